@@ -1,0 +1,270 @@
+/* neoml_hip.h — C ABI of the MI355X (gfx950) math-engine kernels.
+ *
+ * Every entry point below replaces one method of NeoML's IMathEngine interface
+ * (NeoMathEngine/include/NeoMathEngine/NeoMathEngine.h, cited per function as NME.h:<line>).
+ * A handle of the reference (CFloatHandle / CIntHandle = object pointer + byte offset) arrives here
+ * already resolved to a plain device pointer; blob descriptors arrive as plain ints.
+ *
+ * Conventions
+ *   - all pointers are device pointers unless the parameter name ends in _host
+ *   - tensors are dense row-major; images are N,H,W,C (channels last) as in BlobDesc.h:25-35
+ *   - scalars that the reference keeps in engine memory (thresholds, multipliers) are device pointers
+ *   - every function enqueues work on `stream` (a hipStream_t cast to void*, 0 = the null stream)
+ *     and returns without waiting for it
+ *   - return value: NH_OK or an NH_ERR_* code; nhGetLastError() gives the message for the calling thread
+ *   - in-place use (result aliasing an input exactly) is allowed wherever the reference allows it
+ */
+#ifndef NEOML_HIP_H
+#define NEOML_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NH_API __attribute__((visibility("default")))
+
+typedef void* nhStream;
+
+enum {
+	NH_OK = 0,
+	NH_ERR_ARGUMENT = 1,   /* contract violation: the reference would hit ASSERT_EXPR */
+	NH_ERR_HIP = 2,        /* a HIP runtime call failed */
+	NH_ERR_MEMORY = 3,     /* allocation failed or the memory limit was exceeded (OnMemoryError) */
+	NH_ERR_UNSUPPORTED = 4
+};
+
+/* ------------------------------------------------------------------------------------------------
+ * Runtime: device, stream, raw memory, transfers, timing
+ * ---------------------------------------------------------------------------------------------- */
+
+NH_API const char* nhGetLastError(void);
+NH_API int nhGetDeviceCount(int* count);
+/* name_host: at least 256 bytes (CMathEngineInfo::Name, NME.h:1142-1150) */
+NH_API int nhGetDeviceInfo(int device, char* name_host, size_t* total_memory, size_t* free_memory,
+	int* compute_units, int* wave_size);
+NH_API int nhSetDevice(int device);
+NH_API int nhStreamCreate(nhStream* stream);
+NH_API int nhStreamDestroy(nhStream stream);
+NH_API int nhStreamSynchronize(nhStream stream);
+
+/* raw allocator under the caching pool (IRawMemoryManager, src/RawMemoryManager.h:24-29) */
+NH_API int nhRawAlloc(void** ptr, size_t size);
+NH_API int nhRawFree(void* ptr);
+
+/* DataExchangeRaw (NME.h:1219-1220): both wait for completion, like the reference's memcpy */
+NH_API int nhCopyHostToDevice(nhStream stream, void* dst, const void* src_host, size_t size);
+NH_API int nhCopyDeviceToHost(nhStream stream, void* dst_host, const void* src, size_t size);
+NH_API int nhCopyDeviceToDevice(nhStream stream, void* dst, const void* src, size_t size);
+
+/* pinned host staging for GetBuffer/ReleaseBuffer (NME.h:1215-1216) */
+NH_API int nhHostAlloc(void** ptr_host, size_t size);
+NH_API int nhHostFree(void* ptr_host);
+
+/* time between two points of a stream (IPerformanceCounters, PerformanceCounters.h:27-60) */
+typedef void* nhEvent;
+NH_API int nhEventCreate(nhEvent* event);
+NH_API int nhEventDestroy(nhEvent event);
+NH_API int nhEventRecord(nhEvent event, nhStream stream);
+NH_API int nhEventSynchronize(nhEvent event);
+NH_API int nhEventElapsedMs(nhEvent start, nhEvent stop, float* ms_host);
+
+/* ------------------------------------------------------------------------------------------------
+ * Caching device allocator (CMemoryPool + stack allocator behaviour,
+ * src/MemoryPool.cpp:81-88,141-170,275-323; src/MathEngineStackAllocator.cpp:196-320;
+ * src/MemoryEngineMixin.cpp:38-216). kind 0 = device memory, kind 1 = host memory (for tests of the
+ * pool logic on machines without a GPU).
+ * ---------------------------------------------------------------------------------------------- */
+typedef void* nhPool;
+NH_API int nhPoolCreate(nhPool* pool, int kind, size_t memory_limit);
+NH_API int nhPoolDestroy(nhPool pool);
+NH_API int nhPoolSetReuseMemoryMode(nhPool pool, int enable);            /* NME.h:1170 */
+NH_API int nhPoolGetReuseMemoryMode(nhPool pool, int* enabled);          /* NME.h:1171 */
+NH_API int nhPoolSetThreadBufferMemoryThreshold(nhPool pool, size_t t);  /* NME.h:1176 */
+NH_API int nhPoolGetThreadBufferMemoryThreshold(nhPool pool, size_t* t); /* NME.h:1178 */
+NH_API int nhPoolHeapAlloc(nhPool pool, size_t size, void** ptr);        /* NME.h:1180 */
+NH_API int nhPoolHeapFree(nhPool pool, void* ptr);                       /* NME.h:1181 */
+NH_API int nhPoolTransferToThisThread(nhPool pool, void* ptr, size_t size); /* NME.h:1185 */
+NH_API int nhPoolStackAlloc(nhPool pool, size_t size, void** ptr);       /* NME.h:1195 */
+NH_API int nhPoolStackFree(nhPool pool, void* ptr);                      /* NME.h:1196 */
+NH_API int nhPoolCleanUp(nhPool pool);                                   /* NME.h:1211 */
+NH_API int nhPoolGetPeakMemoryUsage(nhPool pool, size_t* bytes);         /* NME.h:1201 */
+NH_API int nhPoolResetPeakMemoryUsage(nhPool pool);                      /* NME.h:1203 */
+NH_API int nhPoolGetCurrentMemoryUsage(nhPool pool, size_t* bytes);      /* NME.h:1205 */
+NH_API int nhPoolGetMemoryInPools(nhPool pool, size_t* bytes);           /* NME.h:1207 */
+
+/* ------------------------------------------------------------------------------------------------
+ * IVectorMathEngine (NME.h:69-387): element-wise kernels, HBM bound
+ * ---------------------------------------------------------------------------------------------- */
+NH_API int nhVectorCopy(nhStream s, float* first, const float* second, int vectorSize);              /* NME.h:73 */
+NH_API int nhVectorCopyInt(nhStream s, int* first, const int* second, int vectorSize);               /* NME.h:74 */
+NH_API int nhVectorFill(nhStream s, float* result, float value, int vectorSize);                     /* NME.h:86 */
+NH_API int nhVectorFillInt(nhStream s, int* result, int value, int vectorSize);                      /* NME.h:87 */
+NH_API int nhVectorFillFromHandle(nhStream s, float* result, int vectorSize, const float* value);    /* NME.h:90 */
+NH_API int nhVectorFillFromHandleInt(nhStream s, int* result, int vectorSize, const int* value);     /* NME.h:91 */
+NH_API int nhVectorConvertFloatToInt(nhStream s, const float* from, int* to, int vectorSize);        /* NME.h:94 */
+NH_API int nhVectorConvertIntToFloat(nhStream s, const int* from, float* to, int vectorSize);        /* NME.h:95 */
+NH_API int nhVectorELU(nhStream s, const float* first, float* result, int vectorSize, const float* alpha);      /* NME.h:136 */
+NH_API int nhVectorReLU(nhStream s, const float* first, float* result, int vectorSize,
+	const float* upperThreshold);                                                                    /* NME.h:144 */
+NH_API int nhVectorLeakyReLU(nhStream s, const float* first, float* result, int vectorSize, const float* alpha); /* NME.h:152 */
+NH_API int nhVectorHSwish(nhStream s, const float* first, float* result, int vectorSize);            /* NME.h:162 */
+NH_API int nhVectorEltwiseMax(nhStream s, const float* first, const float* second, float* result, int vectorSize); /* NME.h:169 */
+NH_API int nhVectorEltwiseMin(nhStream s, const float* first, const float* second, float* result, int vectorSize); /* NME.h:172 */
+NH_API int nhVectorAbs(nhStream s, const float* first, float* result, int vectorSize);               /* NME.h:177 */
+NH_API int nhVectorHardTanh(nhStream s, const float* first, float* result, int vectorSize);          /* NME.h:197 */
+NH_API int nhVectorHardSigmoid(nhStream s, const float* first, float* result, int vectorSize,
+	const float* slope, const float* bias);                                                          /* NME.h:204 */
+NH_API int nhVectorNeg(nhStream s, const float* first, float* result, int vectorSize);               /* NME.h:212 */
+NH_API int nhVectorExp(nhStream s, const float* first, float* result, int vectorSize);               /* NME.h:215 */
+NH_API int nhVectorLog(nhStream s, const float* first, float* result, int vectorSize);               /* NME.h:218 */
+NH_API int nhVectorErf(nhStream s, const float* first, float* result, int vectorSize);               /* NME.h:228 */
+NH_API int nhVectorAdd(nhStream s, const float* first, const float* second, float* result, int vectorSize);     /* NME.h:236 */
+NH_API int nhVectorAddInt(nhStream s, const int* first, const int* second, int* result, int vectorSize);        /* NME.h:238 */
+NH_API int nhVectorAddValue(nhStream s, const float* first, float* result, int vectorSize, const float* addition); /* NME.h:240 */
+NH_API int nhVectorAddValueInt(nhStream s, const int* first, int* result, int vectorSize, const int* addition); /* NME.h:242 */
+NH_API int nhVectorSub(nhStream s, const float* first, const float* second, float* result, int vectorSize);     /* NME.h:249 */
+NH_API int nhVectorSubInt(nhStream s, const int* first, const int* second, int* result, int vectorSize);        /* NME.h:247 */
+NH_API int nhVectorMultiplyAndAdd(nhStream s, const float* first, const float* second, float* result,
+	int vectorSize, const float* mult);                                                              /* NME.h:259 */
+NH_API int nhVectorMultiplyAndSub(nhStream s, const float* first, const float* second, float* result,
+	int vectorSize, const float* mult);                                                              /* NME.h:263 */
+NH_API int nhVectorMultiply(nhStream s, const float* first, float* result, int vectorSize, const float* multiplier); /* NME.h:268 */
+NH_API int nhVectorMultiplyInt(nhStream s, const int* first, int* result, int vectorSize, const int* multiplier);    /* NME.h:270 */
+NH_API int nhVectorNegMultiply(nhStream s, const float* first, float* result, int vectorSize, const float* multiplier); /* NME.h:273 */
+NH_API int nhVectorEltwiseMultiply(nhStream s, const float* first, const float* second, float* result, int vectorSize); /* NME.h:279 */
+NH_API int nhVectorEltwiseMultiplyInt(nhStream s, const int* first, const int* second, int* result, int vectorSize);    /* NME.h:277 */
+NH_API int nhVectorEltwiseMultiplyAdd(nhStream s, const float* first, const float* second, float* result, int vectorSize); /* NME.h:282 */
+NH_API int nhVectorEltwiseNegMultiply(nhStream s, const float* first, const float* second, float* result, int vectorSize); /* NME.h:285 */
+NH_API int nhVectorEltwiseDivide(nhStream s, const float* first, const float* second, float* result, int vectorSize);   /* NME.h:291 */
+NH_API int nhVectorSqrt(nhStream s, const float* first, float* result, int vectorSize);              /* NME.h:299 */
+NH_API int nhVectorInv(nhStream s, const float* first, float* result, int vectorSize);               /* NME.h:302 */
+NH_API int nhVectorMinMax(nhStream s, const float* first, float* result, int vectorSize,
+	const float* minValue, const float* maxValue);                                                   /* NME.h:305 */
+NH_API int nhVectorSigmoid(nhStream s, const float* first, float* result, int vectorSize);           /* NME.h:311 */
+NH_API int nhVectorTanh(nhStream s, const float* first, float* result, int vectorSize);              /* NME.h:319 */
+NH_API int nhVectorSum(nhStream s, const float* first, int vectorSize, float* result);               /* NME.h:105 */
+NH_API int nhVectorDotProduct(nhStream s, const float* first, const float* second, int vectorSize, float* result); /* NME.h:339 */
+
+/* ------------------------------------------------------------------------------------------------
+ * IBlasEngine (NME.h:389-645)
+ * ---------------------------------------------------------------------------------------------- */
+NH_API int nhSetVectorToMatrixRows(nhStream s, float* result, int matrixHeight, int matrixWidth, const float* vector); /* NME.h:393 */
+/* result[b][r][c] = matrix[b][r][c] + vector[b][c] */
+NH_API int nhAddVectorToMatrixRows(nhStream s, int batchSize, const float* matrix, float* result,
+	int matrixHeight, int matrixWidth, const float* vector);                                         /* NME.h:419 */
+/* result[r][c] = matrix[r][c] + vector[r] */
+NH_API int nhAddVectorToMatrixColumns(nhStream s, const float* matrix, float* result,
+	int matrixHeight, int matrixWidth, const float* vector);                                         /* NME.h:423 */
+NH_API int nhSubVectorFromMatrixColumns(nhStream s, const float* matrix, float* result,
+	int matrixHeight, int matrixWidth, const float* vector);                                         /* NME.h:427 */
+/* result[b][c] = sum_r matrix[b][r][c] */
+NH_API int nhSumMatrixRows(nhStream s, int batchSize, float* result, const float* matrix,
+	int matrixHeight, int matrixWidth);                                                              /* NME.h:433 */
+NH_API int nhSumMatrixRowsAdd(nhStream s, int batchSize, float* result, const float* matrix,
+	int matrixHeight, int matrixWidth);                                                              /* NME.h:431 */
+/* result[r] = sum_c matrix[r][c] */
+NH_API int nhSumMatrixColumns(nhStream s, float* result, const float* matrix, int matrixHeight, int matrixWidth); /* NME.h:439 */
+NH_API int nhMatrixSoftmaxByRows(nhStream s, const float* matrix, int height, int width, float* result);          /* NME.h:450 */
+NH_API int nhMatrixLogSumExpByRows(nhStream s, const float* matrix, int height, int width, float* result, int resultSize); /* NME.h:448 */
+/* columnIndices may be null (the overload at NME.h:468) */
+NH_API int nhFindMaxValueInRows(nhStream s, const float* matrix, int matrixHeight, int matrixWidth,
+	float* result, int* columnIndices, int vectorSize);                                              /* NME.h:466-469 */
+NH_API int nhFindMaxValueInColumns(nhStream s, int batchSize, const float* matrix, int matrixHeight,
+	int matrixWidth, float* result, int* rowIndices, int vectorSize);                                /* NME.h:473 */
+/* result[M x N] = first[M x K] * second[N x K]^T with row strides */
+NH_API int nhMultiplyMatrixByTransposedMatrix(nhStream s, const float* first, int firstHeight, int firstWidth,
+	int firstRowSize, const float* second, int secondHeight, int secondRowSize,
+	float* result, int resultRowSize, int resultBufferSize);                                         /* NME.h:529 */
+NH_API int nhBatchMultiplyMatrixByTransposedMatrix(nhStream s, int batchSize, const float* first, int firstHeight,
+	int firstWidth, const float* second, int secondHeight, float* result, int resultBufferSize);     /* NME.h:533 */
+/* result[K1 x N] += first[M x K1]^T * second[M x N] */
+NH_API int nhMultiplyTransposedMatrixByMatrixAndAdd(nhStream s, const float* first, int firstHeight, int firstWidth,
+	int firstRowSize, const float* second, int secondWidth, int secondRowSize,
+	float* result, int resultRowSize, int resultBufferSize);                                         /* NME.h:562 */
+NH_API int nhBatchMultiplyTransposedMatrixByMatrix(nhStream s, int batchSize, const float* first, int firstHeight,
+	int firstWidth, const float* second, int secondWidth, float* result, int resultBufferSize);      /* NME.h:567 */
+NH_API int nhMultiplyDiagMatrixByMatrix(nhStream s, const float* first, int firstSize, const float* second,
+	int secondWidth, float* result, int resultBufferSize);                                           /* NME.h:570 */
+NH_API int nhBatchMultiplyMatrixByMatrix(nhStream s, int batchSize, const float* first, int firstHeight,
+	int firstWidth, const float* second, int secondWidth, float* result, int resultBufferSize);      /* NME.h:580 */
+NH_API int nhBatchMultiplyMatrixByDiagMatrix(nhStream s, int batchSize, const float* first, int height, int width,
+	int firstMatrixOffset, const float* second, int secondMatrixOffset, float* result, int resultBufferSize); /* NME.h:588 */
+/* [b,h,m,w,c] -> [b,w,m,h,c] */
+NH_API int nhTransposeMatrix(nhStream s, int batchSize, const float* first, int height, int medium, int width,
+	int channels, float* result, int resultBufferSize);                                              /* NME.h:599 */
+NH_API int nhTransposeMatrixInt(nhStream s, int batchSize, const int* first, int height, int medium, int width,
+	int channels, int* result, int resultBufferSize);                                                /* NME.h:602 */
+
+/* ------------------------------------------------------------------------------------------------
+ * IDnnEngine (NME.h:691-1113)
+ * ---------------------------------------------------------------------------------------------- */
+
+/* The seven blob dimensions of BlobDesc.h:25-35 in storage order. */
+typedef struct nhBlobDesc {
+	int dims[7]; /* BatchLength, BatchWidth, ListSize, Height, Width, Depth, Channels */
+} nhBlobDesc;
+
+#define NH_MAX_BLOB_DESCS 32 /* MaxBlobDescs, NME.h:1129 */
+
+NH_API int nhBlobMergeByDim(nhStream s, int dim, const nhBlobDesc* from_host, const float* const* fromData_host,
+	int fromCount, const nhBlobDesc* to_host, float* toData);                                        /* NME.h:696 (float) and :698 (int, same bytes) */
+NH_API int nhBlobSplitByDim(nhStream s, int dim, const nhBlobDesc* from_host, const float* fromData,
+	const nhBlobDesc* to_host, float* const* toData_host, int toCount);                              /* NME.h:700,702 */
+
+enum { NH_PAD_CONSTANT = 0, NH_PAD_EDGE = 1, NH_PAD_REFLECT = 2 }; /* TBlobResizePadding, NME.h:62-66 */
+NH_API int nhBlobResizeImage(nhStream s, const nhBlobDesc* from_host, const float* fromData, int deltaLeft,
+	int deltaRight, int deltaTop, int deltaBottom, int padding, float defaultValue,
+	const nhBlobDesc* to_host, float* toData);                                                       /* NME.h:708 */
+
+/* Plain-int form of CCommonConvolutionDesc (src/MathEngineDnnConv.h:24-46).
+ * source N,H,W,Cin (Depth folded into channels); filter [Cout][fh][fw][Cin]; result N,Ho,Wo,Cout. */
+typedef struct nhConvDesc {
+	int batch, height, width, channels;      /* source */
+	int filterCount, filterHeight, filterWidth;
+	int paddingHeight, paddingWidth;
+	int strideHeight, strideWidth;
+	int dilationHeight, dilationWidth;
+	int resultHeight, resultWidth;
+} nhConvDesc;
+
+/* InitBlobConvolution (NME.h:751): fills resultHeight/resultWidth and validates; returns NH_ERR_ARGUMENT
+ * where the reference asserts. */
+NH_API int nhInitBlobConvolution(nhConvDesc* desc_host);
+/* freeTerm may be null */
+NH_API int nhBlobConvolution(nhStream s, const nhConvDesc* desc_host, const float* source, const float* filter,
+	const float* freeTerm, float* result);                                                           /* NME.h:755 */
+
+/* depthwise: filter [fh][fw][C], no dilation (src/MathEngineDnnConv.h:69-90) */
+NH_API int nhInitBlobChannelwiseConvolution(nhConvDesc* desc_host);                                  /* NME.h:766 */
+NH_API int nhBlobChannelwiseConvolution(nhStream s, const nhConvDesc* desc_host, const float* source,
+	const float* filter, const float* freeTerm, float* result);                                      /* NME.h:770 */
+
+/* CCommon2DPoolingDesc (src/MathEngineDnnPoolings.h:24-60): no padding; Ho = (H - fh) / sh + 1 */
+typedef struct nhPoolingDesc {
+	int batch, height, width, channels;
+	int filterHeight, filterWidth, strideHeight, strideWidth;
+	int resultHeight, resultWidth;
+} nhPoolingDesc;
+NH_API int nhInitPooling(nhPoolingDesc* desc_host);                                                  /* NME.h:817,837 */
+/* maxIndices may be null; when given it receives the reference CPU engine's index (see the kernel) */
+NH_API int nhBlobMaxPooling(nhStream s, const nhPoolingDesc* desc_host, const float* source, int* maxIndices,
+	float* result);                                                                                  /* NME.h:821 */
+NH_API int nhBlobMeanPooling(nhStream s, const nhPoolingDesc* desc_host, const float* source, float* result); /* NME.h:841 */
+
+/* LSTM (NME.h:1005-1011). Weights: inputWeights [4H x objectSize], recurrentWeights [4H x H]; gate order in
+ * the 4H vector: main(tanh) | forget | input | output (src/CPU/CpuMathEngineDnnLstm.h:49-90).
+ * Free terms, inputStateBackLink, inputMainBackLink and outputStateBackLink may be null.
+ * workspace: nhLstmWorkspaceSize bytes of device memory, owned by the caller. */
+NH_API int nhLstmWorkspaceSize(int hiddenSize, int objectSize, int sequenceLength, int sequenceCount, size_t* bytes);
+NH_API int nhLstm(nhStream s, int hiddenSize, int objectSize, const float* inputWeights, const float* inputFreeTerm,
+	const float* recurrentWeights, const float* recurrentFreeTerm, int reverse, int sequenceLength,
+	int sequenceCount, const float* inputStateBackLink, const float* inputMainBackLink, const float* input,
+	float* outputStateBackLink, float* outputMainBackLink, void* workspace, size_t workspaceSize);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NEOML_HIP_H */

@@ -1,0 +1,610 @@
+// Bandwidth-bound matrix helpers of IBlasEngine: row/column broadcasts, row/column sums, softmax, arg-max,
+// diagonal products and the blob transpose. Row reductions give one 64-lane wavefront to each row and reduce
+// with cross-lane shuffles; element-wise broadcasts use 128-bit accesses when shapes and pointers allow it.
+#include "common.h"
+#include <float.h>
+
+namespace nh {
+
+// ---------------------------------------------------------------------------------------------------------
+// Broadcast family: result[i] = f( matrix[matIndex( i )], vector[vecIndex( i )] )
+
+enum TBroadcastOp { BO_Add, BO_Sub, BO_Mul, BO_Set };
+
+template<int OP> __device__ __forceinline__ float broadcastApply( float m, float v )
+{
+	switch( OP ) {
+		case BO_Add: return m + v;
+		case BO_Sub: return m - v;
+		case BO_Mul: return m * v;
+		default: return v;
+	}
+}
+
+// Row broadcast: element ( b, r, c ) pairs with vector[b * vecBatchStride + c];
+// the matrix of batch b starts at b * matBatchStride (result is always dense).
+template<int OP, bool VEC>
+__global__ __launch_bounds__( 256 )
+void rowBroadcastKernel( const float* matrix, float* result, const float* vector, int height, int width,
+	long long total, int matBatchStride, int vecBatchStride )
+{
+	const long long step = static_cast<long long>( gridDim.x ) * 256;
+	const int hw = height * width;
+	if( VEC ) {
+		const long long total4 = total >> 2;
+		for( long long i4 = blockIdx.x * 256LL + threadIdx.x; i4 < total4; i4 += step ) {
+			const long long i = i4 << 2;
+			const int b = static_cast<int>( i / hw );
+			const int inMat = static_cast<int>( i - static_cast<long long>( b ) * hw );
+			const int c = inMat % width;
+			const float4 v = *reinterpret_cast<const float4*>( vector + static_cast<long long>( b ) * vecBatchStride + c );
+			float4 m = make_float4( 0.f, 0.f, 0.f, 0.f );
+			if( OP != BO_Set ) {
+				m = *reinterpret_cast<const float4*>( matrix + static_cast<long long>( b ) * matBatchStride + inMat );
+			}
+			float4 r;
+			r.x = broadcastApply<OP>( m.x, v.x );
+			r.y = broadcastApply<OP>( m.y, v.y );
+			r.z = broadcastApply<OP>( m.z, v.z );
+			r.w = broadcastApply<OP>( m.w, v.w );
+			*reinterpret_cast<float4*>( result + i ) = r;
+		}
+	} else {
+		for( long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += step ) {
+			const int b = static_cast<int>( i / hw );
+			const int inMat = static_cast<int>( i - static_cast<long long>( b ) * hw );
+			const int c = inMat % width;
+			const float v = vector[static_cast<long long>( b ) * vecBatchStride + c];
+			const float m = OP != BO_Set ? matrix[static_cast<long long>( b ) * matBatchStride + inMat] : 0.f;
+			result[i] = broadcastApply<OP>( m, v );
+		}
+	}
+}
+
+template<int OP>
+static int launchRowBroadcast( nhStream s, const float* matrix, float* result, const float* vector, int batch,
+	int height, int width, int matBatchStride, int vecBatchStride )
+{
+	const long long total = static_cast<long long>( batch ) * height * width;
+	if( total == 0 ) {
+		return NH_OK;
+	}
+	const bool vec = width % 4 == 0 && matBatchStride % 4 == 0 && vecBatchStride % 4 == 0 && isAligned16( result )
+		&& isAligned16( vector ) && ( OP == BO_Set || isAligned16( matrix ) );
+	const long long work = vec ? total / 4 : total;
+	long long blocks = ( work + 1023 ) / 1024; // 4 items per thread
+	blocks = blocks > 65536 ? 65536 : blocks;
+	if( vec ) {
+		hipLaunchKernelGGL( ( rowBroadcastKernel<OP, true> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			matrix, result, vector, height, width, total, matBatchStride, vecBatchStride );
+	} else {
+		hipLaunchKernelGGL( ( rowBroadcastKernel<OP, false> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			matrix, result, vector, height, width, total, matBatchStride, vecBatchStride );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+// Column broadcast: element ( r, c ) pairs with vector[r].
+template<int OP, bool VEC>
+__global__ __launch_bounds__( 256 )
+void columnBroadcastKernel( const float* matrix, float* result, const float* vector, int width, long long total )
+{
+	const long long step = static_cast<long long>( gridDim.x ) * 256;
+	if( VEC ) {
+		const long long total4 = total >> 2;
+		for( long long i4 = blockIdx.x * 256LL + threadIdx.x; i4 < total4; i4 += step ) {
+			const long long i = i4 << 2;
+			const float v = vector[i / width];
+			const float4 m = *reinterpret_cast<const float4*>( matrix + i );
+			float4 r;
+			r.x = broadcastApply<OP>( m.x, v );
+			r.y = broadcastApply<OP>( m.y, v );
+			r.z = broadcastApply<OP>( m.z, v );
+			r.w = broadcastApply<OP>( m.w, v );
+			*reinterpret_cast<float4*>( result + i ) = r;
+		}
+	} else {
+		for( long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += step ) {
+			result[i] = broadcastApply<OP>( matrix[i], vector[i / width] );
+		}
+	}
+}
+
+template<int OP>
+static int launchColumnBroadcast( nhStream s, const float* matrix, float* result, const float* vector, int height, int width )
+{
+	const long long total = static_cast<long long>( height ) * width;
+	if( total == 0 ) {
+		return NH_OK;
+	}
+	const bool vec = width % 4 == 0 && isAligned16( result ) && isAligned16( matrix );
+	const long long work = vec ? total / 4 : total;
+	long long blocks = ( work + 1023 ) / 1024;
+	blocks = blocks > 65536 ? 65536 : blocks;
+	if( vec ) {
+		hipLaunchKernelGGL( ( columnBroadcastKernel<OP, true> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			matrix, result, vector, width, total );
+	} else {
+		hipLaunchKernelGGL( ( columnBroadcastKernel<OP, false> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			matrix, result, vector, width, total );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Row reductions: one wavefront per row
+
+constexpr int RowsPerBlock = 4; // 256 threads
+
+// result[r] = sum_c matrix[r][c]
+__global__ __launch_bounds__( 256 )
+void sumColumnsKernel( float* result, const float* matrix, int height, int width, int vec )
+{
+	const int row = blockIdx.x * RowsPerBlock + ( threadIdx.x >> 6 );
+	if( row >= height ) {
+		return;
+	}
+	const int lane = threadIdx.x & 63;
+	const float* p = matrix + static_cast<long long>( row ) * width;
+	float s = 0.f;
+	if( vec ) {
+		const int w4 = width >> 2;
+		for( int i = lane; i < w4; i += 64 ) {
+			const float4 v = reinterpret_cast<const float4*>( p )[i];
+			s += ( v.x + v.y ) + ( v.z + v.w );
+		}
+	} else {
+		for( int i = lane; i < width; i += 64 ) {
+			s += p[i];
+		}
+	}
+	s = waveReduceSum( s );
+	if( lane == 0 ) {
+		result[row] = s;
+	}
+}
+
+// result[b][c] (+)= sum_r matrix[b][r][c]; rows [rowBegin, rowEnd) of this slice, one thread per column.
+// With several slices the partial sums meet in the result through atomic adds.
+__global__ __launch_bounds__( 256 )
+void sumRowsKernel( float* result, const float* matrix, int height, int width, int rowsPerSlice, int accumulate )
+{
+	const int c = blockIdx.x * 256 + threadIdx.x;
+	if( c >= width ) {
+		return;
+	}
+	const int b = blockIdx.y;
+	const int rowBegin = blockIdx.z * rowsPerSlice;
+	int rowEnd = rowBegin + rowsPerSlice;
+	rowEnd = rowEnd > height ? height : rowEnd;
+	const float* p = matrix + ( static_cast<long long>( b ) * height + rowBegin ) * width + c;
+	float s = 0.f;
+	for( int r = rowBegin; r < rowEnd; ++r ) {
+		s += *p;
+		p += width;
+	}
+	float* out = result + static_cast<long long>( b ) * width + c;
+	if( gridDim.z > 1 ) {
+		atomicAdd( out, s );
+	} else if( accumulate ) {
+		*out += s;
+	} else {
+		*out = s;
+	}
+}
+
+// Softmax / log-sum-exp of one row per wavefront. Rows of up to 64 * CACHE elements stay in registers between
+// the three passes (max, sum of exp, scale); longer rows are read again from memory.
+// The formula follows the reference: exp( x - max ) * ( 1 / sum ) (src/CPU/CpuMathEngineBlas.cpp:1131-1159).
+template<int CACHE, bool LOGSUMEXP>
+__global__ __launch_bounds__( 256 )
+void softmaxRowsKernel( const float* matrix, int height, int width, float* result )
+{
+	const int row = blockIdx.x * RowsPerBlock + ( threadIdx.x >> 6 );
+	if( row >= height ) {
+		return;
+	}
+	const int lane = threadIdx.x & 63;
+	const float* p = matrix + static_cast<long long>( row ) * width;
+	float cache[CACHE > 0 ? CACHE : 1];
+	float mx = -FLT_MAX;
+	if( CACHE > 0 ) {
+#pragma unroll
+		for( int j = 0; j < CACHE; ++j ) {
+			const int i = lane + j * 64;
+			cache[j] = i < width ? p[i] : -FLT_MAX;
+			mx = fmaxf( mx, cache[j] );
+		}
+	} else {
+		for( int i = lane; i < width; i += 64 ) {
+			mx = fmaxf( mx, p[i] );
+		}
+	}
+	mx = waveReduceMax( mx );
+	float sum = 0.f;
+	if( CACHE > 0 ) {
+#pragma unroll
+		for( int j = 0; j < CACHE; ++j ) {
+			const int i = lane + j * 64;
+			cache[j] = i < width ? expf( cache[j] - mx ) : 0.f;
+			sum += cache[j];
+		}
+	} else {
+		for( int i = lane; i < width; i += 64 ) {
+			sum += expf( p[i] - mx );
+		}
+	}
+	sum = waveReduceSum( sum );
+	if( LOGSUMEXP ) {
+		if( lane == 0 ) {
+			result[row] = mx + logf( sum );
+		}
+		return;
+	}
+	const float inv = 1.f / sum;
+	float* q = result + static_cast<long long>( row ) * width;
+	if( CACHE > 0 ) {
+#pragma unroll
+		for( int j = 0; j < CACHE; ++j ) {
+			const int i = lane + j * 64;
+			if( i < width ) {
+				q[i] = cache[j] * inv;
+			}
+		}
+	} else {
+		for( int i = lane; i < width; i += 64 ) {
+			q[i] = expf( p[i] - mx ) * inv;
+		}
+	}
+}
+
+// Maximum of a row and the index of its first occurrence
+__global__ __launch_bounds__( 256 )
+void findMaxInRowsKernel( const float* matrix, int height, int width, float* result, int* indices )
+{
+	const int row = blockIdx.x * RowsPerBlock + ( threadIdx.x >> 6 );
+	if( row >= height ) {
+		return;
+	}
+	const int lane = threadIdx.x & 63;
+	const float* p = matrix + static_cast<long long>( row ) * width;
+	float best = -FLT_MAX;
+	int bestIdx = 0x7fffffff;
+	for( int i = lane; i < width; i += 64 ) {
+		const float v = p[i];
+		if( bestIdx == 0x7fffffff || v > best ) {
+			best = v;
+			bestIdx = i;
+		}
+	}
+#pragma unroll
+	for( int off = 32; off > 0; off >>= 1 ) {
+		const float ov = __shfl_xor( best, off, 64 );
+		const int oi = __shfl_xor( bestIdx, off, 64 );
+		if( oi != 0x7fffffff && ( bestIdx == 0x7fffffff || ov > best || ( ov == best && oi < bestIdx ) ) ) {
+			best = ov;
+			bestIdx = oi;
+		}
+	}
+	if( lane == 0 ) {
+		result[row] = best;
+		if( indices != nullptr ) {
+			indices[row] = bestIdx;
+		}
+	}
+}
+
+// Maximum of every column of each [height x width] matrix of the batch; first row wins ties
+__global__ __launch_bounds__( 256 )
+void findMaxInColumnsKernel( const float* matrix, int height, int width, float* result, int* indices )
+{
+	const int c = blockIdx.x * 256 + threadIdx.x;
+	if( c >= width ) {
+		return;
+	}
+	const int b = blockIdx.y;
+	const float* p = matrix + static_cast<long long>( b ) * height * width + c;
+	float best = *p;
+	int bestIdx = 0;
+	for( int r = 1; r < height; ++r ) {
+		p += width;
+		const float v = *p;
+		if( v > best ) {
+			best = v;
+			bestIdx = r;
+		}
+	}
+	result[static_cast<long long>( b ) * width + c] = best;
+	indices[static_cast<long long>( b ) * width + c] = bestIdx;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Transpose [b, h, m, w, c] -> [b, w, m, h, c]
+
+// General form: one thread per group of VECW output elements (VECW divides c); reads are contiguous runs of c.
+template<typename T, int VECW>
+__global__ __launch_bounds__( 256 )
+void transposeCellsKernel( const T* in, T* out, int height, int medium, int width, int channels, long long totalGroups )
+{
+	const int cg = channels / VECW;
+	const long long step = static_cast<long long>( gridDim.x ) * 256;
+	for( long long g = blockIdx.x * 256LL + threadIdx.x; g < totalGroups; g += step ) {
+		long long t = g;
+		const int ch = static_cast<int>( t % cg ) * VECW; t /= cg;
+		const int j = static_cast<int>( t % height ); t /= height;
+		const int m = static_cast<int>( t % medium ); t /= medium;
+		const int i = static_cast<int>( t % width ); t /= width;
+		const long long b = t;
+		const long long src = ( ( ( b * height + j ) * medium + m ) * width + i ) * channels + ch;
+		const long long dst = g * VECW;
+		if( VECW == 4 ) {
+			*reinterpret_cast<int4*>( out + dst ) = *reinterpret_cast<const int4*>( in + src );
+		} else {
+			out[dst] = in[src];
+		}
+	}
+}
+
+// Plain matrices (m == 1, c == 1): 64x64 tiles through LDS so that both the read and the write are coalesced.
+template<typename T>
+__global__ __launch_bounds__( 256 )
+void transposePlainKernel( const T* in, T* out, int height, int width )
+{
+	__shared__ T tile[64][65];
+	const long long base = static_cast<long long>( blockIdx.z ) * height * width;
+	const int x0 = blockIdx.x * 64;
+	const int y0 = blockIdx.y * 64;
+	const int tx = threadIdx.x & 63;
+	const int ty = threadIdx.x >> 6;
+	for( int r = ty; r < 64; r += 4 ) {
+		const int y = y0 + r;
+		const int x = x0 + tx;
+		if( y < height && x < width ) {
+			tile[r][tx] = in[base + static_cast<long long>( y ) * width + x];
+		}
+	}
+	__syncthreads();
+	for( int r = ty; r < 64; r += 4 ) {
+		const int x = x0 + r; // row of the result
+		const int y = y0 + tx;
+		if( x < width && y < height ) {
+			out[base + static_cast<long long>( x ) * height + y] = tile[tx][r];
+		}
+	}
+}
+
+template<typename T>
+static int transposeImpl( nhStream s, int batchSize, const T* first, int height, int medium, int width, int channels,
+	T* result, int resultBufferSize )
+{
+	if( batchSize < 0 || height < 0 || medium < 0 || width < 0 || channels < 0 ) {
+		setLastError( "TransposeMatrix: negative dimension" );
+		return NH_ERR_ARGUMENT;
+	}
+	const long long total = static_cast<long long>( batchSize ) * height * medium * width * channels;
+	if( total > resultBufferSize ) {
+		setLastError( "TransposeMatrix: result buffer is too small" );
+		return NH_ERR_ARGUMENT;
+	}
+	if( total == 0 ) {
+		return NH_OK;
+	}
+	if( first == result ) {
+		setLastError( "TransposeMatrix: in-place transposition is not supported" );
+		return NH_ERR_ARGUMENT;
+	}
+	if( height == 1 || width == 1 ) {
+		// [b,1,m,w,c] -> [b,w,m,1,c] moves whole rows when m == 1 and is a (w x m) cell transpose otherwise
+		if( medium == 1 ) {
+			NH_HIP( hipMemcpyAsync( result, first, total * sizeof( T ), hipMemcpyDeviceToDevice, toStream( s ) ) );
+			return NH_OK;
+		}
+	}
+	if( medium == 1 && channels == 1 ) {
+		const dim3 grid( ceilDiv( width, 64 ), ceilDiv( height, 64 ), batchSize );
+		if( grid.y <= 65535 && grid.z <= 65535 ) {
+			hipLaunchKernelGGL( transposePlainKernel<T>, grid, dim3( 256 ), 0, toStream( s ), first, result, height, width );
+			NH_LAUNCH_CHECK();
+			return NH_OK;
+		}
+	}
+	const bool vec = channels % 4 == 0 && isAligned16( first ) && isAligned16( result );
+	const long long groups = vec ? total / 4 : total;
+	long long blocks = ( groups + 255 ) / 256;
+	blocks = blocks > 262144 ? 262144 : blocks;
+	if( vec ) {
+		hipLaunchKernelGGL( ( transposeCellsKernel<T, 4> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			first, result, height, medium, width, channels, groups );
+	} else {
+		hipLaunchKernelGGL( ( transposeCellsKernel<T, 1> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			first, result, height, medium, width, channels, groups );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+} // namespace nh
+
+using namespace nh;
+
+static int sumMatrixRowsImpl( nhStream s, int batchSize, float* result, const float* matrix, int matrixHeight,
+	int matrixWidth, bool accumulate )
+{
+	if( batchSize == 0 || matrixWidth == 0 ) {
+		return NH_OK;
+	}
+	const int colBlocks = ceilDiv( matrixWidth, 256 );
+	// split tall matrices over several workgroups until about 1024 of them exist
+	int slices = 1;
+	const long long base = static_cast<long long>( colBlocks ) * batchSize;
+	if( base < 512 && matrixHeight >= 256 ) {
+		slices = static_cast<int>( 1024 / base );
+		const int maxSlices = matrixHeight / 64;
+		slices = slices > maxSlices ? maxSlices : slices;
+		slices = slices < 1 ? 1 : slices;
+	}
+	if( slices > 1 && !accumulate ) {
+		const int rc = nhVectorFill( s, result, 0.f, batchSize * matrixWidth );
+		if( rc != NH_OK ) {
+			return rc;
+		}
+	}
+	const int rowsPerSlice = ceilDiv( matrixHeight, slices );
+	slices = matrixHeight == 0 ? 1 : ceilDiv( matrixHeight, rowsPerSlice );
+	if( batchSize > 65535 || slices > 65535 ) {
+		setLastError( "SumMatrixRows: batch is too large" );
+		return NH_ERR_ARGUMENT;
+	}
+	hipLaunchKernelGGL( sumRowsKernel, dim3( colBlocks, batchSize, slices ), dim3( 256 ), 0, toStream( s ),
+		result, matrix, matrixHeight, matrixWidth, rowsPerSlice, accumulate ? 1 : 0 );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+template<bool LOGSUMEXP>
+static int softmaxImpl( nhStream s, const float* matrix, int height, int width, float* result )
+{
+	if( height == 0 || width == 0 ) {
+		return NH_OK;
+	}
+	const dim3 grid( ceilDiv( height, RowsPerBlock ) );
+	if( width <= 64 ) {
+		hipLaunchKernelGGL( ( softmaxRowsKernel<1, LOGSUMEXP> ), grid, dim3( 256 ), 0, toStream( s ), matrix, height, width, result );
+	} else if( width <= 256 ) {
+		hipLaunchKernelGGL( ( softmaxRowsKernel<4, LOGSUMEXP> ), grid, dim3( 256 ), 0, toStream( s ), matrix, height, width, result );
+	} else if( width <= 1024 ) {
+		hipLaunchKernelGGL( ( softmaxRowsKernel<16, LOGSUMEXP> ), grid, dim3( 256 ), 0, toStream( s ), matrix, height, width, result );
+	} else {
+		hipLaunchKernelGGL( ( softmaxRowsKernel<0, LOGSUMEXP> ), grid, dim3( 256 ), 0, toStream( s ), matrix, height, width, result );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+extern "C" {
+
+
+int nhSetVectorToMatrixRows( nhStream s, float* result, int matrixHeight, int matrixWidth, const float* vector )
+{
+	NH_REQUIRE( matrixHeight >= 0 && matrixWidth >= 0 );
+	return launchRowBroadcast<BO_Set>( s, nullptr, result, vector, 1, matrixHeight, matrixWidth, 0, 0 );
+}
+
+int nhAddVectorToMatrixRows( nhStream s, int batchSize, const float* matrix, float* result,
+	int matrixHeight, int matrixWidth, const float* vector )
+{
+	NH_REQUIRE( batchSize >= 0 && matrixHeight >= 0 && matrixWidth >= 0 );
+	NH_REQUIRE( static_cast<long long>( matrixHeight ) * matrixWidth <= 0x7fffffffLL );
+	return launchRowBroadcast<BO_Add>( s, matrix, result, vector, batchSize, matrixHeight, matrixWidth,
+		matrixHeight * matrixWidth, matrixWidth );
+}
+
+int nhAddVectorToMatrixColumns( nhStream s, const float* matrix, float* result, int matrixHeight, int matrixWidth,
+	const float* vector )
+{
+	NH_REQUIRE( matrixHeight >= 0 && matrixWidth >= 0 );
+	return launchColumnBroadcast<BO_Add>( s, matrix, result, vector, matrixHeight, matrixWidth );
+}
+
+int nhSubVectorFromMatrixColumns( nhStream s, const float* matrix, float* result, int matrixHeight, int matrixWidth,
+	const float* vector )
+{
+	NH_REQUIRE( matrixHeight >= 0 && matrixWidth >= 0 );
+	return launchColumnBroadcast<BO_Sub>( s, matrix, result, vector, matrixHeight, matrixWidth );
+}
+
+int nhMultiplyDiagMatrixByMatrix( nhStream s, const float* first, int firstSize, const float* second,
+	int secondWidth, float* result, int resultBufferSize )
+{
+	NH_REQUIRE( firstSize >= 0 && secondWidth >= 0 );
+	NH_REQUIRE( static_cast<long long>( firstSize ) * secondWidth <= resultBufferSize );
+	return launchColumnBroadcast<BO_Mul>( s, second, result, first, firstSize, secondWidth );
+}
+
+int nhBatchMultiplyMatrixByDiagMatrix( nhStream s, int batchSize, const float* first, int height, int width,
+	int firstMatrixOffset, const float* second, int secondMatrixOffset, float* result, int resultBufferSize )
+{
+	NH_REQUIRE( batchSize >= 0 && height >= 0 && width >= 0 && firstMatrixOffset >= 0 && secondMatrixOffset >= 0 );
+	NH_REQUIRE( static_cast<long long>( batchSize ) * height * width <= resultBufferSize );
+	return launchRowBroadcast<BO_Mul>( s, first, result, second, batchSize, height, width, firstMatrixOffset, secondMatrixOffset );
+}
+
+int nhSumMatrixRows( nhStream s, int batchSize, float* result, const float* matrix, int matrixHeight, int matrixWidth )
+{
+	NH_REQUIRE( batchSize >= 0 && matrixHeight >= 0 && matrixWidth >= 0 );
+	return sumMatrixRowsImpl( s, batchSize, result, matrix, matrixHeight, matrixWidth, false );
+}
+
+int nhSumMatrixRowsAdd( nhStream s, int batchSize, float* result, const float* matrix, int matrixHeight, int matrixWidth )
+{
+	NH_REQUIRE( batchSize >= 0 && matrixHeight >= 0 && matrixWidth >= 0 );
+	return sumMatrixRowsImpl( s, batchSize, result, matrix, matrixHeight, matrixWidth, true );
+}
+
+int nhSumMatrixColumns( nhStream s, float* result, const float* matrix, int matrixHeight, int matrixWidth )
+{
+	NH_REQUIRE( matrixHeight >= 0 && matrixWidth >= 0 );
+	if( matrixHeight == 0 ) {
+		return NH_OK;
+	}
+	const int vec = ( matrixWidth % 4 == 0 && isAligned16( matrix ) ) ? 1 : 0;
+	hipLaunchKernelGGL( sumColumnsKernel, dim3( ceilDiv( matrixHeight, RowsPerBlock ) ), dim3( 256 ), 0, toStream( s ),
+		result, matrix, matrixHeight, matrixWidth, vec );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+int nhMatrixSoftmaxByRows( nhStream s, const float* matrix, int height, int width, float* result )
+{
+	NH_REQUIRE( height >= 0 && width >= 0 );
+	return softmaxImpl<false>( s, matrix, height, width, result );
+}
+
+int nhMatrixLogSumExpByRows( nhStream s, const float* matrix, int height, int width, float* result, int resultSize )
+{
+	NH_REQUIRE( height >= 0 && width >= 0 && resultSize >= height );
+	return softmaxImpl<true>( s, matrix, height, width, result );
+}
+
+int nhFindMaxValueInRows( nhStream s, const float* matrix, int matrixHeight, int matrixWidth,
+	float* result, int* columnIndices, int vectorSize )
+{
+	NH_REQUIRE( matrixHeight >= 0 && matrixWidth > 0 && vectorSize >= matrixHeight );
+	if( matrixHeight == 0 ) {
+		return NH_OK;
+	}
+	hipLaunchKernelGGL( findMaxInRowsKernel, dim3( ceilDiv( matrixHeight, RowsPerBlock ) ), dim3( 256 ), 0, toStream( s ),
+		matrix, matrixHeight, matrixWidth, result, columnIndices );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+int nhFindMaxValueInColumns( nhStream s, int batchSize, const float* matrix, int matrixHeight,
+	int matrixWidth, float* result, int* rowIndices, int vectorSize )
+{
+	NH_REQUIRE( batchSize >= 0 && matrixHeight > 0 && matrixWidth >= 0 && rowIndices != nullptr );
+	NH_REQUIRE( static_cast<long long>( batchSize ) * matrixWidth <= vectorSize && batchSize <= 65535 );
+	if( batchSize == 0 || matrixWidth == 0 ) {
+		return NH_OK;
+	}
+	hipLaunchKernelGGL( findMaxInColumnsKernel, dim3( ceilDiv( matrixWidth, 256 ), batchSize ), dim3( 256 ), 0, toStream( s ),
+		matrix, matrixHeight, matrixWidth, result, rowIndices );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+int nhTransposeMatrix( nhStream s, int batchSize, const float* first, int height, int medium, int width,
+	int channels, float* result, int resultBufferSize )
+{
+	return transposeImpl<float>( s, batchSize, first, height, medium, width, channels, result, resultBufferSize );
+}
+
+int nhTransposeMatrixInt( nhStream s, int batchSize, const int* first, int height, int medium, int width,
+	int channels, int* result, int resultBufferSize )
+{
+	return transposeImpl<int>( s, batchSize, first, height, medium, width, channels, result, resultBufferSize );
+}
+
+} // extern "C"

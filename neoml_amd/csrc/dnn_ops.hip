@@ -1,0 +1,670 @@
+// Bandwidth-bound blob kernels of IDnnEngine on channels-last images: depthwise (channelwise) convolution,
+// 2-D max / mean pooling, image padding / cropping, split / merge along a blob dimension, and the LSTM
+// recurrence (matrix products on the MFMA kernels + one fused gate kernel per step).
+#include "common.h"
+#include <float.h>
+
+namespace nh {
+
+// matrix products defined in gemm_mfma.hip
+int matMulNT( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
+	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC,
+	const float* bias, bool accumulate );
+
+// ---------------------------------------------------------------------------------------------------------
+// Channelwise convolution: out[n,ho,wo,c] = bias[c] + sum_{kh,kw} in[n, ho*s-p+kh, wo*s-p+kw, c] * filt[kh,kw,c]
+// One thread owns VECW channels of WPT horizontally adjacent output pixels, so that the input columns shared
+// by neighbouring windows are loaded once and the filter taps stay in registers.
+
+template<int VECW> struct CChanVec;
+template<> struct CChanVec<4> {
+	typedef float4 Type;
+	static __device__ __forceinline__ float4 load( const float* p ) { return *reinterpret_cast<const float4*>( p ); }
+	static __device__ __forceinline__ void store( float* p, float4 v ) { *reinterpret_cast<float4*>( p ) = v; }
+	static __device__ __forceinline__ float4 zero() { return make_float4( 0.f, 0.f, 0.f, 0.f ); }
+	static __device__ __forceinline__ float4 fma( float4 a, float4 b, float4 c )
+	{
+		return make_float4( fmaf( a.x, b.x, c.x ), fmaf( a.y, b.y, c.y ), fmaf( a.z, b.z, c.z ), fmaf( a.w, b.w, c.w ) );
+	}
+};
+template<> struct CChanVec<1> {
+	typedef float Type;
+	static __device__ __forceinline__ float load( const float* p ) { return *p; }
+	static __device__ __forceinline__ void store( float* p, float v ) { *p = v; }
+	static __device__ __forceinline__ float zero() { return 0.f; }
+	static __device__ __forceinline__ float fma( float a, float b, float c ) { return fmaf( a, b, c ); }
+};
+
+template<int VECW, int WPT>
+__global__ __launch_bounds__( 256 )
+void channelwiseConvKernel( const nhConvDesc d, const float* source, const float* filter, const float* freeTerm,
+	float* result, int wGroups, long long totalItems )
+{
+	typedef CChanVec<VECW> V;
+	typedef typename V::Type T;
+	const int cg = d.channels / VECW;
+	const long long step = static_cast<long long>( gridDim.x ) * 256;
+	for( long long item = blockIdx.x * 256LL + threadIdx.x; item < totalItems; item += step ) {
+		long long t = item;
+		const int c = static_cast<int>( t % cg ) * VECW; t /= cg;
+		const int wo0 = static_cast<int>( t % wGroups ) * WPT; t /= wGroups;
+		const int ho = static_cast<int>( t % d.resultHeight ); t /= d.resultHeight;
+		const long long n = t;
+
+		T acc[WPT];
+		const T bias = freeTerm != nullptr ? V::load( freeTerm + c ) : V::zero();
+#pragma unroll
+		for( int j = 0; j < WPT; ++j ) {
+			acc[j] = bias;
+		}
+		const float* image = source + n * d.height * d.width * d.channels + c;
+		const int hi0 = ho * d.strideHeight - d.paddingHeight;
+		const int wi0 = wo0 * d.strideWidth - d.paddingWidth;
+		for( int kh = 0; kh < d.filterHeight; ++kh ) {
+			const int hi = hi0 + kh;
+			if( hi < 0 || hi >= d.height ) {
+				continue;
+			}
+			const float* row = image + static_cast<long long>( hi ) * d.width * d.channels;
+			for( int kw = 0; kw < d.filterWidth; ++kw ) {
+				const T f = V::load( filter + ( kh * d.filterWidth + kw ) * d.channels + c );
+#pragma unroll
+				for( int j = 0; j < WPT; ++j ) {
+					const int wi = wi0 + j * d.strideWidth + kw;
+					if( wi >= 0 && wi < d.width && wo0 + j < d.resultWidth ) {
+						acc[j] = V::fma( V::load( row + static_cast<long long>( wi ) * d.channels ), f, acc[j] );
+					}
+				}
+			}
+		}
+		float* out = result + ( ( n * d.resultHeight + ho ) * d.resultWidth + wo0 ) * d.channels + c;
+#pragma unroll
+		for( int j = 0; j < WPT; ++j ) {
+			if( wo0 + j < d.resultWidth ) {
+				V::store( out + static_cast<long long>( j ) * d.channels, acc[j] );
+			}
+		}
+	}
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Pooling, one thread per VECW channels of one output pixel
+
+template<int VECW, bool MEAN>
+__global__ __launch_bounds__( 256 )
+void poolingKernel( const nhPoolingDesc d, const float* source, float* result, long long totalItems )
+{
+	const int cg = d.channels / VECW;
+	const long long step = static_cast<long long>( gridDim.x ) * 256;
+	// ( 1 / fh ) / fw as the reference computes it (src/CPU/CpuMathEngineDnnPooling.h:68-69)
+	const float scale = 1.f / d.filterHeight / d.filterWidth;
+	for( long long item = blockIdx.x * 256LL + threadIdx.x; item < totalItems; item += step ) {
+		long long t = item;
+		const int c = static_cast<int>( t % cg ) * VECW; t /= cg;
+		const int wo = static_cast<int>( t % d.resultWidth ); t /= d.resultWidth;
+		const int ho = static_cast<int>( t % d.resultHeight ); t /= d.resultHeight;
+		const long long n = t;
+		const float* window = source + ( ( n * d.height + ho * d.strideHeight ) * d.width + wo * d.strideWidth ) * d.channels + c;
+		float acc[VECW];
+		// columns outside, rows inside: the reference reduces over the rows of each column first
+		for( int kw = 0; kw < d.filterWidth; ++kw ) {
+			float col[VECW];
+			for( int kh = 0; kh < d.filterHeight; ++kh ) {
+				const float* p = window + ( static_cast<long long>( kh ) * d.width + kw ) * d.channels;
+				float v[VECW];
+				if constexpr( VECW == 4 ) {
+					const float4 q = *reinterpret_cast<const float4*>( p );
+					v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+				} else {
+					v[0] = *p;
+				}
+#pragma unroll
+				for( int e = 0; e < VECW; ++e ) {
+					if( kh == 0 ) {
+						col[e] = v[e];
+					} else if( MEAN ) {
+						col[e] += v[e];
+					} else if( v[e] > col[e] ) {
+						col[e] = v[e];
+					}
+				}
+			}
+#pragma unroll
+			for( int e = 0; e < VECW; ++e ) {
+				if( kw == 0 ) {
+					acc[e] = col[e];
+				} else if( MEAN ) {
+					acc[e] += col[e];
+				} else if( col[e] > acc[e] ) {
+					acc[e] = col[e];
+				}
+			}
+		}
+		float* out = result + item * VECW;
+		if constexpr( VECW == 4 ) {
+			float4 q;
+			q.x = MEAN ? acc[0] * scale : acc[0];
+			q.y = MEAN ? acc[1] * scale : acc[1];
+			q.z = MEAN ? acc[2] * scale : acc[2];
+			q.w = MEAN ? acc[3] * scale : acc[3];
+			*reinterpret_cast<float4*>( out ) = q;
+		} else {
+			*out = MEAN ? acc[0] * scale : acc[0];
+		}
+	}
+}
+
+// Max pooling with the index output used by the backward pass. The index reproduces the reference CPU engine
+// (src/CPU/CpuMathEngineDnnPooling.cpp:40-84) exactly:
+//   - column maxima over the window rows keep the topmost row on ties (strict >);
+//   - the window maximum over those column maxima keeps the leftmost column on ties (strict >);
+//   - the row stored for the winning column is looked up in the row-index buffer at the column's position
+//     RELATIVE to the window ( columnIndex * channels + c ), i.e. it is the arg-max row of image column
+//     `columnIndex` of the same strip, not of column `wo * stride + columnIndex`.
+__global__ __launch_bounds__( 256 )
+void maxPoolingIndexKernel( const nhPoolingDesc d, const float* source, int* maxIndices, float* result, long long total )
+{
+	const long long step = static_cast<long long>( gridDim.x ) * 256;
+	const int rowSize = d.width * d.channels;
+	for( long long item = blockIdx.x * 256LL + threadIdx.x; item < total; item += step ) {
+		long long t = item;
+		const int c = static_cast<int>( t % d.channels ); t /= d.channels;
+		const int wo = static_cast<int>( t % d.resultWidth ); t /= d.resultWidth;
+		const int ho = static_cast<int>( t % d.resultHeight ); t /= d.resultHeight;
+		const long long n = t;
+		const int stripRow = ho * d.strideHeight;
+		const float* strip = source + ( n * d.height + stripRow ) * rowSize;
+		const int windowColumn = wo * d.strideWidth * d.channels;
+		float best = 0.f;
+		int bestCol = 0;
+		for( int kw = 0; kw < d.filterWidth; ++kw ) {
+			const float* p = strip + windowColumn + kw * d.channels + c;
+			float col = *p;
+			for( int kh = 1; kh < d.filterHeight; ++kh ) {
+				const float v = p[static_cast<long long>( kh ) * rowSize];
+				if( v > col ) {
+					col = v;
+				}
+			}
+			if( kw == 0 || col > best ) {
+				best = col;
+				bestCol = kw;
+			}
+		}
+		const int windowIndex = bestCol * d.channels + c;
+		const float* q = strip + windowIndex;
+		float rowBest = *q;
+		int rowIdx = 0;
+		for( int kh = 1; kh < d.filterHeight; ++kh ) {
+			const float v = q[static_cast<long long>( kh ) * rowSize];
+			if( v > rowBest ) {
+				rowBest = v;
+				rowIdx = kh;
+			}
+		}
+		result[item] = best;
+		maxIndices[item] = ( stripRow + rowIdx ) * rowSize + windowColumn + windowIndex;
+	}
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// BlobResizeImage: pad (constant / edge / reflect) or crop the H and W dimensions
+
+__device__ __forceinline__ int resizeInputCoord( int x, int size, int padding )
+{
+	if( x >= 0 && x < size ) {
+		return x;
+	}
+	if( padding == NH_PAD_CONSTANT ) {
+		return -1;
+	}
+	if( padding == NH_PAD_EDGE ) {
+		return x < 0 ? 0 : size - 1;
+	}
+	// reflect, with the reference's arithmetic (src/CPU/Rowwise/CpuRowwiseResizeImage.h:177-195)
+	return x < 0 ? -( x % size ) : ( 2 * size - 2 - ( x % size ) ) % size;
+}
+
+template<int VECW>
+__global__ __launch_bounds__( 256 )
+void resizeImageKernel( const float* from, float* to, int height, int width, int channels, int toHeight, int toWidth,
+	int deltaLeft, int deltaTop, int padding, float defaultValue, long long totalItems )
+{
+	const int cg = channels / VECW;
+	const long long step = static_cast<long long>( gridDim.x ) * 256;
+	for( long long item = blockIdx.x * 256LL + threadIdx.x; item < totalItems; item += step ) {
+		long long t = item;
+		const int c = static_cast<int>( t % cg ) * VECW; t /= cg;
+		const int x = static_cast<int>( t % toWidth ); t /= toWidth;
+		const int y = static_cast<int>( t % toHeight ); t /= toHeight;
+		const long long n = t;
+		const int sy = resizeInputCoord( y - deltaTop, height, padding );
+		const int sx = resizeInputCoord( x - deltaLeft, width, padding );
+		const bool inside = sy >= 0 && sy < height && sx >= 0 && sx < width;
+		const float* p = from + ( ( n * height + sy ) * width + sx ) * channels + c;
+		if( VECW == 4 ) {
+			float4 v = make_float4( defaultValue, defaultValue, defaultValue, defaultValue );
+			if( inside ) {
+				v = *reinterpret_cast<const float4*>( p );
+			}
+			*reinterpret_cast<float4*>( to + item * 4 ) = v;
+		} else {
+			to[item] = inside ? *p : defaultValue;
+		}
+	}
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Split / merge along a blob dimension: the big blob is [objectCount][objectSize]; part i owns the columns
+// [Offset[i], Offset[i+1]) of every row and is itself dense [objectCount][size_i].
+
+struct CSplitParts {
+	float* Data[NH_MAX_BLOB_DESCS];
+	int Offset[NH_MAX_BLOB_DESCS + 1];
+	int Count;
+};
+
+template<int VECW, bool MERGE>
+__global__ __launch_bounds__( 256 )
+void splitMergeKernel( float* big, const CSplitParts parts, int objectSize, long long totalItems )
+{
+	const int rowItems = objectSize / VECW;
+	const long long step = static_cast<long long>( gridDim.x ) * 256;
+	for( long long item = blockIdx.x * 256LL + threadIdx.x; item < totalItems; item += step ) {
+		const long long x = item / rowItems;
+		const int pos = static_cast<int>( item - x * rowItems ) * VECW;
+		int part = 0;
+		while( part + 1 < parts.Count && pos >= parts.Offset[part + 1] ) {
+			++part;
+		}
+		const int size = parts.Offset[part + 1] - parts.Offset[part];
+		float* small = parts.Data[part] + x * size + ( pos - parts.Offset[part] );
+		float* large = big + x * objectSize + pos;
+		if( VECW == 4 ) {
+			if( MERGE ) {
+				*reinterpret_cast<float4*>( large ) = *reinterpret_cast<const float4*>( small );
+			} else {
+				*reinterpret_cast<float4*>( small ) = *reinterpret_cast<const float4*>( large );
+			}
+		} else {
+			if( MERGE ) {
+				*large = *small;
+			} else {
+				*small = *large;
+			}
+		}
+	}
+}
+
+static long long dimProduct( const nhBlobDesc& d, int from, int to )
+{
+	long long p = 1;
+	for( int i = from; i < to; ++i ) {
+		p *= d.dims[i];
+	}
+	return p;
+}
+
+template<bool MERGE>
+static int splitMergeImpl( nhStream s, int dim, const nhBlobDesc& bigDesc, float* big, const nhBlobDesc* partDescs,
+	float* const* partData, int count )
+{
+	if( dim < 0 || dim >= 7 || count < 1 || count > NH_MAX_BLOB_DESCS ) {
+		setLastError( "BlobSplitByDim/BlobMergeByDim: bad dimension or part count" );
+		return NH_ERR_ARGUMENT;
+	}
+	const long long objectCount = dimProduct( bigDesc, 0, dim );
+	const long long blobSize = dimProduct( bigDesc, 0, 7 );
+	CSplitParts parts;
+	parts.Count = count;
+	parts.Offset[0] = 0;
+	bool vec = isAligned16( big );
+	long long objectSize = 0;
+	if( dim == 0 ) {
+		// concatenation of whole blobs: one row, part sizes are the blob sizes
+		for( int i = 0; i < count; ++i ) {
+			objectSize += dimProduct( partDescs[i], 0, 7 );
+			if( objectSize > 0x7fffffffLL ) {
+				setLastError( "BlobSplitByDim/BlobMergeByDim: blob is too large" );
+				return NH_ERR_ARGUMENT;
+			}
+			parts.Offset[i + 1] = static_cast<int>( objectSize );
+		}
+	} else {
+		for( int i = 0; i < count; ++i ) {
+			objectSize += dimProduct( partDescs[i], dim, 7 );
+			if( objectSize > 0x7fffffffLL ) {
+				setLastError( "BlobSplitByDim/BlobMergeByDim: blob is too large" );
+				return NH_ERR_ARGUMENT;
+			}
+			parts.Offset[i + 1] = static_cast<int>( objectSize );
+		}
+	}
+	const long long rows = dim == 0 ? 1 : objectCount;
+	if( rows * objectSize != blobSize ) {
+		setLastError( "BlobSplitByDim/BlobMergeByDim: part sizes do not add up to the blob" );
+		return NH_ERR_ARGUMENT;
+	}
+	if( blobSize == 0 ) {
+		return NH_OK;
+	}
+	for( int i = 0; i < count; ++i ) {
+		parts.Data[i] = partData[i];
+		if( parts.Offset[i + 1] > parts.Offset[i] && partData[i] == nullptr ) {
+			setLastError( "BlobSplitByDim/BlobMergeByDim: null part pointer" );
+			return NH_ERR_ARGUMENT;
+		}
+		vec = vec && isAligned16( partData[i] ) && parts.Offset[i + 1] % 4 == 0;
+	}
+	const long long items = vec ? blobSize / 4 : blobSize;
+	long long blocks = ( items + 255 ) / 256;
+	blocks = blocks > 262144 ? 262144 : blocks;
+	if( vec ) {
+		hipLaunchKernelGGL( ( splitMergeKernel<4, MERGE> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			big, parts, static_cast<int>( objectSize ), items );
+	} else {
+		hipLaunchKernelGGL( ( splitMergeKernel<1, MERGE> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			big, parts, static_cast<int>( objectSize ), items );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// LSTM gate kernel: gates [B x 4H] = main | forget | input | output (pre-activation, free term included)
+//   c = sigmoid( f ) * cPrev + sigmoid( i ) * tanh( a );  h = sigmoid( o ) * tanh( c )
+// (src/CPU/CpuMathEngineDnnLstm.h:49-90)
+
+__device__ __forceinline__ float lstmExp( float x )
+{
+	if( x < -87.33654474f ) return 0.f;
+	if( x > 88.f ) return FLT_MAX;
+	return expf( x );
+}
+__device__ __forceinline__ float lstmSigmoid( float x )
+{
+	const float e = lstmExp( x );
+	return e / ( e + 1.f );
+}
+
+__global__ __launch_bounds__( 256 )
+void lstmGatesKernel( const float* gates, const float* statePrev, float* stateOut, float* mainOut, int hidden, int total )
+{
+	const int i = blockIdx.x * 256 + threadIdx.x;
+	if( i >= total ) {
+		return;
+	}
+	const int b = i / hidden;
+	const int j = i - b * hidden;
+	const float* g = gates + static_cast<long long>( b ) * 4 * hidden + j;
+	const float a = tanhf( g[0] );
+	const float f = lstmSigmoid( g[hidden] );
+	const float in = lstmSigmoid( g[2 * hidden] );
+	const float o = lstmSigmoid( g[3 * hidden] );
+	const float cPrev = statePrev != nullptr ? statePrev[i] : 0.f;
+	const float c = f * cPrev + in * a;
+	stateOut[i] = c;
+	mainOut[i] = o * tanhf( c );
+}
+
+__global__ void addTwoVectorsKernel( const float* a, const float* b, float* out, int n )
+{
+	const int i = blockIdx.x * 256 + threadIdx.x;
+	if( i < n ) {
+		out[i] = ( a != nullptr ? a[i] : 0.f ) + ( b != nullptr ? b[i] : 0.f );
+	}
+}
+
+} // namespace nh
+
+using namespace nh;
+
+extern "C" int nhInitPooling( nhPoolingDesc* d );
+
+static int checkPoolingDesc( const nhPoolingDesc* d )
+{
+	NH_REQUIRE( d != nullptr );
+	nhPoolingDesc check = *d;
+	const int rc = nhInitPooling( &check );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( check.resultHeight == d->resultHeight && check.resultWidth == d->resultWidth );
+	NH_REQUIRE( static_cast<long long>( d->height ) * d->width * d->channels <= 0x7fffffffLL );
+	return NH_OK;
+}
+
+template<bool MEAN>
+static int poolingImpl( nhStream s, const nhPoolingDesc* d, const float* source, float* result )
+{
+	const bool vec = d->channels % 4 == 0 && isAligned16( source ) && isAligned16( result );
+	const long long items = static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * ( vec ? d->channels / 4 : d->channels );
+	if( items == 0 ) {
+		return NH_OK;
+	}
+	long long blocks = ( items + 255 ) / 256;
+	blocks = blocks > 1048576 ? 1048576 : blocks;
+	if( vec ) {
+		hipLaunchKernelGGL( ( poolingKernel<4, MEAN> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			*d, source, result, items );
+	} else {
+		hipLaunchKernelGGL( ( poolingKernel<1, MEAN> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			*d, source, result, items );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+extern "C" {
+
+
+int nhInitBlobChannelwiseConvolution( nhConvDesc* d )
+{
+	NH_REQUIRE( d != nullptr );
+	NH_REQUIRE( d->batch >= 0 && d->height > 0 && d->width > 0 && d->channels > 0 );
+	NH_REQUIRE( d->filterHeight > 0 && d->filterWidth > 0 && d->strideHeight > 0 && d->strideWidth > 0 );
+	NH_REQUIRE( d->paddingHeight >= 0 && d->paddingWidth >= 0 );
+	NH_REQUIRE( d->paddingHeight < d->filterHeight && d->paddingWidth < d->filterWidth );
+	NH_REQUIRE( d->height + 2 * d->paddingHeight >= d->filterHeight && d->width + 2 * d->paddingWidth >= d->filterWidth );
+	d->filterCount = d->channels;
+	d->dilationHeight = 1;
+	d->dilationWidth = 1;
+	d->resultHeight = ( d->height + 2 * d->paddingHeight - d->filterHeight ) / d->strideHeight + 1;
+	d->resultWidth = ( d->width + 2 * d->paddingWidth - d->filterWidth ) / d->strideWidth + 1;
+	return NH_OK;
+}
+
+int nhBlobChannelwiseConvolution( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
+	const float* freeTerm, float* result )
+{
+	NH_REQUIRE( d != nullptr && source != nullptr && filter != nullptr && result != nullptr );
+	nhConvDesc check = *d;
+	const int rc = nhInitBlobChannelwiseConvolution( &check );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( check.resultHeight == d->resultHeight && check.resultWidth == d->resultWidth );
+	if( d->batch == 0 ) {
+		return NH_OK;
+	}
+	const bool vec = d->channels % 4 == 0 && isAligned16( source ) && isAligned16( filter ) && isAligned16( result )
+		&& ( freeTerm == nullptr || isAligned16( freeTerm ) );
+	constexpr int WPT = 4;
+	const int wGroups = ceilDiv( d->resultWidth, WPT );
+	const long long items = static_cast<long long>( d->batch ) * d->resultHeight * wGroups * ( vec ? d->channels / 4 : d->channels );
+	long long blocks = ( items + 255 ) / 256;
+	blocks = blocks > 1048576 ? 1048576 : blocks;
+	if( vec ) {
+		hipLaunchKernelGGL( ( channelwiseConvKernel<4, WPT> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			*d, source, filter, freeTerm, result, wGroups, items );
+	} else {
+		hipLaunchKernelGGL( ( channelwiseConvKernel<1, WPT> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			*d, source, filter, freeTerm, result, wGroups, items );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+int nhInitPooling( nhPoolingDesc* d )
+{
+	NH_REQUIRE( d != nullptr );
+	NH_REQUIRE( d->batch >= 0 && d->height > 0 && d->width > 0 && d->channels > 0 );
+	NH_REQUIRE( d->filterHeight > 0 && d->filterWidth > 0 && d->strideHeight > 0 && d->strideWidth > 0 );
+	NH_REQUIRE( d->filterHeight <= d->height && d->filterWidth <= d->width );
+	d->resultHeight = ( d->height - d->filterHeight ) / d->strideHeight + 1;
+	d->resultWidth = ( d->width - d->filterWidth ) / d->strideWidth + 1;
+	return NH_OK;
+}
+
+int nhBlobMaxPooling( nhStream s, const nhPoolingDesc* d, const float* source, int* maxIndices, float* result )
+{
+	const int rc = checkPoolingDesc( d );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( source != nullptr && result != nullptr );
+	if( maxIndices == nullptr ) {
+		return poolingImpl<false>( s, d, source, result );
+	}
+	const long long total = static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * d->channels;
+	if( total == 0 ) {
+		return NH_OK;
+	}
+	long long blocks = ( total + 255 ) / 256;
+	blocks = blocks > 1048576 ? 1048576 : blocks;
+	hipLaunchKernelGGL( maxPoolingIndexKernel, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+		*d, source, maxIndices, result, total );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+int nhBlobMeanPooling( nhStream s, const nhPoolingDesc* d, const float* source, float* result )
+{
+	const int rc = checkPoolingDesc( d );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( source != nullptr && result != nullptr );
+	return poolingImpl<true>( s, d, source, result );
+}
+
+int nhBlobResizeImage( nhStream s, const nhBlobDesc* from, const float* fromData, int deltaLeft, int deltaRight,
+	int deltaTop, int deltaBottom, int padding, float defaultValue, const nhBlobDesc* to, float* toData )
+{
+	NH_REQUIRE( from != nullptr && to != nullptr && fromData != nullptr && toData != nullptr );
+	NH_REQUIRE( padding == NH_PAD_CONSTANT || padding == NH_PAD_EDGE || padding == NH_PAD_REFLECT );
+	const int height = from->dims[3], width = from->dims[4];
+	const int channels = from->dims[5] * from->dims[6];
+	const long long batch = dimProduct( *from, 0, 3 );
+	const int toHeight = height + deltaTop + deltaBottom;
+	const int toWidth = width + deltaLeft + deltaRight;
+	NH_REQUIRE( height > 0 && width > 0 && channels > 0 && toHeight > 0 && toWidth > 0 );
+	NH_REQUIRE( to->dims[3] == toHeight && to->dims[4] == toWidth && to->dims[5] * to->dims[6] == channels );
+	NH_REQUIRE( dimProduct( *to, 0, 3 ) == batch );
+	if( batch == 0 ) {
+		return NH_OK;
+	}
+	const bool vec = channels % 4 == 0 && isAligned16( fromData ) && isAligned16( toData );
+	const long long items = batch * toHeight * toWidth * ( vec ? channels / 4 : channels );
+	long long blocks = ( items + 255 ) / 256;
+	blocks = blocks > 1048576 ? 1048576 : blocks;
+	if( vec ) {
+		hipLaunchKernelGGL( resizeImageKernel<4>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			fromData, toData, height, width, channels, toHeight, toWidth, deltaLeft, deltaTop, padding, defaultValue, items );
+	} else {
+		hipLaunchKernelGGL( resizeImageKernel<1>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			fromData, toData, height, width, channels, toHeight, toWidth, deltaLeft, deltaTop, padding, defaultValue, items );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+int nhBlobMergeByDim( nhStream s, int dim, const nhBlobDesc* from, const float* const* fromData, int fromCount,
+	const nhBlobDesc* to, float* toData )
+{
+	NH_REQUIRE( from != nullptr && fromData != nullptr && to != nullptr && toData != nullptr );
+	return splitMergeImpl<true>( s, dim, *to, toData, from, const_cast<float* const*>( fromData ), fromCount );
+}
+
+int nhBlobSplitByDim( nhStream s, int dim, const nhBlobDesc* from, const float* fromData,
+	const nhBlobDesc* to, float* const* toData, int toCount )
+{
+	NH_REQUIRE( from != nullptr && fromData != nullptr && to != nullptr && toData != nullptr );
+	return splitMergeImpl<false>( s, dim, *from, const_cast<float*>( fromData ), to, toData, toCount );
+}
+
+// workspace layout: [ gates: T*B*4H ][ free term: 4H ][ state: B*H ]
+int nhLstmWorkspaceSize( int hiddenSize, int objectSize, int sequenceLength, int sequenceCount, size_t* bytes )
+{
+	NH_REQUIRE( bytes != nullptr && hiddenSize > 0 && objectSize > 0 && sequenceLength >= 0 && sequenceCount >= 0 );
+	const size_t gates = static_cast<size_t>( sequenceLength ) * sequenceCount * 4 * hiddenSize;
+	*bytes = ( gates + 4 * static_cast<size_t>( hiddenSize ) + static_cast<size_t>( sequenceCount ) * hiddenSize ) * sizeof( float );
+	return NH_OK;
+}
+
+int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeights, const float* inputFreeTerm,
+	const float* recurrentWeights, const float* recurrentFreeTerm, int reverse, int sequenceLength,
+	int sequenceCount, const float* inputStateBackLink, const float* inputMainBackLink, const float* input,
+	float* outputStateBackLink, float* outputMainBackLink, void* workspace, size_t workspaceSize )
+{
+	size_t need = 0;
+	const int rc0 = nhLstmWorkspaceSize( hiddenSize, objectSize, sequenceLength, sequenceCount, &need );
+	if( rc0 != NH_OK ) {
+		return rc0;
+	}
+	NH_REQUIRE( inputWeights != nullptr && recurrentWeights != nullptr && input != nullptr && outputMainBackLink != nullptr );
+	NH_REQUIRE( workspace != nullptr && workspaceSize >= need && isAligned16( workspace ) );
+	if( sequenceLength == 0 || sequenceCount == 0 ) {
+		return NH_OK;
+	}
+	NH_REQUIRE( static_cast<long long>( sequenceLength ) * sequenceCount * 4 * hiddenSize <= 0x7fffffffLL );
+	hipStream_t stream = toStream( s );
+	const int H = hiddenSize;
+	const int B = sequenceCount;
+	const int T = sequenceLength;
+	float* gates = static_cast<float*>( workspace );
+	float* freeTerm = gates + static_cast<size_t>( T ) * B * 4 * H;
+	float* stateScratch = freeTerm + 4 * H;
+
+	const float* bias = nullptr;
+	if( inputFreeTerm != nullptr || recurrentFreeTerm != nullptr ) {
+		hipLaunchKernelGGL( addTwoVectorsKernel, dim3( ceilDiv( 4 * H, 256 ) ), dim3( 256 ), 0, stream,
+			inputFreeTerm, recurrentFreeTerm, freeTerm, 4 * H );
+		NH_LAUNCH_CHECK();
+		bias = freeTerm;
+	}
+	// every step's input contribution in one product: gates[T*B x 4H] = x[T*B x In] * Win^T + free term
+	int rc = matMulNT( stream, input, objectSize, inputWeights, objectSize, gates, 4 * H, T * B, 4 * H, objectSize,
+		1, 0, 0, 0, bias, false );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	const int stepSize = B * H;
+	for( int i = 0; i < T; ++i ) {
+		const int pos = reverse ? T - 1 - i : i;
+		const int prev = reverse ? pos + 1 : pos - 1;
+		const float* hPrev = i == 0 ? inputMainBackLink : outputMainBackLink + static_cast<size_t>( prev ) * stepSize;
+		const float* cPrev;
+		float* cOut;
+		if( outputStateBackLink != nullptr ) {
+			cPrev = i == 0 ? inputStateBackLink : outputStateBackLink + static_cast<size_t>( prev ) * stepSize;
+			cOut = outputStateBackLink + static_cast<size_t>( pos ) * stepSize;
+		} else {
+			cPrev = i == 0 ? inputStateBackLink : stateScratch;
+			cOut = stateScratch;
+		}
+		float* g = gates + static_cast<size_t>( pos ) * B * 4 * H;
+		if( hPrev != nullptr ) {
+			rc = matMulNT( stream, hPrev, H, recurrentWeights, H, g, 4 * H, B, 4 * H, H, 1, 0, 0, 0, nullptr, true );
+			if( rc != NH_OK ) {
+				return rc;
+			}
+		}
+		hipLaunchKernelGGL( lstmGatesKernel, dim3( ceilDiv( stepSize, 256 ) ), dim3( 256 ), 0, stream,
+			g, cPrev, cOut, outputMainBackLink + static_cast<size_t>( pos ) * stepSize, H, stepSize );
+		NH_LAUNCH_CHECK();
+	}
+	return NH_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,623 @@
+// fp32 matrix products and channels-last convolution on the CDNA4 matrix cores.
+//
+// One kernel template serves every dense contraction of the engine:
+//   C[M x N] (+)= A * B (+ bias[n])
+// with A given K-major (row-major M x K), M-major (a K x M matrix read transposed) or implicitly as the
+// im2col view of an N,H,W,C image (K = fh*fw*Cin gathered on the fly, zero padding), and B given K-major
+// (N x K, i.e. "multiply by transposed matrix" / the filter blob [Cout][fh][fw][Cin]) or N-major (K x N).
+//
+// Tiling: 256 threads = 4 wavefronts per workgroup; workgroup tile BM x BN, K step 16; each wavefront owns
+// a (BM/WAVES_M) x (BN/WAVES_N) sub-tile built from 32x32 blocks of v_mfma_f32_32x32x2_f32 (16 accumulator
+// registers per block). Tiles of A and B are staged through LDS with two buffers and one barrier per K step;
+// the global loads of step k+1 are in flight while step k is multiplied.
+//
+// LDS layout for a K-major operand is [row][16 + 4 pad]; lane (row = lane % 32, half = lane / 32) fetches the
+// four consecutive k values  k0 + 4*half .. +3  with a single 128-bit LDS read and feeds them to four MFMAs.
+// MFMA j of a group therefore reduces over k = {k0 + j, k0 + 4 + j}; both operands use the same permutation of
+// k, which is all the dot product needs.
+#include "common.h"
+
+namespace nh {
+
+typedef float f32x16 __attribute__( ( ext_vector_type( 16 ) ) );
+
+enum TAMode { AM_RowsK = 0, AM_RowsM = 1, AM_Conv = 2 };
+enum TBMode { BM_RowsK = 0, BM_RowsN = 1 };
+
+struct CMatMulArgs {
+	const float* A;
+	const float* B;
+	float* C;
+	const float* Bias; // per column n, may be null
+	int M, N, K;
+	int Lda, Ldb, Ldc;
+	long long BatchStrideA, BatchStrideB, BatchStrideC;
+	int Accumulate; // C += instead of C =
+	int TilesM, TilesN;
+	// convolution geometry (AM_Conv only): A is the image, M = batch * Ho * Wo
+	int H, W, Cin, Ho, Wo, Fw, PadH, PadW, StrideH, StrideW, DilH, DilW;
+};
+
+constexpr int KStep = 16;
+constexpr int LdsK = KStep + 4; // row pitch of a K-major tile in LDS (floats)
+constexpr int Threads = 256;
+
+template<int BX> struct CTileLds {
+	static constexpr int KMajorSize = BX * LdsK;
+	static constexpr int XMajorPitch = BX + 4;
+	static constexpr int XMajorSize = KStep * XMajorPitch;
+};
+
+// Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous range of tiles so that
+// neighbouring tiles (which share rows of A and the halo of the image) meet in the same L2.
+__device__ __forceinline__ int xcdSwizzle( int bid, int total )
+{
+	const int xcd = bid & 7;
+	const int idx = bid >> 3;
+	const int per = total >> 3;
+	const int rem = total & 7;
+	return xcd * per + ( xcd < rem ? xcd : rem ) + idx;
+}
+
+template<int BM, int BN, int WAVES_M, int WAVES_N, int AMODE, int BMODE, bool VEC>
+__global__ __launch_bounds__( Threads, 2 )
+void matMulKernel( const CMatMulArgs args )
+{
+	static_assert( WAVES_M * WAVES_N == 4, "4 wavefronts per workgroup" );
+	constexpr int WM = BM / WAVES_M;
+	constexpr int WN = BN / WAVES_N;
+	constexpr int MI = WM / 32;
+	constexpr int NI = WN / 32;
+	static_assert( MI >= 1 && NI >= 1, "wave tile is at least one 32x32 block" );
+	constexpr bool AK = ( AMODE != AM_RowsM ); // A tile kept K-major in LDS
+	constexpr bool BK = ( BMODE == BM_RowsK );
+	constexpr int ASize = AK ? CTileLds<BM>::KMajorSize : CTileLds<BM>::XMajorSize;
+	constexpr int BSize = BK ? CTileLds<BN>::KMajorSize : CTileLds<BN>::XMajorSize;
+	constexpr int ASlots = ( BM * 4 + Threads - 1 ) / Threads; // float4 slots per thread per K step
+	constexpr int BSlots = ( BN * 4 + Threads - 1 ) / Threads;
+
+	__shared__ __attribute__( ( aligned( 16 ) ) ) float ldsA[2][ASize];
+	__shared__ __attribute__( ( aligned( 16 ) ) ) float ldsB[2][BSize];
+
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = tid >> 6;
+	const int waveM = wave / WAVES_N;
+	const int waveN = wave % WAVES_N;
+	const int l32 = lane & 31;
+	const int half = lane >> 5;
+
+	const int tile = xcdSwizzle( blockIdx.x, gridDim.x );
+	const int tileM = tile / args.TilesN;
+	const int tileN = tile % args.TilesN;
+	const int m0 = tileM * BM;
+	const int n0 = tileN * BN;
+	const int batch = blockIdx.y;
+
+	const float* __restrict__ A = args.A + batch * args.BatchStrideA;
+	const float* __restrict__ B = args.B + batch * args.BatchStrideB;
+	float* C = args.C + batch * args.BatchStrideC;
+	const int M = args.M, N = args.N, K = args.K;
+
+	// ---- per-thread load slots -------------------------------------------------------------------------
+	// K-major tile: slot -> ( row = slot / 4, kq = slot % 4 ); X-major tile: slot -> ( k = slot / (BX/4), xq ).
+	// Convolution: every slot row is one output pixel; its top-left input coordinate is fixed for the kernel.
+	int convBase[ASlots];
+	int convH0[ASlots];
+	int convW0[ASlots];
+	int convCi = 0, convKh = 0, convKw = 0; // tap state of this thread's k (VEC path, advanced every K step)
+	if( AMODE == AM_Conv ) {
+#pragma unroll
+		for( int i = 0; i < ASlots; ++i ) {
+			const int slot = tid + i * Threads;
+			const int m = m0 + ( slot >> 2 );
+			if( m < M && ( BM * 4 % Threads == 0 || slot < BM * 4 ) ) {
+				const int wo = m % args.Wo;
+				const int t = m / args.Wo;
+				const int ho = t % args.Ho;
+				const int n = t / args.Ho;
+				convBase[i] = n * args.H * args.W * args.Cin;
+				convH0[i] = ho * args.StrideH - args.PadH;
+				convW0[i] = wo * args.StrideW - args.PadW;
+			} else {
+				convBase[i] = 0;
+				convH0[i] = -0x40000000; // always out of the image
+				convW0[i] = 0;
+			}
+		}
+		if( VEC ) {
+			const int k = ( tid & 3 ) * 4;
+			const int tap = k / args.Cin;
+			convCi = k - tap * args.Cin;
+			convKh = tap / args.Fw;
+			convKw = tap - convKh * args.Fw;
+		}
+	}
+
+	float4 regA[ASlots];
+	float4 regB[BSlots];
+
+	auto loadConvElement = [&]( int i, int k ) -> float {
+		if( k >= K ) {
+			return 0.f;
+		}
+		const int tap = k / args.Cin;
+		const int ci = k - tap * args.Cin;
+		const int kh = tap / args.Fw;
+		const int kw = tap - kh * args.Fw;
+		const int hi = convH0[i] + kh * args.DilH;
+		const int wi = convW0[i] + kw * args.DilW;
+		if( hi < 0 || hi >= args.H || wi < 0 || wi >= args.W ) {
+			return 0.f;
+		}
+		return A[convBase[i] + ( hi * args.W + wi ) * args.Cin + ci];
+	};
+
+	auto loadTiles = [&]( int kBase ) {
+		// ---- A ----
+#pragma unroll
+		for( int i = 0; i < ASlots; ++i ) {
+			const int slot = tid + i * Threads;
+			float4 v = make_float4( 0.f, 0.f, 0.f, 0.f );
+			if( BM * 4 % Threads == 0 || slot < BM * 4 ) {
+				if( AMODE == AM_RowsK ) {
+					const int m = m0 + ( slot >> 2 );
+					const int k = kBase + ( slot & 3 ) * 4;
+					if( m < M ) {
+						const float* p = A + static_cast<long long>( m ) * args.Lda + k;
+						if( VEC ) {
+							if( k < K ) {
+								v = *reinterpret_cast<const float4*>( p );
+							}
+						} else {
+							if( k < K ) v.x = p[0];
+							if( k + 1 < K ) v.y = p[1];
+							if( k + 2 < K ) v.z = p[2];
+							if( k + 3 < K ) v.w = p[3];
+						}
+					}
+				} else if( AMODE == AM_RowsM ) {
+					const int k = kBase + slot / ( BM / 4 );
+					const int m = m0 + ( slot % ( BM / 4 ) ) * 4;
+					if( k < K ) {
+						const float* p = A + static_cast<long long>( k ) * args.Lda + m;
+						if( VEC ) {
+							if( m < M ) {
+								v = *reinterpret_cast<const float4*>( p );
+							}
+						} else {
+							if( m < M ) v.x = p[0];
+							if( m + 1 < M ) v.y = p[1];
+							if( m + 2 < M ) v.z = p[2];
+							if( m + 3 < M ) v.w = p[3];
+						}
+					}
+				} else { // AM_Conv
+					if( VEC ) {
+						// Cin % 4 == 0: the four k of a slot share one filter tap
+						const int hi = convH0[i] + convKh * args.DilH;
+						const int wi = convW0[i] + convKw * args.DilW;
+						if( kBase + ( tid & 3 ) * 4 < K && hi >= 0 && hi < args.H && wi >= 0 && wi < args.W ) {
+							v = *reinterpret_cast<const float4*>(
+								A + convBase[i] + ( hi * args.W + wi ) * args.Cin + convCi );
+						}
+					} else {
+						const int k = kBase + ( slot & 3 ) * 4;
+						v.x = loadConvElement( i, k );
+						v.y = loadConvElement( i, k + 1 );
+						v.z = loadConvElement( i, k + 2 );
+						v.w = loadConvElement( i, k + 3 );
+					}
+				}
+			}
+			regA[i] = v;
+		}
+		if( AMODE == AM_Conv && VEC ) {
+			convCi += KStep;
+			while( convCi >= args.Cin ) {
+				convCi -= args.Cin;
+				if( ++convKw == args.Fw ) {
+					convKw = 0;
+					++convKh;
+				}
+			}
+		}
+		// ---- B ----
+#pragma unroll
+		for( int i = 0; i < BSlots; ++i ) {
+			const int slot = tid + i * Threads;
+			float4 v = make_float4( 0.f, 0.f, 0.f, 0.f );
+			if( BN * 4 % Threads == 0 || slot < BN * 4 ) {
+				if( BMODE == BM_RowsK ) {
+					const int n = n0 + ( slot >> 2 );
+					const int k = kBase + ( slot & 3 ) * 4;
+					if( n < N ) {
+						const float* p = B + static_cast<long long>( n ) * args.Ldb + k;
+						if( VEC ) {
+							if( k < K ) {
+								v = *reinterpret_cast<const float4*>( p );
+							}
+						} else {
+							if( k < K ) v.x = p[0];
+							if( k + 1 < K ) v.y = p[1];
+							if( k + 2 < K ) v.z = p[2];
+							if( k + 3 < K ) v.w = p[3];
+						}
+					}
+				} else {
+					const int k = kBase + slot / ( BN / 4 );
+					const int n = n0 + ( slot % ( BN / 4 ) ) * 4;
+					if( k < K ) {
+						const float* p = B + static_cast<long long>( k ) * args.Ldb + n;
+						if( VEC ) {
+							if( n < N ) {
+								v = *reinterpret_cast<const float4*>( p );
+							}
+						} else {
+							if( n < N ) v.x = p[0];
+							if( n + 1 < N ) v.y = p[1];
+							if( n + 2 < N ) v.z = p[2];
+							if( n + 3 < N ) v.w = p[3];
+						}
+					}
+				}
+			}
+			regB[i] = v;
+		}
+	};
+
+	auto storeTiles = [&]( int buf ) {
+#pragma unroll
+		for( int i = 0; i < ASlots; ++i ) {
+			const int slot = tid + i * Threads;
+			if( BM * 4 % Threads == 0 || slot < BM * 4 ) {
+				if( AK ) {
+					*reinterpret_cast<float4*>( &ldsA[buf][( slot >> 2 ) * LdsK + ( slot & 3 ) * 4] ) = regA[i];
+				} else {
+					*reinterpret_cast<float4*>( &ldsA[buf][( slot / ( BM / 4 ) ) * CTileLds<BM>::XMajorPitch
+						+ ( slot % ( BM / 4 ) ) * 4] ) = regA[i];
+				}
+			}
+		}
+#pragma unroll
+		for( int i = 0; i < BSlots; ++i ) {
+			const int slot = tid + i * Threads;
+			if( BN * 4 % Threads == 0 || slot < BN * 4 ) {
+				if( BK ) {
+					*reinterpret_cast<float4*>( &ldsB[buf][( slot >> 2 ) * LdsK + ( slot & 3 ) * 4] ) = regB[i];
+				} else {
+					*reinterpret_cast<float4*>( &ldsB[buf][( slot / ( BN / 4 ) ) * CTileLds<BN>::XMajorPitch
+						+ ( slot % ( BN / 4 ) ) * 4] ) = regB[i];
+				}
+			}
+		}
+	};
+
+	f32x16 acc[MI][NI];
+#pragma unroll
+	for( int mi = 0; mi < MI; ++mi ) {
+#pragma unroll
+		for( int ni = 0; ni < NI; ++ni ) {
+#pragma unroll
+			for( int r = 0; r < 16; ++r ) {
+				acc[mi][ni][r] = 0.f;
+			}
+		}
+	}
+
+	const int kSteps = ( K + KStep - 1 ) / KStep;
+	loadTiles( 0 );
+	storeTiles( 0 );
+	__syncthreads();
+
+	for( int ks = 0; ks < kSteps; ++ks ) {
+		const int cur = ks & 1;
+		if( ks + 1 < kSteps ) {
+			loadTiles( ( ks + 1 ) * KStep );
+		}
+		const float* tA = ldsA[cur];
+		const float* tB = ldsB[cur];
+#pragma unroll
+		for( int kc = 0; kc < 2; ++kc ) {
+			float fa[MI][4];
+			float fb[NI][4];
+#pragma unroll
+			for( int mi = 0; mi < MI; ++mi ) {
+				const int row = waveM * WM + mi * 32 + l32;
+				if( AK ) {
+					const float4 v = *reinterpret_cast<const float4*>( &tA[row * LdsK + kc * 8 + half * 4] );
+					fa[mi][0] = v.x; fa[mi][1] = v.y; fa[mi][2] = v.z; fa[mi][3] = v.w;
+				} else {
+#pragma unroll
+					for( int j = 0; j < 4; ++j ) {
+						fa[mi][j] = tA[( kc * 8 + half * 4 + j ) * CTileLds<BM>::XMajorPitch + row];
+					}
+				}
+			}
+#pragma unroll
+			for( int ni = 0; ni < NI; ++ni ) {
+				const int col = waveN * WN + ni * 32 + l32;
+				if( BK ) {
+					const float4 v = *reinterpret_cast<const float4*>( &tB[col * LdsK + kc * 8 + half * 4] );
+					fb[ni][0] = v.x; fb[ni][1] = v.y; fb[ni][2] = v.z; fb[ni][3] = v.w;
+				} else {
+#pragma unroll
+					for( int j = 0; j < 4; ++j ) {
+						fb[ni][j] = tB[( kc * 8 + half * 4 + j ) * CTileLds<BN>::XMajorPitch + col];
+					}
+				}
+			}
+#pragma unroll
+			for( int j = 0; j < 4; ++j ) {
+#pragma unroll
+				for( int mi = 0; mi < MI; ++mi ) {
+#pragma unroll
+					for( int ni = 0; ni < NI; ++ni ) {
+						acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32( fa[mi][j], fb[ni][j], acc[mi][ni], 0, 0, 0 );
+					}
+				}
+			}
+		}
+		if( ks + 1 < kSteps ) {
+			storeTiles( cur ^ 1 );
+		}
+		__syncthreads();
+	}
+
+	// ---- epilogue: accumulator register r of lane holds row 8*(r/4) + 4*half + r%4, column lane%32 ----------
+#pragma unroll
+	for( int ni = 0; ni < NI; ++ni ) {
+		const int n = n0 + waveN * WN + ni * 32 + l32;
+		if( n >= N ) {
+			continue;
+		}
+		const float bias = ( args.Bias != nullptr ) ? args.Bias[n] : 0.f;
+#pragma unroll
+		for( int mi = 0; mi < MI; ++mi ) {
+#pragma unroll
+			for( int r = 0; r < 16; ++r ) {
+				const int m = m0 + waveM * WM + mi * 32 + ( r >> 2 ) * 8 + half * 4 + ( r & 3 );
+				if( m < M ) {
+					float* p = C + static_cast<long long>( m ) * args.Ldc + n;
+					float v = acc[mi][ni][r] + bias;
+					if( args.Accumulate ) {
+						v += *p;
+					}
+					*p = v;
+				}
+			}
+		}
+	}
+}
+
+template<int BM, int BN, int WAVES_M, int WAVES_N, int AMODE, int BMODE>
+static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool vec )
+{
+	args.TilesM = ceilDiv( args.M, BM );
+	args.TilesN = ceilDiv( args.N, BN );
+	const long long tiles = static_cast<long long>( args.TilesM ) * args.TilesN;
+	if( tiles > 0x7fffffffLL ) {
+		setLastError( "matrix product: too many tiles" );
+		return NH_ERR_ARGUMENT;
+	}
+	// blockIdx.y is limited to 65535: walk larger batches in slices
+	for( int b0 = 0; b0 < batch; b0 += 65535 ) {
+		const int nb = batch - b0 < 65535 ? batch - b0 : 65535;
+		CMatMulArgs a = args;
+		a.A += b0 * args.BatchStrideA;
+		a.B += b0 * args.BatchStrideB;
+		a.C += b0 * args.BatchStrideC;
+		const dim3 grid( static_cast<unsigned>( tiles ), nb );
+		if( vec ) {
+			hipLaunchKernelGGL( ( matMulKernel<BM, BN, WAVES_M, WAVES_N, AMODE, BMODE, true> ), grid, dim3( Threads ), 0, stream, a );
+		} else {
+			hipLaunchKernelGGL( ( matMulKernel<BM, BN, WAVES_M, WAVES_N, AMODE, BMODE, false> ), grid, dim3( Threads ), 0, stream, a );
+		}
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+// Picks the workgroup tile: wide N tiles when there are enough columns, and the smaller M tile when the
+// large one would leave most of the 256 compute units without a workgroup.
+template<int AMODE, int BMODE>
+static int launchMatMul( hipStream_t stream, CMatMulArgs& args, int batch, bool vec )
+{
+	const int cus = 256;
+	const int N = args.N;
+	const long long M = args.M;
+	if( N > 64 ) {
+		const long long tiles128 = ( ( M + 127 ) / 128 ) * ( ( N + 127 ) / 128 ) * batch;
+		if( tiles128 >= 2 * cus ) {
+			return launchTile<128, 128, 2, 2, AMODE, BMODE>( stream, args, batch, vec );
+		}
+		const long long tiles64 = ( ( M + 127 ) / 128 ) * ( ( N + 63 ) / 64 ) * batch;
+		if( tiles64 >= 2 * cus ) {
+			return launchTile<128, 64, 2, 2, AMODE, BMODE>( stream, args, batch, vec );
+		}
+		return launchTile<64, 64, 2, 2, AMODE, BMODE>( stream, args, batch, vec );
+	}
+	if( N > 32 ) {
+		const long long tiles = ( ( M + 127 ) / 128 ) * batch;
+		if( tiles >= 2 * cus ) {
+			return launchTile<128, 64, 2, 2, AMODE, BMODE>( stream, args, batch, vec );
+		}
+		return launchTile<64, 64, 2, 2, AMODE, BMODE>( stream, args, batch, vec );
+	}
+	return launchTile<128, 32, 4, 1, AMODE, BMODE>( stream, args, batch, vec );
+}
+
+// C = A * B^T (+ bias) with row strides; also the inner product of the convolution with a 1x1 filter.
+int matMulNT( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
+	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC,
+	const float* bias, bool accumulate )
+{
+	if( M == 0 || N == 0 || batch == 0 ) {
+		return NH_OK;
+	}
+	CMatMulArgs args = {};
+	args.A = a; args.B = b; args.C = c; args.Bias = bias;
+	args.M = M; args.N = N; args.K = K;
+	args.Lda = lda; args.Ldb = ldb; args.Ldc = ldc;
+	args.BatchStrideA = strideA; args.BatchStrideB = strideB; args.BatchStrideC = strideC;
+	args.Accumulate = accumulate ? 1 : 0;
+	const bool vec = isAligned16( a ) && isAligned16( b ) && K % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0
+		&& strideA % 4 == 0 && strideB % 4 == 0;
+	return launchMatMul<AM_RowsK, BM_RowsK>( stream, args, batch, vec );
+}
+
+// C = A * B, A is M x K, B is K x N, all row-major.
+int matMulNN( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
+	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC, bool accumulate )
+{
+	if( M == 0 || N == 0 || batch == 0 ) {
+		return NH_OK;
+	}
+	CMatMulArgs args = {};
+	args.A = a; args.B = b; args.C = c; args.Bias = nullptr;
+	args.M = M; args.N = N; args.K = K;
+	args.Lda = lda; args.Ldb = ldb; args.Ldc = ldc;
+	args.BatchStrideA = strideA; args.BatchStrideB = strideB; args.BatchStrideC = strideC;
+	args.Accumulate = accumulate ? 1 : 0;
+	const bool vec = isAligned16( a ) && isAligned16( b ) && K % 4 == 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0
+		&& strideA % 4 == 0 && strideB % 4 == 0;
+	return launchMatMul<AM_RowsK, BM_RowsN>( stream, args, batch, vec );
+}
+
+// C (+)= A^T * B, A is K x M (stored), B is K x N, all row-major; the reduction runs over the stored rows.
+int matMulTN( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
+	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC, bool accumulate )
+{
+	if( M == 0 || N == 0 || batch == 0 ) {
+		return NH_OK;
+	}
+	CMatMulArgs args = {};
+	args.A = a; args.B = b; args.C = c; args.Bias = nullptr;
+	args.M = M; args.N = N; args.K = K;
+	args.Lda = lda; args.Ldb = ldb; args.Ldc = ldc;
+	args.BatchStrideA = strideA; args.BatchStrideB = strideB; args.BatchStrideC = strideC;
+	args.Accumulate = accumulate ? 1 : 0;
+	const bool vec = isAligned16( a ) && isAligned16( b ) && M % 4 == 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0
+		&& strideA % 4 == 0 && strideB % 4 == 0;
+	return launchMatMul<AM_RowsM, BM_RowsN>( stream, args, batch, vec );
+}
+
+int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* source, const float* filter,
+	const float* freeTerm, float* result )
+{
+	CMatMulArgs args = {};
+	args.A = source; args.B = filter; args.C = result; args.Bias = freeTerm;
+	const long long m = static_cast<long long>( d.batch ) * d.resultHeight * d.resultWidth;
+	args.M = static_cast<int>( m );
+	args.N = d.filterCount;
+	args.K = d.filterHeight * d.filterWidth * d.channels;
+	args.Lda = 0; args.Ldb = args.K; args.Ldc = d.filterCount;
+	args.H = d.height; args.W = d.width; args.Cin = d.channels;
+	args.Ho = d.resultHeight; args.Wo = d.resultWidth; args.Fw = d.filterWidth;
+	args.PadH = d.paddingHeight; args.PadW = d.paddingWidth;
+	args.StrideH = d.strideHeight; args.StrideW = d.strideWidth;
+	args.DilH = d.dilationHeight; args.DilW = d.dilationWidth;
+	if( args.M == 0 || args.N == 0 ) {
+		return NH_OK;
+	}
+	const bool vec = isAligned16( source ) && isAligned16( filter ) && d.channels % 4 == 0;
+	return launchMatMul<AM_Conv, BM_RowsK>( stream, args, 1, vec );
+}
+
+} // namespace nh
+
+// ---------------------------------------------------------------------------------------------------------
+// C ABI
+
+using namespace nh;
+
+extern "C" {
+
+int nhMultiplyMatrixByTransposedMatrix( nhStream s, const float* first, int firstHeight, int firstWidth,
+	int firstRowSize, const float* second, int secondHeight, int secondRowSize,
+	float* result, int resultRowSize, int resultBufferSize )
+{
+	NH_REQUIRE( firstHeight >= 0 && firstWidth >= 0 && secondHeight >= 0 );
+	NH_REQUIRE( firstRowSize >= firstWidth && secondRowSize >= firstWidth && resultRowSize >= secondHeight );
+	NH_REQUIRE( firstHeight == 0 || static_cast<long long>( firstHeight - 1 ) * resultRowSize + secondHeight <= resultBufferSize );
+	return matMulNT( toStream( s ), first, firstRowSize, second, secondRowSize, result, resultRowSize,
+		firstHeight, secondHeight, firstWidth, 1, 0, 0, 0, nullptr, false );
+}
+
+int nhBatchMultiplyMatrixByTransposedMatrix( nhStream s, int batchSize, const float* first, int firstHeight,
+	int firstWidth, const float* second, int secondHeight, float* result, int resultBufferSize )
+{
+	NH_REQUIRE( batchSize >= 0 && firstHeight >= 0 && firstWidth >= 0 && secondHeight >= 0 );
+	NH_REQUIRE( static_cast<long long>( batchSize ) * firstHeight * secondHeight <= resultBufferSize );
+	return matMulNT( toStream( s ), first, firstWidth, second, firstWidth, result, secondHeight,
+		firstHeight, secondHeight, firstWidth, batchSize,
+		static_cast<long long>( firstHeight ) * firstWidth, static_cast<long long>( secondHeight ) * firstWidth,
+		static_cast<long long>( firstHeight ) * secondHeight, nullptr, false );
+}
+
+int nhBatchMultiplyMatrixByMatrix( nhStream s, int batchSize, const float* first, int firstHeight,
+	int firstWidth, const float* second, int secondWidth, float* result, int resultBufferSize )
+{
+	NH_REQUIRE( batchSize >= 0 && firstHeight >= 0 && firstWidth >= 0 && secondWidth >= 0 );
+	NH_REQUIRE( static_cast<long long>( batchSize ) * firstHeight * secondWidth <= resultBufferSize );
+	return matMulNN( toStream( s ), first, firstWidth, second, secondWidth, result, secondWidth,
+		firstHeight, secondWidth, firstWidth, batchSize,
+		static_cast<long long>( firstHeight ) * firstWidth, static_cast<long long>( firstWidth ) * secondWidth,
+		static_cast<long long>( firstHeight ) * secondWidth, false );
+}
+
+int nhMultiplyTransposedMatrixByMatrixAndAdd( nhStream s, const float* first, int firstHeight, int firstWidth,
+	int firstRowSize, const float* second, int secondWidth, int secondRowSize,
+	float* result, int resultRowSize, int resultBufferSize )
+{
+	NH_REQUIRE( firstHeight >= 0 && firstWidth >= 0 && secondWidth >= 0 );
+	NH_REQUIRE( firstRowSize >= firstWidth && secondRowSize >= secondWidth && resultRowSize >= secondWidth );
+	NH_REQUIRE( firstWidth == 0 || static_cast<long long>( firstWidth - 1 ) * resultRowSize + secondWidth <= resultBufferSize );
+	return matMulTN( toStream( s ), first, firstRowSize, second, secondRowSize, result, resultRowSize,
+		firstWidth, secondWidth, firstHeight, 1, 0, 0, 0, true );
+}
+
+int nhBatchMultiplyTransposedMatrixByMatrix( nhStream s, int batchSize, const float* first, int firstHeight,
+	int firstWidth, const float* second, int secondWidth, float* result, int resultBufferSize )
+{
+	NH_REQUIRE( batchSize >= 0 && firstHeight >= 0 && firstWidth >= 0 && secondWidth >= 0 );
+	NH_REQUIRE( static_cast<long long>( batchSize ) * firstWidth * secondWidth <= resultBufferSize );
+	return matMulTN( toStream( s ), first, firstWidth, second, secondWidth, result, secondWidth,
+		firstWidth, secondWidth, firstHeight, batchSize,
+		static_cast<long long>( firstHeight ) * firstWidth, static_cast<long long>( firstHeight ) * secondWidth,
+		static_cast<long long>( firstWidth ) * secondWidth, false );
+}
+
+int nhInitBlobConvolution( nhConvDesc* d )
+{
+	NH_REQUIRE( d != nullptr );
+	NH_REQUIRE( d->batch >= 0 && d->height > 0 && d->width > 0 && d->channels > 0 );
+	NH_REQUIRE( d->filterCount > 0 && d->filterHeight > 0 && d->filterWidth > 0 );
+	NH_REQUIRE( d->paddingHeight >= 0 && d->paddingWidth >= 0 );
+	NH_REQUIRE( d->strideHeight > 0 && d->strideWidth > 0 && d->dilationHeight > 0 && d->dilationWidth > 0 );
+	const int spanH = ( d->filterHeight - 1 ) * d->dilationHeight + 1;
+	const int spanW = ( d->filterWidth - 1 ) * d->dilationWidth + 1;
+	NH_REQUIRE( d->height + 2 * d->paddingHeight >= spanH && d->width + 2 * d->paddingWidth >= spanW );
+	d->resultHeight = ( d->height + 2 * d->paddingHeight - spanH ) / d->strideHeight + 1;
+	d->resultWidth = ( d->width + 2 * d->paddingWidth - spanW ) / d->strideWidth + 1;
+	const long long m = static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth;
+	NH_REQUIRE( m <= 0x7fffffffLL );
+	NH_REQUIRE( static_cast<long long>( d->batch ) * d->height * d->width * d->channels <= 0x7fffffffLL );
+	NH_REQUIRE( m * d->filterCount <= 0x7fffffffLL );
+	return NH_OK;
+}
+
+int nhBlobConvolution( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
+	const float* freeTerm, float* result )
+{
+	NH_REQUIRE( d != nullptr && source != nullptr && filter != nullptr && result != nullptr );
+	nhConvDesc check = *d;
+	const int rc = nhInitBlobConvolution( &check );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( check.resultHeight == d->resultHeight && check.resultWidth == d->resultWidth );
+	return convImplicitGemm( toStream( s ), *d, source, filter, freeTerm, result );
+}
+
+} // extern "C"

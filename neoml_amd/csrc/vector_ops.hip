@@ -1,0 +1,464 @@
+// Element-wise vector kernels (IVectorMathEngine). All of them stream through HBM once: 128-bit loads and
+// stores, four independent 128-bit accesses per thread in flight, one workgroup per 4096 elements so that even a
+// mid-sized vector spreads over all 256 compute units. Pointers that are not 16-byte aligned (handles with an
+// element offset) take the scalar variant of the same kernel.
+//
+// Scalars that the engine keeps in device memory (thresholds, multipliers) are read inside the kernel.
+// Results may alias an input exactly (in-place layers): every element is read before it is written by the
+// same thread, so no __restrict__ is put on the pointers.
+#include "common.h"
+#include <float.h>
+
+namespace nh {
+
+constexpr int EltThreads = 256;
+constexpr int EltUnroll = 4;
+
+template<typename T> struct CVec4;
+template<> struct CVec4<float> { typedef float4 Type; };
+template<> struct CVec4<int> { typedef int4 Type; };
+
+template<int NIN, typename TIn, typename TOut, typename F, bool VEC>
+__global__ __launch_bounds__( EltThreads )
+void eltwiseKernel( const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, F f )
+{
+	f.prepare();
+	if( VEC ) {
+		typedef typename CVec4<TIn>::Type VIn;
+		typedef typename CVec4<TOut>::Type VOut;
+		const int n4 = n >> 2;
+		const int base = blockIdx.x * ( EltThreads * EltUnroll ) + threadIdx.x;
+		VIn va[EltUnroll], vb[EltUnroll], vc[EltUnroll];
+#pragma unroll
+		for( int u = 0; u < EltUnroll; ++u ) {
+			const int i = base + u * EltThreads;
+			if( i < n4 ) {
+				if( NIN >= 1 ) va[u] = reinterpret_cast<const VIn*>( a )[i];
+				if( NIN >= 2 ) vb[u] = reinterpret_cast<const VIn*>( b )[i];
+				if( NIN >= 3 ) vc[u] = reinterpret_cast<const VIn*>( c )[i];
+			}
+		}
+#pragma unroll
+		for( int u = 0; u < EltUnroll; ++u ) {
+			const int i = base + u * EltThreads;
+			if( i < n4 ) {
+				VOut r;
+				r.x = f( va[u].x, vb[u].x, vc[u].x );
+				r.y = f( va[u].y, vb[u].y, vc[u].y );
+				r.z = f( va[u].z, vb[u].z, vc[u].z );
+				r.w = f( va[u].w, vb[u].w, vc[u].w );
+				reinterpret_cast<VOut*>( out )[i] = r;
+			}
+		}
+		// tail of up to 3 elements
+		if( blockIdx.x == 0 && threadIdx.x < ( n & 3 ) ) {
+			const int i = ( n4 << 2 ) + threadIdx.x;
+			const TIn x = NIN >= 1 ? a[i] : TIn();
+			const TIn y = NIN >= 2 ? b[i] : TIn();
+			const TIn z = NIN >= 3 ? c[i] : TIn();
+			out[i] = f( x, y, z );
+		}
+	} else {
+		const int base = blockIdx.x * ( EltThreads * EltUnroll * 4 ) + threadIdx.x;
+#pragma unroll 4
+		for( int u = 0; u < EltUnroll * 4; ++u ) {
+			const int i = base + u * EltThreads;
+			if( i < n ) {
+				const TIn x = NIN >= 1 ? a[i] : TIn();
+				const TIn y = NIN >= 2 ? b[i] : TIn();
+				const TIn z = NIN >= 3 ? c[i] : TIn();
+				out[i] = f( x, y, z );
+			}
+		}
+	}
+}
+
+template<int NIN, typename TIn, typename TOut, typename F>
+static int launchEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, F f )
+{
+	if( n < 0 ) {
+		setLastError( "vector size is negative" );
+		return NH_ERR_ARGUMENT;
+	}
+	if( n == 0 ) {
+		return NH_OK;
+	}
+	if( out == nullptr || ( NIN >= 1 && a == nullptr ) || ( NIN >= 2 && b == nullptr ) || ( NIN >= 3 && c == nullptr ) ) {
+		setLastError( "null vector pointer" );
+		return NH_ERR_ARGUMENT;
+	}
+	const bool vec = isAligned16( out ) && ( NIN < 1 || isAligned16( a ) ) && ( NIN < 2 || isAligned16( b ) )
+		&& ( NIN < 3 || isAligned16( c ) ) && n >= 4;
+	const int perBlock = EltThreads * EltUnroll * 4;
+	const int blocks = ceilDiv( n, perBlock );
+	if( vec ) {
+		hipLaunchKernelGGL( ( eltwiseKernel<NIN, TIn, TOut, F, true> ), dim3( blocks ), dim3( EltThreads ), 0, toStream( s ),
+			a, b, c, out, n, f );
+	} else {
+		hipLaunchKernelGGL( ( eltwiseKernel<NIN, TIn, TOut, F, false> ), dim3( blocks ), dim3( EltThreads ), 0, toStream( s ),
+			a, b, c, out, n, f );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+// exp with the reference's clamps (src/CPU/x86/CpuX86.h:55: below -87.33654474 -> 0, above 88 -> FLT_MAX)
+__device__ __forceinline__ float expClamped( float x )
+{
+	if( x < -87.33654474f ) {
+		return 0.f;
+	}
+	if( x > 88.f ) {
+		return FLT_MAX;
+	}
+	return expf( x );
+}
+
+// ---- functors: operator()( a, b, c ) with unused operands ignored ---------------------------------------
+
+struct CNoScalar { __device__ void prepare() {} };
+
+template<typename T> struct CCopyOp : CNoScalar { __device__ T operator()( T a, T, T ) const { return a; } };
+template<typename T> struct CFillOp : CNoScalar { T Value; __device__ T operator()( T, T, T ) const { return Value; } };
+template<typename T> struct CFillFromOp {
+	const T* Ptr; T Value;
+	__device__ void prepare() { Value = *Ptr; }
+	__device__ T operator()( T, T, T ) const { return Value; }
+};
+struct CFloatToIntOp : CNoScalar { __device__ int operator()( float a, float, float ) const { return static_cast<int>( a ); } };
+struct CIntToFloatOp : CNoScalar { __device__ float operator()( int a, int, int ) const { return static_cast<float>( a ); } };
+
+struct CReLUOp {
+	const float* Ptr; float Threshold;
+	__device__ void prepare() { Threshold = *Ptr; }
+	// max( x, 0 ) written so that NaN becomes 0, as _mm_max_ps( x, 0 ) does
+	// (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:320-337)
+	__device__ float operator()( float a, float, float ) const
+	{
+		float r = a > 0.f ? a : 0.f;
+		if( Threshold > 0.f ) {
+			r = r < Threshold ? r : Threshold;
+		}
+		return r;
+	}
+};
+struct CELUOp {
+	const float* Ptr; float Alpha;
+	__device__ void prepare() { Alpha = *Ptr; }
+	__device__ float operator()( float a, float, float ) const { return a >= 0.f ? a : Alpha * ( expClamped( a ) - 1.f ); }
+};
+struct CLeakyReLUOp {
+	const float* Ptr; float Alpha;
+	__device__ void prepare() { Alpha = *Ptr; }
+	__device__ float operator()( float a, float, float ) const { return a > 0.f ? a : Alpha * a; }
+};
+struct CHSwishOp : CNoScalar {
+	__device__ float operator()( float a, float, float ) const
+	{
+		if( a <= -3.f ) return 0.f;
+		if( a >= 3.f ) return a;
+		return a * ( a + 3.f ) * ( 1.f / 6.f );
+	}
+};
+struct CMaxOp : CNoScalar { __device__ float operator()( float a, float b, float ) const { return a > b ? a : b; } };
+struct CMinOp : CNoScalar { __device__ float operator()( float a, float b, float ) const { return a < b ? a : b; } };
+struct CAbsOp : CNoScalar { __device__ float operator()( float a, float, float ) const { return fabsf( a ); } };
+struct CHardTanhOp : CNoScalar {
+	__device__ float operator()( float a, float, float ) const { return a < -1.f ? -1.f : ( a > 1.f ? 1.f : a ); }
+};
+struct CHardSigmoidOp {
+	const float* SlopePtr; const float* BiasPtr; float Slope, Bias;
+	__device__ void prepare() { Slope = *SlopePtr; Bias = *BiasPtr; }
+	__device__ float operator()( float a, float, float ) const
+	{
+		const float v = a * Slope + Bias;
+		return v < 0.f ? 0.f : ( v > 1.f ? 1.f : v );
+	}
+};
+struct CNegOp : CNoScalar { __device__ float operator()( float a, float, float ) const { return -a; } };
+struct CExpOp : CNoScalar { __device__ float operator()( float a, float, float ) const { return expClamped( a ); } };
+struct CLogOp : CNoScalar {
+	// log( clamp( x, FLT_MIN, FLT_MAX ) ) (src/CPU/x86/CpuX86MathEngineVectorMathMkl.cpp:55-77)
+	__device__ float operator()( float a, float, float ) const
+	{
+		float x = a > FLT_MIN ? a : FLT_MIN; // NaN -> FLT_MIN as std::max( x, FLT_MIN ) gives
+		x = x < FLT_MAX ? x : FLT_MAX;
+		return logf( x );
+	}
+};
+struct CErfOp : CNoScalar { __device__ float operator()( float a, float, float ) const { return erff( a ); } };
+template<typename T> struct CAddOp : CNoScalar { __device__ T operator()( T a, T b, T ) const { return a + b; } };
+template<typename T> struct CSubOp : CNoScalar { __device__ T operator()( T a, T b, T ) const { return a - b; } };
+template<typename T> struct CMulOp : CNoScalar { __device__ T operator()( T a, T b, T ) const { return a * b; } };
+struct CDivOp : CNoScalar { __device__ float operator()( float a, float b, float ) const { return a / b; } };
+struct CNegMulOp : CNoScalar { __device__ float operator()( float a, float b, float ) const { return -a * b; } };
+// result += first * second, two roundings like the reference's mul + add
+struct CMulAddOp : CNoScalar { __device__ float operator()( float a, float b, float c ) const { return __fadd_rn( c, __fmul_rn( a, b ) ); } };
+template<typename T> struct CAddValueOp {
+	const T* Ptr; T Value;
+	__device__ void prepare() { Value = *Ptr; }
+	__device__ T operator()( T a, T, T ) const { return a + Value; }
+};
+template<typename T> struct CMulValueOp {
+	const T* Ptr; T Value;
+	__device__ void prepare() { Value = *Ptr; }
+	__device__ T operator()( T a, T, T ) const { return a * Value; }
+};
+struct CNegMulValueOp {
+	const float* Ptr; float Value;
+	__device__ void prepare() { Value = *Ptr; }
+	__device__ float operator()( float a, float, float ) const { return -a * Value; }
+};
+// first + mult * second with separate rounding of the product
+// (src/CPU/x86/CpuX86MathEngineVectorMathMkl.cpp:79-121)
+struct CMultiplyAndAddOp {
+	const float* Ptr; float Mult;
+	__device__ void prepare() { Mult = *Ptr; }
+	__device__ float operator()( float a, float b, float ) const { return __fadd_rn( a, __fmul_rn( b, Mult ) ); }
+};
+struct CMultiplyAndSubOp {
+	const float* Ptr; float Mult;
+	__device__ void prepare() { Mult = *Ptr; }
+	__device__ float operator()( float a, float b, float ) const { return __fsub_rn( a, __fmul_rn( b, Mult ) ); }
+};
+struct CSqrtOp : CNoScalar { __device__ float operator()( float a, float, float ) const { return sqrtf( a ); } };
+struct CInvOp : CNoScalar {
+	// saturating reciprocal (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:1321-1366):
+	// -FLT_MIN <= x < 0 -> -FLT_MAX; 0 <= x <= FLT_MIN -> FLT_MAX. The reference runs with denormals-are-zero,
+	// so a denormal of either sign counts as +0; the exponent bits are tested so that the answer does not depend
+	// on the denormal mode of the comparison instructions.
+	__device__ float operator()( float a, float, float ) const
+	{
+		if( ( __float_as_uint( a ) & 0x7f800000u ) == 0u ) return FLT_MAX;
+		if( a == FLT_MIN ) return FLT_MAX;
+		if( a == -FLT_MIN ) return -FLT_MAX;
+		return 1.f / a;
+	}
+};
+struct CMinMaxOp {
+	const float* MinPtr; const float* MaxPtr; float Min, Max;
+	__device__ void prepare() { Min = *MinPtr; Max = *MaxPtr; }
+	__device__ float operator()( float a, float, float ) const
+	{
+		const float lo = a > Min ? a : Min;
+		return lo < Max ? lo : Max;
+	}
+};
+struct CSigmoidOp : CNoScalar {
+	// e / ( e + 1 ), e = clamped exp( x ) (src/CPU/x86/CpuX86MathEngineVectorMathPrivate.h:1200-1228)
+	__device__ float operator()( float a, float, float ) const
+	{
+		const float e = expClamped( a );
+		return e / ( e + 1.f );
+	}
+};
+struct CTanhOp : CNoScalar {
+	// -1 + 2 / ( 1 + exp( -2x ) ) (src/CPU/x86/CpuX86MathEngineVectorMathPrivate.h:1178-1187);
+	// tanhf is used for small |x| where that form loses relative accuracy through cancellation
+	__device__ float operator()( float a, float, float ) const { return tanhf( a ); }
+};
+
+// ---- reductions to one value: one workgroup per 16K elements, atomics into a zeroed result -----------------
+
+template<bool DOT>
+__global__ __launch_bounds__( 256 ) void sumKernel( const float* a, const float* b, int n, float* result )
+{
+	__shared__ float part[4];
+	float s = 0.f;
+	const int stride = gridDim.x * 256;
+	for( int i = blockIdx.x * 256 + threadIdx.x; i < n; i += stride ) {
+		s += DOT ? a[i] * b[i] : a[i];
+	}
+	s = waveReduceSum( s );
+	if( ( threadIdx.x & 63 ) == 0 ) {
+		part[threadIdx.x >> 6] = s;
+	}
+	__syncthreads();
+	if( threadIdx.x == 0 ) {
+		atomicAdd( result, part[0] + part[1] + part[2] + part[3] );
+	}
+}
+
+} // namespace nh
+
+using namespace nh;
+
+#define NH_UNARY( name, Op ) \
+	extern "C" int name( nhStream s, const float* first, float* result, int vectorSize ) \
+	{ return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, Op() ); }
+
+#define NH_BINARY( name, T, Op ) \
+	extern "C" int name( nhStream s, const T* first, const T* second, T* result, int vectorSize ) \
+	{ return launchEltwise<2, T, T>( s, first, second, (const T*)nullptr, result, vectorSize, Op() ); }
+
+extern "C" int nhVectorCopy( nhStream s, float* first, const float* second, int vectorSize )
+{
+	return launchEltwise<1, float, float>( s, second, (const float*)nullptr, (const float*)nullptr, first, vectorSize, CCopyOp<float>() );
+}
+extern "C" int nhVectorCopyInt( nhStream s, int* first, const int* second, int vectorSize )
+{
+	return launchEltwise<1, int, int>( s, second, (const int*)nullptr, (const int*)nullptr, first, vectorSize, CCopyOp<int>() );
+}
+extern "C" int nhVectorFill( nhStream s, float* result, float value, int vectorSize )
+{
+	CFillOp<float> op; op.Value = value;
+	return launchEltwise<0, float, float>( s, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorFillInt( nhStream s, int* result, int value, int vectorSize )
+{
+	CFillOp<int> op; op.Value = value;
+	return launchEltwise<0, int, int>( s, (const int*)nullptr, (const int*)nullptr, (const int*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorFillFromHandle( nhStream s, float* result, int vectorSize, const float* value )
+{
+	NH_REQUIRE( value != nullptr );
+	CFillFromOp<float> op; op.Ptr = value; op.Value = 0;
+	return launchEltwise<0, float, float>( s, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorFillFromHandleInt( nhStream s, int* result, int vectorSize, const int* value )
+{
+	NH_REQUIRE( value != nullptr );
+	CFillFromOp<int> op; op.Ptr = value; op.Value = 0;
+	return launchEltwise<0, int, int>( s, (const int*)nullptr, (const int*)nullptr, (const int*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorConvertFloatToInt( nhStream s, const float* from, int* to, int vectorSize )
+{
+	return launchEltwise<1, float, int>( s, from, (const float*)nullptr, (const float*)nullptr, to, vectorSize, CFloatToIntOp() );
+}
+extern "C" int nhVectorConvertIntToFloat( nhStream s, const int* from, float* to, int vectorSize )
+{
+	return launchEltwise<1, int, float>( s, from, (const int*)nullptr, (const int*)nullptr, to, vectorSize, CIntToFloatOp() );
+}
+
+extern "C" int nhVectorReLU( nhStream s, const float* first, float* result, int vectorSize, const float* upperThreshold )
+{
+	NH_REQUIRE( upperThreshold != nullptr );
+	CReLUOp op; op.Ptr = upperThreshold; op.Threshold = 0;
+	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorELU( nhStream s, const float* first, float* result, int vectorSize, const float* alpha )
+{
+	NH_REQUIRE( alpha != nullptr );
+	CELUOp op; op.Ptr = alpha; op.Alpha = 0;
+	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorLeakyReLU( nhStream s, const float* first, float* result, int vectorSize, const float* alpha )
+{
+	NH_REQUIRE( alpha != nullptr );
+	CLeakyReLUOp op; op.Ptr = alpha; op.Alpha = 0;
+	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorHardSigmoid( nhStream s, const float* first, float* result, int vectorSize,
+	const float* slope, const float* bias )
+{
+	NH_REQUIRE( slope != nullptr && bias != nullptr );
+	CHardSigmoidOp op; op.SlopePtr = slope; op.BiasPtr = bias; op.Slope = 0; op.Bias = 0;
+	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorMinMax( nhStream s, const float* first, float* result, int vectorSize,
+	const float* minValue, const float* maxValue )
+{
+	NH_REQUIRE( minValue != nullptr && maxValue != nullptr );
+	CMinMaxOp op; op.MinPtr = minValue; op.MaxPtr = maxValue; op.Min = 0; op.Max = 0;
+	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+
+NH_UNARY( nhVectorHSwish, CHSwishOp )
+NH_UNARY( nhVectorAbs, CAbsOp )
+NH_UNARY( nhVectorHardTanh, CHardTanhOp )
+NH_UNARY( nhVectorNeg, CNegOp )
+NH_UNARY( nhVectorExp, CExpOp )
+NH_UNARY( nhVectorLog, CLogOp )
+NH_UNARY( nhVectorErf, CErfOp )
+NH_UNARY( nhVectorSqrt, CSqrtOp )
+NH_UNARY( nhVectorInv, CInvOp )
+NH_UNARY( nhVectorSigmoid, CSigmoidOp )
+NH_UNARY( nhVectorTanh, CTanhOp )
+
+NH_BINARY( nhVectorEltwiseMax, float, CMaxOp )
+NH_BINARY( nhVectorEltwiseMin, float, CMinOp )
+NH_BINARY( nhVectorAdd, float, CAddOp<float> )
+NH_BINARY( nhVectorAddInt, int, CAddOp<int> )
+NH_BINARY( nhVectorSub, float, CSubOp<float> )
+NH_BINARY( nhVectorSubInt, int, CSubOp<int> )
+NH_BINARY( nhVectorEltwiseMultiply, float, CMulOp<float> )
+NH_BINARY( nhVectorEltwiseMultiplyInt, int, CMulOp<int> )
+NH_BINARY( nhVectorEltwiseNegMultiply, float, CNegMulOp )
+NH_BINARY( nhVectorEltwiseDivide, float, CDivOp )
+
+extern "C" int nhVectorEltwiseMultiplyAdd( nhStream s, const float* first, const float* second, float* result, int vectorSize )
+{
+	return launchEltwise<3, float, float>( s, first, second, result, result, vectorSize, CMulAddOp() );
+}
+
+extern "C" int nhVectorAddValue( nhStream s, const float* first, float* result, int vectorSize, const float* addition )
+{
+	NH_REQUIRE( addition != nullptr );
+	CAddValueOp<float> op; op.Ptr = addition; op.Value = 0;
+	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorAddValueInt( nhStream s, const int* first, int* result, int vectorSize, const int* addition )
+{
+	NH_REQUIRE( addition != nullptr );
+	CAddValueOp<int> op; op.Ptr = addition; op.Value = 0;
+	return launchEltwise<1, int, int>( s, first, (const int*)nullptr, (const int*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorMultiply( nhStream s, const float* first, float* result, int vectorSize, const float* multiplier )
+{
+	NH_REQUIRE( multiplier != nullptr );
+	CMulValueOp<float> op; op.Ptr = multiplier; op.Value = 0;
+	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorMultiplyInt( nhStream s, const int* first, int* result, int vectorSize, const int* multiplier )
+{
+	NH_REQUIRE( multiplier != nullptr );
+	CMulValueOp<int> op; op.Ptr = multiplier; op.Value = 0;
+	return launchEltwise<1, int, int>( s, first, (const int*)nullptr, (const int*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorNegMultiply( nhStream s, const float* first, float* result, int vectorSize, const float* multiplier )
+{
+	NH_REQUIRE( multiplier != nullptr );
+	CNegMulValueOp op; op.Ptr = multiplier; op.Value = 0;
+	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorMultiplyAndAdd( nhStream s, const float* first, const float* second, float* result,
+	int vectorSize, const float* mult )
+{
+	NH_REQUIRE( mult != nullptr );
+	CMultiplyAndAddOp op; op.Ptr = mult; op.Mult = 0;
+	return launchEltwise<2, float, float>( s, first, second, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorMultiplyAndSub( nhStream s, const float* first, const float* second, float* result,
+	int vectorSize, const float* mult )
+{
+	NH_REQUIRE( mult != nullptr );
+	CMultiplyAndSubOp op; op.Ptr = mult; op.Mult = 0;
+	return launchEltwise<2, float, float>( s, first, second, (const float*)nullptr, result, vectorSize, op );
+}
+
+extern "C" int nhVectorSum( nhStream s, const float* first, int vectorSize, float* result )
+{
+	NH_REQUIRE( vectorSize >= 0 && result != nullptr );
+	int rc = nhVectorFill( s, result, 0.f, 1 );
+	if( rc != NH_OK || vectorSize == 0 ) {
+		return rc;
+	}
+	int blocks = ceilDiv( vectorSize, 16384 );
+	blocks = blocks > 2048 ? 2048 : blocks;
+	hipLaunchKernelGGL( sumKernel<false>, dim3( blocks ), dim3( 256 ), 0, toStream( s ), first, (const float*)nullptr, vectorSize, result );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+extern "C" int nhVectorDotProduct( nhStream s, const float* first, const float* second, int vectorSize, float* result )
+{
+	NH_REQUIRE( vectorSize >= 0 && result != nullptr );
+	int rc = nhVectorFill( s, result, 0.f, 1 );
+	if( rc != NH_OK || vectorSize == 0 ) {
+		return rc;
+	}
+	int blocks = ceilDiv( vectorSize, 16384 );
+	blocks = blocks > 2048 ? 2048 : blocks;
+	hipLaunchKernelGGL( sumKernel<true>, dim3( blocks ), dim3( 256 ), 0, toStream( s ), first, second, vectorSize, result );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}

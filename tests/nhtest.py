@@ -1,0 +1,382 @@
+"""Shared helpers of the test-suite: loaders for the checkers (oracle/liboracle.so, oracle/_ref) and thin numpy
+front-ends for them, plus the device-side call helpers for the HIP library.
+
+Only tests, the smoke run and the benchmark's cpu_baseline leg import this module; the product never does.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+ORACLE_LIB = os.path.join(ORACLE_DIR, "liboracle.so")
+SHIM_LIB = os.path.join(ORACLE_DIR, "_ref", "libengine_shim.so")
+
+# tolerance of the parity bar: |a - b| <= ATOL + RTOL * |b|
+RTOL = 1e-4
+ATOL = 1e-5
+
+UNARY = {name: i for i, name in enumerate([
+    "relu", "elu", "leaky_relu", "hswish", "abs", "hard_tanh", "hard_sigmoid", "neg", "exp", "log", "erf", "sqrt",
+    "inv", "minmax", "sigmoid", "tanh", "add_value", "multiply", "neg_multiply", "copy"])}
+BINARY = {name: i for i, name in enumerate([
+    "add", "sub", "eltwise_multiply", "eltwise_neg_multiply", "eltwise_divide", "eltwise_max", "eltwise_min",
+    "multiply_and_add", "multiply_and_sub", "eltwise_multiply_add"])}
+BINARY_INT = {"add": 0, "sub": 1, "multiply": 2}
+
+c_float_p = ctypes.POINTER(ctypes.c_float)
+c_int_p = ctypes.POINTER(ctypes.c_int)
+
+
+def f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def i32(a):
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+def fp(a):
+    return None if a is None else a.ctypes.data_as(c_float_p)
+
+
+def ip(a):
+    return None if a is None else a.ctypes.data_as(c_int_p)
+
+
+def build_oracle():
+    """Compiles oracle/liboracle.so (and oracle/_ref when the reference sources are present)."""
+    import subprocess
+    subprocess.run(["make", "-s", "-C", ORACLE_DIR, "-j8", "all"], check=True)
+
+
+_oracle = None
+
+
+def oracle():
+    global _oracle
+    if _oracle is None:
+        if not os.path.exists(ORACLE_LIB):
+            build_oracle()
+        _oracle = ctypes.CDLL(ORACLE_LIB)
+        _oracle.orc_vector_sum.restype = ctypes.c_float
+        _oracle.orc_vector_dot_product.restype = ctypes.c_float
+    return _oracle
+
+
+def have_reference():
+    return os.path.exists(SHIM_LIB)
+
+
+_shim = None
+_cpu_engine = None
+
+
+def shim():
+    global _shim
+    if _shim is None:
+        _shim = ctypes.CDLL(SHIM_LIB)
+        _shim.shim_create_cpu_engine.restype = ctypes.c_void_p
+        _shim.shim_last_error.restype = ctypes.c_char_p
+    return _shim
+
+
+def cpu_engine():
+    """The reference's CCpuMathEngine (one per process)."""
+    global _cpu_engine
+    if _cpu_engine is None:
+        _cpu_engine = ctypes.c_void_p(shim().shim_create_cpu_engine())
+        assert _cpu_engine.value, "CreateCpuMathEngine failed"
+    return _cpu_engine
+
+
+def conv_out(h, w, fh, fw, ph, pw, sh, sw, dh=1, dw=1):
+    ho = 1 + (h - (fh - 1) * dh + 2 * ph - 1) // sh
+    wo = 1 + (w - (fw - 1) * dw + 2 * pw - 1) // sw
+    return ho, wo
+
+
+class Cpu:
+    """Numpy front-end shared by the oracle ('orc') and the reference engine through the shim ('ref')."""
+
+    def __init__(self, kind):
+        assert kind in ("orc", "ref")
+        self.kind = kind
+        self.lib = oracle() if kind == "orc" else shim()
+        self.pre = "orc_" if kind == "orc" else "shim_"
+        self.eng = () if kind == "orc" else (cpu_engine(),)
+
+    def _call(self, name, *args):
+        rc = getattr(self.lib, self.pre + name)(*self.eng, *args)
+        if self.kind == "ref" and rc != 0:
+            raise RuntimeError("reference engine: " + self.lib.shim_last_error().decode())
+        return rc
+
+    # ---- element-wise
+    def unary(self, op, x, p0=0.0, p1=0.0):
+        x = f32(x)
+        y = np.empty_like(x)
+        self._call("vector_unary", UNARY[op], fp(x), fp(y), x.size, ctypes.c_float(p0), ctypes.c_float(p1))
+        return y
+
+    def binary(self, op, a, b, p0=0.0, result=None):
+        a, b = f32(a), f32(b)
+        y = np.zeros_like(a) if result is None else f32(result).copy()
+        self._call("vector_binary", BINARY[op], fp(a), fp(b), fp(y), a.size, ctypes.c_float(p0))
+        return y
+
+    def binary_int(self, op, a, b):
+        a, b = i32(a), i32(b)
+        y = np.empty_like(a)
+        self._call("vector_binary_int", BINARY_INT[op], ip(a), ip(b), ip(y), a.size)
+        return y
+
+    def float_to_int(self, x):
+        x = f32(x)
+        y = np.empty(x.shape, np.int32)
+        self._call("vector_convert_float_to_int", fp(x), ip(y), x.size)
+        return y
+
+    def int_to_float(self, x):
+        x = i32(x)
+        y = np.empty(x.shape, np.float32)
+        self._call("vector_convert_int_to_float", ip(x), fp(y), x.size)
+        return y
+
+    def vector_sum(self, x):
+        x = f32(x)
+        if self.kind == "orc":
+            return np.float32(self.lib.orc_vector_sum(fp(x), x.size))
+        r = np.zeros(1, np.float32)
+        self._call("vector_sum", fp(x), x.size, fp(r))
+        return r[0]
+
+    def dot(self, a, b):
+        a, b = f32(a), f32(b)
+        if self.kind == "orc":
+            return np.float32(self.lib.orc_vector_dot_product(fp(a), fp(b), a.size))
+        r = np.zeros(1, np.float32)
+        self._call("vector_dot_product", fp(a), fp(b), a.size, fp(r))
+        return r[0]
+
+    # ---- broadcasts, reductions
+    def set_vector_to_matrix_rows(self, h, w, vec):
+        vec = f32(vec)
+        y = np.empty((h, w), np.float32)
+        self._call("set_vector_to_matrix_rows", fp(y), h, w, fp(vec))
+        return y
+
+    def add_vector_to_matrix_rows(self, m, vec):
+        m, vec = f32(m), f32(vec)  # m [b,h,w], vec [b,w]
+        b, h, w = m.shape
+        y = np.empty_like(m)
+        self._call("add_vector_to_matrix_rows", b, fp(m), fp(y), h, w, fp(vec))
+        return y
+
+    def add_vector_to_matrix_columns(self, m, vec, sign=1):
+        m, vec = f32(m), f32(vec)
+        h, w = m.shape
+        y = np.empty_like(m)
+        self._call("add_vector_to_matrix_columns", fp(m), fp(y), h, w, fp(vec), sign)
+        return y
+
+    def sum_matrix_rows(self, m, add_to=None):
+        m = f32(m)
+        b, h, w = m.shape
+        y = np.zeros((b, w), np.float32) if add_to is None else f32(add_to).copy()
+        self._call("sum_matrix_rows", b, fp(y), fp(m), h, w, 0 if add_to is None else 1)
+        return y
+
+    def sum_matrix_columns(self, m):
+        m = f32(m)
+        h, w = m.shape
+        y = np.empty(h, np.float32)
+        self._call("sum_matrix_columns", fp(y), fp(m), h, w)
+        return y
+
+    def multiply_diag_matrix_by_matrix(self, d, m):
+        d, m = f32(d), f32(m)
+        y = np.empty_like(m)
+        self._call("multiply_diag_matrix_by_matrix", fp(d), m.shape[0], fp(m), m.shape[1], fp(y))
+        return y
+
+    def batch_multiply_matrix_by_diag_matrix(self, batch, first, h, w, first_off, second, second_off):
+        first, second = f32(first), f32(second)
+        y = np.empty((batch, h, w), np.float32)
+        self._call("batch_multiply_matrix_by_diag_matrix", batch, fp(first), h, w, first_off, fp(second), second_off, fp(y))
+        return y
+
+    def softmax_rows(self, m):
+        m = f32(m)
+        y = np.empty_like(m)
+        self._call("matrix_softmax_by_rows", fp(m), m.shape[0], m.shape[1], fp(y))
+        return y
+
+    def log_sum_exp_rows(self, m):
+        m = f32(m)
+        y = np.empty(m.shape[0], np.float32)
+        self._call("matrix_log_sum_exp_by_rows", fp(m), m.shape[0], m.shape[1], fp(y))
+        return y
+
+    def find_max_in_rows(self, m, with_indices=True):
+        m = f32(m)
+        v = np.empty(m.shape[0], np.float32)
+        idx = np.empty(m.shape[0], np.int32) if with_indices else None
+        self._call("find_max_value_in_rows", fp(m), m.shape[0], m.shape[1], fp(v), ip(idx))
+        return v, idx
+
+    def find_max_in_columns(self, m):
+        m = f32(m)
+        b, h, w = m.shape
+        v = np.empty((b, w), np.float32)
+        idx = np.empty((b, w), np.int32)
+        self._call("find_max_value_in_columns", b, fp(m), h, w, fp(v), ip(idx))
+        return v, idx
+
+    def transpose(self, x):
+        """x [b,h,m,w,c] -> [b,w,m,h,c]"""
+        x = f32(x)
+        b, h, m, w, c = x.shape
+        y = np.empty((b, w, m, h, c), np.float32)
+        self._call("transpose_matrix", b, fp(x), h, m, w, c, fp(y))
+        return y
+
+    # ---- matrix products (C is M x N, reduction K)
+    def matmul(self, kind, a, b, c=None, lda=None, ldb=None, ldc=None, M=None, N=None, K=None, batch=1):
+        """kind: 'nt' (strided), 'bnt', 'bnn', 'btn' (batched, dense), 'tn_add' (strided, accumulates into c)."""
+        a, b = f32(a), f32(b)
+        if self.kind == "orc":
+            fn = {"nt": "orc_matmul_nt", "bnt": "orc_matmul_nt", "bnn": "orc_matmul_nn", "btn": "orc_matmul_tn",
+                  "tn_add": "orc_matmul_tn"}[kind]
+            if kind in ("nt", "tn_add"):
+                out = np.zeros(((M - 1) * ldc + N,), np.float32) if c is None else f32(c).copy().ravel()
+                getattr(self.lib, fn)(fp(a), lda, fp(b), ldb, fp(out), ldc, M, N, K, 1 if kind == "tn_add" else 0)
+                return out
+            out = np.empty((batch, M, N), np.float32)
+            a_rows, a_cols = (K, M) if kind == "btn" else (M, K)
+            b_rows, b_cols = (N, K) if kind == "bnt" else (K, N)
+            a3 = a.reshape(batch, a_rows, a_cols)
+            b3 = b.reshape(batch, b_rows, b_cols)
+            for i in range(batch):
+                ai, bi, oi = f32(a3[i]), f32(b3[i]), np.empty((M, N), np.float32)
+                getattr(self.lib, fn)(fp(ai), a_cols, fp(bi), b_cols, fp(oi), N, M, N, K, 0)
+                out[i] = oi
+            return out
+        code = {"nt": 0, "bnt": 1, "bnn": 2, "btn": 3, "tn_add": 4}[kind]
+        if kind in ("nt", "tn_add"):
+            out = np.zeros(((M - 1) * ldc + N,), np.float32) if c is None else f32(c).copy().ravel()
+            self._call("matmul", code, 1, fp(a), lda, fp(b), ldb, fp(out), ldc, M, N, K)
+            return out
+        out = np.empty((batch, M, N), np.float32)
+        lda = M if kind == "btn" else K
+        ldb = K if kind == "bnt" else N
+        self._call("matmul", code, batch, fp(a), lda, fp(b), ldb, fp(out), N, M, N, K)
+        return out
+
+    # ---- convolution, pooling
+    def conv(self, x, filt, bias, ph, pw, sh, sw, dh=1, dw=1):
+        x, filt = f32(x), f32(filt)
+        n, h, w, cin = x.shape
+        cout, fh, fw, _ = filt.shape
+        ho, wo = conv_out(h, w, fh, fw, ph, pw, sh, sw, dh, dw)
+        bias = None if bias is None else f32(bias)
+        y = np.empty((n, ho, wo, cout), np.float32)
+        self._call("blob_convolution", fp(x), n, h, w, cin, fp(filt), cout, fh, fw, ph, pw, sh, sw, dh, dw, fp(bias), fp(y))
+        return y
+
+    def channelwise_conv(self, x, filt, bias, ph, pw, sh, sw):
+        x, filt = f32(x), f32(filt)
+        n, h, w, c = x.shape
+        fh, fw, _ = filt.shape
+        ho, wo = conv_out(h, w, fh, fw, ph, pw, sh, sw)
+        bias = None if bias is None else f32(bias)
+        y = np.empty((n, ho, wo, c), np.float32)
+        self._call("blob_channelwise_convolution", fp(x), n, h, w, c, fp(filt), fh, fw, ph, pw, sh, sw, fp(bias), fp(y))
+        return y
+
+    def max_pool(self, x, fh, fw, sh, sw, with_indices=False):
+        x = f32(x)
+        n, h, w, c = x.shape
+        ho, wo = (h - fh) // sh + 1, (w - fw) // sw + 1
+        y = np.empty((n, ho, wo, c), np.float32)
+        idx = np.empty((n, ho, wo, c), np.int32) if with_indices else None
+        self._call("blob_max_pooling", fp(x), n, h, w, c, fh, fw, sh, sw, ip(idx), fp(y))
+        return (y, idx) if with_indices else y
+
+    def mean_pool(self, x, fh, fw, sh, sw):
+        x = f32(x)
+        n, h, w, c = x.shape
+        ho, wo = (h - fh) // sh + 1, (w - fw) // sw + 1
+        y = np.empty((n, ho, wo, c), np.float32)
+        self._call("blob_mean_pooling", fp(x), n, h, w, c, fh, fw, sh, sw, fp(y))
+        return y
+
+    def resize_image(self, x, dl, dr, dt, db, padding=0, value=0.0):
+        x = f32(x)
+        n, h, w, c = x.shape
+        y = np.empty((n, h + dt + db, w + dl + dr, c), np.float32)
+        self._call("blob_resize_image", fp(x), n, h, w, c, dl, dr, dt, db, padding, ctypes.c_float(value), fp(y))
+        return y
+
+    def split(self, big, dim, part_dims):
+        """big: 7-D array; part_dims: list of 7-tuples. Returns the parts."""
+        big = f32(big)
+        parts = [np.empty(d, np.float32) for d in part_dims]
+        self._split_merge(big, dim, parts, merge=0)
+        return parts
+
+    def merge(self, parts, dim, big_dims):
+        parts = [f32(p) for p in parts]
+        big = np.empty(big_dims, np.float32)
+        self._split_merge(big, dim, parts, merge=1)
+        return big
+
+    def _split_merge(self, big, dim, parts, merge):
+        count = len(parts)
+        ptrs = (c_float_p * count)(*[fp(p) for p in parts])
+        if self.kind == "orc":
+            rows = int(np.prod(big.shape[:dim])) if dim > 0 else 1
+            sizes = [int(np.prod(p.shape[dim:])) if dim > 0 else p.size for p in parts]
+            self.lib.orc_blob_split_merge(fp(big), rows, ptrs, ip(i32(sizes)), count, merge)
+        else:
+            pd = i32(np.array([p.shape for p in parts]).ravel())
+            self._call("blob_split_merge", dim, ip(i32(big.shape)), fp(big), ip(pd), ptrs, count, merge)
+
+    def lstm(self, w_in, b_in, w_rec, b_rec, x, reverse=False, c0=None, h0=None, want_state=True):
+        w_in, w_rec, x = f32(w_in), f32(w_rec), f32(x)
+        T, B, In = x.shape
+        H = w_rec.shape[1]
+        b_in = None if b_in is None else f32(b_in)
+        b_rec = None if b_rec is None else f32(b_rec)
+        c0 = None if c0 is None else f32(c0)
+        h0 = None if h0 is None else f32(h0)
+        h = np.empty((T, B, H), np.float32)
+        c = np.empty((T, B, H), np.float32) if want_state else None
+        self._call("lstm", H, In, fp(w_in), fp(b_in), fp(w_rec), fp(b_rec), 1 if reverse else 0, T, B,
+                   fp(c0), fp(h0), fp(x), fp(c), fp(h))
+        return h, c
+
+
+def ctc_greedy_collapse(labels, blank, seq_len=None):
+    """labels [B][T] int32 -> list of label lists (oracle only: the reference does this on the host in the layer)."""
+    labels = i32(labels)
+    B, T = labels.shape
+    out = np.zeros((B, T), np.int32)
+    lengths = np.zeros(B, np.int32)
+    sl = None if seq_len is None else i32(seq_len)
+    oracle().orc_ctc_greedy_collapse(ip(labels), T, B, blank, ip(sl), ip(out), ip(lengths))
+    return [out[b, :lengths[b]].tolist() for b in range(B)]
+
+
+def assert_close(actual, expected, what="", rtol=RTOL, atol=ATOL):
+    actual = np.asarray(actual, dtype=np.float64)
+    expected = np.asarray(expected, dtype=np.float64)
+    assert actual.shape == expected.shape, "%s: shape %s vs %s" % (what, actual.shape, expected.shape)
+    err = np.abs(actual - expected)
+    bound = atol + rtol * np.abs(expected)
+    bad = ~(err <= bound)
+    if bad.any():
+        i = np.unravel_index(np.argmax(np.where(bad, err - bound, -np.inf)), err.shape)
+        raise AssertionError("%s: %d of %d elements outside rtol=%g atol=%g; worst at %s: got %r expected %r" % (
+            what, int(bad.sum()), bad.size, rtol, atol, i, actual[i], expected[i]))

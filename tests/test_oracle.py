@@ -1,0 +1,535 @@
+"""Pins the CPU oracle (oracle/oracle.c).
+
+Two independent anchors for every function:
+  1. the reference's own CCpuMathEngine, compiled from its sources into oracle/_ref (skipped only when that
+     build is absent), called through oracle/engine_shim.cpp;
+  2. formulations that do not share code with the oracle: numpy / scipy routines, closed forms, brute force.
+A dropped term, swapped index or transposed operand in the oracle fails at least one of them.
+"""
+import numpy as np
+import pytest
+import scipy.signal
+import scipy.special
+
+import nhtest
+from nhtest import Cpu, assert_close
+
+orc = Cpu("orc")
+needs_ref = pytest.mark.skipif(not nhtest.have_reference(), reason="oracle/_ref is not built")
+
+
+def ref():
+    return Cpu("ref")
+
+
+def rng(seed):
+    return np.random.default_rng(0xC0FFEE + seed)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# element-wise
+
+UNARY_CASES = [
+    ("relu", 0.0, 0.0), ("relu", 6.0, 0.0), ("elu", 0.7, 0.0), ("leaky_relu", 0.1, 0.0), ("hswish", 0, 0),
+    ("abs", 0, 0), ("hard_tanh", 0, 0), ("hard_sigmoid", 0.2, 0.5), ("neg", 0, 0), ("exp", 0, 0), ("log", 0, 0),
+    ("erf", 0, 0), ("sqrt", 0, 0), ("inv", 0, 0), ("minmax", -0.5, 1.5), ("sigmoid", 0, 0), ("tanh", 0, 0),
+    ("add_value", 1.25, 0), ("multiply", -2.5, 0), ("neg_multiply", 1.702, 0), ("copy", 0, 0),
+]
+
+
+def unary_input(op, n, seed):
+    x = rng(seed).uniform(-10, 10, n).astype(np.float32)
+    if op in ("log", "sqrt"):
+        x = np.abs(x) + 1e-3
+    # special values: zeros, tiny, huge
+    x[:8] = [0.0, -0.0, 1e-38, -1e-38, 3.0, -3.0, 87.0, -87.0]
+    if op in ("log", "sqrt"):
+        x[:8] = np.abs(x[:8])
+    return x
+
+
+NUMPY_UNARY = {
+    "relu": lambda x, p0, p1: np.minimum(np.maximum(x, 0), p0) if p0 > 0 else np.maximum(x, 0),
+    "elu": lambda x, p0, p1: np.where(x >= 0, x, p0 * np.expm1(np.minimum(x, 0).astype(np.float64))),
+    "leaky_relu": lambda x, p0, p1: np.where(x > 0, x, p0 * x),
+    "hswish": lambda x, p0, p1: x * np.clip(x + 3, 0, 6) / 6,
+    "abs": lambda x, p0, p1: np.abs(x),
+    "hard_tanh": lambda x, p0, p1: np.clip(x, -1, 1),
+    "hard_sigmoid": lambda x, p0, p1: np.clip(x * p0 + p1, 0, 1),
+    "neg": lambda x, p0, p1: -x,
+    "exp": lambda x, p0, p1: np.exp(x.astype(np.float64)),
+    "log": lambda x, p0, p1: np.log(np.clip(x.astype(np.float64), np.finfo(np.float32).tiny, None)),
+    "erf": lambda x, p0, p1: scipy.special.erf(x.astype(np.float64)),
+    "sqrt": lambda x, p0, p1: np.sqrt(x.astype(np.float64)),
+    "minmax": lambda x, p0, p1: np.clip(x, p0, p1),
+    "sigmoid": lambda x, p0, p1: scipy.special.expit(x.astype(np.float64)),
+    "tanh": lambda x, p0, p1: np.tanh(x.astype(np.float64)),
+    "add_value": lambda x, p0, p1: x + np.float32(p0),
+    "multiply": lambda x, p0, p1: x * np.float32(p0),
+    "neg_multiply": lambda x, p0, p1: -x * np.float32(p0),
+    "copy": lambda x, p0, p1: x,
+}
+
+
+@pytest.mark.parametrize("op,p0,p1", UNARY_CASES)
+def test_unary_vs_numpy(op, p0, p1):
+    x = unary_input(op, 1003, 1)
+    y = orc.unary(op, x, p0, p1)
+    if op == "inv":
+        big = np.abs(x) > 1e-30
+        assert_close(y[big], 1.0 / x[big].astype(np.float64), op)
+        fmax = np.finfo(np.float32).max
+        # saturation of 0 and of denormals; with denormals-are-zero a negative denormal counts as +0
+        assert y[0] == fmax and y[2] == fmax and y[3] == fmax
+        tiny = np.finfo(np.float32).tiny
+        edge = orc.unary("inv", np.array([tiny, -tiny, 2 * tiny], np.float32))
+        assert edge[0] == fmax and edge[1] == -fmax and edge[2] == np.float32(1.0) / np.float32(2 * tiny)
+        return
+    assert_close(y, NUMPY_UNARY[op](x, p0, p1), op)
+
+
+@needs_ref
+@pytest.mark.parametrize("op,p0,p1", UNARY_CASES)
+def test_unary_vs_reference(op, p0, p1):
+    for n in (1, 3, 4, 7, 64, 1003):
+        x = unary_input(op, max(n, 8), n)[:n] if n < 8 else unary_input(op, n, n)
+        assert_close(orc.unary(op, x, p0, p1), ref().unary(op, x, p0, p1), "%s n=%d" % (op, n))
+
+
+def test_vector_log_and_exp_clamps():
+    fmin, fmax = np.finfo(np.float32).tiny, np.finfo(np.float32).max
+    y = orc.unary("log", np.array([0.0, -5.0, fmin, np.inf], np.float32))
+    assert_close(y, [np.log(np.float64(fmin))] * 3 + [np.log(np.float64(fmax))], "log clamp")
+    e = orc.unary("exp", np.array([-100.0, -87.4, 88.5, 0.0], np.float32))
+    assert e[0] == 0 and e[1] == 0 and e[2] == fmax and e[3] == 1
+
+
+BINARY_CASES = ["add", "sub", "eltwise_multiply", "eltwise_neg_multiply", "eltwise_divide", "eltwise_max",
+                "eltwise_min", "multiply_and_add", "multiply_and_sub", "eltwise_multiply_add"]
+NUMPY_BINARY = {
+    "add": lambda a, b, p, r: a + b, "sub": lambda a, b, p, r: a - b, "eltwise_multiply": lambda a, b, p, r: a * b,
+    "eltwise_neg_multiply": lambda a, b, p, r: -a * b, "eltwise_divide": lambda a, b, p, r: a / b,
+    "eltwise_max": lambda a, b, p, r: np.maximum(a, b), "eltwise_min": lambda a, b, p, r: np.minimum(a, b),
+    "multiply_and_add": lambda a, b, p, r: a + np.float32(p) * b,
+    "multiply_and_sub": lambda a, b, p, r: a - np.float32(p) * b,
+    "eltwise_multiply_add": lambda a, b, p, r: r + a * b,
+}
+
+
+@pytest.mark.parametrize("op", BINARY_CASES)
+def test_binary(op):
+    g = rng(2)
+    for n in (1, 5, 1000):
+        a = g.uniform(-10, 10, n).astype(np.float32)
+        b = g.uniform(0.5, 10, n).astype(np.float32) * np.where(g.random(n) < 0.5, -1, 1).astype(np.float32)
+        r = g.uniform(-10, 10, n).astype(np.float32)
+        y = orc.binary(op, a, b, 0.37, result=r)
+        assert_close(y, NUMPY_BINARY[op](a, b, 0.37, r), op)
+        if nhtest.have_reference():
+            assert_close(y, ref().binary(op, a, b, 0.37, result=r), op + " vs reference")
+
+
+def test_int_ops_and_conversions():
+    g = rng(3)
+    a = g.integers(-1000, 1000, 257).astype(np.int32)
+    b = g.integers(-1000, 1000, 257).astype(np.int32)
+    for op, fn in (("add", np.add), ("sub", np.subtract), ("multiply", np.multiply)):
+        assert np.array_equal(orc.binary_int(op, a, b), fn(a, b))
+        if nhtest.have_reference():
+            assert np.array_equal(ref().binary_int(op, a, b), fn(a, b))
+    x = g.uniform(-100, 100, 257).astype(np.float32)
+    assert np.array_equal(orc.float_to_int(x), np.trunc(x).astype(np.int32))
+    assert np.array_equal(orc.int_to_float(a), a.astype(np.float32))
+    if nhtest.have_reference():
+        assert np.array_equal(ref().float_to_int(x), orc.float_to_int(x))
+        assert np.array_equal(ref().int_to_float(a), orc.int_to_float(a))
+
+
+def test_sum_and_dot():
+    g = rng(4)
+    a = g.uniform(-1, 1, 10007).astype(np.float32)
+    b = g.uniform(-1, 1, 10007).astype(np.float32)
+    assert_close(orc.vector_sum(a), np.sum(a.astype(np.float64)), "sum", atol=1e-4)
+    assert_close(orc.dot(a, b), np.dot(a.astype(np.float64), b.astype(np.float64)), "dot", atol=1e-4)
+    if nhtest.have_reference():
+        assert_close(ref().vector_sum(a), orc.vector_sum(a), "sum vs reference", atol=1e-3)
+        assert_close(ref().dot(a, b), orc.dot(a, b), "dot vs reference", atol=1e-3)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# broadcasts, reductions, softmax, arg-max, transpose
+
+def test_broadcasts_and_sums():
+    g = rng(5)
+    for b, h, w in ((1, 1, 1), (2, 3, 5), (3, 17, 64), (1, 40, 7)):
+        m = g.uniform(-10, 10, (b, h, w)).astype(np.float32)
+        v = g.uniform(-10, 10, (b, w)).astype(np.float32)
+        got = {
+            "add_rows": orc.add_vector_to_matrix_rows(m, v),
+            "set_rows": orc.set_vector_to_matrix_rows(h, w, v[0]),
+            "add_cols": orc.add_vector_to_matrix_columns(m[0], v[0, :1].repeat(h) + np.arange(h, dtype=np.float32)),
+            "sub_cols": orc.add_vector_to_matrix_columns(m[0], np.arange(h, dtype=np.float32), sign=-1),
+            "sum_rows": orc.sum_matrix_rows(m),
+            "sum_rows_add": orc.sum_matrix_rows(m, add_to=v),
+            "sum_cols": orc.sum_matrix_columns(m[0]),
+            "diag_left": orc.multiply_diag_matrix_by_matrix(np.arange(h, dtype=np.float32) - 1, m[0]),
+            "diag_right": orc.batch_multiply_matrix_by_diag_matrix(b, m, h, w, h * w, v, w),
+            "diag_right_bcast": orc.batch_multiply_matrix_by_diag_matrix(b, m, h, w, h * w, v[0], 0),
+        }
+        col = v[0, :1].repeat(h) + np.arange(h, dtype=np.float32)
+        want = {
+            "add_rows": m + v[:, None, :], "set_rows": np.broadcast_to(v[0], (h, w)),
+            "add_cols": m[0] + col[:, None], "sub_cols": m[0] - np.arange(h, dtype=np.float32)[:, None],
+            "sum_rows": m.sum(axis=1, dtype=np.float64), "sum_rows_add": v + m.sum(axis=1, dtype=np.float64),
+            "sum_cols": m[0].sum(axis=1, dtype=np.float64),
+            "diag_left": (np.arange(h, dtype=np.float32) - 1)[:, None] * m[0],
+            "diag_right": m * v[:, None, :], "diag_right_bcast": m * v[0][None, None, :],
+        }
+        for k in got:
+            assert_close(got[k], want[k], "%s %s" % (k, (b, h, w)), atol=1e-4)
+        if nhtest.have_reference():
+            r = ref()
+            assert_close(r.add_vector_to_matrix_rows(m, v), got["add_rows"], "add_rows ref")
+            assert_close(r.set_vector_to_matrix_rows(h, w, v[0]), got["set_rows"], "set_rows ref")
+            assert_close(r.add_vector_to_matrix_columns(m[0], col), got["add_cols"], "add_cols ref")
+            assert_close(r.add_vector_to_matrix_columns(m[0], np.arange(h, dtype=np.float32), sign=-1), got["sub_cols"], "sub ref")
+            assert_close(r.sum_matrix_rows(m), got["sum_rows"], "sum_rows ref", atol=1e-4)
+            assert_close(r.sum_matrix_rows(m, add_to=v), got["sum_rows_add"], "sum_rows_add ref", atol=1e-4)
+            assert_close(r.sum_matrix_columns(m[0]), got["sum_cols"], "sum_cols ref", atol=1e-4)
+            assert_close(r.multiply_diag_matrix_by_matrix(np.arange(h, dtype=np.float32) - 1, m[0]), got["diag_left"], "diag ref")
+            assert_close(r.batch_multiply_matrix_by_diag_matrix(b, m, h, w, h * w, v, w), got["diag_right"], "diagr ref")
+            assert_close(r.batch_multiply_matrix_by_diag_matrix(b, m, h, w, h * w, v[0], 0), got["diag_right_bcast"], "diagb ref")
+
+
+def test_softmax_and_logsumexp():
+    g = rng(6)
+    for h, w in ((1, 1), (3, 2), (7, 101), (5, 256), (2, 1000), (2, 1500)):
+        m = g.uniform(-10, 10, (h, w)).astype(np.float32)
+        assert_close(orc.softmax_rows(m), scipy.special.softmax(m.astype(np.float64), axis=1), "softmax %s" % ((h, w),))
+        assert_close(orc.log_sum_exp_rows(m), scipy.special.logsumexp(m.astype(np.float64), axis=1), "lse %s" % ((h, w),))
+        if nhtest.have_reference():
+            assert_close(ref().softmax_rows(m), orc.softmax_rows(m), "softmax ref")
+            assert_close(ref().log_sum_exp_rows(m), orc.log_sum_exp_rows(m), "lse ref")
+    # rows sum to one; shifting a row by a constant changes nothing
+    m = g.uniform(-5, 5, (4, 33)).astype(np.float32)
+    assert_close(orc.softmax_rows(m).sum(axis=1), np.ones(4), "row sums")
+    assert_close(orc.softmax_rows(m + 3.0), orc.softmax_rows(m), "shift invariance")
+
+
+def test_argmax_rows_and_columns():
+    g = rng(7)
+    for h, w in ((1, 1), (5, 3), (64, 101), (9, 257)):
+        m = g.permutation(h * w).reshape(h, w).astype(np.float32)  # tie-free
+        v, i = orc.find_max_in_rows(m)
+        assert np.array_equal(i, np.argmax(m, axis=1)) and np.array_equal(v, m.max(axis=1))
+        if nhtest.have_reference():
+            rv, ri = ref().find_max_in_rows(m)
+            assert np.array_equal(ri, i) and np.array_equal(rv, v)
+    m = g.permutation(3 * 17 * 9).reshape(3, 17, 9).astype(np.float32)
+    v, i = orc.find_max_in_columns(m)
+    assert np.array_equal(i, np.argmax(m, axis=1)) and np.array_equal(v, m.max(axis=1))
+    # ties: the first row wins in columns (strict >), the first column wins in rows for the oracle
+    t = np.zeros((1, 4, 5), np.float32)
+    assert np.array_equal(orc.find_max_in_columns(t)[1], np.zeros((1, 5), np.int32))
+    if nhtest.have_reference():
+        rv, ri = ref().find_max_in_columns(m)
+        assert np.array_equal(ri, i) and np.array_equal(rv, v)
+        assert np.array_equal(ref().find_max_in_columns(t)[1], np.zeros((1, 5), np.int32))
+
+
+def test_transpose():
+    g = rng(8)
+    for shape in ((1, 1, 1, 1, 1), (2, 3, 1, 5, 1), (2, 4, 3, 5, 2), (1, 1, 3, 4, 2), (3, 7, 1, 1, 4), (2, 16, 1, 8, 64)):
+        x = g.uniform(-1, 1, shape).astype(np.float32)
+        y = orc.transpose(x)
+        assert np.array_equal(y, np.transpose(x, (0, 3, 2, 1, 4)))
+        if nhtest.have_reference():
+            assert np.array_equal(ref().transpose(x), y), shape
+
+
+# ---------------------------------------------------------------------------------------------------------
+# matrix products
+
+def test_matmul_vs_numpy_and_reference():
+    g = rng(9)
+    for M, N, K in ((1, 1, 1), (3, 5, 7), (17, 33, 65), (64, 101, 48)):
+        a = g.uniform(-1, 1, (M, K + 3)).astype(np.float32)  # strided rows
+        b = g.uniform(-1, 1, (N, K + 2)).astype(np.float32)
+        out = orc.matmul("nt", a, b, lda=K + 3, ldb=K + 2, ldc=N + 1, M=M, N=N, K=K)
+        want = a[:, :K].astype(np.float64) @ b[:, :K].astype(np.float64).T
+        got = np.pad(out, (0, M * (N + 1) - out.size)).reshape(M, N + 1)[:, :N]
+        assert_close(got, want, "nt %s" % ((M, N, K),))
+        if nhtest.have_reference():
+            r = ref().matmul("nt", a, b, lda=K + 3, ldb=K + 2, ldc=N + 1, M=M, N=N, K=K)
+            assert_close(np.pad(r, (0, M * (N + 1) - r.size)).reshape(M, N + 1)[:, :N], got, "nt ref")
+        # accumulate A^T B into C
+        at = g.uniform(-1, 1, (K, M + 1)).astype(np.float32)
+        bn = g.uniform(-1, 1, (K, N + 2)).astype(np.float32)
+        c0 = g.uniform(-1, 1, (M, N)).astype(np.float32)
+        out = orc.matmul("tn_add", at, bn, c=c0, lda=M + 1, ldb=N + 2, ldc=N, M=M, N=N, K=K)
+        assert_close(out.reshape(M, N), c0 + at[:, :M].astype(np.float64).T @ bn[:, :N].astype(np.float64), "tn_add")
+        if nhtest.have_reference():
+            r = ref().matmul("tn_add", at, bn, c=c0, lda=M + 1, ldb=N + 2, ldc=N, M=M, N=N, K=K)
+            assert_close(r, out, "tn_add ref")
+    for batch, M, N, K in ((1, 2, 3, 4), (3, 16, 8, 5), (4, 33, 17, 9)):
+        a = g.uniform(-1, 1, (batch, M, K)).astype(np.float32)
+        bt = g.uniform(-1, 1, (batch, N, K)).astype(np.float32)
+        bn = g.uniform(-1, 1, (batch, K, N)).astype(np.float32)
+        at = g.uniform(-1, 1, (batch, K, M)).astype(np.float32)
+        cases = {
+            "bnt": (a, bt, np.einsum("bmk,bnk->bmn", a.astype(np.float64), bt.astype(np.float64))),
+            "bnn": (a, bn, np.einsum("bmk,bkn->bmn", a.astype(np.float64), bn.astype(np.float64))),
+            "btn": (at, bn, np.einsum("bkm,bkn->bmn", at.astype(np.float64), bn.astype(np.float64))),
+        }
+        for kind, (x, y, want) in cases.items():
+            got = orc.matmul(kind, x, y, M=M, N=N, K=K, batch=batch)
+            assert_close(got, want, kind)
+            if nhtest.have_reference():
+                assert_close(ref().matmul(kind, x, y, M=M, N=N, K=K, batch=batch), got, kind + " ref")
+
+
+# ---------------------------------------------------------------------------------------------------------
+# convolution (grid after the reference's BlobConvolutionTest: 1x1, strides, dilations, pad > filter, H x 1 images)
+
+CONV_CASES = [
+    # n, h, w, cin, cout, fh, fw, ph, pw, sh, sw, dh, dw
+    (1, 1, 1, 1, 1, 1, 1, 0, 0, 1, 1, 1, 1),
+    (2, 5, 7, 3, 4, 3, 3, 1, 1, 1, 1, 1, 1),
+    (2, 8, 8, 4, 8, 1, 1, 0, 0, 1, 1, 1, 1),
+    (1, 9, 11, 5, 6, 3, 2, 2, 1, 2, 3, 1, 1),
+    (2, 12, 10, 3, 5, 3, 3, 2, 2, 1, 1, 2, 3),
+    (1, 5, 5, 3, 4, 3, 1, 2, 10, 2, 2, 1, 1),  # padding larger than the filter (BlobConvolutionTest.cpp:236-254)
+    (1, 5, 5, 3, 4, 3, 3, 2, 10, 2, 2, 1, 1),  # BlobConvolutionTest.cpp:255-273
+    (1, 40, 1, 3, 2, 5, 1, 2, 0, 1, 1, 1, 1),
+    (3, 14, 14, 16, 24, 5, 5, 2, 2, 2, 2, 1, 1),
+    (1, 16, 16, 3, 8, 7, 7, 3, 3, 2, 2, 1, 1),  # the stem shape at small size
+    (2, 8, 8, 8, 16, 1, 1, 0, 0, 2, 2, 1, 1),   # 1x1 stride 2 shortcut
+]
+
+
+def conv_via_scipy(x, filt, bias, ph, pw, sh, sw, dh, dw):
+    n, h, w, cin = x.shape
+    cout, fh, fw, _ = filt.shape
+    xp = np.pad(x.astype(np.float64), ((0, 0), (ph, ph), (pw, pw), (0, 0)))
+    fd = np.zeros((cout, (fh - 1) * dh + 1, (fw - 1) * dw + 1, cin))
+    fd[:, ::dh, ::dw, :] = filt
+    outs = []
+    for b in range(n):
+        per_filter = []
+        for co in range(cout):
+            acc = sum(scipy.signal.correlate2d(xp[b, :, :, ci], fd[co, :, :, ci], mode="valid") for ci in range(cin))
+            per_filter.append(acc[::sh, ::sw])
+        outs.append(np.stack(per_filter, axis=-1))
+    y = np.stack(outs)
+    return y + (0 if bias is None else bias.astype(np.float64))
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_convolution(case):
+    n, h, w, cin, cout, fh, fw, ph, pw, sh, sw, dh, dw = case
+    g = rng(10 + h * w)
+    x = g.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    f = g.normal(0, 1, (cout, fh, fw, cin)).astype(np.float32)
+    bias = g.uniform(-1, 1, cout).astype(np.float32)
+    y = orc.conv(x, f, bias, ph, pw, sh, sw, dh, dw)
+    assert_close(y, conv_via_scipy(x, f, bias, ph, pw, sh, sw, dh, dw), "conv %s" % (case,))
+    y0 = orc.conv(x, f, None, ph, pw, sh, sw, dh, dw)
+    assert_close(y0, y - bias, "conv without free term", atol=1e-4)
+    if nhtest.have_reference():
+        assert_close(ref().conv(x, f, bias, ph, pw, sh, sw, dh, dw), y, "conv vs reference %s" % (case,))
+        assert_close(ref().conv(x, f, None, ph, pw, sh, sw, dh, dw), y0, "conv vs reference, no free term")
+
+
+def test_convolution_1x1_is_a_matrix_product():
+    g = rng(11)
+    x = g.uniform(-1, 1, (2, 4, 5, 6)).astype(np.float32)
+    f = g.normal(0, 1, (7, 1, 1, 6)).astype(np.float32)
+    y = orc.conv(x, f, None, 0, 0, 1, 1)
+    assert_close(y.reshape(-1, 7), x.reshape(-1, 6).astype(np.float64) @ f.reshape(7, 6).astype(np.float64).T, "1x1")
+
+
+CHANNELWISE_CASES = [
+    # n, h, w, c, fh, fw, ph, pw, sh, sw
+    (1, 3, 3, 1, 3, 3, 1, 1, 1, 1), (2, 8, 9, 16, 3, 3, 1, 1, 1, 1), (2, 8, 9, 16, 3, 3, 1, 1, 2, 2),
+    (1, 7, 7, 5, 3, 3, 0, 0, 1, 1), (1, 10, 12, 12, 5, 5, 2, 2, 1, 1), (3, 9, 6, 7, 2, 3, 1, 2, 2, 1),
+]
+
+
+@pytest.mark.parametrize("case", CHANNELWISE_CASES)
+def test_channelwise_convolution(case):
+    n, h, w, c, fh, fw, ph, pw, sh, sw = case
+    g = rng(12 + c)
+    x = g.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    f = g.normal(0, 1, (fh, fw, c)).astype(np.float32)
+    bias = g.uniform(-1, 1, c).astype(np.float32)
+    y = orc.channelwise_conv(x, f, bias, ph, pw, sh, sw)
+    # every channel is an independent single-channel convolution
+    for ch in range(c):
+        want = conv_via_scipy(x[..., ch:ch + 1], f[None, :, :, ch:ch + 1], bias[ch:ch + 1], ph, pw, sh, sw, 1, 1)
+        assert_close(y[..., ch:ch + 1], want, "channelwise %s ch %d" % (case, ch))
+    if nhtest.have_reference():
+        assert_close(ref().channelwise_conv(x, f, bias, ph, pw, sh, sw), y, "channelwise vs reference")
+        assert_close(ref().channelwise_conv(x, f, None, ph, pw, sh, sw), orc.channelwise_conv(x, f, None, ph, pw, sh, sw), "no ft")
+
+
+# ---------------------------------------------------------------------------------------------------------
+# pooling
+
+POOL_CASES = [(1, 2, 2, 1, 2, 2, 2, 2), (2, 9, 11, 5, 3, 3, 2, 2), (1, 8, 8, 16, 2, 2, 2, 2), (2, 7, 10, 3, 3, 2, 1, 3),
+              (1, 6, 6, 4, 6, 6, 1, 1), (1, 12, 5, 8, 2, 1, 2, 1)]
+
+
+def windows(x, fh, fw, sh, sw):
+    n, h, w, c = x.shape
+    ho, wo = (h - fh) // sh + 1, (w - fw) // sw + 1
+    out = np.empty((n, ho, wo, fh, fw, c), x.dtype)
+    for y in range(ho):
+        for z in range(wo):
+            out[:, y, z] = x[:, y * sh:y * sh + fh, z * sw:z * sw + fw, :]
+    return out
+
+
+@pytest.mark.parametrize("case", POOL_CASES)
+def test_pooling(case):
+    n, h, w, c, fh, fw, sh, sw = case
+    g = rng(13 + h)
+    x = g.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    win = windows(x, fh, fw, sh, sw)
+    y = orc.max_pool(x, fh, fw, sh, sw)
+    assert np.array_equal(y, win.max(axis=(3, 4)))
+    assert_close(orc.mean_pool(x, fh, fw, sh, sw), win.astype(np.float64).mean(axis=(3, 4)), "mean")
+    yi, idx = orc.max_pool(x, fh, fw, sh, sw, with_indices=True)
+    assert np.array_equal(yi, y)
+    if nhtest.have_reference():
+        assert np.array_equal(ref().max_pool(x, fh, fw, sh, sw), y)
+        assert_close(ref().mean_pool(x, fh, fw, sh, sw), orc.mean_pool(x, fh, fw, sh, sw), "mean vs reference")
+        ry, ridx = ref().max_pool(x, fh, fw, sh, sw, with_indices=True)
+        assert np.array_equal(ry, y)
+        assert np.array_equal(ridx, idx), "max-pool indices differ from the reference engine"
+
+
+def test_max_pool_index_first_window_points_at_the_maximum():
+    # for the first window of every strip (window column 0) the reference's index is the true arg-max position
+    g = rng(14)
+    x = g.permutation(2 * 6 * 4 * 3).reshape(2, 6, 4, 3).astype(np.float32)
+    y, idx = orc.max_pool(x, 2, 2, 2, 2, with_indices=True)
+    flat = x.reshape(2, -1)
+    for b in range(2):
+        for r in range(y.shape[1]):
+            for ch in range(3):
+                assert flat[b, idx[b, r, 0, ch]] == y[b, r, 0, ch]
+
+
+@needs_ref
+def test_max_pool_index_ties_match_reference():
+    # all-zero windows (common after ReLU) and repeated values
+    g = rng(15)
+    x = np.maximum(g.uniform(-1, 0.3, (2, 8, 8, 4)), 0).astype(np.float32)
+    x = np.round(x * 4) / 4
+    for fh, fw, sh, sw in ((2, 2, 2, 2), (3, 3, 2, 2), (3, 3, 1, 1)):
+        y, idx = orc.max_pool(x, fh, fw, sh, sw, with_indices=True)
+        ry, ridx = ref().max_pool(x, fh, fw, sh, sw, with_indices=True)
+        assert np.array_equal(y, ry) and np.array_equal(idx, ridx)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# data movement
+
+def test_resize_image():
+    g = rng(16)
+    x = g.uniform(-1, 1, (2, 5, 6, 3)).astype(np.float32)
+    modes = {0: "constant", 1: "edge", 2: "reflect"}
+    for dl, dr, dt, db in ((1, 1, 1, 1), (2, 0, 0, 3), (0, 0, 0, 0), (3, 2, 1, 4)):
+        for mode, name in modes.items():
+            y = orc.resize_image(x, dl, dr, dt, db, mode, 0.5)
+            kw = {"constant_values": 0.5} if mode == 0 else {}
+            want = np.pad(x, ((0, 0), (dt, db), (dl, dr), (0, 0)), mode=name, **kw)
+            assert np.array_equal(y, want), (dl, dr, dt, db, name)
+            if nhtest.have_reference():
+                assert np.array_equal(ref().resize_image(x, dl, dr, dt, db, mode, 0.5), y), (dl, dr, dt, db, name)
+    # negative deltas crop; mixed crop and pad
+    for dl, dr, dt, db in ((-1, -2, -1, 0), (-1, 2, 1, -2)):
+        y = orc.resize_image(x, dl, dr, dt, db, 0, -1.0)
+        cropped = x[:, max(0, -dt):x.shape[1] - max(0, -db), max(0, -dl):x.shape[2] - max(0, -dr), :]
+        want = np.pad(cropped, ((0, 0), (max(dt, 0), max(db, 0)), (max(dl, 0), max(dr, 0)), (0, 0)), constant_values=-1.0)
+        assert np.array_equal(y, want)
+        if nhtest.have_reference():
+            assert np.array_equal(ref().resize_image(x, dl, dr, dt, db, 0, -1.0), y)
+
+
+def test_split_and_merge():
+    g = rng(17)
+    big = g.uniform(-1, 1, (2, 3, 1, 4, 5, 1, 12)).astype(np.float32)
+    for dim, sizes in ((6, (4, 8)), (6, (3, 4, 5)), (4, (2, 3)), (3, (1, 3)), (0, (1, 1)), (1, (2, 1))):
+        part_dims = []
+        for s in sizes:
+            d = list(big.shape)
+            d[dim] = s
+            part_dims.append(tuple(d))
+        parts = orc.split(big, dim, part_dims)
+        want = np.split(big, np.cumsum(sizes)[:-1], axis=dim)
+        for p, wnt in zip(parts, want):
+            assert np.array_equal(p, wnt), (dim, sizes)
+        assert np.array_equal(orc.merge(parts, dim, big.shape), big)
+        if nhtest.have_reference():
+            for p, q in zip(ref().split(big, dim, part_dims), parts):
+                assert np.array_equal(p, q)
+            assert np.array_equal(ref().merge(parts, dim, big.shape), big)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# LSTM and CTC
+
+def lstm_numpy(w_in, b_in, w_rec, b_rec, x, reverse, c0, h0):
+    T, B, In = x.shape
+    H = w_rec.shape[1]
+    c = np.zeros((B, H)) if c0 is None else c0.astype(np.float64)
+    h = np.zeros((B, H)) if h0 is None else h0.astype(np.float64)
+    hs, cs = np.zeros((T, B, H)), np.zeros((T, B, H))
+    bias = (0 if b_in is None else b_in.astype(np.float64)) + (0 if b_rec is None else b_rec.astype(np.float64))
+    for i in range(T):
+        t = T - 1 - i if reverse else i
+        g = x[t].astype(np.float64) @ w_in.astype(np.float64).T + h @ w_rec.astype(np.float64).T + bias
+        a, f, inp, o = g[:, :H], g[:, H:2 * H], g[:, 2 * H:3 * H], g[:, 3 * H:]
+        c = scipy.special.expit(f) * c + scipy.special.expit(inp) * np.tanh(a)
+        h = scipy.special.expit(o) * np.tanh(c)
+        hs[t], cs[t] = h, c
+    return hs, cs
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+@pytest.mark.parametrize("with_init", [False, True])
+def test_lstm(reverse, with_init):
+    g = rng(18)
+    T, B, In, H = 5, 3, 6, 4
+    w_in = g.uniform(-0.5, 0.5, (4 * H, In)).astype(np.float32)
+    w_rec = g.uniform(-0.5, 0.5, (4 * H, H)).astype(np.float32)
+    b_in = g.uniform(-0.5, 0.5, 4 * H).astype(np.float32)
+    b_rec = g.uniform(-0.5, 0.5, 4 * H).astype(np.float32)
+    x = g.uniform(-1, 1, (T, B, In)).astype(np.float32)
+    c0 = g.uniform(-1, 1, (B, H)).astype(np.float32) if with_init else None
+    h0 = g.uniform(-1, 1, (B, H)).astype(np.float32) if with_init else None
+    for bi, br in ((b_in, b_rec), (b_in, None), (None, None)):
+        h, c = orc.lstm(w_in, bi, w_rec, br, x, reverse, c0, h0)
+        wh, wc = lstm_numpy(w_in, bi, w_rec, br, x, reverse, c0, h0)
+        assert_close(h, wh, "lstm h")
+        assert_close(c, wc, "lstm c")
+        if nhtest.have_reference():
+            rh, rc = ref().lstm(w_in, bi, w_rec, br, x, reverse, c0, h0)
+            assert_close(rh, h, "lstm h vs reference")
+            assert_close(rc, c, "lstm c vs reference")
+            rh2, _ = ref().lstm(w_in, bi, w_rec, br, x, reverse, c0, h0, want_state=False)
+            assert_close(rh2, h, "lstm h vs reference without state output")
+
+
+def test_ctc_greedy_collapse():
+    labels = np.array([[0, 0, 5, 1, 1, 5, 1, 2, 2, 5], [5, 5, 5, 5, 5, 5, 5, 5, 5, 5], [3, 5, 3, 3, 5, 5, 4, 4, 4, 0]], np.int32)
+    got = nhtest.ctc_greedy_collapse(labels, blank=5)
+    assert got == [[0, 1, 1, 2], [], [3, 3, 4, 0]]
+    assert nhtest.ctc_greedy_collapse(labels, blank=5, seq_len=[3, 10, 4]) == [[0], [], [3, 3]]
+    # brute force: itertools.groupby then drop blanks
+    import itertools
+    g = rng(19)
+    rnd = g.integers(0, 4, (6, 40)).astype(np.int32)
+    want = [[k for k, _ in itertools.groupby(row.tolist()) if k != 3] for row in rnd]
+    assert nhtest.ctc_greedy_collapse(rnd, blank=3) == want
