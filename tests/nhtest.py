@@ -380,3 +380,335 @@ def assert_close(actual, expected, what="", rtol=RTOL, atol=ATOL):
         i = np.unravel_index(np.argmax(np.where(bad, err - bound, -np.inf)), err.shape)
         raise AssertionError("%s: %d of %d elements outside rtol=%g atol=%g; worst at %s: got %r expected %r" % (
             what, int(bad.sum()), bad.size, rtol, atol, i, actual[i], expected[i]))
+
+
+# ---------------------------------------------------------------------------------------------------------
+# device side: the same front-end, through the C ABI of libneoml_hip.so on torch-owned device memory
+
+class Hip:
+    """Calls the HIP library through its C ABI. Inputs are numpy arrays; they are uploaded into torch CUDA
+    tensors (plumbing only), the kernel runs on torch's current stream, and the result comes back as numpy."""
+
+    def __init__(self):
+        import torch
+        import neoml_amd
+        self.torch = torch
+        self.na = neoml_amd
+        self.lib = neoml_amd.load()
+        assert torch.cuda.is_available(), "no GPU"
+        self.dev = torch.device("cuda:0")
+
+    # -- plumbing
+    def stream(self):
+        return ctypes.c_void_p(self.torch.cuda.current_stream().cuda_stream)
+
+    def up(self, a):
+        if a is None:
+            return None
+        return self.torch.from_numpy(np.ascontiguousarray(a)).to(self.dev)
+
+    def empty(self, shape, dtype=np.float32):
+        t = self.torch.float32 if dtype == np.float32 else self.torch.int32
+        return self.torch.empty(tuple(int(s) for s in shape), dtype=t, device=self.dev)
+
+    @staticmethod
+    def p(t):
+        return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+    def scalar(self, v, dtype=np.float32):
+        return self.up(np.array([v], dtype=dtype))
+
+    def call(self, name, *args):
+        self.na.check(getattr(self.lib, name)(self.stream(), *args))
+
+    @staticmethod
+    def down(t):
+        return t.cpu().numpy()
+
+    # -- element-wise
+    UNARY_FN = {
+        "relu": ("nhVectorReLU", 1), "elu": ("nhVectorELU", 1), "leaky_relu": ("nhVectorLeakyReLU", 1),
+        "hswish": ("nhVectorHSwish", 0), "abs": ("nhVectorAbs", 0), "hard_tanh": ("nhVectorHardTanh", 0),
+        "hard_sigmoid": ("nhVectorHardSigmoid", 2), "neg": ("nhVectorNeg", 0), "exp": ("nhVectorExp", 0),
+        "log": ("nhVectorLog", 0), "erf": ("nhVectorErf", 0), "sqrt": ("nhVectorSqrt", 0), "inv": ("nhVectorInv", 0),
+        "minmax": ("nhVectorMinMax", 2), "sigmoid": ("nhVectorSigmoid", 0), "tanh": ("nhVectorTanh", 0),
+        "add_value": ("nhVectorAddValue", 1), "multiply": ("nhVectorMultiply", 1),
+        "neg_multiply": ("nhVectorNegMultiply", 1),
+    }
+
+    def unary(self, op, x, p0=0.0, p1=0.0, inplace=False, offset=0):
+        """offset > 0 runs on a view that starts `offset` elements into a buffer (unaligned pointers)."""
+        x = f32(x).ravel()
+        n = x.size
+        buf = self.empty((n + offset,))
+        buf[offset:] = self.up(x)
+        src = buf[offset:]
+        if inplace:
+            dst = src
+        else:
+            dbuf = self.empty((n + offset,))
+            dst = dbuf[offset:]
+        if op == "copy":
+            self.call("nhVectorCopy", self.p(dst), self.p(src), n)
+            return self.down(dst)
+        fn, nscalars = self.UNARY_FN[op]
+        scalars = [self.scalar(p0), self.scalar(p1)][:nscalars]
+        self.call(fn, self.p(src), self.p(dst), n, *[self.p(s) for s in scalars])
+        return self.down(dst)
+
+    BINARY_FN = {
+        "add": "nhVectorAdd", "sub": "nhVectorSub", "eltwise_multiply": "nhVectorEltwiseMultiply",
+        "eltwise_neg_multiply": "nhVectorEltwiseNegMultiply", "eltwise_divide": "nhVectorEltwiseDivide",
+        "eltwise_max": "nhVectorEltwiseMax", "eltwise_min": "nhVectorEltwiseMin",
+        "multiply_and_add": "nhVectorMultiplyAndAdd", "multiply_and_sub": "nhVectorMultiplyAndSub",
+        "eltwise_multiply_add": "nhVectorEltwiseMultiplyAdd",
+    }
+
+    def binary(self, op, a, b, p0=0.0, result=None, inplace_first=False):
+        a, b = self.up(f32(a).ravel()), self.up(f32(b).ravel())
+        n = a.numel()
+        out = a if inplace_first else (self.empty((n,)) if result is None else self.up(f32(result).ravel()))
+        args = [self.p(a), self.p(b), self.p(out), n]
+        if op in ("multiply_and_add", "multiply_and_sub"):
+            s = self.scalar(p0)
+            args.append(self.p(s))
+        self.call(self.BINARY_FN[op], *args)
+        return self.down(out)
+
+    def binary_int(self, op, a, b):
+        fn = {"add": "nhVectorAddInt", "sub": "nhVectorSubInt", "multiply": "nhVectorEltwiseMultiplyInt"}[op]
+        a, b = self.up(i32(a).ravel()), self.up(i32(b).ravel())
+        out = self.empty((a.numel(),), np.int32)
+        self.call(fn, self.p(a), self.p(b), self.p(out), a.numel())
+        return self.down(out)
+
+    def float_to_int(self, x):
+        x = self.up(f32(x).ravel())
+        out = self.empty((x.numel(),), np.int32)
+        self.call("nhVectorConvertFloatToInt", self.p(x), self.p(out), x.numel())
+        return self.down(out)
+
+    def int_to_float(self, x):
+        x = self.up(i32(x).ravel())
+        out = self.empty((x.numel(),))
+        self.call("nhVectorConvertIntToFloat", self.p(x), self.p(out), x.numel())
+        return self.down(out)
+
+    def fill(self, n, value, from_handle=False, integer=False):
+        out = self.empty((n,), np.int32 if integer else np.float32)
+        if from_handle:
+            s = self.scalar(value, np.int32 if integer else np.float32)
+            self.call("nhVectorFillFromHandleInt" if integer else "nhVectorFillFromHandle", self.p(out), n, self.p(s))
+        elif integer:
+            self.call("nhVectorFillInt", self.p(out), int(value), n)
+        else:
+            self.call("nhVectorFill", self.p(out), ctypes.c_float(value), n)
+        return self.down(out)
+
+    def vector_sum(self, x):
+        x = self.up(f32(x).ravel())
+        out = self.empty((1,))
+        self.call("nhVectorSum", self.p(x), x.numel(), self.p(out))
+        return self.down(out)[0]
+
+    def dot(self, a, b):
+        a, b = self.up(f32(a).ravel()), self.up(f32(b).ravel())
+        out = self.empty((1,))
+        self.call("nhVectorDotProduct", self.p(a), self.p(b), a.numel(), self.p(out))
+        return self.down(out)[0]
+
+    # -- broadcasts, reductions
+    def set_vector_to_matrix_rows(self, h, w, vec):
+        v = self.up(f32(vec))
+        out = self.empty((h, w))
+        self.call("nhSetVectorToMatrixRows", self.p(out), h, w, self.p(v))
+        return self.down(out)
+
+    def add_vector_to_matrix_rows(self, m, vec, inplace=False):
+        m, v = self.up(f32(m)), self.up(f32(vec))
+        b, h, w = m.shape
+        out = m if inplace else self.empty(m.shape)
+        self.call("nhAddVectorToMatrixRows", b, self.p(m), self.p(out), h, w, self.p(v))
+        return self.down(out)
+
+    def add_vector_to_matrix_columns(self, m, vec, sign=1):
+        m, v = self.up(f32(m)), self.up(f32(vec))
+        h, w = m.shape
+        out = self.empty(m.shape)
+        self.call("nhAddVectorToMatrixColumns" if sign > 0 else "nhSubVectorFromMatrixColumns",
+                  self.p(m), self.p(out), h, w, self.p(v))
+        return self.down(out)
+
+    def sum_matrix_rows(self, m, add_to=None):
+        m = self.up(f32(m))
+        b, h, w = m.shape
+        out = self.empty((b, w)) if add_to is None else self.up(f32(add_to))
+        self.call("nhSumMatrixRows" if add_to is None else "nhSumMatrixRowsAdd", b, self.p(out), self.p(m), h, w)
+        return self.down(out)
+
+    def sum_matrix_columns(self, m):
+        m = self.up(f32(m))
+        out = self.empty((m.shape[0],))
+        self.call("nhSumMatrixColumns", self.p(out), self.p(m), m.shape[0], m.shape[1])
+        return self.down(out)
+
+    def multiply_diag_matrix_by_matrix(self, d, m):
+        d, m = self.up(f32(d)), self.up(f32(m))
+        out = self.empty(m.shape)
+        self.call("nhMultiplyDiagMatrixByMatrix", self.p(d), m.shape[0], self.p(m), m.shape[1], self.p(out), m.numel())
+        return self.down(out)
+
+    def batch_multiply_matrix_by_diag_matrix(self, batch, first, h, w, first_off, second, second_off):
+        a, b = self.up(f32(first).ravel()), self.up(f32(second).ravel())
+        out = self.empty((batch, h, w))
+        self.call("nhBatchMultiplyMatrixByDiagMatrix", batch, self.p(a), h, w, first_off, self.p(b), second_off,
+                  self.p(out), out.numel())
+        return self.down(out)
+
+    def softmax_rows(self, m, inplace=False):
+        m = self.up(f32(m))
+        out = m if inplace else self.empty(m.shape)
+        self.call("nhMatrixSoftmaxByRows", self.p(m), m.shape[0], m.shape[1], self.p(out))
+        return self.down(out)
+
+    def log_sum_exp_rows(self, m):
+        m = self.up(f32(m))
+        out = self.empty((m.shape[0],))
+        self.call("nhMatrixLogSumExpByRows", self.p(m), m.shape[0], m.shape[1], self.p(out), m.shape[0])
+        return self.down(out)
+
+    def find_max_in_rows(self, m, with_indices=True):
+        m = self.up(f32(m))
+        v = self.empty((m.shape[0],))
+        idx = self.empty((m.shape[0],), np.int32) if with_indices else None
+        self.call("nhFindMaxValueInRows", self.p(m), m.shape[0], m.shape[1], self.p(v), self.p(idx), m.shape[0])
+        return self.down(v), (self.down(idx) if with_indices else None)
+
+    def find_max_in_columns(self, m):
+        m = self.up(f32(m))
+        b, h, w = m.shape
+        v, idx = self.empty((b, w)), self.empty((b, w), np.int32)
+        self.call("nhFindMaxValueInColumns", b, self.p(m), h, w, self.p(v), self.p(idx), b * w)
+        return self.down(v), self.down(idx)
+
+    def transpose(self, x, integer=False):
+        x = self.up(i32(x) if integer else f32(x))
+        b, h, m, w, c = x.shape
+        out = self.empty((b, w, m, h, c), np.int32 if integer else np.float32)
+        self.call("nhTransposeMatrixInt" if integer else "nhTransposeMatrix", b, self.p(x), h, m, w, c, self.p(out), out.numel())
+        return self.down(out)
+
+    # -- matrix products
+    def matmul(self, kind, a, b, c=None, lda=None, ldb=None, ldc=None, M=None, N=None, K=None, batch=1):
+        a, b = self.up(f32(a).ravel()), self.up(f32(b).ravel())
+        if kind == "nt":
+            out = self.torch.zeros(((M - 1) * ldc + N,), dtype=self.torch.float32, device=self.dev)
+            self.call("nhMultiplyMatrixByTransposedMatrix", self.p(a), M, K, lda, self.p(b), N, ldb, self.p(out), ldc, out.numel())
+            return self.down(out)
+        if kind == "tn_add":
+            out = self.up(f32(c).ravel())
+            self.call("nhMultiplyTransposedMatrixByMatrixAndAdd", self.p(a), K, M, lda, self.p(b), N, ldb, self.p(out), ldc, out.numel())
+            return self.down(out)
+        out = self.empty((batch, M, N))
+        if kind == "bnt":
+            self.call("nhBatchMultiplyMatrixByTransposedMatrix", batch, self.p(a), M, K, self.p(b), N, self.p(out), out.numel())
+        elif kind == "bnn":
+            self.call("nhBatchMultiplyMatrixByMatrix", batch, self.p(a), M, K, self.p(b), N, self.p(out), out.numel())
+        else:
+            self.call("nhBatchMultiplyTransposedMatrixByMatrix", batch, self.p(a), K, M, self.p(b), N, self.p(out), out.numel())
+        return self.down(out)
+
+    # -- convolution, pooling
+    def conv_desc(self, n, h, w, cin, cout, fh, fw, ph, pw, sh, sw, dh=1, dw=1, channelwise=False):
+        d = self.na.ConvDesc(n, h, w, cin, cout, fh, fw, ph, pw, sh, sw, dh, dw, 0, 0)
+        fn = self.lib.nhInitBlobChannelwiseConvolution if channelwise else self.lib.nhInitBlobConvolution
+        self.na.check(fn(ctypes.byref(d)))
+        return d
+
+    def conv(self, x, filt, bias, ph, pw, sh, sw, dh=1, dw=1):
+        x, filt = f32(x), f32(filt)
+        n, h, w, cin = x.shape
+        cout, fh, fw, _ = filt.shape
+        d = self.conv_desc(n, h, w, cin, cout, fh, fw, ph, pw, sh, sw, dh, dw)
+        xs, fs, bs = self.up(x), self.up(filt), self.up(None if bias is None else f32(bias))
+        out = self.empty((n, d.resultHeight, d.resultWidth, cout))
+        self.call("nhBlobConvolution", ctypes.byref(d), self.p(xs), self.p(fs), self.p(bs), self.p(out))
+        return self.down(out)
+
+    def channelwise_conv(self, x, filt, bias, ph, pw, sh, sw):
+        x, filt = f32(x), f32(filt)
+        n, h, w, c = x.shape
+        fh, fw, _ = filt.shape
+        d = self.conv_desc(n, h, w, c, c, fh, fw, ph, pw, sh, sw, channelwise=True)
+        xs, fs, bs = self.up(x), self.up(filt), self.up(None if bias is None else f32(bias))
+        out = self.empty((n, d.resultHeight, d.resultWidth, c))
+        self.call("nhBlobChannelwiseConvolution", ctypes.byref(d), self.p(xs), self.p(fs), self.p(bs), self.p(out))
+        return self.down(out)
+
+    def pool_desc(self, n, h, w, c, fh, fw, sh, sw):
+        d = self.na.PoolingDesc(n, h, w, c, fh, fw, sh, sw, 0, 0)
+        self.na.check(self.lib.nhInitPooling(ctypes.byref(d)))
+        return d
+
+    def max_pool(self, x, fh, fw, sh, sw, with_indices=False):
+        x = f32(x)
+        n, h, w, c = x.shape
+        d = self.pool_desc(n, h, w, c, fh, fw, sh, sw)
+        xs = self.up(x)
+        out = self.empty((n, d.resultHeight, d.resultWidth, c))
+        idx = self.empty(out.shape, np.int32) if with_indices else None
+        self.call("nhBlobMaxPooling", ctypes.byref(d), self.p(xs), self.p(idx), self.p(out))
+        return (self.down(out), self.down(idx)) if with_indices else self.down(out)
+
+    def mean_pool(self, x, fh, fw, sh, sw):
+        x = f32(x)
+        n, h, w, c = x.shape
+        d = self.pool_desc(n, h, w, c, fh, fw, sh, sw)
+        xs = self.up(x)
+        out = self.empty((n, d.resultHeight, d.resultWidth, c))
+        self.call("nhBlobMeanPooling", ctypes.byref(d), self.p(xs), self.p(out))
+        return self.down(out)
+
+    def resize_image(self, x, dl, dr, dt, db, padding=0, value=0.0):
+        x = f32(x)
+        n, h, w, c = x.shape
+        fd = self.na.BlobDesc.of(1, n, 1, h, w, 1, c)
+        td = self.na.BlobDesc.of(1, n, 1, h + dt + db, w + dl + dr, 1, c)
+        xs = self.up(x)
+        out = self.empty((n, h + dt + db, w + dl + dr, c))
+        self.call("nhBlobResizeImage", ctypes.byref(fd), self.p(xs), dl, dr, dt, db, padding, ctypes.c_float(value),
+                  ctypes.byref(td), self.p(out))
+        return self.down(out)
+
+    def split(self, big, dim, part_dims):
+        big = f32(big)
+        bs = self.up(big)
+        parts = [self.empty(d) for d in part_dims]
+        descs = (self.na.BlobDesc * len(parts))(*[self.na.BlobDesc.of(*d) for d in part_dims])
+        ptrs = (ctypes.c_void_p * len(parts))(*[p.data_ptr() for p in parts])
+        bd = self.na.BlobDesc.of(*big.shape)
+        self.call("nhBlobSplitByDim", dim, ctypes.byref(bd), self.p(bs), descs, ptrs, len(parts))
+        return [self.down(p) for p in parts]
+
+    def merge(self, parts, dim, big_dims):
+        ps = [self.up(f32(p)) for p in parts]
+        descs = (self.na.BlobDesc * len(ps))(*[self.na.BlobDesc.of(*p.shape) for p in parts])
+        ptrs = (ctypes.c_void_p * len(ps))(*[p.data_ptr() for p in ps])
+        out = self.empty(big_dims)
+        bd = self.na.BlobDesc.of(*big_dims)
+        self.call("nhBlobMergeByDim", dim, descs, ptrs, len(ps), ctypes.byref(bd), self.p(out))
+        return self.down(out)
+
+    def lstm(self, w_in, b_in, w_rec, b_rec, x, reverse=False, c0=None, h0=None, want_state=True):
+        x = f32(x)
+        T, B, In = x.shape
+        H = w_rec.shape[1]
+        ws = [self.up(None if a is None else f32(a)) for a in (w_in, b_in, w_rec, b_rec, c0, h0, x)]
+        h = self.empty((T, B, H))
+        c = self.empty((T, B, H)) if want_state else None
+        size = ctypes.c_size_t(0)
+        self.na.check(self.lib.nhLstmWorkspaceSize(H, In, T, B, ctypes.byref(size)))
+        work = self.torch.empty((size.value + 15) // 4, dtype=self.torch.float32, device=self.dev)
+        self.call("nhLstm", H, In, self.p(ws[0]), self.p(ws[1]), self.p(ws[2]), self.p(ws[3]), 1 if reverse else 0, T, B,
+                  self.p(ws[4]), self.p(ws[5]), self.p(ws[6]), self.p(c), self.p(h), self.p(work), size.value)
+        return self.down(h), (self.down(c) if want_state else None)

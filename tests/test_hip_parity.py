@@ -1,0 +1,389 @@
+"""Parity of the HIP kernels (through the C ABI of libneoml_hip.so) with the CPU oracle.
+
+Bar: int / index results bit-exact; fp32 within |a - b| <= 1e-5 + 1e-4 * |b| (nhtest.ATOL / nhtest.RTOL).
+Where oracle/_ref is present, the reference's own CPU engine is compared as well.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+import nhtest
+from nhtest import Cpu, assert_close
+from test_oracle import (UNARY_CASES, BINARY_CASES, CONV_CASES, CHANNELWISE_CASES, POOL_CASES, unary_input, rng)
+
+pytestmark = pytest.mark.gpu
+
+orc = Cpu("orc")
+_hip = None
+
+
+def hip():
+    global _hip
+    if _hip is None:
+        _hip = nhtest.Hip()
+    return _hip
+
+
+def ref_or_none():
+    return Cpu("ref") if nhtest.have_reference() else None
+
+
+# ---------------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("op,p0,p1", UNARY_CASES)
+def test_unary(op, p0, p1):
+    for n, offset, inplace in ((1, 0, False), (3, 0, False), (1003, 0, False), (4096, 0, True), (70001, 1, False),
+                               (1 << 20, 0, False)):
+        x = unary_input(op, max(n, 8), n)[:n]
+        want = orc.unary(op, x, p0, p1)
+        got = hip().unary(op, x, p0, p1, inplace=inplace, offset=offset)
+        assert_close(got, want, "%s n=%d offset=%d inplace=%s" % (op, n, offset, inplace))
+    r = ref_or_none()
+    if r is not None:
+        x = unary_input(op, 1003, 5)
+        assert_close(hip().unary(op, x, p0, p1), r.unary(op, x, p0, p1), op + " vs reference")
+
+
+def test_relu_nan_and_threshold():
+    x = np.array([np.nan, -1.0, 0.5, 7.0, np.inf, -np.inf, 6.0, 0.0], np.float32)
+    assert np.array_equal(hip().unary("relu", x, 0.0), np.array([0, 0, 0.5, 7, np.inf, 0, 6, 0], np.float32))
+    assert np.array_equal(hip().unary("relu", x, 6.0), np.array([0, 0, 0.5, 6, 6, 0, 6, 0], np.float32))
+
+
+@pytest.mark.parametrize("op", BINARY_CASES)
+def test_binary(op):
+    g = rng(2)
+    for n in (1, 5, 1000, 300003):
+        a = g.uniform(-10, 10, n).astype(np.float32)
+        b = g.uniform(0.5, 10, n).astype(np.float32) * np.where(g.random(n) < 0.5, -1, 1).astype(np.float32)
+        r = g.uniform(-10, 10, n).astype(np.float32)
+        want = orc.binary(op, a, b, 0.37, result=r)
+        assert_close(hip().binary(op, a, b, 0.37, result=r), want, "%s n=%d" % (op, n))
+    if op == "add":  # residual connections write into their first operand
+        assert_close(hip().binary(op, a, b, inplace_first=True), a + b, "add in place")
+
+
+def test_int_ops_fill_convert():
+    g = rng(3)
+    a = g.integers(-1000, 1000, 100003).astype(np.int32)
+    b = g.integers(-1000, 1000, 100003).astype(np.int32)
+    for op in ("add", "sub", "multiply"):
+        assert np.array_equal(hip().binary_int(op, a, b), orc.binary_int(op, a, b))
+    x = g.uniform(-100, 100, 100003).astype(np.float32)
+    assert np.array_equal(hip().float_to_int(x), orc.float_to_int(x))
+    assert np.array_equal(hip().int_to_float(a), orc.int_to_float(a))
+    for n in (1, 7, 4099):
+        assert np.array_equal(hip().fill(n, 2.5), np.full(n, 2.5, np.float32))
+        assert np.array_equal(hip().fill(n, -3, integer=True), np.full(n, -3, np.int32))
+        assert np.array_equal(hip().fill(n, 1.5, from_handle=True), np.full(n, 1.5, np.float32))
+        assert np.array_equal(hip().fill(n, 9, from_handle=True, integer=True), np.full(n, 9, np.int32))
+
+
+def test_sum_and_dot():
+    g = rng(4)
+    for n in (1, 1000, 1 << 20):
+        a = g.uniform(-1, 1, n).astype(np.float32)
+        b = g.uniform(-1, 1, n).astype(np.float32)
+        assert_close(hip().vector_sum(a), orc.vector_sum(a), "sum", atol=1e-2 if n > 1000 else 1e-4)
+        assert_close(hip().dot(a, b), orc.dot(a, b), "dot", atol=1e-2 if n > 1000 else 1e-4)
+
+
+def test_broadcasts_and_sums():
+    g = rng(5)
+    for b, h, w in ((1, 1, 1), (2, 3, 5), (3, 17, 64), (1, 40, 7), (2, 300, 512), (1, 4096, 12), (64, 49, 512)):
+        m = g.uniform(-10, 10, (b, h, w)).astype(np.float32)
+        v = g.uniform(-10, 10, (b, w)).astype(np.float32)
+        col = g.uniform(-10, 10, h).astype(np.float32)
+        tag = str((b, h, w))
+        assert_close(hip().add_vector_to_matrix_rows(m, v), orc.add_vector_to_matrix_rows(m, v), "add rows " + tag)
+        assert_close(hip().add_vector_to_matrix_rows(m, v, inplace=True), orc.add_vector_to_matrix_rows(m, v), "add rows in place")
+        assert_close(hip().set_vector_to_matrix_rows(h, w, v[0]), orc.set_vector_to_matrix_rows(h, w, v[0]), "set rows")
+        assert_close(hip().add_vector_to_matrix_columns(m[0], col), orc.add_vector_to_matrix_columns(m[0], col), "add cols")
+        assert_close(hip().add_vector_to_matrix_columns(m[0], col, -1), orc.add_vector_to_matrix_columns(m[0], col, -1), "sub cols")
+        assert_close(hip().sum_matrix_rows(m), orc.sum_matrix_rows(m), "sum rows " + tag, atol=1e-3)
+        assert_close(hip().sum_matrix_rows(m, add_to=v), orc.sum_matrix_rows(m, add_to=v), "sum rows add", atol=1e-3)
+        assert_close(hip().sum_matrix_columns(m[0]), orc.sum_matrix_columns(m[0]), "sum cols", atol=1e-3)
+        assert_close(hip().multiply_diag_matrix_by_matrix(col, m[0]), orc.multiply_diag_matrix_by_matrix(col, m[0]), "diag")
+        assert_close(hip().batch_multiply_matrix_by_diag_matrix(b, m, h, w, h * w, v, w),
+                     orc.batch_multiply_matrix_by_diag_matrix(b, m, h, w, h * w, v, w), "diag right")
+        assert_close(hip().batch_multiply_matrix_by_diag_matrix(b, m, h, w, h * w, v[0], 0),
+                     orc.batch_multiply_matrix_by_diag_matrix(b, m, h, w, h * w, v[0], 0), "diag right broadcast")
+
+
+def test_softmax_logsumexp():
+    g = rng(6)
+    for h, w in ((1, 1), (3, 2), (7, 64), (9, 101), (513, 256), (64, 1000), (5, 1500), (8192, 101)):
+        m = g.uniform(-10, 10, (h, w)).astype(np.float32)
+        assert_close(hip().softmax_rows(m), orc.softmax_rows(m), "softmax %s" % ((h, w),))
+        assert_close(hip().softmax_rows(m, inplace=True), orc.softmax_rows(m), "softmax in place")
+        assert_close(hip().log_sum_exp_rows(m), orc.log_sum_exp_rows(m), "logsumexp")
+
+
+def test_argmax_bit_exact():
+    g = rng(7)
+    for h, w in ((1, 1), (5, 3), (64, 101), (9, 257), (8192, 101), (3, 5000)):
+        m = g.permutation(h * w).reshape(h, w).astype(np.float32)  # tie-free
+        v, i = hip().find_max_in_rows(m)
+        ov, oi = orc.find_max_in_rows(m)
+        assert np.array_equal(i, oi) and np.array_equal(v, ov)
+        v2, _ = hip().find_max_in_rows(m, with_indices=False)
+        assert np.array_equal(v2, ov)
+    # ties take the first index, as the oracle (and the reference's own test) do
+    t = np.zeros((4, 300), np.float32)
+    t[1, 200] = t[1, 77] = 1.0
+    assert np.array_equal(hip().find_max_in_rows(t)[1], orc.find_max_in_rows(t)[1])
+    for b, h, w in ((1, 1, 1), (3, 17, 9), (2, 128, 300)):
+        m = g.permutation(b * h * w).reshape(b, h, w).astype(np.float32)
+        v, i = hip().find_max_in_columns(m)
+        ov, oi = orc.find_max_in_columns(m)
+        assert np.array_equal(i, oi) and np.array_equal(v, ov)
+
+
+def test_ctc_greedy_pipeline_bit_exact():
+    # softmax -> log -> arg-max -> collapse, as the decoding layer does (CtcLayer.cpp:205-226,342-369)
+    g = rng(20)
+    T, B, C = 32, 8, 101
+    logits = g.uniform(-5, 5, (B * T, C)).astype(np.float32)
+    h = hip()
+    p = h.softmax_rows(logits)
+    lp = h.unary("log", p)
+    _, labels = h.find_max_in_rows(lp.reshape(B * T, C))
+    _, want = orc.find_max_in_rows(orc.unary("log", orc.softmax_rows(logits)).reshape(B * T, C))
+    assert np.array_equal(labels, want)
+    assert nhtest.ctc_greedy_collapse(labels.reshape(B, T), blank=100) == nhtest.ctc_greedy_collapse(want.reshape(B, T), blank=100)
+
+
+def test_transpose():
+    g = rng(8)
+    for shape in ((1, 1, 1, 1, 1), (2, 3, 1, 5, 1), (2, 4, 3, 5, 2), (1, 1, 3, 4, 2), (3, 7, 1, 1, 4), (2, 16, 1, 8, 64),
+                  (2, 100, 1, 130, 1), (4, 256, 1, 8, 64), (2, 70, 2, 33, 3)):
+        x = g.uniform(-1, 1, shape).astype(np.float32)
+        assert np.array_equal(hip().transpose(x), orc.transpose(x)), shape
+    xi = g.integers(-5, 5, (2, 9, 2, 7, 3)).astype(np.int32)
+    assert np.array_equal(hip().transpose(xi, integer=True), np.transpose(xi, (0, 3, 2, 1, 4)))
+
+
+# ---------------------------------------------------------------------------------------------------------
+
+MATMUL_SHAPES = [(1, 1, 1), (3, 5, 7), (17, 33, 65), (64, 101, 48), (128, 128, 16), (129, 65, 17), (200, 300, 100),
+                 (64, 1000, 512), (256, 64, 576), (70, 31, 250)]
+
+
+@pytest.mark.parametrize("shape", MATMUL_SHAPES)
+def test_matmul_strided(shape):
+    M, N, K = shape
+    g = rng(9 + M)
+    for pad_a, pad_b, pad_c in ((0, 0, 0), (3, 2, 1), (4, 8, 4)):
+        a = g.uniform(-1, 1, (M, K + pad_a)).astype(np.float32)
+        b = g.uniform(-1, 1, (N, K + pad_b)).astype(np.float32)
+        kw = dict(lda=K + pad_a, ldb=K + pad_b, ldc=N + pad_c, M=M, N=N, K=K)
+        got, want = hip().matmul("nt", a, b, **kw), orc.matmul("nt", a, b, **kw)
+        assert_close(got, want, "nt %s pads %s" % (shape, (pad_a, pad_b, pad_c)))
+        at = g.uniform(-1, 1, (K, M + pad_a)).astype(np.float32)
+        bn = g.uniform(-1, 1, (K, N + pad_b)).astype(np.float32)
+        c0 = g.uniform(-1, 1, ((M - 1) * (N + pad_c) + N,)).astype(np.float32)
+        kw = dict(c=c0, lda=M + pad_a, ldb=N + pad_b, ldc=N + pad_c, M=M, N=N, K=K)
+        assert_close(hip().matmul("tn_add", at, bn, **kw), orc.matmul("tn_add", at, bn, **kw), "tn_add %s" % (shape,))
+
+
+@pytest.mark.parametrize("batch,M,N,K", [(1, 2, 3, 4), (3, 16, 8, 5), (4, 33, 17, 9), (8, 64, 64, 16), (6, 100, 64, 100),
+                                         (5, 64, 256, 64), (2, 130, 36, 72)])
+def test_matmul_batched(batch, M, N, K):
+    g = rng(30 + M)
+    a = g.uniform(-1, 1, (batch, M, K)).astype(np.float32)
+    bt = g.uniform(-1, 1, (batch, N, K)).astype(np.float32)
+    bn = g.uniform(-1, 1, (batch, K, N)).astype(np.float32)
+    at = g.uniform(-1, 1, (batch, K, M)).astype(np.float32)
+    for kind, x, y in (("bnt", a, bt), ("bnn", a, bn), ("btn", at, bn)):
+        kw = dict(M=M, N=N, K=K, batch=batch)
+        assert_close(hip().matmul(kind, x, y, **kw), orc.matmul(kind, x, y, **kw), "%s %s" % (kind, (batch, M, N, K)))
+
+
+def test_matmul_vs_reference_engine():
+    r = ref_or_none()
+    if r is None:
+        pytest.skip("oracle/_ref is not built")
+    g = rng(31)
+    M, N, K = 300, 200, 160
+    a = g.uniform(-1, 1, (M, K)).astype(np.float32)
+    b = g.uniform(-1, 1, (N, K)).astype(np.float32)
+    kw = dict(lda=K, ldb=K, ldc=N, M=M, N=N, K=K)
+    assert_close(hip().matmul("nt", a, b, **kw), r.matmul("nt", a, b, **kw), "nt vs reference")
+
+
+# ---------------------------------------------------------------------------------------------------------
+
+GPU_CONV_CASES = CONV_CASES + [
+    (2, 16, 16, 64, 64, 3, 3, 1, 1, 1, 1, 1, 1),    # vector path, Cin % 16 == 0
+    (2, 14, 14, 32, 48, 3, 3, 1, 1, 2, 2, 1, 1),
+    (1, 12, 12, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1),     # Cin % 4 == 0, taps straddle a K step
+    (1, 10, 10, 20, 130, 3, 3, 2, 2, 1, 1, 2, 2),   # Cin % 4 == 0, not % 16; N tail; dilation
+    (3, 9, 9, 128, 200, 1, 1, 0, 0, 1, 1, 1, 1),    # 1x1
+    (2, 14, 14, 128, 256, 1, 1, 0, 0, 2, 2, 1, 1),  # 1x1 stride 2 shortcut
+    (2, 32, 32, 3, 64, 7, 7, 3, 3, 2, 2, 1, 1),     # stem
+    (2, 8, 32, 1, 64, 3, 3, 1, 1, 1, 1, 1, 1),      # single input channel
+]
+
+
+@pytest.mark.parametrize("case", GPU_CONV_CASES)
+def test_convolution(case):
+    n, h, w, cin, cout, fh, fw, ph, pw, sh, sw, dh, dw = case
+    g = rng(10 + h * w + cin)
+    x = g.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    f = g.normal(0, 1.0 / np.sqrt(fh * fw * cin), (cout, fh, fw, cin)).astype(np.float32)
+    bias = g.uniform(-1, 1, cout).astype(np.float32)
+    want = orc.conv(x, f, bias, ph, pw, sh, sw, dh, dw)
+    assert_close(hip().conv(x, f, bias, ph, pw, sh, sw, dh, dw), want, "conv %s" % (case,))
+    assert_close(hip().conv(x, f, None, ph, pw, sh, sw, dh, dw), orc.conv(x, f, None, ph, pw, sh, sw, dh, dw), "conv, no free term")
+
+
+def test_convolution_config1_vs_reference_engine():
+    # the single-layer configuration at reduced batch: 32x32x64 image, 3x3 64 -> 64, pad 1, + free term, then ReLU
+    g = rng(1)
+    x = g.uniform(-1, 1, (2, 32, 32, 64)).astype(np.float32)
+    f = g.normal(0, 1.0 / np.sqrt(576.0), (64, 3, 3, 64)).astype(np.float32)
+    bias = np.zeros(64, np.float32)
+    y = hip().conv(x, f, bias, 1, 1, 1, 1)
+    y = hip().unary("relu", y, 0.0).reshape(2, 32, 32, 64)
+    r = ref_or_none() or orc
+    want = r.unary("relu", r.conv(x, f, bias, 1, 1, 1, 1), 0.0).reshape(2, 32, 32, 64)
+    assert_close(y, want, "config 1")
+
+
+def test_convolution_is_linear_at_full_size():
+    # full single-layer configuration (batch 32): conv(a x1 + x2) == a conv(x1) + conv(x2), and the 1x1
+    # identity filter returns the image; both hold for any size without a CPU pass over it
+    h = hip()
+    g = rng(40)
+    x1 = g.uniform(-1, 1, (32, 32, 32, 64)).astype(np.float32)
+    x2 = g.uniform(-1, 1, (32, 32, 32, 64)).astype(np.float32)
+    f = g.normal(0, 1.0 / 24, (64, 3, 3, 64)).astype(np.float32)
+    y1, y2 = h.conv(x1, f, None, 1, 1, 1, 1), h.conv(x2, f, None, 1, 1, 1, 1)
+    y12 = h.conv(0.5 * x1 + x2, f, None, 1, 1, 1, 1)
+    assert_close(y12, 0.5 * y1 + y2, "linearity", atol=1e-4)
+    eye = np.eye(64, dtype=np.float32).reshape(64, 1, 1, 64)
+    assert np.array_equal(h.conv(x1, eye, None, 0, 0, 1, 1), x1)
+
+
+@pytest.mark.parametrize("case", CHANNELWISE_CASES + [(2, 28, 28, 96, 3, 3, 1, 1, 1, 1), (2, 28, 28, 96, 3, 3, 1, 1, 2, 2),
+                                                      (1, 15, 13, 6, 3, 3, 1, 1, 2, 2), (1, 9, 30, 32, 5, 5, 2, 2, 1, 1)])
+def test_channelwise_convolution(case):
+    n, h, w, c, fh, fw, ph, pw, sh, sw = case
+    g = rng(12 + c)
+    x = g.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    f = g.normal(0, 1, (fh, fw, c)).astype(np.float32)
+    bias = g.uniform(-1, 1, c).astype(np.float32)
+    assert_close(hip().channelwise_conv(x, f, bias, ph, pw, sh, sw), orc.channelwise_conv(x, f, bias, ph, pw, sh, sw), str(case))
+    assert_close(hip().channelwise_conv(x, f, None, ph, pw, sh, sw), orc.channelwise_conv(x, f, None, ph, pw, sh, sw), str(case))
+
+
+@pytest.mark.parametrize("case", POOL_CASES + [(2, 57, 57, 64, 3, 3, 2, 2), (3, 16, 64, 7, 2, 2, 2, 2), (2, 4, 128, 256, 2, 1, 2, 1)])
+def test_pooling(case):
+    n, h, w, c, fh, fw, sh, sw = case
+    g = rng(13 + h)
+    x = g.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    assert np.array_equal(hip().max_pool(x, fh, fw, sh, sw), orc.max_pool(x, fh, fw, sh, sw))
+    assert_close(hip().mean_pool(x, fh, fw, sh, sw), orc.mean_pool(x, fh, fw, sh, sw), "mean %s" % (case,))
+    y, idx = hip().max_pool(x, fh, fw, sh, sw, with_indices=True)
+    oy, oidx = orc.max_pool(x, fh, fw, sh, sw, with_indices=True)
+    assert np.array_equal(y, oy)
+    assert np.array_equal(idx, oidx), "pooling indices must be bit-exact"
+
+
+def test_pooling_index_ties_bit_exact():
+    g = rng(15)
+    x = np.maximum(g.uniform(-1, 0.3, (2, 16, 16, 8)), 0).astype(np.float32)  # many all-zero windows, as after ReLU
+    x = np.round(x * 4) / 4
+    r = ref_or_none() or orc
+    for fh, fw, sh, sw in ((2, 2, 2, 2), (3, 3, 2, 2), (3, 3, 1, 1)):
+        y, idx = hip().max_pool(x, fh, fw, sh, sw, with_indices=True)
+        ry, ridx = r.max_pool(x, fh, fw, sh, sw, with_indices=True)
+        assert np.array_equal(y, ry) and np.array_equal(idx, ridx)
+
+
+def test_resize_image():
+    g = rng(16)
+    for shape in ((2, 5, 6, 3), (2, 9, 7, 8)):
+        x = g.uniform(-1, 1, shape).astype(np.float32)
+        for dl, dr, dt, db in ((1, 1, 1, 1), (2, 0, 0, 3), (0, 0, 0, 0), (3, 2, 1, 4), (-1, -2, -1, 0), (-1, 2, 1, -2)):
+            for mode in (0, 1, 2):
+                if mode != 0 and min(dl, dr, dt, db) < 0:
+                    continue
+                assert np.array_equal(hip().resize_image(x, dl, dr, dt, db, mode, 0.5), orc.resize_image(x, dl, dr, dt, db, mode, 0.5))
+
+
+def test_split_and_merge():
+    g = rng(17)
+    big = g.uniform(-1, 1, (2, 3, 1, 4, 5, 1, 12)).astype(np.float32)
+    for dim, sizes in ((6, (4, 8)), (6, (3, 4, 5)), (4, (2, 3)), (3, (1, 3)), (0, (1, 1)), (1, (2, 1))):
+        part_dims = []
+        for s in sizes:
+            d = list(big.shape)
+            d[dim] = s
+            part_dims.append(tuple(d))
+        want = orc.split(big, dim, part_dims)
+        got = hip().split(big, dim, part_dims)
+        for p, q in zip(got, want):
+            assert np.array_equal(p, q), (dim, sizes)
+        assert np.array_equal(hip().merge(want, dim, big.shape), big)
+    # LSTM gate split: 4H -> 4 x H along channels
+    gates = g.uniform(-1, 1, (1, 64, 1, 1, 1, 1, 1024)).astype(np.float32)
+    parts = hip().split(gates, 6, [(1, 64, 1, 1, 1, 1, 256)] * 4)
+    for i, p in enumerate(parts):
+        assert np.array_equal(p, gates[..., 256 * i:256 * (i + 1)])
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+@pytest.mark.parametrize("with_init", [False, True])
+def test_lstm(reverse, with_init):
+    g = rng(18)
+    for T, B, In, H in ((5, 3, 6, 4), (7, 16, 32, 64), (4, 64, 256, 256)):
+        w_in = g.uniform(-0.2, 0.2, (4 * H, In)).astype(np.float32)
+        w_rec = g.uniform(-0.2, 0.2, (4 * H, H)).astype(np.float32)
+        b_in = g.uniform(-0.5, 0.5, 4 * H).astype(np.float32)
+        b_rec = g.uniform(-0.5, 0.5, 4 * H).astype(np.float32)
+        x = g.uniform(-1, 1, (T, B, In)).astype(np.float32)
+        c0 = g.uniform(-1, 1, (B, H)).astype(np.float32) if with_init else None
+        h0 = g.uniform(-1, 1, (B, H)).astype(np.float32) if with_init else None
+        for bi, br in ((b_in, b_rec), (None, b_rec), (None, None)):
+            h, c = hip().lstm(w_in, bi, w_rec, br, x, reverse, c0, h0)
+            oh, oc = orc.lstm(w_in, bi, w_rec, br, x, reverse, c0, h0)
+            assert_close(h, oh, "lstm h %s" % ((T, B, In, H),))
+            assert_close(c, oc, "lstm c")
+            h2, _ = hip().lstm(w_in, bi, w_rec, br, x, reverse, c0, h0, want_state=False)
+            assert_close(h2, oh, "lstm h without state output")
+
+
+# ---------------------------------------------------------------------------------------------------------
+# error convention and allocator on the device
+
+def test_argument_errors_are_reported_not_thrown():
+    import neoml_amd
+    lib = neoml_amd.load()
+    d = neoml_amd.ConvDesc(1, 4, 4, 3, 2, 5, 5, 0, 0, 1, 1, 1, 1, 0, 0)  # filter larger than the image
+    assert lib.nhInitBlobConvolution(ctypes.byref(d)) == 1
+    assert "requirement failed" in neoml_amd.last_error()
+    assert lib.nhVectorReLU(None, None, None, -1, None) == 1
+
+
+def test_device_pool():
+    import neoml_amd
+    lib = neoml_amd.load()
+    pool = ctypes.c_void_p()
+    neoml_amd.check(lib.nhPoolCreate(ctypes.byref(pool), 0, 64 << 20))
+    p1, p2 = ctypes.c_void_p(), ctypes.c_void_p()
+    neoml_amd.check(lib.nhPoolHeapAlloc(pool, 1000, ctypes.byref(p1)))
+    neoml_amd.check(lib.nhPoolHeapFree(pool, p1))
+    neoml_amd.check(lib.nhPoolHeapAlloc(pool, 900, ctypes.byref(p2)))
+    assert p1.value == p2.value  # same size class: the cached block comes back without a raw allocation
+    big = ctypes.c_void_p()
+    assert lib.nhPoolHeapAlloc(pool, 128 << 20, ctypes.byref(big)) == 3  # over the limit: NH_ERR_MEMORY
+    # the block is usable device memory
+    h = hip()
+    neoml_amd.check(lib.nhVectorFill(h.stream(), p2, ctypes.c_float(3.0), 225))
+    host = (ctypes.c_float * 225)()
+    neoml_amd.check(lib.nhCopyDeviceToHost(h.stream(), host, p2, 900))
+    assert list(host) == [3.0] * 225
+    neoml_amd.check(lib.nhPoolHeapFree(pool, p2))
+    neoml_amd.check(lib.nhPoolDestroy(pool))
