@@ -1,0 +1,129 @@
+#!/usr/bin/env python3
+"""Benchmark of the IMathEngine inference hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+A step is one forward pass of the ResNet-18-style network (BASELINE.json configs[1]: batch 64, 224x224x3, fp32)
+issued as engine calls through the C ABI of libneoml_hip.so, input already resident in device memory.
+Prints one JSON line: images/sec, the roofline of the dominant kernel (the 3x3 implicit-GEMM convolutions, timed
+live with events on the launch stream) and the reference CPU engine timed on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP32_MFMA_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBPS = 8000.0
+
+
+def cpu_baseline(batch_sample, image):
+    """The reference's own CPU engine (oracle/_ref, built from its sources) on `batch_sample` images of the same
+    network, one thread. Falls back to the C oracle (kind 'port') when the reference build is absent."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import nhtest
+    from neoml_amd.workloads import ResNet18
+    kind = "ref" if nhtest.have_reference() else "orc"
+    be = nhtest.CpuBackend(kind)
+    net = ResNet18(be, batch=batch_sample, image=image)
+    x = net.make_input()
+    t0 = time.perf_counter()
+    y = net.forward(x)
+    dt = time.perf_counter() - t0
+    return {
+        "value": round(batch_sample / dt, 3), "unit": "images/sec", "cores": 1,
+        "kind": "reference" if kind == "ref" else "port",
+        "sample": "%d images of the same network, 1 pass, %s" % (
+            batch_sample, "reference CCpuMathEngine with its built-in SSE GEMM (no MKL/MLAS)" if kind == "ref" else "C oracle"),
+        "seconds": round(dt, 2),
+    }, y
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--image", type=int, default=224)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample", type=int, default=8, help="images in the CPU baseline sample")
+    ap.add_argument("--per-kernel", action="store_true", help="print a per-op-family timing table to stderr")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus)
+
+    import torch
+    from neoml_amd.workloads import HipBackend, ResNet18
+
+    be = HipBackend(record_events=True)
+    net = ResNet18(be, batch=args.batch, image=args.image)
+    x = be.tensor(net.make_input())
+    for _ in range(args.warmup):
+        net.forward(x)
+    be.synchronize()
+    be.events.clear()
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = net.forward(x)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    ms_per_step = elapsed / args.steps * 1e3
+    images_per_sec = args.batch * args.steps / elapsed
+
+    # per-family totals from the events recorded inside the timed region
+    fam = {}
+    for tag, flops, nbytes, start, stop in be.events:
+        f = fam.setdefault(tag, [0, 0.0, 0, 0])
+        f[0] += 1
+        f[1] += start.elapsed_time(stop)
+        f[2] += flops
+        f[3] += nbytes
+    c3 = fam.get("conv3x3", [0, 1e-9, 0, 0])
+    launches, ms, flops, nbytes = c3
+    achieved = flops / (ms * 1e-3) / 1e12
+    roofline = {
+        "bound": "mfma", "kernel": "matMulKernel<AM_Conv> (3x3 convolutions, %d launches per step)" % (launches // max(args.steps, 1)),
+        "achieved": round(achieved, 2), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
+        "avg_launch_us": round(ms * 1e3 / max(launches, 1), 2),
+        "flop_per_step": flops // max(args.steps, 1),
+    }
+    if args.per_kernel:
+        for tag, (cnt, tms, fl, by) in sorted(fam.items(), key=lambda kv: -kv[1][1]):
+            print("%-10s launches/step %3d  ms/step %8.3f  TFLOP/s %7.2f  GB/s %8.1f" % (
+                tag, cnt // args.steps, tms / args.steps, fl / (tms * 1e-3) / 1e12 if fl else 0.0,
+                by / (tms * 1e-3) / 1e9), file=sys.stderr)
+
+    result = {
+        "metric": "images/sec ResNet-18-style b64 fp32; conv TFLOPS as % of fp32 MFMA peak",
+        "value": round(images_per_sec, 1), "unit": "images/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "ResNet-18-style inference, batch %d, %dx%dx3, fp32, engine calls through the C ABI" % (
+            args.batch, args.image, args.image), "global_batch": args.batch,
+            "gflop_per_step": round(net.conv_flops() / 1e9, 2)},
+        "conv_tflops_overall": round(net.conv_flops() / (ms_per_step * 1e-3) / 1e12, 2),
+        "roofline": roofline,
+    }
+
+    if not args.no_cpu_baseline:
+        base, y_cpu = cpu_baseline(args.cpu_sample, args.image)
+        result["cpu_baseline"] = base
+        # the same images through the GPU path: parity of the whole network on the sample
+        import numpy as np
+        small = ResNet18(HipBackend(), batch=args.cpu_sample, image=args.image)
+        y_gpu = small.be.to_numpy(small.forward(small.be.tensor(small.make_input())))
+        result["parity_max_abs_diff_vs_cpu"] = float(np.max(np.abs(y_gpu - y_cpu)))
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

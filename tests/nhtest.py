@@ -712,3 +712,52 @@ class Hip:
         self.call("nhLstm", H, In, self.p(ws[0]), self.p(ws[1]), self.p(ws[2]), self.p(ws[3]), 1 if reverse else 0, T, B,
                   self.p(ws[4]), self.p(ws[5]), self.p(ws[6]), self.p(c), self.p(h), self.p(work), size.value)
         return self.down(h), (self.down(c) if want_state else None)
+
+
+class CpuBackend:
+    """Host backend for neoml_amd.workloads: the same network code on numpy arrays, executed by the oracle
+    ('orc') or by the reference's CPU engine ('ref')."""
+
+    def __init__(self, kind):
+        self.cpu = Cpu(kind)
+        self.name = kind
+
+    def tensor(self, a):
+        return f32(a)
+
+    def to_numpy(self, t):
+        return t
+
+    def synchronize(self):
+        pass
+
+    def conv(self, x, filt, bias, ph, pw, sh, sw, out=None):
+        return self.cpu.conv(x, filt, bias, ph, pw, sh, sw)
+
+    def relu_(self, x, threshold=None):
+        x[...] = self.cpu.unary("relu", x, 0.0 if threshold is None else threshold).reshape(x.shape)
+        return x
+
+    def add_(self, a, b):
+        a[...] = self.cpu.binary("add", a, b).reshape(a.shape)
+        return a
+
+    def pad(self, x, dl, dr, dt, db, value=0.0, out=None):
+        return self.cpu.resize_image(x, dl, dr, dt, db, 0, value)
+
+    def max_pool(self, x, fh, fw, sh, sw, out=None):
+        return self.cpu.max_pool(x, fh, fw, sh, sw)
+
+    def global_mean(self, x, out=None):
+        n, h, w, c = x.shape
+        s = self.cpu.sum_matrix_rows(x.reshape(n, h * w, c))
+        return self.cpu.unary("multiply", s, np.float32(1.0 / (h * w))).reshape(n, c)
+
+    def fc(self, x, weight, bias, out=None):
+        m, k = x.shape
+        n = weight.shape[0]
+        y = self.cpu.matmul("nt", x, weight, lda=k, ldb=k, ldc=n, M=m, N=n, K=k).reshape(1, m, n)
+        return self.cpu.add_vector_to_matrix_rows(y, bias.reshape(1, n)).reshape(m, n)
+
+    def softmax(self, x, out=None):
+        return self.cpu.softmax_rows(x)
