@@ -45,6 +45,7 @@ class HipBackend:
         self.record_events = record_events
         self.events = []  # (tag, flops, bytes, start, stop)
         self._desc_cache = {}
+        self.plan = None  # when a list: every launch is also appended as (fn, args, tag, flops, bytes)
 
     # ---- memory
     def tensor(self, a):
@@ -64,11 +65,19 @@ class HipBackend:
         return None if t is None else ctypes.c_void_p(t.data_ptr())
 
     def _call(self, fn, *args):
+        if self.plan is not None:
+            self.plan.append((fn, args, None, 0, 0))
         rc = fn(self.stream, *args)
         if rc != 0:
             self.na.check(rc)
 
     def _timed(self, tag, flops, nbytes, fn, *args):
+        if self.plan is not None:
+            self.plan.append((fn, args, tag, flops, nbytes))
+            rc = fn(self.stream, *args)
+            if rc != 0:
+                self.na.check(rc)
+            return
         if not self.record_events:
             self._call(fn, *args)
             return
@@ -157,6 +166,67 @@ class HipBackend:
         return out
 
 
+class LaunchPlan:
+    """A recorded sequence of C-ABI launches with their arguments bound once, replayed with minimal host work
+    (the position a native caller of the engine is in). Optionally brackets the launches of chosen op families
+    with events recorded on the launch stream through nhEventRecord."""
+
+    def __init__(self, backend, launches):
+        self.be = backend
+        self.launches = [(fn, (backend.stream,) + tuple(args), tag, flops, nbytes) for fn, args, tag, flops, nbytes in launches]
+        self.keep_alive = launches  # ctypes objects referenced by the bound arguments
+        self.timed = []  # (tag, flops, bytes, start, stop) of the replays run with events
+
+    def run(self):
+        for fn, args, _, _, _ in self.launches:
+            rc = fn(*args)
+            if rc != 0:
+                self.be.na.check(rc)
+
+    def make_events(self, tags, steps):
+        lib = self.be.lib
+        pools = []
+        for _ in range(steps):
+            step = []
+            for fn, args, tag, flops, nbytes in self.launches:
+                if tag in tags:
+                    a, b = ctypes.c_void_p(), ctypes.c_void_p()
+                    self.be.na.check(lib.nhEventCreate(ctypes.byref(a)))
+                    self.be.na.check(lib.nhEventCreate(ctypes.byref(b)))
+                    step.append((a, b))
+                else:
+                    step.append(None)
+            pools.append(step)
+        return pools
+
+    def run_with_events(self, pool):
+        record, stream = self.be.lib.nhEventRecord, self.be.stream
+        for (fn, args, tag, flops, nbytes), ev in zip(self.launches, pool):
+            if ev is None:
+                rc = fn(*args)
+            else:
+                record(ev[0], stream)
+                rc = fn(*args)
+                record(ev[1], stream)
+                self.timed.append((tag, flops, nbytes, ev[0], ev[1]))
+            if rc != 0:
+                self.be.na.check(rc)
+
+    def family_totals(self):
+        """{tag: [launches, total ms, flops, bytes]} of the replays run with events (after a synchronize)."""
+        lib = self.be.lib
+        fam = {}
+        ms = ctypes.c_float(0)
+        for tag, flops, nbytes, a, b in self.timed:
+            self.be.na.check(lib.nhEventElapsedMs(a, b, ctypes.byref(ms)))
+            f = fam.setdefault(tag, [0, 0.0, 0, 0])
+            f[0] += 1
+            f[1] += ms.value
+            f[2] += flops
+            f[3] += nbytes
+        return fam
+
+
 class ResNet18:
     """ResNet-18-style inference: 7x7/2 stem, pad + 3x3/2 max-pool, 4 stages of 2 basic blocks (64/128/256/512,
     batch-norm folded into the convolution free terms), global mean pool, FC -> classes, softmax."""
@@ -213,9 +283,14 @@ class ResNet18:
         total += 2 * n * self.classes * cin
         return total
 
-    def _buf(self, key, producer):
-        # activations are allocated on the first pass and reused afterwards (what the engine's blob cache does)
-        return self.buffers.get(key)
+    def record_plan(self, x):
+        """Runs one forward pass while recording its launches; returns (LaunchPlan, output tensor).
+        Activation buffers are allocated by this pass and reused by every replay."""
+        self.forward(x)  # allocates the buffers
+        self.be.plan = []
+        out = self.forward(x)
+        launches, self.be.plan = self.be.plan, None
+        return LaunchPlan(self.be, launches), out
 
     def forward(self, x):
         be, B = self.be, self.buffers
