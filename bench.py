@@ -46,8 +46,11 @@ def cpu_baseline(batch_sample, image):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--settle-ms", type=float, default=600.0,
+                    help="after the warm-up steps keep replaying the step untimed for this long, so that the timed region "
+                         "starts with the GPU at its sustained clock instead of ramping up from idle")
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--image", type=int, default=224)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -72,6 +75,13 @@ def main():
     for _ in range(args.warmup):
         plan.run()
     torch.cuda.synchronize()
+    settle_start = time.perf_counter()
+    settle_steps = 0
+    while (time.perf_counter() - settle_start) * 1e3 < args.settle_ms:
+        for _ in range(5):
+            plan.run()
+        torch.cuda.synchronize()
+        settle_steps += 5
 
     t0 = time.perf_counter()
     for step in range(args.steps):
@@ -111,6 +121,7 @@ def main():
             "gflop_per_step": round(net.conv_flops() / 1e9, 2)},
         "conv_tflops_overall": round(net.conv_flops() / (ms_per_step * 1e-3) / 1e12, 2),
         "host_enqueue_ms_per_step": round((host_done - t0) / args.steps * 1e3, 3),
+        "clock_settle": {"ms": args.settle_ms, "untimed_steps": settle_steps},
         "roofline": roofline,
     }
 

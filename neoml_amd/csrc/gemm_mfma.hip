@@ -8,8 +8,14 @@
 //
 // Tiling: 256 threads = 4 wavefronts per workgroup; workgroup tile BM x BN, K step 16; each wavefront owns
 // a (BM/WAVES_M) x (BN/WAVES_N) sub-tile built from 32x32 blocks of v_mfma_f32_32x32x2_f32 (16 accumulator
-// registers per block). Tiles of A and B are staged through LDS with two buffers and one barrier per K step;
-// the global loads of step k+1 are in flight while step k is multiplied.
+// registers per block).
+//
+// Data path: operands are fetched with raw buffer loads (32-bit offsets that only need an add per K step; the
+// memory unit's range check supplies the zeros of padding and of partial tiles), parked in registers for one
+// K step, written to one of three LDS buffers and read back as MFMA operands. Within a wavefront the LDS reads
+// of the next group of 8 k are issued before the MFMAs of the current group, and the single barrier of a K step
+// sits before its last group, so the matrix pipe of a wavefront does not wait for LDS, barrier or memory in steady
+// state.
 //
 // LDS layout for a K-major operand is [row][16 + 4 pad]; lane (row = lane % 32, half = lane / 32) fetches the
 // four consecutive k values  k0 + 4*half .. +3  with a single 128-bit LDS read and feeds them to four MFMAs.
@@ -35,18 +41,14 @@ struct CMatMulArgs {
 	int Accumulate; // C += instead of C =
 	int TilesM, TilesN;
 	// convolution geometry (AM_Conv only): A is the image, M = batch * Ho * Wo
-	int H, W, Cin, Ho, Wo, Fw, PadH, PadW, StrideH, StrideW, DilH, DilW;
+	int H, W, Cin, Ho, Wo, Fh, Fw, PadH, PadW, StrideH, StrideW, DilH, DilW;
 };
 
-constexpr int KStep = 16;
-constexpr int LdsK = KStep + 4; // row pitch of a K-major tile in LDS (floats)
 constexpr int Threads = 256;
 
-template<int BX> struct CTileLds {
-	static constexpr int KMajorSize = BX * LdsK;
-	static constexpr int XMajorPitch = BX + 4;
-	static constexpr int XMajorSize = KStep * XMajorPitch;
-};
+#ifndef NH_KSTEP
+#define NH_KSTEP 16
+#endif
 
 // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous range of tiles so that
 // neighbouring tiles (which share rows of A and the halo of the image) meet in the same L2.
@@ -59,25 +61,47 @@ __device__ __forceinline__ int xcdSwizzle( int bid, int total )
 	return xcd * per + ( xcd < rem ? xcd : rem ) + idx;
 }
 
+// Operands are read with raw buffer loads: a 32-bit byte offset from a base held in scalar registers, and a range
+// check done by the memory unit. An offset at or above BufferBytes reads as zero, which serves as the zero padding
+// of the convolution and as the mask of tile rows / columns / k beyond the matrix, without a branch or a select.
+typedef unsigned int u32x4 __attribute__( ( ext_vector_type( 4 ) ) );
+constexpr unsigned BufferBytes = 0x80000000u;
+constexpr unsigned OutOfRange = 0x80000000u;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t makeBuffer( const float* p )
+{
+	return __builtin_amdgcn_make_buffer_rsrc( const_cast<float*>( p ), 0, BufferBytes, 0x00020000 );
+}
+
+__device__ __forceinline__ float4 bufferLoad4( __amdgpu_buffer_rsrc_t rsrc, unsigned offset )
+{
+	const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128( rsrc, offset, 0, 0 );
+	return make_float4( __uint_as_float( v.x ), __uint_as_float( v.y ), __uint_as_float( v.z ), __uint_as_float( v.w ) );
+}
+
 template<int BM, int BN, int WAVES_M, int WAVES_N, int AMODE, int BMODE, bool VEC>
 __global__ __launch_bounds__( Threads, 2 )
 void matMulKernel( const CMatMulArgs args )
 {
+	constexpr int KS = NH_KSTEP;           // K step per pipeline stage
+	constexpr int KQ = KS / 4;             // float4 slots along K of a K-major tile row
+	constexpr int LdsK = KS + 4;           // row pitch of a K-major tile in LDS
 	static_assert( WAVES_M * WAVES_N == 4, "4 wavefronts per workgroup" );
 	constexpr int WM = BM / WAVES_M;
 	constexpr int WN = BN / WAVES_N;
 	constexpr int MI = WM / 32;
 	constexpr int NI = WN / 32;
-	static_assert( MI >= 1 && NI >= 1, "wave tile is at least one 32x32 block" );
-	constexpr bool AK = ( AMODE != AM_RowsM ); // A tile kept K-major in LDS
+	constexpr bool AK = ( AMODE != AM_RowsM );
 	constexpr bool BK = ( BMODE == BM_RowsK );
-	constexpr int ASize = AK ? CTileLds<BM>::KMajorSize : CTileLds<BM>::XMajorSize;
-	constexpr int BSize = BK ? CTileLds<BN>::KMajorSize : CTileLds<BN>::XMajorSize;
-	constexpr int ASlots = ( BM * 4 + Threads - 1 ) / Threads; // float4 slots per thread per K step
-	constexpr int BSlots = ( BN * 4 + Threads - 1 ) / Threads;
+	constexpr int APitchX = BM + 4, BPitchX = BN + 4;
+	constexpr int ASize = AK ? BM * LdsK : KS * APitchX;
+	constexpr int BSize = BK ? BN * LdsK : KS * BPitchX;
+	constexpr int ATotal = BM * KQ, BTotal = BN * KQ; // float4 slots per tile
+	constexpr int ASlots = ( ATotal + Threads - 1 ) / Threads;
+	constexpr int BSlots = ( BTotal + Threads - 1 ) / Threads;
 
-	__shared__ __attribute__( ( aligned( 16 ) ) ) float ldsA[2][ASize];
-	__shared__ __attribute__( ( aligned( 16 ) ) ) float ldsB[2][BSize];
+	__shared__ __attribute__( ( aligned( 16 ) ) ) float ldsA[3][ASize];
+	__shared__ __attribute__( ( aligned( 16 ) ) ) float ldsB[3][BSize];
 
 	const int tid = threadIdx.x;
 	const int lane = tid & 63;
@@ -94,48 +118,77 @@ void matMulKernel( const CMatMulArgs args )
 	const int n0 = tileN * BN;
 	const int batch = blockIdx.y;
 
-	const float* __restrict__ A = args.A + batch * args.BatchStrideA;
-	const float* __restrict__ B = args.B + batch * args.BatchStrideB;
+	const float* A = args.A + batch * args.BatchStrideA;
+	const float* B = args.B + batch * args.BatchStrideB;
 	float* C = args.C + batch * args.BatchStrideC;
 	const int M = args.M, N = args.N, K = args.K;
+	const __amdgpu_buffer_rsrc_t bufA = makeBuffer( A );
+	const __amdgpu_buffer_rsrc_t bufB = makeBuffer( B );
 
-	// ---- per-thread load slots -------------------------------------------------------------------------
-	// K-major tile: slot -> ( row = slot / 4, kq = slot % 4 ); X-major tile: slot -> ( k = slot / (BX/4), xq ).
-	// Convolution: every slot row is one output pixel; its top-left input coordinate is fixed for the kernel.
-	int convBase[ASlots];
-	int convH0[ASlots];
-	int convW0[ASlots];
-	int convCi = 0, convKh = 0, convKw = 0; // tap state of this thread's k (VEC path, advanced every K step)
-	if( AMODE == AM_Conv ) {
+	// ---- per-thread load slots ---------------------------------------------------------------------------
+	// K-major tile: slot -> ( row = slot / KQ, kq = slot % KQ ); X-major tile: slot -> ( k = slot / (BX/4), xq ).
+	// Vector path: offA / offB hold the byte offset of the slot for the K step that is loaded next.
+	unsigned offA[ASlots], offB[BSlots];
+	int convPixel[ASlots], convH0[ASlots], convW0[ASlots];
+	int convCi = 0, convKh = 0, convKw = 0;
+
+	auto convSlotOffset = [&]( int i ) -> unsigned {
+		const int hi = convH0[i] + convKh * args.DilH;
+		const int wi = convW0[i] + convKw * args.DilW;
+		const bool ok = convKh < args.Fh && hi >= 0 && hi < args.H && wi >= 0 && wi < args.W;
+		return ok ? static_cast<unsigned>( convPixel[i] + ( hi * args.W + wi ) * args.Cin + convCi ) * 4u : OutOfRange;
+	};
+
 #pragma unroll
-		for( int i = 0; i < ASlots; ++i ) {
-			const int slot = tid + i * Threads;
-			const int m = m0 + ( slot >> 2 );
-			if( m < M && ( BM * 4 % Threads == 0 || slot < BM * 4 ) ) {
+	for( int i = 0; i < ASlots; ++i ) {
+		const int slot = tid + i * Threads;
+		const bool inTile = ATotal % Threads == 0 || slot < ATotal;
+		if( AMODE == AM_RowsK ) {
+			const int m = m0 + slot / KQ;
+			offA[i] = ( inTile && m < M ) ? static_cast<unsigned>( m * args.Lda + ( slot % KQ ) * 4 ) * 4u : OutOfRange;
+		} else if( AMODE == AM_RowsM ) {
+			const int m = m0 + ( slot % ( BM / 4 ) ) * 4;
+			offA[i] = ( inTile && m < M ) ? static_cast<unsigned>( ( slot / ( BM / 4 ) ) * args.Lda + m ) * 4u : OutOfRange;
+		} else {
+			const int m = m0 + slot / KQ;
+			if( inTile && m < M ) {
 				const int wo = m % args.Wo;
 				const int t = m / args.Wo;
 				const int ho = t % args.Ho;
 				const int n = t / args.Ho;
-				convBase[i] = n * args.H * args.W * args.Cin;
+				convPixel[i] = n * args.H * args.W * args.Cin;
 				convH0[i] = ho * args.StrideH - args.PadH;
 				convW0[i] = wo * args.StrideW - args.PadW;
 			} else {
-				convBase[i] = 0;
-				convH0[i] = -0x40000000; // always out of the image
+				convPixel[i] = 0;
+				convH0[i] = -0x40000000; // never inside the image
 				convW0[i] = 0;
 			}
 		}
-		if( VEC ) {
-			const int k = ( tid & 3 ) * 4;
-			const int tap = k / args.Cin;
-			convCi = k - tap * args.Cin;
-			convKh = tap / args.Fw;
-			convKw = tap - convKh * args.Fw;
+	}
+	if( AMODE == AM_Conv && VEC ) {
+		const int k = ( tid % KQ ) * 4;
+		const int tap = k / args.Cin;
+		convCi = k - tap * args.Cin;
+		convKh = tap / args.Fw;
+		convKw = tap - convKh * args.Fw;
+#pragma unroll
+		for( int i = 0; i < ASlots; ++i ) {
+			offA[i] = convSlotOffset( i );
 		}
 	}
-
-	float4 regA[ASlots];
-	float4 regB[BSlots];
+#pragma unroll
+	for( int i = 0; i < BSlots; ++i ) {
+		const int slot = tid + i * Threads;
+		const bool inTile = BTotal % Threads == 0 || slot < BTotal;
+		if( BMODE == BM_RowsK ) {
+			const int n = n0 + slot / KQ;
+			offB[i] = ( inTile && n < N ) ? static_cast<unsigned>( n * args.Ldb + ( slot % KQ ) * 4 ) * 4u : OutOfRange;
+		} else {
+			const int n = n0 + ( slot % ( BN / 4 ) ) * 4;
+			offB[i] = ( inTile && n < N ) ? static_cast<unsigned>( ( slot / ( BN / 4 ) ) * args.Ldb + n ) * 4u : OutOfRange;
+		}
+	}
 
 	auto loadConvElement = [&]( int i, int k ) -> float {
 		if( k >= K ) {
@@ -150,115 +203,130 @@ void matMulKernel( const CMatMulArgs args )
 		if( hi < 0 || hi >= args.H || wi < 0 || wi >= args.W ) {
 			return 0.f;
 		}
-		return A[convBase[i] + ( hi * args.W + wi ) * args.Cin + ci];
+		return A[convPixel[i] + ( hi * args.W + wi ) * args.Cin + ci];
 	};
 
-	auto loadTiles = [&]( int kBase ) {
-		// ---- A ----
+	// Loads the tiles of the K step starting at kBase into registers and advances the slot offsets to the next step.
+	auto loadTiles = [&]( int kBase, float4 ( &regA )[ASlots], float4 ( &regB )[BSlots] ) {
+		if( VEC ) {
+			// k of this thread's slots inside the step: fixed column of a K-major tile, fixed row of an X-major one
+			const bool kInA = AMODE == AM_RowsM ? true : ( kBase + ( tid % KQ ) * 4 < K );
+			const bool kInB = BMODE == BM_RowsN ? true : ( kBase + ( tid % KQ ) * 4 < K );
+#pragma unroll
+			for( int i = 0; i < ASlots; ++i ) {
+				unsigned off = offA[i];
+				if( AMODE == AM_RowsK ) {
+					off = kInA ? off : OutOfRange;
+				} else if( AMODE == AM_RowsM ) {
+					off = ( kBase + ( tid + i * Threads ) / ( BM / 4 ) < K ) ? off : OutOfRange;
+				}
+				regA[i] = bufferLoad4( bufA, off );
+			}
+#pragma unroll
+			for( int i = 0; i < BSlots; ++i ) {
+				unsigned off = offB[i];
+				if( BMODE == BM_RowsK ) {
+					off = kInB ? off : OutOfRange;
+				} else {
+					off = ( kBase + ( tid + i * Threads ) / ( BN / 4 ) < K ) ? off : OutOfRange;
+				}
+				regB[i] = bufferLoad4( bufB, off );
+			}
+			// advance
+			if( AMODE == AM_Conv ) {
+				convCi += KS;
+				if( convCi >= args.Cin ) {
+					do {
+						convCi -= args.Cin;
+						if( ++convKw == args.Fw ) {
+							convKw = 0;
+							++convKh;
+						}
+					} while( convCi >= args.Cin );
+#pragma unroll
+					for( int i = 0; i < ASlots; ++i ) {
+						offA[i] = convSlotOffset( i );
+					}
+				} else {
+#pragma unroll
+					for( int i = 0; i < ASlots; ++i ) {
+						offA[i] += KS * 4;
+					}
+				}
+			} else {
+				const unsigned stepA = AMODE == AM_RowsK ? KS * 4u : static_cast<unsigned>( KS * args.Lda ) * 4u;
+#pragma unroll
+				for( int i = 0; i < ASlots; ++i ) {
+					offA[i] += stepA;
+				}
+			}
+			const unsigned stepB = BMODE == BM_RowsK ? KS * 4u : static_cast<unsigned>( KS * args.Ldb ) * 4u;
+#pragma unroll
+			for( int i = 0; i < BSlots; ++i ) {
+				offB[i] += stepB;
+			}
+			return;
+		}
+		// scalar path: any alignment, any shape
 #pragma unroll
 		for( int i = 0; i < ASlots; ++i ) {
 			const int slot = tid + i * Threads;
 			float4 v = make_float4( 0.f, 0.f, 0.f, 0.f );
-			if( BM * 4 % Threads == 0 || slot < BM * 4 ) {
+			if( ATotal % Threads == 0 || slot < ATotal ) {
 				if( AMODE == AM_RowsK ) {
-					const int m = m0 + ( slot >> 2 );
-					const int k = kBase + ( slot & 3 ) * 4;
+					const int m = m0 + slot / KQ;
+					const int k = kBase + ( slot % KQ ) * 4;
 					if( m < M ) {
 						const float* p = A + static_cast<long long>( m ) * args.Lda + k;
-						if( VEC ) {
-							if( k < K ) {
-								v = *reinterpret_cast<const float4*>( p );
-							}
-						} else {
-							if( k < K ) v.x = p[0];
-							if( k + 1 < K ) v.y = p[1];
-							if( k + 2 < K ) v.z = p[2];
-							if( k + 3 < K ) v.w = p[3];
-						}
+						if( k < K ) v.x = p[0];
+						if( k + 1 < K ) v.y = p[1];
+						if( k + 2 < K ) v.z = p[2];
+						if( k + 3 < K ) v.w = p[3];
 					}
 				} else if( AMODE == AM_RowsM ) {
 					const int k = kBase + slot / ( BM / 4 );
 					const int m = m0 + ( slot % ( BM / 4 ) ) * 4;
 					if( k < K ) {
 						const float* p = A + static_cast<long long>( k ) * args.Lda + m;
-						if( VEC ) {
-							if( m < M ) {
-								v = *reinterpret_cast<const float4*>( p );
-							}
-						} else {
-							if( m < M ) v.x = p[0];
-							if( m + 1 < M ) v.y = p[1];
-							if( m + 2 < M ) v.z = p[2];
-							if( m + 3 < M ) v.w = p[3];
-						}
+						if( m < M ) v.x = p[0];
+						if( m + 1 < M ) v.y = p[1];
+						if( m + 2 < M ) v.z = p[2];
+						if( m + 3 < M ) v.w = p[3];
 					}
-				} else { // AM_Conv
-					if( VEC ) {
-						// Cin % 4 == 0: the four k of a slot share one filter tap
-						const int hi = convH0[i] + convKh * args.DilH;
-						const int wi = convW0[i] + convKw * args.DilW;
-						if( kBase + ( tid & 3 ) * 4 < K && hi >= 0 && hi < args.H && wi >= 0 && wi < args.W ) {
-							v = *reinterpret_cast<const float4*>(
-								A + convBase[i] + ( hi * args.W + wi ) * args.Cin + convCi );
-						}
-					} else {
-						const int k = kBase + ( slot & 3 ) * 4;
-						v.x = loadConvElement( i, k );
-						v.y = loadConvElement( i, k + 1 );
-						v.z = loadConvElement( i, k + 2 );
-						v.w = loadConvElement( i, k + 3 );
-					}
+				} else {
+					const int k = kBase + ( slot % KQ ) * 4;
+					v.x = loadConvElement( i, k );
+					v.y = loadConvElement( i, k + 1 );
+					v.z = loadConvElement( i, k + 2 );
+					v.w = loadConvElement( i, k + 3 );
 				}
 			}
 			regA[i] = v;
 		}
-		if( AMODE == AM_Conv && VEC ) {
-			convCi += KStep;
-			while( convCi >= args.Cin ) {
-				convCi -= args.Cin;
-				if( ++convKw == args.Fw ) {
-					convKw = 0;
-					++convKh;
-				}
-			}
-		}
-		// ---- B ----
 #pragma unroll
 		for( int i = 0; i < BSlots; ++i ) {
 			const int slot = tid + i * Threads;
 			float4 v = make_float4( 0.f, 0.f, 0.f, 0.f );
-			if( BN * 4 % Threads == 0 || slot < BN * 4 ) {
+			if( BTotal % Threads == 0 || slot < BTotal ) {
 				if( BMODE == BM_RowsK ) {
-					const int n = n0 + ( slot >> 2 );
-					const int k = kBase + ( slot & 3 ) * 4;
+					const int n = n0 + slot / KQ;
+					const int k = kBase + ( slot % KQ ) * 4;
 					if( n < N ) {
 						const float* p = B + static_cast<long long>( n ) * args.Ldb + k;
-						if( VEC ) {
-							if( k < K ) {
-								v = *reinterpret_cast<const float4*>( p );
-							}
-						} else {
-							if( k < K ) v.x = p[0];
-							if( k + 1 < K ) v.y = p[1];
-							if( k + 2 < K ) v.z = p[2];
-							if( k + 3 < K ) v.w = p[3];
-						}
+						if( k < K ) v.x = p[0];
+						if( k + 1 < K ) v.y = p[1];
+						if( k + 2 < K ) v.z = p[2];
+						if( k + 3 < K ) v.w = p[3];
 					}
 				} else {
 					const int k = kBase + slot / ( BN / 4 );
 					const int n = n0 + ( slot % ( BN / 4 ) ) * 4;
 					if( k < K ) {
 						const float* p = B + static_cast<long long>( k ) * args.Ldb + n;
-						if( VEC ) {
-							if( n < N ) {
-								v = *reinterpret_cast<const float4*>( p );
-							}
-						} else {
-							if( n < N ) v.x = p[0];
-							if( n + 1 < N ) v.y = p[1];
-							if( n + 2 < N ) v.z = p[2];
-							if( n + 3 < N ) v.w = p[3];
-						}
+						if( n < N ) v.x = p[0];
+						if( n + 1 < N ) v.y = p[1];
+						if( n + 2 < N ) v.z = p[2];
+						if( n + 3 < N ) v.w = p[3];
 					}
 				}
 			}
@@ -266,28 +334,26 @@ void matMulKernel( const CMatMulArgs args )
 		}
 	};
 
-	auto storeTiles = [&]( int buf ) {
+	auto storeTiles = [&]( int buf, const float4 ( &regA )[ASlots], const float4 ( &regB )[BSlots] ) {
 #pragma unroll
 		for( int i = 0; i < ASlots; ++i ) {
 			const int slot = tid + i * Threads;
-			if( BM * 4 % Threads == 0 || slot < BM * 4 ) {
+			if( ATotal % Threads == 0 || slot < ATotal ) {
 				if( AK ) {
-					*reinterpret_cast<float4*>( &ldsA[buf][( slot >> 2 ) * LdsK + ( slot & 3 ) * 4] ) = regA[i];
+					*reinterpret_cast<float4*>( &ldsA[buf][( slot / KQ ) * LdsK + ( slot % KQ ) * 4] ) = regA[i];
 				} else {
-					*reinterpret_cast<float4*>( &ldsA[buf][( slot / ( BM / 4 ) ) * CTileLds<BM>::XMajorPitch
-						+ ( slot % ( BM / 4 ) ) * 4] ) = regA[i];
+					*reinterpret_cast<float4*>( &ldsA[buf][( slot / ( BM / 4 ) ) * APitchX + ( slot % ( BM / 4 ) ) * 4] ) = regA[i];
 				}
 			}
 		}
 #pragma unroll
 		for( int i = 0; i < BSlots; ++i ) {
 			const int slot = tid + i * Threads;
-			if( BN * 4 % Threads == 0 || slot < BN * 4 ) {
+			if( BTotal % Threads == 0 || slot < BTotal ) {
 				if( BK ) {
-					*reinterpret_cast<float4*>( &ldsB[buf][( slot >> 2 ) * LdsK + ( slot & 3 ) * 4] ) = regB[i];
+					*reinterpret_cast<float4*>( &ldsB[buf][( slot / KQ ) * LdsK + ( slot % KQ ) * 4] ) = regB[i];
 				} else {
-					*reinterpret_cast<float4*>( &ldsB[buf][( slot / ( BN / 4 ) ) * CTileLds<BN>::XMajorPitch
-						+ ( slot % ( BN / 4 ) ) * 4] ) = regB[i];
+					*reinterpret_cast<float4*>( &ldsB[buf][( slot / ( BN / 4 ) ) * BPitchX + ( slot % ( BN / 4 ) ) * 4] ) = regB[i];
 				}
 			}
 		}
@@ -305,66 +371,99 @@ void matMulKernel( const CMatMulArgs args )
 		}
 	}
 
-	const int kSteps = ( K + KStep - 1 ) / KStep;
-	loadTiles( 0 );
-	storeTiles( 0 );
-	__syncthreads();
-
-	for( int ks = 0; ks < kSteps; ++ks ) {
-		const int cur = ks & 1;
-		if( ks + 1 < kSteps ) {
-			loadTiles( ( ks + 1 ) * KStep );
-		}
-		const float* tA = ldsA[cur];
-		const float* tB = ldsB[cur];
+	// Fragments of one group of 8 k values: four MFMA operands per 32-row block of A and of B.
+	struct CFrag {
+		float A[MI][4];
+		float B[NI][4];
+	};
+	auto readFrag = [&]( int buf, int kc, CFrag& f ) {
+		const float* tA = ldsA[buf];
+		const float* tB = ldsB[buf];
 #pragma unroll
-		for( int kc = 0; kc < 2; ++kc ) {
-			float fa[MI][4];
-			float fb[NI][4];
+		for( int mi = 0; mi < MI; ++mi ) {
+			const int row = waveM * WM + mi * 32 + l32;
+			if( AK ) {
+				const float4 v = *reinterpret_cast<const float4*>( &tA[row * LdsK + kc * 8 + half * 4] );
+				f.A[mi][0] = v.x; f.A[mi][1] = v.y; f.A[mi][2] = v.z; f.A[mi][3] = v.w;
+			} else {
+#pragma unroll
+				for( int j = 0; j < 4; ++j ) {
+					f.A[mi][j] = tA[( kc * 8 + half * 4 + j ) * APitchX + row];
+				}
+			}
+		}
+#pragma unroll
+		for( int ni = 0; ni < NI; ++ni ) {
+			const int col = waveN * WN + ni * 32 + l32;
+			if( BK ) {
+				const float4 v = *reinterpret_cast<const float4*>( &tB[col * LdsK + kc * 8 + half * 4] );
+				f.B[ni][0] = v.x; f.B[ni][1] = v.y; f.B[ni][2] = v.z; f.B[ni][3] = v.w;
+			} else {
+#pragma unroll
+				for( int j = 0; j < 4; ++j ) {
+					f.B[ni][j] = tB[( kc * 8 + half * 4 + j ) * BPitchX + col];
+				}
+			}
+		}
+	};
+	auto multiply = [&]( const CFrag& f ) {
+#pragma unroll
+		for( int j = 0; j < 4; ++j ) {
 #pragma unroll
 			for( int mi = 0; mi < MI; ++mi ) {
-				const int row = waveM * WM + mi * 32 + l32;
-				if( AK ) {
-					const float4 v = *reinterpret_cast<const float4*>( &tA[row * LdsK + kc * 8 + half * 4] );
-					fa[mi][0] = v.x; fa[mi][1] = v.y; fa[mi][2] = v.z; fa[mi][3] = v.w;
-				} else {
 #pragma unroll
-					for( int j = 0; j < 4; ++j ) {
-						fa[mi][j] = tA[( kc * 8 + half * 4 + j ) * CTileLds<BM>::XMajorPitch + row];
-					}
-				}
-			}
-#pragma unroll
-			for( int ni = 0; ni < NI; ++ni ) {
-				const int col = waveN * WN + ni * 32 + l32;
-				if( BK ) {
-					const float4 v = *reinterpret_cast<const float4*>( &tB[col * LdsK + kc * 8 + half * 4] );
-					fb[ni][0] = v.x; fb[ni][1] = v.y; fb[ni][2] = v.z; fb[ni][3] = v.w;
-				} else {
-#pragma unroll
-					for( int j = 0; j < 4; ++j ) {
-						fb[ni][j] = tB[( kc * 8 + half * 4 + j ) * CTileLds<BN>::XMajorPitch + col];
-					}
-				}
-			}
-#pragma unroll
-			for( int j = 0; j < 4; ++j ) {
-#pragma unroll
-				for( int mi = 0; mi < MI; ++mi ) {
-#pragma unroll
-					for( int ni = 0; ni < NI; ++ni ) {
-						acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32( fa[mi][j], fb[ni][j], acc[mi][ni], 0, 0, 0 );
-					}
+				for( int ni = 0; ni < NI; ++ni ) {
+					acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32( f.A[mi][j], f.B[ni][j], acc[mi][ni], 0, 0, 0 );
 				}
 			}
 		}
+	};
+
+	// Software pipeline over K steps of KS, three LDS buffers, one barrier per step:
+	//   top of step ks : the tiles of step ks+1 (loaded from memory during step ks-1) go to LDS buffer (ks+1)%3, then
+	//                    the loads of step ks+2 are issued;
+	//   body           : the MFMAs of each group of 8 k run while the fragments of the following group are being
+	//                    read from LDS; the barrier sits before the last group, after which the first fragments of
+	//                    step ks+1 are fetched, so neither the LDS latency nor the barrier leaves the MFMA pipe idle.
+	// Buffer (ks+1)%3 was last read in step ks-2, and every wave has passed the barrier of step ks-1 since.
+	const int kSteps = ( K + KS - 1 ) / KS;
+	constexpr int Groups = KS / 8;
+	float4 rA[ASlots], rB[BSlots];
+	CFrag frag[2];
+	loadTiles( 0, rA, rB );
+	storeTiles( 0, rA, rB );
+	if( kSteps > 1 ) {
+		loadTiles( KS, rA, rB );
+	}
+	__syncthreads();
+	readFrag( 0, 0, frag[0] );
+	int cur = 0;
+	for( int ks = 0; ks < kSteps; ++ks ) {
+		const int nxt = cur == 2 ? 0 : cur + 1;
 		if( ks + 1 < kSteps ) {
-			storeTiles( cur ^ 1 );
+			storeTiles( nxt, rA, rB );
 		}
-		__syncthreads();
+		if( ks + 2 < kSteps ) {
+			loadTiles( ( ks + 2 ) * KS, rA, rB );
+		}
+		__builtin_amdgcn_sched_barrier( 0 );
+#pragma unroll
+		for( int g = 0; g < Groups; ++g ) {
+			if( g + 1 < Groups ) {
+				readFrag( cur, g + 1, frag[( g + 1 ) & 1] );
+			} else {
+				__syncthreads();
+				if( ks + 1 < kSteps ) {
+					readFrag( nxt, 0, frag[( g + 1 ) & 1] );
+				}
+			}
+			__builtin_amdgcn_sched_barrier( 0 );
+			multiply( frag[g & 1] );
+			__builtin_amdgcn_sched_barrier( 0 );
+		}
+		cur = nxt;
 	}
 
-	// ---- epilogue: accumulator register r of lane holds row 8*(r/4) + 4*half + r%4, column lane%32 ----------
 #pragma unroll
 	for( int ni = 0; ni < NI; ++ni ) {
 		const int n = n0 + waveN * WN + ni * 32 + l32;
@@ -447,6 +546,12 @@ static int launchMatMul( hipStream_t stream, CMatMulArgs& args, int batch, bool 
 	return launchTile<128, 32, 4, 1, AMODE, BMODE>( stream, args, batch, vec );
 }
 
+// The vector path addresses each operand with 32-bit byte offsets below BufferBytes.
+static bool fitsBuffer( long long rows, long long pitch, long long width )
+{
+	return rows <= 0 || ( ( rows - 1 ) * pitch + width ) * 4 < static_cast<long long>( BufferBytes );
+}
+
 // C = A * B^T (+ bias) with row strides; also the inner product of the convolution with a 1x1 filter.
 int matMulNT( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
 	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC,
@@ -462,7 +567,7 @@ int matMulNT( hipStream_t stream, const float* a, int lda, const float* b, int l
 	args.BatchStrideA = strideA; args.BatchStrideB = strideB; args.BatchStrideC = strideC;
 	args.Accumulate = accumulate ? 1 : 0;
 	const bool vec = isAligned16( a ) && isAligned16( b ) && K % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0
-		&& strideA % 4 == 0 && strideB % 4 == 0;
+		&& strideA % 4 == 0 && strideB % 4 == 0 && fitsBuffer( M, lda, K ) && fitsBuffer( N, ldb, K );
 	return launchMatMul<AM_RowsK, BM_RowsK>( stream, args, batch, vec );
 }
 
@@ -480,7 +585,7 @@ int matMulNN( hipStream_t stream, const float* a, int lda, const float* b, int l
 	args.BatchStrideA = strideA; args.BatchStrideB = strideB; args.BatchStrideC = strideC;
 	args.Accumulate = accumulate ? 1 : 0;
 	const bool vec = isAligned16( a ) && isAligned16( b ) && K % 4 == 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0
-		&& strideA % 4 == 0 && strideB % 4 == 0;
+		&& strideA % 4 == 0 && strideB % 4 == 0 && fitsBuffer( M, lda, K ) && fitsBuffer( K, ldb, N );
 	return launchMatMul<AM_RowsK, BM_RowsN>( stream, args, batch, vec );
 }
 
@@ -498,7 +603,7 @@ int matMulTN( hipStream_t stream, const float* a, int lda, const float* b, int l
 	args.BatchStrideA = strideA; args.BatchStrideB = strideB; args.BatchStrideC = strideC;
 	args.Accumulate = accumulate ? 1 : 0;
 	const bool vec = isAligned16( a ) && isAligned16( b ) && M % 4 == 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0
-		&& strideA % 4 == 0 && strideB % 4 == 0;
+		&& strideA % 4 == 0 && strideB % 4 == 0 && fitsBuffer( K, lda, M ) && fitsBuffer( K, ldb, N );
 	return launchMatMul<AM_RowsM, BM_RowsN>( stream, args, batch, vec );
 }
 
@@ -513,14 +618,16 @@ int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* sour
 	args.K = d.filterHeight * d.filterWidth * d.channels;
 	args.Lda = 0; args.Ldb = args.K; args.Ldc = d.filterCount;
 	args.H = d.height; args.W = d.width; args.Cin = d.channels;
-	args.Ho = d.resultHeight; args.Wo = d.resultWidth; args.Fw = d.filterWidth;
+	args.Ho = d.resultHeight; args.Wo = d.resultWidth; args.Fh = d.filterHeight; args.Fw = d.filterWidth;
 	args.PadH = d.paddingHeight; args.PadW = d.paddingWidth;
 	args.StrideH = d.strideHeight; args.StrideW = d.strideWidth;
 	args.DilH = d.dilationHeight; args.DilW = d.dilationWidth;
 	if( args.M == 0 || args.N == 0 ) {
 		return NH_OK;
 	}
-	const bool vec = isAligned16( source ) && isAligned16( filter ) && d.channels % 4 == 0;
+	const bool vec = isAligned16( source ) && isAligned16( filter ) && d.channels % 4 == 0
+		&& fitsBuffer( 1, 0, static_cast<long long>( d.batch ) * d.height * d.width * d.channels )
+		&& fitsBuffer( d.filterCount, args.K, args.K );
 	return launchMatMul<AM_Conv, BM_RowsK>( stream, args, 1, vec );
 }
 
