@@ -56,6 +56,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample", type=int, default=8, help="images in the CPU baseline sample")
     ap.add_argument("--per-kernel", action="store_true", help="print a per-op-family timing table to stderr")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one nhVectorCopy of 2^26 floats (256 MiB read + 256 MiB written): the known-size "
+                         "kernel that scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus)
@@ -69,6 +72,13 @@ def main():
     # the launches of one forward pass, arguments bound once: replaying them costs the host a few microseconds
     # per launch, so the timed region is bound by the GPU, not by the Python interpreter
     plan, out = net.record_plan(x)
+    if args.calibrate_copy:
+        import ctypes
+        src = be.empty(1 << 26).fill_(1.0)
+        dst = be.empty(1 << 26)
+        be.na.check(be.lib.nhVectorCopy(be.stream, ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()), 1 << 26))
+        torch.cuda.synchronize()
+        del src, dst
     timed_tags = None if args.per_kernel else ("conv3x3",)
     all_tags = set(t for _, _, t, _, _ in plan.launches if t)
     pools = plan.make_events(all_tags if timed_tags is None else timed_tags, args.steps)

@@ -1,0 +1,278 @@
+// CHipMathEngine: NeoML's IMathEngine on one MI355X.
+//
+// Host-side C++ adapter between NeoML (its layers call the virtual interface declared in
+// NeoMathEngine/NeoMathEngine.h) and the C ABI of libneoml_hip.so (include/neoml_hip.h): a handle is resolved to
+// a device pointer, blob descriptors to plain ints, and one nh* entry point is called per method. Device memory
+// goes through the caching pool of the C ABI, all work is enqueued on one HIP stream owned by the engine, and
+// errors are routed to NeoML's process-wide exception handler.
+//
+// Only the methods of the inference path are written here; the remaining pure virtuals get asserting bodies
+// generated at build time from the interface header (gen_stubs.py), as the reference's GPU engine does for
+// operations it lacks.
+//
+// Build: compiled against the public headers of the NeoML installation it plugs into; the symbols it needs from
+// libNeoMathEngine (CCrtAllocatedObject::operator new/delete, the interface destructors, the exception handler
+// accessor) are resolved from the host process at load time.
+#pragma once
+
+#include <NeoMathEngine/NeoMathEngine.h>
+
+#include <mutex>
+#include <thread>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/neoml_hip.h"
+
+namespace NeoML {
+
+// CMemoryHandle befriends a class of this name so that an engine can mint handles and read their pointer
+// (MemoryHandle.h:42-53); each engine implementation supplies its own definition.
+class CMemoryHandleInternal {
+public:
+	static void* GetRaw( const CMemoryHandle& handle )
+	{
+		return const_cast<char*>( static_cast<const char*>( handle.Object ) ) + handle.Offset;
+	}
+	static CMemoryHandle Create( IMathEngine* engine, const void* object )
+	{
+		return CMemoryHandle( engine, object, 0 );
+	}
+};
+
+template<class T>
+inline T* GetRaw( const CTypedMemoryHandle<T>& handle )
+{
+	return static_cast<T*>( CMemoryHandleInternal::GetRaw( handle ) );
+}
+
+class CHipMathEngine : public IMathEngine {
+public:
+	CHipMathEngine( int deviceIndex, size_t memoryLimit, int flags );
+	~CHipMathEngine() override;
+
+	// ---- IVectorMathEngine ----
+	void VectorCopy( const CFloatHandle& first, const CConstFloatHandle& second, int vectorSize ) override;
+	void VectorCopy( const CIntHandle& first, const CConstIntHandle& second, int vectorSize ) override;
+	void VectorFill( const CFloatHandle& result, float value, int vectorSize ) override;
+	void VectorFill( const CIntHandle& result, int value, int vectorSize ) override;
+	void VectorFill( const CFloatHandle& result, int vectorSize, const CConstFloatHandle& value ) override;
+	void VectorFill( const CIntHandle& result, int vectorSize, const CConstIntHandle& value ) override;
+	void VectorConvert( const CConstFloatHandle& from, const CIntHandle& to, int vectorSize ) override;
+	void VectorConvert( const CConstIntHandle& from, const CFloatHandle& to, int vectorSize ) override;
+	void VectorSum( const CConstFloatHandle& firstHandle, int vectorSize, const CFloatHandle& resultHandle ) override;
+	void VectorELU( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle,
+		int vectorSize, const CConstFloatHandle& alpha ) override;
+	void VectorReLU( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize,
+		const CConstFloatHandle& upperThresholdHandle ) override;
+	void VectorLeakyReLU( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle,
+		int vectorSize, const CConstFloatHandle& alpha ) override;
+	void VectorHSwish( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseMax( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseMin( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorAbs( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorHardTanh( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorHardSigmoid( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize,
+		const CConstFloatHandle& slopeHandle, const CConstFloatHandle& biasHandle ) override;
+	void VectorNeg( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorExp( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorLog( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorErf( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorAdd( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorAdd( const CConstIntHandle& firstHandle, const CConstIntHandle& secondHandle,
+		const CIntHandle& resultHandle, int vectorSize ) override;
+	void VectorAddValue( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize,
+		const CConstFloatHandle& addition ) override;
+	void VectorAddValue( const CConstIntHandle& firstHandle, const CIntHandle& resultHandle, int vectorSize,
+		const CConstIntHandle& addition ) override;
+	void VectorSub( const CConstIntHandle& firstHandle, const CConstIntHandle& secondHandle,
+		const CIntHandle& resultHandle, int vectorSize ) override;
+	void VectorSub( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorMultiplyAndAdd( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& multHandle ) override;
+	void VectorMultiplyAndSub( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& multHandle ) override;
+	void VectorMultiply( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize,
+		const CConstFloatHandle& multiplierHandle ) override;
+	void VectorMultiply( const CConstIntHandle& firstHandle, const CIntHandle& resultHandle, int vectorSize,
+		const CConstIntHandle& multiplierHandle ) override;
+	void VectorNegMultiply( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize,
+		const CConstFloatHandle& multiplierHandle ) override;
+	void VectorEltwiseMultiply( const CConstIntHandle& firstHandle, const CConstIntHandle& secondHandle,
+		const CIntHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseMultiply( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseMultiplyAdd( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseNegMultiply( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseDivide( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorSqrt( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorInv( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorMinMax( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize,
+		const CConstFloatHandle& minHandle, const CConstFloatHandle& maxHandle ) override;
+	void VectorSigmoid( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorTanh( const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorDotProduct( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle, int vectorSize,
+		const CFloatHandle& resultHandle ) override;
+
+	// ---- IBlasEngine ----
+	void SetVectorToMatrixRows( const CFloatHandle& resultHandle, int matrixHeight, int matrixWidth,
+		const CConstFloatHandle& vectorHandle ) override;
+	void AddVectorToMatrixRows( int batchSize, const CConstFloatHandle& matrixHandle, const CFloatHandle& resultHandle,
+		int matrixHeight, int matrixWidth, const CConstFloatHandle& vectorHandle ) override;
+	void AddVectorToMatrixColumns( const CConstFloatHandle& matrixHandle, const CFloatHandle& resultHandle,
+		int matrixHeight, int matrixWidth, const CConstFloatHandle& vectorHandle ) override;
+	void SubVectorFromMatrixColumns( const CConstFloatHandle& matrixHandle, const CFloatHandle& resultHandle,
+		int matrixHeight, int matrixWidth, const CConstFloatHandle& vectorHandle ) override;
+	void SumMatrixRowsAdd( int batchSize, const CFloatHandle& resultHandle, const CConstFloatHandle& matrixHandle,
+		int matrixHeight, int matrixWidth ) override;
+	void SumMatrixRows( int batchSize, const CFloatHandle& resultHandle, const CConstFloatHandle& matrixHandle,
+		int matrixHeight, int matrixWidth ) override;
+	void SumMatrixColumns( const CFloatHandle& resultHandle, const CConstFloatHandle& matrixHandle,
+		int matrixHeight, int matrixWidth ) override;
+	void MatrixLogSumExpByRows( const CConstFloatHandle& matrix, int height, int width, const CFloatHandle& result,
+		int resultSize ) override;
+	void MatrixSoftmaxByRows( const CConstFloatHandle& matrix, int height, int width, const CFloatHandle& result ) override;
+	void FindMaxValueInRows( const CConstFloatHandle& matrixHandle, int matrixHeight, int matrixWidth,
+		const CFloatHandle& resultHandle, const CIntHandle& columnIndices, int vectorSize ) override;
+	void FindMaxValueInRows( const CConstFloatHandle& matrixHandle, int matrixHeight, int matrixWidth,
+		const CFloatHandle& resultHandle, int vectorSize ) override;
+	void FindMaxValueInColumns( int batchSize, const CConstFloatHandle& matrixHandle, int matrixHeight,
+		int matrixWidth, const CFloatHandle& resultHandle, const CIntHandle& rowIndices, int vectorSize ) override;
+	void MultiplyMatrixByTransposedMatrix( const CConstFloatHandle& firstHandle, int firstHeight, int firstWidth,
+		int firstRowSize, const CConstFloatHandle& secondHandle, int secondHeight, int secondRowSize,
+		const CFloatHandle& resultHandle, int resultRowSize, int resultBufferSize ) override;
+	void MultiplyMatrixByTransposedMatrix( int batchSize, const CConstFloatHandle& firstHandle, int firstHeight,
+		int firstWidth, const CConstFloatHandle& secondHandle, int secondHeight, const CFloatHandle& resultHandle,
+		int resultBufferSize ) override;
+	void MultiplyTransposedMatrixByMatrixAndAdd( const CConstFloatHandle& firstHandle, int firstHeight, int firstWidth,
+		int firstRowSize, const CConstFloatHandle& secondHandle, int secondWidth, int secondRowSize,
+		const CFloatHandle& resultHandle, int resultRowSize, int resultBufferSize ) override;
+	void MultiplyTransposedMatrixByMatrix( int batchSize, const CConstFloatHandle& firstHandle, int firstHeight,
+		int firstWidth, const CConstFloatHandle& secondHandle, int secondWidth, const CFloatHandle& resultHandle,
+		int resultBufferSize ) override;
+	void MultiplyDiagMatrixByMatrix( const CConstFloatHandle& firstHandle, int firstSize,
+		const CConstFloatHandle& secondHandle, int secondWidth, const CFloatHandle& resultHandle,
+		int resultBufferSize ) override;
+	void MultiplyMatrixByMatrix( int batchSize, const CConstFloatHandle& firstHandle, int firstHeight, int firstWidth,
+		const CConstFloatHandle& secondHandle, int secondWidth, const CFloatHandle& resultHandle,
+		int resultBufferSize ) override;
+	void BatchMultiplyMatrixByDiagMatrix( int batchSize, const CConstFloatHandle& firstHandle, int height, int width,
+		int firstMatrixOffset, const CConstFloatHandle& secondHandle, int secondMatrixOffset,
+		const CFloatHandle& resultHandle, int resultBufferSize ) override;
+	void TransposeMatrix( int batchSize, const CConstFloatHandle& firstHandle, int height, int medium, int width,
+		int channels, const CFloatHandle& resultHandle, int resultBufferSize ) override;
+	void TransposeMatrix( int batchSize, const CConstIntHandle& firstHandle, int height, int medium, int width,
+		int channels, const CIntHandle& resultHandle, int resultBufferSize ) override;
+
+	// ---- IDnnEngine ----
+	void BlobMergeByDim( TBlobDim dim, const CBlobDesc* from, const CFloatHandle* fromData, int fromCount,
+		const CBlobDesc& to, const CFloatHandle& toData ) override;
+	void BlobMergeByDim( TBlobDim dim, const CBlobDesc* from, const CIntHandle* fromData, int fromCount,
+		const CBlobDesc& to, const CIntHandle& toData ) override;
+	void BlobSplitByDim( TBlobDim dim, const CBlobDesc& from, const CConstFloatHandle& fromData,
+		const CBlobDesc* to, const CFloatHandle* toData, int toCount ) override;
+	void BlobSplitByDim( TBlobDim dim, const CBlobDesc& from, const CConstIntHandle& fromData,
+		const CBlobDesc* to, const CIntHandle* toData, int toCount ) override;
+	void BlobResizeImage( const CBlobDesc& from, const CFloatHandle& fromData, int deltaLeft, int deltaRight,
+		int deltaTop, int deltaBottom, TBlobResizePadding padding, float defaultValue,
+		const CBlobDesc& to, const CFloatHandle& toData ) override;
+	CConvolutionDesc* InitBlobConvolution( const CBlobDesc& input, int paddingHeight, int paddingWidth,
+		int strideHeight, int strideWidth, int dilationHeight, int dilationWidth, const CBlobDesc& filter,
+		const CBlobDesc& output ) override;
+	void BlobConvolution( const CConvolutionDesc& desc, const CConstFloatHandle& source,
+		const CConstFloatHandle& filter, const CConstFloatHandle* freeTerm, const CFloatHandle& result ) override;
+	CChannelwiseConvolutionDesc* InitBlobChannelwiseConvolution( const CBlobDesc& input, int paddingHeight,
+		int paddingWidth, int strideHeight, int strideWidth, const CBlobDesc& filter, const CBlobDesc* freeTerm,
+		const CBlobDesc& output ) override;
+	void BlobChannelwiseConvolution( const CChannelwiseConvolutionDesc& desc, const CConstFloatHandle& source,
+		const CConstFloatHandle& filter, const CConstFloatHandle* freeTerm, const CFloatHandle& result ) override;
+	CMaxPoolingDesc* InitMaxPooling( const CBlobDesc& source, int filterHeight, int filterWidth,
+		int strideHeight, int strideWidth, const CBlobDesc& result ) override;
+	void BlobMaxPooling( const CMaxPoolingDesc& desc, const CConstFloatHandle& source,
+		const CIntHandle* maxIndices, const CFloatHandle& result ) override;
+	CMeanPoolingDesc* InitMeanPooling( const CBlobDesc& source, int filterHeight, int filterWidth,
+		int strideHeight, int strideWidth, const CBlobDesc& result ) override;
+	void BlobMeanPooling( const CMeanPoolingDesc& desc, const CConstFloatHandle& source,
+		const CFloatHandle& result ) override;
+	CLstmDesc* InitLstm( int hiddenSize, int objectSize, const CConstFloatHandle& inputWeights,
+		const CConstFloatHandle& inputFreeTerm, const CConstFloatHandle& recurrentWeights,
+		const CConstFloatHandle& recurrentFreeTerm ) override;
+	void Lstm( CLstmDesc& desc, bool reverse, int sequenceLength, int sequenceCount,
+		const CConstFloatHandle& inputStateBackLink, const CConstFloatHandle& inputMainBackLink,
+		const CConstFloatHandle& input, const CFloatHandle& outputStateBackLink,
+		const CFloatHandle& outputMainBackLink ) override;
+
+	// ---- IMathEngine ----
+	TMathEngineType GetType() const override;
+	void GetMathEngineInfo( CMathEngineInfo& info ) const override;
+	bool IsInitialized() const override;
+	void SetReuseMemoryMode( bool enable ) override;
+	bool GetReuseMemoryMode() const override;
+	void SetThreadBufferMemoryThreshold( size_t threshold ) override;
+	size_t GetThreadBufferMemoryThreshold() const override;
+	CMemoryHandle HeapAlloc( size_t count ) override;
+	void HeapFree( const CMemoryHandle& handle ) override;
+	void TransferHandleToThisThread( const CMemoryHandle& handle, size_t size ) override;
+	CMemoryHandle StackAlloc( size_t count ) override;
+	void StackFree( const CMemoryHandle& handle ) override;
+	size_t GetFreeMemorySize() const override;
+	size_t GetPeakMemoryUsage() const override;
+	void ResetPeakMemoryUsage() override;
+	size_t GetCurrentMemoryUsage() const override;
+	size_t GetMemoryInPools() const override;
+	void CleanUp() override;
+	void* GetBuffer( const CMemoryHandle& handle, size_t pos, size_t size, bool exchange ) override;
+	void ReleaseBuffer( const CMemoryHandle& handle, void* ptr, bool exchange ) override;
+	void DataExchangeRaw( const CMemoryHandle& result, const void* source, size_t size ) override;
+	void DataExchangeRaw( void* result, const CMemoryHandle& source, size_t size ) override;
+	CMemoryHandle CopyFrom( const CMemoryHandle& handle, size_t size ) override;
+	IPerformanceCounters* CreatePerformanceCounters( bool isTimeOnly ) const override;
+	void AllReduce( const CFloatHandle& handle, int size ) override;
+	void Broadcast( const CFloatHandle& handle, int size, int root ) override;
+
+	// Waits for the engine's stream (used by the performance counters)
+	void Synchronize() const;
+
+	// every other pure virtual of the interface: asserting bodies generated from the interface header
+#include "HipMathEngineStubs.inc"
+
+protected:
+	void CleanUpSpecial() override;
+
+private:
+	const int device;
+	const size_t memoryLimit;
+	nhStream stream;
+	nhPool pool;
+	size_t deviceTotalMemory;
+	char deviceName[256];
+	bool initialized;
+
+	// pinned host staging blocks handed out by GetBuffer, per thread, strictly LIFO
+	struct CHostBuffer {
+		char* Ptr;
+		size_t Size;
+	};
+	mutable std::mutex hostMutex;
+	std::unordered_map<std::thread::id, std::vector<CHostBuffer>> hostBuffers;
+
+	void check( int code, const char* what, int line ) const;
+	template<class T> T* raw( const CTypedMemoryHandle<T>& handle ) const;
+	void* rawBytes( const CMemoryHandle& handle ) const;
+};
+
+} // namespace NeoML
+
+// Creates the engine on the given device (the factory a host application binds; mirrors
+// IGpuMathEngineManager::CreateMathEngine( index, memoryLimit, flags ), NeoMathEngine.h:1299).
+// Returns null instead of throwing. The engine is destroyed by the caller with delete.
+extern "C" __attribute__( ( visibility( "default" ) ) )
+NeoML::IMathEngine* CreateHipMathEngine( int deviceIndex, size_t memoryLimit, int flags );
+extern "C" __attribute__( ( visibility( "default" ) ) ) int GetHipMathEngineCount();

@@ -600,3 +600,14 @@ SHIM_API int shim_clean_up( void* engine )
 {
 	return guarded( [&]() { static_cast<IMathEngine*>( engine )->CleanUp(); } );
 }
+
+// probe for a method outside the inference path (asserts on engines that do not implement it)
+SHIM_API int shim_vector_huber( void* engine, const float* first, float* result, int n )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		CFloatBlob in( e, n, first ), out( e, n );
+		e.VectorHuber( in.Const(), out.Handle(), n );
+		out.CopyTo( result );
+	} );
+}

@@ -91,6 +91,30 @@ def cpu_engine():
     return _cpu_engine
 
 
+ENGINE_LIB = os.path.join(ROOT, "neoml_amd", "lib", "libNeoMathEngineHip.so")
+REF_ENGINE_LIB = os.path.join(ORACLE_DIR, "_ref", "libNeoMathEngine.so")
+_hip_engine = None
+
+
+def have_engine_adapter():
+    return os.path.exists(ENGINE_LIB) and have_reference()
+
+
+def hip_engine():
+    """The CHipMathEngine adapter, created through its C factory. The host process must already hold NeoML's
+    libNeoMathEngine (here: the reference build under oracle/_ref), whose symbols the adapter resolves at load."""
+    global _hip_engine
+    if _hip_engine is None:
+        ctypes.CDLL(REF_ENGINE_LIB, mode=ctypes.RTLD_GLOBAL)
+        lib = ctypes.CDLL(ENGINE_LIB, mode=ctypes.RTLD_GLOBAL)
+        lib.CreateHipMathEngine.restype = ctypes.c_void_p
+        lib.CreateHipMathEngine.argtypes = [ctypes.c_int, ctypes.c_size_t, ctypes.c_int]
+        ptr = lib.CreateHipMathEngine(0, 0, 0)
+        assert ptr, "CreateHipMathEngine returned null"
+        _hip_engine = ctypes.c_void_p(ptr)
+    return _hip_engine
+
+
 def conv_out(h, w, fh, fw, ph, pw, sh, sw, dh=1, dw=1):
     ho = 1 + (h - (fh - 1) * dh + 2 * ph - 1) // sh
     wo = 1 + (w - (fw - 1) * dw + 2 * pw - 1) // sw
@@ -101,16 +125,24 @@ class Cpu:
     """Numpy front-end shared by the oracle ('orc') and the reference engine through the shim ('ref')."""
 
     def __init__(self, kind):
-        assert kind in ("orc", "ref")
-        self.kind = kind
+        # 'orc': the C oracle; 'ref': the reference CPU engine through the shim; 'hipeng': the HIP engine adapter
+        # through the very same shim calls (exercises the IMathEngine boundary; needs a GPU)
+        assert kind in ("orc", "ref", "hipeng")
         self.lib = oracle() if kind == "orc" else shim()
         self.pre = "orc_" if kind == "orc" else "shim_"
-        self.eng = () if kind == "orc" else (cpu_engine(),)
+        if kind == "orc":
+            self.eng = ()
+        elif kind == "ref":
+            self.eng = (cpu_engine(),)
+        else:
+            self.eng = (hip_engine(),)
+        self.kind = "orc" if kind == "orc" else "ref"  # call convention: direct oracle or through the shim
+        self.name = kind
 
     def _call(self, name, *args):
         rc = getattr(self.lib, self.pre + name)(*self.eng, *args)
         if self.kind == "ref" and rc != 0:
-            raise RuntimeError("reference engine: " + self.lib.shim_last_error().decode())
+            raise RuntimeError("%s engine: %s" % (self.name, self.lib.shim_last_error().decode()))
         return rc
 
     # ---- element-wise

@@ -1,0 +1,141 @@
+"""The drop-in boundary: CHipMathEngine (neoml_amd/engine) driven through NeoML's virtual IMathEngine interface by
+the same shim calls that drive the reference's CCpuMathEngine, both engines living in one process. Every case
+compares the two engines on identical inputs (and with the C oracle)."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import nhtest
+from nhtest import Cpu, assert_close
+from test_oracle import UNARY_CASES, BINARY_CASES, unary_input, rng
+
+pytestmark = [pytest.mark.gpu,
+              pytest.mark.skipif(not nhtest.have_engine_adapter(), reason="engine adapter or oracle/_ref not built")]
+
+
+def engines():
+    return Cpu("hipeng"), Cpu("ref")
+
+
+def test_engine_identity_and_memory_interface():
+    hip, _ = engines()
+    s = nhtest.shim()
+    assert s.shim_engine_type(nhtest.hip_engine()) == 2  # MET_Cuda: the generic GPU value of TMathEngineType
+    peak, cur, pools = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    x = np.ones(1000, np.float32)
+    hip.unary("relu", x)  # allocates and frees blobs through HeapAlloc / HeapFree
+    assert s.shim_memory_stats(nhtest.hip_engine(), ctypes.byref(peak), ctypes.byref(cur), ctypes.byref(pools)) == 0
+    assert peak.value >= 4096 and pools.value > 0 and cur.value >= pools.value  # freed blobs stay cached
+    assert s.shim_clean_up(nhtest.hip_engine()) == 0
+    assert s.shim_memory_stats(nhtest.hip_engine(), ctypes.byref(peak), ctypes.byref(cur), ctypes.byref(pools)) == 0
+    assert pools.value == 0
+
+
+@pytest.mark.parametrize("op,p0,p1", UNARY_CASES)
+def test_unary(op, p0, p1):
+    hip, ref = engines()
+    x = unary_input(op, 4099, 3)
+    assert_close(hip.unary(op, x, p0, p1), ref.unary(op, x, p0, p1), op)
+
+
+@pytest.mark.parametrize("op", BINARY_CASES)
+def test_binary(op):
+    hip, ref = engines()
+    g = rng(2)
+    a = g.uniform(-10, 10, 5003).astype(np.float32)
+    b = g.uniform(0.5, 10, 5003).astype(np.float32)
+    r = g.uniform(-10, 10, 5003).astype(np.float32)
+    assert_close(hip.binary(op, a, b, 0.37, result=r), ref.binary(op, a, b, 0.37, result=r), op)
+
+
+def test_blas_family():
+    hip, ref = engines()
+    g = rng(5)
+    m = g.uniform(-10, 10, (3, 17, 64)).astype(np.float32)
+    v = g.uniform(-10, 10, (3, 64)).astype(np.float32)
+    col = g.uniform(-1, 1, 17).astype(np.float32)
+    assert_close(hip.add_vector_to_matrix_rows(m, v), ref.add_vector_to_matrix_rows(m, v), "add rows")
+    assert_close(hip.add_vector_to_matrix_columns(m[0], col), ref.add_vector_to_matrix_columns(m[0], col), "add cols")
+    assert_close(hip.sum_matrix_rows(m), ref.sum_matrix_rows(m), "sum rows", atol=1e-4)
+    assert_close(hip.sum_matrix_columns(m[0]), ref.sum_matrix_columns(m[0]), "sum cols", atol=1e-4)
+    assert_close(hip.multiply_diag_matrix_by_matrix(col, m[0]), ref.multiply_diag_matrix_by_matrix(col, m[0]), "diag")
+    assert_close(hip.batch_multiply_matrix_by_diag_matrix(3, m, 17, 64, 17 * 64, v, 64),
+                 ref.batch_multiply_matrix_by_diag_matrix(3, m, 17, 64, 17 * 64, v, 64), "diag right")
+    assert_close(hip.softmax_rows(m[0]), ref.softmax_rows(m[0]), "softmax")
+    p = g.permutation(64 * 101).reshape(64, 101).astype(np.float32)
+    hv, hi = hip.find_max_in_rows(p)
+    rv, ri = ref.find_max_in_rows(p)
+    assert np.array_equal(hi, ri) and np.array_equal(hv, rv)
+    x = g.uniform(-1, 1, (2, 16, 1, 8, 64)).astype(np.float32)
+    assert np.array_equal(hip.transpose(x), ref.transpose(x))
+
+
+def test_matrix_products():
+    hip, ref = engines()
+    g = rng(9)
+    M, N, K = 130, 70, 96
+    a = g.uniform(-1, 1, (M, K)).astype(np.float32)
+    b = g.uniform(-1, 1, (N, K)).astype(np.float32)
+    kw = dict(lda=K, ldb=K, ldc=N, M=M, N=N, K=K)
+    assert_close(hip.matmul("nt", a, b, **kw), ref.matmul("nt", a, b, **kw), "nt")
+    a3 = g.uniform(-1, 1, (4, 33, 20)).astype(np.float32)
+    bn = g.uniform(-1, 1, (4, 20, 24)).astype(np.float32)
+    bt = g.uniform(-1, 1, (4, 24, 20)).astype(np.float32)
+    at = g.uniform(-1, 1, (4, 20, 33)).astype(np.float32)
+    for kind, x, y in (("bnn", a3, bn), ("bnt", a3, bt), ("btn", at, bn)):
+        kw = dict(M=33, N=24, K=20, batch=4)
+        assert_close(hip.matmul(kind, x, y, **kw), ref.matmul(kind, x, y, **kw), kind)
+
+
+def test_convolution_pooling_resize_split():
+    hip, ref = engines()
+    g = rng(10)
+    x = g.uniform(-1, 1, (2, 16, 16, 32)).astype(np.float32)
+    f = g.normal(0, 0.1, (48, 3, 3, 32)).astype(np.float32)
+    bias = g.uniform(-1, 1, 48).astype(np.float32)
+    assert_close(hip.conv(x, f, bias, 1, 1, 1, 1), ref.conv(x, f, bias, 1, 1, 1, 1), "conv 3x3")
+    assert_close(hip.conv(x, f, None, 1, 1, 2, 2), ref.conv(x, f, None, 1, 1, 2, 2), "conv 3x3/2, no free term")
+    xs = g.uniform(0, 1, (2, 20, 20, 3)).astype(np.float32)
+    fs = g.normal(0, 0.1, (16, 7, 7, 3)).astype(np.float32)
+    assert_close(hip.conv(xs, fs, None, 3, 3, 2, 2), ref.conv(xs, fs, None, 3, 3, 2, 2), "conv 7x7/2")
+    fc = g.normal(0, 1, (3, 3, 32)).astype(np.float32)
+    cb = g.uniform(-1, 1, 32).astype(np.float32)
+    assert_close(hip.channelwise_conv(x, fc, cb, 1, 1, 2, 2), ref.channelwise_conv(x, fc, cb, 1, 1, 2, 2), "channelwise")
+    assert np.array_equal(hip.max_pool(x, 3, 3, 2, 2), ref.max_pool(x, 3, 3, 2, 2))
+    hy, hidx = hip.max_pool(x, 2, 2, 2, 2, with_indices=True)
+    ry, ridx = ref.max_pool(x, 2, 2, 2, 2, with_indices=True)
+    assert np.array_equal(hy, ry) and np.array_equal(hidx, ridx)
+    assert_close(hip.mean_pool(x, 2, 2, 2, 2), ref.mean_pool(x, 2, 2, 2, 2), "mean pool")
+    assert np.array_equal(hip.resize_image(x, 1, 1, 1, 1, 0, 0.0), ref.resize_image(x, 1, 1, 1, 1, 0, 0.0))
+    big = g.uniform(-1, 1, (1, 8, 1, 1, 1, 1, 64)).astype(np.float32)
+    dims = [(1, 8, 1, 1, 1, 1, 16)] * 4
+    for p, q in zip(hip.split(big, 6, dims), ref.split(big, 6, dims)):
+        assert np.array_equal(p, q)
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+def test_lstm_through_the_interface(reverse):
+    hip, ref = engines()
+    g = rng(18)
+    T, B, In, H = 6, 8, 32, 64
+    w_in = g.uniform(-0.2, 0.2, (4 * H, In)).astype(np.float32)
+    w_rec = g.uniform(-0.2, 0.2, (4 * H, H)).astype(np.float32)
+    b_in = g.uniform(-0.5, 0.5, 4 * H).astype(np.float32)
+    b_rec = g.uniform(-0.5, 0.5, 4 * H).astype(np.float32)
+    x = g.uniform(-1, 1, (T, B, In)).astype(np.float32)
+    hh, hc = hip.lstm(w_in, b_in, w_rec, b_rec, x, reverse)
+    rh, rc = ref.lstm(w_in, b_in, w_rec, b_rec, x, reverse)
+    assert_close(hh, rh, "lstm h")
+    assert_close(hc, rc, "lstm c")
+
+
+def test_unimplemented_method_asserts_like_the_reference_gpu_engine():
+    # VectorHuber is outside the inference path: the generated body raises through NeoML's exception handler,
+    # which the shim turns into an error code instead of letting it cross the C boundary
+    s = nhtest.shim()
+    if not hasattr(s, "shim_vector_huber"):
+        pytest.skip("shim has no probe for an unimplemented method")
+    x = np.ones(8, np.float32)
+    y = np.empty(8, np.float32)
+    assert s.shim_vector_huber(nhtest.hip_engine(), nhtest.fp(x), nhtest.fp(y), 8) == 1
