@@ -27,7 +27,9 @@ namespace nh {
 
 typedef float f32x16 __attribute__( ( ext_vector_type( 16 ) ) );
 
-enum TAMode { AM_RowsK = 0, AM_RowsM = 1, AM_Conv = 2 };
+// AM_Conv1x1 runs the same code as AM_Conv; the separate value gives 1x1 convolutions their own kernel symbols, so
+// that profiles tell them apart from the 3x3 ones
+enum TAMode { AM_RowsK = 0, AM_RowsM = 1, AM_Conv = 2, AM_Conv1x1 = 3 };
 enum TBMode { BM_RowsK = 0, BM_RowsN = 1 };
 
 struct CMatMulArgs {
@@ -92,6 +94,7 @@ void matMulKernel( const CMatMulArgs args )
 	constexpr int MI = WM / 32;
 	constexpr int NI = WN / 32;
 	constexpr bool AK = ( AMODE != AM_RowsM );
+	constexpr bool IsConv = ( AMODE == AM_Conv || AMODE == AM_Conv1x1 );
 	constexpr bool BK = ( BMODE == BM_RowsK );
 	constexpr int APitchX = BM + 4, BPitchX = BN + 4;
 	constexpr int ASize = AK ? BM * LdsK : KS * APitchX;
@@ -166,7 +169,7 @@ void matMulKernel( const CMatMulArgs args )
 			}
 		}
 	}
-	if( AMODE == AM_Conv && VEC ) {
+	if( IsConv && VEC ) {
 		const int k = ( tid % KQ ) * 4;
 		const int tap = k / args.Cin;
 		convCi = k - tap * args.Cin;
@@ -233,7 +236,7 @@ void matMulKernel( const CMatMulArgs args )
 				regB[i] = bufferLoad4( bufB, off );
 			}
 			// advance
-			if( AMODE == AM_Conv ) {
+			if( IsConv ) {
 				convCi += KS;
 				if( convCi >= args.Cin ) {
 					do {
@@ -628,6 +631,9 @@ int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* sour
 	const bool vec = isAligned16( source ) && isAligned16( filter ) && d.channels % 4 == 0
 		&& fitsBuffer( 1, 0, static_cast<long long>( d.batch ) * d.height * d.width * d.channels )
 		&& fitsBuffer( d.filterCount, args.K, args.K );
+	if( d.filterHeight == 1 && d.filterWidth == 1 ) {
+		return launchMatMul<AM_Conv1x1, BM_RowsK>( stream, args, 1, vec );
+	}
 	return launchMatMul<AM_Conv, BM_RowsK>( stream, args, 1, vec );
 }
 
