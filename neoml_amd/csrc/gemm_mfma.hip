@@ -6,7 +6,8 @@
 // im2col view of an N,H,W,C image (K = fh*fw*Cin gathered on the fly, zero padding), and B given K-major
 // (N x K, i.e. "multiply by transposed matrix" / the filter blob [Cout][fh][fw][Cin]) or N-major (K x N).
 //
-// Tiling: 256 threads = 4 wavefronts per workgroup; workgroup tile BM x BN, K step 16; each wavefront owns
+// Tiling: 256 threads = 4 wavefronts per workgroup; workgroup tile BM x BN (64x64, or 128x32 for narrow outputs),
+// K step 16; each wavefront owns
 // a (BM/WAVES_M) x (BN/WAVES_N) sub-tile built from 32x32 blocks of v_mfma_f32_32x32x2_f32 (16 accumulator
 // registers per block).
 //
@@ -16,6 +17,10 @@
 // of the next group of 8 k are issued before the MFMAs of the current group, and the single barrier of a K step
 // sits before its last group, so the matrix pipe of a wavefront does not wait for LDS, barrier or memory in steady
 // state.
+//
+// Small grids: when the tiles alone would leave the compute units with one or two workgroups each, K is cut into
+// slices (grid z); the slices add their partial products into C with fp32 atomics after C has been set to the free
+// term. The summation order of the slices then varies from run to run (differences at the 1e-7 relative level).
 //
 // LDS layout for a K-major operand is [row][16 + 4 pad]; lane (row = lane % 32, half = lane / 32) fetches the
 // four consecutive k values  k0 + 4*half .. +3  with a single 128-bit LDS read and feeds them to four MFMAs.
@@ -41,6 +46,8 @@ struct CMatMulArgs {
 	int Lda, Ldb, Ldc;
 	long long BatchStrideA, BatchStrideB, BatchStrideC;
 	int Accumulate; // C += instead of C =
+	int SplitK;     // number of K slices (grid z); > 1: partial products are added to C with atomics
+	int StepsPerSplit;
 	int TilesM, TilesN;
 	// convolution geometry (AM_Conv only): A is the image, M = batch * Ho * Wo
 	int H, W, Cin, Ho, Wo, Fh, Fw, PadH, PadW, StrideH, StrideW, DilH, DilW;
@@ -120,11 +127,13 @@ void matMulKernel( const CMatMulArgs args )
 	const int m0 = tileM * BM;
 	const int n0 = tileN * BN;
 	const int batch = blockIdx.y;
+	const int split = blockIdx.z;
 
 	const float* A = args.A + batch * args.BatchStrideA;
 	const float* B = args.B + batch * args.BatchStrideB;
 	float* C = args.C + batch * args.BatchStrideC;
 	const int M = args.M, N = args.N, K = args.K;
+	const int kStart = split * args.StepsPerSplit * NH_KSTEP; // first k of this workgroup's K slice
 	const __amdgpu_buffer_rsrc_t bufA = makeBuffer( A );
 	const __amdgpu_buffer_rsrc_t bufB = makeBuffer( B );
 
@@ -148,10 +157,10 @@ void matMulKernel( const CMatMulArgs args )
 		const bool inTile = ATotal % Threads == 0 || slot < ATotal;
 		if( AMODE == AM_RowsK ) {
 			const int m = m0 + slot / KQ;
-			offA[i] = ( inTile && m < M ) ? static_cast<unsigned>( m * args.Lda + ( slot % KQ ) * 4 ) * 4u : OutOfRange;
+			offA[i] = ( inTile && m < M ) ? static_cast<unsigned>( m * args.Lda + kStart + ( slot % KQ ) * 4 ) * 4u : OutOfRange;
 		} else if( AMODE == AM_RowsM ) {
 			const int m = m0 + ( slot % ( BM / 4 ) ) * 4;
-			offA[i] = ( inTile && m < M ) ? static_cast<unsigned>( ( slot / ( BM / 4 ) ) * args.Lda + m ) * 4u : OutOfRange;
+			offA[i] = ( inTile && m < M ) ? static_cast<unsigned>( ( kStart + slot / ( BM / 4 ) ) * args.Lda + m ) * 4u : OutOfRange;
 		} else {
 			const int m = m0 + slot / KQ;
 			if( inTile && m < M ) {
@@ -170,7 +179,7 @@ void matMulKernel( const CMatMulArgs args )
 		}
 	}
 	if( IsConv && VEC ) {
-		const int k = ( tid % KQ ) * 4;
+		const int k = kStart + ( tid % KQ ) * 4;
 		const int tap = k / args.Cin;
 		convCi = k - tap * args.Cin;
 		convKh = tap / args.Fw;
@@ -186,10 +195,10 @@ void matMulKernel( const CMatMulArgs args )
 		const bool inTile = BTotal % Threads == 0 || slot < BTotal;
 		if( BMODE == BM_RowsK ) {
 			const int n = n0 + slot / KQ;
-			offB[i] = ( inTile && n < N ) ? static_cast<unsigned>( n * args.Ldb + ( slot % KQ ) * 4 ) * 4u : OutOfRange;
+			offB[i] = ( inTile && n < N ) ? static_cast<unsigned>( n * args.Ldb + kStart + ( slot % KQ ) * 4 ) * 4u : OutOfRange;
 		} else {
 			const int n = n0 + ( slot % ( BN / 4 ) ) * 4;
-			offB[i] = ( inTile && n < N ) ? static_cast<unsigned>( ( slot / ( BN / 4 ) ) * args.Ldb + n ) * 4u : OutOfRange;
+			offB[i] = ( inTile && n < N ) ? static_cast<unsigned>( ( kStart + slot / ( BN / 4 ) ) * args.Ldb + n ) * 4u : OutOfRange;
 		}
 	}
 
@@ -429,14 +438,15 @@ void matMulKernel( const CMatMulArgs args )
 	//                    read from LDS; the barrier sits before the last group, after which the first fragments of
 	//                    step ks+1 are fetched, so neither the LDS latency nor the barrier leaves the MFMA pipe idle.
 	// Buffer (ks+1)%3 was last read in step ks-2, and every wave has passed the barrier of step ks-1 since.
-	const int kSteps = ( K + KS - 1 ) / KS;
+	const int totalSteps = ( K + KS - 1 ) / KS;
+	const int kSteps = min( args.StepsPerSplit, totalSteps - split * args.StepsPerSplit );
 	constexpr int Groups = KS / 8;
 	float4 rA[ASlots], rB[BSlots];
 	CFrag frag[2];
-	loadTiles( 0, rA, rB );
+	loadTiles( kStart, rA, rB );
 	storeTiles( 0, rA, rB );
 	if( kSteps > 1 ) {
-		loadTiles( KS, rA, rB );
+		loadTiles( kStart + KS, rA, rB );
 	}
 	__syncthreads();
 	readFrag( 0, 0, frag[0] );
@@ -447,7 +457,7 @@ void matMulKernel( const CMatMulArgs args )
 			storeTiles( nxt, rA, rB );
 		}
 		if( ks + 2 < kSteps ) {
-			loadTiles( ( ks + 2 ) * KS, rA, rB );
+			loadTiles( kStart + ( ks + 2 ) * KS, rA, rB );
 		}
 		__builtin_amdgcn_sched_barrier( 0 );
 #pragma unroll
@@ -481,15 +491,46 @@ void matMulKernel( const CMatMulArgs args )
 				const int m = m0 + waveM * WM + mi * 32 + ( r >> 2 ) * 8 + half * 4 + ( r & 3 );
 				if( m < M ) {
 					float* p = C + static_cast<long long>( m ) * args.Ldc + n;
-					float v = acc[mi][ni][r] + bias;
-					if( args.Accumulate ) {
-						v += *p;
+					if( args.SplitK > 1 ) {
+						// C was set to the free term (or left as is when accumulating) before the launch
+						unsafeAtomicAdd( p, acc[mi][ni][r] );
+					} else {
+						float v = acc[mi][ni][r] + bias;
+						if( args.Accumulate ) {
+							v += *p;
+						}
+						*p = v;
 					}
-					*p = v;
 				}
 			}
 		}
 	}
+}
+
+// C[b][m][n] = bias[n] (or 0): the starting value that the K slices add their partial products to
+__global__ __launch_bounds__( 256 ) void presetResultKernel( float* c, const float* bias, int M, int N, int ldc, long long batchStride )
+{
+	const long long total = static_cast<long long>( M ) * N;
+	float* base = c + blockIdx.y * batchStride;
+	for( long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += static_cast<long long>( gridDim.x ) * 256 ) {
+		const int m = static_cast<int>( i / N );
+		const int n = static_cast<int>( i - static_cast<long long>( m ) * N );
+		base[static_cast<long long>( m ) * ldc + n] = bias != nullptr ? bias[n] : 0.f;
+	}
+}
+
+static int presetResult( hipStream_t stream, const CMatMulArgs& args, int batch )
+{
+	const long long total = static_cast<long long>( args.M ) * args.N;
+	long long blocks = ( total + 1023 ) / 1024;
+	blocks = blocks > 4096 ? 4096 : blocks;
+	for( int b0 = 0; b0 < batch; b0 += 65535 ) {
+		const int nb = batch - b0 < 65535 ? batch - b0 : 65535;
+		hipLaunchKernelGGL( presetResultKernel, dim3( static_cast<unsigned>( blocks ), nb ), dim3( 256 ), 0, stream,
+			args.C + b0 * args.BatchStrideC, args.Bias, args.M, args.N, args.Ldc, args.BatchStrideC );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
 }
 
 template<int BM, int BN, int WAVES_M, int WAVES_N, int AMODE, int BMODE>
@@ -502,6 +543,26 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 		setLastError( "matrix product: too many tiles" );
 		return NH_ERR_ARGUMENT;
 	}
+	// K slices: when the tiles alone leave most compute units with one or two workgroups, cut K so that about five
+	// workgroups per compute unit exist; the slices meet in C through fp32 atomic adds (C is pre-set to the free term)
+	const int totalSteps = ceilDiv( args.K, NH_KSTEP );
+	int splits = 1;
+	const long long blocks = tiles * batch;
+	if( blocks < 1024 && totalSteps >= 32 ) {
+		splits = static_cast<int>( ( 1280 + blocks / 2 ) / blocks );
+	}
+	splits = splits < 1 ? 1 : splits;
+	if( splits > totalSteps / 8 ) {
+		splits = totalSteps / 8 < 1 ? 1 : totalSteps / 8;
+	}
+	args.StepsPerSplit = ceilDiv( totalSteps, splits );
+	args.SplitK = ceilDiv( totalSteps, args.StepsPerSplit );
+	if( args.SplitK > 1 && !args.Accumulate ) {
+		const int rc = presetResult( stream, args, batch );
+		if( rc != NH_OK ) {
+			return rc;
+		}
+	}
 	// blockIdx.y is limited to 65535: walk larger batches in slices
 	for( int b0 = 0; b0 < batch; b0 += 65535 ) {
 		const int nb = batch - b0 < 65535 ? batch - b0 : 65535;
@@ -509,7 +570,7 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 		a.A += b0 * args.BatchStrideA;
 		a.B += b0 * args.BatchStrideB;
 		a.C += b0 * args.BatchStrideC;
-		const dim3 grid( static_cast<unsigned>( tiles ), nb );
+		const dim3 grid( static_cast<unsigned>( tiles ), nb, args.SplitK );
 		if( vec ) {
 			hipLaunchKernelGGL( ( matMulKernel<BM, BN, WAVES_M, WAVES_N, AMODE, BMODE, true> ), grid, dim3( Threads ), 0, stream, a );
 		} else {
@@ -520,30 +581,14 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 	return NH_OK;
 }
 
-// Picks the workgroup tile: wide N tiles when there are enough columns, and the smaller M tile when the
-// large one would leave most of the 256 compute units without a workgroup.
+// Picks the workgroup tile. Measured on MI355X (convolutions of 64..512 channels, GEMMs up to 8192^3): the 64x64 tile
+// wins or ties everywhere, because it puts the most workgroups on every compute unit (five fit by LDS and registers),
+// and latency hiding across workgroups matters more at fp32 MFMA rates than the smaller tile's extra L2 traffic.
+// Narrow outputs (N <= 32) use 128x32 so that no MFMA block multiplies padding.
 template<int AMODE, int BMODE>
 static int launchMatMul( hipStream_t stream, CMatMulArgs& args, int batch, bool vec )
 {
-	const int cus = 256;
-	const int N = args.N;
-	const long long M = args.M;
-	if( N > 64 ) {
-		const long long tiles128 = ( ( M + 127 ) / 128 ) * ( ( N + 127 ) / 128 ) * batch;
-		if( tiles128 >= 2 * cus ) {
-			return launchTile<128, 128, 2, 2, AMODE, BMODE>( stream, args, batch, vec );
-		}
-		const long long tiles64 = ( ( M + 127 ) / 128 ) * ( ( N + 63 ) / 64 ) * batch;
-		if( tiles64 >= 2 * cus ) {
-			return launchTile<128, 64, 2, 2, AMODE, BMODE>( stream, args, batch, vec );
-		}
-		return launchTile<64, 64, 2, 2, AMODE, BMODE>( stream, args, batch, vec );
-	}
-	if( N > 32 ) {
-		const long long tiles = ( ( M + 127 ) / 128 ) * batch;
-		if( tiles >= 2 * cus ) {
-			return launchTile<128, 64, 2, 2, AMODE, BMODE>( stream, args, batch, vec );
-		}
+	if( args.N > 32 ) {
 		return launchTile<64, 64, 2, 2, AMODE, BMODE>( stream, args, batch, vec );
 	}
 	return launchTile<128, 32, 4, 1, AMODE, BMODE>( stream, args, batch, vec );

@@ -3,7 +3,9 @@
  * TEST INFRASTRUCTURE ONLY. Nothing in the shipped library links, loads or calls this file; it is the checker
  * that tests, the smoke run and the benchmark's cpu_baseline leg compare the HIP kernels against.
  *
- * Plain scalar C, fp32 arithmetic, loops written from the definitions the reference uses
+ * Plain scalar C, fp32 arithmetic (long dot products - matrix products, convolution, LSTM gate sums - accumulate in
+ * double and round once: the reference's fp32 result depends on its blocking order, and both it and the GPU result are
+ * compared with the correctly rounded value), loops written from the definitions the reference uses
  * (paths below are relative to /root/reference/NeoMathEngine/):
  *   - convolution            test/src/common/MeTestCommon.h:67-105 (batchConvolutionForward),
  *                            output size src/CPU/CpuMathEngineDnnConv.cpp:59-62
@@ -294,9 +296,9 @@ ORC_API void orc_matmul_nt(const float* a, int lda, const float* b, int ldb, flo
 {
 	for (int i = 0; i < M; ++i)
 		for (int j = 0; j < N; ++j) {
-			float s = 0.f;
-			for (int k = 0; k < K; ++k) s += a[(size_t)i * lda + k] * b[(size_t)j * ldb + k];
-			if (add) c[(size_t)i * ldc + j] += s; else c[(size_t)i * ldc + j] = s;
+			double s = 0.;
+			for (int k = 0; k < K; ++k) s += (double)a[(size_t)i * lda + k] * (double)b[(size_t)j * ldb + k];
+			if (add) c[(size_t)i * ldc + j] += (float)s; else c[(size_t)i * ldc + j] = (float)s;
 		}
 }
 
@@ -306,9 +308,9 @@ ORC_API void orc_matmul_nn(const float* a, int lda, const float* b, int ldb, flo
 {
 	for (int i = 0; i < M; ++i)
 		for (int j = 0; j < N; ++j) {
-			float s = 0.f;
-			for (int k = 0; k < K; ++k) s += a[(size_t)i * lda + k] * b[(size_t)k * ldb + j];
-			if (add) c[(size_t)i * ldc + j] += s; else c[(size_t)i * ldc + j] = s;
+			double s = 0.;
+			for (int k = 0; k < K; ++k) s += (double)a[(size_t)i * lda + k] * (double)b[(size_t)k * ldb + j];
+			if (add) c[(size_t)i * ldc + j] += (float)s; else c[(size_t)i * ldc + j] = (float)s;
 		}
 }
 
@@ -318,9 +320,9 @@ ORC_API void orc_matmul_tn(const float* a, int lda, const float* b, int ldb, flo
 {
 	for (int i = 0; i < M; ++i)
 		for (int j = 0; j < N; ++j) {
-			float s = 0.f;
-			for (int k = 0; k < K; ++k) s += a[(size_t)k * lda + i] * b[(size_t)k * ldb + j];
-			if (add) c[(size_t)i * ldc + j] += s; else c[(size_t)i * ldc + j] = s;
+			double s = 0.;
+			for (int k = 0; k < K; ++k) s += (double)a[(size_t)k * lda + i] * (double)b[(size_t)k * ldb + j];
+			if (add) c[(size_t)i * ldc + j] += (float)s; else c[(size_t)i * ldc + j] = (float)s;
 		}
 }
 
@@ -344,7 +346,7 @@ ORC_API void orc_blob_convolution(const float* in, int n, int h, int w, int cin,
 		for (int y = 0; y < ho; ++y)
 			for (int x = 0; x < wo; ++x)
 				for (int co = 0; co < cout; ++co) {
-					float s = bias ? bias[co] : 0.f;
+					double s = bias ? bias[co] : 0.;
 					for (int ky = 0; ky < fh; ++ky) {
 						const int iy = y * sh - ph + ky * dh;
 						if (iy < 0 || iy >= h) continue;
@@ -353,10 +355,10 @@ ORC_API void orc_blob_convolution(const float* in, int n, int h, int w, int cin,
 							if (ix < 0 || ix >= w) continue;
 							const float* p = in + (((size_t)b * h + iy) * w + ix) * cin;
 							const float* f = filter + (((size_t)co * fh + ky) * fw + kx) * cin;
-							for (int ci = 0; ci < cin; ++ci) s += p[ci] * f[ci];
+							for (int ci = 0; ci < cin; ++ci) s += (double)p[ci] * (double)f[ci];
 						}
 					}
-					out[(((size_t)b * ho + y) * wo + x) * cout + co] = s;
+					out[(((size_t)b * ho + y) * wo + x) * cout + co] = (float)s;
 				}
 }
 
@@ -503,15 +505,13 @@ ORC_API void orc_lstm(int H, int In, const float* wIn, const float* bIn, const f
 		for (int b = 0; b < B; ++b) {
 			const float* xt = x + ((size_t)t * B + b) * In;
 			for (int g = 0; g < 4 * H; ++g) {
-				float s = 0.f;
-				for (int k = 0; k < In; ++k) s += xt[k] * wIn[(size_t)g * In + k];
-				float r = 0.f;
-				for (int k = 0; k < H; ++k) r += hPrev[(size_t)b * H + k] * wRec[(size_t)g * H + k];
-				s += r;
+				double s = 0.;
+				for (int k = 0; k < In; ++k) s += (double)xt[k] * (double)wIn[(size_t)g * In + k];
+				for (int k = 0; k < H; ++k) s += (double)hPrev[(size_t)b * H + k] * (double)wRec[(size_t)g * H + k];
 				if (bIn && bRec) s += bIn[g] + bRec[g];
 				else if (bIn) s += bIn[g];
 				else if (bRec) s += bRec[g];
-				gates[g] = s;
+				gates[g] = (float)s;
 			}
 			for (int j = 0; j < H; ++j) {
 				float a, f, in, o;
