@@ -19,6 +19,11 @@ sys.path.insert(0, ROOT)
 
 FP32_MFMA_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBPS = 8000.0
+# Bytes crossing the L2 <-> fabric boundary per 3x3-convolution launch, mean over the 16 launches of one step at
+# batch 64, 224x224: rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a known-size copy gives) 53.3 MB + WRITE_SIZE (x1.0)
+# 30.5 MB; profiles/resnet18_b64_conv_hbm_traffic.txt holds the two runs. Counters cannot be read from inside this
+# process, so the figure is a constant of the default workload and null for any other.
+CONV3X3_TRAFFIC_BYTES_B64_224 = 83.8e6
 
 
 def cpu_baseline(batch_sample, image):
@@ -111,7 +116,10 @@ def main():
     roofline = {
         "bound": "mfma", "kernel": "matMulKernel<AM_Conv> (3x3 convolutions, %d launches per step)" % (launches // max(args.steps, 1)),
         "achieved": round(achieved, 2), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-        "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
+        "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
+        "traffic": CONV3X3_TRAFFIC_BYTES_B64_224 if (args.batch, args.image) == (64, 224) else None,
+        "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE, rocprofv3 --pmc, scaled by a known-size copy)",
+        "algorithmic_bytes_per_launch": nbytes // max(launches, 1),
         "avg_launch_us": round(ms * 1e3 / max(launches, 1), 2),
         "flop_per_step": flops // max(args.steps, 1),
     }
