@@ -87,69 +87,173 @@ void channelwiseConvKernel( const nhConvDesc d, const float* source, const float
 	}
 }
 
-// ---------------------------------------------------------------------------------------------------------
-// Pooling, one thread per VECW channels of one output pixel
-
-template<int VECW, bool MEAN>
+// The 3x3 case of the depthwise convolution (every depthwise layer of the MobileNet family), 4 channels per thread.
+// One thread owns a strip WPT output pixels wide and rowsPerItem output rows tall and slides down it with the
+// three input rows of the window in registers: every input row is loaded once per strip instead of once per
+// output row that touches it, and the index arithmetic is paid once per strip. Loads are raw buffer loads, so
+// the zero padding is an out-of-range offset instead of a branch. Workgroups of one XCD cover a contiguous
+// range of strips: the halo rows and columns shared by neighbouring strips meet in that XCD's L2.
+template<int STRIDE, int WPT>
 __global__ __launch_bounds__( 256 )
-void poolingKernel( const nhPoolingDesc d, const float* source, float* result, long long totalItems )
+void channelwiseConv3x3Kernel( const nhConvDesc d, const float* source, const float* filter, const float* freeTerm,
+	float* result, int wGroups, int rowChunks, int rowsPerItem, int totalItems )
 {
+	constexpr int NC = ( WPT - 1 ) * STRIDE + 3;
+	constexpr int Keep = 3 - STRIDE; // input rows shared by two consecutive output rows
+	const int item = xcdSwizzle( blockIdx.x, gridDim.x ) * 256 + threadIdx.x;
+	if( item >= totalItems ) {
+		return;
+	}
+	const int cg = d.channels / 4;
+	int t = item;
+	const int c = ( t % cg ) * 4; t /= cg;
+	const int wo0 = ( t % wGroups ) * WPT; t /= wGroups;
+	const int ho0 = ( t % rowChunks ) * rowsPerItem;
+	const int n = t / rowChunks;
+	const int hoEnd = min( ho0 + rowsPerItem, d.resultHeight );
+
+	const __amdgpu_buffer_rsrc_t image = makeBuffer( source );
+	const unsigned rowBytes = static_cast<unsigned>( d.width ) * d.channels * 4;
+	const unsigned imageBytes = n * d.height * rowBytes;
+	unsigned colOff[NC];
+	const int wi0 = wo0 * STRIDE - d.paddingWidth;
+#pragma unroll
+	for( int j = 0; j < NC; ++j ) {
+		const int wi = wi0 + j;
+		colOff[j] = wi >= 0 && wi < d.width ? static_cast<unsigned>( wi * d.channels + c ) * 4 : OutOfRange;
+	}
+	float4 f[9];
+#pragma unroll
+	for( int k = 0; k < 9; ++k ) {
+		f[k] = *reinterpret_cast<const float4*>( filter + k * d.channels + c );
+	}
+	const float4 bias = freeTerm != nullptr ? *reinterpret_cast<const float4*>( freeTerm + c ) : make_float4( 0.f, 0.f, 0.f, 0.f );
+
+	float4 rows[3][NC];
+	auto loadRow = [&]( float4* row, int hi ) {
+		const bool valid = hi >= 0 && hi < d.height;
+		const unsigned rowOff = imageBytes + static_cast<unsigned>( hi ) * rowBytes;
+#pragma unroll
+		for( int j = 0; j < NC; ++j ) {
+			// a valid row offset is below 2 GiB, so adding an out-of-range column stays out of range
+			row[j] = bufferLoad4( image, valid ? rowOff + colOff[j] : OutOfRange );
+		}
+	};
+	int hi = ho0 * STRIDE - d.paddingHeight;
+#pragma unroll
+	for( int r = 0; r < Keep; ++r ) {
+		loadRow( rows[r], hi + r );
+	}
+	float* out = result + ( ( static_cast<long long>( n ) * d.resultHeight + ho0 ) * d.resultWidth + wo0 ) * d.channels + c;
+	const long long outRow = static_cast<long long>( d.resultWidth ) * d.channels;
+	for( int ho = ho0; ho < hoEnd; ++ho ) {
+#pragma unroll
+		for( int r = Keep; r < 3; ++r ) {
+			loadRow( rows[r], hi + r );
+		}
+#pragma unroll
+		for( int j = 0; j < WPT; ++j ) {
+			float4 acc = bias;
+#pragma unroll
+			for( int kh = 0; kh < 3; ++kh ) {
+#pragma unroll
+				for( int kw = 0; kw < 3; ++kw ) {
+					acc = CChanVec<4>::fma( rows[kh][j * STRIDE + kw], f[kh * 3 + kw], acc );
+				}
+			}
+			if( wo0 + j < d.resultWidth ) {
+				*reinterpret_cast<float4*>( out + j * d.channels ) = acc;
+			}
+		}
+#pragma unroll
+		for( int r = 0; r < Keep; ++r ) {
+#pragma unroll
+			for( int j = 0; j < NC; ++j ) {
+				rows[r][j] = rows[r + STRIDE][j];
+			}
+		}
+		hi += STRIDE;
+		out += outRow;
+	}
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Pooling: one thread owns VECW channels of one output column and walks down rowsPerItem output rows of it.
+// Workgroups of one XCD cover a contiguous range of the image, so the input rows that overlapping windows
+// share are fetched into one L2 only.
+
+// FILTER > 0: the window is FILTER x FILTER and its loops unroll, so all loads of a window are in flight together.
+template<int VECW, bool MEAN, int FILTER>
+__global__ __launch_bounds__( 256 )
+void poolingKernel( const nhPoolingDesc d, const float* source, float* result, int rowChunks, int rowsPerItem, long long totalItems )
+{
+	const int filterHeight = FILTER > 0 ? FILTER : d.filterHeight;
+	const int filterWidth = FILTER > 0 ? FILTER : d.filterWidth;
 	const int cg = d.channels / VECW;
 	const long long step = static_cast<long long>( gridDim.x ) * 256;
 	// ( 1 / fh ) / fw as the reference computes it (src/CPU/CpuMathEngineDnnPooling.h:68-69)
 	const float scale = 1.f / d.filterHeight / d.filterWidth;
-	for( long long item = blockIdx.x * 256LL + threadIdx.x; item < totalItems; item += step ) {
+	const long long inRow = static_cast<long long>( d.width ) * d.channels;
+	const long long outRow = static_cast<long long>( d.resultWidth ) * d.channels;
+	for( long long item = xcdSwizzle( blockIdx.x, gridDim.x ) * 256LL + threadIdx.x; item < totalItems; item += step ) {
 		long long t = item;
 		const int c = static_cast<int>( t % cg ) * VECW; t /= cg;
 		const int wo = static_cast<int>( t % d.resultWidth ); t /= d.resultWidth;
-		const int ho = static_cast<int>( t % d.resultHeight ); t /= d.resultHeight;
+		const int ho0 = static_cast<int>( t % rowChunks ) * rowsPerItem; t /= rowChunks;
 		const long long n = t;
-		const float* window = source + ( ( n * d.height + ho * d.strideHeight ) * d.width + wo * d.strideWidth ) * d.channels + c;
-		float acc[VECW];
-		// columns outside, rows inside: the reference reduces over the rows of each column first
-		for( int kw = 0; kw < d.filterWidth; ++kw ) {
-			float col[VECW];
-			for( int kh = 0; kh < d.filterHeight; ++kh ) {
-				const float* p = window + ( static_cast<long long>( kh ) * d.width + kw ) * d.channels;
-				float v[VECW];
-				if constexpr( VECW == 4 ) {
-					const float4 q = *reinterpret_cast<const float4*>( p );
-					v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
-				} else {
-					v[0] = *p;
+		const int hoEnd = min( ho0 + rowsPerItem, d.resultHeight );
+		const float* window = source + ( ( n * d.height + ho0 * d.strideHeight ) * d.width + wo * d.strideWidth ) * d.channels + c;
+		float* out = result + ( ( n * d.resultHeight + ho0 ) * d.resultWidth + wo ) * d.channels + c;
+		for( int ho = ho0; ho < hoEnd; ++ho ) {
+			float acc[VECW];
+			// columns outside, rows inside: the reference reduces over the rows of each column first
+#pragma unroll
+			for( int kw = 0; kw < filterWidth; ++kw ) {
+				float col[VECW];
+#pragma unroll
+				for( int kh = 0; kh < filterHeight; ++kh ) {
+					const float* p = window + kh * inRow + kw * d.channels;
+					float v[VECW];
+					if constexpr( VECW == 4 ) {
+						const float4 q = *reinterpret_cast<const float4*>( p );
+						v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+					} else {
+						v[0] = *p;
+					}
+#pragma unroll
+					for( int e = 0; e < VECW; ++e ) {
+						if( kh == 0 ) {
+							col[e] = v[e];
+						} else if( MEAN ) {
+							col[e] += v[e];
+						} else if( v[e] > col[e] ) {
+							col[e] = v[e];
+						}
+					}
 				}
 #pragma unroll
 				for( int e = 0; e < VECW; ++e ) {
-					if( kh == 0 ) {
-						col[e] = v[e];
+					if( kw == 0 ) {
+						acc[e] = col[e];
 					} else if( MEAN ) {
-						col[e] += v[e];
-					} else if( v[e] > col[e] ) {
-						col[e] = v[e];
+						acc[e] += col[e];
+					} else if( col[e] > acc[e] ) {
+						acc[e] = col[e];
 					}
 				}
 			}
-#pragma unroll
-			for( int e = 0; e < VECW; ++e ) {
-				if( kw == 0 ) {
-					acc[e] = col[e];
-				} else if( MEAN ) {
-					acc[e] += col[e];
-				} else if( col[e] > acc[e] ) {
-					acc[e] = col[e];
-				}
+			if constexpr( VECW == 4 ) {
+				float4 q;
+				q.x = MEAN ? acc[0] * scale : acc[0];
+				q.y = MEAN ? acc[1] * scale : acc[1];
+				q.z = MEAN ? acc[2] * scale : acc[2];
+				q.w = MEAN ? acc[3] * scale : acc[3];
+				*reinterpret_cast<float4*>( out ) = q;
+			} else {
+				*out = MEAN ? acc[0] * scale : acc[0];
 			}
-		}
-		float* out = result + item * VECW;
-		if constexpr( VECW == 4 ) {
-			float4 q;
-			q.x = MEAN ? acc[0] * scale : acc[0];
-			q.y = MEAN ? acc[1] * scale : acc[1];
-			q.z = MEAN ? acc[2] * scale : acc[2];
-			q.w = MEAN ? acc[3] * scale : acc[3];
-			*reinterpret_cast<float4*>( out ) = q;
-		} else {
-			*out = MEAN ? acc[0] * scale : acc[0];
+			window += d.strideHeight * inRow;
+			out += outRow;
 		}
 	}
 }
@@ -434,23 +538,59 @@ static int checkPoolingDesc( const nhPoolingDesc* d )
 	return NH_OK;
 }
 
+// Splits resultHeight into row chunks, one per work item: as tall as possible (the taller the strip, the fewer
+// halo rows are read twice) while the launch still has `wantedBlocks` workgroups, several rounds of the 256
+// compute units at the kernel's occupancy.
+static void chooseRowChunks( long long itemsPerChunk, int resultHeight, int minRows, int wantedBlocks, int* rowChunks, int* rowsPerItem )
+{
+	const long long blocksPerChunk = ( itemsPerChunk + 255 ) / 256;
+	const long long wanted = ( wantedBlocks + blocksPerChunk - 1 ) / blocksPerChunk;
+	const long long maxChunks = ( resultHeight + minRows - 1 ) / minRows;
+	const int chunks = static_cast<int>( wanted < maxChunks ? wanted : maxChunks );
+	const int rows = ( resultHeight + chunks - 1 ) / chunks;
+	*rowsPerItem = rows;
+	*rowChunks = ( resultHeight + rows - 1 ) / rows;
+}
+
 template<bool MEAN>
 static int poolingImpl( nhStream s, const nhPoolingDesc* d, const float* source, float* result )
 {
 	const bool vec = d->channels % 4 == 0 && isAligned16( source ) && isAligned16( result );
-	const long long items = static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * ( vec ? d->channels / 4 : d->channels );
-	if( items == 0 ) {
+	const long long perRow = static_cast<long long>( d->batch ) * d->resultWidth * ( vec ? d->channels / 4 : d->channels );
+	if( perRow == 0 ) {
 		return NH_OK;
 	}
+	int rowChunks = 1, rowsPerItem = 1;
+	chooseRowChunks( perRow, d->resultHeight, d->filterHeight > d->strideHeight ? 4 : 1, 8192, &rowChunks, &rowsPerItem );
+	const long long items = perRow * rowChunks;
 	long long blocks = ( items + 255 ) / 256;
 	blocks = blocks > 1048576 ? 1048576 : blocks;
-	if( vec ) {
-		hipLaunchKernelGGL( ( poolingKernel<4, MEAN> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
-			*d, source, result, items );
+	const int square = d->filterHeight == d->filterWidth ? d->filterHeight : 0;
+	const dim3 grid( static_cast<unsigned>( blocks ) );
+	if( vec && square == 2 ) {
+		hipLaunchKernelGGL( ( poolingKernel<4, MEAN, 2> ), grid, dim3( 256 ), 0, toStream( s ), *d, source, result, rowChunks, rowsPerItem, items );
+	} else if( vec && square == 3 ) {
+		hipLaunchKernelGGL( ( poolingKernel<4, MEAN, 3> ), grid, dim3( 256 ), 0, toStream( s ), *d, source, result, rowChunks, rowsPerItem, items );
+	} else if( vec ) {
+		hipLaunchKernelGGL( ( poolingKernel<4, MEAN, 0> ), grid, dim3( 256 ), 0, toStream( s ), *d, source, result, rowChunks, rowsPerItem, items );
 	} else {
-		hipLaunchKernelGGL( ( poolingKernel<1, MEAN> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
-			*d, source, result, items );
+		hipLaunchKernelGGL( ( poolingKernel<1, MEAN, 0> ), grid, dim3( 256 ), 0, toStream( s ), *d, source, result, rowChunks, rowsPerItem, items );
 	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+template<int STRIDE, int WPT>
+static int channelwise3x3Impl( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
+	const float* freeTerm, float* result )
+{
+	const int wGroups = ceilDiv( d->resultWidth, WPT );
+	const long long perRow = static_cast<long long>( d->batch ) * wGroups * ( d->channels / 4 );
+	int rowChunks = 1, rowsPerItem = 1;
+	chooseRowChunks( perRow, d->resultHeight, 4, 3072, &rowChunks, &rowsPerItem );
+	const long long items = perRow * rowChunks;
+	hipLaunchKernelGGL( ( channelwiseConv3x3Kernel<STRIDE, WPT> ), dim3( static_cast<unsigned>( ( items + 255 ) / 256 ) ), dim3( 256 ), 0,
+		toStream( s ), *d, source, filter, freeTerm, result, wGroups, rowChunks, rowsPerItem, static_cast<int>( items ) );
 	NH_LAUNCH_CHECK();
 	return NH_OK;
 }
@@ -489,6 +629,15 @@ int nhBlobChannelwiseConvolution( nhStream s, const nhConvDesc* d, const float* 
 	}
 	const bool vec = d->channels % 4 == 0 && isAligned16( source ) && isAligned16( filter ) && isAligned16( result )
 		&& ( freeTerm == nullptr || isAligned16( freeTerm ) );
+	// the strip kernel addresses the image with 32-bit byte offsets and counts work items in an int
+	const long long sourceBytes = static_cast<long long>( d->batch ) * d->height * d->width * d->channels * 4;
+	if( vec && d->filterHeight == 3 && d->filterWidth == 3 && d->strideHeight == d->strideWidth && d->strideHeight <= 2
+		&& sourceBytes < 0x80000000LL
+		&& static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * d->channels < 0x7fffffffLL )
+	{
+		return d->strideHeight == 1 ? channelwise3x3Impl<1, 4>( s, d, source, filter, freeTerm, result )
+			: channelwise3x3Impl<2, 2>( s, d, source, filter, freeTerm, result );
+	}
 	constexpr int WPT = 4;
 	const int wGroups = ceilDiv( d->resultWidth, WPT );
 	const long long items = static_cast<long long>( d->batch ) * d->resultHeight * wGroups * ( vec ? d->channels / 4 : d->channels );

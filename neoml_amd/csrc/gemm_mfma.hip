@@ -59,35 +59,6 @@ constexpr int Threads = 256;
 #define NH_KSTEP 16
 #endif
 
-// Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous range of tiles so that
-// neighbouring tiles (which share rows of A and the halo of the image) meet in the same L2.
-__device__ __forceinline__ int xcdSwizzle( int bid, int total )
-{
-	const int xcd = bid & 7;
-	const int idx = bid >> 3;
-	const int per = total >> 3;
-	const int rem = total & 7;
-	return xcd * per + ( xcd < rem ? xcd : rem ) + idx;
-}
-
-// Operands are read with raw buffer loads: a 32-bit byte offset from a base held in scalar registers, and a range
-// check done by the memory unit. An offset at or above BufferBytes reads as zero, which serves as the zero padding
-// of the convolution and as the mask of tile rows / columns / k beyond the matrix, without a branch or a select.
-typedef unsigned int u32x4 __attribute__( ( ext_vector_type( 4 ) ) );
-constexpr unsigned BufferBytes = 0x80000000u;
-constexpr unsigned OutOfRange = 0x80000000u;
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t makeBuffer( const float* p )
-{
-	return __builtin_amdgcn_make_buffer_rsrc( const_cast<float*>( p ), 0, BufferBytes, 0x00020000 );
-}
-
-__device__ __forceinline__ float4 bufferLoad4( __amdgpu_buffer_rsrc_t rsrc, unsigned offset )
-{
-	const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128( rsrc, offset, 0, 0 );
-	return make_float4( __uint_as_float( v.x ), __uint_as_float( v.y ), __uint_as_float( v.z ), __uint_as_float( v.w ) );
-}
-
 template<int BM, int BN, int WAVES_M, int WAVES_N, int AMODE, int BMODE, bool VEC>
 __global__ __launch_bounds__( Threads, 2 )
 void matMulKernel( const CMatMulArgs args )

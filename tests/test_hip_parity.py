@@ -267,7 +267,13 @@ def test_convolution_is_linear_at_full_size():
 
 
 @pytest.mark.parametrize("case", CHANNELWISE_CASES + [(2, 28, 28, 96, 3, 3, 1, 1, 1, 1), (2, 28, 28, 96, 3, 3, 1, 1, 2, 2),
-                                                      (1, 15, 13, 6, 3, 3, 1, 1, 2, 2), (1, 9, 30, 32, 5, 5, 2, 2, 1, 1)])
+                                                      (1, 15, 13, 6, 3, 3, 1, 1, 2, 2), (1, 9, 30, 32, 5, 5, 2, 2, 1, 1),
+                                                      # the 3x3 strip kernel: ragged row chunks and strip widths, no / wide / uneven padding
+                                                      (2, 30, 17, 8, 3, 3, 1, 1, 1, 1), (1, 11, 11, 4, 3, 3, 0, 0, 1, 1),
+                                                      (1, 7, 9, 12, 3, 3, 2, 2, 2, 2), (3, 13, 21, 16, 3, 3, 2, 0, 1, 1),
+                                                      (2, 21, 13, 20, 3, 3, 0, 2, 2, 2), (1, 3, 3, 4, 3, 3, 1, 1, 1, 1),
+                                                      # one strip of 12 rows per work item (a full-size MobileNet layer)
+                                                      (128, 112, 112, 32, 3, 3, 1, 1, 1, 1)])
 def test_channelwise_convolution(case):
     n, h, w, c, fh, fw, ph, pw, sh, sw = case
     g = rng(12 + c)
@@ -278,7 +284,9 @@ def test_channelwise_convolution(case):
     assert_close(hip().channelwise_conv(x, f, None, ph, pw, sh, sw), orc.channelwise_conv(x, f, None, ph, pw, sh, sw), str(case))
 
 
-@pytest.mark.parametrize("case", POOL_CASES + [(2, 57, 57, 64, 3, 3, 2, 2), (3, 16, 64, 7, 2, 2, 2, 2), (2, 4, 128, 256, 2, 1, 2, 1)])
+@pytest.mark.parametrize("case", POOL_CASES + [(2, 57, 57, 64, 3, 3, 2, 2), (3, 16, 64, 7, 2, 2, 2, 2), (2, 4, 128, 256, 2, 1, 2, 1),
+                                               (2, 23, 19, 8, 3, 3, 1, 1), (1, 31, 9, 12, 2, 2, 2, 2), (2, 9, 9, 4, 4, 4, 1, 1),
+                                               (64, 114, 114, 64, 3, 3, 2, 2)])
 def test_pooling(case):
     n, h, w, c, fh, fw, sh, sw = case
     g = rng(13 + h)
