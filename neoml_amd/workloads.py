@@ -165,6 +165,150 @@ class HipBackend:
         self._timed("softmax", 0, 8 * x.numel(), self.lib.nhMatrixSoftmaxByRows, self._p(x), x.shape[0], x.shape[1], self._p(out))
         return out
 
+    # ---- ops of the depthwise-separable, transformer and line-recogniser configurations
+    def scalar(self, value):
+        """A one-float device buffer: the form the engine takes multipliers, thresholds and addends in."""
+        key = ("scalar", float(value))
+        t = self._desc_cache.get(key)
+        if t is None:
+            t = self._desc_cache[key] = self.tensor(np.array([value], np.float32))
+        return t
+
+    def relu6_(self, x):
+        return self.relu_(x, self.scalar(6.0))
+
+    def channelwise_conv(self, x, filt, bias, ph, pw, sh, sw, out=None):
+        n, h, w, c = x.shape
+        fh, fw, _ = filt.shape
+        key = ("dw", n, h, w, c, fh, fw, ph, pw, sh, sw)
+        d = self._desc_cache.get(key)
+        if d is None:
+            d = self.na.ConvDesc(n, h, w, c, c, fh, fw, ph, pw, sh, sw, 1, 1, 0, 0)
+            self.na.check(self.lib.nhInitBlobChannelwiseConvolution(ctypes.byref(d)))
+            self._desc_cache[key] = d
+        ho, wo = d.resultHeight, d.resultWidth
+        if out is None:
+            out = self.empty(n, ho, wo, c)
+        self._timed("depthwise", 2 * n * ho * wo * c * fh * fw, 4 * (x.numel() + out.numel() + filt.numel() + c),
+                    self.lib.nhBlobChannelwiseConvolution, ctypes.byref(d), self._p(x), self._p(filt), self._p(bias), self._p(out))
+        return out
+
+    def add(self, a, b, out=None):
+        if out is None:
+            out = self.empty(*a.shape)
+        self._timed("add", 0, 12 * a.numel(), self.lib.nhVectorAdd, self._p(a), self._p(b), self._p(out), a.numel())
+        return out
+
+    def mul_scalar_(self, x, value):
+        self._timed("eltwise", 0, 8 * x.numel(), self.lib.nhVectorMultiply, self._p(x), self._p(x), x.numel(), self._p(self.scalar(value)))
+        return x
+
+    def transpose(self, x, out=None):
+        """[b,h,m,w,c] -> [b,w,m,h,c]"""
+        b, h, m, w, c = x.shape
+        if out is None:
+            out = self.empty(b, w, m, h, c)
+        self._timed("transpose", 0, 8 * x.numel(), self.lib.nhTransposeMatrix, b, self._p(x), h, m, w, c, self._p(out), out.numel())
+        return out
+
+    def bmm_nn(self, a, b, out=None):
+        """a [batch,M,K] x b [batch,K,N]"""
+        batch, m, k = a.shape
+        n = b.shape[2]
+        if out is None:
+            out = self.empty(batch, m, n)
+        self._timed("bmm", 2 * batch * m * n * k, 4 * batch * (m * k + k * n + m * n), self.lib.nhBatchMultiplyMatrixByMatrix,
+                    batch, self._p(a), m, k, self._p(b), n, self._p(out), out.numel())
+        return out
+
+    def layer_norm(self, x, scale, bias, out=None, eps=1e-5):
+        """CObjectNormalizationLayer::runOnceImpl (NeoML/src/Dnn/Layers/ObjectNormalizationLayer.cpp:181-242):
+        thirteen engine calls over a [rows x width] matrix."""
+        rows, width = x.shape
+        L, p = self.lib, self._p
+        if out is None:
+            out = self.empty(rows, width)
+        key = ("ln", rows, width)
+        tmp = self._desc_cache.get(key)
+        if tmp is None:
+            tmp = self._desc_cache[key] = (self.empty(rows), self.empty(rows), self.empty(rows, width))
+        neg_mean, inv_std, sq = tmp
+        inv_w, e = self.scalar(1.0 / width), self.scalar(eps)
+        mat = 8 * rows * width
+        t = lambda nbytes, fn, *a: self._timed("layernorm", 0, nbytes, fn, *a)
+        t(mat // 2, L.nhSumMatrixColumns, p(neg_mean), p(x), rows, width)
+        t(8 * rows, L.nhVectorNegMultiply, p(neg_mean), p(neg_mean), rows, p(inv_w))
+        t(mat, L.nhAddVectorToMatrixColumns, p(x), p(sq), rows, width, p(neg_mean))
+        t(mat // 2 * 3, L.nhVectorEltwiseMultiply, p(sq), p(sq), p(sq), rows * width)
+        t(mat // 2, L.nhSumMatrixColumns, p(inv_std), p(sq), rows, width)
+        t(8 * rows, L.nhVectorMultiply, p(inv_std), p(inv_std), rows, p(inv_w))
+        t(8 * rows, L.nhVectorAddValue, p(inv_std), p(inv_std), rows, p(e))
+        t(8 * rows, L.nhVectorSqrt, p(inv_std), p(inv_std), rows)
+        t(8 * rows, L.nhVectorInv, p(inv_std), p(inv_std), rows)
+        t(mat, L.nhAddVectorToMatrixColumns, p(x), p(out), rows, width, p(neg_mean))
+        t(mat, L.nhMultiplyDiagMatrixByMatrix, p(inv_std), rows, p(out), width, p(out), rows * width)
+        t(mat, L.nhBatchMultiplyMatrixByDiagMatrix, 1, p(out), rows, width, 0, p(scale), 0, p(out), rows * width)
+        t(mat, L.nhAddVectorToMatrixRows, 1, p(out), p(out), rows, width, p(bias))
+        return out
+
+    def gelu_(self, x):
+        """CGELULayer, sigmoid approximation (NeoML/src/Dnn/Layers/GELULayer.cpp:146-160): x * sigmoid(1.702 x)"""
+        key = ("gelu", x.numel())
+        tmp = self._desc_cache.get(key)
+        if tmp is None:
+            tmp = self._desc_cache[key] = self.empty(x.numel())
+        n, p = x.numel(), self._p
+        self._timed("gelu", 0, 8 * n, self.lib.nhVectorMultiply, p(x), p(tmp), n, p(self.scalar(1.702)))
+        self._timed("gelu", 0, 8 * n, self.lib.nhVectorSigmoid, p(tmp), p(tmp), n)
+        self._timed("gelu", 0, 12 * n, self.lib.nhVectorEltwiseMultiply, p(x), p(tmp), p(x), n)
+        return x
+
+    def lstm(self, x, w_in, b_in, w_rec, b_rec, reverse=False, out=None):
+        """x [T,B,In] -> h [T,B,H]; zero initial state"""
+        T, B, In = x.shape
+        H = w_rec.shape[1]
+        if out is None:
+            out = self.empty(T, B, H)
+        key = ("lstm", T, B, In, H, bool(reverse))
+        ws = self._desc_cache.get(key)
+        if ws is None:
+            size = ctypes.c_size_t(0)
+            self.na.check(self.lib.nhLstmWorkspaceSize(H, In, T, B, ctypes.byref(size)))
+            ws = self._desc_cache[key] = (self.empty((size.value + 3) // 4), size.value)
+        p = self._p
+        self._timed("lstm", 2 * T * B * 4 * H * (In + H), 4 * (x.numel() + out.numel() + w_in.numel() + w_rec.numel()),
+                    self.lib.nhLstm, H, In, p(w_in), p(b_in), p(w_rec), p(b_rec), 1 if reverse else 0, T, B, None, None, p(x),
+                    None, p(out), p(ws[0]), ws[1])
+        return out
+
+    def merge_channels(self, parts, out=None):
+        """concatenate [rows, c_i] along the channels (BlobMergeByDim on BD_Channels)"""
+        rows = parts[0].shape[0]
+        total = sum(t.shape[1] for t in parts)
+        if out is None:
+            out = self.empty(rows, total)
+        key = ("merge", rows) + tuple(t.data_ptr() for t in parts)
+        d = self._desc_cache.get(key)
+        if d is None:
+            descs = (self.na.BlobDesc * len(parts))(*[self.na.BlobDesc.of(1, rows, 1, 1, 1, 1, t.shape[1]) for t in parts])
+            ptrs = (ctypes.c_void_p * len(parts))(*[t.data_ptr() for t in parts])
+            d = self._desc_cache[key] = (descs, ptrs, self.na.BlobDesc.of(1, rows, 1, 1, 1, 1, total))
+        self._timed("merge", 0, 8 * out.numel(), self.lib.nhBlobMergeByDim, 6, d[0], d[1], len(parts), ctypes.byref(d[2]), self._p(out))
+        return out
+
+    def log_(self, x):
+        self._timed("eltwise", 0, 8 * x.numel(), self.lib.nhVectorLog, self._p(x), self._p(x), x.numel())
+        return x
+
+    def argmax_rows(self, x):
+        rows, width = x.shape
+        key = ("argmax", rows)
+        t = self._desc_cache.get(key)
+        if t is None:
+            t = self._desc_cache[key] = (self.empty(rows), self.torch.empty(rows, dtype=self.torch.int32, device=self.dev))
+        self._timed("argmax", 0, 4 * x.numel(), self.lib.nhFindMaxValueInRows, self._p(x), rows, width, self._p(t[0]), self._p(t[1]), rows)
+        return t[1]
+
 
 class LaunchPlan:
     """A recorded sequence of C-ABI launches with their arguments bound once, replayed with minimal host work
@@ -326,3 +470,202 @@ class ResNet18:
         f, b = self.dev["fc"]
         y = run("fc", be.fc, y, f, b)
         return run("softmax", be.softmax, y)
+
+
+class Network:
+    """Shared plumbing of the configurations: named activation buffers reused across passes, plan recording."""
+
+    def __init__(self, backend):
+        self.be = backend
+        self.buffers = {}
+
+    def run(self, key, fn, *args, **kw):
+        out = fn(*args, out=self.buffers.get(key), **kw)
+        self.buffers[key] = out
+        return out
+
+    def record_plan(self, x):
+        self.forward(x)  # allocates the buffers
+        self.be.plan = []
+        out = self.forward(x)
+        launches, self.be.plan = self.be.plan, None
+        return LaunchPlan(self.be, launches), out
+
+
+class MobileNetV2(Network):
+    """MobileNetV2-style inference: 3x3/2 stem, inverted residual blocks (1x1 expand x t + ReLU6, 3x3 depthwise + ReLU6,
+    1x1 project, residual add when the shape is kept), 1x1 head, global mean pool, FC. Batch-norm folded into the free
+    terms, He-normal weights."""
+
+    TABLE = ((1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2), (6, 320, 1, 1))
+
+    def __init__(self, backend, batch=128, image=224, classes=1000, seed=0xC0FFEE + 3, head=1280):
+        super().__init__(backend)
+        self.batch, self.image, self.classes = batch, image, classes
+        g = np.random.default_rng(seed)
+
+        def conv(cout, f, cin):
+            return (g.normal(0, np.sqrt(2.0 / (f * f * cin)), (cout, f, f, cin)).astype(np.float32),
+                    g.normal(0, 0.01, cout).astype(np.float32))
+
+        def depthwise(c):
+            return g.normal(0, np.sqrt(2.0 / 9), (3, 3, c)).astype(np.float32), g.normal(0, 0.01, c).astype(np.float32)
+
+        self.host = {"stem": conv(32, 3, 3)}
+        self.blocks = []
+        cin = 32
+        for t, c, n, s in self.TABLE:
+            for i in range(n):
+                name = "b%d" % len(self.blocks)
+                stride = s if i == 0 else 1
+                mid = cin * t
+                if t != 1:
+                    self.host[name + "e"] = conv(mid, 1, cin)
+                self.host[name + "d"] = depthwise(mid)
+                self.host[name + "p"] = conv(c, 1, mid)
+                self.blocks.append((name, t != 1, stride, stride == 1 and cin == c))
+                cin = c
+        self.host["head"] = conv(head, 1, cin)
+        self.host["fc"] = (g.normal(0, np.sqrt(1.0 / head), (classes, head)).astype(np.float32), g.normal(0, 0.01, classes).astype(np.float32))
+        self.dev = {k: (backend.tensor(f), backend.tensor(b)) for k, (f, b) in self.host.items()}
+
+    def make_input(self, seed=0xC0FFEE + 103):
+        return np.random.default_rng(seed).uniform(0, 1, (self.batch, self.image, self.image, 3)).astype(np.float32)
+
+    def forward(self, x):
+        be, run, W = self.be, self.run, self.dev
+        y = run("stem", be.conv, x, *W["stem"], 1, 1, 2, 2)
+        be.relu6_(y)
+        for name, expand, stride, residual in self.blocks:
+            t = y
+            if expand:
+                t = run(name + "e", be.conv, t, *W[name + "e"], 0, 0, 1, 1)
+                be.relu6_(t)
+            t = run(name + "d", be.channelwise_conv, t, *W[name + "d"], 1, 1, stride, stride)
+            be.relu6_(t)
+            t = run(name + "p", be.conv, t, *W[name + "p"], 0, 0, 1, 1)
+            if residual:
+                be.add_(t, y)
+            y = t
+        y = run("head", be.conv, y, *W["head"], 0, 0, 1, 1)
+        be.relu6_(y)
+        y = run("gap", be.global_mean, y)
+        return run("fc", be.fc, y, *W["fc"])
+
+
+class TransformerEncoder(Network):
+    """Stack of CTransformerEncoderLayer (post-layernorm, no mask, no dropout, GELU by sigmoid approximation) as
+    the engine calls of NeoML/src/Dnn/Layers/TransformerLayer.cpp:249-329 and MultiheadAttentionLayer.cpp:145-456.
+    Reshapes that the layer graph does with in-place transforms cost nothing here either."""
+
+    def __init__(self, backend, layers=6, d_model=512, heads=8, ffn=2048, seq=256, batch=32, seed=0xC0FFEE + 4):
+        super().__init__(backend)
+        self.layers, self.d, self.heads, self.ffn, self.seq, self.batch = layers, d_model, heads, ffn, seq, batch
+        g = np.random.default_rng(seed)
+
+        def xavier(n_out, n_in):
+            a = np.sqrt(6.0 / (n_in + n_out))
+            return g.uniform(-a, a, (n_out, n_in)).astype(np.float32), g.normal(0, 0.01, n_out).astype(np.float32)
+
+        self.host = {}
+        for l in range(layers):
+            for nm, shape in (("q", (d_model, d_model)), ("k", (d_model, d_model)), ("v", (d_model, d_model)), ("o", (d_model, d_model)),
+                              ("f1", (ffn, d_model)), ("f2", (d_model, ffn))):
+                self.host["l%d%s" % (l, nm)] = xavier(*shape)
+            for nm in ("n1", "n2"):
+                self.host["l%d%s" % (l, nm)] = (g.uniform(0.8, 1.2, d_model).astype(np.float32), g.normal(0, 0.05, d_model).astype(np.float32))
+        self.dev = {k: (backend.tensor(a), backend.tensor(b)) for k, (a, b) in self.host.items()}
+
+    def make_input(self, seed=0xC0FFEE + 104):
+        return np.random.default_rng(seed).normal(0, 1, (self.batch * self.seq, self.d)).astype(np.float32)
+
+    def gemm_flops(self):
+        m, d, f, s = self.batch * self.seq, self.d, self.ffn, self.seq
+        per_layer = 2 * m * d * d * 4 + 2 * m * d * f * 2 + 2 * 2 * self.batch * self.heads * s * s * (d // self.heads)
+        return per_layer * self.layers
+
+    def forward(self, x):
+        be, run, W = self.be, self.run, self.dev
+        B, S, D, h = self.batch, self.seq, self.d, self.heads
+        dk = D // h
+        y = x
+        for l in range(self.layers):
+            n = "l%d" % l
+            q = run(n + "q", be.fc, y, *W[n + "q"])
+            k = run(n + "k", be.fc, y, *W[n + "k"])
+            v = run(n + "v", be.fc, y, *W[n + "v"])
+            qt = run(n + "qt", be.transpose, q.reshape(B, S, 1, h, dk))          # [B,h,1,S,dk]
+            kt = run(n + "kt", be.transpose, k.reshape(B, S, 1, D, 1))           # [B,D,1,S,1] = [B,h,dk,S]
+            vt = run(n + "vt", be.transpose, v.reshape(B, S, 1, h, dk))
+            sc = run(n + "sc", be.bmm_nn, qt.reshape(B * h, S, dk), kt.reshape(B * h, dk, S))
+            be.mul_scalar_(sc, 1.0 / np.sqrt(dk))
+            pr = run(n + "pr", be.softmax, sc.reshape(B * h * S, S))
+            cx = run(n + "cx", be.bmm_nn, pr.reshape(B * h, S, S), vt.reshape(B * h, S, dk))
+            ct = run(n + "ct", be.transpose, cx.reshape(B, h, 1, S, dk))          # [B,S,1,h,dk]
+            o = run(n + "o", be.fc, ct.reshape(B * S, D), *W[n + "o"])
+            a = run(n + "a", be.add, y, o)
+            y1 = run(n + "n1", be.layer_norm, a, *W[n + "n1"])
+            f = run(n + "f1", be.fc, y1, *W[n + "f1"])
+            be.gelu_(f)
+            f2 = run(n + "f2", be.fc, f, *W[n + "f2"])
+            a2 = run(n + "a2", be.add, y1, f2)
+            y = run(n + "n2", be.layer_norm, a2, *W[n + "n2"])
+        return y
+
+
+class LineRecognizer(Network):
+    """OCR line recogniser: 3x3 convolution backbone that pools a 32 x W grey image down to height 1 and width W/4,
+    two bidirectional LSTM layers through the fused Lstm entry point, FC to classes + blank, and the engine part of
+    CCtcDecodingLayer::RunOnce (NeoML/src/Dnn/Layers/CtcLayer.cpp:205-226): transpose, softmax, log, arg-max.
+    The label collapse is host code in the reference too."""
+
+    BACKBONE = ((64, (2, 2)), (128, (2, 2)), (256, None), (256, (2, 1)), (256, (2, 1)), (256, (2, 1)))
+
+    def __init__(self, backend, batch=64, height=32, width=512, hidden=256, classes=100, seed=0xC0FFEE + 5):
+        super().__init__(backend)
+        self.batch, self.height, self.width, self.hidden, self.classes = batch, height, width, hidden, classes
+        g = np.random.default_rng(seed)
+        self.host = {}
+        cin = 1
+        for i, (c, _) in enumerate(self.BACKBONE):
+            self.host["c%d" % i] = (g.normal(0, np.sqrt(2.0 / (9 * cin)), (c, 3, 3, cin)).astype(np.float32), g.normal(0, 0.01, c).astype(np.float32))
+            cin = c
+        feat = cin
+        self.lstm_host = {}
+        for layer in range(2):
+            for direction in ("f", "r"):
+                a = 1.0 / np.sqrt(hidden)
+                self.lstm_host["l%d%s" % (layer, direction)] = (
+                    g.uniform(-a, a, (4 * hidden, feat)).astype(np.float32), g.uniform(-a, a, 4 * hidden).astype(np.float32),
+                    g.uniform(-a, a, (4 * hidden, hidden)).astype(np.float32), g.uniform(-a, a, 4 * hidden).astype(np.float32))
+            feat = 2 * hidden
+        self.host["fc"] = (g.normal(0, np.sqrt(1.0 / feat), (classes + 1, feat)).astype(np.float32), g.normal(0, 0.01, classes + 1).astype(np.float32))
+        self.dev = {k: tuple(backend.tensor(a) for a in v) for k, v in list(self.host.items()) + list(self.lstm_host.items())}
+
+    def make_input(self, seed=0xC0FFEE + 105):
+        return np.random.default_rng(seed).uniform(0, 1, (self.batch, self.height, self.width, 1)).astype(np.float32)
+
+    def forward(self, x):
+        """Returns (labels int32 [B][T], log-probabilities [B*T, classes+1])."""
+        be, run, W = self.be, self.run, self.dev
+        y = x
+        for i, (_, pool) in enumerate(self.BACKBONE):
+            y = run("c%d" % i, be.conv, y, *W["c%d" % i], 1, 1, 1, 1)
+            be.relu_(y)
+            if pool is not None:
+                y = run("p%d" % i, be.max_pool, y, pool[0], pool[1], pool[0], pool[1])
+        B, one, T, C = y.shape
+        assert one == 1
+        seq = run("seq", be.transpose, y.reshape(1, B, 1, T, C)).reshape(T, B, C)   # [T,B,C]
+        for layer in range(2):
+            f = run("l%df" % layer, be.lstm, seq, *W["l%df" % layer], reverse=False)
+            r = run("l%dr" % layer, be.lstm, seq, *W["l%dr" % layer], reverse=True)
+            H = f.shape[2]
+            seq = run("l%dm" % layer, be.merge_channels, [f.reshape(T * B, H), r.reshape(T * B, H)]).reshape(T, B, 2 * H)
+        logits = run("fc", be.fc, seq.reshape(T * B, seq.shape[2]), *W["fc"])
+        K = logits.shape[1]
+        bt = run("bt", be.transpose, logits.reshape(1, T, 1, B, K)).reshape(B * T, K)   # [B,T,K]
+        prob = run("prob", be.softmax, bt)
+        be.log_(prob)
+        labels = be.argmax_rows(prob)
+        return labels.reshape(B, T), prob

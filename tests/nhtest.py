@@ -793,3 +793,60 @@ class CpuBackend:
 
     def softmax(self, x, out=None):
         return self.cpu.softmax_rows(x)
+
+    # ---- ops of the depthwise-separable, transformer and line-recogniser configurations
+    def relu6_(self, x):
+        x[...] = self.cpu.unary("relu", x, 6.0).reshape(x.shape)
+        return x
+
+    def channelwise_conv(self, x, filt, bias, ph, pw, sh, sw, out=None):
+        return self.cpu.channelwise_conv(x, filt, bias, ph, pw, sh, sw)
+
+    def add(self, a, b, out=None):
+        return self.cpu.binary("add", a, b).reshape(a.shape)
+
+    def mul_scalar_(self, x, value):
+        x[...] = self.cpu.unary("multiply", x, np.float32(value)).reshape(x.shape)
+        return x
+
+    def transpose(self, x, out=None):
+        return self.cpu.transpose(x)
+
+    def bmm_nn(self, a, b, out=None):
+        batch, m, k = a.shape
+        return self.cpu.matmul("bnn", a, b, M=m, N=b.shape[2], K=k, batch=batch)
+
+    def layer_norm(self, x, scale, bias, out=None, eps=1e-5):
+        c = self.cpu
+        rows, width = x.shape
+        neg_mean = c.unary("neg_multiply", c.sum_matrix_columns(x), np.float32(1.0 / width))
+        sq = c.add_vector_to_matrix_columns(x, neg_mean)
+        sq = c.binary("eltwise_multiply", sq, sq)
+        var = c.unary("multiply", c.sum_matrix_columns(sq), np.float32(1.0 / width))
+        inv_std = c.unary("inv", c.unary("sqrt", c.unary("add_value", var, np.float32(eps))))
+        y = c.multiply_diag_matrix_by_matrix(inv_std, c.add_vector_to_matrix_columns(x, neg_mean))
+        y = c.batch_multiply_matrix_by_diag_matrix(1, y, rows, width, 0, scale, 0)
+        return c.add_vector_to_matrix_rows(y.reshape(1, rows, width), bias.reshape(1, width)).reshape(rows, width)
+
+    def gelu_(self, x):
+        c = self.cpu
+        t = c.unary("sigmoid", c.unary("multiply", x, np.float32(1.702)))
+        x[...] = c.binary("eltwise_multiply", x, t).reshape(x.shape)
+        return x
+
+    def lstm(self, x, w_in, b_in, w_rec, b_rec, reverse=False, out=None):
+        h, _ = self.cpu.lstm(w_in, b_in, w_rec, b_rec, x, reverse=reverse, want_state=False)
+        return h
+
+    def merge_channels(self, parts, out=None):
+        rows = parts[0].shape[0]
+        total = sum(p.shape[1] for p in parts)
+        parts7 = [f32(p).reshape(1, rows, 1, 1, 1, 1, p.shape[1]) for p in parts]
+        return self.cpu.merge(parts7, 6, (1, rows, 1, 1, 1, 1, total)).reshape(rows, total)
+
+    def log_(self, x):
+        x[...] = self.cpu.unary("log", x).reshape(x.shape)
+        return x
+
+    def argmax_rows(self, x):
+        return self.cpu.find_max_in_rows(x)[1]
