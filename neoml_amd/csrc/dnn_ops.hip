@@ -511,6 +511,106 @@ void lstmGatesKernel( const float* gates, const float* statePrev, float* stateOu
 	mainOut[i] = o * tanhf( c );
 }
 
+// One LSTM step in one launch: gates = pre + hPrev * Wrec^T on the matrix cores, then the gate non-linearities.
+// A workgroup owns 64 sequences x 8 hidden units = a 64 x 32 block of the gate matrix (columns = 4 gates x 8
+// units), so every value the cell update of those units needs meets inside the workgroup. 8 wavefronts: two
+// 32-row halves x four slices of the reduction over H. Operands go from L2 straight into MFMA registers
+// (each lane reads 64 contiguous bytes of its row per 32 k), the four K slices meet in LDS.
+// The step is latency-bound (about 34 MFLOP); the point is one launch instead of a product, a bias add and
+// a gate kernel per step.
+constexpr int LstmRows = 64;
+constexpr int LstmUnits = 8;
+constexpr int LstmKSlices = 4;
+constexpr int LstmThreads = 64 * 2 * LstmKSlices;
+typedef float lstmAcc __attribute__( ( ext_vector_type( 16 ) ) );
+
+__global__ __launch_bounds__( LstmThreads )
+void lstmStepKernel( const float* pre, const float* hPrev, const float* wRec, const float* statePrev,
+	float* stateOut, float* mainOut, int batch, int hidden )
+{
+	__shared__ float partial[LstmKSlices][LstmRows][33];
+	const int wave = threadIdx.x >> 6;
+	const int lane = threadIdx.x & 63;
+	const int l32 = lane & 31;
+	const int half = lane >> 5;
+	const int mHalf = wave & 1;
+	const int slice = wave >> 1;
+	const int unit0 = blockIdx.x * LstmUnits;
+	const int row0 = blockIdx.y * LstmRows;
+
+	// the cell update this thread does after the product: its inputs are requested first, so that their
+	// latency (they were written long ago and come from HBM) hides behind the product
+	const int row = threadIdx.x >> 3;
+	const int unit = threadIdx.x & 7;
+	const int b = row0 + row;
+	const bool active = b < batch;
+	const int cell = b * hidden + unit0 + unit;
+	float g[4] = { 0.f, 0.f, 0.f, 0.f };
+	float cPrev = 0.f;
+	if( active ) {
+#pragma unroll
+		for( int q = 0; q < 4; ++q ) {
+			g[q] = pre[static_cast<long long>( b ) * 4 * hidden + q * hidden + unit0 + unit];
+		}
+		if( statePrev != nullptr ) {
+			cPrev = statePrev[cell];
+		}
+	}
+
+	lstmAcc acc;
+#pragma unroll
+	for( int r = 0; r < 16; ++r ) {
+		acc[r] = 0.f;
+	}
+	if( hPrev != nullptr ) {
+		const __amdgpu_buffer_rsrc_t bufA = makeBuffer( hPrev );
+		const __amdgpu_buffer_rsrc_t bufB = makeBuffer( wRec );
+		const int aRow = row0 + mHalf * 32 + l32;
+		const int bRow = ( l32 >> 3 ) * hidden + unit0 + ( l32 & 7 ); // column l32 of the block = gate l32/8, unit l32%8
+		// lanes 0-31 take k0..k0+15 of their row, lanes 32-63 k0+16..k0+31: MFMA e of a 32-k chunk reduces over
+		// { k0+e, k0+16+e }, the same pairing for both operands
+		const unsigned aBase = aRow < batch ? static_cast<unsigned>( aRow * hidden + half * 16 ) * 4 : OutOfRange;
+		const unsigned bBase = static_cast<unsigned>( bRow * hidden + half * 16 ) * 4;
+		for( int k0 = slice * 32; k0 < hidden; k0 += 32 * LstmKSlices ) {
+			float4 a[4], w[4];
+#pragma unroll
+			for( int q = 0; q < 4; ++q ) {
+				a[q] = bufferLoad4( bufA, aBase + static_cast<unsigned>( k0 + q * 4 ) * 4 );
+				w[q] = bufferLoad4( bufB, bBase + static_cast<unsigned>( k0 + q * 4 ) * 4 );
+			}
+#pragma unroll
+			for( int q = 0; q < 4; ++q ) {
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[q].x, w[q].x, acc, 0, 0, 0 );
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[q].y, w[q].y, acc, 0, 0, 0 );
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[q].z, w[q].z, acc, 0, 0, 0 );
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[q].w, w[q].w, acc, 0, 0, 0 );
+			}
+		}
+	}
+#pragma unroll
+	for( int r = 0; r < 16; ++r ) {
+		partial[slice][mHalf * 32 + ( r >> 2 ) * 8 + half * 4 + ( r & 3 )][l32] = acc[r];
+	}
+	__syncthreads();
+	if( !active ) {
+		return;
+	}
+#pragma unroll
+	for( int q = 0; q < 4; ++q ) {
+#pragma unroll
+		for( int sl = 0; sl < LstmKSlices; ++sl ) {
+			g[q] += partial[sl][row][q * 8 + unit];
+		}
+	}
+	const float a = tanhf( g[0] );
+	const float f = lstmSigmoid( g[1] );
+	const float in = lstmSigmoid( g[2] );
+	const float o = lstmSigmoid( g[3] );
+	const float c = f * cPrev + in * a;
+	stateOut[cell] = c;
+	mainOut[cell] = o * tanhf( c );
+}
+
 __global__ void addTwoVectorsKernel( const float* a, const float* b, float* out, int n )
 {
 	const int i = blockIdx.x * 256 + threadIdx.x;
@@ -789,6 +889,10 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 		return rc;
 	}
 	const int stepSize = B * H;
+	// the one-launch step needs whole 32-k chunks and 8-unit blocks, 16-byte aligned rows and 32-bit byte offsets
+	const bool fusedStep = H % 32 == 0 && isAligned16( recurrentWeights ) && isAligned16( outputMainBackLink )
+		&& ( inputMainBackLink == nullptr || isAligned16( inputMainBackLink ) )
+		&& static_cast<long long>( 4 ) * H * H * 4 < 0x80000000LL && static_cast<long long>( B ) * H * 4 < 0x80000000LL;
 	for( int i = 0; i < T; ++i ) {
 		const int pos = reverse ? T - 1 - i : i;
 		const int prev = reverse ? pos + 1 : pos - 1;
@@ -803,6 +907,12 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 			cOut = stateScratch;
 		}
 		float* g = gates + static_cast<size_t>( pos ) * B * 4 * H;
+		if( fusedStep ) {
+			hipLaunchKernelGGL( lstmStepKernel, dim3( H / LstmUnits, ceilDiv( B, LstmRows ) ), dim3( LstmThreads ), 0, stream,
+				g, hPrev, recurrentWeights, cPrev, cOut, outputMainBackLink + static_cast<size_t>( pos ) * stepSize, B, H );
+			NH_LAUNCH_CHECK();
+			continue;
+		}
 		if( hPrev != nullptr ) {
 			rc = matMulNT( stream, hPrev, H, recurrentWeights, H, g, 4 * H, B, 4 * H, H, 1, 0, 0, 0, nullptr, true );
 			if( rc != NH_OK ) {

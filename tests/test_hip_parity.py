@@ -346,7 +346,7 @@ def test_split_and_merge():
 @pytest.mark.parametrize("with_init", [False, True])
 def test_lstm(reverse, with_init):
     g = rng(18)
-    for T, B, In, H in ((5, 3, 6, 4), (7, 16, 32, 64), (4, 64, 256, 256)):
+    for T, B, In, H in ((5, 3, 6, 4), (7, 16, 32, 64), (4, 64, 256, 256), (6, 70, 48, 96), (33, 5, 16, 32)):
         w_in = g.uniform(-0.2, 0.2, (4 * H, In)).astype(np.float32)
         w_rec = g.uniform(-0.2, 0.2, (4 * H, H)).astype(np.float32)
         b_in = g.uniform(-0.5, 0.5, 4 * H).astype(np.float32)
