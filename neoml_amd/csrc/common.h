@@ -77,6 +77,11 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t makeBuffer( const float* p )
 	return __builtin_amdgcn_make_buffer_rsrc( const_cast<float*>( p ), 0, BufferBytes, 0x00020000 );
 }
 
+__device__ __forceinline__ float bufferLoad1( __amdgpu_buffer_rsrc_t rsrc, unsigned offset )
+{
+	return __uint_as_float( __builtin_amdgcn_raw_buffer_load_b32( rsrc, offset, 0, 0 ) );
+}
+
 __device__ __forceinline__ float4 bufferLoad4( __amdgpu_buffer_rsrc_t rsrc, unsigned offset )
 {
 	const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128( rsrc, offset, 0, 0 );

@@ -34,7 +34,11 @@ typedef float f32x16 __attribute__( ( ext_vector_type( 16 ) ) );
 
 // AM_Conv1x1 runs the same code as AM_Conv; the separate value gives 1x1 convolutions their own kernel symbols, so
 // that profiles tell them apart from the 3x3 ones
-enum TAMode { AM_RowsK = 0, AM_RowsM = 1, AM_Conv = 2, AM_Conv1x1 = 3 };
+// AM_ConvRows serves channel counts that are not a multiple of 4 (grey and RGB inputs): the reduction index runs
+// over Fh filter rows of RowPitch = ceil4( Fw * Cin ) values each. The Fw * Cin values that one filter row meets are
+// contiguous in a channels-last image (no dilation along the width), so they are fetched as 128-bit runs however
+// Cin divides; the 1-3 padding values per row are masked to zero on both operands.
+enum TAMode { AM_RowsK = 0, AM_RowsM = 1, AM_Conv = 2, AM_Conv1x1 = 3, AM_ConvRows = 4 };
 enum TBMode { BM_RowsK = 0, BM_RowsN = 1 };
 
 struct CMatMulArgs {
@@ -51,6 +55,7 @@ struct CMatMulArgs {
 	int TilesM, TilesN;
 	// convolution geometry (AM_Conv only): A is the image, M = batch * Ho * Wo
 	int H, W, Cin, Ho, Wo, Fh, Fw, PadH, PadW, StrideH, StrideW, DilH, DilW;
+	int RowK, RowPitch; // AM_ConvRows: Fw * Cin and its round-up to a multiple of 4; K = Fh * RowPitch
 };
 
 constexpr int Threads = 256;
@@ -73,6 +78,7 @@ void matMulKernel( const CMatMulArgs args )
 	constexpr int NI = WN / 32;
 	constexpr bool AK = ( AMODE != AM_RowsM );
 	constexpr bool IsConv = ( AMODE == AM_Conv || AMODE == AM_Conv1x1 );
+	constexpr bool IsConvRows = ( AMODE == AM_ConvRows );
 	constexpr bool BK = ( BMODE == BM_RowsK );
 	constexpr int APitchX = BM + 4, BPitchX = BN + 4;
 	constexpr int ASize = AK ? BM * LdsK : KS * APitchX;
@@ -141,13 +147,21 @@ void matMulKernel( const CMatMulArgs args )
 				const int n = t / args.Ho;
 				convPixel[i] = n * args.H * args.W * args.Cin;
 				convH0[i] = ho * args.StrideH - args.PadH;
-				convW0[i] = wo * args.StrideW - args.PadW;
+				convW0[i] = ( wo * args.StrideW - args.PadW ) * ( IsConvRows ? args.Cin : 1 ); // AM_ConvRows: in floats
+
 			} else {
 				convPixel[i] = 0;
 				convH0[i] = -0x40000000; // never inside the image
 				convW0[i] = 0;
 			}
 		}
+	}
+	// AM_ConvRows: filter row and position inside the padded row of this thread's k (all its slots share the column)
+	int rowKh = 0, rowR = 0;
+	if( IsConvRows ) {
+		const int k = kStart + ( tid % KQ ) * 4;
+		rowKh = k / args.RowPitch;
+		rowR = k - rowKh * args.RowPitch;
 	}
 	if( IsConv && VEC ) {
 		const int k = kStart + ( tid % KQ ) * 4;
@@ -191,6 +205,51 @@ void matMulKernel( const CMatMulArgs args )
 
 	// Loads the tiles of the K step starting at kBase into registers and advances the slot offsets to the next step.
 	auto loadTiles = [&]( int kBase, float4 ( &regA )[ASlots], float4 ( &regB )[BSlots] ) {
+		if constexpr( IsConvRows ) {
+			const int rowFloats = args.W * args.Cin;
+			const bool khIn = rowKh < args.Fh;
+#pragma unroll
+			for( int i = 0; i < ASlots; ++i ) {
+				const int hi = convH0[i] + rowKh * args.DilH;
+				const bool rowOk = khIn && hi >= 0 && hi < args.H;
+				const int col = convW0[i] + rowR; // position inside the image row, in floats; negative in the left padding
+				const int index = convPixel[i] + hi * rowFloats + col;
+				if( rowOk && rowR + 3 < args.RowK && col >= 0 && col + 3 < rowFloats ) {
+					regA[i] = bufferLoad4( bufA, static_cast<unsigned>( index ) * 4u );
+				} else {
+					float v[4];
+#pragma unroll
+					for( int e = 0; e < 4; ++e ) {
+						const bool ok = rowOk && rowR + e < args.RowK && col + e >= 0 && col + e < rowFloats;
+						v[e] = bufferLoad1( bufA, ok ? static_cast<unsigned>( index + e ) * 4u : OutOfRange );
+					}
+					regA[i] = make_float4( v[0], v[1], v[2], v[3] );
+				}
+			}
+#pragma unroll
+			for( int i = 0; i < BSlots; ++i ) {
+				const int slot = tid + i * Threads;
+				const int n = n0 + slot / KQ;
+				const bool nOk = ( BTotal % Threads == 0 || slot < BTotal ) && n < N && khIn;
+				const int index = n * args.Ldb + rowKh * args.RowK + rowR;
+				if( nOk && rowR + 3 < args.RowK ) {
+					regB[i] = bufferLoad4( bufB, static_cast<unsigned>( index ) * 4u );
+				} else {
+					float v[4];
+#pragma unroll
+					for( int e = 0; e < 4; ++e ) {
+						v[e] = bufferLoad1( bufB, nOk && rowR + e < args.RowK ? static_cast<unsigned>( index + e ) * 4u : OutOfRange );
+					}
+					regB[i] = make_float4( v[0], v[1], v[2], v[3] );
+				}
+			}
+			rowR += KS;
+			while( rowR >= args.RowPitch ) {
+				rowR -= args.RowPitch;
+				++rowKh;
+			}
+			return;
+		}
 		if( VEC ) {
 			// k of this thread's slots inside the step: fixed column of a K-major tile, fixed row of an X-major one
 			const bool kInA = AMODE == AM_RowsM ? true : ( kBase + ( tid % KQ ) * 4 < K );
@@ -649,6 +708,15 @@ int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* sour
 		&& fitsBuffer( d.filterCount, args.K, args.K );
 	if( d.filterHeight == 1 && d.filterWidth == 1 ) {
 		return launchMatMul<AM_Conv1x1, BM_RowsK>( stream, args, 1, vec );
+	}
+	if( d.channels % 4 != 0 && d.dilationWidth == 1
+		&& fitsBuffer( 1, 0, static_cast<long long>( d.batch ) * d.height * d.width * d.channels )
+		&& fitsBuffer( d.filterCount, args.K, args.K ) )
+	{
+		args.RowK = d.filterWidth * d.channels;
+		args.RowPitch = ( args.RowK + 3 ) / 4 * 4;
+		args.K = d.filterHeight * args.RowPitch; // reduction length as the kernel walks it; Ldb keeps the filter's own
+		return launchMatMul<AM_ConvRows, BM_RowsK>( stream, args, 1, true );
 	}
 	return launchMatMul<AM_Conv, BM_RowsK>( stream, args, 1, vec );
 }

@@ -223,6 +223,13 @@ GPU_CONV_CASES = CONV_CASES + [
     (2, 14, 14, 128, 256, 1, 1, 0, 0, 2, 2, 1, 1),  # 1x1 stride 2 shortcut
     (2, 32, 32, 3, 64, 7, 7, 3, 3, 2, 2, 1, 1),     # stem
     (2, 8, 32, 1, 64, 3, 3, 1, 1, 1, 1, 1, 1),      # single input channel
+    # channel counts that are not a multiple of 4: filter rows fetched as contiguous runs
+    (2, 9, 13, 6, 10, 3, 5, 1, 2, 1, 2, 2, 1),      # height dilation, width stride
+    (1, 7, 7, 2, 5, 3, 3, 1, 1, 1, 1, 1, 1),
+    (3, 24, 40, 3, 32, 3, 3, 1, 1, 2, 2, 1, 1),     # RGB 3x3/2 stem
+    (1, 6, 5, 7, 9, 2, 4, 0, 3, 1, 1, 1, 1),        # run longer than the image row is wide
+    (2, 11, 9, 5, 70, 1, 3, 0, 1, 1, 1, 1, 1),      # N tail
+    (4, 32, 64, 1, 64, 3, 3, 1, 1, 1, 1, 1, 1),     # grey line image, split over many tiles
 ]
 
 
@@ -236,6 +243,20 @@ def test_convolution(case):
     want = orc.conv(x, f, bias, ph, pw, sh, sw, dh, dw)
     assert_close(hip().conv(x, f, bias, ph, pw, sh, sw, dh, dw), want, "conv %s" % (case,))
     assert_close(hip().conv(x, f, None, ph, pw, sh, sw, dh, dw), orc.conv(x, f, None, ph, pw, sh, sw, dh, dw), "conv, no free term")
+
+
+def test_convolution_ignores_pixels_outside_the_windows():
+    # stride 4 with a 3-wide filter never touches image columns 3 and 7; whatever they hold (here: infinities)
+    # must not leak into the result through the vector fetches that run past a window's last value
+    g = rng(77)
+    x = g.uniform(-1, 1, (2, 6, 11, 3)).astype(np.float32)
+    x[:, :, 3, :] = np.inf
+    x[:, :, 7, :] = -np.inf
+    f = g.normal(0, 0.3, (8, 3, 3, 3)).astype(np.float32)
+    want = orc.conv(np.nan_to_num(x, posinf=0.0, neginf=0.0), f, None, 0, 0, 1, 4)
+    got = hip().conv(x, f, None, 0, 0, 1, 4)
+    assert np.isfinite(got).all()
+    assert_close(got, want, "unused columns")
 
 
 def test_convolution_config1_vs_reference_engine():
