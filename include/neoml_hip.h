@@ -173,7 +173,8 @@ NH_API int nhFindMaxValueInRows(nhStream s, const float* matrix, int matrixHeigh
 	float* result, int* columnIndices, int vectorSize);                                              /* NME.h:466-469 */
 NH_API int nhFindMaxValueInColumns(nhStream s, int batchSize, const float* matrix, int matrixHeight,
 	int matrixWidth, float* result, int* rowIndices, int vectorSize);                                /* NME.h:473 */
-/* result[M x N] = first[M x K] * second[N x K]^T with row strides */
+/* result[M x N] = first[M x K] * second[N x K]^T with row strides; resultBufferSize is ignored, as the reference
+ * CPU engine ignores it (its fully-connected layer passes 0) */
 NH_API int nhMultiplyMatrixByTransposedMatrix(nhStream s, const float* first, int firstHeight, int firstWidth,
 	int firstRowSize, const float* second, int secondHeight, int secondRowSize,
 	float* result, int resultRowSize, int resultBufferSize);                                         /* NME.h:529 */
@@ -191,7 +192,7 @@ NH_API int nhBatchMultiplyMatrixByMatrix(nhStream s, int batchSize, const float*
 	int firstWidth, const float* second, int secondWidth, float* result, int resultBufferSize);      /* NME.h:580 */
 NH_API int nhBatchMultiplyMatrixByDiagMatrix(nhStream s, int batchSize, const float* first, int height, int width,
 	int firstMatrixOffset, const float* second, int secondMatrixOffset, float* result, int resultBufferSize); /* NME.h:588 */
-/* [b,h,m,w,c] -> [b,w,m,h,c] */
+/* [b,h,m,w,c] -> [b,w,m,h,c]; resultBufferSize is ignored, as in the reference CPU engine */
 NH_API int nhTransposeMatrix(nhStream s, int batchSize, const float* first, int height, int medium, int width,
 	int channels, float* result, int resultBufferSize);                                              /* NME.h:599 */
 NH_API int nhTransposeMatrixInt(nhStream s, int batchSize, const int* first, int height, int medium, int width,

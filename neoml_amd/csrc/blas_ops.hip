@@ -383,11 +383,9 @@ static int transposeImpl( nhStream s, int batchSize, const T* first, int height,
 		setLastError( "TransposeMatrix: negative dimension" );
 		return NH_ERR_ARGUMENT;
 	}
+	// resultBufferSize is not looked at: the reference CPU engine ignores it too (src/CPU/CpuMathEngineBlas.cpp:152-163)
+	( void )resultBufferSize;
 	const long long total = static_cast<long long>( batchSize ) * height * medium * width * channels;
-	if( total > resultBufferSize ) {
-		setLastError( "TransposeMatrix: result buffer is too small" );
-		return NH_ERR_ARGUMENT;
-	}
 	if( total == 0 ) {
 		return NH_OK;
 	}

@@ -736,7 +736,9 @@ int nhMultiplyMatrixByTransposedMatrix( nhStream s, const float* first, int firs
 {
 	NH_REQUIRE( firstHeight >= 0 && firstWidth >= 0 && secondHeight >= 0 );
 	NH_REQUIRE( firstRowSize >= firstWidth && secondRowSize >= firstWidth && resultRowSize >= secondHeight );
-	NH_REQUIRE( firstHeight == 0 || static_cast<long long>( firstHeight - 1 ) * resultRowSize + secondHeight <= resultBufferSize );
+	// resultBufferSize is not looked at: the reference CPU engine ignores it (src/CPU/CpuMathEngineBlas.cpp:906-918)
+	// and CFullyConnectedLayer::RunOnce passes 0 (NeoML/src/Dnn/Layers/FullyConnectedLayer.cpp:91-94)
+	( void )resultBufferSize;
 	return matMulNT( toStream( s ), first, firstRowSize, second, secondRowSize, result, resultRowSize,
 		firstHeight, secondHeight, firstWidth, 1, 0, 0, 0, nullptr, false );
 }

@@ -1,0 +1,247 @@
+// Test infrastructure, not part of the product: C entry points that build small networks out of NeoML's OWN layer
+// classes (CDnn, CConvLayer, CChannelwiseConvLayer, CFullyConnectedLayer, CMaxPoolingLayer, CMeanPoolingLayer,
+// CTransformerEncoderLayer, CLstmLayer; compiled from the reference's sources into _ref/libNeoML.so by the Makefile
+// beside this file) on whatever IMathEngine* they are handed, run one forward pass and return the output.
+// The tests call them once with the reference's CPU engine and once with the HIP engine: same layer code, same
+// CRandom seed for the initialisers, same input, so the two outputs differ only by the engine underneath.
+#include <NeoML/NeoML.h>
+
+#include <exception>
+#include <string>
+#include <string.h>
+
+using namespace NeoML;
+
+static thread_local std::string lastError;
+
+#define EXPORT extern "C" __attribute__( ( visibility( "default" ) ) )
+
+EXPORT const char* dnn_last_error() { return lastError.c_str(); }
+
+template<class T>
+static CPtr<T> add( CDnn& dnn, T* layer, const char* name, CBaseLayer& input, int outputNumber = 0 )
+{
+	CPtr<T> holder = layer;
+	layer->SetName( name );
+	layer->Connect( 0, input, outputNumber );
+	dnn.AddLayer( *layer );
+	return holder;
+}
+
+// kind 0: CNN. Conv 3x3 p1 (16) - ReLU - MaxPool 2x2/2 - ChannelwiseConv 3x3 p1 - ReLU6 - Conv 1x1 (32) - MeanPool 2x2/2
+//         - FullyConnected (10) - Softmax. Input dims: [1, N, 1, H, W, 1, C].
+static CBaseLayer* buildCnn( CDnn& dnn, IMathEngine& e, CBaseLayer& source )
+{
+	CPtr<CConvLayer> conv = add( dnn, new CConvLayer( e ), "conv", source );
+	conv->SetFilterCount( 16 ); conv->SetFilterHeight( 3 ); conv->SetFilterWidth( 3 );
+	conv->SetPaddingHeight( 1 ); conv->SetPaddingWidth( 1 );
+	CPtr<CReLULayer> relu = add( dnn, new CReLULayer( e ), "relu", *conv );
+	CPtr<CMaxPoolingLayer> pool = add( dnn, new CMaxPoolingLayer( e ), "pool", *relu );
+	pool->SetFilterHeight( 2 ); pool->SetFilterWidth( 2 ); pool->SetStrideHeight( 2 ); pool->SetStrideWidth( 2 );
+	CPtr<CChannelwiseConvLayer> dw = add( dnn, new CChannelwiseConvLayer( e ), "dw", *pool );
+	dw->SetFilterCount( 16 ); dw->SetFilterHeight( 3 ); dw->SetFilterWidth( 3 );
+	dw->SetPaddingHeight( 1 ); dw->SetPaddingWidth( 1 );
+	CPtr<CReLULayer> relu6 = add( dnn, new CReLULayer( e ), "relu6", *dw );
+	relu6->SetUpperThreshold( 6.f );
+	CPtr<CConvLayer> project = add( dnn, new CConvLayer( e ), "project", *relu6 );
+	project->SetFilterCount( 32 ); project->SetFilterHeight( 1 ); project->SetFilterWidth( 1 );
+	CPtr<CMeanPoolingLayer> mean = add( dnn, new CMeanPoolingLayer( e ), "mean", *project );
+	mean->SetFilterHeight( 2 ); mean->SetFilterWidth( 2 ); mean->SetStrideHeight( 2 ); mean->SetStrideWidth( 2 );
+	CPtr<CFullyConnectedLayer> fc = add( dnn, new CFullyConnectedLayer( e ), "fc", *mean );
+	fc->SetNumberOfElements( 10 );
+	CPtr<CSoftmaxLayer> softmax = add( dnn, new CSoftmaxLayer( e ), "softmax", *fc );
+	return softmax.Ptr();
+}
+
+// kind 1: two CTransformerEncoderLayer (4 heads, FFN 4x, GELU, post-norm, no dropout). Input: [1, B, S, 1, 1, 1, D].
+static CBaseLayer* buildTransformer( CDnn& dnn, IMathEngine& e, CBaseLayer& source, int hidden )
+{
+	CBaseLayer* last = &source;
+	for( int i = 0; i < 2; ++i ) {
+		CPtr<CTransformerEncoderLayer> layer = add( dnn, new CTransformerEncoderLayer( e ), i == 0 ? "enc0" : "enc1", *last );
+		layer->SetHeadCount( 4 );
+		layer->SetHiddenSize( hidden );
+		layer->SetDropoutRate( 0.f );
+		layer->SetSelfAttentionDropoutRate( 0.f );
+		layer->SetFeedForwardSize( 4 * hidden );
+		layer->SetActivation( CActivationDesc( AF_GELU ) );
+		last = layer.Ptr();
+	}
+	return last;
+}
+
+// kind 2: CLstmLayer (hidden = param) followed by a FullyConnected over every step. Input: [T, B, 1, 1, 1, 1, In].
+static CBaseLayer* buildLstm( CDnn& dnn, IMathEngine& e, CBaseLayer& source, int hidden )
+{
+	CPtr<CLstmLayer> lstm = add( dnn, new CLstmLayer( e ), "lstm", source );
+	lstm->SetHiddenSize( hidden );
+	CPtr<CFullyConnectedLayer> fc = add( dnn, new CFullyConnectedLayer( e ), "fc", *lstm );
+	fc->SetNumberOfElements( 11 );
+	return fc.Ptr();
+}
+
+// kind 3: ResNet-style stem and basic block. Conv 7x7/2 p3 (16) - ReLU - ImageResize (pad 1 each side) - MaxPool 3x3/2
+//         - [Conv 3x3 p1 /2 (32) - ReLU - Conv 3x3 p1 (32)] + [Conv 1x1 /2 (32)] - EltwiseSum - ReLU - GlobalMeanPooling
+//         - FullyConnected (10) - Softmax. Input dims: [1, N, 1, H, W, 1, 3].
+static CBaseLayer* buildResNetBlock( CDnn& dnn, IMathEngine& e, CBaseLayer& source )
+{
+	CPtr<CConvLayer> stem = add( dnn, new CConvLayer( e ), "stem", source );
+	stem->SetFilterCount( 16 ); stem->SetFilterHeight( 7 ); stem->SetFilterWidth( 7 );
+	stem->SetPaddingHeight( 3 ); stem->SetPaddingWidth( 3 ); stem->SetStrideHeight( 2 ); stem->SetStrideWidth( 2 );
+	CPtr<CReLULayer> relu0 = add( dnn, new CReLULayer( e ), "relu0", *stem );
+	CPtr<CImageResizeLayer> pad = add( dnn, new CImageResizeLayer( e ), "pad", *relu0 );
+	pad->SetDelta( CImageResizeLayer::IS_Left, 1 ); pad->SetDelta( CImageResizeLayer::IS_Right, 1 );
+	pad->SetDelta( CImageResizeLayer::IS_Top, 1 ); pad->SetDelta( CImageResizeLayer::IS_Bottom, 1 );
+	CPtr<CMaxPoolingLayer> pool = add( dnn, new CMaxPoolingLayer( e ), "pool", *pad );
+	pool->SetFilterHeight( 3 ); pool->SetFilterWidth( 3 ); pool->SetStrideHeight( 2 ); pool->SetStrideWidth( 2 );
+
+	CPtr<CConvLayer> c1 = add( dnn, new CConvLayer( e ), "c1", *pool );
+	c1->SetFilterCount( 32 ); c1->SetFilterHeight( 3 ); c1->SetFilterWidth( 3 );
+	c1->SetPaddingHeight( 1 ); c1->SetPaddingWidth( 1 ); c1->SetStrideHeight( 2 ); c1->SetStrideWidth( 2 );
+	CPtr<CReLULayer> relu1 = add( dnn, new CReLULayer( e ), "relu1", *c1 );
+	CPtr<CConvLayer> c2 = add( dnn, new CConvLayer( e ), "c2", *relu1 );
+	c2->SetFilterCount( 32 ); c2->SetFilterHeight( 3 ); c2->SetFilterWidth( 3 );
+	c2->SetPaddingHeight( 1 ); c2->SetPaddingWidth( 1 );
+	CPtr<CConvLayer> shortcut = add( dnn, new CConvLayer( e ), "shortcut", *pool );
+	shortcut->SetFilterCount( 32 ); shortcut->SetFilterHeight( 1 ); shortcut->SetFilterWidth( 1 );
+	shortcut->SetStrideHeight( 2 ); shortcut->SetStrideWidth( 2 );
+	CPtr<CEltwiseSumLayer> sum = new CEltwiseSumLayer( e );
+	sum->SetName( "sum" );
+	sum->Connect( 0, *c2 );
+	sum->Connect( 1, *shortcut );
+	dnn.AddLayer( *sum );
+	CPtr<CReLULayer> relu2 = add( dnn, new CReLULayer( e ), "relu2", *sum );
+	CPtr<CGlobalMeanPoolingLayer> gap = add( dnn, new CGlobalMeanPoolingLayer( e ), "gap", *relu2 );
+	CPtr<CFullyConnectedLayer> fc = add( dnn, new CFullyConnectedLayer( e ), "fc", *gap );
+	fc->SetNumberOfElements( 10 );
+	CPtr<CSoftmaxLayer> softmax = add( dnn, new CSoftmaxLayer( e ), "softmax", *fc );
+	return softmax.Ptr();
+}
+
+// kind 4: the tail of the line recogniser. Two CLstmLayer over the same input, one reversed, CConcatChannelsLayer,
+//         FullyConnected to param classes + blank. dnn_run returns the FC output; dnn_run_ctc also attaches a
+//         CCtcDecodingLayer and returns every sequence's best labels. Input: [T, B, 1, 1, 1, 1, In].
+static CBaseLayer* buildRecognizerTail( CDnn& dnn, IMathEngine& e, CBaseLayer& source, int classes )
+{
+	CPtr<CLstmLayer> fwd = add( dnn, new CLstmLayer( e ), "fwd", source );
+	fwd->SetHiddenSize( 32 );
+	CPtr<CLstmLayer> rev = add( dnn, new CLstmLayer( e ), "rev", source );
+	rev->SetHiddenSize( 32 );
+	rev->SetReverseSequence( true );
+	CPtr<CConcatChannelsLayer> concat = new CConcatChannelsLayer( e );
+	concat->SetName( "concat" );
+	concat->Connect( 0, *fwd );
+	concat->Connect( 1, *rev );
+	dnn.AddLayer( *concat );
+	CPtr<CFullyConnectedLayer> fc = add( dnn, new CFullyConnectedLayer( e ), "fc", *concat );
+	fc->SetNumberOfElements( classes + 1 );
+	return fc.Ptr();
+}
+
+// Runs network `kind` on `engine`. dims: the 7 blob dimensions of the input; param: kind-specific size.
+// output receives at most outputCapacity floats; outputDims the 7 dimensions of the result.
+EXPORT int dnn_run( void* engine, int kind, int seed, int param, const int* dims, const float* input,
+	float* output, int outputCapacity, int* outputDims )
+{
+	try {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		CRandom random( seed );
+		CDnn dnn( random, e );
+		CPtr<CSourceLayer> source = new CSourceLayer( e );
+		source->SetName( "source" );
+		dnn.AddLayer( *source );
+
+		CBaseLayer* last = nullptr;
+		switch( kind ) {
+			case 0: last = buildCnn( dnn, e, *source ); break;
+			case 1: last = buildTransformer( dnn, e, *source, param ); break;
+			case 2: last = buildLstm( dnn, e, *source, param ); break;
+			case 3: last = buildResNetBlock( dnn, e, *source ); break;
+			case 4: last = buildRecognizerTail( dnn, e, *source, param ); break;
+			default: lastError = "unknown network kind"; return 1;
+		}
+		CPtr<CSinkLayer> sink = new CSinkLayer( e );
+		sink->SetName( "sink" );
+		sink->Connect( *last );
+		dnn.AddLayer( *sink );
+
+		CBlobDesc desc( CT_Float );
+		for( int d = 0; d < 7; ++d ) {
+			desc.SetDimSize( d, dims[d] );
+		}
+		CPtr<CDnnBlob> blob = CDnnBlob::CreateBlob( e, CT_Float, desc );
+		blob->CopyFrom( input );
+		source->SetBlob( blob );
+
+		dnn.RunOnce();
+		// a second pass over the same network: buffers are reused, results must not change
+		dnn.RunOnce();
+
+		const CPtr<CDnnBlob>& result = sink->GetBlob();
+		for( int d = 0; d < 7; ++d ) {
+			outputDims[d] = result->DimSize( d );
+		}
+		if( result->GetDataSize() > outputCapacity ) {
+			lastError = "output buffer too small";
+			return 2;
+		}
+		result->CopyTo( output );
+		return 0;
+	} catch( std::exception& ex ) {
+		lastError = ex.what();
+	} catch( CException* ex ) {
+		lastError = "NeoML exception";
+		delete ex;
+	} catch( ... ) {
+		lastError = "unknown exception";
+	}
+	return 3;
+}
+
+// The recogniser tail (kind 4) with NeoML's CCtcDecodingLayer on top: labels receives, sequence after sequence,
+// the best label sequence of each of the B inputs (at most T each); lengths[b] its length.
+EXPORT int dnn_run_ctc( void* engine, int seed, int classes, const int* dims, const float* input, int* labels, int* lengths )
+{
+	try {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		CRandom random( seed );
+		CDnn dnn( random, e );
+		CPtr<CSourceLayer> source = new CSourceLayer( e );
+		source->SetName( "source" );
+		dnn.AddLayer( *source );
+		CBaseLayer* fc = buildRecognizerTail( dnn, e, *source, classes );
+		CPtr<CCtcDecodingLayer> ctc = new CCtcDecodingLayer( e );
+		ctc->SetName( "ctc" );
+		ctc->SetBlankLabel( classes );
+		ctc->Connect( *fc );
+		dnn.AddLayer( *ctc );
+
+		CBlobDesc desc( CT_Float );
+		for( int d = 0; d < 7; ++d ) {
+			desc.SetDimSize( d, dims[d] );
+		}
+		CPtr<CDnnBlob> blob = CDnnBlob::CreateBlob( e, CT_Float, desc );
+		blob->CopyFrom( input );
+		source->SetBlob( blob );
+		dnn.RunOnce();
+
+		const int T = dims[0], B = dims[1];
+		for( int b = 0; b < B; ++b ) {
+			CArray<int> best;
+			ctc->GetBestSequence( b, best );
+			lengths[b] = best.Size();
+			for( int i = 0; i < best.Size() && i < T; ++i ) {
+				labels[b * T + i] = best[i];
+			}
+		}
+		return 0;
+	} catch( std::exception& ex ) {
+		lastError = ex.what();
+	} catch( CException* ex ) {
+		lastError = "NeoML exception";
+		delete ex;
+	} catch( ... ) {
+		lastError = "unknown exception";
+	}
+	return 3;
+}

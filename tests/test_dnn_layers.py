@@ -1,0 +1,108 @@
+"""NeoML's own layer classes, unchanged, on the HIP engine.
+
+oracle/_ref/libNeoML.so is the reference's layer library compiled from its sources; oracle/dnn_shim.cpp builds small
+CDnn networks from its CConvLayer, CChannelwiseConvLayer, CFullyConnectedLayer, CMaxPoolingLayer, CMeanPoolingLayer,
+CTransformerEncoderLayer and CLstmLayer on the engine it is handed. The same network (same CRandom seed for the
+initialisers, same input) runs on the reference's CCpuMathEngine and on CHipMathEngine; outputs must agree within
+|a-b| <= 1e-5 + 1e-4 |b|. These tests need the reference build (they are skipped where it is absent).
+"""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+import nhtest
+from nhtest import assert_close, f32, fp, ip, i32
+
+DNN_SHIM = os.path.join(nhtest.ORACLE_DIR, "_ref", "libdnn_shim.so")
+pytestmark = pytest.mark.skipif(not (nhtest.have_reference() and os.path.exists(DNN_SHIM)),
+                                reason="reference NeoML build (oracle/_ref) not present")
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        nhtest.shim()  # loads libNeoMathEngine.so first
+        _lib = ctypes.CDLL(DNN_SHIM, mode=ctypes.RTLD_GLOBAL)
+        _lib.dnn_last_error.restype = ctypes.c_char_p
+    return _lib
+
+
+def dnn_run(engine, kind, dims, x, param=0, seed=451):
+    out = np.empty(1 << 22, np.float32)
+    out_dims = np.zeros(7, np.int32)
+    x = f32(x)
+    assert x.size == int(np.prod(dims))
+    rc = lib().dnn_run(engine, kind, seed, param, ip(i32(dims)), fp(x), fp(out), out.size, ip(out_dims))
+    if rc != 0:
+        raise RuntimeError("dnn_run kind %d: %s" % (kind, lib().dnn_last_error().decode()))
+    return out[:int(np.prod(out_dims))].reshape(tuple(out_dims)).copy()
+
+
+CASES = {
+    # kind, input dims [BL, BW, LS, H, W, D, C], param
+    "cnn": (0, (1, 3, 1, 16, 20, 1, 8), 0),
+    "transformer": (1, (1, 3, 24, 1, 1, 1, 32), 32),
+    "lstm": (2, (9, 5, 1, 1, 1, 1, 24), 32),
+    "resnet_block": (3, (1, 2, 1, 40, 48, 1, 3), 0),
+    "recognizer_tail": (4, (12, 4, 1, 1, 1, 1, 16), 20),
+}
+
+
+def make_input(name):
+    kind, dims, param = CASES[name]
+    g = np.random.default_rng(0xC0FFEE + kind)
+    return g.uniform(-1, 1, dims).astype(np.float32)
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_networks_run_on_the_reference_cpu_engine(name):
+    kind, dims, param = CASES[name]
+    y = dnn_run(nhtest.cpu_engine(), kind, dims, make_input(name), param)
+    assert np.isfinite(y).all() and y.size > 0
+    if name in ("cnn", "resnet_block"):
+        assert y.shape[1] == dims[1] and y.shape[6] == 10
+        assert np.allclose(y.reshape(dims[1], 10).sum(axis=1), 1.0, atol=1e-5)
+    # the initialisers are seeded: a second build of the same network gives the same numbers
+    assert np.array_equal(y, dnn_run(nhtest.cpu_engine(), kind, dims, make_input(name), param))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_layers_unchanged_on_hip_engine(name):
+    kind, dims, param = CASES[name]
+    x = make_input(name)
+    want = dnn_run(nhtest.cpu_engine(), kind, dims, x, param)
+    got = dnn_run(nhtest.hip_engine(), kind, dims, x, param)
+    assert got.shape == want.shape
+    assert_close(got, want, "CDnn %s on CHipMathEngine vs CCpuMathEngine" % name)
+
+
+def dnn_run_ctc(engine, dims, x, classes, seed=451):
+    T, B = dims[0], dims[1]
+    labels = np.full(B * T, -1, np.int32)
+    lengths = np.zeros(B, np.int32)
+    rc = lib().dnn_run_ctc(engine, seed, classes, ip(i32(dims)), fp(f32(x)), ip(labels), ip(lengths))
+    if rc != 0:
+        raise RuntimeError("dnn_run_ctc: %s" % lib().dnn_last_error().decode())
+    return [labels[b * T:b * T + lengths[b]].tolist() for b in range(B)]
+
+
+def test_ctc_decoding_layer_agrees_with_oracle_collapse():
+    """CCtcDecodingLayer::GetBestSequence on the CPU engine = arg-max of the FC output + the oracle's greedy collapse."""
+    kind, dims, classes = CASES["recognizer_tail"]
+    x = make_input("recognizer_tail")
+    logits = dnn_run(nhtest.cpu_engine(), kind, dims, x, classes)      # [T, B, 1, 1, 1, 1, classes + 1]
+    T, B = dims[0], dims[1]
+    best = logits.reshape(T, B, classes + 1).argmax(axis=2).T             # [B][T]
+    assert dnn_run_ctc(nhtest.cpu_engine(), dims, x, classes) == nhtest.ctc_greedy_collapse(best, blank=classes)
+
+
+@pytest.mark.gpu
+def test_ctc_decoding_layer_labels_bit_exact_on_hip_engine():
+    kind, dims, classes = CASES["recognizer_tail"]
+    x = make_input("recognizer_tail")
+    assert dnn_run_ctc(nhtest.hip_engine(), dims, x, classes) == dnn_run_ctc(nhtest.cpu_engine(), dims, x, classes)
