@@ -6,6 +6,7 @@
 // CRandom seed for the initialisers, same input, so the two outputs differ only by the engine underneath.
 #include <NeoML/NeoML.h>
 
+#include <chrono>
 #include <exception>
 #include <string>
 #include <string.h>
@@ -17,6 +18,13 @@ static thread_local std::string lastError;
 #define EXPORT extern "C" __attribute__( ( visibility( "default" ) ) )
 
 EXPORT const char* dnn_last_error() { return lastError.c_str(); }
+
+// dnn_run also times `timedPasses` further forward passes when this is set above zero (wall clock around
+// CDnn::RunOnce calls closed by a read-back of the result, i.e. what an application sees); the last timing is kept here
+static int timedPasses = 0;
+static double lastPassMs = 0;
+EXPORT void dnn_set_timed_passes( int passes ) { timedPasses = passes; }
+EXPORT double dnn_last_pass_ms() { return lastPassMs; }
 
 template<class T>
 static CPtr<T> add( CDnn& dnn, T* layer, const char* name, CBaseLayer& input, int outputNumber = 0 )
@@ -138,6 +146,59 @@ static CBaseLayer* buildRecognizerTail( CDnn& dnn, IMathEngine& e, CBaseLayer& s
 	return fc.Ptr();
 }
 
+// kind 5: the whole ResNet-18-style network of the benchmark: 7x7/2 stem (64), pad + 3x3/2 max-pool, 4 stages of 2
+//         basic blocks (64/128/256/512, 1x1/2 shortcut where the shape changes), global mean pool, FC (param classes),
+//         softmax. Input dims: [1, N, 1, H, W, 1, 3].
+static CPtr<CConvLayer> conv( CDnn& dnn, IMathEngine& e, const CString& name, CBaseLayer& input, int filters, int size,
+	int padding, int stride )
+{
+	CPtr<CConvLayer> layer = add( dnn, new CConvLayer( e ), name, input );
+	layer->SetFilterCount( filters ); layer->SetFilterHeight( size ); layer->SetFilterWidth( size );
+	layer->SetPaddingHeight( padding ); layer->SetPaddingWidth( padding );
+	layer->SetStrideHeight( stride ); layer->SetStrideWidth( stride );
+	return layer;
+}
+
+static CBaseLayer* buildResNet18( CDnn& dnn, IMathEngine& e, CBaseLayer& source, int classes )
+{
+	CPtr<CConvLayer> stem = conv( dnn, e, "stem", source, 64, 7, 3, 2 );
+	CPtr<CReLULayer> relu0 = add( dnn, new CReLULayer( e ), "stem_relu", *stem );
+	CPtr<CImageResizeLayer> pad = add( dnn, new CImageResizeLayer( e ), "pad", *relu0 );
+	pad->SetDelta( CImageResizeLayer::IS_Left, 1 ); pad->SetDelta( CImageResizeLayer::IS_Right, 1 );
+	pad->SetDelta( CImageResizeLayer::IS_Top, 1 ); pad->SetDelta( CImageResizeLayer::IS_Bottom, 1 );
+	CPtr<CMaxPoolingLayer> pool = add( dnn, new CMaxPoolingLayer( e ), "pool", *pad );
+	pool->SetFilterHeight( 3 ); pool->SetFilterWidth( 3 ); pool->SetStrideHeight( 2 ); pool->SetStrideWidth( 2 );
+	CBaseLayer* last = pool.Ptr();
+	const int widths[4] = { 64, 128, 256, 512 };
+	int channels = 64;
+	for( int stage = 0; stage < 4; ++stage ) {
+		for( int block = 0; block < 2; ++block ) {
+			const int stride = ( stage > 0 && block == 0 ) ? 2 : 1;
+			const CString prefix = CString( "s" ) + Str( stage ) + "b" + Str( block );
+			CPtr<CConvLayer> c1 = conv( dnn, e, prefix + "c1", *last, widths[stage], 3, 1, stride );
+			CPtr<CReLULayer> r1 = add( dnn, new CReLULayer( e ), prefix + "r1", *c1 );
+			CPtr<CConvLayer> c2 = conv( dnn, e, prefix + "c2", *r1, widths[stage], 3, 1, 1 );
+			CBaseLayer* shortcut = last;
+			if( stride != 1 || channels != widths[stage] ) {
+				shortcut = conv( dnn, e, prefix + "sc", *last, widths[stage], 1, 0, stride ).Ptr();
+			}
+			CPtr<CEltwiseSumLayer> sum = new CEltwiseSumLayer( e );
+			sum->SetName( prefix + "sum" );
+			sum->Connect( 0, *c2 );
+			sum->Connect( 1, *shortcut );
+			dnn.AddLayer( *sum );
+			CPtr<CReLULayer> r2 = add( dnn, new CReLULayer( e ), prefix + "r2", *sum );
+			last = r2.Ptr();
+			channels = widths[stage];
+		}
+	}
+	CPtr<CGlobalMeanPoolingLayer> gap = add( dnn, new CGlobalMeanPoolingLayer( e ), "gap", *last );
+	CPtr<CFullyConnectedLayer> fc = add( dnn, new CFullyConnectedLayer( e ), "fc", *gap );
+	fc->SetNumberOfElements( classes );
+	CPtr<CSoftmaxLayer> softmax = add( dnn, new CSoftmaxLayer( e ), "softmax", *fc );
+	return softmax.Ptr();
+}
+
 // Runs network `kind` on `engine`. dims: the 7 blob dimensions of the input; param: kind-specific size.
 // output receives at most outputCapacity floats; outputDims the 7 dimensions of the result.
 EXPORT int dnn_run( void* engine, int kind, int seed, int param, const int* dims, const float* input,
@@ -158,6 +219,7 @@ EXPORT int dnn_run( void* engine, int kind, int seed, int param, const int* dims
 			case 2: last = buildLstm( dnn, e, *source, param ); break;
 			case 3: last = buildResNetBlock( dnn, e, *source ); break;
 			case 4: last = buildRecognizerTail( dnn, e, *source, param ); break;
+			case 5: last = buildResNet18( dnn, e, *source, param ); break;
 			default: lastError = "unknown network kind"; return 1;
 		}
 		CPtr<CSinkLayer> sink = new CSinkLayer( e );
@@ -176,6 +238,18 @@ EXPORT int dnn_run( void* engine, int kind, int seed, int param, const int* dims
 		dnn.RunOnce();
 		// a second pass over the same network: buffers are reused, results must not change
 		dnn.RunOnce();
+
+		if( timedPasses > 0 ) {
+			float probe = 0;
+			sink->GetBlob()->GetData().GetValue(); // drains the engine's queue before the clock starts
+			const auto start = std::chrono::steady_clock::now();
+			for( int i = 0; i < timedPasses; ++i ) {
+				dnn.RunOnce();
+			}
+			probe = sink->GetBlob()->GetData().GetValue();
+			( void )probe;
+			lastPassMs = std::chrono::duration<double, std::milli>( std::chrono::steady_clock::now() - start ).count() / timedPasses;
+		}
 
 		const CPtr<CDnnBlob>& result = sink->GetBlob();
 		for( int d = 0; d < 7; ++d ) {

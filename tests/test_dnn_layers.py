@@ -49,6 +49,7 @@ CASES = {
     "lstm": (2, (9, 5, 1, 1, 1, 1, 24), 32),
     "resnet_block": (3, (1, 2, 1, 40, 48, 1, 3), 0),
     "recognizer_tail": (4, (12, 4, 1, 1, 1, 1, 16), 20),
+    "resnet18": (5, (1, 2, 1, 64, 64, 1, 3), 100),
 }
 
 
@@ -63,9 +64,9 @@ def test_networks_run_on_the_reference_cpu_engine(name):
     kind, dims, param = CASES[name]
     y = dnn_run(nhtest.cpu_engine(), kind, dims, make_input(name), param)
     assert np.isfinite(y).all() and y.size > 0
-    if name in ("cnn", "resnet_block"):
-        assert y.shape[1] == dims[1] and y.shape[6] == 10
-        assert np.allclose(y.reshape(dims[1], 10).sum(axis=1), 1.0, atol=1e-5)
+    if name in ("cnn", "resnet_block", "resnet18"):
+        assert y.shape[1] == dims[1] and y.shape[6] == (100 if name == "resnet18" else 10)
+        assert np.allclose(y.reshape(dims[1], -1).sum(axis=1), 1.0, atol=1e-5)
     # the initialisers are seeded: a second build of the same network gives the same numbers
     assert np.array_equal(y, dnn_run(nhtest.cpu_engine(), kind, dims, make_input(name), param))
 
@@ -106,3 +107,27 @@ def test_ctc_decoding_layer_labels_bit_exact_on_hip_engine():
     kind, dims, classes = CASES["recognizer_tail"]
     x = make_input("recognizer_tail")
     assert dnn_run_ctc(nhtest.hip_engine(), dims, x, classes) == dnn_run_ctc(nhtest.cpu_engine(), dims, x, classes)
+
+
+@pytest.mark.gpu
+def test_resnet18_through_cdnn_at_benchmark_size(capsys):
+    """The benchmark network at its full size (batch 64, 224x224x3) as a CDnn of the reference's layers on the HIP
+    engine: the drop-in path an application takes. Prints the time per CDnn::RunOnce; the result must be a valid
+    softmax and must equal what the same network gives at batch 2 for its first two images."""
+    dims = (1, 64, 1, 224, 224, 1, 3)
+    g = np.random.default_rng(0xC0FFEE + 102)
+    x = g.uniform(0, 1, dims).astype(np.float32)
+    lib().dnn_set_timed_passes(20)
+    lib().dnn_last_pass_ms.restype = ctypes.c_double
+    try:
+        y = dnn_run(nhtest.hip_engine(), 5, dims, x, 1000).reshape(64, 1000)
+        ms = lib().dnn_last_pass_ms()
+    finally:
+        lib().dnn_set_timed_passes(0)
+    with capsys.disabled():
+        print("\nResNet-18-style, batch 64, CDnn::RunOnce on CHipMathEngine: %.3f ms per pass = %.0f images/sec" % (ms, 64e3 / ms))
+    assert np.allclose(y.sum(axis=1), 1.0, atol=1e-5)
+    small = dnn_run(nhtest.hip_engine(), 5, (1, 2, 1, 224, 224, 1, 3), x[:, :2], 1000).reshape(2, 1000)
+    assert_close(y[:2], small, "batch 64 vs batch 2")
+    want = dnn_run(nhtest.cpu_engine(), 5, (1, 1, 1, 224, 224, 1, 3), x[:, :1], 1000).reshape(1, 1000)
+    assert_close(y[:1], want, "first image vs the CPU engine")
