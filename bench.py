@@ -113,7 +113,7 @@ def main():
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--image", type=int, default=224)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample", type=int, default=8, help="images in the CPU baseline sample")
+    ap.add_argument("--cpu-sample", type=int, default=24, help="images in the CPU baseline sample")
     ap.add_argument("--per-kernel", action="store_true", help="print a per-op-family timing table to stderr")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one nhVectorCopy of 2^26 floats (256 MiB read + 256 MiB written): the known-size "
