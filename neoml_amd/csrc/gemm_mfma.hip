@@ -27,6 +27,7 @@
 // MFMA j of a group therefore reduces over k = {k0 + j, k0 + 4 + j}; both operands use the same permutation of
 // k, which is all the dot product needs.
 #include "common.h"
+#include <math.h>
 
 namespace nh {
 
@@ -573,17 +574,23 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 		setLastError( "matrix product: too many tiles" );
 		return NH_ERR_ARGUMENT;
 	}
-	// K slices: when the tiles alone leave most compute units with one or two workgroups, cut K so that about five
-	// workgroups per compute unit exist; the slices meet in C through fp32 atomic adds (C is pre-set to the free term)
+	// K slices: when the tiles alone leave most compute units with one or two workgroups, K is cut into slices that
+	// meet in C through fp32 atomic adds (C is pre-set to the free term). 1280 workgroups (5 per compute unit) run
+	// at once; the slice count is the one that wastes least of the last round of 1280, each extra slice priced at 2 %
+	// for its atomics, and every slice keeps at least 8 K steps.
 	const int totalSteps = ceilDiv( args.K, NH_KSTEP );
 	int splits = 1;
 	const long long blocks = tiles * batch;
 	if( blocks < 1024 && totalSteps >= 32 ) {
-		splits = static_cast<int>( ( 1280 + blocks / 2 ) / blocks );
-	}
-	splits = splits < 1 ? 1 : splits;
-	if( splits > totalSteps / 8 ) {
-		splits = totalSteps / 8 < 1 ? 1 : totalSteps / 8;
+		double best = 0;
+		for( int s = 1; s <= 8 && s <= totalSteps / 8; ++s ) {
+			const double rounds = static_cast<double>( blocks * s ) / 1280.0;
+			const double cost = ceil( rounds ) / rounds * ( 1.0 + 0.02 * ( s - 1 ) );
+			if( s == 1 || cost < best ) {
+				best = cost;
+				splits = s;
+			}
+		}
 	}
 	args.StepsPerSplit = ceilDiv( totalSteps, splits );
 	args.SplitK = ceilDiv( totalSteps, args.StepsPerSplit );
@@ -706,6 +713,13 @@ int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* sour
 	const bool vec = isAligned16( source ) && isAligned16( filter ) && d.channels % 4 == 0
 		&& fitsBuffer( 1, 0, static_cast<long long>( d.batch ) * d.height * d.width * d.channels )
 		&& fitsBuffer( d.filterCount, args.K, args.K );
+	if( d.filterHeight == 1 && d.filterWidth == 1 && d.strideHeight == 1 && d.strideWidth == 1
+		&& d.paddingHeight == 0 && d.paddingWidth == 0 )
+	{
+		// a pointwise convolution over a channels-last image is the plain product image[M x Cin] * filter[Cout x Cin]^T
+		return matMulNT( stream, source, d.channels, filter, d.channels, result, d.filterCount, args.M, args.N, d.channels,
+			1, 0, 0, 0, freeTerm, false );
+	}
 	if( d.filterHeight == 1 && d.filterWidth == 1 ) {
 		return launchMatMul<AM_Conv1x1, BM_RowsK>( stream, args, 1, vec );
 	}
