@@ -184,6 +184,12 @@ def main():
         measure("VectorSigmoid n=%d" % n, lambda: lib.nhVectorSigmoid(stream, P(a), P(c), n), 0, 8 * n, 8 * n)
         measure("VectorEltwiseMultiply n=%d" % n, lambda: lib.nhVectorEltwiseMultiply(stream, P(a), P(b), P(c), n), 0, 12 * n, 12 * n)
         del a, b, c
+    for n in (1 << 26, 1 << 28):
+        c = empty(n)
+        measure("VectorFill (write only) n=%d" % n, lambda: lib.nhVectorFill(stream, P(c), ctypes.c_float(1.5), n), 0, 4 * n, 4 * n)
+        a = rand(n)
+        measure("VectorSum (read only) n=%d" % n, lambda: lib.nhVectorSum(stream, P(a), n, P(zero)), 0, 4 * n, 4 * n)
+        del a, c
     n = 8192 * 512
     a, c = rand(n), empty(n)
     measure("VectorTanh n=%d" % n, lambda: lib.nhVectorTanh(stream, P(a), P(c), n), 0, 8 * n, 8 * n)
