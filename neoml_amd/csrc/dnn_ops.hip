@@ -3,6 +3,7 @@
 // recurrence (matrix products on the MFMA kernels + one fused gate kernel per step).
 #include "common.h"
 #include <float.h>
+#include <stdlib.h>
 
 namespace nh {
 
@@ -611,6 +612,317 @@ void lstmStepKernel( const float* pre, const float* hPrev, const float* wRec, co
 	mainOut[cell] = o * tanhf( c );
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// The whole sequence in ONE launch. The per-step launch above costs about 7 us per step, nearly all of it the
+// launch latency between dependent kernels; here the workgroups stay resident for all T steps and hand each
+// step's output to one another through memory.
+//   workgroup  = 4*CB hidden units x RB (16 or 32) sequences, W wavefronts: the gate columns of those units are CB
+//                16-wide MFMA blocks; their rows of Wrec (16*CB x H) are copied to LDS once and stay there for all
+//                steps, the cell state of the workgroup's cells lives in registers for all steps;
+//   per step   : the wavefronts split the reduction over H in chunks of 16 k (v_mfma_f32_16x16x4_f32), meet in
+//                LDS, and every wavefront does the cell update of its share of the (sequence, unit) cells;
+//   exchange   : besides the plain store into the output blob, every h value is published as a 64-bit word
+//                { float bits, step tag } with ONE device-scope relaxed atomic store (it goes to the level where the
+//                eight L2s of the device agree). A consumer loads the words of the rows it multiplies with
+//                device-scope atomic loads and repeats the loads until every tag names the step it needs: value and
+//                "it has been written" arrive in the same word, so a step costs one store-to-load visibility
+//                latency, with no counter, no flag and no fence. (An arrival counter bumped by 256 workgroups cost
+//                6 us per step; device-scope fences, which write back and invalidate L2, 27 us.)
+//                Such loads are not served by L2 and their round trip grows with the volume in flight, so wide
+//                workgroups (many units, every published word read by few workgroups) beat many narrow ones.
+//                Two exchange buffers alternate by step parity: a workgroup can only write step i+2 after it has
+//                read step i+1 from every producer of its rows, i.e. after all of them finished reading step i.
+//                The host clears the buffers before the launch, tags start at 1, so stale memory never matches.
+// All workgroups must be resident together: the host only takes this path when the grid fits the device. The wait
+// is bounded: after MaxSpins rounds of loads, or when another workgroup gave up, a wavefront raises the abort word
+// and the workgroup leaves at its next barrier, so the grid always drains.
+constexpr int SeqUnits = 4; // hidden units per 16-column block: column n = unit n/4, gate n%4
+typedef float f32x4v __attribute__( ( ext_vector_type( 4 ) ) );
+
+struct CLstmSeqArgs {
+	const float* Gates;            // [T][B][4H] input contribution + free term
+	const float* Wrec;             // [4H][H]
+	const float* H0;               // [B][H] or null
+	const float* C0;               // [B][H] or null
+	float* HOut;                   // [T][B][H]
+	float* COut;                   // [T][B][H] or null
+	unsigned long long* Exchange;  // [2][B][H] tagged h values, zero at launch
+	unsigned* Abort;               // one word, zero at launch
+	int T, B, H, Reverse;
+	unsigned MaxSpins;
+};
+
+// Gate non-linearities on the hardware exp2 / reciprocal: 1 ulp each, and the cell update of a step sits on the
+// critical path of the whole device. Saturation: exp2 gives +inf / 0 at the ends, the reciprocal turns them into the
+// 0 / 1 (-1 / 1) that the clamped reference formulas give.
+__device__ __forceinline__ float seqSigmoid( float x )
+{
+	return __builtin_amdgcn_rcpf( 1.f + __builtin_amdgcn_exp2f( -1.4426950408889634f * x ) );
+}
+__device__ __forceinline__ float seqTanh( float x )
+{
+	return 1.f - 2.f * __builtin_amdgcn_rcpf( 1.f + __builtin_amdgcn_exp2f( 2.8853900817779268f * x ) );
+}
+
+
+template<int RB, int CB, int W>
+__global__ __launch_bounds__( 64 * W )
+void lstmSequenceKernel( const CLstmSeqArgs a )
+{
+	extern __shared__ __attribute__( ( aligned( 16 ) ) ) float seqLds[];
+	__shared__ int giveUp;
+	constexpr int Threads = 64 * W;
+	constexpr int RBlocks = RB / 16;
+	constexpr int Units = CB * SeqUnits;  // hidden units of this workgroup
+	constexpr int Cols = CB * 16;         // their gate columns
+	constexpr int PartPitch = Cols + 4;   // rows stay 16-byte aligned: a cell reads its four gates with one 128-bit load
+	constexpr int Batch = 16; // words per thread whose loads are in flight together
+	// The first half of the wavefronts update the cells and publish, the second half fetch the next step's values.
+	// A wavefront's loads and stores complete in issue order, so a wavefront that has just published could only
+	// consume a load once its stores have been acknowledged by the far end (about half a microsecond).
+	constexpr int CellWaves = W / 2;
+	constexpr int CellsPerWave = RB * Units / CellWaves;
+	constexpr int LoadThreads = ( W - CellWaves ) * 64;
+	static_assert( CellsPerWave <= 64 && CellsPerWave * CellWaves == RB * Units, "the cells divide evenly over the cell wavefronts" );
+	const int H = a.H, B = a.B;
+	const int pitch = H + 4;
+	float* wLds = seqLds;                   // [Cols][pitch]  this workgroup's rows of Wrec
+	float* hTile = wLds + Cols * pitch;     // [RB][pitch]    the previous step's output of this workgroup's sequences
+	float* partial = hTile + RB * pitch + 4; // [W][RB][PartPitch]; the 4 floats between are the loaders' spare slot
+	const int tid = threadIdx.x;
+	const int wave = tid >> 6;
+	const int lane = tid & 63;
+	const int col = lane & 15; // MFMA: row of the A block / column of the B block
+	const int kq = lane >> 4;  // MFMA: which 4 of the 16 k of a chunk
+	const int unitBlocks = H / Units;
+	const int unit0 = ( blockIdx.x % unitBlocks ) * Units;
+	const int row0 = ( blockIdx.x / unitBlocks ) * RB;
+	const int rowsHere = min( RB, B - row0 );
+
+	// gate column n of this workgroup = unit unit0 + n/4, gate n%4: the four gates of a cell are neighbours
+	for( int idx = tid; idx < Cols * ( H / 4 ); idx += Threads ) {
+		const int n = idx / ( H / 4 );
+		const int k4 = idx - n * ( H / 4 );
+		const int gate = n & 3;
+		const int unit = unit0 + ( n >> 2 );
+		const float4 v = *reinterpret_cast<const float4*>( a.Wrec + ( static_cast<long long>( gate ) * H + unit ) * H + k4 * 4 );
+		*reinterpret_cast<float4*>( wLds + n * pitch + k4 * 4 ) = v;
+	}
+	// rows of the tile beyond the last sequence stay zero for all steps
+	for( int idx = tid; idx < RB * pitch; idx += Threads ) {
+		hTile[idx] = 0.f;
+	}
+	__syncthreads();
+	if( a.H0 != nullptr ) {
+		const int rows = min( RB, B - row0 );
+		for( int j = tid; j < rows * H; j += Threads ) {
+			hTile[( j / H ) * pitch + j % H] = a.H0[static_cast<long long>( row0 ) * H + j];
+		}
+	}
+	if( tid == 0 ) {
+		giveUp = 0;
+	}
+
+	// the cell this thread updates
+	const int cellId = wave * CellsPerWave + lane;
+	const int cellRow = cellId / Units;
+	const int cellUnit = cellId % Units;
+	const int cellB = row0 + cellRow;
+	const bool cellActive = wave < CellWaves && lane < CellsPerWave && cellB < B;
+	const bool loader = wave >= CellWaves;
+	const int loadTid = tid - CellWaves * 64;
+	const int cellCol = cellUnit * 4; // its four gate columns
+	float cState = ( cellActive && a.C0 != nullptr ) ? a.C0[static_cast<long long>( cellB ) * H + unit0 + cellUnit] : 0.f;
+	const long long stepSize = static_cast<long long>( B ) * H;
+	const int chunks = H / 16;
+	const int tileWords = rowsHere * H; // the tile's rows are contiguous in [B][H]
+	const long long tileBase = static_cast<long long>( row0 ) * H;
+	__syncthreads();
+
+	// the input contribution of the step after the current one is requested a step ahead, before the current
+	// step's stores are issued: loads return in order, so a load issued after the (slow, device-coherent) stores
+	// could only be consumed once those stores have been acknowledged
+	float gNext[4] = { 0.f, 0.f, 0.f, 0.f };
+	auto requestGates = [&]( int step ) {
+		if( cellActive && step < a.T ) {
+			const int p = a.Reverse ? a.T - 1 - step : step;
+			const float* src = a.Gates + ( static_cast<long long>( p ) * B + cellB ) * 4 * H + unit0 + cellUnit;
+#pragma unroll
+			for( int q = 0; q < 4; ++q ) {
+				gNext[q] = src[q * H];
+			}
+		}
+	};
+	requestGates( 0 );
+
+	// Loader thread t fetches words t, t + LoadThreads, ... of the tile ( word j = row j / H, column j % H ): a
+	// wavefront's load covers 64 consecutive words, whole cache lines, each requested once. The positions are worked
+	// out once: integer division by H inside the step loop would cost more than the loads. The host only picks a
+	// shape whose loaders cover the tile in one batch ( RB * H <= Batch * LoadThreads ).
+	int wordIndex[Batch], ldsIndex[Batch];
+	unsigned wordMask[Batch]; // all ones inside the tile, zero beyond it
+#pragma unroll
+	for( int n = 0; n < Batch; ++n ) {
+		const int j = n * LoadThreads + loadTid;
+		const bool inside = loader && j < tileWords;
+		wordIndex[n] = inside ? j : 0;
+		wordMask[n] = inside ? 0xffffffffu : 0u;
+		ldsIndex[n] = inside ? ( j / H ) * pitch + j % H : RB * pitch;
+	}
+
+	for( int i = 0; i < a.T; ++i ) {
+		const int pos = a.Reverse ? a.T - 1 - i : i;
+		const bool havePrev = i > 0 || a.H0 != nullptr;
+		// ---- the previous output of this workgroup's sequences -> hTile (step 0: put there before the loop)
+		if( i > 0 && loader ) {
+			const unsigned long long* published = a.Exchange + ( ( i - 1 ) & 1 ) * stepSize + tileBase;
+			const unsigned tag = static_cast<unsigned>( i ); // step i-1 publishes with tag i
+			// Every load of a round is unconditional and all are in flight together (a conditional atomic load cannot be
+			// hoisted): words beyond the tile read word 0, are not checked and land in the spare LDS slot.
+			unsigned long long word[Batch];
+			unsigned spins = 0;
+			// A round of Batch loads per thread takes about half a microsecond, one load a fifth of that: wait on the
+			// first word of every thread (together they touch every producer) before asking for everything.
+			while( true ) {
+				const unsigned long long first = __hip_atomic_load( published + wordIndex[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT );
+				const unsigned mismatch = ( static_cast<unsigned>( first >> 32 ) ^ tag ) & wordMask[0];
+				if( __builtin_amdgcn_ballot_w64( mismatch != 0 ) == 0 || ++spins > a.MaxSpins ) {
+					break; // ( at the spin limit the full round below fails and gives up )
+				}
+			}
+			while( true ) {
+#pragma unroll
+				for( int n = 0; n < Batch; ++n ) {
+					word[n] = __hip_atomic_load( published + wordIndex[n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT );
+				}
+				unsigned mismatch = 0; // branch-free: every tag xor the wanted one, or-ed
+#pragma unroll
+				for( int n = 0; n < Batch; ++n ) {
+					mismatch |= ( static_cast<unsigned>( word[n] >> 32 ) ^ tag ) & wordMask[n];
+				}
+				if( __builtin_amdgcn_ballot_w64( mismatch != 0 ) == 0 ) {
+					break;
+				}
+				if( ++spins > a.MaxSpins || ( ( spins & 15 ) == 0
+					&& __hip_atomic_load( a.Abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT ) != 0 ) )
+				{
+					__hip_atomic_store( a.Abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT );
+					giveUp = 1; // read by the whole workgroup after the next barrier
+					break;
+				}
+			}
+#pragma unroll
+			for( int n = 0; n < Batch; ++n ) {
+				hTile[ldsIndex[n]] = __uint_as_float( static_cast<unsigned>( word[n] ) );
+			}
+		}
+		__syncthreads();
+		if( giveUp != 0 ) {
+			return; // uniform: every thread reads the same LDS word after the barrier
+		}
+
+		// ---- gates += hTile * Wrec^T for this workgroup's columns; the wavefronts split the reduction over H
+		// One accumulator per ( column block, row block, k lane of the chunk ): consecutive MFMAs never wait for one
+		// another's result; the four k lanes are summed at the end.
+		f32x4v acc[CB][RBlocks][4];
+#pragma unroll
+		for( int cb = 0; cb < CB; ++cb ) {
+#pragma unroll
+			for( int rb = 0; rb < RBlocks; ++rb ) {
+#pragma unroll
+				for( int e = 0; e < 4; ++e ) {
+					acc[cb][rb][e] = f32x4v{ 0.f, 0.f, 0.f, 0.f };
+				}
+			}
+		}
+		if( havePrev ) {
+			for( int chunk = wave; chunk < chunks; chunk += W ) {
+				const int k = chunk * 16 + kq * 4;
+				// MFMA e of the chunk reduces over k = chunk*16 + { e, 4+e, 8+e, 12+e }: the same pairing on both operands
+				float4 w[CB], h[RBlocks];
+#pragma unroll
+				for( int cb = 0; cb < CB; ++cb ) {
+					w[cb] = *reinterpret_cast<const float4*>( wLds + ( cb * 16 + col ) * pitch + k );
+				}
+#pragma unroll
+				for( int rb = 0; rb < RBlocks; ++rb ) {
+					h[rb] = *reinterpret_cast<const float4*>( hTile + ( rb * 16 + col ) * pitch + k );
+				}
+#pragma unroll
+				for( int rb = 0; rb < RBlocks; ++rb ) {
+#pragma unroll
+					for( int cb = 0; cb < CB; ++cb ) {
+						acc[cb][rb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32( h[rb].x, w[cb].x, acc[cb][rb][0], 0, 0, 0 );
+						acc[cb][rb][1] = __builtin_amdgcn_mfma_f32_16x16x4f32( h[rb].y, w[cb].y, acc[cb][rb][1], 0, 0, 0 );
+						acc[cb][rb][2] = __builtin_amdgcn_mfma_f32_16x16x4f32( h[rb].z, w[cb].z, acc[cb][rb][2], 0, 0, 0 );
+						acc[cb][rb][3] = __builtin_amdgcn_mfma_f32_16x16x4f32( h[rb].w, w[cb].w, acc[cb][rb][3], 0, 0, 0 );
+					}
+				}
+			}
+		}
+		// accumulator register r of lane l is element ( row 4*(l/16) + r, column l%16 ) of the 16 x 16 block
+#pragma unroll
+		for( int cb = 0; cb < CB; ++cb ) {
+#pragma unroll
+			for( int rb = 0; rb < RBlocks; ++rb ) {
+#pragma unroll
+				for( int r = 0; r < 4; ++r ) {
+					partial[( wave * RB + rb * 16 + kq * 4 + r ) * PartPitch + cb * 16 + col] =
+						( acc[cb][rb][0][r] + acc[cb][rb][1][r] ) + ( acc[cb][rb][2][r] + acc[cb][rb][3][r] );
+				}
+			}
+		}
+		__syncthreads();
+		float g[4];
+#pragma unroll
+		for( int q = 0; q < 4; ++q ) {
+			g[q] = gNext[q];
+		}
+		if( cellActive ) {
+			float4 part[W];
+#pragma unroll
+			for( int wv = 0; wv < W; ++wv ) {
+				part[wv] = *reinterpret_cast<const float4*>( partial + ( wv * RB + cellRow ) * PartPitch + cellCol );
+			}
+#pragma unroll
+			for( int wv = 0; wv < W; ++wv ) {
+				g[0] += part[wv].x; g[1] += part[wv].y; g[2] += part[wv].z; g[3] += part[wv].w;
+			}
+		}
+		// ( `partial` and `hTile` are next written after the tile barrier of step i+1, which the cell wavefronts only
+		// reach when they are done reading )
+		requestGates( i + 1 );
+		if( cellActive ) {
+			const float m = seqTanh( g[0] );
+			const float f = seqSigmoid( g[1] );
+			const float in = seqSigmoid( g[2] );
+			const float o = seqSigmoid( g[3] );
+			cState = f * cState + in * m;
+			const float h = o * seqTanh( cState );
+			const long long cellInStep = static_cast<long long>( cellB ) * H + unit0 + cellUnit;
+			if( i + 1 < a.T ) {
+				const unsigned long long word = ( static_cast<unsigned long long>( i + 1 ) << 32 ) | __float_as_uint( h );
+				__hip_atomic_store( a.Exchange + ( i & 1 ) * stepSize + cellInStep, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT );
+			}
+			a.HOut[pos * stepSize + cellInStep] = h;
+			if( a.COut != nullptr ) {
+				a.COut[pos * stepSize + cellInStep] = cState;
+			}
+		}
+		// The loader wavefronts start asking for step i's values only now that this workgroup has published its own
+		// (the workgroups run in lockstep, so the others are about as far): a round of loads issued earlier would
+		// come back incomplete and cost a whole round trip.
+		__syncthreads();
+	}
+}
+
+__global__ __launch_bounds__( 256 ) void clearWordsKernel( unsigned long long* words, long long count )
+{
+	for( long long i = blockIdx.x * 256LL + threadIdx.x; i < count; i += gridDim.x * 256LL ) {
+		words[i] = 0;
+	}
+}
+
 __global__ void addTwoVectorsKernel( const float* a, const float* b, float* out, int n )
 {
 	const int i = blockIdx.x * 256 + threadIdx.x;
@@ -624,6 +936,119 @@ __global__ void addTwoVectorsKernel( const float* a, const float* b, float* out,
 using namespace nh;
 
 extern "C" int nhInitPooling( nhPoolingDesc* d );
+
+// ---- whole-sequence LSTM launch ------------------------------------------------------------------------------
+
+// The shapes of the one-launch kernel: Rows sequences x ( 4 * Blocks ) hidden units per workgroup of Waves wavefronts.
+struct CLstmSeqShape {
+	int Rows, Blocks, Waves;
+	const void* Kernel;
+	void ( *Launch )( hipStream_t, unsigned, size_t, const CLstmSeqArgs& );
+};
+
+template<int RB, int CB, int W>
+static void launchSeqShape( hipStream_t stream, unsigned groups, size_t lds, const CLstmSeqArgs& a )
+{
+	hipLaunchKernelGGL( ( lstmSequenceKernel<RB, CB, W> ), dim3( groups ), dim3( 64 * W ), lds, stream, a );
+}
+
+#define NH_SEQ_SHAPE( RB, CB, W ) { RB, CB, W, reinterpret_cast<const void*>( &lstmSequenceKernel<RB, CB, W> ), &launchSeqShape<RB, CB, W> }
+// in order of preference (measured at 64 sequences x 256 units, 128 steps: 433 / 445 / 515 us for the first three;
+// a v_mfma_f32_16x16x4_f32 issues every 64 clocks, so the narrow workgroup has the shortest product phase)
+static const CLstmSeqShape lstmSeqShapes[] = {
+	NH_SEQ_SHAPE( 16, 1, 8 ), NH_SEQ_SHAPE( 16, 2, 8 ), NH_SEQ_SHAPE( 16, 4, 8 ), NH_SEQ_SHAPE( 16, 2, 16 ), NH_SEQ_SHAPE( 16, 4, 16 ),
+	NH_SEQ_SHAPE( 32, 2, 16 ) };
+constexpr size_t LdsLimit = 160 * 1024 - 256; // dynamic part; the kernel also has a static word
+
+static size_t lstmSequenceLds( int H, const CLstmSeqShape& shape )
+{
+	const size_t cols = 16 * static_cast<size_t>( shape.Blocks );
+	return ( ( cols + shape.Rows ) * ( H + 4 ) + 4 + static_cast<size_t>( shape.Waves ) * shape.Rows * ( cols + 4 ) ) * sizeof( float );
+}
+
+// The first shape whose grid fits the device; null = none does.
+static const CLstmSeqShape* lstmSequenceShape( int H, int B )
+{
+	static int computeUnits = 0; // the engine drives one device per process
+	static bool ldsRaised = false;
+	if( computeUnits == 0 ) {
+		int device = 0, count = 0;
+		if( hipGetDevice( &device ) != hipSuccess
+			|| hipDeviceGetAttribute( &count, hipDeviceAttributeMultiprocessorCount, device ) != hipSuccess || count <= 0 )
+		{
+			( void )hipGetLastError();
+			return nullptr;
+		}
+		computeUnits = count;
+	}
+	if( !ldsRaised ) {
+		// beyond 64 KB of dynamic LDS a kernel has to ask
+		for( const CLstmSeqShape& shape : lstmSeqShapes ) {
+			const hipError_t err = hipFuncSetAttribute( shape.Kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>( LdsLimit ) );
+			if( err != hipSuccess ) {
+				setLastError( "lstm: hipFuncSetAttribute failed: %s", hipGetErrorString( err ) );
+				( void )hipGetLastError();
+				return nullptr;
+			}
+		}
+		ldsRaised = true;
+	}
+	for( const CLstmSeqShape& shape : lstmSeqShapes ) {
+		const size_t lds = lstmSequenceLds( H, shape );
+		const int batch = 16; // the kernel's Batch
+		if( H % ( SeqUnits * shape.Blocks ) != 0 || lds > LdsLimit
+			|| static_cast<long long>( shape.Rows ) * H > static_cast<long long>( batch ) * ( shape.Waves / 2 ) * 64 )
+		{
+			continue;
+		}
+		int perUnit = 0;
+		const hipError_t err = hipOccupancyMaxActiveBlocksPerMultiprocessor( &perUnit, shape.Kernel, 64 * shape.Waves, lds );
+		if( err != hipSuccess ) {
+			setLastError( "lstm: occupancy query failed: %s", hipGetErrorString( err ) );
+			( void )hipGetLastError();
+			continue;
+		}
+		// one workgroup per compute unit is what the dispatcher certainly places side by side on an otherwise idle
+		// device; the occupancy figure only confirms that one fits
+		const long long groups = static_cast<long long>( H / ( SeqUnits * shape.Blocks ) ) * ceilDiv( B, shape.Rows );
+		if( perUnit >= 1 && groups <= computeUnits ) {
+			return &shape;
+		}
+	}
+	return nullptr;
+}
+
+static bool lstmSequenceFits( int H, int B, const float* wRec, const float* c0, const float* h0, const float* hOut )
+{
+	( void )c0;
+	return H % 16 == 0 && isAligned16( wRec ) && isAligned16( hOut ) && ( h0 == nullptr || isAligned16( h0 ) )
+		&& lstmSequenceShape( H, B ) != nullptr;
+}
+
+// Rounds of loads a wavefront makes for one step's values before it gives up (a round is a trip to the device-level
+// coherence point: about a microsecond).
+// NH_LSTM_SPIN_LIMIT overrides it; tests use a tiny value to drive the give-up path from the host.
+static unsigned lstmSpinLimit()
+{
+	const char* env = getenv( "NH_LSTM_SPIN_LIMIT" );
+	if( env != nullptr && *env != 0 ) {
+		return static_cast<unsigned>( strtoul( env, nullptr, 10 ) );
+	}
+	return 4u << 20;
+}
+
+static int launchLstmSequence( hipStream_t stream, const CLstmSeqArgs& a )
+{
+	const CLstmSeqShape* shape = lstmSequenceShape( a.H, a.B );
+	NH_REQUIRE( shape != nullptr );
+	const unsigned groups = static_cast<unsigned>( ( a.H / ( SeqUnits * shape->Blocks ) ) * ceilDiv( a.B, shape->Rows ) );
+	// the exchange buffers and the abort word that follows them
+	const long long words = 2LL * a.B * a.H + 1;
+	hipLaunchKernelGGL( clearWordsKernel, dim3( static_cast<unsigned>( ( words + 1023 ) / 1024 ) ), dim3( 256 ), 0, stream, a.Exchange, words );
+	shape->Launch( stream, groups, lstmSequenceLds( a.H, *shape ), a );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
 
 static int checkPoolingDesc( const nhPoolingDesc* d )
 {
@@ -842,12 +1267,12 @@ int nhBlobSplitByDim( nhStream s, int dim, const nhBlobDesc* from, const float* 
 	return splitMergeImpl<false>( s, dim, *from, const_cast<float*>( fromData ), to, toData, toCount );
 }
 
-// workspace layout: [ gates: T*B*4H ][ free term: 4H ][ state: B*H ]
+// workspace layout: [ gates: T*B*4H ][ free term: 4H ][ state: B*H ][ tagged h exchange: 2*B*H 64-bit words ][ abort word: 64 bits ]
 int nhLstmWorkspaceSize( int hiddenSize, int objectSize, int sequenceLength, int sequenceCount, size_t* bytes )
 {
 	NH_REQUIRE( bytes != nullptr && hiddenSize > 0 && objectSize > 0 && sequenceLength >= 0 && sequenceCount >= 0 );
 	const size_t gates = static_cast<size_t>( sequenceLength ) * sequenceCount * 4 * hiddenSize;
-	*bytes = ( gates + 4 * static_cast<size_t>( hiddenSize ) + static_cast<size_t>( sequenceCount ) * hiddenSize ) * sizeof( float );
+	*bytes = ( gates + 4 * static_cast<size_t>( hiddenSize ) + 5 * static_cast<size_t>( sequenceCount ) * hiddenSize + 2 ) * sizeof( float );
 	return NH_OK;
 }
 
@@ -889,6 +1314,16 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 		return rc;
 	}
 	const int stepSize = B * H;
+	if( T > 1 && lstmSequenceFits( H, B, recurrentWeights, inputStateBackLink, inputMainBackLink, outputMainBackLink ) ) {
+		CLstmSeqArgs a = {};
+		a.Gates = gates; a.Wrec = recurrentWeights; a.H0 = inputMainBackLink; a.C0 = inputStateBackLink;
+		a.HOut = outputMainBackLink; a.COut = outputStateBackLink;
+		a.Exchange = reinterpret_cast<unsigned long long*>( stateScratch + static_cast<size_t>( B ) * H );
+		a.Abort = reinterpret_cast<unsigned*>( a.Exchange + 2 * static_cast<size_t>( B ) * H );
+		a.T = T; a.B = B; a.H = H; a.Reverse = reverse ? 1 : 0;
+		a.MaxSpins = lstmSpinLimit();
+		return launchLstmSequence( stream, a );
+	}
 	// the one-launch step needs whole 32-k chunks and 8-unit blocks, 16-byte aligned rows and 32-bit byte offsets
 	const bool fusedStep = H % 32 == 0 && isAligned16( recurrentWeights ) && isAligned16( outputMainBackLink )
 		&& ( inputMainBackLink == nullptr || isAligned16( inputMainBackLink ) )

@@ -731,7 +731,7 @@ class Hip:
         self.call("nhBlobMergeByDim", dim, descs, ptrs, len(ps), ctypes.byref(bd), self.p(out))
         return self.down(out)
 
-    def lstm(self, w_in, b_in, w_rec, b_rec, x, reverse=False, c0=None, h0=None, want_state=True):
+    def lstm(self, w_in, b_in, w_rec, b_rec, x, reverse=False, c0=None, h0=None, want_state=True, return_sync=False):
         x = f32(x)
         T, B, In = x.shape
         H = w_rec.shape[1]
@@ -743,6 +743,10 @@ class Hip:
         work = self.torch.empty((size.value + 15) // 4, dtype=self.torch.float32, device=self.dev)
         self.call("nhLstm", H, In, self.p(ws[0]), self.p(ws[1]), self.p(ws[2]), self.p(ws[3]), 1 if reverse else 0, T, B,
                   self.p(ws[4]), self.p(ws[5]), self.p(ws[6]), self.p(c), self.p(h), self.p(work), size.value)
+        if return_sync:
+            # the last 8 bytes of the workspace hold the abort word of the one-launch path
+            word = int(work.view(self.torch.int32)[size.value // 4 - 2].item())
+            return self.down(h), (self.down(c) if want_state else None), word
         return self.down(h), (self.down(c) if want_state else None)
 
 

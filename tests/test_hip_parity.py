@@ -384,6 +384,42 @@ def test_lstm(reverse, with_init):
             assert_close(h2, oh, "lstm h without state output")
 
 
+def test_lstm_long_sequence():
+    # 128 steps through the one-launch path (H a multiple of 16 and a grid that fits the device), H = 512 through
+    # its 16-wavefront shape, plus a shape whose grid does not fit and takes the launch-per-step path
+    g = rng(181)
+    for T, B, In, H in ((128, 20, 24, 128), (6, 20, 16, 512), (3, 40, 16, 1024)):
+        w_in = g.uniform(-0.2, 0.2, (4 * H, In)).astype(np.float32)
+        w_rec = g.uniform(-2.0 / H ** 0.5, 2.0 / H ** 0.5, (4 * H, H)).astype(np.float32)
+        b_in = g.uniform(-0.5, 0.5, 4 * H).astype(np.float32)
+        x = g.uniform(-1, 1, (T, B, In)).astype(np.float32)
+        for reverse in (False, True):
+            h, c = hip().lstm(w_in, b_in, w_rec, None, x, reverse)
+            oh, oc = orc.lstm(w_in, b_in, w_rec, None, x, reverse)
+            assert_close(h, oh, "lstm h %s" % ((T, B, In, H),))
+            assert_close(c, oc, "lstm c %s" % ((T, B, In, H),))
+
+
+def test_lstm_bounded_wait_gives_up(monkeypatch):
+    # The step wait of the one-launch LSTM is bounded. With a spin limit of zero, forced from the host, a
+    # wavefront that finds a value of the previous step not yet published raises the abort word and every
+    # workgroup leaves: the launch ends normally and the word is visible in the workspace. (If every value
+    # happens to be there in time, the word stays zero and the output is the regular one.)
+    g = rng(182)
+    T, B, In, H = 64, 64, 16, 256
+    w_in = g.uniform(-0.2, 0.2, (4 * H, In)).astype(np.float32)
+    w_rec = g.uniform(-0.1, 0.1, (4 * H, H)).astype(np.float32)
+    x = g.uniform(-1, 1, (T, B, In)).astype(np.float32)
+    monkeypatch.setenv("NH_LSTM_SPIN_LIMIT", "0")
+    h, _, word = hip().lstm(w_in, None, w_rec, None, x, want_state=False, return_sync=True)
+    monkeypatch.delenv("NH_LSTM_SPIN_LIMIT")
+    assert word in (0, 1)
+    h2, _, word2 = hip().lstm(w_in, None, w_rec, None, x, want_state=False, return_sync=True)
+    assert word2 == 0
+    oh, _ = orc.lstm(w_in, None, w_rec, None, x)
+    assert_close(h2, oh, "lstm after a forced give-up")
+
+
 # ---------------------------------------------------------------------------------------------------------
 # error convention and allocator on the device
 
