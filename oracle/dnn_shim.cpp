@@ -5,6 +5,7 @@
 // The tests call them once with the reference's CPU engine and once with the HIP engine: same layer code, same
 // CRandom seed for the initialisers, same input, so the two outputs differ only by the engine underneath.
 #include <NeoML/NeoML.h>
+#include "HipLstmLayer.h" // neoml_amd/engine: the LSTM layer that reaches IMathEngine::Lstm on a non-CPU engine
 
 #include <chrono>
 #include <exception>
@@ -25,6 +26,14 @@ static int timedPasses = 0;
 static double lastPassMs = 0;
 EXPORT void dnn_set_timed_passes( int passes ) { timedPasses = passes; }
 EXPORT double dnn_last_pass_ms() { return lastPassMs; }
+
+// LSTM layers of the networks below: NeoML's own CLstmLayer (0) or this repository's CHipLstmLayer (1); hidden size of
+// the two LSTM layers of network kind 4
+static int fusedLstm = 0;
+static int tailHidden = 32;
+EXPORT void dnn_set_fused_lstm( int on ) { fusedLstm = on; }
+EXPORT void dnn_set_tail_hidden( int hidden ) { tailHidden = hidden; }
+static CLstmLayer* newLstm( IMathEngine& e ) { return fusedLstm != 0 ? new CHipLstmLayer( e ) : new CLstmLayer( e ); }
 
 template<class T>
 static CPtr<T> add( CDnn& dnn, T* layer, const char* name, CBaseLayer& input, int outputNumber = 0 )
@@ -81,7 +90,7 @@ static CBaseLayer* buildTransformer( CDnn& dnn, IMathEngine& e, CBaseLayer& sour
 // kind 2: CLstmLayer (hidden = param) followed by a FullyConnected over every step. Input: [T, B, 1, 1, 1, 1, In].
 static CBaseLayer* buildLstm( CDnn& dnn, IMathEngine& e, CBaseLayer& source, int hidden )
 {
-	CPtr<CLstmLayer> lstm = add( dnn, new CLstmLayer( e ), "lstm", source );
+	CPtr<CLstmLayer> lstm = add( dnn, newLstm( e ), "lstm", source );
 	lstm->SetHiddenSize( hidden );
 	CPtr<CFullyConnectedLayer> fc = add( dnn, new CFullyConnectedLayer( e ), "fc", *lstm );
 	fc->SetNumberOfElements( 11 );
@@ -131,10 +140,10 @@ static CBaseLayer* buildResNetBlock( CDnn& dnn, IMathEngine& e, CBaseLayer& sour
 //         CCtcDecodingLayer and returns every sequence's best labels. Input: [T, B, 1, 1, 1, 1, In].
 static CBaseLayer* buildRecognizerTail( CDnn& dnn, IMathEngine& e, CBaseLayer& source, int classes )
 {
-	CPtr<CLstmLayer> fwd = add( dnn, new CLstmLayer( e ), "fwd", source );
-	fwd->SetHiddenSize( 32 );
-	CPtr<CLstmLayer> rev = add( dnn, new CLstmLayer( e ), "rev", source );
-	rev->SetHiddenSize( 32 );
+	CPtr<CLstmLayer> fwd = add( dnn, newLstm( e ), "fwd", source );
+	fwd->SetHiddenSize( tailHidden );
+	CPtr<CLstmLayer> rev = add( dnn, newLstm( e ), "rev", source );
+	rev->SetHiddenSize( tailHidden );
 	rev->SetReverseSequence( true );
 	CPtr<CConcatChannelsLayer> concat = new CConcatChannelsLayer( e );
 	concat->SetName( "concat" );

@@ -131,3 +131,72 @@ def test_resnet18_through_cdnn_at_benchmark_size(capsys):
     assert_close(y[:2], small, "batch 64 vs batch 2")
     want = dnn_run(nhtest.cpu_engine(), 5, (1, 1, 1, 224, 224, 1, 3), x[:, :1], 1000).reshape(1, 1000)
     assert_close(y[:1], want, "first image vs the CPU engine")
+
+
+# ---------------------------------------------------------------------------------------------------------
+# CHipLstmLayer (neoml_amd/engine/HipLstmLayer.h): CLstmLayer whose RunOnce reaches IMathEngine::Lstm on a non-CPU
+# engine. Same weights (same CRandom seed), so it must reproduce CLstmLayer on the CPU engine.
+
+class fused_lstm:
+    def __init__(self, hidden=32):
+        self.hidden = hidden
+
+    def __enter__(self):
+        lib().dnn_set_fused_lstm(1)
+        lib().dnn_set_tail_hidden(self.hidden)
+
+    def __exit__(self, *exc):
+        lib().dnn_set_fused_lstm(0)
+        lib().dnn_set_tail_hidden(32)
+
+
+def test_hip_lstm_layer_is_clstmlayer_on_the_cpu_engine():
+    # on the CPU engine the subclass defers to its base class: identical numbers
+    for name in ("lstm", "recognizer_tail"):
+        kind, dims, param = CASES[name]
+        x = make_input(name)
+        want = dnn_run(nhtest.cpu_engine(), kind, dims, x, param)
+        with fused_lstm():
+            got = dnn_run(nhtest.cpu_engine(), kind, dims, x, param)
+        assert np.array_equal(got, want), name
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["lstm", "recognizer_tail"])
+def test_hip_lstm_layer_matches_clstmlayer(name):
+    kind, dims, param = CASES[name]
+    x = make_input(name)
+    want = dnn_run(nhtest.cpu_engine(), kind, dims, x, param)
+    with fused_lstm():
+        got = dnn_run(nhtest.hip_engine(), kind, dims, x, param)
+    assert_close(got, want, "CHipLstmLayer on CHipMathEngine vs CLstmLayer on CCpuMathEngine (%s)" % name)
+    if name == "recognizer_tail":
+        with fused_lstm():
+            labels = dnn_run_ctc(nhtest.hip_engine(), dims, x, param)
+        assert labels == dnn_run_ctc(nhtest.cpu_engine(), dims, x, param)
+
+
+@pytest.mark.gpu
+def test_recognizer_tail_at_benchmark_size_fused_vs_composite(capsys):
+    """The BiLSTM tail of the line recogniser at its full size (128 steps, 64 lines, 256 -> 2 x 256 hidden, FC to 101)
+    as a CDnn: CLstmLayer (composite per-step graph on this engine) against CHipLstmLayer (IMathEngine::Lstm).
+    Same weights, so the outputs must agree; the time per CDnn::RunOnce of both is printed."""
+    dims = (128, 64, 1, 1, 1, 1, 256)
+    g = np.random.default_rng(0xC0FFEE + 105)
+    x = g.uniform(-1, 1, dims).astype(np.float32)
+    lib().dnn_last_pass_ms.restype = ctypes.c_double
+    lib().dnn_set_timed_passes(5)
+    try:
+        lib().dnn_set_tail_hidden(256)
+        composite = dnn_run(nhtest.hip_engine(), 4, dims, x, 100)
+        composite_ms = lib().dnn_last_pass_ms()
+        with fused_lstm(256):
+            fused = dnn_run(nhtest.hip_engine(), 4, dims, x, 100)
+            fused_ms = lib().dnn_last_pass_ms()
+    finally:
+        lib().dnn_set_timed_passes(0)
+        lib().dnn_set_tail_hidden(32)
+    with capsys.disabled():
+        print("\nBiLSTM(256) tail, 128 steps x 64 lines, CDnn::RunOnce on CHipMathEngine: CLstmLayer %.2f ms, "
+              "CHipLstmLayer %.2f ms" % (composite_ms, fused_ms))
+    assert_close(fused, composite, "CHipLstmLayer vs CLstmLayer on the same engine")
