@@ -637,6 +637,152 @@ static bool fitsBuffer( long long rows, long long pitch, long long width )
 	return rows <= 0 || ( ( rows - 1 ) * pitch + width ) * 4 < static_cast<long long>( BufferBytes );
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Short reductions over many rows: C[M x N] = A[M x K] * W[N x K]^T (+ bias), K = 8 * KC <= 192, all three dense.
+// These are the pointwise convolutions of a depthwise-separable network at high resolution (16 -> 96, 24 -> 144,
+// 144 -> 24 channels over 10^5..10^6 pixels): bound by HBM, and the tiled kernel above, built around a long K loop,
+// spends its time in prologues and epilogues and re-reads A once per 64 output columns.
+// Here a wavefront owns 32 whole rows: it fetches them straight into MFMA operand registers (every lane its row's
+// K values, 16 bytes per load: together the loads of a wavefront cover one contiguous piece of A), keeps them for
+// all output columns, and walks the columns in blocks of 32 with W read from LDS, where the workgroup put it once.
+// No barrier after that; wavefronts take further row blocks grid-stride.
+// MFMA e of the c-th group of 8 k reduces over { 8c + e, 8c + 4 + e } on both operands.
+template<int KC>
+__global__ __launch_bounds__( Threads )
+void shortReductionKernel( const float* A, const float* W, const float* bias, float* C, int M, int N, int rowBlocks )
+{
+	constexpr int K = KC * 8;
+	constexpr int Pitch = K + 4;
+	// [32 * nBlocks][Pitch], rows beyond N are zero; then one [32][36] output patch per wavefront
+	extern __shared__ __attribute__( ( aligned( 16 ) ) ) float wLds[];
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = tid >> 6;
+	const int l32 = lane & 31;
+	const int half = lane >> 5;
+	const int nBlocks = ( N + 31 ) / 32;
+	for( int idx = tid; idx < nBlocks * 32 * ( K / 4 ); idx += Threads ) {
+		const int n = idx / ( K / 4 );
+		const int k4 = idx - n * ( K / 4 );
+		const float4 v = n < N ? *reinterpret_cast<const float4*>( W + static_cast<long long>( n ) * K + k4 * 4 )
+			: make_float4( 0.f, 0.f, 0.f, 0.f );
+		*reinterpret_cast<float4*>( wLds + n * Pitch + k4 * 4 ) = v;
+	}
+	__syncthreads();
+
+	constexpr int PatchPitch = 36;
+	float* patch = wLds + nBlocks * 32 * Pitch + wave * 32 * PatchPitch;
+	const bool rowsAligned = N % 4 == 0 && ( reinterpret_cast<uintptr_t>( C ) & 15 ) == 0;
+	const __amdgpu_buffer_rsrc_t bufA = makeBuffer( A );
+	// The rows of the next block are requested before the current block is multiplied and stored: a wavefront's
+	// loads and stores complete in issue order, so loads issued after the stores would wait for the stores' round trip.
+	auto requestRows = [&]( int block, float4 ( &rows )[KC] ) {
+		const int m = block * 32 + l32;
+		const unsigned rowOffset = ( block < rowBlocks && m < M ) ? static_cast<unsigned>( m ) * ( K * 4u ) + half * 16u : OutOfRange;
+#pragma unroll
+		for( int c = 0; c < KC; ++c ) {
+			rows[c] = bufferLoad4( bufA, rowOffset + c * 32u ); // an out-of-range row reads zeros
+		}
+	};
+	float4 ahead[KC];
+	requestRows( blockIdx.x * 4 + wave, ahead );
+	for( int block = blockIdx.x * 4 + wave; block < rowBlocks; block += gridDim.x * 4 ) {
+		float4 a[KC];
+#pragma unroll
+		for( int c = 0; c < KC; ++c ) {
+			a[c] = ahead[c];
+		}
+		requestRows( block + gridDim.x * 4, ahead );
+		for( int nb = 0; nb < nBlocks; ++nb ) {
+			f32x16 acc;
+#pragma unroll
+			for( int r = 0; r < 16; ++r ) {
+				acc[r] = 0.f;
+			}
+			const float* wRow = wLds + ( nb * 32 + l32 ) * Pitch + half * 4;
+#pragma unroll
+			for( int c = 0; c < KC; ++c ) {
+				const float4 w = *reinterpret_cast<const float4*>( wRow + c * 8 );
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[c].x, w.x, acc, 0, 0, 0 );
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[c].y, w.y, acc, 0, 0, 0 );
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[c].z, w.z, acc, 0, 0, 0 );
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[c].w, w.w, acc, 0, 0, 0 );
+			}
+			// The block goes out through a wavefront-private patch of LDS, turned so that a lane holds four
+			// neighbouring columns of one row: 4 stores of 16 bytes per lane, each covering whole 128-byte runs of
+			// 8 rows, instead of 16 stores of 4 bytes. (Register r of lane ( l32, half ) is row
+			// ( r / 4 ) * 8 + half * 4 + r % 4, column l32 of the block.)
+			const int n = nb * 32 + l32;
+			const float b = ( bias != nullptr && n < N ) ? bias[n] : 0.f;
+#pragma unroll
+			for( int r = 0; r < 16; ++r ) {
+				patch[( ( r >> 2 ) * 8 + half * 4 + ( r & 3 ) ) * PatchPitch + l32] = acc[r] + b;
+			}
+			// ( same wavefront: the LDS unit executes its reads after its writes, no barrier needed )
+			const int col4 = ( lane & 7 ) * 4;
+			const int n4 = nb * 32 + col4;
+#pragma unroll
+			for( int q = 0; q < 4; ++q ) {
+				const int row = q * 8 + ( lane >> 3 );
+				const float4 v = *reinterpret_cast<const float4*>( patch + row * PatchPitch + col4 );
+				const long long mOut = static_cast<long long>( block ) * 32 + row;
+				if( mOut < M ) {
+					float* out = C + mOut * N + n4;
+					if( rowsAligned && n4 + 3 < N ) {
+						*reinterpret_cast<float4*>( out ) = v;
+					} else {
+						if( n4 < N ) out[0] = v.x;
+						if( n4 + 1 < N ) out[1] = v.y;
+						if( n4 + 2 < N ) out[2] = v.z;
+						if( n4 + 3 < N ) out[3] = v.w;
+					}
+				}
+			}
+		}
+	}
+}
+
+template<int KC>
+static void launchShortReduction( hipStream_t stream, const float* a, const float* w, const float* bias, float* c, int M, int N )
+{
+	const int rowBlocks = ceilDiv( M, 32 );
+	const int groups = ceilDiv( rowBlocks, 4 );
+	const size_t lds = ( static_cast<size_t>( ceilDiv( N, 32 ) ) * 32 * ( KC * 8 + 4 ) + 4 * 32 * 36 ) * sizeof( float );
+	hipLaunchKernelGGL( shortReductionKernel<KC>, dim3( groups < 2048 ? groups : 2048 ), dim3( Threads ), lds, stream,
+		a, w, bias, c, M, N, rowBlocks );
+}
+
+// true (and launched) when the product has the shape this kernel is for
+static bool tryShortReduction( hipStream_t stream, const float* a, int lda, const float* w, int ldb, float* c, int ldc,
+	int M, int N, int K, const float* bias, int* rc )
+{
+	if( lda != K || ldb != K || ldc != N || M < 16384 || K % 8 != 0 || K > 192 || N > 192
+		|| !isAligned16( a ) || !isAligned16( w ) || !fitsBuffer( M, K, K )
+		|| ( static_cast<size_t>( ceilDiv( N, 32 ) ) * 32 * ( K + 4 ) + 4 * 32 * 36 ) * sizeof( float ) > 64 * 1024 )
+	{
+		return false;
+	}
+	switch( K / 8 ) {
+		case 2: launchShortReduction<2>( stream, a, w, bias, c, M, N ); break;
+		case 3: launchShortReduction<3>( stream, a, w, bias, c, M, N ); break;
+		case 4: launchShortReduction<4>( stream, a, w, bias, c, M, N ); break;
+		case 6: launchShortReduction<6>( stream, a, w, bias, c, M, N ); break;
+		case 8: launchShortReduction<8>( stream, a, w, bias, c, M, N ); break;
+		case 12: launchShortReduction<12>( stream, a, w, bias, c, M, N ); break;
+		case 18: launchShortReduction<18>( stream, a, w, bias, c, M, N ); break;
+		case 24: launchShortReduction<24>( stream, a, w, bias, c, M, N ); break;
+		default: return false;
+	}
+	const hipError_t err = hipGetLastError();
+	if( err != hipSuccess ) {
+		setLastError( "short-reduction product: launch failed: %s", hipGetErrorString( err ) );
+		*rc = NH_ERR_HIP;
+	} else {
+		*rc = NH_OK;
+	}
+	return true;
+}
+
 // C = A * B^T (+ bias) with row strides; also the inner product of the convolution with a 1x1 filter.
 int matMulNT( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
 	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC,
@@ -651,6 +797,10 @@ int matMulNT( hipStream_t stream, const float* a, int lda, const float* b, int l
 	args.Lda = lda; args.Ldb = ldb; args.Ldc = ldc;
 	args.BatchStrideA = strideA; args.BatchStrideB = strideB; args.BatchStrideC = strideC;
 	args.Accumulate = accumulate ? 1 : 0;
+	int rc = NH_OK;
+	if( batch == 1 && !accumulate && tryShortReduction( stream, a, lda, b, ldb, c, ldc, M, N, K, bias, &rc ) ) {
+		return rc;
+	}
 	const bool vec = isAligned16( a ) && isAligned16( b ) && K % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0
 		&& strideA % 4 == 0 && strideB % 4 == 0 && fitsBuffer( M, lda, K ) && fitsBuffer( N, ldb, K );
 	return launchMatMul<AM_RowsK, BM_RowsK>( stream, args, batch, vec );

@@ -97,8 +97,13 @@ def main():
     conv("cfg2 s4", 64, 7, 7, 512, 512, 3, 1, 1)
     conv("cfg2 s2 down", 64, 56, 56, 64, 128, 3, 1, 2)
     conv("cfg2 s2 short", 64, 56, 56, 64, 128, 1, 0, 2)
+    conv("cfg3 project", 128, 112, 112, 32, 16, 1, 0, 1)
+    conv("cfg3 expand", 128, 112, 112, 16, 96, 1, 0, 1)
+    conv("cfg3 project", 128, 56, 56, 96, 24, 1, 0, 1)
     conv("cfg3 expand", 128, 56, 56, 24, 144, 1, 0, 1)
     conv("cfg3 project", 128, 56, 56, 144, 24, 1, 0, 1)
+    conv("cfg3 expand", 128, 28, 28, 32, 192, 1, 0, 1)
+    conv("cfg3 project", 128, 28, 28, 192, 32, 1, 0, 1)
     conv("cfg3 expand", 128, 14, 14, 64, 384, 1, 0, 1)
     conv("cfg3 project", 128, 14, 14, 384, 64, 1, 0, 1)
     conv("cfg5 conv1", 64, 32, 512, 1, 64, 3, 1, 1)

@@ -230,6 +230,12 @@ GPU_CONV_CASES = CONV_CASES + [
     (1, 6, 5, 7, 9, 2, 4, 0, 3, 1, 1, 1, 1),        # run longer than the image row is wide
     (2, 11, 9, 5, 70, 1, 3, 0, 1, 1, 1, 1, 1),      # N tail
     (4, 32, 64, 1, 64, 3, 3, 1, 1, 1, 1, 1, 1),     # grey line image, split over many tiles
+    # pointwise convolutions over many pixels with a short reduction: the row-resident kernel
+    (4, 64, 64, 24, 144, 1, 1, 0, 0, 1, 1, 1, 1),   # expand
+    (4, 64, 64, 144, 24, 1, 1, 0, 0, 1, 1, 1, 1),   # project, N < 32
+    (2, 96, 96, 16, 96, 1, 1, 0, 0, 1, 1, 1, 1),
+    (1, 131, 127, 32, 20, 1, 1, 0, 0, 1, 1, 1, 1),  # pixel count not a multiple of 32
+    (1, 128, 130, 192, 40, 1, 1, 0, 0, 1, 1, 1, 1), # longest reduction it takes, N tail
 ]
 
 
