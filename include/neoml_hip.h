@@ -242,6 +242,39 @@ NH_API int nhInitBlobChannelwiseConvolution(nhConvDesc* desc_host);             
 NH_API int nhBlobChannelwiseConvolution(nhStream s, const nhConvDesc* desc_host, const float* source,
 	const float* filter, const float* freeTerm, float* result);                                      /* NME.h:770 */
 
+/* The fused blocks the graph optimizer emits for depthwise-separable networks (NME.h:1066-1072, layer classes
+ * CMobileNetV2BlockLayer / CChannelwiseWith1x1Layer). Activations are TActivationFunction values reduced to what
+ * the blocks support (src/CPU/Rowwise/CpuRowwiseCommon.h:79-86): ReLU with an optional upper threshold (param > 0),
+ * h-swish, anything else = none. The depthwise stage is 3x3, padding 1, stride 1 or 2 (Ho = (H + stride - 1) / stride).
+ * Filters: expand [E][Cin], channelwise [3][3][E], down / conv [Cout][E]; free terms may be null.
+ * residual != 0 adds the block's input to its output (needs Cin == Cout, stride 1); input == output is allowed then.
+ * workspace: the expanded activations between the stages, nh...WorkspaceSize bytes of device memory. */
+#define NH_ACT_NONE 0
+#define NH_ACT_RELU 1
+#define NH_ACT_HSWISH 2
+typedef struct nhSeparableBlockDesc {
+	int batch, height, width;
+	int inputChannels;     /* MobileNetV2Block only */
+	int expandedChannels;  /* channels of the depthwise stage (= input channels of ChannelwiseWith1x1) */
+	int outputChannels;
+	int stride, residual;
+	int expandActivation; float expandParam;           /* MobileNetV2Block only */
+	int channelwiseActivation; float channelwiseParam;
+} nhSeparableBlockDesc;
+NH_API int nhMobileNetV2BlockWorkspaceSize(const nhSeparableBlockDesc* desc_host, size_t* bytes);
+NH_API int nhMobileNetV2Block(nhStream s, const nhSeparableBlockDesc* desc_host, const float* input,
+	const float* expandFilter, const float* expandFreeTerm, const float* channelwiseFilter,
+	const float* channelwiseFreeTerm, const float* downFilter, const float* downFreeTerm, float* output,
+	void* workspace, size_t workspaceSize);                                                          /* NME.h:1069 */
+NH_API int nhChannelwiseWith1x1WorkspaceSize(const nhSeparableBlockDesc* desc_host, size_t* bytes);
+NH_API int nhChannelwiseWith1x1(nhStream s, const nhSeparableBlockDesc* desc_host, const float* input,
+	const float* channelwiseFilter, const float* channelwiseFreeTerm, const float* convFilter,
+	const float* convFreeTerm, float* output, void* workspace, size_t workspaceSize);                /* NME.h:1066 */
+/* A convolution / matrix product with the activation behind it in the same launch, as the rowwise operation chains
+ * pair them (NME.h:1080-1087): result = act( source * filter^T + freeTerm ), 1x1 filter [Cout][Cin], rows = pixels */
+NH_API int nhPointwiseConvolutionWithActivation(nhStream s, const float* source, int rows, int channels,
+	const float* filter, const float* freeTerm, int filterCount, int activation, float param, float* result);
+
 /* CCommon2DPoolingDesc (src/MathEngineDnnPoolings.h:24-60): no padding; Ho = (H - fh) / sh + 1 */
 typedef struct nhPoolingDesc {
 	int batch, height, width, channels;

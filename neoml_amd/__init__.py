@@ -6,5 +6,5 @@ device memory for those comes from torch tensors.
 """
 from .capi import (  # noqa: F401
     NeoMLHipError, load, check, last_error, declared_functions,
-    ConvDesc, PoolingDesc, BlobDesc, LIB_PATH, HEADER_PATH,
+    ConvDesc, PoolingDesc, BlobDesc, SeparableBlockDesc, LIB_PATH, HEADER_PATH,
 )

@@ -36,6 +36,14 @@ class PoolingDesc(ctypes.Structure):
         "resultHeight", "resultWidth")]
 
 
+class SeparableBlockDesc(ctypes.Structure):
+    """nhSeparableBlockDesc"""
+    _fields_ = [(n, ctypes.c_int) for n in (
+        "batch", "height", "width", "inputChannels", "expandedChannels", "outputChannels", "stride", "residual")] + [
+        ("expandActivation", ctypes.c_int), ("expandParam", ctypes.c_float),
+        ("channelwiseActivation", ctypes.c_int), ("channelwiseParam", ctypes.c_float)]
+
+
 class BlobDesc(ctypes.Structure):
     """nhBlobDesc: BatchLength, BatchWidth, ListSize, Height, Width, Depth, Channels"""
     _fields_ = [("dims", ctypes.c_int * 7)]

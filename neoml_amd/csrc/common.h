@@ -65,6 +65,27 @@ __device__ __forceinline__ int xcdSwizzle( int bid, int total )
 	return xcd * per + ( xcd < rem ? xcd : rem ) + idx;
 }
 
+// Activation applied by a producing kernel before it stores: the fused blocks of the MobileNet family put ReLU
+// (optionally clipped at Param > 0) or h-swish behind a convolution; any other type stores the value as it is
+// (src/CPU/Rowwise/CpuRowwiseCommon.h:79-86).
+struct CFusedActivation {
+	int Type;    // NH_ACT_*
+	float Param; // upper threshold of NH_ACT_RELU when above zero
+};
+
+__device__ __forceinline__ float applyActivation( float v, const CFusedActivation& a )
+{
+	if( a.Type == NH_ACT_RELU ) {
+		v = v > 0.f ? v : 0.f; // NaN becomes 0, as in VectorReLU
+		if( a.Param > 0.f ) {
+			v = v < a.Param ? v : a.Param;
+		}
+	} else if( a.Type == NH_ACT_HSWISH ) {
+		v = v <= -3.f ? 0.f : ( v >= 3.f ? v : v * ( v + 3.f ) * ( 1.f / 6.f ) );
+	}
+	return v;
+}
+
 // Operands are read with raw buffer loads: a 32-bit byte offset from a base held in scalar registers, and a range
 // check done by the memory unit. An offset at or above BufferBytes reads as zero, which serves as the zero padding
 // of the convolution and as the mask of tile rows / columns / k beyond the matrix, without a branch or a select.

@@ -11,6 +11,9 @@ namespace nh {
 int matMulNT( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
 	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC,
 	const float* bias, bool accumulate );
+int matMulNTFused( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
+	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC,
+	const float* bias, bool accumulate, const CFusedActivation& act, const float* residual );
 
 // ---------------------------------------------------------------------------------------------------------
 // Channelwise convolution: out[n,ho,wo,c] = bias[c] + sum_{kh,kw} in[n, ho*s-p+kh, wo*s-p+kw, c] * filt[kh,kw,c]
@@ -27,6 +30,10 @@ template<> struct CChanVec<4> {
 	{
 		return make_float4( fmaf( a.x, b.x, c.x ), fmaf( a.y, b.y, c.y ), fmaf( a.z, b.z, c.z ), fmaf( a.w, b.w, c.w ) );
 	}
+	static __device__ __forceinline__ float4 activate( float4 v, const CFusedActivation& a )
+	{
+		return make_float4( applyActivation( v.x, a ), applyActivation( v.y, a ), applyActivation( v.z, a ), applyActivation( v.w, a ) );
+	}
 };
 template<> struct CChanVec<1> {
 	typedef float Type;
@@ -34,12 +41,13 @@ template<> struct CChanVec<1> {
 	static __device__ __forceinline__ void store( float* p, float v ) { *p = v; }
 	static __device__ __forceinline__ float zero() { return 0.f; }
 	static __device__ __forceinline__ float fma( float a, float b, float c ) { return fmaf( a, b, c ); }
+	static __device__ __forceinline__ float activate( float v, const CFusedActivation& a ) { return applyActivation( v, a ); }
 };
 
 template<int VECW, int WPT>
 __global__ __launch_bounds__( 256 )
 void channelwiseConvKernel( const nhConvDesc d, const float* source, const float* filter, const float* freeTerm,
-	float* result, int wGroups, long long totalItems )
+	float* result, int wGroups, long long totalItems, const CFusedActivation act )
 {
 	typedef CChanVec<VECW> V;
 	typedef typename V::Type T;
@@ -82,7 +90,7 @@ void channelwiseConvKernel( const nhConvDesc d, const float* source, const float
 #pragma unroll
 		for( int j = 0; j < WPT; ++j ) {
 			if( wo0 + j < d.resultWidth ) {
-				V::store( out + static_cast<long long>( j ) * d.channels, acc[j] );
+				V::store( out + static_cast<long long>( j ) * d.channels, V::activate( acc[j], act ) );
 			}
 		}
 	}
@@ -97,7 +105,7 @@ void channelwiseConvKernel( const nhConvDesc d, const float* source, const float
 template<int STRIDE, int WPT>
 __global__ __launch_bounds__( 256 )
 void channelwiseConv3x3Kernel( const nhConvDesc d, const float* source, const float* filter, const float* freeTerm,
-	float* result, int wGroups, int rowChunks, int rowsPerItem, int totalItems )
+	float* result, int wGroups, int rowChunks, int rowsPerItem, int totalItems, const CFusedActivation act )
 {
 	constexpr int NC = ( WPT - 1 ) * STRIDE + 3;
 	constexpr int Keep = 3 - STRIDE; // input rows shared by two consecutive output rows
@@ -163,7 +171,7 @@ void channelwiseConv3x3Kernel( const nhConvDesc d, const float* source, const fl
 				}
 			}
 			if( wo0 + j < d.resultWidth ) {
-				*reinterpret_cast<float4*>( out + j * d.channels ) = acc;
+				*reinterpret_cast<float4*>( out + j * d.channels ) = CChanVec<4>::activate( acc, act );
 			}
 		}
 #pragma unroll
@@ -1107,7 +1115,7 @@ static int poolingImpl( nhStream s, const nhPoolingDesc* d, const float* source,
 
 template<int STRIDE, int WPT>
 static int channelwise3x3Impl( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
-	const float* freeTerm, float* result )
+	const float* freeTerm, float* result, const CFusedActivation& act )
 {
 	const int wGroups = ceilDiv( d->resultWidth, WPT );
 	const long long perRow = static_cast<long long>( d->batch ) * wGroups * ( d->channels / 4 );
@@ -1115,7 +1123,7 @@ static int channelwise3x3Impl( nhStream s, const nhConvDesc* d, const float* sou
 	chooseRowChunks( perRow, d->resultHeight, 4, 3072, &rowChunks, &rowsPerItem );
 	const long long items = perRow * rowChunks;
 	hipLaunchKernelGGL( ( channelwiseConv3x3Kernel<STRIDE, WPT> ), dim3( static_cast<unsigned>( ( items + 255 ) / 256 ) ), dim3( 256 ), 0,
-		toStream( s ), *d, source, filter, freeTerm, result, wGroups, rowChunks, rowsPerItem, static_cast<int>( items ) );
+		toStream( s ), *d, source, filter, freeTerm, result, wGroups, rowChunks, rowsPerItem, static_cast<int>( items ), act );
 	NH_LAUNCH_CHECK();
 	return NH_OK;
 }
@@ -1139,8 +1147,18 @@ int nhInitBlobChannelwiseConvolution( nhConvDesc* d )
 	return NH_OK;
 }
 
+static int channelwiseConvolution( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
+	const float* freeTerm, float* result, const CFusedActivation& act );
+
 int nhBlobChannelwiseConvolution( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
 	const float* freeTerm, float* result )
+{
+	const CFusedActivation none = { NH_ACT_NONE, 0.f };
+	return channelwiseConvolution( s, d, source, filter, freeTerm, result, none );
+}
+
+static int channelwiseConvolution( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
+	const float* freeTerm, float* result, const CFusedActivation& act )
 {
 	NH_REQUIRE( d != nullptr && source != nullptr && filter != nullptr && result != nullptr );
 	nhConvDesc check = *d;
@@ -1160,8 +1178,8 @@ int nhBlobChannelwiseConvolution( nhStream s, const nhConvDesc* d, const float* 
 		&& sourceBytes < 0x80000000LL
 		&& static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * d->channels < 0x7fffffffLL )
 	{
-		return d->strideHeight == 1 ? channelwise3x3Impl<1, 4>( s, d, source, filter, freeTerm, result )
-			: channelwise3x3Impl<2, 2>( s, d, source, filter, freeTerm, result );
+		return d->strideHeight == 1 ? channelwise3x3Impl<1, 4>( s, d, source, filter, freeTerm, result, act )
+			: channelwise3x3Impl<2, 2>( s, d, source, filter, freeTerm, result, act );
 	}
 	constexpr int WPT = 4;
 	const int wGroups = ceilDiv( d->resultWidth, WPT );
@@ -1170,10 +1188,10 @@ int nhBlobChannelwiseConvolution( nhStream s, const nhConvDesc* d, const float* 
 	blocks = blocks > 1048576 ? 1048576 : blocks;
 	if( vec ) {
 		hipLaunchKernelGGL( ( channelwiseConvKernel<4, WPT> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
-			*d, source, filter, freeTerm, result, wGroups, items );
+			*d, source, filter, freeTerm, result, wGroups, items, act );
 	} else {
 		hipLaunchKernelGGL( ( channelwiseConvKernel<1, WPT> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
-			*d, source, filter, freeTerm, result, wGroups, items );
+			*d, source, filter, freeTerm, result, wGroups, items, act );
 	}
 	NH_LAUNCH_CHECK();
 	return NH_OK;
@@ -1359,6 +1377,126 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 		NH_LAUNCH_CHECK();
 	}
 	return NH_OK;
+}
+
+// ---- the fused blocks of depthwise-separable networks -----------------------------------------------------------
+// Every stage is one launch with its activation (and the residual sum) in the epilogue of the kernel that produces
+// the values: expand 1x1 (+act) -> depthwise 3x3 (+act) -> down 1x1 (+input). Unfused, the same block costs two
+// activation passes and one sum pass more over the six-fold expanded tensor.
+
+static int checkSeparableDesc( const nhSeparableBlockDesc* d, bool withExpand, nhConvDesc* dw )
+{
+	NH_REQUIRE( d != nullptr );
+	NH_REQUIRE( d->batch >= 0 && d->height > 0 && d->width > 0 && d->expandedChannels > 0 && d->outputChannels > 0 );
+	NH_REQUIRE( !withExpand || d->inputChannels > 0 );
+	NH_REQUIRE( d->stride == 1 || d->stride == 2 );
+	const int blockInput = withExpand ? d->inputChannels : d->expandedChannels;
+	NH_REQUIRE( d->residual == 0 || ( d->stride == 1 && blockInput == d->outputChannels ) );
+	*dw = nhConvDesc();
+	dw->batch = d->batch; dw->height = d->height; dw->width = d->width; dw->channels = d->expandedChannels;
+	dw->filterCount = d->expandedChannels; dw->filterHeight = 3; dw->filterWidth = 3;
+	dw->paddingHeight = 1; dw->paddingWidth = 1; dw->strideHeight = d->stride; dw->strideWidth = d->stride;
+	return nhInitBlobChannelwiseConvolution( dw );
+}
+
+int nhMobileNetV2BlockWorkspaceSize( const nhSeparableBlockDesc* d, size_t* bytes )
+{
+	nhConvDesc dw;
+	const int rc = checkSeparableDesc( d, true, &dw );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( bytes != nullptr );
+	const size_t expanded = static_cast<size_t>( d->batch ) * d->height * d->width * d->expandedChannels;
+	const size_t reduced = static_cast<size_t>( d->batch ) * dw.resultHeight * dw.resultWidth * d->expandedChannels;
+	*bytes = ( ( expanded + 63 ) / 64 * 64 + reduced ) * sizeof( float );
+	return NH_OK;
+}
+
+int nhMobileNetV2Block( nhStream s, const nhSeparableBlockDesc* d, const float* input, const float* expandFilter,
+	const float* expandFreeTerm, const float* channelwiseFilter, const float* channelwiseFreeTerm,
+	const float* downFilter, const float* downFreeTerm, float* output, void* workspace, size_t workspaceSize )
+{
+	nhConvDesc dw;
+	int rc = checkSeparableDesc( d, true, &dw );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	size_t need = 0;
+	rc = nhMobileNetV2BlockWorkspaceSize( d, &need );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( input != nullptr && expandFilter != nullptr && channelwiseFilter != nullptr && downFilter != nullptr && output != nullptr );
+	NH_REQUIRE( workspace != nullptr && workspaceSize >= need && isAligned16( workspace ) );
+	if( d->batch == 0 ) {
+		return NH_OK;
+	}
+	const long long pixelsIn = static_cast<long long>( d->batch ) * d->height * d->width;
+	const long long pixelsOut = static_cast<long long>( d->batch ) * dw.resultHeight * dw.resultWidth;
+	NH_REQUIRE( pixelsIn <= 0x7fffffffLL && pixelsIn * d->expandedChannels <= 0x7fffffffLL );
+	float* expanded = static_cast<float*>( workspace );
+	float* reduced = expanded + ( static_cast<size_t>( pixelsIn ) * d->expandedChannels + 63 ) / 64 * 64;
+	const CFusedActivation expandAct = { d->expandActivation, d->expandParam };
+	const CFusedActivation channelwiseAct = { d->channelwiseActivation, d->channelwiseParam };
+	const CFusedActivation none = { NH_ACT_NONE, 0.f };
+	rc = matMulNTFused( toStream( s ), input, d->inputChannels, expandFilter, d->inputChannels, expanded, d->expandedChannels,
+		static_cast<int>( pixelsIn ), d->expandedChannels, d->inputChannels, 1, 0, 0, 0, expandFreeTerm, false, expandAct, nullptr );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	rc = channelwiseConvolution( s, &dw, expanded, channelwiseFilter, channelwiseFreeTerm, reduced, channelwiseAct );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	return matMulNTFused( toStream( s ), reduced, d->expandedChannels, downFilter, d->expandedChannels, output, d->outputChannels,
+		static_cast<int>( pixelsOut ), d->outputChannels, d->expandedChannels, 1, 0, 0, 0, downFreeTerm, false, none,
+		d->residual != 0 ? input : nullptr );
+}
+
+int nhChannelwiseWith1x1WorkspaceSize( const nhSeparableBlockDesc* d, size_t* bytes )
+{
+	nhConvDesc dw;
+	const int rc = checkSeparableDesc( d, false, &dw );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( bytes != nullptr );
+	*bytes = static_cast<size_t>( d->batch ) * dw.resultHeight * dw.resultWidth * d->expandedChannels * sizeof( float );
+	return NH_OK;
+}
+
+int nhChannelwiseWith1x1( nhStream s, const nhSeparableBlockDesc* d, const float* input, const float* channelwiseFilter,
+	const float* channelwiseFreeTerm, const float* convFilter, const float* convFreeTerm, float* output,
+	void* workspace, size_t workspaceSize )
+{
+	nhConvDesc dw;
+	int rc = checkSeparableDesc( d, false, &dw );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	size_t need = 0;
+	rc = nhChannelwiseWith1x1WorkspaceSize( d, &need );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( input != nullptr && channelwiseFilter != nullptr && convFilter != nullptr && output != nullptr );
+	NH_REQUIRE( workspace != nullptr && workspaceSize >= need && isAligned16( workspace ) );
+	if( d->batch == 0 ) {
+		return NH_OK;
+	}
+	const long long pixelsOut = static_cast<long long>( d->batch ) * dw.resultHeight * dw.resultWidth;
+	NH_REQUIRE( pixelsOut <= 0x7fffffffLL );
+	float* reduced = static_cast<float*>( workspace );
+	const CFusedActivation channelwiseAct = { d->channelwiseActivation, d->channelwiseParam };
+	const CFusedActivation none = { NH_ACT_NONE, 0.f };
+	rc = channelwiseConvolution( s, &dw, input, channelwiseFilter, channelwiseFreeTerm, reduced, channelwiseAct );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	return matMulNTFused( toStream( s ), reduced, d->expandedChannels, convFilter, d->expandedChannels, output, d->outputChannels,
+		static_cast<int>( pixelsOut ), d->outputChannels, d->expandedChannels, 1, 0, 0, 0, convFreeTerm, false, none,
+		d->residual != 0 ? input : nullptr );
 }
 
 } // extern "C"

@@ -57,6 +57,9 @@ struct CMatMulArgs {
 	// convolution geometry (AM_Conv only): A is the image, M = batch * Ho * Wo
 	int H, W, Cin, Ho, Wo, Fh, Fw, PadH, PadW, StrideH, StrideW, DilH, DilW;
 	int RowK, RowPitch; // AM_ConvRows: Fw * Cin and its round-up to a multiple of 4; K = Fh * RowPitch
+	// epilogue of the fused blocks: C = act( A * B + bias ) + Residual; Residual has C's layout, may be C itself
+	CFusedActivation Act;
+	const float* Residual;
 };
 
 constexpr int Threads = 256;
@@ -530,6 +533,10 @@ void matMulKernel( const CMatMulArgs args )
 						if( args.Accumulate ) {
 							v += *p;
 						}
+						v = applyActivation( v, args.Act );
+						if( args.Residual != nullptr ) {
+							v += args.Residual[batch * args.BatchStrideC + static_cast<long long>( m ) * args.Ldc + n];
+						}
 						*p = v;
 					}
 				}
@@ -581,7 +588,8 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 	const int totalSteps = ceilDiv( args.K, NH_KSTEP );
 	int splits = 1;
 	const long long blocks = tiles * batch;
-	if( blocks < 1024 && totalSteps >= 32 ) {
+	const bool plainEpilogue = args.Act.Type == NH_ACT_NONE && args.Residual == nullptr; // K slices cannot apply one
+	if( blocks < 1024 && totalSteps >= 32 && plainEpilogue ) {
 		double best = 0;
 		for( int s = 1; s <= 8 && s <= totalSteps / 8; ++s ) {
 			const double rounds = static_cast<double>( blocks * s ) / 1280.0;
@@ -649,7 +657,8 @@ static bool fitsBuffer( long long rows, long long pitch, long long width )
 // MFMA e of the c-th group of 8 k reduces over { 8c + e, 8c + 4 + e } on both operands.
 template<int KC>
 __global__ __launch_bounds__( Threads )
-void shortReductionKernel( const float* A, const float* W, const float* bias, float* C, int M, int N, int rowBlocks )
+void shortReductionKernel( const float* A, const float* W, const float* bias, float* C, int M, int N, int rowBlocks,
+	const CFusedActivation act, const float* residual )
 {
 	constexpr int K = KC * 8;
 	constexpr int Pitch = K + 4;
@@ -716,7 +725,7 @@ void shortReductionKernel( const float* A, const float* W, const float* bias, fl
 			const float b = ( bias != nullptr && n < N ) ? bias[n] : 0.f;
 #pragma unroll
 			for( int r = 0; r < 16; ++r ) {
-				patch[( ( r >> 2 ) * 8 + half * 4 + ( r & 3 ) ) * PatchPitch + l32] = acc[r] + b;
+				patch[( ( r >> 2 ) * 8 + half * 4 + ( r & 3 ) ) * PatchPitch + l32] = applyActivation( acc[r] + b, act );
 			}
 			// ( same wavefront: the LDS unit executes its reads after its writes, no barrier needed )
 			const int col4 = ( lane & 7 ) * 4;
@@ -724,10 +733,17 @@ void shortReductionKernel( const float* A, const float* W, const float* bias, fl
 #pragma unroll
 			for( int q = 0; q < 4; ++q ) {
 				const int row = q * 8 + ( lane >> 3 );
-				const float4 v = *reinterpret_cast<const float4*>( patch + row * PatchPitch + col4 );
+				float4 v = *reinterpret_cast<const float4*>( patch + row * PatchPitch + col4 );
 				const long long mOut = static_cast<long long>( block ) * 32 + row;
 				if( mOut < M ) {
 					float* out = C + mOut * N + n4;
+					if( residual != nullptr ) {
+						const float* res = residual + mOut * N + n4;
+						if( n4 < N ) v.x += res[0];
+						if( n4 + 1 < N ) v.y += res[1];
+						if( n4 + 2 < N ) v.z += res[2];
+						if( n4 + 3 < N ) v.w += res[3];
+					}
 					if( rowsAligned && n4 + 3 < N ) {
 						*reinterpret_cast<float4*>( out ) = v;
 					} else {
@@ -743,18 +759,19 @@ void shortReductionKernel( const float* A, const float* W, const float* bias, fl
 }
 
 template<int KC>
-static void launchShortReduction( hipStream_t stream, const float* a, const float* w, const float* bias, float* c, int M, int N )
+static void launchShortReduction( hipStream_t stream, const float* a, const float* w, const float* bias, float* c, int M, int N,
+	const CFusedActivation& act, const float* residual )
 {
 	const int rowBlocks = ceilDiv( M, 32 );
 	const int groups = ceilDiv( rowBlocks, 4 );
 	const size_t lds = ( static_cast<size_t>( ceilDiv( N, 32 ) ) * 32 * ( KC * 8 + 4 ) + 4 * 32 * 36 ) * sizeof( float );
 	hipLaunchKernelGGL( shortReductionKernel<KC>, dim3( groups < 2048 ? groups : 2048 ), dim3( Threads ), lds, stream,
-		a, w, bias, c, M, N, rowBlocks );
+		a, w, bias, c, M, N, rowBlocks, act, residual );
 }
 
 // true (and launched) when the product has the shape this kernel is for
 static bool tryShortReduction( hipStream_t stream, const float* a, int lda, const float* w, int ldb, float* c, int ldc,
-	int M, int N, int K, const float* bias, int* rc )
+	int M, int N, int K, const float* bias, const CFusedActivation& act, const float* residual, int* rc )
 {
 	if( lda != K || ldb != K || ldc != N || M < 16384 || K % 8 != 0 || K > 192 || N > 192
 		|| !isAligned16( a ) || !isAligned16( w ) || !fitsBuffer( M, K, K )
@@ -763,14 +780,14 @@ static bool tryShortReduction( hipStream_t stream, const float* a, int lda, cons
 		return false;
 	}
 	switch( K / 8 ) {
-		case 2: launchShortReduction<2>( stream, a, w, bias, c, M, N ); break;
-		case 3: launchShortReduction<3>( stream, a, w, bias, c, M, N ); break;
-		case 4: launchShortReduction<4>( stream, a, w, bias, c, M, N ); break;
-		case 6: launchShortReduction<6>( stream, a, w, bias, c, M, N ); break;
-		case 8: launchShortReduction<8>( stream, a, w, bias, c, M, N ); break;
-		case 12: launchShortReduction<12>( stream, a, w, bias, c, M, N ); break;
-		case 18: launchShortReduction<18>( stream, a, w, bias, c, M, N ); break;
-		case 24: launchShortReduction<24>( stream, a, w, bias, c, M, N ); break;
+		case 2: launchShortReduction<2>( stream, a, w, bias, c, M, N, act, residual ); break;
+		case 3: launchShortReduction<3>( stream, a, w, bias, c, M, N, act, residual ); break;
+		case 4: launchShortReduction<4>( stream, a, w, bias, c, M, N, act, residual ); break;
+		case 6: launchShortReduction<6>( stream, a, w, bias, c, M, N, act, residual ); break;
+		case 8: launchShortReduction<8>( stream, a, w, bias, c, M, N, act, residual ); break;
+		case 12: launchShortReduction<12>( stream, a, w, bias, c, M, N, act, residual ); break;
+		case 18: launchShortReduction<18>( stream, a, w, bias, c, M, N, act, residual ); break;
+		case 24: launchShortReduction<24>( stream, a, w, bias, c, M, N, act, residual ); break;
 		default: return false;
 	}
 	const hipError_t err = hipGetLastError();
@@ -784,9 +801,22 @@ static bool tryShortReduction( hipStream_t stream, const float* a, int lda, cons
 }
 
 // C = A * B^T (+ bias) with row strides; also the inner product of the convolution with a 1x1 filter.
+int matMulNTFused( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
+	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC,
+	const float* bias, bool accumulate, const CFusedActivation& act, const float* residual );
+
 int matMulNT( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
 	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC,
 	const float* bias, bool accumulate )
+{
+	const CFusedActivation none = { NH_ACT_NONE, 0.f };
+	return matMulNTFused( stream, a, lda, b, ldb, c, ldc, M, N, K, batch, strideA, strideB, strideC, bias, accumulate, none, nullptr );
+}
+
+// ... and C = act( A * B^T + bias ) + residual, the epilogue of the fused blocks
+int matMulNTFused( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
+	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC,
+	const float* bias, bool accumulate, const CFusedActivation& act, const float* residual )
 {
 	if( M == 0 || N == 0 || batch == 0 ) {
 		return NH_OK;
@@ -797,8 +827,10 @@ int matMulNT( hipStream_t stream, const float* a, int lda, const float* b, int l
 	args.Lda = lda; args.Ldb = ldb; args.Ldc = ldc;
 	args.BatchStrideA = strideA; args.BatchStrideB = strideB; args.BatchStrideC = strideC;
 	args.Accumulate = accumulate ? 1 : 0;
+	args.Act = act;
+	args.Residual = residual;
 	int rc = NH_OK;
-	if( batch == 1 && !accumulate && tryShortReduction( stream, a, lda, b, ldb, c, ldc, M, N, K, bias, &rc ) ) {
+	if( batch == 1 && !accumulate && tryShortReduction( stream, a, lda, b, ldb, c, ldc, M, N, K, bias, act, residual, &rc ) ) {
 		return rc;
 	}
 	const bool vec = isAligned16( a ) && isAligned16( b ) && K % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0
@@ -949,6 +981,16 @@ int nhBatchMultiplyTransposedMatrixByMatrix( nhStream s, int batchSize, const fl
 		firstWidth, secondWidth, firstHeight, batchSize,
 		static_cast<long long>( firstHeight ) * firstWidth, static_cast<long long>( firstHeight ) * secondWidth,
 		static_cast<long long>( firstWidth ) * secondWidth, false );
+}
+
+int nhPointwiseConvolutionWithActivation( nhStream s, const float* source, int rows, int channels,
+	const float* filter, const float* freeTerm, int filterCount, int activation, float param, float* result )
+{
+	NH_REQUIRE( source != nullptr && filter != nullptr && result != nullptr );
+	NH_REQUIRE( rows >= 0 && channels > 0 && filterCount > 0 );
+	const CFusedActivation act = { activation, param };
+	return matMulNTFused( toStream( s ), source, channels, filter, channels, result, filterCount, rows, filterCount, channels,
+		1, 0, 0, 0, freeTerm, false, act, nullptr );
 }
 
 int nhInitBlobConvolution( nhConvDesc* d )

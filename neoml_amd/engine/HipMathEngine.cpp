@@ -131,13 +131,6 @@ void CHipMathEngine::check( int code, const char* what, int line ) const
 		L"HipMathEngine.cpp", line, code );
 }
 
-template<class T>
-T* CHipMathEngine::raw( const CTypedMemoryHandle<T>& handle ) const
-{
-	ASSERT_EXPR( handle.GetMathEngine() == this );
-	return static_cast<T*>( CMemoryHandleInternal::GetRaw( handle ) );
-}
-
 void* CHipMathEngine::rawBytes( const CMemoryHandle& handle ) const
 {
 	ASSERT_EXPR( handle.GetMathEngine() == this );

@@ -209,6 +209,42 @@ public:
 		const CConstFloatHandle& input, const CFloatHandle& outputStateBackLink,
 		const CFloatHandle& outputMainBackLink ) override;
 
+	// the fused blocks and operation chains of the graph optimizer (HipMathEngineRowwise.cpp)
+	void ChannelwiseWith1x1( const CBlobDesc& inputDesc, const CBlobDesc& outputDesc,
+		const CRowwiseOperationDesc& rowwiseDesc, const CChannelwiseConvolutionDesc& convDesc,
+		const CConstFloatHandle& inputHandle, const CFloatHandle& outputHandle ) override;
+	void MobileNetV2Block( const CBlobDesc& inputDesc, const CBlobDesc& outputDesc,
+		const CRowwiseOperationDesc& rowwiseDesc, const CChannelwiseConvolutionDesc& convDesc,
+		const CConstFloatHandle& inputHandle, const CFloatHandle& outputHandle ) override;
+	CRowwiseOperationDesc* InitRowwiseActivation( const CActivationDesc& desc ) override;
+	CRowwiseOperationDesc* InitRowwiseChWith1x1( int stride, const CConstFloatHandle& channelwiseFilter,
+		const CConstFloatHandle* channelwiseFreeTerm, TActivationFunction activation, float reluParam,
+		const CConstFloatHandle& convFilter, const CConstFloatHandle* convFreeTerm,
+		int outputChannels, bool residual ) override;
+	CRowwiseOperationDesc* InitRowwiseConv( int paddingHeight, int paddingWidth, int strideHeight,
+		int strideWidth, int dilationHeight, int dilationWidth, const CBlobDesc& filterDesc,
+		const CConstFloatHandle& filter, const CConstFloatHandle* freeTerm ) override;
+	CRowwiseOperationDesc* InitRowwiseChConv( int paddingHeight, int paddingWidth, int strideHeight,
+		int strideWidth, const CBlobDesc& filterDesc, const CConstFloatHandle& filter,
+		const CConstFloatHandle* freeTerm ) override;
+	CRowwiseOperationDesc* InitRowwiseMobileNetV2( int inputChannels,
+		const CConstFloatHandle& expandFilter, const CConstFloatHandle* expandFreeTerm, int expandedChannels,
+		TActivationFunction expandActivation, float expandReluParam,
+		const CConstFloatHandle& channelwiseFilter, const CConstFloatHandle* channelwiseFreeTerm, int stride,
+		TActivationFunction channelwiseActivation, float channelwiseReluParam,
+		const CConstFloatHandle& downFilter, const CConstFloatHandle* downFreeTerm,
+		int outputChannels, bool residual ) override;
+	CRowwiseOperationDesc* InitRowwise2DPooling( bool isMax, int filterHeight, int filterWidth,
+		int strideHeight, int strideWidth ) override;
+	CRowwiseOperationDesc* InitRowwiseResizeImage( TBlobResizePadding padding, float defaultValue,
+		int deltaLeft, int deltaRight, int deltaTop, int deltaBottom ) override;
+	CBlobDesc RowwiseReshape( CRowwiseOperationDesc** operations, int operationCount,
+		const CBlobDesc& input ) override;
+	void RowwiseExecute( const CBlobDesc& inputDesc, CRowwiseOperationDesc** operations, int operationCount,
+		const CFloatHandle& input, const CFloatHandle& output ) override;
+	// runs a CHipRowwiseSeparableBlock (either MobileNet block) on whole blobs
+	void RunSeparableBlock( const CRowwiseOperationDesc& block, const CConstFloatHandle& input, const CFloatHandle& output );
+
 	// ---- IMathEngine ----
 	TMathEngineType GetType() const override;
 	void GetMathEngineInfo( CMathEngineInfo& info ) const override;
@@ -267,6 +303,14 @@ private:
 	template<class T> T* raw( const CTypedMemoryHandle<T>& handle ) const;
 	void* rawBytes( const CMemoryHandle& handle ) const;
 };
+
+// the device pointer behind a handle of this engine
+template<class T>
+inline T* CHipMathEngine::raw( const CTypedMemoryHandle<T>& handle ) const
+{
+	ASSERT_EXPR( handle.GetMathEngine() == this );
+	return static_cast<T*>( CMemoryHandleInternal::GetRaw( handle ) );
+}
 
 } // namespace NeoML
 

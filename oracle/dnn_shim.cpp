@@ -208,6 +208,73 @@ static CBaseLayer* buildResNet18( CDnn& dnn, IMathEngine& e, CBaseLayer& source,
 	return softmax.Ptr();
 }
 
+// kind 6: a small depthwise-separable network of plain layers, the patterns NeoML's graph optimizer rewrites:
+//         stem 3x3/2 (16) - ReLU6 - inverted residual block (1x1 to 96 - ReLU6 - channelwise 3x3 - ReLU6 - 1x1 to 16, + input)
+//         - inverted block with stride 2 (to 24 channels, no residual) - channelwise 3x3 - h-swish - 1x1 (32)
+//         - global mean pool - FullyConnected (param) - softmax. Input dims: [1, N, 1, H, W, 1, 3].
+static CBaseLayer* relu6( CDnn& dnn, IMathEngine& e, const CString& name, CBaseLayer& input )
+{
+	CPtr<CReLULayer> layer = add( dnn, new CReLULayer( e ), name, input );
+	layer->SetUpperThreshold( 6.f );
+	return layer.Ptr();
+}
+
+static CBaseLayer* channelwise3x3( CDnn& dnn, IMathEngine& e, const CString& name, CBaseLayer& input, int channels, int stride )
+{
+	CPtr<CChannelwiseConvLayer> layer = add( dnn, new CChannelwiseConvLayer( e ), name, input );
+	layer->SetFilterCount( channels ); layer->SetFilterHeight( 3 ); layer->SetFilterWidth( 3 );
+	layer->SetPaddingHeight( 1 ); layer->SetPaddingWidth( 1 );
+	layer->SetStrideHeight( stride ); layer->SetStrideWidth( stride );
+	return layer.Ptr();
+}
+
+static CBaseLayer* invertedBlock( CDnn& dnn, IMathEngine& e, const CString& name, CBaseLayer& input, int expanded,
+	int outputChannels, int stride, bool residual )
+{
+	CBaseLayer* x = conv( dnn, e, name + "_expand", input, expanded, 1, 0, 1 ).Ptr();
+	x = relu6( dnn, e, name + "_relu1", *x );
+	x = channelwise3x3( dnn, e, name + "_dw", *x, expanded, stride );
+	x = relu6( dnn, e, name + "_relu2", *x );
+	x = conv( dnn, e, name + "_down", *x, outputChannels, 1, 0, 1 ).Ptr();
+	if( residual ) {
+		CPtr<CEltwiseSumLayer> sum = new CEltwiseSumLayer( e );
+		sum->SetName( name + "_sum" );
+		sum->Connect( 0, input );
+		sum->Connect( 1, *x );
+		dnn.AddLayer( *sum );
+		x = sum.Ptr();
+	}
+	return x;
+}
+
+static CBaseLayer* buildSeparableNet( CDnn& dnn, IMathEngine& e, CBaseLayer& source, int classes )
+{
+	CBaseLayer* x = conv( dnn, e, "stem", source, 16, 3, 1, 2 ).Ptr();
+	x = relu6( dnn, e, "stem_relu", *x );
+	x = invertedBlock( dnn, e, "b1", *x, 96, 16, 1, true );
+	x = invertedBlock( dnn, e, "b2", *x, 96, 24, 2, false );
+	x = channelwise3x3( dnn, e, "tail_dw", *x, 24, 1 );
+	CPtr<CHSwishLayer> hswish = add( dnn, new CHSwishLayer( e ), "tail_hswish", *x );
+	x = conv( dnn, e, "tail_conv", *hswish, 32, 1, 0, 1 ).Ptr();
+	CPtr<CGlobalMeanPoolingLayer> gap = add( dnn, new CGlobalMeanPoolingLayer( e ), "gap", *x );
+	CPtr<CFullyConnectedLayer> fc = add( dnn, new CFullyConnectedLayer( e ), "fc", *gap );
+	fc->SetNumberOfElements( classes );
+	CPtr<CSoftmaxLayer> softmax = add( dnn, new CSoftmaxLayer( e ), "softmax", *fc );
+	return softmax.Ptr();
+}
+
+// When set, dnn_run hands the network to NeoML's own graph optimizer (OptimizeDnn) after its first pass (the pass
+// that allocates and initialises the weights) and keeps what the optimizer reports
+static int optimizeNetworks = 0;
+static CDnnOptimizationReport lastReport;
+EXPORT void dnn_set_optimize( int on ) { optimizeNetworks = on; }
+EXPORT void dnn_last_optimization( int* mobileNetV2Blocks, int* channelwiseWith1x1, int* rowwiseChains )
+{
+	*mobileNetV2Blocks = lastReport.MobileNetV2NonResidualBlocks + lastReport.MobileNetV2ResidualBlocks;
+	*channelwiseWith1x1 = lastReport.ChannelwiseWith1x1NonResidual + lastReport.ChannelwiseWith1x1Residual;
+	*rowwiseChains = lastReport.RowwiseChainCount;
+}
+
 // Runs network `kind` on `engine`. dims: the 7 blob dimensions of the input; param: kind-specific size.
 // output receives at most outputCapacity floats; outputDims the 7 dimensions of the result.
 EXPORT int dnn_run( void* engine, int kind, int seed, int param, const int* dims, const float* input,
@@ -229,6 +296,7 @@ EXPORT int dnn_run( void* engine, int kind, int seed, int param, const int* dims
 			case 3: last = buildResNetBlock( dnn, e, *source ); break;
 			case 4: last = buildRecognizerTail( dnn, e, *source, param ); break;
 			case 5: last = buildResNet18( dnn, e, *source, param ); break;
+			case 6: last = buildSeparableNet( dnn, e, *source, param ); break;
 			default: lastError = "unknown network kind"; return 1;
 		}
 		CPtr<CSinkLayer> sink = new CSinkLayer( e );
@@ -245,6 +313,9 @@ EXPORT int dnn_run( void* engine, int kind, int seed, int param, const int* dims
 		source->SetBlob( blob );
 
 		dnn.RunOnce();
+		if( optimizeNetworks != 0 ) {
+			lastReport = OptimizeDnn( dnn );
+		}
 		// a second pass over the same network: buffers are reused, results must not change
 		dnn.RunOnce();
 

@@ -460,6 +460,67 @@ SHIM_API int shim_blob_channelwise_convolution( void* engine, const float* in, i
 	} );
 }
 
+// The two fused blocks of depthwise-separable networks through the interface calls their layers make
+// (MobileNetV2BlockLayer.cpp:205-250, ChannelwiseWith1x1Layer.cpp:150-197). activation codes: 0 none (AF_Linear),
+// 1 ReLU (param = upper threshold when > 0), 2 h-swish. withExpand: MobileNetV2Block, else ChannelwiseWith1x1
+// (then inputChannels is not used and expandedChannels is the input's channel count).
+// inPlace != 0 (residual blocks only): output blob = input blob, as CDnn does when it reuses memory.
+SHIM_API int shim_separable_block( void* engine, int withExpand, const float* in, int n, int h, int w, int inputChannels,
+	int expandedChannels, int outputChannels, int stride, int residual, int expandActivation, float expandParam,
+	int channelwiseActivation, float channelwiseParam, const float* expandFilter, const float* expandFreeTerm,
+	const float* channelwiseFilter, const float* channelwiseFreeTerm, const float* downFilter, const float* downFreeTerm,
+	int inPlace, float* out )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		static const TActivationFunction types[3] = { AF_Linear, AF_ReLU, AF_HSwish };
+		const int blockInput = withExpand ? inputChannels : expandedChannels;
+		const int ho = ( h + stride - 1 ) / stride, wo = ( w + stride - 1 ) / stride;
+		const CBlobDesc inDesc = imageDesc( n, h, w, blockInput ), outDesc = imageDesc( n, ho, wo, outputChannels ),
+			chInDesc = imageDesc( n, h, w, expandedChannels ), chOutDesc = imageDesc( n, ho, wo, expandedChannels ),
+			chFilterDesc = imageDesc( 1, 3, 3, expandedChannels ), chFreeTermDesc = imageDesc( 1, 1, 1, expandedChannels );
+		if( inPlace && inDesc.BlobSize() != outDesc.BlobSize() ) {
+			throw std::logic_error( "in-place block needs equal input and output sizes" );
+		}
+		CFloatBlob src( e, inDesc.BlobSize(), in ),
+			dst( e, outDesc.BlobSize() ),
+			exF( e, withExpand ? expandedChannels * inputChannels : 1, withExpand ? expandFilter : nullptr ),
+			exT( e, expandedChannels, expandFreeTerm ), chF( e, 9 * expandedChannels, channelwiseFilter ),
+			chT( e, expandedChannels, channelwiseFreeTerm ), dnF( e, outputChannels * expandedChannels, downFilter ),
+			dnT( e, outputChannels, downFreeTerm );
+		const CConstFloatHandle exTh = exT.Const(), chTh = chT.Const(), dnTh = dnT.Const();
+		CChannelwiseConvolutionDesc* convDesc = e.InitBlobChannelwiseConvolution( chInDesc, 1, 1, stride, stride, chFilterDesc,
+			channelwiseFreeTerm != nullptr ? &chFreeTermDesc : nullptr, chOutDesc );
+		CRowwiseOperationDesc* rowwise = withExpand
+			? e.InitRowwiseMobileNetV2( inputChannels, exF.Const(), expandFreeTerm != nullptr ? &exTh : nullptr, expandedChannels,
+				types[expandActivation], expandParam, chF.Const(), channelwiseFreeTerm != nullptr ? &chTh : nullptr, stride,
+				types[channelwiseActivation], channelwiseParam, dnF.Const(), downFreeTerm != nullptr ? &dnTh : nullptr,
+				outputChannels, residual != 0 )
+			: e.InitRowwiseChWith1x1( stride, chF.Const(), channelwiseFreeTerm != nullptr ? &chTh : nullptr,
+				types[channelwiseActivation], channelwiseParam, dnF.Const(), downFreeTerm != nullptr ? &dnTh : nullptr,
+				outputChannels, residual != 0 );
+		try {
+			const CFloatHandle target = inPlace ? src.Handle() : dst.Handle();
+			if( withExpand ) {
+				e.MobileNetV2Block( inDesc, outDesc, *rowwise, *convDesc, src.Const(), target );
+			} else {
+				e.ChannelwiseWith1x1( inDesc, outDesc, *rowwise, *convDesc, src.Const(), target );
+			}
+		} catch( ... ) {
+			delete rowwise;
+			delete convDesc;
+			throw;
+		}
+		delete rowwise;
+		delete convDesc;
+		if( inPlace ) {
+			src.CopyTo( out );
+		} else {
+			dst.CopyTo( out );
+		}
+	} );
+}
+
 SHIM_API int shim_blob_max_pooling( void* engine, const float* in, int n, int h, int w, int c, int fh, int fw,
 	int sh, int sw, int* indices, float* out )
 {

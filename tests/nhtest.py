@@ -327,6 +327,44 @@ class Cpu:
         self._call("blob_channelwise_convolution", fp(x), n, h, w, c, fp(filt), fh, fw, ph, pw, sh, sw, fp(bias), fp(y))
         return y
 
+    ACTIVATIONS = {None: 0, "relu": 1, "hswish": 2}
+
+    def separable_block(self, x, expand, channelwise, down, stride=1, residual=False, in_place=False):
+        """The fused blocks of depthwise-separable networks. expand = (filter [E][Cin], free term, activation, param)
+        or None for the channelwise + 1x1 block; channelwise = (filter [3][3][E], free term, activation, param);
+        down = (filter [Cout][E], free term). activation: None, 'relu' (param = upper threshold when > 0), 'hswish'.
+        The oracle composes the block from its own convolution, channelwise convolution and activation functions,
+        stage by stage as src/CPU/Rowwise/CpuRowwiseMobileNetV2.h:150-300 and CpuRowwiseChConvWith1x1.h do; the
+        reference engine runs its MobileNetV2Block / ChannelwiseWith1x1."""
+        x = f32(x)
+        n, h, w, cin = x.shape
+        ch_f, ch_t, ch_act, ch_param = channelwise
+        dn_f, dn_t = down
+        e = ch_f.shape[2]
+        cout = dn_f.shape[0]
+        ho, wo = (h + stride - 1) // stride, (w + stride - 1) // stride
+        if self.kind == "orc":
+            def act(t, name, param):
+                if name is None:
+                    return t
+                return self.unary(name, t, np.float32(param if name == "relu" else 0.0)).reshape(t.shape)
+            t = x
+            if expand is not None:
+                ex_f, ex_t, ex_act, ex_param = expand
+                t = act(self.conv(t, f32(ex_f).reshape(e, 1, 1, cin), ex_t, 0, 0, 1, 1), ex_act, ex_param)
+            t = act(self.channelwise_conv(t, ch_f, ch_t, 1, 1, stride, stride), ch_act, ch_param)
+            y = self.conv(t, f32(dn_f).reshape(cout, 1, 1, e), dn_t, 0, 0, 1, 1)
+            return y + x if residual else y
+        ex_f, ex_t, ex_act, ex_param = expand if expand is not None else (None, None, None, 0.0)
+        y = np.empty((n, ho, wo, cout), np.float32)
+        opt = lambda a: None if a is None else f32(a)
+        keep = [opt(ex_f), opt(ex_t), f32(ch_f), opt(ch_t), f32(dn_f), opt(dn_t)]
+        self._call("separable_block", 1 if expand is not None else 0, fp(x), n, h, w, cin, e, cout, stride,
+                   1 if residual else 0, self.ACTIVATIONS[ex_act], ctypes.c_float(ex_param), self.ACTIVATIONS[ch_act],
+                   ctypes.c_float(ch_param), fp(keep[0]), fp(keep[1]), fp(keep[2]), fp(keep[3]), fp(keep[4]), fp(keep[5]),
+                   1 if in_place else 0, fp(y))
+        return y
+
     def max_pool(self, x, fh, fw, sh, sw, with_indices=False):
         x = f32(x)
         n, h, w, c = x.shape
@@ -676,6 +714,33 @@ class Hip:
         out = self.empty((n, d.resultHeight, d.resultWidth, c))
         self.call("nhBlobChannelwiseConvolution", ctypes.byref(d), self.p(xs), self.p(fs), self.p(bs), self.p(out))
         return self.down(out)
+
+    def separable_block(self, x, expand, channelwise, down, stride=1, residual=False, in_place=False):
+        x = f32(x)
+        n, h, w, cin = x.shape
+        ch_f, ch_t, ch_act, ch_param = channelwise
+        dn_f, dn_t = down
+        e, cout = ch_f.shape[2], dn_f.shape[0]
+        ex_f, ex_t, ex_act, ex_param = expand if expand is not None else (None, None, None, 0.0)
+        acts = Cpu.ACTIVATIONS
+        d = self.na.SeparableBlockDesc(n, h, w, cin if expand is not None else 0, e, cout, stride, 1 if residual else 0,
+                                       acts[ex_act], ex_param, acts[ch_act], ch_param)
+        size = ctypes.c_size_t(0)
+        which = "nhMobileNetV2Block" if expand is not None else "nhChannelwiseWith1x1"
+        self.na.check(getattr(self.lib, which + "WorkspaceSize")(ctypes.byref(d), ctypes.byref(size)))
+        work = self.torch.empty((size.value + 15) // 4 + 4, dtype=self.torch.float32, device=self.dev)
+        xs = self.up(x)
+        ho, wo = (h + stride - 1) // stride, (w + stride - 1) // stride
+        out = xs if in_place else self.empty((n, ho, wo, cout))
+        up = lambda a: self.up(None if a is None else f32(a))
+        ws = [up(ex_f), up(ex_t), up(ch_f), up(ch_t), up(dn_f), up(dn_t)]
+        if expand is not None:
+            self.call(which, ctypes.byref(d), self.p(xs), self.p(ws[0]), self.p(ws[1]), self.p(ws[2]), self.p(ws[3]),
+                      self.p(ws[4]), self.p(ws[5]), self.p(out), self.p(work), size.value)
+        else:
+            self.call(which, ctypes.byref(d), self.p(xs), self.p(ws[2]), self.p(ws[3]), self.p(ws[4]), self.p(ws[5]),
+                      self.p(out), self.p(work), size.value)
+        return self.down(out).reshape(n, ho, wo, cout)
 
     def pool_desc(self, n, h, w, c, fh, fw, sh, sw):
         d = self.na.PoolingDesc(n, h, w, c, fh, fw, sh, sw, 0, 0)

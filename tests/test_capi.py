@@ -62,7 +62,8 @@ def test_lstm_workspace_size():
     lib = neoml_amd.load()
     size = ctypes.c_size_t(0)
     neoml_amd.check(lib.nhLstmWorkspaceSize(256, 512, 128, 64, ctypes.byref(size)))
-    assert size.value == 4 * (128 * 64 * 1024 + 1024 + 64 * 256)
+    # gates for every step, summed free term, one step of cell state, two exchange buffers of 64-bit words, abort word
+    assert size.value == 4 * (128 * 64 * 1024 + 1024 + 64 * 256 + 2 * 2 * 64 * 256 + 2)
 
 
 # ---- caching allocator on host memory (kind 1): same logic as on the device ------------------------------------

@@ -200,3 +200,48 @@ def test_recognizer_tail_at_benchmark_size_fused_vs_composite(capsys):
         print("\nBiLSTM(256) tail, 128 steps x 64 lines, CDnn::RunOnce on CHipMathEngine: CLstmLayer %.2f ms, "
               "CHipLstmLayer %.2f ms" % (composite_ms, fused_ms))
     assert_close(fused, composite, "CHipLstmLayer vs CLstmLayer on the same engine")
+
+
+# ---------------------------------------------------------------------------------------------------------
+# The graph optimizer's fused layers: NeoML's OptimizeDnn rewrites the plain layers of a depthwise-separable network
+# into CMobileNetV2BlockLayer / CChannelwiseWith1x1Layer / CRowwiseOperationChainLayer, whose RunOnce calls
+# IMathEngine::MobileNetV2Block, ChannelwiseWith1x1 and RowwiseExecute.
+
+CASES["separable_net"] = (6, (1, 3, 1, 32, 40, 1, 3), 10)
+
+
+class optimized:
+    def __enter__(self):
+        lib().dnn_set_optimize(1)
+
+    def __exit__(self, *exc):
+        lib().dnn_set_optimize(0)
+
+
+def last_optimization():
+    counts = [ctypes.c_int(0) for _ in range(3)]
+    lib().dnn_last_optimization(*[ctypes.byref(c) for c in counts])
+    return tuple(c.value for c in counts)
+
+
+def test_optimizer_rewrites_the_separable_network_on_the_cpu_engine():
+    kind, dims, param = CASES["separable_net"]
+    x = make_input("separable_net")
+    plain = dnn_run(nhtest.cpu_engine(), kind, dims, x, param)
+    with optimized():
+        fused = dnn_run(nhtest.cpu_engine(), kind, dims, x, param)
+    blocks, with1x1, chains = last_optimization()
+    assert blocks == 2 and with1x1 >= 1 and chains >= 1  # (the 1x1 pass also counts the pairs inside the two blocks)
+    assert_close(fused, plain, "optimized vs plain network on the CPU engine")
+
+
+@pytest.mark.gpu
+def test_optimized_separable_network_on_hip_engine():
+    kind, dims, param = CASES["separable_net"]
+    x = make_input("separable_net")
+    want = dnn_run(nhtest.cpu_engine(), kind, dims, x, param)
+    with optimized():
+        got = dnn_run(nhtest.hip_engine(), kind, dims, x, param)
+    blocks, with1x1, chains = last_optimization()
+    assert blocks == 2 and with1x1 >= 1 and chains >= 1  # (the 1x1 pass also counts the pairs inside the two blocks)
+    assert_close(got, want, "optimized network on CHipMathEngine vs plain network on CCpuMathEngine")

@@ -139,3 +139,18 @@ def test_unimplemented_method_asserts_like_the_reference_gpu_engine():
     x = np.ones(8, np.float32)
     y = np.empty(8, np.float32)
     assert s.shim_vector_huber(nhtest.hip_engine(), nhtest.fp(x), nhtest.fp(y), 8) == 1
+
+
+@pytest.mark.parametrize("with_expand", [True, False])
+def test_fused_separable_blocks_through_the_interface(with_expand):
+    """InitRowwiseMobileNetV2 / InitRowwiseChWith1x1 + MobileNetV2Block / ChannelwiseWith1x1 on both engines."""
+    from test_oracle import SEPARABLE_CASES, separable_operands
+    hip, ref = engines()
+    for case in SEPARABLE_CASES:
+        x, expand, channelwise, down, stride, residual = separable_operands(case, with_expand)
+        want = ref.separable_block(x, expand, channelwise, down, stride, residual)
+        assert_close(hip.separable_block(x, expand, channelwise, down, stride, residual), want,
+                     "separable block %s expand=%s" % (case, with_expand))
+        if residual and with_expand:
+            assert_close(hip.separable_block(x, expand, channelwise, down, stride, residual, in_place=True), want,
+                         "separable block in place %s" % (case,))

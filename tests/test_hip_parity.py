@@ -10,7 +10,8 @@ import pytest
 
 import nhtest
 from nhtest import Cpu, assert_close
-from test_oracle import (UNARY_CASES, BINARY_CASES, CONV_CASES, CHANNELWISE_CASES, POOL_CASES, unary_input, rng)
+from test_oracle import (UNARY_CASES, BINARY_CASES, CONV_CASES, CHANNELWISE_CASES, POOL_CASES, SEPARABLE_CASES,
+                         separable_operands, unary_input, rng)
 
 pytestmark = pytest.mark.gpu
 
@@ -388,6 +389,26 @@ def test_lstm(reverse, with_init):
             assert_close(c, oc, "lstm c")
             h2, _ = hip().lstm(w_in, bi, w_rec, br, x, reverse, c0, h0, want_state=False)
             assert_close(h2, oh, "lstm h without state output")
+
+
+GPU_SEPARABLE_CASES = SEPARABLE_CASES + [
+    (2, 56, 56, 24, 144, 24, 1, True, ("relu", 6.0), ("relu", 6.0)),    # the row-resident pointwise kernel on both 1x1 stages
+    (1, 112, 112, 16, 96, 24, 2, False, ("relu", 6.0), ("relu", 6.0)),
+    (4, 14, 14, 64, 384, 64, 1, True, ("hswish", 0.0), ("hswish", 0.0)),  # the tiled kernel with an epilogue
+]
+
+
+@pytest.mark.parametrize("case", GPU_SEPARABLE_CASES)
+@pytest.mark.parametrize("with_expand", [True, False])
+def test_separable_blocks(case, with_expand):
+    for with_free_terms in (True, False):
+        x, expand, channelwise, down, stride, residual = separable_operands(case, with_expand, with_free_terms)
+        want = orc.separable_block(x, expand, channelwise, down, stride, residual)
+        got = hip().separable_block(x, expand, channelwise, down, stride, residual)
+        assert_close(got, want, "separable block %s expand=%s" % (case, with_expand))
+        if residual and with_expand:  # the layer of the MobileNetV2 block reuses its input blob
+            got = hip().separable_block(x, expand, channelwise, down, stride, residual, in_place=True)
+            assert_close(got, want, "separable block in place %s" % (case,))
 
 
 def test_lstm_long_sequence():

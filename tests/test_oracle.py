@@ -348,6 +348,65 @@ def test_convolution_1x1_is_a_matrix_product():
     assert_close(y.reshape(-1, 7), x.reshape(-1, 6).astype(np.float64) @ f.reshape(7, 6).astype(np.float64).T, "1x1")
 
 
+# (n, h, w, cin, expanded, cout, stride, residual, expand activation, channelwise activation)
+SEPARABLE_CASES = [
+    (2, 9, 11, 8, 48, 8, 1, True, ("relu", 6.0), ("relu", 6.0)),
+    (1, 12, 10, 16, 96, 24, 2, False, ("relu", 0.0), ("hswish", 0.0)),
+    (2, 7, 7, 12, 20, 12, 1, True, ("hswish", 0.0), (None, 0.0)),
+    (1, 5, 6, 3, 5, 7, 2, False, (None, 0.0), ("relu", 2.5)),       # channel counts not a multiple of 4
+    (3, 8, 8, 24, 144, 32, 1, False, ("relu", 6.0), ("relu", 6.0)),
+]
+
+
+def separable_operands(case, with_expand, with_free_terms=True):
+    n, h, w, cin, e, cout, stride, residual, ex_act, ch_act = case
+    g = rng(40 + h * w + e)
+    block_in = cin if with_expand else e
+    if not with_expand and residual:
+        cout = e
+    x = g.uniform(-2, 2, (n, h, w, block_in)).astype(np.float32)
+    ft = (lambda k: g.uniform(-0.5, 0.5, k).astype(np.float32)) if with_free_terms else (lambda k: None)
+    expand = (g.normal(0, 1.0 / np.sqrt(cin), (e, cin)).astype(np.float32), ft(e), ex_act[0], ex_act[1]) if with_expand else None
+    channelwise = (g.normal(0, 0.4, (3, 3, e)).astype(np.float32), ft(e), ch_act[0], ch_act[1])
+    down = (g.normal(0, 1.0 / np.sqrt(e), (cout, e)).astype(np.float32), ft(cout))
+    return x, expand, channelwise, down, stride, residual
+
+
+@pytest.mark.parametrize("case", SEPARABLE_CASES)
+@pytest.mark.parametrize("with_expand", [True, False])
+def test_separable_blocks_against_the_reference_engine(case, with_expand):
+    """MobileNetV2Block / ChannelwiseWith1x1: the oracle's stage-by-stage composition against the reference CPU
+    engine's fused row-by-row implementation, and against an independent numpy formulation."""
+    for with_free_terms in (True, False):
+        x, expand, channelwise, down, stride, residual = separable_operands(case, with_expand, with_free_terms)
+        y = orc.separable_block(x, expand, channelwise, down, stride, residual)
+        # numpy: 1x1 convolutions as matrix products, the depthwise stage per channel through scipy
+        def act(t, name, param):
+            if name == "relu":
+                t = np.maximum(t, 0)
+                return np.minimum(t, param) if param > 0 else t
+            if name == "hswish":
+                return np.where(t <= -3, 0, np.where(t >= 3, t, t * (t + 3) / 6))
+            return t
+        t = x.astype(np.float64)
+        if expand is not None:
+            t = act(t @ expand[0].astype(np.float64).T + (0 if expand[1] is None else expand[1]), expand[2], expand[3])
+        tp = np.pad(t, ((0, 0), (1, 1), (1, 1), (0, 0)))
+        dw = np.stack([np.stack([scipy.signal.correlate2d(tp[b, :, :, c], channelwise[0][:, :, c].astype(np.float64), mode="valid")
+                                 [::stride, ::stride] for c in range(t.shape[3])], axis=-1) for b in range(t.shape[0])])
+        dw = act(dw + (0 if channelwise[1] is None else channelwise[1]), channelwise[2], channelwise[3])
+        want = dw @ down[0].astype(np.float64).T + (0 if down[1] is None else down[1])
+        if residual:
+            want = want + x
+        assert_close(y, want, "separable block %s expand=%s" % (case, with_expand))
+        if nhtest.have_reference():
+            assert_close(ref().separable_block(x, expand, channelwise, down, stride, residual), y,
+                         "separable block vs reference %s expand=%s" % (case, with_expand))
+            if residual and with_expand:  # only the MobileNetV2 block is specified to work in place
+                assert_close(ref().separable_block(x, expand, channelwise, down, stride, residual, in_place=True), y,
+                             "separable block in place vs reference")
+
+
 CHANNELWISE_CASES = [
     # n, h, w, c, fh, fw, ph, pw, sh, sw
     (1, 3, 3, 1, 3, 3, 1, 1, 1, 1), (2, 8, 9, 16, 3, 3, 1, 1, 1, 1), (2, 8, 9, 16, 3, 3, 1, 1, 2, 2),
