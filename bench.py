@@ -54,7 +54,7 @@ def other_workload(args):
     from neoml_amd.workloads import HipBackend, MobileNetV2, TransformerEncoder, LineRecognizer
     be = HipBackend()
     if args.workload == "mobilenetv2":
-        net = MobileNetV2(be, batch=args.batch or 128, image=args.image)
+        net = MobileNetV2(be, batch=args.batch or 128, image=args.image, fused=args.fused)
         unit, items, name = "images/sec", net.batch, "MobileNetV2-style inference, batch %d, %dx%dx3" % (net.batch, args.image, args.image)
     elif args.workload == "transformer":
         net = TransformerEncoder(be, batch=args.batch or 32)
@@ -107,6 +107,8 @@ def main():
     ap.add_argument("--settle-ms", type=float, default=600.0,
                     help="after the warm-up steps keep replaying the step untimed for this long, so that the timed region "
                          "starts with the GPU at its sustained clock instead of ramping up from idle")
+    ap.add_argument("--fused", action="store_true",
+                    help="mobilenetv2: run the inverted-residual blocks as the graph optimizer's fused block calls")
     ap.add_argument("--workload", default="resnet18", choices=("resnet18", "mobilenetv2", "transformer", "ocr"),
                     help="resnet18 (default) is the configuration the metric is quoted on; the others are the remaining "
                          "BASELINE configurations, measured the same way with a per-family table on stderr")

@@ -193,6 +193,49 @@ class HipBackend:
                     self.lib.nhBlobChannelwiseConvolution, ctypes.byref(d), self._p(x), self._p(filt), self._p(bias), self._p(out))
         return out
 
+    def separable_block(self, x, expand, channelwise, down, stride, residual, out=None):
+        """The fused inverted-residual block (nhMobileNetV2Block) or, without an expand stage, channelwise + 1x1
+        (nhChannelwiseWith1x1), ReLU6 behind the expand and channelwise stages as the configuration has it."""
+        n, h, w, cin = x.shape
+        e, cout = channelwise[0].shape[2], down[0].shape[0]
+        ho, wo = (h + stride - 1) // stride, (w + stride - 1) // stride
+        key = ("sep", n, h, w, cin, e, cout, stride, residual, expand is not None)
+        cached = self._desc_cache.get(key)
+        if cached is None:
+            d = self.na.SeparableBlockDesc(n, h, w, cin if expand is not None else 0, e, cout, stride, 1 if residual else 0,
+                                           1, 6.0, 1, 6.0)
+            size = ctypes.c_size_t(0)
+            fn = self.lib.nhMobileNetV2BlockWorkspaceSize if expand is not None else self.lib.nhChannelwiseWith1x1WorkspaceSize
+            self.na.check(fn(ctypes.byref(d), ctypes.byref(size)))
+            cached = self._desc_cache[key] = (d, size.value)
+        d, size = cached
+        work = self._desc_cache.get("sep_workspace")
+        if work is None or work.numel() * 4 < size:
+            work = self._desc_cache["sep_workspace"] = self.torch.empty((size + 3) // 4, dtype=self.torch.float32, device=self.dev)
+        if out is None:
+            out = self.empty(n, ho, wo, cout)
+        flops = 2 * n * ho * wo * e * (9 + cout) + (2 * n * h * w * e * cin if expand is not None else 0)
+        nbytes = 4 * (x.numel() + out.numel())  # what the block has to move; the expanded tensors are its own business
+        if expand is not None:
+            self._timed("mbv2block", flops, nbytes, self.lib.nhMobileNetV2Block, ctypes.byref(d), self._p(x),
+                        self._p(expand[0]), self._p(expand[1]), self._p(channelwise[0]), self._p(channelwise[1]),
+                        self._p(down[0]), self._p(down[1]), self._p(out), self._p(work), size)
+        else:
+            self._timed("dw+1x1", flops, nbytes, self.lib.nhChannelwiseWith1x1, ctypes.byref(d), self._p(x),
+                        self._p(channelwise[0]), self._p(channelwise[1]), self._p(down[0]), self._p(down[1]),
+                        self._p(out), self._p(work), size)
+        return out
+
+    def pointwise_conv_relu6(self, x, filt, bias, out=None):
+        n, h, w, cin = x.shape
+        cout = filt.shape[0]
+        if out is None:
+            out = self.empty(n, h, w, cout)
+        self._timed("conv1x1+act", conv_flops(n, h, w, cout, 1, 1, cin), conv_bytes(n, h, w, cin, h, w, cout, 1, 1),
+                    self.lib.nhPointwiseConvolutionWithActivation, self._p(x), n * h * w, cin, self._p(filt), self._p(bias),
+                    cout, 1, 6.0, self._p(out))
+        return out
+
     def add(self, a, b, out=None):
         if out is None:
             out = self.empty(*a.shape)
@@ -499,9 +542,12 @@ class MobileNetV2(Network):
 
     TABLE = ((1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2), (6, 320, 1, 1))
 
-    def __init__(self, backend, batch=128, image=224, classes=1000, seed=0xC0FFEE + 3, head=1280):
+    def __init__(self, backend, batch=128, image=224, classes=1000, seed=0xC0FFEE + 3, head=1280, fused=False):
         super().__init__(backend)
         self.batch, self.image, self.classes = batch, image, classes
+        # fused: the form NeoML's graph optimizer gives the network (one MobileNetV2Block / ChannelwiseWith1x1 call per
+        # block, activations inside); same arithmetic
+        self.fused = fused
         g = np.random.default_rng(seed)
 
         def conv(cout, f, cin):
@@ -537,6 +583,10 @@ class MobileNetV2(Network):
         y = run("stem", be.conv, x, *W["stem"], 1, 1, 2, 2)
         be.relu6_(y)
         for name, expand, stride, residual in self.blocks:
+            if self.fused:
+                y = run(name + "p", be.separable_block, y, W[name + "e"] if expand else None, W[name + "d"], W[name + "p"],
+                        stride, residual)
+                continue
             t = y
             if expand:
                 t = run(name + "e", be.conv, t, *W[name + "e"], 0, 0, 1, 1)
@@ -547,8 +597,11 @@ class MobileNetV2(Network):
             if residual:
                 be.add_(t, y)
             y = t
-        y = run("head", be.conv, y, *W["head"], 0, 0, 1, 1)
-        be.relu6_(y)
+        if self.fused:
+            y = run("head", be.pointwise_conv_relu6, y, *W["head"])
+        else:
+            y = run("head", be.conv, y, *W["head"], 0, 0, 1, 1)
+            be.relu6_(y)
         y = run("gap", be.global_mean, y)
         return run("fc", be.fc, y, *W["fc"])
 

@@ -871,6 +871,15 @@ class CpuBackend:
     def channelwise_conv(self, x, filt, bias, ph, pw, sh, sw, out=None):
         return self.cpu.channelwise_conv(x, filt, bias, ph, pw, sh, sw)
 
+    def separable_block(self, x, expand, channelwise, down, stride, residual, out=None):
+        ex = None if expand is None else (expand[0].reshape(expand[0].shape[0], -1), expand[1], "relu", 6.0)
+        return self.cpu.separable_block(x, ex, (channelwise[0], channelwise[1], "relu", 6.0),
+                                        (down[0].reshape(down[0].shape[0], -1), down[1]), stride, residual)
+
+    def pointwise_conv_relu6(self, x, filt, bias, out=None):
+        y = self.cpu.conv(x, filt, bias, 0, 0, 1, 1)
+        return self.cpu.unary("relu", y, 6.0).reshape(y.shape)
+
     def add(self, a, b, out=None):
         return self.cpu.binary("add", a, b).reshape(a.shape)
 
