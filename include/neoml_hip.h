@@ -290,7 +290,12 @@ NH_API int nhBlobMeanPooling(nhStream s, const nhPoolingDesc* desc_host, const f
 /* LSTM (NME.h:1005-1011). Weights: inputWeights [4H x objectSize], recurrentWeights [4H x H]; gate order in
  * the 4H vector: main(tanh) | forget | input | output (src/CPU/CpuMathEngineDnnLstm.h:49-90).
  * Free terms, inputStateBackLink, inputMainBackLink and outputStateBackLink may be null.
- * workspace: nhLstmWorkspaceSize bytes of device memory, owned by the caller. */
+ * workspace: nhLstmWorkspaceSize bytes of device memory, owned by the caller.
+ * Sequences of 2+ steps with H a multiple of 16, H <= 512 and a grid that fits the device run as ONE launch whose
+ * workgroups stay resident and hand the step outputs to one another through memory; it needs the device to itself
+ * for that launch (other work on the same stream is ordered before or after it anyway). Its wait for a step's values
+ * is bounded: should it trip (several such launches sharing the device from different streams), the launch ends
+ * normally with invalid output, and the next nhStreamSynchronize / nhCopyDeviceToHost returns NH_ERR_HIP once. */
 NH_API int nhLstmWorkspaceSize(int hiddenSize, int objectSize, int sequenceLength, int sequenceCount, size_t* bytes);
 NH_API int nhLstm(nhStream s, int hiddenSize, int objectSize, const float* inputWeights, const float* inputFreeTerm,
 	const float* recurrentWeights, const float* recurrentFreeTerm, int reverse, int sequenceLength,

@@ -4,6 +4,7 @@
 #include "common.h"
 #include <float.h>
 #include <stdlib.h>
+#include <atomic>
 
 namespace nh {
 
@@ -673,6 +674,11 @@ __device__ __forceinline__ float seqTanh( float x )
 }
 
 
+// Sticky count of wavefronts that gave up a wait, over all launches on this device: the abort word lives in the
+// caller's workspace, which the caller is free to recycle, so the host reads this one after it has drained a stream
+// and reports the give-up through the next synchronising call.
+__device__ unsigned seqGiveUps;
+
 template<int RB, int CB, int W>
 __global__ __launch_bounds__( 64 * W )
 void lstmSequenceKernel( const CLstmSeqArgs a )
@@ -815,6 +821,9 @@ void lstmSequenceKernel( const CLstmSeqArgs a )
 					&& __hip_atomic_load( a.Abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT ) != 0 ) )
 				{
 					__hip_atomic_store( a.Abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT );
+					if( lane == 0 ) {
+						atomicAdd( &seqGiveUps, 1u );
+					}
 					giveUp = 1; // read by the whole workgroup after the next barrier
 					break;
 				}
@@ -945,6 +954,30 @@ using namespace nh;
 
 extern "C" int nhInitPooling( nhPoolingDesc* d );
 
+// set by every launch of the one-launch LSTM, cleared by the check below
+static std::atomic<bool> sequenceLaunched( false );
+
+namespace nh {
+// Called by the synchronising entry points once their stream has drained: a one-launch LSTM whose bounded wait
+// tripped has produced garbage, and that must not pass silently.
+int checkSequenceGiveUps()
+{
+	if( !sequenceLaunched.exchange( false ) ) {
+		return NH_OK;
+	}
+	unsigned count = 0;
+	NH_HIP( hipMemcpyFromSymbol( &count, HIP_SYMBOL( seqGiveUps ), sizeof( count ) ) );
+	if( count == 0 ) {
+		return NH_OK;
+	}
+	const unsigned zero = 0;
+	NH_HIP( hipMemcpyToSymbol( HIP_SYMBOL( seqGiveUps ), &zero, sizeof( zero ) ) );
+	setLastError( "nhLstm: %u wavefronts of a one-launch LSTM gave up waiting for the previous step (the grid was not "
+		"resident as a whole, or the spin limit is too low): its output is invalid", count );
+	return NH_ERR_HIP;
+}
+} // namespace nh
+
 // ---- whole-sequence LSTM launch ------------------------------------------------------------------------------
 
 // The shapes of the one-launch kernel: Rows sequences x ( 4 * Blocks ) hidden units per workgroup of Waves wavefronts.
@@ -1047,6 +1080,7 @@ static unsigned lstmSpinLimit()
 
 static int launchLstmSequence( hipStream_t stream, const CLstmSeqArgs& a )
 {
+	sequenceLaunched.store( true );
 	const CLstmSeqShape* shape = lstmSequenceShape( a.H, a.B );
 	NH_REQUIRE( shape != nullptr );
 	const unsigned groups = static_cast<unsigned>( ( a.H / ( SeqUnits * shape->Blocks ) ) * ceilDiv( a.B, shape->Rows ) );

@@ -17,6 +17,10 @@ void setLastError( const char* fmt, ... )
 
 } // namespace nh
 
+namespace nh {
+int checkSequenceGiveUps(); // dnn_ops.hip
+}
+
 using namespace nh;
 
 extern "C" {
@@ -91,7 +95,7 @@ int nhStreamDestroy( nhStream stream )
 int nhStreamSynchronize( nhStream stream )
 {
 	NH_HIP( hipStreamSynchronize( toStream( stream ) ) );
-	return NH_OK;
+	return checkSequenceGiveUps();
 }
 
 int nhRawAlloc( void** ptr, size_t size )
@@ -131,7 +135,7 @@ int nhCopyDeviceToHost( nhStream stream, void* dst, const void* src, size_t size
 	NH_REQUIRE( dst != nullptr && src != nullptr );
 	NH_HIP( hipMemcpyAsync( dst, src, size, hipMemcpyDeviceToHost, toStream( stream ) ) );
 	NH_HIP( hipStreamSynchronize( toStream( stream ) ) );
-	return NH_OK;
+	return checkSequenceGiveUps();
 }
 
 int nhCopyDeviceToDevice( nhStream stream, void* dst, const void* src, size_t size )

@@ -441,6 +441,13 @@ def test_lstm_bounded_wait_gives_up(monkeypatch):
     h, _, word = hip().lstm(w_in, None, w_rec, None, x, want_state=False, return_sync=True)
     monkeypatch.delenv("NH_LSTM_SPIN_LIMIT")
     assert word in (0, 1)
+    # the give-up is also reported, once, by the next synchronising call of the library
+    import neoml_amd
+    rc = neoml_amd.load().nhStreamSynchronize(hip().stream())
+    assert rc == (2 if word == 1 else 0)
+    if word == 1:
+        assert "gave up" in neoml_amd.last_error()
+    assert neoml_amd.load().nhStreamSynchronize(hip().stream()) == 0
     h2, _, word2 = hip().lstm(w_in, None, w_rec, None, x, want_state=False, return_sync=True)
     assert word2 == 0
     oh, _ = orc.lstm(w_in, None, w_rec, None, x)
