@@ -270,8 +270,11 @@ NH_API int nhChannelwiseWith1x1WorkspaceSize(const nhSeparableBlockDesc* desc_ho
 NH_API int nhChannelwiseWith1x1(nhStream s, const nhSeparableBlockDesc* desc_host, const float* input,
 	const float* channelwiseFilter, const float* channelwiseFreeTerm, const float* convFilter,
 	const float* convFreeTerm, float* output, void* workspace, size_t workspaceSize);                /* NME.h:1066 */
-/* A convolution / matrix product with the activation behind it in the same launch, as the rowwise operation chains
- * pair them (NME.h:1080-1087): result = act( source * filter^T + freeTerm ), 1x1 filter [Cout][Cin], rows = pixels */
+/* A convolution with the activation behind it in the same launch, as the rowwise operation chains pair them
+ * (NME.h:1080-1087): nhBlobConvolution followed by NH_ACT_* (a launch that is cut into K slices applies the activation
+ * as a pass of its own); the pointwise form takes a 1x1 filter [Cout][Cin] over rows = pixels */
+NH_API int nhBlobConvolutionWithActivation(nhStream s, const nhConvDesc* desc_host, const float* source,
+	const float* filter, const float* freeTerm, int activation, float param, float* result);
 NH_API int nhPointwiseConvolutionWithActivation(nhStream s, const float* source, int rows, int channels,
 	const float* filter, const float* freeTerm, int filterCount, int activation, float param, float* result);
 

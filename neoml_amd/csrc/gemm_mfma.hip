@@ -557,6 +557,19 @@ __global__ __launch_bounds__( 256 ) void presetResultKernel( float* c, const flo
 	}
 }
 
+// C[b][m][n] = act( C[b][m][n] ): the activation pass behind a launch that met in C through K slices
+__global__ __launch_bounds__( 256 ) void activateResultKernel( float* c, int M, int N, int ldc, long long batchStride, const CFusedActivation act )
+{
+	const long long total = static_cast<long long>( M ) * N;
+	float* base = c + blockIdx.y * batchStride;
+	for( long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += static_cast<long long>( gridDim.x ) * 256 ) {
+		const int m = static_cast<int>( i / N );
+		const int n = static_cast<int>( i - static_cast<long long>( m ) * N );
+		float* p = base + static_cast<long long>( m ) * ldc + n;
+		*p = applyActivation( *p, act );
+	}
+}
+
 static int presetResult( hipStream_t stream, const CMatMulArgs& args, int batch )
 {
 	const long long total = static_cast<long long>( args.M ) * args.N;
@@ -588,8 +601,8 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 	const int totalSteps = ceilDiv( args.K, NH_KSTEP );
 	int splits = 1;
 	const long long blocks = tiles * batch;
-	const bool plainEpilogue = args.Act.Type == NH_ACT_NONE && args.Residual == nullptr; // K slices cannot apply one
-	if( blocks < 1024 && totalSteps >= 32 && plainEpilogue ) {
+	// K slices cannot add a residual; an activation follows them as a pass of its own
+	if( blocks < 1024 && totalSteps >= 32 && args.Residual == nullptr ) {
 		double best = 0;
 		for( int s = 1; s <= 8 && s <= totalSteps / 8; ++s ) {
 			const double rounds = static_cast<double>( blocks * s ) / 1280.0;
@@ -608,6 +621,10 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 			return rc;
 		}
 	}
+	const CFusedActivation actAfter = args.Act;
+	if( args.SplitK > 1 ) {
+		args.Act.Type = NH_ACT_NONE;
+	}
 	// blockIdx.y is limited to 65535: walk larger batches in slices
 	for( int b0 = 0; b0 < batch; b0 += 65535 ) {
 		const int nb = batch - b0 < 65535 ? batch - b0 : 65535;
@@ -620,6 +637,12 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 			hipLaunchKernelGGL( ( matMulKernel<BM, BN, WAVES_M, WAVES_N, AMODE, BMODE, true> ), grid, dim3( Threads ), 0, stream, a );
 		} else {
 			hipLaunchKernelGGL( ( matMulKernel<BM, BN, WAVES_M, WAVES_N, AMODE, BMODE, false> ), grid, dim3( Threads ), 0, stream, a );
+		}
+		if( args.SplitK > 1 && actAfter.Type != NH_ACT_NONE ) {
+			const long long total = static_cast<long long>( args.M ) * args.N;
+			const long long blocksAct = ( total + 1023 ) / 1024;
+			hipLaunchKernelGGL( activateResultKernel, dim3( static_cast<unsigned>( blocksAct > 4096 ? 4096 : blocksAct ), nb ), dim3( 256 ), 0,
+				stream, a.C, args.M, args.N, args.Ldc, args.BatchStrideC, actAfter );
 		}
 	}
 	NH_LAUNCH_CHECK();
@@ -875,9 +898,10 @@ int matMulTN( hipStream_t stream, const float* a, int lda, const float* b, int l
 }
 
 int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* source, const float* filter,
-	const float* freeTerm, float* result )
+	const float* freeTerm, float* result, const CFusedActivation& act )
 {
 	CMatMulArgs args = {};
+	args.Act = act;
 	args.A = source; args.B = filter; args.C = result; args.Bias = freeTerm;
 	const long long m = static_cast<long long>( d.batch ) * d.resultHeight * d.resultWidth;
 	args.M = static_cast<int>( m );
@@ -899,8 +923,8 @@ int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* sour
 		&& d.paddingHeight == 0 && d.paddingWidth == 0 )
 	{
 		// a pointwise convolution over a channels-last image is the plain product image[M x Cin] * filter[Cout x Cin]^T
-		return matMulNT( stream, source, d.channels, filter, d.channels, result, d.filterCount, args.M, args.N, d.channels,
-			1, 0, 0, 0, freeTerm, false );
+		return matMulNTFused( stream, source, d.channels, filter, d.channels, result, d.filterCount, args.M, args.N, d.channels,
+			1, 0, 0, 0, freeTerm, false, act, nullptr );
 	}
 	if( d.filterHeight == 1 && d.filterWidth == 1 ) {
 		return launchMatMul<AM_Conv1x1, BM_RowsK>( stream, args, 1, vec );
@@ -1015,6 +1039,12 @@ int nhInitBlobConvolution( nhConvDesc* d )
 int nhBlobConvolution( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
 	const float* freeTerm, float* result )
 {
+	return nhBlobConvolutionWithActivation( s, d, source, filter, freeTerm, NH_ACT_NONE, 0.f, result );
+}
+
+int nhBlobConvolutionWithActivation( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
+	const float* freeTerm, int activation, float param, float* result )
+{
 	NH_REQUIRE( d != nullptr && source != nullptr && filter != nullptr && result != nullptr );
 	nhConvDesc check = *d;
 	const int rc = nhInitBlobConvolution( &check );
@@ -1022,7 +1052,8 @@ int nhBlobConvolution( nhStream s, const nhConvDesc* d, const float* source, con
 		return rc;
 	}
 	NH_REQUIRE( check.resultHeight == d->resultHeight && check.resultWidth == d->resultWidth );
-	return convImplicitGemm( toStream( s ), *d, source, filter, freeTerm, result );
+	const CFusedActivation act = { activation, param };
+	return convImplicitGemm( toStream( s ), *d, source, filter, freeTerm, result, act );
 }
 
 } // extern "C"

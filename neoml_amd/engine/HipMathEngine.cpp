@@ -540,6 +540,15 @@ void CHipMathEngine::BlobConvolution( const CConvolutionDesc& desc, const CConst
 		freeTerm != nullptr ? raw( *freeTerm ) : nullptr, raw( result ) ) );
 }
 
+void CHipMathEngine::BlobConvolutionWithActivation( const CConvolutionDesc& desc, const CConstFloatHandle& source,
+	const CConstFloatHandle& filter, const CConstFloatHandle* freeTerm, int activation, float param,
+	const CFloatHandle& result )
+{
+	const CHipConvolutionDesc& d = static_cast<const CHipConvolutionDesc&>( desc );
+	NH_CALL( nhBlobConvolutionWithActivation( stream, &d.D, raw( source ), raw( filter ),
+		freeTerm != nullptr ? raw( *freeTerm ) : nullptr, activation, param, raw( result ) ) );
+}
+
 CChannelwiseConvolutionDesc* CHipMathEngine::InitBlobChannelwiseConvolution( const CBlobDesc& input, int paddingHeight,
 	int paddingWidth, int strideHeight, int strideWidth, const CBlobDesc& filter, const CBlobDesc* freeTerm,
 	const CBlobDesc& output )

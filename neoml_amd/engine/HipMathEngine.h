@@ -242,6 +242,10 @@ public:
 		const CBlobDesc& input ) override;
 	void RowwiseExecute( const CBlobDesc& inputDesc, CRowwiseOperationDesc** operations, int operationCount,
 		const CFloatHandle& input, const CFloatHandle& output ) override;
+	// BlobConvolution with NH_ACT_RELU / NH_ACT_HSWISH applied by the same launch (rowwise chains pair them)
+	void BlobConvolutionWithActivation( const CConvolutionDesc& desc, const CConstFloatHandle& source,
+		const CConstFloatHandle& filter, const CConstFloatHandle* freeTerm, int activation, float param,
+		const CFloatHandle& result );
 	// runs a CHipRowwiseSeparableBlock (either MobileNet block) on whole blobs
 	void RunSeparableBlock( const CRowwiseOperationDesc& block, const CConstFloatHandle& input, const CFloatHandle& output );
 

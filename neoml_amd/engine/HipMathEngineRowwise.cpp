@@ -123,11 +123,18 @@ struct CHipRowwiseConv : public IHipRowwiseOperation {
 	int OutputSize() const override { return Output.BlobSize(); }
 	void Process( CHipMathEngine& engine, const CConstFloatHandle& input, const CFloatHandle& output ) override
 	{
+		ProcessWithActivation( engine, input, output, NH_ACT_NONE, 0.f );
+	}
+	// the convolution and the ReLU / h-swish that follows it in the chain as one launch
+	void ProcessWithActivation( CHipMathEngine& engine, const CConstFloatHandle& input, const CFloatHandle& output,
+		int activation, float param )
+	{
 		if( Desc == nullptr ) {
 			Desc.reset( engine.InitBlobConvolution( Input, PaddingHeight, PaddingWidth, StrideHeight, StrideWidth,
 				DilationHeight, DilationWidth, FilterDesc, Output ) );
 		}
-		engine.BlobConvolution( *Desc, input, Filter, FreeTerm.IsNull() ? nullptr : &FreeTerm, output );
+		engine.BlobConvolutionWithActivation( *Desc, input, Filter, FreeTerm.IsNull() ? nullptr : &FreeTerm, activation,
+			param, output );
 	}
 };
 
@@ -438,8 +445,19 @@ void CHipMathEngine::RowwiseExecute( const CBlobDesc& /*inputDesc*/, CRowwiseOpe
 			}
 			target = buffer->GetHandle();
 		}
-		stages[i][0]->Process( *this, current, target );
-		for( size_t j = 1; j < stages[i].size(); ++j ) {
+		size_t next = 1;
+		CHipRowwiseConv* conv = dynamic_cast<CHipRowwiseConv*>( stages[i][0] );
+		CHipRowwiseActivation* activation = stages[i].size() > 1 ? dynamic_cast<CHipRowwiseActivation*>( stages[i][1] ) : nullptr;
+		if( conv != nullptr && activation != nullptr && fusedActivation( activation->Desc.GetType() ) != NH_ACT_NONE ) {
+			// convolution + ReLU / h-swish: the activation rides in the epilogue of the convolution
+			const float param = activation->Desc.GetType() == AF_ReLU
+				? activation->Desc.GetParam<CReLUActivationParam>().UpperThreshold : 0.f;
+			conv->ProcessWithActivation( *this, current, target, fusedActivation( activation->Desc.GetType() ), param );
+			next = 2;
+		} else {
+			stages[i][0]->Process( *this, current, target );
+		}
+		for( size_t j = next; j < stages[i].size(); ++j ) {
 			stages[i][j]->Process( *this, target, target );
 		}
 		current = target;

@@ -695,14 +695,18 @@ class Hip:
         self.na.check(fn(ctypes.byref(d)))
         return d
 
-    def conv(self, x, filt, bias, ph, pw, sh, sw, dh=1, dw=1):
+    def conv(self, x, filt, bias, ph, pw, sh, sw, dh=1, dw=1, activation=None, param=0.0):
         x, filt = f32(x), f32(filt)
         n, h, w, cin = x.shape
         cout, fh, fw, _ = filt.shape
         d = self.conv_desc(n, h, w, cin, cout, fh, fw, ph, pw, sh, sw, dh, dw)
         xs, fs, bs = self.up(x), self.up(filt), self.up(None if bias is None else f32(bias))
         out = self.empty((n, d.resultHeight, d.resultWidth, cout))
-        self.call("nhBlobConvolution", ctypes.byref(d), self.p(xs), self.p(fs), self.p(bs), self.p(out))
+        if activation is None:
+            self.call("nhBlobConvolution", ctypes.byref(d), self.p(xs), self.p(fs), self.p(bs), self.p(out))
+        else:
+            self.call("nhBlobConvolutionWithActivation", ctypes.byref(d), self.p(xs), self.p(fs), self.p(bs),
+                      Cpu.ACTIVATIONS[activation], param, self.p(out))
         return self.down(out)
 
     def channelwise_conv(self, x, filt, bias, ph, pw, sh, sw):

@@ -245,3 +245,28 @@ def test_optimized_separable_network_on_hip_engine():
     blocks, with1x1, chains = last_optimization()
     assert blocks == 2 and with1x1 >= 1 and chains >= 1  # (the 1x1 pass also counts the pairs inside the two blocks)
     assert_close(got, want, "optimized network on CHipMathEngine vs plain network on CCpuMathEngine")
+
+
+@pytest.mark.gpu
+def test_optimized_resnet18_through_cdnn_at_benchmark_size(capsys):
+    """The benchmark network after NeoML's OptimizeDnn: its convolution + ReLU pairs become rowwise operation chains,
+    which the engine runs as one launch per pair. Same result as the plain network; time per CDnn::RunOnce printed."""
+    dims = (1, 64, 1, 224, 224, 1, 3)
+    g = np.random.default_rng(0xC0FFEE + 102)
+    x = g.uniform(0, 1, dims).astype(np.float32)
+    lib().dnn_last_pass_ms.restype = ctypes.c_double
+    lib().dnn_set_timed_passes(20)
+    try:
+        plain = dnn_run(nhtest.hip_engine(), 5, dims, x, 1000).reshape(64, 1000)
+        plain_ms = lib().dnn_last_pass_ms()
+        with optimized():
+            fused = dnn_run(nhtest.hip_engine(), 5, dims, x, 1000).reshape(64, 1000)
+            fused_ms = lib().dnn_last_pass_ms()
+    finally:
+        lib().dnn_set_timed_passes(0)
+    chains = last_optimization()[2]
+    with capsys.disabled():
+        print("\nResNet-18-style, batch 64, CDnn::RunOnce on CHipMathEngine: plain layers %.3f ms, after OptimizeDnn "
+              "(%d rowwise chains) %.3f ms = %.0f images/sec" % (plain_ms, chains, fused_ms, 64e3 / fused_ms))
+    assert chains >= 1
+    assert_close(fused, plain, "optimized vs plain ResNet-18 on the HIP engine")

@@ -252,6 +252,26 @@ def test_convolution(case):
     assert_close(hip().conv(x, f, None, ph, pw, sh, sw, dh, dw), orc.conv(x, f, None, ph, pw, sh, sw, dh, dw), "conv, no free term")
 
 
+@pytest.mark.parametrize("case", [
+    (2, 16, 16, 64, 64, 3, 3, 1, 1, 1, 1, 1, 1),     # whole tiles, activation in the epilogue
+    (1, 7, 7, 512, 96, 3, 3, 1, 1, 1, 1, 1, 1),      # few tiles, long reduction: K slices, activation as a pass of its own
+    (3, 9, 9, 128, 200, 1, 1, 0, 0, 1, 1, 1, 1),     # 1x1 through the matrix-product path
+    (2, 32, 32, 3, 64, 7, 7, 3, 3, 2, 2, 1, 1),      # stem
+    (4, 64, 64, 24, 144, 1, 1, 0, 0, 1, 1, 1, 1),    # the row-resident pointwise kernel
+])
+@pytest.mark.parametrize("activation,param", [("relu", 0.0), ("relu", 0.5), ("hswish", 0.0)])
+def test_convolution_with_activation(case, activation, param):
+    n, h, w, cin, cout, fh, fw, ph, pw, sh, sw, dh, dw = case
+    g = rng(310 + cin + fh)
+    x = g.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    f = g.normal(0, 1.0 / np.sqrt(fh * fw * cin), (cout, fh, fw, cin)).astype(np.float32)
+    bias = g.uniform(-1, 1, cout).astype(np.float32)
+    plain = orc.conv(x, f, bias, ph, pw, sh, sw, dh, dw)
+    want = orc.unary(activation, plain, param).reshape(plain.shape)
+    got = hip().conv(x, f, bias, ph, pw, sh, sw, dh, dw, activation=activation, param=param)
+    assert_close(got, want, "conv + %s %s" % (activation, case))
+
+
 def test_convolution_ignores_pixels_outside_the_windows():
     # stride 4 with a 3-wide filter never touches image columns 3 and 7; whatever they hold (here: infinities)
     # must not leak into the result through the vector fetches that run past a window's last value
