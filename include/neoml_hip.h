@@ -144,6 +144,17 @@ NH_API int nhVectorMinMax(nhStream s, const float* first, float* result, int vec
 	const float* minValue, const float* maxValue);                                                   /* NME.h:305 */
 NH_API int nhVectorSigmoid(nhStream s, const float* first, float* result, int vectorSize);           /* NME.h:311 */
 NH_API int nhVectorTanh(nhStream s, const float* first, float* result, int vectorSize);              /* NME.h:319 */
+
+/* ---- derivatives of the activations, backward pass: result = f'(first) * second; the ...DiffOp forms take the
+ * activation's OUTPUT as first (NME.h:146-149, 164, 225, 313-325). upperThreshold: device scalar, as for nhVectorReLU */
+NH_API int nhVectorNegLog(nhStream s, const float* first, float* result, int vectorSize);            /* NME.h:225 */
+NH_API int nhVectorReLUDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize,
+	const float* upperThreshold);                                                                    /* NME.h:146,148 */
+NH_API int nhVectorHSwishDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize);   /* NME.h:164 */
+NH_API int nhVectorSigmoidDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize);  /* NME.h:313 */
+NH_API int nhVectorSigmoidDiffOp(nhStream s, const float* first, const float* second, float* result, int vectorSize); /* NME.h:316 */
+NH_API int nhVectorTanhDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize);     /* NME.h:321 */
+NH_API int nhVectorTanhDiffOp(nhStream s, const float* first, const float* second, float* result, int vectorSize);   /* NME.h:324 */
 NH_API int nhVectorSum(nhStream s, const float* first, int vectorSize, float* result);               /* NME.h:105 */
 NH_API int nhVectorDotProduct(nhStream s, const float* first, const float* second, int vectorSize, float* result); /* NME.h:339 */
 
@@ -237,6 +248,18 @@ NH_API int nhInitBlobConvolution(nhConvDesc* desc_host);
 NH_API int nhBlobConvolution(nhStream s, const nhConvDesc* desc_host, const float* source, const float* filter,
 	const float* freeTerm, float* result);                                                           /* NME.h:755 */
 
+/* Gradients of the convolution (NME.h:757-761), same descriptor as the forward pass.
+ * Backward: inputDiff = the gradient by the source; freeTerm (per source channel, may be null) is added, as the
+ * reference does for the layers that run a convolution backwards as their forward pass. workspace: the filter with its
+ * channel axes swapped, nhBlobConvolutionBackwardWorkspaceSize bytes.
+ * LearnAdd: filterDiff += the gradient by the filter. The gradient by the free term is a column sum of outputDiff
+ * (nhSumMatrixRowsAdd over [pixels x filterCount]). */
+NH_API int nhBlobConvolutionBackwardWorkspaceSize(const nhConvDesc* desc_host, size_t* bytes);
+NH_API int nhBlobConvolutionBackward(nhStream s, const nhConvDesc* desc_host, const float* outputDiff,
+	const float* filter, const float* freeTerm, float* inputDiff, void* workspace, size_t workspaceSize); /* NME.h:757 */
+NH_API int nhBlobConvolutionLearnAdd(nhStream s, const nhConvDesc* desc_host, const float* input,
+	const float* outputDiff, float* filterDiff);                                                     /* NME.h:759 */
+
 /* depthwise: filter [fh][fw][C], no dilation (src/MathEngineDnnConv.h:69-90) */
 NH_API int nhInitBlobChannelwiseConvolution(nhConvDesc* desc_host);                                  /* NME.h:766 */
 NH_API int nhBlobChannelwiseConvolution(nhStream s, const nhConvDesc* desc_host, const float* source,
@@ -289,6 +312,12 @@ NH_API int nhInitPooling(nhPoolingDesc* desc_host);                             
 NH_API int nhBlobMaxPooling(nhStream s, const nhPoolingDesc* desc_host, const float* source, int* maxIndices,
 	float* result);                                                                                  /* NME.h:821 */
 NH_API int nhBlobMeanPooling(nhStream s, const nhPoolingDesc* desc_host, const float* source, float* result); /* NME.h:841 */
+/* backward passes (NME.h:823-824, 842): sourceDiff receives the gradient by the pooling input; maxIndices are the
+ * ones the forward pass wrote */
+NH_API int nhBlobMaxPoolingBackward(nhStream s, const nhPoolingDesc* desc_host, const float* resultDiff,
+	const int* maxIndices, float* sourceDiff);                                                       /* NME.h:823 */
+NH_API int nhBlobMeanPoolingBackward(nhStream s, const nhPoolingDesc* desc_host, const float* resultDiff,
+	float* sourceDiff);                                                                              /* NME.h:842 */
 
 /* LSTM (NME.h:1005-1011). Weights: inputWeights [4H x objectSize], recurrentWeights [4H x H]; gate order in
  * the 4H vector: main(tanh) | forget | input | output (src/CPU/CpuMathEngineDnnLstm.h:49-90).

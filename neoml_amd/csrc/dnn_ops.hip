@@ -940,6 +940,46 @@ __global__ __launch_bounds__( 256 ) void clearWordsKernel( unsigned long long* w
 	}
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Pooling, backward. Max: every output element sends its gradient to the input element its index names (index
+// inside the image, as the forward pass wrote it); overlapping windows may name the same element, so the sums meet
+// through atomic adds in a zeroed blob. Mean: every input element gathers the gradients of the windows that cover
+// it, times 1 / fh / fw.
+__global__ __launch_bounds__( 256 )
+void maxPoolingBackwardKernel( const float* resultDiff, const int* maxIndices, float* sourceDiff, long long total,
+	int resultObjectSize, int sourceObjectSize )
+{
+	for( long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += static_cast<long long>( gridDim.x ) * 256 ) {
+		const long long object = i / resultObjectSize;
+		unsafeAtomicAdd( sourceDiff + object * sourceObjectSize + maxIndices[i], resultDiff[i] );
+	}
+}
+
+__global__ __launch_bounds__( 256 )
+void meanPoolingBackwardKernel( const nhPoolingDesc d, const float* resultDiff, float* sourceDiff, long long total )
+{
+	const float scale = 1.f / d.filterHeight / d.filterWidth;
+	for( long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += static_cast<long long>( gridDim.x ) * 256 ) {
+		long long t = i;
+		const int c = static_cast<int>( t % d.channels ); t /= d.channels;
+		const int wi = static_cast<int>( t % d.width ); t /= d.width;
+		const int hi = static_cast<int>( t % d.height );
+		const long long n = t / d.height;
+		// windows ho with ho * s <= hi < ho * s + fh
+		const int hoFirst = hi >= d.filterHeight ? ( hi - d.filterHeight ) / d.strideHeight + 1 : 0;
+		const int hoLast = min( hi / d.strideHeight, d.resultHeight - 1 );
+		const int woFirst = wi >= d.filterWidth ? ( wi - d.filterWidth ) / d.strideWidth + 1 : 0;
+		const int woLast = min( wi / d.strideWidth, d.resultWidth - 1 );
+		float sum = 0.f;
+		for( int ho = hoFirst; ho <= hoLast; ++ho ) {
+			for( int wo = woFirst; wo <= woLast; ++wo ) {
+				sum += resultDiff[( ( n * d.resultHeight + ho ) * d.resultWidth + wo ) * d.channels + c];
+			}
+		}
+		sourceDiff[i] = sum * scale;
+	}
+}
+
 __global__ void addTwoVectorsKernel( const float* a, const float* b, float* out, int n )
 {
 	const int i = blockIdx.x * 256 + threadIdx.x;
@@ -1260,6 +1300,52 @@ int nhBlobMaxPooling( nhStream s, const nhPoolingDesc* d, const float* source, i
 	blocks = blocks > 1048576 ? 1048576 : blocks;
 	hipLaunchKernelGGL( maxPoolingIndexKernel, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
 		*d, source, maxIndices, result, total );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+int nhBlobMaxPoolingBackward( nhStream s, const nhPoolingDesc* d, const float* resultDiff, const int* maxIndices,
+	float* sourceDiff )
+{
+	const int rc = checkPoolingDesc( d );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( resultDiff != nullptr && maxIndices != nullptr && sourceDiff != nullptr );
+	const int sourceObjectSize = d->height * d->width * d->channels;
+	const int resultObjectSize = d->resultHeight * d->resultWidth * d->channels;
+	const long long sourceTotal = static_cast<long long>( d->batch ) * sourceObjectSize;
+	const long long total = static_cast<long long>( d->batch ) * resultObjectSize;
+	if( sourceTotal == 0 ) {
+		return NH_OK;
+	}
+	NH_HIP( hipMemsetAsync( sourceDiff, 0, sourceTotal * sizeof( float ), toStream( s ) ) );
+	if( total == 0 ) {
+		return NH_OK;
+	}
+	long long blocks = ( total + 255 ) / 256;
+	blocks = blocks > 1048576 ? 1048576 : blocks;
+	hipLaunchKernelGGL( maxPoolingBackwardKernel, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+		resultDiff, maxIndices, sourceDiff, total, resultObjectSize, sourceObjectSize );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+int nhBlobMeanPoolingBackward( nhStream s, const nhPoolingDesc* d, const float* resultDiff, float* sourceDiff )
+{
+	const int rc = checkPoolingDesc( d );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( resultDiff != nullptr && sourceDiff != nullptr );
+	const long long total = static_cast<long long>( d->batch ) * d->height * d->width * d->channels;
+	if( total == 0 ) {
+		return NH_OK;
+	}
+	long long blocks = ( total + 255 ) / 256;
+	blocks = blocks > 1048576 ? 1048576 : blocks;
+	hipLaunchKernelGGL( meanPoolingBackwardKernel, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+		*d, resultDiff, sourceDiff, total );
 	NH_LAUNCH_CHECK();
 	return NH_OK;
 }

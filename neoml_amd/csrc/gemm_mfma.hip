@@ -40,7 +40,9 @@ typedef float f32x16 __attribute__( ( ext_vector_type( 16 ) ) );
 // contiguous in a channels-last image (no dilation along the width), so they are fetched as 128-bit runs however
 // Cin divides; the 1-3 padding values per row are masked to zero on both operands.
 enum TAMode { AM_RowsK = 0, AM_RowsM = 1, AM_Conv = 2, AM_Conv1x1 = 3, AM_ConvRows = 4 };
-enum TBMode { BM_RowsK = 0, BM_RowsN = 1 };
+// BM_ConvN: B is the im2col view of an N,H,W,C image read N-major: row k = output pixel, column n = ( kh, kw, ci ).
+// With A = the gradient by the convolution's output read M-major this is the gradient by the filter.
+enum TBMode { BM_RowsK = 0, BM_RowsN = 1, BM_ConvN = 2 };
 
 struct CMatMulArgs {
 	const float* A;
@@ -57,6 +59,10 @@ struct CMatMulArgs {
 	// convolution geometry (AM_Conv only): A is the image, M = batch * Ho * Wo
 	int H, W, Cin, Ho, Wo, Fh, Fw, PadH, PadW, StrideH, StrideW, DilH, DilW;
 	int RowK, RowPitch; // AM_ConvRows: Fw * Cin and its round-up to a multiple of 4; K = Fh * RowPitch
+	// AM_Conv as the gradient by the input of a strided convolution: the tap's source coordinate is
+	// ( ho * StrideH - PadH + kh * DilH ) / UpH and only exists where that division is exact (values <= 1: no division)
+	int UpH, UpW;
+	int ManySlices; // the reduction is far longer than the output is large: as many K slices as fill the device
 	// epilogue of the fused blocks: C = act( A * B + bias ) + Residual; Residual has C's layout, may be C itself
 	CFusedActivation Act;
 	const float* Residual;
@@ -126,9 +132,15 @@ void matMulKernel( const CMatMulArgs args )
 	int convCi = 0, convKh = 0, convKw = 0;
 
 	auto convSlotOffset = [&]( int i ) -> unsigned {
-		const int hi = convH0[i] + convKh * args.DilH;
-		const int wi = convW0[i] + convKw * args.DilW;
-		const bool ok = convKh < args.Fh && hi >= 0 && hi < args.H && wi >= 0 && wi < args.W;
+		int hi = convH0[i] + convKh * args.DilH;
+		int wi = convW0[i] + convKw * args.DilW;
+		bool ok = convKh < args.Fh;
+		if( args.UpH > 1 || args.UpW > 1 ) {
+			ok = ok && hi >= 0 && wi >= 0 && hi % args.UpH == 0 && wi % args.UpW == 0;
+			hi /= args.UpH;
+			wi /= args.UpW;
+		}
+		ok = ok && hi >= 0 && hi < args.H && wi >= 0 && wi < args.W;
 		return ok ? static_cast<unsigned>( convPixel[i] + ( hi * args.W + wi ) * args.Cin + convCi ) * 4u : OutOfRange;
 	};
 
@@ -178,11 +190,30 @@ void matMulKernel( const CMatMulArgs args )
 			offA[i] = convSlotOffset( i );
 		}
 	}
+	// BM_ConvN: per slot, the tap of its four columns ( fixed for the whole launch ) and the output pixel of its row
+	// ( advances by KS pixels per K step )
+	int bDh[BSlots], bDw[BSlots], bCi[BSlots], bImg[BSlots], bHo[BSlots], bWo[BSlots];
+	long long bPixel[BSlots];
 #pragma unroll
 	for( int i = 0; i < BSlots; ++i ) {
 		const int slot = tid + i * Threads;
 		const bool inTile = BTotal % Threads == 0 || slot < BTotal;
-		if( BMODE == BM_RowsK ) {
+		if( BMODE == BM_ConvN ) {
+			const int n = n0 + ( slot % ( BN / 4 ) ) * 4;
+			const bool nOk = inTile && n < N;
+			const int tap = n / args.Cin;
+			bCi[i] = n - tap * args.Cin;
+			const int kh = tap / args.Fw;
+			bDh[i] = nOk ? kh * args.DilH - args.PadH : -0x40000000; // never inside the image
+			bDw[i] = ( tap - kh * args.Fw ) * args.DilW - args.PadW;
+			const long long pixel = static_cast<long long>( kStart ) + slot / ( BN / 4 );
+			bPixel[i] = pixel;
+			bWo[i] = static_cast<int>( pixel % args.Wo );
+			const long long t = pixel / args.Wo;
+			bHo[i] = static_cast<int>( t % args.Ho );
+			bImg[i] = static_cast<int>( t / args.Ho );
+			offB[i] = 0;
+		} else if( BMODE == BM_RowsK ) {
 			const int n = n0 + slot / KQ;
 			offB[i] = ( inTile && n < N ) ? static_cast<unsigned>( n * args.Ldb + kStart + ( slot % KQ ) * 4 ) * 4u : OutOfRange;
 		} else {
@@ -199,12 +230,40 @@ void matMulKernel( const CMatMulArgs args )
 		const int ci = k - tap * args.Cin;
 		const int kh = tap / args.Fw;
 		const int kw = tap - kh * args.Fw;
-		const int hi = convH0[i] + kh * args.DilH;
-		const int wi = convW0[i] + kw * args.DilW;
+		int hi = convH0[i] + kh * args.DilH;
+		int wi = convW0[i] + kw * args.DilW;
+		if( args.UpH > 1 || args.UpW > 1 ) {
+			if( hi < 0 || wi < 0 || hi % args.UpH != 0 || wi % args.UpW != 0 ) {
+				return 0.f;
+			}
+			hi /= args.UpH;
+			wi /= args.UpW;
+		}
 		if( hi < 0 || hi >= args.H || wi < 0 || wi >= args.W ) {
 			return 0.f;
 		}
 		return A[convPixel[i] + ( hi * args.W + wi ) * args.Cin + ci];
+	};
+
+	// im2col element ( output pixel, column n ) of the image B, zero outside (BM_ConvN, scalar path)
+	auto loadIm2colElement = [&]( long long pixel, int n ) -> float {
+		if( pixel >= K || n >= N ) {
+			return 0.f;
+		}
+		const int wo = static_cast<int>( pixel % args.Wo );
+		const long long t = pixel / args.Wo;
+		const int ho = static_cast<int>( t % args.Ho );
+		const long long img = t / args.Ho;
+		const int tap = n / args.Cin;
+		const int ci = n - tap * args.Cin;
+		const int kh = tap / args.Fw;
+		const int kw = tap - kh * args.Fw;
+		const int hi = ho * args.StrideH - args.PadH + kh * args.DilH;
+		const int wi = wo * args.StrideW - args.PadW + kw * args.DilW;
+		if( hi < 0 || hi >= args.H || wi < 0 || wi >= args.W ) {
+			return 0.f;
+		}
+		return B[( ( img * args.H + hi ) * args.W + wi ) * args.Cin + ci];
 	};
 
 	// Loads the tiles of the K step starting at kBase into registers and advances the slot offsets to the next step.
@@ -257,7 +316,7 @@ void matMulKernel( const CMatMulArgs args )
 		if( VEC ) {
 			// k of this thread's slots inside the step: fixed column of a K-major tile, fixed row of an X-major one
 			const bool kInA = AMODE == AM_RowsM ? true : ( kBase + ( tid % KQ ) * 4 < K );
-			const bool kInB = BMODE == BM_RowsN ? true : ( kBase + ( tid % KQ ) * 4 < K );
+			const bool kInB = BMODE != BM_RowsK ? true : ( kBase + ( tid % KQ ) * 4 < K );
 #pragma unroll
 			for( int i = 0; i < ASlots; ++i ) {
 				unsigned off = offA[i];
@@ -271,7 +330,22 @@ void matMulKernel( const CMatMulArgs args )
 #pragma unroll
 			for( int i = 0; i < BSlots; ++i ) {
 				unsigned off = offB[i];
-				if( BMODE == BM_RowsK ) {
+				if( BMODE == BM_ConvN ) {
+					const int hi = bHo[i] * args.StrideH + bDh[i];
+					const int wi = bWo[i] * args.StrideW + bDw[i];
+					const bool ok = bPixel[i] < K && hi >= 0 && hi < args.H && wi >= 0 && wi < args.W;
+					off = ok ? static_cast<unsigned>( ( ( bImg[i] * args.H + hi ) * args.W + wi ) * args.Cin + bCi[i] ) * 4u : OutOfRange;
+					// the row of this slot in the next K step
+					bPixel[i] += KS;
+					bWo[i] += KS;
+					while( bWo[i] >= args.Wo ) {
+						bWo[i] -= args.Wo;
+						if( ++bHo[i] == args.Ho ) {
+							bHo[i] = 0;
+							++bImg[i];
+						}
+					}
+				} else if( BMODE == BM_RowsK ) {
 					off = kInB ? off : OutOfRange;
 				} else {
 					off = ( kBase + ( tid + i * Threads ) / ( BN / 4 ) < K ) ? off : OutOfRange;
@@ -306,10 +380,12 @@ void matMulKernel( const CMatMulArgs args )
 					offA[i] += stepA;
 				}
 			}
-			const unsigned stepB = BMODE == BM_RowsK ? KS * 4u : static_cast<unsigned>( KS * args.Ldb ) * 4u;
+			if( BMODE != BM_ConvN ) {
+				const unsigned stepB = BMODE == BM_RowsK ? KS * 4u : static_cast<unsigned>( KS * args.Ldb ) * 4u;
 #pragma unroll
-			for( int i = 0; i < BSlots; ++i ) {
-				offB[i] += stepB;
+				for( int i = 0; i < BSlots; ++i ) {
+					offB[i] += stepB;
+				}
 			}
 			return;
 		}
@@ -364,6 +440,13 @@ void matMulKernel( const CMatMulArgs args )
 						if( k + 2 < K ) v.z = p[2];
 						if( k + 3 < K ) v.w = p[3];
 					}
+				} else if( BMODE == BM_ConvN ) {
+					const long long pixel = static_cast<long long>( kBase ) + slot / ( BN / 4 );
+					const int n = n0 + ( slot % ( BN / 4 ) ) * 4;
+					v.x = loadIm2colElement( pixel, n );
+					v.y = loadIm2colElement( pixel, n + 1 );
+					v.z = loadIm2colElement( pixel, n + 2 );
+					v.w = loadIm2colElement( pixel, n + 3 );
 				} else {
 					const int k = kBase + slot / ( BN / 4 );
 					const int n = n0 + ( slot % ( BN / 4 ) ) * 4;
@@ -601,8 +684,13 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 	const int totalSteps = ceilDiv( args.K, NH_KSTEP );
 	int splits = 1;
 	const long long blocks = tiles * batch;
+	if( args.ManySlices != 0 ) {
+		// a gradient by a filter: a few tiles, a reduction over every pixel of the batch
+		const long long fill = blocks >= 1280 ? 1 : 1280 / blocks;
+		const long long most = totalSteps / 8 > 0 ? totalSteps / 8 : 1;
+		splits = static_cast<int>( fill < most ? fill : most );
 	// K slices cannot add a residual; an activation follows them as a pass of its own
-	if( blocks < 1024 && totalSteps >= 32 && args.Residual == nullptr ) {
+	} else if( blocks < 1024 && totalSteps >= 32 && args.Residual == nullptr ) {
 		double best = 0;
 		for( int s = 1; s <= 8 && s <= totalSteps / 8; ++s ) {
 			const double rounds = static_cast<double>( blocks * s ) / 1280.0;
@@ -941,6 +1029,78 @@ int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* sour
 	return launchMatMul<AM_Conv, BM_RowsK>( stream, args, 1, vec );
 }
 
+// ---- gradients of the convolution ------------------------------------------------------------------------------
+
+// filter [Cout][taps][Cin] -> [Cin][taps][Cout]: the filter of the convolution that maps the output gradient back
+__global__ __launch_bounds__( 256 ) void swapFilterChannelsKernel( const float* filter, float* swapped, int cout, int taps, int cin )
+{
+	const int total = cout * taps * cin;
+	for( int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256 ) {
+		const int co = i % cout;
+		const int t = ( i / cout ) % taps;
+		const int ci = i / ( cout * taps );
+		swapped[i] = filter[( co * taps + t ) * cin + ci];
+	}
+}
+
+// inputDiff[n,hi,wi,ci] = freeTerm[ci] + sum over ( kh, kw, co ) of outputDiff[n, (hi+p-kh*d)/s, (wi+p-kw*d)/s, co] *
+// filter[co,kh,kw,ci], the terms whose divisions are exact and in range: the forward kernel on the output gradient as
+// its image, with padding -p, dilation -d, the division by the stride, and the filter with its channel axes swapped.
+int convBackwardData( hipStream_t stream, const nhConvDesc& d, const float* outputDiff, const float* filter,
+	const float* freeTerm, float* inputDiff, float* swappedFilter )
+{
+	const int taps = d.filterHeight * d.filterWidth;
+	const int filterSize = d.filterCount * taps * d.channels;
+	hipLaunchKernelGGL( swapFilterChannelsKernel, dim3( ceilDiv( filterSize, 1024 ) ), dim3( 256 ), 0, stream,
+		filter, swappedFilter, d.filterCount, taps, d.channels );
+	CMatMulArgs args = {};
+	args.A = outputDiff; args.B = swappedFilter; args.C = inputDiff; args.Bias = freeTerm;
+	const long long m = static_cast<long long>( d.batch ) * d.height * d.width;
+	args.M = static_cast<int>( m );
+	args.N = d.channels;
+	args.K = taps * d.filterCount;
+	args.Lda = 0; args.Ldb = args.K; args.Ldc = d.channels;
+	args.H = d.resultHeight; args.W = d.resultWidth; args.Cin = d.filterCount;
+	args.Ho = d.height; args.Wo = d.width; args.Fh = d.filterHeight; args.Fw = d.filterWidth;
+	args.PadH = -d.paddingHeight; args.PadW = -d.paddingWidth;
+	args.StrideH = 1; args.StrideW = 1;
+	args.DilH = -d.dilationHeight; args.DilW = -d.dilationWidth;
+	args.UpH = d.strideHeight; args.UpW = d.strideWidth;
+	if( args.M == 0 || args.N == 0 ) {
+		return NH_OK;
+	}
+	const bool vec = isAligned16( outputDiff ) && isAligned16( swappedFilter ) && d.filterCount % 4 == 0
+		&& fitsBuffer( 1, 0, static_cast<long long>( d.batch ) * d.resultHeight * d.resultWidth * d.filterCount )
+		&& fitsBuffer( d.channels, args.K, args.K );
+	return launchMatMul<AM_Conv, BM_RowsK>( stream, args, 1, vec );
+}
+
+// filterDiff[co][kh,kw,ci] += sum over output pixels of outputDiff[pixel][co] * im2col( input )[pixel][kh,kw,ci]
+int convLearnAdd( hipStream_t stream, const nhConvDesc& d, const float* input, const float* outputDiff, float* filterDiff )
+{
+	CMatMulArgs args = {};
+	args.A = outputDiff; args.B = input; args.C = filterDiff;
+	const long long pixels = static_cast<long long>( d.batch ) * d.resultHeight * d.resultWidth;
+	args.M = d.filterCount;
+	args.N = d.filterHeight * d.filterWidth * d.channels;
+	args.K = static_cast<int>( pixels );
+	args.Lda = d.filterCount; args.Ldb = 0; args.Ldc = args.N;
+	args.H = d.height; args.W = d.width; args.Cin = d.channels;
+	args.Ho = d.resultHeight; args.Wo = d.resultWidth; args.Fh = d.filterHeight; args.Fw = d.filterWidth;
+	args.PadH = d.paddingHeight; args.PadW = d.paddingWidth;
+	args.StrideH = d.strideHeight; args.StrideW = d.strideWidth;
+	args.DilH = d.dilationHeight; args.DilW = d.dilationWidth;
+	args.Accumulate = 1;
+	args.ManySlices = 1;
+	if( args.M == 0 || args.N == 0 || args.K == 0 ) {
+		return NH_OK;
+	}
+	const bool vec = isAligned16( outputDiff ) && isAligned16( input ) && d.filterCount % 4 == 0 && d.channels % 4 == 0
+		&& fitsBuffer( pixels, d.filterCount, d.filterCount )
+		&& fitsBuffer( 1, 0, static_cast<long long>( d.batch ) * d.height * d.width * d.channels );
+	return launchMatMul<AM_RowsM, BM_ConvN>( stream, args, 1, vec );
+}
+
 } // namespace nh
 
 // ---------------------------------------------------------------------------------------------------------
@@ -1034,6 +1194,53 @@ int nhInitBlobConvolution( nhConvDesc* d )
 	NH_REQUIRE( static_cast<long long>( d->batch ) * d->height * d->width * d->channels <= 0x7fffffffLL );
 	NH_REQUIRE( m * d->filterCount <= 0x7fffffffLL );
 	return NH_OK;
+}
+
+static int checkedConvDesc( const nhConvDesc* d )
+{
+	NH_REQUIRE( d != nullptr );
+	nhConvDesc check = *d;
+	const int rc = nhInitBlobConvolution( &check );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( check.resultHeight == d->resultHeight && check.resultWidth == d->resultWidth );
+	return NH_OK;
+}
+
+int nhBlobConvolutionBackwardWorkspaceSize( const nhConvDesc* d, size_t* bytes )
+{
+	const int rc = checkedConvDesc( d );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( bytes != nullptr );
+	*bytes = static_cast<size_t>( d->filterCount ) * d->filterHeight * d->filterWidth * d->channels * sizeof( float );
+	return NH_OK;
+}
+
+int nhBlobConvolutionBackward( nhStream s, const nhConvDesc* d, const float* outputDiff, const float* filter,
+	const float* freeTerm, float* inputDiff, void* workspace, size_t workspaceSize )
+{
+	size_t need = 0;
+	const int rc = nhBlobConvolutionBackwardWorkspaceSize( d, &need );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( outputDiff != nullptr && filter != nullptr && inputDiff != nullptr );
+	NH_REQUIRE( workspace != nullptr && workspaceSize >= need && isAligned16( workspace ) );
+	NH_REQUIRE( static_cast<long long>( d->filterCount ) * d->filterHeight * d->filterWidth * d->channels <= 0x7fffffffLL );
+	return convBackwardData( toStream( s ), *d, outputDiff, filter, freeTerm, inputDiff, static_cast<float*>( workspace ) );
+}
+
+int nhBlobConvolutionLearnAdd( nhStream s, const nhConvDesc* d, const float* input, const float* outputDiff, float* filterDiff )
+{
+	const int rc = checkedConvDesc( d );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( input != nullptr && outputDiff != nullptr && filterDiff != nullptr );
+	return convLearnAdd( toStream( s ), *d, input, outputDiff, filterDiff );
 }
 
 int nhBlobConvolution( nhStream s, const nhConvDesc* d, const float* source, const float* filter,

@@ -258,6 +258,50 @@ struct CTanhOp : CNoScalar {
 	__device__ float operator()( float a, float, float ) const { return tanhf( a ); }
 };
 
+// ---- derivatives of the activations (backward pass): result = f'( first ) * second, or, for the ...DiffOp forms,
+// the same derivative expressed through the activation's OUTPUT given as first
+struct CNegLogOp : CNoScalar {
+	// -log( clamp( x, FLT_MIN, FLT_MAX ) ): VectorLog with the sign flipped (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:1692-1720)
+	__device__ float operator()( float a, float, float ) const
+	{
+		float x = a > FLT_MIN ? a : FLT_MIN;
+		x = x < FLT_MAX ? x : FLT_MAX;
+		return -logf( x );
+	}
+};
+struct CReLUDiffOp {
+	// second where 0 < first ( < threshold when the threshold is positive ), else 0; the same expression serves the
+	// input and the output form (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:339-395)
+	const float* Ptr; float Threshold;
+	__device__ void prepare() { Threshold = *Ptr; }
+	__device__ float operator()( float a, float b, float ) const
+	{
+		const bool pass = a > 0.f && ( Threshold <= 0.f || a < Threshold );
+		return pass ? b : 0.f;
+	}
+};
+struct CHSwishDiffOp : CNoScalar {
+	// 0 below -3, second above 3, second * ( first / 3 + 1/2 ) between (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:433-480)
+	__device__ float operator()( float a, float b, float ) const
+	{
+		if( !( -3.f < a ) ) return 0.f;
+		return a < 3.f ? b * ( a * ( 1.f / 3.f ) + 0.5f ) : b;
+	}
+};
+struct CSigmoidDiffOp : CNoScalar {
+	// second / ( 2 + e + 1 / e ), e = clamped exp( -first ) (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:1377-1412)
+	__device__ float operator()( float a, float b, float ) const
+	{
+		const float e = expClamped( -a );
+		return b / ( 2.f + e + 1.f / e );
+	}
+};
+struct CSigmoidDiffOutOp : CNoScalar { __device__ float operator()( float y, float b, float ) const { return y * ( 1.f - y ) * b; } };
+struct CTanhDiffOp : CNoScalar {
+	__device__ float operator()( float a, float b, float ) const { const float t = tanhf( a ); return b * ( 1.f - t * t ); }
+};
+struct CTanhDiffOutOp : CNoScalar { __device__ float operator()( float y, float b, float ) const { return ( 1.f - y * y ) * b; } };
+
 // ---- reductions to one value: one workgroup per 16K elements, atomics into a zeroed result -----------------
 
 template<bool DOT>
@@ -374,6 +418,21 @@ NH_UNARY( nhVectorSqrt, CSqrtOp )
 NH_UNARY( nhVectorInv, CInvOp )
 NH_UNARY( nhVectorSigmoid, CSigmoidOp )
 NH_UNARY( nhVectorTanh, CTanhOp )
+
+NH_UNARY( nhVectorNegLog, CNegLogOp )
+NH_BINARY( nhVectorHSwishDiff, float, CHSwishDiffOp )
+NH_BINARY( nhVectorSigmoidDiff, float, CSigmoidDiffOp )
+NH_BINARY( nhVectorSigmoidDiffOp, float, CSigmoidDiffOutOp )
+NH_BINARY( nhVectorTanhDiff, float, CTanhDiffOp )
+NH_BINARY( nhVectorTanhDiffOp, float, CTanhDiffOutOp )
+
+extern "C" int nhVectorReLUDiff( nhStream s, const float* first, const float* second, float* result, int vectorSize,
+	const float* upperThreshold )
+{
+	NH_REQUIRE( upperThreshold != nullptr );
+	CReLUDiffOp op; op.Ptr = upperThreshold; op.Threshold = 0;
+	return launchEltwise<2, float, float>( s, first, second, (const float*)nullptr, result, vectorSize, op );
+}
 
 NH_BINARY( nhVectorEltwiseMax, float, CMaxOp )
 NH_BINARY( nhVectorEltwiseMin, float, CMinOp )

@@ -225,6 +225,8 @@ HIP_UNARY( VectorInv, nhVectorInv )
 HIP_UNARY( VectorSigmoid, nhVectorSigmoid )
 HIP_UNARY( VectorTanh, nhVectorTanh )
 
+HIP_UNARY( VectorNegLog, nhVectorNegLog )
+
 HIP_UNARY_SCALAR( VectorELU, nhVectorELU )
 HIP_UNARY_SCALAR( VectorReLU, nhVectorReLU )
 HIP_UNARY_SCALAR( VectorLeakyReLU, nhVectorLeakyReLU )
@@ -243,6 +245,28 @@ HIP_BINARY( VectorEltwiseMultiply, CIntHandle, CConstIntHandle, nhVectorEltwiseM
 HIP_BINARY( VectorEltwiseMultiplyAdd, CFloatHandle, CConstFloatHandle, nhVectorEltwiseMultiplyAdd )
 HIP_BINARY( VectorEltwiseNegMultiply, CFloatHandle, CConstFloatHandle, nhVectorEltwiseNegMultiply )
 HIP_BINARY( VectorEltwiseDivide, CFloatHandle, CConstFloatHandle, nhVectorEltwiseDivide )
+
+// derivatives of the activations: result = f'( first ) * second; the Op forms take the activation's output as first
+HIP_BINARY( VectorHSwishDiff, CFloatHandle, CConstFloatHandle, nhVectorHSwishDiff )
+HIP_BINARY( VectorSigmoidDiff, CFloatHandle, CConstFloatHandle, nhVectorSigmoidDiff )
+HIP_BINARY( VectorSigmoidDiffOp, CFloatHandle, CConstFloatHandle, nhVectorSigmoidDiffOp )
+HIP_BINARY( VectorTanhDiff, CFloatHandle, CConstFloatHandle, nhVectorTanhDiff )
+HIP_BINARY( VectorTanhDiffOp, CFloatHandle, CConstFloatHandle, nhVectorTanhDiffOp )
+
+void CHipMathEngine::VectorReLUDiff( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+	const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& upperThresholdHandle )
+{
+	NH_CALL( nhVectorReLUDiff( stream, raw( firstHandle ), raw( secondHandle ), raw( resultHandle ), vectorSize,
+		raw( upperThresholdHandle ) ) );
+}
+
+// ReLU's output is positive and below the threshold exactly where its input is: the same test on either
+// (CpuMathEngine.h:763-767)
+void CHipMathEngine::VectorReLUDiffOp( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+	const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& upperThresholdHandle )
+{
+	VectorReLUDiff( firstHandle, secondHandle, resultHandle, vectorSize, upperThresholdHandle );
+}
 
 void CHipMathEngine::VectorAddValue( const CConstIntHandle& firstHandle, const CIntHandle& resultHandle, int vectorSize,
 	const CConstIntHandle& addition )
@@ -549,6 +573,36 @@ void CHipMathEngine::BlobConvolutionWithActivation( const CConvolutionDesc& desc
 		freeTerm != nullptr ? raw( *freeTerm ) : nullptr, activation, param, raw( result ) ) );
 }
 
+void CHipMathEngine::BlobConvolutionBackward( const CConvolutionDesc& desc, const CConstFloatHandle& outputDiff,
+	const CConstFloatHandle& filter, const CConstFloatHandle* freeTerm, const CFloatHandle& inputDiff )
+{
+	const CHipConvolutionDesc& d = static_cast<const CHipConvolutionDesc&>( desc );
+	size_t workspaceSize = 0;
+	NH_CALL( nhBlobConvolutionBackwardWorkspaceSize( &d.D, &workspaceSize ) );
+	const CMemoryHandle workspace = StackAlloc( std::max<size_t>( workspaceSize, 16 ) );
+	NH_CALL( nhBlobConvolutionBackward( stream, &d.D, raw( outputDiff ), raw( filter ),
+		freeTerm != nullptr ? raw( *freeTerm ) : nullptr, raw( inputDiff ), rawBytes( workspace ), workspaceSize ) );
+	StackFree( workspace );
+}
+
+void CHipMathEngine::BlobConvolutionLearnAdd( const CConvolutionDesc& desc, const CConstFloatHandle& input,
+	const CConstFloatHandle& outputDiff, const CFloatHandle& filterDiff, const CFloatHandle* freeTermDiff,
+	bool isFreeTermDiffFromInput )
+{
+	const CHipConvolutionDesc& d = static_cast<const CHipConvolutionDesc&>( desc );
+	NH_CALL( nhBlobConvolutionLearnAdd( stream, &d.D, raw( input ), raw( outputDiff ), raw( filterDiff ) ) );
+	if( freeTermDiff != nullptr ) {
+		// the free term's gradient is the sum of the pixels of outputDiff, channel by channel; the transposed
+		// convolution asks for the same over the input instead (CpuMathEngineDnnConv.cpp:860-883)
+		if( isFreeTermDiffFromInput ) {
+			SumMatrixRowsAdd( 1, *freeTermDiff, input, d.D.batch * d.D.height * d.D.width, d.D.channels );
+		} else {
+			SumMatrixRowsAdd( 1, *freeTermDiff, outputDiff, d.D.batch * d.D.resultHeight * d.D.resultWidth,
+				d.D.filterCount );
+		}
+	}
+}
+
 CChannelwiseConvolutionDesc* CHipMathEngine::InitBlobChannelwiseConvolution( const CBlobDesc& input, int paddingHeight,
 	int paddingWidth, int strideHeight, int strideWidth, const CBlobDesc& filter, const CBlobDesc* freeTerm,
 	const CBlobDesc& output )
@@ -616,6 +670,13 @@ void CHipMathEngine::BlobMaxPooling( const CMaxPoolingDesc& desc, const CConstFl
 		raw( result ) ) );
 }
 
+void CHipMathEngine::BlobMaxPoolingBackward( const CMaxPoolingDesc& desc, const CConstFloatHandle& resultDiff,
+	const CConstIntHandle& maxIndices, const CFloatHandle& sourceDiff )
+{
+	const CHipMaxPoolingDesc& d = static_cast<const CHipMaxPoolingDesc&>( desc );
+	NH_CALL( nhBlobMaxPoolingBackward( stream, &d.D, raw( resultDiff ), raw( maxIndices ), raw( sourceDiff ) ) );
+}
+
 CMeanPoolingDesc* CHipMathEngine::InitMeanPooling( const CBlobDesc& source, int filterHeight, int filterWidth,
 	int strideHeight, int strideWidth, const CBlobDesc& result )
 {
@@ -631,6 +692,13 @@ void CHipMathEngine::BlobMeanPooling( const CMeanPoolingDesc& desc, const CConst
 {
 	const CHipMeanPoolingDesc& d = static_cast<const CHipMeanPoolingDesc&>( desc );
 	NH_CALL( nhBlobMeanPooling( stream, &d.D, raw( source ), raw( result ) ) );
+}
+
+void CHipMathEngine::BlobMeanPoolingBackward( const CMeanPoolingDesc& desc, const CConstFloatHandle& resultDiff,
+	const CFloatHandle& sourceDiff )
+{
+	const CHipMeanPoolingDesc& d = static_cast<const CHipMeanPoolingDesc&>( desc );
+	NH_CALL( nhBlobMeanPoolingBackward( stream, &d.D, raw( resultDiff ), raw( sourceDiff ) ) );
 }
 
 CLstmDesc* CHipMathEngine::InitLstm( int hiddenSize, int objectSize, const CConstFloatHandle& inputWeights,

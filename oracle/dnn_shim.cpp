@@ -352,6 +352,122 @@ EXPORT int dnn_run( void* engine, int kind, int seed, int param, const int* dims
 	return 3;
 }
 
+// Training: a small classifier, CCrossEntropyLossLayer on float labels, CDnnSimpleGradientSolver (momentum 0.9),
+// `steps` calls of CDnn::RunAndLearnOnce on the same batch. kind 0: FullyConnected (32) - ReLU - FullyConnected
+// (classes); kind 1: Conv 3x3 p1 (8) - ReLU - MaxPool 2x2/2 - Conv 3x3 p1 stride 2 (16) - ReLU - FullyConnected (classes).
+// kind 2: Conv 3x3 p1 (16) - HSwish - [Conv 3x3 p1 (16) - ReLU - Conv 3x3 p1 (16)] + shortcut - ReLU - MeanPool 2x2/2 -
+// FullyConnected (classes); kind 3: Lstm (24 units, over BatchLength) - FullyConnected (classes) at every step.
+// solver 0: CDnnSimpleGradientSolver, 1: CDnnAdaptiveGradientSolver (Adam), both with L2 regularisation 1e-3.
+// losses receives the loss of every step, output the logits of a final forward pass with the trained weights.
+EXPORT int dnn_train( void* engine, int kind, int solverKind, int seed, int classes, int steps, float learningRate,
+	const int* dims, const float* input, const float* labels, float* losses, float* output, int outputCapacity )
+{
+	try {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		CRandom random( seed );
+		CDnn dnn( random, e );
+		CPtr<CSourceLayer> source = new CSourceLayer( e );
+		source->SetName( "source" );
+		dnn.AddLayer( *source );
+		CPtr<CSourceLayer> labelSource = new CSourceLayer( e );
+		labelSource->SetName( "labels" );
+		dnn.AddLayer( *labelSource );
+
+		CBaseLayer* last = source.Ptr();
+		if( kind == 0 ) {
+			CPtr<CFullyConnectedLayer> fc1 = add( dnn, new CFullyConnectedLayer( e ), "fc1", *last );
+			fc1->SetNumberOfElements( 32 );
+			CPtr<CReLULayer> relu = add( dnn, new CReLULayer( e ), "relu", *fc1 );
+			last = relu.Ptr();
+		} else if( kind == 2 ) {
+			CPtr<CConvLayer> c0 = conv( dnn, e, "conv0", *last, 16, 3, 1, 1 );
+			CPtr<CHSwishLayer> a0 = add( dnn, new CHSwishLayer( e ), "hswish0", *c0 );
+			CPtr<CConvLayer> c1 = conv( dnn, e, "conv1", *a0, 16, 3, 1, 1 );
+			CPtr<CReLULayer> r1 = add( dnn, new CReLULayer( e ), "relu1", *c1 );
+			CPtr<CConvLayer> c2 = conv( dnn, e, "conv2", *r1, 16, 3, 1, 1 );
+			CPtr<CEltwiseSumLayer> sum = add( dnn, new CEltwiseSumLayer( e ), "sum", *c2 );
+			sum->Connect( 1, *a0 );
+			CPtr<CReLULayer> r2 = add( dnn, new CReLULayer( e ), "relu2", *sum );
+			CPtr<CMeanPoolingLayer> pool = add( dnn, new CMeanPoolingLayer( e ), "pool", *r2 );
+			pool->SetFilterHeight( 2 ); pool->SetFilterWidth( 2 ); pool->SetStrideHeight( 2 ); pool->SetStrideWidth( 2 );
+			last = pool.Ptr();
+		} else if( kind == 3 ) {
+			CPtr<CLstmLayer> lstm = add( dnn, new CLstmLayer( e ), "lstm", *last );
+			lstm->SetHiddenSize( 24 );
+			last = lstm.Ptr();
+		} else {
+			CPtr<CConvLayer> c1 = conv( dnn, e, "conv1", *last, 8, 3, 1, 1 );
+			CPtr<CReLULayer> r1 = add( dnn, new CReLULayer( e ), "relu1", *c1 );
+			CPtr<CMaxPoolingLayer> pool = add( dnn, new CMaxPoolingLayer( e ), "pool", *r1 );
+			pool->SetFilterHeight( 2 ); pool->SetFilterWidth( 2 ); pool->SetStrideHeight( 2 ); pool->SetStrideWidth( 2 );
+			CPtr<CConvLayer> c2 = conv( dnn, e, "conv2", *pool, 16, 3, 1, 2 );
+			CPtr<CReLULayer> r2 = add( dnn, new CReLULayer( e ), "relu2", *c2 );
+			last = r2.Ptr();
+		}
+		CPtr<CFullyConnectedLayer> fc = add( dnn, new CFullyConnectedLayer( e ), "fc", *last );
+		fc->SetNumberOfElements( classes );
+		CPtr<CCrossEntropyLossLayer> loss = new CCrossEntropyLossLayer( e );
+		loss->SetName( "loss" );
+		loss->Connect( 0, *fc );
+		loss->Connect( 1, *labelSource );
+		dnn.AddLayer( *loss );
+		CPtr<CSinkLayer> sink = new CSinkLayer( e );
+		sink->SetName( "sink" );
+		sink->Connect( *fc );
+		dnn.AddLayer( *sink );
+
+		if( solverKind == 0 ) {
+			CPtr<CDnnSimpleGradientSolver> solver = new CDnnSimpleGradientSolver( e );
+			solver->SetMomentDecayRate( 0.9f );
+			solver->SetLearningRate( learningRate );
+			solver->SetL2Regularization( 1e-3f );
+			dnn.SetSolver( solver );
+		} else {
+			CPtr<CDnnAdaptiveGradientSolver> solver = new CDnnAdaptiveGradientSolver( e );
+			solver->SetLearningRate( learningRate );
+			solver->SetL2Regularization( 1e-3f );
+			dnn.SetSolver( solver );
+		}
+
+		CBlobDesc desc( CT_Float );
+		for( int d = 0; d < 7; ++d ) {
+			desc.SetDimSize( d, dims[d] );
+		}
+		CPtr<CDnnBlob> blob = CDnnBlob::CreateBlob( e, CT_Float, desc );
+		blob->CopyFrom( input );
+		source->SetBlob( blob );
+		CBlobDesc labelDesc( CT_Float );
+		labelDesc.SetDimSize( BD_BatchLength, dims[0] );
+		labelDesc.SetDimSize( BD_BatchWidth, dims[1] );
+		labelDesc.SetDimSize( BD_ListSize, dims[2] );
+		labelDesc.SetDimSize( BD_Channels, classes );
+		CPtr<CDnnBlob> labelBlob = CDnnBlob::CreateBlob( e, CT_Float, labelDesc );
+		labelBlob->CopyFrom( labels );
+		labelSource->SetBlob( labelBlob );
+
+		for( int i = 0; i < steps; ++i ) {
+			dnn.RunAndLearnOnce();
+			losses[i] = loss->GetLastLoss();
+		}
+		dnn.RunOnce();
+		const CPtr<CDnnBlob>& result = sink->GetBlob();
+		if( result->GetDataSize() > outputCapacity ) {
+			lastError = "output buffer too small";
+			return 2;
+		}
+		result->CopyTo( output );
+		return 0;
+	} catch( std::exception& ex ) {
+		lastError = ex.what();
+	} catch( CException* ex ) {
+		lastError = "NeoML exception";
+		delete ex;
+	} catch( ... ) {
+		lastError = "unknown exception";
+	}
+	return 3;
+}
+
 // The recogniser tail (kind 4) with NeoML's CCtcDecodingLayer on top: labels receives, sequence after sequence,
 // the best label sequence of each of the B inputs (at most T each); lengths[b] its length.
 EXPORT int dnn_run_ctc( void* engine, int seed, int classes, const int* dims, const float* input, int* labels, int* lengths )

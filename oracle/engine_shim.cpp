@@ -104,7 +104,7 @@ SHIM_API int shim_engine_type( void* engine ) { return static_cast<IMathEngine*>
 enum {
 	OP_RELU = 0, OP_ELU, OP_LEAKY_RELU, OP_HSWISH, OP_ABS, OP_HARD_TANH, OP_HARD_SIGMOID, OP_NEG,
 	OP_EXP, OP_LOG, OP_ERF, OP_SQRT, OP_INV, OP_MINMAX, OP_SIGMOID, OP_TANH,
-	OP_ADD_VALUE, OP_MULTIPLY, OP_NEG_MULTIPLY, OP_COPY
+	OP_ADD_VALUE, OP_MULTIPLY, OP_NEG_MULTIPLY, OP_COPY, OP_NEG_LOG
 };
 
 SHIM_API int shim_vector_unary( void* engine, int op, const float* first, float* result, int n, float p0, float p1 )
@@ -133,6 +133,7 @@ SHIM_API int shim_vector_unary( void* engine, int op, const float* first, float*
 			case OP_MULTIPLY: e.VectorMultiply( in.Const(), out.Handle(), n, s0.Const() ); break;
 			case OP_NEG_MULTIPLY: e.VectorNegMultiply( in.Const(), out.Handle(), n, s0.Const() ); break;
 			case OP_COPY: e.VectorCopy( out.Handle(), in.Const(), n ); break;
+			case OP_NEG_LOG: e.VectorNegLog( in.Const(), out.Handle(), n ); break;
 			default: throw std::logic_error( "bad unary op" );
 		}
 		out.CopyTo( result );
@@ -141,7 +142,8 @@ SHIM_API int shim_vector_unary( void* engine, int op, const float* first, float*
 
 enum {
 	OP_ADD = 0, OP_SUB, OP_ELTWISE_MULTIPLY, OP_ELTWISE_NEG_MULTIPLY, OP_ELTWISE_DIVIDE, OP_ELTWISE_MAX,
-	OP_ELTWISE_MIN, OP_MULTIPLY_AND_ADD, OP_MULTIPLY_AND_SUB, OP_ELTWISE_MULTIPLY_ADD
+	OP_ELTWISE_MIN, OP_MULTIPLY_AND_ADD, OP_MULTIPLY_AND_SUB, OP_ELTWISE_MULTIPLY_ADD,
+	OP_RELU_DIFF, OP_HSWISH_DIFF, OP_SIGMOID_DIFF, OP_SIGMOID_DIFF_OP, OP_TANH_DIFF, OP_TANH_DIFF_OP
 };
 
 SHIM_API int shim_vector_binary( void* engine, int op, const float* first, const float* second, float* result, int n, float p0 )
@@ -160,6 +162,13 @@ SHIM_API int shim_vector_binary( void* engine, int op, const float* first, const
 			case OP_MULTIPLY_AND_ADD: e.VectorMultiplyAndAdd( a.Const(), b.Const(), out.Handle(), n, s0.Const() ); break;
 			case OP_MULTIPLY_AND_SUB: e.VectorMultiplyAndSub( a.Const(), b.Const(), out.Handle(), n, s0.Const() ); break;
 			case OP_ELTWISE_MULTIPLY_ADD: e.VectorEltwiseMultiplyAdd( a.Const(), b.Const(), out.Handle(), n ); break;
+			// both forms of the ReLU derivative are checked against each other: the second through the ReLU's output
+			case OP_RELU_DIFF: e.VectorReLUDiff( a.Const(), b.Const(), out.Handle(), n, s0.Const() ); break;
+			case OP_HSWISH_DIFF: e.VectorHSwishDiff( a.Const(), b.Const(), out.Handle(), n ); break;
+			case OP_SIGMOID_DIFF: e.VectorSigmoidDiff( a.Const(), b.Const(), out.Handle(), n ); break;
+			case OP_SIGMOID_DIFF_OP: e.VectorSigmoidDiffOp( a.Const(), b.Const(), out.Handle(), n ); break;
+			case OP_TANH_DIFF: e.VectorTanhDiff( a.Const(), b.Const(), out.Handle(), n ); break;
+			case OP_TANH_DIFF_OP: e.VectorTanhDiffOp( a.Const(), b.Const(), out.Handle(), n ); break;
 			default: throw std::logic_error( "bad binary op" );
 		}
 		out.CopyTo( result );
@@ -518,6 +527,97 @@ SHIM_API int shim_separable_block( void* engine, int withExpand, const float* in
 		} else {
 			dst.CopyTo( out );
 		}
+	} );
+}
+
+// gradients of the convolution through BlobConvolutionBackward / BlobConvolutionLearnAdd (NeoMathEngine.h:757-761);
+// filterDiff and freeTermDiff (may be null) are accumulated into
+SHIM_API int shim_blob_convolution_backward( void* engine, const float* outDiff, int n, int h, int w, int cin,
+	const float* filter, int cout, int fh, int fw, int ph, int pw, int sh, int sw, int dh, int dw, const float* bias,
+	float* inDiff )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		const int ho = 1 + ( h - ( fh - 1 ) * dh + 2 * ph - 1 ) / sh;
+		const int wo = 1 + ( w - ( fw - 1 ) * dw + 2 * pw - 1 ) / sw;
+		const CBlobDesc inDesc = imageDesc( n, h, w, cin ), filterDesc = imageDesc( cout, fh, fw, cin ),
+			outDesc = imageDesc( n, ho, wo, cout );
+		CFloatBlob src( e, outDesc.BlobSize(), outDiff ), flt( e, filterDesc.BlobSize(), filter ), ft( e, cin, bias ),
+			dst( e, inDesc.BlobSize() );
+		CConvolutionDesc* desc = e.InitBlobConvolution( inDesc, ph, pw, sh, sw, dh, dw, filterDesc, outDesc );
+		const CConstFloatHandle ftHandle = ft.Const();
+		try {
+			e.BlobConvolutionBackward( *desc, src.Const(), flt.Const(), bias != nullptr ? &ftHandle : nullptr, dst.Handle() );
+		} catch( ... ) {
+			delete desc;
+			throw;
+		}
+		delete desc;
+		dst.CopyTo( inDiff );
+	} );
+}
+
+SHIM_API int shim_blob_convolution_learn_add( void* engine, const float* in, int n, int h, int w, int cin,
+	const float* outDiff, int cout, int fh, int fw, int ph, int pw, int sh, int sw, int dh, int dw, float* filterDiff,
+	float* freeTermDiff )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		const int ho = 1 + ( h - ( fh - 1 ) * dh + 2 * ph - 1 ) / sh;
+		const int wo = 1 + ( w - ( fw - 1 ) * dw + 2 * pw - 1 ) / sw;
+		const CBlobDesc inDesc = imageDesc( n, h, w, cin ), filterDesc = imageDesc( cout, fh, fw, cin ),
+			outDesc = imageDesc( n, ho, wo, cout );
+		CFloatBlob src( e, inDesc.BlobSize(), in ), grad( e, outDesc.BlobSize(), outDiff ),
+			fd( e, filterDesc.BlobSize(), filterDiff ), ftd( e, cout, freeTermDiff );
+		CConvolutionDesc* desc = e.InitBlobConvolution( inDesc, ph, pw, sh, sw, dh, dw, filterDesc, outDesc );
+		const CFloatHandle ftdHandle = ftd.Handle();
+		try {
+			e.BlobConvolutionLearnAdd( *desc, src.Const(), grad.Const(), fd.Handle(), freeTermDiff != nullptr ? &ftdHandle : nullptr, false );
+		} catch( ... ) {
+			delete desc;
+			throw;
+		}
+		delete desc;
+		fd.CopyTo( filterDiff );
+		if( freeTermDiff != nullptr ) {
+			ftd.CopyTo( freeTermDiff );
+		}
+	} );
+}
+
+// forward max pooling with indices, then BlobMaxPoolingBackward with them (isMax) / BlobMeanPoolingBackward
+SHIM_API int shim_blob_pooling_backward( void* engine, int isMax, const float* in, const float* resultDiff, int n, int h, int w,
+	int c, int fh, int fw, int sh, int sw, float* sourceDiff )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		const int ho = ( h - fh ) / sh + 1, wo = ( w - fw ) / sw + 1;
+		const CBlobDesc inDesc = imageDesc( n, h, w, c ), outDesc = imageDesc( n, ho, wo, c );
+		CFloatBlob src( e, inDesc.BlobSize(), in ), out( e, outDesc.BlobSize() ), grad( e, outDesc.BlobSize(), resultDiff ),
+			dst( e, inDesc.BlobSize() );
+		if( isMax ) {
+			CIntBlob idx( e, outDesc.BlobSize() );
+			CMaxPoolingDesc* desc = e.InitMaxPooling( inDesc, fh, fw, sh, sw, outDesc );
+			const CIntHandle idxHandle = idx.Handle();
+			try {
+				e.BlobMaxPooling( *desc, src.Const(), &idxHandle, out.Handle() );
+				e.BlobMaxPoolingBackward( *desc, grad.Const(), idx.Const(), dst.Handle() );
+			} catch( ... ) {
+				delete desc;
+				throw;
+			}
+			delete desc;
+		} else {
+			CMeanPoolingDesc* desc = e.InitMeanPooling( inDesc, fh, fw, sh, sw, outDesc );
+			try {
+				e.BlobMeanPoolingBackward( *desc, grad.Const(), dst.Handle() );
+			} catch( ... ) {
+				delete desc;
+				throw;
+			}
+			delete desc;
+		}
+		dst.CopyTo( sourceDiff );
 	} );
 }
 

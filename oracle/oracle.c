@@ -57,7 +57,7 @@ static float orc_exp_clamped(float x)
 enum {
 	ORC_RELU = 0, ORC_ELU, ORC_LEAKY_RELU, ORC_HSWISH, ORC_ABS, ORC_HARD_TANH, ORC_HARD_SIGMOID, ORC_NEG,
 	ORC_EXP, ORC_LOG, ORC_ERF, ORC_SQRT, ORC_INV, ORC_MINMAX, ORC_SIGMOID, ORC_TANH,
-	ORC_ADD_VALUE, ORC_MULTIPLY, ORC_NEG_MULTIPLY, ORC_COPY
+	ORC_ADD_VALUE, ORC_MULTIPLY, ORC_NEG_MULTIPLY, ORC_COPY, ORC_NEG_LOG
 };
 
 /* result[i] = f(first[i]; p0, p1) */
@@ -93,6 +93,8 @@ ORC_API void orc_vector_unary(int op, const float* first, float* result, int n, 
 		case ORC_MULTIPLY: y = x * p0; break;
 		case ORC_NEG_MULTIPLY: y = -x * p0; break;
 		case ORC_COPY: y = x; break;
+		/* VectorLog with the sign flipped (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:1692-1720) */
+		case ORC_NEG_LOG: { float c = x > FLT_MIN ? x : FLT_MIN; c = c < FLT_MAX ? c : FLT_MAX; y = -logf(c); } break;
 		default: y = NAN; break;
 		}
 		result[i] = y;
@@ -101,7 +103,10 @@ ORC_API void orc_vector_unary(int op, const float* first, float* result, int n, 
 
 enum {
 	ORC_ADD = 0, ORC_SUB, ORC_ELTWISE_MULTIPLY, ORC_ELTWISE_NEG_MULTIPLY, ORC_ELTWISE_DIVIDE, ORC_ELTWISE_MAX,
-	ORC_ELTWISE_MIN, ORC_MULTIPLY_AND_ADD, ORC_MULTIPLY_AND_SUB, ORC_ELTWISE_MULTIPLY_ADD
+	ORC_ELTWISE_MIN, ORC_MULTIPLY_AND_ADD, ORC_MULTIPLY_AND_SUB, ORC_ELTWISE_MULTIPLY_ADD,
+	/* derivatives of the activations times second; the _OP forms take the activation's output as first
+	 * (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:339-395, 433-480, 1377-1520) */
+	ORC_RELU_DIFF, ORC_HSWISH_DIFF, ORC_SIGMOID_DIFF, ORC_SIGMOID_DIFF_OP, ORC_TANH_DIFF, ORC_TANH_DIFF_OP
 };
 
 /* result[i] = f(first[i], second[i]; p0); ORC_ELTWISE_MULTIPLY_ADD reads result[i] as the addend */
@@ -121,6 +126,12 @@ ORC_API void orc_vector_binary(int op, const float* first, const float* second, 
 		case ORC_MULTIPLY_AND_ADD: { volatile float m = b * p0; y = a + m; } break;
 		case ORC_MULTIPLY_AND_SUB: { volatile float m = b * p0; y = a - m; } break;
 		case ORC_ELTWISE_MULTIPLY_ADD: { volatile float m = a * b; y = result[i] + m; } break;
+		case ORC_RELU_DIFF: y = (a > 0.f && (p0 <= 0.f || a < p0)) ? b : 0.f; break;
+		case ORC_HSWISH_DIFF: y = !(-3.f < a) ? 0.f : (a < 3.f ? b * (a * (1.f / 3.f) + 0.5f) : b); break;
+		case ORC_SIGMOID_DIFF: { const float e = orc_exp_clamped(-a); y = b / (2.f + e + 1.f / e); } break;
+		case ORC_SIGMOID_DIFF_OP: y = a * (1.f - a) * b; break;
+		case ORC_TANH_DIFF: { const float t = -1.f + 2.f / (1.f + orc_exp_clamped(-2.f * a)); y = b * (1.f - t * t); } break;
+		case ORC_TANH_DIFF_OP: y = (1.f - a * a) * b; break;
 		default: y = NAN; break;
 		}
 		result[i] = y;
@@ -384,6 +395,94 @@ ORC_API void orc_blob_channelwise_convolution(const float* in, int n, int h, int
 					}
 					out[(((size_t)b * ho + y) * wo + x) * c + ch] = s;
 				}
+}
+
+/* Gradient of the convolution by its input, written as the scatter that transposes the forward loop nest: every
+ * output pixel sends outputDiff * filter to the input pixels of its window (the definition behind
+ * src/CPU/CpuMathEngineDnnConv.cpp:620-805; bias, when given, is a per-channel start value, :758-762). */
+ORC_API void orc_blob_convolution_backward(const float* outDiff, int n, int h, int w, int cin, const float* filter, int cout,
+	int fh, int fw, int ph, int pw, int sh, int sw, int dh, int dw, const float* bias, float* inDiff)
+{
+	int ho, wo;
+	orc_conv_output_size(h, w, fh, fw, ph, pw, sh, sw, dh, dw, &ho, &wo);
+	const size_t total = (size_t)n * h * w * cin;
+	double* acc = (double*)calloc(total, sizeof(double));
+	for (int b = 0; b < n; ++b)
+		for (int y = 0; y < ho; ++y)
+			for (int x = 0; x < wo; ++x)
+				for (int co = 0; co < cout; ++co) {
+					const double g = outDiff[(((size_t)b * ho + y) * wo + x) * cout + co];
+					for (int ky = 0; ky < fh; ++ky) {
+						const int iy = y * sh - ph + ky * dh;
+						if (iy < 0 || iy >= h) continue;
+						for (int kx = 0; kx < fw; ++kx) {
+							const int ix = x * sw - pw + kx * dw;
+							if (ix < 0 || ix >= w) continue;
+							const float* f = filter + (((size_t)co * fh + ky) * fw + kx) * cin;
+							double* dst = acc + (((size_t)b * h + iy) * w + ix) * cin;
+							for (int ci = 0; ci < cin; ++ci) dst[ci] += g * f[ci];
+						}
+					}
+				}
+	for (size_t i = 0; i < total; ++i) inDiff[i] = (float)(acc[i] + (bias ? bias[i % cin] : 0.f));
+	free(acc);
+}
+
+/* filterDiff += gradient of the convolution by its filter (src/CPU/CpuMathEngineDnnConv.cpp:808-987) */
+ORC_API void orc_blob_convolution_learn_add(const float* in, int n, int h, int w, int cin, const float* outDiff, int cout,
+	int fh, int fw, int ph, int pw, int sh, int sw, int dh, int dw, float* filterDiff)
+{
+	int ho, wo;
+	orc_conv_output_size(h, w, fh, fw, ph, pw, sh, sw, dh, dw, &ho, &wo);
+	for (int co = 0; co < cout; ++co)
+		for (int ky = 0; ky < fh; ++ky)
+			for (int kx = 0; kx < fw; ++kx)
+				for (int ci = 0; ci < cin; ++ci) {
+					double s = 0;
+					for (int b = 0; b < n; ++b)
+						for (int y = 0; y < ho; ++y) {
+							const int iy = y * sh - ph + ky * dh;
+							if (iy < 0 || iy >= h) continue;
+							for (int x = 0; x < wo; ++x) {
+								const int ix = x * sw - pw + kx * dw;
+								if (ix < 0 || ix >= w) continue;
+								s += (double)outDiff[(((size_t)b * ho + y) * wo + x) * cout + co]
+									* in[(((size_t)b * h + iy) * w + ix) * cin + ci];
+							}
+						}
+					float* d = filterDiff + (((size_t)co * fh + ky) * fw + kx) * cin + ci;
+					*d = (float)(*d + s);
+				}
+}
+
+/* sourceDiff = 0, then every output element adds its gradient at the index the forward pass stored
+ * (src/CPU/CpuMathEngineDnnPooling.cpp:146-175) */
+ORC_API void orc_blob_max_pooling_backward(const float* resultDiff, const int* indices, int n, int sourceObjectSize,
+	int resultObjectSize, float* sourceDiff)
+{
+	memset(sourceDiff, 0, (size_t)n * sourceObjectSize * sizeof(float));
+	for (int b = 0; b < n; ++b)
+		for (int j = 0; j < resultObjectSize; ++j)
+			sourceDiff[(size_t)b * sourceObjectSize + indices[(size_t)b * resultObjectSize + j]] += resultDiff[(size_t)b * resultObjectSize + j];
+}
+
+/* every window spreads its gradient over its elements, the sums are scaled by 1 / fh / fw at the end
+ * (src/CPU/CpuMathEngineDnnPooling.cpp:202-242) */
+ORC_API void orc_blob_mean_pooling_backward(const float* resultDiff, int n, int h, int w, int c, int fh, int fw, int sh, int sw,
+	float* sourceDiff)
+{
+	const int ho = (h - fh) / sh + 1, wo = (w - fw) / sw + 1;
+	memset(sourceDiff, 0, (size_t)n * h * w * c * sizeof(float));
+	for (int b = 0; b < n; ++b)
+		for (int y = 0; y < ho; ++y)
+			for (int x = 0; x < wo; ++x)
+				for (int ky = 0; ky < fh; ++ky)
+					for (int kx = 0; kx < fw; ++kx)
+						for (int ch = 0; ch < c; ++ch)
+							sourceDiff[(((size_t)b * h + y * sh + ky) * w + x * sw + kx) * c + ch]
+								+= resultDiff[(((size_t)b * ho + y) * wo + x) * c + ch];
+	const float scale = 1.f / fh / fw;
+	for (size_t i = 0; i < (size_t)n * h * w * c; ++i) sourceDiff[i] *= scale;
 }
 
 /* Max pooling without padding. indices may be null. The index follows the reference CPU engine literally:

@@ -19,10 +19,11 @@ ATOL = 1e-5
 
 UNARY = {name: i for i, name in enumerate([
     "relu", "elu", "leaky_relu", "hswish", "abs", "hard_tanh", "hard_sigmoid", "neg", "exp", "log", "erf", "sqrt",
-    "inv", "minmax", "sigmoid", "tanh", "add_value", "multiply", "neg_multiply", "copy"])}
+    "inv", "minmax", "sigmoid", "tanh", "add_value", "multiply", "neg_multiply", "copy", "neg_log"])}
 BINARY = {name: i for i, name in enumerate([
     "add", "sub", "eltwise_multiply", "eltwise_neg_multiply", "eltwise_divide", "eltwise_max", "eltwise_min",
-    "multiply_and_add", "multiply_and_sub", "eltwise_multiply_add"])}
+    "multiply_and_add", "multiply_and_sub", "eltwise_multiply_add", "relu_diff", "hswish_diff", "sigmoid_diff",
+    "sigmoid_diff_op", "tanh_diff", "tanh_diff_op"])}
 BINARY_INT = {"add": 0, "sub": 1, "multiply": 2}
 
 c_float_p = ctypes.POINTER(ctypes.c_float)
@@ -365,6 +366,59 @@ class Cpu:
                    1 if in_place else 0, fp(y))
         return y
 
+    # ---- gradients (what the layers' backward and learn passes call)
+    def conv_backward(self, out_diff, filt, bias, in_shape, ph, pw, sh, sw, dh=1, dw=1):
+        """Gradient by the input; bias [Cin] or None is added to every pixel."""
+        out_diff, filt = f32(out_diff), f32(filt)
+        n, h, w, cin = in_shape
+        cout, fh, fw, _ = filt.shape
+        assert out_diff.shape == (n, *conv_out(h, w, fh, fw, ph, pw, sh, sw, dh, dw), cout)
+        bias = None if bias is None else f32(bias)
+        y = np.empty(in_shape, np.float32)
+        self._call("blob_convolution_backward", fp(out_diff), n, h, w, cin, fp(filt), cout, fh, fw, ph, pw, sh, sw, dh, dw,
+                   fp(bias), fp(y))
+        return y
+
+    def conv_learn_add(self, x, out_diff, filter_diff, ph, pw, sh, sw, dh=1, dw=1, free_term_diff=None):
+        """filter_diff [Cout][fh][fw][Cin] += gradient by the filter; free_term_diff [Cout] += column sums of out_diff
+        (through the reference interface only: the oracle's form of it is numpy's sum)."""
+        x, out_diff = f32(x), f32(out_diff)
+        n, h, w, cin = x.shape
+        cout, fh, fw, _ = filter_diff.shape
+        fd = f32(filter_diff).copy()
+        if self.kind == "orc":
+            self._call("blob_convolution_learn_add", fp(x), n, h, w, cin, fp(out_diff), cout, fh, fw, ph, pw, sh, sw, dh, dw,
+                       fp(fd))
+            if free_term_diff is None:
+                return fd
+            return fd, (f32(free_term_diff) + out_diff.reshape(-1, cout).astype(np.float64).sum(axis=0)).astype(np.float32)
+        ftd = None if free_term_diff is None else f32(free_term_diff).copy()
+        self._call("blob_convolution_learn_add", fp(x), n, h, w, cin, fp(out_diff), cout, fh, fw, ph, pw, sh, sw, dh, dw,
+                   fp(fd), fp(ftd))
+        return fd if ftd is None else (fd, ftd)
+
+    def max_pool_backward(self, x, result_diff, fh, fw, sh, sw):
+        """Forward pass over x for the indices, then the gradient by x."""
+        x, result_diff = f32(x), f32(result_diff)
+        n, h, w, c = x.shape
+        y = np.empty_like(x)
+        if self.kind == "orc":
+            _, idx = self.max_pool(x, fh, fw, sh, sw, with_indices=True)
+            self._call("blob_max_pooling_backward", fp(result_diff), ip(idx), n, h * w * c, idx[0].size, fp(y))
+        else:
+            self._call("blob_pooling_backward", 1, fp(x), fp(result_diff), n, h, w, c, fh, fw, sh, sw, fp(y))
+        return y
+
+    def mean_pool_backward(self, in_shape, result_diff, fh, fw, sh, sw):
+        result_diff = f32(result_diff)
+        n, h, w, c = in_shape
+        y = np.empty(in_shape, np.float32)
+        if self.kind == "orc":
+            self._call("blob_mean_pooling_backward", fp(result_diff), n, h, w, c, fh, fw, sh, sw, fp(y))
+        else:
+            self._call("blob_pooling_backward", 0, None, fp(result_diff), n, h, w, c, fh, fw, sh, sw, fp(y))
+        return y
+
     def max_pool(self, x, fh, fw, sh, sw, with_indices=False):
         x = f32(x)
         n, h, w, c = x.shape
@@ -503,7 +557,7 @@ class Hip:
         "log": ("nhVectorLog", 0), "erf": ("nhVectorErf", 0), "sqrt": ("nhVectorSqrt", 0), "inv": ("nhVectorInv", 0),
         "minmax": ("nhVectorMinMax", 2), "sigmoid": ("nhVectorSigmoid", 0), "tanh": ("nhVectorTanh", 0),
         "add_value": ("nhVectorAddValue", 1), "multiply": ("nhVectorMultiply", 1),
-        "neg_multiply": ("nhVectorNegMultiply", 1),
+        "neg_multiply": ("nhVectorNegMultiply", 1), "neg_log": ("nhVectorNegLog", 0),
     }
 
     def unary(self, op, x, p0=0.0, p1=0.0, inplace=False, offset=0):
@@ -531,7 +585,9 @@ class Hip:
         "eltwise_neg_multiply": "nhVectorEltwiseNegMultiply", "eltwise_divide": "nhVectorEltwiseDivide",
         "eltwise_max": "nhVectorEltwiseMax", "eltwise_min": "nhVectorEltwiseMin",
         "multiply_and_add": "nhVectorMultiplyAndAdd", "multiply_and_sub": "nhVectorMultiplyAndSub",
-        "eltwise_multiply_add": "nhVectorEltwiseMultiplyAdd",
+        "eltwise_multiply_add": "nhVectorEltwiseMultiplyAdd", "relu_diff": "nhVectorReLUDiff",
+        "hswish_diff": "nhVectorHSwishDiff", "sigmoid_diff": "nhVectorSigmoidDiff",
+        "sigmoid_diff_op": "nhVectorSigmoidDiffOp", "tanh_diff": "nhVectorTanhDiff", "tanh_diff_op": "nhVectorTanhDiffOp",
     }
 
     def binary(self, op, a, b, p0=0.0, result=None, inplace_first=False):
@@ -539,7 +595,7 @@ class Hip:
         n = a.numel()
         out = a if inplace_first else (self.empty((n,)) if result is None else self.up(f32(result).ravel()))
         args = [self.p(a), self.p(b), self.p(out), n]
-        if op in ("multiply_and_add", "multiply_and_sub"):
+        if op in ("multiply_and_add", "multiply_and_sub", "relu_diff"):
             s = self.scalar(p0)
             args.append(self.p(s))
         self.call(self.BINARY_FN[op], *args)
@@ -745,6 +801,50 @@ class Hip:
             self.call(which, ctypes.byref(d), self.p(xs), self.p(ws[2]), self.p(ws[3]), self.p(ws[4]), self.p(ws[5]),
                       self.p(out), self.p(work), size.value)
         return self.down(out).reshape(n, ho, wo, cout)
+
+    # -- gradients
+    def conv_backward(self, out_diff, filt, bias, in_shape, ph, pw, sh, sw, dh=1, dw=1):
+        out_diff, filt = f32(out_diff), f32(filt)
+        n, h, w, cin = in_shape
+        cout, fh, fw, _ = filt.shape
+        d = self.conv_desc(n, h, w, cin, cout, fh, fw, ph, pw, sh, sw, dh, dw)
+        size = ctypes.c_size_t(0)
+        self.na.check(self.lib.nhBlobConvolutionBackwardWorkspaceSize(ctypes.byref(d), ctypes.byref(size)))
+        work = self.torch.empty((size.value + 15) // 4 + 4, dtype=self.torch.float32, device=self.dev)
+        gs, fs, bs = self.up(out_diff), self.up(filt), self.up(None if bias is None else f32(bias))
+        out = self.empty(in_shape)
+        self.call("nhBlobConvolutionBackward", ctypes.byref(d), self.p(gs), self.p(fs), self.p(bs), self.p(out),
+                  self.p(work), size.value)
+        return self.down(out)
+
+    def conv_learn_add(self, x, out_diff, filter_diff, ph, pw, sh, sw, dh=1, dw=1):
+        x, out_diff, filter_diff = f32(x), f32(out_diff), f32(filter_diff)
+        n, h, w, cin = x.shape
+        cout, fh, fw, _ = filter_diff.shape
+        d = self.conv_desc(n, h, w, cin, cout, fh, fw, ph, pw, sh, sw, dh, dw)
+        xs, gs, fd = self.up(x), self.up(out_diff), self.up(filter_diff)
+        self.call("nhBlobConvolutionLearnAdd", ctypes.byref(d), self.p(xs), self.p(gs), self.p(fd))
+        return self.down(fd)
+
+    def max_pool_backward(self, x, result_diff, fh, fw, sh, sw):
+        x = f32(x)
+        n, h, w, c = x.shape
+        d = self.pool_desc(n, h, w, c, fh, fw, sh, sw)
+        xs, gs = self.up(x), self.up(f32(result_diff))
+        out = self.empty((n, d.resultHeight, d.resultWidth, c))
+        idx = self.empty(out.shape, np.int32)
+        self.call("nhBlobMaxPooling", ctypes.byref(d), self.p(xs), self.p(idx), self.p(out))
+        src_diff = self.empty(x.shape)
+        self.call("nhBlobMaxPoolingBackward", ctypes.byref(d), self.p(gs), self.p(idx), self.p(src_diff))
+        return self.down(src_diff)
+
+    def mean_pool_backward(self, in_shape, result_diff, fh, fw, sh, sw):
+        n, h, w, c = in_shape
+        d = self.pool_desc(n, h, w, c, fh, fw, sh, sw)
+        gs = self.up(f32(result_diff))
+        src_diff = self.empty(in_shape)
+        self.call("nhBlobMeanPoolingBackward", ctypes.byref(d), self.p(gs), self.p(src_diff))
+        return self.down(src_diff)
 
     def pool_desc(self, n, h, w, c, fh, fw, sh, sw):
         d = self.na.PoolingDesc(n, h, w, c, fh, fw, sh, sw, 0, 0)

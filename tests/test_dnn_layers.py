@@ -270,3 +270,50 @@ def test_optimized_resnet18_through_cdnn_at_benchmark_size(capsys):
               "(%d rowwise chains) %.3f ms = %.0f images/sec" % (plain_ms, chains, fused_ms, 64e3 / fused_ms))
     assert chains >= 1
     assert_close(fused, plain, "optimized vs plain ResNet-18 on the HIP engine")
+
+
+# ---------------------------------------------------------------------------------------------------------
+# training: CDnn::RunAndLearnOnce (backward and learn passes of the layers, the loss layer, the solvers)
+
+# name: (kind, input dims, solver: 0 SGD with momentum / 1 Adam, learning rate)
+TRAIN_CASES = {
+    "mlp_sgd": (0, (1, 16, 1, 1, 1, 1, 24), 0, 0.05),
+    "mlp_adam": (0, (1, 16, 1, 1, 1, 1, 24), 1, 0.01),
+    "cnn_sgd": (1, (1, 6, 1, 12, 12, 1, 3), 0, 0.05),
+    "residual_cnn_adam": (2, (1, 4, 1, 10, 10, 1, 3), 1, 0.01),
+    "residual_cnn_sgd_wide": (2, (1, 8, 1, 32, 32, 1, 16), 0, 0.02),
+    "lstm_adam": (3, (7, 5, 1, 1, 1, 1, 12), 1, 0.01),
+}
+
+
+def dnn_train(engine, name, classes=5, steps=4):
+    kind, dims, solver, rate = TRAIN_CASES[name]
+    g = np.random.default_rng(0xC0FFEE + 7 * kind + solver)
+    x = g.uniform(-1, 1, dims).astype(np.float32)
+    n = dims[0] * dims[1] * dims[2]
+    labels = np.zeros((n, classes), np.float32)
+    labels[np.arange(n), g.integers(0, classes, n)] = 1
+    losses = np.zeros(steps, np.float32)
+    out = np.zeros(n * classes, np.float32)
+    rc = lib().dnn_train(engine, kind, solver, 11, classes, steps, ctypes.c_float(rate), ip(i32(dims)), fp(x), fp(labels),
+                         fp(losses), fp(out), out.size)
+    if rc != 0:
+        raise RuntimeError("dnn_train %s: %s" % (name, lib().dnn_last_error().decode()))
+    return losses, out
+
+
+@pytest.mark.parametrize("name", sorted(TRAIN_CASES))
+def test_training_reduces_the_loss_on_the_reference_cpu_engine(name):
+    losses, out = dnn_train(nhtest.cpu_engine(), name)
+    assert np.isfinite(out).all() and (np.diff(losses) < 0).all(), losses
+    assert abs(losses[0] - np.log(5)) < 0.4  # an untrained 5-class classifier
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(TRAIN_CASES))
+def test_training_on_hip_engine_follows_the_cpu_engine(name):
+    want_losses, want = dnn_train(nhtest.cpu_engine(), name)
+    losses, got = dnn_train(nhtest.hip_engine(), name)
+    # four steps of forward, backward, learn and solver: every gradient kernel feeds the weights of the next step
+    assert_close(losses, want_losses, "loss per step, %s" % name, atol=2e-5)
+    assert_close(got, want, "logits after training, %s" % name, atol=1e-4, rtol=1e-3)

@@ -11,7 +11,7 @@ import pytest
 import nhtest
 from nhtest import Cpu, assert_close
 from test_oracle import (UNARY_CASES, BINARY_CASES, CONV_CASES, CHANNELWISE_CASES, POOL_CASES, SEPARABLE_CASES,
-                         separable_operands, unary_input, rng)
+                         DIFF_CASES, diff_operands, separable_operands, unary_input, rng)
 
 pytestmark = pytest.mark.gpu
 
@@ -63,6 +63,15 @@ def test_binary(op):
         assert_close(hip().binary(op, a, b, 0.37, result=r), want, "%s n=%d" % (op, n))
     if op == "add":  # residual connections write into their first operand
         assert_close(hip().binary(op, a, b, inplace_first=True), a + b, "add in place")
+
+
+@pytest.mark.parametrize("op,p", DIFF_CASES)
+def test_activation_derivatives(op, p):
+    for n in (1, 5, 1003, 300003):
+        a, b = diff_operands(op, n, 70 + n)
+        assert_close(hip().binary(op, a, b, p), orc.binary(op, a, b, p), "%s n=%d" % (op, n))
+    a, b = diff_operands(op, 4099, 3)
+    assert_close(hip().binary(op, a, b, p, inplace_first=True), orc.binary(op, a, b, p), op + " into its first operand")
 
 
 def test_int_ops_fill_convert():
@@ -270,6 +279,73 @@ def test_convolution_with_activation(case, activation, param):
     want = orc.unary(activation, plain, param).reshape(plain.shape)
     got = hip().conv(x, f, bias, ph, pw, sh, sw, dh, dw, activation=activation, param=param)
     assert_close(got, want, "conv + %s %s" % (activation, case))
+
+
+# the training-step shapes on top of the forward cases: whole tiles, strides that leave holes in the input gradient,
+# a stem with few input channels, 1x1 shortcuts
+GPU_CONV_GRADIENT_CASES = CONV_CASES + [
+    (2, 16, 16, 64, 64, 3, 3, 1, 1, 1, 1, 1, 1),
+    (2, 14, 14, 32, 48, 3, 3, 1, 1, 2, 2, 1, 1),
+    (2, 15, 15, 32, 48, 3, 3, 1, 1, 2, 2, 1, 1),    # stride 2 over an odd size: the last input row has no window of its own
+    (1, 10, 10, 20, 130, 3, 3, 2, 2, 1, 1, 2, 2),
+    (3, 9, 9, 128, 200, 1, 1, 0, 0, 1, 1, 1, 1),
+    (2, 14, 14, 128, 256, 1, 1, 0, 0, 2, 2, 1, 1),
+    (2, 32, 32, 3, 64, 7, 7, 3, 3, 2, 2, 1, 1),
+    (2, 8, 32, 1, 64, 3, 3, 1, 1, 1, 1, 1, 1),
+    (2, 9, 13, 6, 10, 3, 5, 1, 2, 1, 2, 2, 1),
+    (1, 6, 5, 7, 9, 2, 4, 0, 3, 1, 1, 1, 1),
+    (2, 12, 12, 8, 16, 3, 3, 0, 0, 3, 3, 1, 1),     # stride as large as the filter
+    (8, 32, 32, 64, 64, 3, 3, 1, 1, 1, 1, 1, 1),    # many pixels: the filter gradient's reduction is split over the grid
+]
+
+
+@pytest.mark.parametrize("case", GPU_CONV_GRADIENT_CASES)
+def test_convolution_gradients(case):
+    n, h, w, cin, cout, fh, fw, ph, pw, sh, sw, dh, dw = case
+    g = rng(410 + h * w + cin)
+    ho, wo = nhtest.conv_out(h, w, fh, fw, ph, pw, sh, sw, dh, dw)
+    x = g.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    f = g.normal(0, 1.0 / np.sqrt(fh * fw * cin), (cout, fh, fw, cin)).astype(np.float32)
+    grad = g.uniform(-1, 1, (n, ho, wo, cout)).astype(np.float32)
+    bias = g.uniform(-1, 1, cin).astype(np.float32)
+    want = orc.conv_backward(grad, f, None, x.shape, ph, pw, sh, sw, dh, dw)
+    assert_close(hip().conv_backward(grad, f, None, x.shape, ph, pw, sh, sw, dh, dw), want, "backward %s" % (case,), atol=2e-5)
+    assert_close(hip().conv_backward(grad, f, bias, x.shape, ph, pw, sh, sw, dh, dw), want + bias, "backward + free term", atol=2e-5)
+    start = g.uniform(-1, 1, f.shape).astype(np.float32)
+    want = orc.conv_learn_add(x, grad, start, ph, pw, sh, sw, dh, dw)
+    # sums over every pixel of the batch: the bar is relative to the size of the terms, as for the dot product
+    scale = np.sqrt(n * ho * wo)
+    assert_close(hip().conv_learn_add(x, grad, start, ph, pw, sh, sw, dh, dw), want, "learn %s" % (case,), atol=1e-5 * scale)
+
+
+def test_convolution_gradients_are_adjoints_at_full_size():
+    # the single-layer configuration, batch 32: <conv(x, f), g> == <x, backward(g, f)> == <f, learn(x, g)>
+    h = hip()
+    g = rng(41)
+    x = g.uniform(-1, 1, (32, 32, 32, 64)).astype(np.float32)
+    f = g.normal(0, 1.0 / 24, (64, 3, 3, 64)).astype(np.float32)
+    grad = g.uniform(-1, 1, (32, 32, 32, 64)).astype(np.float32)
+    y = h.conv(x, f, None, 1, 1, 1, 1).astype(np.float64)
+    pairing = np.vdot(y, grad)
+    size = np.abs(y * grad).sum()
+    dx = h.conv_backward(grad, f, None, x.shape, 1, 1, 1, 1)
+    assert abs(np.vdot(dx.astype(np.float64), x) - pairing) <= 1e-5 * size
+    df = h.conv_learn_add(x, grad, np.zeros_like(f), 1, 1, 1, 1)
+    assert abs(np.vdot(df.astype(np.float64), f) - pairing) <= 1e-5 * size
+
+
+@pytest.mark.parametrize("case", POOL_CASES + [(2, 57, 57, 64, 3, 3, 2, 2), (3, 16, 64, 7, 2, 2, 2, 2), (2, 23, 19, 8, 3, 3, 1, 1),
+                                               (2, 9, 9, 4, 4, 4, 1, 1), (2, 10, 10, 6, 2, 2, 3, 3)])
+def test_pooling_gradients(case):
+    n, h, w, c, fh, fw, sh, sw = case
+    g = rng(113 + h)
+    x = g.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    ho, wo = (h - fh) // sh + 1, (w - fw) // sw + 1
+    grad = g.uniform(-1, 1, (n, ho, wo, c)).astype(np.float32)
+    assert_close(hip().max_pool_backward(x, grad, fh, fw, sh, sw), orc.max_pool_backward(x, grad, fh, fw, sh, sw),
+                 "max pooling backward %s" % (case,))
+    assert_close(hip().mean_pool_backward(x.shape, grad, fh, fw, sh, sw), orc.mean_pool_backward(x.shape, grad, fh, fw, sh, sw),
+                 "mean pooling backward %s" % (case,))
 
 
 def test_convolution_ignores_pixels_outside_the_windows():

@@ -33,17 +33,17 @@ UNARY_CASES = [
     ("relu", 0.0, 0.0), ("relu", 6.0, 0.0), ("elu", 0.7, 0.0), ("leaky_relu", 0.1, 0.0), ("hswish", 0, 0),
     ("abs", 0, 0), ("hard_tanh", 0, 0), ("hard_sigmoid", 0.2, 0.5), ("neg", 0, 0), ("exp", 0, 0), ("log", 0, 0),
     ("erf", 0, 0), ("sqrt", 0, 0), ("inv", 0, 0), ("minmax", -0.5, 1.5), ("sigmoid", 0, 0), ("tanh", 0, 0),
-    ("add_value", 1.25, 0), ("multiply", -2.5, 0), ("neg_multiply", 1.702, 0), ("copy", 0, 0),
+    ("add_value", 1.25, 0), ("multiply", -2.5, 0), ("neg_multiply", 1.702, 0), ("copy", 0, 0), ("neg_log", 0, 0),
 ]
 
 
 def unary_input(op, n, seed):
     x = rng(seed).uniform(-10, 10, n).astype(np.float32)
-    if op in ("log", "sqrt"):
+    if op in ("log", "sqrt", "neg_log"):
         x = np.abs(x) + 1e-3
     # special values: zeros, tiny, huge
     x[:8] = [0.0, -0.0, 1e-38, -1e-38, 3.0, -3.0, 87.0, -87.0]
-    if op in ("log", "sqrt"):
+    if op in ("log", "sqrt", "neg_log"):
         x[:8] = np.abs(x[:8])
     return x
 
@@ -68,6 +68,7 @@ NUMPY_UNARY = {
     "multiply": lambda x, p0, p1: x * np.float32(p0),
     "neg_multiply": lambda x, p0, p1: -x * np.float32(p0),
     "copy": lambda x, p0, p1: x,
+    "neg_log": lambda x, p0, p1: -np.log(np.clip(x.astype(np.float64), np.finfo(np.float32).tiny, None)),
 }
 
 
@@ -127,6 +128,60 @@ def test_binary(op):
         assert_close(y, NUMPY_BINARY[op](a, b, 0.37, r), op)
         if nhtest.have_reference():
             assert_close(y, ref().binary(op, a, b, 0.37, result=r), op + " vs reference")
+
+
+# derivatives of the activations: first = the activation's input (or its output for the _op forms), second = the
+# gradient that arrives from above, p = ReLU's upper threshold
+DIFF_CASES = [("relu_diff", 0.0), ("relu_diff", 6.0), ("hswish_diff", 0.0), ("sigmoid_diff", 0.0), ("sigmoid_diff_op", 0.0),
+              ("tanh_diff", 0.0), ("tanh_diff_op", 0.0)]
+_expit = lambda a: scipy.special.expit(a.astype(np.float64))
+NUMPY_DIFF = {
+    "relu_diff": lambda a, b, p: np.where((a > 0) & ((a < p) if p > 0 else True), b, 0),
+    "hswish_diff": lambda a, b, p: np.where(a <= -3, 0, np.where(a >= 3, b, b * (2 * a.astype(np.float64) + 3) / 6)),
+    "sigmoid_diff": lambda a, b, p: _expit(a) * (1 - _expit(a)) * b,
+    "sigmoid_diff_op": lambda a, b, p: a.astype(np.float64) * (1 - a) * b,
+    "tanh_diff": lambda a, b, p: (1 - np.tanh(a.astype(np.float64)) ** 2) * b,
+    "tanh_diff_op": lambda a, b, p: (1 - a.astype(np.float64) ** 2) * b,
+}
+# the activation each derivative belongs to, for the finite-difference check
+DIFF_FORWARD = {"relu_diff": "relu", "hswish_diff": "hswish", "sigmoid_diff": "sigmoid", "tanh_diff": "tanh"}
+
+
+def diff_operands(op, n, seed):
+    g = rng(seed)
+    a = g.uniform(-8, 8, n).astype(np.float32)
+    if op.endswith("_op"):
+        a = g.uniform(-0.99 if op.startswith("tanh") else 0.01, 0.99, n).astype(np.float32)
+    elif n >= 8:
+        a[:8] = [0.0, 3.0, -3.0, 6.0, 2.999, -2.999, 40.0, -40.0]
+    b = g.uniform(-2, 2, n).astype(np.float32)
+    return a, b
+
+
+@pytest.mark.parametrize("op,p", DIFF_CASES)
+def test_activation_derivatives(op, p):
+    for n in (1, 5, 1003):
+        a, b = diff_operands(op, n, 70 + n)
+        y = orc.binary(op, a, b, p)
+        assert_close(y, NUMPY_DIFF[op](a, b, p), "%s n=%d" % (op, n))
+        if nhtest.have_reference():
+            assert_close(ref().binary(op, a, b, p), y, "%s vs reference n=%d" % (op, n))
+
+
+@pytest.mark.parametrize("op,p", [c for c in DIFF_CASES if c[0] in DIFF_FORWARD])
+def test_activation_derivatives_are_the_slopes_of_the_activations(op, p):
+    # central differences of the forward function in float64-friendly ranges, away from the kinks
+    g = rng(75)
+    a = g.uniform(-2.9, 2.9, 500).astype(np.float32)
+    a = a[(np.abs(a) > 0.05)]
+    eps = np.float32(1.0 / 256)
+    fwd = DIFF_FORWARD[op]
+    slope = (orc.unary(fwd, a + eps, p).astype(np.float64) - orc.unary(fwd, a - eps, p)) / (2.0 * float(eps))
+    y = orc.binary(op, a, np.ones_like(a), p)
+    np.testing.assert_allclose(y, slope, rtol=2e-3, atol=2e-4)
+    if op in ("sigmoid_diff", "tanh_diff"):  # the _op form on the activation's output is the same derivative
+        out = orc.unary(fwd, a)
+        assert_close(orc.binary(op + "_op", out, np.ones_like(a)), y, op + " through the output", atol=1e-5)
 
 
 def test_int_ops_and_conversions():
@@ -340,6 +395,47 @@ def test_convolution(case):
         assert_close(ref().conv(x, f, None, ph, pw, sh, sw, dh, dw), y0, "conv vs reference, no free term")
 
 
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_convolution_gradients_are_the_adjoints_of_the_forward_pass(case):
+    """<conv(x, f), g> is bilinear in (x, f): its gradient by x is conv_backward(g, f), by f is learn(x, g). With the
+    forward oracle pinned above, a wrong index, stride or dilation in either gradient breaks one of the identities."""
+    n, h, w, cin, cout, fh, fw, ph, pw, sh, sw, dh, dw = case
+    g = rng(20 + h * w)
+    x = g.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    f = g.normal(0, 1, (cout, fh, fw, cin)).astype(np.float32)
+    y = orc.conv(x, f, None, ph, pw, sh, sw, dh, dw)
+    grad = g.uniform(-1, 1, y.shape).astype(np.float32)
+    bias = g.uniform(-1, 1, cin).astype(np.float32)
+    dx = orc.conv_backward(grad, f, None, x.shape, ph, pw, sh, sw, dh, dw)
+    pairing = np.vdot(y.astype(np.float64), grad)
+    assert abs(np.vdot(dx.astype(np.float64), x) - pairing) <= 1e-4 * np.abs(y.astype(np.float64) * grad).sum()
+    # every component, not only the pairing with x: the forward pass of a unit impulse picks one column of the adjoint
+    for _ in range(6):
+        at = tuple(g.integers(0, d) for d in x.shape)
+        e = np.zeros_like(x)
+        e[at] = 1
+        assert abs(np.vdot(orc.conv(e, f, None, ph, pw, sh, sw, dh, dw).astype(np.float64), grad) - dx[at]) <= 1e-4 * (1 + abs(dx[at]))
+    assert_close(orc.conv_backward(grad, f, bias, x.shape, ph, pw, sh, sw, dh, dw), dx + bias, "free term of the backward pass", atol=1e-5)
+    start = g.uniform(-1, 1, f.shape).astype(np.float32)
+    df = orc.conv_learn_add(x, grad, start, ph, pw, sh, sw, dh, dw)
+    assert abs(np.vdot((df - start).astype(np.float64), f) - pairing) <= 2e-4 * np.abs(y.astype(np.float64) * grad).sum()
+    for _ in range(6):
+        at = tuple(g.integers(0, d) for d in f.shape)
+        e = np.zeros_like(f)
+        e[at] = 1
+        want = np.vdot(orc.conv(x, e, None, ph, pw, sh, sw, dh, dw).astype(np.float64), grad) + start[at]
+        assert abs(want - df[at]) <= 1e-4 * (1 + abs(want))
+    if nhtest.have_reference():
+        r = ref()
+        assert_close(r.conv_backward(grad, f, None, x.shape, ph, pw, sh, sw, dh, dw), dx, "backward vs reference %s" % (case,), atol=1e-4)
+        assert_close(r.conv_backward(grad, f, bias, x.shape, ph, pw, sh, sw, dh, dw), dx + bias, "backward + free term vs reference", atol=1e-4)
+        ft0 = g.uniform(-1, 1, cout).astype(np.float32)
+        rdf, rft = r.conv_learn_add(x, grad, start, ph, pw, sh, sw, dh, dw, free_term_diff=ft0)
+        odf, oft = orc.conv_learn_add(x, grad, start, ph, pw, sh, sw, dh, dw, free_term_diff=ft0)
+        assert_close(rdf, df, "learn vs reference %s" % (case,), atol=2e-4)
+        assert_close(rft, oft, "free term diff vs reference", atol=1e-4)
+
+
 def test_convolution_1x1_is_a_matrix_product():
     g = rng(11)
     x = g.uniform(-1, 1, (2, 4, 5, 6)).astype(np.float32)
@@ -465,6 +561,43 @@ def test_pooling(case):
         ry, ridx = ref().max_pool(x, fh, fw, sh, sw, with_indices=True)
         assert np.array_equal(ry, y)
         assert np.array_equal(ridx, idx), "max-pool indices differ from the reference engine"
+
+
+def wo_is_one(w, fw, sw):
+    return (w - fw) // sw + 1 == 1
+
+
+@pytest.mark.parametrize("case", POOL_CASES)
+def test_pooling_gradients(case):
+    n, h, w, c, fh, fw, sh, sw = case
+    g = rng(60 + h * w)
+    x = g.permutation(n * h * w * c).reshape(n, h, w, c).astype(np.float32)  # distinct values: one maximum per window
+    y = orc.mean_pool(x, fh, fw, sh, sw)
+    grad = g.uniform(-1, 1, y.shape).astype(np.float32)
+    # mean pooling is linear: its gradient is its adjoint
+    dmean = orc.mean_pool_backward(x.shape, grad, fh, fw, sh, sw)
+    assert abs(np.vdot(dmean.astype(np.float64), x) - np.vdot(y.astype(np.float64), grad)) <= 1e-4 * np.abs(y * grad).sum()
+    for _ in range(5):
+        at = tuple(g.integers(0, d) for d in x.shape)
+        e = np.zeros_like(x)
+        e[at] = 1
+        assert abs(np.vdot(orc.mean_pool(e, fh, fw, sh, sw), grad) - dmean[at]) <= 1e-5
+    # max pooling: a scatter-add of the gradient at the indices the forward pass stored (which follow the reference's
+    # CPU engine literally, see the index tests below), restated with numpy's unbuffered add
+    dmax = orc.max_pool_backward(x, grad, fh, fw, sh, sw)
+    _, idx = orc.max_pool(x, fh, fw, sh, sw, with_indices=True)
+    want = np.zeros((n, h * w * c))
+    for b in range(n):
+        np.add.at(want[b], idx[b].ravel(), grad[b].ravel().astype(np.float64))
+    assert_close(dmax, want.reshape(x.shape), "max pooling backward", atol=1e-5)
+    if wo_is_one(w, fw, sw):  # windows in the first column: the index is the arg max, the scatter the gradient
+        step = g.integers(-3, 4, x.shape).astype(np.float32) / 8  # exact in fp32, below half the gap between values
+        moved = orc.max_pool(x + step, fh, fw, sh, sw).astype(np.float64) - orc.max_pool(x, fh, fw, sh, sw)
+        assert abs(np.vdot(moved, grad) - np.vdot(dmax.astype(np.float64), step)) <= 1e-5 * np.abs(grad).sum()
+    assert abs(dmax.astype(np.float64).sum() - grad.astype(np.float64).sum()) <= 1e-3
+    if nhtest.have_reference():
+        assert_close(ref().mean_pool_backward(x.shape, grad, fh, fw, sh, sw), dmean, "mean pooling backward vs reference")
+        assert_close(ref().max_pool_backward(x, grad, fh, fw, sh, sw), dmax, "max pooling backward vs reference", atol=1e-5)
 
 
 def test_max_pool_index_first_window_points_at_the_maximum():
