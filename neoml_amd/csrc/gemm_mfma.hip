@@ -39,10 +39,23 @@ typedef float f32x16 __attribute__( ( ext_vector_type( 16 ) ) );
 // over Fh filter rows of RowPitch = ceil4( Fw * Cin ) values each. The Fw * Cin values that one filter row meets are
 // contiguous in a channels-last image (no dilation along the width), so they are fetched as 128-bit runs however
 // Cin divides; the 1-3 padding values per row are masked to zero on both operands.
-enum TAMode { AM_RowsK = 0, AM_RowsM = 1, AM_Conv = 2, AM_Conv1x1 = 3, AM_ConvRows = 4 };
+// AM_ConvClasses: the gradient by the input of a strided convolution, one stride-1 convolution per residue class of the
+// input pixels (blockIdx.y = class): AM_Conv whose geometry, filter and output rows come from args.Class[class].
+enum TAMode { AM_RowsK = 0, AM_RowsM = 1, AM_Conv = 2, AM_Conv1x1 = 3, AM_ConvRows = 4, AM_ConvClasses = 5 };
 // BM_ConvN: B is the im2col view of an N,H,W,C image read N-major: row k = output pixel, column n = ( kh, kw, ci ).
 // With A = the gradient by the convolution's output read M-major this is the gradient by the filter.
 enum TBMode { BM_RowsK = 0, BM_RowsN = 1, BM_ConvN = 2 };
+
+// One residue class ( ( hi + pad ) mod stride, same along the width ) of the input pixels of a strided convolution. Only
+// the filter taps kh with kh * dilation in the same class reach its pixels, Fh x Fw of them, and through them the
+// class is a stride-1 convolution over the output gradient. Its result rows are the pixels
+// ( OutH0 + j * strideH, OutW0 + i * strideW ), j < Ho, i < Wo, of every image.
+struct CConvClass {
+	int K, Fh, Fw, PadH, PadW, Ho, Wo, M, OutH0, OutW0;
+	long long BOffset; // of the class's filter [N][Fh][Fw][Cin] inside B, in floats
+};
+
+constexpr int MaxConvClasses = 4;
 
 struct CMatMulArgs {
 	const float* A;
@@ -63,6 +76,9 @@ struct CMatMulArgs {
 	// ( ho * StrideH - PadH + kh * DilH ) / UpH and only exists where that division is exact (values <= 1: no division)
 	int UpH, UpW;
 	int ManySlices; // the reduction is far longer than the output is large: as many K slices as fill the device
+	// AM_ConvClasses: the dense result is [images][OutH][OutW][Ldc], DenseM pixels in all
+	int OutH, OutW, OutUpH, OutUpW, DenseM;
+	CConvClass Class[MaxConvClasses];
 	// epilogue of the fused blocks: C = act( A * B + bias ) + Residual; Residual has C's layout, may be C itself
 	CFusedActivation Act;
 	const float* Residual;
@@ -76,8 +92,18 @@ constexpr int Threads = 256;
 
 template<int BM, int BN, int WAVES_M, int WAVES_N, int AMODE, int BMODE, bool VEC>
 __global__ __launch_bounds__( Threads, 2 )
-void matMulKernel( const CMatMulArgs args )
+void matMulKernel( const CMatMulArgs launchArgs )
 {
+	constexpr bool IsClasses = ( AMODE == AM_ConvClasses );
+	CMatMulArgs args = launchArgs;
+	int outH0 = 0, outW0 = 0;
+	if constexpr( IsClasses ) {
+		const CConvClass& c = launchArgs.Class[blockIdx.y];
+		args.K = c.K; args.Ldb = c.K; args.B += c.BOffset;
+		args.Fh = c.Fh; args.Fw = c.Fw; args.PadH = c.PadH; args.PadW = c.PadW;
+		args.Ho = c.Ho; args.Wo = c.Wo; args.M = c.M;
+		outH0 = c.OutH0; outW0 = c.OutW0;
+	}
 	constexpr int KS = NH_KSTEP;           // K step per pipeline stage
 	constexpr int KQ = KS / 4;             // float4 slots along K of a K-major tile row
 	constexpr int LdsK = KS + 4;           // row pitch of a K-major tile in LDS
@@ -87,7 +113,7 @@ void matMulKernel( const CMatMulArgs args )
 	constexpr int MI = WM / 32;
 	constexpr int NI = WN / 32;
 	constexpr bool AK = ( AMODE != AM_RowsM );
-	constexpr bool IsConv = ( AMODE == AM_Conv || AMODE == AM_Conv1x1 );
+	constexpr bool IsConv = ( AMODE == AM_Conv || AMODE == AM_Conv1x1 || AMODE == AM_ConvClasses );
 	constexpr bool IsConvRows = ( AMODE == AM_ConvRows );
 	constexpr bool BK = ( BMODE == BM_RowsK );
 	constexpr int APitchX = BM + 4, BPitchX = BN + 4;
@@ -121,6 +147,12 @@ void matMulKernel( const CMatMulArgs args )
 	float* C = args.C + batch * args.BatchStrideC;
 	const int M = args.M, N = args.N, K = args.K;
 	const int kStart = split * args.StepsPerSplit * NH_KSTEP; // first k of this workgroup's K slice
+	if constexpr( IsClasses ) {
+		// classes differ in their row and reduction counts; the grid is sized for the largest
+		if( m0 >= M || ( split > 0 && kStart >= K ) ) {
+			return;
+		}
+	}
 	const __amdgpu_buffer_rsrc_t bufA = makeBuffer( A );
 	const __amdgpu_buffer_rsrc_t bufB = makeBuffer( B );
 
@@ -560,13 +592,16 @@ void matMulKernel( const CMatMulArgs args )
 	constexpr int Groups = KS / 8;
 	float4 rA[ASlots], rB[BSlots];
 	CFrag frag[2];
-	loadTiles( kStart, rA, rB );
-	storeTiles( 0, rA, rB );
-	if( kSteps > 1 ) {
-		loadTiles( kStart + KS, rA, rB );
+	// a class without taps ( kSteps == 0 ) only writes the free term
+	if( !IsClasses || kSteps > 0 ) {
+		loadTiles( kStart, rA, rB );
+		storeTiles( 0, rA, rB );
+		if( kSteps > 1 ) {
+			loadTiles( kStart + KS, rA, rB );
+		}
+		__syncthreads();
+		readFrag( 0, 0, frag[0] );
 	}
-	__syncthreads();
-	readFrag( 0, 0, frag[0] );
 	int cur = 0;
 	for( int ks = 0; ks < kSteps; ++ks ) {
 		const int nxt = cur == 2 ? 0 : cur + 1;
@@ -607,7 +642,15 @@ void matMulKernel( const CMatMulArgs args )
 			for( int r = 0; r < 16; ++r ) {
 				const int m = m0 + waveM * WM + mi * 32 + ( r >> 2 ) * 8 + half * 4 + ( r & 3 );
 				if( m < M ) {
-					float* p = C + static_cast<long long>( m ) * args.Ldc + n;
+					long long row = m;
+					if constexpr( IsClasses ) {
+						const int wo = m % args.Wo;
+						const int t = m / args.Wo;
+						const int ho = t % args.Ho;
+						row = ( static_cast<long long>( t / args.Ho ) * args.OutH + outH0 + ho * args.OutUpH ) * args.OutW
+							+ outW0 + wo * args.OutUpW;
+					}
+					float* p = C + row * args.Ldc + n;
 					if( args.SplitK > 1 ) {
 						// C was set to the free term (or left as is when accumulating) before the launch
 						unsafeAtomicAdd( p, acc[mi][ni][r] );
@@ -618,7 +661,7 @@ void matMulKernel( const CMatMulArgs args )
 						}
 						v = applyActivation( v, args.Act );
 						if( args.Residual != nullptr ) {
-							v += args.Residual[batch * args.BatchStrideC + static_cast<long long>( m ) * args.Ldc + n];
+							v += args.Residual[batch * args.BatchStrideC + row * args.Ldc + n];
 						}
 						*p = v;
 					}
@@ -704,7 +747,11 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 	args.StepsPerSplit = ceilDiv( totalSteps, splits );
 	args.SplitK = ceilDiv( totalSteps, args.StepsPerSplit );
 	if( args.SplitK > 1 && !args.Accumulate ) {
-		const int rc = presetResult( stream, args, batch );
+		CMatMulArgs dense = args;
+		if( AMODE == AM_ConvClasses ) {
+			dense.M = args.DenseM; // the classes interleave in one dense result
+		}
+		const int rc = presetResult( stream, dense, AMODE == AM_ConvClasses ? 1 : batch );
 		if( rc != NH_OK ) {
 			return rc;
 		}
@@ -1046,9 +1093,115 @@ __global__ __launch_bounds__( 256 ) void swapFilterChannelsKernel( const float* 
 // inputDiff[n,hi,wi,ci] = freeTerm[ci] + sum over ( kh, kw, co ) of outputDiff[n, (hi+p-kh*d)/s, (wi+p-kw*d)/s, co] *
 // filter[co,kh,kw,ci], the terms whose divisions are exact and in range: the forward kernel on the output gradient as
 // its image, with padding -p, dilation -d, the division by the stride, and the filter with its channel axes swapped.
+// Which class a filter tap belongs to and where it goes inside the class's filter
+struct CTapClasses {
+	int StrideH, StrideW, DilH, DilW;
+	int FirstH[2], FirstW[2];   // by residue: the first tap of the class along that axis
+	int CountW[2];              // by residue: taps of the class along the width
+	int K[MaxConvClasses];
+	long long BOffset[MaxConvClasses];
+};
+
+// filter [Cout][Fh][Fw][Cin] -> per class [Cin][its taps][Cout]
+__global__ __launch_bounds__( 256 ) void packClassFiltersKernel( const float* filter, float* packed, int cout, int fh, int fw,
+	int cin, const CTapClasses t )
+{
+	const int total = cout * fh * fw * cin;
+	for( int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256 ) {
+		const int ci = i % cin;
+		const int kw = ( i / cin ) % fw;
+		const int kh = ( i / ( cin * fw ) ) % fh;
+		const int co = i / ( cin * fw * fh );
+		const int rh = ( kh * t.DilH ) % t.StrideH;
+		const int rw = ( kw * t.DilW ) % t.StrideW;
+		const int cls = rh * t.StrideW + rw;
+		const int tap = ( kh - t.FirstH[rh] ) / t.StrideH * t.CountW[rw] + ( kw - t.FirstW[rw] ) / t.StrideW;
+		packed[t.BOffset[cls] + static_cast<long long>( ci ) * t.K[cls] + tap * cout + co] = filter[i];
+	}
+}
+
+static int gcd( int a, int b ) { return b == 0 ? a : gcd( b, a % b ); }
+
+// The strided case of convBackwardData: true when it took the launch. A pixel hi of the input meets tap kh only when
+// hi + pad - kh * dil is a multiple of the stride, so the pixels fall into stride^2 classes by ( hi + pad ) mod stride,
+// each with its own subset of the taps; per class the sum is a stride-1 convolution without a single masked tap.
+static bool convBackwardDataByClasses( hipStream_t stream, const nhConvDesc& d, const float* outputDiff, const float* filter,
+	const float* freeTerm, float* inputDiff, float* packedFilter, int& rc )
+{
+	const int sh = d.strideHeight, sw = d.strideWidth;
+	if( ( sh == 1 && sw == 1 ) || sh > 2 || sw > 2 || gcd( d.dilationHeight, sh ) != 1 || gcd( d.dilationWidth, sw ) != 1 ) {
+		return false;
+	}
+	CMatMulArgs args = {};
+	CTapClasses taps = {};
+	taps.StrideH = sh; taps.StrideW = sw; taps.DilH = d.dilationHeight; taps.DilW = d.dilationWidth;
+	// per axis and residue r: first pixel of the class, pixel count, first tap, tap count, source offset of pixel 0 / tap 0
+	struct CAxis { int First, Count, FirstTap, Taps, Base; };
+	auto axis = []( int size, int pad, int stride, int dil, int filterSize, int r ) {
+		CAxis a = {};
+		a.First = ( ( r - pad ) % stride + stride ) % stride;
+		a.Count = a.First < size ? ( size - a.First + stride - 1 ) / stride : 0;
+		a.FirstTap = 0;
+		while( ( a.FirstTap * dil ) % stride != r ) {
+			++a.FirstTap; // exists below stride: dil and stride are coprime
+		}
+		a.Taps = a.FirstTap < filterSize ? ( filterSize - a.FirstTap + stride - 1 ) / stride : 0;
+		a.Base = ( a.First + pad - a.FirstTap * dil ) / stride; // exact
+		return a;
+	};
+	long long offset = 0;
+	int maxM = 0, maxK = 0;
+	for( int rh = 0; rh < sh; ++rh ) {
+		const CAxis h = axis( d.height, d.paddingHeight, sh, d.dilationHeight, d.filterHeight, rh );
+		taps.FirstH[rh] = h.FirstTap;
+		for( int rw = 0; rw < sw; ++rw ) {
+			const CAxis w = axis( d.width, d.paddingWidth, sw, d.dilationWidth, d.filterWidth, rw );
+			taps.FirstW[rw] = w.FirstTap;
+			taps.CountW[rw] = w.Taps;
+			CConvClass& c = args.Class[rh * sw + rw];
+			c.Fh = h.Taps; c.Fw = w.Taps;
+			c.K = h.Taps * w.Taps * d.filterCount;
+			// source pixel of result pixel j through tap t: Base + j - t * dil
+			c.PadH = -h.Base; c.PadW = -w.Base;
+			c.Ho = h.Count; c.Wo = w.Count;
+			c.M = d.batch * h.Count * w.Count;
+			c.OutH0 = h.First; c.OutW0 = w.First;
+			c.BOffset = offset;
+			taps.K[rh * sw + rw] = c.K;
+			taps.BOffset[rh * sw + rw] = offset;
+			offset += static_cast<long long>( c.K ) * d.channels;
+			maxM = c.M > maxM ? c.M : maxM;
+			maxK = c.K > maxK ? c.K : maxK;
+		}
+	}
+	const int filterSize = d.filterCount * d.filterHeight * d.filterWidth * d.channels;
+	hipLaunchKernelGGL( packClassFiltersKernel, dim3( ceilDiv( filterSize, 1024 ) ), dim3( 256 ), 0, stream,
+		filter, packedFilter, d.filterCount, d.filterHeight, d.filterWidth, d.channels, taps );
+	args.A = outputDiff; args.B = packedFilter; args.C = inputDiff; args.Bias = freeTerm;
+	args.M = maxM; args.N = d.channels; args.K = maxK;
+	args.Lda = 0; args.Ldb = maxK; args.Ldc = d.channels;
+	args.H = d.resultHeight; args.W = d.resultWidth; args.Cin = d.filterCount;
+	args.StrideH = 1; args.StrideW = 1;
+	args.DilH = -d.dilationHeight; args.DilW = -d.dilationWidth;
+	args.OutH = d.height; args.OutW = d.width; args.OutUpH = sh; args.OutUpW = sw;
+	args.DenseM = d.batch * d.height * d.width;
+	const bool vec = isAligned16( outputDiff ) && isAligned16( packedFilter ) && d.filterCount % 4 == 0
+		&& fitsBuffer( 1, 0, static_cast<long long>( d.batch ) * d.resultHeight * d.resultWidth * d.filterCount )
+		&& fitsBuffer( 1, 0, static_cast<long long>( filterSize ) );
+	rc = launchMatMul<AM_ConvClasses, BM_RowsK>( stream, args, sh * sw, vec );
+	return true;
+}
+
 int convBackwardData( hipStream_t stream, const nhConvDesc& d, const float* outputDiff, const float* filter,
 	const float* freeTerm, float* inputDiff, float* swappedFilter )
 {
+	if( static_cast<long long>( d.batch ) * d.height * d.width == 0 || d.channels == 0 ) {
+		return NH_OK;
+	}
+	int rc = NH_OK;
+	if( convBackwardDataByClasses( stream, d, outputDiff, filter, freeTerm, inputDiff, swappedFilter, rc ) ) {
+		return rc;
+	}
 	const int taps = d.filterHeight * d.filterWidth;
 	const int filterSize = d.filterCount * taps * d.channels;
 	hipLaunchKernelGGL( swapFilterChannelsKernel, dim3( ceilDiv( filterSize, 1024 ) ), dim3( 256 ), 0, stream,

@@ -109,6 +109,33 @@ def main():
     conv("cfg5 conv1", 64, 32, 512, 1, 64, 3, 1, 1)
     conv("cfg5 conv3", 64, 16, 256, 64, 128, 3, 1, 1)
 
+    # ---- gradients of the convolutions (a training step of config 1 / 2)
+    def conv_grad(tag, n, h, w, cin, cout, f, p, s):
+        d = neoml_amd.ConvDesc(n, h, w, cin, cout, f, f, p, p, s, s, 1, 1, 0, 0)
+        neoml_amd.check(lib.nhInitBlobConvolution(ctypes.byref(d)))
+        x, flt = rand(n, h, w, cin), rand(cout, f, f, cin) * 0.05
+        g = rand(n, d.resultHeight, d.resultWidth, cout)
+        dx, dflt = empty(n, h, w, cin), torch.zeros_like(flt)
+        size = ctypes.c_size_t(0)
+        neoml_amd.check(lib.nhBlobConvolutionBackwardWorkspaceSize(ctypes.byref(d), ctypes.byref(size)))
+        work = torch.empty((size.value + 15) // 4 + 4, dtype=torch.float32, device=dev)
+        fl = 2 * n * d.resultHeight * d.resultWidth * cout * f * f * cin
+        by = 4 * (x.numel() + g.numel() + flt.numel())
+        shape = "%s %dx%dx%dx%d->%d %dx%d/%d" % (tag, n, h, w, cin, cout, f, f, s)
+        measure("BlobConvolutionBackward " + shape, lambda: lib.nhBlobConvolutionBackward(
+            stream, ctypes.byref(d), P(g), P(flt), None, P(dx), P(work), size.value), fl, by, by)
+        measure("BlobConvolutionLearnAdd " + shape, lambda: lib.nhBlobConvolutionLearnAdd(
+            stream, ctypes.byref(d), P(x), P(g), P(dflt)), fl, by, by)
+
+    conv_grad("cfg1", 32, 32, 32, 64, 64, 3, 1, 1)
+    conv_grad("cfg2 stem", 64, 224, 224, 3, 64, 7, 3, 2)
+    conv_grad("cfg2 s1", 64, 56, 56, 64, 64, 3, 1, 1)
+    conv_grad("cfg2 s2", 64, 28, 28, 128, 128, 3, 1, 1)
+    conv_grad("cfg2 s3", 64, 14, 14, 256, 256, 3, 1, 1)
+    conv_grad("cfg2 s4", 64, 7, 7, 512, 512, 3, 1, 1)
+    conv_grad("cfg2 s2 down", 64, 56, 56, 64, 128, 3, 1, 2)
+    conv_grad("cfg2 s2 short", 64, 56, 56, 64, 128, 1, 0, 2)
+
     # ---- matrix products (config 2 FC, config 4, config 5)
     def gemm_nt(tag, m, n, k):
         a, b, c = rand(m, k), rand(n, k), empty(m, n)
@@ -174,6 +201,22 @@ def main():
     pool("cfg5", 64, 32, 512, 64, 2, 2, 2, 2)
     pool("cfg2", 64, 114, 114, 64, 3, 3, 2, 2, mean=True)
 
+    def pool_grad(n, h, w, c, f, s_):
+        d = neoml_amd.PoolingDesc(n, h, w, c, f, f, s_, s_, 0, 0)
+        neoml_amd.check(lib.nhInitPooling(ctypes.byref(d)))
+        x, y = rand(n, h, w, c), empty(n, d.resultHeight, d.resultWidth, c)
+        idx = torch.empty(y.shape, dtype=torch.int32, device=dev)
+        neoml_amd.check(lib.nhBlobMaxPooling(stream, ctypes.byref(d), P(x), P(idx), P(y)))
+        g, dx = rand(*y.shape), empty(n, h, w, c)
+        measure("BlobMaxPoolingBackward cfg2 %dx%dx%dx%d %dx%d/%d" % (n, h, w, c, f, f, s_),
+                lambda: lib.nhBlobMaxPoolingBackward(stream, ctypes.byref(d), P(g), P(idx), P(dx)),
+                0, 4 * (2 * g.numel() + dx.numel()), 4 * (2 * g.numel() + dx.numel()))
+        measure("BlobMeanPoolingBackward cfg2 %dx%dx%dx%d %dx%d/%d" % (n, h, w, c, f, f, s_),
+                lambda: lib.nhBlobMeanPoolingBackward(stream, ctypes.byref(d), P(g), P(dx)),
+                0, 4 * (g.numel() + dx.numel()), 4 * (g.numel() + dx.numel()))
+
+    pool_grad(64, 114, 114, 64, 3, 2)
+
     x, y = rand(64, 112, 112, 64), empty(64, 114, 114, 64)
     fd, td = neoml_amd.BlobDesc.of(1, 64, 1, 112, 112, 1, 64), neoml_amd.BlobDesc.of(1, 64, 1, 114, 114, 1, 64)
     measure("BlobResizeImage cfg2 pad 112->114 x64ch", lambda: lib.nhBlobResizeImage(
@@ -187,6 +230,7 @@ def main():
         measure("VectorReLU6 n=%d" % n, lambda: lib.nhVectorReLU(stream, P(a), P(c), n, P(six)), 0, 8 * n, 8 * n)
         measure("VectorAdd n=%d" % n, lambda: lib.nhVectorAdd(stream, P(a), P(b), P(c), n), 0, 12 * n, 12 * n)
         measure("VectorSigmoid n=%d" % n, lambda: lib.nhVectorSigmoid(stream, P(a), P(c), n), 0, 8 * n, 8 * n)
+        measure("VectorReLUDiff n=%d" % n, lambda: lib.nhVectorReLUDiff(stream, P(a), P(b), P(c), n, P(zero)), 0, 12 * n, 12 * n)
         measure("VectorEltwiseMultiply n=%d" % n, lambda: lib.nhVectorEltwiseMultiply(stream, P(a), P(b), P(c), n), 0, 12 * n, 12 * n)
         del a, b, c
     for n in (1 << 26, 1 << 28):

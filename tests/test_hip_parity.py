@@ -296,6 +296,15 @@ GPU_CONV_GRADIENT_CASES = CONV_CASES + [
     (1, 6, 5, 7, 9, 2, 4, 0, 3, 1, 1, 1, 1),
     (2, 12, 12, 8, 16, 3, 3, 0, 0, 3, 3, 1, 1),     # stride as large as the filter
     (8, 32, 32, 64, 64, 3, 3, 1, 1, 1, 1, 1, 1),    # many pixels: the filter gradient's reduction is split over the grid
+    # strided: the input gradient runs class by class of ( pixel + padding ) mod stride
+    (1, 11, 10, 8, 12, 3, 3, 0, 0, 2, 2, 3, 3),     # dilation 3 against stride 2
+    (2, 12, 12, 8, 16, 2, 2, 0, 0, 2, 2, 1, 1),     # one tap per class
+    (2, 13, 9, 4, 8, 3, 3, 1, 1, 2, 1, 1, 1),       # stride along the height only, odd size: classes of 7 and 6 rows
+    (2, 9, 14, 4, 8, 3, 4, 1, 2, 1, 2, 1, 1),       # stride along the width only
+    (1, 9, 9, 4, 8, 5, 5, 2, 2, 2, 2, 2, 2),        # dilation and stride share a factor: the masked form
+    (1, 13, 13, 4, 8, 3, 3, 1, 1, 3, 3, 1, 1),      # stride 3: the masked form
+    (1, 3, 3, 4, 8, 3, 3, 0, 0, 2, 2, 1, 1),        # a single window: classes without pixels of their own
+    (8, 14, 14, 256, 512, 3, 3, 1, 1, 2, 2, 1, 1),  # few tiles per class, long reduction: K slices over a preset result
 ]
 
 
