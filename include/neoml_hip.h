@@ -265,6 +265,13 @@ NH_API int nhInitBlobChannelwiseConvolution(nhConvDesc* desc_host);             
 NH_API int nhBlobChannelwiseConvolution(nhStream s, const nhConvDesc* desc_host, const float* source,
 	const float* filter, const float* freeTerm, float* result);                                      /* NME.h:770 */
 
+/* Gradients of the depthwise convolution. Backward: inputDiff = the gradient by the source. LearnAdd: filterDiff +=
+ * the gradient by the filter, freeTermDiff (may be null) += the sum of outputDiff over the pixels. */
+NH_API int nhBlobChannelwiseConvolutionBackward(nhStream s, const nhConvDesc* desc_host, const float* outputDiff,
+	const float* filter, float* inputDiff);                                                          /* NME.h:774 */
+NH_API int nhBlobChannelwiseConvolutionLearnAdd(nhStream s, const nhConvDesc* desc_host, const float* input,
+	const float* outputDiff, float* filterDiff, float* freeTermDiff);                                /* NME.h:778 */
+
 /* The fused blocks the graph optimizer emits for depthwise-separable networks (NME.h:1066-1072, layer classes
  * CMobileNetV2BlockLayer / CChannelwiseWith1x1Layer). Activations are TActivationFunction values reduced to what
  * the blocks support (src/CPU/Rowwise/CpuRowwiseCommon.h:79-86): ReLU with an optional upper threshold (param > 0),

@@ -195,6 +195,58 @@ void sumRowsKernel( float* result, const float* matrix, int height, int width, i
 	}
 }
 
+// The same sums for a tall matrix of few columns (the free-term gradient of a convolution: one row per pixel of the
+// batch). The 256 threads of a workgroup form 256 / groups row lanes of `groups` float4 columns, so that a wave reads
+// whole rows back to back; every lane keeps four loads in flight, the lanes meet in LDS, one atomic add per column.
+__global__ __launch_bounds__( 256 )
+void sumTallRowsKernel( float* result, const float* matrix, int height, int width, int groups, int rowsPerSlice )
+{
+	__shared__ float4 meet[256];
+	const int group = threadIdx.x % groups;
+	const int lane = threadIdx.x / groups;
+	const int lanes = 256 / groups;
+	const int b = blockIdx.y;
+	const int rowBegin = blockIdx.x * rowsPerSlice;
+	const int rowEnd = min( rowBegin + rowsPerSlice, height );
+	float4 sum[4];
+#pragma unroll
+	for( int j = 0; j < 4; ++j ) {
+		sum[j] = make_float4( 0.f, 0.f, 0.f, 0.f );
+	}
+	if( group * 4 < width ) {
+		const float* p = matrix + static_cast<long long>( b ) * height * width + group * 4;
+		int r = rowBegin + lane;
+		for( ; r + 3 * lanes < rowEnd; r += 4 * lanes ) {
+			float4 v[4];
+#pragma unroll
+			for( int j = 0; j < 4; ++j ) {
+				v[j] = *reinterpret_cast<const float4*>( p + static_cast<long long>( r + j * lanes ) * width );
+			}
+#pragma unroll
+			for( int j = 0; j < 4; ++j ) {
+				sum[j].x += v[j].x; sum[j].y += v[j].y; sum[j].z += v[j].z; sum[j].w += v[j].w;
+			}
+		}
+		for( ; r < rowEnd; r += lanes ) {
+			const float4 v = *reinterpret_cast<const float4*>( p + static_cast<long long>( r ) * width );
+			sum[0].x += v.x; sum[0].y += v.y; sum[0].z += v.z; sum[0].w += v.w;
+		}
+	}
+	meet[threadIdx.x] = make_float4( sum[0].x + sum[1].x + sum[2].x + sum[3].x, sum[0].y + sum[1].y + sum[2].y + sum[3].y,
+		sum[0].z + sum[1].z + sum[2].z + sum[3].z, sum[0].w + sum[1].w + sum[2].w + sum[3].w );
+	__syncthreads();
+	// one thread per column adds up its lanes
+	const int c = threadIdx.x;
+	if( c < width ) {
+		const float* column = reinterpret_cast<const float*>( meet ) + c;
+		float total = 0.f;
+		for( int l = 0; l < lanes; ++l ) {
+			total += column[l * groups * 4];
+		}
+		atomicAdd( result + static_cast<long long>( b ) * width + c, total );
+	}
+}
+
 // Softmax / log-sum-exp of one row per wavefront. Rows of up to 64 * CACHE elements stay in registers between
 // the three passes (max, sum of exp, scale); longer rows are read again from memory.
 // The formula follows the reference: exp( x - max ) * ( 1 / sum ) (src/CPU/CpuMathEngineBlas.cpp:1131-1159).
@@ -431,6 +483,29 @@ static int sumMatrixRowsImpl( nhStream s, int batchSize, float* result, const fl
 	int matrixWidth, bool accumulate )
 {
 	if( batchSize == 0 || matrixWidth == 0 ) {
+		return NH_OK;
+	}
+	if( matrixWidth % 4 == 0 && matrixWidth <= 256 && matrixHeight >= 2048 && batchSize <= 65535 && isAligned16( matrix ) ) {
+		int groups = 1;
+		while( groups * 4 < matrixWidth ) {
+			groups *= 2;
+		}
+		const int lanes = 256 / groups;
+		// about 2048 workgroups, at least 16 rows per lane
+		int slices = 2048 / batchSize > 0 ? 2048 / batchSize : 1;
+		const int most = matrixHeight / ( 16 * lanes ) > 0 ? matrixHeight / ( 16 * lanes ) : 1;
+		slices = slices < most ? slices : most;
+		const int rowsPerSlice = ceilDiv( matrixHeight, slices );
+		slices = ceilDiv( matrixHeight, rowsPerSlice );
+		if( !accumulate ) {
+			const int rc = nhVectorFill( s, result, 0.f, batchSize * matrixWidth );
+			if( rc != NH_OK ) {
+				return rc;
+			}
+		}
+		hipLaunchKernelGGL( sumTallRowsKernel, dim3( slices, batchSize ), dim3( 256 ), 0, toStream( s ),
+			result, matrix, matrixHeight, matrixWidth, groups, rowsPerSlice );
+		NH_LAUNCH_CHECK();
 		return NH_OK;
 	}
 	const int colBlocks = ceilDiv( matrixWidth, 256 );

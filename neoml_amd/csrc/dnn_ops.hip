@@ -980,6 +980,138 @@ void meanPoolingBackwardKernel( const nhPoolingDesc d, const float* resultDiff, 
 	}
 }
 
+// Gradient of the channelwise convolution by its input: every input pixel gathers, tap by tap, the output pixels whose
+// window holds it: ( hi + pad - kh ) / stride where that division is exact and in range.
+template<int VECW>
+__global__ __launch_bounds__( 256 )
+void channelwiseConvBackwardKernel( const nhConvDesc d, const float* outputDiff, const float* filter, float* inputDiff,
+	long long totalItems )
+{
+	typedef CChanVec<VECW> V;
+	typedef typename V::Type T;
+	const int cg = d.channels / VECW;
+	const long long step = static_cast<long long>( gridDim.x ) * 256;
+	for( long long item = blockIdx.x * 256LL + threadIdx.x; item < totalItems; item += step ) {
+		long long t = item;
+		const int c = static_cast<int>( t % cg ) * VECW; t /= cg;
+		const int wi = static_cast<int>( t % d.width ); t /= d.width;
+		const int hi = static_cast<int>( t % d.height );
+		const long long n = t / d.height;
+		const float* image = outputDiff + n * d.resultHeight * d.resultWidth * d.channels + c;
+		T acc = V::zero();
+		for( int kh = 0; kh < d.filterHeight; ++kh ) {
+			const int hs = hi + d.paddingHeight - kh;
+			if( hs < 0 || hs % d.strideHeight != 0 || hs / d.strideHeight >= d.resultHeight ) {
+				continue;
+			}
+			const float* row = image + static_cast<long long>( hs / d.strideHeight ) * d.resultWidth * d.channels;
+			for( int kw = 0; kw < d.filterWidth; ++kw ) {
+				const int ws = wi + d.paddingWidth - kw;
+				if( ws < 0 || ws % d.strideWidth != 0 || ws / d.strideWidth >= d.resultWidth ) {
+					continue;
+				}
+				acc = V::fma( V::load( row + ( ws / d.strideWidth ) * d.channels ),
+					V::load( filter + ( kh * d.filterWidth + kw ) * d.channels + c ), acc );
+			}
+		}
+		V::store( inputDiff + item * VECW, acc );
+	}
+}
+
+template<int VECW> struct CChanAtomic;
+template<> struct CChanAtomic<4> {
+	static __device__ __forceinline__ void add( float* p, float4 v )
+	{
+		unsafeAtomicAdd( p, v.x ); unsafeAtomicAdd( p + 1, v.y ); unsafeAtomicAdd( p + 2, v.z ); unsafeAtomicAdd( p + 3, v.w );
+	}
+	static __device__ __forceinline__ float4 sum( float4 a, float4 b ) { return make_float4( a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w ); }
+};
+template<> struct CChanAtomic<1> {
+	static __device__ __forceinline__ void add( float* p, float v ) { unsafeAtomicAdd( p, v ); }
+	static __device__ __forceinline__ float sum( float a, float b ) { return a + b; }
+};
+
+// Gradient of the channelwise convolution by its filter (and free term): sums over every output pixel of the batch.
+// A workgroup owns a block of GROUPS channel groups and a slice of the output pixels; its 256 / GROUPS pixel lanes keep
+// the TAPS + 1 sums of their channel group in registers, meet in LDS and leave with one atomic add per sum.
+// TAPS == 0: any filter size, one tap per pass over the slice.
+template<int VECW, int TAPS>
+__global__ __launch_bounds__( 256 )
+void channelwiseConvLearnKernel( const nhConvDesc d, const float* input, const float* outputDiff, float* filterDiff,
+	float* freeTermDiff, int groups, int groupBlocks, long long pixelsPerSlice )
+{
+	typedef CChanVec<VECW> V;
+	typedef CChanAtomic<VECW> At;
+	typedef typename V::Type T;
+	constexpr int Sums = ( TAPS > 0 ? TAPS : 1 ) + 1;
+	__shared__ T meet[256];
+	const int lanes = 256 / groups;
+	const int group = threadIdx.x % groups;
+	const int lane = threadIdx.x / groups;
+	const int cgTotal = d.channels / VECW;
+	const int cgIndex = ( blockIdx.x % groupBlocks ) * groups + group;
+	const bool active = cgIndex < cgTotal && lane < lanes;
+	const int c = cgIndex * VECW;
+	const long long slice = blockIdx.x / groupBlocks;
+	const long long pixels = static_cast<long long>( d.batch ) * d.resultHeight * d.resultWidth;
+	const long long first = slice * pixelsPerSlice;
+	const long long last = min( first + pixelsPerSlice, pixels );
+	const int taps = d.filterHeight * d.filterWidth;
+	const int passes = TAPS > 0 ? 1 : taps;
+	for( int pass = 0; pass < passes; ++pass ) {
+		T sums[Sums];
+#pragma unroll
+		for( int i = 0; i < Sums; ++i ) {
+			sums[i] = V::zero();
+		}
+		if( active ) {
+			for( long long pixel = first + lane; pixel < last; pixel += lanes ) {
+				const int wo = static_cast<int>( pixel % d.resultWidth );
+				const long long t = pixel / d.resultWidth;
+				const int ho = static_cast<int>( t % d.resultHeight );
+				const long long n = t / d.resultHeight;
+				const T g = V::load( outputDiff + pixel * d.channels + c );
+				sums[Sums - 1] = At::sum( sums[Sums - 1], g );
+				const float* image = input + n * d.height * d.width * d.channels + c;
+				const int hi0 = ho * d.strideHeight - d.paddingHeight;
+				const int wi0 = wo * d.strideWidth - d.paddingWidth;
+				if( TAPS > 0 ) {
+#pragma unroll
+					for( int tap = 0; tap < ( TAPS > 0 ? TAPS : 1 ); ++tap ) {
+						const int hi = hi0 + tap / 3, wi = wi0 + tap % 3; // TAPS == 9: the 3x3 filter
+						if( hi >= 0 && hi < d.height && wi >= 0 && wi < d.width ) {
+							sums[tap] = V::fma( V::load( image + ( static_cast<long long>( hi ) * d.width + wi ) * d.channels ), g, sums[tap] );
+						}
+					}
+				} else {
+					const int hi = hi0 + pass / d.filterWidth, wi = wi0 + pass % d.filterWidth;
+					if( hi >= 0 && hi < d.height && wi >= 0 && wi < d.width ) {
+						sums[0] = V::fma( V::load( image + ( static_cast<long long>( hi ) * d.width + wi ) * d.channels ), g, sums[0] );
+					}
+				}
+			}
+		}
+		// the lanes of a channel group meet: lane 0 adds up and leaves
+#pragma unroll
+		for( int i = 0; i < Sums; ++i ) {
+			__syncthreads();
+			meet[threadIdx.x] = sums[i];
+			__syncthreads();
+			if( active && lane == 0 ) {
+				T total = meet[group];
+				for( int l = 1; l < lanes; ++l ) {
+					total = At::sum( total, meet[l * groups + group] );
+				}
+				if( i < Sums - 1 ) {
+					At::add( filterDiff + ( ( TAPS > 0 ? i : pass ) ) * d.channels + c, total );
+				} else if( freeTermDiff != nullptr && pass == 0 ) {
+					At::add( freeTermDiff + c, total );
+				}
+			}
+		}
+	}
+}
+
 __global__ void addTwoVectorsKernel( const float* a, const float* b, float* out, int n )
 {
 	const int i = blockIdx.x * 256 + threadIdx.x;
@@ -1346,6 +1478,85 @@ int nhBlobMeanPoolingBackward( nhStream s, const nhPoolingDesc* d, const float* 
 	blocks = blocks > 1048576 ? 1048576 : blocks;
 	hipLaunchKernelGGL( meanPoolingBackwardKernel, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
 		*d, resultDiff, sourceDiff, total );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+static int checkedChannelwiseDesc( const nhConvDesc* d )
+{
+	NH_REQUIRE( d != nullptr );
+	nhConvDesc check = *d;
+	const int rc = nhInitBlobChannelwiseConvolution( &check );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( check.resultHeight == d->resultHeight && check.resultWidth == d->resultWidth );
+	return NH_OK;
+}
+
+int nhBlobChannelwiseConvolutionBackward( nhStream s, const nhConvDesc* d, const float* outputDiff, const float* filter,
+	float* inputDiff )
+{
+	const int rc = checkedChannelwiseDesc( d );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( outputDiff != nullptr && filter != nullptr && inputDiff != nullptr );
+	if( d->batch == 0 ) {
+		return NH_OK;
+	}
+	const bool vec = d->channels % 4 == 0 && isAligned16( outputDiff ) && isAligned16( filter ) && isAligned16( inputDiff );
+	const long long items = static_cast<long long>( d->batch ) * d->height * d->width * ( vec ? d->channels / 4 : d->channels );
+	long long blocks = ( items + 255 ) / 256;
+	blocks = blocks > 1048576 ? 1048576 : blocks;
+	if( vec ) {
+		hipLaunchKernelGGL( channelwiseConvBackwardKernel<4>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			*d, outputDiff, filter, inputDiff, items );
+	} else {
+		hipLaunchKernelGGL( channelwiseConvBackwardKernel<1>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			*d, outputDiff, filter, inputDiff, items );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+int nhBlobChannelwiseConvolutionLearnAdd( nhStream s, const nhConvDesc* d, const float* input, const float* outputDiff,
+	float* filterDiff, float* freeTermDiff )
+{
+	const int rc = checkedChannelwiseDesc( d );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( input != nullptr && outputDiff != nullptr && filterDiff != nullptr );
+	if( d->batch == 0 ) {
+		return NH_OK;
+	}
+	const bool vec = d->channels % 4 == 0 && isAligned16( input ) && isAligned16( outputDiff );
+	const int cg = vec ? d->channels / 4 : d->channels;
+	// channel groups per workgroup: a power of two up to 64, so that a wave reads whole runs of channels
+	int groups = 1;
+	while( groups < cg && groups < 64 ) {
+		groups *= 2;
+	}
+	const int groupBlocks = ceilDiv( cg, groups );
+	const long long pixels = static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth;
+	// about 2048 workgroups, each lane at least 8 pixels of its own
+	const int lanes = 256 / groups;
+	long long slices = 2048 / groupBlocks > 0 ? 2048 / groupBlocks : 1;
+	const long long most = pixels / ( 8LL * lanes ) > 0 ? pixels / ( 8LL * lanes ) : 1;
+	slices = slices < most ? slices : most;
+	const long long pixelsPerSlice = ( pixels + slices - 1 ) / slices;
+	slices = ( pixels + pixelsPerSlice - 1 ) / pixelsPerSlice;
+	const dim3 grid( static_cast<unsigned>( slices * groupBlocks ) );
+	const bool is3x3 = d->filterHeight == 3 && d->filterWidth == 3;
+#define NH_LAUNCH_LEARN( VECW, TAPS ) hipLaunchKernelGGL( ( channelwiseConvLearnKernel<VECW, TAPS> ), grid, dim3( 256 ), 0, \
+	toStream( s ), *d, input, outputDiff, filterDiff, freeTermDiff, groups, groupBlocks, pixelsPerSlice )
+	if( vec ) {
+		if( is3x3 ) { NH_LAUNCH_LEARN( 4, 9 ); } else { NH_LAUNCH_LEARN( 4, 0 ); }
+	} else {
+		if( is3x3 ) { NH_LAUNCH_LEARN( 1, 9 ); } else { NH_LAUNCH_LEARN( 1, 0 ); }
+	}
+#undef NH_LAUNCH_LEARN
 	NH_LAUNCH_CHECK();
 	return NH_OK;
 }

@@ -652,6 +652,22 @@ static nhPoolingDesc makePoolingDesc( const CBlobDesc& source, int filterHeight,
 	return d;
 }
 
+void CHipMathEngine::BlobChannelwiseConvolutionBackward( const CChannelwiseConvolutionDesc& desc,
+	const CConstFloatHandle& source, const CConstFloatHandle& filter, const CFloatHandle& result )
+{
+	const CHipChannelwiseConvolutionDesc& d = static_cast<const CHipChannelwiseConvolutionDesc&>( desc );
+	NH_CALL( nhBlobChannelwiseConvolutionBackward( stream, &d.D, raw( source ), raw( filter ), raw( result ) ) );
+}
+
+void CHipMathEngine::BlobChannelwiseConvolutionLearnAdd( const CChannelwiseConvolutionDesc& desc,
+	const CConstFloatHandle& input, const CConstFloatHandle& outputDiff, const CFloatHandle& filterDiff,
+	const CFloatHandle* freeTermDiff )
+{
+	const CHipChannelwiseConvolutionDesc& d = static_cast<const CHipChannelwiseConvolutionDesc&>( desc );
+	NH_CALL( nhBlobChannelwiseConvolutionLearnAdd( stream, &d.D, raw( input ), raw( outputDiff ), raw( filterDiff ),
+		freeTermDiff != nullptr ? raw( *freeTermDiff ) : nullptr ) );
+}
+
 CMaxPoolingDesc* CHipMathEngine::InitMaxPooling( const CBlobDesc& source, int filterHeight, int filterWidth,
 	int strideHeight, int strideWidth, const CBlobDesc& result )
 {

@@ -214,6 +214,10 @@ public:
 		const CBlobDesc& output ) override;
 	void BlobChannelwiseConvolution( const CChannelwiseConvolutionDesc& desc, const CConstFloatHandle& source,
 		const CConstFloatHandle& filter, const CConstFloatHandle* freeTerm, const CFloatHandle& result ) override;
+	void BlobChannelwiseConvolutionBackward( const CChannelwiseConvolutionDesc& desc, const CConstFloatHandle& source,
+		const CConstFloatHandle& filter, const CFloatHandle& result ) override;
+	void BlobChannelwiseConvolutionLearnAdd( const CChannelwiseConvolutionDesc& desc, const CConstFloatHandle& input,
+		const CConstFloatHandle& outputDiff, const CFloatHandle& filterDiff, const CFloatHandle* freeTermDiff ) override;
 	CMaxPoolingDesc* InitMaxPooling( const CBlobDesc& source, int filterHeight, int filterWidth,
 		int strideHeight, int strideWidth, const CBlobDesc& result ) override;
 	void BlobMaxPooling( const CMaxPoolingDesc& desc, const CConstFloatHandle& source,

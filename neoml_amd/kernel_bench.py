@@ -262,6 +262,9 @@ def main():
     mv, mi = empty(8192), torch.empty(8192, dtype=torch.int32, device=dev)
     measure("FindMaxValueInRows 8192x101", lambda: lib.nhFindMaxValueInRows(stream, P(s_in), 8192, 101, P(mv), P(mi), 8192),
             0, 4 * 8192 * 101, 4 * 8192 * 101)
+    t_in, t_out = rand(64 * 56 * 56, 64), empty(64)
+    measure("SumMatrixRowsAdd free-term gradient 200704x64", lambda: lib.nhSumMatrixRowsAdd(stream, 1, P(t_out), P(t_in), 64 * 56 * 56, 64),
+            0, 4 * t_in.numel(), 4 * t_in.numel())
     g_in, g_out = rand(64, 49, 512), empty(64, 512)
     measure("SumMatrixRows cfg2 global mean 64x49x512", lambda: lib.nhSumMatrixRows(stream, 64, P(g_out), P(g_in), 49, 512),
             0, 4 * g_in.numel(), 4 * g_in.numel())

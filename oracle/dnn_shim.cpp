@@ -168,7 +168,7 @@ static CPtr<CConvLayer> conv( CDnn& dnn, IMathEngine& e, const CString& name, CB
 	return layer;
 }
 
-static CBaseLayer* buildResNet18( CDnn& dnn, IMathEngine& e, CBaseLayer& source, int classes )
+static CBaseLayer* buildResNet18( CDnn& dnn, IMathEngine& e, CBaseLayer& source, int classes, bool withSoftmax = true )
 {
 	CPtr<CConvLayer> stem = conv( dnn, e, "stem", source, 64, 7, 3, 2 );
 	CPtr<CReLULayer> relu0 = add( dnn, new CReLULayer( e ), "stem_relu", *stem );
@@ -204,6 +204,9 @@ static CBaseLayer* buildResNet18( CDnn& dnn, IMathEngine& e, CBaseLayer& source,
 	CPtr<CGlobalMeanPoolingLayer> gap = add( dnn, new CGlobalMeanPoolingLayer( e ), "gap", *last );
 	CPtr<CFullyConnectedLayer> fc = add( dnn, new CFullyConnectedLayer( e ), "fc", *gap );
 	fc->SetNumberOfElements( classes );
+	if( !withSoftmax ) {
+		return fc.Ptr(); // the loss layer applies its own softmax
+	}
 	CPtr<CSoftmaxLayer> softmax = add( dnn, new CSoftmaxLayer( e ), "softmax", *fc );
 	return softmax.Ptr();
 }
@@ -247,7 +250,7 @@ static CBaseLayer* invertedBlock( CDnn& dnn, IMathEngine& e, const CString& name
 	return x;
 }
 
-static CBaseLayer* buildSeparableNet( CDnn& dnn, IMathEngine& e, CBaseLayer& source, int classes )
+static CBaseLayer* buildSeparableNet( CDnn& dnn, IMathEngine& e, CBaseLayer& source, int classes, bool withSoftmax = true )
 {
 	CBaseLayer* x = conv( dnn, e, "stem", source, 16, 3, 1, 2 ).Ptr();
 	x = relu6( dnn, e, "stem_relu", *x );
@@ -259,6 +262,9 @@ static CBaseLayer* buildSeparableNet( CDnn& dnn, IMathEngine& e, CBaseLayer& sou
 	CPtr<CGlobalMeanPoolingLayer> gap = add( dnn, new CGlobalMeanPoolingLayer( e ), "gap", *x );
 	CPtr<CFullyConnectedLayer> fc = add( dnn, new CFullyConnectedLayer( e ), "fc", *gap );
 	fc->SetNumberOfElements( classes );
+	if( !withSoftmax ) {
+		return fc.Ptr(); // the loss layer applies its own softmax
+	}
 	CPtr<CSoftmaxLayer> softmax = add( dnn, new CSoftmaxLayer( e ), "softmax", *fc );
 	return softmax.Ptr();
 }
@@ -357,10 +363,14 @@ EXPORT int dnn_run( void* engine, int kind, int seed, int param, const int* dims
 // (classes); kind 1: Conv 3x3 p1 (8) - ReLU - MaxPool 2x2/2 - Conv 3x3 p1 stride 2 (16) - ReLU - FullyConnected (classes).
 // kind 2: Conv 3x3 p1 (16) - HSwish - [Conv 3x3 p1 (16) - ReLU - Conv 3x3 p1 (16)] + shortcut - ReLU - MeanPool 2x2/2 -
 // FullyConnected (classes); kind 3: Lstm (24 units, over BatchLength) - FullyConnected (classes) at every step.
+// kind 4: the ResNet-18-style network of dnn_run's kind 5; kind 5: the depthwise-separable network of its kind 6.
 // solver 0: CDnnSimpleGradientSolver, 1: CDnnAdaptiveGradientSolver (Adam), both with L2 regularisation 1e-3.
 // losses receives the loss of every step, output the logits of a final forward pass with the trained weights.
+// timedSteps > 0: that many further steps are timed (the loss is read after the last one, which waits for the device)
+// and *msPerStep receives the mean.
 EXPORT int dnn_train( void* engine, int kind, int solverKind, int seed, int classes, int steps, float learningRate,
-	const int* dims, const float* input, const float* labels, float* losses, float* output, int outputCapacity )
+	const int* dims, const float* input, const float* labels, float* losses, float* output, int outputCapacity,
+	int timedSteps, float* msPerStep )
 {
 	try {
 		IMathEngine& e = *static_cast<IMathEngine*>( engine );
@@ -374,7 +384,12 @@ EXPORT int dnn_train( void* engine, int kind, int solverKind, int seed, int clas
 		dnn.AddLayer( *labelSource );
 
 		CBaseLayer* last = source.Ptr();
-		if( kind == 0 ) {
+		CBaseLayer* logits = nullptr;
+		if( kind == 4 ) {
+			logits = buildResNet18( dnn, e, *source, classes, false );
+		} else if( kind == 5 ) {
+			logits = buildSeparableNet( dnn, e, *source, classes, false );
+		} else if( kind == 0 ) {
 			CPtr<CFullyConnectedLayer> fc1 = add( dnn, new CFullyConnectedLayer( e ), "fc1", *last );
 			fc1->SetNumberOfElements( 32 );
 			CPtr<CReLULayer> relu = add( dnn, new CReLULayer( e ), "relu", *fc1 );
@@ -404,8 +419,12 @@ EXPORT int dnn_train( void* engine, int kind, int solverKind, int seed, int clas
 			CPtr<CReLULayer> r2 = add( dnn, new CReLULayer( e ), "relu2", *c2 );
 			last = r2.Ptr();
 		}
-		CPtr<CFullyConnectedLayer> fc = add( dnn, new CFullyConnectedLayer( e ), "fc", *last );
-		fc->SetNumberOfElements( classes );
+		if( logits == nullptr ) {
+			CPtr<CFullyConnectedLayer> fcLast = add( dnn, new CFullyConnectedLayer( e ), "fc", *last );
+			fcLast->SetNumberOfElements( classes );
+			logits = fcLast.Ptr();
+		}
+		CBaseLayer* fc = logits;
 		CPtr<CCrossEntropyLossLayer> loss = new CCrossEntropyLossLayer( e );
 		loss->SetName( "loss" );
 		loss->Connect( 0, *fc );
@@ -448,6 +467,14 @@ EXPORT int dnn_train( void* engine, int kind, int solverKind, int seed, int clas
 		for( int i = 0; i < steps; ++i ) {
 			dnn.RunAndLearnOnce();
 			losses[i] = loss->GetLastLoss();
+		}
+		if( timedSteps > 0 ) {
+			const auto start = std::chrono::steady_clock::now();
+			for( int i = 0; i < timedSteps; ++i ) {
+				dnn.RunAndLearnOnce();
+			}
+			( void )loss->GetLastLoss();
+			*msPerStep = std::chrono::duration<float, std::milli>( std::chrono::steady_clock::now() - start ).count() / timedSteps;
 		}
 		dnn.RunOnce();
 		const CPtr<CDnnBlob>& result = sink->GetBlob();

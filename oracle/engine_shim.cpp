@@ -469,6 +469,59 @@ SHIM_API int shim_blob_channelwise_convolution( void* engine, const float* in, i
 	} );
 }
 
+// gradients of the channelwise convolution (NeoMathEngine.h:774-780); filterDiff and freeTermDiff (may be null) are
+// accumulated into
+SHIM_API int shim_blob_channelwise_convolution_backward( void* engine, const float* outDiff, int n, int h, int w, int c,
+	const float* filter, int fh, int fw, int ph, int pw, int sh, int sw, float* inDiff )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		const int ho = 1 + ( h - fh + 2 * ph ) / sh;
+		const int wo = 1 + ( w - fw + 2 * pw ) / sw;
+		const CBlobDesc inDesc = imageDesc( n, h, w, c ), filterDesc = imageDesc( 1, fh, fw, c ),
+			outDesc = imageDesc( n, ho, wo, c );
+		CFloatBlob grad( e, outDesc.BlobSize(), outDiff ), flt( e, filterDesc.BlobSize(), filter ), dst( e, inDesc.BlobSize() );
+		CChannelwiseConvolutionDesc* desc = e.InitBlobChannelwiseConvolution( inDesc, ph, pw, sh, sw, filterDesc, nullptr, outDesc );
+		try {
+			e.BlobChannelwiseConvolutionBackward( *desc, grad.Const(), flt.Const(), dst.Handle() );
+		} catch( ... ) {
+			delete desc;
+			throw;
+		}
+		delete desc;
+		dst.CopyTo( inDiff );
+	} );
+}
+
+SHIM_API int shim_blob_channelwise_convolution_learn_add( void* engine, const float* in, int n, int h, int w, int c,
+	const float* outDiff, int fh, int fw, int ph, int pw, int sh, int sw, float* filterDiff, float* freeTermDiff )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		const int ho = 1 + ( h - fh + 2 * ph ) / sh;
+		const int wo = 1 + ( w - fw + 2 * pw ) / sw;
+		const CBlobDesc inDesc = imageDesc( n, h, w, c ), filterDesc = imageDesc( 1, fh, fw, c ),
+			outDesc = imageDesc( n, ho, wo, c ), ftDesc = imageDesc( 1, 1, 1, c );
+		CFloatBlob src( e, inDesc.BlobSize(), in ), grad( e, outDesc.BlobSize(), outDiff ),
+			fd( e, filterDesc.BlobSize(), filterDiff ), ftd( e, c, freeTermDiff );
+		CChannelwiseConvolutionDesc* desc = e.InitBlobChannelwiseConvolution( inDesc, ph, pw, sh, sw, filterDesc,
+			freeTermDiff != nullptr ? &ftDesc : nullptr, outDesc );
+		const CFloatHandle ftdHandle = ftd.Handle();
+		try {
+			e.BlobChannelwiseConvolutionLearnAdd( *desc, src.Const(), grad.Const(), fd.Handle(),
+				freeTermDiff != nullptr ? &ftdHandle : nullptr );
+		} catch( ... ) {
+			delete desc;
+			throw;
+		}
+		delete desc;
+		fd.CopyTo( filterDiff );
+		if( freeTermDiff != nullptr ) {
+			ftd.CopyTo( freeTermDiff );
+		}
+	} );
+}
+
 // The two fused blocks of depthwise-separable networks through the interface calls their layers make
 // (MobileNetV2BlockLayer.cpp:205-250, ChannelwiseWith1x1Layer.cpp:150-197). activation codes: 0 none (AF_Linear),
 // 1 ReLU (param = upper threshold when > 0), 2 h-swish. withExpand: MobileNetV2Block, else ChannelwiseWith1x1

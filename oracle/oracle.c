@@ -455,6 +455,62 @@ ORC_API void orc_blob_convolution_learn_add(const float* in, int n, int h, int w
 				}
 }
 
+/* Gradients of the channelwise convolution, as the transposes of its forward loop nest
+ * (src/CPU/CpuMathEngineDnnConv.cpp:1017-1200): by the input (scatter of outputDiff * filter), by the filter
+ * and by the free term (sums over the pixels, added to what the buffers hold) */
+ORC_API void orc_blob_channelwise_convolution_backward(const float* outDiff, int n, int h, int w, int c, const float* filter,
+	int fh, int fw, int ph, int pw, int sh, int sw, float* inDiff)
+{
+	const int ho = (h + 2 * ph - fh) / sh + 1, wo = (w + 2 * pw - fw) / sw + 1;
+	const size_t total = (size_t)n * h * w * c;
+	double* acc = (double*)calloc(total, sizeof(double));
+	for (int b = 0; b < n; ++b)
+		for (int y = 0; y < ho; ++y)
+			for (int x = 0; x < wo; ++x)
+				for (int ky = 0; ky < fh; ++ky) {
+					const int iy = y * sh - ph + ky;
+					if (iy < 0 || iy >= h) continue;
+					for (int kx = 0; kx < fw; ++kx) {
+						const int ix = x * sw - pw + kx;
+						if (ix < 0 || ix >= w) continue;
+						for (int ch = 0; ch < c; ++ch)
+							acc[(((size_t)b * h + iy) * w + ix) * c + ch] +=
+								(double)outDiff[(((size_t)b * ho + y) * wo + x) * c + ch] * filter[((size_t)ky * fw + kx) * c + ch];
+					}
+				}
+	for (size_t i = 0; i < total; ++i) inDiff[i] = (float)acc[i];
+	free(acc);
+}
+
+ORC_API void orc_blob_channelwise_convolution_learn_add(const float* in, int n, int h, int w, int c, const float* outDiff,
+	int fh, int fw, int ph, int pw, int sh, int sw, float* filterDiff, float* freeTermDiff)
+{
+	const int ho = (h + 2 * ph - fh) / sh + 1, wo = (w + 2 * pw - fw) / sw + 1;
+	for (int ch = 0; ch < c; ++ch) {
+		for (int ky = 0; ky < fh; ++ky)
+			for (int kx = 0; kx < fw; ++kx) {
+				double s = 0;
+				for (int b = 0; b < n; ++b)
+					for (int y = 0; y < ho; ++y) {
+						const int iy = y * sh - ph + ky;
+						if (iy < 0 || iy >= h) continue;
+						for (int x = 0; x < wo; ++x) {
+							const int ix = x * sw - pw + kx;
+							if (ix < 0 || ix >= w) continue;
+							s += (double)outDiff[(((size_t)b * ho + y) * wo + x) * c + ch] * in[(((size_t)b * h + iy) * w + ix) * c + ch];
+						}
+					}
+				float* d = filterDiff + ((size_t)ky * fw + kx) * c + ch;
+				*d = (float)(*d + s);
+			}
+		if (freeTermDiff) {
+			double s = 0;
+			for (size_t p = 0; p < (size_t)n * ho * wo; ++p) s += outDiff[p * c + ch];
+			freeTermDiff[ch] = (float)(freeTermDiff[ch] + s);
+		}
+	}
+}
+
 /* sourceDiff = 0, then every output element adds its gradient at the index the forward pass stored
  * (src/CPU/CpuMathEngineDnnPooling.cpp:146-175) */
 ORC_API void orc_blob_max_pooling_backward(const float* resultDiff, const int* indices, int n, int sourceObjectSize,

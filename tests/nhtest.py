@@ -397,6 +397,24 @@ class Cpu:
                    fp(fd), fp(ftd))
         return fd if ftd is None else (fd, ftd)
 
+    def channelwise_conv_backward(self, out_diff, filt, in_shape, ph, pw, sh, sw):
+        out_diff, filt = f32(out_diff), f32(filt)
+        n, h, w, c = in_shape
+        fh, fw, _ = filt.shape
+        assert out_diff.shape == (n, *conv_out(h, w, fh, fw, ph, pw, sh, sw), c)
+        y = np.empty(in_shape, np.float32)
+        self._call("blob_channelwise_convolution_backward", fp(out_diff), n, h, w, c, fp(filt), fh, fw, ph, pw, sh, sw, fp(y))
+        return y
+
+    def channelwise_conv_learn_add(self, x, out_diff, filter_diff, ph, pw, sh, sw, free_term_diff=None):
+        x, out_diff = f32(x), f32(out_diff)
+        n, h, w, c = x.shape
+        fh, fw, _ = filter_diff.shape
+        fd = f32(filter_diff).copy()
+        ftd = None if free_term_diff is None else f32(free_term_diff).copy()
+        self._call("blob_channelwise_convolution_learn_add", fp(x), n, h, w, c, fp(out_diff), fh, fw, ph, pw, sh, sw, fp(fd), fp(ftd))
+        return fd if ftd is None else (fd, ftd)
+
     def max_pool_backward(self, x, result_diff, fh, fw, sh, sw):
         """Forward pass over x for the indices, then the gradient by x."""
         x, result_diff = f32(x), f32(result_diff)
@@ -825,6 +843,26 @@ class Hip:
         xs, gs, fd = self.up(x), self.up(out_diff), self.up(filter_diff)
         self.call("nhBlobConvolutionLearnAdd", ctypes.byref(d), self.p(xs), self.p(gs), self.p(fd))
         return self.down(fd)
+
+    def channelwise_conv_backward(self, out_diff, filt, in_shape, ph, pw, sh, sw):
+        out_diff, filt = f32(out_diff), f32(filt)
+        n, h, w, c = in_shape
+        fh, fw, _ = filt.shape
+        d = self.conv_desc(n, h, w, c, c, fh, fw, ph, pw, sh, sw, channelwise=True)
+        gs, fs = self.up(out_diff), self.up(filt)
+        out = self.empty(in_shape)
+        self.call("nhBlobChannelwiseConvolutionBackward", ctypes.byref(d), self.p(gs), self.p(fs), self.p(out))
+        return self.down(out)
+
+    def channelwise_conv_learn_add(self, x, out_diff, filter_diff, ph, pw, sh, sw, free_term_diff=None):
+        x, out_diff = f32(x), f32(out_diff)
+        n, h, w, c = x.shape
+        fh, fw, _ = filter_diff.shape
+        d = self.conv_desc(n, h, w, c, c, fh, fw, ph, pw, sh, sw, channelwise=True)
+        xs, gs, fd = self.up(x), self.up(out_diff), self.up(f32(filter_diff))
+        ftd = self.up(None if free_term_diff is None else f32(free_term_diff))
+        self.call("nhBlobChannelwiseConvolutionLearnAdd", ctypes.byref(d), self.p(xs), self.p(gs), self.p(fd), self.p(ftd))
+        return self.down(fd) if ftd is None else (self.down(fd), self.down(ftd))
 
     def max_pool_backward(self, x, result_diff, fh, fw, sh, sw):
         x = f32(x)

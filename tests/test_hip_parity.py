@@ -121,6 +121,18 @@ def test_broadcasts_and_sums():
                      orc.batch_multiply_matrix_by_diag_matrix(b, m, h, w, h * w, v[0], 0), "diag right broadcast")
 
 
+@pytest.mark.parametrize("b,h,w", [(1, 2048, 4), (1, 12544, 64), (2, 5000, 12), (1, 3000, 256), (3, 2049, 100), (1, 100352, 128)])
+def test_sums_over_the_rows_of_tall_matrices(b, h, w):
+    # the free-term gradient of a convolution: one row per pixel of the batch, one column per filter
+    g = rng(55 + w)
+    m = g.uniform(-1, 1, (b, h, w)).astype(np.float32)
+    v = g.uniform(-10, 10, (b, w)).astype(np.float32)
+    want = m.astype(np.float64).sum(axis=1)
+    tol = 1e-5 * np.sqrt(h)
+    assert_close(hip().sum_matrix_rows(m), want, "sum rows %s" % ((b, h, w),), atol=tol)
+    assert_close(hip().sum_matrix_rows(m, add_to=v), want + v, "sum rows add", atol=tol)
+
+
 def test_softmax_logsumexp():
     g = rng(6)
     for h, w in ((1, 1), (3, 2), (7, 64), (9, 101), (513, 256), (64, 1000), (5, 1500), (8192, 101)):
@@ -341,6 +353,28 @@ def test_convolution_gradients_are_adjoints_at_full_size():
     assert abs(np.vdot(dx.astype(np.float64), x) - pairing) <= 1e-5 * size
     df = h.conv_learn_add(x, grad, np.zeros_like(f), 1, 1, 1, 1)
     assert abs(np.vdot(df.astype(np.float64), f) - pairing) <= 1e-5 * size
+
+
+@pytest.mark.parametrize("case", CHANNELWISE_CASES + [(2, 28, 28, 96, 3, 3, 1, 1, 1, 1), (2, 28, 28, 96, 3, 3, 1, 1, 2, 2),
+                                                      (1, 15, 13, 6, 3, 3, 1, 1, 2, 2), (1, 9, 30, 32, 5, 5, 2, 2, 1, 1),
+                                                      (2, 21, 13, 20, 3, 3, 0, 2, 2, 2), (1, 3, 3, 4, 3, 3, 1, 1, 1, 1),
+                                                      (4, 14, 14, 384, 3, 3, 1, 1, 1, 1), (16, 56, 56, 144, 3, 3, 1, 1, 1, 1)])
+def test_channelwise_convolution_gradients(case):
+    n, h, w, c, fh, fw, ph, pw, sh, sw = case
+    g = rng(212 + c)
+    x = g.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    f = g.normal(0, 1, (fh, fw, c)).astype(np.float32)
+    ho, wo = nhtest.conv_out(h, w, fh, fw, ph, pw, sh, sw)
+    grad = g.uniform(-1, 1, (n, ho, wo, c)).astype(np.float32)
+    assert_close(hip().channelwise_conv_backward(grad, f, x.shape, ph, pw, sh, sw),
+                 orc.channelwise_conv_backward(grad, f, x.shape, ph, pw, sh, sw), "backward %s" % (case,))
+    start, ft0 = g.uniform(-1, 1, f.shape).astype(np.float32), g.uniform(-1, 1, c).astype(np.float32)
+    want, want_ft = orc.channelwise_conv_learn_add(x, grad, start, ph, pw, sh, sw, free_term_diff=ft0)
+    got, got_ft = hip().channelwise_conv_learn_add(x, grad, start, ph, pw, sh, sw, free_term_diff=ft0)
+    scale = np.sqrt(n * ho * wo)  # sums over every pixel of the batch
+    assert_close(got, want, "learn %s" % (case,), atol=1e-5 * scale)
+    assert_close(got_ft, want_ft, "free term gradient %s" % (case,), atol=1e-5 * scale)
+    assert_close(hip().channelwise_conv_learn_add(x, grad, start, ph, pw, sh, sw), want, "learn, no free term", atol=1e-5 * scale)
 
 
 @pytest.mark.parametrize("case", POOL_CASES + [(2, 57, 57, 64, 3, 3, 2, 2), (3, 16, 64, 7, 2, 2, 2, 2), (2, 23, 19, 8, 3, 3, 1, 1),

@@ -530,6 +530,40 @@ def test_channelwise_convolution(case):
 # ---------------------------------------------------------------------------------------------------------
 # pooling
 
+@pytest.mark.parametrize("case", CHANNELWISE_CASES)
+def test_channelwise_convolution_gradients_are_adjoints(case):
+    n, h, w, c, fh, fw, ph, pw, sh, sw = case
+    g = rng(112 + c)
+    x = g.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    f = g.normal(0, 1, (fh, fw, c)).astype(np.float32)
+    y = orc.channelwise_conv(x, f, None, ph, pw, sh, sw)
+    grad = g.uniform(-1, 1, y.shape).astype(np.float32)
+    pairing = np.vdot(y.astype(np.float64), grad)
+    size = np.abs(y.astype(np.float64) * grad).sum()
+    dx = orc.channelwise_conv_backward(grad, f, x.shape, ph, pw, sh, sw)
+    assert abs(np.vdot(dx.astype(np.float64), x) - pairing) <= 1e-4 * size
+    start, ft0 = g.uniform(-1, 1, f.shape).astype(np.float32), g.uniform(-1, 1, c).astype(np.float32)
+    df, dft = orc.channelwise_conv_learn_add(x, grad, start, ph, pw, sh, sw, free_term_diff=ft0)
+    assert abs(np.vdot((df - start).astype(np.float64), f) - pairing) <= 1e-4 * size
+    assert_close(dft, ft0 + grad.reshape(-1, c).astype(np.float64).sum(axis=0), "free term gradient", atol=1e-5)
+    for _ in range(6):  # single components through unit impulses
+        at = tuple(g.integers(0, d) for d in x.shape)
+        e = np.zeros_like(x)
+        e[at] = 1
+        assert abs(np.vdot(orc.channelwise_conv(e, f, None, ph, pw, sh, sw).astype(np.float64), grad) - dx[at]) <= 1e-4 * (1 + abs(dx[at]))
+        at = tuple(g.integers(0, d) for d in f.shape)
+        e = np.zeros_like(f)
+        e[at] = 1
+        want = np.vdot(orc.channelwise_conv(x, e, None, ph, pw, sh, sw).astype(np.float64), grad) + start[at]
+        assert abs(want - df[at]) <= 1e-4 * (1 + abs(want))
+    if nhtest.have_reference():
+        assert_close(ref().channelwise_conv_backward(grad, f, x.shape, ph, pw, sh, sw), dx, "backward vs reference %s" % (case,), atol=1e-4)
+        rdf, rdft = ref().channelwise_conv_learn_add(x, grad, start, ph, pw, sh, sw, free_term_diff=ft0)
+        assert_close(rdf, df, "learn vs reference %s" % (case,), atol=1e-4)
+        assert_close(rdft, dft, "free term gradient vs reference", atol=1e-4)
+        assert_close(ref().channelwise_conv_learn_add(x, grad, start, ph, pw, sh, sw), df, "learn without free term", atol=1e-4)
+
+
 POOL_CASES = [(1, 2, 2, 1, 2, 2, 2, 2), (2, 9, 11, 5, 3, 3, 2, 2), (1, 8, 8, 16, 2, 2, 2, 2), (2, 7, 10, 3, 3, 2, 1, 3),
               (1, 6, 6, 4, 6, 6, 1, 1), (1, 12, 5, 8, 2, 1, 2, 1)]
 
