@@ -225,6 +225,12 @@ NH_API int nhBlobMergeByDim(nhStream s, int dim, const nhBlobDesc* from_host, co
 NH_API int nhBlobSplitByDim(nhStream s, int dim, const nhBlobDesc* from_host, const float* fromData,
 	const nhBlobDesc* to_host, float* const* toData_host, int toCount);                              /* NME.h:700,702 */
 
+/* BroadcastCopy: every dimension of `from` is 1 or equal to the one of `to`; values repeat along the dimensions of
+ * size 1. additionalWidth (>= 1) is one more, innermost, unbroadcast dimension. 4-byte elements: serves the float
+ * and the int member alike. */
+NH_API int nhBroadcastCopy(nhStream s, void* to, const void* from, const nhBlobDesc* to_host,
+	const nhBlobDesc* from_host, int additionalWidth);                                               /* NME.h:80,82 */
+
 enum { NH_PAD_CONSTANT = 0, NH_PAD_EDGE = 1, NH_PAD_REFLECT = 2 }; /* TBlobResizePadding, NME.h:62-66 */
 NH_API int nhBlobResizeImage(nhStream s, const nhBlobDesc* from_host, const float* fromData, int deltaLeft,
 	int deltaRight, int deltaTop, int deltaBottom, int padding, float defaultValue,
@@ -300,6 +306,22 @@ NH_API int nhChannelwiseWith1x1WorkspaceSize(const nhSeparableBlockDesc* desc_ho
 NH_API int nhChannelwiseWith1x1(nhStream s, const nhSeparableBlockDesc* desc_host, const float* input,
 	const float* channelwiseFilter, const float* channelwiseFreeTerm, const float* convFilter,
 	const float* convFreeTerm, float* output, void* workspace, size_t workspaceSize);                /* NME.h:1066 */
+
+/* The two halves of a MobileNetV3 block, before and after its squeeze-and-excite branch (NME.h:1073-1083, layer classes
+ * CMobileNetV3PreSEBlockLayer / CMobileNetV3PostSEBlockLayer). Pre: expand 1x1 (+act) -> depthwise of any
+ * nhInitBlobChannelwiseConvolution descriptor (+act); channelwise_desc describes the depthwise stage, its `channels` is
+ * the expanded width; workspace holds the expanded tensor (nhMobileNetV3PreSEBlockWorkspaceSize bytes).
+ * Post: output = down 1x1( act( channelwiseOutput * squeezeAndExcite[image][channel] ) ) + residual (may be null);
+ * workspace: batch * pixelsPerImage * channels floats. Activations as for the blocks above. */
+NH_API int nhMobileNetV3PreSEBlockWorkspaceSize(const nhConvDesc* channelwise_desc_host, size_t* bytes);
+NH_API int nhMobileNetV3PreSEBlock(nhStream s, const nhConvDesc* channelwise_desc_host, int inputChannels,
+	const float* input, const float* expandFilter, const float* expandFreeTerm, int expandActivation,
+	float expandParam, const float* channelwiseFilter, const float* channelwiseFreeTerm, int channelwiseActivation,
+	float channelwiseParam, float* output, void* workspace, size_t workspaceSize);                  /* NME.h:1073 */
+NH_API int nhMobileNetV3PostSEBlock(nhStream s, int batch, int pixelsPerImage, int channels, int outputChannels,
+	const float* channelwiseOutput, const float* squeezeAndExcite, const float* residual, int activation,
+	float param, const float* downFilter, const float* downFreeTerm, float* output, void* workspace,
+	size_t workspaceSize);                                                                          /* NME.h:1079 */
 /* A convolution with the activation behind it in the same launch, as the rowwise operation chains pair them
  * (NME.h:1080-1087): nhBlobConvolution followed by NH_ACT_* (a launch that is cut into K slices applies the activation
  * as a pass of its own); the pointwise form takes a 1x1 filter [Cout][Cin] over rows = pixels */

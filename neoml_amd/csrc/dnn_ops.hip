@@ -1112,6 +1112,45 @@ void channelwiseConvLearnKernel( const nhConvDesc d, const float* input, const f
 	}
 }
 
+// out[b][pixel][c] = act( in[b][pixel][c] * scale[b][c] ): the squeeze-and-excite gate of a MobileNetV3 block
+template<int VECW>
+__global__ __launch_bounds__( 256 )
+void scaleChannelsKernel( const float* in, const float* scale, float* out, int pixelsPerImage, int channels, long long totalItems,
+	const CFusedActivation act )
+{
+	typedef CChanVec<VECW> V;
+	const int cg = channels / VECW;
+	const long long perImage = static_cast<long long>( pixelsPerImage ) * cg;
+	for( long long item = blockIdx.x * 256LL + threadIdx.x; item < totalItems; item += static_cast<long long>( gridDim.x ) * 256 ) {
+		const int c = static_cast<int>( item % cg ) * VECW;
+		const long long b = item / perImage;
+		const typename V::Type v = V::fma( V::load( in + item * VECW ), V::load( scale + b * channels + c ), V::zero() );
+		V::store( out + item * VECW, V::activate( v, act ) );
+	}
+}
+
+// to[i0..i7] = from[the same index with 0 where from's dimension is 1]; dimension 7 is the additional width
+struct CBroadcastShape {
+	int ToDims[8];
+	int FromStrides[8]; // 0 along broadcast dimensions
+};
+
+__global__ __launch_bounds__( 256 )
+void broadcastCopyKernel( unsigned* to, const unsigned* from, const CBroadcastShape shape, long long total )
+{
+	for( long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += static_cast<long long>( gridDim.x ) * 256 ) {
+		long long rest = i;
+		long long source = 0;
+#pragma unroll
+		for( int d = 7; d >= 0; --d ) {
+			const int index = static_cast<int>( rest % shape.ToDims[d] );
+			rest /= shape.ToDims[d];
+			source += static_cast<long long>( index ) * shape.FromStrides[d];
+		}
+		to[i] = from[source];
+	}
+}
+
 __global__ void addTwoVectorsKernel( const float* a, const float* b, float* out, int n )
 {
 	const int i = blockIdx.x * 256 + threadIdx.x;
@@ -1609,6 +1648,30 @@ int nhBlobMergeByDim( nhStream s, int dim, const nhBlobDesc* from, const float* 
 	return splitMergeImpl<true>( s, dim, *to, toData, from, const_cast<float* const*>( fromData ), fromCount );
 }
 
+int nhBroadcastCopy( nhStream s, void* to, const void* from, const nhBlobDesc* toDesc, const nhBlobDesc* fromDesc,
+	int additionalWidth )
+{
+	NH_REQUIRE( to != nullptr && from != nullptr && toDesc != nullptr && fromDesc != nullptr && additionalWidth >= 1 );
+	CBroadcastShape shape;
+	long long total = additionalWidth, stride = additionalWidth;
+	shape.ToDims[7] = additionalWidth;
+	shape.FromStrides[7] = 1;
+	for( int d = 6; d >= 0; --d ) {
+		NH_REQUIRE( toDesc->dims[d] >= 1 && ( fromDesc->dims[d] == 1 || fromDesc->dims[d] == toDesc->dims[d] ) );
+		shape.ToDims[d] = toDesc->dims[d];
+		shape.FromStrides[d] = fromDesc->dims[d] == toDesc->dims[d] ? static_cast<int>( stride ) : 0;
+		stride *= fromDesc->dims[d];
+		total *= toDesc->dims[d];
+	}
+	NH_REQUIRE( stride <= 0x7fffffffLL );
+	long long blocks = ( total + 255 ) / 256;
+	blocks = blocks > 1048576 ? 1048576 : blocks;
+	hipLaunchKernelGGL( broadcastCopyKernel, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+		static_cast<unsigned*>( to ), static_cast<const unsigned*>( from ), shape, total );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
 int nhBlobSplitByDim( nhStream s, int dim, const nhBlobDesc* from, const float* fromData,
 	const nhBlobDesc* to, float* const* toData, int toCount )
 {
@@ -1783,6 +1846,91 @@ int nhMobileNetV2Block( nhStream s, const nhSeparableBlockDesc* d, const float* 
 	return matMulNTFused( toStream( s ), reduced, d->expandedChannels, downFilter, d->expandedChannels, output, d->outputChannels,
 		static_cast<int>( pixelsOut ), d->outputChannels, d->expandedChannels, 1, 0, 0, 0, downFreeTerm, false, none,
 		d->residual != 0 ? input : nullptr );
+}
+
+// The two halves of a MobileNetV3 block, around its squeeze-and-excite branch: expand 1x1 (+act) -> depthwise (+act), and
+// gate (+act) -> down 1x1 (+residual). The depthwise stage takes any channelwise descriptor (3x3 and 5x5 occur).
+static int checkPreSE( const nhConvDesc* dw, int inputChannels )
+{
+	NH_REQUIRE( dw != nullptr && inputChannels > 0 );
+	nhConvDesc check = *dw;
+	const int rc = nhInitBlobChannelwiseConvolution( &check );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( check.resultHeight == dw->resultHeight && check.resultWidth == dw->resultWidth );
+	const long long expanded = static_cast<long long>( dw->batch ) * dw->height * dw->width * dw->channels;
+	NH_REQUIRE( expanded <= 0x7fffffffLL );
+	return NH_OK;
+}
+
+int nhMobileNetV3PreSEBlockWorkspaceSize( const nhConvDesc* dw, size_t* bytes )
+{
+	const int rc = checkPreSE( dw, 1 );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( bytes != nullptr );
+	*bytes = static_cast<size_t>( dw->batch ) * dw->height * dw->width * dw->channels * sizeof( float );
+	return NH_OK;
+}
+
+int nhMobileNetV3PreSEBlock( nhStream s, const nhConvDesc* dw, int inputChannels, const float* input,
+	const float* expandFilter, const float* expandFreeTerm, int expandActivation, float expandParam,
+	const float* channelwiseFilter, const float* channelwiseFreeTerm, int channelwiseActivation, float channelwiseParam,
+	float* output, void* workspace, size_t workspaceSize )
+{
+	const int rc = checkPreSE( dw, inputChannels );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( input != nullptr && expandFilter != nullptr && channelwiseFilter != nullptr && output != nullptr );
+	const size_t need = static_cast<size_t>( dw->batch ) * dw->height * dw->width * dw->channels * sizeof( float );
+	NH_REQUIRE( workspace != nullptr && workspaceSize >= need && isAligned16( workspace ) );
+	if( dw->batch == 0 ) {
+		return NH_OK;
+	}
+	float* expanded = static_cast<float*>( workspace );
+	const CFusedActivation expandAct = { expandActivation, expandParam };
+	const CFusedActivation channelwiseAct = { channelwiseActivation, channelwiseParam };
+	const int pixels = dw->batch * dw->height * dw->width;
+	const int rcExpand = matMulNTFused( toStream( s ), input, inputChannels, expandFilter, inputChannels, expanded, dw->channels,
+		pixels, dw->channels, inputChannels, 1, 0, 0, 0, expandFreeTerm, false, expandAct, nullptr );
+	if( rcExpand != NH_OK ) {
+		return rcExpand;
+	}
+	return channelwiseConvolution( s, dw, expanded, channelwiseFilter, channelwiseFreeTerm, output, channelwiseAct );
+}
+
+int nhMobileNetV3PostSEBlock( nhStream s, int batch, int pixelsPerImage, int channels, int outputChannels,
+	const float* channelwiseOutput, const float* squeezeAndExcite, const float* residual, int activation, float param,
+	const float* downFilter, const float* downFreeTerm, float* output, void* workspace, size_t workspaceSize )
+{
+	NH_REQUIRE( batch >= 0 && pixelsPerImage > 0 && channels > 0 && outputChannels > 0 );
+	const long long total = static_cast<long long>( batch ) * pixelsPerImage * channels;
+	NH_REQUIRE( total <= 0x7fffffffLL );
+	NH_REQUIRE( channelwiseOutput != nullptr && squeezeAndExcite != nullptr && downFilter != nullptr && output != nullptr );
+	NH_REQUIRE( workspace != nullptr && workspaceSize >= static_cast<size_t>( total ) * sizeof( float ) && isAligned16( workspace ) );
+	if( batch == 0 ) {
+		return NH_OK;
+	}
+	float* gated = static_cast<float*>( workspace );
+	const CFusedActivation act = { activation, param };
+	const bool vec = channels % 4 == 0 && isAligned16( channelwiseOutput ) && isAligned16( squeezeAndExcite );
+	const long long items = vec ? total / 4 : total;
+	long long blocks = ( items + 255 ) / 256;
+	blocks = blocks > 1048576 ? 1048576 : blocks;
+	if( vec ) {
+		hipLaunchKernelGGL( scaleChannelsKernel<4>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			channelwiseOutput, squeezeAndExcite, gated, pixelsPerImage, channels, items, act );
+	} else {
+		hipLaunchKernelGGL( scaleChannelsKernel<1>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			channelwiseOutput, squeezeAndExcite, gated, pixelsPerImage, channels, items, act );
+	}
+	NH_LAUNCH_CHECK();
+	const CFusedActivation none = { NH_ACT_NONE, 0.f };
+	return matMulNTFused( toStream( s ), gated, channels, downFilter, channels, output, outputChannels,
+		batch * pixelsPerImage, outputChannels, channels, 1, 0, 0, 0, downFreeTerm, false, none, residual );
 }
 
 int nhChannelwiseWith1x1WorkspaceSize( const nhSeparableBlockDesc* d, size_t* bytes )

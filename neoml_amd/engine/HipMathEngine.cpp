@@ -14,14 +14,6 @@ namespace NeoML {
 // ---------------------------------------------------------------------------------------------------------
 // descriptors (deleted by the caller with plain delete, hence CCrtAllocatedObject through the base structs)
 
-struct CHipConvolutionDesc : public CConvolutionDesc {
-	nhConvDesc D;
-};
-
-struct CHipChannelwiseConvolutionDesc : public CChannelwiseConvolutionDesc {
-	nhConvDesc D;
-};
-
 struct CHipMaxPoolingDesc : public CMaxPoolingDesc {
 	nhPoolingDesc D;
 };
@@ -153,6 +145,20 @@ void CHipMathEngine::VectorCopy( const CFloatHandle& first, const CConstFloatHan
 void CHipMathEngine::VectorCopy( const CIntHandle& first, const CConstIntHandle& second, int vectorSize )
 {
 	NH_CALL( nhVectorCopyInt( stream, raw( first ), raw( second ), vectorSize ) );
+}
+
+void CHipMathEngine::BroadcastCopy( const CIntHandle& toHandle, const CConstIntHandle& fromHandle, const CBlobDesc& toDesc,
+	const CBlobDesc& fromDesc, int additionalWidth )
+{
+	const nhBlobDesc to = toBlobDesc( toDesc ), from = toBlobDesc( fromDesc );
+	NH_CALL( nhBroadcastCopy( stream, raw( toHandle ), raw( fromHandle ), &to, &from, additionalWidth ) );
+}
+
+void CHipMathEngine::BroadcastCopy( const CFloatHandle& toHandle, const CConstFloatHandle& fromHandle,
+	const CBlobDesc& toDesc, const CBlobDesc& fromDesc, int additionalWidth )
+{
+	const nhBlobDesc to = toBlobDesc( toDesc ), from = toBlobDesc( fromDesc );
+	NH_CALL( nhBroadcastCopy( stream, raw( toHandle ), raw( fromHandle ), &to, &from, additionalWidth ) );
 }
 
 void CHipMathEngine::VectorFill( const CFloatHandle& result, float value, int vectorSize )

@@ -46,6 +46,16 @@ inline T* GetRaw( const CTypedMemoryHandle<T>& handle )
 	return static_cast<T*>( CMemoryHandleInternal::GetRaw( handle ) );
 }
 
+// Convolution descriptors (deleted by the caller with plain delete, hence CCrtAllocatedObject through the base structs);
+// shared by the engine's source files
+struct CHipConvolutionDesc : public CConvolutionDesc {
+	nhConvDesc D;
+};
+
+struct CHipChannelwiseConvolutionDesc : public CChannelwiseConvolutionDesc {
+	nhConvDesc D;
+};
+
 class CHipMathEngine : public IMathEngine {
 public:
 	CHipMathEngine( int deviceIndex, size_t memoryLimit, int flags );
@@ -54,6 +64,10 @@ public:
 	// ---- IVectorMathEngine ----
 	void VectorCopy( const CFloatHandle& first, const CConstFloatHandle& second, int vectorSize ) override;
 	void VectorCopy( const CIntHandle& first, const CConstIntHandle& second, int vectorSize ) override;
+	void BroadcastCopy( const CIntHandle& toHandle, const CConstIntHandle& fromHandle, const CBlobDesc& toDesc,
+		const CBlobDesc& fromDesc, int additionalWidth ) override;
+	void BroadcastCopy( const CFloatHandle& toHandle, const CConstFloatHandle& fromHandle, const CBlobDesc& toDesc,
+		const CBlobDesc& fromDesc, int additionalWidth ) override;
 	void VectorFill( const CFloatHandle& result, float value, int vectorSize ) override;
 	void VectorFill( const CIntHandle& result, int value, int vectorSize ) override;
 	void VectorFill( const CFloatHandle& result, int vectorSize, const CConstFloatHandle& value ) override;
@@ -238,6 +252,17 @@ public:
 		const CConstFloatHandle& input, const CFloatHandle& outputStateBackLink,
 		const CFloatHandle& outputMainBackLink ) override;
 
+	void MobileNetV3PreSEBlock( const CBlobDesc& inputDesc, const CBlobDesc& outputDesc,
+		const CChannelwiseConvolutionDesc& convDesc, const CConstFloatHandle& inputHandle,
+		const CConstFloatHandle& expandFilter, const CConstFloatHandle* expandFreeTerm,
+		TActivationFunction expandActivation, float expandReluParam, const CConstFloatHandle& channelwiseFilter,
+		const CConstFloatHandle* channelwiseFreeTerm, TActivationFunction channelwiseActivation,
+		float channelwiseReluParam, const CFloatHandle& outputHandle ) override;
+	void MobileNetV3PostSEBlock( const CBlobDesc& channelwiseOutputDesc, int outputChannels,
+		const CConstFloatHandle& channelwiseOutputHandle, const CConstFloatHandle& squeezeAndExciteHandle,
+		const CConstFloatHandle* residualHandle, TActivationFunction activation, float reluParam,
+		const CConstFloatHandle& downFilterHandle, const CConstFloatHandle* downFreeTermHandle,
+		const CFloatHandle& outputHandle ) override;
 	// the fused blocks and operation chains of the graph optimizer (HipMathEngineRowwise.cpp)
 	void ChannelwiseWith1x1( const CBlobDesc& inputDesc, const CBlobDesc& outputDesc,
 		const CRowwiseOperationDesc& rowwiseDesc, const CChannelwiseConvolutionDesc& convDesc,

@@ -304,6 +304,48 @@ void CHipMathEngine::MobileNetV2Block( const CBlobDesc& inputDesc, const CBlobDe
 	RunSeparableBlock( block, inputHandle, outputHandle );
 }
 
+// The halves of a MobileNetV3 block around its squeeze-and-excite branch (CMobileNetV3PreSEBlockLayer /
+// CMobileNetV3PostSEBlockLayer call these directly with their parameter blobs)
+void CHipMathEngine::MobileNetV3PreSEBlock( const CBlobDesc& inputDesc, const CBlobDesc& outputDesc,
+	const CChannelwiseConvolutionDesc& convDesc, const CConstFloatHandle& inputHandle,
+	const CConstFloatHandle& expandFilter, const CConstFloatHandle* expandFreeTerm,
+	TActivationFunction expandActivation, float expandReluParam, const CConstFloatHandle& channelwiseFilter,
+	const CConstFloatHandle* channelwiseFreeTerm, TActivationFunction channelwiseActivation,
+	float channelwiseReluParam, const CFloatHandle& outputHandle )
+{
+	const CHipChannelwiseConvolutionDesc& d = static_cast<const CHipChannelwiseConvolutionDesc&>( convDesc );
+	ASSERT_EXPR( outputDesc.Channels() == d.D.channels && inputDesc.ObjectCount() == d.D.batch );
+	ASSERT_EXPR( inputDesc.Height() == d.D.height && inputDesc.Width() == d.D.width );
+	size_t workspaceSize = 0;
+	NH_CALL( nhMobileNetV3PreSEBlockWorkspaceSize( &d.D, &workspaceSize ) );
+	const CMemoryHandle workspace = StackAlloc( std::max<size_t>( workspaceSize, 16 ) );
+	NH_CALL( nhMobileNetV3PreSEBlock( stream, &d.D, inputDesc.Channels(), raw( inputHandle ), raw( expandFilter ),
+		expandFreeTerm != nullptr ? raw( *expandFreeTerm ) : nullptr, fusedActivation( expandActivation ), expandReluParam,
+		raw( channelwiseFilter ), channelwiseFreeTerm != nullptr ? raw( *channelwiseFreeTerm ) : nullptr,
+		fusedActivation( channelwiseActivation ), channelwiseReluParam, raw( outputHandle ), rawBytes( workspace ),
+		workspaceSize ) );
+	StackFree( workspace );
+}
+
+void CHipMathEngine::MobileNetV3PostSEBlock( const CBlobDesc& channelwiseOutputDesc, int outputChannels,
+	const CConstFloatHandle& channelwiseOutputHandle, const CConstFloatHandle& squeezeAndExciteHandle,
+	const CConstFloatHandle* residualHandle, TActivationFunction activation, float reluParam,
+	const CConstFloatHandle& downFilterHandle, const CConstFloatHandle* downFreeTermHandle,
+	const CFloatHandle& outputHandle )
+{
+	const int batch = channelwiseOutputDesc.ObjectCount();
+	const int pixels = channelwiseOutputDesc.Height() * channelwiseOutputDesc.Width();
+	const int channels = channelwiseOutputDesc.Channels();
+	const size_t workspaceSize = static_cast<size_t>( batch ) * pixels * channels * sizeof( float );
+	const CMemoryHandle workspace = StackAlloc( std::max<size_t>( workspaceSize, 16 ) );
+	NH_CALL( nhMobileNetV3PostSEBlock( stream, batch, pixels, channels, outputChannels, raw( channelwiseOutputHandle ),
+		raw( squeezeAndExciteHandle ), residualHandle != nullptr ? raw( *residualHandle ) : nullptr,
+		fusedActivation( activation ), reluParam, raw( downFilterHandle ),
+		downFreeTermHandle != nullptr ? raw( *downFreeTermHandle ) : nullptr, raw( outputHandle ), rawBytes( workspace ),
+		workspaceSize ) );
+	StackFree( workspace );
+}
+
 // ---- descriptors ----------------------------------------------------------------------------------------------
 
 CRowwiseOperationDesc* CHipMathEngine::InitRowwiseActivation( const CActivationDesc& desc )

@@ -5,6 +5,7 @@
 // The tests call them once with the reference's CPU engine and once with the HIP engine: same layer code, same
 // CRandom seed for the initialisers, same input, so the two outputs differ only by the engine underneath.
 #include <NeoML/NeoML.h>
+#include <NeoML/Dnn/Layers/Onnx/OnnxEltwiseLayer.h>
 #include "HipLstmLayer.h" // neoml_amd/engine: the LSTM layer that reaches IMathEngine::Lstm on a non-CPU engine
 
 #include <chrono>
@@ -269,6 +270,67 @@ static CBaseLayer* buildSeparableNet( CDnn& dnn, IMathEngine& e, CBaseLayer& sou
 	return softmax.Ptr();
 }
 
+// kind 7: a MobileNetV3-style network of plain layers: stem 3x3/2 (16) - h-swish - two blocks of
+//         [1x1 expand - act - channelwise FxF - act - squeeze-and-excite (global mean - FC / 4 - ReLU - FC - hard sigmoid,
+//         multiplied back through COnnxEltwiseLayer) - act - 1x1 down ( + input )]: (F 3, 64 wide, ReLU, residual) and
+//         (F 5, 96 wide, h-swish, stride 2, to 24 channels) - global mean pool - FullyConnected (param) - softmax.
+static CBaseLayer* blockActivation( CDnn& dnn, IMathEngine& e, const CString& name, CBaseLayer& input, bool hswish )
+{
+	if( hswish ) {
+		return add( dnn, new CHSwishLayer( e ), name, input ).Ptr();
+	}
+	return add( dnn, new CReLULayer( e ), name, input ).Ptr();
+}
+
+static CBaseLayer* squeezeExciteBlock( CDnn& dnn, IMathEngine& e, const CString& name, CBaseLayer& input, int filterSize,
+	int expanded, int outputChannels, int stride, bool hswish, bool residual )
+{
+	CBaseLayer* x = conv( dnn, e, name + "_expand", input, expanded, 1, 0, 1 ).Ptr();
+	x = blockActivation( dnn, e, name + "_act1", *x, hswish );
+	CPtr<CChannelwiseConvLayer> dw = add( dnn, new CChannelwiseConvLayer( e ), name + "_dw", *x );
+	dw->SetFilterCount( expanded ); dw->SetFilterHeight( filterSize ); dw->SetFilterWidth( filterSize );
+	dw->SetPaddingHeight( filterSize / 2 ); dw->SetPaddingWidth( filterSize / 2 );
+	dw->SetStrideHeight( stride ); dw->SetStrideWidth( stride );
+	x = blockActivation( dnn, e, name + "_act2", *dw, hswish );
+	CPtr<CGlobalMeanPoolingLayer> pool = add( dnn, new CGlobalMeanPoolingLayer( e ), name + "_se_pool", *x );
+	CPtr<CFullyConnectedLayer> fc1 = add( dnn, new CFullyConnectedLayer( e ), name + "_se_fc1", *pool );
+	fc1->SetNumberOfElements( expanded / 4 );
+	CPtr<CReLULayer> seRelu = add( dnn, new CReLULayer( e ), name + "_se_relu", *fc1 );
+	CPtr<CFullyConnectedLayer> fc2 = add( dnn, new CFullyConnectedLayer( e ), name + "_se_fc2", *seRelu );
+	fc2->SetNumberOfElements( expanded );
+	CPtr<CHardSigmoidLayer> gate = add( dnn, new CHardSigmoidLayer( e ), name + "_se_gate", *fc2 );
+	CPtr<COnnxEltwiseLayer> mul = new COnnxEltwiseLayer( e );
+	mul->SetName( name + "_se_mul" );
+	mul->SetOperation( COnnxEltwiseLayer::TOperation::Mul );
+	mul->Connect( 0, *x );
+	mul->Connect( 1, *gate );
+	dnn.AddLayer( *mul );
+	x = blockActivation( dnn, e, name + "_act3", *mul, hswish );
+	x = conv( dnn, e, name + "_down", *x, outputChannels, 1, 0, 1 ).Ptr();
+	if( residual ) {
+		CPtr<CEltwiseSumLayer> sum = new CEltwiseSumLayer( e );
+		sum->SetName( name + "_sum" );
+		sum->Connect( 0, input );
+		sum->Connect( 1, *x );
+		dnn.AddLayer( *sum );
+		x = sum.Ptr();
+	}
+	return x;
+}
+
+static CBaseLayer* buildSqueezeExciteNet( CDnn& dnn, IMathEngine& e, CBaseLayer& source, int classes )
+{
+	CBaseLayer* x = conv( dnn, e, "stem", source, 16, 3, 1, 2 ).Ptr();
+	x = add( dnn, new CHSwishLayer( e ), "stem_hswish", *x ).Ptr();
+	x = squeezeExciteBlock( dnn, e, "b1", *x, 3, 64, 16, 1, false, true );
+	x = squeezeExciteBlock( dnn, e, "b2", *x, 5, 96, 24, 2, true, false );
+	CPtr<CGlobalMeanPoolingLayer> gap = add( dnn, new CGlobalMeanPoolingLayer( e ), "gap", *x );
+	CPtr<CFullyConnectedLayer> fc = add( dnn, new CFullyConnectedLayer( e ), "fc", *gap );
+	fc->SetNumberOfElements( classes );
+	CPtr<CSoftmaxLayer> softmax = add( dnn, new CSoftmaxLayer( e ), "softmax", *fc );
+	return softmax.Ptr();
+}
+
 // When set, dnn_run hands the network to NeoML's own graph optimizer (OptimizeDnn) after its first pass (the pass
 // that allocates and initialises the weights) and keeps what the optimizer reports
 static int optimizeNetworks = 0;
@@ -279,6 +341,10 @@ EXPORT void dnn_last_optimization( int* mobileNetV2Blocks, int* channelwiseWith1
 	*mobileNetV2Blocks = lastReport.MobileNetV2NonResidualBlocks + lastReport.MobileNetV2ResidualBlocks;
 	*channelwiseWith1x1 = lastReport.ChannelwiseWith1x1NonResidual + lastReport.ChannelwiseWith1x1Residual;
 	*rowwiseChains = lastReport.RowwiseChainCount;
+}
+EXPORT int dnn_last_optimization_mobilenetv3_blocks()
+{
+	return lastReport.MobileNetV3NonResidualBlocks + lastReport.MobileNetV3ResidualBlocks;
 }
 
 // Runs network `kind` on `engine`. dims: the 7 blob dimensions of the input; param: kind-specific size.
@@ -303,6 +369,7 @@ EXPORT int dnn_run( void* engine, int kind, int seed, int param, const int* dims
 			case 4: last = buildRecognizerTail( dnn, e, *source, param ); break;
 			case 5: last = buildResNet18( dnn, e, *source, param ); break;
 			case 6: last = buildSeparableNet( dnn, e, *source, param ); break;
+			case 7: last = buildSqueezeExciteNet( dnn, e, *source, param ); break;
 			default: lastError = "unknown network kind"; return 1;
 		}
 		CPtr<CSinkLayer> sink = new CSinkLayer( e );

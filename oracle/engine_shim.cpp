@@ -583,6 +583,59 @@ SHIM_API int shim_separable_block( void* engine, int withExpand, const float* in
 	} );
 }
 
+// The halves of a MobileNetV3 block around its squeeze-and-excite branch, as CMobileNetV3PreSEBlockLayer and
+// CMobileNetV3PostSEBlockLayer call them (MobileNetV3BlockLayer.cpp:150-175, 245-265). The depthwise stage has a square
+// filter of `filterSize` (3 or 5) with padding ( filterSize - 1 ) / 2. Activation codes as for shim_separable_block.
+SHIM_API int shim_mobilenetv3_pre_se( void* engine, const float* in, int n, int h, int w, int inputChannels,
+	int expandedChannels, int filterSize, int stride, int expandActivation, float expandParam, int channelwiseActivation,
+	float channelwiseParam, const float* expandFilter, const float* expandFreeTerm, const float* channelwiseFilter,
+	const float* channelwiseFreeTerm, float* out )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		static const TActivationFunction types[3] = { AF_Linear, AF_ReLU, AF_HSwish };
+		const int pad = ( filterSize - 1 ) / 2;
+		const int ho = ( h + 2 * pad - filterSize ) / stride + 1, wo = ( w + 2 * pad - filterSize ) / stride + 1;
+		const CBlobDesc inDesc = imageDesc( n, h, w, inputChannels ), chInDesc = imageDesc( n, h, w, expandedChannels ),
+			outDesc = imageDesc( n, ho, wo, expandedChannels ), chFilterDesc = imageDesc( 1, filterSize, filterSize, expandedChannels ),
+			chFreeTermDesc = imageDesc( 1, 1, 1, expandedChannels );
+		CFloatBlob src( e, inDesc.BlobSize(), in ), dst( e, outDesc.BlobSize() ),
+			exF( e, expandedChannels * inputChannels, expandFilter ), exT( e, expandedChannels, expandFreeTerm ),
+			chF( e, filterSize * filterSize * expandedChannels, channelwiseFilter ), chT( e, expandedChannels, channelwiseFreeTerm );
+		const CConstFloatHandle exTh = exT.Const(), chTh = chT.Const();
+		CChannelwiseConvolutionDesc* convDesc = e.InitBlobChannelwiseConvolution( chInDesc, pad, pad, stride, stride, chFilterDesc,
+			channelwiseFreeTerm != nullptr ? &chFreeTermDesc : nullptr, outDesc );
+		try {
+			e.MobileNetV3PreSEBlock( inDesc, outDesc, *convDesc, src.Const(), exF.Const(),
+				expandFreeTerm != nullptr ? &exTh : nullptr, types[expandActivation], expandParam, chF.Const(),
+				channelwiseFreeTerm != nullptr ? &chTh : nullptr, types[channelwiseActivation], channelwiseParam, dst.Handle() );
+		} catch( ... ) {
+			delete convDesc;
+			throw;
+		}
+		delete convDesc;
+		dst.CopyTo( out );
+	} );
+}
+
+SHIM_API int shim_mobilenetv3_post_se( void* engine, const float* in, int n, int h, int w, int channels, int outputChannels,
+	const float* squeezeAndExcite, const float* residual, int activation, float param, const float* downFilter,
+	const float* downFreeTerm, float* out )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		static const TActivationFunction types[3] = { AF_Linear, AF_ReLU, AF_HSwish };
+		const CBlobDesc inDesc = imageDesc( n, h, w, channels ), outDesc = imageDesc( n, h, w, outputChannels );
+		CFloatBlob src( e, inDesc.BlobSize(), in ), dst( e, outDesc.BlobSize() ), se( e, n * channels, squeezeAndExcite ),
+			res( e, outDesc.BlobSize(), residual ), dnF( e, outputChannels * channels, downFilter ),
+			dnT( e, outputChannels, downFreeTerm );
+		const CConstFloatHandle resH = res.Const(), dnTh = dnT.Const();
+		e.MobileNetV3PostSEBlock( inDesc, outputChannels, src.Const(), se.Const(), residual != nullptr ? &resH : nullptr,
+			types[activation], param, dnF.Const(), downFreeTerm != nullptr ? &dnTh : nullptr, dst.Handle() );
+		dst.CopyTo( out );
+	} );
+}
+
 // gradients of the convolution through BlobConvolutionBackward / BlobConvolutionLearnAdd (NeoMathEngine.h:757-761);
 // filterDiff and freeTermDiff (may be null) are accumulated into
 SHIM_API int shim_blob_convolution_backward( void* engine, const float* outDiff, int n, int h, int w, int cin,
@@ -729,6 +782,23 @@ SHIM_API int shim_blob_resize_image( void* engine, const float* from, int n, int
 		const TBlobResizePadding mode = padding == 0 ? TBlobResizePadding::Constant
 			: ( padding == 1 ? TBlobResizePadding::Edge : TBlobResizePadding::Reflect );
 		e.BlobResizeImage( inDesc, src.Handle(), dl, dr, dt, db, mode, value, outDesc, dst.Handle() );
+		dst.CopyTo( to );
+	} );
+}
+
+// BroadcastCopy (NeoMathEngine.h:75-83): toDims / fromDims are the 7 blob dimensions, without the additional width
+SHIM_API int shim_broadcast_copy( void* engine, const int* toDims, const int* fromDims, int additionalWidth, const float* from,
+	float* to )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		CBlobDesc toDesc( CT_Float ), fromDesc( CT_Float );
+		for( int i = 0; i < 7; ++i ) {
+			toDesc.SetDimSize( i, toDims[i] );
+			fromDesc.SetDimSize( i, fromDims[i] );
+		}
+		CFloatBlob src( e, fromDesc.BlobSize() * additionalWidth, from ), dst( e, toDesc.BlobSize() * additionalWidth );
+		e.BroadcastCopy( dst.Handle(), src.Const(), toDesc, fromDesc, additionalWidth );
 		dst.CopyTo( to );
 	} );
 }

@@ -455,6 +455,28 @@ ORC_API void orc_blob_convolution_learn_add(const float* in, int n, int h, int w
 				}
 }
 
+/* BroadcastCopy: `from` repeats along every dimension where it has size 1 and `to` does not; width is one more,
+ * innermost, dimension that both share (src/CPU/CpuMathEngineVectorMath.cpp:69-95 builds the same result by growing
+ * the copied block dimension by dimension from the innermost) */
+ORC_API void orc_broadcast_copy(const int* toDims, const int* fromDims, int width, const float* from, float* to)
+{
+	size_t fromStride[7];
+	size_t stride = (size_t)width, total = (size_t)width;
+	for (int d = 6; d >= 0; --d) {
+		fromStride[d] = fromDims[d] == toDims[d] ? stride : 0;
+		stride *= (size_t)fromDims[d];
+		total *= (size_t)toDims[d];
+	}
+	for (size_t i = 0; i < total; ++i) {
+		size_t rest = i / (size_t)width, source = i % (size_t)width;
+		for (int d = 6; d >= 0; --d) {
+			source += (rest % (size_t)toDims[d]) * fromStride[d];
+			rest /= (size_t)toDims[d];
+		}
+		to[i] = from[source];
+	}
+}
+
 /* Gradients of the channelwise convolution, as the transposes of its forward loop nest
  * (src/CPU/CpuMathEngineDnnConv.cpp:1017-1200): by the input (scatter of outputDiff * filter), by the filter
  * and by the free term (sums over the pixels, added to what the buffers hold) */

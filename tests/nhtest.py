@@ -366,6 +366,49 @@ class Cpu:
                    1 if in_place else 0, fp(y))
         return y
 
+    def mobilenetv3_pre_se(self, x, expand, channelwise, stride=1):
+        """expand = (filter [E][Cin], free term, activation, param); channelwise = (filter [F][F][E], free term,
+        activation, param), F = 3 or 5, padding (F - 1) / 2. The oracle composes its own convolution, channelwise
+        convolution and activations; the reference engine runs its MobileNetV3PreSEBlock."""
+        x = f32(x)
+        n, h, w, cin = x.shape
+        ex_f, ex_t, ex_act, ex_param = expand
+        ch_f, ch_t, ch_act, ch_param = channelwise
+        fsize, e = ch_f.shape[0], ch_f.shape[2]
+        pad = (fsize - 1) // 2
+        if self.kind == "orc":
+            def act(t, name, param):
+                return t if name is None else self.unary(name, t, np.float32(param if name == "relu" else 0.0)).reshape(t.shape)
+            t = act(self.conv(x, f32(ex_f).reshape(e, 1, 1, cin), ex_t, 0, 0, 1, 1), ex_act, ex_param)
+            return act(self.channelwise_conv(t, ch_f, ch_t, pad, pad, stride, stride), ch_act, ch_param)
+        ho, wo = conv_out(h, w, fsize, fsize, pad, pad, stride, stride)
+        y = np.empty((n, ho, wo, e), np.float32)
+        opt = lambda a: None if a is None else f32(a)
+        keep = [f32(ex_f), opt(ex_t), f32(ch_f), opt(ch_t)]
+        self._call("mobilenetv3_pre_se", fp(x), n, h, w, cin, e, fsize, stride, self.ACTIVATIONS[ex_act], ctypes.c_float(ex_param),
+                   self.ACTIVATIONS[ch_act], ctypes.c_float(ch_param), fp(keep[0]), fp(keep[1]), fp(keep[2]), fp(keep[3]), fp(y))
+        return y
+
+    def mobilenetv3_post_se(self, x, gate, residual, activation, param, down):
+        """x [N][H][W][C] (the depthwise stage's output), gate [N][C], residual [N][H][W][Cout] or None,
+        down = (filter [Cout][C], free term)."""
+        x, gate = f32(x), f32(gate)
+        n, h, w, c = x.shape
+        dn_f, dn_t = down
+        cout = dn_f.shape[0]
+        if self.kind == "orc":
+            t = x * gate.reshape(n, 1, 1, c)
+            if activation is not None:
+                t = self.unary(activation, t, np.float32(param if activation == "relu" else 0.0)).reshape(t.shape)
+            y = self.conv(t, f32(dn_f).reshape(cout, 1, 1, c), dn_t, 0, 0, 1, 1)
+            return y if residual is None else y + f32(residual)
+        y = np.empty((n, h, w, cout), np.float32)
+        opt = lambda a: None if a is None else f32(a)
+        keep = [opt(residual), f32(dn_f), opt(dn_t)]
+        self._call("mobilenetv3_post_se", fp(x), n, h, w, c, cout, fp(gate), fp(keep[0]), self.ACTIVATIONS[activation],
+                   ctypes.c_float(param), fp(keep[1]), fp(keep[2]), fp(y))
+        return y
+
     # ---- gradients (what the layers' backward and learn passes call)
     def conv_backward(self, out_diff, filt, bias, in_shape, ph, pw, sh, sw, dh=1, dw=1):
         """Gradient by the input; bias [Cin] or None is added to every pixel."""
@@ -473,6 +516,14 @@ class Cpu:
         big = np.empty(big_dims, np.float32)
         self._split_merge(big, dim, parts, merge=1)
         return big
+
+    def broadcast_copy(self, x, to_dims, width=1):
+        """x: array of shape from_dims (7) + (width,); returns to_dims + (width,)."""
+        x = f32(x)
+        from_dims = x.shape[:7]
+        y = np.empty(tuple(to_dims) + (width,), np.float32)
+        self._call("broadcast_copy", ip(i32(to_dims)), ip(i32(from_dims)), width, fp(x), fp(y))
+        return y
 
     def _split_merge(self, big, dim, parts, merge):
         count = len(parts)
@@ -820,6 +871,38 @@ class Hip:
                       self.p(out), self.p(work), size.value)
         return self.down(out).reshape(n, ho, wo, cout)
 
+    def mobilenetv3_pre_se(self, x, expand, channelwise, stride=1):
+        x = f32(x)
+        n, h, w, cin = x.shape
+        ex_f, ex_t, ex_act, ex_param = expand
+        ch_f, ch_t, ch_act, ch_param = channelwise
+        fsize, e = ch_f.shape[0], ch_f.shape[2]
+        pad = (fsize - 1) // 2
+        d = self.conv_desc(n, h, w, e, e, fsize, fsize, pad, pad, stride, stride, channelwise=True)
+        size = ctypes.c_size_t(0)
+        self.na.check(self.lib.nhMobileNetV3PreSEBlockWorkspaceSize(ctypes.byref(d), ctypes.byref(size)))
+        work = self.torch.empty((size.value + 15) // 4 + 4, dtype=self.torch.float32, device=self.dev)
+        up = lambda a: self.up(None if a is None else f32(a))
+        xs, ws = self.up(x), [up(ex_f), up(ex_t), up(ch_f), up(ch_t)]
+        out = self.empty((n, d.resultHeight, d.resultWidth, e))
+        acts = Cpu.ACTIVATIONS
+        self.call("nhMobileNetV3PreSEBlock", ctypes.byref(d), cin, self.p(xs), self.p(ws[0]), self.p(ws[1]), acts[ex_act],
+                  ex_param, self.p(ws[2]), self.p(ws[3]), acts[ch_act], ch_param, self.p(out), self.p(work), size.value)
+        return self.down(out)
+
+    def mobilenetv3_post_se(self, x, gate, residual, activation, param, down, in_place_residual=False):
+        x, gate = f32(x), f32(gate)
+        n, h, w, c = x.shape
+        dn_f, dn_t = down
+        cout = dn_f.shape[0]
+        up = lambda a: self.up(None if a is None else f32(a))
+        xs, gs, rs, fs, ts = self.up(x), self.up(gate), up(residual), up(dn_f), up(dn_t)
+        work = self.torch.empty(x.size + 4, dtype=self.torch.float32, device=self.dev)
+        out = rs if in_place_residual else self.empty((n, h, w, cout))
+        self.call("nhMobileNetV3PostSEBlock", n, h * w, c, cout, self.p(xs), self.p(gs), self.p(rs), Cpu.ACTIVATIONS[activation],
+                  param, self.p(fs), self.p(ts), self.p(out), self.p(work), x.size * 4)
+        return self.down(out).reshape(n, h, w, cout)
+
     # -- gradients
     def conv_backward(self, out_diff, filt, bias, in_shape, ph, pw, sh, sw, dh=1, dw=1):
         out_diff, filt = f32(out_diff), f32(filt)
@@ -917,6 +1000,14 @@ class Hip:
         out = self.empty((n, h + dt + db, w + dl + dr, c))
         self.call("nhBlobResizeImage", ctypes.byref(fd), self.p(xs), dl, dr, dt, db, padding, ctypes.c_float(value),
                   ctypes.byref(td), self.p(out))
+        return self.down(out)
+
+    def broadcast_copy(self, x, to_dims, width=1):
+        x = f32(x)
+        xs = self.up(x)
+        out = self.empty(tuple(to_dims) + (width,))
+        self.call("nhBroadcastCopy", self.p(out), self.p(xs), ctypes.byref(self.na.BlobDesc.of(*to_dims)),
+                  ctypes.byref(self.na.BlobDesc.of(*x.shape[:7])), width)
         return self.down(out)
 
     def split(self, big, dim, part_dims):

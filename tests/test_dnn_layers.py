@@ -247,6 +247,41 @@ def test_optimized_separable_network_on_hip_engine():
     assert_close(got, want, "optimized network on CHipMathEngine vs plain network on CCpuMathEngine")
 
 
+# the MobileNetV3-style network: squeeze-and-excite branches multiplied back through COnnxEltwiseLayer
+SQUEEZE_EXCITE_NET = (7, (1, 3, 1, 32, 40, 1, 3), 10)
+
+
+def test_optimizer_rewrites_the_squeeze_excite_network_on_the_cpu_engine():
+    kind, dims, param = SQUEEZE_EXCITE_NET
+    x = np.random.default_rng(0xC0FFEE + kind).uniform(-1, 1, dims).astype(np.float32)
+    plain = dnn_run(nhtest.cpu_engine(), kind, dims, x, param)
+    assert np.allclose(plain.reshape(dims[1], -1).sum(axis=1), 1.0, atol=1e-5)
+    with optimized():
+        fused = dnn_run(nhtest.cpu_engine(), kind, dims, x, param)
+    assert lib().dnn_last_optimization_mobilenetv3_blocks() == 2
+    assert_close(fused, plain, "optimized vs plain network on the CPU engine")
+
+
+@pytest.mark.gpu
+def test_plain_squeeze_excite_network_on_hip_engine():
+    # COnnxEltwiseLayer's multiplication of [N, H, W, C] by [N, 1, 1, C] goes through BroadcastCopy
+    kind, dims, param = SQUEEZE_EXCITE_NET
+    x = np.random.default_rng(0xC0FFEE + kind).uniform(-1, 1, dims).astype(np.float32)
+    assert_close(dnn_run(nhtest.hip_engine(), kind, dims, x, param), dnn_run(nhtest.cpu_engine(), kind, dims, x, param),
+                 "plain squeeze-and-excite network on CHipMathEngine vs CCpuMathEngine")
+
+
+@pytest.mark.gpu
+def test_optimized_squeeze_excite_network_on_hip_engine():
+    kind, dims, param = SQUEEZE_EXCITE_NET
+    x = np.random.default_rng(0xC0FFEE + kind).uniform(-1, 1, dims).astype(np.float32)
+    want = dnn_run(nhtest.cpu_engine(), kind, dims, x, param)
+    with optimized():
+        got = dnn_run(nhtest.hip_engine(), kind, dims, x, param)
+    assert lib().dnn_last_optimization_mobilenetv3_blocks() == 2
+    assert_close(got, want, "optimized network on CHipMathEngine vs plain network on CCpuMathEngine")
+
+
 @pytest.mark.gpu
 def test_optimized_resnet18_through_cdnn_at_benchmark_size(capsys):
     """The benchmark network after NeoML's OptimizeDnn: its convolution + ReLU pairs become rowwise operation chains,

@@ -11,7 +11,7 @@ import pytest
 import nhtest
 from nhtest import Cpu, assert_close
 from test_oracle import (UNARY_CASES, BINARY_CASES, CONV_CASES, CHANNELWISE_CASES, POOL_CASES, SEPARABLE_CASES,
-                         DIFF_CASES, diff_operands, separable_operands, unary_input, rng)
+                         BROADCAST_CASES, DIFF_CASES, MOBILENETV3_CASES, diff_operands, mobilenetv3_operands, separable_operands, unary_input, rng)
 
 pytestmark = pytest.mark.gpu
 
@@ -488,6 +488,13 @@ def test_resize_image():
                 assert np.array_equal(hip().resize_image(x, dl, dr, dt, db, mode, 0.5), orc.resize_image(x, dl, dr, dt, db, mode, 0.5))
 
 
+@pytest.mark.parametrize("from_dims,to_dims,width", BROADCAST_CASES + [((1, 64, 1, 1, 1, 1, 96), (1, 64, 1, 28, 28, 1, 96), 1)])
+def test_broadcast_copy(from_dims, to_dims, width):
+    g = rng(170 + sum(from_dims))
+    x = g.uniform(-1, 1, from_dims + (width,)).astype(np.float32)
+    assert np.array_equal(hip().broadcast_copy(x, to_dims, width), np.broadcast_to(x, to_dims + (width,)))
+
+
 def test_split_and_merge():
     g = rng(17)
     big = g.uniform(-1, 1, (2, 3, 1, 4, 5, 1, 12)).astype(np.float32)
@@ -548,6 +555,25 @@ def test_separable_blocks(case, with_expand):
         if residual and with_expand:  # the layer of the MobileNetV2 block reuses its input blob
             got = hip().separable_block(x, expand, channelwise, down, stride, residual, in_place=True)
             assert_close(got, want, "separable block in place %s" % (case,))
+
+
+@pytest.mark.parametrize("case", MOBILENETV3_CASES + [
+    (4, 28, 28, 40, 120, 40, 5, 1, True, ("relu", 0.0), ("relu", 0.0), ("relu", 0.0)),
+    (2, 14, 14, 80, 480, 112, 3, 1, False, ("hswish", 0.0), ("hswish", 0.0), ("hswish", 0.0)),
+    (2, 14, 14, 112, 672, 160, 5, 2, False, ("hswish", 0.0), ("hswish", 0.0), ("hswish", 0.0))])
+def test_mobilenetv3_blocks(case):
+    n, h, w, cin, e, cout, fsize, stride, residual, ex_act, ch_act, gate_act = case
+    x, expand, channelwise, gate, down = mobilenetv3_operands(case)
+    pre = orc.mobilenetv3_pre_se(x, expand, channelwise, stride)
+    assert_close(hip().mobilenetv3_pre_se(x, expand, channelwise, stride), pre, "pre-SE %s" % (case,), atol=2e-5)
+    res = x if residual and stride == 1 and cin == cout else None
+    want = orc.mobilenetv3_post_se(pre, gate, res, gate_act[0], gate_act[1], down)
+    assert_close(hip().mobilenetv3_post_se(pre, gate, res, gate_act[0], gate_act[1], down), want, "post-SE %s" % (case,), atol=2e-5)
+    assert_close(hip().mobilenetv3_post_se(pre, gate, None, gate_act[0], gate_act[1], (down[0], None)),
+                 orc.mobilenetv3_post_se(pre, gate, None, gate_act[0], gate_act[1], (down[0], None)), "post-SE, bare", atol=2e-5)
+    if res is not None:  # the layer may hand the residual blob over as the output blob
+        got = hip().mobilenetv3_post_se(pre, gate, res, gate_act[0], gate_act[1], down, in_place_residual=True)
+        assert_close(got, want, "post-SE into its residual", atol=2e-5)
 
 
 def test_lstm_long_sequence():

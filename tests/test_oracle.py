@@ -503,6 +503,51 @@ def test_separable_blocks_against_the_reference_engine(case, with_expand):
                              "separable block in place vs reference")
 
 
+# (n, h, w, cin, expanded, cout, filter size, stride, residual, expand activation, channelwise activation, gate activation)
+MOBILENETV3_CASES = [
+    (2, 9, 11, 8, 48, 8, 3, 1, True, ("hswish", 0.0), ("hswish", 0.0), ("hswish", 0.0)),
+    (1, 12, 10, 16, 64, 24, 5, 2, False, ("relu", 0.0), ("relu", 6.0), ("relu", 0.0)),
+    (2, 7, 7, 12, 20, 12, 5, 1, True, ("hswish", 0.0), (None, 0.0), (None, 0.0)),
+    (1, 6, 5, 3, 5, 7, 3, 2, False, (None, 0.0), ("relu", 2.5), ("hswish", 0.0)),      # channel counts not a multiple of 4
+    (3, 14, 14, 40, 240, 40, 5, 1, True, ("hswish", 0.0), ("hswish", 0.0), ("hswish", 0.0)),
+]
+
+
+def mobilenetv3_operands(case):
+    n, h, w, cin, e, cout, fsize, stride, residual, ex_act, ch_act, gate_act = case
+    g = rng(140 + h * w + e)
+    x = g.uniform(-2, 2, (n, h, w, cin)).astype(np.float32)
+    ft = lambda k: g.uniform(-0.5, 0.5, k).astype(np.float32)
+    expand = (g.normal(0, 1.0 / np.sqrt(cin), (e, cin)).astype(np.float32), ft(e), ex_act[0], ex_act[1])
+    channelwise = (g.normal(0, 0.4, (fsize, fsize, e)).astype(np.float32), ft(e), ch_act[0], ch_act[1])
+    gate = g.uniform(0, 1, (n, e)).astype(np.float32)  # what the squeeze-and-excite branch's hard sigmoid delivers
+    down = (g.normal(0, 1.0 / np.sqrt(e), (cout, e)).astype(np.float32), ft(cout))
+    return x, expand, channelwise, gate, down
+
+
+@needs_ref
+@pytest.mark.parametrize("case", MOBILENETV3_CASES)
+def test_mobilenetv3_blocks_against_the_reference_engine(case):
+    n, h, w, cin, e, cout, fsize, stride, residual, ex_act, ch_act, gate_act = case
+    x, expand, channelwise, gate, down = mobilenetv3_operands(case)
+    pre = orc.mobilenetv3_pre_se(x, expand, channelwise, stride)
+    assert_close(ref().mobilenetv3_pre_se(x, expand, channelwise, stride), pre, "pre-SE %s" % (case,), atol=2e-5)
+    assert_close(ref().mobilenetv3_pre_se(x, expand[:1] + (None,) + expand[2:], channelwise[:1] + (None,) + channelwise[2:], stride),
+                 orc.mobilenetv3_pre_se(x, expand[:1] + (None,) + expand[2:], channelwise[:1] + (None,) + channelwise[2:], stride),
+                 "pre-SE without free terms", atol=2e-5)
+    res = x[:, ::stride, ::stride, :][:, :pre.shape[1], :pre.shape[2], :] if residual and stride == 1 and cin == cout else None
+    post = orc.mobilenetv3_post_se(pre, gate, res, gate_act[0], gate_act[1], down)
+    assert_close(ref().mobilenetv3_post_se(pre, gate, res, gate_act[0], gate_act[1], down), post, "post-SE %s" % (case,), atol=2e-5)
+    # numpy for the post-SE half: gate, activation, matrix product, sum
+    t = pre.astype(np.float64) * gate.reshape(n, 1, 1, e)
+    if gate_act[0] == "relu":
+        t = np.clip(t, 0, gate_act[1]) if gate_act[1] > 0 else np.maximum(t, 0)
+    elif gate_act[0] == "hswish":
+        t = t * np.clip(t + 3, 0, 6) / 6
+    want = t @ down[0].astype(np.float64).T + down[1]
+    assert_close(post, want + (0 if res is None else res), "post-SE vs numpy", atol=2e-5)
+
+
 CHANNELWISE_CASES = [
     # n, h, w, c, fh, fw, ph, pw, sh, sw
     (1, 3, 3, 1, 3, 3, 1, 1, 1, 1), (2, 8, 9, 16, 3, 3, 1, 1, 1, 1), (2, 8, 9, 16, 3, 3, 1, 1, 2, 2),
@@ -681,6 +726,27 @@ def test_resize_image():
         assert np.array_equal(y, want)
         if nhtest.have_reference():
             assert np.array_equal(ref().resize_image(x, dl, dr, dt, db, 0, -1.0), y)
+
+
+BROADCAST_CASES = [
+    # from dims, to dims, additional width
+    ((1, 1, 1, 1, 1, 1, 1), (2, 3, 1, 4, 5, 1, 6), 1),
+    ((1, 3, 1, 1, 1, 1, 6), (1, 3, 1, 4, 5, 1, 6), 1),       # a squeeze-and-excite gate over the pixels
+    ((2, 1, 1, 4, 1, 1, 6), (2, 3, 1, 4, 5, 1, 6), 1),
+    ((2, 3, 1, 4, 5, 1, 1), (2, 3, 1, 4, 5, 1, 6), 1),
+    ((1, 3, 1, 1, 5, 1, 1), (2, 3, 2, 4, 5, 2, 3), 4),
+    ((2, 3, 1, 4, 5, 1, 6), (2, 3, 1, 4, 5, 1, 6), 1),       # nothing to broadcast
+]
+
+
+@pytest.mark.parametrize("from_dims,to_dims,width", BROADCAST_CASES)
+def test_broadcast_copy(from_dims, to_dims, width):
+    g = rng(170 + sum(from_dims))
+    x = g.uniform(-1, 1, from_dims + (width,)).astype(np.float32)
+    y = orc.broadcast_copy(x, to_dims, width)
+    assert np.array_equal(y, np.broadcast_to(x, to_dims + (width,)))
+    if nhtest.have_reference():
+        assert np.array_equal(ref().broadcast_copy(x, to_dims, width), y)
 
 
 def test_split_and_merge():
