@@ -76,6 +76,10 @@ struct CMatMulArgs {
 	// ( ho * StrideH - PadH + kh * DilH ) / UpH and only exists where that division is exact (values <= 1: no division)
 	int UpH, UpW;
 	int ManySlices; // the reduction is far longer than the output is large: as many K slices as fill the device
+	// Tail mode (FullTiles > 0, grid z = 1): the first FullTiles workgroups compute one whole tile each; the workgroups
+	// behind them share the TailTiles remaining tiles, TailSplit slices of TailSteps K steps per tile, and meet in C
+	// through atomic adds like the K slices above
+	int FullTiles, TailTiles, TailSplit, TailSteps;
 	// AM_ConvClasses: the dense result is [images][OutH][OutW][Ldc], DenseM pixels in all
 	int OutH, OutW, OutUpH, OutUpW, DenseM;
 	CConvClass Class[MaxConvClasses];
@@ -134,19 +138,31 @@ void matMulKernel( const CMatMulArgs launchArgs )
 	const int l32 = lane & 31;
 	const int half = lane >> 5;
 
-	const int tile = xcdSwizzle( blockIdx.x, gridDim.x );
+	int tile = xcdSwizzle( blockIdx.x, gridDim.x );
+	int split = blockIdx.z;
+	int splitK = args.SplitK, stepsPerSplit = args.StepsPerSplit;
+	if( args.FullTiles > 0 ) {
+		if( blockIdx.x < args.FullTiles ) {
+			tile = xcdSwizzle( blockIdx.x, args.FullTiles );
+		} else {
+			const int j = blockIdx.x - args.FullTiles;
+			split = j / args.TailTiles;
+			tile = args.FullTiles + ( j - split * args.TailTiles );
+			splitK = args.TailSplit;
+			stepsPerSplit = args.TailSteps;
+		}
+	}
 	const int tileM = tile / args.TilesN;
 	const int tileN = tile % args.TilesN;
 	const int m0 = tileM * BM;
 	const int n0 = tileN * BN;
 	const int batch = blockIdx.y;
-	const int split = blockIdx.z;
 
 	const float* A = args.A + batch * args.BatchStrideA;
 	const float* B = args.B + batch * args.BatchStrideB;
 	float* C = args.C + batch * args.BatchStrideC;
 	const int M = args.M, N = args.N, K = args.K;
-	const int kStart = split * args.StepsPerSplit * NH_KSTEP; // first k of this workgroup's K slice
+	const int kStart = split * stepsPerSplit * NH_KSTEP; // first k of this workgroup's K slice
 	if constexpr( IsClasses ) {
 		// classes differ in their row and reduction counts; the grid is sized for the largest
 		if( m0 >= M || ( split > 0 && kStart >= K ) ) {
@@ -588,7 +604,7 @@ void matMulKernel( const CMatMulArgs launchArgs )
 	//                    step ks+1 are fetched, so neither the LDS latency nor the barrier leaves the MFMA pipe idle.
 	// Buffer (ks+1)%3 was last read in step ks-2, and every wave has passed the barrier of step ks-1 since.
 	const int totalSteps = ( K + KS - 1 ) / KS;
-	const int kSteps = min( args.StepsPerSplit, totalSteps - split * args.StepsPerSplit );
+	const int kSteps = min( stepsPerSplit, totalSteps - split * stepsPerSplit );
 	constexpr int Groups = KS / 8;
 	float4 rA[ASlots], rB[BSlots];
 	CFrag frag[2];
@@ -651,7 +667,7 @@ void matMulKernel( const CMatMulArgs launchArgs )
 							+ outW0 + wo * args.OutUpW;
 					}
 					float* p = C + row * args.Ldc + n;
-					if( args.SplitK > 1 ) {
+					if( splitK > 1 ) {
 						// C was set to the free term (or left as is when accumulating) before the launch
 						unsafeAtomicAdd( p, acc[mi][ni][r] );
 					} else {
@@ -746,6 +762,59 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 	}
 	args.StepsPerSplit = ceilDiv( totalSteps, splits );
 	args.SplitK = ceilDiv( totalSteps, args.StepsPerSplit );
+	// Tail mode: more tiles than run at once, and the last round of them would leave most of the device idle. The tiles
+	// of the whole rounds run as they are; the rest is cut into K slices that fill that last round. Priced in rounds of
+	// whole tiles, from measurements of the 3x3 convolutions: a round filled to the fraction f takes 0.17 + 0.85 f of a
+	// full one (fewer workgroups per compute unit run faster, but not in proportion), a workgroup costs about 4 K steps
+	// beyond its own, and the preset of the tail rows about 2 K steps of a round.
+	const int slots = 256 * ( BM * BN <= 64 * 64 ? 5 : 4 );
+	long long gridX = tiles;
+	int tailRow = 0;
+	if( splits == 1 && batch == 1 && AMODE != AM_ConvClasses && args.Residual == nullptr && tiles >= slots && totalSteps >= 16 ) {
+		long long full = tiles / slots * slots;
+		full -= full % args.TilesN; // whole rows of tiles: the preset below covers the rows behind them
+		const long long rest = tiles - full;
+		auto roundsFor = []( double fill ) {
+			const double whole = floor( fill );
+			const double part = fill - whole;
+			return whole + ( part > 0 ? 0.17 + 0.85 * part : 0.0 );
+		};
+		int best = 1;
+		double bestCost = 0, unsplitCost = 0;
+		for( int slices = 1; slices <= 8 && slices <= totalSteps / 8; ++slices ) {
+			const double length = ( static_cast<double>( totalSteps ) / slices + 4.0 ) / ( totalSteps + 4.0 );
+			const double cost = roundsFor( static_cast<double>( rest * slices ) / slots ) * length
+				+ ( slices > 1 ? 2.0 / totalSteps : 0.0 );
+			if( slices == 1 ) {
+				unsplitCost = cost;
+			}
+			if( slices == 1 || cost < bestCost ) {
+				bestCost = cost;
+				best = slices;
+			}
+		}
+		if( bestCost > unsplitCost - 0.03 ) {
+			best = 1; // not worth the atomics
+		}
+		if( rest > 0 && best > 1 ) {
+			args.FullTiles = static_cast<int>( full );
+			args.TailTiles = static_cast<int>( rest );
+			args.TailSteps = ceilDiv( totalSteps, best );
+			args.TailSplit = ceilDiv( totalSteps, args.TailSteps );
+			gridX = full + rest * args.TailSplit;
+			tailRow = static_cast<int>( full / args.TilesN ) * BM;
+		}
+	}
+	// the rows of the tail tiles as a matrix product of their own: what the preset and the activation pass cover
+	CMatMulArgs tail = args;
+	tail.C += static_cast<long long>( tailRow ) * args.Ldc;
+	tail.M = args.M - tailRow;
+	if( args.FullTiles > 0 && !args.Accumulate ) {
+		const int rc = presetResult( stream, tail, 1 );
+		if( rc != NH_OK ) {
+			return rc;
+		}
+	}
 	if( args.SplitK > 1 && !args.Accumulate ) {
 		CMatMulArgs dense = args;
 		if( AMODE == AM_ConvClasses ) {
@@ -767,11 +836,17 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 		a.A += b0 * args.BatchStrideA;
 		a.B += b0 * args.BatchStrideB;
 		a.C += b0 * args.BatchStrideC;
-		const dim3 grid( static_cast<unsigned>( tiles ), nb, args.SplitK );
+		const dim3 grid( static_cast<unsigned>( gridX ), nb, args.SplitK );
 		if( vec ) {
 			hipLaunchKernelGGL( ( matMulKernel<BM, BN, WAVES_M, WAVES_N, AMODE, BMODE, true> ), grid, dim3( Threads ), 0, stream, a );
 		} else {
 			hipLaunchKernelGGL( ( matMulKernel<BM, BN, WAVES_M, WAVES_N, AMODE, BMODE, false> ), grid, dim3( Threads ), 0, stream, a );
+		}
+		if( args.FullTiles > 0 && actAfter.Type != NH_ACT_NONE ) {
+			const long long total = static_cast<long long>( tail.M ) * args.N;
+			const long long blocksAct = ( total + 1023 ) / 1024;
+			hipLaunchKernelGGL( activateResultKernel, dim3( static_cast<unsigned>( blocksAct > 4096 ? 4096 : blocksAct ), 1 ), dim3( 256 ), 0,
+				stream, tail.C, tail.M, args.N, args.Ldc, args.BatchStrideC, actAfter );
 		}
 		if( args.SplitK > 1 && actAfter.Type != NH_ACT_NONE ) {
 			const long long total = static_cast<long long>( args.M ) * args.N;
