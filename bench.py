@@ -108,7 +108,8 @@ def main():
                     help="after the warm-up steps keep replaying the step untimed for this long, so that the timed region "
                          "starts with the GPU at its sustained clock instead of ramping up from idle")
     ap.add_argument("--fused", action="store_true",
-                    help="mobilenetv2: run the inverted-residual blocks as the graph optimizer's fused block calls")
+                    help="the network as NeoML's graph optimizer rewrites it: resnet18: convolution + ReLU pairs as one "
+                         "engine call; mobilenetv2: the inverted-residual blocks as fused block calls")
     ap.add_argument("--workload", default="resnet18", choices=("resnet18", "mobilenetv2", "transformer", "ocr"),
                     help="resnet18 (default) is the configuration the metric is quoted on; the others are the remaining "
                          "BASELINE configurations, measured the same way with a per-family table on stderr")
@@ -133,7 +134,7 @@ def main():
     from neoml_amd.workloads import HipBackend, ResNet18
 
     be = HipBackend()
-    net = ResNet18(be, batch=args.batch, image=args.image)
+    net = ResNet18(be, batch=args.batch, image=args.image, fused=args.fused)
     x = be.tensor(net.make_input())
     # the launches of one forward pass, arguments bound once: replaying them costs the host a few microseconds
     # per launch, so the timed region is bound by the GPU, not by the Python interpreter
@@ -195,14 +196,34 @@ def main():
         "value": round(images_per_sec, 1), "unit": "images/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "ResNet-18-style inference, batch %d, %dx%dx3, fp32, engine calls through the C ABI" % (
-            args.batch, args.image, args.image), "global_batch": args.batch,
+        "config": {"workload": "ResNet-18-style inference, batch %d, %dx%dx3, fp32, engine calls through the C ABI%s" % (
+            args.batch, args.image, args.image,
+            ", graph as rewritten by OptimizeDnn (convolution + ReLU in one call)" if args.fused else ""),
+            "global_batch": args.batch,
             "gflop_per_step": round(net.conv_flops() / 1e9, 2)},
         "conv_tflops_overall": round(net.conv_flops() / (ms_per_step * 1e-3) / 1e12, 2),
         "host_enqueue_ms_per_step": round((host_done - t0) / args.steps * 1e3, 3),
         "clock_settle": {"ms": args.settle_ms, "untimed_steps": settle_steps},
         "roofline": roofline,
     }
+
+    if not args.fused:
+        # beside the headline: the same network after NeoML's own graph optimizer (OptimizeDnn turns each convolution that
+        # feeds only a ReLU into a rowwise chain = one engine call); same result, fewer passes over the activations
+        opt = ResNet18(be, batch=args.batch, image=args.image, fused=True)
+        opt_plan, opt_out = opt.record_plan(x)
+        torch.cuda.synchronize()
+        steps = max(10, min(args.steps, 50))
+        for _ in range(10):
+            opt_plan.run()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(steps):
+            opt_plan.run()
+        torch.cuda.synchronize()
+        opt_ms = (time.perf_counter() - t1) / steps * 1e3
+        result["optimized_graph"] = {"ms_per_step": round(opt_ms, 3), "images_per_sec": round(args.batch / opt_ms * 1e3, 1),
+                                     "steps": steps, "max_abs_diff_vs_plain": float((opt_out - out).abs().max().item())}
 
     if not args.no_cpu_baseline:
         base, y_cpu = cpu_baseline(args.cpu_sample, args.image)

@@ -89,7 +89,9 @@ class HipBackend:
         self.events.append((tag, flops, nbytes, start, stop))
 
     # ---- ops (shapes are N,H,W,C)
-    def conv(self, x, filt, bias, ph, pw, sh, sw, out=None):
+    def conv(self, x, filt, bias, ph, pw, sh, sw, out=None, relu=False):
+        """relu: the activation in the convolution's own launch, what a rowwise chain of NeoML's graph optimizer
+        (convolution + ReLU) asks of the engine."""
         n, h, w, cin = x.shape
         cout, fh, fw, _ = filt.shape
         key = ("conv", n, h, w, cin, cout, fh, fw, ph, pw, sh, sw)
@@ -102,6 +104,11 @@ class HipBackend:
         if out is None:
             out = self.empty(n, ho, wo, cout)
         tag = "conv%dx%d" % (fh, fw)
+        if relu:
+            self._timed(tag, conv_flops(n, ho, wo, cout, fh, fw, cin), conv_bytes(n, h, w, cin, ho, wo, cout, fh, fw),
+                        self.lib.nhBlobConvolutionWithActivation, ctypes.byref(d), self._p(x), self._p(filt), self._p(bias),
+                        1, ctypes.c_float(0.0), self._p(out))
+            return out
         self._timed(tag, conv_flops(n, ho, wo, cout, fh, fw, cin), conv_bytes(n, h, w, cin, ho, wo, cout, fh, fw),
                     self.lib.nhBlobConvolution, ctypes.byref(d), self._p(x), self._p(filt), self._p(bias), self._p(out))
         return out
@@ -420,8 +427,11 @@ class ResNet18:
 
     STAGES = (64, 128, 256, 512)
 
-    def __init__(self, backend, batch=64, image=224, classes=1000, seed=0xC0FFEE + 2, width_scale=1.0):
+    def __init__(self, backend, batch=64, image=224, classes=1000, seed=0xC0FFEE + 2, width_scale=1.0, fused=False):
+        """fused: the network as NeoML's OptimizeDnn leaves it: every convolution that feeds a ReLU and nothing else
+        (the stem and the first convolution of each block) forms a rowwise chain with it, one engine call."""
         self.be = backend
+        self.fused = fused
         self.batch, self.image, self.classes = batch, image, classes
         g = np.random.default_rng(seed)
         self.widths = [max(4, int(round(c * width_scale / 4)) * 4) for c in self.STAGES]
@@ -488,8 +498,9 @@ class ResNet18:
             return out
 
         f, b = self.dev["stem"]
-        y = run("stem", be.conv, x, f, b, 3, 3, 2, 2)
-        be.relu_(y)
+        y = run("stem", be.conv, x, f, b, 3, 3, 2, 2, relu=self.fused)
+        if not self.fused:
+            be.relu_(y)
         y = run("pad", be.pad, y, 1, 1, 1, 1, 0.0)
         y = run("pool", be.max_pool, y, 3, 3, 2, 2)
         for s in range(len(self.widths)):
@@ -498,8 +509,9 @@ class ResNet18:
                 name = "s%db%d" % (s, blk)
                 f1, b1 = self.dev[name + "c1"]
                 f2, b2 = self.dev[name + "c2"]
-                t = run(name + "c1", be.conv, y, f1, b1, 1, 1, stride, stride)
-                be.relu_(t)
+                t = run(name + "c1", be.conv, y, f1, b1, 1, 1, stride, stride, relu=self.fused)
+                if not self.fused:
+                    be.relu_(t)
                 t = run(name + "c2", be.conv, t, f2, b2, 1, 1, 1, 1)
                 if (name + "sc") in self.dev:
                     fs, bs = self.dev[name + "sc"]

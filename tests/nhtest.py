@@ -1065,8 +1065,9 @@ class CpuBackend:
     def synchronize(self):
         pass
 
-    def conv(self, x, filt, bias, ph, pw, sh, sw, out=None):
-        return self.cpu.conv(x, filt, bias, ph, pw, sh, sw)
+    def conv(self, x, filt, bias, ph, pw, sh, sw, out=None, relu=False):
+        y = self.cpu.conv(x, filt, bias, ph, pw, sh, sw)
+        return self.cpu.unary("relu", y, 0.0).reshape(y.shape) if relu else y
 
     def relu_(self, x, threshold=None):
         x[...] = self.cpu.unary("relu", x, 0.0 if threshold is None else threshold).reshape(x.shape)

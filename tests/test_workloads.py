@@ -22,6 +22,7 @@ def checker():
 
 SMALL = {
     "resnet": lambda be: ResNet18(be, batch=1, image=32, classes=10, width_scale=0.125),
+    "resnet_fused": lambda be: ResNet18(be, batch=1, image=32, classes=10, width_scale=0.125, fused=True),
     "mobilenet": lambda be: MobileNetV2(be, batch=1, image=32, classes=10, head=64),
     "mobilenet_fused": lambda be: MobileNetV2(be, batch=1, image=32, classes=10, head=64, fused=True),
     "transformer": lambda be: TransformerEncoder(be, layers=1, d_model=32, heads=4, ffn=64, seq=8, batch=2),
@@ -30,6 +31,7 @@ SMALL = {
 
 REDUCED = {
     "resnet": lambda be: ResNet18(be, batch=2, image=96, classes=100, width_scale=0.5),
+    "resnet_fused": lambda be: ResNet18(be, batch=2, image=96, classes=100, width_scale=0.5, fused=True),
     "mobilenet": lambda be: MobileNetV2(be, batch=2, image=96, classes=100, head=320),
     "mobilenet_fused": lambda be: MobileNetV2(be, batch=2, image=96, classes=100, head=320, fused=True),
     "transformer": lambda be: TransformerEncoder(be, layers=2, d_model=128, heads=4, ffn=512, seq=64, batch=4),
