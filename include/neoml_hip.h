@@ -150,6 +150,23 @@ NH_API int nhVectorTanh(nhStream s, const float* first, float* result, int vecto
 NH_API int nhVectorNegLog(nhStream s, const float* first, float* result, int vectorSize);            /* NME.h:225 */
 NH_API int nhVectorReLUDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize,
 	const float* upperThreshold);                                                                    /* NME.h:146,148 */
+/* The other activations' derivatives, same convention (Op = through the activation's output). alpha, slope, bias are
+ * read from device memory like the forward parameters. Leaky ReLU and hard tanh have one entry for both forms: the
+ * test is the same on either side of the activation. */
+NH_API int nhVectorELUDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize,
+	const float* alpha_dev);                                                                         /* NME.h:138 */
+NH_API int nhVectorELUDiffOp(nhStream s, const float* first, const float* second, float* result, int vectorSize,
+	const float* alpha_dev);                                                                         /* NME.h:140 */
+NH_API int nhVectorLeakyReLUDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize,
+	const float* alpha_dev);                                                                         /* NME.h:154,157 */
+NH_API int nhVectorHardTanhDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize); /* NME.h:198,200 */
+NH_API int nhVectorHardSigmoidDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize,
+	const float* slope_dev, const float* bias_dev);                                                  /* NME.h:206 */
+NH_API int nhVectorHardSigmoidDiffOp(nhStream s, const float* first, const float* second, float* result, int vectorSize,
+	const float* slope_dev);                                                                         /* NME.h:208 */
+NH_API int nhVectorAbsDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize); /* NME.h:178 */
+/* first - value, or value - first when reverse != 0: the two scalar overloads of VectorSub */
+NH_API int nhVectorSubValue(nhStream s, const float* first, float value, int reverse, float* result, int vectorSize); /* NME.h:251,253 */
 NH_API int nhVectorHSwishDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize);   /* NME.h:164 */
 NH_API int nhVectorSigmoidDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize);  /* NME.h:313 */
 NH_API int nhVectorSigmoidDiffOp(nhStream s, const float* first, const float* second, float* result, int vectorSize); /* NME.h:316 */
@@ -197,6 +214,15 @@ NH_API int nhMultiplyTransposedMatrixByMatrixAndAdd(nhStream s, const float* fir
 	float* result, int resultRowSize, int resultBufferSize);                                         /* NME.h:562 */
 NH_API int nhBatchMultiplyTransposedMatrixByMatrix(nhStream s, int batchSize, const float* first, int firstHeight,
 	int firstWidth, const float* second, int secondWidth, float* result, int resultBufferSize);      /* NME.h:567 */
+/* result[firstSize x secondWidth] += sum over the batch of diag( first[b] ) * second[b] */
+NH_API int nhMultiplyDiagMatrixByMatrixAndAdd(nhStream s, int batchSize, const float* first, int firstSize,
+	const float* second, int secondWidth, float* result);                                            /* NME.h:607 */
+/* result[r] = dot product of row r of first and of second */
+NH_API int nhRowMultiplyMatrixByMatrix(nhStream s, const float* first, const float* second, int height, int width,
+	float* result);                                                                                  /* NME.h:611 */
+/* softmax derivative through its output: result = first * ( second - rowwise <first, second> ), first = softmax(x) */
+NH_API int nhMatrixSoftmaxDiffOpByRows(nhStream s, const float* first, const float* second, int height, int width,
+	float* result);                                                                                  /* NME.h:453 */
 NH_API int nhMultiplyDiagMatrixByMatrix(nhStream s, const float* first, int firstSize, const float* second,
 	int secondWidth, float* result, int resultBufferSize);                                           /* NME.h:570 */
 NH_API int nhBatchMultiplyMatrixByMatrix(nhStream s, int batchSize, const float* first, int firstHeight,

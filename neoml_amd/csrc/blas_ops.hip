@@ -247,6 +247,51 @@ void sumTallRowsKernel( float* result, const float* matrix, int height, int widt
 	}
 }
 
+// result[r] = <first[r], second[r]> (DIFF == false), or the softmax derivative expressed through the softmax's output:
+// result[r][c] = first[r][c] * ( second[r][c] - <first[r], second[r]> ) with first = y, second = dE/dy
+// (src/CPU/CpuMathEngineBlas.cpp:1161-1179). One row per wavefront.
+template<bool DIFF>
+__global__ __launch_bounds__( 256 )
+void rowDotKernel( const float* first, const float* second, int height, int width, float* result )
+{
+	const int row = blockIdx.x * RowsPerBlock + ( threadIdx.x >> 6 );
+	if( row >= height ) {
+		return;
+	}
+	const int lane = threadIdx.x & 63;
+	const float* a = first + static_cast<long long>( row ) * width;
+	const float* b = second + static_cast<long long>( row ) * width;
+	float dot = 0.f;
+	for( int c = lane; c < width; c += 64 ) {
+		dot += a[c] * b[c];
+	}
+	dot = waveReduceSum( dot );
+	if( DIFF ) {
+		float* out = result + static_cast<long long>( row ) * width;
+		for( int c = lane; c < width; c += 64 ) {
+			out[c] = a[c] * ( b[c] - dot );
+		}
+	} else if( lane == 0 ) {
+		result[row] = dot;
+	}
+}
+
+// result[j][c] += sum over b of first[b][j] * second[b][j][c]: one result matrix for the whole batch
+// (src/CPU/x86/CpuX86MathEngineBlas.cpp:401-456)
+__global__ __launch_bounds__( 256 )
+void diagByMatrixAddKernel( int batchSize, const float* first, int firstSize, const float* second, int secondWidth, float* result )
+{
+	const long long total = static_cast<long long>( firstSize ) * secondWidth;
+	for( long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += static_cast<long long>( gridDim.x ) * 256 ) {
+		const int j = static_cast<int>( i / secondWidth );
+		float sum = result[i];
+		for( int b = 0; b < batchSize; ++b ) {
+			sum += first[static_cast<long long>( b ) * firstSize + j] * second[b * total + i];
+		}
+		result[i] = sum;
+	}
+}
+
 // Softmax / log-sum-exp of one row per wavefront. Rows of up to 64 * CACHE elements stay in registers between
 // the three passes (max, sum of exp, scale); longer rows are read again from memory.
 // The formula follows the reference: exp( x - max ) * ( 1 / sum ) (src/CPU/CpuMathEngineBlas.cpp:1131-1159).
@@ -594,6 +639,49 @@ int nhMultiplyDiagMatrixByMatrix( nhStream s, const float* first, int firstSize,
 	NH_REQUIRE( firstSize >= 0 && secondWidth >= 0 );
 	NH_REQUIRE( static_cast<long long>( firstSize ) * secondWidth <= resultBufferSize );
 	return launchColumnBroadcast<BO_Mul>( s, second, result, first, firstSize, secondWidth );
+}
+
+int nhMultiplyDiagMatrixByMatrixAndAdd( nhStream s, int batchSize, const float* first, int firstSize, const float* second,
+	int secondWidth, float* result )
+{
+	NH_REQUIRE( batchSize >= 0 && firstSize >= 0 && secondWidth >= 0 );
+	const long long total = static_cast<long long>( firstSize ) * secondWidth;
+	if( total == 0 || batchSize == 0 ) {
+		return NH_OK;
+	}
+	NH_REQUIRE( first != nullptr && second != nullptr && result != nullptr );
+	long long blocks = ( total + 255 ) / 256;
+	blocks = blocks > 1048576 ? 1048576 : blocks;
+	hipLaunchKernelGGL( diagByMatrixAddKernel, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+		batchSize, first, firstSize, second, secondWidth, result );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+int nhRowMultiplyMatrixByMatrix( nhStream s, const float* first, const float* second, int height, int width, float* result )
+{
+	NH_REQUIRE( height >= 0 && width >= 0 );
+	if( height == 0 ) {
+		return NH_OK;
+	}
+	NH_REQUIRE( first != nullptr && second != nullptr && result != nullptr );
+	hipLaunchKernelGGL( rowDotKernel<false>, dim3( ceilDiv( height, RowsPerBlock ) ), dim3( 256 ), 0, toStream( s ),
+		first, second, height, width, result );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+int nhMatrixSoftmaxDiffOpByRows( nhStream s, const float* first, const float* second, int height, int width, float* result )
+{
+	NH_REQUIRE( height >= 0 && width >= 0 );
+	if( height == 0 || width == 0 ) {
+		return NH_OK;
+	}
+	NH_REQUIRE( first != nullptr && second != nullptr && result != nullptr );
+	hipLaunchKernelGGL( rowDotKernel<true>, dim3( ceilDiv( height, RowsPerBlock ) ), dim3( 256 ), 0, toStream( s ),
+		first, second, height, width, result );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
 }
 
 int nhBatchMultiplyMatrixByDiagMatrix( nhStream s, int batchSize, const float* first, int height, int width,

@@ -280,6 +280,56 @@ struct CReLUDiffOp {
 		return pass ? b : 0.f;
 	}
 };
+struct CELUDiffOp {
+	// first = the input: second where exp( first ) >= 1, else second * exp( first ) * alpha
+	// (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:232-273)
+	const float* Ptr; float Alpha;
+	__device__ void prepare() { Alpha = *Ptr; }
+	__device__ float operator()( float a, float b, float ) const
+	{
+		const float e = expClamped( a );
+		return e >= 1.f ? b : b * e * Alpha;
+	}
+};
+struct CELUDiffOutOp {
+	// first = the output: second where first >= 0, else second * ( first + alpha ) (:275-318)
+	const float* Ptr; float Alpha;
+	__device__ void prepare() { Alpha = *Ptr; }
+	__device__ float operator()( float a, float b, float ) const { return a >= 0.f ? b : b * ( a + Alpha ); }
+};
+struct CLeakyReLUDiffOp {
+	// second above 0, second * alpha below, 0 at 0 as the reference's vector lanes have it (:394-432); the output
+	// form is the same test, alpha being positive
+	const float* Ptr; float Alpha;
+	__device__ void prepare() { Alpha = *Ptr; }
+	__device__ float operator()( float a, float b, float ) const { return a > 0.f ? b : ( a < 0.f ? b * Alpha : 0.f ); }
+};
+struct CHardTanhDiffOp : CNoScalar {
+	// second inside ( -1, 1 ), else 0 (:783-812); serves the output form as well
+	__device__ float operator()( float a, float b, float ) const { return ( -1.f < a && a < 1.f ) ? b : 0.f; }
+};
+struct CHardSigmoidDiffOp {
+	// first = the input: second * slope inside ( -bias / slope, ( 1 - bias ) / slope ), else 0 (:825-875)
+	const float* SlopePtr; const float* BiasPtr; float Slope, Low, High;
+	__device__ void prepare() { Slope = *SlopePtr; const float bias = *BiasPtr; Low = -bias / Slope; High = ( 1.f - bias ) / Slope; }
+	__device__ float operator()( float a, float b, float ) const { return ( Low < a && a < High ) ? b * Slope : 0.f; }
+};
+struct CHardSigmoidDiffOutOp {
+	// first = the output: second * slope inside ( 0, 1 ), else 0 (:877-920)
+	const float* SlopePtr; float Slope;
+	__device__ void prepare() { Slope = *SlopePtr; }
+	__device__ float operator()( float a, float b, float ) const { return ( 0.f < a && a < 1.f ) ? b * Slope : 0.f; }
+};
+struct CAbsDiffOp : CNoScalar {
+	// second above 0, -second otherwise (:550-580)
+	__device__ float operator()( float a, float b, float ) const { return a > 0.f ? b : -b; }
+};
+struct CSubValueOp {
+	// first - Value, or Value - first when Reverse (the scalar forms of VectorSub)
+	float Value; int Reverse;
+	__device__ void prepare() {}
+	__device__ float operator()( float a, float, float ) const { return Reverse ? Value - a : a - Value; }
+};
 struct CHSwishDiffOp : CNoScalar {
 	// 0 below -3, second above 3, second * ( first / 3 + 1/2 ) between (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:433-480)
 	__device__ float operator()( float a, float b, float ) const
@@ -432,6 +482,39 @@ extern "C" int nhVectorReLUDiff( nhStream s, const float* first, const float* se
 	NH_REQUIRE( upperThreshold != nullptr );
 	CReLUDiffOp op; op.Ptr = upperThreshold; op.Threshold = 0;
 	return launchEltwise<2, float, float>( s, first, second, (const float*)nullptr, result, vectorSize, op );
+}
+
+#define NH_BINARY_ALPHA( name, Op ) \
+	extern "C" int name( nhStream s, const float* first, const float* second, float* result, int vectorSize, const float* alpha ) \
+	{ \
+		NH_REQUIRE( alpha != nullptr ); \
+		Op op; op.Ptr = alpha; op.Alpha = 0; \
+		return launchEltwise<2, float, float>( s, first, second, (const float*)nullptr, result, vectorSize, op ); \
+	}
+NH_BINARY_ALPHA( nhVectorELUDiff, CELUDiffOp )
+NH_BINARY_ALPHA( nhVectorELUDiffOp, CELUDiffOutOp )
+NH_BINARY_ALPHA( nhVectorLeakyReLUDiff, CLeakyReLUDiffOp )
+NH_BINARY( nhVectorHardTanhDiff, float, CHardTanhDiffOp )
+NH_BINARY( nhVectorAbsDiff, float, CAbsDiffOp )
+
+extern "C" int nhVectorHardSigmoidDiff( nhStream s, const float* first, const float* second, float* result, int vectorSize,
+	const float* slope, const float* bias )
+{
+	NH_REQUIRE( slope != nullptr && bias != nullptr );
+	CHardSigmoidDiffOp op; op.SlopePtr = slope; op.BiasPtr = bias; op.Slope = op.Low = op.High = 0;
+	return launchEltwise<2, float, float>( s, first, second, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorHardSigmoidDiffOp( nhStream s, const float* first, const float* second, float* result, int vectorSize,
+	const float* slope )
+{
+	NH_REQUIRE( slope != nullptr );
+	CHardSigmoidDiffOutOp op; op.SlopePtr = slope; op.Slope = 0;
+	return launchEltwise<2, float, float>( s, first, second, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorSubValue( nhStream s, const float* first, float value, int reverse, float* result, int vectorSize )
+{
+	CSubValueOp op; op.Value = value; op.Reverse = reverse;
+	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
 }
 
 NH_BINARY( nhVectorEltwiseMax, float, CMaxOp )

@@ -274,6 +274,69 @@ void CHipMathEngine::VectorReLUDiffOp( const CConstFloatHandle& firstHandle, con
 	VectorReLUDiff( firstHandle, secondHandle, resultHandle, vectorSize, upperThresholdHandle );
 }
 
+HIP_BINARY( VectorAbsDiff, CFloatHandle, CConstFloatHandle, nhVectorAbsDiff )
+// inside ( -1, 1 ) on the input exactly where the output is: one test for both forms, as for ReLU
+HIP_BINARY( VectorHardTanhDiff, CFloatHandle, CConstFloatHandle, nhVectorHardTanhDiff )
+HIP_BINARY( VectorHardTanhDiffOp, CFloatHandle, CConstFloatHandle, nhVectorHardTanhDiff )
+
+// result = f'( first; alpha in engine memory ) * second
+#define HIP_BINARY_ALPHA( Method, entry ) \
+	void CHipMathEngine::Method( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle, \
+		const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& alpha ) \
+	{ NH_CALL( entry( stream, raw( firstHandle ), raw( secondHandle ), raw( resultHandle ), vectorSize, raw( alpha ) ) ); }
+
+HIP_BINARY_ALPHA( VectorELUDiff, nhVectorELUDiff )
+HIP_BINARY_ALPHA( VectorELUDiffOp, nhVectorELUDiffOp )
+HIP_BINARY_ALPHA( VectorLeakyReLUDiff, nhVectorLeakyReLUDiff )
+HIP_BINARY_ALPHA( VectorLeakyReLUDiffOp, nhVectorLeakyReLUDiff ) // a positive alpha keeps the sign: same test
+
+void CHipMathEngine::VectorHardSigmoidDiff( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+	const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& slopeHandle,
+	const CConstFloatHandle& biasHandle )
+{
+	NH_CALL( nhVectorHardSigmoidDiff( stream, raw( firstHandle ), raw( secondHandle ), raw( resultHandle ), vectorSize,
+		raw( slopeHandle ), raw( biasHandle ) ) );
+}
+
+void CHipMathEngine::VectorHardSigmoidDiffOp( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+	const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& slopeHandle,
+	const CConstFloatHandle& /*biasHandle*/ )
+{
+	NH_CALL( nhVectorHardSigmoidDiffOp( stream, raw( firstHandle ), raw( secondHandle ), raw( resultHandle ), vectorSize,
+		raw( slopeHandle ) ) );
+}
+
+void CHipMathEngine::VectorSub( const CConstFloatHandle& firstHandle, float second, const CFloatHandle& resultHandle,
+	int vectorSize )
+{
+	NH_CALL( nhVectorSubValue( stream, raw( firstHandle ), second, 0, raw( resultHandle ), vectorSize ) );
+}
+
+void CHipMathEngine::VectorSub( float first, const CConstFloatHandle& secondHandle, const CFloatHandle& resultHandle,
+	int vectorSize )
+{
+	NH_CALL( nhVectorSubValue( stream, raw( secondHandle ), first, 1, raw( resultHandle ), vectorSize ) );
+}
+
+void CHipMathEngine::MatrixSoftmaxDiffOpByRows( const CConstFloatHandle& first, const CConstFloatHandle& second,
+	int height, int width, const CFloatHandle& result )
+{
+	NH_CALL( nhMatrixSoftmaxDiffOpByRows( stream, raw( first ), raw( second ), height, width, raw( result ) ) );
+}
+
+void CHipMathEngine::MultiplyDiagMatrixByMatrixAndAdd( int batchSize, const CConstFloatHandle& firstHandle,
+	int firstSize, const CConstFloatHandle& secondHandle, int secondWidth, const CFloatHandle& resultHandle )
+{
+	NH_CALL( nhMultiplyDiagMatrixByMatrixAndAdd( stream, batchSize, raw( firstHandle ), firstSize, raw( secondHandle ),
+		secondWidth, raw( resultHandle ) ) );
+}
+
+void CHipMathEngine::RowMultiplyMatrixByMatrix( const CConstFloatHandle& firstHandle,
+	const CConstFloatHandle& secondHandle, int height, int width, const CFloatHandle& result )
+{
+	NH_CALL( nhRowMultiplyMatrixByMatrix( stream, raw( firstHandle ), raw( secondHandle ), height, width, raw( result ) ) );
+}
+
 void CHipMathEngine::VectorAddValue( const CConstIntHandle& firstHandle, const CIntHandle& resultHandle, int vectorSize,
 	const CConstIntHandle& addition )
 {

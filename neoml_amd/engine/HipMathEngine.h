@@ -150,6 +150,36 @@ public:
 		const CFloatHandle& resultHandle, int vectorSize ) override;
 	void VectorTanhDiffOp( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
 		const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorELUDiff( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& alpha ) override;
+	void VectorELUDiffOp( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& alpha ) override;
+	void VectorLeakyReLUDiff( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& alpha ) override;
+	void VectorLeakyReLUDiffOp( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& alpha ) override;
+	void VectorAbsDiff( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorHardTanhDiff( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorHardTanhDiffOp( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorHardSigmoidDiff( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& slopeHandle,
+		const CConstFloatHandle& biasHandle ) override;
+	void VectorHardSigmoidDiffOp( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& slopeHandle,
+		const CConstFloatHandle& biasHandle ) override;
+	void VectorSub( const CConstFloatHandle& firstHandle, float second, const CFloatHandle& resultHandle,
+		int vectorSize ) override;
+	void VectorSub( float first, const CConstFloatHandle& secondHandle, const CFloatHandle& resultHandle,
+		int vectorSize ) override;
+	void MatrixSoftmaxDiffOpByRows( const CConstFloatHandle& first, const CConstFloatHandle& second, int height,
+		int width, const CFloatHandle& result ) override;
+	void MultiplyDiagMatrixByMatrixAndAdd( int batchSize, const CConstFloatHandle& firstHandle, int firstSize,
+		const CConstFloatHandle& secondHandle, int secondWidth, const CFloatHandle& resultHandle ) override;
+	void RowMultiplyMatrixByMatrix( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+		int height, int width, const CFloatHandle& result ) override;
 
 	// ---- IBlasEngine ----
 	void SetVectorToMatrixRows( const CFloatHandle& resultHandle, int matrixHeight, int matrixWidth,

@@ -430,7 +430,8 @@ EXPORT int dnn_run( void* engine, int kind, int seed, int param, const int* dims
 // (classes); kind 1: Conv 3x3 p1 (8) - ReLU - MaxPool 2x2/2 - Conv 3x3 p1 stride 2 (16) - ReLU - FullyConnected (classes).
 // kind 2: Conv 3x3 p1 (16) - HSwish - [Conv 3x3 p1 (16) - ReLU - Conv 3x3 p1 (16)] + shortcut - ReLU - MeanPool 2x2/2 -
 // FullyConnected (classes); kind 3: Lstm (24 units, over BatchLength) - FullyConnected (classes) at every step.
-// kind 4: the ResNet-18-style network of dnn_run's kind 5; kind 5: the depthwise-separable network of its kind 6.
+// kind 4: the ResNet-18-style network of dnn_run's kind 5; kind 5: the depthwise-separable network of its kind 6;
+// kind 6: the transformer encoder of its kind 1 with a classifier over every position (input [1, B, seq, 1, 1, 1, hidden]).
 // solver 0: CDnnSimpleGradientSolver, 1: CDnnAdaptiveGradientSolver (Adam), both with L2 regularisation 1e-3.
 // losses receives the loss of every step, output the logits of a final forward pass with the trained weights.
 // timedSteps > 0: that many further steps are timed (the loss is read after the last one, which waits for the device)
@@ -452,7 +453,10 @@ EXPORT int dnn_train( void* engine, int kind, int solverKind, int seed, int clas
 
 		CBaseLayer* last = source.Ptr();
 		CBaseLayer* logits = nullptr;
-		if( kind == 4 ) {
+		if( kind == 6 ) {
+			// two CTransformerEncoderLayers (hidden = the input's channel count), a classifier over every position
+			last = buildTransformer( dnn, e, *source, dims[6] );
+		} else if( kind == 4 ) {
 			logits = buildResNet18( dnn, e, *source, classes, false );
 		} else if( kind == 5 ) {
 			logits = buildSeparableNet( dnn, e, *source, classes, false );

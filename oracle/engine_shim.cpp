@@ -104,7 +104,7 @@ SHIM_API int shim_engine_type( void* engine ) { return static_cast<IMathEngine*>
 enum {
 	OP_RELU = 0, OP_ELU, OP_LEAKY_RELU, OP_HSWISH, OP_ABS, OP_HARD_TANH, OP_HARD_SIGMOID, OP_NEG,
 	OP_EXP, OP_LOG, OP_ERF, OP_SQRT, OP_INV, OP_MINMAX, OP_SIGMOID, OP_TANH,
-	OP_ADD_VALUE, OP_MULTIPLY, OP_NEG_MULTIPLY, OP_COPY, OP_NEG_LOG
+	OP_ADD_VALUE, OP_MULTIPLY, OP_NEG_MULTIPLY, OP_COPY, OP_NEG_LOG, OP_SUB_VALUE, OP_VALUE_SUB
 };
 
 SHIM_API int shim_vector_unary( void* engine, int op, const float* first, float* result, int n, float p0, float p1 )
@@ -134,6 +134,8 @@ SHIM_API int shim_vector_unary( void* engine, int op, const float* first, float*
 			case OP_NEG_MULTIPLY: e.VectorNegMultiply( in.Const(), out.Handle(), n, s0.Const() ); break;
 			case OP_COPY: e.VectorCopy( out.Handle(), in.Const(), n ); break;
 			case OP_NEG_LOG: e.VectorNegLog( in.Const(), out.Handle(), n ); break;
+			case OP_SUB_VALUE: e.VectorSub( in.Const(), p0, out.Handle(), n ); break;
+			case OP_VALUE_SUB: e.VectorSub( p0, in.Const(), out.Handle(), n ); break;
 			default: throw std::logic_error( "bad unary op" );
 		}
 		out.CopyTo( result );
@@ -143,14 +145,17 @@ SHIM_API int shim_vector_unary( void* engine, int op, const float* first, float*
 enum {
 	OP_ADD = 0, OP_SUB, OP_ELTWISE_MULTIPLY, OP_ELTWISE_NEG_MULTIPLY, OP_ELTWISE_DIVIDE, OP_ELTWISE_MAX,
 	OP_ELTWISE_MIN, OP_MULTIPLY_AND_ADD, OP_MULTIPLY_AND_SUB, OP_ELTWISE_MULTIPLY_ADD,
-	OP_RELU_DIFF, OP_HSWISH_DIFF, OP_SIGMOID_DIFF, OP_SIGMOID_DIFF_OP, OP_TANH_DIFF, OP_TANH_DIFF_OP
+	OP_RELU_DIFF, OP_HSWISH_DIFF, OP_SIGMOID_DIFF, OP_SIGMOID_DIFF_OP, OP_TANH_DIFF, OP_TANH_DIFF_OP,
+	OP_ELU_DIFF, OP_ELU_DIFF_OP, OP_LEAKY_RELU_DIFF, OP_HARD_TANH_DIFF, OP_HARD_SIGMOID_DIFF, OP_HARD_SIGMOID_DIFF_OP,
+	OP_ABS_DIFF
 };
 
-SHIM_API int shim_vector_binary( void* engine, int op, const float* first, const float* second, float* result, int n, float p0 )
+SHIM_API int shim_vector_binary( void* engine, int op, const float* first, const float* second, float* result, int n, float p0,
+	float p1 )
 {
 	return guarded( [&]() {
 		IMathEngine& e = *static_cast<IMathEngine*>( engine );
-		CFloatBlob a( e, n, first ), b( e, n, second ), out( e, n, result ), s0( e, 1, &p0 );
+		CFloatBlob a( e, n, first ), b( e, n, second ), out( e, n, result ), s0( e, 1, &p0 ), s1( e, 1, &p1 );
 		switch( op ) {
 			case OP_ADD: e.VectorAdd( a.Const(), b.Const(), out.Handle(), n ); break;
 			case OP_SUB: e.VectorSub( a.Const(), b.Const(), out.Handle(), n ); break;
@@ -169,6 +174,13 @@ SHIM_API int shim_vector_binary( void* engine, int op, const float* first, const
 			case OP_SIGMOID_DIFF_OP: e.VectorSigmoidDiffOp( a.Const(), b.Const(), out.Handle(), n ); break;
 			case OP_TANH_DIFF: e.VectorTanhDiff( a.Const(), b.Const(), out.Handle(), n ); break;
 			case OP_TANH_DIFF_OP: e.VectorTanhDiffOp( a.Const(), b.Const(), out.Handle(), n ); break;
+			case OP_ELU_DIFF: e.VectorELUDiff( a.Const(), b.Const(), out.Handle(), n, s0.Const() ); break;
+			case OP_ELU_DIFF_OP: e.VectorELUDiffOp( a.Const(), b.Const(), out.Handle(), n, s0.Const() ); break;
+			case OP_LEAKY_RELU_DIFF: e.VectorLeakyReLUDiff( a.Const(), b.Const(), out.Handle(), n, s0.Const() ); break;
+			case OP_HARD_TANH_DIFF: e.VectorHardTanhDiff( a.Const(), b.Const(), out.Handle(), n ); break;
+			case OP_HARD_SIGMOID_DIFF: e.VectorHardSigmoidDiff( a.Const(), b.Const(), out.Handle(), n, s0.Const(), s1.Const() ); break;
+			case OP_HARD_SIGMOID_DIFF_OP: e.VectorHardSigmoidDiffOp( a.Const(), b.Const(), out.Handle(), n, s0.Const(), s1.Const() ); break;
+			case OP_ABS_DIFF: e.VectorAbsDiff( a.Const(), b.Const(), out.Handle(), n ); break;
 			default: throw std::logic_error( "bad binary op" );
 		}
 		out.CopyTo( result );
@@ -783,6 +795,37 @@ SHIM_API int shim_blob_resize_image( void* engine, const float* from, int n, int
 			: ( padding == 1 ? TBlobResizePadding::Edge : TBlobResizePadding::Reflect );
 		e.BlobResizeImage( inDesc, src.Handle(), dl, dr, dt, db, mode, value, outDesc, dst.Handle() );
 		dst.CopyTo( to );
+	} );
+}
+
+SHIM_API int shim_row_multiply_matrix_by_matrix( void* engine, const float* first, const float* second, int h, int w, float* result )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		CFloatBlob a( e, h * w, first ), b( e, h * w, second ), out( e, h );
+		e.RowMultiplyMatrixByMatrix( a.Const(), b.Const(), h, w, out.Handle() );
+		out.CopyTo( result );
+	} );
+}
+
+SHIM_API int shim_matrix_softmax_diff_op_by_rows( void* engine, const float* first, const float* second, int h, int w, float* result )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		CFloatBlob a( e, h * w, first ), b( e, h * w, second ), out( e, h * w );
+		e.MatrixSoftmaxDiffOpByRows( a.Const(), b.Const(), h, w, out.Handle() );
+		out.CopyTo( result );
+	} );
+}
+
+SHIM_API int shim_multiply_diag_matrix_by_matrix_and_add( void* engine, int batch, const float* first, int size, const float* second,
+	int width, float* result )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		CFloatBlob a( e, batch * size, first ), b( e, batch * size * width, second ), out( e, size * width, result );
+		e.MultiplyDiagMatrixByMatrixAndAdd( batch, a.Const(), size, b.Const(), width, out.Handle() );
+		out.CopyTo( result );
 	} );
 }
 

@@ -57,7 +57,8 @@ static float orc_exp_clamped(float x)
 enum {
 	ORC_RELU = 0, ORC_ELU, ORC_LEAKY_RELU, ORC_HSWISH, ORC_ABS, ORC_HARD_TANH, ORC_HARD_SIGMOID, ORC_NEG,
 	ORC_EXP, ORC_LOG, ORC_ERF, ORC_SQRT, ORC_INV, ORC_MINMAX, ORC_SIGMOID, ORC_TANH,
-	ORC_ADD_VALUE, ORC_MULTIPLY, ORC_NEG_MULTIPLY, ORC_COPY, ORC_NEG_LOG
+	ORC_ADD_VALUE, ORC_MULTIPLY, ORC_NEG_MULTIPLY, ORC_COPY, ORC_NEG_LOG,
+	ORC_SUB_VALUE, ORC_VALUE_SUB /* x - p0 and p0 - x: the scalar forms of VectorSub */
 };
 
 /* result[i] = f(first[i]; p0, p1) */
@@ -94,6 +95,8 @@ ORC_API void orc_vector_unary(int op, const float* first, float* result, int n, 
 		case ORC_NEG_MULTIPLY: y = -x * p0; break;
 		case ORC_COPY: y = x; break;
 		/* VectorLog with the sign flipped (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:1692-1720) */
+		case ORC_SUB_VALUE: y = x - p0; break;
+		case ORC_VALUE_SUB: y = p0 - x; break;
 		case ORC_NEG_LOG: { float c = x > FLT_MIN ? x : FLT_MIN; c = c < FLT_MAX ? c : FLT_MAX; y = -logf(c); } break;
 		default: y = NAN; break;
 		}
@@ -106,11 +109,15 @@ enum {
 	ORC_ELTWISE_MIN, ORC_MULTIPLY_AND_ADD, ORC_MULTIPLY_AND_SUB, ORC_ELTWISE_MULTIPLY_ADD,
 	/* derivatives of the activations times second; the _OP forms take the activation's output as first
 	 * (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:339-395, 433-480, 1377-1520) */
-	ORC_RELU_DIFF, ORC_HSWISH_DIFF, ORC_SIGMOID_DIFF, ORC_SIGMOID_DIFF_OP, ORC_TANH_DIFF, ORC_TANH_DIFF_OP
+	ORC_RELU_DIFF, ORC_HSWISH_DIFF, ORC_SIGMOID_DIFF, ORC_SIGMOID_DIFF_OP, ORC_TANH_DIFF, ORC_TANH_DIFF_OP,
+	/* (:232-318 ELU, p0 = alpha; :394-432 leaky ReLU, p0 = alpha; :783-812 hard tanh; :825-920 hard sigmoid, p0 = slope,
+	 * p1 = bias; :550-580 abs) */
+	ORC_ELU_DIFF, ORC_ELU_DIFF_OP, ORC_LEAKY_RELU_DIFF, ORC_HARD_TANH_DIFF, ORC_HARD_SIGMOID_DIFF, ORC_HARD_SIGMOID_DIFF_OP,
+	ORC_ABS_DIFF
 };
 
-/* result[i] = f(first[i], second[i]; p0); ORC_ELTWISE_MULTIPLY_ADD reads result[i] as the addend */
-ORC_API void orc_vector_binary(int op, const float* first, const float* second, float* result, int n, float p0)
+/* result[i] = f(first[i], second[i]; p0, p1); ORC_ELTWISE_MULTIPLY_ADD reads result[i] as the addend */
+ORC_API void orc_vector_binary(int op, const float* first, const float* second, float* result, int n, float p0, float p1)
 {
 	for (int i = 0; i < n; ++i) {
 		const float a = first[i], b = second[i];
@@ -132,6 +139,13 @@ ORC_API void orc_vector_binary(int op, const float* first, const float* second, 
 		case ORC_SIGMOID_DIFF_OP: y = a * (1.f - a) * b; break;
 		case ORC_TANH_DIFF: { const float t = -1.f + 2.f / (1.f + orc_exp_clamped(-2.f * a)); y = b * (1.f - t * t); } break;
 		case ORC_TANH_DIFF_OP: y = (1.f - a * a) * b; break;
+		case ORC_ELU_DIFF: { const float e = orc_exp_clamped(a); y = e >= 1.f ? b : b * e * p0; } break;
+		case ORC_ELU_DIFF_OP: y = a >= 0.f ? b : b * (a + p0); break;
+		case ORC_LEAKY_RELU_DIFF: y = a > 0.f ? b : (a < 0.f ? b * p0 : 0.f); break;
+		case ORC_HARD_TANH_DIFF: y = (-1.f < a && a < 1.f) ? b : 0.f; break;
+		case ORC_HARD_SIGMOID_DIFF: y = (-p1 / p0 < a && a < (1.f - p1) / p0) ? b * p0 : 0.f; break;
+		case ORC_HARD_SIGMOID_DIFF_OP: y = (0.f < a && a < 1.f) ? b * p0 : 0.f; break;
+		case ORC_ABS_DIFF: y = a > 0.f ? b : -b; break;
 		default: y = NAN; break;
 		}
 		result[i] = y;
@@ -453,6 +467,41 @@ ORC_API void orc_blob_convolution_learn_add(const float* in, int n, int h, int w
 					float* d = filterDiff + (((size_t)co * fh + ky) * fw + kx) * cin + ci;
 					*d = (float)(*d + s);
 				}
+}
+
+/* result[r] = <first[r], second[r]> (src/CPU/CpuMathEngineBlas.cpp RowMultiplyMatrixByMatrix) */
+ORC_API void orc_row_multiply_matrix_by_matrix(const float* first, const float* second, int h, int w, float* result)
+{
+	for (int r = 0; r < h; ++r) {
+		double s = 0;
+		for (int c = 0; c < w; ++c) s += (double)first[(size_t)r * w + c] * second[(size_t)r * w + c];
+		result[r] = (float)s;
+	}
+}
+
+/* dE/dx of a softmax over rows from its output y = first and dE/dy = second: y * ( dE/dy - <dE/dy, y> )
+ * (src/CPU/CpuMathEngineBlas.cpp:1161-1179) */
+ORC_API void orc_matrix_softmax_diff_op_by_rows(const float* first, const float* second, int h, int w, float* result)
+{
+	for (int r = 0; r < h; ++r) {
+		double dot = 0;
+		for (int c = 0; c < w; ++c) dot += (double)first[(size_t)r * w + c] * second[(size_t)r * w + c];
+		for (int c = 0; c < w; ++c)
+			result[(size_t)r * w + c] = first[(size_t)r * w + c] * (second[(size_t)r * w + c] - (float)dot);
+	}
+}
+
+/* result[j][c] += sum over b of first[b][j] * second[b][j][c] (src/CPU/x86/CpuX86MathEngineBlas.cpp:401-456) */
+ORC_API void orc_multiply_diag_matrix_by_matrix_and_add(int batch, const float* first, int size, const float* second, int width,
+	float* result)
+{
+	for (int j = 0; j < size; ++j)
+		for (int c = 0; c < width; ++c) {
+			double s = result[(size_t)j * width + c];
+			for (int b = 0; b < batch; ++b)
+				s += (double)first[(size_t)b * size + j] * second[((size_t)b * size + j) * width + c];
+			result[(size_t)j * width + c] = (float)s;
+		}
 }
 
 /* BroadcastCopy: `from` repeats along every dimension where it has size 1 and `to` does not; width is one more,

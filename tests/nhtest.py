@@ -19,11 +19,12 @@ ATOL = 1e-5
 
 UNARY = {name: i for i, name in enumerate([
     "relu", "elu", "leaky_relu", "hswish", "abs", "hard_tanh", "hard_sigmoid", "neg", "exp", "log", "erf", "sqrt",
-    "inv", "minmax", "sigmoid", "tanh", "add_value", "multiply", "neg_multiply", "copy", "neg_log"])}
+    "inv", "minmax", "sigmoid", "tanh", "add_value", "multiply", "neg_multiply", "copy", "neg_log", "sub_value", "value_sub"])}
 BINARY = {name: i for i, name in enumerate([
     "add", "sub", "eltwise_multiply", "eltwise_neg_multiply", "eltwise_divide", "eltwise_max", "eltwise_min",
     "multiply_and_add", "multiply_and_sub", "eltwise_multiply_add", "relu_diff", "hswish_diff", "sigmoid_diff",
-    "sigmoid_diff_op", "tanh_diff", "tanh_diff_op"])}
+    "sigmoid_diff_op", "tanh_diff", "tanh_diff_op", "elu_diff", "elu_diff_op", "leaky_relu_diff", "hard_tanh_diff",
+    "hard_sigmoid_diff", "hard_sigmoid_diff_op", "abs_diff"])}
 BINARY_INT = {"add": 0, "sub": 1, "multiply": 2}
 
 c_float_p = ctypes.POINTER(ctypes.c_float)
@@ -153,11 +154,30 @@ class Cpu:
         self._call("vector_unary", UNARY[op], fp(x), fp(y), x.size, ctypes.c_float(p0), ctypes.c_float(p1))
         return y
 
-    def binary(self, op, a, b, p0=0.0, result=None):
+    def binary(self, op, a, b, p0=0.0, result=None, p1=0.0):
         a, b = f32(a), f32(b)
         y = np.zeros_like(a) if result is None else f32(result).copy()
-        self._call("vector_binary", BINARY[op], fp(a), fp(b), fp(y), a.size, ctypes.c_float(p0))
+        self._call("vector_binary", BINARY[op], fp(a), fp(b), fp(y), a.size, ctypes.c_float(p0), ctypes.c_float(p1))
         return y
+
+    def row_dot(self, a, b):
+        a, b = f32(a), f32(b)
+        y = np.empty(a.shape[0], np.float32)
+        self._call("row_multiply_matrix_by_matrix", fp(a), fp(b), a.shape[0], a.shape[1], fp(y))
+        return y
+
+    def softmax_diff_rows(self, y, grad):
+        y, grad = f32(y), f32(grad)
+        out = np.empty_like(y)
+        self._call("matrix_softmax_diff_op_by_rows", fp(y), fp(grad), y.shape[0], y.shape[1], fp(out))
+        return out
+
+    def diag_by_matrix_add(self, diag, matrix, result):
+        """diag [B][n], matrix [B][n][w], result [n][w] (accumulated into)."""
+        diag, matrix = f32(diag), f32(matrix)
+        out = f32(result).copy()
+        self._call("multiply_diag_matrix_by_matrix_and_add", diag.shape[0], fp(diag), diag.shape[1], fp(matrix), matrix.shape[2], fp(out))
+        return out
 
     def binary_int(self, op, a, b):
         a, b = i32(a), i32(b)
@@ -629,6 +649,7 @@ class Hip:
         "neg_multiply": ("nhVectorNegMultiply", 1), "neg_log": ("nhVectorNegLog", 0),
     }
 
+
     def unary(self, op, x, p0=0.0, p1=0.0, inplace=False, offset=0):
         """offset > 0 runs on a view that starts `offset` elements into a buffer (unaligned pointers)."""
         x = f32(x).ravel()
@@ -644,6 +665,9 @@ class Hip:
         if op == "copy":
             self.call("nhVectorCopy", self.p(dst), self.p(src), n)
             return self.down(dst)
+        if op in ("sub_value", "value_sub"):
+            self.call("nhVectorSubValue", self.p(src), p0, 1 if op == "value_sub" else 0, self.p(dst), n)
+            return self.down(dst)
         fn, nscalars = self.UNARY_FN[op]
         scalars = [self.scalar(p0), self.scalar(p1)][:nscalars]
         self.call(fn, self.p(src), self.p(dst), n, *[self.p(s) for s in scalars])
@@ -657,17 +681,45 @@ class Hip:
         "eltwise_multiply_add": "nhVectorEltwiseMultiplyAdd", "relu_diff": "nhVectorReLUDiff",
         "hswish_diff": "nhVectorHSwishDiff", "sigmoid_diff": "nhVectorSigmoidDiff",
         "sigmoid_diff_op": "nhVectorSigmoidDiffOp", "tanh_diff": "nhVectorTanhDiff", "tanh_diff_op": "nhVectorTanhDiffOp",
+        "elu_diff": "nhVectorELUDiff", "elu_diff_op": "nhVectorELUDiffOp", "leaky_relu_diff": "nhVectorLeakyReLUDiff",
+        "hard_tanh_diff": "nhVectorHardTanhDiff", "hard_sigmoid_diff": "nhVectorHardSigmoidDiff",
+        "hard_sigmoid_diff_op": "nhVectorHardSigmoidDiffOp", "abs_diff": "nhVectorAbsDiff",
     }
 
-    def binary(self, op, a, b, p0=0.0, result=None, inplace_first=False):
+    def binary(self, op, a, b, p0=0.0, result=None, inplace_first=False, p1=0.0):
         a, b = self.up(f32(a).ravel()), self.up(f32(b).ravel())
         n = a.numel()
         out = a if inplace_first else (self.empty((n,)) if result is None else self.up(f32(result).ravel()))
         args = [self.p(a), self.p(b), self.p(out), n]
-        if op in ("multiply_and_add", "multiply_and_sub", "relu_diff"):
+        keep = []
+        if op in ("multiply_and_add", "multiply_and_sub", "relu_diff", "elu_diff", "elu_diff_op", "leaky_relu_diff",
+                  "hard_sigmoid_diff", "hard_sigmoid_diff_op"):
             s = self.scalar(p0)
             args.append(self.p(s))
+        if op == "hard_sigmoid_diff":
+            keep.append(self.scalar(p1))
+            args.append(self.p(keep[0]))
         self.call(self.BINARY_FN[op], *args)
+        return self.down(out)
+
+    def row_dot(self, a, b):
+        a, b = f32(a), f32(b)
+        xa, xb = self.up(a), self.up(b)
+        out = self.empty((a.shape[0],))
+        self.call("nhRowMultiplyMatrixByMatrix", self.p(xa), self.p(xb), a.shape[0], a.shape[1], self.p(out))
+        return self.down(out)
+
+    def softmax_diff_rows(self, y, grad, inplace=False):
+        y, grad = f32(y), f32(grad)
+        xa, xb = self.up(y), self.up(grad)
+        out = xb if inplace else self.empty(y.shape)
+        self.call("nhMatrixSoftmaxDiffOpByRows", self.p(xa), self.p(xb), y.shape[0], y.shape[1], self.p(out))
+        return self.down(out)
+
+    def diag_by_matrix_add(self, diag, matrix, result):
+        diag, matrix = f32(diag), f32(matrix)
+        xd, xm, out = self.up(diag), self.up(matrix), self.up(f32(result))
+        self.call("nhMultiplyDiagMatrixByMatrixAndAdd", diag.shape[0], self.p(xd), diag.shape[1], self.p(xm), matrix.shape[2], self.p(out))
         return self.down(out)
 
     def binary_int(self, op, a, b):

@@ -10,7 +10,7 @@ import pytest
 
 import nhtest
 from nhtest import Cpu, assert_close
-from test_oracle import (UNARY_CASES, BINARY_CASES, CONV_CASES, CHANNELWISE_CASES, POOL_CASES, SEPARABLE_CASES,
+from test_oracle import (HARD_SIGMOID_BIAS, UNARY_CASES, BINARY_CASES, CONV_CASES, CHANNELWISE_CASES, POOL_CASES, SEPARABLE_CASES,
                          BROADCAST_CASES, DIFF_CASES, MOBILENETV3_CASES, diff_operands, mobilenetv3_operands, separable_operands, unary_input, rng)
 
 pytestmark = pytest.mark.gpu
@@ -69,9 +69,27 @@ def test_binary(op):
 def test_activation_derivatives(op, p):
     for n in (1, 5, 1003, 300003):
         a, b = diff_operands(op, n, 70 + n)
-        assert_close(hip().binary(op, a, b, p), orc.binary(op, a, b, p), "%s n=%d" % (op, n))
+        assert_close(hip().binary(op, a, b, p, p1=HARD_SIGMOID_BIAS), orc.binary(op, a, b, p, p1=HARD_SIGMOID_BIAS), "%s n=%d" % (op, n))
     a, b = diff_operands(op, 4099, 3)
-    assert_close(hip().binary(op, a, b, p, inplace_first=True), orc.binary(op, a, b, p), op + " into its first operand")
+    assert_close(hip().binary(op, a, b, p, inplace_first=True, p1=HARD_SIGMOID_BIAS), orc.binary(op, a, b, p, p1=HARD_SIGMOID_BIAS),
+                 op + " into its first operand")
+
+
+def test_row_products_softmax_derivative_and_diag_accumulation():
+    g = rng(81)
+    for h, w in ((1, 1), (3, 5), (17, 64), (40, 101), (9, 300), (8192, 256), (2048, 1000)):
+        a = g.uniform(-1, 1, (h, w)).astype(np.float32)
+        b = g.uniform(-1, 1, (h, w)).astype(np.float32)
+        assert_close(hip().row_dot(a, b), orc.row_dot(a, b), "row dot %s" % ((h, w),), atol=1e-5 * np.sqrt(w))
+        y = orc.softmax_rows(a)
+        want = orc.softmax_diff_rows(y, b)
+        assert_close(hip().softmax_diff_rows(y, b), want, "softmax derivative %s" % ((h, w),), atol=1e-6)
+        assert_close(hip().softmax_diff_rows(y, b, inplace=True), want, "softmax derivative into the gradient", atol=1e-6)
+    for batch, n, w in ((1, 1, 1), (1, 7, 5), (3, 6, 33), (2, 40, 64), (1, 8192, 512)):
+        diag = g.uniform(-1, 1, (batch, n)).astype(np.float32)
+        m = g.uniform(-1, 1, (batch, n, w)).astype(np.float32)
+        start = g.uniform(-1, 1, (n, w)).astype(np.float32)
+        assert_close(hip().diag_by_matrix_add(diag, m, start), orc.diag_by_matrix_add(diag, m, start), "diag accumulate %s" % ((batch, n, w),))
 
 
 def test_int_ops_fill_convert():

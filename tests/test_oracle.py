@@ -34,6 +34,7 @@ UNARY_CASES = [
     ("abs", 0, 0), ("hard_tanh", 0, 0), ("hard_sigmoid", 0.2, 0.5), ("neg", 0, 0), ("exp", 0, 0), ("log", 0, 0),
     ("erf", 0, 0), ("sqrt", 0, 0), ("inv", 0, 0), ("minmax", -0.5, 1.5), ("sigmoid", 0, 0), ("tanh", 0, 0),
     ("add_value", 1.25, 0), ("multiply", -2.5, 0), ("neg_multiply", 1.702, 0), ("copy", 0, 0), ("neg_log", 0, 0),
+    ("sub_value", 0.75, 0), ("value_sub", 0.75, 0),
 ]
 
 
@@ -69,6 +70,8 @@ NUMPY_UNARY = {
     "neg_multiply": lambda x, p0, p1: -x * np.float32(p0),
     "copy": lambda x, p0, p1: x,
     "neg_log": lambda x, p0, p1: -np.log(np.clip(x.astype(np.float64), np.finfo(np.float32).tiny, None)),
+    "sub_value": lambda x, p0, p1: x - np.float32(p0),
+    "value_sub": lambda x, p0, p1: np.float32(p0) - x,
 }
 
 
@@ -133,7 +136,9 @@ def test_binary(op):
 # derivatives of the activations: first = the activation's input (or its output for the _op forms), second = the
 # gradient that arrives from above, p = ReLU's upper threshold
 DIFF_CASES = [("relu_diff", 0.0), ("relu_diff", 6.0), ("hswish_diff", 0.0), ("sigmoid_diff", 0.0), ("sigmoid_diff_op", 0.0),
-              ("tanh_diff", 0.0), ("tanh_diff_op", 0.0)]
+              ("tanh_diff", 0.0), ("tanh_diff_op", 0.0), ("elu_diff", 0.7), ("elu_diff_op", 0.7), ("leaky_relu_diff", 0.1),
+              ("hard_tanh_diff", 0.0), ("hard_sigmoid_diff", 0.2), ("hard_sigmoid_diff_op", 0.2), ("abs_diff", 0.0)]
+HARD_SIGMOID_BIAS = 0.5  # second parameter of the hard sigmoid cases
 _expit = lambda a: scipy.special.expit(a.astype(np.float64))
 NUMPY_DIFF = {
     "relu_diff": lambda a, b, p: np.where((a > 0) & ((a < p) if p > 0 else True), b, 0),
@@ -142,16 +147,28 @@ NUMPY_DIFF = {
     "sigmoid_diff_op": lambda a, b, p: a.astype(np.float64) * (1 - a) * b,
     "tanh_diff": lambda a, b, p: (1 - np.tanh(a.astype(np.float64)) ** 2) * b,
     "tanh_diff_op": lambda a, b, p: (1 - a.astype(np.float64) ** 2) * b,
+    "elu_diff": lambda a, b, p: np.where(a >= 0, b, b * p * np.exp(np.minimum(a, 0).astype(np.float64))),
+    "elu_diff_op": lambda a, b, p: np.where(a >= 0, b, b * (a.astype(np.float64) + p)),
+    "leaky_relu_diff": lambda a, b, p: np.where(a > 0, b, b * np.float32(p)),
+    "hard_tanh_diff": lambda a, b, p: np.where(np.abs(a) < 1, b, 0),
+    "hard_sigmoid_diff": lambda a, b, p: np.where((a * p + HARD_SIGMOID_BIAS > 0) & (a * p + HARD_SIGMOID_BIAS < 1), b * np.float32(p), 0),
+    "hard_sigmoid_diff_op": lambda a, b, p: np.where((a > 0) & (a < 1), b * np.float32(p), 0),
+    "abs_diff": lambda a, b, p: np.where(a > 0, b, -b),
 }
 # the activation each derivative belongs to, for the finite-difference check
-DIFF_FORWARD = {"relu_diff": "relu", "hswish_diff": "hswish", "sigmoid_diff": "sigmoid", "tanh_diff": "tanh"}
+DIFF_FORWARD = {"relu_diff": "relu", "hswish_diff": "hswish", "sigmoid_diff": "sigmoid", "tanh_diff": "tanh", "elu_diff": "elu",
+                "leaky_relu_diff": "leaky_relu", "hard_tanh_diff": "hard_tanh", "hard_sigmoid_diff": "hard_sigmoid", "abs_diff": "abs"}
 
 
 def diff_operands(op, n, seed):
     g = rng(seed)
     a = g.uniform(-8, 8, n).astype(np.float32)
-    if op.endswith("_op"):
+    if op in ("sigmoid_diff_op", "tanh_diff_op"):
         a = g.uniform(-0.99 if op.startswith("tanh") else 0.01, 0.99, n).astype(np.float32)
+    elif op in ("elu_diff_op", "hard_sigmoid_diff_op"):  # outputs of the activation: ELU above -alpha, hard sigmoid in [0, 1]
+        a = g.uniform(-0.69, 3, n).astype(np.float32) if op == "elu_diff_op" else np.clip(g.uniform(-0.5, 1.5, n), 0, 1).astype(np.float32)
+    elif op in ("leaky_relu_diff", "abs_diff"):
+        pass  # no special values: at exactly 0 the reference's vector lanes and its scalar tail disagree
     elif n >= 8:
         a[:8] = [0.0, 3.0, -3.0, 6.0, 2.999, -2.999, 40.0, -40.0]
     b = g.uniform(-2, 2, n).astype(np.float32)
@@ -162,10 +179,10 @@ def diff_operands(op, n, seed):
 def test_activation_derivatives(op, p):
     for n in (1, 5, 1003):
         a, b = diff_operands(op, n, 70 + n)
-        y = orc.binary(op, a, b, p)
+        y = orc.binary(op, a, b, p, p1=HARD_SIGMOID_BIAS)
         assert_close(y, NUMPY_DIFF[op](a, b, p), "%s n=%d" % (op, n))
         if nhtest.have_reference():
-            assert_close(ref().binary(op, a, b, p), y, "%s vs reference n=%d" % (op, n))
+            assert_close(ref().binary(op, a, b, p, p1=HARD_SIGMOID_BIAS), y, "%s vs reference n=%d" % (op, n))
 
 
 @pytest.mark.parametrize("op,p", [c for c in DIFF_CASES if c[0] in DIFF_FORWARD])
@@ -176,12 +193,39 @@ def test_activation_derivatives_are_the_slopes_of_the_activations(op, p):
     a = a[(np.abs(a) > 0.05)]
     eps = np.float32(1.0 / 256)
     fwd = DIFF_FORWARD[op]
-    slope = (orc.unary(fwd, a + eps, p).astype(np.float64) - orc.unary(fwd, a - eps, p)) / (2.0 * float(eps))
-    y = orc.binary(op, a, np.ones_like(a), p)
+    if op in ("hard_tanh_diff", "hard_sigmoid_diff"):
+        a = a[np.abs(np.abs(a) - (1.0 if op == "hard_tanh_diff" else 2.5)) > 0.05]  # away from their kinks as well
+    slope = (orc.unary(fwd, a + eps, p, HARD_SIGMOID_BIAS).astype(np.float64) - orc.unary(fwd, a - eps, p, HARD_SIGMOID_BIAS)) / (2.0 * float(eps))
+    y = orc.binary(op, a, np.ones_like(a), p, p1=HARD_SIGMOID_BIAS)
     np.testing.assert_allclose(y, slope, rtol=2e-3, atol=2e-4)
     if op in ("sigmoid_diff", "tanh_diff"):  # the _op form on the activation's output is the same derivative
         out = orc.unary(fwd, a)
         assert_close(orc.binary(op + "_op", out, np.ones_like(a)), y, op + " through the output", atol=1e-5)
+
+
+def test_row_products_softmax_derivative_and_diag_accumulation():
+    g = rng(81)
+    for h, w in ((1, 1), (3, 5), (17, 64), (40, 101), (9, 300)):
+        a = g.uniform(-1, 1, (h, w)).astype(np.float32)
+        b = g.uniform(-1, 1, (h, w)).astype(np.float32)
+        dot = orc.row_dot(a, b)
+        assert_close(dot, np.einsum("rc,rc->r", a.astype(np.float64), b), "row dot %s" % ((h, w),))
+        y = scipy.special.softmax(a.astype(np.float64), axis=1).astype(np.float32)
+        d = orc.softmax_diff_rows(y, b)
+        # the Jacobian of softmax, written out: diag(y) - y y^T, applied to the incoming gradient
+        want = np.stack([(np.diag(y[r].astype(np.float64)) - np.outer(y[r], y[r])) @ b[r] for r in range(h)])
+        assert_close(d, want, "softmax derivative %s" % ((h, w),), atol=1e-6)
+        if nhtest.have_reference():
+            assert_close(ref().row_dot(a, b), dot, "row dot vs reference")
+            assert_close(ref().softmax_diff_rows(y, b), d, "softmax derivative vs reference", atol=1e-6)
+    for batch, n, w in ((1, 1, 1), (1, 7, 5), (3, 6, 33), (2, 40, 64)):
+        diag = g.uniform(-1, 1, (batch, n)).astype(np.float32)
+        m = g.uniform(-1, 1, (batch, n, w)).astype(np.float32)
+        start = g.uniform(-1, 1, (n, w)).astype(np.float32)
+        got = orc.diag_by_matrix_add(diag, m, start)
+        assert_close(got, start + np.einsum("bn,bnw->nw", diag.astype(np.float64), m), "diag accumulate %s" % ((batch, n, w),))
+        if nhtest.have_reference():
+            assert_close(ref().diag_by_matrix_add(diag, m, start), got, "diag accumulate vs reference")
 
 
 def test_int_ops_and_conversions():
