@@ -257,6 +257,12 @@ NH_API int nhBlobSplitByDim(nhStream s, int dim, const nhBlobDesc* from_host, co
 NH_API int nhBroadcastCopy(nhStream s, void* to, const void* from, const nhBlobDesc* to_host,
 	const nhBlobDesc* from_host, int additionalWidth);                                               /* NME.h:80,82 */
 
+/* Dropout (InitDropout + Dropout, NME.h:932-935) with the very mask the reference's CPU engine draws for the same seed
+ * (src/CPU/CpuRandom.h): out = in * mask / (1 - rate). Spatial: whole channels of an object; batchwise: the same mask
+ * for every object. in == out is allowed. */
+NH_API int nhDropout(nhStream s, const nhBlobDesc* input_host, float rate, int isSpatial, int isBatchwise, int seed,
+	const float* in, float* out);
+
 enum { NH_PAD_CONSTANT = 0, NH_PAD_EDGE = 1, NH_PAD_REFLECT = 2 }; /* TBlobResizePadding, NME.h:62-66 */
 NH_API int nhBlobResizeImage(nhStream s, const nhBlobDesc* from_host, const float* fromData, int deltaLeft,
 	int deltaRight, int deltaTop, int deltaBottom, int padding, float defaultValue,

@@ -1151,6 +1151,53 @@ void broadcastCopyKernel( unsigned* to, const unsigned* from, const CBroadcastSh
 	}
 }
 
+// Dropout with the mask of the reference's CPU engine: the counter-based generator of src/CPU/CpuRandom.h (ten rounds of
+// Philox 4x32 on the counter { n, 0, seed ^ 0xBADFACE, seed ^ 0xBADBEEF }, key { seed, seed ^ 0xBADF00D }), four mask
+// values per counter value n, kept where the 32-bit value is <= threshold. Being counter-based it needs no state: every
+// thread computes the word of its own mask element.
+__device__ __forceinline__ unsigned dropoutWord( unsigned generation, int lane, unsigned seed )
+{
+	unsigned c0 = generation, c1 = 0, c2 = seed ^ 0xBADFACEu, c3 = seed ^ 0xBADBEEFu;
+	unsigned k0 = seed, k1 = seed ^ 0xBADF00Du;
+#pragma unroll
+	for( int round = 0; round < 10; ++round ) {
+		const unsigned long long first = 0xD2511F53ull * c0;
+		const unsigned long long second = 0xCD9E8D57ull * c2;
+		const unsigned n0 = static_cast<unsigned>( second >> 32 ) ^ c1 ^ k0;
+		const unsigned n1 = static_cast<unsigned>( second );
+		const unsigned n2 = static_cast<unsigned>( first >> 32 ) ^ c3 ^ k1;
+		const unsigned n3 = static_cast<unsigned>( first );
+		c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+		k0 += 0x9E3779B9u;
+		k1 += 0xBB67AE85u;
+	}
+	return lane == 0 ? c0 : ( lane == 1 ? c1 : ( lane == 2 ? c2 : c3 ) );
+}
+
+// Mask layout (src/CPU/CpuMathEngineDnnDropout.cpp:33-96). Plain: one mask of batchWidth * objectSize values, shared by
+// the batchLength outer slices. Spatial: one value per ( object of the batch width, channel ), shared by every pixel and
+// by the outer slices; the generator runs on from object to object, ceil( channels / 4 ) counter values each.
+__global__ __launch_bounds__( 256 )
+void dropoutKernel( const float* in, float* out, long long total, int maskSize, int objectSize, int channels, int batchWidth,
+	int spatial, unsigned seed, unsigned threshold, float value )
+{
+	for( long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += static_cast<long long>( gridDim.x ) * 256 ) {
+		unsigned generation;
+		int lane;
+		if( spatial ) {
+			const int c = static_cast<int>( i % channels );
+			const int object = static_cast<int>( ( i / objectSize ) % batchWidth );
+			generation = static_cast<unsigned>( object ) * ( ( channels + 3 ) / 4 ) + c / 4;
+			lane = c & 3;
+		} else {
+			const int m = static_cast<int>( i % maskSize );
+			generation = m / 4;
+			lane = m & 3;
+		}
+		out[i] = dropoutWord( generation, lane, seed ) <= threshold ? in[i] * value : in[i] * 0.f;
+	}
+}
+
 __global__ void addTwoVectorsKernel( const float* a, const float* b, float* out, int n )
 {
 	const int i = blockIdx.x * 256 + threadIdx.x;
@@ -1668,6 +1715,36 @@ int nhBroadcastCopy( nhStream s, void* to, const void* from, const nhBlobDesc* t
 	blocks = blocks > 1048576 ? 1048576 : blocks;
 	hipLaunchKernelGGL( broadcastCopyKernel, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
 		static_cast<unsigned*>( to ), static_cast<const unsigned*>( from ), shape, total );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+int nhDropout( nhStream s, const nhBlobDesc* input, float rate, int isSpatial, int isBatchwise, int seed, const float* in,
+	float* out )
+{
+	NH_REQUIRE( input != nullptr && rate >= 0.f && rate < 1.f );
+	const long long objectCount = dimProduct( *input, 0, 3 );
+	const long long objectSize = dimProduct( *input, 3, 7 );
+	const long long total = objectCount * objectSize;
+	if( total == 0 ) {
+		return NH_OK;
+	}
+	NH_REQUIRE( in != nullptr && out != nullptr && total <= 0x7fffffffLL );
+	const float forwardRate = 1.f - rate;
+	if( forwardRate == 1.f ) {
+		return nhVectorCopy( s, out, in, static_cast<int>( total ) );
+	}
+	// batchwise: every object is its own outer slice, the mask covers one object
+	const long long batchLength = isBatchwise ? objectCount : input->dims[0];
+	const int batchWidth = static_cast<int>( objectCount / batchLength );
+	const int channels = input->dims[6];
+	const long long maskSize = isSpatial ? static_cast<long long>( batchWidth ) * channels : batchWidth * objectSize;
+	const unsigned threshold = static_cast<unsigned>( static_cast<double>( forwardRate ) * 4294967295.0 );
+	long long blocks = ( total + 255 ) / 256;
+	blocks = blocks > 1048576 ? 1048576 : blocks;
+	hipLaunchKernelGGL( dropoutKernel, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+		in, out, total, static_cast<int>( maskSize ), static_cast<int>( objectSize ), channels, batchWidth, isSpatial ? 1 : 0,
+		static_cast<unsigned>( seed ), threshold, 1.f / forwardRate );
 	NH_LAUNCH_CHECK();
 	return NH_OK;
 }

@@ -786,6 +786,34 @@ void CHipMathEngine::BlobMeanPoolingBackward( const CMeanPoolingDesc& desc, cons
 	NH_CALL( nhBlobMeanPoolingBackward( stream, &d.D, raw( resultDiff ), raw( sourceDiff ) ) );
 }
 
+struct CHipDropoutDesc : public CDropoutDesc {
+	nhBlobDesc Input;
+	float Rate;
+	bool IsSpatial, IsBatchwise;
+	int Seed;
+};
+
+CDropoutDesc* CHipMathEngine::InitDropout( float rate, bool isSpatial, bool isBatchwise, const CBlobDesc& input,
+	const CBlobDesc& output, int seed )
+{
+	ASSERT_EXPR( rate >= 0.f && rate < 1.f );
+	ASSERT_EXPR( input.HasEqualDimensions( output ) );
+	CHipDropoutDesc* desc = new CHipDropoutDesc();
+	desc->Input = toBlobDesc( input );
+	desc->Rate = rate;
+	desc->IsSpatial = isSpatial;
+	desc->IsBatchwise = isBatchwise;
+	desc->Seed = seed;
+	return desc;
+}
+
+void CHipMathEngine::Dropout( const CDropoutDesc& desc, const CFloatHandle& input, const CFloatHandle& output )
+{
+	const CHipDropoutDesc& d = static_cast<const CHipDropoutDesc&>( desc );
+	NH_CALL( nhDropout( stream, &d.Input, d.Rate, d.IsSpatial ? 1 : 0, d.IsBatchwise ? 1 : 0, d.Seed, raw( input ),
+		raw( output ) ) );
+}
+
 CLstmDesc* CHipMathEngine::InitLstm( int hiddenSize, int objectSize, const CConstFloatHandle& inputWeights,
 	const CConstFloatHandle& inputFreeTerm, const CConstFloatHandle& recurrentWeights,
 	const CConstFloatHandle& recurrentFreeTerm )

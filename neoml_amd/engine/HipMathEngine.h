@@ -274,6 +274,9 @@ public:
 		const CFloatHandle& result ) override;
 	void BlobMeanPoolingBackward( const CMeanPoolingDesc& desc, const CConstFloatHandle& resultDiff,
 		const CFloatHandle& sourceDiff ) override;
+	CDropoutDesc* InitDropout( float rate, bool isSpatial, bool isBatchwise, const CBlobDesc& input,
+		const CBlobDesc& output, int seed ) override;
+	void Dropout( const CDropoutDesc& desc, const CFloatHandle& input, const CFloatHandle& output ) override;
 	CLstmDesc* InitLstm( int hiddenSize, int objectSize, const CConstFloatHandle& inputWeights,
 		const CConstFloatHandle& inputFreeTerm, const CConstFloatHandle& recurrentWeights,
 		const CConstFloatHandle& recurrentFreeTerm ) override;

@@ -72,15 +72,15 @@ static CBaseLayer* buildCnn( CDnn& dnn, IMathEngine& e, CBaseLayer& source )
 }
 
 // kind 1: two CTransformerEncoderLayer (4 heads, FFN 4x, GELU, post-norm, no dropout). Input: [1, B, S, 1, 1, 1, D].
-static CBaseLayer* buildTransformer( CDnn& dnn, IMathEngine& e, CBaseLayer& source, int hidden )
+static CBaseLayer* buildTransformer( CDnn& dnn, IMathEngine& e, CBaseLayer& source, int hidden, float dropout = 0.f )
 {
 	CBaseLayer* last = &source;
 	for( int i = 0; i < 2; ++i ) {
 		CPtr<CTransformerEncoderLayer> layer = add( dnn, new CTransformerEncoderLayer( e ), i == 0 ? "enc0" : "enc1", *last );
 		layer->SetHeadCount( 4 );
 		layer->SetHiddenSize( hidden );
-		layer->SetDropoutRate( 0.f );
-		layer->SetSelfAttentionDropoutRate( 0.f );
+		layer->SetDropoutRate( dropout );
+		layer->SetSelfAttentionDropoutRate( dropout );
 		layer->SetFeedForwardSize( 4 * hidden );
 		layer->SetActivation( CActivationDesc( AF_GELU ) );
 		last = layer.Ptr();
@@ -453,9 +453,10 @@ EXPORT int dnn_train( void* engine, int kind, int solverKind, int seed, int clas
 
 		CBaseLayer* last = source.Ptr();
 		CBaseLayer* logits = nullptr;
-		if( kind == 6 ) {
-			// two CTransformerEncoderLayers (hidden = the input's channel count), a classifier over every position
-			last = buildTransformer( dnn, e, *source, dims[6] );
+		if( kind == 6 || kind == 7 ) {
+			// two CTransformerEncoderLayers (hidden = the input's channel count), a classifier over every position;
+			// kind 7: with dropout 0.1 inside the layers (the masks come from the network's CRandom seeds)
+			last = buildTransformer( dnn, e, *source, dims[6], kind == 7 ? 0.1f : 0.f );
 		} else if( kind == 4 ) {
 			logits = buildResNet18( dnn, e, *source, classes, false );
 		} else if( kind == 5 ) {

@@ -829,6 +829,29 @@ SHIM_API int shim_multiply_diag_matrix_by_matrix_and_add( void* engine, int batc
 	} );
 }
 
+// InitDropout + Dropout (NeoMathEngine.h:930-935); dims: the 7 blob dimensions
+SHIM_API int shim_dropout( void* engine, const int* dims, float rate, int isSpatial, int isBatchwise, int seed, const float* in,
+	float* out )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		CBlobDesc desc( CT_Float );
+		for( int i = 0; i < 7; ++i ) {
+			desc.SetDimSize( i, dims[i] );
+		}
+		CFloatBlob src( e, desc.BlobSize(), in ), dst( e, desc.BlobSize() );
+		CDropoutDesc* dropout = e.InitDropout( rate, isSpatial != 0, isBatchwise != 0, desc, desc, seed );
+		try {
+			e.Dropout( *dropout, src.Handle(), dst.Handle() );
+		} catch( ... ) {
+			delete dropout;
+			throw;
+		}
+		delete dropout;
+		dst.CopyTo( out );
+	} );
+}
+
 // BroadcastCopy (NeoMathEngine.h:75-83): toDims / fromDims are the 7 blob dimensions, without the additional width
 SHIM_API int shim_broadcast_copy( void* engine, const int* toDims, const int* fromDims, int additionalWidth, const float* from,
 	float* to )

@@ -504,6 +504,67 @@ ORC_API void orc_multiply_diag_matrix_by_matrix_and_add(int batch, const float* 
 		}
 }
 
+/* Dropout as the reference's CPU engine draws it (src/CPU/CpuMathEngineDnnDropout.cpp:33-96, generator src/CPU/CpuRandom.h):
+ * ten rounds of Philox 4x32 on a running 128-bit counter, four mask values per counter value, consumed in the loop
+ * order of the engine (mask chunks of 64 values; spatial: object after object of the batch width). */
+typedef struct { unsigned seed; unsigned counter[4]; } orc_random;
+
+static void orc_random_next(orc_random* r, unsigned out[4])
+{
+	unsigned key[2] = { r->seed, r->seed ^ 0xBADF00Du };
+	unsigned c[4] = { r->counter[0], r->counter[1], r->counter[2], r->counter[3] };
+	for (int round = 0; round < 10; ++round) {
+		const unsigned long long first = 0xD2511F53ull * c[0];
+		const unsigned long long second = 0xCD9E8D57ull * c[2];
+		const unsigned n0 = (unsigned)(second >> 32) ^ c[1] ^ key[0];
+		const unsigned n2 = (unsigned)(first >> 32) ^ c[3] ^ key[1];
+		c[1] = (unsigned)second; c[3] = (unsigned)first; c[0] = n0; c[2] = n2;
+		key[0] += 0x9E3779B9u;
+		key[1] += 0xBB67AE85u;
+	}
+	for (int k = 0; k < 4; ++k) out[k] = c[k];
+	if (++r->counter[0] == 0 && ++r->counter[1] == 0 && ++r->counter[2] == 0) ++r->counter[3];
+}
+
+/* dims: the 7 blob dimensions */
+ORC_API void orc_dropout(const int* dims, float rate, int isSpatial, int isBatchwise, int seed, const float* in, float* out)
+{
+	const float forwardRate = 1.f - rate;
+	const int objectCount = dims[0] * dims[1] * dims[2];
+	const int inputObjectSize = dims[3] * dims[4] * dims[5] * dims[6];
+	if (forwardRate == 1.f) {
+		memcpy(out, in, sizeof(float) * (size_t)objectCount * inputObjectSize);
+		return;
+	}
+	const float value = 1.f / forwardRate;
+	const unsigned threshold = (unsigned)((double)forwardRate * 4294967295.0);
+	const int objectSize = isSpatial ? dims[6] : inputObjectSize;
+	const int batchLength = isBatchwise ? objectCount : dims[0];
+	const int batchWidth = objectCount / batchLength;
+	const int unitSize = isSpatial ? objectSize : batchWidth * objectSize;
+	const int pixels = isSpatial ? inputObjectSize / objectSize : 1;
+	const int objects = isSpatial ? batchWidth : 1;
+	const size_t sliceStep = isSpatial ? (size_t)batchWidth * inputObjectSize : (size_t)unitSize;
+	orc_random random = { (unsigned)seed, { 0, 0, (unsigned)seed ^ 0xBADFACEu, (unsigned)seed ^ 0xBADBEEFu } };
+	float mask[64];
+	for (int object = 0; object < objects; ++object) {
+		const size_t base = isSpatial ? (size_t)object * inputObjectSize : 0;
+		for (int chunk = 0; chunk * 64 < unitSize; ++chunk) {
+			const int size = unitSize - chunk * 64 < 64 ? unitSize - chunk * 64 : 64;
+			for (int g = 0; g * 4 < size; ++g) {
+				unsigned word[4];
+				orc_random_next(&random, word);
+				for (int k = 0; k < 4; ++k) mask[g * 4 + k] = word[k] <= threshold ? value : 0.f;
+			}
+			for (int b = 0; b < batchLength; ++b)
+				for (int p = 0; p < pixels; ++p) {
+					const size_t at = base + b * sliceStep + (size_t)p * objectSize + (size_t)chunk * 64;
+					for (int k = 0; k < size; ++k) out[at + k] = in[at + k] * mask[k];
+				}
+		}
+	}
+}
+
 /* BroadcastCopy: `from` repeats along every dimension where it has size 1 and `to` does not; width is one more,
  * innermost, dimension that both share (src/CPU/CpuMathEngineVectorMath.cpp:69-95 builds the same result by growing
  * the copied block dimension by dimension from the innermost) */

@@ -537,6 +537,13 @@ class Cpu:
         self._split_merge(big, dim, parts, merge=1)
         return big
 
+    def dropout(self, x, rate, spatial=False, batchwise=False, seed=1):
+        """x: 7-D blob."""
+        x = f32(x)
+        y = np.empty_like(x)
+        self._call("dropout", ip(i32(x.shape)), ctypes.c_float(rate), 1 if spatial else 0, 1 if batchwise else 0, seed, fp(x), fp(y))
+        return y
+
     def broadcast_copy(self, x, to_dims, width=1):
         """x: array of shape from_dims (7) + (width,); returns to_dims + (width,)."""
         x = f32(x)
@@ -1052,6 +1059,14 @@ class Hip:
         out = self.empty((n, h + dt + db, w + dl + dr, c))
         self.call("nhBlobResizeImage", ctypes.byref(fd), self.p(xs), dl, dr, dt, db, padding, ctypes.c_float(value),
                   ctypes.byref(td), self.p(out))
+        return self.down(out)
+
+    def dropout(self, x, rate, spatial=False, batchwise=False, seed=1, inplace=False):
+        x = f32(x)
+        xs = self.up(x)
+        out = xs if inplace else self.empty(x.shape)
+        self.call("nhDropout", ctypes.byref(self.na.BlobDesc.of(*x.shape)), rate, 1 if spatial else 0, 1 if batchwise else 0, seed,
+                  self.p(xs), self.p(out))
         return self.down(out)
 
     def broadcast_copy(self, x, to_dims, width=1):

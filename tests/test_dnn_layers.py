@@ -321,6 +321,7 @@ TRAIN_CASES = {
     "resnet18_sgd": (4, (1, 2, 1, 64, 64, 1, 3), 0, 0.002),
     "separable_sgd": (5, (1, 3, 1, 24, 24, 1, 3), 0, 0.02),
     "transformer_adam": (6, (1, 2, 8, 1, 1, 1, 32), 1, 0.003),
+    "transformer_dropout_adam": (7, (1, 2, 8, 1, 1, 1, 32), 1, 0.003),
 }
 
 

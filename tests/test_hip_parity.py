@@ -11,7 +11,7 @@ import pytest
 import nhtest
 from nhtest import Cpu, assert_close
 from test_oracle import (HARD_SIGMOID_BIAS, UNARY_CASES, BINARY_CASES, CONV_CASES, CHANNELWISE_CASES, POOL_CASES, SEPARABLE_CASES,
-                         BROADCAST_CASES, DIFF_CASES, MOBILENETV3_CASES, diff_operands, mobilenetv3_operands, separable_operands, unary_input, rng)
+                         BROADCAST_CASES, DIFF_CASES, DROPOUT_CASES, MOBILENETV3_CASES, diff_operands, mobilenetv3_operands, separable_operands, unary_input, rng)
 
 pytestmark = pytest.mark.gpu
 
@@ -511,6 +511,19 @@ def test_broadcast_copy(from_dims, to_dims, width):
     g = rng(170 + sum(from_dims))
     x = g.uniform(-1, 1, from_dims + (width,)).astype(np.float32)
     assert np.array_equal(hip().broadcast_copy(x, to_dims, width), np.broadcast_to(x, to_dims + (width,)))
+
+
+@pytest.mark.parametrize("dims,rate,spatial,batchwise", DROPOUT_CASES + [((1, 64, 1, 28, 28, 1, 96), 0.2, False, False),
+                                                                          ((1, 64, 1, 28, 28, 1, 96), 0.2, True, False)])
+def test_dropout_mask_bit_exact(dims, rate, spatial, batchwise):
+    g = rng(180 + sum(dims))
+    x = g.uniform(0.5, 1.5, dims).astype(np.float32)
+    for seed in (1, 12345, -7):
+        want = orc.dropout(x, rate, spatial, batchwise, seed)
+        got = hip().dropout(x, rate, spatial, batchwise, seed)
+        assert np.array_equal(got != 0, want != 0), "dropout mask"
+        assert_close(got, want, "dropout values")
+    assert np.array_equal(hip().dropout(x, rate, spatial, batchwise, 5, inplace=True) != 0, orc.dropout(x, rate, spatial, batchwise, 5) != 0)
 
 
 def test_split_and_merge():

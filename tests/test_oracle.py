@@ -793,6 +793,40 @@ def test_broadcast_copy(from_dims, to_dims, width):
         assert np.array_equal(ref().broadcast_copy(x, to_dims, width), y)
 
 
+# blob dims, rate, spatial, batchwise
+DROPOUT_CASES = [
+    ((1, 4, 1, 1, 1, 1, 10), 0.3, False, False), ((3, 4, 1, 5, 6, 1, 7), 0.5, False, False),
+    ((3, 4, 1, 5, 6, 1, 7), 0.5, False, True), ((2, 3, 2, 4, 4, 1, 70), 0.25, True, False),
+    ((2, 3, 1, 4, 4, 1, 9), 0.6, True, True), ((1, 2, 1, 1, 1, 1, 1000), 0.1, False, False),
+    ((1, 5, 1, 3, 3, 1, 130), 0.4, True, False), ((2, 2, 1, 2, 2, 1, 3), 0.0, False, False),
+]
+
+
+@pytest.mark.parametrize("dims,rate,spatial,batchwise", DROPOUT_CASES)
+def test_dropout_draws_the_reference_mask(dims, rate, spatial, batchwise):
+    g = rng(180 + sum(dims))
+    x = g.uniform(0.5, 1.5, dims).astype(np.float32)
+    for seed in (1, 12345, -7):
+        y = orc.dropout(x, rate, spatial, batchwise, seed)
+        kept = y != 0
+        assert np.array_equal(y[kept], (x * np.float32(1.0 / (1.0 - rate)))[kept]) or np.allclose(y[kept], x[kept] / (1 - rate), rtol=1e-6)
+        if rate == 0.0:
+            assert kept.all()
+        # the mask repeats over the outer slices; the spatial one also over the pixels of an object
+        objects = dims[0] * dims[1] * dims[2]
+        outer = objects if batchwise else dims[0]
+        per = kept.reshape(outer, -1)
+        assert (per == per[0]).all()
+        if spatial:
+            pix = kept.reshape(objects, -1, dims[6])
+            assert (pix == pix[:, :1, :]).all()
+        if nhtest.have_reference():
+            assert np.array_equal(ref().dropout(x, rate, spatial, batchwise, seed), y), "mask differs from the reference's"
+    if x.size >= 1000 and not spatial:
+        frac = np.mean([(orc.dropout(x, rate, spatial, batchwise, s) != 0).mean() for s in range(20)])
+        assert abs(frac - (1 - rate)) < 0.03
+
+
 def test_split_and_merge():
     g = rng(17)
     big = g.uniform(-1, 1, (2, 3, 1, 4, 5, 1, 12)).astype(np.float32)
