@@ -94,8 +94,12 @@ constexpr int Threads = 256;
 #define NH_KSTEP 16
 #endif
 
-template<int BM, int BN, int WAVES_M, int WAVES_N, int AMODE, int BMODE, bool VEC>
-__global__ __launch_bounds__( Threads, 2 )
+// KGROUPS == 2: the workgroup has two groups of 4 wavefronts; each group runs the whole pipeline on its own LDS buffers
+// over one half of the K steps of the tile, then the second group hands its accumulators to the first through LDS.
+// For problems of a few hundred tiles with a reduction long enough to cut in two: the same number of waves per compute
+// unit as two K slices in separate workgroups, without the preset of C, the atomics and the separate activation pass.
+template<int BM, int BN, int WAVES_M, int WAVES_N, int AMODE, int BMODE, bool VEC, int KGROUPS = 1>
+__global__ __launch_bounds__( Threads * KGROUPS, KGROUPS == 1 ? 2 : 1 )
 void matMulKernel( const CMatMulArgs launchArgs )
 {
 	constexpr bool IsClasses = ( AMODE == AM_ConvClasses );
@@ -127,10 +131,12 @@ void matMulKernel( const CMatMulArgs launchArgs )
 	constexpr int ASlots = ( ATotal + Threads - 1 ) / Threads;
 	constexpr int BSlots = ( BTotal + Threads - 1 ) / Threads;
 
-	__shared__ __attribute__( ( aligned( 16 ) ) ) float ldsA[3][ASize];
-	__shared__ __attribute__( ( aligned( 16 ) ) ) float ldsB[3][BSize];
+	__shared__ __attribute__( ( aligned( 16 ) ) ) float lds[KGROUPS][3][ASize + BSize];
 
-	const int tid = threadIdx.x;
+	const int kGroup = KGROUPS == 1 ? 0 : threadIdx.x / Threads;
+	const int tid = KGROUPS == 1 ? threadIdx.x : threadIdx.x % Threads; // inside the group
+	auto ldsA = [&]( int buf ) -> float* { return lds[kGroup][buf]; };
+	auto ldsB = [&]( int buf ) -> float* { return lds[kGroup][buf] + ASize; };
 	const int lane = tid & 63;
 	const int wave = tid >> 6;
 	const int waveM = wave / WAVES_N;
@@ -162,6 +168,11 @@ void matMulKernel( const CMatMulArgs launchArgs )
 	const float* B = args.B + batch * args.BatchStrideB;
 	float* C = args.C + batch * args.BatchStrideC;
 	const int M = args.M, N = args.N, K = args.K;
+	if constexpr( KGROUPS == 2 ) {
+		// the launch has one slice ( split == 0 ) of an even number of steps: this group's half of it
+		stepsPerSplit = ( ( K + NH_KSTEP - 1 ) / NH_KSTEP ) / 2;
+		split = kGroup;
+	}
 	const int kStart = split * stepsPerSplit * NH_KSTEP; // first k of this workgroup's K slice
 	if constexpr( IsClasses ) {
 		// classes differ in their row and reduction counts; the grid is sized for the largest
@@ -517,9 +528,9 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			const int slot = tid + i * Threads;
 			if( ATotal % Threads == 0 || slot < ATotal ) {
 				if( AK ) {
-					*reinterpret_cast<float4*>( &ldsA[buf][( slot / KQ ) * LdsK + ( slot % KQ ) * 4] ) = regA[i];
+					*reinterpret_cast<float4*>( &ldsA( buf )[( slot / KQ ) * LdsK + ( slot % KQ ) * 4] ) = regA[i];
 				} else {
-					*reinterpret_cast<float4*>( &ldsA[buf][( slot / ( BM / 4 ) ) * APitchX + ( slot % ( BM / 4 ) ) * 4] ) = regA[i];
+					*reinterpret_cast<float4*>( &ldsA( buf )[( slot / ( BM / 4 ) ) * APitchX + ( slot % ( BM / 4 ) ) * 4] ) = regA[i];
 				}
 			}
 		}
@@ -528,9 +539,9 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			const int slot = tid + i * Threads;
 			if( BTotal % Threads == 0 || slot < BTotal ) {
 				if( BK ) {
-					*reinterpret_cast<float4*>( &ldsB[buf][( slot / KQ ) * LdsK + ( slot % KQ ) * 4] ) = regB[i];
+					*reinterpret_cast<float4*>( &ldsB( buf )[( slot / KQ ) * LdsK + ( slot % KQ ) * 4] ) = regB[i];
 				} else {
-					*reinterpret_cast<float4*>( &ldsB[buf][( slot / ( BN / 4 ) ) * BPitchX + ( slot % ( BN / 4 ) ) * 4] ) = regB[i];
+					*reinterpret_cast<float4*>( &ldsB( buf )[( slot / ( BN / 4 ) ) * BPitchX + ( slot % ( BN / 4 ) ) * 4] ) = regB[i];
 				}
 			}
 		}
@@ -554,8 +565,8 @@ void matMulKernel( const CMatMulArgs launchArgs )
 		float B[NI][4];
 	};
 	auto readFrag = [&]( int buf, int kc, CFrag& f ) {
-		const float* tA = ldsA[buf];
-		const float* tB = ldsB[buf];
+		const float* tA = ldsA( buf );
+		const float* tB = ldsB( buf );
 #pragma unroll
 		for( int mi = 0; mi < MI; ++mi ) {
 			const int row = waveM * WM + mi * 32 + l32;
@@ -643,6 +654,37 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			__builtin_amdgcn_sched_barrier( 0 );
 		}
 		cur = nxt;
+	}
+
+	if constexpr( KGROUPS == 2 ) {
+		// every wave has passed the last barrier of its loop behind its last LDS read: the buffers are free
+		float* hand = &lds[1][0][0] + wave * ( MI * NI * 16 * 64 ) + lane;
+		if( kGroup == 1 ) {
+#pragma unroll
+			for( int mi = 0; mi < MI; ++mi ) {
+#pragma unroll
+				for( int ni = 0; ni < NI; ++ni ) {
+#pragma unroll
+					for( int r = 0; r < 16; ++r ) {
+						hand[( ( mi * NI + ni ) * 16 + r ) * 64] = acc[mi][ni][r];
+					}
+				}
+			}
+		}
+		__syncthreads();
+		if( kGroup == 1 ) {
+			return;
+		}
+#pragma unroll
+		for( int mi = 0; mi < MI; ++mi ) {
+#pragma unroll
+			for( int ni = 0; ni < NI; ++ni ) {
+#pragma unroll
+				for( int r = 0; r < 16; ++r ) {
+					acc[mi][ni][r] += hand[( ( mi * NI + ni ) * 16 + r ) * 64];
+				}
+			}
+		}
 	}
 
 #pragma unroll
@@ -760,6 +802,14 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 			}
 		}
 	}
+	// two slices of an even number of steps: the two halves share a workgroup of 8 wavefronts instead (KGROUPS = 2)
+	bool twoGroups = false;
+	if constexpr( BM == 64 && BN == 64 && BMODE == BM_RowsK && ( AMODE == AM_Conv || AMODE == AM_RowsK ) ) {
+		if( vec && splits == 2 && totalSteps % 2 == 0 && batch == 1 && args.ManySlices == 0 ) {
+			twoGroups = true;
+			splits = 1;
+		}
+	}
 	args.StepsPerSplit = ceilDiv( totalSteps, splits );
 	args.SplitK = ceilDiv( totalSteps, args.StepsPerSplit );
 	// Tail mode: more tiles than run at once, and the last round of them would leave most of the device idle. The tiles
@@ -770,7 +820,7 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 	const int slots = 256 * ( BM * BN <= 64 * 64 ? 5 : 4 );
 	long long gridX = tiles;
 	int tailRow = 0;
-	if( splits == 1 && batch == 1 && AMODE != AM_ConvClasses && args.Residual == nullptr && tiles >= slots && totalSteps >= 16 ) {
+	if( splits == 1 && !twoGroups && batch == 1 && AMODE != AM_ConvClasses && args.Residual == nullptr && tiles >= slots && totalSteps >= 16 ) {
 		long long full = tiles / slots * slots;
 		full -= full % args.TilesN; // whole rows of tiles: the preset below covers the rows behind them
 		const long long rest = tiles - full;
@@ -837,7 +887,11 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 		a.B += b0 * args.BatchStrideB;
 		a.C += b0 * args.BatchStrideC;
 		const dim3 grid( static_cast<unsigned>( gridX ), nb, args.SplitK );
-		if( vec ) {
+		if( twoGroups ) {
+			if constexpr( BM == 64 && BN == 64 && BMODE == BM_RowsK && ( AMODE == AM_Conv || AMODE == AM_RowsK ) ) {
+				hipLaunchKernelGGL( ( matMulKernel<BM, BN, WAVES_M, WAVES_N, AMODE, BMODE, true, 2> ), grid, dim3( Threads * 2 ), 0, stream, a );
+			}
+		} else if( vec ) {
 			hipLaunchKernelGGL( ( matMulKernel<BM, BN, WAVES_M, WAVES_N, AMODE, BMODE, true> ), grid, dim3( Threads ), 0, stream, a );
 		} else {
 			hipLaunchKernelGGL( ( matMulKernel<BM, BN, WAVES_M, WAVES_N, AMODE, BMODE, false> ), grid, dim3( Threads ), 0, stream, a );

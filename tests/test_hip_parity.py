@@ -227,6 +227,23 @@ def test_matmul_strided(shape):
         assert_close(hip().matmul("tn_add", at, bn, **kw), orc.matmul("tn_add", at, bn, **kw), "tn_add %s" % (shape,))
 
 
+def test_matmul_k_halves_in_one_workgroup():
+    # 448 tiles and 32 K steps: the two halves of K run in the two wave groups of one workgroup. Positive operands: over
+    # 1.8 M sums of 512 products the few that cancel to almost nothing would otherwise sit at the edge of the absolute bar
+    M, N, K = 1792, 1024, 512
+    g = rng(91)
+    a = g.uniform(0, 1, (M, K)).astype(np.float32)
+    b = g.uniform(0, 1, (N, K)).astype(np.float32)
+    kw = dict(lda=K, ldb=K, ldc=N, M=M, N=N, K=K)
+    got = hip().matmul("nt", a, b, **kw)
+    assert_close(got, orc.matmul("nt", a, b, **kw), "nt, K halves")
+    # every k must be counted once: a one-hot column of A picks one column of B
+    a[:] = 0
+    a[np.arange(M), np.arange(M) % K] = 1
+    got = hip().matmul("nt", a, b, **kw).reshape(M, N)
+    assert np.array_equal(got, b[:, np.arange(M) % K].T)
+
+
 @pytest.mark.parametrize("batch,M,N,K", [(1, 2, 3, 4), (3, 16, 8, 5), (4, 33, 17, 9), (8, 64, 64, 16), (6, 100, 64, 100),
                                          (5, 64, 256, 64), (2, 130, 36, 72)])
 def test_matmul_batched(batch, M, N, K):
@@ -276,6 +293,7 @@ GPU_CONV_CASES = CONV_CASES + [
     (2, 96, 96, 16, 96, 1, 1, 0, 0, 1, 1, 1, 1),
     (1, 131, 127, 32, 20, 1, 1, 0, 0, 1, 1, 1, 1),  # pixel count not a multiple of 32
     (1, 128, 130, 192, 40, 1, 1, 0, 0, 1, 1, 1, 1), # longest reduction it takes, N tail
+    (7, 64, 64, 64, 64, 3, 3, 1, 1, 1, 1, 1, 1),    # 448 tiles, 36 K steps: the two halves of K share a workgroup
 ]
 
 
@@ -297,6 +315,7 @@ def test_convolution(case):
     (3, 9, 9, 128, 200, 1, 1, 0, 0, 1, 1, 1, 1),     # 1x1 through the matrix-product path
     (2, 32, 32, 3, 64, 7, 7, 3, 3, 2, 2, 1, 1),      # stem
     (4, 64, 64, 24, 144, 1, 1, 0, 0, 1, 1, 1, 1),    # the row-resident pointwise kernel
+    (7, 64, 64, 64, 64, 3, 3, 1, 1, 1, 1, 1, 1),     # two K groups in a workgroup: activation in the epilogue again
 ])
 @pytest.mark.parametrize("activation,param", [("relu", 0.0), ("relu", 0.5), ("hswish", 0.0)])
 def test_convolution_with_activation(case, activation, param):
