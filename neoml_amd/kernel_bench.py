@@ -200,6 +200,8 @@ def main():
     pool("cfg2", 64, 114, 114, 64, 3, 3, 2, 2)
     pool("cfg5", 64, 32, 512, 64, 2, 2, 2, 2)
     pool("cfg2", 64, 114, 114, 64, 3, 3, 2, 2, mean=True)
+    pool("at the depthwise shape", 128, 112, 112, 96, 3, 3, 2, 2)
+    pool("at the depthwise shape", 128, 112, 112, 32, 3, 3, 1, 1)
 
     def pool_grad(n, h, w, c, f, s_):
         d = neoml_amd.PoolingDesc(n, h, w, c, f, f, s_, s_, 0, 0)
