@@ -940,28 +940,20 @@ __global__ __launch_bounds__( 256 ) void clearWordsKernel( unsigned long long* w
 	}
 }
 
-// ---------------------------------------------------------------------------------------------------------
-// Pooling, backward. Max: every output element sends its gradient to the input element its index names (index
-// inside the image, as the forward pass wrote it); overlapping windows may name the same element, so the sums meet
-// through atomic adds in a zeroed blob. Mean: every input element gathers the gradients of the windows that cover
-// it, times 1 / fh / fw.
+// Pooling gradients as gathers. Max: the gradient of an output element goes to the input element its stored index names
+// (always inside the window, as the forward pass wrote it). Mean: every window spreads its gradient, times 1 / fh / fw.
+// One kernel for both: every input element ( VECW channels of a pixel ) walks the windows that cover it, in the order
+// the reference's loop adds them. MAX: a window contributes where its stored index names this element.
+template<int VECW, bool MAX>
 __global__ __launch_bounds__( 256 )
-void maxPoolingBackwardKernel( const float* resultDiff, const int* maxIndices, float* sourceDiff, long long total,
-	int resultObjectSize, int sourceObjectSize )
-{
-	for( long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += static_cast<long long>( gridDim.x ) * 256 ) {
-		const long long object = i / resultObjectSize;
-		unsafeAtomicAdd( sourceDiff + object * sourceObjectSize + maxIndices[i], resultDiff[i] );
-	}
-}
-
-__global__ __launch_bounds__( 256 )
-void meanPoolingBackwardKernel( const nhPoolingDesc d, const float* resultDiff, float* sourceDiff, long long total )
+void poolingBackwardKernel( const nhPoolingDesc d, const float* resultDiff, const int* maxIndices, float* sourceDiff,
+	long long totalItems )
 {
 	const float scale = 1.f / d.filterHeight / d.filterWidth;
-	for( long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += static_cast<long long>( gridDim.x ) * 256 ) {
-		long long t = i;
-		const int c = static_cast<int>( t % d.channels ); t /= d.channels;
+	const int cg = d.channels / VECW;
+	for( long long item = blockIdx.x * 256LL + threadIdx.x; item < totalItems; item += static_cast<long long>( gridDim.x ) * 256 ) {
+		long long t = item;
+		const int c = static_cast<int>( t % cg ) * VECW; t /= cg;
 		const int wi = static_cast<int>( t % d.width ); t /= d.width;
 		const int hi = static_cast<int>( t % d.height );
 		const long long n = t / d.height;
@@ -970,13 +962,45 @@ void meanPoolingBackwardKernel( const nhPoolingDesc d, const float* resultDiff, 
 		const int hoLast = min( hi / d.strideHeight, d.resultHeight - 1 );
 		const int woFirst = wi >= d.filterWidth ? ( wi - d.filterWidth ) / d.strideWidth + 1 : 0;
 		const int woLast = min( wi / d.strideWidth, d.resultWidth - 1 );
-		float sum = 0.f;
+		const int own = ( hi * d.width + wi ) * d.channels + c; // index inside the object, as the forward pass stores it
+		float sum[VECW];
+#pragma unroll
+		for( int e = 0; e < VECW; ++e ) {
+			sum[e] = 0.f;
+		}
 		for( int ho = hoFirst; ho <= hoLast; ++ho ) {
 			for( int wo = woFirst; wo <= woLast; ++wo ) {
-				sum += resultDiff[( ( n * d.resultHeight + ho ) * d.resultWidth + wo ) * d.channels + c];
+				const long long at = ( ( n * d.resultHeight + ho ) * d.resultWidth + wo ) * d.channels + c;
+				float g[VECW];
+				int index[VECW];
+				if( VECW == 4 ) {
+					const float4 v = *reinterpret_cast<const float4*>( resultDiff + at );
+					g[0] = v.x; g[1] = v.y; g[2] = v.z; g[3] = v.w;
+					if( MAX ) {
+						const int4 k = *reinterpret_cast<const int4*>( maxIndices + at );
+						index[0] = k.x; index[1] = k.y; index[2] = k.z; index[3] = k.w;
+					}
+				} else {
+					g[0] = resultDiff[at];
+					if( MAX ) {
+						index[0] = maxIndices[at];
+					}
+				}
+#pragma unroll
+				for( int e = 0; e < VECW; ++e ) {
+					if( !MAX || index[e] == own + e ) {
+						sum[e] += g[e];
+					}
+				}
 			}
 		}
-		sourceDiff[i] = sum * scale;
+		float* out = sourceDiff + item * VECW;
+		if( VECW == 4 ) {
+			*reinterpret_cast<float4*>( out ) = MAX ? make_float4( sum[0], sum[1], sum[2], sum[3] )
+				: make_float4( sum[0] * scale, sum[1] * scale, sum[2] * scale, sum[3] * scale );
+		} else {
+			out[0] = MAX ? sum[0] : sum[0] * scale;
+		}
 	}
 }
 
@@ -1420,6 +1444,30 @@ static int channelwise3x3Impl( nhStream s, const nhConvDesc* d, const float* sou
 	return NH_OK;
 }
 
+template<bool MAX>
+static int poolingBackwardImpl( nhStream s, const nhPoolingDesc* d, const float* resultDiff, const int* maxIndices,
+	float* sourceDiff )
+{
+	const long long total = static_cast<long long>( d->batch ) * d->height * d->width * d->channels;
+	if( total == 0 ) {
+		return NH_OK;
+	}
+	const bool vec = d->channels % 4 == 0 && isAligned16( resultDiff ) && isAligned16( sourceDiff )
+		&& ( !MAX || isAligned16( maxIndices ) );
+	const long long items = vec ? total / 4 : total;
+	long long blocks = ( items + 255 ) / 256;
+	blocks = blocks > 1048576 ? 1048576 : blocks;
+	if( vec ) {
+		hipLaunchKernelGGL( ( poolingBackwardKernel<4, MAX> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			*d, resultDiff, maxIndices, sourceDiff, items );
+	} else {
+		hipLaunchKernelGGL( ( poolingBackwardKernel<1, MAX> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			*d, resultDiff, maxIndices, sourceDiff, items );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
 extern "C" {
 
 
@@ -1530,23 +1578,7 @@ int nhBlobMaxPoolingBackward( nhStream s, const nhPoolingDesc* d, const float* r
 		return rc;
 	}
 	NH_REQUIRE( resultDiff != nullptr && maxIndices != nullptr && sourceDiff != nullptr );
-	const int sourceObjectSize = d->height * d->width * d->channels;
-	const int resultObjectSize = d->resultHeight * d->resultWidth * d->channels;
-	const long long sourceTotal = static_cast<long long>( d->batch ) * sourceObjectSize;
-	const long long total = static_cast<long long>( d->batch ) * resultObjectSize;
-	if( sourceTotal == 0 ) {
-		return NH_OK;
-	}
-	NH_HIP( hipMemsetAsync( sourceDiff, 0, sourceTotal * sizeof( float ), toStream( s ) ) );
-	if( total == 0 ) {
-		return NH_OK;
-	}
-	long long blocks = ( total + 255 ) / 256;
-	blocks = blocks > 1048576 ? 1048576 : blocks;
-	hipLaunchKernelGGL( maxPoolingBackwardKernel, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
-		resultDiff, maxIndices, sourceDiff, total, resultObjectSize, sourceObjectSize );
-	NH_LAUNCH_CHECK();
-	return NH_OK;
+	return poolingBackwardImpl<true>( s, d, resultDiff, maxIndices, sourceDiff );
 }
 
 int nhBlobMeanPoolingBackward( nhStream s, const nhPoolingDesc* d, const float* resultDiff, float* sourceDiff )
@@ -1556,16 +1588,7 @@ int nhBlobMeanPoolingBackward( nhStream s, const nhPoolingDesc* d, const float* 
 		return rc;
 	}
 	NH_REQUIRE( resultDiff != nullptr && sourceDiff != nullptr );
-	const long long total = static_cast<long long>( d->batch ) * d->height * d->width * d->channels;
-	if( total == 0 ) {
-		return NH_OK;
-	}
-	long long blocks = ( total + 255 ) / 256;
-	blocks = blocks > 1048576 ? 1048576 : blocks;
-	hipLaunchKernelGGL( meanPoolingBackwardKernel, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
-		*d, resultDiff, sourceDiff, total );
-	NH_LAUNCH_CHECK();
-	return NH_OK;
+	return poolingBackwardImpl<false>( s, d, resultDiff, nullptr, sourceDiff );
 }
 
 static int checkedChannelwiseDesc( const nhConvDesc* d )
