@@ -354,14 +354,55 @@ struct CTanhDiffOutOp : CNoScalar { __device__ float operator()( float y, float 
 
 // ---- reductions to one value: one workgroup per 16K elements, atomics into a zeroed result -----------------
 
-template<bool DOT>
+// VEC: 128-bit loads, four of them in flight per thread and operand (both pointers 16-byte aligned); the up to three
+// elements behind the last whole vector are added by the first thread.
+template<bool DOT, bool VEC>
 __global__ __launch_bounds__( 256 ) void sumKernel( const float* a, const float* b, int n, float* result )
 {
 	__shared__ float part[4];
 	float s = 0.f;
 	const int stride = gridDim.x * 256;
-	for( int i = blockIdx.x * 256 + threadIdx.x; i < n; i += stride ) {
-		s += DOT ? a[i] * b[i] : a[i];
+	const int start = blockIdx.x * 256 + threadIdx.x;
+	if( VEC ) {
+		const int n4 = n >> 2;
+		const float4* a4 = reinterpret_cast<const float4*>( a );
+		const float4* b4 = reinterpret_cast<const float4*>( b );
+		float acc[4] = { 0.f, 0.f, 0.f, 0.f };
+		int i = start;
+		for( ; i + 3 * stride < n4; i += 4 * stride ) {
+			float4 va[4], vb[4];
+#pragma unroll
+			for( int j = 0; j < 4; ++j ) {
+				va[j] = a4[i + j * stride];
+				if( DOT ) {
+					vb[j] = b4[i + j * stride];
+				}
+			}
+#pragma unroll
+			for( int j = 0; j < 4; ++j ) {
+				acc[j] += DOT ? ( va[j].x * vb[j].x + va[j].y * vb[j].y ) + ( va[j].z * vb[j].z + va[j].w * vb[j].w )
+					: ( va[j].x + va[j].y ) + ( va[j].z + va[j].w );
+			}
+		}
+		for( ; i < n4; i += stride ) {
+			const float4 va = a4[i];
+			if( DOT ) {
+				const float4 vb = b4[i];
+				acc[0] += ( va.x * vb.x + va.y * vb.y ) + ( va.z * vb.z + va.w * vb.w );
+			} else {
+				acc[0] += ( va.x + va.y ) + ( va.z + va.w );
+			}
+		}
+		s = ( acc[0] + acc[1] ) + ( acc[2] + acc[3] );
+		if( start == 0 ) {
+			for( int k = n4 << 2; k < n; ++k ) {
+				s += DOT ? a[k] * b[k] : a[k];
+			}
+		}
+	} else {
+		for( int i = start; i < n; i += stride ) {
+			s += DOT ? a[i] * b[i] : a[i];
+		}
 	}
 	s = waveReduceSum( s );
 	if( ( threadIdx.x & 63 ) == 0 ) {
@@ -371,6 +412,25 @@ __global__ __launch_bounds__( 256 ) void sumKernel( const float* a, const float*
 	if( threadIdx.x == 0 ) {
 		atomicAdd( result, part[0] + part[1] + part[2] + part[3] );
 	}
+}
+
+template<bool DOT>
+static int launchSum( nhStream s, const float* first, const float* second, int vectorSize, float* result )
+{
+	int rc = nhVectorFill( s, result, 0.f, 1 );
+	if( rc != NH_OK || vectorSize == 0 ) {
+		return rc;
+	}
+	NH_REQUIRE( first != nullptr && ( !DOT || second != nullptr ) );
+	int blocks = ceilDiv( vectorSize, 16384 );
+	blocks = blocks > 2048 ? 2048 : blocks;
+	if( isAligned16( first ) && ( !DOT || isAligned16( second ) ) ) {
+		hipLaunchKernelGGL( ( sumKernel<DOT, true> ), dim3( blocks ), dim3( 256 ), 0, toStream( s ), first, second, vectorSize, result );
+	} else {
+		hipLaunchKernelGGL( ( sumKernel<DOT, false> ), dim3( blocks ), dim3( 256 ), 0, toStream( s ), first, second, vectorSize, result );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
 }
 
 } // namespace nh
@@ -581,26 +641,10 @@ extern "C" int nhVectorMultiplyAndSub( nhStream s, const float* first, const flo
 extern "C" int nhVectorSum( nhStream s, const float* first, int vectorSize, float* result )
 {
 	NH_REQUIRE( vectorSize >= 0 && result != nullptr );
-	int rc = nhVectorFill( s, result, 0.f, 1 );
-	if( rc != NH_OK || vectorSize == 0 ) {
-		return rc;
-	}
-	int blocks = ceilDiv( vectorSize, 16384 );
-	blocks = blocks > 2048 ? 2048 : blocks;
-	hipLaunchKernelGGL( sumKernel<false>, dim3( blocks ), dim3( 256 ), 0, toStream( s ), first, (const float*)nullptr, vectorSize, result );
-	NH_LAUNCH_CHECK();
-	return NH_OK;
+	return launchSum<false>( s, first, nullptr, vectorSize, result );
 }
 extern "C" int nhVectorDotProduct( nhStream s, const float* first, const float* second, int vectorSize, float* result )
 {
 	NH_REQUIRE( vectorSize >= 0 && result != nullptr );
-	int rc = nhVectorFill( s, result, 0.f, 1 );
-	if( rc != NH_OK || vectorSize == 0 ) {
-		return rc;
-	}
-	int blocks = ceilDiv( vectorSize, 16384 );
-	blocks = blocks > 2048 ? 2048 : blocks;
-	hipLaunchKernelGGL( sumKernel<true>, dim3( blocks ), dim3( 256 ), 0, toStream( s ), first, second, vectorSize, result );
-	NH_LAUNCH_CHECK();
-	return NH_OK;
+	return launchSum<true>( s, first, second, vectorSize, result );
 }

@@ -110,11 +110,16 @@ def test_int_ops_fill_convert():
 
 def test_sum_and_dot():
     g = rng(4)
-    for n in (1, 1000, 1 << 20):
+    for n in (1, 2, 3, 5, 1000, 1003, 4099, 1 << 20, (1 << 22) + 7):
         a = g.uniform(-1, 1, n).astype(np.float32)
         b = g.uniform(-1, 1, n).astype(np.float32)
-        assert_close(hip().vector_sum(a), orc.vector_sum(a), "sum", atol=1e-2 if n > 1000 else 1e-4)
-        assert_close(hip().dot(a, b), orc.dot(a, b), "dot", atol=1e-2 if n > 1000 else 1e-4)
+        assert_close(hip().vector_sum(a), orc.vector_sum(a), "sum n=%d" % n, atol=1e-2 if n > 1000 else 1e-4)
+        assert_close(hip().dot(a, b), orc.dot(a, b), "dot n=%d" % n, atol=1e-2 if n > 1000 else 1e-4)
+    # every element counted exactly once, whatever the vector / tail split: sums of small integers are exact in fp32
+    for n in (7, 1026, 70001):
+        a = g.integers(0, 4, n).astype(np.float32)
+        assert hip().vector_sum(a) == a.sum(dtype=np.float64)
+        assert hip().dot(a, np.ones_like(a)) == a.sum(dtype=np.float64)
 
 
 def test_broadcasts_and_sums():
