@@ -782,7 +782,8 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 	// meet in C through fp32 atomic adds (C is pre-set to the free term). 1280 workgroups (5 per compute unit) run
 	// at once; the slice count is the one that wastes least of the last round of 1280, each extra slice priced at 2 %
 	// for its atomics, and every slice keeps at least 8 K steps.
-	const int totalSteps = ceilDiv( args.K, NH_KSTEP );
+	// an empty reduction ( K == 0 ) still launches: one step of masked loads, C receives the free term or keeps its value
+	const int totalSteps = args.K > 0 ? ceilDiv( args.K, NH_KSTEP ) : 1;
 	int splits = 1;
 	const long long blocks = tiles * batch;
 	if( args.ManySlices != 0 ) {

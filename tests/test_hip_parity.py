@@ -677,6 +677,40 @@ def test_lstm_bounded_wait_gives_up(monkeypatch):
 # ---------------------------------------------------------------------------------------------------------
 # error convention and allocator on the device
 
+def test_empty_inputs_are_accepted():
+    """Zero-sized operands (an empty batch, a vector of no elements, a product over no terms) return NH_OK and leave
+    memory they do not own alone; a product over K = 0 terms is the free term / zero."""
+    import neoml_amd
+    h = hip()
+    lib, P = h.lib, h.p
+    guard = h.up(np.full(64, 7.0, np.float32))
+    zero = h.scalar(0.0)
+    ok = lambda rc: neoml_amd.check(rc)
+    ok(lib.nhVectorAdd(h.stream(), P(guard), P(guard), P(guard), 0))
+    ok(lib.nhVectorReLU(h.stream(), P(guard), P(guard), 0, P(zero)))
+    ok(lib.nhVectorCopy(h.stream(), P(guard), P(guard), 0))
+    total = h.up(np.full(1, 5.0, np.float32))
+    ok(lib.nhVectorSum(h.stream(), P(guard), 0, P(total)))
+    assert h.down(total)[0] == 0.0
+    ok(lib.nhMatrixSoftmaxByRows(h.stream(), P(guard), 0, 16, P(guard)))
+    ok(lib.nhSumMatrixRows(h.stream(), 0, P(guard), P(guard), 4, 4))
+    ok(lib.nhMultiplyMatrixByTransposedMatrix(h.stream(), P(guard), 0, 8, 8, P(guard), 4, 8, P(guard), 4, 0))
+    d = neoml_amd.ConvDesc(0, 8, 8, 4, 4, 3, 3, 1, 1, 1, 1, 1, 1, 0, 0)
+    ok(lib.nhInitBlobConvolution(ctypes.byref(d)))
+    ok(lib.nhBlobConvolution(h.stream(), ctypes.byref(d), P(guard), P(guard), None, P(guard)))
+    p = neoml_amd.PoolingDesc(0, 8, 8, 4, 2, 2, 2, 2, 0, 0)
+    ok(lib.nhInitPooling(ctypes.byref(p)))
+    ok(lib.nhBlobMaxPooling(h.stream(), ctypes.byref(p), P(guard), None, P(guard)))
+    ok(lib.nhBlobMeanPoolingBackward(h.stream(), ctypes.byref(p), P(guard), P(guard)))
+    assert np.array_equal(h.down(guard), np.full(64, 7.0, np.float32))
+    # K = 0: [4 x 0] * [0 x 5] is a matrix of zeros
+    a = np.zeros((4, 0), np.float32)
+    b = np.zeros((5, 0), np.float32)
+    out = h.up(np.full(20, 3.0, np.float32))
+    ok(lib.nhMultiplyMatrixByTransposedMatrix(h.stream(), P(guard), 4, 0, 0, P(guard), 5, 0, P(out), 5, 20))
+    assert np.array_equal(h.down(out), np.zeros(20, np.float32))
+
+
 def test_argument_errors_are_reported_not_thrown():
     import neoml_amd
     lib = neoml_amd.load()
