@@ -23,7 +23,7 @@ HBM_PEAK_GBPS = 8000.0
 # batch 64, 224x224: rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a known-size copy gives) 53.2 MB + WRITE_SIZE (x1.0)
 # 33.7 MB; profiles/resnet18_b64_conv_hbm_traffic.txt holds the two runs. Counters cannot be read from inside this
 # process, so the figure is a constant of the default workload and null for any other.
-CONV3X3_TRAFFIC_BYTES_B64_224 = 86.9e6
+CONV3X3_TRAFFIC_BYTES_B64_224 = 91.5e6
 
 
 def cpu_baseline(batch_sample, image):
