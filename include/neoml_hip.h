@@ -165,6 +165,16 @@ NH_API int nhVectorHardSigmoidDiff(nhStream s, const float* first, const float* 
 NH_API int nhVectorHardSigmoidDiffOp(nhStream s, const float* first, const float* second, float* result, int vectorSize,
 	const float* slope_dev);                                                                         /* NME.h:208 */
 NH_API int nhVectorAbsDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize); /* NME.h:178 */
+/* element-wise parts of the hinge / squared hinge / Huber losses and their derivatives (times second), and of the L1
+ * regulariser: result = first + mult * clamp( second, -threshold, threshold ), both scalars in device memory */
+NH_API int nhVectorHinge(nhStream s, const float* first, float* result, int vectorSize);             /* NME.h:184 */
+NH_API int nhVectorHingeDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize); /* NME.h:185 */
+NH_API int nhVectorSquaredHinge(nhStream s, const float* first, float* result, int vectorSize);      /* NME.h:188 */
+NH_API int nhVectorSquaredHingeDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize); /* NME.h:189 */
+NH_API int nhVectorHuber(nhStream s, const float* first, float* result, int vectorSize);             /* NME.h:193 */
+NH_API int nhVectorHuberDerivative(nhStream s, const float* first, float* result, int vectorSize);   /* NME.h:194 */
+NH_API int nhVectorL1DiffAdd(nhStream s, const float* first, const float* second, float* result, int vectorSize,
+	const float* threshold_dev, const float* mult_dev);                                              /* NME.h:335 */
 /* first - value, or value - first when reverse != 0: the two scalar overloads of VectorSub */
 NH_API int nhVectorSubValue(nhStream s, const float* first, float value, int reverse, float* result, int vectorSize); /* NME.h:251,253 */
 NH_API int nhVectorHSwishDiff(nhStream s, const float* first, const float* second, float* result, int vectorSize);   /* NME.h:164 */

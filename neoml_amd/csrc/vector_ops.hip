@@ -330,6 +330,41 @@ struct CSubValueOp {
 	__device__ void prepare() {}
 	__device__ float operator()( float a, float, float ) const { return Reverse ? Value - a : a - Value; }
 };
+// The element-wise parts of the hinge, squared hinge and Huber losses and of the L1 regulariser
+// (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:584-782, 924-975, 1598-1640)
+struct CHingeOp : CNoScalar { __device__ float operator()( float a, float, float ) const { return fmaxf( 0.f, 1.f - a ); } };
+struct CSquaredHingeOp : CNoScalar {
+	__device__ float operator()( float a, float, float ) const
+	{
+		if( a < -1.f ) return -4.f * a;
+		const float t = fmaxf( 0.f, 1.f - a );
+		return t * t;
+	}
+};
+struct CHuberOp : CNoScalar {
+	__device__ float operator()( float a, float, float ) const { return a > 1.f ? a - 0.5f : ( a < -1.f ? -a - 0.5f : a * a / 2 ); }
+};
+struct CHuberDerivativeOp : CNoScalar {
+	__device__ float operator()( float a, float, float ) const { return a > 1.f ? 1.f : ( a < -1.f ? -1.f : a ); }
+};
+struct CHingeDiffOp : CNoScalar { __device__ float operator()( float a, float b, float ) const { return a < 1.f ? -b : 0.f; } };
+struct CSquaredHingeDiffOp : CNoScalar {
+	__device__ float operator()( float a, float b, float ) const
+	{
+		if( a < -1.f ) return -4.f * b;
+		return -2.f * fmaxf( 0.f, 1.f - a ) * b;
+	}
+};
+struct CL1DiffAddOp {
+	// first + mult * clamp( second, -threshold, threshold )
+	const float* ThresholdPtr; const float* MultPtr; float Threshold, Mult;
+	__device__ void prepare() { Threshold = *ThresholdPtr; Mult = *MultPtr; }
+	__device__ float operator()( float a, float b, float ) const
+	{
+		const float x = b < -Threshold ? -Threshold : ( b > Threshold ? Threshold : b );
+		return a + Mult * x;
+	}
+};
 struct CHSwishDiffOp : CNoScalar {
 	// 0 below -3, second above 3, second * ( first / 3 + 1/2 ) between (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:433-480)
 	__device__ float operator()( float a, float b, float ) const
@@ -575,6 +610,20 @@ extern "C" int nhVectorSubValue( nhStream s, const float* first, float value, in
 {
 	CSubValueOp op; op.Value = value; op.Reverse = reverse;
 	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+
+NH_UNARY( nhVectorHinge, CHingeOp )
+NH_UNARY( nhVectorSquaredHinge, CSquaredHingeOp )
+NH_UNARY( nhVectorHuber, CHuberOp )
+NH_UNARY( nhVectorHuberDerivative, CHuberDerivativeOp )
+NH_BINARY( nhVectorHingeDiff, float, CHingeDiffOp )
+NH_BINARY( nhVectorSquaredHingeDiff, float, CSquaredHingeDiffOp )
+extern "C" int nhVectorL1DiffAdd( nhStream s, const float* first, const float* second, float* result, int vectorSize,
+	const float* threshold, const float* mult )
+{
+	NH_REQUIRE( threshold != nullptr && mult != nullptr );
+	CL1DiffAddOp op; op.ThresholdPtr = threshold; op.MultPtr = mult; op.Threshold = op.Mult = 0;
+	return launchEltwise<2, float, float>( s, first, second, (const float*)nullptr, result, vectorSize, op );
 }
 
 NH_BINARY( nhVectorEltwiseMax, float, CMaxOp )

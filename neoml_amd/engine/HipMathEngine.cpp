@@ -233,6 +233,11 @@ HIP_UNARY( VectorTanh, nhVectorTanh )
 
 HIP_UNARY( VectorNegLog, nhVectorNegLog )
 
+HIP_UNARY( VectorHinge, nhVectorHinge )
+HIP_UNARY( VectorSquaredHinge, nhVectorSquaredHinge )
+HIP_UNARY( VectorHuber, nhVectorHuber )
+HIP_UNARY( VectorHuberDerivative, nhVectorHuberDerivative )
+
 HIP_UNARY_SCALAR( VectorELU, nhVectorELU )
 HIP_UNARY_SCALAR( VectorReLU, nhVectorReLU )
 HIP_UNARY_SCALAR( VectorLeakyReLU, nhVectorLeakyReLU )
@@ -272,6 +277,17 @@ void CHipMathEngine::VectorReLUDiffOp( const CConstFloatHandle& firstHandle, con
 	const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& upperThresholdHandle )
 {
 	VectorReLUDiff( firstHandle, secondHandle, resultHandle, vectorSize, upperThresholdHandle );
+}
+
+HIP_BINARY( VectorHingeDiff, CFloatHandle, CConstFloatHandle, nhVectorHingeDiff )
+HIP_BINARY( VectorSquaredHingeDiff, CFloatHandle, CConstFloatHandle, nhVectorSquaredHingeDiff )
+
+void CHipMathEngine::VectorL1DiffAdd( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle,
+	const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& hubertThresholdHandle,
+	const CConstFloatHandle& multHandle )
+{
+	NH_CALL( nhVectorL1DiffAdd( stream, raw( firstHandle ), raw( secondHandle ), raw( resultHandle ), vectorSize,
+		raw( hubertThresholdHandle ), raw( multHandle ) ) );
 }
 
 HIP_BINARY( VectorAbsDiff, CFloatHandle, CConstFloatHandle, nhVectorAbsDiff )

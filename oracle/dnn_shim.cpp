@@ -431,7 +431,8 @@ EXPORT int dnn_run( void* engine, int kind, int seed, int param, const int* dims
 // kind 2: Conv 3x3 p1 (16) - HSwish - [Conv 3x3 p1 (16) - ReLU - Conv 3x3 p1 (16)] + shortcut - ReLU - MeanPool 2x2/2 -
 // FullyConnected (classes); kind 3: Lstm (24 units, over BatchLength) - FullyConnected (classes) at every step.
 // kind 4: the ResNet-18-style network of dnn_run's kind 5; kind 5: the depthwise-separable network of its kind 6;
-// kind 6: the transformer encoder of its kind 1 with a classifier over every position (input [1, B, seq, 1, 1, 1, hidden]).
+// kind 6: the transformer encoder of its kind 1 with a classifier over every position (input [1, B, seq, 1, 1, 1, hidden]);
+// kind 7: the same with dropout; kind 8: a small CNN with CBatchNormalizationLayer behind each convolution.
 // solver 0: CDnnSimpleGradientSolver, 1: CDnnAdaptiveGradientSolver (Adam), both with L2 regularisation 1e-3.
 // losses receives the loss of every step, output the logits of a final forward pass with the trained weights.
 // timedSteps > 0: that many further steps are timed (the loss is read after the last one, which waits for the device)
@@ -453,7 +454,22 @@ EXPORT int dnn_train( void* engine, int kind, int solverKind, int seed, int clas
 
 		CBaseLayer* last = source.Ptr();
 		CBaseLayer* logits = nullptr;
-		if( kind == 6 || kind == 7 ) {
+		if( kind == 8 ) {
+			// Conv 3x3 (8) - BatchNormalization (per channel) - ReLU - Conv 3x3 /2 (16) - BatchNormalization - ReLU - GlobalMeanPooling
+			CPtr<CConvLayer> c1 = conv( dnn, e, "conv1", *last, 8, 3, 1, 1 );
+			// (the normalization mode can only be set before the layer joins the network)
+			CBatchNormalizationLayer* newBn1 = new CBatchNormalizationLayer( e );
+			newBn1->SetChannelBased( true );
+			CPtr<CBatchNormalizationLayer> bn1 = add( dnn, newBn1, "bn1", *c1 );
+			CPtr<CReLULayer> r1 = add( dnn, new CReLULayer( e ), "relu1", *bn1 );
+			CPtr<CConvLayer> c2 = conv( dnn, e, "conv2", *r1, 16, 3, 1, 2 );
+			CBatchNormalizationLayer* newBn2 = new CBatchNormalizationLayer( e );
+			newBn2->SetChannelBased( true );
+			CPtr<CBatchNormalizationLayer> bn2 = add( dnn, newBn2, "bn2", *c2 );
+			CPtr<CReLULayer> r2 = add( dnn, new CReLULayer( e ), "relu2", *bn2 );
+			CPtr<CGlobalMeanPoolingLayer> gap = add( dnn, new CGlobalMeanPoolingLayer( e ), "gap", *r2 );
+			last = gap.Ptr();
+		} else if( kind == 6 || kind == 7 ) {
 			// two CTransformerEncoderLayers (hidden = the input's channel count), a classifier over every position;
 			// kind 7: with dropout 0.1 inside the layers (the masks come from the network's CRandom seeds)
 			last = buildTransformer( dnn, e, *source, dims[6], kind == 7 ? 0.1f : 0.f );

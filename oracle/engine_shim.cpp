@@ -104,7 +104,8 @@ SHIM_API int shim_engine_type( void* engine ) { return static_cast<IMathEngine*>
 enum {
 	OP_RELU = 0, OP_ELU, OP_LEAKY_RELU, OP_HSWISH, OP_ABS, OP_HARD_TANH, OP_HARD_SIGMOID, OP_NEG,
 	OP_EXP, OP_LOG, OP_ERF, OP_SQRT, OP_INV, OP_MINMAX, OP_SIGMOID, OP_TANH,
-	OP_ADD_VALUE, OP_MULTIPLY, OP_NEG_MULTIPLY, OP_COPY, OP_NEG_LOG, OP_SUB_VALUE, OP_VALUE_SUB
+	OP_ADD_VALUE, OP_MULTIPLY, OP_NEG_MULTIPLY, OP_COPY, OP_NEG_LOG, OP_SUB_VALUE, OP_VALUE_SUB,
+	OP_HINGE, OP_SQUARED_HINGE, OP_HUBER, OP_HUBER_DERIVATIVE
 };
 
 SHIM_API int shim_vector_unary( void* engine, int op, const float* first, float* result, int n, float p0, float p1 )
@@ -134,6 +135,10 @@ SHIM_API int shim_vector_unary( void* engine, int op, const float* first, float*
 			case OP_NEG_MULTIPLY: e.VectorNegMultiply( in.Const(), out.Handle(), n, s0.Const() ); break;
 			case OP_COPY: e.VectorCopy( out.Handle(), in.Const(), n ); break;
 			case OP_NEG_LOG: e.VectorNegLog( in.Const(), out.Handle(), n ); break;
+			case OP_HINGE: e.VectorHinge( in.Const(), out.Handle(), n ); break;
+			case OP_SQUARED_HINGE: e.VectorSquaredHinge( in.Const(), out.Handle(), n ); break;
+			case OP_HUBER: e.VectorHuber( in.Const(), out.Handle(), n ); break;
+			case OP_HUBER_DERIVATIVE: e.VectorHuberDerivative( in.Const(), out.Handle(), n ); break;
 			case OP_SUB_VALUE: e.VectorSub( in.Const(), p0, out.Handle(), n ); break;
 			case OP_VALUE_SUB: e.VectorSub( p0, in.Const(), out.Handle(), n ); break;
 			default: throw std::logic_error( "bad unary op" );
@@ -147,7 +152,7 @@ enum {
 	OP_ELTWISE_MIN, OP_MULTIPLY_AND_ADD, OP_MULTIPLY_AND_SUB, OP_ELTWISE_MULTIPLY_ADD,
 	OP_RELU_DIFF, OP_HSWISH_DIFF, OP_SIGMOID_DIFF, OP_SIGMOID_DIFF_OP, OP_TANH_DIFF, OP_TANH_DIFF_OP,
 	OP_ELU_DIFF, OP_ELU_DIFF_OP, OP_LEAKY_RELU_DIFF, OP_HARD_TANH_DIFF, OP_HARD_SIGMOID_DIFF, OP_HARD_SIGMOID_DIFF_OP,
-	OP_ABS_DIFF
+	OP_ABS_DIFF, OP_HINGE_DIFF, OP_SQUARED_HINGE_DIFF, OP_L1_DIFF_ADD
 };
 
 SHIM_API int shim_vector_binary( void* engine, int op, const float* first, const float* second, float* result, int n, float p0,
@@ -181,6 +186,9 @@ SHIM_API int shim_vector_binary( void* engine, int op, const float* first, const
 			case OP_HARD_SIGMOID_DIFF: e.VectorHardSigmoidDiff( a.Const(), b.Const(), out.Handle(), n, s0.Const(), s1.Const() ); break;
 			case OP_HARD_SIGMOID_DIFF_OP: e.VectorHardSigmoidDiffOp( a.Const(), b.Const(), out.Handle(), n, s0.Const(), s1.Const() ); break;
 			case OP_ABS_DIFF: e.VectorAbsDiff( a.Const(), b.Const(), out.Handle(), n ); break;
+			case OP_HINGE_DIFF: e.VectorHingeDiff( a.Const(), b.Const(), out.Handle(), n ); break;
+			case OP_SQUARED_HINGE_DIFF: e.VectorSquaredHingeDiff( a.Const(), b.Const(), out.Handle(), n ); break;
+			case OP_L1_DIFF_ADD: e.VectorL1DiffAdd( a.Const(), b.Const(), out.Handle(), n, s0.Const(), s1.Const() ); break;
 			default: throw std::logic_error( "bad binary op" );
 		}
 		out.CopyTo( result );

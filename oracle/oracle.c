@@ -58,7 +58,9 @@ enum {
 	ORC_RELU = 0, ORC_ELU, ORC_LEAKY_RELU, ORC_HSWISH, ORC_ABS, ORC_HARD_TANH, ORC_HARD_SIGMOID, ORC_NEG,
 	ORC_EXP, ORC_LOG, ORC_ERF, ORC_SQRT, ORC_INV, ORC_MINMAX, ORC_SIGMOID, ORC_TANH,
 	ORC_ADD_VALUE, ORC_MULTIPLY, ORC_NEG_MULTIPLY, ORC_COPY, ORC_NEG_LOG,
-	ORC_SUB_VALUE, ORC_VALUE_SUB /* x - p0 and p0 - x: the scalar forms of VectorSub */
+	ORC_SUB_VALUE, ORC_VALUE_SUB, /* x - p0 and p0 - x: the scalar forms of VectorSub */
+	/* element-wise parts of the losses (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:584-782) */
+	ORC_HINGE, ORC_SQUARED_HINGE, ORC_HUBER, ORC_HUBER_DERIVATIVE
 };
 
 /* result[i] = f(first[i]; p0, p1) */
@@ -95,6 +97,10 @@ ORC_API void orc_vector_unary(int op, const float* first, float* result, int n, 
 		case ORC_NEG_MULTIPLY: y = -x * p0; break;
 		case ORC_COPY: y = x; break;
 		/* VectorLog with the sign flipped (src/CPU/x86/CpuX86MathEngineVectorMath.cpp:1692-1720) */
+		case ORC_HINGE: y = 1.f - x > 0.f ? 1.f - x : 0.f; break;
+		case ORC_SQUARED_HINGE: { const float t = 1.f - x > 0.f ? 1.f - x : 0.f; y = x < -1.f ? -4.f * x : t * t; } break;
+		case ORC_HUBER: y = x > 1.f ? x - 0.5f : (x < -1.f ? -x - 0.5f : x * x / 2); break;
+		case ORC_HUBER_DERIVATIVE: y = x > 1.f ? 1.f : (x < -1.f ? -1.f : x); break;
 		case ORC_SUB_VALUE: y = x - p0; break;
 		case ORC_VALUE_SUB: y = p0 - x; break;
 		case ORC_NEG_LOG: { float c = x > FLT_MIN ? x : FLT_MIN; c = c < FLT_MAX ? c : FLT_MAX; y = -logf(c); } break;
@@ -113,7 +119,9 @@ enum {
 	/* (:232-318 ELU, p0 = alpha; :394-432 leaky ReLU, p0 = alpha; :783-812 hard tanh; :825-920 hard sigmoid, p0 = slope,
 	 * p1 = bias; :550-580 abs) */
 	ORC_ELU_DIFF, ORC_ELU_DIFF_OP, ORC_LEAKY_RELU_DIFF, ORC_HARD_TANH_DIFF, ORC_HARD_SIGMOID_DIFF, ORC_HARD_SIGMOID_DIFF_OP,
-	ORC_ABS_DIFF
+	ORC_ABS_DIFF,
+	/* (:614-649 hinge, :924-975 squared hinge; :1598-1640 L1 regulariser, p0 = threshold, p1 = multiplier) */
+	ORC_HINGE_DIFF, ORC_SQUARED_HINGE_DIFF, ORC_L1_DIFF_ADD
 };
 
 /* result[i] = f(first[i], second[i]; p0, p1); ORC_ELTWISE_MULTIPLY_ADD reads result[i] as the addend */
@@ -146,6 +154,9 @@ ORC_API void orc_vector_binary(int op, const float* first, const float* second, 
 		case ORC_HARD_SIGMOID_DIFF: y = (-p1 / p0 < a && a < (1.f - p1) / p0) ? b * p0 : 0.f; break;
 		case ORC_HARD_SIGMOID_DIFF_OP: y = (0.f < a && a < 1.f) ? b * p0 : 0.f; break;
 		case ORC_ABS_DIFF: y = a > 0.f ? b : -b; break;
+		case ORC_HINGE_DIFF: y = a < 1.f ? -b : 0.f; break;
+		case ORC_SQUARED_HINGE_DIFF: { const float t = 1.f - a > 0.f ? 1.f - a : 0.f; y = a < -1.f ? -4.f * b : -2.f * t * b; } break;
+		case ORC_L1_DIFF_ADD: { const float x = b < -p0 ? -p0 : (b > p0 ? p0 : b); y = a + p1 * x; } break;
 		default: y = NAN; break;
 		}
 		result[i] = y;

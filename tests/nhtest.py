@@ -19,12 +19,12 @@ ATOL = 1e-5
 
 UNARY = {name: i for i, name in enumerate([
     "relu", "elu", "leaky_relu", "hswish", "abs", "hard_tanh", "hard_sigmoid", "neg", "exp", "log", "erf", "sqrt",
-    "inv", "minmax", "sigmoid", "tanh", "add_value", "multiply", "neg_multiply", "copy", "neg_log", "sub_value", "value_sub"])}
+    "inv", "minmax", "sigmoid", "tanh", "add_value", "multiply", "neg_multiply", "copy", "neg_log", "sub_value", "value_sub", "hinge", "squared_hinge", "huber", "huber_derivative"])}
 BINARY = {name: i for i, name in enumerate([
     "add", "sub", "eltwise_multiply", "eltwise_neg_multiply", "eltwise_divide", "eltwise_max", "eltwise_min",
     "multiply_and_add", "multiply_and_sub", "eltwise_multiply_add", "relu_diff", "hswish_diff", "sigmoid_diff",
     "sigmoid_diff_op", "tanh_diff", "tanh_diff_op", "elu_diff", "elu_diff_op", "leaky_relu_diff", "hard_tanh_diff",
-    "hard_sigmoid_diff", "hard_sigmoid_diff_op", "abs_diff"])}
+    "hard_sigmoid_diff", "hard_sigmoid_diff_op", "abs_diff", "hinge_diff", "squared_hinge_diff", "l1_diff_add"])}
 BINARY_INT = {"add": 0, "sub": 1, "multiply": 2}
 
 c_float_p = ctypes.POINTER(ctypes.c_float)
@@ -653,7 +653,9 @@ class Hip:
         "log": ("nhVectorLog", 0), "erf": ("nhVectorErf", 0), "sqrt": ("nhVectorSqrt", 0), "inv": ("nhVectorInv", 0),
         "minmax": ("nhVectorMinMax", 2), "sigmoid": ("nhVectorSigmoid", 0), "tanh": ("nhVectorTanh", 0),
         "add_value": ("nhVectorAddValue", 1), "multiply": ("nhVectorMultiply", 1),
-        "neg_multiply": ("nhVectorNegMultiply", 1), "neg_log": ("nhVectorNegLog", 0),
+        "neg_multiply": ("nhVectorNegMultiply", 1), "neg_log": ("nhVectorNegLog", 0), "hinge": ("nhVectorHinge", 0),
+        "squared_hinge": ("nhVectorSquaredHinge", 0), "huber": ("nhVectorHuber", 0),
+        "huber_derivative": ("nhVectorHuberDerivative", 0),
     }
 
 
@@ -691,6 +693,7 @@ class Hip:
         "elu_diff": "nhVectorELUDiff", "elu_diff_op": "nhVectorELUDiffOp", "leaky_relu_diff": "nhVectorLeakyReLUDiff",
         "hard_tanh_diff": "nhVectorHardTanhDiff", "hard_sigmoid_diff": "nhVectorHardSigmoidDiff",
         "hard_sigmoid_diff_op": "nhVectorHardSigmoidDiffOp", "abs_diff": "nhVectorAbsDiff",
+        "hinge_diff": "nhVectorHingeDiff", "squared_hinge_diff": "nhVectorSquaredHingeDiff", "l1_diff_add": "nhVectorL1DiffAdd",
     }
 
     def binary(self, op, a, b, p0=0.0, result=None, inplace_first=False, p1=0.0):
@@ -700,10 +703,10 @@ class Hip:
         args = [self.p(a), self.p(b), self.p(out), n]
         keep = []
         if op in ("multiply_and_add", "multiply_and_sub", "relu_diff", "elu_diff", "elu_diff_op", "leaky_relu_diff",
-                  "hard_sigmoid_diff", "hard_sigmoid_diff_op"):
+                  "hard_sigmoid_diff", "hard_sigmoid_diff_op", "l1_diff_add"):
             s = self.scalar(p0)
             args.append(self.p(s))
-        if op == "hard_sigmoid_diff":
+        if op in ("hard_sigmoid_diff", "l1_diff_add"):
             keep.append(self.scalar(p1))
             args.append(self.p(keep[0]))
         self.call(self.BINARY_FN[op], *args)

@@ -322,6 +322,7 @@ TRAIN_CASES = {
     "separable_sgd": (5, (1, 3, 1, 24, 24, 1, 3), 0, 0.02),
     "transformer_adam": (6, (1, 2, 8, 1, 1, 1, 32), 1, 0.003),
     "transformer_dropout_adam": (7, (1, 2, 8, 1, 1, 1, 32), 1, 0.003),
+    "batchnorm_cnn_sgd": (8, (1, 8, 1, 12, 12, 1, 3), 0, 0.05),
 }
 
 

@@ -34,7 +34,8 @@ UNARY_CASES = [
     ("abs", 0, 0), ("hard_tanh", 0, 0), ("hard_sigmoid", 0.2, 0.5), ("neg", 0, 0), ("exp", 0, 0), ("log", 0, 0),
     ("erf", 0, 0), ("sqrt", 0, 0), ("inv", 0, 0), ("minmax", -0.5, 1.5), ("sigmoid", 0, 0), ("tanh", 0, 0),
     ("add_value", 1.25, 0), ("multiply", -2.5, 0), ("neg_multiply", 1.702, 0), ("copy", 0, 0), ("neg_log", 0, 0),
-    ("sub_value", 0.75, 0), ("value_sub", 0.75, 0),
+    ("sub_value", 0.75, 0), ("value_sub", 0.75, 0), ("hinge", 0, 0), ("squared_hinge", 0, 0), ("huber", 0, 0),
+    ("huber_derivative", 0, 0),
 ]
 
 
@@ -72,6 +73,10 @@ NUMPY_UNARY = {
     "neg_log": lambda x, p0, p1: -np.log(np.clip(x.astype(np.float64), np.finfo(np.float32).tiny, None)),
     "sub_value": lambda x, p0, p1: x - np.float32(p0),
     "value_sub": lambda x, p0, p1: np.float32(p0) - x,
+    "hinge": lambda x, p0, p1: np.maximum(0, 1 - x),
+    "squared_hinge": lambda x, p0, p1: np.where(x < -1, -4 * x, np.maximum(0, 1 - x.astype(np.float64)) ** 2),
+    "huber": lambda x, p0, p1: np.where(np.abs(x) > 1, np.abs(x) - 0.5, x.astype(np.float64) ** 2 / 2),
+    "huber_derivative": lambda x, p0, p1: np.clip(x, -1, 1),
 }
 
 
@@ -137,7 +142,8 @@ def test_binary(op):
 # gradient that arrives from above, p = ReLU's upper threshold
 DIFF_CASES = [("relu_diff", 0.0), ("relu_diff", 6.0), ("hswish_diff", 0.0), ("sigmoid_diff", 0.0), ("sigmoid_diff_op", 0.0),
               ("tanh_diff", 0.0), ("tanh_diff_op", 0.0), ("elu_diff", 0.7), ("elu_diff_op", 0.7), ("leaky_relu_diff", 0.1),
-              ("hard_tanh_diff", 0.0), ("hard_sigmoid_diff", 0.2), ("hard_sigmoid_diff_op", 0.2), ("abs_diff", 0.0)]
+              ("hard_tanh_diff", 0.0), ("hard_sigmoid_diff", 0.2), ("hard_sigmoid_diff_op", 0.2), ("abs_diff", 0.0),
+              ("hinge_diff", 0.0), ("squared_hinge_diff", 0.0), ("l1_diff_add", 0.3)]
 HARD_SIGMOID_BIAS = 0.5  # second parameter of the hard sigmoid cases
 _expit = lambda a: scipy.special.expit(a.astype(np.float64))
 NUMPY_DIFF = {
@@ -154,10 +160,15 @@ NUMPY_DIFF = {
     "hard_sigmoid_diff": lambda a, b, p: np.where((a * p + HARD_SIGMOID_BIAS > 0) & (a * p + HARD_SIGMOID_BIAS < 1), b * np.float32(p), 0),
     "hard_sigmoid_diff_op": lambda a, b, p: np.where((a > 0) & (a < 1), b * np.float32(p), 0),
     "abs_diff": lambda a, b, p: np.where(a > 0, b, -b),
+    "hinge_diff": lambda a, b, p: np.where(a < 1, -b, 0),
+    "squared_hinge_diff": lambda a, b, p: np.where(a < -1, -4 * b, -2 * np.maximum(0, 1 - a.astype(np.float64)) * b),
+    # (p = the clamp threshold; the multiplier travels as the second parameter, HARD_SIGMOID_BIAS in these tests)
+    "l1_diff_add": lambda a, b, p: a + np.float32(HARD_SIGMOID_BIAS) * np.clip(b, -np.float32(p), np.float32(p)),
 }
 # the activation each derivative belongs to, for the finite-difference check
 DIFF_FORWARD = {"relu_diff": "relu", "hswish_diff": "hswish", "sigmoid_diff": "sigmoid", "tanh_diff": "tanh", "elu_diff": "elu",
-                "leaky_relu_diff": "leaky_relu", "hard_tanh_diff": "hard_tanh", "hard_sigmoid_diff": "hard_sigmoid", "abs_diff": "abs"}
+                "leaky_relu_diff": "leaky_relu", "hard_tanh_diff": "hard_tanh", "hard_sigmoid_diff": "hard_sigmoid", "abs_diff": "abs",
+                "hinge_diff": "hinge", "squared_hinge_diff": "squared_hinge"}
 
 
 def diff_operands(op, n, seed):
@@ -193,8 +204,8 @@ def test_activation_derivatives_are_the_slopes_of_the_activations(op, p):
     a = a[(np.abs(a) > 0.05)]
     eps = np.float32(1.0 / 256)
     fwd = DIFF_FORWARD[op]
-    if op in ("hard_tanh_diff", "hard_sigmoid_diff"):
-        a = a[np.abs(np.abs(a) - (1.0 if op == "hard_tanh_diff" else 2.5)) > 0.05]  # away from their kinks as well
+    if op in ("hard_tanh_diff", "hard_sigmoid_diff", "hinge_diff", "squared_hinge_diff"):
+        a = a[np.abs(np.abs(a) - (2.5 if op == "hard_sigmoid_diff" else 1.0)) > 0.05]  # away from their kinks as well
     slope = (orc.unary(fwd, a + eps, p, HARD_SIGMOID_BIAS).astype(np.float64) - orc.unary(fwd, a - eps, p, HARD_SIGMOID_BIAS)) / (2.0 * float(eps))
     y = orc.binary(op, a, np.ones_like(a), p, p1=HARD_SIGMOID_BIAS)
     np.testing.assert_allclose(y, slope, rtol=2e-3, atol=2e-4)
