@@ -959,13 +959,13 @@ SHIM_API int shim_clean_up( void* engine )
 	return guarded( [&]() { static_cast<IMathEngine*>( engine )->CleanUp(); } );
 }
 
-// probe for a method outside the inference path (asserts on engines that do not implement it)
-SHIM_API int shim_vector_huber( void* engine, const float* first, float* result, int n )
+// probe for a method outside the implemented paths (asserts on engines that do not implement it)
+SHIM_API int shim_vector_power( void* engine, float exponent, const float* first, float* result, int n )
 {
 	return guarded( [&]() {
 		IMathEngine& e = *static_cast<IMathEngine*>( engine );
 		CFloatBlob in( e, n, first ), out( e, n );
-		e.VectorHuber( in.Const(), out.Handle(), n );
+		e.VectorPower( exponent, in.Const(), out.Handle(), n );
 		out.CopyTo( result );
 	} );
 }

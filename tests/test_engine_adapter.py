@@ -8,7 +8,8 @@ import pytest
 
 import nhtest
 from nhtest import Cpu, assert_close
-from test_oracle import UNARY_CASES, BINARY_CASES, unary_input, rng
+from test_oracle import (UNARY_CASES, BINARY_CASES, DIFF_CASES, HARD_SIGMOID_BIAS, DROPOUT_CASES, BROADCAST_CASES,
+                         MOBILENETV3_CASES, diff_operands, mobilenetv3_operands, unary_input, rng)
 
 pytestmark = [pytest.mark.gpu,
               pytest.mark.skipif(not nhtest.have_engine_adapter(), reason="engine adapter or oracle/_ref not built")]
@@ -131,14 +132,13 @@ def test_lstm_through_the_interface(reverse):
 
 
 def test_unimplemented_method_asserts_like_the_reference_gpu_engine():
-    # VectorHuber is outside the inference path: the generated body raises through NeoML's exception handler,
+    # VectorPower is outside the implemented paths: the generated body raises through NeoML's exception handler,
     # which the shim turns into an error code instead of letting it cross the C boundary
     s = nhtest.shim()
-    if not hasattr(s, "shim_vector_huber"):
-        pytest.skip("shim has no probe for an unimplemented method")
-    x = np.ones(8, np.float32)
+    x = np.full(8, 2.0, np.float32)
     y = np.empty(8, np.float32)
-    assert s.shim_vector_huber(nhtest.hip_engine(), nhtest.fp(x), nhtest.fp(y), 8) == 1
+    assert s.shim_vector_power(nhtest.hip_engine(), ctypes.c_float(2.0), nhtest.fp(x), nhtest.fp(y), 8) == 1
+    assert s.shim_vector_power(nhtest.cpu_engine(), ctypes.c_float(2.0), nhtest.fp(x), nhtest.fp(y), 8) == 0 and y[0] == 4.0
 
 
 @pytest.mark.parametrize("with_expand", [True, False])
@@ -154,3 +154,77 @@ def test_fused_separable_blocks_through_the_interface(with_expand):
         if residual and with_expand:
             assert_close(hip.separable_block(x, expand, channelwise, down, stride, residual, in_place=True), want,
                          "separable block in place %s" % (case,))
+
+
+# ---- what the backward and learn passes of the layers call, through the interface -----------------------------
+
+@pytest.mark.parametrize("op,p", DIFF_CASES)
+def test_activation_derivatives_through_the_interface(op, p):
+    hip, ref = engines()
+    a, b = diff_operands(op, 4099, 3)
+    assert_close(hip.binary(op, a, b, p, p1=HARD_SIGMOID_BIAS), ref.binary(op, a, b, p, p1=HARD_SIGMOID_BIAS), op)
+
+
+def test_gradients_through_the_interface():
+    hip, ref = engines()
+    g = rng(501)
+    # convolution: stride 2 with an odd size (class-by-class input gradient), free terms on both sides
+    n, h, w, cin, cout, fh, fw, ph, pw, sh, sw = 2, 15, 13, 8, 12, 3, 3, 1, 1, 2, 2
+    ho, wo = nhtest.conv_out(h, w, fh, fw, ph, pw, sh, sw)
+    x = g.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    f = g.normal(0, 0.2, (cout, fh, fw, cin)).astype(np.float32)
+    grad = g.uniform(-1, 1, (n, ho, wo, cout)).astype(np.float32)
+    bias = g.uniform(-1, 1, cin).astype(np.float32)
+    assert_close(hip.conv_backward(grad, f, bias, x.shape, ph, pw, sh, sw), ref.conv_backward(grad, f, bias, x.shape, ph, pw, sh, sw),
+                 "BlobConvolutionBackward", atol=2e-5)
+    start, ft0 = g.uniform(-1, 1, f.shape).astype(np.float32), g.uniform(-1, 1, cout).astype(np.float32)
+    got, want = (e.conv_learn_add(x, grad, start, ph, pw, sh, sw, free_term_diff=ft0) for e in (hip, ref))
+    assert_close(got[0], want[0], "BlobConvolutionLearnAdd", atol=1e-4)
+    assert_close(got[1], want[1], "free term gradient", atol=1e-4)
+    # channelwise convolution
+    fc = g.normal(0, 0.5, (3, 3, cin)).astype(np.float32)
+    gc = g.uniform(-1, 1, (n, ho, wo, cin)).astype(np.float32)
+    assert_close(hip.channelwise_conv_backward(gc, fc, x.shape, 1, 1, 2, 2), ref.channelwise_conv_backward(gc, fc, x.shape, 1, 1, 2, 2),
+                 "BlobChannelwiseConvolutionBackward")
+    got, want = (e.channelwise_conv_learn_add(x, gc, fc, 1, 1, 2, 2, free_term_diff=bias) for e in (hip, ref))
+    assert_close(got[0], want[0], "BlobChannelwiseConvolutionLearnAdd", atol=1e-4)
+    assert_close(got[1], want[1], "channelwise free term gradient", atol=1e-4)
+    # pooling
+    gp = g.uniform(-1, 1, (n, 7, 6, cin)).astype(np.float32)
+    assert_close(hip.max_pool_backward(x, gp, 3, 3, 2, 2), ref.max_pool_backward(x, gp, 3, 3, 2, 2), "BlobMaxPoolingBackward")
+    assert_close(hip.mean_pool_backward(x.shape, gp, 3, 3, 2, 2), ref.mean_pool_backward(x.shape, gp, 3, 3, 2, 2), "BlobMeanPoolingBackward")
+    # softmax derivative, row products, diagonal accumulation
+    y = ref.softmax_rows(g.uniform(-3, 3, (33, 101)).astype(np.float32))
+    d = g.uniform(-1, 1, y.shape).astype(np.float32)
+    assert_close(hip.softmax_diff_rows(y, d), ref.softmax_diff_rows(y, d), "MatrixSoftmaxDiffOpByRows", atol=1e-6)
+    assert_close(hip.row_dot(y, d), ref.row_dot(y, d), "RowMultiplyMatrixByMatrix")
+    diag, m, acc = g.uniform(-1, 1, (2, 9)).astype(np.float32), g.uniform(-1, 1, (2, 9, 20)).astype(np.float32), g.uniform(-1, 1, (9, 20)).astype(np.float32)
+    assert_close(hip.diag_by_matrix_add(diag, m, acc), ref.diag_by_matrix_add(diag, m, acc), "MultiplyDiagMatrixByMatrixAndAdd")
+
+
+@pytest.mark.parametrize("dims,rate,spatial,batchwise", DROPOUT_CASES[:5])
+def test_dropout_through_the_interface(dims, rate, spatial, batchwise):
+    hip, ref = engines()
+    x = rng(502).uniform(0.5, 1.5, dims).astype(np.float32)
+    got, want = hip.dropout(x, rate, spatial, batchwise, 77), ref.dropout(x, rate, spatial, batchwise, 77)
+    assert np.array_equal(got != 0, want != 0)
+    assert_close(got, want, "Dropout")
+
+
+@pytest.mark.parametrize("from_dims,to_dims,width", BROADCAST_CASES)
+def test_broadcast_copy_through_the_interface(from_dims, to_dims, width):
+    hip, ref = engines()
+    x = rng(503).uniform(-1, 1, from_dims + (width,)).astype(np.float32)
+    assert np.array_equal(hip.broadcast_copy(x, to_dims, width), ref.broadcast_copy(x, to_dims, width))
+
+
+@pytest.mark.parametrize("case", MOBILENETV3_CASES[:3])
+def test_mobilenetv3_blocks_through_the_interface(case):
+    hip, ref = engines()
+    n, h, w, cin, e, cout, fsize, stride, residual, ex_act, ch_act, gate_act = case
+    x, expand, channelwise, gate, down = mobilenetv3_operands(case)
+    pre = ref.mobilenetv3_pre_se(x, expand, channelwise, stride)
+    assert_close(hip.mobilenetv3_pre_se(x, expand, channelwise, stride), pre, "MobileNetV3PreSEBlock", atol=2e-5)
+    res = x if residual and stride == 1 and cin == cout else None
+    assert_close(hip.mobilenetv3_post_se(pre, gate, res, gate_act[0], gate_act[1], down),
+                 ref.mobilenetv3_post_se(pre, gate, res, gate_act[0], gate_act[1], down), "MobileNetV3PostSEBlock", atol=2e-5)
