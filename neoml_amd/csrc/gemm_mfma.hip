@@ -28,6 +28,9 @@
 // k, which is all the dot product needs.
 #include "common.h"
 #include <math.h>
+#include <map>
+#include <mutex>
+#include <utility>
 
 namespace nh {
 
@@ -80,6 +83,11 @@ struct CMatMulArgs {
 	// behind them share the TailTiles remaining tiles, TailSplit slices of TailSteps K steps per tile, and meet in C
 	// through atomic adds like the K slices above
 	int FullTiles, TailTiles, TailSplit, TailSteps;
+	// K slices that meet without atomics (Partials != null): every slice leaves its accumulators in Partials
+	// [ sliced tile ][ slice ][ 4096 ] and counts itself in Counters[ sliced tile ]; the slice that counts last adds
+	// them up in slice order, runs the ordinary epilogue and sets the counter back to zero for the next launch.
+	float* Partials;
+	unsigned* Counters;
 	// AM_ConvClasses: the dense result is [images][OutH][OutW][Ldc], DenseM pixels in all
 	int OutH, OutW, OutUpH, OutUpW, DenseM;
 	CConvClass Class[MaxConvClasses];
@@ -687,6 +695,56 @@ void matMulKernel( const CMatMulArgs launchArgs )
 		}
 	}
 
+	if constexpr( MI * NI == 1 && KGROUPS == 1 ) {
+		if( splitK > 1 && args.Partials != nullptr ) {
+			// Values cross between workgroups (and so between the L2 caches of the XCDs) through device-scope atomic
+			// stores and loads, which go past those caches. A wave's stores are complete when the barrier lets it
+			// through, the count follows the barrier: whoever reads the full count finds every slice's values.
+			const int slicedTile = args.FullTiles > 0 ? tile - args.FullTiles : tile;
+			unsigned* mine = reinterpret_cast<unsigned*>( args.Partials )
+				+ ( static_cast<long long>( slicedTile ) * splitK + split ) * ( BM * BN ) + wave * 64 + lane;
+#pragma unroll
+			for( int r = 0; r < 16; ++r ) {
+				__hip_atomic_store( mine + r * Threads, __float_as_uint( acc[0][0][r] ), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT );
+			}
+			__builtin_amdgcn_s_waitcnt( 0x0F70 ); // vmcnt( 0 ): this wave's stores have been acknowledged
+			__syncthreads();
+			unsigned* arrived = reinterpret_cast<unsigned*>( &lds[0][0][0] );
+			if( tid == 0 ) {
+				*arrived = __hip_atomic_fetch_add( args.Counters + slicedTile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT );
+			}
+			__syncthreads();
+			if( *arrived != static_cast<unsigned>( splitK - 1 ) ) {
+				return;
+			}
+			f32x16 total;
+#pragma unroll
+			for( int r = 0; r < 16; ++r ) {
+				total[r] = 0.f;
+			}
+			const unsigned* first = mine - static_cast<long long>( split ) * ( BM * BN );
+			for( int slice = 0; slice < splitK; ++slice ) {
+				if( slice == split ) {
+#pragma unroll
+					for( int r = 0; r < 16; ++r ) {
+						total[r] += acc[0][0][r];
+					}
+				} else {
+					const unsigned* theirs = first + static_cast<long long>( slice ) * ( BM * BN );
+#pragma unroll
+					for( int r = 0; r < 16; ++r ) {
+						total[r] += __uint_as_float( __hip_atomic_load( theirs + r * Threads, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT ) );
+					}
+				}
+			}
+			acc[0][0] = total;
+			if( tid == 0 ) {
+				__hip_atomic_store( args.Counters + slicedTile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT );
+			}
+			splitK = 1; // from here on: the one workgroup that writes the tile
+		}
+	}
+
 #pragma unroll
 	for( int ni = 0; ni < NI; ++ni ) {
 		const int n = n0 + waveN * WN + ni * 32 + l32;
@@ -727,6 +785,72 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			}
 		}
 	}
+}
+
+// Scratch of the K slices that meet without atomics: partial tiles and arrival counters, one pair per stream (launches
+// of one stream run in order and may share it; two streams must not). Grown on demand, kept until the process ends.
+// The counters start at zero and every launch leaves them at zero.
+struct CSliceScratch {
+	float* Partials = nullptr;
+	size_t PartialFloats = 0;
+	unsigned* Counters = nullptr;
+	size_t CounterCount = 0;
+};
+
+static bool sliceScratch( hipStream_t stream, size_t partialFloats, size_t counters, CSliceScratch& out )
+{
+	static std::mutex lock;
+	static std::map<std::pair<int, hipStream_t>, CSliceScratch> byStream;
+	int device = 0;
+	if( hipGetDevice( &device ) != hipSuccess ) {
+		return false;
+	}
+	std::lock_guard<std::mutex> guard( lock );
+	// A recorded graph would keep the address of a block that a later, larger launch frees, and may replay on another
+	// stream: launches under capture take the atomic path.
+	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+	if( hipStreamIsCapturing( stream, &capture ) != hipSuccess || capture != hipStreamCaptureStatusNone ) {
+		( void )hipGetLastError();
+		return false;
+	}
+	CSliceScratch& scratch = byStream[std::make_pair( device, stream )];
+	if( scratch.PartialFloats < partialFloats ) {
+		// work that still reads the old block must finish first
+		if( hipStreamSynchronize( stream ) != hipSuccess ) {
+			return false;
+		}
+		if( scratch.Partials != nullptr ) {
+			( void )hipFree( scratch.Partials );
+			scratch.Partials = nullptr;
+			scratch.PartialFloats = 0;
+		}
+		const size_t grown = partialFloats + partialFloats / 4;
+		if( hipMalloc( reinterpret_cast<void**>( &scratch.Partials ), grown * sizeof( float ) ) != hipSuccess ) {
+			( void )hipGetLastError();
+			return false;
+		}
+		scratch.PartialFloats = grown;
+	}
+	if( scratch.CounterCount < counters ) {
+		if( hipStreamSynchronize( stream ) != hipSuccess ) {
+			return false;
+		}
+		if( scratch.Counters != nullptr ) {
+			( void )hipFree( scratch.Counters );
+			scratch.Counters = nullptr;
+			scratch.CounterCount = 0;
+		}
+		const size_t grown = counters * 2 > 4096 ? counters * 2 : 4096;
+		if( hipMalloc( reinterpret_cast<void**>( &scratch.Counters ), grown * sizeof( unsigned ) ) != hipSuccess
+			|| hipMemset( scratch.Counters, 0, grown * sizeof( unsigned ) ) != hipSuccess )
+		{
+			( void )hipGetLastError();
+			return false;
+		}
+		scratch.CounterCount = grown;
+	}
+	out = scratch;
+	return true;
 }
 
 // C[b][m][n] = bias[n] (or 0): the starting value that the K slices add their partial products to
@@ -856,17 +980,33 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 			tailRow = static_cast<int>( full / args.TilesN ) * BM;
 		}
 	}
+	// Few slices per tile, one matrix: the slices meet through partial tiles in scratch memory and the last one to arrive
+	// runs the epilogue, so there is no preset of C, no atomic add and no separate activation pass, and the sum has a
+	// fixed order. (Not for the gradient by a filter with its dozens of slices, nor for the per-class launches, whose
+	// slices may have nothing to do and would never arrive.) Falls back to atomics when the scratch cannot be had.
+	if( ( args.SplitK > 1 || args.FullTiles > 0 ) && batch == 1 && args.ManySlices == 0 && AMODE != AM_ConvClasses
+		&& BM * BN == 4096 )
+	{
+		const size_t slicedTiles = args.FullTiles > 0 ? args.TailTiles : static_cast<size_t>( tiles );
+		const size_t slices = args.FullTiles > 0 ? args.TailSplit : args.SplitK;
+		CSliceScratch scratch;
+		if( sliceScratch( stream, slicedTiles * slices * 4096, slicedTiles, scratch ) ) {
+			args.Partials = scratch.Partials;
+			args.Counters = scratch.Counters;
+		}
+	}
+	const bool meetInScratch = args.Partials != nullptr;
 	// the rows of the tail tiles as a matrix product of their own: what the preset and the activation pass cover
 	CMatMulArgs tail = args;
 	tail.C += static_cast<long long>( tailRow ) * args.Ldc;
 	tail.M = args.M - tailRow;
-	if( args.FullTiles > 0 && !args.Accumulate ) {
+	if( args.FullTiles > 0 && !args.Accumulate && !meetInScratch ) {
 		const int rc = presetResult( stream, tail, 1 );
 		if( rc != NH_OK ) {
 			return rc;
 		}
 	}
-	if( args.SplitK > 1 && !args.Accumulate ) {
+	if( args.SplitK > 1 && !args.Accumulate && !meetInScratch ) {
 		CMatMulArgs dense = args;
 		if( AMODE == AM_ConvClasses ) {
 			dense.M = args.DenseM; // the classes interleave in one dense result
@@ -877,7 +1017,7 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 		}
 	}
 	const CFusedActivation actAfter = args.Act;
-	if( args.SplitK > 1 ) {
+	if( args.SplitK > 1 && !meetInScratch ) {
 		args.Act.Type = NH_ACT_NONE;
 	}
 	// blockIdx.y is limited to 65535: walk larger batches in slices
@@ -897,13 +1037,13 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 		} else {
 			hipLaunchKernelGGL( ( matMulKernel<BM, BN, WAVES_M, WAVES_N, AMODE, BMODE, false> ), grid, dim3( Threads ), 0, stream, a );
 		}
-		if( args.FullTiles > 0 && actAfter.Type != NH_ACT_NONE ) {
+		if( args.FullTiles > 0 && actAfter.Type != NH_ACT_NONE && !meetInScratch ) {
 			const long long total = static_cast<long long>( tail.M ) * args.N;
 			const long long blocksAct = ( total + 1023 ) / 1024;
 			hipLaunchKernelGGL( activateResultKernel, dim3( static_cast<unsigned>( blocksAct > 4096 ? 4096 : blocksAct ), 1 ), dim3( 256 ), 0,
 				stream, tail.C, tail.M, args.N, args.Ldc, args.BatchStrideC, actAfter );
 		}
-		if( args.SplitK > 1 && actAfter.Type != NH_ACT_NONE ) {
+		if( args.SplitK > 1 && actAfter.Type != NH_ACT_NONE && !meetInScratch ) {
 			const long long total = static_cast<long long>( args.M ) * args.N;
 			const long long blocksAct = ( total + 1023 ) / 1024;
 			hipLaunchKernelGGL( activateResultKernel, dim3( static_cast<unsigned>( blocksAct > 4096 ? 4096 : blocksAct ), nb ), dim3( 256 ), 0,

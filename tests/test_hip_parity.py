@@ -433,6 +433,27 @@ def test_pooling_gradients(case):
                  "mean pooling backward %s" % (case,))
 
 
+def test_k_sliced_convolutions_are_bit_reproducible():
+    # K slices meet through partial tiles that the last slice to arrive adds up in slice order: whichever slice that is,
+    # the sum has one order. Alternating shapes also checks that every launch leaves the arrival counters at zero.
+    h = hip()
+    g = rng(93)
+    cases = [(4, 14, 14, 256, 256), (2, 7, 7, 512, 512), (24, 28, 28, 128, 128)]  # 3 slices; 8 slices; whole tiles + sliced tail
+    data = []
+    for n, hw, _, cin, cout in cases:
+        x = g.uniform(-1, 1, (n, hw, hw, cin)).astype(np.float32)
+        f = g.normal(0, 1.0 / np.sqrt(9 * cin), (cout, 3, 3, cin)).astype(np.float32)
+        b = g.uniform(-1, 1, cout).astype(np.float32)
+        data.append((x, f, b, h.conv(x, f, b, 1, 1, 1, 1)))
+    for _ in range(3):
+        for x, f, b, first in data:
+            assert np.array_equal(h.conv(x, f, b, 1, 1, 1, 1), first)
+    x, f, b, first = data[0]
+    assert_close(first, orc.conv(x, f, b, 1, 1, 1, 1), "sliced convolution vs oracle")
+    relu = h.conv(x, f, b, 1, 1, 1, 1, activation="relu")
+    assert np.array_equal(relu, np.maximum(first, 0)), "activation in the last slice's epilogue"
+
+
 def test_convolution_ignores_pixels_outside_the_windows():
     # stride 4 with a 3-wide filter never touches image columns 3 and 7; whatever they hold (here: infinities)
     # must not leak into the result through the vector fetches that run past a window's last value
