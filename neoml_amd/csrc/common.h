@@ -109,5 +109,13 @@ __device__ __forceinline__ float4 bufferLoad4( __amdgpu_buffer_rsrc_t rsrc, unsi
 	return make_float4( __uint_as_float( v.x ), __uint_as_float( v.y ), __uint_as_float( v.z ), __uint_as_float( v.w ) );
 }
 
+// The same with a second, wave-uniform byte offset that travels in a scalar register: what a loop adds per iteration
+// costs no vector instruction. The range check looks at the per-lane offset, so OutOfRange still reads as zero.
+__device__ __forceinline__ float4 bufferLoad4( __amdgpu_buffer_rsrc_t rsrc, unsigned offset, unsigned uniformOffset )
+{
+	const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128( rsrc, offset, uniformOffset, 0 );
+	return make_float4( __uint_as_float( v.x ), __uint_as_float( v.y ), __uint_as_float( v.z ), __uint_as_float( v.w ) );
+}
+
 } // namespace nh
 #endif

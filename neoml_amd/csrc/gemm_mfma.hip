@@ -11,16 +11,19 @@
 // a (BM/WAVES_M) x (BN/WAVES_N) sub-tile built from 32x32 blocks of v_mfma_f32_32x32x2_f32 (16 accumulator
 // registers per block).
 //
-// Data path: operands are fetched with raw buffer loads (32-bit offsets that only need an add per K step; the
-// memory unit's range check supplies the zeros of padding and of partial tiles), parked in registers for one
-// K step, written to one of three LDS buffers and read back as MFMA operands. Within a wavefront the LDS reads
+// Data path: operands are fetched with raw buffer loads (a 32-bit offset per lane that stays put, plus what a K step
+// adds in a scalar register; the memory unit's range check supplies the zeros of padding and of partial tiles),
+// parked in registers for one K step, written to one of two LDS buffers (20 KB per workgroup: seven workgroups
+// per compute unit) and read back as MFMA operands. Within a wavefront the LDS reads
 // of the next group of 8 k are issued before the MFMAs of the current group, and the single barrier of a K step
 // sits before its last group, so the matrix pipe of a wavefront does not wait for LDS, barrier or memory in steady
 // state.
 //
 // Small grids: when the tiles alone would leave the compute units with one or two workgroups each, K is cut into
-// slices (grid z); the slices add their partial products into C with fp32 atomics after C has been set to the free
-// term. The summation order of the slices then varies from run to run (differences at the 1e-7 relative level).
+// slices (grid z). The slices of one matrix meet inside the launch through partial tiles in scratch memory, summed
+// in slice order by the slice that arrives last; batched products, the gradient by a filter and launches recorded
+// into a graph add their partial products into C with fp32 atomics after C has been set to the free term (the
+// summation order of those slices varies from run to run, differences at the 1e-7 relative level).
 //
 // LDS layout for a K-major operand is [row][16 + 4 pad]; lane (row = lane % 32, half = lane / 32) fetches the
 // four consecutive k values  k0 + 4*half .. +3  with a single 128-bit LDS read and feeds them to four MFMAs.
@@ -139,9 +142,9 @@ void matMulKernel( const CMatMulArgs launchArgs )
 	constexpr int ASlots = ( ATotal + Threads - 1 ) / Threads;
 	constexpr int BSlots = ( BTotal + Threads - 1 ) / Threads;
 
-	__shared__ __attribute__( ( aligned( 16 ) ) ) float lds[KGROUPS][3][ASize + BSize];
+	__shared__ __attribute__( ( aligned( 16 ) ) ) float lds[KGROUPS][2][ASize + BSize];
 
-	const int kGroup = KGROUPS == 1 ? 0 : threadIdx.x / Threads;
+	const int kGroup = KGROUPS == 1 ? 0 : __builtin_amdgcn_readfirstlane( threadIdx.x / Threads ); // same for a whole wave
 	const int tid = KGROUPS == 1 ? threadIdx.x : threadIdx.x % Threads; // inside the group
 	auto ldsA = [&]( int buf ) -> float* { return lds[kGroup][buf]; };
 	auto ldsB = [&]( int buf ) -> float* { return lds[kGroup][buf] + ASize; };
@@ -246,15 +249,43 @@ void matMulKernel( const CMatMulArgs launchArgs )
 		rowKh = k / args.RowPitch;
 		rowR = k - rowKh * args.RowPitch;
 	}
+	// Channel counts that are a multiple of the K step: every lane of the workgroup is in the same filter tap during a
+	// step, so the tap and the channel inside it live in scalar registers, the channel reaches the loads as their
+	// uniform offset, and a step inside a tap costs no vector instruction for addresses.
+	const bool uniformTap = IsConv && VEC && args.Cin % KS == 0;
+	int tapCi = 0, tapKh = 0, tapKw = 0;
+	auto tapSlotOffset = [&]( int i ) -> unsigned {
+		int hi = convH0[i] + tapKh * args.DilH;
+		int wi = convW0[i] + tapKw * args.DilW;
+		bool ok = tapKh < args.Fh;
+		if( args.UpH > 1 || args.UpW > 1 ) {
+			ok = ok && hi >= 0 && wi >= 0 && hi % args.UpH == 0 && wi % args.UpW == 0;
+			hi /= args.UpH;
+			wi /= args.UpW;
+		}
+		ok = ok && hi >= 0 && hi < args.H && wi >= 0 && wi < args.W;
+		return ok ? static_cast<unsigned>( convPixel[i] + ( hi * args.W + wi ) * args.Cin + ( tid % KQ ) * 4 ) * 4u : OutOfRange;
+	};
 	if( IsConv && VEC ) {
-		const int k = kStart + ( tid % KQ ) * 4;
-		const int tap = k / args.Cin;
-		convCi = k - tap * args.Cin;
-		convKh = tap / args.Fw;
-		convKw = tap - convKh * args.Fw;
+		if( uniformTap ) {
+			const int tap = kStart / args.Cin;
+			tapCi = kStart - tap * args.Cin;
+			tapKh = tap / args.Fw;
+			tapKw = tap - tapKh * args.Fw;
 #pragma unroll
-		for( int i = 0; i < ASlots; ++i ) {
-			offA[i] = convSlotOffset( i );
+			for( int i = 0; i < ASlots; ++i ) {
+				offA[i] = tapSlotOffset( i );
+			}
+		} else {
+			const int k = kStart + ( tid % KQ ) * 4;
+			const int tap = k / args.Cin;
+			convCi = k - tap * args.Cin;
+			convKh = tap / args.Fw;
+			convKw = tap - convKh * args.Fw;
+#pragma unroll
+			for( int i = 0; i < ASlots; ++i ) {
+				offA[i] = convSlotOffset( i );
+			}
 		}
 	}
 	// BM_ConvN: per slot, the tap of its four columns ( fixed for the whole launch ) and the output pixel of its row
@@ -381,27 +412,35 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			return;
 		}
 		if( VEC ) {
-			// k of this thread's slots inside the step: fixed column of a K-major tile, fixed row of an X-major one
-			const bool kInA = AMODE == AM_RowsM ? true : ( kBase + ( tid % KQ ) * 4 < K );
-			const bool kInB = BMODE != BM_RowsK ? true : ( kBase + ( tid % KQ ) * 4 < K );
+			// Offsets of the slots stay where the slice begins; what a step adds is the same for every lane and goes to
+			// the loads as their uniform offset. Only the last step of a K that is not a multiple of the step masks k.
+			const unsigned stepK = static_cast<unsigned>( kBase - kStart );
+			const unsigned uniA = IsConv ? ( uniformTap ? static_cast<unsigned>( tapCi ) * 4u : 0u )
+				: ( AMODE == AM_RowsK ? stepK * 4u : stepK * static_cast<unsigned>( args.Lda ) * 4u );
+			const unsigned uniB = BMODE == BM_ConvN ? 0u
+				: ( BMODE == BM_RowsK ? stepK * 4u : stepK * static_cast<unsigned>( args.Ldb ) * 4u );
+			const bool partialStep = kBase + KS > K;
+			if( IsConv || !partialStep ) {
+				// the image's own zero padding covers k beyond K: such taps lie below the filter ( kh >= Fh )
 #pragma unroll
-			for( int i = 0; i < ASlots; ++i ) {
-				unsigned off = offA[i];
-				if( AMODE == AM_RowsK ) {
-					off = kInA ? off : OutOfRange;
-				} else if( AMODE == AM_RowsM ) {
-					off = ( kBase + ( tid + i * Threads ) / ( BM / 4 ) < K ) ? off : OutOfRange;
+				for( int i = 0; i < ASlots; ++i ) {
+					regA[i] = bufferLoad4( bufA, offA[i], uniA );
 				}
-				regA[i] = bufferLoad4( bufA, off );
-			}
+			} else {
+				asm volatile( "" ); // keeps this rare case a branch of its own instead of selects in every step
 #pragma unroll
-			for( int i = 0; i < BSlots; ++i ) {
-				unsigned off = offB[i];
-				if( BMODE == BM_ConvN ) {
+				for( int i = 0; i < ASlots; ++i ) {
+					const int kOfSlot = AMODE == AM_RowsM ? ( tid + i * Threads ) / ( BM / 4 ) : ( tid % KQ ) * 4;
+					regA[i] = bufferLoad4( bufA, kBase + kOfSlot < K ? offA[i] : OutOfRange, uniA );
+				}
+			}
+			if( BMODE == BM_ConvN ) {
+#pragma unroll
+				for( int i = 0; i < BSlots; ++i ) {
 					const int hi = bHo[i] * args.StrideH + bDh[i];
 					const int wi = bWo[i] * args.StrideW + bDw[i];
 					const bool ok = bPixel[i] < K && hi >= 0 && hi < args.H && wi >= 0 && wi < args.W;
-					off = ok ? static_cast<unsigned>( ( ( bImg[i] * args.H + hi ) * args.W + wi ) * args.Cin + bCi[i] ) * 4u : OutOfRange;
+					const unsigned off = ok ? static_cast<unsigned>( ( ( bImg[i] * args.H + hi ) * args.W + wi ) * args.Cin + bCi[i] ) * 4u : OutOfRange;
 					// the row of this slot in the next K step
 					bPixel[i] += KS;
 					bWo[i] += KS;
@@ -412,46 +451,56 @@ void matMulKernel( const CMatMulArgs launchArgs )
 							++bImg[i];
 						}
 					}
-				} else if( BMODE == BM_RowsK ) {
-					off = kInB ? off : OutOfRange;
-				} else {
-					off = ( kBase + ( tid + i * Threads ) / ( BN / 4 ) < K ) ? off : OutOfRange;
+					regB[i] = bufferLoad4( bufB, off );
 				}
-				regB[i] = bufferLoad4( bufB, off );
-			}
-			// advance
-			if( IsConv ) {
-				convCi += KS;
-				if( convCi >= args.Cin ) {
-					do {
-						convCi -= args.Cin;
-						if( ++convKw == args.Fw ) {
-							convKw = 0;
-							++convKh;
-						}
-					} while( convCi >= args.Cin );
-#pragma unroll
-					for( int i = 0; i < ASlots; ++i ) {
-						offA[i] = convSlotOffset( i );
-					}
-				} else {
-#pragma unroll
-					for( int i = 0; i < ASlots; ++i ) {
-						offA[i] += KS * 4;
-					}
-				}
-			} else {
-				const unsigned stepA = AMODE == AM_RowsK ? KS * 4u : static_cast<unsigned>( KS * args.Lda ) * 4u;
-#pragma unroll
-				for( int i = 0; i < ASlots; ++i ) {
-					offA[i] += stepA;
-				}
-			}
-			if( BMODE != BM_ConvN ) {
-				const unsigned stepB = BMODE == BM_RowsK ? KS * 4u : static_cast<unsigned>( KS * args.Ldb ) * 4u;
+			} else if( !partialStep ) {
 #pragma unroll
 				for( int i = 0; i < BSlots; ++i ) {
-					offB[i] += stepB;
+					regB[i] = bufferLoad4( bufB, offB[i], uniB );
+				}
+			} else {
+				asm volatile( "" );
+#pragma unroll
+				for( int i = 0; i < BSlots; ++i ) {
+					const int kOfSlot = BMODE == BM_RowsK ? ( tid % KQ ) * 4 : ( tid + i * Threads ) / ( BN / 4 );
+					regB[i] = bufferLoad4( bufB, kBase + kOfSlot < K ? offB[i] : OutOfRange, uniB );
+				}
+			}
+			// advance the convolution's tap
+			if( IsConv ) {
+				if( uniformTap ) {
+					tapCi += KS;
+					if( tapCi >= args.Cin ) {
+						tapCi = 0;
+						if( ++tapKw == args.Fw ) {
+							tapKw = 0;
+							++tapKh;
+						}
+#pragma unroll
+						for( int i = 0; i < ASlots; ++i ) {
+							offA[i] = tapSlotOffset( i );
+						}
+					}
+				} else {
+					convCi += KS;
+					if( convCi >= args.Cin ) {
+						do {
+							convCi -= args.Cin;
+							if( ++convKw == args.Fw ) {
+								convKw = 0;
+								++convKh;
+							}
+						} while( convCi >= args.Cin );
+#pragma unroll
+						for( int i = 0; i < ASlots; ++i ) {
+							offA[i] = convSlotOffset( i );
+						}
+					} else {
+#pragma unroll
+						for( int i = 0; i < ASlots; ++i ) {
+							offA[i] += KS * 4;
+						}
+					}
 				}
 			}
 			return;
@@ -615,13 +664,16 @@ void matMulKernel( const CMatMulArgs launchArgs )
 		}
 	};
 
-	// Software pipeline over K steps of KS, three LDS buffers, one barrier per step:
-	//   top of step ks : the tiles of step ks+1 (loaded from memory during step ks-1) go to LDS buffer (ks+1)%3, then
+	// Software pipeline over K steps of KS, two LDS buffers, one barrier per step:
+	//   top of step ks : the tiles of step ks+1 (loaded from memory during step ks-1) go to LDS buffer (ks+1)%2, then
 	//                    the loads of step ks+2 are issued;
 	//   body           : the MFMAs of each group of 8 k run while the fragments of the following group are being
 	//                    read from LDS; the barrier sits before the last group, after which the first fragments of
 	//                    step ks+1 are fetched, so neither the LDS latency nor the barrier leaves the MFMA pipe idle.
-	// Buffer (ks+1)%3 was last read in step ks-2, and every wave has passed the barrier of step ks-1 since.
+	// Buffer (ks+1)%2 was last read in step ks-1 BEFORE that step's barrier (the fragments of a step's last group are
+	// fetched ahead of the barrier, and a wave waits for its LDS reads before it enters the barrier; behind the barrier
+	// a wave only reads the other buffer), and a wave that stores at the top of step ks has passed that barrier: two
+	// buffers are enough, and the smaller footprint puts seven workgroups instead of five on a compute unit.
 	const int totalSteps = ( K + KS - 1 ) / KS;
 	const int kSteps = min( stepsPerSplit, totalSteps - split * stepsPerSplit );
 	constexpr int Groups = KS / 8;
@@ -639,7 +691,7 @@ void matMulKernel( const CMatMulArgs launchArgs )
 	}
 	int cur = 0;
 	for( int ks = 0; ks < kSteps; ++ks ) {
-		const int nxt = cur == 2 ? 0 : cur + 1;
+		const int nxt = cur ^ 1;
 		if( ks + 1 < kSteps ) {
 			storeTiles( nxt, rA, rB );
 		}
@@ -903,8 +955,9 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 		return NH_ERR_ARGUMENT;
 	}
 	// K slices: when the tiles alone leave most compute units with one or two workgroups, K is cut into slices that
-	// meet in C through fp32 atomic adds (C is pre-set to the free term). 1280 workgroups (5 per compute unit) run
-	// at once; the slice count is the one that wastes least of the last round of 1280, each extra slice priced at 2 %
+	// meet in scratch memory or, where that is not possible, in C through fp32 atomic adds. Seven workgroups fit a compute
+	// unit, five saturate it: the grid is planned in rounds of 1280 (measured: planning with 1792 is slower everywhere);
+	// the slice count is the one that wastes least of the last round of 1280, each extra slice priced at 2 %
 	// for its atomics, and every slice keeps at least 8 K steps.
 	// an empty reduction ( K == 0 ) still launches: one step of masked loads, C receives the free term or keeps its value
 	const int totalSteps = args.K > 0 ? ceilDiv( args.K, NH_KSTEP ) : 1;
@@ -942,7 +995,7 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 	// whole tiles, from measurements of the 3x3 convolutions: a round filled to the fraction f takes 0.17 + 0.85 f of a
 	// full one (fewer workgroups per compute unit run faster, but not in proportion), a workgroup costs about 4 K steps
 	// beyond its own, and the preset of the tail rows about 2 K steps of a round.
-	const int slots = 256 * ( BM * BN <= 64 * 64 ? 5 : 4 );
+	const int slots = 256 * 5; // planned as above: the five that saturate a compute unit, not the seven that fit
 	long long gridX = tiles;
 	int tailRow = 0;
 	if( splits == 1 && !twoGroups && batch == 1 && AMODE != AM_ConvClasses && args.Residual == nullptr && tiles >= slots && totalSteps >= 16 ) {
@@ -1055,7 +1108,7 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 }
 
 // Picks the workgroup tile. Measured on MI355X (convolutions of 64..512 channels, GEMMs up to 8192^3): the 64x64 tile
-// wins or ties everywhere, because it puts the most workgroups on every compute unit (five fit by LDS and registers),
+// wins or ties everywhere, because it puts the most workgroups on every compute unit (seven fit by LDS and registers),
 // and latency hiding across workgroups matters more at fp32 MFMA rates than the smaller tile's extra L2 traffic.
 // Narrow outputs (N <= 32) use 128x32 so that no MFMA block multiplies padding.
 template<int AMODE, int BMODE>
