@@ -299,6 +299,10 @@ GPU_CONV_CASES = CONV_CASES + [
     (1, 131, 127, 32, 20, 1, 1, 0, 0, 1, 1, 1, 1),  # pixel count not a multiple of 32
     (1, 128, 130, 192, 40, 1, 1, 0, 0, 1, 1, 1, 1), # longest reduction it takes, N tail
     (7, 64, 64, 64, 64, 3, 3, 1, 1, 1, 1, 1, 1),    # 448 tiles, 36 K steps: the two halves of K share a workgroup
+    # channel counts that are a multiple of the K step: the filter tap is kept in scalar registers
+    (2, 13, 11, 48, 40, 3, 5, 2, 4, 2, 1, 2, 3),    # dilation, padding wider than the filter's reach, stride along the height
+    (1, 7, 7, 32, 64, 5, 5, 2, 2, 1, 1, 1, 1),      # one tile, 50 K steps: K slices that begin in the middle of a tap
+    (3, 10, 10, 16, 24, 2, 2, 0, 0, 1, 1, 1, 1),    # a tap per K step
 ]
 
 
@@ -358,6 +362,8 @@ GPU_CONV_GRADIENT_CASES = CONV_CASES + [
     (1, 9, 9, 4, 8, 5, 5, 2, 2, 2, 2, 2, 2),        # dilation and stride share a factor: the masked form
     (1, 13, 13, 4, 8, 3, 3, 1, 1, 3, 3, 1, 1),      # stride 3: the masked form
     (1, 3, 3, 4, 8, 3, 3, 0, 0, 2, 2, 1, 1),        # a single window: classes without pixels of their own
+    (1, 13, 13, 4, 16, 3, 3, 1, 1, 3, 3, 1, 1),     # the masked form over 16 gradient channels: taps in scalar registers
+    (1, 9, 9, 4, 32, 5, 5, 2, 2, 2, 2, 2, 2),
     (8, 14, 14, 256, 512, 3, 3, 1, 1, 2, 2, 1, 1),  # few tiles per class, long reduction: K slices over a preset result
 ]
 
