@@ -460,6 +460,51 @@ def test_k_sliced_convolutions_are_bit_reproducible():
     assert np.array_equal(relu, np.maximum(first, 0)), "activation in the last slice's epilogue"
 
 
+def test_k_sliced_convolution_replays_from_a_captured_graph():
+    # A launch recorded into a HIP graph must not keep the address of the slices' scratch block (a later, larger launch
+    # frees it): under capture the slices meet in the result through atomic adds instead. The graph holds kernels only;
+    # it is replayed several times with eager launches of other sizes between the replays.
+    import ctypes
+    import torch
+    import neoml_amd
+    lib = neoml_amd.load()
+    g = rng(95)
+    n, hw, cin, cout = 4, 14, 256, 256
+    x = g.uniform(-1, 1, (n, hw, hw, cin)).astype(np.float32)
+    f = g.normal(0, 1.0 / np.sqrt(9 * cin), (cout, 3, 3, cin)).astype(np.float32)
+    b = g.uniform(-1, 1, cout).astype(np.float32)
+    want = orc.conv(x, f, b, 1, 1, 1, 1)
+    dev = torch.device("cuda:0")
+    dx, df, db = (torch.from_numpy(a).to(dev) for a in (x, f, b))
+    dy = torch.zeros((n, hw, hw, cout), device=dev)
+    d = neoml_amd.ConvDesc(n, hw, hw, cin, cout, 3, 3, 1, 1, 1, 1, 1, 1, 0, 0)
+    neoml_amd.check(lib.nhInitBlobConvolution(ctypes.byref(d)))
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def launch():
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        neoml_amd.check(lib.nhBlobConvolution(stream, ctypes.byref(d), P(dx), P(df), P(db), P(dy)))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    assert_close(dy.cpu().numpy(), want, "eager, slices meeting in scratch memory")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        launch()
+    for replay in range(3):
+        dy.zero_()
+        # eager work between the replays: a larger sliced convolution, which grows the scratch block
+        big = g.uniform(-1, 1, (8 + 8 * replay, hw, hw, cin)).astype(np.float32)
+        assert_close(hip().conv(big, f, b, 1, 1, 1, 1)[:1], orc.conv(big[:1], f, b, 1, 1, 1, 1), "eager between replays")
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_close(dy.cpu().numpy(), want, "replay %d" % replay)
+
+
 def test_convolution_ignores_pixels_outside_the_windows():
     # stride 4 with a 3-wide filter never touches image columns 3 and 7; whatever they hold (here: infinities)
     # must not leak into the result through the vector fetches that run past a window's last value
