@@ -954,11 +954,14 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 		setLastError( "matrix product: too many tiles" );
 		return NH_ERR_ARGUMENT;
 	}
-	// K slices: when the tiles alone leave most compute units with one or two workgroups, K is cut into slices that
-	// meet in scratch memory or, where that is not possible, in C through fp32 atomic adds. Seven workgroups fit a compute
-	// unit, five saturate it: the grid is planned in rounds of 1280 (measured: planning with 1792 is slower everywhere);
-	// the slice count is the one that wastes least of the last round of 1280, each extra slice priced at 2 %
-	// for its atomics, and every slice keeps at least 8 K steps.
+	// K slices: when the tiles alone leave most compute units with a few workgroups, K is cut into slices that meet in
+	// scratch memory or, where that is not possible, in C through fp32 atomic adds. Eight workgroups fit a compute unit.
+	// The slice count is picked by a small model of the launch, fitted to measurements of 3x3 convolutions and of matrix
+	// products: with w workgroups in all, the fullest compute unit runs n = ceil( w / 256 ) of them side by side when they
+	// all fit at once ( w <= 2048 ), each as long as its K steps plus about 8 steps for its prologue, epilogue and the
+	// meeting, and the matrix pipe is busy n / ( n + 1.7 ) of the time with n wavefronts per SIMD to pick from; beyond
+	// 2048 the compute units refill as workgroups end and the imbalance shrinks to about 0.6 of a workgroup.
+	// Every slice keeps at least 8 K steps.
 	// an empty reduction ( K == 0 ) still launches: one step of masked loads, C receives the free term or keeps its value
 	const int totalSteps = args.K > 0 ? ceilDiv( args.K, NH_KSTEP ) : 1;
 	int splits = 1;
@@ -968,12 +971,19 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 		const long long fill = blocks >= 1280 ? 1 : 1280 / blocks;
 		const long long most = totalSteps / 8 > 0 ? totalSteps / 8 : 1;
 		splits = static_cast<int>( fill < most ? fill : most );
-	// K slices cannot add a residual; an activation follows them as a pass of its own
+	// K slices cannot add a residual
 	} else if( blocks < 1024 && totalSteps >= 32 && args.Residual == nullptr ) {
 		double best = 0;
 		for( int s = 1; s <= 8 && s <= totalSteps / 8; ++s ) {
-			const double rounds = static_cast<double>( blocks * s ) / 1280.0;
-			const double cost = ceil( rounds ) / rounds * ( 1.0 + 0.02 * ( s - 1 ) );
+			const double perUnit = static_cast<double>( blocks * s ) / 256.0;
+			const double length = static_cast<double>( ceilDiv( totalSteps, s ) ) + 8.0;
+			double cost;
+			if( blocks * s <= 2048 ) {
+				const double sideBySide = ceil( perUnit );
+				cost = sideBySide * length * ( sideBySide + 1.7 ) / sideBySide;
+			} else {
+				cost = ( perUnit + 0.6 ) * length * ( 8.0 + 1.7 ) / 8.0;
+			}
 			if( s == 1 || cost < best ) {
 				best = cost;
 				splits = s;
