@@ -20,10 +20,10 @@ sys.path.insert(0, ROOT)
 FP32_MFMA_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBPS = 8000.0
 # Bytes crossing the L2 <-> fabric boundary per 3x3-convolution launch, mean over the 16 launches of one step at
-# batch 64, 224x224: rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a known-size copy gives) 67.7 MB + WRITE_SIZE (x1.0)
-# 42.1 MB; profiles/resnet18_b64_conv_hbm_traffic.txt holds the two runs. Counters cannot be read from inside this
+# batch 64, 224x224: rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a known-size copy gives) 81.0 MB + WRITE_SIZE (x1.0)
+# 43.4 MB; profiles/resnet18_b64_conv_hbm_traffic.txt holds the two runs. Counters cannot be read from inside this
 # process, so the figure is a constant of the default workload and null for any other.
-CONV3X3_TRAFFIC_BYTES_B64_224 = 109.9e6
+CONV3X3_TRAFFIC_BYTES_B64_224 = 124.4e6
 
 
 def cpu_baseline(batch_sample, image):

@@ -195,7 +195,14 @@ void matMulKernel( const CMatMulArgs launchArgs )
 	const __amdgpu_buffer_rsrc_t bufB = makeBuffer( B );
 
 	// ---- per-thread load slots ---------------------------------------------------------------------------
-	// K-major tile: slot -> ( row = slot / KQ, kq = slot % KQ ); X-major tile: slot -> ( k = slot / (BX/4), xq ).
+	// K-major tile: slot -> ( row = rowOfSlot( slot ), kq = slot % KQ ); X-major tile: slot -> ( k = slot / (BX/4), xq ).
+	// The rows of a K-major tile are dealt to the slots so that the two rows which eight consecutive lanes write with
+	// one 128-bit LDS store are four rows apart: at a pitch of 20 floats they then cover all 32 banks once ( rows next to
+	// each other share four banks, which doubles the time of every store ). Memory still sees 64 contiguous bytes per row.
+	auto rowOfSlot = []( int slot ) -> int {
+		const int q = slot / KQ;
+		return ( q & ~7 ) | ( ( q & 1 ) << 2 ) | ( ( q & 6 ) >> 1 );
+	};
 	// Vector path: offA / offB hold the byte offset of the slot for the K step that is loaded next.
 	unsigned offA[ASlots], offB[BSlots];
 	int convPixel[ASlots], convH0[ASlots], convW0[ASlots];
@@ -219,13 +226,13 @@ void matMulKernel( const CMatMulArgs launchArgs )
 		const int slot = tid + i * Threads;
 		const bool inTile = ATotal % Threads == 0 || slot < ATotal;
 		if( AMODE == AM_RowsK ) {
-			const int m = m0 + slot / KQ;
+			const int m = m0 + rowOfSlot( slot );
 			offA[i] = ( inTile && m < M ) ? static_cast<unsigned>( m * args.Lda + kStart + ( slot % KQ ) * 4 ) * 4u : OutOfRange;
 		} else if( AMODE == AM_RowsM ) {
 			const int m = m0 + ( slot % ( BM / 4 ) ) * 4;
 			offA[i] = ( inTile && m < M ) ? static_cast<unsigned>( ( kStart + slot / ( BM / 4 ) ) * args.Lda + m ) * 4u : OutOfRange;
 		} else {
-			const int m = m0 + slot / KQ;
+			const int m = m0 + rowOfSlot( slot );
 			if( inTile && m < M ) {
 				const int wo = m % args.Wo;
 				const int t = m / args.Wo;
@@ -312,7 +319,7 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			bImg[i] = static_cast<int>( t / args.Ho );
 			offB[i] = 0;
 		} else if( BMODE == BM_RowsK ) {
-			const int n = n0 + slot / KQ;
+			const int n = n0 + rowOfSlot( slot );
 			offB[i] = ( inTile && n < N ) ? static_cast<unsigned>( n * args.Ldb + kStart + ( slot % KQ ) * 4 ) * 4u : OutOfRange;
 		} else {
 			const int n = n0 + ( slot % ( BN / 4 ) ) * 4;
@@ -390,7 +397,7 @@ void matMulKernel( const CMatMulArgs launchArgs )
 #pragma unroll
 			for( int i = 0; i < BSlots; ++i ) {
 				const int slot = tid + i * Threads;
-				const int n = n0 + slot / KQ;
+				const int n = n0 + rowOfSlot( slot );
 				const bool nOk = ( BTotal % Threads == 0 || slot < BTotal ) && n < N && khIn;
 				const int index = n * args.Ldb + rowKh * args.RowK + rowR;
 				if( nOk && rowR + 3 < args.RowK ) {
@@ -512,7 +519,7 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			float4 v = make_float4( 0.f, 0.f, 0.f, 0.f );
 			if( ATotal % Threads == 0 || slot < ATotal ) {
 				if( AMODE == AM_RowsK ) {
-					const int m = m0 + slot / KQ;
+					const int m = m0 + rowOfSlot( slot );
 					const int k = kBase + ( slot % KQ ) * 4;
 					if( m < M ) {
 						const float* p = A + static_cast<long long>( m ) * args.Lda + k;
@@ -547,7 +554,7 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			float4 v = make_float4( 0.f, 0.f, 0.f, 0.f );
 			if( BTotal % Threads == 0 || slot < BTotal ) {
 				if( BMODE == BM_RowsK ) {
-					const int n = n0 + slot / KQ;
+					const int n = n0 + rowOfSlot( slot );
 					const int k = kBase + ( slot % KQ ) * 4;
 					if( n < N ) {
 						const float* p = B + static_cast<long long>( n ) * args.Ldb + k;
@@ -585,7 +592,7 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			const int slot = tid + i * Threads;
 			if( ATotal % Threads == 0 || slot < ATotal ) {
 				if( AK ) {
-					*reinterpret_cast<float4*>( &ldsA( buf )[( slot / KQ ) * LdsK + ( slot % KQ ) * 4] ) = regA[i];
+					*reinterpret_cast<float4*>( &ldsA( buf )[rowOfSlot( slot ) * LdsK + ( slot % KQ ) * 4] ) = regA[i];
 				} else {
 					*reinterpret_cast<float4*>( &ldsA( buf )[( slot / ( BM / 4 ) ) * APitchX + ( slot % ( BM / 4 ) ) * 4] ) = regA[i];
 				}
@@ -596,7 +603,7 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			const int slot = tid + i * Threads;
 			if( BTotal % Threads == 0 || slot < BTotal ) {
 				if( BK ) {
-					*reinterpret_cast<float4*>( &ldsB( buf )[( slot / KQ ) * LdsK + ( slot % KQ ) * 4] ) = regB[i];
+					*reinterpret_cast<float4*>( &ldsB( buf )[rowOfSlot( slot ) * LdsK + ( slot % KQ ) * 4] ) = regB[i];
 				} else {
 					*reinterpret_cast<float4*>( &ldsB( buf )[( slot / ( BN / 4 ) ) * BPitchX + ( slot % ( BN / 4 ) ) * 4] ) = regB[i];
 				}
