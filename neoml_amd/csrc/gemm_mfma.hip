@@ -847,7 +847,9 @@ void matMulKernel( const CMatMulArgs launchArgs )
 }
 
 // Scratch of the K slices that meet without atomics: partial tiles and arrival counters, one pair per stream (launches
-// of one stream run in order and may share it; two streams must not). Grown on demand, kept until the process ends.
+// of one stream run in order and may share it; two streams must not). Grown on demand by doubling; a block that has been
+// outgrown is NOT freed: another thread may be about to launch on the same stream with the address it was handed a
+// moment ago. All blocks live until the process ends (together at most twice the largest request).
 // The counters start at zero and every launch leaves them at zero.
 struct CSliceScratch {
 	float* Partials = nullptr;
@@ -865,8 +867,8 @@ static bool sliceScratch( hipStream_t stream, size_t partialFloats, size_t count
 		return false;
 	}
 	std::lock_guard<std::mutex> guard( lock );
-	// A recorded graph would keep the address of a block that a later, larger launch frees, and may replay on another
-	// stream: launches under capture take the atomic path.
+	// A recorded graph may replay on another stream, beside launches that use this stream's block: launches under
+	// capture take the atomic path.
 	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
 	if( hipStreamIsCapturing( stream, &capture ) != hipSuccess || capture != hipStreamCaptureStatusNone ) {
 		( void )hipGetLastError();
@@ -874,38 +876,27 @@ static bool sliceScratch( hipStream_t stream, size_t partialFloats, size_t count
 	}
 	CSliceScratch& scratch = byStream[std::make_pair( device, stream )];
 	if( scratch.PartialFloats < partialFloats ) {
-		// work that still reads the old block must finish first
-		if( hipStreamSynchronize( stream ) != hipSuccess ) {
-			return false;
-		}
-		if( scratch.Partials != nullptr ) {
-			( void )hipFree( scratch.Partials );
-			scratch.Partials = nullptr;
-			scratch.PartialFloats = 0;
-		}
-		const size_t grown = partialFloats + partialFloats / 4;
-		if( hipMalloc( reinterpret_cast<void**>( &scratch.Partials ), grown * sizeof( float ) ) != hipSuccess ) {
+		const size_t grown = partialFloats > 2 * scratch.PartialFloats ? partialFloats : 2 * scratch.PartialFloats;
+		float* block = nullptr;
+		if( hipMalloc( reinterpret_cast<void**>( &block ), grown * sizeof( float ) ) != hipSuccess ) {
 			( void )hipGetLastError();
 			return false;
 		}
+		scratch.Partials = block;
 		scratch.PartialFloats = grown;
 	}
 	if( scratch.CounterCount < counters ) {
-		if( hipStreamSynchronize( stream ) != hipSuccess ) {
-			return false;
-		}
-		if( scratch.Counters != nullptr ) {
-			( void )hipFree( scratch.Counters );
-			scratch.Counters = nullptr;
-			scratch.CounterCount = 0;
-		}
-		const size_t grown = counters * 2 > 4096 ? counters * 2 : 4096;
-		if( hipMalloc( reinterpret_cast<void**>( &scratch.Counters ), grown * sizeof( unsigned ) ) != hipSuccess
-			|| hipMemset( scratch.Counters, 0, grown * sizeof( unsigned ) ) != hipSuccess )
+		size_t grown = counters > 2 * scratch.CounterCount ? counters : 2 * scratch.CounterCount;
+		grown = grown > 4096 ? grown : 4096;
+		unsigned* block = nullptr;
+		// cleared on the launch stream, ahead of the launch that first uses it
+		if( hipMalloc( reinterpret_cast<void**>( &block ), grown * sizeof( unsigned ) ) != hipSuccess
+			|| hipMemsetAsync( block, 0, grown * sizeof( unsigned ), stream ) != hipSuccess )
 		{
 			( void )hipGetLastError();
 			return false;
 		}
+		scratch.Counters = block;
 		scratch.CounterCount = grown;
 	}
 	out = scratch;
