@@ -13,7 +13,7 @@
 //
 // Data path: operands are fetched with raw buffer loads (a 32-bit offset per lane that stays put, plus what a K step
 // adds in a scalar register; the memory unit's range check supplies the zeros of padding and of partial tiles),
-// parked in registers for one K step, written to one of two LDS buffers (20 KB per workgroup: seven workgroups
+// parked in registers for one K step, written to one of two LDS buffers (20 KB per workgroup: eight workgroups
 // per compute unit) and read back as MFMA operands. Within a wavefront the LDS reads
 // of the next group of 8 k are issued before the MFMAs of the current group, and the single barrier of a K step
 // sits before its last group, so the matrix pipe of a wavefront does not wait for LDS, barrier or memory in steady
@@ -680,7 +680,7 @@ void matMulKernel( const CMatMulArgs launchArgs )
 	// Buffer (ks+1)%2 was last read in step ks-1 BEFORE that step's barrier (the fragments of a step's last group are
 	// fetched ahead of the barrier, and a wave waits for its LDS reads before it enters the barrier; behind the barrier
 	// a wave only reads the other buffer), and a wave that stores at the top of step ks has passed that barrier: two
-	// buffers are enough, and the smaller footprint puts seven workgroups instead of five on a compute unit.
+	// buffers are enough, and the smaller footprint puts eight workgroups instead of five on a compute unit.
 	const int totalSteps = ( K + KS - 1 ) / KS;
 	const int kSteps = min( stepsPerSplit, totalSteps - split * stepsPerSplit );
 	constexpr int Groups = KS / 8;
@@ -1116,7 +1116,9 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 }
 
 // Picks the workgroup tile. Measured on MI355X (convolutions of 64..512 channels, GEMMs up to 8192^3): the 64x64 tile
-// wins or ties everywhere, because it puts the most workgroups on every compute unit (seven fit by LDS and registers),
+// wins or ties everywhere, because it puts the most workgroups on every compute unit (eight fit by LDS and registers; a 128x64 tile, five per compute unit with two
+// accumulators per wavefront, is 0-25 % slower on the shapes of the benchmarks and 2 % faster only on 256 -> 256 channels
+// over 65 536 pixels),
 // and latency hiding across workgroups matters more at fp32 MFMA rates than the smaller tile's extra L2 traffic.
 // Narrow outputs (N <= 32) use 128x32 so that no MFMA block multiplies padding.
 template<int AMODE, int BMODE>
