@@ -1003,7 +1003,7 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 	// whole tiles, from measurements of the 3x3 convolutions: a round filled to the fraction f takes 0.17 + 0.85 f of a
 	// full one (fewer workgroups per compute unit run faster, but not in proportion), a workgroup costs about 4 K steps
 	// beyond its own, and the preset of the tail rows about 2 K steps of a round.
-	const int slots = 256 * 5; // planned as above: the five that saturate a compute unit, not the seven that fit
+	const int slots = 256 * 5; // planned as above: the five that saturate a compute unit, not the eight that fit
 	long long gridX = tiles;
 	int tailRow = 0;
 	if( splits == 1 && !twoGroups && batch == 1 && AMODE != AM_ConvClasses && args.Residual == nullptr && tiles >= slots && totalSteps >= 16 ) {

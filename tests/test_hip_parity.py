@@ -387,6 +387,61 @@ def test_convolution_gradients(case):
     assert_close(hip().conv_learn_add(x, grad, start, ph, pw, sh, sw, dh, dw), want, "learn %s" % (case,), atol=1e-5 * scale)
 
 
+def _random_conv_case(g):
+    """A convolution whose result is not empty: channel counts drawn from the loader's three regimes (not a multiple of
+    4, a multiple of 4, a multiple of the K step), any filter, stride, dilation and padding up to beyond the filter."""
+    cin = int(g.choice([1, 3, 5, 4, 8, 12, 20, 16, 32, 48, 64]))
+    cout = int(g.choice([1, 7, 16, 33, 64, 70]))
+    fh, fw = int(g.integers(1, 6)), int(g.integers(1, 6))
+    dh, dw = int(g.integers(1, 4)), int(g.integers(1, 4))
+    sh, sw = int(g.integers(1, 4)), int(g.integers(1, 4))
+    ph, pw = int(g.integers(0, fh * dh + 1)), int(g.integers(0, fw * dw + 1))
+    h = int(g.integers(max(1, (fh - 1) * dh + 1 - 2 * ph), 20))
+    w = int(g.integers(max(1, (fw - 1) * dw + 1 - 2 * pw), 20))
+    n = int(g.integers(1, 5))
+    return n, h, w, cin, cout, fh, fw, ph, pw, sh, sw, dh, dw
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_convolution_and_gradients_on_random_shapes(seed):
+    g = rng(7000 + seed)
+    for _ in range(12):
+        case = _random_conv_case(g)
+        n, h, w, cin, cout, fh, fw, ph, pw, sh, sw, dh, dw = case
+        ho, wo = nhtest.conv_out(h, w, fh, fw, ph, pw, sh, sw, dh, dw)
+        x = g.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+        f = g.normal(0, 1.0 / np.sqrt(fh * fw * cin), (cout, fh, fw, cin)).astype(np.float32)
+        bias = g.uniform(-1, 1, cout).astype(np.float32)
+        grad = g.uniform(-1, 1, (n, ho, wo, cout)).astype(np.float32)
+        assert_close(hip().conv(x, f, bias, ph, pw, sh, sw, dh, dw), orc.conv(x, f, bias, ph, pw, sh, sw, dh, dw), "conv %s" % (case,))
+        assert_close(hip().conv_backward(grad, f, None, x.shape, ph, pw, sh, sw, dh, dw),
+                     orc.conv_backward(grad, f, None, x.shape, ph, pw, sh, sw, dh, dw), "backward %s" % (case,), atol=2e-5)
+        start = g.uniform(-1, 1, f.shape).astype(np.float32)
+        assert_close(hip().conv_learn_add(x, grad, start, ph, pw, sh, sw, dh, dw),
+                     orc.conv_learn_add(x, grad, start, ph, pw, sh, sw, dh, dw), "learn %s" % (case,), atol=1e-5 * np.sqrt(n * ho * wo))
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_matmul_on_random_shapes(seed):
+    # row strides with padding, reductions that are and are not multiples of the K step, long reductions over few
+    # tiles ( K slices ), all three operand orders
+    g = rng(7100 + seed)
+    for _ in range(10):
+        M, N = int(g.integers(1, 200)), int(g.integers(1, 200))
+        K = int(g.choice([1, 3, 16, 17, 64, 100, 512, 1000, 2048]))
+        pa, pb, pc = (int(v) for v in g.integers(0, 5, 3))
+        a = g.uniform(-1, 1, (M, K + pa)).astype(np.float32)
+        b = g.uniform(-1, 1, (N, K + pb)).astype(np.float32)
+        kw = dict(lda=K + pa, ldb=K + pb, ldc=N + pc, M=M, N=N, K=K)
+        tol = dict(atol=1e-5 * max(1.0, np.sqrt(K / 64.0)))
+        assert_close(hip().matmul("nt", a, b, **kw), orc.matmul("nt", a, b, **kw), "nt %s" % ((M, N, K, pa, pb, pc),), **tol)
+        at = g.uniform(-1, 1, (K, M + pa)).astype(np.float32)
+        bn = g.uniform(-1, 1, (K, N + pb)).astype(np.float32)
+        c0 = g.uniform(-1, 1, ((M - 1) * (N + pc) + N,)).astype(np.float32)
+        kw = dict(c=c0, lda=M + pa, ldb=N + pb, ldc=N + pc, M=M, N=N, K=K)
+        assert_close(hip().matmul("tn_add", at, bn, **kw), orc.matmul("tn_add", at, bn, **kw), "tn_add %s" % ((M, N, K),), **tol)
+
+
 def test_convolution_gradients_are_adjoints_at_full_size():
     # the single-layer configuration, batch 32: <conv(x, f), g> == <x, backward(g, f)> == <f, learn(x, g)>
     h = hip()
