@@ -560,6 +560,62 @@ def test_k_sliced_convolution_replays_from_a_captured_graph():
         assert_close(dy.cpu().numpy(), want, "replay %d" % replay)
 
 
+def test_k_sliced_convolutions_from_two_threads_on_one_stream():
+    # The engine interface is thread-safe: two threads may enqueue on the engine's one stream at the same time. K-sliced
+    # launches of one stream share a scratch block, which is replaced by larger ones while the other thread is launching
+    # (the stream is new, so its block starts empty); every result must still be the one a single thread gets, bit for
+    # bit: the slices are summed in a fixed order.
+    import ctypes
+    import threading
+    import torch
+    import neoml_amd
+    lib = neoml_amd.load()
+    g = rng(96)
+    dev = torch.device("cuda:0")
+    side = torch.cuda.Stream()
+    stream = ctypes.c_void_p(side.cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    cin = cout = 256
+    f = torch.from_numpy(g.normal(0, 1.0 / 48, (cout, 3, 3, cin)).astype(np.float32)).to(dev)
+    b = torch.from_numpy(g.uniform(-1, 1, cout).astype(np.float32)).to(dev)
+
+    def make(n):
+        x = torch.from_numpy(g.uniform(-1, 1, (n, 14, 14, cin)).astype(np.float32)).to(dev)
+        d = neoml_amd.ConvDesc(n, 14, 14, cin, cout, 3, 3, 1, 1, 1, 1, 1, 1, 0, 0)
+        neoml_amd.check(lib.nhInitBlobConvolution(ctypes.byref(d)))
+        return d, x, torch.zeros((n, 14, 14, cout), device=dev)
+
+    jobs = [[make(n) for n in sizes] for sizes in ((1, 3, 6, 12, 20), (2, 4, 8, 16, 24))]
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(thread_jobs):
+        try:
+            for _ in range(20):
+                for d, x, y in thread_jobs:
+                    neoml_amd.check(lib.nhBlobConvolution(stream, ctypes.byref(d), P(x), P(f), P(b), P(y)))
+        except Exception as e:  # reported by the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(tj,)) for tj in jobs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    side.synchronize()
+    assert not errors, errors
+    threaded = [[y.cpu().numpy().copy() for _, _, y in tj] for tj in jobs]
+    for thread_jobs, got in zip(jobs, threaded):
+        for (d, x, y), have in zip(thread_jobs, got):
+            y.zero_()
+            torch.cuda.synchronize()
+            neoml_amd.check(lib.nhBlobConvolution(stream, ctypes.byref(d), P(x), P(f), P(b), P(y)))
+            side.synchronize()
+            assert np.array_equal(y.cpu().numpy(), have)
+    d, x, _ = jobs[1][2]
+    assert_close(threaded[1][2], orc.conv(x.cpu().numpy(), f.cpu().numpy(), b.cpu().numpy(), 1, 1, 1, 1), "vs oracle")
+
+
 def test_convolution_ignores_pixels_outside_the_windows():
     # stride 4 with a 3-wide filter never touches image columns 3 and 7; whatever they hold (here: infinities)
     # must not leak into the result through the vector fetches that run past a window's last value
