@@ -78,6 +78,7 @@ struct CMatMulArgs {
 	// convolution geometry (AM_Conv only): A is the image, M = batch * Ho * Wo
 	int H, W, Cin, Ho, Wo, Fh, Fw, PadH, PadW, StrideH, StrideW, DilH, DilW;
 	int RowK, RowPitch; // AM_ConvRows: Fw * Cin and its round-up to a multiple of 4; K = Fh * RowPitch
+	int AFloats, BFloats; // AM_ConvRows: sizes of the image and of the filter, the limit of a 128-bit load that reads past a run
 	// AM_Conv as the gradient by the input of a strided convolution: the tap's source coordinate is
 	// ( ho * StrideH - PadH + kh * DilH ) / UpH and only exists where that division is exact (values <= 1: no division)
 	int UpH, UpW;
@@ -376,19 +377,30 @@ void matMulKernel( const CMatMulArgs launchArgs )
 		if constexpr( IsConvRows ) {
 			const int rowFloats = args.W * args.Cin;
 			const bool khIn = rowKh < args.Fh;
+			// A run that ends inside these four values ( the last values of a filter row, the right edge of the image ) is
+			// still fetched with one 128-bit load, as long as the load stays inside the tensor, and the values beyond the
+			// run's end are replaced by zeros: what lies there is the next pixels, not padding. Only a run that BEGINS inside
+			// the four values ( the left edge ) or touches the tensor's end is fetched value by value.
+			const int leftInRow = args.RowK - rowR; // values of the filter row from this lane's k on; <= 0 in the padding of K
+			auto maskTail = []( float4 v, int valid ) -> float4 {
+				return make_float4( v.x, valid > 1 ? v.y : 0.f, valid > 2 ? v.z : 0.f, valid > 3 ? v.w : 0.f );
+			};
 #pragma unroll
 			for( int i = 0; i < ASlots; ++i ) {
 				const int hi = convH0[i] + rowKh * args.DilH;
 				const bool rowOk = khIn && hi >= 0 && hi < args.H;
 				const int col = convW0[i] + rowR; // position inside the image row, in floats; negative in the left padding
 				const int index = convPixel[i] + hi * rowFloats + col;
-				if( rowOk && rowR + 3 < args.RowK && col >= 0 && col + 3 < rowFloats ) {
-					regA[i] = bufferLoad4( bufA, static_cast<unsigned>( index ) * 4u );
+				const int valid = min( leftInRow, rowFloats - col );
+				if( !rowOk || valid <= 0 || col <= -4 ) {
+					regA[i] = make_float4( 0.f, 0.f, 0.f, 0.f );
+				} else if( col >= 0 && index + 3 < args.AFloats ) {
+					regA[i] = maskTail( bufferLoad4( bufA, static_cast<unsigned>( index ) * 4u ), valid );
 				} else {
 					float v[4];
 #pragma unroll
 					for( int e = 0; e < 4; ++e ) {
-						const bool ok = rowOk && rowR + e < args.RowK && col + e >= 0 && col + e < rowFloats;
+						const bool ok = e < valid && col + e >= 0;
 						v[e] = bufferLoad1( bufA, ok ? static_cast<unsigned>( index + e ) * 4u : OutOfRange );
 					}
 					regA[i] = make_float4( v[0], v[1], v[2], v[3] );
@@ -400,13 +412,15 @@ void matMulKernel( const CMatMulArgs launchArgs )
 				const int n = n0 + rowOfSlot( slot );
 				const bool nOk = ( BTotal % Threads == 0 || slot < BTotal ) && n < N && khIn;
 				const int index = n * args.Ldb + rowKh * args.RowK + rowR;
-				if( nOk && rowR + 3 < args.RowK ) {
-					regB[i] = bufferLoad4( bufB, static_cast<unsigned>( index ) * 4u );
+				if( !nOk || leftInRow <= 0 ) {
+					regB[i] = make_float4( 0.f, 0.f, 0.f, 0.f );
+				} else if( index + 3 < args.BFloats ) {
+					regB[i] = maskTail( bufferLoad4( bufB, static_cast<unsigned>( index ) * 4u ), leftInRow );
 				} else {
 					float v[4];
 #pragma unroll
 					for( int e = 0; e < 4; ++e ) {
-						v[e] = bufferLoad1( bufB, nOk && rowR + e < args.RowK ? static_cast<unsigned>( index + e ) * 4u : OutOfRange );
+						v[e] = bufferLoad1( bufB, e < leftInRow ? static_cast<unsigned>( index + e ) * 4u : OutOfRange );
 					}
 					regB[i] = make_float4( v[0], v[1], v[2], v[3] );
 				}
@@ -1434,6 +1448,8 @@ int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* sour
 	{
 		args.RowK = d.filterWidth * d.channels;
 		args.RowPitch = ( args.RowK + 3 ) / 4 * 4;
+		args.AFloats = d.batch * d.height * d.width * d.channels;
+		args.BFloats = d.filterCount * d.filterHeight * args.RowK;
 		args.K = d.filterHeight * args.RowPitch; // reduction length as the kernel walks it; Ldb keeps the filter's own
 		return launchMatMul<AM_ConvRows, BM_RowsK>( stream, args, 1, true );
 	}
