@@ -978,24 +978,31 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 	const int totalSteps = args.K > 0 ? ceilDiv( args.K, NH_KSTEP ) : 1;
 	int splits = 1;
 	const long long blocks = tiles * batch;
+	auto launchCost = [&]( int slices ) -> double {
+		const double perUnit = static_cast<double>( blocks * slices ) / 256.0;
+		const double length = static_cast<double>( ceilDiv( totalSteps, slices ) ) + 8.0;
+		if( blocks * slices <= 2048 ) {
+			const double sideBySide = ceil( perUnit );
+			return sideBySide * length * ( sideBySide + 1.7 ) / sideBySide;
+		}
+		return ( perUnit + 0.6 ) * length * ( 8.0 + 1.7 ) / 8.0;
+	};
 	if( args.ManySlices != 0 ) {
-		// a gradient by a filter: a few tiles, a reduction over every pixel of the batch
-		const long long fill = blocks >= 1280 ? 1 : 1280 / blocks;
-		const long long most = totalSteps / 8 > 0 ? totalSteps / 8 : 1;
-		splits = static_cast<int>( fill < most ? fill : most );
+		// a gradient by a filter: a few tiles, a reduction over every pixel of the batch, up to hundreds of slices
+		const int most = totalSteps / 8 > 0 ? totalSteps / 8 : 1;
+		double best = 0;
+		for( int s = 1; s <= most && ( s == 1 || blocks * s <= 4096 ); ++s ) {
+			const double cost = launchCost( s );
+			if( s == 1 || cost < best ) {
+				best = cost;
+				splits = s;
+			}
+		}
 	// K slices cannot add a residual
 	} else if( blocks < 1024 && totalSteps >= 32 && args.Residual == nullptr ) {
 		double best = 0;
 		for( int s = 1; s <= 8 && s <= totalSteps / 8; ++s ) {
-			const double perUnit = static_cast<double>( blocks * s ) / 256.0;
-			const double length = static_cast<double>( ceilDiv( totalSteps, s ) ) + 8.0;
-			double cost;
-			if( blocks * s <= 2048 ) {
-				const double sideBySide = ceil( perUnit );
-				cost = sideBySide * length * ( sideBySide + 1.7 ) / sideBySide;
-			} else {
-				cost = ( perUnit + 0.6 ) * length * ( 8.0 + 1.7 ) / 8.0;
-			}
+			const double cost = launchCost( s );
 			if( s == 1 || cost < best ) {
 				best = cost;
 				splits = s;
