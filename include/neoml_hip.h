@@ -14,7 +14,7 @@
  *   - return value: NH_OK or an NH_ERR_* code; nhGetLastError() gives the message for the calling thread
  *   - in-place use (result aliasing an input exactly) is allowed wherever the reference allows it
  *   - convolutions and matrix products with few output tiles cut their reduction into slices that meet in a scratch
- *     block which the library allocates per (device, stream) on first need and keeps until the process ends; their
+ *     block which the library allocates per (device, stream) on first need and keeps until nhStreamDestroy; their
  *     results do not depend on timing. Calls on one stream may come from several threads; do not share the block
  *     across streams by replaying a captured graph elsewhere: while a stream is being captured these calls neither
  *     allocate nor use the block (the slices then meet through fp32 atomic adds, reproducible to rounding) and

@@ -14,6 +14,10 @@ void setLastError( const char* fmt, ... );
 
 inline hipStream_t toStream( nhStream s ) { return reinterpret_cast<hipStream_t>( s ); }
 
+// Frees the scratch blocks that sliced reductions keep for a stream of the current device ( gemm_mfma.hip ); the stream
+// must have been drained. Called when the stream is destroyed.
+void releaseSliceScratch( hipStream_t stream );
+
 constexpr int WaveSize = 64;
 
 inline int ceilDiv( long long a, long long b ) { return static_cast<int>( ( a + b - 1 ) / b ); }

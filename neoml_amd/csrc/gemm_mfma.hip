@@ -34,6 +34,7 @@
 #include <map>
 #include <mutex>
 #include <utility>
+#include <vector>
 
 namespace nh {
 
@@ -862,25 +863,52 @@ void matMulKernel( const CMatMulArgs launchArgs )
 
 // Scratch of the K slices that meet without atomics: partial tiles and arrival counters, one pair per stream (launches
 // of one stream run in order and may share it; two streams must not). Grown on demand by doubling; a block that has been
-// outgrown is NOT freed: another thread may be about to launch on the same stream with the address it was handed a
-// moment ago. All blocks live until the process ends (together at most twice the largest request).
+// outgrown is NOT freed while the stream lives: another thread may be about to launch on the same stream with the address
+// it was handed a moment ago. All blocks of a stream (together at most twice the largest request) are freed when the
+// stream is destroyed through nhStreamDestroy, those of other streams live until the process ends.
 // The counters start at zero and every launch leaves them at zero.
 struct CSliceScratch {
 	float* Partials = nullptr;
 	size_t PartialFloats = 0;
 	unsigned* Counters = nullptr;
 	size_t CounterCount = 0;
+	std::vector<void*> Blocks; // every allocation made for the stream
 };
+
+static std::mutex sliceScratchLock;
+static std::map<std::pair<int, hipStream_t>, CSliceScratch>& sliceScratchByStream()
+{
+	static std::map<std::pair<int, hipStream_t>, CSliceScratch> byStream;
+	return byStream;
+}
+
+void releaseSliceScratch( hipStream_t stream )
+{
+	int device = 0;
+	if( hipGetDevice( &device ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return;
+	}
+	std::lock_guard<std::mutex> guard( sliceScratchLock );
+	auto& byStream = sliceScratchByStream();
+	auto found = byStream.find( std::make_pair( device, stream ) );
+	if( found == byStream.end() ) {
+		return;
+	}
+	for( void* block : found->second.Blocks ) {
+		( void )hipFree( block );
+	}
+	byStream.erase( found );
+}
 
 static bool sliceScratch( hipStream_t stream, size_t partialFloats, size_t counters, CSliceScratch& out )
 {
-	static std::mutex lock;
-	static std::map<std::pair<int, hipStream_t>, CSliceScratch> byStream;
 	int device = 0;
 	if( hipGetDevice( &device ) != hipSuccess ) {
 		return false;
 	}
-	std::lock_guard<std::mutex> guard( lock );
+	std::lock_guard<std::mutex> guard( sliceScratchLock );
+	auto& byStream = sliceScratchByStream();
 	// A recorded graph may replay on another stream, beside launches that use this stream's block: launches under
 	// capture take the atomic path.
 	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
@@ -896,6 +924,7 @@ static bool sliceScratch( hipStream_t stream, size_t partialFloats, size_t count
 			( void )hipGetLastError();
 			return false;
 		}
+		scratch.Blocks.push_back( block );
 		scratch.Partials = block;
 		scratch.PartialFloats = grown;
 	}
@@ -904,16 +933,20 @@ static bool sliceScratch( hipStream_t stream, size_t partialFloats, size_t count
 		grown = grown > 4096 ? grown : 4096;
 		unsigned* block = nullptr;
 		// cleared on the launch stream, ahead of the launch that first uses it
-		if( hipMalloc( reinterpret_cast<void**>( &block ), grown * sizeof( unsigned ) ) != hipSuccess
-			|| hipMemsetAsync( block, 0, grown * sizeof( unsigned ), stream ) != hipSuccess )
-		{
+		if( hipMalloc( reinterpret_cast<void**>( &block ), grown * sizeof( unsigned ) ) != hipSuccess ) {
+			( void )hipGetLastError();
+			return false;
+		}
+		scratch.Blocks.push_back( block );
+		if( hipMemsetAsync( block, 0, grown * sizeof( unsigned ), stream ) != hipSuccess ) {
 			( void )hipGetLastError();
 			return false;
 		}
 		scratch.Counters = block;
 		scratch.CounterCount = grown;
 	}
-	out = scratch;
+	out.Partials = scratch.Partials;
+	out.Counters = scratch.Counters;
 	return true;
 }
 

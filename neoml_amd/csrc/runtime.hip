@@ -87,6 +87,9 @@ int nhStreamCreate( nhStream* stream )
 int nhStreamDestroy( nhStream stream )
 {
 	if( stream != nullptr ) {
+		// what the library keeps for the stream goes with it ( a later stream may be handed the same handle )
+		NH_HIP( hipStreamSynchronize( toStream( stream ) ) );
+		releaseSliceScratch( toStream( stream ) );
 		NH_HIP( hipStreamDestroy( toStream( stream ) ) );
 	}
 	return NH_OK;

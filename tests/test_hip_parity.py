@@ -616,6 +616,40 @@ def test_k_sliced_convolutions_from_two_threads_on_one_stream():
     assert_close(threaded[1][2], orc.conv(x.cpu().numpy(), f.cpu().numpy(), b.cpu().numpy(), 1, 1, 1, 1), "vs oracle")
 
 
+def test_stream_destroy_frees_the_slices_scratch():
+    # an application that makes an engine (= a stream) per request must not pile up scratch blocks
+    import ctypes
+    import torch
+    import neoml_amd
+    lib = neoml_amd.load()
+    g = rng(97)
+    dev = torch.device("cuda:0")
+    n, hw, cin, cout = 16, 14, 256, 256   # 3 slices x 392 tiles x 16 KB = 19 MB of partial tiles
+    x = torch.from_numpy(g.uniform(-1, 1, (n, hw, hw, cin)).astype(np.float32)).to(dev)
+    f = torch.from_numpy(g.normal(0, 1.0 / 48, (cout, 3, 3, cin)).astype(np.float32)).to(dev)
+    y = torch.zeros((n, hw, hw, cout), device=dev)
+    d = neoml_amd.ConvDesc(n, hw, hw, cin, cout, 3, 3, 1, 1, 1, 1, 1, 1, 0, 0)
+    neoml_amd.check(lib.nhInitBlobConvolution(ctypes.byref(d)))
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    torch.cuda.synchronize()
+
+    def once():
+        stream = ctypes.c_void_p()
+        neoml_amd.check(lib.nhStreamCreate(ctypes.byref(stream)))
+        neoml_amd.check(lib.nhBlobConvolution(stream, ctypes.byref(d), P(x), P(f), None, P(y)))
+        neoml_amd.check(lib.nhStreamSynchronize(stream))
+        neoml_amd.check(lib.nhStreamDestroy(stream))
+        return y.cpu().numpy().copy()
+
+    first = once()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(12):
+        assert np.array_equal(once(), first)
+    free_after = torch.cuda.mem_get_info()[0]
+    assert free_before - free_after < 32 * 1024 * 1024, (free_before, free_after)  # 12 leaked blocks would be 230 MB
+    assert_close(first[:1], orc.conv(x[:1].cpu().numpy(), f.cpu().numpy(), None, 1, 1, 1, 1), "vs oracle")
+
+
 def test_convolution_ignores_pixels_outside_the_windows():
     # stride 4 with a 3-wide filter never touches image columns 3 and 7; whatever they hold (here: infinities)
     # must not leak into the result through the vector fetches that run past a window's last value
