@@ -308,11 +308,20 @@ void matMulKernel( const CMatMulArgs launchArgs )
 		if( BMODE == BM_ConvN ) {
 			const int n = n0 + ( slot % ( BN / 4 ) ) * 4;
 			const bool nOk = inTile && n < N;
-			const int tap = n / args.Cin;
-			bCi[i] = n - tap * args.Cin;
-			const int kh = tap / args.Fw;
-			bDh[i] = nOk ? kh * args.DilH - args.PadH : -0x40000000; // never inside the image
-			bDw[i] = ( tap - kh * args.Fw ) * args.DilW - args.PadW;
+			if( args.RowPitch > 0 ) {
+				// channel counts that are not a multiple of 4: column n = kh * RowPitch + r, r = position inside the run of
+				// Fw * Cin values that a filter row meets in an image row ( r >= RowK: padding of the run, dropped on output )
+				const int kh = n / args.RowPitch;
+				bCi[i] = n - kh * args.RowPitch;
+				bDh[i] = nOk ? kh * args.DilH - args.PadH : -0x40000000; // never inside the image
+				bDw[i] = bCi[i] - args.PadW * args.Cin; // in floats, from the image row's position of the output column
+			} else {
+				const int tap = n / args.Cin;
+				bCi[i] = n - tap * args.Cin;
+				const int kh = tap / args.Fw;
+				bDh[i] = nOk ? kh * args.DilH - args.PadH : -0x40000000; // never inside the image
+				bDw[i] = ( tap - kh * args.Fw ) * args.DilW - args.PadW;
+			}
 			const long long pixel = static_cast<long long>( kStart ) + slot / ( BN / 4 );
 			bPixel[i] = pixel;
 			bWo[i] = static_cast<int>( pixel % args.Wo );
@@ -460,6 +469,29 @@ void matMulKernel( const CMatMulArgs launchArgs )
 #pragma unroll
 				for( int i = 0; i < BSlots; ++i ) {
 					const int hi = bHo[i] * args.StrideH + bDh[i];
+					if( args.RowPitch > 0 ) {
+						// four values of a filter row's run in the image row: one 128-bit load at 4-byte alignment whose
+						// values beyond the run's end or the row's end are replaced by zeros; element-wise only where the
+						// run begins inside the four ( left edge ) or the load would leave the tensor
+						const int rowFloats = args.W * args.Cin;
+						const int col = bWo[i] * args.StrideW * args.Cin + bDw[i];
+						const bool rowOk = bPixel[i] < K && hi >= 0 && hi < args.H;
+						const int valid = min( args.RowK - bCi[i], rowFloats - col );
+						const int index = ( bImg[i] * args.H + hi ) * rowFloats + col;
+						if( !rowOk || valid <= 0 || col <= -4 ) {
+							regB[i] = make_float4( 0.f, 0.f, 0.f, 0.f );
+						} else if( col >= 0 && index + 3 < args.BFloats ) {
+							const float4 v = bufferLoad4( bufB, static_cast<unsigned>( index ) * 4u );
+							regB[i] = make_float4( v.x, valid > 1 ? v.y : 0.f, valid > 2 ? v.z : 0.f, valid > 3 ? v.w : 0.f );
+						} else {
+							float v[4];
+#pragma unroll
+							for( int e = 0; e < 4; ++e ) {
+								v[e] = bufferLoad1( bufB, ( e < valid && col + e >= 0 ) ? static_cast<unsigned>( index + e ) * 4u : OutOfRange );
+							}
+							regB[i] = make_float4( v[0], v[1], v[2], v[3] );
+						}
+					}
 					const int wi = bWo[i] * args.StrideW + bDw[i];
 					const bool ok = bPixel[i] < K && hi >= 0 && hi < args.H && wi >= 0 && wi < args.W;
 					const unsigned off = ok ? static_cast<unsigned>( ( ( bImg[i] * args.H + hi ) * args.W + wi ) * args.Cin + bCi[i] ) * 4u : OutOfRange;
@@ -473,7 +505,9 @@ void matMulKernel( const CMatMulArgs launchArgs )
 							++bImg[i];
 						}
 					}
-					regB[i] = bufferLoad4( bufB, off );
+					if( args.RowPitch <= 0 ) {
+						regB[i] = bufferLoad4( bufB, off );
+					}
 				}
 			} else if( !partialStep ) {
 #pragma unroll
@@ -821,9 +855,18 @@ void matMulKernel( const CMatMulArgs launchArgs )
 
 #pragma unroll
 	for( int ni = 0; ni < NI; ++ni ) {
-		const int n = n0 + waveN * WN + ni * 32 + l32;
+		int n = n0 + waveN * WN + ni * 32 + l32;
 		if( n >= N ) {
 			continue;
+		}
+		if( BMODE == BM_ConvN && args.RowPitch > 0 ) {
+			// the padded runs of the columns close up: ( kh, r ) -> kh * RowK + r
+			const int kh = n / args.RowPitch;
+			const int r = n - kh * args.RowPitch;
+			if( r >= args.RowK ) {
+				continue;
+			}
+			n = kh * args.RowK + r;
 		}
 		const float bias = ( args.Bias != nullptr ) ? args.Bias[n] : 0.f;
 #pragma unroll
@@ -1668,9 +1711,18 @@ int convLearnAdd( hipStream_t stream, const nhConvDesc& d, const float* input, c
 	if( args.M == 0 || args.N == 0 || args.K == 0 ) {
 		return NH_OK;
 	}
-	const bool vec = isAligned16( outputDiff ) && isAligned16( input ) && d.filterCount % 4 == 0 && d.channels % 4 == 0
+	const bool fits = isAligned16( outputDiff ) && d.filterCount % 4 == 0
 		&& fitsBuffer( pixels, d.filterCount, d.filterCount )
 		&& fitsBuffer( 1, 0, static_cast<long long>( d.batch ) * d.height * d.width * d.channels );
+	bool vec = fits && isAligned16( input ) && d.channels % 4 == 0;
+	if( fits && d.channels % 4 != 0 && d.dilationWidth == 1 ) {
+		// grey and RGB inputs: the columns walk each filter row's run of Fw * Cin image values, padded to a multiple of 4
+		args.RowK = d.filterWidth * d.channels;
+		args.RowPitch = ( args.RowK + 3 ) / 4 * 4;
+		args.BFloats = d.batch * d.height * d.width * d.channels;
+		args.N = d.filterHeight * args.RowPitch; // Ldc keeps the filter's own row length
+		vec = true;
+	}
 	return launchMatMul<AM_RowsM, BM_ConvN>( stream, args, 1, vec );
 }
 
