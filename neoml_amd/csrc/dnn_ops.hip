@@ -275,49 +275,79 @@ void poolingKernel( const nhPoolingDesc d, const float* source, float* result, i
 //   - the row stored for the winning column is looked up in the row-index buffer at the column's position
 //     RELATIVE to the window ( columnIndex * channels + c ), i.e. it is the arg-max row of image column
 //     `columnIndex` of the same strip, not of column `wo * stride + columnIndex`.
+// VECW channels per thread ( 4: 128-bit loads and stores when the channel count allows ).
+template<int VECW>
 __global__ __launch_bounds__( 256 )
 void maxPoolingIndexKernel( const nhPoolingDesc d, const float* source, int* maxIndices, float* result, long long total )
 {
 	const long long step = static_cast<long long>( gridDim.x ) * 256;
 	const int rowSize = d.width * d.channels;
+	const int channelGroups = d.channels / VECW;
+	auto load = []( const float* p, float ( &v )[VECW] ) {
+		if( VECW == 4 ) {
+			const float4 q = *reinterpret_cast<const float4*>( p );
+			v[0] = q.x; v[1 % VECW] = q.y; v[2 % VECW] = q.z; v[3 % VECW] = q.w;
+		} else {
+			v[0] = *p;
+		}
+	};
 	for( long long item = blockIdx.x * 256LL + threadIdx.x; item < total; item += step ) {
 		long long t = item;
-		const int c = static_cast<int>( t % d.channels ); t /= d.channels;
+		const int c = static_cast<int>( t % channelGroups ) * VECW; t /= channelGroups;
 		const int wo = static_cast<int>( t % d.resultWidth ); t /= d.resultWidth;
 		const int ho = static_cast<int>( t % d.resultHeight ); t /= d.resultHeight;
 		const long long n = t;
 		const int stripRow = ho * d.strideHeight;
 		const float* strip = source + ( n * d.height + stripRow ) * rowSize;
 		const int windowColumn = wo * d.strideWidth * d.channels;
-		float best = 0.f;
-		int bestCol = 0;
+		float best[VECW];
+		int bestCol[VECW];
 		for( int kw = 0; kw < d.filterWidth; ++kw ) {
 			const float* p = strip + windowColumn + kw * d.channels + c;
-			float col = *p;
+			float col[VECW];
+			load( p, col );
 			for( int kh = 1; kh < d.filterHeight; ++kh ) {
-				const float v = p[static_cast<long long>( kh ) * rowSize];
-				if( v > col ) {
-					col = v;
+				float v[VECW];
+				load( p + static_cast<long long>( kh ) * rowSize, v );
+#pragma unroll
+				for( int e = 0; e < VECW; ++e ) {
+					if( v[e] > col[e] ) {
+						col[e] = v[e];
+					}
 				}
 			}
-			if( kw == 0 || col > best ) {
-				best = col;
-				bestCol = kw;
+#pragma unroll
+			for( int e = 0; e < VECW; ++e ) {
+				if( kw == 0 || col[e] > best[e] ) {
+					best[e] = col[e];
+					bestCol[e] = kw;
+				}
 			}
 		}
-		const int windowIndex = bestCol * d.channels + c;
-		const float* q = strip + windowIndex;
-		float rowBest = *q;
-		int rowIdx = 0;
-		for( int kh = 1; kh < d.filterHeight; ++kh ) {
-			const float v = q[static_cast<long long>( kh ) * rowSize];
-			if( v > rowBest ) {
-				rowBest = v;
-				rowIdx = kh;
+		int index[VECW];
+#pragma unroll
+		for( int e = 0; e < VECW; ++e ) {
+			const int windowIndex = bestCol[e] * d.channels + c + e;
+			const float* q = strip + windowIndex;
+			float rowBest = *q;
+			int rowIdx = 0;
+			for( int kh = 1; kh < d.filterHeight; ++kh ) {
+				const float v = q[static_cast<long long>( kh ) * rowSize];
+				if( v > rowBest ) {
+					rowBest = v;
+					rowIdx = kh;
+				}
 			}
+			index[e] = ( stripRow + rowIdx ) * rowSize + windowColumn + windowIndex;
 		}
-		result[item] = best;
-		maxIndices[item] = ( stripRow + rowIdx ) * rowSize + windowColumn + windowIndex;
+		const long long out = item * VECW;
+		if( VECW == 4 ) {
+			*reinterpret_cast<float4*>( result + out ) = make_float4( best[0], best[1 % VECW], best[2 % VECW], best[3 % VECW] );
+			*reinterpret_cast<int4*>( maxIndices + out ) = make_int4( index[0], index[1 % VECW], index[2 % VECW], index[3 % VECW] );
+		} else {
+			result[out] = best[0];
+			maxIndices[out] = index[0];
+		}
 	}
 }
 
@@ -1562,10 +1592,17 @@ int nhBlobMaxPooling( nhStream s, const nhPoolingDesc* d, const float* source, i
 	if( total == 0 ) {
 		return NH_OK;
 	}
-	long long blocks = ( total + 255 ) / 256;
+	const bool vec = d->channels % 4 == 0 && isAligned16( source ) && isAligned16( result ) && isAligned16( maxIndices );
+	const long long items = vec ? total / 4 : total;
+	long long blocks = ( items + 255 ) / 256;
 	blocks = blocks > 1048576 ? 1048576 : blocks;
-	hipLaunchKernelGGL( maxPoolingIndexKernel, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
-		*d, source, maxIndices, result, total );
+	if( vec ) {
+		hipLaunchKernelGGL( maxPoolingIndexKernel<4>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			*d, source, maxIndices, result, items );
+	} else {
+		hipLaunchKernelGGL( maxPoolingIndexKernel<1>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			*d, source, maxIndices, result, items );
+	}
 	NH_LAUNCH_CHECK();
 	return NH_OK;
 }
