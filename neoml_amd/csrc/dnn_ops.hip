@@ -106,7 +106,7 @@ void channelwiseConvKernel( const nhConvDesc d, const float* source, const float
 template<int STRIDE, int WPT>
 __global__ __launch_bounds__( 256 )
 void channelwiseConv3x3Kernel( const nhConvDesc d, const float* source, const float* filter, const float* freeTerm,
-	float* result, int wGroups, int rowChunks, int rowsPerItem, int totalItems, const CFusedActivation act )
+	float* result, int wGroups, int rowChunks, int rowsPerItem, int totalItems, const CFusedActivation act, int flipTaps )
 {
 	constexpr int NC = ( WPT - 1 ) * STRIDE + 3;
 	constexpr int Keep = 3 - STRIDE; // input rows shared by two consecutive output rows
@@ -135,7 +135,8 @@ void channelwiseConv3x3Kernel( const nhConvDesc d, const float* source, const fl
 	float4 f[9];
 #pragma unroll
 	for( int k = 0; k < 9; ++k ) {
-		f[k] = *reinterpret_cast<const float4*>( filter + k * d.channels + c );
+		// flipTaps: the filter turned by 180 degrees, which makes this kernel the gradient by the input of the stride-1 case
+		f[k] = *reinterpret_cast<const float4*>( filter + ( flipTaps != 0 ? 8 - k : k ) * d.channels + c );
 	}
 	const float4 bias = freeTerm != nullptr ? *reinterpret_cast<const float4*>( freeTerm + c ) : make_float4( 0.f, 0.f, 0.f, 0.f );
 
@@ -1461,7 +1462,7 @@ static int poolingImpl( nhStream s, const nhPoolingDesc* d, const float* source,
 
 template<int STRIDE, int WPT>
 static int channelwise3x3Impl( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
-	const float* freeTerm, float* result, const CFusedActivation& act )
+	const float* freeTerm, float* result, const CFusedActivation& act, bool flipTaps = false )
 {
 	const int wGroups = ceilDiv( d->resultWidth, WPT );
 	const long long perRow = static_cast<long long>( d->batch ) * wGroups * ( d->channels / 4 );
@@ -1469,7 +1470,8 @@ static int channelwise3x3Impl( nhStream s, const nhConvDesc* d, const float* sou
 	chooseRowChunks( perRow, d->resultHeight, 4, 3072, &rowChunks, &rowsPerItem );
 	const long long items = perRow * rowChunks;
 	hipLaunchKernelGGL( ( channelwiseConv3x3Kernel<STRIDE, WPT> ), dim3( static_cast<unsigned>( ( items + 255 ) / 256 ) ), dim3( 256 ), 0,
-		toStream( s ), *d, source, filter, freeTerm, result, wGroups, rowChunks, rowsPerItem, static_cast<int>( items ), act );
+		toStream( s ), *d, source, filter, freeTerm, result, wGroups, rowChunks, rowsPerItem, static_cast<int>( items ), act,
+		flipTaps ? 1 : 0 );
 	NH_LAUNCH_CHECK();
 	return NH_OK;
 }
@@ -1652,6 +1654,23 @@ int nhBlobChannelwiseConvolutionBackward( nhStream s, const nhConvDesc* d, const
 		return NH_OK;
 	}
 	const bool vec = d->channels % 4 == 0 && isAligned16( outputDiff ) && isAligned16( filter ) && isAligned16( inputDiff );
+	if( vec && d->filterHeight == 3 && d->filterWidth == 3 && d->strideHeight == 1 && d->strideWidth == 1
+		&& d->dilationHeight == 1 && d->dilationWidth == 1 && d->paddingHeight <= 2 && d->paddingWidth <= 2
+		&& static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * d->channels * 4 < 0x7fffffffLL
+		&& static_cast<long long>( d->batch ) * d->height * d->width * d->channels < 0x7fffffffLL )
+	{
+		// Stride 1: the gradient by the input is the depthwise convolution of the output gradient with the filter turned
+		// by 180 degrees and padding 2 - p: the forward pass's strip kernel ( every row of the gradient read once per strip ).
+		nhConvDesc turned = *d;
+		turned.height = d->resultHeight;
+		turned.width = d->resultWidth;
+		turned.paddingHeight = 2 - d->paddingHeight;
+		turned.paddingWidth = 2 - d->paddingWidth;
+		turned.resultHeight = d->height;
+		turned.resultWidth = d->width;
+		const CFusedActivation none = { NH_ACT_NONE, 0.f };
+		return channelwise3x3Impl<1, 4>( s, &turned, outputDiff, filter, nullptr, inputDiff, none, true );
+	}
 	const long long items = static_cast<long long>( d->batch ) * d->height * d->width * ( vec ? d->channels / 4 : d->channels );
 	long long blocks = ( items + 255 ) / 256;
 	blocks = blocks > 1048576 ? 1048576 : blocks;
@@ -1686,9 +1705,9 @@ int nhBlobChannelwiseConvolutionLearnAdd( nhStream s, const nhConvDesc* d, const
 	}
 	const int groupBlocks = ceilDiv( cg, groups );
 	const long long pixels = static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth;
-	// about 2048 workgroups, each lane at least 8 pixels of its own
+	// about 1024 workgroups ( measured best of 256..2048 ), each lane at least 8 pixels of its own
 	const int lanes = 256 / groups;
-	long long slices = 2048 / groupBlocks > 0 ? 2048 / groupBlocks : 1;
+	long long slices = 1024 / groupBlocks > 0 ? 1024 / groupBlocks : 1;
 	const long long most = pixels / ( 8LL * lanes ) > 0 ? pixels / ( 8LL * lanes ) : 1;
 	slices = slices < most ? slices : most;
 	const long long pixelsPerSlice = ( pixels + slices - 1 ) / slices;

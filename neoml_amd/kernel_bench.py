@@ -177,12 +177,30 @@ def main():
                 lambda: lib.nhBlobChannelwiseConvolution(stream, ctypes.byref(d), P(x), P(flt), P(b), P(y)),
                 2 * n * d.resultHeight * d.resultWidth * c * 9, by, by)
 
+    def dw_gradients(n, h, w, c, s):
+        d = neoml_amd.ConvDesc(n, h, w, c, c, 3, 3, 1, 1, s, s, 1, 1, 0, 0)
+        neoml_amd.check(lib.nhInitBlobChannelwiseConvolution(ctypes.byref(d)))
+        x, flt = rand(n, h, w, c), rand(3, 3, c)
+        g = rand(n, d.resultHeight, d.resultWidth, c)
+        dx, dflt, dfree = empty(n, h, w, c), torch.zeros((3, 3, c), device=dev), torch.zeros(c, device=dev)
+        by = 4 * (x.numel() + g.numel())
+        tag = "cfg3 %dx%dx%dx%d 3x3/%d" % (n, h, w, c, s)
+        measure("BlobChannelwiseConvolutionBackward " + tag,
+                lambda: lib.nhBlobChannelwiseConvolutionBackward(stream, ctypes.byref(d), P(g), P(flt), P(dx)),
+                2 * g.numel() * 9, by, by)
+        measure("BlobChannelwiseConvolutionLearnAdd " + tag,
+                lambda: lib.nhBlobChannelwiseConvolutionLearnAdd(stream, ctypes.byref(d), P(x), P(g), P(dflt), P(dfree)),
+                2 * g.numel() * 9, by, by)
+
     dw(128, 112, 112, 96, 2)
     dw(128, 112, 112, 32, 1)
     dw(128, 56, 56, 144, 1)
     dw(128, 28, 28, 192, 2)
     dw(128, 14, 14, 384, 1)
     dw(128, 7, 7, 960, 1)
+    dw_gradients(128, 56, 56, 144, 1)
+    dw_gradients(128, 112, 112, 96, 2)
+    dw_gradients(128, 14, 14, 384, 1)
 
     # ---- pooling, padding (config 2, 5)
     def pool(tag, n, h, w, c, f_h, f_w, s_h, s_w, mean=False):
