@@ -1086,6 +1086,118 @@ template<> struct CChanAtomic<1> {
 	static __device__ __forceinline__ float sum( float a, float b ) { return a + b; }
 };
 
+// The 3x3 case of the gradient by the filter, on the forward pass's strips: a thread owns 4 channels of a strip WPT
+// output pixels wide and rowsPerItem output rows tall, slides down it with the three input rows of the window in
+// registers ( every input row loaded once per strip ) and keeps the nine tap sums and the free-term sum of its strip in
+// registers. The threads of a workgroup then meet per channel in an LDS table ( LDS atomics ), and the workgroup leaves
+// with one global atomic add per table entry: a few hundred adds per address over the whole launch.
+template<int STRIDE, int WPT>
+__global__ __launch_bounds__( 256 )
+void channelwiseLearn3x3Kernel( const nhConvDesc d, const float* input, const float* outputDiff, float* filterDiff,
+	float* freeTermDiff, int wGroups, int rowChunks, int rowsPerItem, int totalItems )
+{
+	constexpr int NC = ( WPT - 1 ) * STRIDE + 3;
+	constexpr int Keep = 3 - STRIDE;
+	constexpr int Sums = 10; // nine taps and the free term
+	__shared__ float table[Sums * 4 * 256];
+	const int cg = d.channels / 4; // at most 256: the table has a column per channel group
+	const int tableWidth = cg;
+	for( int idx = threadIdx.x; idx < Sums * 4 * tableWidth; idx += blockDim.x ) {
+		table[idx] = 0.f;
+	}
+	__syncthreads();
+	// a few hundred workgroups walk the strips grid-stride and collect in their table: the global adds at the end are what
+	// limits this kernel when thousands of workgroups bring their own
+	for( int item = blockIdx.x * blockDim.x + threadIdx.x; item < totalItems; item += gridDim.x * blockDim.x ) {
+		int t = item;
+		const int group = t % cg;
+		const int c = group * 4; t /= cg;
+		const int wo0 = ( t % wGroups ) * WPT; t /= wGroups;
+		const int ho0 = ( t % rowChunks ) * rowsPerItem;
+		const int n = t / rowChunks;
+		const int hoEnd = min( ho0 + rowsPerItem, d.resultHeight );
+
+		const __amdgpu_buffer_rsrc_t image = makeBuffer( input );
+		const unsigned rowBytes = static_cast<unsigned>( d.width ) * d.channels * 4;
+		const unsigned imageBytes = n * d.height * rowBytes;
+		unsigned colOff[NC];
+		const int wi0 = wo0 * STRIDE - d.paddingWidth;
+#pragma unroll
+		for( int j = 0; j < NC; ++j ) {
+			const int wi = wi0 + j;
+			colOff[j] = wi >= 0 && wi < d.width ? static_cast<unsigned>( wi * d.channels + c ) * 4 : OutOfRange;
+		}
+		float4 rows[3][NC];
+		auto loadRow = [&]( float4* row, int hi ) {
+			const bool valid = hi >= 0 && hi < d.height;
+			const unsigned rowOff = imageBytes + static_cast<unsigned>( hi ) * rowBytes;
+#pragma unroll
+			for( int j = 0; j < NC; ++j ) {
+				row[j] = bufferLoad4( image, valid ? rowOff + colOff[j] : OutOfRange );
+			}
+		};
+		float4 sums[Sums];
+#pragma unroll
+		for( int k = 0; k < Sums; ++k ) {
+			sums[k] = make_float4( 0.f, 0.f, 0.f, 0.f );
+		}
+		int hi = ho0 * STRIDE - d.paddingHeight;
+#pragma unroll
+		for( int r = 0; r < Keep; ++r ) {
+			loadRow( rows[r], hi + r );
+		}
+		const float* diff = outputDiff + ( ( static_cast<long long>( n ) * d.resultHeight + ho0 ) * d.resultWidth + wo0 ) * d.channels + c;
+		const long long diffRow = static_cast<long long>( d.resultWidth ) * d.channels;
+		for( int ho = ho0; ho < hoEnd; ++ho ) {
+#pragma unroll
+			for( int r = Keep; r < 3; ++r ) {
+				loadRow( rows[r], hi + r );
+			}
+#pragma unroll
+			for( int j = 0; j < WPT; ++j ) {
+				const float4 g = wo0 + j < d.resultWidth ? *reinterpret_cast<const float4*>( diff + j * d.channels )
+					: make_float4( 0.f, 0.f, 0.f, 0.f );
+#pragma unroll
+				for( int kh = 0; kh < 3; ++kh ) {
+#pragma unroll
+					for( int kw = 0; kw < 3; ++kw ) {
+						sums[kh * 3 + kw] = CChanVec<4>::fma( rows[kh][j * STRIDE + kw], g, sums[kh * 3 + kw] );
+					}
+				}
+				sums[9].x += g.x; sums[9].y += g.y; sums[9].z += g.z; sums[9].w += g.w;
+			}
+#pragma unroll
+			for( int r = 0; r < Keep; ++r ) {
+#pragma unroll
+				for( int j = 0; j < NC; ++j ) {
+					rows[r][j] = rows[r + STRIDE][j];
+				}
+			}
+			hi += STRIDE;
+			diff += diffRow;
+		}
+#pragma unroll
+		for( int k = 0; k < Sums; ++k ) {
+			atomicAdd( &table[( k * 4 + 0 ) * tableWidth + group], sums[k].x );
+			atomicAdd( &table[( k * 4 + 1 ) * tableWidth + group], sums[k].y );
+			atomicAdd( &table[( k * 4 + 2 ) * tableWidth + group], sums[k].z );
+			atomicAdd( &table[( k * 4 + 3 ) * tableWidth + group], sums[k].w );
+		}
+	}
+	__syncthreads();
+	for( int idx = threadIdx.x; idx < Sums * 4 * tableWidth; idx += blockDim.x ) {
+		const int k4 = idx / tableWidth;
+		const int group = idx - k4 * tableWidth;
+		const int channel = group * 4 + ( k4 & 3 );
+		const float v = table[idx];
+		if( k4 < 36 ) {
+			unsafeAtomicAdd( filterDiff + ( k4 >> 2 ) * d.channels + channel, v );
+		} else if( freeTermDiff != nullptr ) {
+			unsafeAtomicAdd( freeTermDiff + channel, v );
+		}
+	}
+}
+
 // Gradient of the channelwise convolution by its filter (and free term): sums over every output pixel of the batch.
 // A workgroup owns a block of GROUPS channel groups and a slice of the output pixels; its 256 / GROUPS pixel lanes keep
 // the TAPS + 1 sums of their channel group in registers, meet in LDS and leave with one atomic add per sum.
@@ -1476,6 +1588,26 @@ static int channelwise3x3Impl( nhStream s, const nhConvDesc* d, const float* sou
 	return NH_OK;
 }
 
+template<int STRIDE, int WPT>
+static int channelwiseLearn3x3Impl( nhStream s, const nhConvDesc* d, const float* input, const float* outputDiff,
+	float* filterDiff, float* freeTermDiff )
+{
+	const int wGroups = ceilDiv( d->resultWidth, WPT );
+	const long long perRow = static_cast<long long>( d->batch ) * wGroups * ( d->channels / 4 );
+	int rowChunks = 1, rowsPerItem = 1;
+	// tall strips ( few row chunks ): every chunk re-reads two halo rows and ends with 40 LDS adds per thread
+	chooseRowChunks( perRow, d->resultHeight, 4, 256, &rowChunks, &rowsPerItem );
+	const long long items = perRow * rowChunks;
+	// one workgroup per compute unit: measured best of 64..2048 ( more workgroups bring more global adds, fewer leave
+	// compute units idle; larger workgroups change nothing )
+	const long long cap = 256;
+	const long long blocks = ( items + 255 ) / 256 < cap ? ( items + 255 ) / 256 : cap;
+	hipLaunchKernelGGL( ( channelwiseLearn3x3Kernel<STRIDE, WPT> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0,
+		toStream( s ), *d, input, outputDiff, filterDiff, freeTermDiff, wGroups, rowChunks, rowsPerItem, static_cast<int>( items ) );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
 template<bool MAX>
 static int poolingBackwardImpl( nhStream s, const nhPoolingDesc* d, const float* resultDiff, const int* maxIndices,
 	float* sourceDiff )
@@ -1697,6 +1829,14 @@ int nhBlobChannelwiseConvolutionLearnAdd( nhStream s, const nhConvDesc* d, const
 		return NH_OK;
 	}
 	const bool vec = d->channels % 4 == 0 && isAligned16( input ) && isAligned16( outputDiff );
+	if( vec && d->filterHeight == 3 && d->filterWidth == 3 && d->strideHeight == d->strideWidth && d->strideHeight <= 2
+		&& d->channels <= 1024
+		&& static_cast<long long>( d->batch ) * d->height * d->width * d->channels * 4 < 0x80000000LL
+		&& static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * d->channels < 0x7fffffffLL )
+	{
+		return d->strideHeight == 1 ? channelwiseLearn3x3Impl<1, 4>( s, d, input, outputDiff, filterDiff, freeTermDiff )
+			: channelwiseLearn3x3Impl<2, 2>( s, d, input, outputDiff, filterDiff, freeTermDiff );
+	}
 	const int cg = vec ? d->channels / 4 : d->channels;
 	// channel groups per workgroup: a power of two up to 64, so that a wave reads whole runs of channels
 	int groups = 1;
