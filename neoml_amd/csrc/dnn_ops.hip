@@ -1073,6 +1073,47 @@ void channelwiseConvBackwardKernel( const nhConvDesc d, const float* outputDiff,
 	}
 }
 
+// The 3x3, stride 2 case of the gradient by the input, 4 channels per thread: an input pixel lies in one or two window
+// rows ( hi + pad even: taps 0 and 2, odd: tap 1 ) and one or two window columns, so it gathers at most four output
+// pixels; which ones follows from the parity, without divisions or a loop over the nine taps. Out-of-range output pixels
+// are out-of-range buffer offsets ( they read as zero ).
+__global__ __launch_bounds__( 256 )
+void channelwiseBackward3x3Stride2Kernel( const nhConvDesc d, const float* outputDiff, const float* filter, float* inputDiff,
+	int totalItems )
+{
+	const int item = blockIdx.x * 256 + threadIdx.x;
+	if( item >= totalItems ) {
+		return;
+	}
+	const int cg = d.channels / 4;
+	int t = item;
+	const int c = ( t % cg ) * 4; t /= cg;
+	const int wi = t % d.width; t /= d.width;
+	const int hi = t % d.height;
+	const int n = t / d.height;
+	const __amdgpu_buffer_rsrc_t diff = makeBuffer( outputDiff );
+	const int a = hi + d.paddingHeight, b = wi + d.paddingWidth;
+	int kh[2], ho[2], kw[2], wo[2];
+	kh[0] = a & 1; ho[0] = ( a - kh[0] ) >> 1; kh[1] = kh[0] + 2; ho[1] = ho[0] - 1;
+	kw[0] = b & 1; wo[0] = ( b - kw[0] ) >> 1; kw[1] = kw[0] + 2; wo[1] = wo[0] - 1;
+	float4 acc = make_float4( 0.f, 0.f, 0.f, 0.f );
+#pragma unroll
+	for( int r = 0; r < 2; ++r ) {
+		const bool rowOk = kh[r] <= 2 && ho[r] >= 0 && ho[r] < d.resultHeight;
+#pragma unroll
+		for( int q = 0; q < 2; ++q ) {
+			const bool ok = rowOk && kw[q] <= 2 && wo[q] >= 0 && wo[q] < d.resultWidth;
+			const unsigned offset = ok ? static_cast<unsigned>( ( ( n * d.resultHeight + ho[r] ) * d.resultWidth + wo[q] ) * d.channels + c ) * 4u
+				: OutOfRange;
+			const float4 g = bufferLoad4( diff, offset );
+			const int tap = ok ? kh[r] * 3 + kw[q] : 0;
+			const float4 f = *reinterpret_cast<const float4*>( filter + tap * d.channels + c );
+			acc = CChanVec<4>::fma( g, f, acc );
+		}
+	}
+	*reinterpret_cast<float4*>( inputDiff + static_cast<long long>( item ) * 4 ) = acc;
+}
+
 template<int VECW> struct CChanAtomic;
 template<> struct CChanAtomic<4> {
 	static __device__ __forceinline__ void add( float* p, float4 v )
@@ -1802,6 +1843,16 @@ int nhBlobChannelwiseConvolutionBackward( nhStream s, const nhConvDesc* d, const
 		turned.resultWidth = d->width;
 		const CFusedActivation none = { NH_ACT_NONE, 0.f };
 		return channelwise3x3Impl<1, 4>( s, &turned, outputDiff, filter, nullptr, inputDiff, none, true );
+	}
+	if( vec && d->filterHeight == 3 && d->filterWidth == 3 && d->strideHeight == 2 && d->strideWidth == 2
+		&& static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * d->channels * 4 < 0x7fffffffLL
+		&& static_cast<long long>( d->batch ) * d->height * d->width * ( d->channels / 4 ) < 0x7fffff00LL )
+	{
+		const int total = d->batch * d->height * d->width * ( d->channels / 4 );
+		hipLaunchKernelGGL( channelwiseBackward3x3Stride2Kernel, dim3( static_cast<unsigned>( ( total + 255 ) / 256 ) ), dim3( 256 ), 0,
+			toStream( s ), *d, outputDiff, filter, inputDiff, total );
+		NH_LAUNCH_CHECK();
+		return NH_OK;
 	}
 	const long long items = static_cast<long long>( d->batch ) * d->height * d->width * ( vec ? d->channels / 4 : d->channels );
 	long long blocks = ( items + 255 ) / 256;
