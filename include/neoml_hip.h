@@ -54,6 +54,15 @@ NH_API int nhSetDevice(int device);
 NH_API int nhStreamCreate(nhStream* stream);
 NH_API int nhStreamDestroy(nhStream stream);
 NH_API int nhStreamSynchronize(nhStream stream);
+/* The scratch block of a stream (see the conventions above) normally comes from the raw allocator. After
+ * nhStreamBindPool it is taken from `pool` instead, so that the pool's memory limit, statistics and clean-up cover
+ * everything an engine allocates (HeapAlloc's contract, src/MemoryEngineMixin.cpp:99-115); when the pool cannot give the
+ * block the launch still runs, its slices meeting through atomic adds. Binding to another pool or to null hands the blocks
+ * back first: the stream must be idle, and a bound pool must outlive the binding (rebind to null, release or destroy the
+ * stream before nhPoolDestroy). nhStreamReleaseScratch drains the stream and frees its block, for CleanUp (NME.h:1211)
+ * and for streams the library did not create; the next launch that needs a block allocates a new one. */
+NH_API int nhStreamBindPool(nhStream stream, void* pool);
+NH_API int nhStreamReleaseScratch(nhStream stream);
 
 /* raw allocator under the caching pool (IRawMemoryManager, src/RawMemoryManager.h:24-29) */
 NH_API int nhRawAlloc(void** ptr, size_t size);
@@ -402,9 +411,11 @@ NH_API int nhBlobMeanPoolingBackward(nhStream s, const nhPoolingDesc* desc_host,
  * workspace: nhLstmWorkspaceSize bytes of device memory, owned by the caller.
  * Sequences of 2+ steps with H a multiple of 16, H <= 512 and a grid that fits the device run as ONE launch whose
  * workgroups stay resident and hand the step outputs to one another through memory; it needs the device to itself
- * for that launch (other work on the same stream is ordered before or after it anyway). Its wait for a step's values
- * is bounded: should it trip (several such launches sharing the device from different streams), the launch ends
- * normally with invalid output, and the next nhStreamSynchronize / nhCopyDeviceToHost returns NH_ERR_HIP once. */
+ * for that launch. The library therefore orders every such launch of the process behind the previous one on the device
+ * (an event wait; the host does not block), whichever streams they use, and takes the launch-per-step kernels while the
+ * stream is being captured into a graph. Its wait for a step's values is bounded: should it still trip (another process
+ * occupying the device for seconds), the launch ends normally with invalid output, and the next nhStreamSynchronize /
+ * nhCopyDeviceToHost ON THAT STREAM returns NH_ERR_HIP once; no other stream is told or touched. */
 NH_API int nhLstmWorkspaceSize(int hiddenSize, int objectSize, int sequenceLength, int sequenceCount, size_t* bytes);
 NH_API int nhLstm(nhStream s, int hiddenSize, int objectSize, const float* inputWeights, const float* inputFreeTerm,
 	const float* recurrentWeights, const float* recurrentFreeTerm, int reverse, int sequenceLength,

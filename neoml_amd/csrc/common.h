@@ -15,8 +15,8 @@ void setLastError( const char* fmt, ... );
 inline hipStream_t toStream( nhStream s ) { return reinterpret_cast<hipStream_t>( s ); }
 
 // Frees the scratch blocks that sliced reductions keep for a stream of the current device ( gemm_mfma.hip ); the stream
-// must have been drained. Called when the stream is destroyed.
-void releaseSliceScratch( hipStream_t stream );
+// must have been drained. unbind: the stream is going away, its binding to a pool goes with the blocks.
+void releaseSliceScratch( hipStream_t stream, bool unbind );
 
 constexpr int WaveSize = 64;
 

@@ -4,7 +4,9 @@
 #include "common.h"
 #include <float.h>
 #include <stdlib.h>
-#include <atomic>
+#include <map>
+#include <mutex>
+#include <utility>
 
 namespace nh {
 
@@ -688,6 +690,7 @@ struct CLstmSeqArgs {
 	float* COut;                   // [T][B][H] or null
 	unsigned long long* Exchange;  // [2][B][H] tagged h values, zero at launch
 	unsigned* Abort;               // one word, zero at launch
+	unsigned* GaveUp;              // host-visible word of the launch stream: set when a wavefront gives up
 	int T, B, H, Reverse;
 	unsigned MaxSpins;
 };
@@ -704,11 +707,6 @@ __device__ __forceinline__ float seqTanh( float x )
 	return 1.f - 2.f * __builtin_amdgcn_rcpf( 1.f + __builtin_amdgcn_exp2f( 2.8853900817779268f * x ) );
 }
 
-
-// Sticky count of wavefronts that gave up a wait, over all launches on this device: the abort word lives in the
-// caller's workspace, which the caller is free to recycle, so the host reads this one after it has drained a stream
-// and reports the give-up through the next synchronising call.
-__device__ unsigned seqGiveUps;
 
 template<int RB, int CB, int W>
 __global__ __launch_bounds__( 64 * W )
@@ -853,7 +851,9 @@ void lstmSequenceKernel( const CLstmSeqArgs a )
 				{
 					__hip_atomic_store( a.Abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT );
 					if( lane == 0 ) {
-						atomicAdd( &seqGiveUps, 1u );
+						// the abort word lives in the caller's workspace, which the caller is free to recycle: the host
+						// learns of the give-up through this word of pinned host memory that belongs to the launch stream
+						__hip_atomic_store( a.GaveUp, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM );
 					}
 					giveUp = 1; // read by the whole workgroup after the next barrier
 					break;
@@ -1420,28 +1420,86 @@ using namespace nh;
 
 extern "C" int nhInitPooling( nhPoolingDesc* d );
 
-// set by every launch of the one-launch LSTM, cleared by the check below
-static std::atomic<bool> sequenceLaunched( false );
-
+// ---- bookkeeping of the one-launch LSTM ------------------------------------------------------------------------
+// Per ( device, stream ): one word of pinned host memory that a launch on that stream sets when its bounded wait
+// trips. The synchronising entry points read the word of THEIR stream once it has drained, so a give-up is reported to
+// whoever waits for the stream it happened on, once, and to nobody else; no copy, no other stream is touched.
+// Per device: the event of the last one-launch LSTM. The kernel needs all its workgroups resident together; two such
+// grids from different streams could each hold half of the device and starve one another until their waits expire.
+// A launch on another stream is therefore ordered behind the previous one through that event ( a wait on the device,
+// the host does not block ).
 namespace nh {
-// Called by the synchronising entry points once their stream has drained: a one-launch LSTM whose bounded wait
-// tripped has produced garbage, and that must not pass silently.
-int checkSequenceGiveUps()
+
+struct CSequenceStream {
+	unsigned* GaveUp = nullptr; // pinned host memory, device-visible
+	bool Launched = false;      // a one-launch LSTM was issued since the word was last looked at
+};
+
+struct CSequenceDevice {
+	hipEvent_t LastDone = nullptr;
+	hipStream_t LastStream = nullptr;
+	bool Any = false;
+};
+
+static std::mutex sequenceLock;
+static std::map<std::pair<int, hipStream_t>, CSequenceStream>& sequenceStreams()
 {
-	if( !sequenceLaunched.exchange( false ) ) {
+	static std::map<std::pair<int, hipStream_t>, CSequenceStream> streams;
+	return streams;
+}
+static std::map<int, CSequenceDevice>& sequenceDevices()
+{
+	static std::map<int, CSequenceDevice> devices;
+	return devices;
+}
+
+// Called by the synchronising entry points once `stream` has drained: a one-launch LSTM of this stream whose bounded
+// wait tripped has produced garbage, and that must not pass silently.
+int checkSequenceGiveUps( hipStream_t stream )
+{
+	int device = 0;
+	if( hipGetDevice( &device ) != hipSuccess ) {
+		( void )hipGetLastError();
 		return NH_OK;
 	}
-	unsigned count = 0;
-	NH_HIP( hipMemcpyFromSymbol( &count, HIP_SYMBOL( seqGiveUps ), sizeof( count ) ) );
-	if( count == 0 ) {
+	std::lock_guard<std::mutex> guard( sequenceLock );
+	auto& streams = sequenceStreams();
+	auto found = streams.find( std::make_pair( device, stream ) );
+	if( found == streams.end() || !found->second.Launched ) {
 		return NH_OK;
 	}
-	const unsigned zero = 0;
-	NH_HIP( hipMemcpyToSymbol( HIP_SYMBOL( seqGiveUps ), &zero, sizeof( zero ) ) );
-	setLastError( "nhLstm: %u wavefronts of a one-launch LSTM gave up waiting for the previous step (the grid was not "
-		"resident as a whole, or the spin limit is too low): its output is invalid", count );
+	found->second.Launched = false;
+	volatile unsigned* word = found->second.GaveUp;
+	if( *word == 0 ) {
+		return NH_OK;
+	}
+	*word = 0;
+	setLastError( "nhLstm: a one-launch LSTM on this stream gave up waiting for the previous step (its grid was not "
+		"resident as a whole, or the spin limit is too low): its output is invalid" );
 	return NH_ERR_HIP;
 }
+
+// the stream is going away ( it has been drained )
+void releaseSequenceStream( hipStream_t stream )
+{
+	int device = 0;
+	if( hipGetDevice( &device ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return;
+	}
+	std::lock_guard<std::mutex> guard( sequenceLock );
+	auto& streams = sequenceStreams();
+	auto found = streams.find( std::make_pair( device, stream ) );
+	if( found != streams.end() ) {
+		( void )hipHostFree( found->second.GaveUp );
+		streams.erase( found );
+	}
+	auto dev = sequenceDevices().find( device );
+	if( dev != sequenceDevices().end() && dev->second.LastStream == stream ) {
+		dev->second.Any = false; // drained: nothing of it is in flight
+	}
+}
+
 } // namespace nh
 
 // ---- whole-sequence LSTM launch ------------------------------------------------------------------------------
@@ -1544,17 +1602,51 @@ static unsigned lstmSpinLimit()
 	return 4u << 20;
 }
 
-static int launchLstmSequence( hipStream_t stream, const CLstmSeqArgs& a )
+// false: the one-launch path cannot be taken for this stream right now ( it is being captured into a graph, whose
+// replays nothing here could order ); the caller runs the launch-per-step kernels instead
+static bool lstmSequenceAllowed( hipStream_t stream )
 {
-	sequenceLaunched.store( true );
+	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+	if( hipStreamIsCapturing( stream, &capture ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return false;
+	}
+	return capture == hipStreamCaptureStatusNone;
+}
+
+static int launchLstmSequence( hipStream_t stream, CLstmSeqArgs a )
+{
 	const CLstmSeqShape* shape = lstmSequenceShape( a.H, a.B );
 	NH_REQUIRE( shape != nullptr );
+	int device = 0;
+	NH_HIP( hipGetDevice( &device ) );
+	std::lock_guard<std::mutex> guard( sequenceLock );
+	CSequenceStream& own = sequenceStreams()[std::make_pair( device, stream )];
+	if( own.GaveUp == nullptr ) {
+		void* word = nullptr;
+		NH_HIP( hipHostMalloc( &word, 64, hipHostMallocDefault ) );
+		own.GaveUp = static_cast<unsigned*>( word );
+		*own.GaveUp = 0;
+	}
+	CSequenceDevice& dev = sequenceDevices()[device];
+	if( dev.LastDone == nullptr ) {
+		NH_HIP( hipEventCreateWithFlags( &dev.LastDone, hipEventDisableTiming ) );
+	}
+	if( dev.Any ) {
+		// behind the one-launch LSTM issued last, whichever stream it went to ( on the same stream the wait is free )
+		NH_HIP( hipStreamWaitEvent( stream, dev.LastDone, 0 ) );
+	}
+	a.GaveUp = own.GaveUp;
+	own.Launched = true;
 	const unsigned groups = static_cast<unsigned>( ( a.H / ( SeqUnits * shape->Blocks ) ) * ceilDiv( a.B, shape->Rows ) );
 	// the exchange buffers and the abort word that follows them
 	const long long words = 2LL * a.B * a.H + 1;
 	hipLaunchKernelGGL( clearWordsKernel, dim3( static_cast<unsigned>( ( words + 1023 ) / 1024 ) ), dim3( 256 ), 0, stream, a.Exchange, words );
 	shape->Launch( stream, groups, lstmSequenceLds( a.H, *shape ), a );
 	NH_LAUNCH_CHECK();
+	NH_HIP( hipEventRecord( dev.LastDone, stream ) );
+	dev.LastStream = stream;
+	dev.Any = true;
 	return NH_OK;
 }
 
@@ -2073,7 +2165,9 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 		return rc;
 	}
 	const int stepSize = B * H;
-	if( T > 1 && lstmSequenceFits( H, B, recurrentWeights, inputStateBackLink, inputMainBackLink, outputMainBackLink ) ) {
+	if( T > 1 && lstmSequenceFits( H, B, recurrentWeights, inputStateBackLink, inputMainBackLink, outputMainBackLink )
+		&& lstmSequenceAllowed( stream ) )
+	{
 		CLstmSeqArgs a = {};
 		a.Gates = gates; a.Wrec = recurrentWeights; a.H0 = inputMainBackLink; a.C0 = inputStateBackLink;
 		a.HOut = outputMainBackLink; a.COut = outputStateBackLink;

@@ -906,9 +906,12 @@ void matMulKernel( const CMatMulArgs launchArgs )
 
 // Scratch of the K slices that meet without atomics: partial tiles and arrival counters, one pair per stream (launches
 // of one stream run in order and may share it; two streams must not). Grown on demand by doubling; a block that has been
-// outgrown is NOT freed while the stream lives: another thread may be about to launch on the same stream with the address
-// it was handed a moment ago. All blocks of a stream (together at most twice the largest request) are freed when the
-// stream is destroyed through nhStreamDestroy, those of other streams live until the process ends.
+// outgrown is NOT freed while the stream keeps its scratch: another thread may be about to launch on the same stream with
+// the address it was handed a moment ago. All blocks of a stream (together at most twice the largest request) are freed by
+// releaseSliceScratch: when the stream is destroyed through nhStreamDestroy, or when its owner asks
+// (nhStreamReleaseScratch); those of other streams live until the process ends.
+// A stream that has been bound to a caching pool (nhStreamBindPool) takes its blocks from that pool and gives them back
+// to it, so the pool's memory limit, statistics and clean-up cover them; other streams use the raw allocator.
 // The counters start at zero and every launch leaves them at zero.
 struct CSliceScratch {
 	float* Partials = nullptr;
@@ -916,6 +919,7 @@ struct CSliceScratch {
 	unsigned* Counters = nullptr;
 	size_t CounterCount = 0;
 	std::vector<void*> Blocks; // every allocation made for the stream
+	nhPool Pool = nullptr;     // where the blocks came from; null = the raw allocator
 };
 
 static std::mutex sliceScratchLock;
@@ -924,8 +928,25 @@ static std::map<std::pair<int, hipStream_t>, CSliceScratch>& sliceScratchByStrea
 	static std::map<std::pair<int, hipStream_t>, CSliceScratch> byStream;
 	return byStream;
 }
+static std::map<std::pair<int, hipStream_t>, nhPool>& poolByStream()
+{
+	static std::map<std::pair<int, hipStream_t>, nhPool> byStream;
+	return byStream;
+}
 
-void releaseSliceScratch( hipStream_t stream )
+static void freeSliceBlocks( CSliceScratch& scratch )
+{
+	for( void* block : scratch.Blocks ) {
+		if( scratch.Pool != nullptr ) {
+			( void )nhPoolHeapFree( scratch.Pool, block );
+		} else {
+			( void )hipFree( block );
+		}
+	}
+	scratch = CSliceScratch();
+}
+
+void releaseSliceScratch( hipStream_t stream, bool unbind )
 {
 	int device = 0;
 	if( hipGetDevice( &device ) != hipSuccess ) {
@@ -933,19 +954,52 @@ void releaseSliceScratch( hipStream_t stream )
 		return;
 	}
 	std::lock_guard<std::mutex> guard( sliceScratchLock );
+	const std::pair<int, hipStream_t> key = std::make_pair( device, stream );
 	auto& byStream = sliceScratchByStream();
-	auto found = byStream.find( std::make_pair( device, stream ) );
-	if( found == byStream.end() ) {
-		return;
+	auto found = byStream.find( key );
+	if( found != byStream.end() ) {
+		freeSliceBlocks( found->second );
+		byStream.erase( found );
 	}
-	for( void* block : found->second.Blocks ) {
-		( void )hipFree( block );
+	if( unbind ) {
+		poolByStream().erase( key );
 	}
-	byStream.erase( found );
+}
+
+int bindSliceScratchPool( hipStream_t stream, nhPool pool )
+{
+	int device = 0;
+	NH_HIP( hipGetDevice( &device ) );
+	std::lock_guard<std::mutex> guard( sliceScratchLock );
+	const std::pair<int, hipStream_t> key = std::make_pair( device, stream );
+	auto& byStream = sliceScratchByStream();
+	auto found = byStream.find( key );
+	if( found != byStream.end() && found->second.Pool != pool ) {
+		// blocks from the previous source go back there ( the caller has drained the stream )
+		freeSliceBlocks( found->second );
+		byStream.erase( found );
+	}
+	if( pool != nullptr ) {
+		poolByStream()[key] = pool;
+	} else {
+		poolByStream().erase( key );
+	}
+	return NH_OK;
+}
+
+// hipStreamPerThread names a different queue in every thread: launches of two threads on that handle may run side by
+// side, so it never gets a block ( its slices meet through atomic adds ). The null stream and hipStreamLegacy name the
+// one legacy queue of the device, whose launches run in order whoever issues them.
+static bool isSharedStreamHandle( hipStream_t stream )
+{
+	return stream == hipStreamPerThread;
 }
 
 static bool sliceScratch( hipStream_t stream, size_t partialFloats, size_t counters, CSliceScratch& out )
 {
+	if( isSharedStreamHandle( stream ) ) {
+		return false;
+	}
 	int device = 0;
 	if( hipGetDevice( &device ) != hipSuccess ) {
 		return false;
@@ -959,28 +1013,43 @@ static bool sliceScratch( hipStream_t stream, size_t partialFloats, size_t count
 		( void )hipGetLastError();
 		return false;
 	}
-	CSliceScratch& scratch = byStream[std::make_pair( device, stream )];
-	if( scratch.PartialFloats < partialFloats ) {
-		const size_t grown = partialFloats > 2 * scratch.PartialFloats ? partialFloats : 2 * scratch.PartialFloats;
-		float* block = nullptr;
-		if( hipMalloc( reinterpret_cast<void**>( &block ), grown * sizeof( float ) ) != hipSuccess ) {
+	const std::pair<int, hipStream_t> key = std::make_pair( device, stream );
+	CSliceScratch& scratch = byStream[key];
+	if( scratch.Blocks.empty() ) {
+		auto bound = poolByStream().find( key );
+		scratch.Pool = bound != poolByStream().end() ? bound->second : nullptr;
+	}
+	// a pool that cannot give the block ( its memory limit ) is not an error here: the slices then meet through atomics
+	auto allocate = [&]( size_t bytes ) -> void* {
+		void* block = nullptr;
+		if( scratch.Pool != nullptr ) {
+			if( nhPoolHeapAlloc( scratch.Pool, bytes, &block ) != NH_OK ) {
+				return nullptr;
+			}
+		} else if( hipMalloc( &block, bytes ) != hipSuccess ) {
 			( void )hipGetLastError();
-			return false;
+			return nullptr;
 		}
 		scratch.Blocks.push_back( block );
+		return block;
+	};
+	if( scratch.PartialFloats < partialFloats ) {
+		const size_t grown = partialFloats > 2 * scratch.PartialFloats ? partialFloats : 2 * scratch.PartialFloats;
+		float* block = static_cast<float*>( allocate( grown * sizeof( float ) ) );
+		if( block == nullptr ) {
+			return false;
+		}
 		scratch.Partials = block;
 		scratch.PartialFloats = grown;
 	}
 	if( scratch.CounterCount < counters ) {
 		size_t grown = counters > 2 * scratch.CounterCount ? counters : 2 * scratch.CounterCount;
 		grown = grown > 4096 ? grown : 4096;
-		unsigned* block = nullptr;
-		// cleared on the launch stream, ahead of the launch that first uses it
-		if( hipMalloc( reinterpret_cast<void**>( &block ), grown * sizeof( unsigned ) ) != hipSuccess ) {
-			( void )hipGetLastError();
+		unsigned* block = static_cast<unsigned*>( allocate( grown * sizeof( unsigned ) ) );
+		if( block == nullptr ) {
 			return false;
 		}
-		scratch.Blocks.push_back( block );
+		// cleared on the launch stream, ahead of the launch that first uses it
 		if( hipMemsetAsync( block, 0, grown * sizeof( unsigned ), stream ) != hipSuccess ) {
 			( void )hipGetLastError();
 			return false;
@@ -991,6 +1060,23 @@ static bool sliceScratch( hipStream_t stream, size_t partialFloats, size_t count
 	out.Partials = scratch.Partials;
 	out.Counters = scratch.Counters;
 	return true;
+}
+
+// A meeting place handed in by the caller instead of the stream's block: the launch neither allocates nor looks the
+// stream up, and fails when the place is too small.
+struct CSliceMeeting {
+	float* Partials;
+	size_t PartialFloats;
+	unsigned* Counters;
+	size_t CounterCount;
+};
+
+// a fill kernel rather than a memset: callers may be recording a graph
+__global__ __launch_bounds__( 256 ) void clearCountersKernel( unsigned* counters, int count )
+{
+	for( int i = blockIdx.x * 256 + threadIdx.x; i < count; i += gridDim.x * 256 ) {
+		counters[i] = 0u;
+	}
 }
 
 // C[b][m][n] = bias[n] (or 0): the starting value that the K slices add their partial products to
@@ -1033,7 +1119,7 @@ static int presetResult( hipStream_t stream, const CMatMulArgs& args, int batch 
 }
 
 template<int BM, int BN, int WAVES_M, int WAVES_N, int AMODE, int BMODE>
-static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool vec )
+static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool vec, const CSliceMeeting* fixedMeeting )
 {
 	args.TilesM = ceilDiv( args.M, BM );
 	args.TilesN = ceilDiv( args.N, BN );
@@ -1148,7 +1234,19 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 		const size_t slicedTiles = args.FullTiles > 0 ? args.TailTiles : static_cast<size_t>( tiles );
 		const size_t slices = args.FullTiles > 0 ? args.TailSplit : args.SplitK;
 		CSliceScratch scratch;
-		if( sliceScratch( stream, slicedTiles * slices * 4096, slicedTiles, scratch ) ) {
+		if( fixedMeeting != nullptr ) {
+			// the caller's place: no allocation, no look at the stream; the contents are whatever the last call left
+			if( slicedTiles * slices * 4096 > fixedMeeting->PartialFloats || slicedTiles > fixedMeeting->CounterCount ) {
+				setLastError( "the K slices of this launch need %zu bytes of partial tiles and %zu counters; the fixed scratch holds "
+					"%zu bytes and %zu counters", slicedTiles * slices * 4096 * sizeof( float ), slicedTiles,
+					fixedMeeting->PartialFloats * sizeof( float ), fixedMeeting->CounterCount );
+				return NH_ERR_ARGUMENT;
+			}
+			hipLaunchKernelGGL( clearCountersKernel, dim3( ceilDiv( static_cast<long long>( slicedTiles ), 1024 ) ), dim3( 256 ), 0, stream,
+				fixedMeeting->Counters, static_cast<int>( slicedTiles ) );
+			args.Partials = fixedMeeting->Partials;
+			args.Counters = fixedMeeting->Counters;
+		} else if( sliceScratch( stream, slicedTiles * slices * 4096, slicedTiles, scratch ) ) {
 			args.Partials = scratch.Partials;
 			args.Counters = scratch.Counters;
 		}
@@ -1219,12 +1317,12 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 // and latency hiding across workgroups matters more at fp32 MFMA rates than the smaller tile's extra L2 traffic.
 // Narrow outputs (N <= 32) use 128x32 so that no MFMA block multiplies padding.
 template<int AMODE, int BMODE>
-static int launchMatMul( hipStream_t stream, CMatMulArgs& args, int batch, bool vec )
+static int launchMatMul( hipStream_t stream, CMatMulArgs& args, int batch, bool vec, const CSliceMeeting* fixedMeeting = nullptr )
 {
 	if( args.N > 32 ) {
-		return launchTile<64, 64, 2, 2, AMODE, BMODE>( stream, args, batch, vec );
+		return launchTile<64, 64, 2, 2, AMODE, BMODE>( stream, args, batch, vec, fixedMeeting );
 	}
-	return launchTile<128, 32, 4, 1, AMODE, BMODE>( stream, args, batch, vec );
+	return launchTile<128, 32, 4, 1, AMODE, BMODE>( stream, args, batch, vec, fixedMeeting );
 }
 
 // The vector path addresses each operand with 32-bit byte offsets below BufferBytes.
@@ -1432,10 +1530,22 @@ int matMulNT( hipStream_t stream, const float* a, int lda, const float* b, int l
 	return matMulNTFused( stream, a, lda, b, ldb, c, ldc, M, N, K, batch, strideA, strideB, strideC, bias, accumulate, none, nullptr );
 }
 
+static int matMulNTMeeting( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
+	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC,
+	const float* bias, bool accumulate, const CFusedActivation& act, const float* residual, const CSliceMeeting* fixedMeeting );
+
 // ... and C = act( A * B^T + bias ) + residual, the epilogue of the fused blocks
 int matMulNTFused( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
 	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC,
 	const float* bias, bool accumulate, const CFusedActivation& act, const float* residual )
+{
+	return matMulNTMeeting( stream, a, lda, b, ldb, c, ldc, M, N, K, batch, strideA, strideB, strideC, bias, accumulate, act,
+		residual, nullptr );
+}
+
+static int matMulNTMeeting( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
+	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC,
+	const float* bias, bool accumulate, const CFusedActivation& act, const float* residual, const CSliceMeeting* fixedMeeting )
 {
 	if( M == 0 || N == 0 || batch == 0 ) {
 		return NH_OK;
@@ -1454,7 +1564,7 @@ int matMulNTFused( hipStream_t stream, const float* a, int lda, const float* b, 
 	}
 	const bool vec = isAligned16( a ) && isAligned16( b ) && K % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0
 		&& strideA % 4 == 0 && strideB % 4 == 0 && fitsBuffer( M, lda, K ) && fitsBuffer( N, ldb, K );
-	return launchMatMul<AM_RowsK, BM_RowsK>( stream, args, batch, vec );
+	return launchMatMul<AM_RowsK, BM_RowsK>( stream, args, batch, vec, fixedMeeting );
 }
 
 // C = A * B, A is M x K, B is K x N, all row-major.
@@ -1494,7 +1604,7 @@ int matMulTN( hipStream_t stream, const float* a, int lda, const float* b, int l
 }
 
 int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* source, const float* filter,
-	const float* freeTerm, float* result, const CFusedActivation& act )
+	const float* freeTerm, float* result, const CFusedActivation& act, const CSliceMeeting* fixedMeeting = nullptr )
 {
 	CMatMulArgs args = {};
 	args.Act = act;
@@ -1519,11 +1629,11 @@ int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* sour
 		&& d.paddingHeight == 0 && d.paddingWidth == 0 )
 	{
 		// a pointwise convolution over a channels-last image is the plain product image[M x Cin] * filter[Cout x Cin]^T
-		return matMulNTFused( stream, source, d.channels, filter, d.channels, result, d.filterCount, args.M, args.N, d.channels,
-			1, 0, 0, 0, freeTerm, false, act, nullptr );
+		return matMulNTMeeting( stream, source, d.channels, filter, d.channels, result, d.filterCount, args.M, args.N, d.channels,
+			1, 0, 0, 0, freeTerm, false, act, nullptr, fixedMeeting );
 	}
 	if( d.filterHeight == 1 && d.filterWidth == 1 ) {
-		return launchMatMul<AM_Conv1x1, BM_RowsK>( stream, args, 1, vec );
+		return launchMatMul<AM_Conv1x1, BM_RowsK>( stream, args, 1, vec, fixedMeeting );
 	}
 	if( d.channels % 4 != 0 && d.dilationWidth == 1
 		&& fitsBuffer( 1, 0, static_cast<long long>( d.batch ) * d.height * d.width * d.channels )
@@ -1534,9 +1644,9 @@ int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* sour
 		args.AFloats = d.batch * d.height * d.width * d.channels;
 		args.BFloats = d.filterCount * d.filterHeight * args.RowK;
 		args.K = d.filterHeight * args.RowPitch; // reduction length as the kernel walks it; Ldb keeps the filter's own
-		return launchMatMul<AM_ConvRows, BM_RowsK>( stream, args, 1, true );
+		return launchMatMul<AM_ConvRows, BM_RowsK>( stream, args, 1, true, fixedMeeting );
 	}
-	return launchMatMul<AM_Conv, BM_RowsK>( stream, args, 1, vec );
+	return launchMatMul<AM_Conv, BM_RowsK>( stream, args, 1, vec, fixedMeeting );
 }
 
 // ---- gradients of the convolution ------------------------------------------------------------------------------
@@ -1872,6 +1982,18 @@ int nhBlobConvolution( nhStream s, const nhConvDesc* d, const float* source, con
 	const float* freeTerm, float* result )
 {
 	return nhBlobConvolutionWithActivation( s, d, source, filter, freeTerm, NH_ACT_NONE, 0.f, result );
+}
+
+int nhStreamBindPool( nhStream s, nhPool pool )
+{
+	return bindSliceScratchPool( toStream( s ), pool );
+}
+
+int nhStreamReleaseScratch( nhStream s )
+{
+	NH_HIP( hipStreamSynchronize( toStream( s ) ) );
+	releaseSliceScratch( toStream( s ), false );
+	return NH_OK;
 }
 
 int nhBlobConvolutionWithActivation( nhStream s, const nhConvDesc* d, const float* source, const float* filter,

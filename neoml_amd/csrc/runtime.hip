@@ -18,7 +18,9 @@ void setLastError( const char* fmt, ... )
 } // namespace nh
 
 namespace nh {
-int checkSequenceGiveUps(); // dnn_ops.hip
+// dnn_ops.hip
+int checkSequenceGiveUps( hipStream_t stream );
+void releaseSequenceStream( hipStream_t stream );
 }
 
 using namespace nh;
@@ -89,7 +91,8 @@ int nhStreamDestroy( nhStream stream )
 	if( stream != nullptr ) {
 		// what the library keeps for the stream goes with it ( a later stream may be handed the same handle )
 		NH_HIP( hipStreamSynchronize( toStream( stream ) ) );
-		releaseSliceScratch( toStream( stream ) );
+		releaseSliceScratch( toStream( stream ), true );
+		releaseSequenceStream( toStream( stream ) );
 		NH_HIP( hipStreamDestroy( toStream( stream ) ) );
 	}
 	return NH_OK;
@@ -98,7 +101,7 @@ int nhStreamDestroy( nhStream stream )
 int nhStreamSynchronize( nhStream stream )
 {
 	NH_HIP( hipStreamSynchronize( toStream( stream ) ) );
-	return checkSequenceGiveUps();
+	return checkSequenceGiveUps( toStream( stream ) );
 }
 
 int nhRawAlloc( void** ptr, size_t size )
@@ -138,7 +141,7 @@ int nhCopyDeviceToHost( nhStream stream, void* dst, const void* src, size_t size
 	NH_REQUIRE( dst != nullptr && src != nullptr );
 	NH_HIP( hipMemcpyAsync( dst, src, size, hipMemcpyDeviceToHost, toStream( stream ) ) );
 	NH_HIP( hipStreamSynchronize( toStream( stream ) ) );
-	return checkSequenceGiveUps();
+	return checkSequenceGiveUps( toStream( stream ) );
 }
 
 int nhCopyDeviceToDevice( nhStream stream, void* dst, const void* src, size_t size )

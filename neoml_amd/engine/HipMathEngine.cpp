@@ -87,6 +87,8 @@ CHipMathEngine::CHipMathEngine( int deviceIndex, size_t memoryLimit, int /*flags
 	NH_CALL( nhGetDeviceInfo( device, deviceName, &deviceTotalMemory, nullptr, nullptr, nullptr ) );
 	NH_CALL( nhStreamCreate( &stream ) );
 	NH_CALL( nhPoolCreate( &pool, 0, memoryLimit ) );
+	// what the kernels allocate behind the scenes for this stream is charged to the engine's pool
+	NH_CALL( nhStreamBindPool( stream, pool ) );
 	initialized = true;
 }
 
@@ -96,9 +98,12 @@ CHipMathEngine::~CHipMathEngine()
 		nhStreamSynchronize( stream );
 	}
 	for( auto& t : hostBuffers ) {
-		for( CHostBuffer& b : t.second ) {
+		for( CHostBuffer& b : t.second.Blocks ) {
 			nhHostFree( b.Ptr );
 		}
+	}
+	if( stream != nullptr ) {
+		nhStreamBindPool( stream, nullptr ); // the stream's scratch goes back to the pool before the pool goes
 	}
 	if( pool != nullptr ) {
 		nhPoolDestroy( pool );
@@ -989,11 +994,20 @@ void CHipMathEngine::CleanUp()
 	{
 		std::lock_guard<std::mutex> lock( hostMutex );
 		auto it = hostBuffers.find( std::this_thread::get_id() );
-		if( it != hostBuffers.end() && it->second.empty() ) {
-			hostBuffers.erase( it );
+		if( it != hostBuffers.end() ) {
+			CHostStack& stack = it->second;
+			while( stack.Blocks.size() > stack.Depth ) {
+				nhHostFree( stack.Blocks.back().Ptr );
+				stack.Blocks.pop_back();
+			}
+			if( stack.Blocks.empty() ) {
+				hostBuffers.erase( it );
+			}
 		}
 	}
 	CleanUpSpecial();
+	// the scratch block the kernels keep for the stream came from the pool: back it goes, then the pool lets go
+	NH_CALL( nhStreamReleaseScratch( stream ) );
 	NH_CALL( nhPoolCleanUp( pool ) );
 }
 
@@ -1008,16 +1022,30 @@ void* CHipMathEngine::GetBuffer( const CMemoryHandle& handle, size_t pos, size_t
 {
 	OWN( handle );
 	constexpr size_t headerSize = 2 * sizeof( size_t );
-	void* block = nullptr;
-	NH_CALL( nhHostAlloc( &block, size + headerSize ) );
-	size_t* header = static_cast<size_t*>( block );
-	header[0] = pos;
-	header[1] = size;
-	char* data = static_cast<char*>( block ) + headerSize;
+	char* block = nullptr;
 	{
 		std::lock_guard<std::mutex> lock( hostMutex );
-		hostBuffers[std::this_thread::get_id()].push_back( CHostBuffer{ static_cast<char*>( block ), size + headerSize } );
+		CHostStack& stack = hostBuffers[std::this_thread::get_id()];
+		const size_t need = size + headerSize;
+		if( stack.Blocks.size() > stack.Depth && stack.Blocks[stack.Depth].Size < need ) {
+			// the idle block at this depth is too small; the ones behind it are idle too
+			while( stack.Blocks.size() > stack.Depth ) {
+				nhHostFree( stack.Blocks.back().Ptr );
+				stack.Blocks.pop_back();
+			}
+		}
+		if( stack.Blocks.size() == stack.Depth ) {
+			void* fresh = nullptr;
+			NH_CALL( nhHostAlloc( &fresh, need ) );
+			stack.Blocks.push_back( CHostBuffer{ static_cast<char*>( fresh ), need } );
+		}
+		block = stack.Blocks[stack.Depth].Ptr;
+		++stack.Depth;
 	}
+	size_t* header = reinterpret_cast<size_t*>( block );
+	header[0] = pos;
+	header[1] = size;
+	char* data = block + headerSize;
 	if( exchange ) {
 		NH_CALL( nhCopyDeviceToHost( stream, data, static_cast<char*>( CMemoryHandleInternal::GetRaw( handle ) ) + pos, size ) );
 	}
@@ -1031,16 +1059,17 @@ void CHipMathEngine::ReleaseBuffer( const CMemoryHandle& handle, void* ptr, bool
 	char* block = static_cast<char*>( ptr ) - headerSize;
 	{
 		std::lock_guard<std::mutex> lock( hostMutex );
-		std::vector<CHostBuffer>& stack = hostBuffers[std::this_thread::get_id()];
-		ASSERT_EXPR( !stack.empty() && stack.back().Ptr == block );
-		stack.pop_back();
+		CHostStack& stack = hostBuffers[std::this_thread::get_id()];
+		ASSERT_EXPR( stack.Depth > 0 && stack.Blocks[stack.Depth - 1].Ptr == block );
 	}
 	if( exchange ) {
+		// ( waits for the copy: the block may be handed out again right away )
 		const size_t* header = reinterpret_cast<const size_t*>( block );
 		NH_CALL( nhCopyHostToDevice( stream, static_cast<char*>( CMemoryHandleInternal::GetRaw( handle ) ) + header[0],
 			ptr, header[1] ) );
 	}
-	NH_CALL( nhHostFree( block ) );
+	std::lock_guard<std::mutex> lock( hostMutex );
+	--hostBuffers[std::this_thread::get_id()].Depth;
 }
 
 void CHipMathEngine::DataExchangeRaw( const CMemoryHandle& result, const void* source, size_t size )

@@ -393,13 +393,19 @@ private:
 	char deviceName[256];
 	bool initialized;
 
-	// pinned host staging blocks handed out by GetBuffer, per thread, strictly LIFO
+	// Pinned host staging blocks handed out by GetBuffer, per thread, strictly LIFO. Allocating and freeing pinned
+	// memory synchronises the device, so the blocks are kept: the first Depth blocks of a thread are handed out, the
+	// ones behind them wait for the next GetBuffer at that depth (regrown when too small); CleanUp frees the idle ones.
 	struct CHostBuffer {
 		char* Ptr;
 		size_t Size;
 	};
+	struct CHostStack {
+		std::vector<CHostBuffer> Blocks;
+		size_t Depth = 0;
+	};
 	mutable std::mutex hostMutex;
-	std::unordered_map<std::thread::id, std::vector<CHostBuffer>> hostBuffers;
+	std::unordered_map<std::thread::id, CHostStack> hostBuffers;
 
 	void check( int code, const char* what, int line ) const;
 	template<class T> T* raw( const CTypedMemoryHandle<T>& handle ) const;

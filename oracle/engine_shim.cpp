@@ -959,6 +959,37 @@ SHIM_API int shim_clean_up( void* engine )
 	return guarded( [&]() { static_cast<IMathEngine*>( engine )->CleanUp(); } );
 }
 
+// IPerformanceCounters of the engine (PerformanceCounters.h:27-60), as CDnn::EnableProfile drives them: Synchronise(),
+// work, Synchronise(), read. Two measurements, a small and a large element-wise pass; name64 receives counter 0's name.
+SHIM_API int shim_performance_counters( void* engine, int smallSize, int largeSize, int repeats, char* name64, int* counterCount,
+	unsigned long long* smallValue, unsigned long long* largeValue )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		CFloatBlob in( e, largeSize ), out( e, largeSize );
+		e.VectorFill( in.Handle(), 1.5f, largeSize );
+		IPerformanceCounters* counters = e.CreatePerformanceCounters( true );
+		if( counters == nullptr ) {
+			throw std::runtime_error( "CreatePerformanceCounters returned null" );
+		}
+		*counterCount = static_cast<int>( counters->size() );
+		std::strncpy( name64, ( *counters )[0].Name, 63 );
+		name64[63] = 0;
+		counters->Synchronise();
+		for( int i = 0; i < repeats; ++i ) {
+			e.VectorAbs( in.Const(), out.Handle(), smallSize );
+		}
+		counters->Synchronise();
+		*smallValue = ( *counters )[0].Value;
+		for( int i = 0; i < repeats; ++i ) {
+			e.VectorAbs( in.Const(), out.Handle(), largeSize );
+		}
+		counters->Synchronise();
+		*largeValue = ( *counters )[0].Value;
+		delete counters;
+	} );
+}
+
 // probe for a method outside the implemented paths (asserts on engines that do not implement it)
 SHIM_API int shim_vector_power( void* engine, float exponent, const float* first, float* result, int n )
 {

@@ -33,6 +33,83 @@ def test_engine_identity_and_memory_interface():
     assert pools.value == 0
 
 
+def test_performance_counters_measure_the_device_work_between_synchronise_calls():
+    """IPerformanceCounters as CDnn::EnableProfile uses them (PerformanceCounters.h:27-60): counter 0 is "time ns", its
+    value is the time since the previous Synchronise(), and Synchronise() drains the stream first, so device work shows
+    up in it: 20 passes over 64 M floats (0.5 GB each way per pass, >= 3 ms of HBM time) must read far longer than 20
+    passes over 1 K floats, and longer than the memory system could possibly make them."""
+    s = nhtest.shim()
+    name = ctypes.create_string_buffer(64)
+    count = ctypes.c_int()
+    small, large = ctypes.c_ulonglong(), ctypes.c_ulonglong()
+    n_large = 64 << 20
+    rc = s.shim_performance_counters(nhtest.hip_engine(), 1024, n_large, 20, name, ctypes.byref(count),
+                                     ctypes.byref(small), ctypes.byref(large))
+    assert rc == 0, s.shim_last_error().decode()
+    assert count.value == 1 and name.value == b"time ns"
+    assert small.value > 0
+    floor_ns = 20 * 8 * n_large / 8e12 * 1e9  # 20 passes at the 8 TB/s peak
+    assert large.value > floor_ns, (large.value, floor_ns)
+    assert large.value > 5 * small.value, (small.value, large.value)
+    assert large.value < 2e9  # and it is a time in nanoseconds, not in another unit
+
+
+def _create_engine(limit):
+    lib = ctypes.CDLL(nhtest.ENGINE_LIB, mode=ctypes.RTLD_GLOBAL)
+    lib.CreateHipMathEngine.restype = ctypes.c_void_p
+    lib.CreateHipMathEngine.argtypes = [ctypes.c_int, ctypes.c_size_t, ctypes.c_int]
+    ptr = lib.CreateHipMathEngine(0, limit, 0)
+    assert ptr
+    return ctypes.c_void_p(ptr)
+
+
+def test_memory_limit_covers_the_scratch_of_sliced_convolutions():
+    """Everything the engine allocates counts against memoryLimit (MemoryEngineMixin.cpp:99-115), also the block in
+    which the K slices of a convolution meet. The last ResNet-18 stage at batch 64 (392 tiles, cut into 5 slices) asks
+    for a 30.6 MiB block next to 28 MiB of blobs: without a limit the block shows in the peak and CleanUp gives it
+    back; with a limit that holds the blobs but not the block the convolution still gives the right answer (its slices
+    then meet through atomic adds) and the peak stays under the limit."""
+    nhtest.hip_engine()  # loads the libraries
+    s = nhtest.shim()
+    g = rng(77)
+    x = g.uniform(-1, 1, (64, 7, 7, 512)).astype(np.float32)
+    f = g.normal(0, 1.0 / 68.0, (512, 3, 3, 512)).astype(np.float32)
+    bias = g.uniform(-0.5, 0.5, 512).astype(np.float32)
+    peak, cur, pools = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    stats = lambda e: (s.shim_memory_stats(e, ctypes.byref(peak), ctypes.byref(cur), ctypes.byref(pools)),
+                       peak.value, cur.value, pools.value)[1:]
+    results = {}
+    MiB = 1 << 20
+    for limit in (0, 40 * MiB):
+        eng = _create_engine(limit)
+        try:
+            hip = Cpu("hipeng")
+            hip.eng = (eng,)
+            results[limit] = hip.conv(x, f, bias, 1, 1, 1, 1)
+            p, c, _ = stats(eng)
+            if limit == 0:
+                assert p >= 58 * MiB, p      # blobs (8 + 12 + 8 MiB size classes) and the 32 MiB class of the block
+                assert c >= 30 * MiB, c      # the block stays with the stream ...
+                assert s.shim_clean_up(eng) == 0
+                assert stats(eng)[1] == 0    # ... until CleanUp returns it with the cached blobs
+            else:
+                assert p <= limit, (p, limit)
+        finally:
+            s.shim_destroy_engine(eng)
+    want = Cpu("orc").conv(x[:4], f, bias, 1, 1, 1, 1)
+    assert_close(results[0][:4], want, "sliced convolution, scratch from the pool")
+    assert_close(results[40 * MiB], results[0], "sliced convolution under a memory limit vs without")
+    # a limit below the blobs themselves is the caller's memory error, as on every engine
+    eng = _create_engine(16 * MiB)
+    try:
+        hip = Cpu("hipeng")
+        hip.eng = (eng,)
+        with pytest.raises(RuntimeError, match="memory"):
+            hip.conv(x, f, bias, 1, 1, 1, 1)
+    finally:
+        s.shim_destroy_engine(eng)
+
+
 @pytest.mark.parametrize("op,p0,p1", UNARY_CASES)
 def test_unary(op, p0, p1):
     hip, ref = engines()

@@ -893,6 +893,61 @@ def test_lstm_bounded_wait_gives_up(monkeypatch):
     assert_close(h2, oh, "lstm after a forced give-up")
 
 
+def _enqueue_lstm(h, stream, w_in, w_rec, x):
+    """nhLstm on `stream` without waiting for it; returns the output tensor and what must stay alive."""
+    import torch
+    T, B, In = x.shape
+    H = w_rec.shape[1]
+    with torch.cuda.stream(stream):
+        ws = [h.up(a) for a in (w_in, w_rec, x)]
+        out = h.empty((T, B, H))
+        size = ctypes.c_size_t(0)
+        h.na.check(h.lib.nhLstmWorkspaceSize(H, In, T, B, ctypes.byref(size)))
+        work = torch.empty((size.value + 15) // 4, dtype=torch.float32, device=h.dev)
+        h.call("nhLstm", H, In, h.p(ws[0]), None, h.p(ws[1]), None, 0, T, B, None, None, h.p(ws[2]), None, h.p(out),
+               h.p(work), size.value)
+    return out, (ws, work)
+
+
+def test_lstm_on_two_streams_and_give_up_reported_to_its_own_stream(monkeypatch):
+    """Two one-launch LSTMs issued on two streams without a wait between them: the library orders the second behind the
+    first on the device (each needs the whole device resident), both give the oracle's result. Then a give-up forced
+    from the host (spin limit zero) on the first stream is reported by that stream's next synchronising call only: the
+    other stream's synchronise stays clean."""
+    import torch
+    import neoml_amd
+    h = hip()
+    lib = neoml_amd.load()
+    g = rng(183)
+    T, B, In, H = 48, 64, 32, 256
+    w_in = g.uniform(-0.2, 0.2, (4 * H, In)).astype(np.float32)
+    w_rec = g.uniform(-0.1, 0.1, (4 * H, H)).astype(np.float32)
+    xa = g.uniform(-1, 1, (T, B, In)).astype(np.float32)
+    xb = g.uniform(-1, 1, (T, B, In)).astype(np.float32)
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    pa, pb = ctypes.c_void_p(sa.cuda_stream), ctypes.c_void_p(sb.cuda_stream)
+    torch.cuda.synchronize()
+    out_a, keep_a = _enqueue_lstm(h, sa, w_in, w_rec, xa)
+    out_b, keep_b = _enqueue_lstm(h, sb, w_in, w_rec, xb)
+    assert lib.nhStreamSynchronize(pa) == 0 and lib.nhStreamSynchronize(pb) == 0
+    assert_close(out_a.cpu().numpy(), orc.lstm(w_in, None, w_rec, None, xa)[0], "lstm on stream a")
+    assert_close(out_b.cpu().numpy(), orc.lstm(w_in, None, w_rec, None, xb)[0], "lstm on stream b")
+    # forced give-up on stream a, a regular run on stream b
+    monkeypatch.setenv("NH_LSTM_SPIN_LIMIT", "0")
+    out_a2, keep_a2 = _enqueue_lstm(h, sa, w_in, w_rec, xa)
+    monkeypatch.delenv("NH_LSTM_SPIN_LIMIT")
+    out_b2, keep_b2 = _enqueue_lstm(h, sb, w_in, w_rec, xb)
+    rc_b = lib.nhStreamSynchronize(pb)
+    rc_a = lib.nhStreamSynchronize(pa)
+    assert rc_b == 0
+    assert_close(out_b2.cpu().numpy(), out_b.cpu().numpy(), "lstm on stream b beside a give-up on stream a")
+    assert rc_a in (0, 2)  # 0: every value happened to be there in time
+    if rc_a == 2:
+        assert "gave up" in neoml_amd.last_error()
+    assert lib.nhStreamSynchronize(pa) == 0  # reported once
+    del keep_a, keep_b, keep_a2, keep_b2
+
+
 # ---------------------------------------------------------------------------------------------------------
 # error convention and allocator on the device
 
