@@ -311,6 +311,21 @@ NH_API int nhInitBlobConvolution(nhConvDesc* desc_host);
 NH_API int nhBlobConvolution(nhStream s, const nhConvDesc* desc_host, const float* source, const float* filter,
 	const float* freeTerm, float* result);                                                           /* NME.h:755 */
 
+/* nhBlobConvolution for callers that cannot allocate device memory: code recording a HIP graph, serving loops and
+ * harnesses that forbid hipMalloc. No counterpart in the reference. Same arguments and results as nhBlobConvolution
+ * (bit for bit: the same kernels and the same summation order). Where nhBlobConvolution lets the K slices of a launch
+ * meet in a block it allocates per stream, this one uses a fixed array inside the library's device image: it never
+ * calls hipMalloc / hipFree, also not while the stream is being captured (its counters are cleared by a fill kernel).
+ * Limits: the partial tiles of one launch (sliced tiles x slices x 16 KiB) must fit NH_NOALLOC_SCRATCH_BYTES and the
+ * sliced tiles NH_NOALLOC_MAX_SLICED_TILES, otherwise NH_ERR_ARGUMENT and nothing is launched (the ResNet-18 stages at
+ * batch 64 need up to 38.5 MB). Every GPU the library runs on holds its own copy of the array until the process ends.
+ * All calls on one GPU share that copy: calls that may overlap there (different streams, replays of graphs recorded
+ * from it) race; serialise them. */
+#define NH_NOALLOC_SCRATCH_BYTES (64u << 20)
+#define NH_NOALLOC_MAX_SLICED_TILES 16384
+NH_API int nhBlobConvolutionNoAlloc(nhStream s, const nhConvDesc* desc_host, const float* source, const float* filter,
+	const float* freeTerm, float* result);
+
 /* Gradients of the convolution (NME.h:757-761), same descriptor as the forward pass.
  * Backward: inputDiff = the gradient by the source; freeTerm (per source channel, may be null) is added, as the
  * reference does for the layers that run a convolution backwards as their forward pass. workspace: the filter with its

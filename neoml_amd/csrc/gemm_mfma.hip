@@ -1071,6 +1071,42 @@ struct CSliceMeeting {
 	size_t CounterCount;
 };
 
+// The meeting place of nhBlobConvolutionNoAlloc: a fixed array in the library's own device image, one copy per GPU,
+// held from the moment the library is loaded on that GPU until the process ends. Partial tiles first, the arrival
+// counters behind them. Every call on a GPU shares that GPU's copy, so calls that overlap there race.
+constexpr size_t NoAllocPartialFloats = NH_NOALLOC_SCRATCH_BYTES / sizeof( float );
+constexpr size_t NoAllocCounters = NH_NOALLOC_MAX_SLICED_TILES;
+static __device__ __align__( 256 ) unsigned char scratch[NH_NOALLOC_SCRATCH_BYTES + NoAllocCounters * sizeof( unsigned )];
+
+// The array's address on the current device. In host code the array's name is only a stand-in for the symbol, not a
+// device address: the address is asked for once per device, with that device current, and kept.
+constexpr int MaxDevices = 64;
+static std::mutex noAllocLock;
+static unsigned char* noAllocScratch[MaxDevices] = {};
+
+static int noAllocMeeting( CSliceMeeting& meeting )
+{
+	int device = 0;
+	NH_HIP( hipGetDevice( &device ) );
+	if( device < 0 || device >= MaxDevices ) {
+		setLastError( "nhBlobConvolutionNoAlloc: device index %d is beyond the %d devices the library keeps scratch for", device, MaxDevices );
+		return NH_ERR_UNSUPPORTED;
+	}
+	std::lock_guard<std::mutex> guard( noAllocLock );
+	if( noAllocScratch[device] == nullptr ) {
+		unsigned char* ptr = nullptr;
+		NH_HIP( hipGetSymbolAddress( reinterpret_cast<void**>( &ptr ), HIP_SYMBOL( scratch ) ) );
+		NH_REQUIRE( ptr != nullptr );
+		noAllocScratch[device] = ptr;
+	}
+	unsigned char* base = noAllocScratch[device];
+	meeting.Partials = reinterpret_cast<float*>( base );
+	meeting.PartialFloats = NoAllocPartialFloats;
+	meeting.Counters = reinterpret_cast<unsigned*>( base + NH_NOALLOC_SCRATCH_BYTES );
+	meeting.CounterCount = NoAllocCounters;
+	return NH_OK;
+}
+
 // a fill kernel rather than a memset: callers may be recording a graph
 __global__ __launch_bounds__( 256 ) void clearCountersKernel( unsigned* counters, int count )
 {
@@ -1982,6 +2018,25 @@ int nhBlobConvolution( nhStream s, const nhConvDesc* d, const float* source, con
 	const float* freeTerm, float* result )
 {
 	return nhBlobConvolutionWithActivation( s, d, source, filter, freeTerm, NH_ACT_NONE, 0.f, result );
+}
+
+int nhBlobConvolutionNoAlloc( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
+	const float* freeTerm, float* result )
+{
+	NH_REQUIRE( d != nullptr && source != nullptr && filter != nullptr && result != nullptr );
+	nhConvDesc check = *d;
+	int rc = nhInitBlobConvolution( &check );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( check.resultHeight == d->resultHeight && check.resultWidth == d->resultWidth );
+	CSliceMeeting meeting = {};
+	rc = noAllocMeeting( meeting );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	const CFusedActivation none = { NH_ACT_NONE, 0.f };
+	return convImplicitGemm( toStream( s ), *d, source, filter, freeTerm, result, none, &meeting );
 }
 
 int nhStreamBindPool( nhStream s, nhPool pool )
