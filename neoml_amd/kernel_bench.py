@@ -1,6 +1,6 @@
 """Per-kernel measurements at the sizes of the BASELINE configurations.
 
-    python -m neoml_amd.kernel_bench [--reps N] [--filter substring]
+    python -m neoml_amd.kernel_bench [--reps N] [--filter substring[,substring...]]
 
 Every line is one C-ABI entry point at one shape: time per launch (events on the launch stream around a run of
 back-to-back launches, after a clock warm-up), algorithmic FLOP and bytes (the formulas of the measurement
@@ -43,9 +43,10 @@ def main():
         return torch.empty(shape, device=dev, dtype=torch.float32)
 
     rows = []
+    wanted = [w for w in args.filter.split(",") if w]
 
     def measure(name, fn, flops, nbytes, footprint):
-        if args.filter and args.filter not in name:
+        if wanted and not any(w in name for w in wanted):
             return
         neoml_amd.check(fn())
         torch.cuda.synchronize()
@@ -258,6 +259,12 @@ def main():
         measure("VectorFill (write only) n=%d" % n, lambda: lib.nhVectorFill(stream, P(c), ctypes.c_float(1.5), n), 0, 4 * n, 4 * n)
         a = rand(n)
         measure("VectorSum (read only) n=%d" % n, lambda: lib.nhVectorSum(stream, P(a), n, P(zero)), 0, 4 * n, 4 * n)
+        del a, c
+    if any("calibrate" in w for w in wanted):
+        # a copy of known size (256 MiB read, 256 MiB written): the scale of the FETCH_SIZE / WRITE_SIZE counters
+        n = 1 << 26
+        a, c = rand(n), empty(n)
+        measure("VectorCopy calibrate n=%d" % n, lambda: lib.nhVectorCopy(stream, P(c), P(a), n), 0, 8 * n, 8 * n)
         del a, c
     n = 8192 * 512
     a, c = rand(n), empty(n)
