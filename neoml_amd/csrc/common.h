@@ -113,6 +113,13 @@ __device__ __forceinline__ float4 bufferLoad4( __amdgpu_buffer_rsrc_t rsrc, unsi
 	return make_float4( __uint_as_float( v.x ), __uint_as_float( v.y ), __uint_as_float( v.z ), __uint_as_float( v.w ) );
 }
 
+// Streaming variant: the line is marked for early replacement in the caches ( data that is read once ).
+__device__ __forceinline__ float4 bufferLoad4Stream( __amdgpu_buffer_rsrc_t rsrc, unsigned offset )
+{
+	const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128( rsrc, offset, 0, 2 ); // aux bit 1: nt
+	return make_float4( __uint_as_float( v.x ), __uint_as_float( v.y ), __uint_as_float( v.z ), __uint_as_float( v.w ) );
+}
+
 // The same with a second, wave-uniform byte offset that travels in a scalar register: what a loop adds per iteration
 // costs no vector instruction. The range check looks at the per-lane offset, so OutOfRange still reads as zero.
 __device__ __forceinline__ float4 bufferLoad4( __amdgpu_buffer_rsrc_t rsrc, unsigned offset, unsigned uniformOffset )

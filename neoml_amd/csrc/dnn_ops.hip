@@ -3,6 +3,7 @@
 // recurrence (matrix products on the MFMA kernels + one fused gate kernel per step).
 #include "common.h"
 #include <float.h>
+#include <math.h>
 #include <stdlib.h>
 #include <map>
 #include <mutex>
@@ -101,18 +102,22 @@ void channelwiseConvKernel( const nhConvDesc d, const float* source, const float
 
 // The 3x3 case of the depthwise convolution (every depthwise layer of the MobileNet family), 4 channels per thread.
 // One thread owns a strip WPT output pixels wide and rowsPerItem output rows tall and slides down it with the
-// three input rows of the window in registers: every input row is loaded once per strip instead of once per
-// output row that touches it, and the index arithmetic is paid once per strip. Loads are raw buffer loads, so
-// the zero padding is an out-of-range offset instead of a branch. Workgroups of one XCD cover a contiguous
-// range of strips: the halo rows and columns shared by neighbouring strips meet in that XCD's L2.
-template<int STRIDE, int WPT>
+// input rows of the window in registers: every input row is loaded once per strip instead of once per output row
+// that touches it, and the index arithmetic is paid once per strip. The registers form a ring of 3 + PRE * STRIDE
+// rows: the rows that enter the window for the output row PRE steps ahead are requested before the current row is
+// computed and stored, so a thread always has PRE rows' worth of loads in flight ( the ring turns by renaming: the
+// row loop is unrolled by the ring size, no register is moved ). Loads are raw buffer loads, so the zero padding is an
+// out-of-range offset instead of a branch. Workgroups of one XCD cover a contiguous range of strips: the halo columns
+// shared by neighbouring strips meet in that XCD's L2.
+// STREAM: loads carry the streaming hint ( tensors far larger than the caches, every line used by one strip ).
+template<int STRIDE, int WPT, int PRE, bool STREAM>
 __global__ __launch_bounds__( 256 )
 void channelwiseConv3x3Kernel( const nhConvDesc d, const float* source, const float* filter, const float* freeTerm,
 	float* result, int wGroups, int rowChunks, int rowsPerItem, int totalItems, const CFusedActivation act, int flipTaps )
 {
 	constexpr int NC = ( WPT - 1 ) * STRIDE + 3;
-	constexpr int Keep = 3 - STRIDE; // input rows shared by two consecutive output rows
-	const int item = xcdSwizzle( blockIdx.x, gridDim.x ) * 256 + threadIdx.x;
+	constexpr int Ring = 3 + PRE * STRIDE;
+	const int item = xcdSwizzle( blockIdx.x, gridDim.x ) * blockDim.x + threadIdx.x;
 	if( item >= totalItems ) {
 		return;
 	}
@@ -142,51 +147,55 @@ void channelwiseConv3x3Kernel( const nhConvDesc d, const float* source, const fl
 	}
 	const float4 bias = freeTerm != nullptr ? *reinterpret_cast<const float4*>( freeTerm + c ) : make_float4( 0.f, 0.f, 0.f, 0.f );
 
-	float4 rows[3][NC];
+	// input row hi of the strip lives in ring[ ( hi - hiFirst ) % Ring ]
+	float4 ring[Ring][NC];
+	const int hiFirst = ho0 * STRIDE - d.paddingHeight;
+	const int hiLast = ( hoEnd - 1 ) * STRIDE - d.paddingHeight + 2; // last input row any output row of the strip needs
 	auto loadRow = [&]( float4* row, int hi ) {
-		const bool valid = hi >= 0 && hi < d.height;
+		const bool valid = hi >= 0 && hi < d.height && hi <= hiLast;
 		const unsigned rowOff = imageBytes + static_cast<unsigned>( hi ) * rowBytes;
 #pragma unroll
 		for( int j = 0; j < NC; ++j ) {
 			// a valid row offset is below 2 GiB, so adding an out-of-range column stays out of range
-			row[j] = bufferLoad4( image, valid ? rowOff + colOff[j] : OutOfRange );
+			const unsigned offset = valid ? rowOff + colOff[j] : OutOfRange;
+			row[j] = STREAM ? bufferLoad4Stream( image, offset ) : bufferLoad4( image, offset );
 		}
 	};
-	int hi = ho0 * STRIDE - d.paddingHeight;
 #pragma unroll
-	for( int r = 0; r < Keep; ++r ) {
-		loadRow( rows[r], hi + r );
+	for( int r = 0; r < Ring - STRIDE; ++r ) {
+		loadRow( ring[r], hiFirst + r );
 	}
 	float* out = result + ( ( static_cast<long long>( n ) * d.resultHeight + ho0 ) * d.resultWidth + wo0 ) * d.channels + c;
 	const long long outRow = static_cast<long long>( d.resultWidth ) * d.channels;
-	for( int ho = ho0; ho < hoEnd; ++ho ) {
+	for( int hoBase = ho0; hoBase < hoEnd; hoBase += Ring ) {
 #pragma unroll
-		for( int r = Keep; r < 3; ++r ) {
-			loadRow( rows[r], hi + r );
-		}
+		for( int k = 0; k < Ring; ++k ) {
+			if( hoBase + k < hoEnd ) {
+				// output row hoBase + k: its window starts at ring position ( k * STRIDE ) % Ring ( Ring output rows
+				// advance the window by Ring * STRIDE rows: a whole number of turns ); the rows PRE steps ahead go in
+				// behind the ones already there
 #pragma unroll
-		for( int j = 0; j < WPT; ++j ) {
-			float4 acc = bias;
-#pragma unroll
-			for( int kh = 0; kh < 3; ++kh ) {
-#pragma unroll
-				for( int kw = 0; kw < 3; ++kw ) {
-					acc = CChanVec<4>::fma( rows[kh][j * STRIDE + kw], f[kh * 3 + kw], acc );
+				for( int r = 0; r < STRIDE; ++r ) {
+					const int ahead = k * STRIDE + Ring - STRIDE + r;
+					loadRow( ring[ahead % Ring], hiFirst + ( hoBase - ho0 ) * STRIDE + ahead );
 				}
-			}
-			if( wo0 + j < d.resultWidth ) {
-				*reinterpret_cast<float4*>( out + j * d.channels ) = CChanVec<4>::activate( acc, act );
+#pragma unroll
+				for( int j = 0; j < WPT; ++j ) {
+					float4 acc = bias;
+#pragma unroll
+					for( int kh = 0; kh < 3; ++kh ) {
+#pragma unroll
+						for( int kw = 0; kw < 3; ++kw ) {
+							acc = CChanVec<4>::fma( ring[( k * STRIDE + kh ) % Ring][j * STRIDE + kw], f[kh * 3 + kw], acc );
+						}
+					}
+					if( wo0 + j < d.resultWidth ) {
+						*reinterpret_cast<float4*>( out + j * d.channels ) = CChanVec<4>::activate( acc, act );
+					}
+				}
+				out += outRow;
 			}
 		}
-#pragma unroll
-		for( int r = 0; r < Keep; ++r ) {
-#pragma unroll
-			for( int j = 0; j < NC; ++j ) {
-				rows[r][j] = rows[r + STRIDE][j];
-			}
-		}
-		hi += STRIDE;
-		out += outRow;
 	}
 }
 
@@ -1705,20 +1714,115 @@ static int poolingImpl( nhStream s, const nhPoolingDesc* d, const float* source,
 	return NH_OK;
 }
 
+// ---- strips of the 3x3 depthwise kernel ------------------------------------------------------------------------
+// How wide and how tall the strips of a launch are decides three things at once: how many input rows are read twice
+// ( every strip re-reads the two rows above its first output row ), how many bytes the device has in flight ( a wave asks
+// for one row of its strip ahead; about 10 MB in flight saturate HBM ), and how evenly the waves fill the device ( waves
+// beyond what is resident at once form a second, partly filled round ). Measured on the three large layers of a
+// MobileNetV2 at batch 128 with 7 to 56 rows per strip: the estimate below picks strips within 2.5 % of the best of each
+// ( 5.5 / 6.05 / 5.6 TB/s ). Strips of more than 30 rows were slower than it says on every shape, hence the last term.
+static double stripTimeEstimate( const nhConvDesc& d, int stride, int wpt, int chunks, int residentWaves )
+{
+	const int rows = ceilDiv( d.resultHeight, chunks );
+	const double waves = static_cast<double>( d.batch ) * ceilDiv( d.resultWidth, wpt ) * ( d.channels / 4 ) * chunks / 64.0;
+	const int columns = ( wpt - 1 ) * stride + 3;
+	const double rounds = ceil( waves / residentWaves );
+	const double fill = waves / ( rounds * residentWaves );
+	const double inFlight = ( waves < residentWaves ? waves : residentWaves ) * 64.0 * columns * stride * 16.0;
+	const double haloRows = static_cast<double>( rows * stride + 2 ) / ( rows * stride );
+	const double haloColumns = pow( static_cast<double>( columns ) / ( wpt * stride ), 0.1 ); // mostly served by the L1
+	double time = static_cast<double>( d.height ) * d.width * haloRows * haloColumns
+		+ static_cast<double>( d.resultHeight ) * d.resultWidth;
+	if( inFlight < 10e6 ) {
+		time *= 10e6 / inFlight;
+	}
+	if( rounds > 1 ) {
+		time *= 1.0 + 0.5 * ( 1.0 / fill - 1.0 );
+	}
+	if( rows > 30 ) {
+		time /= 0.85;
+	}
+	return time;
+}
+
+static int residentWavesFor( const void* kernel )
+{
+	static std::mutex lock;
+	static std::map<std::pair<int, const void*>, int> known;
+	int device = 0;
+	( void )hipGetDevice( &device );
+	std::lock_guard<std::mutex> guard( lock );
+	int& waves = known[std::make_pair( device, kernel )];
+	if( waves == 0 ) {
+		int perUnit = 0, units = 0;
+		if( hipOccupancyMaxActiveBlocksPerMultiprocessor( &perUnit, kernel, 64, 0 ) != hipSuccess
+			|| hipDeviceGetAttribute( &units, hipDeviceAttributeMultiprocessorCount, device ) != hipSuccess || perUnit <= 0 || units <= 0 )
+		{
+			( void )hipGetLastError();
+			perUnit = 4;
+			units = 256;
+		}
+		waves = perUnit * units;
+	}
+	return waves;
+}
+
+template<int STRIDE, int WPT, bool STREAM>
+static int channelwise3x3Launch( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
+	const float* freeTerm, float* result, const CFusedActivation& act, bool flipTaps, int rowChunks )
+{
+	const int wGroups = ceilDiv( d->resultWidth, WPT );
+	const long long perRow = static_cast<long long>( d->batch ) * wGroups * ( d->channels / 4 );
+	const int rowsPerItem = ceilDiv( d->resultHeight, rowChunks );
+	rowChunks = ceilDiv( d->resultHeight, rowsPerItem );
+	const long long items = perRow * rowChunks;
+	// workgroups of one wave: the strips need nothing from one another, and single waves spread most evenly
+	hipLaunchKernelGGL( ( channelwiseConv3x3Kernel<STRIDE, WPT, 1, STREAM> ), dim3( static_cast<unsigned>( ( items + 63 ) / 64 ) ),
+		dim3( 64 ), 0, toStream( s ), *d, source, filter, freeTerm, result, wGroups, rowChunks, rowsPerItem,
+		static_cast<int>( items ), act, flipTaps ? 1 : 0 );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
 template<int STRIDE, int WPT>
 static int channelwise3x3Impl( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
 	const float* freeTerm, float* result, const CFusedActivation& act, bool flipTaps = false )
 {
-	const int wGroups = ceilDiv( d->resultWidth, WPT );
-	const long long perRow = static_cast<long long>( d->batch ) * wGroups * ( d->channels / 4 );
-	int rowChunks = 1, rowsPerItem = 1;
-	chooseRowChunks( perRow, d->resultHeight, 4, 3072, &rowChunks, &rowsPerItem );
-	const long long items = perRow * rowChunks;
-	hipLaunchKernelGGL( ( channelwiseConv3x3Kernel<STRIDE, WPT> ), dim3( static_cast<unsigned>( ( items + 255 ) / 256 ) ), dim3( 256 ), 0,
-		toStream( s ), *d, source, filter, freeTerm, result, wGroups, rowChunks, rowsPerItem, static_cast<int>( items ), act,
-		flipTaps ? 1 : 0 );
-	NH_LAUNCH_CHECK();
-	return NH_OK;
+	const long long sourceBytes = static_cast<long long>( d->batch ) * d->height * d->width * d->channels * 4;
+	if( sourceBytes < ( 64LL << 20 ) ) {
+		// served by the caches: what counts is how many waves work at once, not what is read twice
+		const long long perRow = static_cast<long long>( d->batch ) * ceilDiv( d->resultWidth, WPT ) * ( d->channels / 4 );
+		int rowChunks = 1, rowsPerItem = 1;
+		chooseRowChunks( perRow, d->resultHeight, 4, 3072, &rowChunks, &rowsPerItem );
+		return channelwise3x3Launch<STRIDE, WPT, false>( s, d, source, filter, freeTerm, result, act, flipTaps, rowChunks );
+	}
+	// Strips twice as wide halve the columns read twice but need twice the registers: measured, they pay at stride 2
+	// ( 9 columns for 4 output pixels instead of 5 for 2 ) and lose at stride 1.
+	constexpr int Widths = STRIDE == 2 ? 2 : 1;
+	const int resident[2] = {
+		residentWavesFor( reinterpret_cast<const void*>( &channelwiseConv3x3Kernel<STRIDE, WPT, 1, true> ) ),
+		residentWavesFor( reinterpret_cast<const void*>( &channelwiseConv3x3Kernel<STRIDE, WPT * 2, 1, true> ) ) };
+	bool wide = false;
+	int chunks = 1;
+	double best = -1;
+	const int mostChunks = ceilDiv( d->resultHeight, 4 );
+	for( int w = 0; w < Widths; ++w ) {
+		for( int c = 1; c <= mostChunks; ++c ) {
+			if( c > 1 && ceilDiv( d->resultHeight, c ) == ceilDiv( d->resultHeight, c - 1 ) ) {
+				continue; // the same strip height
+			}
+			const double time = stripTimeEstimate( *d, STRIDE, w == 0 ? WPT : WPT * 2, c, resident[w] );
+			if( best < 0 || time < best ) {
+				best = time;
+				wide = w != 0;
+				chunks = c;
+			}
+		}
+	}
+	if( wide ) {
+		return channelwise3x3Launch<STRIDE, WPT * 2, true>( s, d, source, filter, freeTerm, result, act, flipTaps, chunks );
+	}
+	return channelwise3x3Launch<STRIDE, WPT, true>( s, d, source, filter, freeTerm, result, act, flipTaps, chunks );
 }
 
 template<int STRIDE, int WPT>

@@ -18,7 +18,26 @@ template<typename T> struct CVec4;
 template<> struct CVec4<float> { typedef float4 Type; };
 template<> struct CVec4<int> { typedef int4 Type; };
 
-template<int NIN, typename TIn, typename TOut, typename F, bool VEC>
+// 128-bit access with the streaming hint: the line is marked for early replacement in the caches. Vectors far larger
+// than the caches are read and written once; measured on MI355X, a copy of 617 MB goes from 5.7 to 6.3 TB/s with it.
+template<typename V> __device__ __forceinline__ V loadStreaming( const V* p )
+{
+	typedef unsigned raw4 __attribute__( ( ext_vector_type( 4 ) ) );
+	const raw4 r = __builtin_nontemporal_load( reinterpret_cast<const raw4*>( p ) );
+	V v;
+	__builtin_memcpy( &v, &r, sizeof( V ) );
+	return v;
+}
+template<typename V> __device__ __forceinline__ void storeStreaming( V* p, const V& v )
+{
+	typedef unsigned raw4 __attribute__( ( ext_vector_type( 4 ) ) );
+	raw4 r;
+	__builtin_memcpy( &r, &v, sizeof( V ) );
+	__builtin_nontemporal_store( r, reinterpret_cast<raw4*>( p ) );
+}
+
+// STREAM bit 0: streaming loads, bit 1: streaming stores ( vector path only )
+template<int NIN, typename TIn, typename TOut, typename F, bool VEC, int STREAM = 0>
 __global__ __launch_bounds__( EltThreads )
 void eltwiseKernel( const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, F f )
 {
@@ -33,9 +52,15 @@ void eltwiseKernel( const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, 
 		for( int u = 0; u < EltUnroll; ++u ) {
 			const int i = base + u * EltThreads;
 			if( i < n4 ) {
-				if( NIN >= 1 ) va[u] = reinterpret_cast<const VIn*>( a )[i];
-				if( NIN >= 2 ) vb[u] = reinterpret_cast<const VIn*>( b )[i];
-				if( NIN >= 3 ) vc[u] = reinterpret_cast<const VIn*>( c )[i];
+				if( ( STREAM & 1 ) != 0 ) {
+					if( NIN >= 1 ) va[u] = loadStreaming( reinterpret_cast<const VIn*>( a ) + i );
+					if( NIN >= 2 ) vb[u] = loadStreaming( reinterpret_cast<const VIn*>( b ) + i );
+					if( NIN >= 3 ) vc[u] = loadStreaming( reinterpret_cast<const VIn*>( c ) + i );
+				} else {
+					if( NIN >= 1 ) va[u] = reinterpret_cast<const VIn*>( a )[i];
+					if( NIN >= 2 ) vb[u] = reinterpret_cast<const VIn*>( b )[i];
+					if( NIN >= 3 ) vc[u] = reinterpret_cast<const VIn*>( c )[i];
+				}
 			}
 		}
 #pragma unroll
@@ -47,7 +72,11 @@ void eltwiseKernel( const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, 
 				r.y = f( va[u].y, vb[u].y, vc[u].y );
 				r.z = f( va[u].z, vb[u].z, vc[u].z );
 				r.w = f( va[u].w, vb[u].w, vc[u].w );
-				reinterpret_cast<VOut*>( out )[i] = r;
+				if( ( STREAM & 2 ) != 0 ) {
+					storeStreaming( reinterpret_cast<VOut*>( out ) + i, r );
+				} else {
+					reinterpret_cast<VOut*>( out )[i] = r;
+				}
 			}
 		}
 		// tail of up to 3 elements
@@ -91,7 +120,17 @@ static int launchEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 		&& ( NIN < 3 || isAligned16( c ) ) && n >= 4;
 	const int perBlock = EltThreads * EltUnroll * 4;
 	const int blocks = ceilDiv( n, perBlock );
-	if( vec ) {
+	// Vectors that cannot stay in the 256 MB last-level cache next to their result are read with the streaming hint
+	// ( 51 M floats: 5.7 -> 6.8 TB/s ), the largest ones are written with it too ( 154 M floats: 5.8 -> 6.1 TB/s; for the
+	// mid-sized ones streaming stores cost what streaming loads gain ). Below that the hint only loses cache hits.
+	constexpr int StreamLoadsFrom = 24 << 20, StreamStoresFrom = 100 << 20;
+	if( vec && NIN >= 1 && n >= StreamStoresFrom ) {
+		hipLaunchKernelGGL( ( eltwiseKernel<NIN, TIn, TOut, F, true, 3> ), dim3( blocks ), dim3( EltThreads ), 0, toStream( s ),
+			a, b, c, out, n, f );
+	} else if( vec && NIN >= 1 && n >= StreamLoadsFrom ) {
+		hipLaunchKernelGGL( ( eltwiseKernel<NIN, TIn, TOut, F, true, 1> ), dim3( blocks ), dim3( EltThreads ), 0, toStream( s ),
+			a, b, c, out, n, f );
+	} else if( vec ) {
 		hipLaunchKernelGGL( ( eltwiseKernel<NIN, TIn, TOut, F, true> ), dim3( blocks ), dim3( EltThreads ), 0, toStream( s ),
 			a, b, c, out, n, f );
 	} else {
