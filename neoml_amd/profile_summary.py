@@ -34,7 +34,7 @@ def _demangle(names):
         return {n: n for n in names}
 
 
-def summarize(path, match, demangle, out=sys.stdout):
+def summarize(path, match, demangle, out=sys.stdout, width=110):
     conn = sqlite3.connect(path)
     suf = _suffix(conn, "rocpd_kernel_dispatch")
     if suf is None:
@@ -48,10 +48,10 @@ def summarize(path, match, demangle, out=sys.stdout):
     keep = lambda name: not match or any(m in name or m in names[name] for m in match)
     total = sum(r[6] for r in rows) or 1.0
     print("== %s" % path, file=out)
-    print("%-110s %16s %6s %10s %10s %6s" % ("kernel", "grid (work-items)", "calls", "avg_us", "total_ms", "share"), file=out)
+    print("%-*s %16s %6s %10s %10s %6s" % (width, "kernel", "grid (work-items)", "calls", "avg_us", "total_ms", "share"), file=out)
     for name, gx, gy, gz, calls, avg_us, total_ms in rows:
         if keep(name):
-            print("%-110s %16s %6d %10.2f %10.3f %5.1f%%" % (names[name][:110], "%dx%dx%d" % (gx, gy, gz), calls, avg_us,
+            print("%-*s %16s %6d %10.2f %10.3f %5.1f%%" % (width, names[name][:width], "%dx%dx%d" % (gx, gy, gz), calls, avg_us,
                                                               total_ms, 100 * total_ms / total), file=out)
     psuf = _suffix(conn, "rocpd_pmc_event")
     if psuf is None or conn.execute("select count(*) from rocpd_pmc_event%s" % psuf).fetchone()[0] == 0:
@@ -61,10 +61,22 @@ def summarize(path, match, demangle, out=sys.stdout):
              "sum(e.value) / count(distinct d.id) from rocpd_pmc_event%s e join rocpd_info_pmc%s p on e.pmc_id = p.id "
              "join rocpd_kernel_dispatch%s d on e.event_id = d.event_id join rocpd_info_kernel_symbol%s s on d.kernel_id = s.id "
              "group by s.kernel_name, d.grid_size_x, d.grid_size_y, d.grid_size_z, p.name order by 1, 2, 5" % (psuf, psuf, psuf, psuf))
+    values = {}
     for name, gx, gy, gz, counter, calls, value in conn.execute(query):
         if keep(name):
-            print("%-110s %16s %-28s calls=%5d per_dispatch=%.1f" % (names.get(name, name)[:110], "%dx%dx%d" % (gx, gy, gz),
+            print("%-*s %16s %-28s calls=%5d per_dispatch=%.1f" % (width, names.get(name, name)[:width], "%dx%dx%d" % (gx, gy, gz),
                                                                    counter, calls, value), file=out)
+            values.setdefault((name, gx, gy, gz), {})[counter] = value
+    derived = [(k, v) for k, v in values.items() if "SQ_VALU_MFMA_BUSY_CYCLES" in v and "SQ_BUSY_CU_CYCLES" in v]
+    if derived:
+        # a compute unit has four SIMDs, each with its own matrix pipe; SQ_BUSY_CU_CYCLES counts the cycles a unit holds waves
+        print("\nmatrix pipe busy = SQ_VALU_MFMA_BUSY_CYCLES / ( 4 * SQ_BUSY_CU_CYCLES )", file=out)
+        for (name, gx, gy, gz), v in derived:
+            line = "%-*s %16s %5.1f%%" % (width, names.get(name, name)[:width], "%dx%dx%d" % (gx, gy, gz),
+                                           100.0 * v["SQ_VALU_MFMA_BUSY_CYCLES"] / (4.0 * v["SQ_BUSY_CU_CYCLES"]))
+            if "SQ_WAIT_INST_ANY" in v and "SQ_WAVE_CYCLES" in v:
+                line += "   waves waiting on an instruction: %4.1f%% of wave cycles" % (100.0 * v["SQ_WAIT_INST_ANY"] / v["SQ_WAVE_CYCLES"])
+            print(line, file=out)
 
 
 def main():
@@ -72,10 +84,11 @@ def main():
     ap.add_argument("databases", nargs="+")
     ap.add_argument("--match", default="", help="only kernels whose (demangled) name contains one of these substrings")
     ap.add_argument("--demangle", action="store_true")
+    ap.add_argument("--width", type=int, default=110, help="columns kept of a kernel name")
     args = ap.parse_args()
     match = [m for m in args.match.split(",") if m]
     for path in args.databases:
-        summarize(path, match, args.demangle)
+        summarize(path, match, args.demangle, width=args.width)
         print()
 
 
