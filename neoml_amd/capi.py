@@ -8,7 +8,8 @@ import os
 import re
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "lib", "libneoml_hip.so")
+# NEOML_HIP_LIBRARY names another build of the library (a debug or experimental one)
+LIB_PATH = os.environ.get("NEOML_HIP_LIBRARY") or os.path.join(HERE, "lib", "libneoml_hip.so")
 HEADER_PATH = os.path.join(os.path.dirname(HERE), "include", "neoml_hip.h")
 
 NH_OK = 0

@@ -120,6 +120,17 @@ __device__ __forceinline__ float4 bufferLoad4Stream( __amdgpu_buffer_rsrc_t rsrc
 	return make_float4( __uint_as_float( v.x ), __uint_as_float( v.y ), __uint_as_float( v.z ), __uint_as_float( v.w ) );
 }
 
+// Store through a buffer descriptor: an offset at or beyond the descriptor's size drops the store.
+__device__ __forceinline__ void bufferStore4( __amdgpu_buffer_rsrc_t rsrc, unsigned offset, const float4& v )
+{
+	u32x4 u;
+	u.x = __float_as_uint( v.x );
+	u.y = __float_as_uint( v.y );
+	u.z = __float_as_uint( v.z );
+	u.w = __float_as_uint( v.w );
+	__builtin_amdgcn_raw_buffer_store_b128( u, rsrc, offset, 0, 0 );
+}
+
 // The same with a second, wave-uniform byte offset that travels in a scalar register: what a loop adds per iteration
 // costs no vector instruction. The range check looks at the per-lane offset, so OutOfRange still reads as zero.
 __device__ __forceinline__ float4 bufferLoad4( __amdgpu_buffer_rsrc_t rsrc, unsigned offset, unsigned uniformOffset )

@@ -1368,180 +1368,294 @@ static bool fitsBuffer( long long rows, long long pitch, long long width )
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Short reductions over many rows: C[M x N] = A[M x K] * W[N x K]^T (+ bias), K = 8 * KC <= 192, all three dense.
-// These are the pointwise convolutions of a depthwise-separable network at high resolution (16 -> 96, 24 -> 144,
-// 144 -> 24 channels over 10^5..10^6 pixels): bound by HBM, and the tiled kernel above, built around a long K loop,
-// spends its time in prologues and epilogues and re-reads A once per 64 output columns.
+// Short reductions over many rows: C[M x N] = act( A[M x K] * W[N x K]^T + bias ) (+ residual), K = 8 * KC <= 192,
+// N <= 32 * NB, all dense. These are the pointwise convolutions of a depthwise-separable network at high resolution
+// (16 -> 96, 24 -> 144, 144 -> 24 channels over 10^5..10^6 pixels): they move 4 ( K + N ) bytes per row for 2 K N
+// flops, which at fp32 MFMA rates puts the matrix pipe at 25-50 % of its peak while the memory runs at full rate, so
+// the two must overlap. The tiled kernel above, built around a long K loop, spends its time in prologues and
+// epilogues and re-reads A once per 64 output columns.
 // Here a wavefront owns 32 whole rows: it fetches them straight into MFMA operand registers (every lane its row's
 // K values, 16 bytes per load: together the loads of a wavefront cover one contiguous piece of A), keeps them for
-// all output columns, and walks the columns in blocks of 32 with W read from LDS, where the workgroup put it once.
-// No barrier after that; wavefronts take further row blocks grid-stride.
+// all output columns, and walks the columns in blocks of 32 with W and the bias read from LDS, where the workgroup
+// put them once. No barrier after that; wavefronts take further row blocks grid-stride.
+// A wavefront's loads and stores complete in issue order, and the wait in front of a use counts the operations issued
+// after the awaited one, so that count must be known when the kernel is compiled: every memory operation of the row-block
+// loop is unconditional (raw buffer accesses; rows beyond M and columns beyond N get an out-of-range offset, which
+// reads zeros and drops stores), the column blocks are unrolled (NB), and nothing but A, the residual and C touches
+// memory inside the loop. The registers of A are refilled with the next row block's values right behind the last
+// MFMAs that read them, the residual of a column block is requested one block ahead: in the steady state no
+// wavefront waits for its own stores.
 // MFMA e of the c-th group of 8 k reduces over { 8c + e, 8c + 4 + e } on both operands.
-template<int KC>
-__global__ __launch_bounds__( Threads )
+__device__ __forceinline__ float hSwishOf( float v )
+{
+	const float mid = v * ( v + 3.f ) * ( 1.f / 6.f );
+	return v <= -3.f ? 0.f : ( v >= 3.f ? v : mid );
+}
+
+// ( W is the MFMA's first operand and A its second: the 32 x 32 block comes out transposed, lane ( l32, half ) holding
+// row l32 and, in registers 4g..4g+3, its columns 8g + 4 half .. + 3. The accumulator starts as the bias of those columns. )
+template<int KC, int NB, bool RES>
+__global__ __launch_bounds__( Threads, 2 )
 void shortReductionKernel( const float* A, const float* W, const float* bias, float* C, int M, int N, int rowBlocks,
 	const CFusedActivation act, const float* residual )
 {
 	constexpr int K = KC * 8;
 	constexpr int Pitch = K + 4;
-	// [32 * nBlocks][Pitch], rows beyond N are zero; then one [32][36] output patch per wavefront
+	constexpr int PatchPitch = 36;
+	// [32 * NB][Pitch], rows beyond N are zero; the bias, [32 * NB]; then one [32][36] output patch per wavefront
 	extern __shared__ __attribute__( ( aligned( 16 ) ) ) float wLds[];
 	const int tid = threadIdx.x;
 	const int lane = tid & 63;
 	const int wave = tid >> 6;
 	const int l32 = lane & 31;
 	const int half = lane >> 5;
-	const int nBlocks = ( N + 31 ) / 32;
-	for( int idx = tid; idx < nBlocks * 32 * ( K / 4 ); idx += Threads ) {
+
+	float* biasLds = wLds + NB * 32 * Pitch;
+	float* patch = biasLds + NB * 32 + wave * 32 * PatchPitch;
+	const __amdgpu_buffer_rsrc_t bufA = makeBuffer( A );
+	// C and the residual end where the matrix ends: rows beyond M are out of range by themselves
+	const unsigned cBytes = static_cast<unsigned>( M ) * static_cast<unsigned>( N ) * 4u;
+	const __amdgpu_buffer_rsrc_t bufC = __builtin_amdgcn_make_buffer_rsrc( C, 0, cBytes, 0x00020000 );
+	const __amdgpu_buffer_rsrc_t bufR = __builtin_amdgcn_make_buffer_rsrc( const_cast<float*>( RES ? residual : C ), 0, cBytes, 0x00020000 );
+	const unsigned rowBytes = static_cast<unsigned>( N ) * 4u;
+	// a lane stores 16 bytes: columns col4..col4+3 of row q * 8 + lane / 8 of the 32 x 32 block, q = 0..3
+	const int col4 = ( lane & 7 ) * 4;
+	const unsigned laneOut = static_cast<unsigned>( lane >> 3 ) * rowBytes + col4 * 4u;
+	const int stride = gridDim.x * 4;
+	const float reluTop = act.Param > 0.f ? act.Param : __builtin_inff(); // the upper threshold of ReLU, if any
+
+	auto rowOffset = [&]( int block ) -> unsigned {
+		const int m = block * 32 + l32;
+		return ( block < rowBlocks && m < M ) ? static_cast<unsigned>( m ) * ( K * 4u ) + half * 16u : OutOfRange;
+	};
+	auto outOffset = [&]( int block, int nb ) -> unsigned {
+		// ( blocks beyond the last one start beyond cBytes )
+		return nb * 32 + col4 < N ? static_cast<unsigned>( block ) * 32u * rowBytes + nb * 128u + laneOut : OutOfRange;
+	};
+
+	for( int idx = tid; idx < NB * 32 * ( K / 4 ); idx += Threads ) {
 		const int n = idx / ( K / 4 );
 		const int k4 = idx - n * ( K / 4 );
 		const float4 v = n < N ? *reinterpret_cast<const float4*>( W + static_cast<long long>( n ) * K + k4 * 4 )
 			: make_float4( 0.f, 0.f, 0.f, 0.f );
 		*reinterpret_cast<float4*>( wLds + n * Pitch + k4 * 4 ) = v;
 	}
+	for( int n = tid; n < NB * 32; n += Threads ) {
+		biasLds[n] = ( bias != nullptr && n < N ) ? bias[n] : 0.f;
+	}
 	__syncthreads();
 
-	constexpr int PatchPitch = 36;
-	float* patch = wLds + nBlocks * 32 * Pitch + wave * 32 * PatchPitch;
-	const bool rowsAligned = N % 4 == 0 && ( reinterpret_cast<uintptr_t>( C ) & 15 ) == 0;
-	const __amdgpu_buffer_rsrc_t bufA = makeBuffer( A );
-	// The rows of the next block are requested before the current block is multiplied and stored: a wavefront's
-	// loads and stores complete in issue order, so loads issued after the stores would wait for the stores' round trip.
-	auto requestRows = [&]( int block, float4 ( &rows )[KC] ) {
-		const int m = block * 32 + l32;
-		const unsigned rowOffset = ( block < rowBlocks && m < M ) ? static_cast<unsigned>( m ) * ( K * 4u ) + half * 16u : OutOfRange;
+	int block = blockIdx.x * 4 + wave;
+	float4 a[KC];
+	{
+		const unsigned first = rowOffset( block );
 #pragma unroll
 		for( int c = 0; c < KC; ++c ) {
-			rows[c] = bufferLoad4( bufA, rowOffset + c * 32u ); // an out-of-range row reads zeros
+			a[c] = bufferLoad4( bufA, first + c * 32u ); // an out-of-range row reads zeros
 		}
-	};
-	float4 ahead[KC];
-	requestRows( blockIdx.x * 4 + wave, ahead );
-	for( int block = blockIdx.x * 4 + wave; block < rowBlocks; block += gridDim.x * 4 ) {
-		float4 a[KC];
+	}
+
+	float4 res[4];
+	{
+		if( RES ) {
+			const unsigned o = outOffset( block, 0 );
 #pragma unroll
-		for( int c = 0; c < KC; ++c ) {
-			a[c] = ahead[c];
+			for( int q = 0; q < 4; ++q ) {
+				res[q] = bufferLoad4( bufR, o + q * 8u * rowBytes );
+			}
 		}
-		requestRows( block + gridDim.x * 4, ahead );
-		for( int nb = 0; nb < nBlocks; ++nb ) {
+		// Four stores that go nowhere: the loop is entered with the same sequence of outstanding operations that its
+		// own last column block leaves behind, so the compiler's wait counts for the first MFMAs skip the stores.
+#pragma unroll
+		for( int q = 0; q < 4; ++q ) {
+			bufferStore4( bufC, OutOfRange + q * 16u, make_float4( 0.f, 0.f, 0.f, 0.f ) );
+		}
+	}
+	for( ; block < rowBlocks; block += stride ) {
+		const unsigned nextRows = rowOffset( block + stride );
+#pragma unroll
+		for( int nb = 0; nb < NB; ++nb ) {
+			const bool lastColumns = nb == NB - 1; // known when the loop is unrolled
 			f32x16 acc;
+			{
+				const float* b = biasLds + nb * 32 + half * 4;
 #pragma unroll
-			for( int r = 0; r < 16; ++r ) {
-				acc[r] = 0.f;
+				for( int g = 0; g < 4; ++g ) {
+					const float4 v = *reinterpret_cast<const float4*>( b + g * 8 );
+					acc[g * 4] = v.x;
+					acc[g * 4 + 1] = v.y;
+					acc[g * 4 + 2] = v.z;
+					acc[g * 4 + 3] = v.w;
+				}
 			}
 			const float* wRow = wLds + ( nb * 32 + l32 ) * Pitch + half * 4;
 #pragma unroll
 			for( int c = 0; c < KC; ++c ) {
 				const float4 w = *reinterpret_cast<const float4*>( wRow + c * 8 );
-				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[c].x, w.x, acc, 0, 0, 0 );
-				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[c].y, w.y, acc, 0, 0, 0 );
-				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[c].z, w.z, acc, 0, 0, 0 );
-				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[c].w, w.w, acc, 0, 0, 0 );
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( w.x, a[c].x, acc, 0, 0, 0 );
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( w.y, a[c].y, acc, 0, 0, 0 );
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( w.z, a[c].z, acc, 0, 0, 0 );
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( w.w, a[c].w, acc, 0, 0, 0 );
+				if( lastColumns ) {
+					a[c] = bufferLoad4( bufA, nextRows + c * 32u );
+				}
 			}
-			// The block goes out through a wavefront-private patch of LDS, turned so that a lane holds four
-			// neighbouring columns of one row: 4 stores of 16 bytes per lane, each covering whole 128-byte runs of
-			// 8 rows, instead of 16 stores of 4 bytes. (Register r of lane ( l32, half ) is row
-			// ( r / 4 ) * 8 + half * 4 + r % 4, column l32 of the block.)
-			const int n = nb * 32 + l32;
-			const float b = ( bias != nullptr && n < N ) ? bias[n] : 0.f;
+			// the residual of the column block that follows ( of the next row block behind the last one )
+			float4 resNext[4];
+			if( RES ) {
+				const unsigned o = lastColumns ? outOffset( block + stride, 0 ) : outOffset( block, nb + 1 );
 #pragma unroll
-			for( int r = 0; r < 16; ++r ) {
-				patch[( ( r >> 2 ) * 8 + half * 4 + ( r & 3 ) ) * PatchPitch + l32] = applyActivation( acc[r] + b, act );
+				for( int q = 0; q < 4; ++q ) {
+					resNext[q] = bufferLoad4( bufR, o + q * 8u * rowBytes );
+				}
+			}
+			// The block goes out through a wavefront-private patch of LDS in which the lanes regroup: a lane then holds
+			// four neighbouring columns of a row such that one store instruction covers whole 128-byte runs of 8 rows
+			// ( stored as they come out of the MFMA, an instruction would touch 32 rows with 32 bytes each ).
+			// Nothing but the move to the patch stands between the MFMAs and the first use of their result, in one
+			// basic block: the activation, with its branches on the type, is applied to what comes back from the patch.
+			float* mine = patch + l32 * PatchPitch + half * 4;
+#pragma unroll
+			for( int g = 0; g < 4; ++g ) {
+				*reinterpret_cast<float4*>( mine + g * 8 ) = make_float4( acc[g * 4], acc[g * 4 + 1], acc[g * 4 + 2], acc[g * 4 + 3] );
 			}
 			// ( same wavefront: the LDS unit executes its reads after its writes, no barrier needed )
-			const int col4 = ( lane & 7 ) * 4;
-			const int n4 = nb * 32 + col4;
+			float4 v[4];
 #pragma unroll
 			for( int q = 0; q < 4; ++q ) {
-				const int row = q * 8 + ( lane >> 3 );
-				float4 v = *reinterpret_cast<const float4*>( patch + row * PatchPitch + col4 );
-				const long long mOut = static_cast<long long>( block ) * 32 + row;
-				if( mOut < M ) {
-					float* out = C + mOut * N + n4;
-					if( residual != nullptr ) {
-						const float* res = residual + mOut * N + n4;
-						if( n4 < N ) v.x += res[0];
-						if( n4 + 1 < N ) v.y += res[1];
-						if( n4 + 2 < N ) v.z += res[2];
-						if( n4 + 3 < N ) v.w += res[3];
-					}
-					if( rowsAligned && n4 + 3 < N ) {
-						*reinterpret_cast<float4*>( out ) = v;
-					} else {
-						if( n4 < N ) out[0] = v.x;
-						if( n4 + 1 < N ) out[1] = v.y;
-						if( n4 + 2 < N ) out[2] = v.z;
-						if( n4 + 3 < N ) out[3] = v.w;
-					}
+				v[q] = *reinterpret_cast<const float4*>( patch + ( q * 8 + ( lane >> 3 ) ) * PatchPitch + col4 );
+			}
+			if( act.Type == NH_ACT_RELU ) {
+#pragma unroll
+				for( int q = 0; q < 4; ++q ) {
+					// NaN becomes 0, as in VectorReLU: the maximum of a NaN and a number is the number
+					v[q].x = __builtin_fminf( __builtin_fmaxf( v[q].x, 0.f ), reluTop );
+					v[q].y = __builtin_fminf( __builtin_fmaxf( v[q].y, 0.f ), reluTop );
+					v[q].z = __builtin_fminf( __builtin_fmaxf( v[q].z, 0.f ), reluTop );
+					v[q].w = __builtin_fminf( __builtin_fmaxf( v[q].w, 0.f ), reluTop );
+				}
+			} else if( act.Type == NH_ACT_HSWISH ) {
+#pragma unroll
+				for( int q = 0; q < 4; ++q ) {
+					v[q].x = hSwishOf( v[q].x );
+					v[q].y = hSwishOf( v[q].y );
+					v[q].z = hSwishOf( v[q].z );
+					v[q].w = hSwishOf( v[q].w );
+				}
+			}
+			const unsigned o = outOffset( block, nb );
+#pragma unroll
+			for( int q = 0; q < 4; ++q ) {
+				if( RES ) {
+					v[q].x += res[q].x;
+					v[q].y += res[q].y;
+					v[q].z += res[q].z;
+					v[q].w += res[q].w;
+				}
+				bufferStore4( bufC, o + q * 8u * rowBytes, v[q] );
+			}
+			if( RES ) {
+#pragma unroll
+				for( int q = 0; q < 4; ++q ) {
+					res[q] = resNext[q];
 				}
 			}
 		}
 	}
 }
 
-template<int KC>
+static constexpr size_t shortReductionLds( int K, int nb )
+{
+	return ( static_cast<size_t>( nb ) * 32 * ( K + 4 ) + nb * 32 + 4 * 32 * 36 ) * sizeof( float );
+}
+
+template<int KC, int NB, bool RES>
 static void launchShortReduction( hipStream_t stream, const float* a, const float* w, const float* bias, float* c, int M, int N,
 	const CFusedActivation& act, const float* residual )
 {
 	const int rowBlocks = ceilDiv( M, 32 );
 	const int groups = ceilDiv( rowBlocks, 4 );
-	const size_t lds = ( static_cast<size_t>( ceilDiv( N, 32 ) ) * 32 * ( KC * 8 + 4 ) + 4 * 32 * 36 ) * sizeof( float );
+	const size_t lds = shortReductionLds( KC * 8, NB );
 	// The wavefronts walk the row blocks grid-stride. Narrow outputs ( one block of columns: read-bound, a long prologue
 	// that copies W to LDS ): the grid is what the device holds at once ( registers and LDS decide, both depend on KC and
-	// N ), so that no second, partly filled round of workgroups trails behind the first: 15-25 % faster than a fixed
-	// 2048, and up to 35 % faster than a workgroup per four row blocks. Wide outputs ( write-bound ) are the opposite:
-	// with one resident round every wavefront loads and stores in step with all others; eight rounds' worth of
-	// workgroups, which drift apart, are up to 24 % faster ( 16 -> 96 channels over 1.6 M pixels: 198 -> 152 us ).
+	// NB ), so that no second, partly filled round of workgroups trails behind the first. Wide outputs ( write-bound ):
+	// four rounds' worth of workgroups, which drift apart instead of loading and storing in step with each other
+	// ( 16 -> 96 channels over 1.6 M pixels: 144 -> 133 us ).
 	static std::mutex lock;
-	static std::map<std::pair<int, size_t>, int> residentFor;
+	static std::map<int, int> residentFor;
 	int resident = 0;
 	{
 		int device = 0;
 		( void )hipGetDevice( &device );
 		std::lock_guard<std::mutex> guard( lock );
-		int& known = residentFor[std::make_pair( device, lds )];
+		int& known = residentFor[device];
 		if( known == 0 ) {
 			int perUnit = 0, units = 0;
-			if( hipOccupancyMaxActiveBlocksPerMultiprocessor( &perUnit, shortReductionKernel<KC>, Threads, lds ) != hipSuccess
+			if( hipOccupancyMaxActiveBlocksPerMultiprocessor( &perUnit, shortReductionKernel<KC, NB, RES>, Threads, lds ) != hipSuccess
 				|| hipDeviceGetAttribute( &units, hipDeviceAttributeMultiprocessorCount, device ) != hipSuccess
 				|| perUnit <= 0 || units <= 0 )
 			{
 				( void )hipGetLastError();
-				perUnit = 8;
+				perUnit = 2;
 				units = 256;
 			}
 			known = perUnit * units;
 		}
 		resident = known;
 	}
-	if( N > 32 ) {
-		resident *= 8;
+	if( NB > 1 ) {
+		resident *= 4;
 	}
-	hipLaunchKernelGGL( shortReductionKernel<KC>, dim3( groups < resident ? groups : resident ), dim3( Threads ), lds, stream,
+	hipLaunchKernelGGL( ( shortReductionKernel<KC, NB, RES> ), dim3( groups < resident ? groups : resident ), dim3( Threads ), lds, stream,
 		a, w, bias, c, M, N, rowBlocks, act, residual );
+}
+
+// One kernel per count of column blocks that 64 KB of LDS hold next to the output patches.
+template<int KC, int NB>
+static bool launchShortReductionColumns( hipStream_t stream, const float* a, const float* w, const float* bias, float* c, int M, int N,
+	const CFusedActivation& act, const float* residual )
+{
+	if constexpr( NB >= 1 && shortReductionLds( KC * 8, NB >= 1 ? NB : 1 ) <= 64 * 1024 ) {
+		if( ceilDiv( N, 32 ) == NB ) {
+			if( residual != nullptr ) {
+				launchShortReduction<KC, NB, true>( stream, a, w, bias, c, M, N, act, residual );
+			} else {
+				launchShortReduction<KC, NB, false>( stream, a, w, bias, c, M, N, act, residual );
+			}
+			return true;
+		}
+		return launchShortReductionColumns<KC, NB - 1>( stream, a, w, bias, c, M, N, act, residual );
+	} else if constexpr( NB >= 1 ) {
+		return launchShortReductionColumns<KC, NB - 1>( stream, a, w, bias, c, M, N, act, residual );
+	} else {
+		return false;
+	}
 }
 
 // true (and launched) when the product has the shape this kernel is for
 static bool tryShortReduction( hipStream_t stream, const float* a, int lda, const float* w, int ldb, float* c, int ldc,
 	int M, int N, int K, const float* bias, const CFusedActivation& act, const float* residual, int* rc )
 {
-	if( lda != K || ldb != K || ldc != N || M < 16384 || K % 8 != 0 || K > 192 || N > 192
-		|| !isAligned16( a ) || !isAligned16( w ) || !fitsBuffer( M, K, K )
-		|| ( static_cast<size_t>( ceilDiv( N, 32 ) ) * 32 * ( K + 4 ) + 4 * 32 * 36 ) * sizeof( float ) > 64 * 1024 )
+	if( lda != K || ldb != K || ldc != N || M < 16384 || K % 8 != 0 || K > 192 || N > 192 || N % 4 != 0
+		|| !isAligned16( a ) || !isAligned16( w ) || !isAligned16( c ) || !isAligned16( residual )
+		|| !fitsBuffer( M, K, K ) || !fitsBuffer( M + 32, N, N ) )
 	{
 		return false;
 	}
+	bool launched = false;
 	switch( K / 8 ) {
-		case 2: launchShortReduction<2>( stream, a, w, bias, c, M, N, act, residual ); break;
-		case 3: launchShortReduction<3>( stream, a, w, bias, c, M, N, act, residual ); break;
-		case 4: launchShortReduction<4>( stream, a, w, bias, c, M, N, act, residual ); break;
-		case 6: launchShortReduction<6>( stream, a, w, bias, c, M, N, act, residual ); break;
-		case 8: launchShortReduction<8>( stream, a, w, bias, c, M, N, act, residual ); break;
-		case 12: launchShortReduction<12>( stream, a, w, bias, c, M, N, act, residual ); break;
-		case 18: launchShortReduction<18>( stream, a, w, bias, c, M, N, act, residual ); break;
-		case 24: launchShortReduction<24>( stream, a, w, bias, c, M, N, act, residual ); break;
-		default: return false;
+		case 2: launched = launchShortReductionColumns<2, 6>( stream, a, w, bias, c, M, N, act, residual ); break;
+		case 3: launched = launchShortReductionColumns<3, 6>( stream, a, w, bias, c, M, N, act, residual ); break;
+		case 4: launched = launchShortReductionColumns<4, 6>( stream, a, w, bias, c, M, N, act, residual ); break;
+		case 6: launched = launchShortReductionColumns<6, 6>( stream, a, w, bias, c, M, N, act, residual ); break;
+		case 8: launched = launchShortReductionColumns<8, 6>( stream, a, w, bias, c, M, N, act, residual ); break;
+		case 12: launched = launchShortReductionColumns<12, 6>( stream, a, w, bias, c, M, N, act, residual ); break;
+		case 18: launched = launchShortReductionColumns<18, 6>( stream, a, w, bias, c, M, N, act, residual ); break;
+		case 24: launched = launchShortReductionColumns<24, 6>( stream, a, w, bias, c, M, N, act, residual ); break;
+		default: break;
+	}
+	if( !launched ) {
+		return false;
 	}
 	const hipError_t err = hipGetLastError();
 	if( err != hipSuccess ) {
