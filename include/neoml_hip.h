@@ -437,6 +437,57 @@ NH_API int nhLstm(nhStream s, int hiddenSize, int objectSize, const float* input
 	int sequenceCount, const float* inputStateBackLink, const float* inputMainBackLink, const float* input,
 	float* outputStateBackLink, float* outputMainBackLink, void* workspace, size_t workspaceSize);
 
+/* ---- Element-wise members beyond the inference path: comparisons, selections, powers, masked gradients, sums along a
+ * dimension (what losses, ONNX-style operators and NeoML's automatic differentiation call). Semantics are the
+ * reference CPU engine's (src/CPU/CpuMathEngineVectorMath.cpp, src/CPU/x86/CpuX86MathEngineVectorMath.cpp). */
+NH_API int nhVectorFillBernoulli(nhStream s, float* result, float p, int vectorSize, float value, int seed);           /* NME.h:99, the CPU engine's generator */
+NH_API int nhFilterSmallValues(nhStream s, float* data, int dataSize, float threshold);                              /* NME.h:102 */
+NH_API int nhVectorSumAdd(nhStream s, const float* first, int vectorSize, float* result);                            /* NME.h:107 */
+NH_API int nhVectorSumAlongDimension(nhStream s, const float* first, int precedingDimension, int dimension,
+	int followingDimension, float* result);                                                                          /* NME.h:109 */
+NH_API int nhVectorCumSumAlongDimension(nhStream s, const float* first, int precedingDimension, int dimension,
+	int followingDimension, float* result, int reverse);                                                             /* NME.h:112 */
+NH_API int nhVectorCumSumAlongDimensionInt(nhStream s, const int* first, int precedingDimension, int dimension,
+	int followingDimension, int* result, int reverse);                                                               /* NME.h:114 */
+/* cumulative = 0: VectorSumAlongDimensionDiag (NME.h:117), 1: VectorCumSumAlongDimensionDiag (NME.h:119) */
+NH_API int nhVectorSumAlongDimensionDiag(nhStream s, const float* first, int precedingDimension, int dimension,
+	int followingDimension, float* result, int cumulative);
+NH_API int nhVectorEqualInt(nhStream s, const int* first, const int* second, float* result, int vectorSize);         /* NME.h:123 */
+NH_API int nhVectorEqualValueInt(nhStream s, const int* first, float* result, int vectorSize, const int* value);     /* NME.h:126 */
+NH_API int nhVectorMax(nhStream s, const float* first, float secondValue, float* result, int vectorSize);            /* NME.h:130 */
+NH_API int nhVectorMaxDiff(nhStream s, const float* first, float secondValue, float* grad, int gradHeight, int gradWidth); /* NME.h:132 */
+NH_API int nhVectorAbsDiffRows(nhStream s, const float* sourceGrad, int gradHeight, int gradWidth, const float* first,
+	float* result);                                                                                                  /* NME.h:180 */
+NH_API int nhVectorLogDiff(nhStream s, const float* sourceGrad, int gradHeight, int gradWidth, const float* value,
+	float* result);                                                                                                  /* NME.h:221 */
+NH_API int nhVectorBernulliKLDerivative(nhStream s, const float* estimation, float* result, int vectorSize,
+	const float* target);                                                                                            /* NME.h:231 */
+NH_API int nhVectorEltwiseDivideInt(nhStream s, const int* first, const int* second, int* result, int vectorSize);   /* NME.h:289 */
+NH_API int nhVectorEltwisePower(nhStream s, const float* first, const float* second, float* result, int vectorSize); /* NME.h:295 */
+NH_API int nhVectorMinMaxDiff(nhStream s, const float* sourceGrad, int gradHeight, int gradWidth, const float* first,
+	float* result, const float* minValue, const float* maxValue);                                                    /* NME.h:307 */
+NH_API int nhVectorPower(nhStream s, float exponent, const float* first, float* result, int vectorSize);             /* NME.h:327 */
+NH_API int nhVectorPowerDiff(nhStream s, float exponent, const float* first, const float* second, float* result,
+	int vectorSize);                                                                                                 /* NME.h:328 */
+NH_API int nhVectorPowerDiffOp(nhStream s, float exponent, const float* first, const float* second, float* result,
+	int vectorSize);                                                                                                 /* NME.h:330 */
+NH_API int nhVectorEltwiseNotInt(nhStream s, const int* first, int* result, int vectorSize);                         /* NME.h:343 */
+NH_API int nhVectorEltwiseNotNegative(nhStream s, const int* first, float* result, int vectorSize);                  /* NME.h:346 */
+NH_API int nhVectorEltwiseLess(nhStream s, const float* first, const float* second, float* result, int vectorSize);  /* NME.h:349 */
+/* valueFirst = 0: first[i] < second (NME.h:351); 1: second < first[i] (NME.h:353) */
+NH_API int nhVectorEltwiseLessValue(nhStream s, const float* first, float second, float* result, int vectorSize, int valueFirst);
+NH_API int nhVectorEltwiseLessToInt(nhStream s, const float* first, const float* second, int* result, int vectorSize); /* NME.h:357 */
+NH_API int nhVectorEltwiseLessInt(nhStream s, const int* first, const int* second, int* result, int vectorSize);     /* NME.h:359 */
+NH_API int nhVectorEltwiseEqualToInt(nhStream s, const float* first, const float* second, int* result, int vectorSize); /* NME.h:363 */
+NH_API int nhVectorEltwiseEqualInt(nhStream s, const int* first, const int* second, int* result, int vectorSize);    /* NME.h:365 */
+/* result = first != 0 ? second : third on 32-bit elements: the float (NME.h:369) and the int (NME.h:371) overload */
+NH_API int nhVectorEltwiseWhere(nhStream s, const int* first, const void* second, const void* third, void* result, int vectorSize);
+/* One step of VectorFindMaxValueInSet with indices (NME.h:375): where candidate[i] > result[i], both result[i] and
+ * indices[i] = index follow; the caller starts from the first vector with indices 0. */
+NH_API int nhVectorMaxWithIndex(nhStream s, const float* candidate, float* result, int* indices, int index, int vectorSize);
+/* One target of VectorSpreadValues (NME.h:377): target[i] = source[i] where indices[i] == index. */
+NH_API int nhVectorSpreadValuesTo(nhStream s, const float* source, float* target, const int* indices, int index, int vectorSize);
+
 #ifdef __cplusplus
 }
 #endif

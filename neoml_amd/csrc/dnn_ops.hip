@@ -1415,6 +1415,17 @@ void dropoutKernel( const float* in, float* out, long long total, int maskSize, 
 	}
 }
 
+// VectorFillBernoulli with the same generator ( src/CPU/CpuMathEngineVectorMath.cpp:267-284 ): element i takes word i % 4 of
+// counter value i / 4.
+__global__ __launch_bounds__( 256 )
+void fillBernoulliKernel( float* result, int n, unsigned seed, unsigned threshold, float value )
+{
+	const int i = blockIdx.x * 256 + threadIdx.x;
+	if( i < n ) {
+		result[i] = dropoutWord( static_cast<unsigned>( i ) / 4, i & 3, seed ) <= threshold ? value : 0.f;
+	}
+}
+
 __global__ void addTwoVectorsKernel( const float* a, const float* b, float* out, int n )
 {
 	const int i = blockIdx.x * 256 + threadIdx.x;
@@ -2524,3 +2535,17 @@ int nhChannelwiseWith1x1( nhStream s, const nhSeparableBlockDesc* d, const float
 }
 
 } // extern "C"
+
+extern "C" int nhVectorFillBernoulli( nhStream s, float* result, float p, int vectorSize, float value, int seed )
+{
+	NH_REQUIRE( vectorSize >= 0 );
+	if( vectorSize == 0 ) {
+		return NH_OK;
+	}
+	NH_REQUIRE( result != nullptr );
+	const unsigned threshold = static_cast<unsigned>( static_cast<double>( p ) * 4294967295.0 );
+	hipLaunchKernelGGL( fillBernoulliKernel, dim3( ceilDiv( vectorSize, 256 ) ), dim3( 256 ), 0, toStream( s ), result, vectorSize,
+		static_cast<unsigned>( seed ), threshold, value );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}

@@ -489,9 +489,9 @@ __global__ __launch_bounds__( 256 ) void sumKernel( const float* a, const float*
 }
 
 template<bool DOT>
-static int launchSum( nhStream s, const float* first, const float* second, int vectorSize, float* result )
+static int launchSum( nhStream s, const float* first, const float* second, int vectorSize, float* result, bool addToResult = false )
 {
-	int rc = nhVectorFill( s, result, 0.f, 1 );
+	int rc = addToResult ? NH_OK : nhVectorFill( s, result, 0.f, 1 );
 	if( rc != NH_OK || vectorSize == 0 ) {
 		return rc;
 	}
@@ -735,4 +735,344 @@ extern "C" int nhVectorDotProduct( nhStream s, const float* first, const float* 
 {
 	NH_REQUIRE( vectorSize >= 0 && result != nullptr );
 	return launchSum<true>( s, first, second, vectorSize, result );
+}
+
+// ---- comparisons, selections, powers, masked gradients: the element-wise members that losses, ONNX-style operators
+// ---- and the automatic differentiation of NeoML call (semantics: src/CPU/CpuMathEngineVectorMath.cpp and
+// ---- src/CPU/x86/CpuX86MathEngineVectorMath.cpp, lines cited per functor) ------------------------------------------
+
+namespace nh {
+
+struct CFilterSmallOp { // x86/CpuX86MathEngineVectorMath.cpp:99-126: kept when x >= t or x <= -t
+	float Threshold;
+	__device__ void prepare() {}
+	__device__ float operator()( float a, float, float ) const { return ( a >= Threshold || a <= -Threshold ) ? a : 0.f; }
+};
+struct CEqualToFloatOp : CNoScalar { __device__ float operator()( int a, int b, int ) const { return a == b ? 1.f : 0.f; } }; // x86:166
+struct CEqualValueOp { // x86:199
+	const int* Ptr; int Value;
+	__device__ void prepare() { Value = *Ptr; }
+	__device__ float operator()( int a, int, int ) const { return a == Value ? 1.f : 0.f; }
+};
+struct CMaxValueOp { // CpuMathEngineVectorMath.cpp:551
+	float Value;
+	__device__ void prepare() {}
+	__device__ float operator()( float a, float, float ) const { return a >= Value ? a : Value; }
+};
+struct CBernulliKLOp { // x86:980-1025: -t / e + ( 1 - t ) / ( 1 - e ), cut to [-10, 10] (min first, as the SSE code does)
+	const float* Ptr; float Target;
+	__device__ void prepare() { Target = *Ptr; }
+	__device__ float operator()( float e, float, float ) const
+	{
+		float d = -Target / e + ( 1.f - Target ) / ( 1.f - e );
+		d = d < 10.f ? d : 10.f;   // _mm_min_ps( d, 10 ): the second operand when either is NaN
+		return d > -10.f ? d : -10.f;
+	}
+};
+struct CDivIntOp : CNoScalar { __device__ int operator()( int a, int b, int ) const { return b != 0 ? a / b : 0; } }; // :814 ( a zero divisor traps there )
+struct CEltwisePowerOp : CNoScalar { __device__ float operator()( float a, float b, float ) const { return b == 1.f ? a : powf( a, b ); } }; // x86:1277
+struct CPowerOp { // x86/CpuX86MathEngineVectorMathMkl.cpp:129-153
+	float Exponent;
+	__device__ void prepare() {}
+	__device__ float operator()( float a, float, float ) const { return powf( a, Exponent ); }
+};
+struct CPowerDiffOp { // x86:1522-1595: second * exponent * first ^ Power
+	float Exponent, Power;
+	__device__ void prepare() {}
+	__device__ float operator()( float a, float b, float ) const { return b * ( Exponent * powf( a, Power ) ); }
+};
+struct CNotOp : CNoScalar { __device__ int operator()( int a, int, int ) const { return a == 0 ? 1 : 0; } };              // x86:1648
+struct CNotNegativeOp : CNoScalar { __device__ float operator()( int a, int, int ) const { return a >= 0 ? 1.f : 0.f; } }; // x86:1677
+template<typename TIn, typename TOut> struct CLessOp : CNoScalar { // :688-760
+	__device__ TOut operator()( TIn a, TIn b, TIn ) const { return static_cast<TOut>( a < b ? 1 : 0 ); }
+};
+struct CLessValueOp { // :713-741; Reverse: value < x
+	float Value; int Reverse;
+	__device__ void prepare() {}
+	__device__ float operator()( float a, float, float ) const { return ( Reverse ? Value < a : a < Value ) ? 1.f : 0.f; }
+};
+template<typename TIn> struct CEqualToIntOp : CNoScalar { __device__ int operator()( TIn a, TIn b, TIn ) const { return a == b ? 1 : 0; } }; // :764-786
+// first != 0 ? second : third, on the 32-bit patterns (serves the float and the int overload, :788-812)
+struct CWhereOp : CNoScalar { __device__ int operator()( int a, int b, int c ) const { return a != 0 ? b : c; } };
+
+// result[i][j] = f( first[i], grad[i][j] ): the gradient forms whose condition is one value per row of the gradient
+// ( firstSize = gradHeight == 1 ? gradWidth : gradHeight rows of gradSize = gradHeight == 1 ? 1 : gradWidth values )
+template<typename F>
+__global__ __launch_bounds__( 256 )
+void rowConditionKernel( const float* first, const float* grad, float* result, long long total, int gradSize, F f )
+{
+	for( long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += static_cast<long long>( gridDim.x ) * 256 ) {
+		result[i] = f( first[i / gradSize], grad[i] );
+	}
+}
+
+struct CRowAbsDiff { __device__ float operator()( float x, float g ) const { return x > 0.f ? g : -g; } };              // :516-549
+struct CRowMaxDiff { float Value; __device__ float operator()( float x, float g ) const { return x < Value ? 0.f : g; } }; // :567-589
+struct CRowLogDiff { // :591-619
+	__device__ float operator()( float x, float g ) const { return ( -FLT_MIN <= x && x <= FLT_MIN ) ? 0.f : g / x; }
+};
+struct CRowMinMaxDiff { // :649-686
+	const float* MinPtr; const float* MaxPtr;
+	__device__ float operator()( float x, float g ) const { return ( x < *MinPtr || x > *MaxPtr ) ? 0.f : g; }
+};
+
+template<typename F>
+static int launchRowCondition( nhStream s, const float* first, const float* grad, float* result, int gradHeight, int gradWidth, F f )
+{
+	NH_REQUIRE( gradHeight > 0 && gradWidth > 0 && first != nullptr && grad != nullptr && result != nullptr );
+	const int gradSize = gradHeight == 1 ? 1 : gradWidth;
+	const long long total = static_cast<long long>( gradHeight ) * gradWidth;
+	const long long blocks = ( total + 255 ) / 256;
+	hipLaunchKernelGGL( rowConditionKernel<F>, dim3( static_cast<unsigned>( blocks > 8192 ? 8192 : blocks ) ), dim3( 256 ), 0, toStream( s ),
+		first, grad, result, total, gradSize, f );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+__global__ __launch_bounds__( 256 )
+void maxWithIndexKernel( const float* candidate, float* result, int* indices, int index, int n )
+{
+	const int i = blockIdx.x * 256 + threadIdx.x;
+	if( i < n && candidate[i] > result[i] ) {
+		result[i] = candidate[i];
+		indices[i] = index;
+	}
+}
+
+__global__ __launch_bounds__( 256 )
+void spreadValuesKernel( const float* source, float* target, const int* indices, int index, int n )
+{
+	const int i = blockIdx.x * 256 + threadIdx.x;
+	if( i < n && indices[i] == index ) {
+		target[i] = source[i];
+	}
+}
+
+// sums over the middle one of three dimensions: first is [following][dimension][preceding] ( :146-207 )
+template<typename T, bool CUMULATIVE>
+__global__ __launch_bounds__( 256 )
+void sumAlongDimensionKernel( const T* first, T* result, int preceding, int dimension, int following, int reverse )
+{
+	const long long lines = static_cast<long long>( preceding ) * following;
+	for( long long line = blockIdx.x * 256LL + threadIdx.x; line < lines; line += static_cast<long long>( gridDim.x ) * 256 ) {
+		const long long f = line / preceding;
+		const int p = static_cast<int>( line - f * preceding );
+		const T* in = first + f * dimension * preceding + p;
+		T sum = T();
+		if( CUMULATIVE ) {
+			T* out = result + f * dimension * preceding + p;
+			for( int d = 0; d < dimension; ++d ) {
+				const int at = reverse ? dimension - 1 - d : d;
+				sum = d == 0 ? in[static_cast<long long>( at ) * preceding] : in[static_cast<long long>( at ) * preceding] + sum;
+				out[static_cast<long long>( at ) * preceding] = sum;
+			}
+		} else {
+			for( int d = 0; d < dimension; ++d ) {
+				sum = d == 0 ? in[0] : in[static_cast<long long>( d ) * preceding] + sum;
+			}
+			result[line] = sum;
+		}
+	}
+}
+
+// The Jacobians of the two sums above as dense matrices ( :209-264 ): row ( f, p [, d] ), column ( f, k, p ) holds
+// first[f][k][p] for every k ( for k <= d in the cumulative form ), zero elsewhere.
+template<bool CUMULATIVE>
+__global__ __launch_bounds__( 256 )
+void sumAlongDimensionDiagKernel( const float* first, float* result, int preceding, int dimension, int following, long long total )
+{
+	const long long width = static_cast<long long>( preceding ) * dimension * following;
+	for( long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += static_cast<long long>( gridDim.x ) * 256 ) {
+		const long long row = i / width;
+		const long long column = i - row * width;
+		// row = ( f * preceding + p ) [ * dimension + d ]
+		const long long fp = CUMULATIVE ? row / dimension : row;
+		const int d = CUMULATIVE ? static_cast<int>( row - fp * dimension ) : dimension - 1;
+		const long long f = fp / preceding;
+		const int p = static_cast<int>( fp - f * preceding );
+		const long long cf = column / ( static_cast<long long>( dimension ) * preceding );
+		const long long rest = column - cf * dimension * preceding;
+		const int k = static_cast<int>( rest / preceding );
+		const int cp = static_cast<int>( rest - static_cast<long long>( k ) * preceding );
+		result[i] = ( cf == f && cp == p && k <= d ) ? first[( f * dimension + k ) * preceding + p] : 0.f;
+	}
+}
+
+} // namespace nh
+
+extern "C" int nhFilterSmallValues( nhStream s, float* data, int dataSize, float threshold )
+{
+	CFilterSmallOp op; op.Threshold = threshold;
+	return launchEltwise<1, float, float>( s, data, (const float*)nullptr, (const float*)nullptr, data, dataSize, op );
+}
+extern "C" int nhVectorSumAdd( nhStream s, const float* first, int vectorSize, float* result )
+{
+	NH_REQUIRE( vectorSize >= 0 && result != nullptr );
+	return launchSum<false>( s, first, nullptr, vectorSize, result, true );
+}
+extern "C" int nhVectorEqualInt( nhStream s, const int* first, const int* second, float* result, int vectorSize )
+{
+	return launchEltwise<2, int, float>( s, first, second, (const int*)nullptr, result, vectorSize, CEqualToFloatOp() );
+}
+extern "C" int nhVectorEqualValueInt( nhStream s, const int* first, float* result, int vectorSize, const int* value )
+{
+	NH_REQUIRE( value != nullptr );
+	CEqualValueOp op; op.Ptr = value; op.Value = 0;
+	return launchEltwise<1, int, float>( s, first, (const int*)nullptr, (const int*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorMax( nhStream s, const float* first, float secondValue, float* result, int vectorSize )
+{
+	CMaxValueOp op; op.Value = secondValue;
+	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorMaxDiff( nhStream s, const float* first, float secondValue, float* grad, int gradHeight, int gradWidth )
+{
+	CRowMaxDiff f; f.Value = secondValue;
+	return launchRowCondition( s, first, grad, grad, gradHeight, gradWidth, f );
+}
+extern "C" int nhVectorAbsDiffRows( nhStream s, const float* sourceGrad, int gradHeight, int gradWidth, const float* first, float* result )
+{
+	return launchRowCondition( s, first, sourceGrad, result, gradHeight, gradWidth, CRowAbsDiff() );
+}
+extern "C" int nhVectorLogDiff( nhStream s, const float* sourceGrad, int gradHeight, int gradWidth, const float* value, float* result )
+{
+	return launchRowCondition( s, value, sourceGrad, result, gradHeight, gradWidth, CRowLogDiff() );
+}
+extern "C" int nhVectorMinMaxDiff( nhStream s, const float* sourceGrad, int gradHeight, int gradWidth, const float* first, float* result,
+	const float* minValue, const float* maxValue )
+{
+	NH_REQUIRE( minValue != nullptr && maxValue != nullptr );
+	CRowMinMaxDiff f; f.MinPtr = minValue; f.MaxPtr = maxValue;
+	return launchRowCondition( s, first, sourceGrad, result, gradHeight, gradWidth, f );
+}
+extern "C" int nhVectorBernulliKLDerivative( nhStream s, const float* estimation, float* result, int vectorSize, const float* target )
+{
+	NH_REQUIRE( target != nullptr );
+	CBernulliKLOp op; op.Ptr = target; op.Target = 0;
+	return launchEltwise<1, float, float>( s, estimation, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+NH_BINARY( nhVectorEltwiseDivideInt, int, CDivIntOp )
+NH_BINARY( nhVectorEltwisePower, float, CEltwisePowerOp )
+extern "C" int nhVectorPower( nhStream s, float exponent, const float* first, float* result, int vectorSize )
+{
+	CPowerOp op; op.Exponent = exponent;
+	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorPowerDiff( nhStream s, float exponent, const float* first, const float* second, float* result, int vectorSize )
+{
+	CPowerDiffOp op; op.Exponent = exponent; op.Power = exponent - 1.f;
+	return launchEltwise<2, float, float>( s, first, second, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorPowerDiffOp( nhStream s, float exponent, const float* first, const float* second, float* result, int vectorSize )
+{
+	CPowerDiffOp op; op.Exponent = exponent; op.Power = ( exponent - 1.f ) / exponent;
+	return launchEltwise<2, float, float>( s, first, second, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorEltwiseNotInt( nhStream s, const int* first, int* result, int vectorSize )
+{
+	return launchEltwise<1, int, int>( s, first, (const int*)nullptr, (const int*)nullptr, result, vectorSize, CNotOp() );
+}
+extern "C" int nhVectorEltwiseNotNegative( nhStream s, const int* first, float* result, int vectorSize )
+{
+	return launchEltwise<1, int, float>( s, first, (const int*)nullptr, (const int*)nullptr, result, vectorSize, CNotNegativeOp() );
+}
+extern "C" int nhVectorEltwiseLess( nhStream s, const float* first, const float* second, float* result, int vectorSize )
+{
+	return launchEltwise<2, float, float>( s, first, second, (const float*)nullptr, result, vectorSize, CLessOp<float, float>() );
+}
+extern "C" int nhVectorEltwiseLessValue( nhStream s, const float* first, float second, float* result, int vectorSize, int valueFirst )
+{
+	CLessValueOp op; op.Value = second; op.Reverse = valueFirst;
+	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
+}
+extern "C" int nhVectorEltwiseLessToInt( nhStream s, const float* first, const float* second, int* result, int vectorSize )
+{
+	return launchEltwise<2, float, int>( s, first, second, (const float*)nullptr, result, vectorSize, CLessOp<float, int>() );
+}
+extern "C" int nhVectorEltwiseLessInt( nhStream s, const int* first, const int* second, int* result, int vectorSize )
+{
+	return launchEltwise<2, int, int>( s, first, second, (const int*)nullptr, result, vectorSize, CLessOp<int, int>() );
+}
+extern "C" int nhVectorEltwiseEqualToInt( nhStream s, const float* first, const float* second, int* result, int vectorSize )
+{
+	return launchEltwise<2, float, int>( s, first, second, (const float*)nullptr, result, vectorSize, CEqualToIntOp<float>() );
+}
+extern "C" int nhVectorEltwiseEqualInt( nhStream s, const int* first, const int* second, int* result, int vectorSize )
+{
+	return launchEltwise<2, int, int>( s, first, second, (const int*)nullptr, result, vectorSize, CEqualToIntOp<int>() );
+}
+extern "C" int nhVectorEltwiseWhere( nhStream s, const int* first, const void* second, const void* third, void* result, int vectorSize )
+{
+	return launchEltwise<3, int, int>( s, first, static_cast<const int*>( second ), static_cast<const int*>( third ),
+		static_cast<int*>( result ), vectorSize, CWhereOp() );
+}
+extern "C" int nhVectorMaxWithIndex( nhStream s, const float* candidate, float* result, int* indices, int index, int vectorSize )
+{
+	NH_REQUIRE( vectorSize >= 0 );
+	if( vectorSize == 0 ) {
+		return NH_OK;
+	}
+	NH_REQUIRE( candidate != nullptr && result != nullptr && indices != nullptr );
+	hipLaunchKernelGGL( maxWithIndexKernel, dim3( ceilDiv( vectorSize, 256 ) ), dim3( 256 ), 0, toStream( s ), candidate, result, indices,
+		index, vectorSize );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+extern "C" int nhVectorSpreadValuesTo( nhStream s, const float* source, float* target, const int* indices, int index, int vectorSize )
+{
+	NH_REQUIRE( vectorSize >= 0 );
+	if( vectorSize == 0 ) {
+		return NH_OK;
+	}
+	NH_REQUIRE( source != nullptr && target != nullptr && indices != nullptr );
+	hipLaunchKernelGGL( spreadValuesKernel, dim3( ceilDiv( vectorSize, 256 ) ), dim3( 256 ), 0, toStream( s ), source, target, indices,
+		index, vectorSize );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+template<typename T, bool CUMULATIVE>
+static int launchSumAlongDimension( nhStream s, const T* first, int preceding, int dimension, int following, T* result, int reverse )
+{
+	NH_REQUIRE( preceding > 0 && dimension > 0 && following > 0 && first != nullptr && result != nullptr );
+	const long long lines = static_cast<long long>( preceding ) * following;
+	const long long blocks = ( lines + 255 ) / 256;
+	hipLaunchKernelGGL( ( sumAlongDimensionKernel<T, CUMULATIVE> ), dim3( static_cast<unsigned>( blocks > 8192 ? 8192 : blocks ) ), dim3( 256 ), 0,
+		toStream( s ), first, result, preceding, dimension, following, reverse );
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+extern "C" int nhVectorSumAlongDimension( nhStream s, const float* first, int precedingDimension, int dimension, int followingDimension,
+	float* result )
+{
+	return launchSumAlongDimension<float, false>( s, first, precedingDimension, dimension, followingDimension, result, 0 );
+}
+extern "C" int nhVectorCumSumAlongDimension( nhStream s, const float* first, int precedingDimension, int dimension, int followingDimension,
+	float* result, int reverse )
+{
+	return launchSumAlongDimension<float, true>( s, first, precedingDimension, dimension, followingDimension, result, reverse );
+}
+extern "C" int nhVectorCumSumAlongDimensionInt( nhStream s, const int* first, int precedingDimension, int dimension, int followingDimension,
+	int* result, int reverse )
+{
+	return launchSumAlongDimension<int, true>( s, first, precedingDimension, dimension, followingDimension, result, reverse );
+}
+extern "C" int nhVectorSumAlongDimensionDiag( nhStream s, const float* first, int precedingDimension, int dimension, int followingDimension,
+	float* result, int cumulative )
+{
+	NH_REQUIRE( precedingDimension > 0 && dimension > 0 && followingDimension > 0 && first != nullptr && result != nullptr );
+	const long long width = static_cast<long long>( precedingDimension ) * dimension * followingDimension;
+	const long long rows = static_cast<long long>( precedingDimension ) * followingDimension * ( cumulative ? dimension : 1 );
+	const long long total = width * rows;
+	const long long blocks = ( total + 255 ) / 256;
+	const dim3 grid( static_cast<unsigned>( blocks > 8192 ? 8192 : blocks ) );
+	if( cumulative ) {
+		hipLaunchKernelGGL( sumAlongDimensionDiagKernel<true>, grid, dim3( 256 ), 0, toStream( s ), first, result, precedingDimension, dimension,
+			followingDimension, total );
+	} else {
+		hipLaunchKernelGGL( sumAlongDimensionDiagKernel<false>, grid, dim3( 256 ), 0, toStream( s ), first, result, precedingDimension, dimension,
+			followingDimension, total );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
 }

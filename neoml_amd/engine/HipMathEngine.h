@@ -378,6 +378,45 @@ public:
 	// Waits for the engine's stream (used by the performance counters)
 	void Synchronize() const;
 
+	// ---- members beyond the inference path ( HipMathEngineWide.cpp ): comparisons, selections, powers, masked
+	// ---- gradients, sums along a dimension ----
+	void VectorFillBernoulli( const CFloatHandle& result, float p, int vectorSize, float value, int seed ) override;
+	void FilterSmallValues( const CFloatHandle& data, int dataSize, float threshold ) override;
+	void VectorSumAdd( const CConstFloatHandle& firstHandle, int vectorSize, const CFloatHandle& resultHandle ) override;
+	void VectorSumAlongDimension( const CConstFloatHandle& firstHandle, int precedingDimension, int dimension, int followingDimension, const CFloatHandle& resultHandle ) override;
+	void VectorCumSumAlongDimension( const CConstFloatHandle& firstHandle, int precedingDimension, int dimension, int followingDimension, const CFloatHandle& resultHandle, bool reverse ) override;
+	void VectorCumSumAlongDimension( const CConstIntHandle& firstHandle, int precedingDimension, int dimension, int followingDimension, const CIntHandle& resultHandle, bool reverse ) override;
+	void VectorSumAlongDimensionDiag( const CConstFloatHandle& firstHandle, int precedingDimension, int dimension, int followingDimension, const CFloatHandle& resultHandle ) override;
+	void VectorCumSumAlongDimensionDiag( const CConstFloatHandle& firstHandle, int precedingDimension, int dimension, int followingDimension, const CFloatHandle& resultHandle ) override;
+	void VectorEqual( const CConstIntHandle& firstHandle, const CConstIntHandle& secondHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorEqualValue( const CConstIntHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize, const CConstIntHandle& valueHandle ) override;
+	void VectorMax( const CConstFloatHandle& firstHandle, float secondValue, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorMaxDiff( const CConstFloatHandle& firstHandle, float secondValue, const CFloatHandle& gradHandle, int gradHeight, int gradWidth ) override;
+	void VectorAbsDiff( const CConstFloatHandle& sourceGradHandle, int gradHeight, int gradWidth, const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle ) override;
+	void VectorLogDiff( const CConstFloatHandle& sourceGradHandle, int sourceGradHeight, int sourceGradWidth, const CConstFloatHandle& valueHandle, const CFloatHandle& resultHandle ) override;
+	void VectorBernulliKLDerivative( const CConstFloatHandle& estimationHandle, const CFloatHandle& resultHandle, int vectorSize, const CConstFloatHandle& target ) override;
+	void VectorEltwiseDivide( const CConstIntHandle& firstHandle, const CConstIntHandle& secondHandle, const CIntHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwisePower( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorMinMaxDiff( const CConstFloatHandle& sourceGradHandle, int gradHeight, int gradWidth, const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, const CConstFloatHandle& minHandle, const CConstFloatHandle& maxHandle ) override;
+	void VectorPower( float exponent, const CConstFloatHandle& firstHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorPowerDiff( float exponent, const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorPowerDiffOp( float exponent, const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseNot( const CConstIntHandle& firstHandle, const CIntHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseNotNegative( const CConstIntHandle& firstHanle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseLess( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseLess( const CConstFloatHandle& firstHandle, float second, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseLess( float firstHandle, const CConstFloatHandle& secondHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseLess( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle, const CIntHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseLess( const CConstIntHandle& firstHandle, const CConstIntHandle& secondHandle, const CIntHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseEqual( const CConstFloatHandle& firstHandle, const CConstFloatHandle& secondHandle, const CIntHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseEqual( const CConstIntHandle& firstHandle, const CConstIntHandle& secondHandle, const CIntHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseWhere( const CConstIntHandle& firstHandle, const CConstFloatHandle& secondHandle, const CConstFloatHandle& thirdHandle, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorEltwiseWhere( const CConstIntHandle& firstHandle, const CConstIntHandle& secondHandle, const CConstIntHandle& thirdHandle, const CIntHandle& resultHandle, int vectorSize ) override;
+	void VectorFindMaxValueInSet( const CConstFloatHandle* vectors, int vectorCount, const CFloatHandle& resultHandle, int vectorSize ) override;
+	void VectorFindMaxValueInSet( const CConstFloatHandle* vectors, int vectorCount, const CFloatHandle& resultHandle, const CIntHandle& indexHandle, int vectorSize ) override;
+	void VectorSpreadValues( const CConstFloatHandle& sourceHandle, CFloatHandle* vectors, int vectorCount, const CConstIntHandle& indexHandle, int vectorSize ) override;
+	// ---- end of the members beyond the inference path ----
+
 	// every other pure virtual of the interface: asserting bodies generated from the interface header
 #include "HipMathEngineStubs.inc"
 
