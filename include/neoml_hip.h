@@ -488,6 +488,75 @@ NH_API int nhVectorMaxWithIndex(nhStream s, const float* candidate, float* resul
 /* One target of VectorSpreadValues (NME.h:377): target[i] = source[i] where indices[i] == index. */
 NH_API int nhVectorSpreadValuesTo(nhStream s, const float* source, float* target, const int* indices, int index, int vectorSize);
 
+/* ---- Indexed additions, row scatters, lookups (embeddings), binarizations, column-wise softmax, index planes,
+ * sub-sequences, up-sampling, space <-> depth: members beyond the benchmark networks' path. Semantics are the
+ * reference CPU engine's (src/CPU/CpuMathEngineBlas.cpp, CpuMathEngineDnn.cpp, CpuMathEngineDnnPooling.cpp). */
+NH_API int nhAddVectorToMatrixColumnsInt(nhStream s, const int* matrix, int* result, int matrixHeight, int matrixWidth,
+	const int* vector);                                                                                              /* NME.h:425 */
+NH_API int nhSumMatrixRowsInt(nhStream s, int batchSize, int* result, const int* matrix, int matrixHeight, int matrixWidth); /* NME.h:435 */
+NH_API int nhAddDiagMatrixToMatrix(nhStream s, const float* diagMatrix, const float* matrix, int height, int width, float* result); /* NME.h:411 */
+NH_API int nhMatrixColumnsEltwiseDivide(nhStream s, const float* matrix, int matrixHeight, int matrixWidth, const float* vector,
+	float* result);                                                                                                  /* NME.h:443 */
+NH_API int nhMultiply1DiagMatrixByMatrix(nhStream s, int batchSize, const float* first, int firstSize, const float* second,
+	int secondWidth, float* result);                                                                                 /* NME.h:575 */
+NH_API int nhMatrixSoftmaxByColumns(nhStream s, const float* matrix, int height, int width, float* result);          /* NME.h:458 */
+NH_API int nhMatrixSoftmaxDiffOpByColumns(nhStream s, const float* first, const float* second, int height, int width,
+	float* result);                                                                                                  /* NME.h:462 */
+NH_API int nhFindMinValueInColumns(nhStream s, const float* matrix, int matrixHeight, int matrixWidth, float* result,
+	int* rowIndices);                                                                                                /* NME.h:477 */
+NH_API int nhMatrixRowsToVectorSquaredL2Distance(nhStream s, const float* matrix, int matrixHeight, int matrixWidth,
+	const float* vector, float* result);                                                                             /* NME.h:865 */
+/* 32-bit elements, float (NME.h:616) or int (NME.h:621); fillValue: device pointer or null for zero. Rows with a negative
+ * index go nowhere; when two rows name the same target, which one stays is unspecified. */
+NH_API int nhMatrixSpreadRows(nhStream s, const void* source, int height, int width, void* result, int resultHeight,
+	const int* indices, const void* fillValue);
+NH_API int nhMatrixSpreadRowsAdd(nhStream s, const float* source, int height, int width, float* result, const int* indices); /* NME.h:619 */
+/* The indexed additions. mode 0: to[j] += from[j][first[j]] (AddMatrixElementsToVector, NME.h:404); 1: to[j][first[j]] +=
+ * from[j][first[j]] (AddMatrixElementsToMatrix, NME.h:415); 2: to[i] += from[first[i]][second[i]] (NME.h:406);
+ * 3: to[j][first[j]] += from[j] (AddVectorToMatrixElements, NME.h:397); 4: to[first[i]][second[i]] += from[i] (NME.h:400).
+ * count = rows (modes 0, 1, 3) or elements (2, 4); width = the matrix width; indices outside the row are skipped in 0, 1, 3. */
+NH_API int nhIndexedAdd(nhStream s, int mode, const float* from, float* to, int count, int width, const int* first, const int* second);
+NH_API int nhBuildIntegerHist(nhStream s, const int* numbers, int numbersCount, int* result, int maxNumber);         /* NME.h:861 */
+NH_API int nhEnumBinarization(nhStream s, int batchSize, const void* input, int inputIsFloat, int enumSize, float* result); /* NME.h:506, 508 */
+NH_API int nhBitSetBinarization(nhStream s, int batchSize, int bitSetSize, const int* input, int outputVectorSize, float* result); /* NME.h:513 */
+/* One lookup table of VectorMultichannelLookupAndCopy (NME.h:483-489): channel `channel` of each of the batchSize input
+ * rows (float or int) indexes `table` (32-bit elements); the vector goes to output columns [outputOffset, +vectorSize). */
+NH_API int nhLookupAndCopy(nhStream s, int batchSize, int channelCount, const void* input, int inputIsFloat, int channel,
+	const void* table, int vectorCount, int vectorSize, void* output, int outputChannels, int outputOffset);
+/* columns [inputOffset, +count) of every row to columns [outputOffset, +count): the channels behind the last table */
+NH_API int nhCopyColumns(nhStream s, int rows, const void* input, int inputWidth, int inputOffset, void* output, int outputWidth,
+	int outputOffset, int count);
+/* One table of VectorMultichannelLookupAndAddToTable (NME.h:493-496): table[index] += *mult * matrix[row][matrixOffset..] */
+NH_API int nhLookupAndAddToTable(nhStream s, int batchSize, int channelCount, const void* input, int inputIsFloat, int channel,
+	float* table, int vectorCount, int vectorSize, const float* mult, const float* matrix, int matrixWidth, int matrixOffset);
+NH_API int nhLookupAndSum(nhStream s, const int* indices, int batchSize, int indexCount, const float* table, int vectorSize,
+	float* result);                                                                                                  /* NME.h:500 */
+NH_API int nhLookupAndAddToWholeTable(nhStream s, const int* indices, int batchSize, int indexCount, const float* additions,
+	int vectorSize, float* table, int vectorCount);                                                                  /* LookupAndAddToTable, NME.h:502 */
+NH_API int nhMultiplyLookupMatrixByLookupVector(nhStream s, int batchSize, const float* matrixTable, const int* rows, int rowCount,
+	int width, const float* vectorTable, const int* vectors, float* result);                                         /* NME.h:518 */
+/* add = 0: NME.h:520, 1: ...AndAdd, NME.h:522 */
+NH_API int nhMultiplyTransposedLookupMatrixByVector(nhStream s, int batchSize, const float* table, const int* rows, int rowCount,
+	int width, const float* vector, float* result, int add);
+NH_API int nhMultiplyVectorByTransposedLookupVectorAndAddToTable(nhStream s, int batchSize, float* table, int vectorSize,
+	const int* index, const float* first, int firstSize, const float* secondTable, const int* secondVector);         /* NME.h:524 */
+/* result = source +- the index along the middle one of [outer][indexed][inner]: AddWidthIndex (NME.h:919-920) with
+ * indexed = width, AddHeightIndex (NME.h:927-928) with indexed = height */
+NH_API int nhAddDimIndex(nhStream s, const void* source, void* result, int isFloat, int outerSize, int indexedSize, int innerSize,
+	int forward);
+NH_API int nhBlobGetSubSequence(nhStream s, const float* from, int fromLength, int batchWidth, int objectSize, int* indices,
+	float* to, int toLength, int startPos, int isRev);                                                               /* NME.h:719 */
+NH_API int nhUpsampling2DForward(nhStream s, int objectCount, int height, int width, int pixelSize, const void* input,
+	int heightCopyCount, int widthCopyCount, void* result);                                                          /* NME.h:853, 855; 32-bit elements */
+NH_API int nhUpsampling2DBackward(nhStream s, int objectCount, int height, int width, int pixelSize, const float* input,
+	int heightCopyCount, int widthCopyCount, float* result);                                                         /* NME.h:857; height, width: of the result */
+/* SpaceToDepth (isForward, NME.h:902-904) and DepthToSpace (NME.h:909-911) on 32-bit elements; dataRowCount = objects x rows
+ * of blocks, dataRowWidth = blocks per row, blockChannels = channels of the "space" side */
+NH_API int nhSpaceToDepth(nhStream s, const void* source, int dataRowCount, int dataRowWidth, int blockChannels, int blockSize,
+	int isForward, void* result);
+NH_API int nhReorg(nhStream s, const void* source, int stride, int isForward, int batchSize, int channels, int height, int width,
+	void* result);                                                                                                   /* NME.h:895-897; 32-bit elements */
+
 #ifdef __cplusplus
 }
 #endif

@@ -415,6 +415,54 @@ public:
 	void VectorFindMaxValueInSet( const CConstFloatHandle* vectors, int vectorCount, const CFloatHandle& resultHandle, int vectorSize ) override;
 	void VectorFindMaxValueInSet( const CConstFloatHandle* vectors, int vectorCount, const CFloatHandle& resultHandle, const CIntHandle& indexHandle, int vectorSize ) override;
 	void VectorSpreadValues( const CConstFloatHandle& sourceHandle, CFloatHandle* vectors, int vectorCount, const CConstIntHandle& indexHandle, int vectorSize ) override;
+	// indexed additions, row scatters, lookups, binarizations, column-wise softmax, index planes, sub-sequences,
+	// up-sampling, space <-> depth
+	void AddVectorToMatrixElements( const CFloatHandle& matrix, int height, int width, const CConstIntHandle& indices, const CConstFloatHandle& vector ) override;
+	void AddVectorToMatrixElements( const CFloatHandle& matrix, int height, int width, const CConstIntHandle& rowIndices, const CConstIntHandle& columnIndices, const CConstFloatHandle& vector, int vectorSize ) override;
+	void AddMatrixElementsToVector( const CConstFloatHandle& matrix, int height, int width, const CConstIntHandle& indices, const CFloatHandle& result, int vectorSize ) override;
+	void AddMatrixElementsToVector( const CConstFloatHandle& matrix, int height, int width, const CConstIntHandle& rowIndices, const CConstIntHandle& columnIndices, const CFloatHandle& result, int vectorSize ) override;
+	void AddDiagMatrixToMatrix( const CConstFloatHandle& diagMatrix, const CConstFloatHandle& matrix, int height, int width, const CFloatHandle& result ) override;
+	void AddMatrixElementsToMatrix( const CConstFloatHandle& matrix, int height, int width, const CFloatHandle& result, const CConstIntHandle& indices ) override;
+	void AddVectorToMatrixColumns( const CConstIntHandle& matrixHandle, const CIntHandle& resultHandle, int matrixHeight, int matrixWidth, const CConstIntHandle& vectorHandle ) override;
+	void SumMatrixRows( int batchSize, const CIntHandle& resultHandle, const CConstIntHandle& matrixHandle, int matrixHeight, int matrixWidth ) override;
+	void MatrixColumnsEltwiseDivide( const CConstFloatHandle& matrix, int matrixHeight, int matrixWidth, const CConstFloatHandle& vector, const CFloatHandle& resultHandle ) override;
+	void MatrixSoftmaxByColumns( const CConstFloatHandle& matrix, int height, int width, const CFloatHandle& result ) override;
+	void MatrixSoftmaxDiffOpByColumns( const CConstFloatHandle& first, const CConstFloatHandle& second, int height, int width, const CFloatHandle& result ) override;
+	void FindMinValueInColumns( const CConstFloatHandle& matrixHandle, int matrixHeight, int matrixWidth, const CFloatHandle& resultHandle, const CIntHandle& columnIndices ) override;
+	void VectorMultichannelLookupAndCopy( int batchSize, int channelCount, const CConstFloatHandle& inputHandle, const CConstFloatHandle* lookupHandles, const CLookupDimension* lookupDimensions, int lookupCount, const CFloatHandle& outputHandle, int outputChannels ) override;
+	void VectorMultichannelLookupAndCopy( int batchSize, int channelCount, const CConstIntHandle& inputHandle, const CConstFloatHandle* lookupHandles, const CLookupDimension* lookupDimensions, int lookupCount, const CFloatHandle& outputHandle, int outputChannels ) override;
+	void VectorMultichannelLookupAndCopy( int batchSize, int channelCount, const CConstIntHandle& inputHandle, const CConstIntHandle* lookupHandles, const CLookupDimension* lookupDimensions, int lookupCount, const CIntHandle& outputHandle, int outputChannels ) override;
+	void VectorMultichannelLookupAndAddToTable( int batchSize, int channelCount, const CConstFloatHandle& inputHandle, const CFloatHandle* lookupHandles, const CLookupDimension* lookupDimensions, int lookupCount, const CConstFloatHandle& multHandle, const CConstFloatHandle& matrixHandle, int outputChannels ) override;
+	void VectorMultichannelLookupAndAddToTable( int batchSize, int channelCount, const CConstIntHandle& inputHandle, const CFloatHandle* lookupHandles, const CLookupDimension* lookupDimensions, int lookupCount, const CConstFloatHandle& multHandle, const CConstFloatHandle& matrixHandle, int outputChannels ) override;
+	void LookupAndSum( const CConstIntHandle& indicesHandle, int batchSize, int indexCount, const CConstFloatHandle& tableHandle, int vectorSize, const CFloatHandle& result ) override;
+	void LookupAndAddToTable( const CConstIntHandle& indicesHandle, int batchSize, int indexCount, const CConstFloatHandle& additionsHandle, int vectorSize, const CFloatHandle& tableHandle, int vectorCount ) override;
+	void EnumBinarization( int batchSize, const CConstFloatHandle& inputHandle, int enumSize, const CFloatHandle& resultHandle ) override;
+	void EnumBinarization( int batchSize, const CConstIntHandle& inputHandle, int enumSize, const CFloatHandle& resultHandle ) override;
+	void BitSetBinarization( int batchSize, int bitSetSize, const CConstIntHandle& inputHandle, int outputVectorSize, const CFloatHandle& resultHandle ) override;
+	void MultiplyLookupMatrixByLookupVector( int batchSize, const CLookupMatrix& matrix, const CLookupVector& vector, const CFloatHandle& result, int resultSize ) override;
+	void MultiplyTransposedLookupMatrixByVector( int batchSize, const CLookupMatrix& matrix, const CConstFloatHandle& vectorHandle, const CFloatHandle& resultHandle, int resultSize ) override;
+	void MultiplyTransposedLookupMatrixByVectorAndAdd( int batchSize, const CLookupMatrix& matrix, const CConstFloatHandle& vectorHandle, const CFloatHandle& resultHandle, int resultSize ) override;
+	void MultiplyVectorByTransposedLookupVectorAndAddToTable( int batchSize, const CFloatHandle& tableHandle, int vectorCount, int vectorSize, const CConstIntHandle& indices, const CConstFloatHandle& firstHandle, int firstSize, const CLookupVector& secondVector ) override;
+	void Multiply1DiagMatrixByMatrix( int batchSize, const CConstFloatHandle& firstHandle, int firstSize, const CConstFloatHandle& secondHandle, int secondWidth, const CFloatHandle& resultHandle, int resultBufferSize ) override;
+	void MatrixSpreadRows( const CConstFloatHandle& sourceHandle, int height, int width, const CFloatHandle& resultHandle, int resultHeight, const CConstIntHandle& indexHandle, const CConstFloatHandle& fillValue ) override;
+	void MatrixSpreadRowsAdd( const CConstFloatHandle& sourceHandle, int height, int width, const CFloatHandle& resultHandle, int resultHeight, const CConstIntHandle& indexHandle ) override;
+	void MatrixSpreadRows( const CConstIntHandle& sourceHandle, int height, int width, const CIntHandle& resultHandle, int resultHeight, const CConstIntHandle& indexHandle, const CConstIntHandle& fillValue ) override;
+	void BlobGetSubSequence( const CBlobDesc& from, const CFloatHandle& fromData, const CIntHandle& indexHandle, const CBlobDesc& to, const CFloatHandle& toData, int startPos, bool isRev ) override;
+	void Upsampling2DForward( const CBlobDesc& input, const CConstIntHandle& inputData, int heightCopyCount, int widthCopyCount, const CBlobDesc& result, const CIntHandle& resultData ) override;
+	void Upsampling2DForward( const CBlobDesc& input, const CConstFloatHandle& inputData, int heightCopyCount, int widthCopyCount, const CBlobDesc& result, const CFloatHandle& resultData ) override;
+	void Upsampling2DBackward( const CBlobDesc& input, const CConstFloatHandle& inputData, int heightCopyCount, int widthCopyCount, const CBlobDesc& result, const CFloatHandle& resultData ) override;
+	void BuildIntegerHist( const CConstIntHandle& numbersHandle, int numbersCount, const CIntHandle& resultHandle, int maxNumber ) override;
+	void MatrixRowsToVectorSquaredL2Distance( const CConstFloatHandle& matrixHandle, const int matrixHeight, const int matrixWidth, const CConstFloatHandle& vectorHandle, const CFloatHandle& resultHandle ) override;
+	void Reorg( const CBlobDesc& source, const CFloatHandle& sourceData, int stride, bool isForward, const CBlobDesc& result, const CFloatHandle& resultData ) override;
+	void Reorg( const CBlobDesc& source, const CIntHandle& sourceData, int stride, bool isForward, const CBlobDesc& result, const CIntHandle& resultData ) override;
+	void SpaceToDepth( const CBlobDesc& source, const CConstFloatHandle& sourceData, int blockSize, const CBlobDesc& result, const CFloatHandle& resultData ) override;
+	void SpaceToDepth( const CBlobDesc& source, const CConstIntHandle& sourceData, int blockSize, const CBlobDesc& result, const CIntHandle& resultData ) override;
+	void DepthToSpace( const CBlobDesc& source, const CConstFloatHandle& sourceData, int blockSize, const CBlobDesc& result, const CFloatHandle& resultData ) override;
+	void DepthToSpace( const CBlobDesc& source, const CConstIntHandle& sourceData, int blockSize, const CBlobDesc& result, const CIntHandle& resultData ) override;
+	void AddWidthIndex( const CBlobDesc& source, const CConstFloatHandle& sourceData, bool isForward, const CFloatHandle& result ) override;
+	void AddWidthIndex( const CBlobDesc& source, const CConstIntHandle& sourceData, bool isForward, const CIntHandle& result ) override;
+	void AddHeightIndex( const CBlobDesc& source, const CConstFloatHandle& sourceData, bool isForward, const CFloatHandle& result ) override;
+	void AddHeightIndex( const CBlobDesc& source, const CConstIntHandle& sourceData, bool isForward, const CIntHandle& result ) override;
 	// ---- end of the members beyond the inference path ----
 
 	// every other pure virtual of the interface: asserting bodies generated from the interface header

@@ -229,4 +229,360 @@ void CHipMathEngine::VectorSpreadValues( const CConstFloatHandle& sourceHandle, 
 	}
 }
 
+// ---- indexed additions ( one entry point, the mode names the member ) ----------------------------------------
+
+void CHipMathEngine::AddMatrixElementsToVector( const CConstFloatHandle& matrix, int height, int width, const CConstIntHandle& indices,
+	const CFloatHandle& result, int vectorSize )
+{
+	ASSERT_EXPR( vectorSize >= height );
+	NH_CALL( nhIndexedAdd( stream, 0, raw( matrix ), raw( result ), height, width, raw( indices ), nullptr ) );
+}
+
+void CHipMathEngine::AddMatrixElementsToMatrix( const CConstFloatHandle& matrix, int height, int width, const CFloatHandle& result,
+	const CConstIntHandle& indices )
+{
+	NH_CALL( nhIndexedAdd( stream, 1, raw( matrix ), raw( result ), height, width, raw( indices ), nullptr ) );
+}
+
+void CHipMathEngine::AddMatrixElementsToVector( const CConstFloatHandle& matrix, int height, int width, const CConstIntHandle& rowIndices,
+	const CConstIntHandle& columnIndices, const CFloatHandle& result, int vectorSize )
+{
+	NH_CALL( nhIndexedAdd( stream, 2, raw( matrix ), raw( result ), vectorSize, width, raw( rowIndices ), raw( columnIndices ) ) );
+}
+
+void CHipMathEngine::AddVectorToMatrixElements( const CFloatHandle& matrix, int height, int width, const CConstIntHandle& indices,
+	const CConstFloatHandle& vector )
+{
+	NH_CALL( nhIndexedAdd( stream, 3, raw( vector ), raw( matrix ), height, width, raw( indices ), nullptr ) );
+}
+
+void CHipMathEngine::AddVectorToMatrixElements( const CFloatHandle& matrix, int height, int width, const CConstIntHandle& rowIndices,
+	const CConstIntHandle& columnIndices, const CConstFloatHandle& vector, int vectorSize )
+{
+	NH_CALL( nhIndexedAdd( stream, 4, raw( vector ), raw( matrix ), vectorSize, width, raw( rowIndices ), raw( columnIndices ) ) );
+}
+
+// ---- matrices -------------------------------------------------------------------------------------------------
+
+void CHipMathEngine::AddDiagMatrixToMatrix( const CConstFloatHandle& diagMatrix, const CConstFloatHandle& matrix, int height, int width,
+	const CFloatHandle& result )
+{
+	NH_CALL( nhAddDiagMatrixToMatrix( stream, raw( diagMatrix ), raw( matrix ), height, width, raw( result ) ) );
+}
+
+void CHipMathEngine::AddVectorToMatrixColumns( const CConstIntHandle& matrixHandle, const CIntHandle& resultHandle, int matrixHeight,
+	int matrixWidth, const CConstIntHandle& vectorHandle )
+{
+	NH_CALL( nhAddVectorToMatrixColumnsInt( stream, raw( matrixHandle ), raw( resultHandle ), matrixHeight, matrixWidth, raw( vectorHandle ) ) );
+}
+
+void CHipMathEngine::SumMatrixRows( int batchSize, const CIntHandle& resultHandle, const CConstIntHandle& matrixHandle, int matrixHeight,
+	int matrixWidth )
+{
+	NH_CALL( nhSumMatrixRowsInt( stream, batchSize, raw( resultHandle ), raw( matrixHandle ), matrixHeight, matrixWidth ) );
+}
+
+void CHipMathEngine::MatrixColumnsEltwiseDivide( const CConstFloatHandle& matrix, int matrixHeight, int matrixWidth,
+	const CConstFloatHandle& vector, const CFloatHandle& resultHandle )
+{
+	NH_CALL( nhMatrixColumnsEltwiseDivide( stream, raw( matrix ), matrixHeight, matrixWidth, raw( vector ), raw( resultHandle ) ) );
+}
+
+void CHipMathEngine::MatrixSoftmaxByColumns( const CConstFloatHandle& matrix, int height, int width, const CFloatHandle& result )
+{
+	NH_CALL( nhMatrixSoftmaxByColumns( stream, raw( matrix ), height, width, raw( result ) ) );
+}
+
+void CHipMathEngine::MatrixSoftmaxDiffOpByColumns( const CConstFloatHandle& first, const CConstFloatHandle& second, int height, int width,
+	const CFloatHandle& result )
+{
+	NH_CALL( nhMatrixSoftmaxDiffOpByColumns( stream, raw( first ), raw( second ), height, width, raw( result ) ) );
+}
+
+void CHipMathEngine::FindMinValueInColumns( const CConstFloatHandle& matrixHandle, int matrixHeight, int matrixWidth,
+	const CFloatHandle& resultHandle, const CIntHandle& columnIndices )
+{
+	NH_CALL( nhFindMinValueInColumns( stream, raw( matrixHandle ), matrixHeight, matrixWidth, raw( resultHandle ), raw( columnIndices ) ) );
+}
+
+void CHipMathEngine::Multiply1DiagMatrixByMatrix( int batchSize, const CConstFloatHandle& firstHandle, int firstSize,
+	const CConstFloatHandle& secondHandle, int secondWidth, const CFloatHandle& resultHandle, int )
+{
+	NH_CALL( nhMultiply1DiagMatrixByMatrix( stream, batchSize, raw( firstHandle ), firstSize, raw( secondHandle ), secondWidth, raw( resultHandle ) ) );
+}
+
+void CHipMathEngine::MatrixRowsToVectorSquaredL2Distance( const CConstFloatHandle& matrixHandle, const int matrixHeight, const int matrixWidth,
+	const CConstFloatHandle& vectorHandle, const CFloatHandle& resultHandle )
+{
+	NH_CALL( nhMatrixRowsToVectorSquaredL2Distance( stream, raw( matrixHandle ), matrixHeight, matrixWidth, raw( vectorHandle ), raw( resultHandle ) ) );
+}
+
+void CHipMathEngine::MatrixSpreadRows( const CConstFloatHandle& sourceHandle, int height, int width, const CFloatHandle& resultHandle,
+	int resultHeight, const CConstIntHandle& indexHandle, const CConstFloatHandle& fillValue )
+{
+	NH_CALL( nhMatrixSpreadRows( stream, raw( sourceHandle ), height, width, raw( resultHandle ), resultHeight, raw( indexHandle ),
+		fillValue.IsNull() ? nullptr : raw( fillValue ) ) );
+}
+
+void CHipMathEngine::MatrixSpreadRows( const CConstIntHandle& sourceHandle, int height, int width, const CIntHandle& resultHandle,
+	int resultHeight, const CConstIntHandle& indexHandle, const CConstIntHandle& fillValue )
+{
+	NH_CALL( nhMatrixSpreadRows( stream, raw( sourceHandle ), height, width, raw( resultHandle ), resultHeight, raw( indexHandle ),
+		fillValue.IsNull() ? nullptr : raw( fillValue ) ) );
+}
+
+void CHipMathEngine::MatrixSpreadRowsAdd( const CConstFloatHandle& sourceHandle, int height, int width, const CFloatHandle& resultHandle,
+	int, const CConstIntHandle& indexHandle )
+{
+	NH_CALL( nhMatrixSpreadRowsAdd( stream, raw( sourceHandle ), height, width, raw( resultHandle ), raw( indexHandle ) ) );
+}
+
+void CHipMathEngine::BuildIntegerHist( const CConstIntHandle& numbersHandle, int numbersCount, const CIntHandle& resultHandle, int maxNumber )
+{
+	NH_CALL( nhBuildIntegerHist( stream, raw( numbersHandle ), numbersCount, raw( resultHandle ), maxNumber ) );
+}
+
+void CHipMathEngine::EnumBinarization( int batchSize, const CConstFloatHandle& inputHandle, int enumSize, const CFloatHandle& resultHandle )
+{
+	NH_CALL( nhEnumBinarization( stream, batchSize, raw( inputHandle ), 1, enumSize, raw( resultHandle ) ) );
+}
+
+void CHipMathEngine::EnumBinarization( int batchSize, const CConstIntHandle& inputHandle, int enumSize, const CFloatHandle& resultHandle )
+{
+	NH_CALL( nhEnumBinarization( stream, batchSize, raw( inputHandle ), 0, enumSize, raw( resultHandle ) ) );
+}
+
+void CHipMathEngine::BitSetBinarization( int batchSize, int bitSetSize, const CConstIntHandle& inputHandle, int outputVectorSize,
+	const CFloatHandle& resultHandle )
+{
+	NH_CALL( nhBitSetBinarization( stream, batchSize, bitSetSize, raw( inputHandle ), outputVectorSize, raw( resultHandle ) ) );
+}
+
+// ---- lookups: one launch per table, as the tables are separate blobs ( src/CPU/CpuMathEngineBlas.cpp:432-571 ) ----------
+
+void CHipMathEngine::VectorMultichannelLookupAndCopy( int batchSize, int channelCount, const CConstFloatHandle& inputHandle,
+	const CConstFloatHandle* lookupHandles, const CLookupDimension* lookupDimensions, int lookupCount, const CFloatHandle& outputHandle,
+	int outputChannels )
+{
+	int offset = 0;
+	for( int j = 0; j < lookupCount; ++j ) {
+		NH_CALL( nhLookupAndCopy( stream, batchSize, channelCount, raw( inputHandle ), 1, j, raw( lookupHandles[j] ),
+			lookupDimensions[j].VectorCount, lookupDimensions[j].VectorSize, raw( outputHandle ), outputChannels, offset ) );
+		offset += lookupDimensions[j].VectorSize;
+	}
+	if( channelCount > lookupCount ) {
+		NH_CALL( nhCopyColumns( stream, batchSize, raw( inputHandle ), channelCount, lookupCount, raw( outputHandle ), outputChannels, offset,
+			channelCount - lookupCount ) );
+	}
+}
+
+void CHipMathEngine::VectorMultichannelLookupAndCopy( int batchSize, int channelCount, const CConstIntHandle& inputHandle,
+	const CConstFloatHandle* lookupHandles, const CLookupDimension* lookupDimensions, int lookupCount, const CFloatHandle& outputHandle,
+	int outputChannels )
+{
+	int offset = 0;
+	for( int j = 0; j < lookupCount && j < channelCount; ++j ) {
+		NH_CALL( nhLookupAndCopy( stream, batchSize, channelCount, raw( inputHandle ), 0, j, raw( lookupHandles[j] ),
+			lookupDimensions[j].VectorCount, lookupDimensions[j].VectorSize, raw( outputHandle ), outputChannels, offset ) );
+		offset += lookupDimensions[j].VectorSize;
+	}
+}
+
+void CHipMathEngine::VectorMultichannelLookupAndCopy( int batchSize, int channelCount, const CConstIntHandle& inputHandle,
+	const CConstIntHandle* lookupHandles, const CLookupDimension* lookupDimensions, int lookupCount, const CIntHandle& outputHandle,
+	int outputChannels )
+{
+	int offset = 0;
+	for( int j = 0; j < lookupCount; ++j ) {
+		NH_CALL( nhLookupAndCopy( stream, batchSize, channelCount, raw( inputHandle ), 0, j, raw( lookupHandles[j] ),
+			lookupDimensions[j].VectorCount, lookupDimensions[j].VectorSize, raw( outputHandle ), outputChannels, offset ) );
+		offset += lookupDimensions[j].VectorSize;
+	}
+	if( channelCount > lookupCount ) {
+		NH_CALL( nhCopyColumns( stream, batchSize, raw( inputHandle ), channelCount, lookupCount, raw( outputHandle ), outputChannels, offset,
+			channelCount - lookupCount ) );
+	}
+}
+
+// the gradient matrix has a row per input row: the tables' vectors side by side, then the unmapped channels
+static int lookupMatrixWidth( const CLookupDimension* lookupDimensions, int lookupCount, int channelCount )
+{
+	int width = 0;
+	for( int j = 0; j < lookupCount && j < channelCount; ++j ) {
+		width += lookupDimensions[j].VectorSize;
+	}
+	return width + ( channelCount > lookupCount ? channelCount - lookupCount : 0 );
+}
+
+void CHipMathEngine::VectorMultichannelLookupAndAddToTable( int batchSize, int channelCount, const CConstFloatHandle& inputHandle,
+	const CFloatHandle* lookupHandles, const CLookupDimension* lookupDimensions, int lookupCount, const CConstFloatHandle& multHandle,
+	const CConstFloatHandle& matrixHandle, int )
+{
+	const int matrixWidth = lookupMatrixWidth( lookupDimensions, lookupCount, channelCount );
+	int offset = 0;
+	for( int j = 0; j < lookupCount && j < channelCount; ++j ) {
+		NH_CALL( nhLookupAndAddToTable( stream, batchSize, channelCount, raw( inputHandle ), 1, j, raw( lookupHandles[j] ),
+			lookupDimensions[j].VectorCount, lookupDimensions[j].VectorSize, raw( multHandle ), raw( matrixHandle ), matrixWidth, offset ) );
+		offset += lookupDimensions[j].VectorSize;
+	}
+}
+
+void CHipMathEngine::VectorMultichannelLookupAndAddToTable( int batchSize, int channelCount, const CConstIntHandle& inputHandle,
+	const CFloatHandle* lookupHandles, const CLookupDimension* lookupDimensions, int lookupCount, const CConstFloatHandle& multHandle,
+	const CConstFloatHandle& matrixHandle, int )
+{
+	const int matrixWidth = lookupMatrixWidth( lookupDimensions, lookupCount, channelCount );
+	int offset = 0;
+	for( int j = 0; j < lookupCount && j < channelCount; ++j ) {
+		NH_CALL( nhLookupAndAddToTable( stream, batchSize, channelCount, raw( inputHandle ), 0, j, raw( lookupHandles[j] ),
+			lookupDimensions[j].VectorCount, lookupDimensions[j].VectorSize, raw( multHandle ), raw( matrixHandle ), matrixWidth, offset ) );
+		offset += lookupDimensions[j].VectorSize;
+	}
+}
+
+void CHipMathEngine::LookupAndSum( const CConstIntHandle& indicesHandle, int batchSize, int indexCount, const CConstFloatHandle& tableHandle,
+	int vectorSize, const CFloatHandle& result )
+{
+	NH_CALL( nhLookupAndSum( stream, raw( indicesHandle ), batchSize, indexCount, raw( tableHandle ), vectorSize, raw( result ) ) );
+}
+
+void CHipMathEngine::LookupAndAddToTable( const CConstIntHandle& indicesHandle, int batchSize, int indexCount,
+	const CConstFloatHandle& additionsHandle, int vectorSize, const CFloatHandle& tableHandle, int vectorCount )
+{
+	NH_CALL( nhLookupAndAddToWholeTable( stream, raw( indicesHandle ), batchSize, indexCount, raw( additionsHandle ), vectorSize,
+		raw( tableHandle ), vectorCount ) );
+}
+
+void CHipMathEngine::MultiplyLookupMatrixByLookupVector( int batchSize, const CLookupMatrix& matrix, const CLookupVector& vector,
+	const CFloatHandle& result, int )
+{
+	ASSERT_EXPR( matrix.Width() == vector.VectorSize() );
+	NH_CALL( nhMultiplyLookupMatrixByLookupVector( stream, batchSize, raw( matrix.Table ), raw( matrix.Rows ), matrix.RowCount, matrix.Width(),
+		raw( vector.Table ), raw( vector.Vector ), raw( result ) ) );
+}
+
+void CHipMathEngine::MultiplyTransposedLookupMatrixByVector( int batchSize, const CLookupMatrix& matrix, const CConstFloatHandle& vectorHandle,
+	const CFloatHandle& resultHandle, int )
+{
+	NH_CALL( nhMultiplyTransposedLookupMatrixByVector( stream, batchSize, raw( matrix.Table ), raw( matrix.Rows ), matrix.RowCount, matrix.Width(),
+		raw( vectorHandle ), raw( resultHandle ), 0 ) );
+}
+
+void CHipMathEngine::MultiplyTransposedLookupMatrixByVectorAndAdd( int batchSize, const CLookupMatrix& matrix,
+	const CConstFloatHandle& vectorHandle, const CFloatHandle& resultHandle, int )
+{
+	NH_CALL( nhMultiplyTransposedLookupMatrixByVector( stream, batchSize, raw( matrix.Table ), raw( matrix.Rows ), matrix.RowCount, matrix.Width(),
+		raw( vectorHandle ), raw( resultHandle ), 1 ) );
+}
+
+void CHipMathEngine::MultiplyVectorByTransposedLookupVectorAndAddToTable( int batchSize, const CFloatHandle& tableHandle, int, int vectorSize,
+	const CConstIntHandle& indices, const CConstFloatHandle& firstHandle, int firstSize, const CLookupVector& secondVector )
+{
+	ASSERT_EXPR( vectorSize == secondVector.VectorSize() );
+	NH_CALL( nhMultiplyVectorByTransposedLookupVectorAndAddToTable( stream, batchSize, raw( tableHandle ), vectorSize, raw( indices ),
+		raw( firstHandle ), firstSize, raw( secondVector.Table ), raw( secondVector.Vector ) ) );
+}
+
+// ---- blobs ------------------------------------------------------------------------------------------------------
+
+void CHipMathEngine::AddWidthIndex( const CBlobDesc& source, const CConstFloatHandle& sourceData, bool isForward, const CFloatHandle& result )
+{
+	NH_CALL( nhAddDimIndex( stream, raw( sourceData ), raw( result ), 1, source.ObjectCount() * source.Height(), source.Width(),
+		source.Depth() * source.Channels(), isForward ? 1 : 0 ) );
+}
+
+void CHipMathEngine::AddWidthIndex( const CBlobDesc& source, const CConstIntHandle& sourceData, bool isForward, const CIntHandle& result )
+{
+	NH_CALL( nhAddDimIndex( stream, raw( sourceData ), raw( result ), 0, source.ObjectCount() * source.Height(), source.Width(),
+		source.Depth() * source.Channels(), isForward ? 1 : 0 ) );
+}
+
+void CHipMathEngine::AddHeightIndex( const CBlobDesc& source, const CConstFloatHandle& sourceData, bool isForward, const CFloatHandle& result )
+{
+	NH_CALL( nhAddDimIndex( stream, raw( sourceData ), raw( result ), 1, source.ObjectCount(), source.Height(),
+		source.Width() * source.Depth() * source.Channels(), isForward ? 1 : 0 ) );
+}
+
+void CHipMathEngine::AddHeightIndex( const CBlobDesc& source, const CConstIntHandle& sourceData, bool isForward, const CIntHandle& result )
+{
+	NH_CALL( nhAddDimIndex( stream, raw( sourceData ), raw( result ), 0, source.ObjectCount(), source.Height(),
+		source.Width() * source.Depth() * source.Channels(), isForward ? 1 : 0 ) );
+}
+
+void CHipMathEngine::BlobGetSubSequence( const CBlobDesc& from, const CFloatHandle& fromData, const CIntHandle& indexHandle,
+	const CBlobDesc& to, const CFloatHandle& toData, int startPos, bool isRev )
+{
+	ASSERT_EXPR( from.BatchWidth() == to.BatchWidth() && from.ObjectSize() == to.ObjectSize() && from.ListSize() == to.ListSize() );
+	NH_CALL( nhBlobGetSubSequence( stream, raw( fromData ), from.BatchLength(), from.BatchWidth(), from.ObjectSize() * from.ListSize(),
+		indexHandle.IsNull() ? nullptr : raw( indexHandle ), raw( toData ), to.BatchLength(), startPos, isRev ? 1 : 0 ) );
+}
+
+void CHipMathEngine::Upsampling2DForward( const CBlobDesc& input, const CConstIntHandle& inputData, int heightCopyCount, int widthCopyCount,
+	const CBlobDesc& result, const CIntHandle& resultData )
+{
+	ASSERT_EXPR( result.Height() == input.Height() * heightCopyCount && result.Width() == input.Width() * widthCopyCount );
+	NH_CALL( nhUpsampling2DForward( stream, input.ObjectCount(), input.Height(), input.Width(), input.Depth() * input.Channels(),
+		raw( inputData ), heightCopyCount, widthCopyCount, raw( resultData ) ) );
+}
+
+void CHipMathEngine::Upsampling2DForward( const CBlobDesc& input, const CConstFloatHandle& inputData, int heightCopyCount, int widthCopyCount,
+	const CBlobDesc& result, const CFloatHandle& resultData )
+{
+	ASSERT_EXPR( result.Height() == input.Height() * heightCopyCount && result.Width() == input.Width() * widthCopyCount );
+	NH_CALL( nhUpsampling2DForward( stream, input.ObjectCount(), input.Height(), input.Width(), input.Depth() * input.Channels(),
+		raw( inputData ), heightCopyCount, widthCopyCount, raw( resultData ) ) );
+}
+
+void CHipMathEngine::Upsampling2DBackward( const CBlobDesc& input, const CConstFloatHandle& inputData, int heightCopyCount, int widthCopyCount,
+	const CBlobDesc& result, const CFloatHandle& resultData )
+{
+	ASSERT_EXPR( input.Height() == result.Height() * heightCopyCount && input.Width() == result.Width() * widthCopyCount );
+	NH_CALL( nhUpsampling2DBackward( stream, input.ObjectCount(), result.Height(), result.Width(), input.Depth() * input.Channels(),
+		raw( inputData ), heightCopyCount, widthCopyCount, raw( resultData ) ) );
+}
+
+void CHipMathEngine::Reorg( const CBlobDesc& source, const CFloatHandle& sourceData, int stride, bool isForward, const CBlobDesc& result,
+	const CFloatHandle& resultData )
+{
+	const CBlobDesc& dims = isForward ? source : result;
+	NH_CALL( nhReorg( stream, raw( sourceData ), stride, isForward ? 1 : 0, source.ObjectCount(), dims.Channels(), dims.Height(), dims.Width(),
+		raw( resultData ) ) );
+}
+
+void CHipMathEngine::Reorg( const CBlobDesc& source, const CIntHandle& sourceData, int stride, bool isForward, const CBlobDesc& result,
+	const CIntHandle& resultData )
+{
+	const CBlobDesc& dims = isForward ? source : result;
+	NH_CALL( nhReorg( stream, raw( sourceData ), stride, isForward ? 1 : 0, source.ObjectCount(), dims.Channels(), dims.Height(), dims.Width(),
+		raw( resultData ) ) );
+}
+
+void CHipMathEngine::SpaceToDepth( const CBlobDesc& source, const CConstFloatHandle& sourceData, int blockSize, const CBlobDesc& result,
+	const CFloatHandle& resultData )
+{
+	NH_CALL( nhSpaceToDepth( stream, raw( sourceData ), source.ObjectCount() * result.Height(), result.Width(), source.Channels(), blockSize, 1,
+		raw( resultData ) ) );
+}
+
+void CHipMathEngine::SpaceToDepth( const CBlobDesc& source, const CConstIntHandle& sourceData, int blockSize, const CBlobDesc& result,
+	const CIntHandle& resultData )
+{
+	NH_CALL( nhSpaceToDepth( stream, raw( sourceData ), source.ObjectCount() * result.Height(), result.Width(), source.Channels(), blockSize, 1,
+		raw( resultData ) ) );
+}
+
+void CHipMathEngine::DepthToSpace( const CBlobDesc& source, const CConstFloatHandle& sourceData, int blockSize, const CBlobDesc& result,
+	const CFloatHandle& resultData )
+{
+	NH_CALL( nhSpaceToDepth( stream, raw( sourceData ), source.ObjectCount() * source.Height(), source.Width(), result.Channels(), blockSize, 0,
+		raw( resultData ) ) );
+}
+
+void CHipMathEngine::DepthToSpace( const CBlobDesc& source, const CConstIntHandle& sourceData, int blockSize, const CBlobDesc& result,
+	const CIntHandle& resultData )
+{
+	NH_CALL( nhSpaceToDepth( stream, raw( sourceData ), source.ObjectCount() * source.Height(), source.Width(), result.Channels(), blockSize, 0,
+		raw( resultData ) ) );
+}
+
 } // namespace NeoML
