@@ -305,7 +305,10 @@ typedef struct nhConvDesc {
 } nhConvDesc;
 
 /* InitBlobConvolution (NME.h:751): fills resultHeight/resultWidth and validates; returns NH_ERR_ARGUMENT
- * where the reference asserts. */
+ * where the reference asserts. The convolution entry points also accept other result sizes: fewer or more rows (columns)
+ * than equal padding on both sides gives stand for a different padding at the end (below the filter's span), which is how
+ * the convolution over time runs through them (InitTimeConvolution / BlobTimeConvolution*, NME.h:724-731: the sequence
+ * axis as the height, the batch width as the width, paddingFront as paddingHeight, paddingBack implied by the length). */
 NH_API int nhInitBlobConvolution(nhConvDesc* desc_host);
 /* freeTerm may be null */
 NH_API int nhBlobConvolution(nhStream s, const nhConvDesc* desc_host, const float* source, const float* filter,
@@ -556,6 +559,27 @@ NH_API int nhSpaceToDepth(nhStream s, const void* source, int dataRowCount, int 
 	int isForward, void* result);
 NH_API int nhReorg(nhStream s, const void* source, int stride, int isForward, int batchSize, int channels, int height, int width,
 	void* result);                                                                                                   /* NME.h:895-897; 32-bit elements */
+
+/* BlobGlobalMaxPooling (NME.h:787): per (object, channel) the maxCount largest of poolSize values, descending, with their
+ * pixel indices; equal values: the later pixel first; empty slots hold -FLT_MAX / -1. source [objects][poolSize][channels],
+ * result and maxIndices [objects][maxCount][channels]. */
+NH_API int nhBlobGlobalMaxPooling(nhStream s, int objectCount, int poolSize, int channels, int maxCount, const float* source,
+	int* maxIndices, float* result);
+NH_API int nhBlobGlobalMaxPoolingBackward(nhStream s, int objectCount, int poolSize, int channels, int maxCount,
+	const float* resultDiff, const int* maxIndices, float* sourceDiff);                                              /* NME.h:789 */
+/* BlobMaxOverTimePooling (NME.h:830): source [sourceLength][seqElemSize]; maxIndices may be null */
+NH_API int nhBlobMaxOverTimePooling(nhStream s, int sourceLength, int seqElemSize, int filterLen, int strideLen, const float* source,
+	int* maxIndices, float* result);
+/* global = 0: BlobMaxOverTimePoolingBackward (NME.h:832, additions); 1: BlobGlobalMaxOverTimePoolingBackward (NME.h:850, stores).
+ * The forward pass of the global form is nhFindMaxValueInColumns over [sourceLength][seqElemSize]. */
+NH_API int nhBlobOverTimePoolingBackward(nhStream s, int sourceLength, int resultLength, int seqElemSize, const float* resultDiff,
+	const int* maxIndices, float* sourceDiff, int global);
+/* LinearInterpolation (NME.h:1049). coords: 0 half pixel, 1 PyTorch half pixel, 2 align corners, 3 asymmetric
+ * (TInterpolationCoords, NME.h:40-46); round: 0 none, 1 half down, 2 half up, 3 floor, 4 ceil (TInterpolationRound, NME.h:51-57) */
+NH_API int nhLinearInterpolation(nhStream s, const float* data, float* result, int coords, int round, int objectCount, int scaledAxis,
+	int objectSize, float scale);
+NH_API int nhScatterND(nhStream s, const int* indices, const void* updates, void* data, const nhBlobDesc* dataDesc_host, int updateCount,
+	int indexDims);                                                                                                  /* NME.h:1061-1063; 32-bit elements */
 
 #ifdef __cplusplus
 }

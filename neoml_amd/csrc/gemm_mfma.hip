@@ -2081,15 +2081,27 @@ int nhInitBlobConvolution( nhConvDesc* d )
 	return NH_OK;
 }
 
+// What every convolution entry point asks of a descriptor. The result sizes need not be the ones nhInitBlobConvolution
+// computes for equal padding on both sides: fewer or more rows ( columns ) are taken as a different padding at the end,
+// as long as the padding at the end stays within the larger of the padding at the beginning and the filter's span - 1.
+// The kernels read whatever lies beyond the image as zeros wherever it is, so the padding at the end needs no field.
 static int checkedConvDesc( const nhConvDesc* d )
 {
 	NH_REQUIRE( d != nullptr );
-	nhConvDesc check = *d;
-	const int rc = nhInitBlobConvolution( &check );
-	if( rc != NH_OK ) {
-		return rc;
-	}
-	NH_REQUIRE( check.resultHeight == d->resultHeight && check.resultWidth == d->resultWidth );
+	NH_REQUIRE( d->batch >= 0 && d->height > 0 && d->width > 0 && d->channels > 0 );
+	NH_REQUIRE( d->filterCount > 0 && d->filterHeight > 0 && d->filterWidth > 0 );
+	NH_REQUIRE( d->paddingHeight >= 0 && d->paddingWidth >= 0 );
+	NH_REQUIRE( d->strideHeight > 0 && d->strideWidth > 0 && d->dilationHeight > 0 && d->dilationWidth > 0 );
+	const int spanH = ( d->filterHeight - 1 ) * d->dilationHeight + 1;
+	const int spanW = ( d->filterWidth - 1 ) * d->dilationWidth + 1;
+	const int endH = d->paddingHeight > spanH - 1 ? d->paddingHeight : spanH - 1;
+	const int endW = d->paddingWidth > spanW - 1 ? d->paddingWidth : spanW - 1;
+	NH_REQUIRE( d->resultHeight >= 1 && d->resultHeight <= ( d->height + d->paddingHeight + endH - spanH ) / d->strideHeight + 1 );
+	NH_REQUIRE( d->resultWidth >= 1 && d->resultWidth <= ( d->width + d->paddingWidth + endW - spanW ) / d->strideWidth + 1 );
+	const long long m = static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth;
+	NH_REQUIRE( m <= 0x7fffffffLL );
+	NH_REQUIRE( static_cast<long long>( d->batch ) * d->height * d->width * d->channels <= 0x7fffffffLL );
+	NH_REQUIRE( m * d->filterCount <= 0x7fffffffLL );
 	return NH_OK;
 }
 
@@ -2138,12 +2150,10 @@ int nhBlobConvolutionNoAlloc( nhStream s, const nhConvDesc* d, const float* sour
 	const float* freeTerm, float* result )
 {
 	NH_REQUIRE( d != nullptr && source != nullptr && filter != nullptr && result != nullptr );
-	nhConvDesc check = *d;
-	int rc = nhInitBlobConvolution( &check );
+	int rc = checkedConvDesc( d );
 	if( rc != NH_OK ) {
 		return rc;
 	}
-	NH_REQUIRE( check.resultHeight == d->resultHeight && check.resultWidth == d->resultWidth );
 	CSliceMeeting meeting = {};
 	rc = noAllocMeeting( meeting );
 	if( rc != NH_OK ) {
@@ -2169,12 +2179,10 @@ int nhBlobConvolutionWithActivation( nhStream s, const nhConvDesc* d, const floa
 	const float* freeTerm, int activation, float param, float* result )
 {
 	NH_REQUIRE( d != nullptr && source != nullptr && filter != nullptr && result != nullptr );
-	nhConvDesc check = *d;
-	const int rc = nhInitBlobConvolution( &check );
+	const int rc = checkedConvDesc( d );
 	if( rc != NH_OK ) {
 		return rc;
 	}
-	NH_REQUIRE( check.resultHeight == d->resultHeight && check.resultWidth == d->resultWidth );
 	const CFusedActivation act = { activation, param };
 	return convImplicitGemm( toStream( s ), *d, source, filter, freeTerm, result, act );
 }

@@ -519,6 +519,174 @@ void reorgKernel( const int* source, int* result, int stride, int forward, int c
 	}
 }
 
+// ---- poolings over a whole object or over time ------------------------------------------------------------------
+
+// src/CPU/x86/CpuX86MathEngineDnn.cpp:33-140: per ( object, channel ) the maxCount largest of the poolSize values in
+// descending order with their pixel indices; a value that equals a kept one goes in front of it ( the comparison is
+// >= ), slots that stay empty hold -FLT_MAX / -1. One thread per ( object, channel ) keeps its list in the result
+// itself, as the reference does; a value below the smallest kept one is dropped without walking the list.
+__global__ __launch_bounds__( 256 )
+void globalMaxPoolingKernel( const float* source, int* maxIndices, float* result, long long columns, int poolSize, int channels, int maxCount )
+{
+	NH_FOR_EACH( column, columns ) {
+		const long long b = column / channels;
+		const int c = static_cast<int>( column - b * channels );
+		const float* in = source + b * poolSize * channels + c;
+		float* values = result + b * maxCount * channels + c;
+		int* indices = maxIndices + b * maxCount * channels + c;
+		for( int k = 0; k < maxCount; ++k ) {
+			values[static_cast<long long>( k ) * channels] = -FLT_MAX;
+			indices[static_cast<long long>( k ) * channels] = -1;
+		}
+		float smallest = -FLT_MAX;
+		for( int i = 0; i < poolSize; ++i ) {
+			float next = in[static_cast<long long>( i ) * channels];
+			if( !( next >= smallest ) ) {
+				continue;
+			}
+			int nextIndex = i;
+			for( int k = 0; k < maxCount; ++k ) {
+				const long long at = static_cast<long long>( k ) * channels;
+				const float current = values[at];
+				if( next >= current ) {
+					const int currentIndex = indices[at];
+					values[at] = next;
+					indices[at] = nextIndex;
+					next = current;
+					nextIndex = currentIndex;
+				}
+			}
+			smallest = values[static_cast<long long>( maxCount - 1 ) * channels];
+		}
+	}
+}
+
+// src/CPU/CpuMathEngineDnnPooling.cpp:318-350 ( the gradient blob is cleared by the caller )
+__global__ __launch_bounds__( 256 )
+void globalMaxPoolingBackwardKernel( const float* resultDiff, const int* maxIndices, float* sourceDiff, long long total, int poolSize,
+	int channels, int maxCount )
+{
+	NH_FOR_EACH( i, total ) {
+		const int index = maxIndices[i];
+		if( index >= 0 && index < poolSize ) {
+			const long long b = i / ( static_cast<long long>( maxCount ) * channels );
+			const int c = static_cast<int>( i % channels );
+			sourceDiff[( b * poolSize + index ) * channels + c] = resultDiff[i];
+		}
+	}
+}
+
+// src/CPU/x86/CpuX86MathEngineDnn.cpp:336-440: windows of filterLen steps, strideLen apart, over the sequence axis; the
+// first of equal maxima keeps its step
+__global__ __launch_bounds__( 256 )
+void maxOverTimePoolingKernel( const float* source, int* maxIndices, float* result, long long total, int seqElemSize, int filterLen,
+	int strideLen )
+{
+	NH_FOR_EACH( i, total ) {
+		const long long l = i / seqElemSize;
+		const int e = static_cast<int>( i - l * seqElemSize );
+		const long long first = l * strideLen;
+		float best = source[first * seqElemSize + e];
+		int bestStep = static_cast<int>( first );
+		for( int n = 1; n < filterLen; ++n ) {
+			const float v = source[( first + n ) * seqElemSize + e];
+			if( v > best ) {
+				best = v;
+				bestStep = static_cast<int>( first + n );
+			}
+		}
+		result[i] = best;
+		if( maxIndices != nullptr ) {
+			maxIndices[i] = bestStep;
+		}
+	}
+}
+
+// src/CPU/CpuMathEngineDnnPooling.cpp:480-500 ( windows overlap: atomic additions into the cleared gradient ); with
+// assign != 0 the plain store of the global form, :300-316
+__global__ __launch_bounds__( 256 )
+void overTimePoolingBackwardKernel( const float* resultDiff, const int* maxIndices, float* sourceDiff, long long total, int seqElemSize,
+	int assign )
+{
+	NH_FOR_EACH( i, total ) {
+		const int e = static_cast<int>( i % seqElemSize );
+		float* to = sourceDiff + static_cast<long long>( maxIndices[i] ) * seqElemSize + e;
+		if( assign ) {
+			*to = resultDiff[i];
+		} else {
+			atomicAdd( to, resultDiff[i] );
+		}
+	}
+}
+
+// src/CPU/CpuMathEngineDnn.cpp:1016-1110: linear interpolation along the middle axis of [objectCount][scaledAxis][objectSize]
+// coords 0 half pixel, 1 PyTorch half pixel, 2 align corners, 3 asymmetric; round 0 none, 1 half down, 2 half up, 3 floor, 4 ceil
+__global__ __launch_bounds__( 256 )
+void linearInterpolationKernel( const float* data, float* result, long long total, int scaledAxis, int newAxis, int objectSize, float scale,
+	int coords, int round )
+{
+	NH_FOR_EACH( i, total ) {
+		const int k = static_cast<int>( i % objectSize );
+		const long long rest = i / objectSize;
+		const int at = static_cast<int>( rest % newAxis );
+		const long long b = rest / newAxis;
+		float old;
+		if( coords == 3 ) {
+			old = at / scale;
+		} else if( coords == 0 ) {
+			old = ( at + 0.5f ) / scale - 0.5f;
+		} else if( coords == 1 ) {
+			old = newAxis > 1 ? ( at + 0.5f ) / scale - 0.5f : 0.f;
+		} else {
+			old = static_cast<float>( at * ( scaledAxis - 1 ) ) / ( newAxis - 1 );
+		}
+		if( round == 1 ) {
+			old = old == static_cast<int>( old ) + 0.5f ? floorf( old ) : roundf( old );
+		} else if( round == 2 ) {
+			old = roundf( old );
+		} else if( round == 3 ) {
+			old = floorf( old );
+		} else if( round == 4 ) {
+			old = ceilf( old );
+		}
+		const float* in = data + b * scaledAxis * objectSize + k;
+		float value;
+		if( old <= 0.f ) {
+			value = in[0];
+		} else if( old >= static_cast<float>( scaledAxis - 1 ) ) {
+			value = in[static_cast<long long>( scaledAxis - 1 ) * objectSize];
+		} else {
+			const float left = floorf( old );
+			const float rightMul = old - left;
+			const float leftMul = 1.f - rightMul;
+			const long long cell = static_cast<long long>( static_cast<int>( old ) ) * objectSize;
+			// two products, one sum, as the reference's multiply / multiply / add
+			value = __fadd_rn( __fmul_rn( in[cell + objectSize], rightMul ), __fmul_rn( in[cell], leftMul ) );
+		}
+		result[i] = value;
+	}
+}
+
+// :1112-1140: objects of 32-bit values to the places their index tuples name ( the strides of the indexed dimensions
+// arrive precomputed; a repeated target keeps an unspecified one of its updates )
+struct CScatterStrides {
+	int Count;
+	long long Stride[8];
+};
+
+__global__ __launch_bounds__( 256 )
+void scatterNDKernel( const int* updates, const int* indices, int* data, long long total, int objectSize, CScatterStrides strides )
+{
+	NH_FOR_EACH( i, total ) {
+		const long long update = i / objectSize;
+		long long flat = 0;
+		for( int d = 0; d < strides.Count; ++d ) {
+			flat += strides.Stride[d] * indices[update * strides.Count + d];
+		}
+		data[flat + ( i - update * objectSize )] = updates[i];
+	}
+}
+
 } // namespace nh
 
 using namespace nh;
@@ -876,5 +1044,97 @@ extern "C" int nhReorg( nhStream s, const void* source, int stride, int isForwar
 	const long long total = static_cast<long long>( batchSize ) * channels * height * width;
 	NH_REQUIRE( total == 0 || ( source != nullptr && result != nullptr ) );
 	NH_LAUNCH( reorgKernel, total, static_cast<const int*>( source ), static_cast<int*>( result ), stride, isForward, channels, height, width, total );
+	return NH_OK;
+}
+
+extern "C" int nhBlobGlobalMaxPooling( nhStream s, int objectCount, int poolSize, int channels, int maxCount, const float* source, int* maxIndices,
+	float* result )
+{
+	NH_REQUIRE( objectCount >= 0 && poolSize > 0 && channels > 0 && maxCount > 0 );
+	const long long columns = static_cast<long long>( objectCount ) * channels;
+	NH_REQUIRE( columns == 0 || ( source != nullptr && maxIndices != nullptr && result != nullptr ) );
+	NH_LAUNCH( globalMaxPoolingKernel, columns, source, maxIndices, result, columns, poolSize, channels, maxCount );
+	return NH_OK;
+}
+
+extern "C" int nhBlobGlobalMaxPoolingBackward( nhStream s, int objectCount, int poolSize, int channels, int maxCount, const float* resultDiff,
+	const int* maxIndices, float* sourceDiff )
+{
+	NH_REQUIRE( objectCount >= 0 && poolSize > 0 && channels > 0 && maxCount > 0 );
+	const long long sourceTotal = static_cast<long long>( objectCount ) * poolSize * channels;
+	NH_REQUIRE( sourceTotal <= 0x7fffffff );
+	if( sourceTotal == 0 ) {
+		return NH_OK;
+	}
+	NH_REQUIRE( resultDiff != nullptr && maxIndices != nullptr && sourceDiff != nullptr );
+	const int rc = nhVectorFill( s, sourceDiff, 0.f, static_cast<int>( sourceTotal ) );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	const long long total = static_cast<long long>( objectCount ) * maxCount * channels;
+	NH_LAUNCH( globalMaxPoolingBackwardKernel, total, resultDiff, maxIndices, sourceDiff, total, poolSize, channels, maxCount );
+	return NH_OK;
+}
+
+extern "C" int nhBlobMaxOverTimePooling( nhStream s, int sourceLength, int seqElemSize, int filterLen, int strideLen, const float* source,
+	int* maxIndices, float* result )
+{
+	NH_REQUIRE( sourceLength > 0 && seqElemSize >= 0 && filterLen > 0 && strideLen > 0 && filterLen <= sourceLength );
+	const int resultLength = ( sourceLength - filterLen ) / strideLen + 1;
+	const long long total = static_cast<long long>( resultLength ) * seqElemSize;
+	NH_REQUIRE( total == 0 || ( source != nullptr && result != nullptr ) );
+	NH_LAUNCH( maxOverTimePoolingKernel, total, source, maxIndices, result, total, seqElemSize, filterLen, strideLen );
+	return NH_OK;
+}
+
+extern "C" int nhBlobOverTimePoolingBackward( nhStream s, int sourceLength, int resultLength, int seqElemSize, const float* resultDiff,
+	const int* maxIndices, float* sourceDiff, int global )
+{
+	NH_REQUIRE( sourceLength > 0 && resultLength > 0 && seqElemSize >= 0 );
+	const long long sourceTotal = static_cast<long long>( sourceLength ) * seqElemSize;
+	NH_REQUIRE( sourceTotal <= 0x7fffffff );
+	if( sourceTotal == 0 ) {
+		return NH_OK;
+	}
+	NH_REQUIRE( resultDiff != nullptr && maxIndices != nullptr && sourceDiff != nullptr );
+	const int rc = nhVectorFill( s, sourceDiff, 0.f, static_cast<int>( sourceTotal ) );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	const long long total = static_cast<long long>( resultLength ) * seqElemSize;
+	NH_LAUNCH( overTimePoolingBackwardKernel, total, resultDiff, maxIndices, sourceDiff, total, seqElemSize, global );
+	return NH_OK;
+}
+
+extern "C" int nhLinearInterpolation( nhStream s, const float* data, float* result, int coords, int round, int objectCount, int scaledAxis,
+	int objectSize, float scale )
+{
+	NH_REQUIRE( coords >= 0 && coords <= 3 && round >= 0 && round <= 4 && objectCount >= 0 && scaledAxis > 0 && objectSize >= 0 && scale > 0.f );
+	const int newAxis = static_cast<int>( scaledAxis * scale );
+	const long long total = static_cast<long long>( objectCount ) * newAxis * objectSize;
+	NH_REQUIRE( total == 0 || ( data != nullptr && result != nullptr ) );
+	NH_LAUNCH( linearInterpolationKernel, total, data, result, total, scaledAxis, newAxis, objectSize, scale, coords, round );
+	return NH_OK;
+}
+
+extern "C" int nhScatterND( nhStream s, const int* indices, const void* updates, void* data, const nhBlobDesc* dataDesc, int updateCount,
+	int indexDims )
+{
+	NH_REQUIRE( dataDesc != nullptr && updateCount >= 0 && indexDims >= 1 && indexDims <= 7 );
+	long long objectSize = 1;
+	for( int i = indexDims; i < 7; ++i ) {
+		objectSize *= dataDesc->dims[i];
+	}
+	CScatterStrides strides = {};
+	strides.Count = indexDims;
+	strides.Stride[indexDims - 1] = objectSize;
+	for( int i = indexDims - 2; i >= 0; --i ) {
+		strides.Stride[i] = strides.Stride[i + 1] * dataDesc->dims[i + 1];
+	}
+	NH_REQUIRE( objectSize <= 0x7fffffff );
+	const long long total = static_cast<long long>( updateCount ) * objectSize;
+	NH_REQUIRE( total == 0 || ( indices != nullptr && updates != nullptr && data != nullptr ) );
+	NH_LAUNCH( scatterNDKernel, total, static_cast<const int*>( updates ), indices, static_cast<int*>( data ), total, static_cast<int>( objectSize ),
+		strides );
 	return NH_OK;
 }

@@ -3,6 +3,9 @@
 // resolves its handles and calls entry points of the C ABI; semantics are the reference CPU engine's.
 #include "HipMathEngine.h"
 
+#include <algorithm>
+#include <memory>
+
 namespace NeoML {
 
 #define NH_CALL( expr ) check( ( expr ), #expr, __LINE__ )
@@ -583,6 +586,197 @@ void CHipMathEngine::DepthToSpace( const CBlobDesc& source, const CConstIntHandl
 {
 	NH_CALL( nhSpaceToDepth( stream, raw( sourceData ), source.ObjectCount() * source.Height(), source.Width(), result.Channels(), blockSize, 0,
 		raw( resultData ) ) );
+}
+
+// ---- convolution over time: the 2-D convolution with the sequence axis as the height and the batch width as the width
+// ---- ( src/CPU/CpuMathEngineDnnTimeConv.cpp:27-208 ); the padding at the back is implied by the result's length ----
+
+struct CHipTimeConvolutionDesc : public CTimeConvolutionDesc {
+	nhConvDesc D;
+};
+
+CTimeConvolutionDesc* CHipMathEngine::InitTimeConvolution( const CBlobDesc& source, int stride, int paddingFront, int paddingBack,
+	int dilation, const CBlobDesc& filter, const CBlobDesc& result )
+{
+	ASSERT_EXPR( stride > 0 && paddingFront >= 0 && paddingBack >= 0 && dilation > 0 );
+	ASSERT_EXPR( filter.BatchLength() == 1 && filter.Width() == 1 && filter.Depth() == 1 );
+	ASSERT_EXPR( filter.Channels() == source.ObjectSize() );
+	const int span = ( filter.Height() - 1 ) * dilation + 1;
+	ASSERT_EXPR( source.BatchLength() + paddingFront + paddingBack >= span );
+	ASSERT_EXPR( result.BatchLength() == ( source.BatchLength() - span + paddingFront + paddingBack ) / stride + 1 );
+	ASSERT_EXPR( result.BatchWidth() == source.BatchWidth() && result.ListSize() == 1 && source.ListSize() == 1 );
+	ASSERT_EXPR( result.Width() == 1 && result.Height() == 1 && result.Depth() == 1 && result.Channels() == filter.BatchWidth() );
+	ASSERT_EXPR( paddingFront < span && paddingBack < span );
+	std::unique_ptr<CHipTimeConvolutionDesc> desc( new CHipTimeConvolutionDesc() );
+	nhConvDesc& d = desc->D;
+	d.batch = 1;
+	d.height = source.BatchLength();
+	d.width = source.BatchWidth();
+	d.channels = source.ObjectSize();
+	d.filterCount = filter.BatchWidth();
+	d.filterHeight = filter.Height();
+	d.filterWidth = 1;
+	d.paddingHeight = paddingFront;
+	d.paddingWidth = 0;
+	d.strideHeight = stride;
+	d.strideWidth = 1;
+	d.dilationHeight = dilation;
+	d.dilationWidth = 1;
+	d.resultHeight = result.BatchLength();
+	d.resultWidth = source.BatchWidth();
+	return desc.release();
+}
+
+void CHipMathEngine::BlobTimeConvolution( const CTimeConvolutionDesc& desc, const CConstFloatHandle& source, const CConstFloatHandle& filter,
+	const CConstFloatHandle& freeTerm, const CFloatHandle& result )
+{
+	const CHipTimeConvolutionDesc& d = static_cast<const CHipTimeConvolutionDesc&>( desc );
+	NH_CALL( nhBlobConvolution( stream, &d.D, raw( source ), raw( filter ), raw( freeTerm ), raw( result ) ) );
+}
+
+// ( the free term does not enter the input's gradient, :117-166 )
+void CHipMathEngine::BlobTimeConvolutionBackward( const CTimeConvolutionDesc& desc, const CConstFloatHandle& outputDiff,
+	const CConstFloatHandle& filter, const CConstFloatHandle&, const CFloatHandle& inputDiff )
+{
+	const CHipTimeConvolutionDesc& d = static_cast<const CHipTimeConvolutionDesc&>( desc );
+	size_t workspaceSize = 0;
+	NH_CALL( nhBlobConvolutionBackwardWorkspaceSize( &d.D, &workspaceSize ) );
+	const CMemoryHandle workspace = StackAlloc( std::max<size_t>( workspaceSize, 16 ) );
+	NH_CALL( nhBlobConvolutionBackward( stream, &d.D, raw( outputDiff ), raw( filter ), nullptr, raw( inputDiff ), rawBytes( workspace ),
+		workspaceSize ) );
+	StackFree( workspace );
+}
+
+void CHipMathEngine::BlobTimeConvolutionLearnAdd( const CTimeConvolutionDesc& desc, const CConstFloatHandle& input,
+	const CConstFloatHandle& outputDiff, const CFloatHandle& filterDiff, const CFloatHandle& freeTermDiff )
+{
+	const CHipTimeConvolutionDesc& d = static_cast<const CHipTimeConvolutionDesc&>( desc );
+	NH_CALL( nhBlobConvolutionLearnAdd( stream, &d.D, raw( input ), raw( outputDiff ), raw( filterDiff ) ) );
+	SumMatrixRowsAdd( 1, freeTermDiff, outputDiff, d.D.resultHeight * d.D.resultWidth, d.D.filterCount );
+}
+
+// ---- poolings over an object and over time ---------------------------------------------------------------------
+
+struct CHipGlobalMaxPoolingDesc : public CGlobalMaxPoolingDesc {
+	int Objects, PoolSize, Channels, MaxCount;
+};
+
+CGlobalMaxPoolingDesc* CHipMathEngine::InitGlobalMaxPooling( const CBlobDesc& source, const CBlobDesc& maxIndices, const CBlobDesc& result )
+{
+	ASSERT_EXPR( result.ObjectCount() == source.ObjectCount() && result.Channels() == source.Channels() );
+	ASSERT_EXPR( maxIndices.BlobSize() == result.BlobSize() );
+	std::unique_ptr<CHipGlobalMaxPoolingDesc> desc( new CHipGlobalMaxPoolingDesc() );
+	desc->Objects = source.ObjectCount();
+	desc->PoolSize = source.Height() * source.Width() * source.Depth();
+	desc->Channels = source.Channels();
+	desc->MaxCount = result.Height() * result.Width() * result.Depth();
+	return desc.release();
+}
+
+void CHipMathEngine::BlobGlobalMaxPooling( const CGlobalMaxPoolingDesc& desc, const CConstFloatHandle& source, const CIntHandle& maxIndices,
+	const CFloatHandle& result )
+{
+	const CHipGlobalMaxPoolingDesc& d = static_cast<const CHipGlobalMaxPoolingDesc&>( desc );
+	NH_CALL( nhBlobGlobalMaxPooling( stream, d.Objects, d.PoolSize, d.Channels, d.MaxCount, raw( source ), raw( maxIndices ), raw( result ) ) );
+}
+
+void CHipMathEngine::BlobGlobalMaxPoolingBackward( const CGlobalMaxPoolingDesc& desc, const CConstFloatHandle& resultDiff,
+	const CConstIntHandle& maxIndices, const CFloatHandle& sourceDiff )
+{
+	const CHipGlobalMaxPoolingDesc& d = static_cast<const CHipGlobalMaxPoolingDesc&>( desc );
+	NH_CALL( nhBlobGlobalMaxPoolingBackward( stream, d.Objects, d.PoolSize, d.Channels, d.MaxCount, raw( resultDiff ), raw( maxIndices ),
+		raw( sourceDiff ) ) );
+}
+
+struct CHipMaxOverTimePoolingDesc : public CMaxOverTimePoolingDesc {
+	int SourceLength, ResultLength, SeqElemSize, FilterLen, StrideLen;
+};
+
+CMaxOverTimePoolingDesc* CHipMathEngine::InitMaxOverTimePooling( const CBlobDesc& source, int filterLen, int strideLen, const CBlobDesc& result )
+{
+	ASSERT_EXPR( filterLen > 0 && strideLen > 0 && source.BatchLength() >= filterLen );
+	ASSERT_EXPR( result.BatchLength() == ( source.BatchLength() - filterLen ) / strideLen + 1 );
+	ASSERT_EXPR( result.BatchWidth() == source.BatchWidth() && result.ObjectSize() == source.ObjectSize() );
+	std::unique_ptr<CHipMaxOverTimePoolingDesc> desc( new CHipMaxOverTimePoolingDesc() );
+	desc->SourceLength = source.BatchLength();
+	desc->ResultLength = result.BatchLength();
+	desc->SeqElemSize = source.BlobSize() / source.BatchLength();
+	desc->FilterLen = filterLen;
+	desc->StrideLen = strideLen;
+	return desc.release();
+}
+
+void CHipMathEngine::BlobMaxOverTimePooling( const CMaxOverTimePoolingDesc& desc, const CConstFloatHandle& source, const CIntHandle* maxIndices,
+	const CFloatHandle& result )
+{
+	const CHipMaxOverTimePoolingDesc& d = static_cast<const CHipMaxOverTimePoolingDesc&>( desc );
+	NH_CALL( nhBlobMaxOverTimePooling( stream, d.SourceLength, d.SeqElemSize, d.FilterLen, d.StrideLen, raw( source ),
+		maxIndices != nullptr ? raw( *maxIndices ) : nullptr, raw( result ) ) );
+}
+
+void CHipMathEngine::BlobMaxOverTimePoolingBackward( const CMaxOverTimePoolingDesc& desc, const CConstFloatHandle& resultDiff,
+	const CConstIntHandle& maxIndices, const CFloatHandle& sourceDiff )
+{
+	const CHipMaxOverTimePoolingDesc& d = static_cast<const CHipMaxOverTimePoolingDesc&>( desc );
+	NH_CALL( nhBlobOverTimePoolingBackward( stream, d.SourceLength, d.ResultLength, d.SeqElemSize, raw( resultDiff ), raw( maxIndices ),
+		raw( sourceDiff ), 0 ) );
+}
+
+struct CHipGlobalMaxOverTimePoolingDesc : public CGlobalMaxOverTimePoolingDesc {
+	int SourceLength, SeqElemSize;
+};
+
+CGlobalMaxOverTimePoolingDesc* CHipMathEngine::InitGlobalMaxOverTimePooling( const CBlobDesc& source, const CBlobDesc& result )
+{
+	ASSERT_EXPR( result.BatchLength() == 1 && result.BatchWidth() == source.BatchWidth() && result.ObjectSize() == source.ObjectSize() );
+	std::unique_ptr<CHipGlobalMaxOverTimePoolingDesc> desc( new CHipGlobalMaxOverTimePoolingDesc() );
+	desc->SourceLength = source.BatchLength();
+	desc->SeqElemSize = source.BatchWidth() * source.ObjectSize();
+	return desc.release();
+}
+
+// the maximum of every column of [length][batch width x object size], the first of equal maxima keeps its step
+// ( src/CPU/CpuMathEngineDnnPooling.cpp:274-298 )
+void CHipMathEngine::BlobGlobalMaxOverTimePooling( const CGlobalMaxOverTimePoolingDesc& desc, const CConstFloatHandle& source,
+	const CIntHandle* maxIndices, const CFloatHandle& result )
+{
+	const CHipGlobalMaxOverTimePoolingDesc& d = static_cast<const CHipGlobalMaxOverTimePoolingDesc&>( desc );
+	NH_CALL( nhBlobMaxOverTimePooling( stream, d.SourceLength, d.SeqElemSize, d.SourceLength, 1, raw( source ),
+		maxIndices != nullptr ? raw( *maxIndices ) : nullptr, raw( result ) ) );
+}
+
+void CHipMathEngine::BlobGlobalMaxOverTimePoolingBackward( const CGlobalMaxOverTimePoolingDesc& desc, const CConstFloatHandle& resultDiff,
+	const CConstIntHandle& maxIndices, const CFloatHandle& sourceDiff )
+{
+	const CHipGlobalMaxOverTimePoolingDesc& d = static_cast<const CHipGlobalMaxOverTimePoolingDesc&>( desc );
+	NH_CALL( nhBlobOverTimePoolingBackward( stream, d.SourceLength, 1, d.SeqElemSize, raw( resultDiff ), raw( maxIndices ), raw( sourceDiff ), 1 ) );
+}
+
+void CHipMathEngine::LinearInterpolation( const CConstFloatHandle& dataHandle, const CFloatHandle& resultHandle, TInterpolationCoords coords,
+	TInterpolationRound round, int objectCount, int scaledAxis, int objectSize, float scale )
+{
+	NH_CALL( nhLinearInterpolation( stream, raw( dataHandle ), raw( resultHandle ), static_cast<int>( coords ), static_cast<int>( round ),
+		objectCount, scaledAxis, objectSize, scale ) );
+}
+
+void CHipMathEngine::ScatterND( const CConstIntHandle& indicesHandle, const CConstFloatHandle& updatesHandle, const CFloatHandle& dataHandle,
+	const CBlobDesc& dataDesc, int updateCount, int indexDims )
+{
+	nhBlobDesc desc;
+	for( int i = 0; i < 7; ++i ) {
+		desc.dims[i] = dataDesc.DimSize( i );
+	}
+	NH_CALL( nhScatterND( stream, raw( indicesHandle ), raw( updatesHandle ), raw( dataHandle ), &desc, updateCount, indexDims ) );
+}
+
+void CHipMathEngine::ScatterND( const CConstIntHandle& indicesHandle, const CConstIntHandle& updatesHandle, const CIntHandle& dataHandle,
+	const CBlobDesc& dataDesc, int updateCount, int indexDims )
+{
+	nhBlobDesc desc;
+	for( int i = 0; i < 7; ++i ) {
+		desc.dims[i] = dataDesc.DimSize( i );
+	}
+	NH_CALL( nhScatterND( stream, raw( indicesHandle ), raw( updatesHandle ), raw( dataHandle ), &desc, updateCount, indexDims ) );
 }
 
 } // namespace NeoML

@@ -991,6 +991,18 @@ SHIM_API int shim_performance_counters( void* engine, int smallSize, int largeSi
 }
 
 // probe for a method outside the implemented paths (asserts on engines that do not implement it)
+SHIM_API int shim_vector_top_k( void* engine, const float* first, int n, int k, float* result, int* indices )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		CFloatBlob in( e, n, first ), out( e, k );
+		CIntHandleVar found( e, k );
+		e.VectorTopK( in.Const(), n, k, out.Handle(), found.GetHandle() );
+		out.CopyTo( result );
+		e.DataExchangeTyped<int>( indices, found.GetHandle(), k );
+	} );
+}
+
 SHIM_API int shim_vector_power( void* engine, float exponent, const float* first, float* result, int n )
 {
 	return guarded( [&]() {

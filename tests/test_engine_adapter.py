@@ -209,13 +209,25 @@ def test_lstm_through_the_interface(reverse):
 
 
 def test_unimplemented_method_asserts_like_the_reference_gpu_engine():
-    # VectorPower is outside the implemented paths: the generated body raises through NeoML's exception handler,
+    # VectorTopK is outside the implemented paths: the generated body raises through NeoML's exception handler,
     # which the shim turns into an error code instead of letting it cross the C boundary
     s = nhtest.shim()
-    x = np.full(8, 2.0, np.float32)
+    x = np.arange(8, dtype=np.float32)
+    y = np.empty(2, np.float32)
+    idx = np.empty(2, np.int32)
+    ip = idx.ctypes.data_as(ctypes.POINTER(ctypes.c_int))
+    assert s.shim_vector_top_k(nhtest.hip_engine(), nhtest.fp(x), 8, 2, nhtest.fp(y), ip) == 1
+    assert s.shim_vector_top_k(nhtest.cpu_engine(), nhtest.fp(x), 8, 2, nhtest.fp(y), ip) == 0 and y[0] == 7.0 and idx[0] == 7
+
+
+def test_vector_power_on_both_engines():
+    s = nhtest.shim()
+    x = np.linspace(0.5, 3.0, 8).astype(np.float32)
     y = np.empty(8, np.float32)
-    assert s.shim_vector_power(nhtest.hip_engine(), ctypes.c_float(2.0), nhtest.fp(x), nhtest.fp(y), 8) == 1
-    assert s.shim_vector_power(nhtest.cpu_engine(), ctypes.c_float(2.0), nhtest.fp(x), nhtest.fp(y), 8) == 0 and y[0] == 4.0
+    z = np.empty(8, np.float32)
+    assert s.shim_vector_power(nhtest.hip_engine(), ctypes.c_float(2.5), nhtest.fp(x), nhtest.fp(y), 8) == 0
+    assert s.shim_vector_power(nhtest.cpu_engine(), ctypes.c_float(2.5), nhtest.fp(x), nhtest.fp(z), 8) == 0
+    assert_close(y, z, "VectorPower")
 
 
 @pytest.mark.parametrize("with_expand", [True, False])
