@@ -6,7 +6,8 @@
 A step is one forward pass of the ResNet-18-style network (BASELINE.json configs[1]: batch 64, 224x224x3, fp32)
 issued as engine calls through the C ABI of libneoml_hip.so, input already resident in device memory.
 Prints one JSON line: images/sec, the roofline of the dominant kernel (the 3x3 implicit-GEMM convolutions, timed
-live with events on the launch stream) and the reference CPU engine timed on a bounded sample of the same workload.
+live with events on the launch stream) and the reference CPU engine (its MLAS build) timed on the same batch: one thread,
+and one engine per host core with the batch split between them.
 """
 import argparse
 import json
@@ -22,30 +23,81 @@ HBM_PEAK_GBPS = 8000.0
 # Bytes crossing the L2 <-> fabric boundary per 3x3-convolution launch, mean over the 16 launches of one step at
 # batch 64, 224x224: rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a known-size copy gives) 81.0 MB + WRITE_SIZE (x1.0)
 # 43.4 MB; profiles/resnet18_b64_conv_hbm_traffic.txt holds the two runs. Counters cannot be read from inside this
-# process, so the figure is a constant of the default workload and null for any other.
+# process, so the figure is a constant of the default workload (labelled as coming from that profile) and null for any other.
 CONV3X3_TRAFFIC_BYTES_B64_224 = 124.4e6
+CONV3X3_TRAFFIC_SOURCE = "offline_profile: profiles/resnet18_b64_conv_hbm_traffic.txt"
 
 
-def cpu_baseline(batch_sample, image):
-    """The reference's own CPU engine (oracle/_ref, built from its sources) on `batch_sample` images of the same
-    network, one thread. Falls back to the C oracle (kind 'port') when the reference build is absent."""
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    import nhtest
-    from neoml_amd.workloads import ResNet18
-    kind = "ref" if nhtest.have_reference() else "orc"
-    be = nhtest.CpuBackend(kind)
-    net = ResNet18(be, batch=batch_sample, image=image)
-    x = net.make_input()
-    t0 = time.perf_counter()
-    y = net.forward(x)
-    dt = time.perf_counter() - t0
-    return {
-        "value": round(batch_sample / dt, 3), "unit": "images/sec", "cores": 1,
-        "kind": "reference" if kind == "ref" else "port",
-        "sample": "%d images of the same network, 1 pass, %s" % (
-            batch_sample, "reference CCpuMathEngine with its built-in SSE GEMM (no MKL/MLAS)" if kind == "ref" else "C oracle"),
-        "seconds": round(dt, 2),
-    }, y
+def _cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(batch, image, replicas):
+    """The reference's own CPU engine (oracle/_ref, compiled from its sources, with the MLAS GEMM it ships with on Linux) on
+    the same network and the same batch: (1) one engine, one thread, the whole batch; (2) `replicas` engines side by side,
+    one thread and one network each, the batch split between them, started together
+    (NeoML/test/src/InferencePerformanceMultiThreadingTest.cpp:238-262). Every engine runs in a process of its own
+    (oracle/cpu_baseline.py). Returns the JSON object and the arrays of the single-thread pass (softmax, logits)."""
+    import subprocess
+    import tempfile
+    import numpy as np
+    script = os.path.join(ROOT, "oracle", "cpu_baseline.py")
+    mlas = os.path.exists(os.path.join(ROOT, "oracle", "_ref", "mlas", "libengine_shim.so"))
+    common = [sys.executable, script, "--image", str(image)] + (["--mlas"] if mlas else [])
+    with tempfile.TemporaryDirectory() as tmp:
+        saved = os.path.join(tmp, "single.npz")
+        one = json.loads(subprocess.run(common + ["--images", str(batch), "--passes", "2", "--save", saved], check=True, stdout=subprocess.PIPE,
+                                        text=True).stdout.strip().splitlines()[-1])
+        arrays = dict(np.load(saved))
+        # the first images once more on the engine's built-in GEMM (no MLAS), the build the parity tests check against:
+        # how far the reference's own two backends are from each other is the scale for the GPU's distance from either
+        if mlas:
+            first = os.path.join(tmp, "first.npz")
+            n_first = min(4, batch)
+            subprocess.run([sys.executable, script, "--image", str(image), "--images", str(n_first), "--save", first], check=True,
+                           stdout=subprocess.DEVNULL)
+            arrays["logits_builtin_gemm"] = np.load(first)["logits"]
+    base = {
+        "value": round(one["images"] / one["seconds"], 3), "unit": "images/sec", "cores": 1, "kind": one["kind"],
+        "sample": "the whole batch of %d images, mean of 2 passes, 1 thread, %s" % (batch, one["backend"]),
+        "seconds": round(one["seconds"], 2), "cpu": _cpu_model(),
+    }
+    if replicas > 1:
+        share = [batch // replicas + (1 if i < batch % replicas else 0) for i in range(replicas)]
+        share = [n for n in share if n > 0]
+        start_at = time.time() + 6.0  # past every replica's start-up (imports, weights)
+        procs = [subprocess.Popen(common + ["--images", str(n), "--passes", "4", "--start-at", repr(start_at)], stdout=subprocess.PIPE, text=True)
+                 for n in share]
+        done = [json.loads(p.communicate()[0].strip().splitlines()[-1]) for p in procs]
+        slowest = max(d["seconds"] for d in done)
+        base["replicas"] = {
+            "value": round(batch / slowest, 3), "unit": "images/sec", "cores": len(share),
+            "sample": "the same batch split over %d engines (one thread, one network each, %d-%d images), started together, 4 passes each; "
+                      "rate = batch / slowest replica's mean pass" % (len(share), min(share), max(share)),
+            "seconds": round(slowest, 2),
+        }
+    return base, arrays
+
+
+def cdnn_run_once(batch, image):
+    """CDnn::RunOnce (NeoML/src/Dnn/Dnn.cpp:626-658) of the benchmark network on CHipMathEngine, measured by
+    oracle/cdnn_run_once.py; None where the reference's layer library was not built."""
+    import subprocess
+    if not os.path.exists(os.path.join(ROOT, "oracle", "_ref", "libdnn_shim.so")):
+        return None
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "oracle", "cdnn_run_once.py"), "--batch", str(batch), "--image", str(image)],
+                         stdout=subprocess.PIPE, text=True)
+    if res.returncode != 0:
+        return {"error": "oracle/cdnn_run_once.py exited with %d" % res.returncode}
+    fig = json.loads(res.stdout.strip().splitlines()[-1])
+    fig["what"] = "NeoML's CDnn + layer classes (reference sources) on CHipMathEngine, wall time per RunOnce closed by a read-back"
+    return fig
 
 
 def other_workload(args):
@@ -116,7 +168,8 @@ def main():
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--image", type=int, default=224)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample", type=int, default=24, help="images in the CPU baseline sample")
+    ap.add_argument("--cpu-replicas", type=int, default=min(16, os.cpu_count() or 1),
+                    help="engines of the multi-replica CPU baseline (one thread each; 16 = the host cores that go with one GPU)")
     ap.add_argument("--per-kernel", action="store_true", help="print a per-op-family timing table to stderr")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one nhVectorCopy of 2^26 floats (256 MiB read + 256 MiB written): the known-size "
@@ -160,17 +213,22 @@ def main():
         torch.cuda.synchronize()
         settle_steps += 5
 
+    # the throughput figure: the plain replay, nothing but the step's own launches on the stream
     t0 = time.perf_counter()
     for step in range(args.steps):
-        plan.run_with_events(pools[step])
+        plan.run()
     host_done = time.perf_counter()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    # the roofline figure: the same steps again with an event pair around every 3x3 convolution (on the launch stream)
+    for step in range(args.steps):
+        plan.run_with_events(pools[step])
+    torch.cuda.synchronize()
 
     ms_per_step = elapsed / args.steps * 1e3
     images_per_sec = args.batch * args.steps / elapsed
 
-    # per-family totals from the events recorded inside the timed region (on the launch stream)
+    # per-family totals from the events of the second pass
     fam = plan.family_totals()
     c3 = fam.get("conv3x3", [0, 1e-9, 0, 0])
     launches, ms, flops, nbytes = c3
@@ -181,6 +239,7 @@ def main():
         "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
         "traffic": CONV3X3_TRAFFIC_BYTES_B64_224 if (args.batch, args.image) == (64, 224) else None,
         "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE, rocprofv3 --pmc, scaled by a known-size copy)",
+        "traffic_source": CONV3X3_TRAFFIC_SOURCE if (args.batch, args.image) == (64, 224) else None,
         "algorithmic_bytes_per_launch": nbytes // max(launches, 1),
         "avg_launch_us": round(ms * 1e3 / max(launches, 1), 2),
         "flop_per_step": flops // max(args.steps, 1),
@@ -226,13 +285,32 @@ def main():
                                      "steps": steps, "max_abs_diff_vs_plain": float((opt_out - out).abs().max().item())}
 
     if not args.no_cpu_baseline:
-        base, y_cpu = cpu_baseline(args.cpu_sample, args.image)
-        result["cpu_baseline"] = base
-        # the same images through the GPU path: parity of the whole network on the sample
         import numpy as np
-        small = ResNet18(HipBackend(), batch=args.cpu_sample, image=args.image)
-        y_gpu = small.be.to_numpy(small.forward(small.be.tensor(small.make_input())))
-        result["parity_max_abs_diff_vs_cpu"] = float(np.max(np.abs(y_gpu - y_cpu)))
+        base, cpu = cpu_baseline(args.batch, args.image, args.cpu_replicas)
+        result["cpu_baseline"] = base
+        # parity of the whole network on the whole batch, against the CPU engine's single-thread pass: the softmax output
+        # and the logits in front of it (1000 probabilities of ~1e-3 pass an absolute bar easily, the logits do not)
+        y_gpu = be.to_numpy(out)
+        logits_gpu = be.to_numpy(net.buffers["fc"])
+        logits_cpu = cpu["logits"].reshape(logits_gpu.shape)
+
+        def distance(a, b):
+            d = np.abs(a - b)
+            return {"max_abs_diff": float(d.max()), "max_abs_value": float(np.abs(b).max()),
+                    "worst_fraction_of_bar": round(float((d / (1e-5 + 1e-4 * np.abs(b))).max()), 3), "images": int(a.shape[0])}
+
+        result["parity_max_abs_diff_vs_cpu"] = float(np.max(np.abs(y_gpu - cpu["softmax"].reshape(y_gpu.shape))))
+        result["parity_logits_vs_cpu"] = dict(distance(logits_gpu, logits_cpu), bar="|a - b| <= 1e-5 + 1e-4 |b| per element")
+        if "logits_builtin_gemm" in cpu:
+            # logits near zero are sums of 512 products that cancel: their absolute error follows the size of the products,
+            # not of the sum, so the per-element bar is a strict one here; the reference's two GEMM backends show the scale
+            builtin = cpu["logits_builtin_gemm"].reshape(-1, logits_gpu.shape[1])
+            n = builtin.shape[0]
+            result["parity_logits_vs_cpu"]["vs_builtin_gemm_engine"] = distance(logits_gpu[:n], builtin)
+            result["parity_logits_vs_cpu"]["reference_mlas_vs_builtin_gemm"] = distance(logits_cpu[:n], builtin)
+        # the same network as an application of the reference runs it: NeoML's own CDnn and layer classes (compiled from the
+        # reference's sources) calling the HIP engine through IMathEngine, timed per CDnn::RunOnce in a process of its own
+        result["cdnn_run_once"] = cdnn_run_once(args.batch, args.image)
     print(json.dumps(result))
 
 

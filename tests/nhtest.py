@@ -11,7 +11,8 @@ import numpy as np
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 ORACLE_LIB = os.path.join(ORACLE_DIR, "liboracle.so")
-SHIM_LIB = os.path.join(ORACLE_DIR, "_ref", "libengine_shim.so")
+# NHTEST_SHIM_LIB: another build of the shim + reference engine (the MLAS-backed one of the benchmark's CPU baseline)
+SHIM_LIB = os.environ.get("NHTEST_SHIM_LIB") or os.path.join(ORACLE_DIR, "_ref", "libengine_shim.so")
 
 # tolerance of the parity bar: |a - b| <= ATOL + RTOL * |b|
 RTOL = 1e-4
