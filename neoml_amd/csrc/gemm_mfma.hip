@@ -33,6 +33,7 @@
 #include <math.h>
 #include <map>
 #include <mutex>
+#include <type_traits>
 #include <utility>
 #include <vector>
 
@@ -1392,16 +1393,53 @@ __device__ __forceinline__ float hSwishOf( float v )
 	return v <= -3.f ? 0.f : ( v >= 3.f ? v : mid );
 }
 
+//
+// The same kernel is the first layer of an image network ( RP > 0 ): a convolution over an image with one or three
+// channels, whose reduction is short ( 3 x 3 x 3 = 27, 7 x 7 x 3 = 147 ) and whose result is many times larger than its
+// input. A row of A is then the window of one output pixel: Fh runs of RowK = Fw * Cin consecutive floats of a
+// channels-last image, laid out as Fh rows of RP = RowK rounded up to a multiple of 4 ( k = r * RP + j ). A lane's 16
+// bytes of chunk c are four consecutive j of one filter row r, both known at compile time per half-wavefront, fetched
+// with one 128-bit load at 4-byte alignment. What such a load brings along beyond the run ( j >= RowK: the next
+// pixels ), before the image row's first element ( padding on the left: the row above ) or behind its last one is
+// replaced by zeros when the registers are first used; filter rows above and below the image get an out-of-range offset;
+// the descriptor ends with the image blob, and a 128-bit load is range-checked per component, so nothing is read
+// beyond it. Offsets cannot be negative: the few pixels of the first image whose window begins in front of the blob
+// ( top left corner, padding on the left ) lie in the first row blocks, which are the ones the prologue fetches, and
+// those it fetches element by element.
+struct CRowRuns {
+	int H, W, Cin, Ho, Wo, Fh, RowK;
+	int PadH, PadW, StrideH, StrideW;
+	unsigned ABytes; // size of the image blob
+	int SlowRows; // output pixels below this index: fetched element by element ( all of them in prologue blocks )
+};
+
+// where a lane's output pixel sits in the image
+struct CRunState {
+	int PixBytes; // byte offset of filter row 0, j = 0 ( negative where that lies in front of the blob )
+	int Hi0; // image row of filter row 0
+	int Lb, Span; // j is inside the image row and the run for Lb <= j < Lb + Span
+};
+
 // ( W is the MFMA's first operand and A its second: the 32 x 32 block comes out transposed, lane ( l32, half ) holding
 // row l32 and, in registers 4g..4g+3, its columns 8g + 4 half .. + 3. The accumulator starts as the bias of those columns. )
-template<int KC, int NB, bool RES>
+template<int KC, int NB, bool RES, int RP>
 __global__ __launch_bounds__( Threads, 2 )
 void shortReductionKernel( const float* A, const float* W, const float* bias, float* C, int M, int N, int rowBlocks,
-	const CFusedActivation act, const float* residual )
+	const CFusedActivation act, const float* residual, const CRowRuns geo )
 {
 	constexpr int K = KC * 8;
 	constexpr int Pitch = K + 4;
 	constexpr int PatchPitch = 36;
+	constexpr int RP_OR_ONE = RP > 0 ? RP : 1;
+	constexpr int KR = RP > 0 ? ( K + RP - 1 ) / RP : 1; // filter rows that K spans ( those beyond Fh only round K up )
+	// Column blocks worked on together, each with its own accumulator. The window loader's long reductions are bound by
+	// the matrix pipe, and the two wavefronts per SIMD that registers and LDS leave room for keep it only half busy with
+	// one chain of dependent MFMAs each; two independent chains per wavefront do what four wavefronts would.
+	constexpr int Together = ( RP > 0 && NB % 2 == 0 ) ? 2 : 1;
+	static_assert( !RES || Together == 1, "the residual is requested one column block ahead" );
+	// ... and the chunks of a long reduction alternate between two chains per column block, added up at the end
+	// ( measured: no gain on any shape once two column blocks run together; kept for single column blocks of the window loader )
+	constexpr int Chains = ( RP > 0 && Together == 1 ) ? 2 : 1;
 	// [32 * NB][Pitch], rows beyond N are zero; the bias, [32 * NB]; then one [32][36] output patch per wavefront
 	extern __shared__ __attribute__( ( aligned( 16 ) ) ) float wLds[];
 	const int tid = threadIdx.x;
@@ -1412,7 +1450,8 @@ void shortReductionKernel( const float* A, const float* W, const float* bias, fl
 
 	float* biasLds = wLds + NB * 32 * Pitch;
 	float* patch = biasLds + NB * 32 + wave * 32 * PatchPitch;
-	const __amdgpu_buffer_rsrc_t bufA = makeBuffer( A );
+	const __amdgpu_buffer_rsrc_t bufA = RP > 0 ? __builtin_amdgcn_make_buffer_rsrc( const_cast<float*>( A ), 0, geo.ABytes, 0x00020000 )
+		: makeBuffer( A );
 	// C and the residual end where the matrix ends: rows beyond M are out of range by themselves
 	const unsigned cBytes = static_cast<unsigned>( M ) * static_cast<unsigned>( N ) * 4u;
 	const __amdgpu_buffer_rsrc_t bufC = __builtin_amdgcn_make_buffer_rsrc( C, 0, cBytes, 0x00020000 );
@@ -1433,12 +1472,76 @@ void shortReductionKernel( const float* A, const float* W, const float* bias, fl
 		return nb * 32 + col4 < N ? static_cast<unsigned>( block ) * 32u * rowBytes + nb * 128u + laneOut : OutOfRange;
 	};
 
-	for( int idx = tid; idx < NB * 32 * ( K / 4 ); idx += Threads ) {
-		const int n = idx / ( K / 4 );
-		const int k4 = idx - n * ( K / 4 );
-		const float4 v = n < N ? *reinterpret_cast<const float4*>( W + static_cast<long long>( n ) * K + k4 * 4 )
-			: make_float4( 0.f, 0.f, 0.f, 0.f );
-		*reinterpret_cast<float4*>( wLds + n * Pitch + k4 * 4 ) = v;
+	// the pixel of this lane in row block `block` ( RP > 0 )
+	const int rowBytesIn = RP > 0 ? geo.W * geo.Cin * 4 : 0;
+	auto locate = [&]( int block ) -> CRunState {
+		CRunState s = { 0, -0x40000000, 0, 0 }; // no filter row meets the image: every chunk out of range
+		const int m = block * 32 + l32;
+		if( block < rowBlocks && m < M ) {
+			const int wo = m % geo.Wo;
+			const int t = m / geo.Wo;
+			const int ho = t % geo.Ho;
+			const int n = t / geo.Ho;
+			const int wc0 = ( wo * geo.StrideW - geo.PadW ) * geo.Cin;
+			s.Hi0 = ho * geo.StrideH - geo.PadH;
+			s.PixBytes = ( n * geo.H + s.Hi0 ) * rowBytesIn + wc0 * 4;
+			s.Lb = wc0 < 0 ? -wc0 : 0;
+			const int inRow = geo.W * geo.Cin - wc0;
+			const int ub = geo.RowK < inRow ? geo.RowK : inRow;
+			s.Span = ub > s.Lb ? ub - s.Lb : 0;
+		}
+		return s;
+	};
+	// filter row and position in it of this lane's piece of chunk c
+	auto chunkRow = [&]( int c ) -> int { return half != 0 ? ( 8 * c + 4 ) / RP_OR_ONE : ( 8 * c ) / RP_OR_ONE; };
+	auto chunkPos = [&]( int c ) -> int { return half != 0 ? ( 8 * c + 4 ) % RP_OR_ONE : ( 8 * c ) % RP_OR_ONE; };
+	auto chunkOffset = [&]( const CRunState& s, int c ) -> unsigned {
+		const int r = chunkRow( c );
+		const bool meets = static_cast<unsigned>( s.Hi0 + r ) < static_cast<unsigned>( geo.H ) && r < geo.Fh;
+		return meets ? static_cast<unsigned>( s.PixBytes + r * rowBytesIn + chunkPos( c ) * 4 ) : OutOfRange;
+	};
+	// zeros behind the run's end, for lanes whose window lies inside the image row ( j < RowK is all that can fail, and
+	// only in the last positions of a filter row )
+	auto maskRunEnd = [&]( int c, float4 v ) -> float4 {
+		const int j0 = ( 8 * c ) % RP_OR_ONE;
+		const int j1 = ( 8 * c + 4 ) % RP_OR_ONE;
+		if( j0 + 3 >= RP_OR_ONE - 3 || j1 + 3 >= RP_OR_ONE - 3 ) {
+			const int j = half != 0 ? j1 : j0;
+			v.x = j < geo.RowK ? v.x : 0.f;
+			v.y = j + 1 < geo.RowK ? v.y : 0.f;
+			v.z = j + 2 < geo.RowK ? v.z : 0.f;
+			v.w = j + 3 < geo.RowK ? v.w : 0.f;
+		}
+		return v;
+	};
+	auto maskChunk = [&]( const CRunState& s, int c, float4 v ) -> float4 {
+		const unsigned t = static_cast<unsigned>( chunkPos( c ) - s.Lb );
+		const unsigned span = static_cast<unsigned>( s.Span );
+		v.x = t < span ? v.x : 0.f;
+		v.y = t + 1u < span ? v.y : 0.f;
+		v.z = t + 2u < span ? v.z : 0.f;
+		v.w = t + 3u < span ? v.w : 0.f;
+		return v;
+	};
+
+	if( RP > 0 ) {
+		// the filter [N][Fh][RowK] into rows of Fh x RP ( + what rounds K up ), zeros in the padding
+#pragma unroll 8
+		for( int idx = tid; idx < NB * 32 * K; idx += Threads ) {
+			const int n = idx / K;
+			const int k = idx - n * K;
+			const int r = k / RP_OR_ONE;
+			const int j = k - r * RP_OR_ONE;
+			wLds[n * Pitch + k] = ( n < N && r < geo.Fh && j < geo.RowK ) ? W[( static_cast<long long>( n ) * geo.Fh + r ) * geo.RowK + j] : 0.f;
+		}
+	} else {
+		for( int idx = tid; idx < NB * 32 * ( K / 4 ); idx += Threads ) {
+			const int n = idx / ( K / 4 );
+			const int k4 = idx - n * ( K / 4 );
+			const float4 v = n < N ? *reinterpret_cast<const float4*>( W + static_cast<long long>( n ) * K + k4 * 4 )
+				: make_float4( 0.f, 0.f, 0.f, 0.f );
+			*reinterpret_cast<float4*>( wLds + n * Pitch + k4 * 4 ) = v;
+		}
 	}
 	for( int n = tid; n < NB * 32; n += Threads ) {
 		biasLds[n] = ( bias != nullptr && n < N ) ? bias[n] : 0.f;
@@ -1447,7 +1550,33 @@ void shortReductionKernel( const float* A, const float* W, const float* bias, fl
 
 	int block = blockIdx.x * 4 + wave;
 	float4 a[KC];
-	{
+	CRunState cur = { 0, 0, 0, 0 };
+	if( RP > 0 ) {
+		cur = locate( block );
+		if( block * 32 < geo.SlowRows ) {
+			// a block with pixels whose window begins in front of the blob: element by element, nothing out of bounds
+			const long long pixFloats = cur.PixBytes / 4; // ( exact: a multiple of 4, also when negative )
+#pragma unroll
+			for( int c = 0; c < KC; ++c ) {
+				const int r = chunkRow( c );
+				const int j0 = chunkPos( c );
+				const bool meets = static_cast<unsigned>( cur.Hi0 + r ) < static_cast<unsigned>( geo.H ) && r < geo.Fh;
+				const float* from = A + ( pixFloats + static_cast<long long>( r ) * ( rowBytesIn / 4 ) + j0 );
+				float e[4];
+#pragma unroll
+				for( int i = 0; i < 4; ++i ) {
+					const bool inside = meets && static_cast<unsigned>( j0 + i - cur.Lb ) < static_cast<unsigned>( cur.Span );
+					e[i] = inside ? from[i] : 0.f;
+				}
+				a[c] = make_float4( e[0], e[1], e[2], e[3] );
+			}
+		} else {
+#pragma unroll
+			for( int c = 0; c < KC; ++c ) {
+				a[c] = bufferLoad4( bufA, chunkOffset( cur, c ) );
+			}
+		}
+	} else {
 		const unsigned first = rowOffset( block );
 #pragma unroll
 		for( int c = 0; c < KC; ++c ) {
@@ -1464,95 +1593,190 @@ void shortReductionKernel( const float* A, const float* W, const float* bias, fl
 				res[q] = bufferLoad4( bufR, o + q * 8u * rowBytes );
 			}
 		}
-		// Four stores that go nowhere: the loop is entered with the same sequence of outstanding operations that its
+		// Stores that go nowhere, as many as a pass over the last column blocks issues: the loop is entered with the same sequence of outstanding operations that its
 		// own last column block leaves behind, so the compiler's wait counts for the first MFMAs skip the stores.
 #pragma unroll
-		for( int q = 0; q < 4; ++q ) {
+		for( int q = 0; q < 4 * Together; ++q ) {
 			bufferStore4( bufC, OutOfRange + q * 16u, make_float4( 0.f, 0.f, 0.f, 0.f ) );
 		}
 	}
 	for( ; block < rowBlocks; block += stride ) {
-		const unsigned nextRows = rowOffset( block + stride );
+		const unsigned nextRows = RP > 0 ? 0u : rowOffset( block + stride );
+		// RP > 0: what the loads for the next row block need, per filter row: its byte offset at j = 0, out of range
+		// where the row lies above or below the image
+		CRunState next = { 0, 0, 0, 0 };
+		unsigned nextRow[KR];
+		if( RP > 0 ) {
+			next = locate( block + stride );
 #pragma unroll
-		for( int nb = 0; nb < NB; ++nb ) {
-			const bool lastColumns = nb == NB - 1; // known when the loop is unrolled
-			f32x16 acc;
-			{
-				const float* b = biasLds + nb * 32 + half * 4;
+			for( int r = 0; r < KR; ++r ) {
+				const bool meets = static_cast<unsigned>( next.Hi0 + r ) < static_cast<unsigned>( geo.H ) && r < geo.Fh;
+				nextRow[r] = meets ? static_cast<unsigned>( next.PixBytes + r * rowBytesIn ) : OutOfRange;
+			}
+		}
+		// every lane's window inside its image row ( wave-uniform ): only the run's end needs zeros then
+		// ( the other wavefronts, those with a pixel at the left or right border or behind the last one, first put zeros
+		// wherever a lane's bounds ask for them; the registers are changed in place, under a branch without MFMAs )
+		const bool plain = RP > 0 && __builtin_amdgcn_ballot_w64( cur.Lb != 0 || cur.Span != geo.RowK ) == 0;
+		if( RP > 0 && !plain ) {
+#pragma unroll
+			for( int c = 0; c < KC; ++c ) {
+				a[c] = maskChunk( cur, c, a[c] );
+			}
+		}
+#pragma unroll
+		for( int nb = 0; nb < NB; nb += Together ) {
+			const bool lastColumns = nb + Together >= NB; // known when the loop is unrolled
+			f32x16 accs[Together * Chains];
+#pragma unroll
+			for( int t = 0; t < Together; ++t ) {
+				const float* b = biasLds + ( nb + t ) * 32 + half * 4;
 #pragma unroll
 				for( int g = 0; g < 4; ++g ) {
 					const float4 v = *reinterpret_cast<const float4*>( b + g * 8 );
-					acc[g * 4] = v.x;
-					acc[g * 4 + 1] = v.y;
-					acc[g * 4 + 2] = v.z;
-					acc[g * 4 + 3] = v.w;
+					accs[t][g * 4] = v.x;
+					accs[t][g * 4 + 1] = v.y;
+					accs[t][g * 4 + 2] = v.z;
+					accs[t][g * 4 + 3] = v.w;
+				}
+				if constexpr( Chains > 1 ) {
+#pragma unroll
+					for( int i = 0; i < 16; ++i ) {
+						accs[Together + t][i] = 0.f;
+					}
 				}
 			}
 			const float* wRow = wLds + ( nb * 32 + l32 ) * Pitch + half * 4;
-#pragma unroll
-			for( int c = 0; c < KC; ++c ) {
-				const float4 w = *reinterpret_cast<const float4*>( wRow + c * 8 );
-				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( w.x, a[c].x, acc, 0, 0, 0 );
-				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( w.y, a[c].y, acc, 0, 0, 0 );
-				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( w.z, a[c].z, acc, 0, 0, 0 );
-				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( w.w, a[c].w, acc, 0, 0, 0 );
-				if( lastColumns ) {
-					a[c] = bufferLoad4( bufA, nextRows + c * 32u );
-				}
-			}
-			// the residual of the column block that follows ( of the next row block behind the last one )
 			float4 resNext[4];
-			if( RES ) {
-				const unsigned o = lastColumns ? outOffset( block + stride, 0 ) : outOffset( block, nb + 1 );
+			float* mine = patch + l32 * PatchPitch + half * 4;
+			// The MFMAs of the column blocks, and the first block's move to the LDS patch: nothing else stands between the
+			// MFMAs and the first use of their result, in one basic block. Masks: 0 none, 1 the run's end.
+			auto pass = [&]( auto masks ) {
+				constexpr int Masks = decltype( masks )::value;
 #pragma unroll
-				for( int q = 0; q < 4; ++q ) {
-					resNext[q] = bufferLoad4( bufR, o + q * 8u * rowBytes );
+				for( int c = 0; c < KC; ++c ) {
+					float4 w[Together];
+#pragma unroll
+					for( int t = 0; t < Together; ++t ) {
+						w[t] = *reinterpret_cast<const float4*>( wRow + t * 32 * Pitch + c * 8 );
+					}
+					if( Masks == 1 ) {
+						a[c] = maskRunEnd( c, a[c] ); // first use of what the loads brought
+					}
+					// ( the later column block first: its chain is the older one when the blocks go out in ascending order )
+#pragma unroll
+					for( int t = Together - 1; t >= 0; --t ) {
+						f32x16& chain = accs[( c % Chains ) * Together + t];
+						chain = __builtin_amdgcn_mfma_f32_32x32x2f32( w[t].x, a[c].x, chain, 0, 0, 0 );
+					}
+#pragma unroll
+					for( int t = Together - 1; t >= 0; --t ) {
+						f32x16& chain = accs[( c % Chains ) * Together + t];
+						chain = __builtin_amdgcn_mfma_f32_32x32x2f32( w[t].y, a[c].y, chain, 0, 0, 0 );
+					}
+#pragma unroll
+					for( int t = Together - 1; t >= 0; --t ) {
+						f32x16& chain = accs[( c % Chains ) * Together + t];
+						chain = __builtin_amdgcn_mfma_f32_32x32x2f32( w[t].z, a[c].z, chain, 0, 0, 0 );
+					}
+#pragma unroll
+					for( int t = Together - 1; t >= 0; --t ) {
+						f32x16& chain = accs[( c % Chains ) * Together + t];
+						chain = __builtin_amdgcn_mfma_f32_32x32x2f32( w[t].w, a[c].w, chain, 0, 0, 0 );
+					}
+					if( lastColumns ) {
+						if( RP > 0 ) {
+							const unsigned o0 = nextRow[( 8 * c ) / RP_OR_ONE] + ( ( 8 * c ) % RP_OR_ONE ) * 4u;
+							const unsigned o1 = nextRow[( 8 * c + 4 ) / RP_OR_ONE] + ( ( 8 * c + 4 ) % RP_OR_ONE ) * 4u;
+							a[c] = bufferLoad4( bufA, half != 0 ? o1 : o0 );
+							// ( left to itself the scheduler gathers these loads behind the last MFMA, and the next row
+							// block begins by waiting for them )
+							__builtin_amdgcn_sched_barrier( 0 );
+						} else {
+							a[c] = bufferLoad4( bufA, nextRows + c * 32u );
+						}
+					}
 				}
+				// the residual of the column block that follows ( of the next row block behind the last one )
+				if( RES ) {
+					const unsigned o = lastColumns ? outOffset( block + stride, 0 ) : outOffset( block, nb + 1 );
+#pragma unroll
+					for( int q = 0; q < 4; ++q ) {
+						resNext[q] = bufferLoad4( bufR, o + q * 8u * rowBytes );
+					}
+				}
+				f32x16 acc = accs[0];
+				if constexpr( Chains > 1 ) {
+#pragma unroll
+					for( int i = 0; i < 16; ++i ) {
+						acc[i] += accs[Together][i];
+					}
+				}
+#pragma unroll
+				for( int g = 0; g < 4; ++g ) {
+					*reinterpret_cast<float4*>( mine + g * 8 ) = make_float4( acc[g * 4], acc[g * 4 + 1], acc[g * 4 + 2], acc[g * 4 + 3] );
+				}
+			};
+			if( RP > 0 && nb == 0 ) {
+				pass( std::integral_constant<int, 1>() );
+			} else {
+				pass( std::integral_constant<int, 0>() );
 			}
 			// The block goes out through a wavefront-private patch of LDS in which the lanes regroup: a lane then holds
 			// four neighbouring columns of a row such that one store instruction covers whole 128-byte runs of 8 rows
-			// ( stored as they come out of the MFMA, an instruction would touch 32 rows with 32 bytes each ).
-			// Nothing but the move to the patch stands between the MFMAs and the first use of their result, in one
-			// basic block: the activation, with its branches on the type, is applied to what comes back from the patch.
-			float* mine = patch + l32 * PatchPitch + half * 4;
+			// ( stored as they come out of the MFMA, an instruction would touch 32 rows with 32 bytes each ). The
+			// activation, with its branches on the type, is applied to what comes back from the patch.
 #pragma unroll
-			for( int g = 0; g < 4; ++g ) {
-				*reinterpret_cast<float4*>( mine + g * 8 ) = make_float4( acc[g * 4], acc[g * 4 + 1], acc[g * 4 + 2], acc[g * 4 + 3] );
-			}
-			// ( same wavefront: the LDS unit executes its reads after its writes, no barrier needed )
-			float4 v[4];
+			for( int t = 0; t < Together; ++t ) {
+				if( t > 0 ) {
+					// ( a later block of the group: its MFMAs were issued before the first block's last ones )
+					f32x16 acc = accs[t];
+					if constexpr( Chains > 1 ) {
 #pragma unroll
-			for( int q = 0; q < 4; ++q ) {
-				v[q] = *reinterpret_cast<const float4*>( patch + ( q * 8 + ( lane >> 3 ) ) * PatchPitch + col4 );
-			}
-			if( act.Type == NH_ACT_RELU ) {
+						for( int i = 0; i < 16; ++i ) {
+							acc[i] += accs[Together + t][i];
+						}
+					}
+#pragma unroll
+					for( int g = 0; g < 4; ++g ) {
+						*reinterpret_cast<float4*>( mine + g * 8 ) = make_float4( acc[g * 4], acc[g * 4 + 1], acc[g * 4 + 2], acc[g * 4 + 3] );
+					}
+				}
+				// ( same wavefront: the LDS unit executes its reads after its writes, no barrier needed )
+				float4 v[4];
 #pragma unroll
 				for( int q = 0; q < 4; ++q ) {
-					// NaN becomes 0, as in VectorReLU: the maximum of a NaN and a number is the number
-					v[q].x = __builtin_fminf( __builtin_fmaxf( v[q].x, 0.f ), reluTop );
-					v[q].y = __builtin_fminf( __builtin_fmaxf( v[q].y, 0.f ), reluTop );
-					v[q].z = __builtin_fminf( __builtin_fmaxf( v[q].z, 0.f ), reluTop );
-					v[q].w = __builtin_fminf( __builtin_fmaxf( v[q].w, 0.f ), reluTop );
+					v[q] = *reinterpret_cast<const float4*>( patch + ( q * 8 + ( lane >> 3 ) ) * PatchPitch + col4 );
 				}
-			} else if( act.Type == NH_ACT_HSWISH ) {
+				if( act.Type == NH_ACT_RELU ) {
+#pragma unroll
+					for( int q = 0; q < 4; ++q ) {
+						// NaN becomes 0, as in VectorReLU: the maximum of a NaN and a number is the number
+						v[q].x = __builtin_fminf( __builtin_fmaxf( v[q].x, 0.f ), reluTop );
+						v[q].y = __builtin_fminf( __builtin_fmaxf( v[q].y, 0.f ), reluTop );
+						v[q].z = __builtin_fminf( __builtin_fmaxf( v[q].z, 0.f ), reluTop );
+						v[q].w = __builtin_fminf( __builtin_fmaxf( v[q].w, 0.f ), reluTop );
+					}
+				} else if( act.Type == NH_ACT_HSWISH ) {
+#pragma unroll
+					for( int q = 0; q < 4; ++q ) {
+						v[q].x = hSwishOf( v[q].x );
+						v[q].y = hSwishOf( v[q].y );
+						v[q].z = hSwishOf( v[q].z );
+						v[q].w = hSwishOf( v[q].w );
+					}
+				}
+				const unsigned o = outOffset( block, nb + t );
 #pragma unroll
 				for( int q = 0; q < 4; ++q ) {
-					v[q].x = hSwishOf( v[q].x );
-					v[q].y = hSwishOf( v[q].y );
-					v[q].z = hSwishOf( v[q].z );
-					v[q].w = hSwishOf( v[q].w );
+					if( RES ) {
+						v[q].x += res[q].x;
+						v[q].y += res[q].y;
+						v[q].z += res[q].z;
+						v[q].w += res[q].w;
+					}
+					bufferStore4( bufC, o + q * 8u * rowBytes, v[q] );
 				}
-			}
-			const unsigned o = outOffset( block, nb );
-#pragma unroll
-			for( int q = 0; q < 4; ++q ) {
-				if( RES ) {
-					v[q].x += res[q].x;
-					v[q].y += res[q].y;
-					v[q].z += res[q].z;
-					v[q].w += res[q].w;
-				}
-				bufferStore4( bufC, o + q * 8u * rowBytes, v[q] );
 			}
 			if( RES ) {
 #pragma unroll
@@ -1561,6 +1785,7 @@ void shortReductionKernel( const float* A, const float* W, const float* bias, fl
 				}
 			}
 		}
+		cur = next;
 	}
 }
 
@@ -1569,9 +1794,10 @@ static constexpr size_t shortReductionLds( int K, int nb )
 	return ( static_cast<size_t>( nb ) * 32 * ( K + 4 ) + nb * 32 + 4 * 32 * 36 ) * sizeof( float );
 }
 
-template<int KC, int NB, bool RES>
-static void launchShortReduction( hipStream_t stream, const float* a, const float* w, const float* bias, float* c, int M, int N,
-	const CFusedActivation& act, const float* residual )
+// ( false, and nothing launched: a window loader whose element-wise blocks would not all be first blocks )
+template<int KC, int NB, bool RES, int RP = 0>
+static bool launchShortReduction( hipStream_t stream, const float* a, const float* w, const float* bias, float* c, int M, int N,
+	const CFusedActivation& act, const float* residual, const CRowRuns& geo = CRowRuns() )
 {
 	const int rowBlocks = ceilDiv( M, 32 );
 	const int groups = ceilDiv( rowBlocks, 4 );
@@ -1591,7 +1817,7 @@ static void launchShortReduction( hipStream_t stream, const float* a, const floa
 		int& known = residentFor[device];
 		if( known == 0 ) {
 			int perUnit = 0, units = 0;
-			if( hipOccupancyMaxActiveBlocksPerMultiprocessor( &perUnit, shortReductionKernel<KC, NB, RES>, Threads, lds ) != hipSuccess
+			if( hipOccupancyMaxActiveBlocksPerMultiprocessor( &perUnit, shortReductionKernel<KC, NB, RES, RP>, Threads, lds ) != hipSuccess
 				|| hipDeviceGetAttribute( &units, hipDeviceAttributeMultiprocessorCount, device ) != hipSuccess
 				|| perUnit <= 0 || units <= 0 )
 			{
@@ -1603,11 +1829,16 @@ static void launchShortReduction( hipStream_t stream, const float* a, const floa
 		}
 		resident = known;
 	}
-	if( NB > 1 ) {
-		resident *= 4;
+	if( NB > 1 && RP == 0 ) {
+		resident *= 4; // ( the window loader's reductions are long enough to be bound by the matrix pipe: one round )
 	}
-	hipLaunchKernelGGL( ( shortReductionKernel<KC, NB, RES> ), dim3( groups < resident ? groups : resident ), dim3( Threads ), lds, stream,
-		a, w, bias, c, M, N, rowBlocks, act, residual );
+	const int grid = groups < resident ? groups : resident;
+	if( RP > 0 && geo.SlowRows > grid * 128 ) {
+		return false;
+	}
+	hipLaunchKernelGGL( ( shortReductionKernel<KC, NB, RES, RP> ), dim3( grid ), dim3( Threads ), lds, stream,
+		a, w, bias, c, M, N, rowBlocks, act, residual, geo );
+	return true;
 }
 
 // One kernel per count of column blocks that 64 KB of LDS hold next to the output patches.
@@ -1618,11 +1849,9 @@ static bool launchShortReductionColumns( hipStream_t stream, const float* a, con
 	if constexpr( NB >= 1 && shortReductionLds( KC * 8, NB >= 1 ? NB : 1 ) <= 64 * 1024 ) {
 		if( ceilDiv( N, 32 ) == NB ) {
 			if( residual != nullptr ) {
-				launchShortReduction<KC, NB, true>( stream, a, w, bias, c, M, N, act, residual );
-			} else {
-				launchShortReduction<KC, NB, false>( stream, a, w, bias, c, M, N, act, residual );
+				return launchShortReduction<KC, NB, true>( stream, a, w, bias, c, M, N, act, residual );
 			}
-			return true;
+			return launchShortReduction<KC, NB, false>( stream, a, w, bias, c, M, N, act, residual );
 		}
 		return launchShortReductionColumns<KC, NB - 1>( stream, a, w, bias, c, M, N, act, residual );
 	} else if constexpr( NB >= 1 ) {
@@ -1753,6 +1982,62 @@ int matMulTN( hipStream_t stream, const float* a, int lda, const float* b, int l
 	return launchMatMul<AM_RowsM, BM_RowsN>( stream, args, batch, vec );
 }
 
+// The first layer of an image network through the short-reduction kernel's window loader: true (and launched) for the
+// filter shapes it is built for.
+template<int KC, int RP>
+static bool launchWindowReduction( hipStream_t stream, const float* a, const float* w, const float* bias, float* c, int M, int N,
+	const CFusedActivation& act, const CRowRuns& geo )
+{
+	if( N <= 32 ) {
+		return launchShortReduction<KC, 1, false, RP>( stream, a, w, bias, c, M, N, act, nullptr, geo );
+	}
+	return launchShortReduction<KC, 2, false, RP>( stream, a, w, bias, c, M, N, act, nullptr, geo );
+}
+
+static bool tryWindowReduction( hipStream_t stream, const nhConvDesc& d, const float* source, const float* filter,
+	const float* freeTerm, float* result, const CFusedActivation& act, int* rc )
+{
+	const long long m = static_cast<long long>( d.batch ) * d.resultHeight * d.resultWidth;
+	const long long imageFloats = static_cast<long long>( d.batch ) * d.height * d.width * d.channels;
+	const int rowK = d.filterWidth * d.channels;
+	const int rowPitch = ( rowK + 3 ) / 4 * 4;
+	if( d.dilationHeight != 1 || d.dilationWidth != 1 || m < 16384 || d.filterCount > 64 || d.filterCount % 4 != 0
+		|| !isAligned16( result ) || imageFloats * 4 >= static_cast<long long>( BufferBytes )
+		|| !fitsBuffer( m + 32, d.filterCount, d.filterCount ) )
+	{
+		return false;
+	}
+	CRowRuns geo = {};
+	geo.H = d.height; geo.W = d.width; geo.Cin = d.channels; geo.Ho = d.resultHeight; geo.Wo = d.resultWidth;
+	geo.Fh = d.filterHeight; geo.RowK = rowK;
+	geo.PadH = d.paddingHeight; geo.PadW = d.paddingWidth; geo.StrideH = d.strideHeight; geo.StrideW = d.strideWidth;
+	geo.ABytes = static_cast<unsigned>( imageFloats * 4 );
+	// windows that begin in front of the blob: first image, filter row on image row 0, padding on the left
+	geo.SlowRows = d.paddingWidth > 0 ? ( d.paddingHeight / d.strideHeight + 1 ) * d.resultWidth : 0;
+	const int M = static_cast<int>( m );
+	const int N = d.filterCount;
+	const int kc = ( d.filterHeight * rowPitch + 7 ) / 8;
+	bool launched = false;
+	if( rowPitch == 12 && kc == 5 ) { // 3 x 3 over RGB
+		launched = launchWindowReduction<5, 12>( stream, source, filter, freeTerm, result, M, N, act, geo );
+	} else if( rowPitch == 24 && kc == 21 ) { // 7 x 7 over RGB
+		launched = launchWindowReduction<21, 24>( stream, source, filter, freeTerm, result, M, N, act, geo );
+	} else if( rowPitch == 4 && kc == 2 ) { // 3 x 3 over one channel
+		launched = launchWindowReduction<2, 4>( stream, source, filter, freeTerm, result, M, N, act, geo );
+	}
+	if( !launched ) {
+		return false;
+	}
+	const hipError_t err = hipGetLastError();
+	if( err != hipSuccess ) {
+		setLastError( "window reduction: launch failed: %s", hipGetErrorString( err ) );
+		*rc = NH_ERR_HIP;
+	} else {
+		*rc = NH_OK;
+	}
+	return true;
+}
+
 int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* source, const float* filter,
 	const float* freeTerm, float* result, const CFusedActivation& act, const CSliceMeeting* fixedMeeting = nullptr )
 {
@@ -1784,6 +2069,12 @@ int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* sour
 	}
 	if( d.filterHeight == 1 && d.filterWidth == 1 ) {
 		return launchMatMul<AM_Conv1x1, BM_RowsK>( stream, args, 1, vec, fixedMeeting );
+	}
+	if( d.channels % 4 != 0 ) {
+		int rc = NH_OK;
+		if( tryWindowReduction( stream, d, source, filter, freeTerm, result, act, &rc ) ) {
+			return rc;
+		}
 	}
 	if( d.channels % 4 != 0 && d.dilationWidth == 1
 		&& fitsBuffer( 1, 0, static_cast<long long>( d.batch ) * d.height * d.width * d.channels )

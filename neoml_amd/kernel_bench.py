@@ -98,6 +98,7 @@ def main():
     conv("cfg2 s4", 64, 7, 7, 512, 512, 3, 1, 1)
     conv("cfg2 s2 down", 64, 56, 56, 64, 128, 3, 1, 2)
     conv("cfg2 s2 short", 64, 56, 56, 64, 128, 1, 0, 2)
+    conv("cfg3 stem", 128, 224, 224, 3, 32, 3, 1, 2)
     conv("cfg3 project", 128, 112, 112, 32, 16, 1, 0, 1)
     conv("cfg3 expand", 128, 112, 112, 16, 96, 1, 0, 1)
     conv("cfg3 project", 128, 56, 56, 96, 24, 1, 0, 1)

@@ -91,7 +91,7 @@ class HipBackend:
     # ---- ops (shapes are N,H,W,C)
     def conv(self, x, filt, bias, ph, pw, sh, sw, out=None, relu=False):
         """relu: the activation in the convolution's own launch, what a rowwise chain of NeoML's graph optimizer
-        (convolution + ReLU) asks of the engine."""
+        (convolution + ReLU) asks of the engine; True for the plain ReLU, a number for ReLU with that upper threshold."""
         n, h, w, cin = x.shape
         cout, fh, fw, _ = filt.shape
         key = ("conv", n, h, w, cin, cout, fh, fw, ph, pw, sh, sw)
@@ -107,7 +107,7 @@ class HipBackend:
         if relu:
             self._timed(tag, conv_flops(n, ho, wo, cout, fh, fw, cin), conv_bytes(n, h, w, cin, ho, wo, cout, fh, fw),
                         self.lib.nhBlobConvolutionWithActivation, ctypes.byref(d), self._p(x), self._p(filt), self._p(bias),
-                        1, ctypes.c_float(0.0), self._p(out))
+                        1, ctypes.c_float(0.0 if relu is True else float(relu)), self._p(out))
             return out
         self._timed(tag, conv_flops(n, ho, wo, cout, fh, fw, cin), conv_bytes(n, h, w, cin, ho, wo, cout, fh, fw),
                     self.lib.nhBlobConvolution, ctypes.byref(d), self._p(x), self._p(filt), self._p(bias), self._p(out))
@@ -592,8 +592,10 @@ class MobileNetV2(Network):
 
     def forward(self, x):
         be, run, W = self.be, self.run, self.dev
-        y = run("stem", be.conv, x, *W["stem"], 1, 1, 2, 2)
-        be.relu6_(y)
+        # ( the optimizer's form: the stem and its ReLU6 are a rowwise chain = one engine call )
+        y = run("stem", be.conv, x, *W["stem"], 1, 1, 2, 2, relu=6.0 if self.fused else False)
+        if not self.fused:
+            be.relu6_(y)
         for name, expand, stride, residual in self.blocks:
             if self.fused:
                 y = run(name + "p", be.separable_block, y, W[name + "e"] if expand else None, W[name + "d"], W[name + "p"],

@@ -1138,7 +1138,7 @@ class CpuBackend:
 
     def conv(self, x, filt, bias, ph, pw, sh, sw, out=None, relu=False):
         y = self.cpu.conv(x, filt, bias, ph, pw, sh, sw)
-        return self.cpu.unary("relu", y, 0.0).reshape(y.shape) if relu else y
+        return self.cpu.unary("relu", y, 0.0 if relu is True else float(relu)).reshape(y.shape) if relu else y
 
     def relu_(self, x, threshold=None):
         x[...] = self.cpu.unary("relu", x, 0.0 if threshold is None else threshold).reshape(x.shape)

@@ -666,6 +666,81 @@ def test_convolution_ignores_pixels_outside_the_windows():
     assert_close(got, want, "unused columns")
 
 
+# The first layer of an image network: one or three channels, 3 x 3 or 7 x 7 filter, up to 64 filters, 16384 output
+# pixels or more. These go through the window loader of the short-reduction kernel (128-bit loads at 4-byte alignment
+# that bring along what lies next to a window; zeros by masks and by the memory unit's range check).
+# (n, h, w, cin, cout, fh, fw, ph, pw, sh, sw)
+WINDOW_CASES = [
+    (2, 184, 200, 3, 32, 3, 3, 1, 1, 2, 2),   # the depthwise-separable network's stem, reduced
+    (2, 190, 182, 3, 64, 7, 7, 3, 3, 2, 2),   # the residual network's stem, reduced: two rows of pixels begin in front of the blob
+    (2, 96, 100, 1, 64, 3, 3, 1, 1, 1, 1),    # the line recogniser's first layer, reduced
+    (1, 130, 140, 3, 20, 3, 3, 0, 0, 1, 1),   # no padding, a filter count that fills no column block
+    (1, 400, 400, 3, 48, 3, 3, 2, 2, 3, 3),   # padding beyond the filter's reach on the left and at the top
+    (1, 130, 131, 3, 8, 7, 7, 3, 3, 1, 1),    # windows that hang over the right border by up to three pixels
+    (3, 151, 149, 1, 36, 3, 3, 1, 1, 2, 2),   # odd sizes: the last row block is ragged
+    (1, 136, 129, 3, 64, 7, 7, 0, 5, 1, 1),   # wide padding on the left only
+]
+
+
+@pytest.mark.parametrize("case", WINDOW_CASES)
+def test_first_layer_convolution(case):
+    n, h, w, cin, cout, fh, fw, ph, pw, sh, sw = case
+    g = rng(sum(case))
+    x = g.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    f = g.normal(0, 1.0 / np.sqrt(fh * fw * cin), (cout, fh, fw, cin)).astype(np.float32)
+    bias = g.uniform(-1, 1, cout).astype(np.float32)
+    want = orc.conv(x, f, bias, ph, pw, sh, sw)
+    assert want.shape[0] * want.shape[1] * want.shape[2] >= 16384
+    assert_close(hip().conv(x, f, bias, ph, pw, sh, sw), want, "first layer %s" % (case,))
+    assert_close(hip().conv(x, f, None, ph, pw, sh, sw), want - bias, "without free term", atol=2e-5)
+    assert_close(hip().conv(x, f, bias, ph, pw, sh, sw, activation="relu", param=0.5),
+                 np.clip(want, 0.0, 0.5), "with ReLU clipped at 0.5")
+
+
+def test_first_layer_convolution_reads_nothing_beside_its_windows():
+    """Infinities in the image columns that no window touches (stride 4, filter 3 wide), and the image blob placed
+    between two blocks of infinities: nothing of either may reach the result."""
+    import ctypes
+    import torch
+    import neoml_amd
+    lib = neoml_amd.load()
+    g = rng(79)
+    n, h, w, cin, cout = 2, 130, 267, 3, 24
+    x = g.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    x[:, :, 3::4, :] = np.inf
+    f = g.normal(0, 0.3, (cout, 3, 3, cin)).astype(np.float32)
+    want = orc.conv(np.nan_to_num(x, posinf=0.0), f, None, 0, 0, 1, 4)
+    assert want.shape == (n, 128, 67, cout)
+    dev = torch.device("cuda:0")
+    guard = 1024  # floats, keeps the blob 16-byte aligned
+    room = torch.full((guard + x.size + guard,), float("inf"), device=dev)
+    room[guard:guard + x.size] = torch.from_numpy(x.reshape(-1)).to(dev)
+    y = torch.zeros(want.shape, device=dev)
+    fd = torch.from_numpy(f).to(dev)
+    d = neoml_amd.ConvDesc(n, h, w, cin, cout, 3, 3, 0, 0, 1, 4, 1, 1, 0, 0)
+    neoml_amd.check(lib.nhInitBlobConvolution(ctypes.byref(d)))
+    torch.cuda.synchronize()
+    neoml_amd.check(lib.nhBlobConvolution(None, ctypes.byref(d), ctypes.c_void_p(room.data_ptr() + 4 * guard),
+                                          ctypes.c_void_p(fd.data_ptr()), None, ctypes.c_void_p(y.data_ptr())))
+    torch.cuda.synchronize()
+    got = y.cpu().numpy()
+    assert np.isfinite(got).all()
+    assert_close(got, want, "unused columns and guards")
+    # with padding: the windows of the first pixels begin in front of the blob, those of the last ones end behind it
+    x2 = g.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    room[guard:guard + x.size] = torch.from_numpy(x2.reshape(-1)).to(dev)
+    want2 = orc.conv(x2, f, None, 1, 1, 1, 1)
+    y2 = torch.zeros(want2.shape, device=dev)
+    d2 = neoml_amd.ConvDesc(n, h, w, cin, cout, 3, 3, 1, 1, 1, 1, 1, 1, 0, 0)
+    neoml_amd.check(lib.nhInitBlobConvolution(ctypes.byref(d2)))
+    neoml_amd.check(lib.nhBlobConvolution(None, ctypes.byref(d2), ctypes.c_void_p(room.data_ptr() + 4 * guard),
+                                          ctypes.c_void_p(fd.data_ptr()), None, ctypes.c_void_p(y2.data_ptr())))
+    torch.cuda.synchronize()
+    got2 = y2.cpu().numpy()
+    assert np.isfinite(got2).all()
+    assert_close(got2, want2, "padded windows between guards")
+
+
 def test_convolution_config1_vs_reference_engine():
     # the single-layer configuration at reduced batch: 32x32x64 image, 3x3 64 -> 64, pad 1, + free term, then ReLU
     g = rng(1)
