@@ -581,6 +581,81 @@ NH_API int nhLinearInterpolation(nhStream s, const float* data, float* result, i
 NH_API int nhScatterND(nhStream s, const int* indices, const void* updates, void* data, const nhBlobDesc* dataDesc_host, int updateCount,
 	int indexDims);                                                                                                  /* NME.h:1061-1063; 32-bit elements */
 
+/* ---- members that no network of the benchmark configurations calls (rare_ops.hip): plain kernels -------------------- */
+/* QRNN poolings (NME.h:943-962). reverse != 0: the sequence is walked from its last element. initialState may be null.
+ * The backward passes walk in the same direction, read the state "before" an element at the next position of the walk and
+ * add every element's recurrent share onto resultDiff there: resultDiff is modified, as in the reference. */
+NH_API int nhQrnnFPooling(nhStream s, int reverse, int sequenceLength, int objectSize, const float* update, const float* forget,
+	const float* initialState, float* result);                                                                        /* NME.h:943 */
+NH_API int nhQrnnFPoolingBackward(nhStream s, int reverse, int sequenceLength, int objectSize, const float* update, const float* forget,
+	const float* initialState, const float* result, float* resultDiff, float* updateDiff, float* forgetDiff);         /* NME.h:948 */
+NH_API int nhQrnnIfPooling(nhStream s, int reverse, int sequenceLength, int objectSize, const float* update, const float* forget,
+	const float* input, const float* initialState, float* result);                                                    /* NME.h:954 */
+NH_API int nhQrnnIfPoolingBackward(nhStream s, int reverse, int sequenceLength, int objectSize, const float* update, const float* forget,
+	const float* input, const float* initialState, const float* result, float* resultDiff, float* updateDiff, float* forgetDiff,
+	float* inputDiff);                                                                                                /* NME.h:959 */
+/* IndRNN (NME.h:979-990): h_t = activation( wx_t + u * mask * h_(t-1) ); mask [batch x object] may be null; uDiff is added to */
+#define NH_INDRNN_SIGMOID 0
+#define NH_INDRNN_RELU 1
+NH_API int nhIndRnnRecurrent(nhStream s, int reverse, int sequenceLength, int batchSize, int objectSize, int activation, const float* wx,
+	const float* mask, const float* u, float* h);                                                                     /* NME.h:979 */
+NH_API int nhIndRnnRecurrentBackward(nhStream s, int reverse, int sequenceLength, int batchSize, int objectSize, int activation,
+	const float* mask, const float* u, const float* h, const float* hDiff, float* wxDiff);                            /* NME.h:983 */
+NH_API int nhIndRnnRecurrentLearn(nhStream s, int reverse, int sequenceLength, int batchSize, int objectSize, int activation,
+	const float* mask, const float* u, const float* h, const float* hDiff, float* uDiff);                             /* NME.h:988 */
+/* BERT's light-weight convolution (NME.h:1039-1043): data [seqLen][batch][heads x headSize], kernel [seqLen][batch x heads][kernelSize] */
+NH_API int nhBertConv(nhStream s, const float* data, const float* kernel, int seqLen, int batchSize, int numHeads, int headSize,
+	int kernelSize, float* output);
+NH_API int nhBertConvBackward(nhStream s, const float* data, const float* kernel, const float* outDiff, int seqLen, int batchSize,
+	int numHeads, int headSize, int kernelSize, float* dataDiff, float* kernelDiff);
+/* Local response normalization over the channels (NME.h:994-1002; CMathEngineLrnDesc: vectorCount = objects x positions,
+ * vectorSize = channels). invSum and invSumBeta may be null in the forward pass (they are what the backward pass needs). */
+NH_API int nhLrn(nhStream s, const float* input, int vectorCount, int vectorSize, int windowSize, float bias, float alpha, float beta,
+	float* invSum, float* invSumBeta, float* output);
+NH_API int nhLrnBackward(nhStream s, const float* input, const float* output, const float* outputDiff, const float* invSum,
+	const float* invSumBeta, int vectorCount, int vectorSize, int windowSize, float alpha, float beta, float* inputDiff);
+/* Products with a sparse matrix in CSR form (CSparseMatrixDesc: rows [height + 1], columns and values [elements]; NME.h:541-559) */
+NH_API int nhMultiplySparseMatrixByTransposedMatrix(nhStream s, int firstHeight, int firstWidth, int secondHeight, const int* rows,
+	const int* columns, const float* values, const float* second, float* result);                                     /* NME.h:541 */
+/* isTransposedSparse: the sparse matrix is [resultWidth x firstHeight]; add: onto result (NME.h:550) instead of into it (NME.h:545) */
+NH_API int nhMultiplyTransposedMatrixBySparseMatrix(nhStream s, int firstHeight, int firstWidth, int resultWidth, const float* first,
+	const int* rows, const int* columns, const float* values, float* result, int isTransposedSparse, int add);
+NH_API int nhMultiplySparseMatrixByMatrix(nhStream s, int firstHeight, int firstWidth, int secondWidth, const int* rows,
+	const int* columns, const float* values, const float* second, float* result);                                     /* NME.h:554 */
+NH_API int nhMultiplyTransposedSparseMatrixByMatrix(nhStream s, int firstHeight, int firstWidth, int secondWidth, const int* rows,
+	const int* columns, const float* values, const float* second, float* result);                                     /* NME.h:558 */
+/* the k largest values in descending order and their positions, equal values in the order of their positions (NME.h:380-383) */
+NH_API int nhVectorTopK(nhStream s, const float* first, int firstSize, int k, float* result, int* indices);
+NH_API int nhVectorTopKDiff(nhStream s, const float* sourceGrad, int sourceGradHeight, int sourceGradWidth, const int* indices, int k,
+	float* resultGrad);
+/* 3-D convolution and pooling over blobs [batch][height][width][depth][channels] (CCommon3dConvolutionDesc,
+ * CCommon3dMaxPoolingDesc, CCommon3dMeanPoolingDesc); filter [filterCount][fh][fw][fd][channels]; poolings have no padding and
+ * filterCount is unused there */
+typedef struct nh3dDesc {
+	int batch, height, width, depth, channels;
+	int filterCount, filterHeight, filterWidth, filterDepth;
+	int paddingHeight, paddingWidth, paddingDepth;
+	int strideHeight, strideWidth, strideDepth;
+	int resultHeight, resultWidth, resultDepth;
+} nh3dDesc;
+NH_API int nhBlob3dConvolution(nhStream s, const nh3dDesc* desc_host, const float* source, const float* filter, const float* freeTerm,
+	float* result);                                                                                                   /* NME.h:741 */
+/* freeTerm [channels] or null is added to every position of inputDiff */
+NH_API int nhBlob3dConvolutionBackward(nhStream s, const nh3dDesc* desc_host, const float* outputDiff, const float* filter,
+	const float* freeTerm, float* inputDiff);                                                                         /* NME.h:743 */
+NH_API int nhBlob3dConvolutionLearnAdd(nhStream s, const nh3dDesc* desc_host, const float* input, const float* outputDiff,
+	float* filterDiff, float* freeTermDiff, int freeTermDiffFromInput);                                               /* NME.h:745 */
+/* maxIndices (may be null in the forward pass): offset of channel 0 of the winning position inside the source object */
+NH_API int nhBlob3dMaxPooling(nhStream s, const nh3dDesc* desc_host, const float* source, int* maxIndices, float* result);   /* NME.h:798 */
+NH_API int nhBlob3dMaxPoolingBackward(nhStream s, const nh3dDesc* desc_host, const float* resultDiff, const int* maxIndices,
+	float* sourceDiff);                                                                                               /* NME.h:800 */
+NH_API int nhBlob3dMeanPooling(nhStream s, const nh3dDesc* desc_host, const float* source, float* result);                  /* NME.h:810 */
+NH_API int nhBlob3dMeanPoolingBackward(nhStream s, const nh3dDesc* desc_host, const float* resultDiff, float* sourceDiff);  /* NME.h:812 */
+/* Run-length encoded black-and-white images (CRleImage, NME.h:664-686) to dense ones of stroke / non-stroke values: what
+ * BlobRleConvolution and BlobRleConvolutionLearnAdd (NME.h:871-878) run in front of the ordinary convolution entry points */
+NH_API int nhRleImagesToDense(nhStream s, const void* rle, int batch, int height, int width, float strokeValue, float nonStrokeValue,
+	float* dense);
+
 #ifdef __cplusplus
 }
 #endif

@@ -12,7 +12,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libneoml_hip.so")
 
-SOURCES = ["runtime.hip", "mem_pool.cpp", "vector_ops.hip", "blas_ops.hip", "dnn_ops.hip", "wide_ops.hip", "gemm_mfma.hip"]
+SOURCES = ["runtime.hip", "mem_pool.cpp", "vector_ops.hip", "blas_ops.hip", "dnn_ops.hip", "wide_ops.hip", "rare_ops.hip", "gemm_mfma.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming packed fp32 VALU instructions
 HIPCC_FLAGS = [

@@ -480,6 +480,39 @@ public:
 	void LinearInterpolation( const CConstFloatHandle& dataHandle, const CFloatHandle& resultHandle, TInterpolationCoords coords, TInterpolationRound round, int objectCount, int scaledAxis, int objectSize, float scale ) override;
 	void ScatterND( const CConstIntHandle& indicesHandle, const CConstFloatHandle& updatesHandle, const CFloatHandle& dataHandle, const CBlobDesc& dataDesc, int updateCount, int indexDims ) override;
 	void ScatterND( const CConstIntHandle& indicesHandle, const CConstIntHandle& updatesHandle, const CIntHandle& dataHandle, const CBlobDesc& dataDesc, int updateCount, int indexDims ) override;
+	// recurrent poolings, BERT convolution, LRN, sparse products, top-k, 3-D convolution and pooling, RLE convolution ( HipMathEngineRare.cpp )
+	void QrnnFPooling( bool reverse, int sequenceLength, int objectSize, const CConstFloatHandle& update, const CConstFloatHandle& forget, const CConstFloatHandle& initialState, const CFloatHandle& result ) override;
+	void QrnnFPoolingBackward( bool reverse, int sequenceLength, int objectSize, const CConstFloatHandle& update, const CConstFloatHandle& forget, const CConstFloatHandle& initialState, const CConstFloatHandle& result, const CFloatHandle& resultDiff, const CFloatHandle& updateDiff, const CFloatHandle& forgetDiff ) override;
+	void QrnnIfPooling( bool reverse, int sequenceLength, int objectSize, const CConstFloatHandle& update, const CConstFloatHandle& forget, const CConstFloatHandle& input, const CConstFloatHandle& initialState, const CFloatHandle& result ) override;
+	void QrnnIfPoolingBackward( bool reverse, int sequenceLength, int objectSize, const CConstFloatHandle& update, const CConstFloatHandle& forget, const CConstFloatHandle& input, const CConstFloatHandle& initialState, const CConstFloatHandle& result, const CFloatHandle& resultDiff, const CFloatHandle& updateDiff, const CFloatHandle& forgetDiff, const CFloatHandle& inputDiff ) override;
+	void IndRnnRecurrent( bool reverse, int sequenceLength, int batchSize, int objectSize, TActivationFunction activation, const CConstFloatHandle& wx, const CConstFloatHandle& mask, const CConstFloatHandle& u, const CFloatHandle& h ) override;
+	void IndRnnRecurrentBackward( bool reverse, int sequenceLength, int batchSize, int objectSize, TActivationFunction activation, const CConstFloatHandle& mask, const CConstFloatHandle& u, const CConstFloatHandle& h, const CConstFloatHandle& hDiff, const CFloatHandle& wxDiff ) override;
+	void IndRnnRecurrentLearn( bool reverse, int sequenceLength, int batchSize, int objectSize, TActivationFunction activation, const CConstFloatHandle& mask, const CConstFloatHandle& u, const CConstFloatHandle& h, const CConstFloatHandle& hDiff, const CFloatHandle& uDiff ) override;
+	void BertConv( const CConstFloatHandle& dataHandle, const CConstFloatHandle& kernelHandle, int seqLen, int batchSize, int numHeads, int headSize, int kernelSize, const CFloatHandle& outputHandle ) override;
+	void BertConvBackward( const CConstFloatHandle& dataHandle, const CConstFloatHandle& kernelHandle, const CConstFloatHandle& outDiffHandle, int seqLen, int batchSize, int numHeads, int headSize, int kernelSize, const CFloatHandle& dataDiffHandle, const CFloatHandle& kernelDiffHandle ) override;
+	CLrnDesc* InitLrn( const CBlobDesc& source, int windowSize, float bias, float alpha, float beta ) override;
+	void Lrn( const CLrnDesc& desc, const CConstFloatHandle& input, const CFloatHandle& invSum, const CFloatHandle& invSumBeta, const CFloatHandle& outputHandle ) override;
+	void LrnBackward( const CLrnDesc& desc, const CConstFloatHandle& input, const CConstFloatHandle& output, const CConstFloatHandle& outputDiff, const CConstFloatHandle& invSum, const CConstFloatHandle& invSumBeta, const CFloatHandle& inputDiff ) override;
+	void MultiplySparseMatrixByTransposedMatrix( int firstHeight, int firstWidth, int secondHeight, const CSparseMatrixDesc& firstDesc, const CConstFloatHandle& secondHandle, const CFloatHandle& resultHandle ) override;
+	void MultiplyTransposedMatrixBySparseMatrix( int firstHeight, int firstWidth, int resultWidth, const CConstFloatHandle& firstHandle, const CSparseMatrixDesc& secondDesc, const CFloatHandle& resultHandle, bool isTransposedSparse ) override;
+	void MultiplyTransposedMatrixBySparseMatrixAndAdd( int firstHeight, int firstWidth, int secondWidth, const CConstFloatHandle& firstHandle, const CSparseMatrixDesc& secondDesc, const CFloatHandle& resultHandle ) override;
+	void MultiplySparseMatrixByMatrix( int firstHeight, int firstWidth, int secondWidth, const CSparseMatrixDesc& firstDesc, const CConstFloatHandle& secondHandle, const CFloatHandle& resultHandle ) override;
+	void MultiplyTransposedSparseMatrixByMatrix( int firstHeight, int firstWidth, int secondWidth, const CSparseMatrixDesc& firstDesc, const CConstFloatHandle& secondHandle, const CFloatHandle& resultHandle ) override;
+	void VectorTopK( const CConstFloatHandle& first, int firstSize, int k, const CFloatHandle& result, const CIntHandle& indices ) override;
+	void VectorTopKDiff( const CConstFloatHandle& sourceGrad, int sourceGradHeight, int sourceGradWidth, const CConstIntHandle& indices, int k, const CFloatHandle& resultGrad ) override;
+	C3dConvolutionDesc* InitBlob3dConvolution( const CBlobDesc& input, int paddingHeight, int paddingWidth, int paddingDepth, int strideHeight, int strideWidth, int strideDepth, const CBlobDesc& filter, const CBlobDesc& output ) override;
+	void Blob3dConvolution( const C3dConvolutionDesc& desc, const CConstFloatHandle& source, const CConstFloatHandle& filter, const CConstFloatHandle* freeTerm, const CFloatHandle& result ) override;
+	void Blob3dConvolutionBackward( const C3dConvolutionDesc& desc, const CConstFloatHandle& source, const CConstFloatHandle& filter, const CConstFloatHandle* freeTerm, const CFloatHandle& result ) override;
+	void Blob3dConvolutionLearnAdd( const C3dConvolutionDesc& desc, const CConstFloatHandle& input, const CConstFloatHandle& outputDiff, const CFloatHandle& filterDiff, const CFloatHandle* freeTermDiff, bool isFreeTermDiffFromInput ) override;
+	C3dMaxPoolingDesc* Init3dMaxPooling( const CBlobDesc& source, int filterHeight, int filterWidth, int filterDepth, int strideHeight, int strideWidth, int strideDepth, const CBlobDesc& result ) override;
+	void Blob3dMaxPooling( const C3dMaxPoolingDesc& desc, const CConstFloatHandle& source, const CIntHandle* maxIndices, const CFloatHandle& result ) override;
+	void Blob3dMaxPoolingBackward( const C3dMaxPoolingDesc& desc, const CConstFloatHandle& resultDiff, const CConstIntHandle& maxIndices, const CFloatHandle& sourceDiff ) override;
+	C3dMeanPoolingDesc* Init3dMeanPooling( const CBlobDesc& source, int filterHeight, int filterWidth, int filterDepth, int strideHeight, int strideWidth, int strideDepth, const CBlobDesc& result ) override;
+	void Blob3dMeanPooling( const C3dMeanPoolingDesc& desc, const CConstFloatHandle& source, const CFloatHandle& result ) override;
+	void Blob3dMeanPoolingBackward( const C3dMeanPoolingDesc& desc, const CConstFloatHandle& resultDiff, const CFloatHandle& sourceDiff ) override;
+	CRleConvolutionDesc* InitBlobRleConvolution( const CBlobDesc& input, float strokeValue, float nonStrokeValue, int strideHeight, int strideWidth, const CBlobDesc& filter, const CBlobDesc& output ) override;
+	void BlobRleConvolution( const CRleConvolutionDesc& desc, const CConstFloatHandle& source, const CConstFloatHandle& filter, const CConstFloatHandle* freeTerm, const CFloatHandle& result ) override;
+	void BlobRleConvolutionLearnAdd( const CRleConvolutionDesc& desc, const CConstFloatHandle& input, const CConstFloatHandle& outputDiff, const CFloatHandle& filterDiff, const CFloatHandle* freeTermDiff ) override;
 	// ---- end of the members beyond the inference path ----
 
 	// every other pure virtual of the interface: asserting bodies generated from the interface header

@@ -990,7 +990,19 @@ SHIM_API int shim_performance_counters( void* engine, int smallSize, int largeSi
 	} );
 }
 
-// probe for a method outside the implemented paths (asserts on engines that do not implement it)
+// probe for a method outside the implemented paths (asserts on engines that do not implement it, and on the reference CPU
+// engine where it is built without MKL)
+SHIM_API int shim_singular_value_decomposition( void* engine, const float* matrix, int height, int width, float* singular )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		const int rank = height < width ? height : width;
+		CFloatBlob a( e, height * width, matrix ), u( e, height * rank ), sv( e, rank ), vt( e, rank * width ), superb( e, rank );
+		e.SingularValueDecomposition( a.Handle(), height, width, u.Handle(), sv.Handle(), vt.Handle(), superb.Handle(), true, true );
+		sv.CopyTo( singular );
+	} );
+}
+
 SHIM_API int shim_vector_top_k( void* engine, const float* first, int n, int k, float* result, int* indices )
 {
 	return guarded( [&]() {

@@ -209,15 +209,25 @@ def test_lstm_through_the_interface(reverse):
 
 
 def test_unimplemented_method_asserts_like_the_reference_gpu_engine():
-    # VectorTopK is outside the implemented paths: the generated body raises through NeoML's exception handler,
-    # which the shim turns into an error code instead of letting it cross the C boundary
+    # SingularValueDecomposition is one of the four members left as generated bodies: it raises through NeoML's exception
+    # handler, which the shim turns into an error code instead of letting it cross the C boundary
     s = nhtest.shim()
-    x = np.arange(8, dtype=np.float32)
-    y = np.empty(2, np.float32)
-    idx = np.empty(2, np.int32)
-    ip = idx.ctypes.data_as(ctypes.POINTER(ctypes.c_int))
-    assert s.shim_vector_top_k(nhtest.hip_engine(), nhtest.fp(x), 8, 2, nhtest.fp(y), ip) == 1
-    assert s.shim_vector_top_k(nhtest.cpu_engine(), nhtest.fp(x), 8, 2, nhtest.fp(y), ip) == 0 and y[0] == 7.0 and idx[0] == 7
+    a = np.array([[3.0, 1.0], [1.0, 2.0]], np.float32)
+    sv = np.empty(2, np.float32)
+    assert s.shim_singular_value_decomposition(nhtest.hip_engine(), nhtest.fp(a), 2, 2, nhtest.fp(sv)) == 1
+
+
+def test_vector_top_k_on_both_engines():
+    # descending values with their positions; of equal values the one met first comes first
+    s = nhtest.shim()
+    x = np.array([1.0, 7.0, 3.0, 7.0, -2.0, 5.0, 7.0, 0.5], np.float32)
+    got, want = np.empty(5, np.float32), np.empty(5, np.float32)
+    got_idx, want_idx = np.empty(5, np.int32), np.empty(5, np.int32)
+    ip = lambda a: a.ctypes.data_as(ctypes.POINTER(ctypes.c_int))
+    assert s.shim_vector_top_k(nhtest.hip_engine(), nhtest.fp(x), 8, 5, nhtest.fp(got), ip(got_idx)) == 0
+    assert s.shim_vector_top_k(nhtest.cpu_engine(), nhtest.fp(x), 8, 5, nhtest.fp(want), ip(want_idx)) == 0
+    assert list(want_idx) == [1, 3, 6, 5, 2]
+    assert np.array_equal(got, want) and np.array_equal(got_idx, want_idx)
 
 
 def test_vector_power_on_both_engines():
