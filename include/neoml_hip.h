@@ -651,6 +651,14 @@ NH_API int nhBlob3dMaxPoolingBackward(nhStream s, const nh3dDesc* desc_host, con
 	float* sourceDiff);                                                                                               /* NME.h:800 */
 NH_API int nhBlob3dMeanPooling(nhStream s, const nh3dDesc* desc_host, const float* source, float* result);                  /* NME.h:810 */
 NH_API int nhBlob3dMeanPoolingBackward(nhStream s, const nh3dDesc* desc_host, const float* resultDiff, float* sourceDiff);  /* NME.h:812 */
+/* CTC loss (NME.h:1033-1036): result [resultLen][batch][classCount] before its softmax, labels [labelLen][batch]; labelLens,
+ * resultLens, labelWeights and lossGradient may be null; loss receives - sum( weight * log p( labels ) ) / batch, lossGradient the
+ * gradient by result (not weighted, not divided by the batch: the loss layer does both). workspace: device memory of at
+ * least nhCtcLossWorkspaceSize bytes. */
+NH_API int nhCtcLossWorkspaceSize(int resultLen, int batchSize, int classCount, int labelLen, size_t* bytes);
+NH_API int nhCtcLossForward(nhStream s, int resultLen, int batchSize, int classCount, int labelLen, int blankLabel, int skipBlanks,
+	const float* result, const int* labels, const int* labelLens, const int* resultLens, const float* labelWeights, float* loss,
+	float* lossGradient, void* workspace, size_t workspaceBytes);
 /* Run-length encoded black-and-white images (CRleImage, NME.h:664-686) to dense ones of stroke / non-stroke values: what
  * BlobRleConvolution and BlobRleConvolutionLearnAdd (NME.h:871-878) run in front of the ordinary convolution entry points */
 NH_API int nhRleImagesToDense(nhStream s, const void* rle, int batch, int height, int width, float strokeValue, float nonStrokeValue,

@@ -677,6 +677,202 @@ void rleDecodeKernel( const int* rle, int batch, int height, int width, float st
 	}
 }
 
+
+// ---- CTC loss ( src/CPU/CpuMathEngineDnnCtc.cpp:202-403 ) ----------------------------------------------------------
+// The lattice of a sequence: U = 2 * labelLen + 1 positions ( blank, label 0, blank, label 1, ..., blank ), T frames.
+// logAlpha[t][u] / logBeta[t][u] are the reference's forward / backward variables in the log domain, computed by the same
+// operations in the same order ( its log-sum-exp of two values, its "log zero" of -FLT_MAX / 4, its padding of frames beyond
+// a sequence's length with a certain blank ), so that both engines agree to rounding. One workgroup walks one sequence of
+// the batch: the frames one after the other, the positions side by side.
+
+constexpr float CtcLogZero = -FLT_MAX / 4;
+
+__device__ __forceinline__ float ctcExp( float x )
+{
+	return x < -87.33654474f ? 0.f : ( x > 88.f ? FLT_MAX : expf( x ) );
+}
+
+// ( x86/CpuX86MathEngineVectorMathMkl.cpp:155-213 )
+__device__ __forceinline__ float ctcLogSumExp( float a, float b )
+{
+	const float e = ctcExp( -fabsf( a - b ) );
+	return fmaxf( a, b ) + logf( fminf( 1.f + fmaxf( e, FLT_MIN ), FLT_MAX ) );
+}
+
+struct CCtcShape {
+	int T, B, C, L, U, Blank, SkipBlanks;
+};
+
+__device__ __forceinline__ int ctcPaddedLabel( const CCtcShape& n, const int* labels, int b, int u )
+{
+	return ( u & 1 ) != 0 ? labels[( u >> 1 ) * n.B + b] : n.Blank;
+}
+
+// log( I{ u < U - 2 } * I{ label[u] != label[u + 2] } ): what a step over a blank adds
+__device__ __forceinline__ float ctcSkipMask( const CCtcShape& n, const int* labels, int b, int u )
+{
+	return ( u < n.U - 2 && ctcPaddedLabel( n, labels, b, u ) != ctcPaddedLabel( n, labels, b, u + 2 ) ) ? 0.f : CtcLogZero;
+}
+
+// log-probability of class k in frame t; frames beyond the sequence's length emit a blank for certain
+__device__ __forceinline__ float ctcEmission( const CCtcShape& n, const float* logProb, const int* resultLens, int t, int b, int k )
+{
+	if( resultLens != nullptr && t >= resultLens[b] ) {
+		return k == n.Blank ? -FLT_MIN * 2 : CtcLogZero;
+	}
+	return logProb[( static_cast<long long>( t ) * n.B + b ) * n.C + k];
+}
+
+// the reference's column-wise log-sum-exp: maximum, sum of exp( x - maximum ) in ascending order, clamped log
+__device__ float ctcLogSumExpOf( const float* values, int count )
+{
+	float top = values[0];
+	for( int i = 1; i < count; ++i ) {
+		top = values[i] > top ? values[i] : top;
+	}
+	float sum = 0.f;
+	for( int i = 0; i < count; ++i ) {
+		sum += ctcExp( values[i] - top );
+	}
+	return top + logf( fminf( fmaxf( sum, FLT_MIN ), FLT_MAX ) );
+}
+
+__global__ __launch_bounds__( 256 )
+void ctcLatticeKernel( const CCtcShape n, const float* logProb, const int* labels, const int* labelLens, const int* resultLens,
+	float* logAlpha, float* logBeta, float* total )
+{
+	extern __shared__ float lattice[]; // [3][U]
+	float* previous = lattice;
+	float* current = lattice + n.U;
+	float* shifted = lattice + 2 * n.U;
+	const int b = blockIdx.x;
+	const int U = n.U;
+	const long long frame = static_cast<long long>( U ) * n.B;
+
+	// forward: a sequence begins with a blank or with its first label
+	for( int u = threadIdx.x; u < U; u += 256 ) {
+		const float v = ( u < 2 ? 0.f : CtcLogZero ) + ctcEmission( n, logProb, resultLens, 0, b, ctcPaddedLabel( n, labels, b, u ) );
+		previous[u] = v;
+		logAlpha[static_cast<long long>( u ) * n.B + b] = v;
+	}
+	__syncthreads();
+	for( int t = 1; t < n.T; ++t ) {
+		for( int u = threadIdx.x; u < U; u += 256 ) {
+			float v = u == 0 ? previous[0] : ctcLogSumExp( previous[u - 1], previous[u] );
+			if( n.SkipBlanks && u >= 2 ) {
+				v = ctcLogSumExp( v, previous[u - 2] + ctcSkipMask( n, labels, b, u - 2 ) );
+			}
+			v += ctcEmission( n, logProb, resultLens, t, b, ctcPaddedLabel( n, labels, b, u ) );
+			current[u] = v;
+			logAlpha[t * frame + static_cast<long long>( u ) * n.B + b] = v;
+		}
+		__syncthreads();
+		float* swap = previous;
+		previous = current;
+		current = swap;
+	}
+
+	// backward: a sequence ends with its last label or with the blank behind it ( with the blank only where frames
+	// beyond its length follow: CpuMathEngineDnnCtc.cpp:350-376 )
+	__syncthreads();
+	{
+		int endA = U - 1, endB = U - 2;
+		if( labelLens != nullptr ) {
+			endA = 2 * labelLens[b];
+			endB = endA - 1 + ( ( resultLens != nullptr && resultLens[b] < n.T ) ? 1 : 0 );
+		}
+		for( int u = threadIdx.x; u < U; u += 256 ) {
+			const float v = ( u == endA || u == endB ) ? 0.f : CtcLogZero;
+			previous[u] = v;
+			logBeta[( n.T - 1 ) * frame + static_cast<long long>( u ) * n.B + b] = v;
+		}
+	}
+	__syncthreads();
+	for( int t = n.T - 2; t >= 0; --t ) {
+		for( int u = threadIdx.x; u < U; u += 256 ) {
+			shifted[u] = previous[u] + ctcEmission( n, logProb, resultLens, t + 1, b, ctcPaddedLabel( n, labels, b, u ) );
+		}
+		__syncthreads();
+		for( int u = threadIdx.x; u < U; u += 256 ) {
+			float v = shifted[u];
+			if( u < U - 1 ) {
+				v = ctcLogSumExp( shifted[u], shifted[u + 1] );
+				if( n.SkipBlanks && u < U - 2 ) {
+					v = ctcLogSumExp( v, shifted[u + 2] + ctcSkipMask( n, labels, b, u ) );
+				}
+			}
+			current[u] = v;
+			logBeta[t * frame + static_cast<long long>( u ) * n.B + b] = v;
+		}
+		__syncthreads();
+		float* swap = previous;
+		previous = current;
+		current = swap;
+	}
+
+	// log-probability of the labelling: over the positions of frame 0
+	for( int u = threadIdx.x; u < U; u += 256 ) {
+		shifted[u] = logAlpha[static_cast<long long>( u ) * n.B + b] + logBeta[static_cast<long long>( u ) * n.B + b];
+	}
+	__syncthreads();
+	if( threadIdx.x == 0 ) {
+		total[b] = ctcLogSumExpOf( shifted, U );
+	}
+}
+
+// loss = - sum( weight * total ) / batch
+__global__ void ctcLossKernel( const float* total, const float* weights, int batch, float* loss )
+{
+	if( blockIdx.x == 0 && threadIdx.x == 0 ) {
+		float sum = 0.f;
+		for( int b = 0; b < batch; ++b ) {
+			sum += weights != nullptr ? weights[b] * total[b] : total[b];
+		}
+		*loss = -sum / batch;
+	}
+}
+
+// gradient by the network's result ( before its softmax ): prob - exp( logsumexp over the positions of class k of
+// ( logAlpha + logBeta ) - total ); one workgroup per ( frame, sequence )
+__global__ __launch_bounds__( 256 )
+void ctcGradientKernel( const CCtcShape n, const float* prob, const int* labels, const int* resultLens, const float* logAlpha,
+	const float* logBeta, const float* total, float* gradient )
+{
+	extern __shared__ float both[]; // [U] + 1
+	const int t = blockIdx.x / n.B;
+	const int b = blockIdx.x - t * n.B;
+	const long long frame = static_cast<long long>( n.U ) * n.B;
+	float* out = gradient + ( static_cast<long long>( t ) * n.B + b ) * n.C;
+	if( resultLens != nullptr && t >= resultLens[b] ) {
+		for( int k = threadIdx.x; k < n.C; k += 256 ) {
+			out[k] = 0.f;
+		}
+		return;
+	}
+	for( int u = threadIdx.x; u < n.U; u += 256 ) {
+		const long long at = t * frame + static_cast<long long>( u ) * n.B + b;
+		both[u] = logAlpha[at] + logBeta[at];
+	}
+	__syncthreads();
+	if( threadIdx.x == 0 ) {
+		// ( with skipped blanks the reference takes the total of the frame itself, for stability )
+		both[n.U] = n.SkipBlanks ? ctcLogSumExpOf( both, n.U ) : total[b];
+	}
+	__syncthreads();
+	const float all = both[n.U];
+	const float* p = prob + ( static_cast<long long>( t ) * n.B + b ) * n.C;
+	for( int k = threadIdx.x; k < n.C; k += 256 ) {
+		float sum = CtcLogZero;
+		for( int u = 0; u < n.U; ++u ) {
+			if( ctcPaddedLabel( n, labels, b, u ) == k ) {
+				const float f = both[u];
+				sum = f >= sum ? f + log1pf( expf( sum - f ) ) : sum + log1pf( expf( f - sum ) );
+			}
+		}
+		out[k] = p[k] - ctcExp( sum - all );
+	}
+}
+
 static bool valid3d( const nh3dDesc* d )
 {
 	return d != nullptr && d->batch >= 0 && d->height > 0 && d->width > 0 && d->depth > 0 && d->channels > 0
@@ -967,6 +1163,57 @@ int nhRleImagesToDense( nhStream s, const void* rle, int batch, int height, int 
 	hipLaunchKernelGGL( rleDecodeKernel, dim3( ( batch + 63 ) / 64 ), dim3( 64 ), 0, toStream( s ), static_cast<const int*>( rle ), batch,
 		height, width, strokeValue, nonStrokeValue, dense );
 	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+int nhCtcLossWorkspaceSize( int resultLen, int batchSize, int classCount, int labelLen, size_t* bytes )
+{
+	NH_REQUIRE( bytes != nullptr && resultLen >= 1 && batchSize >= 1 && classCount >= 1 && labelLen >= 1 );
+	const size_t frames = static_cast<size_t>( resultLen ) * batchSize;
+	const size_t padded = 2 * static_cast<size_t>( labelLen ) + 1;
+	*bytes = ( 2 * frames * classCount + 2 * frames * padded + batchSize ) * sizeof( float );
+	return NH_OK;
+}
+
+int nhCtcLossForward( nhStream s, int resultLen, int batchSize, int classCount, int labelLen, int blankLabel, int skipBlanks,
+	const float* result, const int* labels, const int* labelLens, const int* resultLens, const float* labelWeights, float* loss,
+	float* lossGradient, void* workspace, size_t workspaceBytes )
+{
+	size_t needed = 0;
+	const int rc = nhCtcLossWorkspaceSize( resultLen, batchSize, classCount, labelLen, &needed );
+	if( rc != NH_OK ) {
+		return rc;
+	}
+	NH_REQUIRE( result != nullptr && loss != nullptr && labels != nullptr );
+	NH_REQUIRE( blankLabel >= 0 && blankLabel < classCount );
+	NH_REQUIRE( workspace != nullptr && workspaceBytes >= needed );
+	const long long frames = static_cast<long long>( resultLen ) * batchSize;
+	NH_REQUIRE( frames * classCount <= 0x7fffffffLL );
+	CCtcShape n = { resultLen, batchSize, classCount, labelLen, 2 * labelLen + 1, blankLabel, skipBlanks ? 1 : 0 };
+	NH_REQUIRE( 3 * static_cast<size_t>( n.U ) * sizeof( float ) <= 60 * 1024 );
+	float* prob = static_cast<float*>( workspace );
+	float* logProb = prob + frames * classCount;
+	float* logAlpha = logProb + frames * classCount;
+	float* logBeta = logAlpha + frames * n.U;
+	float* total = logBeta + frames * n.U;
+	int step = nhMatrixSoftmaxByRows( s, result, static_cast<int>( frames ), classCount, prob );
+	if( step != NH_OK ) {
+		return step;
+	}
+	step = nhVectorLog( s, prob, logProb, static_cast<int>( frames * classCount ) );
+	if( step != NH_OK ) {
+		return step;
+	}
+	hipLaunchKernelGGL( ctcLatticeKernel, dim3( batchSize ), dim3( 256 ), 3 * n.U * sizeof( float ), toStream( s ), n, logProb, labels,
+		labelLens, resultLens, logAlpha, logBeta, total );
+	NH_LAUNCH_CHECK();
+	hipLaunchKernelGGL( ctcLossKernel, dim3( 1 ), dim3( 64 ), 0, toStream( s ), total, labelWeights, batchSize, loss );
+	NH_LAUNCH_CHECK();
+	if( lossGradient != nullptr ) {
+		hipLaunchKernelGGL( ctcGradientKernel, dim3( static_cast<unsigned>( frames ) ), dim3( 256 ), ( n.U + 1 ) * sizeof( float ), toStream( s ), n,
+			prob, labels, resultLens, logAlpha, logBeta, total, lossGradient );
+		NH_LAUNCH_CHECK();
+	}
 	return NH_OK;
 }
 

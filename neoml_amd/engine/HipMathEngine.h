@@ -513,6 +513,7 @@ public:
 	CRleConvolutionDesc* InitBlobRleConvolution( const CBlobDesc& input, float strokeValue, float nonStrokeValue, int strideHeight, int strideWidth, const CBlobDesc& filter, const CBlobDesc& output ) override;
 	void BlobRleConvolution( const CRleConvolutionDesc& desc, const CConstFloatHandle& source, const CConstFloatHandle& filter, const CConstFloatHandle* freeTerm, const CFloatHandle& result ) override;
 	void BlobRleConvolutionLearnAdd( const CRleConvolutionDesc& desc, const CConstFloatHandle& input, const CConstFloatHandle& outputDiff, const CFloatHandle& filterDiff, const CFloatHandle* freeTermDiff ) override;
+	void CtcLossForward( int resultLen, int batchSize, int classCount, int labelLen, int blankLabel, bool skipBlanks, const CConstFloatHandle& result, const CConstIntHandle& labels, const CConstIntHandle& labelLens, const CConstIntHandle& resultLens, const CConstFloatHandle& labelWeights, const CFloatHandle& loss, const CFloatHandle& lossGradient ) override;
 	// ---- end of the members beyond the inference path ----
 
 	// every other pure virtual of the interface: asserting bodies generated from the interface header

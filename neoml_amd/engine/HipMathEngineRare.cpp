@@ -168,6 +168,19 @@ void CHipMathEngine::VectorTopKDiff( const CConstFloatHandle& sourceGrad, int so
 	NH_CALL( nhVectorTopKDiff( stream, raw( sourceGrad ), sourceGradHeight, sourceGradWidth, raw( indices ), k, raw( resultGrad ) ) );
 }
 
+void CHipMathEngine::CtcLossForward( int resultLen, int batchSize, int classCount, int labelLen, int blankLabel, bool skipBlanks,
+	const CConstFloatHandle& result, const CConstIntHandle& labels, const CConstIntHandle& labelLens, const CConstIntHandle& resultLens,
+	const CConstFloatHandle& labelWeights, const CFloatHandle& loss, const CFloatHandle& lossGradient )
+{
+	size_t workspaceSize = 0;
+	NH_CALL( nhCtcLossWorkspaceSize( resultLen, batchSize, classCount, labelLen, &workspaceSize ) );
+	const CMemoryHandle workspace = StackAlloc( workspaceSize );
+	NH_CALL( nhCtcLossForward( stream, resultLen, batchSize, classCount, labelLen, blankLabel, skipBlanks ? 1 : 0, raw( result ),
+		OPTIONAL( labels ), OPTIONAL( labelLens ), OPTIONAL( resultLens ), OPTIONAL( labelWeights ), raw( loss ), OPTIONAL( lossGradient ),
+		rawBytes( workspace ), workspaceSize ) );
+	StackFree( workspace );
+}
+
 // ---- 3-D convolution and pooling ---------------------------------------------------------------------------------
 
 struct CHip3dConvolutionDesc : public C3dConvolutionDesc {

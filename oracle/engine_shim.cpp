@@ -1003,6 +1003,39 @@ SHIM_API int shim_singular_value_decomposition( void* engine, const float* matri
 	} );
 }
 
+// IMathEngine::CtcLossForward; label_lens, result_lens, weights and gradient may be null
+SHIM_API int shim_ctc_loss_forward( void* engine, int result_len, int batch, int classes, int label_len, int blank, int skip_blanks,
+	const float* result, const int* labels, const int* label_lens, const int* result_lens, const float* weights, float* loss,
+	float* gradient )
+{
+	return guarded( [&]() {
+		IMathEngine& e = *static_cast<IMathEngine*>( engine );
+		const int frames = result_len * batch * classes;
+		CFloatBlob in( e, frames, result ), lossOut( e, 1 ), grad( e, frames ), w( e, batch );
+		CIntHandleVar lab( e, label_len * batch + 1 ), labLens( e, batch ), resLens( e, batch );
+		if( label_len > 0 ) {
+			e.DataExchangeTyped<int>( lab.GetHandle(), labels, label_len * batch );
+		}
+		if( label_lens != nullptr ) {
+			e.DataExchangeTyped<int>( labLens.GetHandle(), label_lens, batch );
+		}
+		if( result_lens != nullptr ) {
+			e.DataExchangeTyped<int>( resLens.GetHandle(), result_lens, batch );
+		}
+		if( weights != nullptr ) {
+			e.DataExchangeTyped<float>( w.Handle(), weights, batch );
+		}
+		e.CtcLossForward( result_len, batch, classes, label_len, blank, skip_blanks != 0, in.Const(), lab.GetHandle(),
+			label_lens != nullptr ? CConstIntHandle( labLens.GetHandle() ) : CConstIntHandle(),
+			result_lens != nullptr ? CConstIntHandle( resLens.GetHandle() ) : CConstIntHandle(),
+			weights != nullptr ? w.Const() : CConstFloatHandle(), lossOut.Handle(), gradient != nullptr ? grad.Handle() : CFloatHandle() );
+		lossOut.CopyTo( loss );
+		if( gradient != nullptr ) {
+			grad.CopyTo( gradient );
+		}
+	} );
+}
+
 SHIM_API int shim_vector_top_k( void* engine, const float* first, int n, int k, float* result, int* indices )
 {
 	return guarded( [&]() {
