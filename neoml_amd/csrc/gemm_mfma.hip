@@ -1197,8 +1197,8 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 				splits = s;
 			}
 		}
-	// K slices cannot add a residual
-	} else if( blocks < 1024 && totalSteps >= 32 && args.Residual == nullptr ) {
+	// ( with a residual only slices that meet in scratch memory will do, see below )
+	} else if( blocks < 1024 && totalSteps >= 32 && ( args.Residual == nullptr || ( batch == 1 && AMODE != AM_ConvClasses && BM * BN == 4096 ) ) ) {
 		double best = 0;
 		for( int s = 1; s <= 8 && s <= totalSteps / 8; ++s ) {
 			const double cost = launchCost( s );
@@ -1289,6 +1289,12 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 		}
 	}
 	const bool meetInScratch = args.Partials != nullptr;
+	if( args.Residual != nullptr && args.SplitK > 1 && !meetInScratch ) {
+		// The residual is added by the one workgroup that writes a tile, which is the last slice to arrive at the meeting;
+		// slices that add onto C with atomics have no such workgroup. No scratch ( a capturing stream ): one slice.
+		args.StepsPerSplit = totalSteps;
+		args.SplitK = 1;
+	}
 	// the rows of the tail tiles as a matrix product of their own: what the preset and the activation pass cover
 	CMatMulArgs tail = args;
 	tail.C += static_cast<long long>( tailRow ) * args.Ldc;

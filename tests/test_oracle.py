@@ -506,6 +506,9 @@ SEPARABLE_CASES = [
     (2, 7, 7, 12, 20, 12, 1, True, ("hswish", 0.0), (None, 0.0)),
     (1, 5, 6, 3, 5, 7, 2, False, (None, 0.0), ("relu", 2.5)),       # channel counts not a multiple of 4
     (3, 8, 8, 24, 144, 32, 1, False, ("relu", 6.0), ("relu", 6.0)),
+    # few pixels, long reductions, a residual: the down convolution's reduction is cut into slices whose last one adds the input
+    (2, 7, 7, 160, 960, 160, 1, True, ("relu", 6.0), ("relu", 6.0)),
+    (1, 14, 14, 96, 576, 96, 1, True, ("relu", 6.0), ("relu", 6.0)),
 ]
 
 
