@@ -18,6 +18,10 @@ inline hipStream_t toStream( nhStream s ) { return reinterpret_cast<hipStream_t>
 // must have been drained. unbind: the stream is going away, its binding to a pool goes with the blocks.
 void releaseSliceScratch( hipStream_t stream, bool unbind );
 
+// Scratch of the stream for reductions that meet inside a launch ( gemm_mfma.hip ): `partialFloats` floats and one arrival
+// counter that is zero between launches and must be left at zero. false: none to be had, take another way.
+bool streamMeetingPlace( hipStream_t stream, size_t partialFloats, float** partials, unsigned** counter );
+
 constexpr int WaveSize = 64;
 
 inline int ceilDiv( long long a, long long b ) { return static_cast<int>( ( a + b - 1 ) / b ); }

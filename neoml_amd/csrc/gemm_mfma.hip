@@ -1063,6 +1063,19 @@ static bool sliceScratch( hipStream_t stream, size_t partialFloats, size_t count
 	return true;
 }
 
+// The same block for other reductions that meet inside a launch ( vector sums ): partial results and one arrival counter,
+// which every user leaves at zero. false: none to be had ( a capturing stream, a shared stream handle, no memory ).
+bool streamMeetingPlace( hipStream_t stream, size_t partialFloats, float** partials, unsigned** counter )
+{
+	CSliceScratch scratch;
+	if( !sliceScratch( stream, partialFloats, 1, scratch ) ) {
+		return false;
+	}
+	*partials = scratch.Partials;
+	*counter = scratch.Counters;
+	return true;
+}
+
 // A meeting place handed in by the caller instead of the stream's block: the launch neither allocates nor looks the
 // stream up, and fails when the place is too small.
 struct CSliceMeeting {

@@ -426,14 +426,21 @@ struct CTanhDiffOp : CNoScalar {
 };
 struct CTanhDiffOutOp : CNoScalar { __device__ float operator()( float y, float b, float ) const { return ( 1.f - y * y ) * b; } };
 
-// ---- reductions to one value: one workgroup per 16K elements, atomics into a zeroed result -----------------
+// ---- reductions to one value: one workgroup per 16K elements ------------------------------------------------------
+// The workgroups meet in the stream's scratch: each leaves its partial sum there and draws a ticket; the one that draws
+// the last ticket adds the partial sums up in a fixed order and only then touches the result ( stores, or adds onto it ).
+// So the value does not depend on the order in which the workgroups finish, and a result that lies inside an operand
+// is read before it is written, as on the CPU engine. Without scratch ( a capturing stream ): atomic adds onto a
+// result that a launch in front has set to zero.
 
 // VEC: 128-bit loads, four of them in flight per thread and operand (both pointers 16-byte aligned); the up to three
 // elements behind the last whole vector are added by the first thread.
 template<bool DOT, bool VEC>
-__global__ __launch_bounds__( 256 ) void sumKernel( const float* a, const float* b, int n, float* result )
+__global__ __launch_bounds__( 256 ) void sumKernel( const float* a, const float* b, int n, float* result, float* partials,
+	unsigned* counter, int addToResult )
 {
 	__shared__ float part[4];
+	__shared__ unsigned ticket;
 	float s = 0.f;
 	const int stride = gridDim.x * 256;
 	const int start = blockIdx.x * 256 + threadIdx.x;
@@ -483,25 +490,70 @@ __global__ __launch_bounds__( 256 ) void sumKernel( const float* a, const float*
 		part[threadIdx.x >> 6] = s;
 	}
 	__syncthreads();
+	const float mine = part[0] + part[1] + part[2] + part[3];
+	if( partials == nullptr ) {
+		if( threadIdx.x == 0 ) {
+			atomicAdd( result, mine );
+		}
+		return;
+	}
+	if( gridDim.x == 1 ) {
+		if( threadIdx.x == 0 ) {
+			*result = addToResult ? *result + mine : mine;
+		}
+		return;
+	}
+	// ( values cross between workgroups through device-scope accesses, past the L2 of the XCD they run on )
 	if( threadIdx.x == 0 ) {
-		atomicAdd( result, part[0] + part[1] + part[2] + part[3] );
+		__hip_atomic_store( reinterpret_cast<unsigned*>( partials ) + blockIdx.x, __float_as_uint( mine ), __ATOMIC_RELAXED,
+			__HIP_MEMORY_SCOPE_AGENT );
+		__builtin_amdgcn_s_waitcnt( 0x0F70 ); // vmcnt( 0 ): the store has been acknowledged
+		ticket = __hip_atomic_fetch_add( counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT );
+	}
+	__syncthreads();
+	if( ticket != gridDim.x - 1 || threadIdx.x >= 64 ) {
+		return;
+	}
+	float total = 0.f;
+	for( unsigned i = threadIdx.x; i < gridDim.x; i += 64 ) {
+		total += __uint_as_float( __hip_atomic_load( reinterpret_cast<unsigned*>( partials ) + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT ) );
+	}
+	total = waveReduceSum( total );
+	if( threadIdx.x == 0 ) {
+		*result = addToResult ? *result + total : total;
+		__hip_atomic_store( counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT );
 	}
 }
 
 template<bool DOT>
 static int launchSum( nhStream s, const float* first, const float* second, int vectorSize, float* result, bool addToResult = false )
 {
-	int rc = addToResult ? NH_OK : nhVectorFill( s, result, 0.f, 1 );
-	if( rc != NH_OK || vectorSize == 0 ) {
-		return rc;
+	if( vectorSize == 0 ) {
+		return addToResult ? NH_OK : nhVectorFill( s, result, 0.f, 1 );
 	}
-	NH_REQUIRE( first != nullptr && ( !DOT || second != nullptr ) );
+	NH_REQUIRE( first != nullptr && ( !DOT || second != nullptr ) && result != nullptr );
 	int blocks = ceilDiv( vectorSize, 16384 );
 	blocks = blocks > 2048 ? 2048 : blocks;
+	float* partials = nullptr;
+	unsigned* counter = nullptr;
+	if( !streamMeetingPlace( toStream( s ), 2048, &partials, &counter ) ) {
+		partials = nullptr;
+		if( blocks == 1 ) {
+			partials = result; // ( not used by a single workgroup: only says that it may write the result itself )
+		} else if( !addToResult ) {
+			const int rc = nhVectorFill( s, result, 0.f, 1 );
+			if( rc != NH_OK ) {
+				return rc;
+			}
+		}
+	}
+	const int add = addToResult ? 1 : 0;
 	if( isAligned16( first ) && ( !DOT || isAligned16( second ) ) ) {
-		hipLaunchKernelGGL( ( sumKernel<DOT, true> ), dim3( blocks ), dim3( 256 ), 0, toStream( s ), first, second, vectorSize, result );
+		hipLaunchKernelGGL( ( sumKernel<DOT, true> ), dim3( blocks ), dim3( 256 ), 0, toStream( s ), first, second, vectorSize, result, partials,
+			counter, add );
 	} else {
-		hipLaunchKernelGGL( ( sumKernel<DOT, false> ), dim3( blocks ), dim3( 256 ), 0, toStream( s ), first, second, vectorSize, result );
+		hipLaunchKernelGGL( ( sumKernel<DOT, false> ), dim3( blocks ), dim3( 256 ), 0, toStream( s ), first, second, vectorSize, result, partials,
+			counter, add );
 	}
 	NH_LAUNCH_CHECK();
 	return NH_OK;

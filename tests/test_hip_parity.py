@@ -652,6 +652,43 @@ def test_stream_destroy_frees_the_slices_scratch():
     assert_close(first[:1], orc.conv(x[:1].cpu().numpy(), f.cpu().numpy(), None, 1, 1, 1, 1), "vs oracle")
 
 
+def test_vector_sum_is_reproducible_and_may_write_into_its_operand():
+    """Sums over many workgroups: the same bits on every run (the partial sums are added in a fixed order), and a result
+    that lies inside the operand is read before it is written (the CPU engine computes first and stores last)."""
+    import ctypes
+    import torch
+    import neoml_amd
+    lib = neoml_amd.load()
+    g = rng(123)
+    n = 5_000_011
+    host = g.normal(0, 1, n).astype(np.float32)
+    dev = torch.device("cuda:0")
+    x = torch.from_numpy(host).to(dev)
+    y = torch.from_numpy(g.normal(0, 1, n).astype(np.float32)).to(dev)
+    out = torch.zeros(4, device=dev)
+    P = lambda t, offset=0: ctypes.c_void_p(t.data_ptr() + 4 * offset)
+    runs = []
+    for _ in range(5):
+        neoml_amd.check(lib.nhVectorSum(None, P(x), n, P(out)))
+        neoml_amd.check(lib.nhVectorDotProduct(None, P(x), P(y), n, P(out, 1)))
+        torch.cuda.synchronize()
+        runs.append(out[:2].cpu().numpy().copy())
+    assert all(np.array_equal(r, runs[0]) for r in runs[1:]), runs
+    assert abs(runs[0][0] - host.astype(np.float64).sum()) < 1.0
+    # the result in the middle of the operand
+    want = float(host.astype(np.float64).sum())
+    neoml_amd.check(lib.nhVectorSum(None, P(x), n, P(x, 2_500_000)))
+    torch.cuda.synchronize()
+    got = float(x[2_500_000].item())
+    assert abs(got - want) < 1.0 and got == float(runs[0][0]), (got, want, runs[0][0])
+    # adding onto a value
+    out[2] = 10.0
+    neoml_amd.check(lib.nhVectorSumAdd(None, P(y), n, P(out, 2)))
+    neoml_amd.check(lib.nhVectorSum(None, P(y), n, P(out, 3)))
+    torch.cuda.synchronize()
+    assert abs(float(out[2].item()) - 10.0 - float(out[3].item())) < 1e-3 * max(1.0, abs(float(out[3].item())))
+
+
 def test_convolution_ignores_pixels_outside_the_windows():
     # stride 4 with a 3-wide filter never touches image columns 3 and 7; whatever they hold (here: infinities)
     # must not leak into the result through the vector fetches that run past a window's last value
