@@ -423,6 +423,13 @@ NH_API int nhBlobMaxPoolingBackward(nhStream s, const nhPoolingDesc* desc_host, 
 NH_API int nhBlobMeanPoolingBackward(nhStream s, const nhPoolingDesc* desc_host, const float* resultDiff,
 	float* sourceDiff);                                                                              /* NME.h:842 */
 
+/* Two one-launch LSTMs side by side. No counterpart in the reference: its bidirectional layers are two CLstmLayer calls in
+ * stream order. On a stream that has asked for it (enable != 0) a whole-sequence nhLstm launch takes at most half of the
+ * compute units, and an nhLstm that follows it directly (nothing else enqueued on the stream through this library in
+ * between) and touches none of its inputs, results or workspace runs beside it on a stream of the library's own; the
+ * caller's stream waits for it right there, so work enqueued later is ordered behind both. Only for streams whose work
+ * all goes through this library (an engine's own stream). Results are those of the calls in order. */
+NH_API int nhStreamOverlapLstm(nhStream s, int enable);
 /* LSTM (NME.h:1005-1011). Weights: inputWeights [4H x objectSize], recurrentWeights [4H x H]; gate order in
  * the 4H vector: main(tanh) | forget | input | output (src/CPU/CpuMathEngineDnnLstm.h:49-90).
  * Free terms, inputStateBackLink, inputMainBackLink and outputStateBackLink may be null.

@@ -12,7 +12,20 @@ namespace nh {
 // Stores the message returned by nhGetLastError() for the calling thread.
 void setLastError( const char* fmt, ... );
 
-inline hipStream_t toStream( nhStream s ) { return reinterpret_cast<hipStream_t>( s ); }
+// Streams on which two one-launch LSTMs that do not depend on each other may run side by side ( nhStreamOverlapLstm,
+// dnn_ops.hip ) need to know whether anything was enqueued between two nhLstm calls: every entry point turns its stream
+// handle into a stream here, so here is where that is noted. Costs one relaxed load while no stream has asked for it.
+extern int overlapLstmStreams;
+void noteStreamUse( hipStream_t stream );
+
+inline hipStream_t toStream( nhStream s )
+{
+	const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
+	if( __atomic_load_n( &overlapLstmStreams, __ATOMIC_RELAXED ) != 0 ) {
+		noteStreamUse( stream );
+	}
+	return stream;
+}
 
 // Frees the scratch blocks that sliced reductions keep for a stream of the current device ( gemm_mfma.hip ); the stream
 // must have been drained. unbind: the stream is going away, its binding to a pool goes with the blocks.

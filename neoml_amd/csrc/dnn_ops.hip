@@ -1459,6 +1459,31 @@ struct CSequenceDevice {
 	hipEvent_t LastDone = nullptr;
 	hipStream_t LastStream = nullptr;
 	bool Any = false;
+	// the one before the last: what the partner of an overlapped pair waits for instead of its own partner
+	hipEvent_t OlderDone = nullptr;
+	bool AnyOlder = false;
+};
+
+// Two one-launch LSTMs side by side ( nhStreamOverlapLstm ): the two directions of a bidirectional layer read the same
+// input and write different outputs, arrive as two nhLstm calls one behind the other, and each keeps its cell state for
+// itself; in stream order the second waits for the first and the device is half idle. On a stream that has asked for it
+// a one-launch LSTM takes a grid of at most half the compute units, and a second nhLstm that follows it directly ( nothing
+// else was enqueued through this library in between ) and touches none of its memory runs on a side stream: the side
+// stream waits for what was in front of the first, the main stream waits for the side stream right behind the first, so
+// whatever is enqueued later, through this library or not, is ordered behind both.
+struct CByteRange {
+	const char* Lo = nullptr;
+	const char* Hi = nullptr;
+};
+
+struct CLstmOverlap {
+	bool Enabled = false;
+	hipStream_t Side = nullptr;
+	hipEvent_t Before = nullptr;   // recorded on the main stream in front of a one-launch LSTM
+	hipEvent_t SideDone = nullptr; // recorded on the side stream behind its LSTM
+	bool LastWasLstm = false;      // that LSTM was the last thing enqueued on the main stream
+	CByteRange Written[3];         // what it writes: results, workspace
+	CByteRange Read[4];            // what it reads: input, initial states ( the weights are constant )
 };
 
 static std::mutex sequenceLock;
@@ -1472,6 +1497,33 @@ static std::map<int, CSequenceDevice>& sequenceDevices()
 	static std::map<int, CSequenceDevice> devices;
 	return devices;
 }
+static std::map<std::pair<int, hipStream_t>, CLstmOverlap>& lstmOverlaps()
+{
+	static std::map<std::pair<int, hipStream_t>, CLstmOverlap> overlaps;
+	return overlaps;
+}
+
+int overlapLstmStreams = 0;
+
+// something is being enqueued on `stream` through this library: a one-launch LSTM on it has no partner any more
+void noteStreamUse( hipStream_t stream )
+{
+	int device = 0;
+	if( hipGetDevice( &device ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return;
+	}
+	std::lock_guard<std::mutex> guard( sequenceLock );
+	auto found = lstmOverlaps().find( std::make_pair( device, stream ) );
+	if( found != lstmOverlaps().end() ) {
+		found->second.LastWasLstm = false;
+	}
+}
+
+static bool rangesMeet( const CByteRange& a, const CByteRange& b )
+{
+	return a.Lo != nullptr && b.Lo != nullptr && a.Lo < b.Hi && b.Lo < a.Hi;
+}
 
 // Called by the synchronising entry points once `stream` has drained: a one-launch LSTM of this stream whose bounded
 // wait tripped has produced garbage, and that must not pass silently.
@@ -1484,16 +1536,31 @@ int checkSequenceGiveUps( hipStream_t stream )
 	}
 	std::lock_guard<std::mutex> guard( sequenceLock );
 	auto& streams = sequenceStreams();
-	auto found = streams.find( std::make_pair( device, stream ) );
-	if( found == streams.end() || !found->second.Launched ) {
+	bool gaveUp = false;
+	// the stream's own launches, and those of its side stream ( the main stream has waited for them )
+	hipStream_t both[2] = { stream, nullptr };
+	auto overlap = lstmOverlaps().find( std::make_pair( device, stream ) );
+	if( overlap != lstmOverlaps().end() ) {
+		both[1] = overlap->second.Side;
+	}
+	for( int i = 0; i < 2; ++i ) {
+		if( i == 1 && both[1] == nullptr ) {
+			break;
+		}
+		auto found = streams.find( std::make_pair( device, both[i] ) );
+		if( found == streams.end() || !found->second.Launched ) {
+			continue;
+		}
+		found->second.Launched = false;
+		volatile unsigned* word = found->second.GaveUp;
+		if( *word != 0 ) {
+			*word = 0;
+			gaveUp = true;
+		}
+	}
+	if( !gaveUp ) {
 		return NH_OK;
 	}
-	found->second.Launched = false;
-	volatile unsigned* word = found->second.GaveUp;
-	if( *word == 0 ) {
-		return NH_OK;
-	}
-	*word = 0;
 	setLastError( "nhLstm: a one-launch LSTM on this stream gave up waiting for the previous step (its grid was not "
 		"resident as a whole, or the spin limit is too low): its output is invalid" );
 	return NH_ERR_HIP;
@@ -1517,6 +1584,26 @@ void releaseSequenceStream( hipStream_t stream )
 	auto dev = sequenceDevices().find( device );
 	if( dev != sequenceDevices().end() && dev->second.LastStream == stream ) {
 		dev->second.Any = false; // drained: nothing of it is in flight
+		dev->second.AnyOlder = false;
+	}
+	auto overlap = lstmOverlaps().find( std::make_pair( device, stream ) );
+	if( overlap != lstmOverlaps().end() ) {
+		CLstmOverlap& o = overlap->second;
+		if( o.Side != nullptr ) {
+			auto side = streams.find( std::make_pair( device, o.Side ) );
+			if( side != streams.end() ) {
+				( void )hipHostFree( side->second.GaveUp );
+				streams.erase( side );
+			}
+			releaseSliceScratch( o.Side, true );
+			( void )hipStreamDestroy( o.Side );
+			( void )hipEventDestroy( o.Before );
+			( void )hipEventDestroy( o.SideDone );
+		}
+		if( o.Enabled ) {
+			__atomic_fetch_sub( &overlapLstmStreams, 1, __ATOMIC_RELAXED );
+		}
+		lstmOverlaps().erase( overlap );
 	}
 }
 
@@ -1552,7 +1639,7 @@ static size_t lstmSequenceLds( int H, const CLstmSeqShape& shape )
 }
 
 // The first shape whose grid fits the device; null = none does.
-static const CLstmSeqShape* lstmSequenceShape( int H, int B )
+static const CLstmSeqShape* lstmSequenceShape( int H, int B, bool halfDevice = false )
 {
 	static int computeUnits = 0; // the engine drives one device per process
 	static bool ldsRaised = false;
@@ -1596,11 +1683,12 @@ static const CLstmSeqShape* lstmSequenceShape( int H, int B )
 		// one workgroup per compute unit is what the dispatcher certainly places side by side on an otherwise idle
 		// device; the occupancy figure only confirms that one fits
 		const long long groups = static_cast<long long>( H / ( SeqUnits * shape.Blocks ) ) * ceilDiv( B, shape.Rows );
-		if( perUnit >= 1 && groups <= computeUnits ) {
+		if( perUnit >= 1 && groups <= ( halfDevice ? computeUnits / 2 : computeUnits ) ) {
 			return &shape;
 		}
 	}
-	return nullptr;
+	// ( no shape of half the device: the whole one, and no partner beside it )
+	return halfDevice ? lstmSequenceShape( H, B, false ) : nullptr;
 }
 
 static bool lstmSequenceFits( int H, int B, const float* wRec, const float* c0, const float* h0, const float* hOut )
@@ -1634,12 +1722,22 @@ static bool lstmSequenceAllowed( hipStream_t stream )
 	return capture == hipStreamCaptureStatusNone;
 }
 
-static int launchLstmSequence( hipStream_t stream, CLstmSeqArgs a )
+// halfDevice: a grid of at most half the compute units if there is such a shape ( *tookHalf says whether ).
+// partner: this launch runs beside the one issued last ( its partner, on the main stream ) instead of behind it.
+static int launchLstmSequence( hipStream_t stream, CLstmSeqArgs a, bool halfDevice = false, bool partner = false, bool* tookHalf = nullptr )
 {
-	const CLstmSeqShape* shape = lstmSequenceShape( a.H, a.B );
+	const CLstmSeqShape* shape = lstmSequenceShape( a.H, a.B, halfDevice );
 	NH_REQUIRE( shape != nullptr );
 	int device = 0;
 	NH_HIP( hipGetDevice( &device ) );
+	int computeUnits = 0;
+	NH_HIP( hipDeviceGetAttribute( &computeUnits, hipDeviceAttributeMultiprocessorCount, device ) );
+	const long long shapeGroups = static_cast<long long>( a.H / ( SeqUnits * shape->Blocks ) ) * ceilDiv( a.B, shape->Rows );
+	const bool isHalf = shapeGroups <= computeUnits / 2;
+	if( tookHalf != nullptr ) {
+		*tookHalf = isHalf;
+	}
+	NH_REQUIRE( !partner || isHalf );
 	std::lock_guard<std::mutex> guard( sequenceLock );
 	CSequenceStream& own = sequenceStreams()[std::make_pair( device, stream )];
 	if( own.GaveUp == nullptr ) {
@@ -1651,8 +1749,14 @@ static int launchLstmSequence( hipStream_t stream, CLstmSeqArgs a )
 	CSequenceDevice& dev = sequenceDevices()[device];
 	if( dev.LastDone == nullptr ) {
 		NH_HIP( hipEventCreateWithFlags( &dev.LastDone, hipEventDisableTiming ) );
+		NH_HIP( hipEventCreateWithFlags( &dev.OlderDone, hipEventDisableTiming ) );
 	}
-	if( dev.Any ) {
+	if( partner ) {
+		// beside the one issued last, behind the one in front of that
+		if( dev.AnyOlder ) {
+			NH_HIP( hipStreamWaitEvent( stream, dev.OlderDone, 0 ) );
+		}
+	} else if( dev.Any ) {
 		// behind the one-launch LSTM issued last, whichever stream it went to ( on the same stream the wait is free )
 		NH_HIP( hipStreamWaitEvent( stream, dev.LastDone, 0 ) );
 	}
@@ -1664,8 +1768,26 @@ static int launchLstmSequence( hipStream_t stream, CLstmSeqArgs a )
 	hipLaunchKernelGGL( clearWordsKernel, dim3( static_cast<unsigned>( ( words + 1023 ) / 1024 ) ), dim3( 256 ), 0, stream, a.Exchange, words );
 	shape->Launch( stream, groups, lstmSequenceLds( a.H, *shape ), a );
 	NH_LAUNCH_CHECK();
-	NH_HIP( hipEventRecord( dev.LastDone, stream ) );
-	dev.LastStream = stream;
+	if( !partner ) {
+		// ( a partner's completion is recorded by its caller, on the main stream, once that stream waits for both )
+		std::swap( dev.LastDone, dev.OlderDone );
+		dev.AnyOlder = dev.Any;
+		NH_HIP( hipEventRecord( dev.LastDone, stream ) );
+		dev.LastStream = stream;
+		dev.Any = true;
+	}
+	return NH_OK;
+}
+
+// both LSTMs of a pair are behind the main stream's last wait: later one-launch LSTMs wait for this point
+static int recordPairDone( hipStream_t mainStream )
+{
+	int device = 0;
+	NH_HIP( hipGetDevice( &device ) );
+	std::lock_guard<std::mutex> guard( sequenceLock );
+	CSequenceDevice& dev = sequenceDevices()[device];
+	NH_HIP( hipEventRecord( dev.LastDone, mainStream ) );
+	dev.LastStream = mainStream;
 	dev.Any = true;
 	return NH_OK;
 }
@@ -2233,6 +2355,30 @@ int nhBlobSplitByDim( nhStream s, int dim, const nhBlobDesc* from, const float* 
 	return splitMergeImpl<false>( s, dim, *from, const_cast<float*>( fromData ), to, toData, toCount );
 }
 
+int nhStreamOverlapLstm( nhStream s, int enable )
+{
+	const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
+	int device = 0;
+	NH_HIP( hipGetDevice( &device ) );
+	std::lock_guard<std::mutex> guard( sequenceLock );
+	CLstmOverlap& o = lstmOverlaps()[std::make_pair( device, stream )];
+	if( enable != 0 && o.Side == nullptr ) {
+		NH_HIP( hipStreamCreateWithFlags( &o.Side, hipStreamNonBlocking ) );
+		NH_HIP( hipEventCreateWithFlags( &o.Before, hipEventDisableTiming ) );
+		NH_HIP( hipEventCreateWithFlags( &o.SideDone, hipEventDisableTiming ) );
+	}
+	if( ( enable != 0 ) != o.Enabled ) {
+		if( enable != 0 ) {
+			__atomic_fetch_add( &overlapLstmStreams, 1, __ATOMIC_RELAXED );
+		} else {
+			__atomic_fetch_sub( &overlapLstmStreams, 1, __ATOMIC_RELAXED );
+		}
+		o.Enabled = enable != 0;
+	}
+	o.LastWasLstm = false;
+	return NH_OK;
+}
+
 // workspace layout: [ gates: T*B*4H ][ free term: 4H ][ state: B*H ][ tagged h exchange: 2*B*H 64-bit words ][ abort word: 64 bits ]
 int nhLstmWorkspaceSize( int hiddenSize, int objectSize, int sequenceLength, int sequenceCount, size_t* bytes )
 {
@@ -2258,10 +2404,68 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 		return NH_OK;
 	}
 	NH_REQUIRE( static_cast<long long>( sequenceLength ) * sequenceCount * 4 * hiddenSize <= 0x7fffffffLL );
-	hipStream_t stream = toStream( s );
 	const int H = hiddenSize;
 	const int B = sequenceCount;
 	const int T = sequenceLength;
+	// ( not through toStream: whether something was enqueued since the last nhLstm is what is asked here )
+	const hipStream_t mainStream = reinterpret_cast<hipStream_t>( s );
+	hipStream_t stream = mainStream;
+	const bool sequencePath = T > 1 && lstmSequenceFits( H, B, recurrentWeights, inputStateBackLink, inputMainBackLink, outputMainBackLink )
+		&& lstmSequenceAllowed( mainStream );
+	// what this call writes and reads
+	CByteRange written[3], read[4];
+	{
+		const size_t stateBytes = static_cast<size_t>( T ) * B * H * sizeof( float );
+		const size_t oneState = static_cast<size_t>( B ) * H * sizeof( float );
+		auto range = []( const void* p, size_t bytes ) {
+			CByteRange r;
+			if( p != nullptr ) {
+				r.Lo = static_cast<const char*>( p );
+				r.Hi = r.Lo + bytes;
+			}
+			return r;
+		};
+		written[0] = range( outputMainBackLink, stateBytes );
+		written[1] = range( outputStateBackLink, stateBytes );
+		written[2] = range( workspace, need );
+		read[0] = range( input, static_cast<size_t>( T ) * B * objectSize * sizeof( float ) );
+		read[1] = range( inputMainBackLink, oneState );
+		read[2] = range( inputStateBackLink, oneState );
+	}
+	bool overlapEnabled = false;
+	bool beside = false; // this call runs on the side stream, beside the one-launch LSTM issued just before
+	CLstmOverlap pair;
+	if( __atomic_load_n( &overlapLstmStreams, __ATOMIC_RELAXED ) != 0 ) {
+		int device = 0;
+		NH_HIP( hipGetDevice( &device ) );
+		std::lock_guard<std::mutex> guard( sequenceLock );
+		auto found = lstmOverlaps().find( std::make_pair( device, mainStream ) );
+		if( found != lstmOverlaps().end() && found->second.Enabled ) {
+			CLstmOverlap& o = found->second;
+			overlapEnabled = true;
+			beside = o.LastWasLstm && sequencePath && lstmSequenceShape( H, B, true ) != nullptr;
+			if( beside ) {
+				const long long groups = static_cast<long long>( H / ( SeqUnits * lstmSequenceShape( H, B, true )->Blocks ) )
+					* ceilDiv( B, lstmSequenceShape( H, B, true )->Rows );
+				int units = 0;
+				beside = hipDeviceGetAttribute( &units, hipDeviceAttributeMultiprocessorCount, device ) == hipSuccess && groups <= units / 2;
+			}
+			for( int i = 0; beside && i < 3; ++i ) {
+				for( int j = 0; j < 3; ++j ) {
+					beside = beside && !rangesMeet( written[i], o.Written[j] ) && !rangesMeet( read[i], o.Written[j] )
+						&& !rangesMeet( written[i], o.Read[j] );
+				}
+			}
+			o.LastWasLstm = false;
+			pair = o;
+		}
+	}
+	if( beside ) {
+		stream = pair.Side;
+		NH_HIP( hipStreamWaitEvent( stream, pair.Before, 0 ) ); // everything in front of the partner
+	} else if( overlapEnabled && sequencePath ) {
+		NH_HIP( hipEventRecord( pair.Before, mainStream ) ); // in case a partner follows
+	}
 	float* gates = static_cast<float*>( workspace );
 	float* freeTerm = gates + static_cast<size_t>( T ) * B * 4 * H;
 	float* stateScratch = freeTerm + 4 * H;
@@ -2280,9 +2484,7 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 		return rc;
 	}
 	const int stepSize = B * H;
-	if( T > 1 && lstmSequenceFits( H, B, recurrentWeights, inputStateBackLink, inputMainBackLink, outputMainBackLink )
-		&& lstmSequenceAllowed( stream ) )
-	{
+	if( sequencePath ) {
 		CLstmSeqArgs a = {};
 		a.Gates = gates; a.Wrec = recurrentWeights; a.H0 = inputMainBackLink; a.C0 = inputStateBackLink;
 		a.HOut = outputMainBackLink; a.COut = outputStateBackLink;
@@ -2290,7 +2492,32 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 		a.Abort = reinterpret_cast<unsigned*>( a.Exchange + 2 * static_cast<size_t>( B ) * H );
 		a.T = T; a.B = B; a.H = H; a.Reverse = reverse ? 1 : 0;
 		a.MaxSpins = lstmSpinLimit();
-		return launchLstmSequence( stream, a );
+		bool tookHalf = false;
+		rc = launchLstmSequence( stream, a, overlapEnabled, beside, &tookHalf );
+		if( rc != NH_OK ) {
+			return rc;
+		}
+		if( beside ) {
+			// the main stream goes on behind both
+			NH_HIP( hipEventRecord( pair.SideDone, stream ) );
+			NH_HIP( hipStreamWaitEvent( mainStream, pair.SideDone, 0 ) );
+			return recordPairDone( mainStream );
+		}
+		if( overlapEnabled && tookHalf ) {
+			int device = 0;
+			NH_HIP( hipGetDevice( &device ) );
+			std::lock_guard<std::mutex> guard( sequenceLock );
+			auto found = lstmOverlaps().find( std::make_pair( device, mainStream ) );
+			if( found != lstmOverlaps().end() ) {
+				CLstmOverlap& o = found->second;
+				o.LastWasLstm = true;
+				for( int i = 0; i < 3; ++i ) {
+					o.Written[i] = written[i];
+					o.Read[i] = read[i];
+				}
+			}
+		}
+		return NH_OK;
 	}
 	// the one-launch step needs whole 32-k chunks and 8-unit blocks, 16-byte aligned rows and 32-bit byte offsets
 	const bool fusedStep = H % 32 == 0 && isAligned16( recurrentWeights ) && isAligned16( outputMainBackLink )

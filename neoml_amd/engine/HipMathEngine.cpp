@@ -28,6 +28,19 @@ struct CHipLstmDesc : public CLstmDesc {
 	int HiddenSize;
 	int ObjectSize;
 	CConstFloatHandle InputWeights, InputFreeTerm, RecurrentWeights, RecurrentFreeTerm;
+	// The workspace of the calls with this descriptor, grown on demand and kept: two LSTMs with descriptors of their
+	// own ( the two directions of a bidirectional layer ) then work in different memory, which is what lets the second
+	// run beside the first ( nhStreamOverlapLstm ). Blocks handed back go to the engine's pool and are reused in stream
+	// order, behind the kernels that used them.
+	IMathEngine* Engine = nullptr;
+	CMemoryHandle Workspace;
+	size_t WorkspaceSize = 0;
+	~CHipLstmDesc() override
+	{
+		if( !Workspace.IsNull() ) {
+			Engine->HeapFree( Workspace );
+		}
+	}
 };
 
 static nhBlobDesc toBlobDesc( const CBlobDesc& desc )
@@ -89,6 +102,8 @@ CHipMathEngine::CHipMathEngine( int deviceIndex, size_t memoryLimit, int /*flags
 	NH_CALL( nhPoolCreate( &pool, 0, memoryLimit ) );
 	// what the kernels allocate behind the scenes for this stream is charged to the engine's pool
 	NH_CALL( nhStreamBindPool( stream, pool ) );
+	// all of this engine's work is enqueued through the library: independent one-launch LSTMs may run side by side
+	NH_CALL( nhStreamOverlapLstm( stream, 1 ) );
 	initialized = true;
 }
 
@@ -846,6 +861,7 @@ CLstmDesc* CHipMathEngine::InitLstm( int hiddenSize, int objectSize, const CCons
 	desc->InputFreeTerm = inputFreeTerm;
 	desc->RecurrentWeights = recurrentWeights;
 	desc->RecurrentFreeTerm = recurrentFreeTerm;
+	desc->Engine = this;
 	return desc;
 }
 
@@ -856,7 +872,16 @@ void CHipMathEngine::Lstm( CLstmDesc& desc, bool reverse, int sequenceLength, in
 	CHipLstmDesc& d = static_cast<CHipLstmDesc&>( desc );
 	size_t workspaceSize = 0;
 	NH_CALL( nhLstmWorkspaceSize( d.HiddenSize, d.ObjectSize, sequenceLength, sequenceCount, &workspaceSize ) );
-	const CMemoryHandle workspace = StackAlloc( workspaceSize );
+	if( d.WorkspaceSize < workspaceSize ) {
+		if( !d.Workspace.IsNull() ) {
+			HeapFree( d.Workspace );
+			d.Workspace = CMemoryHandle();
+			d.WorkspaceSize = 0;
+		}
+		d.Workspace = HeapAlloc( workspaceSize );
+		d.WorkspaceSize = workspaceSize;
+	}
+	const CMemoryHandle& workspace = d.Workspace;
 	NH_CALL( nhLstm( stream, d.HiddenSize, d.ObjectSize, raw( d.InputWeights ),
 		d.InputFreeTerm.IsNull() ? nullptr : raw( d.InputFreeTerm ), raw( d.RecurrentWeights ),
 		d.RecurrentFreeTerm.IsNull() ? nullptr : raw( d.RecurrentFreeTerm ), reverse ? 1 : 0, sequenceLength,
@@ -864,8 +889,6 @@ void CHipMathEngine::Lstm( CLstmDesc& desc, bool reverse, int sequenceLength, in
 		inputMainBackLink.IsNull() ? nullptr : raw( inputMainBackLink ), raw( input ),
 		outputStateBackLink.IsNull() ? nullptr : raw( outputStateBackLink ), raw( outputMainBackLink ),
 		rawBytes( workspace ), workspaceSize ) );
-	// the stack block is recycled in stream order: later work on the same stream cannot overtake the LSTM kernels
-	StackFree( workspace );
 }
 
 // ---------------------------------------------------------------------------------------------------------

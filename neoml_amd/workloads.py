@@ -691,6 +691,11 @@ class LineRecognizer(Network):
     def __init__(self, backend, batch=64, height=32, width=512, hidden=256, classes=100, seed=0xC0FFEE + 5):
         super().__init__(backend)
         self.batch, self.height, self.width, self.hidden, self.classes = batch, height, width, hidden, classes
+        if hasattr(backend, "lib") and hasattr(backend, "stream"):
+            # every launch of this network goes through the library: the two directions of a bidirectional layer, two
+            # nhLstm calls one behind the other with workspaces of their own, may run side by side (what the engine
+            # adapter asks for its own stream)
+            backend.na.check(backend.lib.nhStreamOverlapLstm(backend.stream, 1))
         g = np.random.default_rng(seed)
         self.host = {}
         cin = 1

@@ -1060,6 +1060,87 @@ def test_lstm_on_two_streams_and_give_up_reported_to_its_own_stream(monkeypatch)
     del keep_a, keep_b, keep_a2, keep_b2
 
 
+def test_independent_lstms_side_by_side(capsys):
+    """nhStreamOverlapLstm: the two directions of a bidirectional layer, two nhLstm calls one behind the other on one
+    stream with workspaces of their own, run side by side and give what the calls give in order. A second call that
+    reads the first one's result, or whose input is produced by a launch in between, does not overtake anything."""
+    import torch
+    import neoml_amd
+    h = hip()
+    lib = neoml_amd.load()
+    g = rng(185)
+    T, B, In, H = 64, 64, 256, 256
+    dev = h.dev
+
+    def operands(n_in):
+        w_in = g.uniform(-0.2, 0.2, (4 * H, n_in)).astype(np.float32)
+        w_rec = g.uniform(-0.1, 0.1, (4 * H, H)).astype(np.float32)
+        bias = g.uniform(-0.5, 0.5, 4 * H).astype(np.float32)
+        return w_in, w_rec, bias
+
+    fwd, rev = operands(In), operands(In)
+    x = g.uniform(-1, 1, (T, B, In)).astype(np.float32)
+    s = torch.cuda.Stream()
+    ps = ctypes.c_void_p(s.cuda_stream)
+    size = ctypes.c_size_t(0)
+    neoml_amd.check(lib.nhLstmWorkspaceSize(H, In, T, B, ctypes.byref(size)))
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    d_fwd, d_rev, d_x = [up(a) for a in fwd], [up(a) for a in rev], up(x)
+    work = [torch.empty((size.value + 15) // 4, dtype=torch.float32, device=dev) for _ in range(2)]
+    out = [torch.zeros((T, B, H), device=dev) for _ in range(3)]
+    torch.cuda.synchronize()
+
+    def lstm(weights, source, reverse, result, workspace):
+        neoml_amd.check(lib.nhLstm(ps, H, In, P(weights[0]), P(weights[2]), P(weights[1]), None, reverse, T, B, None, None, P(source),
+                                   None, P(result), P(workspace), size.value))
+
+    def both_directions():
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(s)
+        lstm(d_fwd, d_x, 0, out[0], work[0])
+        lstm(d_rev, d_x, 1, out[1], work[1])
+        stop.record(s)
+        assert lib.nhStreamSynchronize(ps) == 0
+        return start.elapsed_time(stop), out[0].cpu().numpy().copy(), out[1].cpu().numpy().copy()
+
+    both_directions()
+    in_order_ms, f0, r0 = both_directions()
+    neoml_amd.check(lib.nhStreamOverlapLstm(ps, 1))
+    try:
+        both_directions()
+        side_by_side_ms, f1, r1 = both_directions()
+        with capsys.disabled():
+            print("\ntwo LSTM directions, %d steps, %d sequences, %d units: %.0f us in order, %.0f us side by side" % (
+                T, B, H, in_order_ms * 1e3, side_by_side_ms * 1e3))
+        want_f = orc.lstm(fwd[0], fwd[2], fwd[1], None, x, False)[0]
+        want_r = orc.lstm(rev[0], rev[2], rev[1], None, x, True)[0]
+        assert_close(f1, want_f, "forward direction, side by side")
+        assert_close(r1, want_r, "reverse direction, side by side")
+        assert_close(f1, f0, "forward direction: side by side vs in order")
+        assert_close(r1, r0, "reverse direction: side by side vs in order")
+        # the second reads what the first writes ( In == H ): it must wait
+        lstm(d_fwd, d_x, 0, out[0], work[0])
+        lstm(d_rev, out[0], 1, out[1], work[1])
+        assert lib.nhStreamSynchronize(ps) == 0
+        assert_close(out[1].cpu().numpy(), orc.lstm(rev[0], rev[2], rev[1], None, want_f, True)[0], "stacked: the second reads the first",
+                     atol=2e-5)
+        # a launch between the two produces the second one's input
+        lstm(d_fwd, d_x, 0, out[0], work[0])
+        neoml_amd.check(lib.nhVectorCopy(ps, P(out[2]), P(d_x), d_x.numel()))
+        lstm(d_rev, out[2], 1, out[1], work[1])
+        assert lib.nhStreamSynchronize(ps) == 0
+        assert_close(out[1].cpu().numpy(), want_r, "a launch between the two")
+        # the same workspace for both: in order again
+        lstm(d_fwd, d_x, 0, out[0], work[0])
+        lstm(d_rev, d_x, 1, out[1], work[0])
+        assert lib.nhStreamSynchronize(ps) == 0
+        assert_close(out[0].cpu().numpy(), want_f, "shared workspace, first")
+        assert_close(out[1].cpu().numpy(), want_r, "shared workspace, second")
+    finally:
+        neoml_amd.check(lib.nhStreamOverlapLstm(ps, 0))
+
+
 # ---------------------------------------------------------------------------------------------------------
 # error convention and allocator on the device
 
