@@ -34,6 +34,7 @@ template<> struct CChanVec<4> {
 	{
 		return make_float4( fmaf( a.x, b.x, c.x ), fmaf( a.y, b.y, c.y ), fmaf( a.z, b.z, c.z ), fmaf( a.w, b.w, c.w ) );
 	}
+	static __device__ __forceinline__ float4 mul( float4 a, float4 b ) { return make_float4( a.x * b.x, a.y * b.y, a.z * b.z, a.w * b.w ); }
 	static __device__ __forceinline__ float4 activate( float4 v, const CFusedActivation& a )
 	{
 		return make_float4( applyActivation( v.x, a ), applyActivation( v.y, a ), applyActivation( v.z, a ), applyActivation( v.w, a ) );
@@ -1082,45 +1083,101 @@ void channelwiseConvBackwardKernel( const nhConvDesc d, const float* outputDiff,
 	}
 }
 
-// The 3x3, stride 2 case of the gradient by the input, 4 channels per thread: an input pixel lies in one or two window
-// rows ( hi + pad even: taps 0 and 2, odd: tap 1 ) and one or two window columns, so it gathers at most four output
-// pixels; which ones follows from the parity, without divisions or a loop over the nine taps. Out-of-range output pixels
-// are out-of-range buffer offsets ( they read as zero ).
+// The 3x3, stride 2 case of the gradient by the input, 4 channels per thread. With a = hi + padH and b = wi + padW an
+// input pixel lies in the window rows kh of a's parity: a = 2r meets output row r through tap row 0 and output row r - 1
+// through tap row 2, a = 2r + 1 meets output row r through tap row 1; the same along the width. A thread owns a strip
+// of 8 columns of b that starts at an even b and pairsPerItem row pairs ( 2r, 2r + 1 ): the strip reads 5 columns of the
+// output gradient, and walking down it needs output row r - 1 and r for the pair r, so every row of the output
+// gradient is loaded once per strip ( a ring of three rows in registers: the row of the next pair is requested before
+// the current pair is computed and stored ) and which taps meet which pixel is known at compile time. Out-of-range
+// output pixels are out-of-range buffer offsets ( they read as zero ); input pixels outside the image are not stored.
 __global__ __launch_bounds__( 256 )
 void channelwiseBackward3x3Stride2Kernel( const nhConvDesc d, const float* outputDiff, const float* filter, float* inputDiff,
-	int totalItems )
+	int wGroups, int rowChunks, int pairsPerItem, int pairs, int totalItems )
 {
-	const int item = blockIdx.x * 256 + threadIdx.x;
+	const int item = xcdSwizzle( blockIdx.x, gridDim.x ) * 256 + threadIdx.x;
 	if( item >= totalItems ) {
 		return;
 	}
 	const int cg = d.channels / 4;
 	int t = item;
 	const int c = ( t % cg ) * 4; t /= cg;
-	const int wi = t % d.width; t /= d.width;
-	const int hi = t % d.height;
-	const int n = t / d.height;
+	const int b0 = ( t % wGroups ) * 8; t /= wGroups;
+	const int r0 = ( t % rowChunks ) * pairsPerItem;
+	const int n = t / rowChunks;
+	const int rEnd = min( r0 + pairsPerItem, pairs );
+
 	const __amdgpu_buffer_rsrc_t diff = makeBuffer( outputDiff );
-	const int a = hi + d.paddingHeight, b = wi + d.paddingWidth;
-	int kh[2], ho[2], kw[2], wo[2];
-	kh[0] = a & 1; ho[0] = ( a - kh[0] ) >> 1; kh[1] = kh[0] + 2; ho[1] = ho[0] - 1;
-	kw[0] = b & 1; wo[0] = ( b - kw[0] ) >> 1; kw[1] = kw[0] + 2; wo[1] = wo[0] - 1;
-	float4 acc = make_float4( 0.f, 0.f, 0.f, 0.f );
+	const unsigned rowBytes = static_cast<unsigned>( d.resultWidth ) * d.channels * 4;
+	const unsigned imageBytes = n * d.resultHeight * rowBytes;
+	unsigned colOff[5];
 #pragma unroll
-	for( int r = 0; r < 2; ++r ) {
-		const bool rowOk = kh[r] <= 2 && ho[r] >= 0 && ho[r] < d.resultHeight;
+	for( int j = 0; j < 5; ++j ) {
+		const int wo = b0 / 2 - 1 + j;
+		colOff[j] = wo >= 0 && wo < d.resultWidth ? static_cast<unsigned>( wo * d.channels + c ) * 4 : OutOfRange;
+	}
+	float4 f[9];
 #pragma unroll
-		for( int q = 0; q < 2; ++q ) {
-			const bool ok = rowOk && kw[q] <= 2 && wo[q] >= 0 && wo[q] < d.resultWidth;
-			const unsigned offset = ok ? static_cast<unsigned>( ( ( n * d.resultHeight + ho[r] ) * d.resultWidth + wo[q] ) * d.channels + c ) * 4u
-				: OutOfRange;
-			const float4 g = bufferLoad4( diff, offset );
-			const int tap = ok ? kh[r] * 3 + kw[q] : 0;
-			const float4 f = *reinterpret_cast<const float4*>( filter + tap * d.channels + c );
-			acc = CChanVec<4>::fma( g, f, acc );
+	for( int k = 0; k < 9; ++k ) {
+		f[k] = *reinterpret_cast<const float4*>( filter + k * d.channels + c );
+	}
+	float4 ring[3][5];
+	auto loadRow = [&]( float4* row, int ho ) {
+		const bool valid = ho >= 0 && ho < d.resultHeight && ho < rEnd;
+		const unsigned rowOff = imageBytes + static_cast<unsigned>( ho ) * rowBytes;
+#pragma unroll
+		for( int j = 0; j < 5; ++j ) {
+			// a valid row offset is below 2 GiB, so adding an out-of-range column stays out of range
+			row[j] = bufferLoad4( diff, valid ? rowOff + colOff[j] : OutOfRange );
+		}
+	};
+	loadRow( ring[0], r0 - 1 );
+	loadRow( ring[1], r0 );
+	const long long inRow = static_cast<long long>( d.width ) * d.channels;
+	float* const image = inputDiff + static_cast<long long>( n ) * d.height * inRow + c;
+	const int wi0 = b0 - d.paddingWidth;
+	for( int rBase = r0; rBase < rEnd; rBase += 3 ) {
+#pragma unroll
+		for( int k = 0; k < 3; ++k ) {
+			const int r = rBase + k;
+			if( r < rEnd ) {
+				const float4* prev = ring[k % 3];
+				const float4* cur = ring[( k + 1 ) % 3];
+				loadRow( ring[( k + 2 ) % 3], r + 1 );
+#pragma unroll
+				for( int odd = 0; odd < 2; ++odd ) {
+					const int hi = 2 * r + odd - d.paddingHeight;
+					if( hi < 0 || hi >= d.height ) {
+						continue;
+					}
+					float* out = image + hi * inRow + static_cast<long long>( wi0 ) * d.channels;
+#pragma unroll
+					for( int m = 0; m < 4; ++m ) {
+						float4 even, uneven;
+						if( odd == 0 ) {
+							even = CChanVec<4>::mul( cur[m + 1], f[0] );
+							even = CChanVec<4>::fma( cur[m], f[2], even );
+							even = CChanVec<4>::fma( prev[m + 1], f[6], even );
+							even = CChanVec<4>::fma( prev[m], f[8], even );
+							uneven = CChanVec<4>::mul( cur[m + 1], f[1] );
+							uneven = CChanVec<4>::fma( prev[m + 1], f[7], uneven );
+						} else {
+							even = CChanVec<4>::mul( cur[m + 1], f[3] );
+							even = CChanVec<4>::fma( cur[m], f[5], even );
+							uneven = CChanVec<4>::mul( cur[m + 1], f[4] );
+						}
+						const int wi = wi0 + 2 * m;
+						if( wi >= 0 && wi < d.width ) {
+							*reinterpret_cast<float4*>( out + ( 2 * m ) * d.channels ) = even;
+						}
+						if( wi + 1 >= 0 && wi + 1 < d.width ) {
+							*reinterpret_cast<float4*>( out + ( 2 * m + 1 ) * d.channels ) = uneven;
+						}
+					}
+				}
+			}
 		}
 	}
-	*reinterpret_cast<float4*>( inputDiff + static_cast<long long>( item ) * 4 ) = acc;
 }
 
 template<int VECW> struct CChanAtomic;
@@ -2177,9 +2234,17 @@ int nhBlobChannelwiseConvolutionBackward( nhStream s, const nhConvDesc* d, const
 		&& static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * d->channels * 4 < 0x7fffffffLL
 		&& static_cast<long long>( d->batch ) * d->height * d->width * ( d->channels / 4 ) < 0x7fffff00LL )
 	{
-		const int total = d->batch * d->height * d->width * ( d->channels / 4 );
+		// strips of 8 columns of wi + padW, and as many row pairs per strip as still leave every SIMD a few waves
+		const int pairs = ( d->height + d->paddingHeight + 1 ) / 2;
+		const int wGroups = ( d->width + d->paddingWidth + 7 ) / 8;
+		const long long perChunk = static_cast<long long>( d->batch ) * wGroups * ( d->channels / 4 );
+		const long long wanted = ( 8LL * 64 * 1024 + perChunk - 1 ) / perChunk; // 8 waves for each of the 1024 SIMDs
+		const int rowChunks = static_cast<int>( std::max( 1LL, std::min<long long>( ( pairs + 3 ) / 4, wanted ) ) );
+		const int pairsPerItem = ( pairs + rowChunks - 1 ) / rowChunks;
+		const int chunks = ( pairs + pairsPerItem - 1 ) / pairsPerItem;
+		const int total = static_cast<int>( perChunk * chunks );
 		hipLaunchKernelGGL( channelwiseBackward3x3Stride2Kernel, dim3( static_cast<unsigned>( ( total + 255 ) / 256 ) ), dim3( 256 ), 0,
-			toStream( s ), *d, outputDiff, filter, inputDiff, total );
+			toStream( s ), *d, outputDiff, filter, inputDiff, wGroups, chunks, pairsPerItem, pairs, total );
 		NH_LAUNCH_CHECK();
 		return NH_OK;
 	}

@@ -463,7 +463,11 @@ def test_convolution_gradients_are_adjoints_at_full_size():
                                                       (2, 21, 13, 20, 3, 3, 0, 2, 2, 2), (1, 3, 3, 4, 3, 3, 1, 1, 1, 1),
                                                       (4, 14, 14, 384, 3, 3, 1, 1, 1, 1), (16, 56, 56, 144, 3, 3, 1, 1, 1, 1),
                                                       # stride 1 with padding 0, 2 and mixed: the input gradient runs as a forward pass with the filter turned
-                                                      (2, 12, 10, 8, 3, 3, 0, 0, 1, 1), (2, 9, 11, 12, 3, 3, 2, 2, 1, 1), (1, 7, 16, 4, 3, 3, 0, 2, 1, 1)])
+                                                      (2, 12, 10, 8, 3, 3, 0, 0, 1, 1), (2, 9, 11, 12, 3, 3, 2, 2, 1, 1), (1, 7, 16, 4, 3, 3, 0, 2, 1, 1),
+                                                      # stride 2: strips of 8 columns and of row pairs, with even and odd sizes, padding 0, 1 and 2, rows
+                                                      # and columns that no window reaches, several row chunks per image
+                                                      (2, 16, 16, 8, 3, 3, 0, 0, 2, 2), (3, 57, 45, 32, 3, 3, 1, 1, 2, 2), (1, 5, 4, 4, 3, 3, 2, 1, 2, 2),
+                                                      (2, 18, 35, 12, 3, 3, 1, 0, 2, 2), (16, 112, 112, 96, 3, 3, 1, 1, 2, 2)])
 def test_channelwise_convolution_gradients(case):
     n, h, w, c, fh, fw, ph, pw, sh, sw = case
     g = rng(212 + c)
