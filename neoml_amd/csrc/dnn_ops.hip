@@ -2234,13 +2234,12 @@ int nhBlobChannelwiseConvolutionBackward( nhStream s, const nhConvDesc* d, const
 		&& static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * d->channels * 4 < 0x7fffffffLL
 		&& static_cast<long long>( d->batch ) * d->height * d->width * ( d->channels / 4 ) < 0x7fffff00LL )
 	{
-		// strips of 8 columns of wi + padW, and as many row pairs per strip as still leave every SIMD a few waves
+		// strips of 8 columns of wi + padW and of 2 row pairs: measured on 128 x 112 x 112 x 96, strips of 2 / 3 / 6 / 12 / 29
+		// pairs take 150 / 153 / 162 / 171 / 184 us although the short ones read every second row of the output gradient twice
 		const int pairs = ( d->height + d->paddingHeight + 1 ) / 2;
 		const int wGroups = ( d->width + d->paddingWidth + 7 ) / 8;
 		const long long perChunk = static_cast<long long>( d->batch ) * wGroups * ( d->channels / 4 );
-		const long long wanted = ( 8LL * 64 * 1024 + perChunk - 1 ) / perChunk; // 8 waves for each of the 1024 SIMDs
-		const int rowChunks = static_cast<int>( std::max( 1LL, std::min<long long>( ( pairs + 3 ) / 4, wanted ) ) );
-		const int pairsPerItem = ( pairs + rowChunks - 1 ) / rowChunks;
+		const int pairsPerItem = 2;
 		const int chunks = ( pairs + pairsPerItem - 1 ) / pairsPerItem;
 		const int total = static_cast<int>( perChunk * chunks );
 		hipLaunchKernelGGL( channelwiseBackward3x3Stride2Kernel, dim3( static_cast<unsigned>( ( total + 255 ) / 256 ) ), dim3( 256 ), 0,

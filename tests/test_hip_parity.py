@@ -250,7 +250,11 @@ def test_matmul_k_halves_in_one_workgroup():
 
 
 @pytest.mark.parametrize("batch,M,N,K", [(1, 2, 3, 4), (3, 16, 8, 5), (4, 33, 17, 9), (8, 64, 64, 16), (6, 100, 64, 100),
-                                         (5, 64, 256, 64), (2, 130, 36, 72)])
+                                         (5, 64, 256, 64), (2, 130, 36, 72),
+                                         # many small products (the strips of 64 rows that walk over all of their tiles): the two
+                                         # products of an attention head, ragged rows, columns and reductions, one and several k chunks
+                                         (256, 256, 256, 64), (256, 256, 64, 256), (130, 200, 52, 36), (600, 50, 132, 100),
+                                         (512, 64, 68, 256), (300, 70, 4, 4)])
 def test_matmul_batched(batch, M, N, K):
     g = rng(30 + M)
     a = g.uniform(-1, 1, (batch, M, K)).astype(np.float32)
