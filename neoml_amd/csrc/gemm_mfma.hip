@@ -734,26 +734,23 @@ void matMulKernel( const CMatMulArgs launchArgs )
 	const int totalSteps = ( K + KS - 1 ) / KS;
 	const int kSteps = min( stepsPerSplit, totalSteps - split * stepsPerSplit );
 	constexpr int Groups = KS / 8;
-	float4 rA[ASlots], rB[BSlots];
+	// Two sets of load registers: the operands of step ks + 1 wait in set ( ks + 1 ) % 2 while those of step ks + 2 are on
+	// their way into the other set, so a load has two steps' time before its values are needed. The steps are unrolled
+	// by two ( set and LDS buffer are compile-time constants ), and the steady state is a loop of its own in which every
+	// step stores and reloads unconditionally: the wait in front of the store then counts exactly the loads of the
+	// other set as still outstanding.
+	float4 rA[2][ASlots], rB[2][BSlots];
 	CFrag frag[2];
 	// a class without taps ( kSteps == 0 ) only writes the free term
-	if( !IsClasses || kSteps > 0 ) {
-		loadTiles( kStart, rA, rB );
-		storeTiles( 0, rA, rB );
-		if( kSteps > 1 ) {
-			loadTiles( kStart + KS, rA, rB );
+	auto step = [&]( int ks, auto setOf, auto steadyOf ) {
+		constexpr int set = decltype( setOf )::value; // == ( ks + 1 ) % 2: register set of step ks + 1 and the LDS buffer it goes to
+		constexpr bool steady = decltype( steadyOf )::value;
+		constexpr int cur = set ^ 1, nxt = set;
+		if( steady || ks + 1 < kSteps ) {
+			storeTiles( nxt, rA[set], rB[set] );
 		}
-		__syncthreads();
-		readFrag( 0, 0, frag[0] );
-	}
-	int cur = 0;
-	for( int ks = 0; ks < kSteps; ++ks ) {
-		const int nxt = cur ^ 1;
-		if( ks + 1 < kSteps ) {
-			storeTiles( nxt, rA, rB );
-		}
-		if( ks + 2 < kSteps ) {
-			loadTiles( kStart + ( ks + 2 ) * KS, rA, rB );
+		if( steady || ks + 3 < kSteps ) {
+			loadTiles( kStart + ( ks + 3 ) * KS, rA[set], rB[set] );
 		}
 		__builtin_amdgcn_sched_barrier( 0 );
 #pragma unroll
@@ -762,7 +759,7 @@ void matMulKernel( const CMatMulArgs launchArgs )
 				readFrag( cur, g + 1, frag[( g + 1 ) & 1] );
 			} else {
 				__syncthreads();
-				if( ks + 1 < kSteps ) {
+				if( steady || ks + 1 < kSteps ) {
 					readFrag( nxt, 0, frag[( g + 1 ) & 1] );
 				}
 			}
@@ -770,7 +767,41 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			multiply( frag[g & 1] );
 			__builtin_amdgcn_sched_barrier( 0 );
 		}
-		cur = nxt;
+	};
+	int ks = 0;
+	const bool hasSteadySteps = kSteps > 4;
+	if( hasSteadySteps ) {
+		// ( a branch of its own: on the way into the steady loop every one of these loads has been issued, which is what
+		// lets the waits in that loop leave the younger set's loads outstanding )
+		loadTiles( kStart, rA[0], rB[0] );
+		storeTiles( 0, rA[0], rB[0] );
+		loadTiles( kStart + KS, rA[1], rB[1] );
+		loadTiles( kStart + 2 * KS, rA[0], rB[0] );
+		__syncthreads();
+		readFrag( 0, 0, frag[0] );
+		asm volatile( "; into the steady loop" ); // keeps this path apart from the one below up to the loop
+		for( ; ks + 4 < kSteps; ks += 2 ) {
+			step( ks, std::integral_constant<int, 1>(), std::true_type() );
+			step( ks + 1, std::integral_constant<int, 0>(), std::true_type() );
+		}
+	} else if( !IsClasses || kSteps > 0 ) {
+		loadTiles( kStart, rA[0], rB[0] );
+		storeTiles( 0, rA[0], rB[0] );
+		if( kSteps > 1 ) {
+			loadTiles( kStart + KS, rA[1], rB[1] );
+		}
+		if( kSteps > 2 ) {
+			loadTiles( kStart + 2 * KS, rA[0], rB[0] );
+		}
+		__syncthreads();
+		readFrag( 0, 0, frag[0] );
+	}
+	static_assert( Groups % 2 == 0, "the fragment buffers are back where they started after a step" );
+	for( ; ks < kSteps; ks += 2 ) {
+		step( ks, std::integral_constant<int, 1>(), std::false_type() );
+		if( ks + 1 < kSteps ) {
+			step( ks + 1, std::integral_constant<int, 0>(), std::false_type() );
+		}
 	}
 
 	if constexpr( KGROUPS == 2 ) {

@@ -25,6 +25,10 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=0, help="launches per measurement (default: enough for ~0.3 s)")
     ap.add_argument("--filter", default="")
+    ap.add_argument("--vendor", action="store_true",
+                    help="under every convolution and matrix product line, time the vendor library at the same shape "
+                         "(torch.nn.functional.conv2d = MIOpen, torch.matmul / torch.bmm = hipBLASLt or rocBLAS, fp32): "
+                         "a yardstick on the same device, nothing the engine calls")
     args = ap.parse_args()
 
     import torch
@@ -76,6 +80,22 @@ def main():
         print("%-58s %9.1f us %7.1f TFLOP/s %5.1f%%  %8.1f GB/s%s %5.1f%%" % (
             name, us, tf, 100 * mfma_frac, gbs, cached, 100 * hbm_frac), flush=True)
 
+    def vendor(name, op, flops, nbytes):
+        """op() runs the vendor library's routine on torch's current stream (the one the engine's launches use here)"""
+        if not args.vendor or (wanted and not any(w in name for w in wanted)):
+            return
+        try:
+            op()
+            torch.cuda.synchronize()
+        except Exception as e:  # a shape the library refuses is reported, not fatal
+            print("%-58s vendor library: %s" % ("  " + name[:56], str(e).splitlines()[0][:60]), flush=True)
+            return
+
+        def call():
+            op()
+            return 0
+        measure(("  vendor: " + name)[:58], call, flops, nbytes, nbytes)
+
     zero = torch.zeros(1, device=dev)
     six = torch.full((1,), 6.0, device=dev)
 
@@ -89,6 +109,14 @@ def main():
         by = 4 * (x.numel() + y.numel() + flt.numel() + cout)
         measure("BlobConvolution %s %dx%dx%dx%d->%d %dx%d/%d" % (tag, n, h, w, cin, cout, f, f, s),
                 lambda: lib.nhBlobConvolution(stream, ctypes.byref(d), P(x), P(flt), P(b), P(y)), fl, by, by)
+        if args.vendor:
+            # the same tensors as logical NCHW views of channels-last memory, and as plain NCHW
+            xl, wl = x.permute(0, 3, 1, 2), flt.permute(0, 3, 1, 2)
+            vendor("conv2d channels-last %s %dx%dx%dx%d->%d %dx%d/%d" % (tag, n, h, w, cin, cout, f, f, s),
+                   lambda: torch.nn.functional.conv2d(xl, wl, b, stride=s, padding=p), fl, by)
+            xc, wc = xl.contiguous(), wl.contiguous()
+            vendor("conv2d NCHW %s %dx%dx%dx%d->%d %dx%d/%d" % (tag, n, h, w, cin, cout, f, f, s),
+                   lambda: torch.nn.functional.conv2d(xc, wc, b, stride=s, padding=p), fl, by)
 
     conv("cfg1", 32, 32, 32, 64, 64, 3, 1, 1)
     conv("cfg2 stem", 64, 224, 224, 3, 64, 7, 3, 2)
@@ -144,6 +172,8 @@ def main():
         measure("MultiplyMatrixByTransposedMatrix %s %dx%dx%d" % (tag, m, n, k),
                 lambda: lib.nhMultiplyMatrixByTransposedMatrix(stream, P(a), m, k, k, P(b), n, k, P(c), n, m * n),
                 2 * m * n * k, 4 * (m * k + n * k + m * n), 4 * (m * k + n * k + m * n))
+        vendor("matmul A B^T %s %dx%dx%d" % (tag, m, n, k), lambda: torch.matmul(a, b.t(), out=c),
+               2 * m * n * k, 4 * (m * k + n * k + m * n))
 
     gemm_nt("cfg2 fc", 64, 1000, 512)
     gemm_nt("cfg4 qkv/out", 8192, 512, 512)
@@ -163,6 +193,8 @@ def main():
         by = 4 * batch * (m * k + k * n + m * n)
         measure("%s %s b%d %dx%dx%d" % ("MultiplyMatrixByMatrix" if kind == "nn" else "MultiplyTransposedMatrixByMatrix",
                                          tag, batch, m, n, k), call, 2 * batch * m * n * k, by, by)
+        if kind == "nn":
+            vendor("bmm %s b%d %dx%dx%d" % (tag, batch, m, n, k), lambda: torch.bmm(a, b, out=c), 2 * batch * m * n * k, by)
 
     gemm_batched("cfg4 QK^T", "nn", 256, 256, 256, 64)
     gemm_batched("cfg4 PV", "nn", 256, 256, 64, 256)
