@@ -2059,6 +2059,225 @@ static int poolingBackwardImpl( nhStream s, const nhPoolingDesc* d, const float*
 	return NH_OK;
 }
 
+// Expand 1x1 (+act) -> depthwise 3x3, padding 1 (+act) in one launch, the expanded tensor never in memory: for the blocks
+// of a MobileNetV2 whose expanded tensor is several times the size of the last-level cache (16 -> 96 channels at
+// 112 x 112, 24 -> 144 at 56 x 56, 32 -> 192 at 28 x 28, batch 128) writing it and reading it back is most of the block's
+// time. Every wavefront works alone, no barrier anywhere: it owns a patch of PH x PW <= 64 input pixels ( 8 x 8 at
+// stride 1 for 6 x 6 output pixels, 7 x 9 at stride 2 for 3 x 4 ), holds them as the operand of two 32 x 32 MFMA blocks
+// in registers for the whole launch ( each lane its pixel's channels, fetched with 128-bit buffer loads; pixels
+// outside the image are out-of-range offsets ) and walks the expanded channels 32 at a time: multiply by that chunk of
+// the expand filter ( its rows straight from memory into the other operand ), add the free term, activate, put zeros
+// where the pixel lies outside the image ( the depthwise convolution pads the expanded tensor, not the input ), write
+// the 64 x 32 values to the wave's own LDS tile, and sum the nine taps of every output from there, four channels per lane,
+// eight lanes per pixel = one 128-byte store per pixel and chunk. A wave's LDS operations complete in order, so the
+// tile needs no synchronisation beyond the wave. The patches overlap by two pixels, i.e. the expand product is computed
+// 1.8 times ( the matrix pipe is idle otherwise: the reduction is 16 to 32 long ).
+namespace nh {
+
+typedef float expandAcc __attribute__( ( ext_vector_type( 16 ) ) );
+
+// CLIPPED: both activations are ReLU with an upper threshold ( ReLU6, what MobileNetV2 uses ): two instructions per value
+template<bool CLIPPED>
+__device__ __forceinline__ float activateExpanded( float v, const CFusedActivation& a )
+{
+	if( CLIPPED ) {
+		return fminf( fmaxf( v, 0.f ), a.Param ); // NaN becomes 0, as in VectorReLU
+	}
+	return applyActivation( v, a );
+}
+
+template<int STRIDE, int KIN, bool CLIPPED>
+__global__ __launch_bounds__( 256, 2 )
+void expandDepthwiseKernel( const nhSeparableBlockDesc d, int outH, int outW, const float* input, const float* expandFilter,
+	const float* expandBias, const float* dwFilter, const float* dwBias, float* result, int tilesX, int tilesY, int totalTiles,
+	const CFusedActivation expandAct, const CFusedActivation dwAct )
+{
+	constexpr int PH = STRIDE == 1 ? 8 : 7, PW = STRIDE == 1 ? 8 : 9;
+	constexpr int OH = ( PH - 3 ) / STRIDE + 1, OW = ( PW - 3 ) / STRIDE + 1;
+	constexpr int PitchE = 36;
+	constexpr int KG = KIN / 8;
+	static_assert( PH * PW <= 64 && KIN % 8 == 0, "one pixel per accumulator row of two blocks, whole groups of 8 k" );
+	__shared__ __attribute__( ( aligned( 16 ) ) ) float ldsE[4][64 * PitchE];
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, half = lane >> 5;
+	int t = xcdSwizzle( blockIdx.x, gridDim.x ) * 4 + wave;
+	if( t >= totalTiles ) {
+		return;
+	}
+	const int tx = t % tilesX; t /= tilesX;
+	const int ty = t % tilesY;
+	const int n = t / tilesY;
+	const int cexp = d.expandedChannels;
+	const int hy0 = ty * OH * STRIDE - 1, wx0 = tx * OW * STRIDE - 1;
+	auto insideImage = [&]( int p ) -> bool {
+		const int py = p / PW, px = p - py * PW;
+		const int hy = hy0 + py, wx = wx0 + px;
+		return p < PH * PW && hy >= 0 && hy < d.height && wx >= 0 && wx < d.width;
+	};
+	// the patch as MFMA operand: lane ( l32, half ) holds k = 8 g + 4 half .. + 3 of pixel 32 b + l32
+	const __amdgpu_buffer_rsrc_t image = makeBuffer( input + static_cast<long long>( n ) * d.height * d.width * KIN );
+	float4 a[2][KG];
+	unsigned insideBits[2];
+#pragma unroll
+	for( int b = 0; b < 2; ++b ) {
+		const int p = b * 32 + l32;
+		const int py = p / PW, px = p - py * PW;
+		const unsigned base = insideImage( p ) ? static_cast<unsigned>( ( ( hy0 + py ) * d.width + wx0 + px ) * KIN + half * 4 ) * 4u : OutOfRange;
+#pragma unroll
+		for( int g = 0; g < KG; ++g ) {
+			// a valid offset is below 2 GiB, so adding to an out-of-range one stays out of range
+			a[b][g] = bufferLoad4( image, base + g * 32u );
+		}
+		// bit r: accumulator register r of this lane in block b is a pixel of the image
+		insideBits[b] = 0;
+#pragma unroll
+		for( int r = 0; r < 16; ++r ) {
+			insideBits[b] |= insideImage( b * 32 + ( r >> 2 ) * 8 + half * 4 + ( r & 3 ) ) ? ( 1u << r ) : 0u;
+		}
+	}
+	// ( rows beyond PH x PW are never read by a window, so "inside" only matters for the patch's own pixels )
+	const bool wholePatchInside = hy0 >= 0 && wx0 >= 0 && hy0 + PH <= d.height && wx0 + PW <= d.width;
+	float* const tile = ldsE[wave];
+	const int q4 = ( lane & 7 ) * 4;
+	// lane ( q, o ) sums 4 channels of the output pixels 8 pass + o: where their windows begin in the tile and where they go
+	constexpr int Passes = ( OH * OW + 7 ) / 8;
+	int windowAt[Passes];
+	long long storeAt[Passes]; // in floats from result, without the channel; negative: no such pixel
+#pragma unroll
+	for( int pass = 0; pass < Passes; ++pass ) {
+		const int op = pass * 8 + ( lane >> 3 );
+		const int oy = op / OW, ox = op - oy * OW;
+		const int gy = ty * OH + oy, gx = tx * OW + ox;
+		windowAt[pass] = ( oy * STRIDE * PW + ox * STRIDE ) * PitchE + q4;
+		storeAt[pass] = ( op < OH * OW && gy < outH && gx < outW )
+			? ( ( static_cast<long long>( n ) * outH + gy ) * outW + gx ) * cexp + q4 : -1;
+	}
+	// a chunk's rows of the expand filter ( lane = channel c0 + l32 ) and its free term are requested one chunk ahead
+	float4 wNext[KG];
+	float biasNext = 0.f;
+	auto requestChunk = [&]( int c0 ) {
+		const bool rowOk = c0 + l32 < cexp;
+		const float* wRow = expandFilter + static_cast<long long>( rowOk ? c0 + l32 : 0 ) * KIN + half * 4;
+#pragma unroll
+		for( int g = 0; g < KG; ++g ) {
+			wNext[g] = *reinterpret_cast<const float4*>( wRow + g * 8 );
+		}
+		biasNext = expandBias != nullptr ? expandBias[rowOk ? c0 + l32 : 0] : 0.f;
+	};
+	requestChunk( 0 );
+	for( int c0 = 0; c0 < cexp; c0 += 32 ) {
+		const bool rowOk = c0 + l32 < cexp;
+		float4 w[KG];
+#pragma unroll
+		for( int g = 0; g < KG; ++g ) {
+			w[g] = rowOk ? wNext[g] : make_float4( 0.f, 0.f, 0.f, 0.f );
+		}
+		const float bias = rowOk ? biasNext : 0.f;
+		if( c0 + 32 < cexp ) {
+			requestChunk( c0 + 32 );
+		}
+		const bool quadOk = c0 + q4 < cexp;
+		float4 f[9];
+#pragma unroll
+		for( int k = 0; k < 9; ++k ) {
+			f[k] = quadOk ? *reinterpret_cast<const float4*>( dwFilter + k * cexp + c0 + q4 ) : make_float4( 0.f, 0.f, 0.f, 0.f );
+		}
+		const float4 bias4 = ( dwBias != nullptr && quadOk ) ? *reinterpret_cast<const float4*>( dwBias + c0 + q4 )
+			: make_float4( 0.f, 0.f, 0.f, 0.f );
+#pragma unroll
+		for( int b = 0; b < 2; ++b ) {
+			// the accumulator starts as the free term: every register of a lane belongs to the lane's channel
+			expandAcc acc;
+#pragma unroll
+			for( int r = 0; r < 16; ++r ) {
+				acc[r] = bias;
+			}
+#pragma unroll
+			for( int g = 0; g < KG; ++g ) {
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[b][g].x, w[g].x, acc, 0, 0, 0 );
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[b][g].y, w[g].y, acc, 0, 0, 0 );
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[b][g].z, w[g].z, acc, 0, 0, 0 );
+				acc = __builtin_amdgcn_mfma_f32_32x32x2f32( a[b][g].w, w[g].w, acc, 0, 0, 0 );
+			}
+			if( wholePatchInside ) {
+#pragma unroll
+				for( int r = 0; r < 16; ++r ) {
+					tile[( b * 32 + ( r >> 2 ) * 8 + half * 4 + ( r & 3 ) ) * PitchE + l32] = activateExpanded<CLIPPED>( acc[r], expandAct );
+				}
+			} else {
+#pragma unroll
+				for( int r = 0; r < 16; ++r ) {
+					const float v = activateExpanded<CLIPPED>( acc[r], expandAct );
+					tile[( b * 32 + ( r >> 2 ) * 8 + half * 4 + ( r & 3 ) ) * PitchE + l32] = ( ( insideBits[b] >> r ) & 1u ) != 0 ? v : 0.f;
+				}
+			}
+		}
+		// the wave's own writes, read back by other lanes of the same wave: ordered by the LDS, kept in order by the fence
+		__builtin_amdgcn_fence( __ATOMIC_RELEASE, "wavefront" );
+		__builtin_amdgcn_wave_barrier();
+		__builtin_amdgcn_fence( __ATOMIC_ACQUIRE, "wavefront" );
+#pragma unroll
+		for( int pass = 0; pass < Passes; ++pass ) {
+			if( storeAt[pass] >= 0 && quadOk ) {
+				const float* e = tile + windowAt[pass];
+				float4 acc = bias4;
+#pragma unroll
+				for( int ky = 0; ky < 3; ++ky ) {
+#pragma unroll
+					for( int kx = 0; kx < 3; ++kx ) {
+						acc = CChanVec<4>::fma( *reinterpret_cast<const float4*>( e + ( ky * PW + kx ) * PitchE ), f[ky * 3 + kx], acc );
+					}
+				}
+				*reinterpret_cast<float4*>( result + storeAt[pass] + c0 )
+					= make_float4( activateExpanded<CLIPPED>( acc.x, dwAct ), activateExpanded<CLIPPED>( acc.y, dwAct ),
+						activateExpanded<CLIPPED>( acc.z, dwAct ), activateExpanded<CLIPPED>( acc.w, dwAct ) );
+			}
+		}
+		__builtin_amdgcn_fence( __ATOMIC_RELEASE, "wavefront" );
+		__builtin_amdgcn_wave_barrier();
+		__builtin_amdgcn_fence( __ATOMIC_ACQUIRE, "wavefront" );
+	}
+}
+
+} // namespace nh
+
+// true ( and launched ) where the fused kernel is built for the block and the expanded tensor is too large for the caches
+static bool tryExpandDepthwise( nhStream s, const nhSeparableBlockDesc* d, const nhConvDesc& dw, const float* input,
+	const float* expandFilter, const float* expandBias, const float* dwFilter, const float* dwBias, float* reduced )
+{
+	const long long expandedBytes = static_cast<long long>( d->batch ) * d->height * d->width * d->expandedChannels * 4;
+	if( expandedBytes < ( 64LL << 20 ) || d->expandedChannels % 4 != 0 || !isAligned16( input ) || !isAligned16( expandFilter )
+		|| !isAligned16( dwFilter ) || ( dwBias != nullptr && !isAligned16( dwBias ) ) || !isAligned16( reduced )
+		|| ( d->inputChannels != 16 && d->inputChannels != 24 && d->inputChannels != 32 )
+		|| static_cast<long long>( d->height ) * d->width * d->inputChannels * 4 >= 0x7fffffffLL )
+	{
+		return false;
+	}
+	const int oh = d->stride == 1 ? 6 : 3, ow = d->stride == 1 ? 6 : 4;
+	const int tilesX = ceilDiv( dw.resultWidth, ow ), tilesY = ceilDiv( dw.resultHeight, oh );
+	const long long tiles = static_cast<long long>( d->batch ) * tilesX * tilesY;
+	if( tiles < 4096 || tiles > 0x7ffffff0LL ) {
+		return false;
+	}
+	const unsigned groups = static_cast<unsigned>( ( tiles + 3 ) / 4 );
+	const CFusedActivation expandAct = { d->expandActivation, d->expandParam };
+	const CFusedActivation dwAct = { d->channelwiseActivation, d->channelwiseParam };
+	const bool clipped = d->expandActivation == NH_ACT_RELU && d->expandParam > 0.f && d->channelwiseActivation == NH_ACT_RELU
+		&& d->channelwiseParam > 0.f;
+#define NH_EXPAND_DW( STRIDE, KIN, CLIPPED ) hipLaunchKernelGGL( ( expandDepthwiseKernel<STRIDE, KIN, CLIPPED> ), dim3( groups ), \
+		dim3( 256 ), 0, toStream( s ), *d, dw.resultHeight, dw.resultWidth, input, expandFilter, expandBias, dwFilter, dwBias, reduced, \
+		tilesX, tilesY, static_cast<int>( tiles ), expandAct, dwAct )
+#define NH_EXPAND_DW_K( STRIDE, CLIPPED ) if( d->inputChannels == 16 ) { NH_EXPAND_DW( STRIDE, 16, CLIPPED ); } \
+	else if( d->inputChannels == 24 ) { NH_EXPAND_DW( STRIDE, 24, CLIPPED ); } else { NH_EXPAND_DW( STRIDE, 32, CLIPPED ); }
+	if( d->stride == 1 ) {
+		if( clipped ) { NH_EXPAND_DW_K( 1, true ) } else { NH_EXPAND_DW_K( 1, false ) }
+	} else {
+		if( clipped ) { NH_EXPAND_DW_K( 2, true ) } else { NH_EXPAND_DW_K( 2, false ) }
+	}
+#undef NH_EXPAND_DW_K
+#undef NH_EXPAND_DW
+	return true;
+}
+
 extern "C" {
 
 
@@ -2681,14 +2900,18 @@ int nhMobileNetV2Block( nhStream s, const nhSeparableBlockDesc* d, const float* 
 	const CFusedActivation expandAct = { d->expandActivation, d->expandParam };
 	const CFusedActivation channelwiseAct = { d->channelwiseActivation, d->channelwiseParam };
 	const CFusedActivation none = { NH_ACT_NONE, 0.f };
-	rc = matMulNTFused( toStream( s ), input, d->inputChannels, expandFilter, d->inputChannels, expanded, d->expandedChannels,
-		static_cast<int>( pixelsIn ), d->expandedChannels, d->inputChannels, 1, 0, 0, 0, expandFreeTerm, false, expandAct, nullptr );
-	if( rc != NH_OK ) {
-		return rc;
-	}
-	rc = channelwiseConvolution( s, &dw, expanded, channelwiseFilter, channelwiseFreeTerm, reduced, channelwiseAct );
-	if( rc != NH_OK ) {
-		return rc;
+	if( tryExpandDepthwise( s, d, dw, input, expandFilter, expandFreeTerm, channelwiseFilter, channelwiseFreeTerm, reduced ) ) {
+		NH_LAUNCH_CHECK();
+	} else {
+		rc = matMulNTFused( toStream( s ), input, d->inputChannels, expandFilter, d->inputChannels, expanded, d->expandedChannels,
+			static_cast<int>( pixelsIn ), d->expandedChannels, d->inputChannels, 1, 0, 0, 0, expandFreeTerm, false, expandAct, nullptr );
+		if( rc != NH_OK ) {
+			return rc;
+		}
+		rc = channelwiseConvolution( s, &dw, expanded, channelwiseFilter, channelwiseFreeTerm, reduced, channelwiseAct );
+		if( rc != NH_OK ) {
+			return rc;
+		}
 	}
 	return matMulNTFused( toStream( s ), reduced, d->expandedChannels, downFilter, d->expandedChannels, output, d->outputChannels,
 		static_cast<int>( pixelsOut ), d->outputChannels, d->expandedChannels, 1, 0, 0, 0, downFreeTerm, false, none,

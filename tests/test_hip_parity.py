@@ -951,6 +951,32 @@ def test_separable_blocks(case, with_expand):
             assert_close(got, want, "separable block in place %s" % (case,))
 
 
+# Blocks whose expanded tensor would be far larger than the caches: expand and depthwise stage run as one launch that
+# keeps the expanded values of a tile of pixels in LDS (tiles of 14 x 14 / 7 x 7 output pixels, 32 expanded channels at a
+# time). Sizes that are and are not multiples of the tile, a last chunk of 16 and of 4 channels, both strides, with and
+# without free terms, a residual that reuses the input blob.
+LARGE_SEPARABLE_CASES = [
+    (16, 112, 112, 16, 96, 24, 2, False, ("relu", 6.0), ("relu", 6.0)),
+    (40, 56, 56, 24, 144, 24, 1, True, ("relu", 6.0), ("relu", 6.0)),
+    (40, 56, 56, 24, 144, 32, 2, False, ("relu", 6.0), ("relu", 6.0)),
+    (128, 28, 28, 32, 192, 32, 1, True, ("relu", 6.0), ("relu", 6.0)),
+    (24, 100, 90, 16, 100, 24, 1, False, ("hswish", 0.0), ("relu", 0.0)),
+    (24, 101, 91, 16, 96, 24, 2, False, ("relu", 6.0), (None, 0.0)),
+]
+
+
+@pytest.mark.parametrize("case", LARGE_SEPARABLE_CASES)
+def test_separable_blocks_without_the_expanded_tensor(case):
+    for with_free_terms in (True, False):
+        x, expand, channelwise, down, stride, residual = separable_operands(case, True, with_free_terms)
+        want = orc.separable_block(x, expand, channelwise, down, stride, residual)
+        got = hip().separable_block(x, expand, channelwise, down, stride, residual)
+        assert_close(got, want, "separable block %s free terms=%s" % (case, with_free_terms))
+        if residual:
+            got = hip().separable_block(x, expand, channelwise, down, stride, residual, in_place=True)
+            assert_close(got, want, "separable block in place %s" % (case,))
+
+
 @pytest.mark.parametrize("case", MOBILENETV3_CASES + [
     (4, 28, 28, 40, 120, 40, 5, 1, True, ("relu", 0.0), ("relu", 0.0), ("relu", 0.0)),
     (2, 14, 14, 80, 480, 112, 3, 1, False, ("hswish", 0.0), ("hswish", 0.0), ("hswish", 0.0)),
