@@ -200,6 +200,27 @@ def main():
     gemm_batched("cfg4 PV", "nn", 256, 256, 64, 256)
     gemm_batched("fc grad", "tn", 1, 512, 2048, 8192)
 
+    # ---- the fused block of the graph optimizer (config 3): expand 1x1 -> depthwise 3x3 -> down 1x1 (+ input)
+    def block(n, h, w, cin, e, cout, stride, residual):
+        d = neoml_amd.SeparableBlockDesc(n, h, w, cin, e, cout, stride, 1 if residual else 0, 1, 6.0, 1, 6.0)  # ReLU6 twice
+        size = ctypes.c_size_t(0)
+        neoml_amd.check(lib.nhMobileNetV2BlockWorkspaceSize(ctypes.byref(d), ctypes.byref(size)))
+        work = empty((size.value + 15) // 4 + 4)
+        x, ef, eb, cf, cb, df, db = rand(n, h, w, cin), rand(e, cin), rand(e), rand(3, 3, e), rand(e), rand(cout, e), rand(cout)
+        ho, wo = (h + stride - 1) // stride, (w + stride - 1) // stride
+        out = empty(n, ho, wo, cout)
+        fl = 2 * n * (h * w * cin * e + ho * wo * e * (9 + cout))
+        by = 4 * (x.numel() + out.numel() + ef.numel() + cf.numel() + df.numel() + 2 * e + cout)
+        measure("MobileNetV2Block cfg3 %dx%dx%dx%d->%d->%d /%d" % (n, h, w, cin, e, cout, stride),
+                lambda: lib.nhMobileNetV2Block(stream, ctypes.byref(d), P(x), P(ef), P(eb), P(cf), P(cb), P(df), P(db), P(out),
+                                               P(work), size.value), fl, by, by)
+
+    block(128, 112, 112, 16, 96, 24, 2, False)
+    block(128, 56, 56, 24, 144, 24, 1, True)
+    block(128, 56, 56, 24, 144, 32, 2, False)
+    block(128, 28, 28, 32, 192, 32, 1, True)
+    block(128, 14, 14, 64, 384, 64, 1, True)
+
     # ---- depthwise convolution (config 3)
     def dw(n, h, w, c, s):
         d = neoml_amd.ConvDesc(n, h, w, c, c, 3, 3, 1, 1, s, s, 1, 1, 0, 0)
