@@ -2963,6 +2963,21 @@ int nhMobileNetV3PreSEBlock( nhStream s, const nhConvDesc* dw, int inputChannels
 	float* expanded = static_cast<float*>( workspace );
 	const CFusedActivation expandAct = { expandActivation, expandParam };
 	const CFusedActivation channelwiseAct = { channelwiseActivation, channelwiseParam };
+	if( dw->filterHeight == 3 && dw->filterWidth == 3 && dw->paddingHeight == 1 && dw->paddingWidth == 1
+		&& dw->strideHeight == dw->strideWidth && ( dw->strideHeight == 1 || dw->strideHeight == 2 ) )
+	{
+		// the 3x3 case is the MobileNetV2 block's pair of stages: one launch where the expanded tensor would be large
+		nhSeparableBlockDesc pair = {};
+		pair.batch = dw->batch; pair.height = dw->height; pair.width = dw->width;
+		pair.inputChannels = inputChannels; pair.expandedChannels = dw->channels; pair.outputChannels = dw->channels;
+		pair.stride = dw->strideHeight;
+		pair.expandActivation = expandActivation; pair.expandParam = expandParam;
+		pair.channelwiseActivation = channelwiseActivation; pair.channelwiseParam = channelwiseParam;
+		if( tryExpandDepthwise( s, &pair, *dw, input, expandFilter, expandFreeTerm, channelwiseFilter, channelwiseFreeTerm, output ) ) {
+			NH_LAUNCH_CHECK();
+			return NH_OK;
+		}
+	}
 	const int pixels = dw->batch * dw->height * dw->width;
 	const int rcExpand = matMulNTFused( toStream( s ), input, inputChannels, expandFilter, inputChannels, expanded, dw->channels,
 		pixels, dw->channels, inputChannels, 1, 0, 0, 0, expandFreeTerm, false, expandAct, nullptr );

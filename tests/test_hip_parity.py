@@ -980,7 +980,10 @@ def test_separable_blocks_without_the_expanded_tensor(case):
 @pytest.mark.parametrize("case", MOBILENETV3_CASES + [
     (4, 28, 28, 40, 120, 40, 5, 1, True, ("relu", 0.0), ("relu", 0.0), ("relu", 0.0)),
     (2, 14, 14, 80, 480, 112, 3, 1, False, ("hswish", 0.0), ("hswish", 0.0), ("hswish", 0.0)),
-    (2, 14, 14, 112, 672, 160, 5, 2, False, ("hswish", 0.0), ("hswish", 0.0), ("hswish", 0.0))])
+    (2, 14, 14, 112, 672, 160, 5, 2, False, ("hswish", 0.0), ("hswish", 0.0), ("hswish", 0.0)),
+    # an expanded tensor far larger than the caches behind a 3x3 depthwise stage: expand and depthwise in one launch
+    (32, 112, 112, 16, 64, 24, 3, 2, False, ("relu", 0.0), ("hswish", 0.0), ("relu", 0.0)),
+    (72, 56, 56, 24, 72, 24, 3, 1, True, ("hswish", 0.0), ("relu", 0.0), ("hswish", 0.0))])
 def test_mobilenetv3_blocks(case):
     n, h, w, cin, e, cout, fsize, stride, residual, ex_act, ch_act, gate_act = case
     x, expand, channelwise, gate, down = mobilenetv3_operands(case)
