@@ -2081,7 +2081,9 @@ template<bool CLIPPED>
 __device__ __forceinline__ float activateExpanded( float v, const CFusedActivation& a )
 {
 	if( CLIPPED ) {
-		return fminf( fmaxf( v, 0.f ), a.Param ); // NaN becomes 0, as in VectorReLU
+		// the median of ( v, 0, threshold ) in one instruction; with a NaN among its operands the instruction returns the
+		// smallest of the others, so NaN becomes 0, as in VectorReLU
+		return __builtin_amdgcn_fmed3f( v, 0.f, a.Param );
 	}
 	return applyActivation( v, a );
 }
@@ -2219,13 +2221,10 @@ void expandDepthwiseKernel( const nhSeparableBlockDesc d, int outH, int outW, co
 		for( int pass = 0; pass < Passes; ++pass ) {
 			if( storeAt[pass] >= 0 && quadOk ) {
 				const float* e = tile + windowAt[pass];
-				float4 acc = bias4;
+				float4 acc = CChanVec<4>::fma( *reinterpret_cast<const float4*>( e ), f[0], bias4 );
 #pragma unroll
-				for( int ky = 0; ky < 3; ++ky ) {
-#pragma unroll
-					for( int kx = 0; kx < 3; ++kx ) {
-						acc = CChanVec<4>::fma( *reinterpret_cast<const float4*>( e + ( ky * PW + kx ) * PitchE ), f[ky * 3 + kx], acc );
-					}
+				for( int k = 1; k < 9; ++k ) {
+					acc = CChanVec<4>::fma( *reinterpret_cast<const float4*>( e + ( ( k / 3 ) * PW + k % 3 ) * PitchE ), f[k], acc );
 				}
 				*reinterpret_cast<float4*>( result + storeAt[pass] + c0 )
 					= make_float4( activateExpanded<CLIPPED>( acc.x, dwAct ), activateExpanded<CLIPPED>( acc.y, dwAct ),

@@ -977,6 +977,19 @@ def test_separable_blocks_without_the_expanded_tensor(case):
             assert_close(got, want, "separable block in place %s" % (case,))
 
 
+def test_fused_expand_depthwise_treats_nan_like_the_separate_launches():
+    """ReLU turns NaN into 0 (VectorReLU's rule, the vector maximum of the CPU engine): the one-launch expand + depthwise
+    stage must do so as well. The same images run in one large batch (one launch) and two at a time (three launches)."""
+    case = (16, 112, 112, 16, 96, 24, 2, False, ("relu", 6.0), ("relu", 6.0))
+    x, expand, channelwise, down, stride, residual = separable_operands(case, True, True)
+    x[:, 5, 7, 3] = np.nan
+    x[3, 111, 111, 0] = np.inf
+    whole = hip().separable_block(x, expand, channelwise, down, stride, residual)
+    parts = np.concatenate([hip().separable_block(x[i:i + 2], expand, channelwise, down, stride, residual) for i in range(0, 16, 2)])
+    assert np.isfinite(whole).all() and np.isfinite(parts).all()
+    assert_close(whole, parts, "one launch vs three launches, NaN and infinity in the input")
+
+
 @pytest.mark.parametrize("case", MOBILENETV3_CASES + [
     (4, 28, 28, 40, 120, 40, 5, 1, True, ("relu", 0.0), ("relu", 0.0), ("relu", 0.0)),
     (2, 14, 14, 80, 480, 112, 3, 1, False, ("hswish", 0.0), ("hswish", 0.0), ("hswish", 0.0)),
