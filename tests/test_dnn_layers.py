@@ -247,6 +247,21 @@ def test_optimized_separable_network_on_hip_engine():
     assert_close(got, want, "optimized network on CHipMathEngine vs plain network on CCpuMathEngine")
 
 
+@pytest.mark.gpu
+def test_optimized_separable_network_on_hip_engine_with_blocks_too_large_for_the_caches():
+    """The same network on 16 images of 224 x 224: the expanded tensors of its two CMobileNetV2BlockLayers (16 x 112 x 112 x 96,
+    77 MB) are beyond the size at which the engine runs the expand and depthwise stages as one launch (both strides)."""
+    kind, _, param = CASES["separable_net"]
+    dims = (1, 16, 1, 224, 224, 1, 3)
+    x = np.random.default_rng(0xC0FFEE + 61).uniform(-1, 1, dims).astype(np.float32)
+    want = dnn_run(nhtest.cpu_engine(), kind, dims, x, param)
+    with optimized():
+        got = dnn_run(nhtest.hip_engine(), kind, dims, x, param)
+    blocks, with1x1, chains = last_optimization()
+    assert blocks == 2
+    assert_close(got, want, "optimized network on CHipMathEngine vs plain network on CCpuMathEngine, 16 x 224 x 224")
+
+
 # the MobileNetV3-style network: squeeze-and-excite branches multiplied back through COnnxEltwiseLayer
 SQUEEZE_EXCITE_NET = (7, (1, 3, 1, 32, 40, 1, 3), 10)
 
