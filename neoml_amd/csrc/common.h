@@ -107,6 +107,21 @@ __device__ __forceinline__ float applyActivation( float v, const CFusedActivatio
 	return v;
 }
 
+// The same activation with its type fixed at compile time and the upper threshold of ReLU given as a value that is
+// +infinity when there is none: what the epilogue of a matrix product applies to every element of a tile, after one
+// decision per tile instead of one per element.
+template<int TYPE>
+__device__ __forceinline__ float applyActivationOf( float v, float reluTop )
+{
+	if constexpr( TYPE == NH_ACT_RELU ) {
+		v = v > 0.f ? v : 0.f; // NaN becomes 0, as in VectorReLU
+		v = v < reluTop ? v : reluTop;
+	} else if constexpr( TYPE == NH_ACT_HSWISH ) {
+		v = v <= -3.f ? 0.f : ( v >= 3.f ? v : v * ( v + 3.f ) * ( 1.f / 6.f ) );
+	}
+	return v;
+}
+
 // Operands are read with raw buffer loads: a 32-bit byte offset from a base held in scalar registers, and a range
 // check done by the memory unit. An offset at or above BufferBytes reads as zero, which serves as the zero padding
 // of the convolution and as the mask of tile rows / columns / k beyond the matrix, without a branch or a select.

@@ -901,37 +901,65 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			n = kh * args.RowK + r;
 		}
 		const float bias = ( args.Bias != nullptr ) ? args.Bias[n] : 0.f;
+		const float reluTop = args.Act.Param > 0.f ? args.Act.Param : __builtin_inff();
+		// Mode: 0 adds onto C with atomics ( K slices that meet in C: it was set to the free term, or left as it was when
+		// accumulating, before the launch ), 1 stores act( acc + bias ), 2 also accumulates and / or adds the residual.
+		// What is the same for the whole tile is decided once per tile, not per element: with up to eight wavefronts per SIMD
+		// a handful of branches in front of every one of a lane's 16 or 32 stores costs microseconds per launch.
+		auto write = [&]( auto modeOf, auto typeOf ) {
+			constexpr int Mode = decltype( modeOf )::value;
+			constexpr int Type = decltype( typeOf )::value;
 #pragma unroll
-		for( int mi = 0; mi < MI; ++mi ) {
+			for( int mi = 0; mi < MI; ++mi ) {
 #pragma unroll
-			for( int r = 0; r < 16; ++r ) {
-				const int m = m0 + waveM * WM + mi * 32 + ( r >> 2 ) * 8 + half * 4 + ( r & 3 );
-				if( m < M ) {
-					long long row = m;
-					if constexpr( IsClasses ) {
-						const int wo = m % args.Wo;
-						const int t = m / args.Wo;
-						const int ho = t % args.Ho;
-						row = ( static_cast<long long>( t / args.Ho ) * args.OutH + outH0 + ho * args.OutUpH ) * args.OutW
-							+ outW0 + wo * args.OutUpW;
-					}
-					float* p = C + row * args.Ldc + n;
-					if( splitK > 1 ) {
-						// C was set to the free term (or left as is when accumulating) before the launch
-						unsafeAtomicAdd( p, acc[mi][ni][r] );
-					} else {
-						float v = acc[mi][ni][r] + bias;
-						if( args.Accumulate ) {
-							v += *p;
+				for( int r = 0; r < 16; ++r ) {
+					const int m = m0 + waveM * WM + mi * 32 + ( r >> 2 ) * 8 + half * 4 + ( r & 3 );
+					if( m < M ) {
+						long long row = m;
+						if constexpr( IsClasses ) {
+							const int wo = m % args.Wo;
+							const int t = m / args.Wo;
+							const int ho = t % args.Ho;
+							row = ( static_cast<long long>( t / args.Ho ) * args.OutH + outH0 + ho * args.OutUpH ) * args.OutW
+								+ outW0 + wo * args.OutUpW;
 						}
-						v = applyActivation( v, args.Act );
-						if( args.Residual != nullptr ) {
-							v += args.Residual[batch * args.BatchStrideC + row * args.Ldc + n];
+						float* p = C + row * args.Ldc + n;
+						if constexpr( Mode == 0 ) {
+							unsafeAtomicAdd( p, acc[mi][ni][r] );
+						} else {
+							float v = acc[mi][ni][r] + bias;
+							if constexpr( Mode == 2 ) {
+								if( args.Accumulate ) {
+									v += *p;
+								}
+							}
+							v = applyActivationOf<Type>( v, reluTop );
+							if constexpr( Mode == 2 ) {
+								if( args.Residual != nullptr ) {
+									v += args.Residual[batch * args.BatchStrideC + row * args.Ldc + n];
+								}
+							}
+							*p = v;
 						}
-						*p = v;
 					}
 				}
 			}
+		};
+		auto writeAs = [&]( auto typeOf ) {
+			if( args.Accumulate || args.Residual != nullptr ) {
+				write( std::integral_constant<int, 2>(), typeOf );
+			} else {
+				write( std::integral_constant<int, 1>(), typeOf );
+			}
+		};
+		if( splitK > 1 ) {
+			write( std::integral_constant<int, 0>(), std::integral_constant<int, NH_ACT_NONE>() );
+		} else if( args.Act.Type == NH_ACT_RELU ) {
+			writeAs( std::integral_constant<int, NH_ACT_RELU>() );
+		} else if( args.Act.Type == NH_ACT_HSWISH ) {
+			writeAs( std::integral_constant<int, NH_ACT_HSWISH>() );
+		} else {
+			writeAs( std::integral_constant<int, NH_ACT_NONE>() );
 		}
 	}
 }
@@ -1946,6 +1974,329 @@ static bool tryShortReduction( hipStream_t stream, const float* a, int lda, cons
 	return true;
 }
 
+// ---- plain products with long reductions and large results -------------------------------------------------------
+// C[M x N] (+)= act( A[M x K] * B[N x K]^T + bias ) (+ residual), both operands K-major: the products of fully connected
+// layers over thousands of rows ( transformer feed-forward 8192 x 2048 x 512 and 8192 x 512 x 2048, the input product of
+// an LSTM layer 8192 x 1024 x 256 ).
+// Workgroup tile 128 x 128, K step 16, two LDS buffers of [row][16 + 4], in two shapes:
+//   eight wavefronts ( 2 x 4 ), each 64 rows x 32 columns = two 32 x 32 MFMA blocks that share their B operand; three
+//   workgroups fit a compute unit;
+//   four wavefronts ( 2 x 2 ), each 64 x 64 = four blocks; four workgroups fit a compute unit.
+// Against the 64 x 64 tile of matMulKernel every value that reaches LDS feeds twice as many MFMAs and every fragment
+// read 1.5 to 2 times as many, which on this part shows as a higher sustained clock as much as in fewer stalls, and
+// eight waves per workgroup keep two to six waves on every SIMD even when the tiles only just cover the compute units.
+// Measured against the 64 x 64 tile ( us ): 8192 x 512 x 2048 129 -> 123, 8192 x 512 x 512 39 -> 35, 8192 x 1024 x 256
+// 40 -> 36.5, 8192 x 2048 x 2048 550 -> 469 ( 146.5 TFLOP/s ) with eight wavefronts. With 1024 tiles and a reduction of 32
+// steps ( 8192 x 2048 x 512 ) the eight-wave shape runs 768 workgroups at once and the remaining 256 afterwards on a
+// device that is three quarters idle: 130 to 150 us, depending on how far the first ones had drifted apart; four
+// workgroups of four waves per compute unit hold all 1024 at once: 130 us.
+// Each thread fetches 128-bit pieces of A and B ( raw buffer loads: rows beyond the matrix read as zeros ) into SETS
+// register sets; with one set the values wait a whole step before they go to LDS, which is enough while several
+// workgroups share a compute unit; two sets pay where a compute unit holds one workgroup.
+struct CLongProductArgs {
+	const float* A;
+	const float* B;
+	float* C;
+	const float* Bias;     // per column, may be null
+	const float* Residual; // C's layout, may be null, may be C
+	int M, N, K;
+	int Lda, Ldb, Ldc;
+	long long BatchStrideA, BatchStrideB, BatchStrideC;
+	int TilesN;
+	int Accumulate;
+	CFusedActivation Act;
+};
+
+constexpr int LongTile = 128;
+
+// WGM x WGN wavefronts, each MI x NI blocks of 32 x 32; WPE: wavefronts per SIMD the registers must leave room for
+// RAGGED: K is not a multiple of the step
+template<int WGM, int WGN, int MI, int NI, int SETS, int WPE, bool RAGGED>
+__global__ __launch_bounds__( 64 * WGM * WGN, WPE )
+void longProductKernel( const CLongProductArgs args )
+{
+	constexpr int KS = NH_KSTEP, LdsK = KS + 4, KQ = KS / 4;
+	constexpr int T = 64 * WGM * WGN;
+	constexpr int BM = 32 * WGM * MI, BN = 32 * WGN * NI;
+	constexpr int ASlots = BM * KQ / T, BSlots = BN * KQ / T;
+	static_assert( KS == 16 && BM * KQ % T == 0 && BN * KQ % T == 0, "whole load slots per thread" );
+	__shared__ __attribute__( ( aligned( 16 ) ) ) float lds[2][( BM + BN ) * LdsK];
+
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = tid >> 6;
+	const int waveM = wave / WGN, waveN = wave % WGN;
+	const int l32 = lane & 31, half = lane >> 5;
+
+	const int tile = xcdSwizzle( blockIdx.x, gridDim.x );
+	const int m0 = ( tile / args.TilesN ) * BM;
+	const int n0 = ( tile % args.TilesN ) * BN;
+	const int batch = blockIdx.y;
+	const int M = args.M, N = args.N, K = args.K;
+	const float* baseA = args.A + batch * args.BatchStrideA;
+	const float* baseB = args.B + batch * args.BatchStrideB;
+
+	// load slots of this thread: tile row ( dealt so that the two rows eight neighbouring lanes store to LDS are four
+	// apart: conflict-free at a pitch of 20 floats ) and 128-bit column
+	const int kq = ( tid & 3 ) * 4;
+	auto rowOfSlot = [&]( int i ) -> int {
+		const int q = ( tid + i * T ) >> 2;
+		return ( q & ~7 ) | ( ( q & 1 ) << 2 ) | ( ( q & 6 ) >> 1 );
+	};
+	unsigned offA[ASlots], offB[BSlots];
+#pragma unroll
+	for( int i = 0; i < ASlots; ++i ) {
+		const int m = m0 + rowOfSlot( i );
+		offA[i] = m < M ? static_cast<unsigned>( m * args.Lda + kq ) * 4u : OutOfRange;
+	}
+#pragma unroll
+	for( int i = 0; i < BSlots; ++i ) {
+		const int n = n0 + rowOfSlot( i );
+		offB[i] = n < N ? static_cast<unsigned>( n * args.Ldb + kq ) * 4u : OutOfRange;
+	}
+	const int kSteps = ( K + KS - 1 ) / KS;
+	const bool inLastStep = ( kSteps - 1 ) * KS + kq < K; // RAGGED: the last step has columns beyond K, they must read as zeros
+
+	float4 rA[SETS][ASlots], rB[SETS][BSlots];
+	// Every step of the reduction, the last ones included, runs the same code with the same number of loads in flight
+	// ( the waits in front of the LDS stores count them ): a step behind the last one is requested through a descriptor of
+	// size zero, which answers with zeros without touching memory and costs two scalar instructions. No vector
+	// instruction: a wave's vector instructions wait for its MFMAs in flight, and two selects per step on the lanes'
+	// offsets cost 3 % ( 8192 x 2048 x 2048: 469 -> 484 us ). Only a K that ends inside a step ( RAGGED, a kernel of its
+	// own ) pays them, for the per-lane mask of its last step.
+	auto load = [&]( int step, int set ) {
+		const unsigned uni = static_cast<unsigned>( step ) * ( KS * 4u );
+		const unsigned range = step < kSteps ? BufferBytes : 0u;
+		const __amdgpu_buffer_rsrc_t bufA = __builtin_amdgcn_make_buffer_rsrc( const_cast<float*>( baseA ), 0, range, 0x00020000 );
+		const __amdgpu_buffer_rsrc_t bufB = __builtin_amdgcn_make_buffer_rsrc( const_cast<float*>( baseB ), 0, range, 0x00020000 );
+		const bool masked = RAGGED && step == kSteps - 1 && !inLastStep;
+#pragma unroll
+		for( int i = 0; i < ASlots; ++i ) {
+			rA[set][i] = bufferLoad4( bufA, masked ? OutOfRange : offA[i], uni );
+		}
+#pragma unroll
+		for( int i = 0; i < BSlots; ++i ) {
+			rB[set][i] = bufferLoad4( bufB, masked ? OutOfRange : offB[i], uni );
+		}
+	};
+	auto store = [&]( int buf, int set ) {
+#pragma unroll
+		for( int i = 0; i < ASlots; ++i ) {
+			*reinterpret_cast<float4*>( &lds[buf][rowOfSlot( i ) * LdsK + kq] ) = rA[set][i];
+		}
+#pragma unroll
+		for( int i = 0; i < BSlots; ++i ) {
+			*reinterpret_cast<float4*>( &lds[buf][( BM + rowOfSlot( i ) ) * LdsK + kq] ) = rB[set][i];
+		}
+	};
+
+	f32x16 acc[MI][NI];
+#pragma unroll
+	for( int mi = 0; mi < MI; ++mi ) {
+#pragma unroll
+		for( int ni = 0; ni < NI; ++ni ) {
+#pragma unroll
+			for( int r = 0; r < 16; ++r ) {
+				acc[mi][ni][r] = 0.f;
+			}
+		}
+	}
+	// fragments of one group of 8 k: lane ( l32, half ) holds k = 8 g + 4 half .. + 3 of its row, MFMA j reduces over
+	// { 8 g + j, 8 g + 4 + j } on both operands
+	struct CFrag {
+		float A[MI][4];
+		float B[NI][4];
+	};
+	CFrag frag[2];
+	const int fragA = ( waveM * 32 * MI + l32 ) * LdsK + half * 4;
+	const int fragB = ( BM + waveN * 32 * NI + l32 ) * LdsK + half * 4;
+	auto readFrag = [&]( int buf, int g, CFrag& f ) {
+#pragma unroll
+		for( int mi = 0; mi < MI; ++mi ) {
+			const float4 v = *reinterpret_cast<const float4*>( &lds[buf][fragA + mi * 32 * LdsK + g * 8] );
+			f.A[mi][0] = v.x; f.A[mi][1] = v.y; f.A[mi][2] = v.z; f.A[mi][3] = v.w;
+		}
+#pragma unroll
+		for( int ni = 0; ni < NI; ++ni ) {
+			const float4 v = *reinterpret_cast<const float4*>( &lds[buf][fragB + ni * 32 * LdsK + g * 8] );
+			f.B[ni][0] = v.x; f.B[ni][1] = v.y; f.B[ni][2] = v.z; f.B[ni][3] = v.w;
+		}
+	};
+	auto multiply = [&]( const CFrag& f ) {
+#pragma unroll
+		for( int j = 0; j < 4; ++j ) {
+#pragma unroll
+			for( int mi = 0; mi < MI; ++mi ) {
+#pragma unroll
+				for( int ni = 0; ni < NI; ++ni ) {
+					acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32( f.A[mi][j], f.B[ni][j], acc[mi][ni], 0, 0, 0 );
+				}
+			}
+		}
+	};
+
+	// Step ks multiplies out of LDS buffer ks % 2 while the operands of step ks + 1 go from registers to the other buffer
+	// and those of step ks + 1 + SETS are requested. The one barrier of a step sits between its two groups of 8 k: the
+	// second group's fragments were fetched ahead of it, so behind it nobody reads the buffer any more ( it is the one
+	// the next step stores to ), and the first fragments of the next step are fetched right behind it.
+	constexpr int Ahead = SETS + 1;
+	auto step = [&]( int ks, auto parity ) {
+		constexpr int nxt = decltype( parity )::value; // == ( ks + 1 ) % 2
+		constexpr int cur = nxt ^ 1;
+		constexpr int set = SETS == 2 ? nxt : 0;
+		store( nxt, set ); // ( behind the last step: zeros that nobody multiplies )
+		load( ks + Ahead, set );
+		__builtin_amdgcn_sched_barrier( 0 );
+		readFrag( cur, 1, frag[1] );
+		__builtin_amdgcn_sched_barrier( 0 );
+		multiply( frag[0] );
+		__builtin_amdgcn_sched_barrier( 0 );
+		__syncthreads();
+		readFrag( nxt, 0, frag[0] );
+		__builtin_amdgcn_sched_barrier( 0 );
+		multiply( frag[1] );
+		__builtin_amdgcn_sched_barrier( 0 );
+	};
+
+	load( 0, 0 );
+	store( 0, 0 );
+	if( SETS == 2 ) {
+		load( 1, 1 );
+		load( 2, 0 );
+	} else {
+		load( 1, 0 );
+	}
+	__syncthreads();
+	readFrag( 0, 0, frag[0] );
+	int ks = 0;
+	for( ; ks + 1 < kSteps; ks += 2 ) {
+		step( ks, std::integral_constant<int, 1>() );
+		step( ks + 1, std::integral_constant<int, 0>() );
+	}
+	if( ks < kSteps ) {
+		step( ks, std::integral_constant<int, 1>() );
+	}
+
+	// lane ( l32, half ) holds, of each block, one column of rows ( r / 4 ) * 8 + half * 4 + r % 4
+	float* C = args.C + batch * args.BatchStrideC;
+	const float* residual = args.Residual != nullptr ? args.Residual + batch * args.BatchStrideC : nullptr;
+	const float reluTop = args.Act.Param > 0.f ? args.Act.Param : __builtin_inff();
+	const bool accumulate = args.Accumulate != 0;
+	const int rowBase = m0 + waveM * 32 * MI + half * 4;
+	// what is the same for the whole tile is decided once, here, and not per element: 32 or 64 elements per lane and up
+	// to six wavefronts per SIMD make an epilogue with a handful of branches per element cost microseconds
+	auto write = [&]( auto typeOf, auto extraOf, auto checkedOf ) {
+		constexpr int Type = decltype( typeOf )::value;
+		constexpr bool Extra = decltype( extraOf )::value;     // accumulate and / or residual
+		constexpr bool Checked = decltype( checkedOf )::value; // the tile hangs over the last row
+#pragma unroll
+		for( int ni = 0; ni < NI; ++ni ) {
+			const int n = n0 + waveN * 32 * NI + ni * 32 + l32;
+			if( n >= N ) {
+				continue;
+			}
+			const float bias = args.Bias != nullptr ? args.Bias[n] : 0.f;
+#pragma unroll
+			for( int mi = 0; mi < MI; ++mi ) {
+#pragma unroll
+				for( int r = 0; r < 16; ++r ) {
+					const int m = rowBase + mi * 32 + ( r >> 2 ) * 8 + ( r & 3 );
+					if( !Checked || m < M ) {
+						const long long at = static_cast<long long>( m ) * args.Ldc + n;
+						float v = acc[mi][ni][r] + bias;
+						if constexpr( Extra ) {
+							if( accumulate ) {
+								v += C[at];
+							}
+						}
+						v = applyActivationOf<Type>( v, reluTop );
+						if constexpr( Extra ) {
+							if( residual != nullptr ) {
+								v += residual[at];
+							}
+						}
+						C[at] = v;
+					}
+				}
+			}
+		}
+	};
+	auto writeAs = [&]( auto typeOf ) {
+		if( accumulate || residual != nullptr ) {
+			write( typeOf, std::true_type(), std::true_type() );
+		} else if( m0 + BM > M ) {
+			write( typeOf, std::false_type(), std::true_type() );
+		} else {
+			write( typeOf, std::false_type(), std::false_type() );
+		}
+	};
+	if( args.Act.Type == NH_ACT_RELU ) {
+		writeAs( std::integral_constant<int, NH_ACT_RELU>() );
+	} else if( args.Act.Type == NH_ACT_HSWISH ) {
+		writeAs( std::integral_constant<int, NH_ACT_HSWISH>() );
+	} else {
+		writeAs( std::integral_constant<int, NH_ACT_NONE>() );
+	}
+}
+
+// true ( and launched ) when the product is one this kernel is for: vector loads possible, a reduction of at least eight
+// steps, and enough 128 x 128 tiles to give every compute unit the same number of workgroups to within a quarter ( results
+// with fewer tiles, or tiles that would be mostly padding, stay with the 64 x 64 tiles and their K slices )
+static bool tryLongProduct( hipStream_t stream, const CMatMulArgs& a, int batch, bool vec, int* rc )
+{
+	if( !vec || a.K < 8 * NH_KSTEP || a.M < LongTile || a.N < LongTile / 2 || batch > 65535 ) {
+		return false;
+	}
+	const long long tilesM = ceilDiv( a.M, LongTile ), tilesN = ceilDiv( a.N, LongTile );
+	const long long tiles = tilesM * tilesN * batch;
+	if( tilesM * tilesN > 0x7fffffffLL ) {
+		return false;
+	}
+	const double covered = static_cast<double>( a.M ) * a.N / ( static_cast<double>( tilesM * LongTile ) * ( tilesN * LongTile ) );
+	const long long unitsAtOnce = 256;
+	const long long deepest = ( tiles + unitsAtOnce - 1 ) / unitsAtOnce;
+	const double balance = static_cast<double>( tiles ) / static_cast<double>( deepest * unitsAtOnce );
+	if( covered < 0.85 || ( tiles < 3 * unitsAtOnce && balance < 0.75 ) ) {
+		return false;
+	}
+	CLongProductArgs args = {};
+	args.A = a.A; args.B = a.B; args.C = a.C; args.Bias = a.Bias; args.Residual = a.Residual;
+	args.M = a.M; args.N = a.N; args.K = a.K;
+	args.Lda = a.Lda; args.Ldb = a.Ldb; args.Ldc = a.Ldc;
+	args.BatchStrideA = a.BatchStrideA; args.BatchStrideB = a.BatchStrideB; args.BatchStrideC = a.BatchStrideC;
+	args.TilesN = static_cast<int>( tilesN );
+	args.Accumulate = a.Accumulate;
+	args.Act = a.Act;
+	const dim3 grid( static_cast<unsigned>( tilesM * tilesN ), batch );
+	const int kSteps = ceilDiv( a.K, NH_KSTEP );
+	auto launch = [&]( auto ragged ) {
+		constexpr bool Ragged = decltype( ragged )::value;
+		if( tiles <= unitsAtOnce ) {
+			// one workgroup per compute unit: two waves per SIMD, the operands get two steps to arrive
+			hipLaunchKernelGGL( ( longProductKernel<2, 4, 2, 1, 2, 4, Ragged> ), grid, dim3( 512 ), 0, stream, args );
+		} else if( tiles > 3 * unitsAtOnce && tiles <= 4 * unitsAtOnce && kSteps <= 64 ) {
+			// more than the three workgroups of eight waves that fit a compute unit, and a reduction too short for them
+			// to drift apart: four workgroups of four waves hold all the tiles at once
+			hipLaunchKernelGGL( ( longProductKernel<2, 2, 2, 2, 1, 4, Ragged> ), grid, dim3( 256 ), 0, stream, args );
+		} else {
+			hipLaunchKernelGGL( ( longProductKernel<2, 4, 2, 1, 1, 6, Ragged> ), grid, dim3( 512 ), 0, stream, args );
+		}
+	};
+	if( a.K % NH_KSTEP != 0 ) {
+		launch( std::true_type() );
+	} else {
+		launch( std::false_type() );
+	}
+	const hipError_t err = hipGetLastError();
+	if( err != hipSuccess ) {
+		setLastError( "long product: launch failed: %s", hipGetErrorString( err ) );
+		*rc = NH_ERR_HIP;
+	} else {
+		*rc = NH_OK;
+	}
+	return true;
+}
+
 // C = A * B^T (+ bias) with row strides; also the inner product of the convolution with a 1x1 filter.
 int matMulNTFused( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
 	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC,
@@ -1993,6 +2344,9 @@ static int matMulNTMeeting( hipStream_t stream, const float* a, int lda, const f
 	}
 	const bool vec = isAligned16( a ) && isAligned16( b ) && K % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0
 		&& strideA % 4 == 0 && strideB % 4 == 0 && fitsBuffer( M, lda, K ) && fitsBuffer( N, ldb, K );
+	if( fixedMeeting == nullptr && tryLongProduct( stream, args, batch, vec, &rc ) ) {
+		return rc;
+	}
 	return launchMatMul<AM_RowsK, BM_RowsK>( stream, args, batch, vec, fixedMeeting );
 }
 

@@ -232,6 +232,51 @@ def test_matmul_strided(shape):
         assert_close(hip().matmul("tn_add", at, bn, **kw), orc.matmul("tn_add", at, bn, **kw), "tn_add %s" % (shape,))
 
 
+# results of a few hundred 128 x 128 tiles with reductions of eight steps and more: the tile of eight wavefronts. Rows
+# and columns that end inside a tile, reductions that end inside a step ( multiples of 4: the vector path ), row strides
+# with padding, exactly one workgroup per compute unit ( two sets of load registers ) and more
+LONG_PRODUCT_SHAPES = [(2000, 1990, 264), (2048, 2048, 128), (3000, 2040, 132), (1990, 2000, 1000), (8192, 512, 520),
+                       (1200, 4000, 136), (4096, 1024, 2048)]
+
+
+@pytest.mark.parametrize("shape", LONG_PRODUCT_SHAPES)
+def test_matmul_long_products(shape):
+    M, N, K = shape
+    g = rng(77 + M + K)
+    for pad_a, pad_b, pad_c in ((0, 0, 0), (4, 8, 3)):
+        a = g.uniform(-1, 1, (M, K + pad_a)).astype(np.float32)
+        b = g.uniform(-1, 1, (N, K + pad_b)).astype(np.float32)
+        kw = dict(lda=K + pad_a, ldb=K + pad_b, ldc=N + pad_c, M=M, N=N, K=K)
+        got, want = hip().matmul("nt", a, b, **kw), orc.matmul("nt", a, b, **kw)
+        # sums of K products of values below one: two summation orders differ by a few ulps of sqrt( K )
+        assert_close(got, want, "nt %s pads %s" % (shape, (pad_a, pad_b, pad_c)), atol=1e-5 * max(1.0, np.sqrt(K / 64.0)))
+        if pad_c:
+            continue
+        # every k counted exactly once, every row and column in its place: a one-hot A picks columns of B
+        a[:] = 0
+        a[np.arange(M), (np.arange(M) * 7) % K] = 1
+        got = hip().matmul("nt", a, b, **kw).reshape(M, N)
+        assert np.array_equal(got, b[:, (np.arange(M) * 7) % K].T)
+
+
+def test_matmul_long_product_batched_and_fused():
+    # the same tile behind the batched entry point and behind the pointwise convolution with its epilogue
+    g = rng(78)
+    batch, M, N, K = 3, 1024, 1100, 160
+    a = g.uniform(-1, 1, (batch, M, K)).astype(np.float32)
+    bt = g.uniform(-1, 1, (batch, N, K)).astype(np.float32)
+    kw = dict(M=M, N=N, K=K, batch=batch)
+    assert_close(hip().matmul("bnt", a, bt, **kw), orc.matmul("bnt", a, bt, **kw), "bnt long")
+    # free term, residual and no activation in the epilogue: the down convolution of a gated block, 12 544 pixels 128 -> 256
+    n, h, w, c, cout = 4, 56, 56, 128, 256
+    x = g.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    gate = g.uniform(0, 1, (n, c)).astype(np.float32)
+    res = g.uniform(-1, 1, (n, h, w, cout)).astype(np.float32)
+    down = (g.normal(0, 0.1, (cout, c)).astype(np.float32), g.uniform(-1, 1, cout).astype(np.float32))
+    assert_close(hip().mobilenetv3_post_se(x, gate, res, "hswish", 0.0, down),
+                 orc.mobilenetv3_post_se(x, gate, res, "hswish", 0.0, down), "down convolution with residual, long tile", atol=2e-5)
+
+
 def test_matmul_k_halves_in_one_workgroup():
     # 448 tiles and 32 K steps: the two halves of K run in the two wave groups of one workgroup. Positive operands: over
     # 1.8 M sums of 512 products the few that cancel to almost nothing would otherwise sit at the edge of the absolute bar
