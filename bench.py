@@ -103,7 +103,7 @@ def cdnn_run_once(batch, image):
 def other_workload(args):
     """BASELINE configurations 3-5 at full size: same replay + event method, one JSON line with the per-family split."""
     import torch
-    from neoml_amd.workloads import HipBackend, MobileNetV2, TransformerEncoder, LineRecognizer
+    from workloads import HipBackend, MobileNetV2, TransformerEncoder, LineRecognizer
     be = HipBackend()
     if args.workload == "mobilenetv2":
         net = MobileNetV2(be, batch=args.batch or 128, image=args.image, fused=args.fused)
@@ -184,7 +184,7 @@ def main():
         args.batch = 64
 
     import torch
-    from neoml_amd.workloads import HipBackend, ResNet18
+    from workloads import HipBackend, ResNet18
 
     be = HipBackend()
     net = ResNet18(be, batch=args.batch, image=args.image, fused=args.fused)

@@ -1,6 +1,6 @@
 """Per-kernel measurements at the sizes of the BASELINE configurations.
 
-    python -m neoml_amd.kernel_bench [--reps N] [--filter substring[,substring...]]
+    python kernel_bench.py [--reps N] [--filter substring[,substring...]]
 
 Every line is one C-ABI entry point at one shape: time per launch (events on the launch stream around a run of
 back-to-back launches, after a clock warm-up), algorithmic FLOP and bytes (the formulas of the measurement

@@ -1512,13 +1512,18 @@ struct CSequenceStream {
 	bool Launched = false;      // a one-launch LSTM was issued since the word was last looked at
 };
 
+// `Last` is the one-launch LSTM issued last on the device ( not counting partners ), `Older` the one in front of it. Each
+// may have a partner that runs beside it on a side stream, with a completion event of its own. A launch is ordered
+// behind Last and Last's partner; a partner behind Older and Older's partner. Generation counts the launches that are
+// not partners: a second nhLstm call may only become the partner of the launch it follows on its stream while that
+// launch is still the device's last one, i.e. while no other stream, thread or engine has issued one in between ( such
+// a launch waits for Last only: it would run beside the partner, and it may be a whole-device grid ).
 struct CSequenceDevice {
-	hipEvent_t LastDone = nullptr;
+	hipEvent_t LastDone = nullptr, LastPartnerDone = nullptr;
+	hipEvent_t OlderDone = nullptr, OlderPartnerDone = nullptr;
+	bool Any = false, AnyLastPartner = false, AnyOlder = false, AnyOlderPartner = false;
 	hipStream_t LastStream = nullptr;
-	bool Any = false;
-	// the one before the last: what the partner of an overlapped pair waits for instead of its own partner
-	hipEvent_t OlderDone = nullptr;
-	bool AnyOlder = false;
+	unsigned long long Generation = 0;
 };
 
 // Two one-launch LSTMs side by side ( nhStreamOverlapLstm ): the two directions of a bidirectional layer read the same
@@ -1539,6 +1544,7 @@ struct CLstmOverlap {
 	hipEvent_t Before = nullptr;   // recorded on the main stream in front of a one-launch LSTM
 	hipEvent_t SideDone = nullptr; // recorded on the side stream behind its LSTM
 	bool LastWasLstm = false;      // that LSTM was the last thing enqueued on the main stream
+	unsigned long long Generation = 0; // ... and this was the device's launch count right behind it
 	CByteRange Written[3];         // what it writes: results, workspace
 	CByteRange Read[4];            // what it reads: input, initial states ( the weights are constant )
 };
@@ -1640,8 +1646,9 @@ void releaseSequenceStream( hipStream_t stream )
 	}
 	auto dev = sequenceDevices().find( device );
 	if( dev != sequenceDevices().end() && dev->second.LastStream == stream ) {
-		dev->second.Any = false; // drained: nothing of it is in flight
-		dev->second.AnyOlder = false;
+		// drained: nothing of it is in flight, nor anything it had waited for
+		dev->second.Any = dev->second.AnyLastPartner = false;
+		dev->second.AnyOlder = dev->second.AnyOlderPartner = false;
 	}
 	auto overlap = lstmOverlaps().find( std::make_pair( device, stream ) );
 	if( overlap != lstmOverlaps().end() ) {
@@ -1780,8 +1787,11 @@ static bool lstmSequenceAllowed( hipStream_t stream )
 }
 
 // halfDevice: a grid of at most half the compute units if there is such a shape ( *tookHalf says whether ).
-// partner: this launch runs beside the one issued last ( its partner, on the main stream ) instead of behind it.
-static int launchLstmSequence( hipStream_t stream, CLstmSeqArgs a, bool halfDevice = false, bool partner = false, bool* tookHalf = nullptr )
+// partnerOf: not null = this launch, on a side stream, wants to run beside the launch that made the device's count
+// *partnerOf; it does if that launch is still the device's last one and has no partner yet ( *ranBeside ), otherwise it
+// is ordered like any other launch. *generation receives the device's count behind a launch that is not a partner.
+static int launchLstmSequence( hipStream_t stream, CLstmSeqArgs a, bool halfDevice = false, const unsigned long long* partnerOf = nullptr,
+	bool* tookHalf = nullptr, unsigned long long* generation = nullptr, bool* ranBeside = nullptr )
 {
 	const CLstmSeqShape* shape = lstmSequenceShape( a.H, a.B, halfDevice );
 	NH_REQUIRE( shape != nullptr );
@@ -1794,7 +1804,6 @@ static int launchLstmSequence( hipStream_t stream, CLstmSeqArgs a, bool halfDevi
 	if( tookHalf != nullptr ) {
 		*tookHalf = isHalf;
 	}
-	NH_REQUIRE( !partner || isHalf );
 	std::lock_guard<std::mutex> guard( sequenceLock );
 	CSequenceStream& own = sequenceStreams()[std::make_pair( device, stream )];
 	if( own.GaveUp == nullptr ) {
@@ -1807,15 +1816,30 @@ static int launchLstmSequence( hipStream_t stream, CLstmSeqArgs a, bool halfDevi
 	if( dev.LastDone == nullptr ) {
 		NH_HIP( hipEventCreateWithFlags( &dev.LastDone, hipEventDisableTiming ) );
 		NH_HIP( hipEventCreateWithFlags( &dev.OlderDone, hipEventDisableTiming ) );
+		NH_HIP( hipEventCreateWithFlags( &dev.LastPartnerDone, hipEventDisableTiming ) );
+		NH_HIP( hipEventCreateWithFlags( &dev.OlderPartnerDone, hipEventDisableTiming ) );
+	}
+	const bool partner = partnerOf != nullptr && isHalf && dev.Any && dev.Generation == *partnerOf && !dev.AnyLastPartner;
+	if( ranBeside != nullptr ) {
+		*ranBeside = partner;
 	}
 	if( partner ) {
-		// beside the one issued last, behind the one in front of that
+		// beside the one issued last, behind the one in front of that and its partner
 		if( dev.AnyOlder ) {
 			NH_HIP( hipStreamWaitEvent( stream, dev.OlderDone, 0 ) );
 		}
-	} else if( dev.Any ) {
-		// behind the one-launch LSTM issued last, whichever stream it went to ( on the same stream the wait is free )
-		NH_HIP( hipStreamWaitEvent( stream, dev.LastDone, 0 ) );
+		if( dev.AnyOlderPartner ) {
+			NH_HIP( hipStreamWaitEvent( stream, dev.OlderPartnerDone, 0 ) );
+		}
+	} else {
+		// behind the one-launch LSTM issued last and its partner, whichever streams they went to ( on the same stream
+		// the wait is free )
+		if( dev.Any ) {
+			NH_HIP( hipStreamWaitEvent( stream, dev.LastDone, 0 ) );
+		}
+		if( dev.AnyLastPartner ) {
+			NH_HIP( hipStreamWaitEvent( stream, dev.LastPartnerDone, 0 ) );
+		}
 	}
 	a.GaveUp = own.GaveUp;
 	own.Launched = true;
@@ -1825,27 +1849,23 @@ static int launchLstmSequence( hipStream_t stream, CLstmSeqArgs a, bool halfDevi
 	hipLaunchKernelGGL( clearWordsKernel, dim3( static_cast<unsigned>( ( words + 1023 ) / 1024 ) ), dim3( 256 ), 0, stream, a.Exchange, words );
 	shape->Launch( stream, groups, lstmSequenceLds( a.H, *shape ), a );
 	NH_LAUNCH_CHECK();
-	if( !partner ) {
-		// ( a partner's completion is recorded by its caller, on the main stream, once that stream waits for both )
+	if( partner ) {
+		NH_HIP( hipEventRecord( dev.LastPartnerDone, stream ) );
+		dev.AnyLastPartner = true;
+	} else {
 		std::swap( dev.LastDone, dev.OlderDone );
+		std::swap( dev.LastPartnerDone, dev.OlderPartnerDone );
 		dev.AnyOlder = dev.Any;
+		dev.AnyOlderPartner = dev.AnyLastPartner;
 		NH_HIP( hipEventRecord( dev.LastDone, stream ) );
 		dev.LastStream = stream;
 		dev.Any = true;
+		dev.AnyLastPartner = false;
+		++dev.Generation;
+		if( generation != nullptr ) {
+			*generation = dev.Generation;
+		}
 	}
-	return NH_OK;
-}
-
-// both LSTMs of a pair are behind the main stream's last wait: later one-launch LSTMs wait for this point
-static int recordPairDone( hipStream_t mainStream )
-{
-	int device = 0;
-	NH_HIP( hipGetDevice( &device ) );
-	std::lock_guard<std::mutex> guard( sequenceLock );
-	CSequenceDevice& dev = sequenceDevices()[device];
-	NH_HIP( hipEventRecord( dev.LastDone, mainStream ) );
-	dev.LastStream = mainStream;
-	dev.Any = true;
 	return NH_OK;
 }
 
@@ -2774,16 +2794,18 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 		a.Abort = reinterpret_cast<unsigned*>( a.Exchange + 2 * static_cast<size_t>( B ) * H );
 		a.T = T; a.B = B; a.H = H; a.Reverse = reverse ? 1 : 0;
 		a.MaxSpins = lstmSpinLimit();
-		bool tookHalf = false;
-		rc = launchLstmSequence( stream, a, overlapEnabled, beside, &tookHalf );
+		bool tookHalf = false, ranBeside = false;
+		unsigned long long generation = 0;
+		rc = launchLstmSequence( stream, a, overlapEnabled, beside ? &pair.Generation : nullptr, &tookHalf, &generation, &ranBeside );
 		if( rc != NH_OK ) {
 			return rc;
 		}
 		if( beside ) {
-			// the main stream goes on behind both
+			// the main stream goes on behind both ( also where another stream's launch had come in between and this one
+			// ran behind it instead of beside its partner: it is on the side stream all the same )
 			NH_HIP( hipEventRecord( pair.SideDone, stream ) );
 			NH_HIP( hipStreamWaitEvent( mainStream, pair.SideDone, 0 ) );
-			return recordPairDone( mainStream );
+			return NH_OK;
 		}
 		if( overlapEnabled && tookHalf ) {
 			int device = 0;
@@ -2793,6 +2815,7 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 			if( found != lstmOverlaps().end() ) {
 				CLstmOverlap& o = found->second;
 				o.LastWasLstm = true;
+				o.Generation = generation;
 				for( int i = 0; i < 3; ++i ) {
 					o.Written[i] = written[i];
 					o.Read[i] = read[i];

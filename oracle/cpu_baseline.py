@@ -37,7 +37,7 @@ def main():
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import numpy as np
     import nhtest
-    from neoml_amd.workloads import ResNet18
+    from workloads import ResNet18
 
     kind = "ref" if nhtest.have_reference() else "orc"
     be = nhtest.CpuBackend(kind)

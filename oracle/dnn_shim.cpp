@@ -8,10 +8,13 @@
 #include <NeoML/Dnn/Layers/Onnx/OnnxEltwiseLayer.h>
 #include "HipLstmLayer.h" // neoml_amd/engine: the LSTM layer that reaches IMathEngine::Lstm on a non-CPU engine
 
+#include <atomic>
 #include <chrono>
 #include <exception>
 #include <string>
 #include <string.h>
+#include <thread>
+#include <vector>
 
 using namespace NeoML;
 
@@ -423,6 +426,118 @@ EXPORT int dnn_run( void* engine, int kind, int seed, int param, const int* dims
 		lastError = "unknown exception";
 	}
 	return 3;
+}
+
+// The engine interface from several threads at once ( the reference: "the math engine interface is thread-safe; the same
+// instance may be used in different networks and different threads", README.md:116-118; its own idiom is one engine and
+// one CDnn per thread, NeoML/test/src/InferencePerformanceMultiThreadingTest.cpp:236-262 ).
+// Thread t builds network kinds[t] ( dnn_run's kinds, params[t] ) on engines[t] - all the same engine, or one each -
+// and runs `passes` forward passes over its own input, all threads released together; between the passes it asks the
+// engine for its peak memory and calls CleanUp(), so that those run while the other threads' launches are in flight.
+// outputs[t] receives the result of thread t's last pass. dims: 7 per thread; outputDims: 7 per thread.
+// Returns 0, or 1 + the index of the first thread that failed ( dnn_last_error() then holds its message ).
+EXPORT int dnn_run_threads( int threads, void* const* engines, const int* kinds, const int* params, int seed, const int* dims,
+	const float* const* inputs, float* const* outputs, const int* capacities, int* outputDims, int passes )
+{
+	std::vector<std::string> errors( threads );
+	std::vector<int> codes( threads, 0 );
+	std::atomic<int> ready( 0 );
+	std::atomic<bool> go( false );
+	auto body = [&]( int t ) {
+		bool counted = false; // in `ready`: a thread that fails while building must not leave the others waiting for ever
+		try {
+			IMathEngine& e = *static_cast<IMathEngine*>( engines[t] );
+			CRandom random( seed );
+			CDnn dnn( random, e );
+			CPtr<CSourceLayer> source = new CSourceLayer( e );
+			source->SetName( "source" );
+			dnn.AddLayer( *source );
+			CBaseLayer* last = nullptr;
+			switch( kinds[t] ) {
+				case 0: last = buildCnn( dnn, e, *source ); break;
+				case 1: last = buildTransformer( dnn, e, *source, params[t] ); break;
+				case 2: last = buildLstm( dnn, e, *source, params[t] ); break;
+				case 3: last = buildResNetBlock( dnn, e, *source ); break;
+				case 4: last = buildRecognizerTail( dnn, e, *source, params[t] ); break;
+				case 5: last = buildResNet18( dnn, e, *source, params[t] ); break;
+				case 6: last = buildSeparableNet( dnn, e, *source, params[t] ); break;
+				default: errors[t] = "unknown network kind"; codes[t] = 1; break;
+			}
+			CPtr<CSinkLayer> sink;
+			if( codes[t] == 0 ) {
+				sink = new CSinkLayer( e );
+				sink->SetName( "sink" );
+				sink->Connect( *last );
+				dnn.AddLayer( *sink );
+				CBlobDesc desc( CT_Float );
+				for( int d = 0; d < 7; ++d ) {
+					desc.SetDimSize( d, dims[7 * t + d] );
+				}
+				CPtr<CDnnBlob> blob = CDnnBlob::CreateBlob( e, CT_Float, desc );
+				blob->CopyFrom( inputs[t] );
+				source->SetBlob( blob );
+			}
+			// every thread has built its network: from here on they all run at once
+			counted = true;
+			ready.fetch_add( 1 );
+			while( !go.load() ) {
+				std::this_thread::yield();
+			}
+			if( codes[t] != 0 ) {
+				return;
+			}
+			size_t peak = 0;
+			for( int pass = 0; pass < passes; ++pass ) {
+				dnn.RunOnce();
+				peak = e.GetPeakMemoryUsage() > peak ? e.GetPeakMemoryUsage() : peak;
+				e.CleanUp();
+			}
+			const CPtr<CDnnBlob>& result = sink->GetBlob();
+			for( int d = 0; d < 7; ++d ) {
+				outputDims[7 * t + d] = result->DimSize( d );
+			}
+			if( peak == 0 ) {
+				errors[t] = "GetPeakMemoryUsage returned zero while a network was running";
+				codes[t] = 4;
+			} else if( result->GetDataSize() > capacities[t] ) {
+				errors[t] = "output buffer too small";
+				codes[t] = 2;
+			} else {
+				result->CopyTo( outputs[t] );
+			}
+		} catch( std::exception& ex ) {
+			errors[t] = ex.what();
+			codes[t] = 3;
+		} catch( CException* ex ) {
+			errors[t] = "NeoML exception";
+			codes[t] = 3;
+			delete ex;
+		} catch( ... ) {
+			errors[t] = "unknown exception";
+			codes[t] = 3;
+		}
+		if( !counted ) {
+			ready.fetch_add( 1 );
+		}
+	};
+	std::vector<std::thread> pool;
+	for( int t = 0; t < threads; ++t ) {
+		pool.emplace_back( body, t );
+	}
+	while( ready.load() < threads ) {
+		std::this_thread::yield();
+	}
+	go.store( true );
+	for( std::thread& th : pool ) {
+		th.join();
+	}
+	for( int t = 0; t < threads; ++t ) {
+		if( codes[t] != 0 ) {
+			lastError = "thread " + std::to_string( t ) + ": " + errors[t];
+			return 1 + t;
+		}
+	}
+	return 0;
 }
 
 // Training: a small classifier, CCrossEntropyLossLayer on float labels, CDnnSimpleGradientSolver (momentum 0.9),

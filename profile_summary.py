@@ -1,7 +1,7 @@
 """Reduces rocprofv3 output (the rocpd SQLite database it writes, `<name>_results.db`) to the text tables kept under
 profiles/.
 
-    python -m neoml_amd.profile_summary <results.db> [<results.db> ...] [--match substring[,substring...]] [--demangle]
+    python profile_summary.py <results.db> [<results.db> ...] [--match substring[,substring...]] [--demangle]
 
 Per database it prints
   * the kernel table: per (kernel, grid) the number of dispatches, the average and the total duration, and the share of

@@ -1120,7 +1120,7 @@ class Hip:
 
 
 class CpuBackend:
-    """Host backend for neoml_amd.workloads: the same network code on numpy arrays, executed by the oracle
+    """Host backend for workloads: the same network code on numpy arrays, executed by the oracle
     ('orc') or by the reference's CPU engine ('ref')."""
 
     def __init__(self, kind):

@@ -176,6 +176,101 @@ def test_hip_lstm_layer_matches_clstmlayer(name):
         assert labels == dnn_run_ctc(nhtest.cpu_engine(), dims, x, param)
 
 
+# ---------------------------------------------------------------------------------------------------------
+# Threads. "The math engine interface is thread-safe; the same instance may be used in different networks and different
+# threads" (the reference's README.md:116-118); its own idiom is one engine and one CDnn per thread
+# (NeoML/test/src/InferencePerformanceMultiThreadingTest.cpp:236-262). Both are run here: every thread builds its own
+# CDnn, all threads run their passes at once, calling GetPeakMemoryUsage() and CleanUp() between passes, and every
+# thread's result must be what the same network gives when it runs alone.
+
+THREAD_CASES = [
+    # kind, input dims, param: the small ResNet, the BiLSTM tail of the recogniser at its real width (CHipLstmLayer:
+    # the one-launch LSTM, both directions side by side), a transformer encoder layer, the small CNN
+    (5, (1, 2, 1, 64, 64, 1, 3), 100),
+    (4, (32, 64, 1, 1, 1, 1, 256), 100),
+    (1, (1, 3, 24, 1, 1, 1, 32), 32),
+    (0, (1, 3, 1, 16, 20, 1, 8), 0),
+]
+
+
+def thread_inputs():
+    g = np.random.default_rng(0xC0FFEE + 77)
+    return [g.uniform(-1, 1, dims).astype(np.float32) for _, dims, _ in THREAD_CASES]
+
+
+def dnn_run_threads(engines, inputs, passes=4, seed=451):
+    n = len(THREAD_CASES)
+    outs = [np.empty(1 << 20, np.float32) for _ in range(n)]
+    out_dims = np.zeros(7 * n, np.int32)
+    rc = lib().dnn_run_threads(
+        n, (ctypes.c_void_p * n)(*[e.value for e in engines]), ip(i32([c[0] for c in THREAD_CASES])),
+        ip(i32([c[2] for c in THREAD_CASES])), seed, ip(i32(np.concatenate([c[1] for c in THREAD_CASES]))),
+        (ctypes.c_void_p * n)(*[x.ctypes.data for x in inputs]), (ctypes.c_void_p * n)(*[o.ctypes.data for o in outs]),
+        ip(i32([o.size for o in outs])), ip(out_dims), passes)
+    if rc != 0:
+        raise RuntimeError("dnn_run_threads: %s" % lib().dnn_last_error().decode())
+    return [o[:int(np.prod(out_dims[7 * t:7 * t + 7]))].copy() for t, o in enumerate(outs)]
+
+
+def alone(engine, inputs):
+    return [dnn_run(engine, kind, dims, x, param).ravel() for (kind, dims, param), x in zip(THREAD_CASES, inputs)]
+
+
+@pytest.mark.gpu
+def test_four_threads_share_one_engine():
+    """Four threads, four networks, ONE CHipMathEngine: the same stream, pool and scratch under all of them. The kernels
+    on this path are deterministic (K slices meet in a fixed order), so every result must be bit for bit what the
+    network gives alone; any give-up of a one-launch LSTM would surface as an exception from the read-back."""
+    inputs = thread_inputs()
+    engine = nhtest.hip_engine()
+    with fused_lstm(256):
+        want = alone(engine, inputs)
+        for _ in range(2):
+            got = dnn_run_threads([engine] * len(THREAD_CASES), inputs)
+            for t, (a, b) in enumerate(zip(got, want)):
+                assert np.array_equal(a, b), "thread %d differs from the single-threaded run (max |diff| %g)" % (t, np.abs(a - b).max())
+        # ... and against the reference engine
+        cpu = alone(nhtest.cpu_engine(), inputs)
+    for t, (a, b) in enumerate(zip(got, cpu)):
+        assert_close(a, b, "thread %d vs the CPU engine" % t)
+
+
+@pytest.mark.gpu
+def test_one_engine_per_thread_on_one_device():
+    """The reference's idiom: every thread its own engine (own stream, own pool) on the one GPU. The one-launch LSTMs of
+    different engines are ordered behind one another on the device, their give-up words belong to their own streams:
+    every thread's read-back, which checks its own stream's word, must come back clean and with the right numbers."""
+    inputs = thread_inputs()
+    elib = ctypes.CDLL(nhtest.ENGINE_LIB, mode=ctypes.RTLD_GLOBAL)
+    first = nhtest.hip_engine()
+    elib.CreateHipMathEngine.restype = ctypes.c_void_p
+    elib.CreateHipMathEngine.argtypes = [ctypes.c_int, ctypes.c_size_t, ctypes.c_int]
+    extra = [ctypes.c_void_p(elib.CreateHipMathEngine(0, 0, 0)) for _ in range(len(THREAD_CASES) - 1)]
+    assert all(e.value for e in extra)
+    try:
+        with fused_lstm(256):
+            want = alone(first, inputs)
+            for _ in range(2):
+                got = dnn_run_threads([first] + extra, inputs)
+                for t, (a, b) in enumerate(zip(got, want)):
+                    assert np.array_equal(a, b), "thread %d differs from the single-threaded run (max |diff| %g)" % (t, np.abs(a - b).max())
+            # two engines, both running the BiLSTM tail at once: their one-launch LSTMs meet on the device
+            both = [THREAD_CASES[1]] * 2
+            x = inputs[1]
+            outs = [np.empty(1 << 20, np.float32) for _ in both]
+            out_dims = np.zeros(14, np.int32)
+            rc = lib().dnn_run_threads(
+                2, (ctypes.c_void_p * 2)(first.value, extra[0].value), ip(i32([c[0] for c in both])), ip(i32([c[2] for c in both])),
+                451, ip(i32(np.concatenate([c[1] for c in both]))), (ctypes.c_void_p * 2)(x.ctypes.data, x.ctypes.data),
+                (ctypes.c_void_p * 2)(*[o.ctypes.data for o in outs]), ip(i32([o.size for o in outs])), ip(out_dims), 6)
+            assert rc == 0, lib().dnn_last_error().decode()
+            for o in outs:
+                assert np.array_equal(o[:want[1].size], want[1])
+    finally:
+        for e in extra:
+            nhtest.shim().shim_destroy_engine(e)
+
+
 @pytest.mark.gpu
 def test_recognizer_tail_at_benchmark_size_fused_vs_composite(capsys):
     """The BiLSTM tail of the line recogniser at its full size (128 steps, 64 lines, 256 -> 2 x 256 hidden, FC to 101)
