@@ -49,7 +49,10 @@ typedef float f32x16 __attribute__( ( ext_vector_type( 16 ) ) );
 // Cin divides; the 1-3 padding values per row are masked to zero on both operands.
 // AM_ConvClasses: the gradient by the input of a strided convolution, one stride-1 convolution per residue class of the
 // input pixels (blockIdx.y = class): AM_Conv whose geometry, filter and output rows come from args.Class[class].
-enum TAMode { AM_RowsK = 0, AM_RowsM = 1, AM_Conv = 2, AM_Conv1x1 = 3, AM_ConvRows = 4, AM_ConvClasses = 5 };
+// AM_ConvTaps: AM_Conv for channel counts that are a multiple of the K step, without the strided gradient's exact-division
+// test: a step never straddles two taps, the reduction ends on a step, and everything that is only needed otherwise is
+// compiled out of the loop ( the 3x3 convolutions of the image networks ).
+enum TAMode { AM_RowsK = 0, AM_RowsM = 1, AM_Conv = 2, AM_Conv1x1 = 3, AM_ConvRows = 4, AM_ConvClasses = 5, AM_ConvTaps = 6 };
 // BM_ConvN: B is the im2col view of an N,H,W,C image read N-major: row k = output pixel, column n = ( kh, kw, ci ).
 // With A = the gradient by the convolution's output read M-major this is the gradient by the filter.
 enum TBMode { BM_RowsK = 0, BM_RowsN = 1, BM_ConvN = 2 };
@@ -100,7 +103,29 @@ struct CMatMulArgs {
 	// epilogue of the fused blocks: C = act( A * B + bias ) + Residual; Residual has C's layout, may be C itself
 	CFusedActivation Act;
 	const float* Residual;
+	// floor( 2^32 / divisor ) for the divisions of the prologue ( pixel -> image, row, column; workgroup -> tile ): a
+	// multiplication and one correction instead of the twenty-odd instructions of a division by a run-time value
+	unsigned WoMagic, HoMagic, TilesNMagic;
+	// size of C in bytes when its rows can be addressed by 32-bit offsets from its start ( 0: they cannot ): the
+	// epilogue then stores through a buffer descriptor of that size, which drops the rows of a last tile that lie
+	// beyond the matrix by itself
+	unsigned CBytes;
 };
+
+// floor( 2^32 / d ), capped: with it q = mulhi( x, magic ) is floor( x / d ) or one less for every x < 2^32
+inline unsigned divisionMagic( int d )
+{
+	return d <= 1 ? 0xFFFFFFFFu : static_cast<unsigned>( 0x100000000ULL / static_cast<unsigned>( d ) );
+}
+
+__device__ __forceinline__ void fastDivMod( int x, int d, unsigned magic, int& quotient, int& remainder )
+{
+	unsigned q = __umulhi( static_cast<unsigned>( x ), magic );
+	unsigned r = static_cast<unsigned>( x ) - q * static_cast<unsigned>( d );
+	const bool low = r >= static_cast<unsigned>( d );
+	quotient = static_cast<int>( low ? q + 1 : q );
+	remainder = static_cast<int>( low ? r - static_cast<unsigned>( d ) : r );
+}
 
 constexpr int Threads = 256;
 
@@ -135,7 +160,9 @@ void matMulKernel( const CMatMulArgs launchArgs )
 	constexpr int MI = WM / 32;
 	constexpr int NI = WN / 32;
 	constexpr bool AK = ( AMODE != AM_RowsM );
-	constexpr bool IsConv = ( AMODE == AM_Conv || AMODE == AM_Conv1x1 || AMODE == AM_ConvClasses );
+	constexpr bool IsTaps = ( AMODE == AM_ConvTaps );
+	constexpr bool IsConv = ( AMODE == AM_Conv || AMODE == AM_Conv1x1 || AMODE == AM_ConvClasses || IsTaps );
+	static_assert( !IsTaps || VEC, "whole taps per step go with vector loads" );
 	constexpr bool IsConvRows = ( AMODE == AM_ConvRows );
 	constexpr bool BK = ( BMODE == BM_RowsK );
 	constexpr int APitchX = BM + 4, BPitchX = BN + 4;
@@ -172,8 +199,8 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			stepsPerSplit = args.TailSteps;
 		}
 	}
-	const int tileM = tile / args.TilesN;
-	const int tileN = tile % args.TilesN;
+	int tileM, tileN;
+	fastDivMod( tile, args.TilesN, args.TilesNMagic, tileM, tileN );
 	const int m0 = tileM * BM;
 	const int n0 = tileN * BN;
 	const int batch = blockIdx.y;
@@ -215,7 +242,7 @@ void matMulKernel( const CMatMulArgs launchArgs )
 		int hi = convH0[i] + convKh * args.DilH;
 		int wi = convW0[i] + convKw * args.DilW;
 		bool ok = convKh < args.Fh;
-		if( args.UpH > 1 || args.UpW > 1 ) {
+		if( !IsTaps && ( args.UpH > 1 || args.UpW > 1 ) ) {
 			ok = ok && hi >= 0 && wi >= 0 && hi % args.UpH == 0 && wi % args.UpW == 0;
 			hi /= args.UpH;
 			wi /= args.UpW;
@@ -237,10 +264,17 @@ void matMulKernel( const CMatMulArgs launchArgs )
 		} else {
 			const int m = m0 + rowOfSlot( slot );
 			if( inTile && m < M ) {
-				const int wo = m % args.Wo;
-				const int t = m / args.Wo;
-				const int ho = t % args.Ho;
-				const int n = t / args.Ho;
+				int wo, t, ho, n;
+				if constexpr( IsClasses ) {
+					// ( every class has its own grid of result pixels )
+					wo = m % args.Wo;
+					t = m / args.Wo;
+					ho = t % args.Ho;
+					n = t / args.Ho;
+				} else {
+					fastDivMod( m, args.Wo, args.WoMagic, t, wo );
+					fastDivMod( t, args.Ho, args.HoMagic, n, ho );
+				}
 				convPixel[i] = n * args.H * args.W * args.Cin;
 				convH0[i] = ho * args.StrideH - args.PadH;
 				convW0[i] = ( wo * args.StrideW - args.PadW ) * ( IsConvRows ? args.Cin : 1 ); // AM_ConvRows: in floats
@@ -262,13 +296,13 @@ void matMulKernel( const CMatMulArgs launchArgs )
 	// Channel counts that are a multiple of the K step: every lane of the workgroup is in the same filter tap during a
 	// step, so the tap and the channel inside it live in scalar registers, the channel reaches the loads as their
 	// uniform offset, and a step inside a tap costs no vector instruction for addresses.
-	const bool uniformTap = IsConv && VEC && args.Cin % KS == 0;
+	const bool uniformTap = IsTaps || ( IsConv && VEC && args.Cin % KS == 0 );
 	int tapCi = 0, tapKh = 0, tapKw = 0;
 	auto tapSlotOffset = [&]( int i ) -> unsigned {
 		int hi = convH0[i] + tapKh * args.DilH;
 		int wi = convW0[i] + tapKw * args.DilW;
 		bool ok = tapKh < args.Fh;
-		if( args.UpH > 1 || args.UpW > 1 ) {
+		if( !IsTaps && ( args.UpH > 1 || args.UpW > 1 ) ) {
 			ok = ok && hi >= 0 && wi >= 0 && hi % args.UpH == 0 && wi % args.UpW == 0;
 			hi /= args.UpH;
 			wi /= args.UpW;
@@ -278,10 +312,12 @@ void matMulKernel( const CMatMulArgs launchArgs )
 	};
 	if( IsConv && VEC ) {
 		if( uniformTap ) {
-			const int tap = kStart / args.Cin;
-			tapCi = kStart - tap * args.Cin;
-			tapKh = tap / args.Fw;
-			tapKw = tap - tapKh * args.Fw;
+			if( kStart != 0 ) { // ( a slice behind the first: the only case that pays for the two divisions )
+				const int tap = kStart / args.Cin;
+				tapCi = kStart - tap * args.Cin;
+				tapKh = tap / args.Fw;
+				tapKw = tap - tapKh * args.Fw;
+			}
 #pragma unroll
 			for( int i = 0; i < ASlots; ++i ) {
 				offA[i] = tapSlotOffset( i );
@@ -451,7 +487,7 @@ void matMulKernel( const CMatMulArgs launchArgs )
 				: ( AMODE == AM_RowsK ? stepK * 4u : stepK * static_cast<unsigned>( args.Lda ) * 4u );
 			const unsigned uniB = BMODE == BM_ConvN ? 0u
 				: ( BMODE == BM_RowsK ? stepK * 4u : stepK * static_cast<unsigned>( args.Ldb ) * 4u );
-			const bool partialStep = kBase + KS > K;
+			const bool partialStep = !IsTaps && kBase + KS > K; // ( whole taps of whole steps: K ends on a step )
 			if( IsConv || !partialStep ) {
 				// the image's own zero padding covers k beyond K: such taps lie below the filter ( kh >= Fh )
 #pragma unroll
@@ -840,6 +876,20 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			// Values cross between workgroups (and so between the L2 caches of the XCDs) through device-scope atomic
 			// stores and loads, which go past those caches. A wave's stores are complete when the barrier lets it
 			// through, the count follows the barrier: whoever reads the full count finds every slice's values.
+			// Why relaxed operations are enough here, and what holds them in place:
+			//  - every access to the partial tiles and to the counter is an agent-scope ATOMIC: the compiler may neither
+			//    drop, merge nor cache one, and emits each as an access that is coherent across the XCDs ( write-through
+			//    stores, loads that miss the XCD's L2 ), so no cache has to be written back or invalidated;
+			//  - the partial stores cannot sink below the ticket: between them lie the explicit wait for the wave's own
+			//    stores and __syncthreads(), which is a workgroup-scope release fence, the barrier, and an acquire fence;
+			//    the fences order ALL earlier memory operations of the wave, atomic or not, before all later ones for the
+			//    compiler, and the wait makes the hardware's stores complete ( acknowledged by the memory side ) first;
+			//  - the last arriver's loads cannot rise above the ticket: they come behind the second __syncthreads() and
+			//    depend on the ticket's value through the branch.
+			// A release on the ticket and an acquire in front of the loads would say the same in the language's terms; at
+			// agent scope they make this part write back and invalidate the XCD's whole L2, result tiles of other
+			// workgroups included: measured once, an acq_rel ticket took the K-sliced 3x3 convolutions from 122 / 127 /
+			// 123 us to 145 / 166 / 159 us ( 64 x 28 x 28 x 128, 64 x 14 x 14 x 256, 64 x 7 x 7 x 512 ).
 			const int slicedTile = args.FullTiles > 0 ? tile - args.FullTiles : tile;
 			unsigned* mine = reinterpret_cast<unsigned*>( args.Partials )
 				+ ( static_cast<long long>( slicedTile ) * splitK + split ) * ( BM * BN ) + wave * 64 + lane;
@@ -882,6 +932,60 @@ void matMulKernel( const CMatMulArgs launchArgs )
 				__hip_atomic_store( args.Counters + slicedTile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT );
 			}
 			splitK = 1; // from here on: the one workgroup that writes the tile
+		}
+	}
+
+	// The common case - C = act( acc + bias ), rows addressable by 32-bit offsets - stores through a buffer descriptor that
+	// ends with the matrix: a lane's offset is computed once per 32-column block, a row adds a multiple of the row pitch
+	// ( in a scalar register for tiles that lie inside the matrix: no vector instruction per element beyond the bias and
+	// the activation; as a vector addition for the last tile row, whose rows beyond M the range check drops ). Per tile
+	// and wavefront this takes some 150 vector instructions out of an epilogue that cost as much as ten K steps.
+	if constexpr( !IsClasses && BMODE != BM_ConvN ) {
+		if( args.CBytes != 0 && splitK == 1 && !args.Accumulate && args.Residual == nullptr ) {
+			const __amdgpu_buffer_rsrc_t bufC = __builtin_amdgcn_make_buffer_rsrc( C, 0, args.CBytes, 0x00020000 );
+			const float reluTop = args.Act.Param > 0.f ? args.Act.Param : __builtin_inff();
+			const unsigned pitchBytes = static_cast<unsigned>( args.Ldc ) * 4u;
+			const bool inside = m0 + BM <= M;
+			auto store = [&]( auto typeOf, auto insideOf ) {
+				constexpr int Type = decltype( typeOf )::value;
+				constexpr bool Inside = decltype( insideOf )::value;
+#pragma unroll
+				for( int ni = 0; ni < NI; ++ni ) {
+					const int n = n0 + waveN * WN + ni * 32 + l32;
+					const float bias = ( args.Bias != nullptr && n < N ) ? args.Bias[n] : 0.f;
+					const unsigned laneOffset = n < N
+						? static_cast<unsigned>( ( m0 + waveM * WM + half * 4 ) * args.Ldc + n ) * 4u : OutOfRange;
+#pragma unroll
+					for( int mi = 0; mi < MI; ++mi ) {
+#pragma unroll
+						for( int r = 0; r < 16; ++r ) {
+							const unsigned rowBytes = static_cast<unsigned>( mi * 32 + ( r >> 2 ) * 8 + ( r & 3 ) ) * pitchBytes;
+							const float v = applyActivationOf<Type>( acc[mi][ni][r] + bias, reluTop );
+							if constexpr( Inside ) {
+								__builtin_amdgcn_raw_buffer_store_b32( __float_as_uint( v ), bufC, laneOffset, rowBytes, 0 );
+							} else {
+								// ( an offset that was out of range stays so: rowBytes is below 2^31 )
+								__builtin_amdgcn_raw_buffer_store_b32( __float_as_uint( v ), bufC, laneOffset + rowBytes, 0, 0 );
+							}
+						}
+					}
+				}
+			};
+			auto storeAs = [&]( auto typeOf ) {
+				if( inside ) {
+					store( typeOf, std::true_type() );
+				} else {
+					store( typeOf, std::false_type() );
+				}
+			};
+			if( args.Act.Type == NH_ACT_RELU ) {
+				storeAs( std::integral_constant<int, NH_ACT_RELU>() );
+			} else if( args.Act.Type == NH_ACT_HSWISH ) {
+				storeAs( std::integral_constant<int, NH_ACT_HSWISH>() );
+			} else {
+				storeAs( std::integral_constant<int, NH_ACT_NONE>() );
+			}
+			return;
 		}
 	}
 
@@ -1232,6 +1336,13 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 {
 	args.TilesM = ceilDiv( args.M, BM );
 	args.TilesN = ceilDiv( args.N, BN );
+	args.TilesNMagic = divisionMagic( args.TilesN );
+	args.WoMagic = divisionMagic( args.Wo );
+	args.HoMagic = divisionMagic( args.Ho );
+	{
+		const long long cBytes = ( static_cast<long long>( args.M - 1 ) * args.Ldc + args.N ) * 4;
+		args.CBytes = ( args.Ldc >= args.N && cBytes > 0 && cBytes < 0x7fffff00LL ) ? static_cast<unsigned>( cBytes ) : 0u;
+	}
 	const long long tiles = static_cast<long long>( args.TilesM ) * args.TilesN;
 	if( tiles > 0x7fffffffLL ) {
 		setLastError( "matrix product: too many tiles" );
@@ -1282,7 +1393,7 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 	}
 	// two slices of an even number of steps: the two halves share a workgroup of 8 wavefronts instead (KGROUPS = 2)
 	bool twoGroups = false;
-	if constexpr( BM == 64 && BN == 64 && BMODE == BM_RowsK && ( AMODE == AM_Conv || AMODE == AM_RowsK ) ) {
+	if constexpr( BM == 64 && BN == 64 && BMODE == BM_RowsK && ( AMODE == AM_Conv || AMODE == AM_ConvTaps || AMODE == AM_RowsK ) ) {
 		if( vec && splits == 2 && totalSteps % 2 == 0 && batch == 1 && args.ManySlices == 0 ) {
 			twoGroups = true;
 			splits = 1;
@@ -1400,12 +1511,12 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 		a.C += b0 * args.BatchStrideC;
 		const dim3 grid( static_cast<unsigned>( gridX ), nb, args.SplitK );
 		if( twoGroups ) {
-			if constexpr( BM == 64 && BN == 64 && BMODE == BM_RowsK && ( AMODE == AM_Conv || AMODE == AM_RowsK ) ) {
+			if constexpr( BM == 64 && BN == 64 && BMODE == BM_RowsK && ( AMODE == AM_Conv || AMODE == AM_ConvTaps || AMODE == AM_RowsK ) ) {
 				hipLaunchKernelGGL( ( matMulKernel<BM, BN, WAVES_M, WAVES_N, AMODE, BMODE, true, 2> ), grid, dim3( Threads * 2 ), 0, stream, a );
 			}
 		} else if( vec ) {
 			hipLaunchKernelGGL( ( matMulKernel<BM, BN, WAVES_M, WAVES_N, AMODE, BMODE, true> ), grid, dim3( Threads ), 0, stream, a );
-		} else {
+		} else if constexpr( AMODE != AM_ConvTaps ) {
 			hipLaunchKernelGGL( ( matMulKernel<BM, BN, WAVES_M, WAVES_N, AMODE, BMODE, false> ), grid, dim3( Threads ), 0, stream, a );
 		}
 		if( args.FullTiles > 0 && actAfter.Type != NH_ACT_NONE && !meetInScratch ) {
@@ -2658,6 +2769,9 @@ int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* sour
 		args.K = d.filterHeight * args.RowPitch; // reduction length as the kernel walks it; Ldb keeps the filter's own
 		return launchMatMul<AM_ConvRows, BM_RowsK>( stream, args, 1, true, fixedMeeting );
 	}
+	if( vec && d.channels % NH_KSTEP == 0 ) {
+		return launchMatMul<AM_ConvTaps, BM_RowsK>( stream, args, 1, true, fixedMeeting );
+	}
 	return launchMatMul<AM_Conv, BM_RowsK>( stream, args, 1, vec, fixedMeeting );
 }
 
@@ -2810,6 +2924,9 @@ int convBackwardData( hipStream_t stream, const nhConvDesc& d, const float* outp
 	const bool vec = isAligned16( outputDiff ) && isAligned16( swappedFilter ) && d.filterCount % 4 == 0
 		&& fitsBuffer( 1, 0, static_cast<long long>( d.batch ) * d.resultHeight * d.resultWidth * d.filterCount )
 		&& fitsBuffer( d.channels, args.K, args.K );
+	if( vec && d.filterCount % NH_KSTEP == 0 && d.strideHeight == 1 && d.strideWidth == 1 ) {
+		return launchMatMul<AM_ConvTaps, BM_RowsK>( stream, args, 1, true );
+	}
 	return launchMatMul<AM_Conv, BM_RowsK>( stream, args, 1, vec );
 }
 
