@@ -298,17 +298,32 @@ void matMulKernel( const CMatMulArgs launchArgs )
 	// uniform offset, and a step inside a tap costs no vector instruction for addresses.
 	const bool uniformTap = IsTaps || ( IsConv && VEC && args.Cin % KS == 0 );
 	int tapCi = 0, tapKh = 0, tapKw = 0;
+	// Without the strided gradient's division a tap moves every lane's address by the same amount: per slot the position
+	// of tap ( 0, 0 ) is kept ( in floats, as unsigned arithmetic: it may lie in front of the image ), a tap adds
+	// ( kh dilation W + kw dilation ) Cin from a scalar register, and the two unsigned comparisons say whether the tap
+	// meets the image: six vector instructions per slot and tap.
+	unsigned convBase[ASlots] = {};
+#pragma unroll
+	for( int i = 0; IsConv && i < ASlots; ++i ) {
+		convBase[i] = static_cast<unsigned>( convPixel[i] ) + ( static_cast<unsigned>( convH0[i] ) * static_cast<unsigned>( args.W )
+			+ static_cast<unsigned>( convW0[i] ) ) * static_cast<unsigned>( args.Cin ) + static_cast<unsigned>( ( tid % KQ ) * 4 );
+	}
 	auto tapSlotOffset = [&]( int i ) -> unsigned {
-		int hi = convH0[i] + tapKh * args.DilH;
-		int wi = convW0[i] + tapKw * args.DilW;
-		bool ok = tapKh < args.Fh;
 		if( !IsTaps && ( args.UpH > 1 || args.UpW > 1 ) ) {
-			ok = ok && hi >= 0 && wi >= 0 && hi % args.UpH == 0 && wi % args.UpW == 0;
+			int hi = convH0[i] + tapKh * args.DilH;
+			int wi = convW0[i] + tapKw * args.DilW;
+			bool ok = tapKh < args.Fh && hi >= 0 && wi >= 0 && hi % args.UpH == 0 && wi % args.UpW == 0;
 			hi /= args.UpH;
 			wi /= args.UpW;
+			ok = ok && hi >= 0 && hi < args.H && wi >= 0 && wi < args.W;
+			return ok ? static_cast<unsigned>( convPixel[i] + ( hi * args.W + wi ) * args.Cin + ( tid % KQ ) * 4 ) * 4u : OutOfRange;
 		}
-		ok = ok && hi >= 0 && hi < args.H && wi >= 0 && wi < args.W;
-		return ok ? static_cast<unsigned>( convPixel[i] + ( hi * args.W + wi ) * args.Cin + ( tid % KQ ) * 4 ) * 4u : OutOfRange;
+		const int dh = tapKh * args.DilH, dw = tapKw * args.DilW; // ( scalar )
+		const unsigned tapFloats = ( static_cast<unsigned>( dh ) * static_cast<unsigned>( args.W ) + static_cast<unsigned>( dw ) )
+			* static_cast<unsigned>( args.Cin );
+		const bool ok = tapKh < args.Fh && static_cast<unsigned>( convH0[i] + dh ) < static_cast<unsigned>( args.H )
+			&& static_cast<unsigned>( convW0[i] + dw ) < static_cast<unsigned>( args.W );
+		return ok ? ( convBase[i] + tapFloats ) * 4u : OutOfRange;
 	};
 	if( IsConv && VEC ) {
 		if( uniformTap ) {
