@@ -376,15 +376,7 @@ void findMaxInRowsKernel( const float* matrix, int height, int width, float* res
 			bestIdx = i;
 		}
 	}
-#pragma unroll
-	for( int off = 32; off > 0; off >>= 1 ) {
-		const float ov = __shfl_xor( best, off, 64 );
-		const int oi = __shfl_xor( bestIdx, off, 64 );
-		if( oi != 0x7fffffff && ( bestIdx == 0x7fffffff || ov > best || ( ov == best && oi < bestIdx ) ) ) {
-			best = ov;
-			bestIdx = oi;
-		}
-	}
+	waveReduceArgMax( best, bestIdx );
 	if( lane == 0 ) {
 		result[row] = best;
 		if( indices != nullptr ) {

@@ -57,22 +57,69 @@ inline bool isAligned16( const void* p ) { return ( reinterpret_cast<uintptr_t>(
 #ifdef __HIPCC__
 namespace nh {
 
+// Wavefront reductions on the data-parallel-primitive path of the vector ALU: a DPP operand reads another lane's
+// register as part of the arithmetic instruction itself, where a shuffle is a round trip through the LDS crossbar
+// ( ds_bpermute + wait ) per step. Four shifts inside each row of 16 lanes ( a lane outside the row contributes the
+// operation's identity ), then lane 15 of a row is broadcast into the following row, then lane 31 into the upper half:
+// lane 63 holds the result of all 64 lanes, and a read of that lane hands it to every lane as a scalar.
+// All 64 lanes must be active ( the callers reduce in wave-uniform control flow ).
+constexpr int DppRowShr1 = 0x111, DppRowShr2 = 0x112, DppRowShr4 = 0x114, DppRowShr8 = 0x118;
+constexpr int DppRowBcast15 = 0x142, DppRowBcast31 = 0x143;
+
+template<int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ float dppMove( float identity, float v )
+{
+	return __uint_as_float( static_cast<unsigned>( __builtin_amdgcn_update_dpp( static_cast<int>( __float_as_uint( identity ) ),
+		static_cast<int>( __float_as_uint( v ) ), CTRL, ROW_MASK, 0xF, false ) ) );
+}
+
+template<int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ int dppMove( int identity, int v )
+{
+	return __builtin_amdgcn_update_dpp( identity, v, CTRL, ROW_MASK, 0xF, false );
+}
+
 __device__ __forceinline__ float waveReduceSum( float v )
 {
-#pragma unroll
-	for( int off = 32; off > 0; off >>= 1 ) {
-		v += __shfl_xor( v, off, 64 );
-	}
-	return v;
+	v += dppMove<DppRowShr1>( 0.f, v );
+	v += dppMove<DppRowShr2>( 0.f, v );
+	v += dppMove<DppRowShr4>( 0.f, v );
+	v += dppMove<DppRowShr8>( 0.f, v );
+	v += dppMove<DppRowBcast15, 0xA>( 0.f, v );
+	v += dppMove<DppRowBcast31, 0xC>( 0.f, v );
+	return __uint_as_float( static_cast<unsigned>( __builtin_amdgcn_readlane( static_cast<int>( __float_as_uint( v ) ), 63 ) ) );
 }
 
 __device__ __forceinline__ float waveReduceMax( float v )
 {
-#pragma unroll
-	for( int off = 32; off > 0; off >>= 1 ) {
-		v = fmaxf( v, __shfl_xor( v, off, 64 ) );
-	}
-	return v;
+	const float lowest = -__builtin_inff();
+	v = fmaxf( v, dppMove<DppRowShr1>( lowest, v ) );
+	v = fmaxf( v, dppMove<DppRowShr2>( lowest, v ) );
+	v = fmaxf( v, dppMove<DppRowShr4>( lowest, v ) );
+	v = fmaxf( v, dppMove<DppRowShr8>( lowest, v ) );
+	v = fmaxf( v, dppMove<DppRowBcast15, 0xA>( lowest, v ) );
+	v = fmaxf( v, dppMove<DppRowBcast31, 0xC>( lowest, v ) );
+	return __uint_as_float( static_cast<unsigned>( __builtin_amdgcn_readlane( static_cast<int>( __float_as_uint( v ) ), 63 ) ) );
+}
+
+// The largest value of the wavefront and the smallest index among the lanes that hold it. A lane without a candidate
+// passes index 0x7fffffff, which loses against every real one.
+__device__ __forceinline__ void waveReduceArgMax( float& best, int& bestIndex )
+{
+	auto take = [&]( float otherValue, int otherIndex ) {
+		const bool better = otherIndex != 0x7fffffff
+			&& ( bestIndex == 0x7fffffff || otherValue > best || ( otherValue == best && otherIndex < bestIndex ) );
+		best = better ? otherValue : best;
+		bestIndex = better ? otherIndex : bestIndex;
+	};
+	take( dppMove<DppRowShr1>( 0.f, best ), dppMove<DppRowShr1>( 0x7fffffff, bestIndex ) );
+	take( dppMove<DppRowShr2>( 0.f, best ), dppMove<DppRowShr2>( 0x7fffffff, bestIndex ) );
+	take( dppMove<DppRowShr4>( 0.f, best ), dppMove<DppRowShr4>( 0x7fffffff, bestIndex ) );
+	take( dppMove<DppRowShr8>( 0.f, best ), dppMove<DppRowShr8>( 0x7fffffff, bestIndex ) );
+	take( dppMove<DppRowBcast15, 0xA>( 0.f, best ), dppMove<DppRowBcast15, 0xA>( 0x7fffffff, bestIndex ) );
+	take( dppMove<DppRowBcast31, 0xC>( 0.f, best ), dppMove<DppRowBcast31, 0xC>( 0x7fffffff, bestIndex ) );
+	best = __uint_as_float( static_cast<unsigned>( __builtin_amdgcn_readlane( static_cast<int>( __float_as_uint( best ) ), 63 ) ) );
+	bestIndex = __builtin_amdgcn_readlane( bestIndex, 63 );
 }
 
 // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous range of tiles so that
