@@ -231,6 +231,18 @@ def main():
         measure("BlobChannelwiseConvolution cfg3 %dx%dx%dx%d 3x3/%d" % (n, h, w, c, s),
                 lambda: lib.nhBlobChannelwiseConvolution(stream, ctypes.byref(d), P(x), P(flt), P(b), P(y)),
                 2 * n * d.resultHeight * d.resultWidth * c * 9, by, by)
+        if by >= 200e6:
+            # as inside a network, where the input was written by the layer in front and is not in the last-level cache:
+            # the launches rotate through enough input / output pairs to exceed it several times
+            pairs = [(x, y)] + [(rand(n, h, w, c), empty(n, d.resultHeight, d.resultWidth, c)) for _ in range(max(1, int(1.2e9 // by)))]
+            turn = [0]
+
+            def cold():
+                xi, yi = pairs[turn[0] % len(pairs)]
+                turn[0] += 1
+                return lib.nhBlobChannelwiseConvolution(stream, ctypes.byref(d), P(xi), P(flt), P(b), P(yi))
+            measure("BlobChannelwiseConvolution cold %dx%dx%dx%d 3x3/%d" % (n, h, w, c, s), cold,
+                    2 * n * d.resultHeight * d.resultWidth * c * 9, by, 2e9)
 
     def dw_gradients(n, h, w, c, s):
         d = neoml_amd.ConvDesc(n, h, w, c, c, 3, 3, 1, 1, s, s, 1, 1, 0, 0)

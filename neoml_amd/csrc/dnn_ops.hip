@@ -7,6 +7,7 @@
 #include <stdlib.h>
 #include <map>
 #include <mutex>
+#include <type_traits>
 #include <utility>
 
 namespace nh {
@@ -111,10 +112,17 @@ void channelwiseConvKernel( const nhConvDesc d, const float* source, const float
 // out-of-range offset instead of a branch. Workgroups of one XCD cover a contiguous range of strips: the halo columns
 // shared by neighbouring strips meet in that XCD's L2.
 // STREAM: loads carry the streaming hint ( tensors far larger than the caches, every line used by one strip ).
-template<int STRIDE, int WPT, int PRE, bool STREAM>
+// The row loop has no branch: rows below the strip and columns beyond the image get out-of-range offsets, for the
+// loads ( zeros ) and for the stores ( dropped: the result is written through a buffer descriptor ), and the activation's
+// type ( ACT ) is fixed when the kernel is compiled. With a branch per output pixel in the loop ( is the row inside? the
+// column? which activation? ) the compiler no longer knew how many loads and stores were in flight at the top of the
+// loop and waited for all of them, stores included, once per turn of the ring: every few rows each wave stood still
+// for a whole memory round trip.
+template<int STRIDE, int WPT, int PRE, bool STREAM, int ACT>
 __global__ __launch_bounds__( 256 )
 void channelwiseConv3x3Kernel( const nhConvDesc d, const float* source, const float* filter, const float* freeTerm,
-	float* result, int wGroups, int rowChunks, int rowsPerItem, int totalItems, const CFusedActivation act, int flipTaps )
+	float* result, int wGroups, int rowChunks, int rowsPerItem, int totalItems, const CFusedActivation act, int flipTaps,
+	unsigned resultBytes )
 {
 	constexpr int NC = ( WPT - 1 ) * STRIDE + 3;
 	constexpr int Ring = 3 + PRE * STRIDE;
@@ -144,7 +152,7 @@ void channelwiseConv3x3Kernel( const nhConvDesc d, const float* source, const fl
 #pragma unroll
 	for( int k = 0; k < 9; ++k ) {
 		// flipTaps: the filter turned by 180 degrees, which makes this kernel the gradient by the input of the stride-1 case
-		f[k] = *reinterpret_cast<const float4*>( filter + ( flipTaps != 0 ? 8 - k : k ) * d.channels + c );
+		f[k] = *reinterpret_cast<const float4*>( filter + ( ( flipTaps & 1 ) != 0 ? 8 - k : k ) * d.channels + c );
 	}
 	const float4 bias = freeTerm != nullptr ? *reinterpret_cast<const float4*>( freeTerm + c ) : make_float4( 0.f, 0.f, 0.f, 0.f );
 
@@ -166,36 +174,51 @@ void channelwiseConv3x3Kernel( const nhConvDesc d, const float* source, const fl
 	for( int r = 0; r < Ring - STRIDE; ++r ) {
 		loadRow( ring[r], hiFirst + r );
 	}
-	float* out = result + ( ( static_cast<long long>( n ) * d.resultHeight + ho0 ) * d.resultWidth + wo0 ) * d.channels + c;
-	const long long outRow = static_cast<long long>( d.resultWidth ) * d.channels;
+	const __amdgpu_buffer_rsrc_t outBuffer = __builtin_amdgcn_make_buffer_rsrc( result, 0, resultBytes, 0x00020000 );
+	const unsigned outRowBytes = static_cast<unsigned>( d.resultWidth ) * d.channels * 4;
+	unsigned outCol[WPT];
+#pragma unroll
+	for( int j = 0; j < WPT; ++j ) {
+		outCol[j] = wo0 + j < d.resultWidth ? static_cast<unsigned>( ( wo0 + j ) * d.channels + c ) * 4 : OutOfRange;
+	}
+	unsigned outRowOffset = static_cast<unsigned>( n * d.resultHeight + ho0 ) * outRowBytes;
+	const float reluTop = act.Param > 0.f ? act.Param : __builtin_inff();
 	for( int hoBase = ho0; hoBase < hoEnd; hoBase += Ring ) {
 #pragma unroll
 		for( int k = 0; k < Ring; ++k ) {
-			if( hoBase + k < hoEnd ) {
-				// output row hoBase + k: its window starts at ring position ( k * STRIDE ) % Ring ( Ring output rows
-				// advance the window by Ring * STRIDE rows: a whole number of turns ); the rows PRE steps ahead go in
-				// behind the ones already there
+			// output row hoBase + k: its window starts at ring position ( k * STRIDE ) % Ring ( Ring output rows
+			// advance the window by Ring * STRIDE rows: a whole number of turns ); the rows PRE steps ahead go in
+			// behind the ones already there. Behind the strip's last row nothing is fetched and nothing stored.
 #pragma unroll
-				for( int r = 0; r < STRIDE; ++r ) {
-					const int ahead = k * STRIDE + Ring - STRIDE + r;
-					loadRow( ring[ahead % Ring], hiFirst + ( hoBase - ho0 ) * STRIDE + ahead );
-				}
-#pragma unroll
-				for( int j = 0; j < WPT; ++j ) {
-					float4 acc = bias;
-#pragma unroll
-					for( int kh = 0; kh < 3; ++kh ) {
-#pragma unroll
-						for( int kw = 0; kw < 3; ++kw ) {
-							acc = CChanVec<4>::fma( ring[( k * STRIDE + kh ) % Ring][j * STRIDE + kw], f[kh * 3 + kw], acc );
-						}
-					}
-					if( wo0 + j < d.resultWidth ) {
-						*reinterpret_cast<float4*>( out + j * d.channels ) = CChanVec<4>::activate( acc, act );
-					}
-				}
-				out += outRow;
+			for( int r = 0; r < STRIDE; ++r ) {
+				const int ahead = k * STRIDE + Ring - STRIDE + r;
+				loadRow( ring[ahead % Ring], hiFirst + ( hoBase - ho0 ) * STRIDE + ahead );
 			}
+			const bool rowInside = hoBase + k < hoEnd;
+#pragma unroll
+			for( int j = 0; j < WPT; ++j ) {
+				float4 acc = bias;
+#pragma unroll
+				for( int kh = 0; kh < 3; ++kh ) {
+#pragma unroll
+					for( int kw = 0; kw < 3; ++kw ) {
+						acc = CChanVec<4>::fma( ring[( k * STRIDE + kh ) % Ring][j * STRIDE + kw], f[kh * 3 + kw], acc );
+					}
+				}
+				acc.x = applyActivationOf<ACT>( acc.x, reluTop );
+				acc.y = applyActivationOf<ACT>( acc.y, reluTop );
+				acc.z = applyActivationOf<ACT>( acc.z, reluTop );
+				acc.w = applyActivationOf<ACT>( acc.w, reluTop );
+				// ( a valid row offset is below 2 GiB, so adding an out-of-range column stays out of range )
+				if( STREAM && flipTaps >= 2 ) {
+					u32x4 u;
+					u.x = __float_as_uint( acc.x ); u.y = __float_as_uint( acc.y ); u.z = __float_as_uint( acc.z ); u.w = __float_as_uint( acc.w );
+					__builtin_amdgcn_raw_buffer_store_b128( u, outBuffer, rowInside ? outRowOffset + outCol[j] : OutOfRange, 0, 2 );
+				} else {
+					bufferStore4( outBuffer, rowInside ? outRowOffset + outCol[j] : OutOfRange, acc );
+				}
+			}
+			outRowOffset += outRowBytes;
 		}
 	}
 }
@@ -1987,9 +2010,28 @@ static int channelwise3x3Launch( nhStream s, const nhConvDesc* d, const float* s
 	rowChunks = ceilDiv( d->resultHeight, rowsPerItem );
 	const long long items = perRow * rowChunks;
 	// workgroups of one wave: the strips need nothing from one another, and single waves spread most evenly
-	hipLaunchKernelGGL( ( channelwiseConv3x3Kernel<STRIDE, WPT, 1, STREAM> ), dim3( static_cast<unsigned>( ( items + 63 ) / 64 ) ),
-		dim3( 64 ), 0, toStream( s ), *d, source, filter, freeTerm, result, wGroups, rowChunks, rowsPerItem,
-		static_cast<int>( items ), act, flipTaps ? 1 : 0 );
+	const unsigned resultBytes = static_cast<unsigned>( static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * d->channels * 4 );
+	const dim3 grid( static_cast<unsigned>( ( items + 63 ) / 64 ) );
+	static const char* ntEnv = getenv( "NH_DW_NT" );
+	const int flipArg = ( flipTaps ? 1 : 0 ) + ( ntEnv != nullptr ? 2 : 0 );
+	auto launch = [&]( auto actOf ) {
+		constexpr int Act = decltype( actOf )::value;
+		static const char* preEnv = getenv( "NH_DW_PRE" );
+		if( preEnv != nullptr && preEnv[0] == '2' && STREAM ) {
+			hipLaunchKernelGGL( ( channelwiseConv3x3Kernel<STRIDE, WPT, STREAM ? 2 : 1, STREAM, Act> ), grid, dim3( 64 ), 0, toStream( s ), *d, source, filter,
+				freeTerm, result, wGroups, rowChunks, rowsPerItem, static_cast<int>( items ), act, flipArg, resultBytes );
+			return;
+		}
+		hipLaunchKernelGGL( ( channelwiseConv3x3Kernel<STRIDE, WPT, 1, STREAM, Act> ), grid, dim3( 64 ), 0, toStream( s ), *d, source, filter,
+			freeTerm, result, wGroups, rowChunks, rowsPerItem, static_cast<int>( items ), act, flipArg, resultBytes );
+	};
+	if( act.Type == NH_ACT_RELU ) {
+		launch( std::integral_constant<int, NH_ACT_RELU>() );
+	} else if( act.Type == NH_ACT_HSWISH ) {
+		launch( std::integral_constant<int, NH_ACT_HSWISH>() );
+	} else {
+		launch( std::integral_constant<int, NH_ACT_NONE>() );
+	}
 	NH_LAUNCH_CHECK();
 	return NH_OK;
 }
@@ -2010,8 +2052,8 @@ static int channelwise3x3Impl( nhStream s, const nhConvDesc* d, const float* sou
 	// ( 9 columns for 4 output pixels instead of 5 for 2 ) and lose at stride 1.
 	constexpr int Widths = STRIDE == 2 ? 2 : 1;
 	const int resident[2] = {
-		residentWavesFor( reinterpret_cast<const void*>( &channelwiseConv3x3Kernel<STRIDE, WPT, 1, true> ) ),
-		residentWavesFor( reinterpret_cast<const void*>( &channelwiseConv3x3Kernel<STRIDE, WPT * 2, 1, true> ) ) };
+		residentWavesFor( reinterpret_cast<const void*>( &channelwiseConv3x3Kernel<STRIDE, WPT, 1, true, NH_ACT_NONE> ) ),
+		residentWavesFor( reinterpret_cast<const void*>( &channelwiseConv3x3Kernel<STRIDE, WPT * 2, 1, true, NH_ACT_NONE> ) ) };
 	bool wide = false;
 	int chunks = 1;
 	double best = -1;
@@ -2345,7 +2387,7 @@ static int channelwiseConvolution( nhStream s, const nhConvDesc* d, const float*
 	const long long sourceBytes = static_cast<long long>( d->batch ) * d->height * d->width * d->channels * 4;
 	if( vec && d->filterHeight == 3 && d->filterWidth == 3 && d->strideHeight == d->strideWidth && d->strideHeight <= 2
 		&& sourceBytes < 0x80000000LL
-		&& static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * d->channels < 0x7fffffffLL )
+		&& static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * d->channels * 4 < 0x80000000LL )
 	{
 		return d->strideHeight == 1 ? channelwise3x3Impl<1, 4>( s, d, source, filter, freeTerm, result, act )
 			: channelwise3x3Impl<2, 2>( s, d, source, filter, freeTerm, result, act );
@@ -2454,7 +2496,7 @@ int nhBlobChannelwiseConvolutionBackward( nhStream s, const nhConvDesc* d, const
 	if( vec && d->filterHeight == 3 && d->filterWidth == 3 && d->strideHeight == 1 && d->strideWidth == 1
 		&& d->dilationHeight == 1 && d->dilationWidth == 1 && d->paddingHeight <= 2 && d->paddingWidth <= 2
 		&& static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * d->channels * 4 < 0x7fffffffLL
-		&& static_cast<long long>( d->batch ) * d->height * d->width * d->channels < 0x7fffffffLL )
+		&& static_cast<long long>( d->batch ) * d->height * d->width * d->channels * 4 < 0x7fffffffLL )
 	{
 		// Stride 1: the gradient by the input is the depthwise convolution of the output gradient with the filter turned
 		// by 180 degrees and padding 2 - p: the forward pass's strip kernel ( every row of the gradient read once per strip ).
