@@ -117,7 +117,11 @@ void channelwiseConvKernel( const nhConvDesc d, const float* source, const float
 // type ( ACT ) is fixed when the kernel is compiled. With a branch per output pixel in the loop ( is the row inside? the
 // column? which activation? ) the compiler no longer knew how many loads and stores were in flight at the top of the
 // loop and waited for all of them, stores included, once per turn of the ring: every few rows each wave stood still
-// for a whole memory round trip.
+// for a whole memory round trip ( layers that fit the caches: 14 x 14 x 384 17.4 -> 13.8 us, 7 x 7 x 960 10.6 -> 8.7 us ).
+// On inputs that come from memory ( measured with launches that rotate through 1.2 GB of input / output pairs, as
+// inside a network: 112 x 112 x 32 90 us = 4.6 TB/s, 56 x 56 x 144 113 us = 4.1 TB/s, against 68 and 84 us on repeated
+// buffers ) neither a second row of loads in flight ( PRE = 2: 88 / 106 us ) nor stores with the streaming hint ( 85 /
+// 106 us, and 83 / 104 us on repeated buffers ) change the picture: not a matter of loads in flight.
 template<int STRIDE, int WPT, int PRE, bool STREAM, int ACT>
 __global__ __launch_bounds__( 256 )
 void channelwiseConv3x3Kernel( const nhConvDesc d, const float* source, const float* filter, const float* freeTerm,
@@ -152,7 +156,7 @@ void channelwiseConv3x3Kernel( const nhConvDesc d, const float* source, const fl
 #pragma unroll
 	for( int k = 0; k < 9; ++k ) {
 		// flipTaps: the filter turned by 180 degrees, which makes this kernel the gradient by the input of the stride-1 case
-		f[k] = *reinterpret_cast<const float4*>( filter + ( ( flipTaps & 1 ) != 0 ? 8 - k : k ) * d.channels + c );
+		f[k] = *reinterpret_cast<const float4*>( filter + ( flipTaps != 0 ? 8 - k : k ) * d.channels + c );
 	}
 	const float4 bias = freeTerm != nullptr ? *reinterpret_cast<const float4*>( freeTerm + c ) : make_float4( 0.f, 0.f, 0.f, 0.f );
 
@@ -210,13 +214,7 @@ void channelwiseConv3x3Kernel( const nhConvDesc d, const float* source, const fl
 				acc.z = applyActivationOf<ACT>( acc.z, reluTop );
 				acc.w = applyActivationOf<ACT>( acc.w, reluTop );
 				// ( a valid row offset is below 2 GiB, so adding an out-of-range column stays out of range )
-				if( STREAM && flipTaps >= 2 ) {
-					u32x4 u;
-					u.x = __float_as_uint( acc.x ); u.y = __float_as_uint( acc.y ); u.z = __float_as_uint( acc.z ); u.w = __float_as_uint( acc.w );
-					__builtin_amdgcn_raw_buffer_store_b128( u, outBuffer, rowInside ? outRowOffset + outCol[j] : OutOfRange, 0, 2 );
-				} else {
-					bufferStore4( outBuffer, rowInside ? outRowOffset + outCol[j] : OutOfRange, acc );
-				}
+				bufferStore4( outBuffer, rowInside ? outRowOffset + outCol[j] : OutOfRange, acc );
 			}
 			outRowOffset += outRowBytes;
 		}
@@ -2012,16 +2010,9 @@ static int channelwise3x3Launch( nhStream s, const nhConvDesc* d, const float* s
 	// workgroups of one wave: the strips need nothing from one another, and single waves spread most evenly
 	const unsigned resultBytes = static_cast<unsigned>( static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * d->channels * 4 );
 	const dim3 grid( static_cast<unsigned>( ( items + 63 ) / 64 ) );
-	static const char* ntEnv = getenv( "NH_DW_NT" );
-	const int flipArg = ( flipTaps ? 1 : 0 ) + ( ntEnv != nullptr ? 2 : 0 );
+	const int flipArg = flipTaps ? 1 : 0;
 	auto launch = [&]( auto actOf ) {
 		constexpr int Act = decltype( actOf )::value;
-		static const char* preEnv = getenv( "NH_DW_PRE" );
-		if( preEnv != nullptr && preEnv[0] == '2' && STREAM ) {
-			hipLaunchKernelGGL( ( channelwiseConv3x3Kernel<STRIDE, WPT, STREAM ? 2 : 1, STREAM, Act> ), grid, dim3( 64 ), 0, toStream( s ), *d, source, filter,
-				freeTerm, result, wGroups, rowChunks, rowsPerItem, static_cast<int>( items ), act, flipArg, resultBytes );
-			return;
-		}
 		hipLaunchKernelGGL( ( channelwiseConv3x3Kernel<STRIDE, WPT, 1, STREAM, Act> ), grid, dim3( 64 ), 0, toStream( s ), *d, source, filter,
 			freeTerm, result, wGroups, rowChunks, rowsPerItem, static_cast<int>( items ), act, flipArg, resultBytes );
 	};
