@@ -63,3 +63,49 @@ def test_no_alloc_convolution_without_slices_and_with_a_tail():
         fixed, plain = _both(hip, x, f, bias, k // 2, 1)
         nhtest.assert_close(fixed, plain, "no-alloc vs allocating convolution %dx%dx%d" % (h, w, cin))
         assert np.array_equal(fixed, plain)
+
+
+def test_no_alloc_convolution_leaves_device_memory_as_it_is():
+    """The property itself: a warm call allocates nothing on the device. hipMemGetInfo (through torch) reports the same free
+    bytes before and after, with torch's caching allocator out of the picture (the buffers exist before the first reading,
+    nothing of torch's is allocated or freed in between), and the library's own per-stream scratch does not grow."""
+    import torch
+    hip = nhtest.Hip()
+    x, f, bias = _inputs(0xA1111, 64, 7, 7, 512, 512, 3)
+    d = hip.conv_desc(64, 7, 7, 512, 512, 3, 3, 1, 1, 1, 1)
+    xs, fs, bs = hip.up(x), hip.up(f), hip.up(bias)
+    out = hip.empty((64, d.resultHeight, d.resultWidth, 512))
+    call = lambda: hip.call("nhBlobConvolutionNoAlloc", ctypes.byref(d), hip.p(xs), hip.p(fs), hip.p(bs), hip.p(out))
+    call()  # the first call on a device looks the array's address up
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    reserved_before = torch.cuda.memory_reserved()
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert torch.cuda.memory_reserved() == reserved_before
+    assert free_after == free_before, "device memory in use changed by %d bytes across nhBlobConvolutionNoAlloc" % (free_before - free_after)
+
+
+def test_no_alloc_convolution_refuses_what_does_not_fit_its_array():
+    """K slices whose partial tiles exceed the fixed array (sliced tiles x slices x 16 KiB > 64 MiB): NH_ERR_ARGUMENT with a
+    message that names the limit, and nothing launched: the result buffer keeps its contents. How many slices a launch
+    takes is the launch planner's decision, so a few shapes with many tiles and long reductions are tried."""
+    import neoml_amd
+    hip = nhtest.Hip()
+    g = np.random.default_rng(5)
+    refused = 0
+    for n, h, w, cin, cout in [(144, 7, 7, 1024, 512), (200, 7, 7, 512, 320), (100, 7, 7, 2048, 640), (250, 5, 5, 1024, 512)]:
+        d = hip.conv_desc(n, h, w, cin, cout, 3, 3, 1, 1, 1, 1)
+        xs = hip.up(g.uniform(-1, 1, (n, h, w, cin)).astype(np.float32))
+        fs = hip.up(g.normal(0, 0.01, (cout, 3, 3, cin)).astype(np.float32))
+        out = hip.empty((n, d.resultHeight, d.resultWidth, cout))
+        out.fill_(7.0)
+        rc = hip.lib.nhBlobConvolutionNoAlloc(hip.stream(), ctypes.byref(d), hip.p(xs), hip.p(fs), None, hip.p(out))
+        if rc != 0:
+            refused += 1
+            assert "fixed scratch" in neoml_amd.last_error()
+            assert (hip.down(out) == 7.0).all()
+    if refused == 0:
+        pytest.skip("none of the shapes tried was cut into more slices than the fixed array holds")
