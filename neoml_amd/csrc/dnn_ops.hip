@@ -724,7 +724,16 @@ struct CLstmSeqArgs {
 	unsigned* GaveUp;              // host-visible word of the launch stream: set when a wavefront gives up
 	int T, B, H, Reverse;
 	unsigned MaxSpins;
+	// ( lstmDirectKernel ) XcdLayout != 0: the workgroups that share a block of sequences are meant to sit on one XCD
+	// ( workgroup i of a launch goes to XCD i mod 8: that is how the dispatcher deals them out ) and publish into
+	// ExchangeLocal as well, with plain stores, which stay in that XCD's L2; XcdTable[ workgroup ] receives 1 + the XCD
+	// each one really runs on, and only when all of a block's workgroups report the same one is ExchangeLocal read
+	int XcdLayout, XcdBase, RowBlocks;
+	unsigned long long* ExchangeLocal; // [2][B][H], zero at launch
+	unsigned* XcdTable;                // [ LstmXcdTableWords ], zero at launch
 };
+constexpr int LstmXcdTableWords = 256; // one word per workgroup of the layout by XCDs ( 8 x 32 )
+typedef unsigned u32x2 __attribute__( ( ext_vector_type( 2 ) ) );
 
 // Gate non-linearities on the hardware exp2 / reciprocal: 1 ulp each, and the cell update of a step sits on the
 // critical path of the whole device. Saturation: exp2 gives +inf / 0 at the ends, the reciprocal turns them into the
@@ -992,6 +1001,281 @@ void lstmSequenceKernel( const CLstmSeqArgs a )
 		// (the workgroups run in lockstep, so the others are about as far): a round of loads issued earlier would
 		// come back incomplete and cost a whole round trip.
 		__syncthreads();
+	}
+}
+
+// The same recurrence laid out by XCDs, for a device of 8 XCDs x 32 compute units: the workgroups that exchange values
+// sit on one XCD and talk through that XCD's L2 with plain stores and loads that pass the L1 ( a third of the latency of
+// a device-coherent store and load ), and the product takes its operand straight from the exchange: no staging of the
+// previous output in LDS, one barrier per step instead of three.
+//   workgroup  = 4 sequences x 32 hidden units ( 128 gate columns ); H / 64 product wavefronts + 2 cell wavefronts.
+//                What a step has to move grows with the sequences a workgroup holds ( every workgroup reads the whole
+//                previous output of its sequences: 4 x H tagged words ), and all of an XCD's workgroups ask the same L2
+//                for it at the same time: with 16 sequences per workgroup those loads alone took a microsecond.
+//   product    : v_mfma_f32_4x4x1_16b_f32, sixteen 4 x 4 rank-1 updates per instruction, with the A operand of one of
+//                the sixteen blocks broadcast to all: A = h[ 4 sequences ][ k ], B = Wrec[ k ][ 64 columns ], so four
+//                sequences fill the instruction. Wavefront m reduces over k = 64m .. 64m+63 for all 128 columns; its
+//                64 x 128 weights never leave its registers ( 128 per lane ). Lane ( b, i ) loads the tagged word
+//                h[ i ][ 64m + 16q + b ], q = 0..3: one register feeds sixteen instructions ( block b's value is
+//                broadcast by instruction b ), four 64-bit loads per lane and step.
+//                A wavefront waits with a light load ( one word of every store instruction that publishes into its k
+//                range ) and then asks for everything; what it uses is checked word by word.
+//   cells      : 128 cells, two wavefronts. Every load and store is a buffer access issued on every path ( a lane or
+//                step with nothing to move gets an offset beyond the range, which the hardware drops ), so the compiler
+//                can count what is in flight and wait for the gate loads alone; the wavefronts that publish never wait
+//                for a load of the exchange. The sums of the product wavefronts meet in LDS ( two buffers, by step
+//                parity ), one barrier, and the cell wavefronts finish the step while the product wavefronts already wait
+//                for the next one.
+//   placement  : the launch has 8 x 32 workgroups. The dispatcher deals a launch's workgroups out to the XCDs in turn,
+//                so every XCD receives 32; which XCD comes first is not known, so a workgroup asks where it runs and
+//                takes the next role of that XCD ( a counter per XCD ). XCDs without sequences have nothing to do:
+//                their workgroups leave at once ( the partner of a pair of launches uses them ).
+//   step 0     : the initial output ( or zero ) is published like a step's output before the loop, so every step is
+//                the same code. Step i reads buffer ( i+1 )&1 with tag i+1 and publishes into buffer i&1 with tag i+2:
+//                by the time a workgroup can publish step i, every workgroup of its sequences has published step i-1,
+//                i.e. has the values of step i-2, which this store overwrites, in registers.
+// set when a one-launch LSTM gave up ( for one, the device may not deal workgroups out as the layout by XCDs assumes ):
+// the process goes on without that layout
+static int xcdLayoutFailed = 0;
+constexpr int RowsKernelRows = 4;
+constexpr int RowsKernelUnits = 32;
+// f( integral_constant<int, 0> ) ... f( integral_constant<int, N-1> ), for arguments that have to be constants
+template<int N, class F>
+__device__ __forceinline__ void staticFor( F&& f )
+{
+	if constexpr( N > 0 ) {
+		staticFor<N - 1>( f );
+		f( std::integral_constant<int, N - 1>() );
+	}
+}
+template<int PW>
+__global__ __launch_bounds__( 64 * ( PW + 2 ) )
+void lstmRowsKernel( const CLstmSeqArgs a )
+{
+	__shared__ __attribute__( ( aligned( 16 ) ) ) float sumsLds[2][PW][RowsKernelRows][132];
+	__shared__ int giveUp;
+	__shared__ int role;
+	constexpr int H = 64 * PW;
+	constexpr int UnitGroups = H / RowsKernelUnits;
+	const int B = a.B;
+	const int tid = threadIdx.x;
+	const int wave = tid >> 6;
+	const int lane = tid & 63;
+	unsigned xcd = 0;
+	asm volatile( "s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"( xcd ) );
+	const int slot = ( static_cast<int>( xcd & 7 ) - a.XcdBase ) & 7;
+	if( slot >= a.RowBlocks ) {
+		return;
+	}
+	if( tid == 0 ) {
+		role = static_cast<int>( __hip_atomic_fetch_add( a.XcdTable + ( xcd & 7 ), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT ) );
+		giveUp = 0;
+	}
+	__syncthreads();
+	const int ticket = role;
+	const int unit0 = ( ticket % UnitGroups ) * RowsKernelUnits;
+	const int row0 = ( slot * ( 32 / UnitGroups ) + ticket / UnitGroups ) * RowsKernelRows;
+	if( ticket >= 32 || row0 >= B ) {
+		return; // ( more workgroups on this XCD than the dealing in turn gives it, or no sequences left for this role )
+	}
+	// ( 32-bit products on purpose: the scalar unit has no 64-bit multiply, and a 64-bit product would put every address
+	// derived from it, buffer descriptors included, into vector registers; the host checks that T * B * 4H fits 31 bits )
+	const unsigned stepSize = static_cast<unsigned>( B ) * static_cast<unsigned>( H );
+	const unsigned stepBytes = stepSize * 4u;
+	const bool product = wave < PW;
+	const __amdgpu_buffer_rsrc_t exchange = __builtin_amdgcn_make_buffer_rsrc( a.ExchangeLocal, 0, stepBytes * 4u, 0x00020000 );
+
+	// ---- cell wavefronts: the cell of this lane
+	const int cellId = ( wave - PW ) * 64 + lane;
+	const int cellRow = ( cellId / RowsKernelUnits ) & ( RowsKernelRows - 1 );
+	const int cellUnit = cellId % RowsKernelUnits;
+	const int cellB = row0 + cellRow;
+	const bool cellActive = !product && cellB < B;
+	const unsigned cellInStep = static_cast<unsigned>( cellB ) * H + unit0 + cellUnit;
+	float cState = ( cellActive && a.C0 != nullptr ) ? a.C0[cellInStep] : 0.f;
+	float gNext[4] = { 0.f, 0.f, 0.f, 0.f };
+	const unsigned gateOffset = cellActive ? ( static_cast<unsigned>( cellB ) * 4u * H + unit0 + cellUnit ) * 4u : OutOfRange;
+	auto requestGates = [&]( int step ) {
+		const int p = a.Reverse ? a.T - 1 - step : step;
+		const __amdgpu_buffer_rsrc_t gates = __builtin_amdgcn_make_buffer_rsrc(
+			const_cast<float*>( a.Gates + static_cast<size_t>( step < a.T ? static_cast<unsigned>( p ) * ( stepSize * 4u ) : 0u ) ), 0,
+			step < a.T ? stepBytes * 4u : 0u, 0x00020000 );
+#pragma unroll
+		for( int q = 0; q < 4; ++q ) {
+			gNext[q] = __uint_as_float( __builtin_amdgcn_raw_buffer_load_b32( gates, gateOffset, q * H * 4, 0 ) );
+		}
+	};
+	auto publish = [&]( float h, unsigned tag, unsigned parity ) {
+		// one 64-bit store that this XCD's L2 holds: value and "it has been written" arrive in the same word
+		const u32x2 word = { __float_as_uint( h ), tag };
+		__builtin_amdgcn_raw_buffer_store_b64( word, exchange, cellActive ? ( parity * stepSize + cellInStep ) * 8u : OutOfRange, 0, 0 );
+	};
+	float h0 = 0.f;
+	if( cellActive && a.H0 != nullptr ) {
+		h0 = a.H0[cellInStep];
+	}
+	requestGates( 0 );
+	publish( h0, 1u, 1u );
+	// ( the compiler's count of what may be in flight at the top of the loop is the worse of the two ways there: the two
+	// output stores that follow a step's publication follow the first one too, beyond every range )
+	__builtin_amdgcn_raw_buffer_store_b32( 0u, exchange, OutOfRange, 0, 0 );
+	__builtin_amdgcn_raw_buffer_store_b32( 0u, exchange, OutOfRange, 0, 0 );
+
+	// ---- product wavefronts
+	// lane ( b, j ) of the B operand: column 4b + j of a 64-column half = gate j of unit 16 * half + b
+	// lane ( b, i ) of the A operand: sequence i of the workgroup, k = 16q + b of the wavefront's 64
+	const int lb = lane >> 2;
+	const int li = lane & 3;
+	float weights[2][64];
+	if( product ) {
+#pragma unroll
+		for( int half = 0; half < 2; ++half ) {
+			const float* from = a.Wrec + ( static_cast<size_t>( li ) * H + unit0 + half * 16 + lb ) * H + wave * 64;
+#pragma unroll
+			for( int k4 = 0; k4 < 16; ++k4 ) {
+				const float4 v = *reinterpret_cast<const float4*>( from + k4 * 4 );
+				weights[half][k4 * 4] = v.x; weights[half][k4 * 4 + 1] = v.y; weights[half][k4 * 4 + 2] = v.z; weights[half][k4 * 4 + 3] = v.w;
+			}
+		}
+	}
+	const bool rowValid = row0 + li < B;
+	const unsigned laneWords = rowValid ? ( static_cast<unsigned>( row0 + li ) * H + wave * 64 + lb ) * 8u : OutOfRange;
+	const unsigned rowMask = rowValid ? 0xffffffffu : 0u;
+	// The light load: the wavefront's 64 k are two producers of 32 units, each with two cell wavefronts of two sequences:
+	// lane l < 4 looks at producer l / 2, sequence 2 * ( l % 2 ).
+	unsigned lightWords = OutOfRange;
+	if( lane < 4 && row0 + 2 * ( lane & 1 ) < B ) {
+		lightWords = ( static_cast<unsigned>( row0 + 2 * ( lane & 1 ) ) * H + wave * 64 + ( lane >> 1 ) * RowsKernelUnits ) * 8u;
+	}
+	const unsigned lightMask = lightWords != OutOfRange ? 0xffffffffu : 0u;
+
+	for( int counter = 0; counter < a.T; ++counter ) {
+		// ( the counter of a loop that lanes can leave at different times, as the compiler sees the give-up exit, lives in a
+		// vector register; buffer descriptors derived from it would be rebuilt lane by lane )
+		const int i = __builtin_amdgcn_readfirstlane( counter );
+		const int pos = a.Reverse ? a.T - 1 - i : i;
+		if( product ) {
+			const unsigned tag = static_cast<unsigned>( i + 1 );
+			const unsigned parityBytes = static_cast<unsigned>( ( i + 1 ) & 1 ) * stepBytes * 2u;
+			// ( ACCS accumulators per half take the instructions in turn, so that one does not wait for the one before it;
+			// the widest shape has no registers to spare for a second one )
+			constexpr int ACCS = PW < 8 ? 2 : 1;
+			f32x4v acc[2][ACCS];
+#pragma unroll
+			for( int half = 0; half < 2; ++half ) {
+#pragma unroll
+				for( int e = 0; e < ACCS; ++e ) {
+					acc[half][e] = f32x4v{ 0.f, 0.f, 0.f, 0.f };
+				}
+			}
+			unsigned spins = 0;
+			while( true ) {
+				asm volatile( "" ::: "memory" ); // ( every round asks the memory again )
+				const u32x2 first = __builtin_amdgcn_raw_buffer_load_b64( exchange, lightWords, parityBytes, 2 );
+				if( __builtin_amdgcn_ballot_w64( ( ( first.y ^ tag ) & lightMask ) != 0 ) == 0 || ++spins > a.MaxSpins ) {
+					break; // ( at the spin limit the rounds below fail and give up )
+				}
+			}
+			u32x2 word[4];
+			auto arrived = [&]( int q ) {
+				return __builtin_amdgcn_ballot_w64( ( ( word[q].y ^ tag ) & rowMask ) != 0 ) == 0;
+			};
+			auto multiply = [&]( int q ) {
+				const float h = __uint_as_float( word[q].x );
+				staticFor<16>( [&]( auto blockOf ) {
+					constexpr int b = decltype( blockOf )::value;
+					// cbsz 4: the A operand of block `b` goes to all sixteen blocks ( the block is part of the instruction )
+					acc[0][b % ACCS] = __builtin_amdgcn_mfma_f32_4x4x1f32( h, weights[0][q * 16 + b], acc[0][b % ACCS], 4, b, 0 );
+					acc[1][b % ACCS] = __builtin_amdgcn_mfma_f32_4x4x1f32( h, weights[1][q * 16 + b], acc[1][b % ACCS], 4, b, 0 );
+				} );
+			};
+			// All four loads are asked for at once ( aux 2: past the L1, into this XCD's L2 ) and a quarter is multiplied
+			// as soon as its load has come back, always in order: the sum does not depend on what arrived when.
+			asm volatile( "" ::: "memory" );
+#pragma unroll
+			for( int q = 0; q < 4; ++q ) {
+				word[q] = __builtin_amdgcn_raw_buffer_load_b64( exchange, laneWords, parityBytes + q * 128, 2 );
+			}
+			int good = 0;
+#pragma unroll
+			for( int q = 0; q < 4; ++q ) {
+				if( good == q && arrived( q ) ) {
+					multiply( q );
+					good = q + 1;
+				}
+			}
+			bool gone = false;
+#pragma unroll
+			for( int q = 0; q < 4; ++q ) {
+				if( q < good || gone ) {
+					continue;
+				}
+				// this quarter was not there yet: its load again until it is
+				while( true ) {
+					if( ++spins > a.MaxSpins || ( ( spins & 15 ) == 0
+						&& __hip_atomic_load( a.Abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT ) != 0 ) )
+					{
+						__hip_atomic_store( a.Abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT );
+						if( lane == 0 ) {
+							// the abort word lives in the caller's workspace, which the caller is free to recycle: the host
+							// learns of the give-up through this word of pinned host memory that belongs to the launch stream
+							__hip_atomic_store( a.GaveUp, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM );
+						}
+						giveUp = 1; // read by the whole workgroup after the barrier
+						gone = true;
+						break;
+					}
+					asm volatile( "" ::: "memory" );
+					word[q] = __builtin_amdgcn_raw_buffer_load_b64( exchange, laneWords, parityBytes + q * 128, 2 );
+					if( arrived( q ) ) {
+						break;
+					}
+				}
+				if( !gone ) {
+					multiply( q );
+				}
+			}
+			// accumulator register r of lane ( b, j ) is ( sequence r, column 4b + j ) of the half
+#pragma unroll
+			for( int half = 0; half < 2; ++half ) {
+#pragma unroll
+				for( int r = 0; r < 4; ++r ) {
+					sumsLds[i & 1][wave][r][half * 64 + lane] = ACCS == 2 ? acc[half][0][r] + acc[half][ACCS - 1][r] : acc[half][0][r];
+				}
+			}
+		}
+		__syncthreads();
+		if( giveUp != 0 ) {
+			return; // uniform: every thread reads the same LDS word after the barrier
+		}
+		if( !product ) {
+			float g[4];
+#pragma unroll
+			for( int q = 0; q < 4; ++q ) {
+				g[q] = gNext[q];
+			}
+#pragma unroll
+			for( int wv = 0; wv < PW; ++wv ) {
+				const float4 part = *reinterpret_cast<const float4*>( &sumsLds[i & 1][wv][cellRow][cellUnit * 4] );
+				g[0] += part.x; g[1] += part.y; g[2] += part.z; g[3] += part.w;
+			}
+			requestGates( i + 1 );
+			const float m = seqTanh( g[0] );
+			const float f = seqSigmoid( g[1] );
+			const float in = seqSigmoid( g[2] );
+			const float o = seqSigmoid( g[3] );
+			cState = f * cState + in * m;
+			const float h = o * seqTanh( cState );
+			// ( the last step publishes too: nobody reads it, and the next launch starts from cleared buffers )
+			publish( h, static_cast<unsigned>( i + 2 ), static_cast<unsigned>( i & 1 ) );
+			const unsigned outOffset = cellActive ? cellInStep * 4u : OutOfRange;
+			const size_t outAt = static_cast<size_t>( static_cast<unsigned>( pos ) * stepSize );
+			const __amdgpu_buffer_rsrc_t hOut = __builtin_amdgcn_make_buffer_rsrc( a.HOut + outAt, 0, stepBytes, 0x00020000 );
+			const __amdgpu_buffer_rsrc_t cOut = __builtin_amdgcn_make_buffer_rsrc(
+				a.COut != nullptr ? a.COut + outAt : a.HOut, 0, a.COut != nullptr ? stepBytes : 0u, 0x00020000 );
+			__builtin_amdgcn_raw_buffer_store_b32( __float_as_uint( h ), hOut, outOffset, 0, 0 );
+			__builtin_amdgcn_raw_buffer_store_b32( __float_as_uint( cState ), cOut, outOffset, 0, 0 );
+		}
 	}
 }
 
@@ -1640,6 +1924,9 @@ int checkSequenceGiveUps( hipStream_t stream )
 		if( *word != 0 ) {
 			*word = 0;
 			gaveUp = true;
+			if( getenv( "NH_LSTM_SPIN_LIMIT" ) == nullptr ) { // ( not when a test forces the give-up through the spin limit )
+				__atomic_store_n( &xcdLayoutFailed, 1, __ATOMIC_RELAXED ); // ( whichever layout it was: the plain one asks less )
+			}
 		}
 	}
 	if( !gaveUp ) {
@@ -1696,9 +1983,11 @@ void releaseSequenceStream( hipStream_t stream )
 
 // ---- whole-sequence LSTM launch ------------------------------------------------------------------------------
 
-// The shapes of the one-launch kernel: Rows sequences x ( 4 * Blocks ) hidden units per workgroup of Waves wavefronts.
+// The shapes of the one-launch kernels: Rows sequences x ( 4 * Blocks ) hidden units per workgroup of Waves wavefronts.
+// ByXcd: lstmRowsKernel ( the layout by XCDs ), otherwise lstmSequenceKernel.
 struct CLstmSeqShape {
 	int Rows, Blocks, Waves;
+	bool ByXcd;
 	const void* Kernel;
 	void ( *Launch )( hipStream_t, unsigned, size_t, const CLstmSeqArgs& );
 };
@@ -1709,18 +1998,43 @@ static void launchSeqShape( hipStream_t stream, unsigned groups, size_t lds, con
 	hipLaunchKernelGGL( ( lstmSequenceKernel<RB, CB, W> ), dim3( groups ), dim3( 64 * W ), lds, stream, a );
 }
 
-#define NH_SEQ_SHAPE( RB, CB, W ) { RB, CB, W, reinterpret_cast<const void*>( &lstmSequenceKernel<RB, CB, W> ), &launchSeqShape<RB, CB, W> }
-// in order of preference (measured at 64 sequences x 256 units, 128 steps: 433 / 445 / 515 us for the first three;
-// a v_mfma_f32_16x16x4_f32 issues every 64 clocks, so the narrow workgroup has the shortest product phase)
+template<int PW>
+static void launchRowsShape( hipStream_t stream, unsigned groups, size_t, const CLstmSeqArgs& a )
+{
+	hipLaunchKernelGGL( ( lstmRowsKernel<PW> ), dim3( groups ), dim3( 64 * ( PW + 2 ) ), 0, stream, a );
+}
+
+#define NH_SEQ_SHAPE( RB, CB, W ) { RB, CB, W, false, reinterpret_cast<const void*>( &lstmSequenceKernel<RB, CB, W> ), &launchSeqShape<RB, CB, W> }
+#define NH_ROWS_SHAPE( PW ) { RowsKernelRows, RowsKernelUnits / SeqUnits, PW + 2, true, reinterpret_cast<const void*>( &lstmRowsKernel<PW> ), &launchRowsShape<PW> }
+// in order of preference (measured at 64 sequences x 256 units, 128 steps: 433 / 445 / 515 us for the first three
+// lstmSequenceKernel shapes; a v_mfma_f32_16x16x4_f32 issues every 64 clocks, so the narrow workgroup has the shortest
+// product phase)
 static const CLstmSeqShape lstmSeqShapes[] = {
+	NH_ROWS_SHAPE( 1 ), NH_ROWS_SHAPE( 2 ), NH_ROWS_SHAPE( 4 ), NH_ROWS_SHAPE( 8 ),
 	NH_SEQ_SHAPE( 16, 1, 8 ), NH_SEQ_SHAPE( 16, 2, 8 ), NH_SEQ_SHAPE( 16, 4, 8 ), NH_SEQ_SHAPE( 16, 2, 16 ), NH_SEQ_SHAPE( 16, 4, 16 ),
 	NH_SEQ_SHAPE( 32, 2, 16 ) };
 constexpr size_t LdsLimit = 160 * 1024 - 256; // dynamic part; the kernel also has a static word
 
 static size_t lstmSequenceLds( int H, const CLstmSeqShape& shape )
 {
+	if( shape.ByXcd ) {
+		return 0; // ( its LDS is static )
+	}
 	const size_t cols = 16 * static_cast<size_t>( shape.Blocks );
 	return ( ( cols + shape.Rows ) * ( H + 4 ) + 4 + static_cast<size_t>( shape.Waves ) * shape.Rows * ( cols + 4 ) ) * sizeof( float );
+}
+
+// Can the shape's kernel run this size at all ( the grid aside )?
+static bool lstmShapeTakes( int H, const CLstmSeqShape& shape )
+{
+	if( shape.ByXcd ) {
+		return H == 64 * ( shape.Waves - 2 ); // one product wavefront per 64 k
+	}
+	if( H % ( SeqUnits * shape.Blocks ) != 0 || lstmSequenceLds( H, shape ) > LdsLimit ) {
+		return false;
+	}
+	const int batch = 16; // lstmSequenceKernel's Batch: its loaders cover the tile in one batch
+	return static_cast<long long>( shape.Rows ) * H <= static_cast<long long>( batch ) * ( shape.Waves / 2 ) * 64;
 }
 
 // The first shape whose grid fits the device; null = none does.
@@ -1741,6 +2055,9 @@ static const CLstmSeqShape* lstmSequenceShape( int H, int B, bool halfDevice = f
 	if( !ldsRaised ) {
 		// beyond 64 KB of dynamic LDS a kernel has to ask
 		for( const CLstmSeqShape& shape : lstmSeqShapes ) {
+			if( shape.ByXcd ) {
+				continue;
+			}
 			const hipError_t err = hipFuncSetAttribute( shape.Kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>( LdsLimit ) );
 			if( err != hipSuccess ) {
 				setLastError( "lstm: hipFuncSetAttribute failed: %s", hipGetErrorString( err ) );
@@ -1752,10 +2069,7 @@ static const CLstmSeqShape* lstmSequenceShape( int H, int B, bool halfDevice = f
 	}
 	for( const CLstmSeqShape& shape : lstmSeqShapes ) {
 		const size_t lds = lstmSequenceLds( H, shape );
-		const int batch = 16; // the kernel's Batch
-		if( H % ( SeqUnits * shape.Blocks ) != 0 || lds > LdsLimit
-			|| static_cast<long long>( shape.Rows ) * H > static_cast<long long>( batch ) * ( shape.Waves / 2 ) * 64 )
-		{
+		if( shape.ByXcd || !lstmShapeTakes( H, shape ) ) {
 			continue;
 		}
 		int perUnit = 0;
@@ -1774,6 +2088,44 @@ static const CLstmSeqShape* lstmSequenceShape( int H, int B, bool halfDevice = f
 	}
 	// ( no shape of half the device: the whole one, and no partner beside it )
 	return halfDevice ? lstmSequenceShape( H, B, false ) : nullptr;
+}
+
+// How many XCDs the layout by XCDs needs for B sequences of H units: an XCD's 32 workgroups hold 4 sequences x 32 units each.
+static int lstmXcdsNeeded( int H, int B )
+{
+	const int rowsPerXcd = RowsKernelRows * ( 32 / ( H / RowsKernelUnits ) );
+	return ceilDiv( B, rowsPerXcd );
+}
+
+// The shape of the layout by XCDs ( lstmRowsKernel ) if the device has 8 XCDs of 32 compute units and the sequences fit
+// the XCDs the launch may use ( all eight, or four when two launches share the device ); null: the plain layout.
+static const CLstmSeqShape* lstmXcdShape( int H, int B, bool halfDevice )
+{
+	static const bool enabled = []() {
+		const char* env = getenv( "NH_LSTM_XCD_LAYOUT" ); // "0" switches the layout off ( measurements )
+		return env == nullptr || env[0] != '0';
+	}();
+	int device = 0, units = 0;
+	if( !enabled || __atomic_load_n( &xcdLayoutFailed, __ATOMIC_RELAXED ) != 0 || hipGetDevice( &device ) != hipSuccess
+		|| hipDeviceGetAttribute( &units, hipDeviceAttributeMultiprocessorCount, device ) != hipSuccess || units != 256 )
+	{
+		( void )hipGetLastError();
+		return nullptr;
+	}
+	for( const CLstmSeqShape& shape : lstmSeqShapes ) {
+		if( !shape.ByXcd || !lstmShapeTakes( H, shape ) ) {
+			continue;
+		}
+		int perUnit = 0;
+		if( lstmXcdsNeeded( H, B ) > ( halfDevice ? 4 : 8 )
+			|| hipOccupancyMaxActiveBlocksPerMultiprocessor( &perUnit, shape.Kernel, 64 * shape.Waves, 0 ) != hipSuccess || perUnit < 1 )
+		{
+			( void )hipGetLastError();
+			return nullptr;
+		}
+		return &shape;
+	}
+	return nullptr;
 }
 
 static bool lstmSequenceFits( int H, int B, const float* wRec, const float* c0, const float* h0, const float* hOut )
@@ -1814,14 +2166,18 @@ static bool lstmSequenceAllowed( hipStream_t stream )
 static int launchLstmSequence( hipStream_t stream, CLstmSeqArgs a, bool halfDevice = false, const unsigned long long* partnerOf = nullptr,
 	bool* tookHalf = nullptr, unsigned long long* generation = nullptr, bool* ranBeside = nullptr )
 {
-	const CLstmSeqShape* shape = lstmSequenceShape( a.H, a.B, halfDevice );
+	const CLstmSeqShape* xcdShape = lstmXcdShape( a.H, a.B, halfDevice );
+	const CLstmSeqShape* shape = xcdShape != nullptr ? xcdShape : lstmSequenceShape( a.H, a.B, halfDevice );
 	NH_REQUIRE( shape != nullptr );
 	int device = 0;
 	NH_HIP( hipGetDevice( &device ) );
 	int computeUnits = 0;
 	NH_HIP( hipDeviceGetAttribute( &computeUnits, hipDeviceAttributeMultiprocessorCount, device ) );
 	const long long shapeGroups = static_cast<long long>( a.H / ( SeqUnits * shape->Blocks ) ) * ceilDiv( a.B, shape->Rows );
-	const bool isHalf = shapeGroups <= computeUnits / 2;
+	// ( in the layout by XCDs a launch holds as many XCDs as it has blocks of sequences )
+	const bool isHalf = xcdShape != nullptr ? lstmXcdsNeeded( a.H, a.B ) <= 4 : shapeGroups <= computeUnits / 2;
+	a.XcdLayout = xcdShape != nullptr ? 1 : 0;
+	a.RowBlocks = xcdShape != nullptr ? lstmXcdsNeeded( a.H, a.B ) : ceilDiv( a.B, shape->Rows ); // ( by XCDs: the XCDs in use )
 	if( tookHalf != nullptr ) {
 		*tookHalf = isHalf;
 	}
@@ -1864,9 +2220,13 @@ static int launchLstmSequence( hipStream_t stream, CLstmSeqArgs a, bool halfDevi
 	}
 	a.GaveUp = own.GaveUp;
 	own.Launched = true;
-	const unsigned groups = static_cast<unsigned>( ( a.H / ( SeqUnits * shape->Blocks ) ) * ceilDiv( a.B, shape->Rows ) );
+	// a partner takes the XCDs its partner leaves free
+	a.XcdBase = partner ? 4 : 0;
+	const unsigned groups = a.XcdLayout != 0 ? 256u
+		: static_cast<unsigned>( ( a.H / ( SeqUnits * shape->Blocks ) ) * ceilDiv( a.B, shape->Rows ) );
 	// the exchange buffers and the abort word that follows them
-	const long long words = 2LL * a.B * a.H + 1;
+	// both sets of exchange buffers, the table of XCDs and the abort word that follow them
+	const long long words = 4LL * a.B * a.H + LstmXcdTableWords / 2 + 1;
 	hipLaunchKernelGGL( clearWordsKernel, dim3( static_cast<unsigned>( ( words + 1023 ) / 1024 ) ), dim3( 256 ), 0, stream, a.Exchange, words );
 	shape->Launch( stream, groups, lstmSequenceLds( a.H, *shape ), a );
 	NH_LAUNCH_CHECK();
@@ -2714,12 +3074,13 @@ int nhStreamOverlapLstm( nhStream s, int enable )
 	return NH_OK;
 }
 
-// workspace layout: [ gates: T*B*4H ][ free term: 4H ][ state: B*H ][ tagged h exchange: 2*B*H 64-bit words ][ abort word: 64 bits ]
+// workspace layout: [ gates: T*B*4H ][ free term: 4H ][ state: B*H ][ tagged h exchange: 2*B*H 64-bit words ]
+// [ the same for readers on the writer's XCD ][ table of XCDs: 256 words ][ abort word: 64 bits ]
 int nhLstmWorkspaceSize( int hiddenSize, int objectSize, int sequenceLength, int sequenceCount, size_t* bytes )
 {
 	NH_REQUIRE( bytes != nullptr && hiddenSize > 0 && objectSize > 0 && sequenceLength >= 0 && sequenceCount >= 0 );
 	const size_t gates = static_cast<size_t>( sequenceLength ) * sequenceCount * 4 * hiddenSize;
-	*bytes = ( gates + 4 * static_cast<size_t>( hiddenSize ) + 5 * static_cast<size_t>( sequenceCount ) * hiddenSize + 2 ) * sizeof( float );
+	*bytes = ( gates + 4 * static_cast<size_t>( hiddenSize ) + 9 * static_cast<size_t>( sequenceCount ) * hiddenSize + LstmXcdTableWords + 2 ) * sizeof( float );
 	return NH_OK;
 }
 
@@ -2783,7 +3144,8 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 				const long long groups = static_cast<long long>( H / ( SeqUnits * lstmSequenceShape( H, B, true )->Blocks ) )
 					* ceilDiv( B, lstmSequenceShape( H, B, true )->Rows );
 				int units = 0;
-				beside = hipDeviceGetAttribute( &units, hipDeviceAttributeMultiprocessorCount, device ) == hipSuccess && groups <= units / 2;
+				beside = lstmXcdShape( H, B, true ) != nullptr
+					|| ( hipDeviceGetAttribute( &units, hipDeviceAttributeMultiprocessorCount, device ) == hipSuccess && groups <= units / 2 );
 			}
 			for( int i = 0; beside && i < 3; ++i ) {
 				for( int j = 0; j < 3; ++j ) {
@@ -2824,7 +3186,9 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 		a.Gates = gates; a.Wrec = recurrentWeights; a.H0 = inputMainBackLink; a.C0 = inputStateBackLink;
 		a.HOut = outputMainBackLink; a.COut = outputStateBackLink;
 		a.Exchange = reinterpret_cast<unsigned long long*>( stateScratch + static_cast<size_t>( B ) * H );
-		a.Abort = reinterpret_cast<unsigned*>( a.Exchange + 2 * static_cast<size_t>( B ) * H );
+		a.ExchangeLocal = a.Exchange + 2 * static_cast<size_t>( B ) * H;
+		a.XcdTable = reinterpret_cast<unsigned*>( a.ExchangeLocal + 2 * static_cast<size_t>( B ) * H );
+		a.Abort = a.XcdTable + LstmXcdTableWords; // ( the last 8 bytes of the workspace )
 		a.T = T; a.B = B; a.H = H; a.Reverse = reverse ? 1 : 0;
 		a.MaxSpins = lstmSpinLimit();
 		bool tookHalf = false, ranBeside = false;

@@ -1057,6 +1057,25 @@ def test_mobilenetv3_blocks(case):
         assert_close(got, want, "post-SE into its residual", atol=2e-5)
 
 
+def test_lstm_layout_by_xcds_ragged_and_full():
+    """The one-launch kernel that lays the sequences out by XCDs ( H = 64, 128, 256, 512 ): sequence counts that are no
+    multiple of a workgroup's four, one that leaves whole XCDs without work and the most that fit the eight XCDs, with and
+    without initial state, both directions, cell state asked for."""
+    g = rng(186)
+    for T, B, In, H in ((9, 13, 24, 64), (5, 130, 16, 128), (4, 128, 32, 256), (6, 127, 8, 256), (3, 1, 8, 512), (12, 64, 16, 512)):
+        w_in = g.uniform(-0.2, 0.2, (4 * H, In)).astype(np.float32)
+        w_rec = g.uniform(-2.0 / H ** 0.5, 2.0 / H ** 0.5, (4 * H, H)).astype(np.float32)
+        b_in = g.uniform(-0.5, 0.5, 4 * H).astype(np.float32)
+        x = g.uniform(-1, 1, (T, B, In)).astype(np.float32)
+        for reverse, with_init in ((False, True), (True, False)):
+            c0 = g.uniform(-1, 1, (B, H)).astype(np.float32) if with_init else None
+            h0 = g.uniform(-1, 1, (B, H)).astype(np.float32) if with_init else None
+            h, c = hip().lstm(w_in, b_in, w_rec, None, x, reverse, c0, h0)
+            oh, oc = orc.lstm(w_in, b_in, w_rec, None, x, reverse, c0, h0)
+            assert_close(h, oh, "lstm h %s" % ((T, B, In, H, reverse),))
+            assert_close(c, oc, "lstm c %s" % ((T, B, In, H, reverse),))
+
+
 def test_lstm_long_sequence():
     # 128 steps through the one-launch path (H a multiple of 16 and a grid that fits the device), H = 512 through
     # its 16-wavefront shape, plus a shape whose grid does not fit and takes the launch-per-step path
@@ -1199,12 +1218,16 @@ def test_independent_lstms_side_by_side(capsys):
         assert lib.nhStreamSynchronize(ps) == 0
         return start.elapsed_time(stop), out[0].cpu().numpy().copy(), out[1].cpu().numpy().copy()
 
+    def best_of(times):
+        runs = [both_directions() for _ in range(times)]
+        return (min(r[0] for r in runs),) + runs[-1][1:]
+
     both_directions()
-    in_order_ms, f0, r0 = both_directions()
+    in_order_ms, f0, r0 = best_of(4)
     neoml_amd.check(lib.nhStreamOverlapLstm(ps, 1))
     try:
         both_directions()
-        side_by_side_ms, f1, r1 = both_directions()
+        side_by_side_ms, f1, r1 = best_of(4)
         with capsys.disabled():
             print("\ntwo LSTM directions, %d steps, %d sequences, %d units: %.0f us in order, %.0f us side by side" % (
                 T, B, H, in_order_ms * 1e3, side_by_side_ms * 1e3))
