@@ -100,6 +100,52 @@ def cdnn_run_once(batch, image):
     return fig
 
 
+def lstm_overlap_report(be, plan, steps):
+    """Did the two directions of the bidirectional layers run side by side? The same replay with nhStreamOverlapLstm on and
+    off: the step time, and the span of a layer's pair of nhLstm calls (event before the first call, event behind the
+    second, both on the launch stream, which waits for the side stream behind the second call)."""
+    import ctypes
+    import torch
+    lib, ms = be.lib, ctypes.c_float(0)
+    report = {}
+    for mode, enable in (("in_order", 0), ("side_by_side", 1)):  # ( ends with the overlap on, as the network asked )
+        be.na.check(lib.nhStreamOverlapLstm(be.stream, enable))
+        for _ in range(3):
+            plan.run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            plan.run()
+        torch.cuda.synchronize()
+        step_ms = (time.perf_counter() - t0) / steps * 1e3
+        # events around each pair only: one between the two calls would be a launch between them, and the second call
+        # then has to stay behind the first
+        record, check = lib.nhEventRecord, be.na.check
+        pairs = []
+        for _ in range(steps):
+            seen = 0
+            for fn, fargs, tag, _, _ in plan.launches:
+                if tag == "lstm" and seen % 2 == 0:
+                    start, stop = ctypes.c_void_p(), ctypes.c_void_p()
+                    check(lib.nhEventCreate(ctypes.byref(start)))
+                    check(lib.nhEventCreate(ctypes.byref(stop)))
+                    record(start, be.stream)
+                check(fn(*fargs))
+                if tag == "lstm":
+                    seen += 1
+                    if seen % 2 == 0:
+                        record(stop, be.stream)
+                        pairs.append((start, stop))
+        torch.cuda.synchronize()
+        spans = []
+        for start, stop in pairs:
+            check(lib.nhEventElapsedMs(start, stop, ctypes.byref(ms)))
+            spans.append(ms.value * 1e3)
+        report[mode] = {"ms_per_step": round(step_ms, 3), "pair_span_us": round(sum(spans) / max(len(spans), 1), 1)}
+    report["ran_side_by_side"] = report["side_by_side"]["pair_span_us"] < 0.9 * report["in_order"]["pair_span_us"]
+    return report
+
+
 def other_workload(args):
     """BASELINE configurations 3-5 at full size: same replay + event method, one JSON line with the per-family split."""
     import torch
@@ -143,12 +189,15 @@ def other_workload(args):
                       "gb_per_s": round(by / (tms * 1e-3) / 1e9, 1)}
         print("%-10s launches/step %4d  ms/step %8.3f  TFLOP/s %7.2f  GB/s %8.1f" % (
             tag, cnt // steps, tms / steps, fl / (tms * 1e-3) / 1e12 if fl else 0.0, by / (tms * 1e-3) / 1e9), file=sys.stderr)
+    extra = {}
+    if args.workload == "ocr":
+        extra["lstm_overlap"] = lstm_overlap_report(be, plan, steps)
     print(json.dumps({
         "metric": "%s (not the headline metric)" % unit, "value": round(items * steps / elapsed, 1), "unit": unit, "n_gpus": 1,
         "steps": steps, "warmup": args.warmup, "ms_per_step": round(elapsed / steps * 1e3, 3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": name + ", fp32, engine calls through the C ABI", "launches_per_step": len(plan.launches)},
-        "families": split}))
+        "families": split, **extra}))
 
 
 def main():
