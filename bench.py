@@ -21,21 +21,32 @@ sys.path.insert(0, ROOT)
 FP32_MFMA_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBPS = 8000.0
 # Bytes crossing the L2 <-> fabric boundary per 3x3-convolution launch, mean over the 16 launches of one step at
-# batch 64, 224x224: rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a known-size copy gives) 81.0 MB + WRITE_SIZE (x1.0)
-# 43.4 MB; profiles/resnet18_b64_conv_hbm_traffic.txt holds the two runs. Counters cannot be read from inside this
+# batch 64, 224x224: rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a known-size copy gives) 71.9 MB + WRITE_SIZE (x1.0)
+# 45.3 MB; profiles/resnet18_b64_conv_hbm_traffic.txt holds the two runs. Counters cannot be read from inside this
 # process, so the figure is a constant of the default workload (labelled as coming from that profile) and null for any other.
-CONV3X3_TRAFFIC_BYTES_B64_224 = 124.4e6
+CONV3X3_TRAFFIC_BYTES_B64_224 = 117.2e6
 CONV3X3_TRAFFIC_SOURCE = "offline_profile: profiles/resnet18_b64_conv_hbm_traffic.txt"
 
 
 def _cpu_model():
+    """What /proc/cpuinfo says of the host's first processor: the model name (a virtual machine may only give the brand)
+    with family / model / stepping and the clock it reports, which identify the part where the name does not."""
+    fields = {}
     try:
         for line in open("/proc/cpuinfo"):
-            if line.startswith("model name"):
-                return line.split(":", 1)[1].strip()
+            if ":" not in line:
+                if fields:
+                    break
+                continue
+            key, value = (t.strip() for t in line.split(":", 1))
+            fields.setdefault(key, value)
     except OSError:
-        pass
-    return "unknown"
+        return "unknown"
+    if "model name" not in fields:
+        return "unknown"
+    detail = ", ".join("%s %s" % (k, fields[k]) for k in ("cpu family", "model", "stepping") if k in fields)
+    mhz = " at %.0f MHz" % float(fields["cpu MHz"]) if "cpu MHz" in fields else ""
+    return "%s (%s%s)" % (fields["model name"], detail, mhz)
 
 
 def cpu_baseline(batch, image, replicas):
@@ -283,7 +294,7 @@ def main():
     launches, ms, flops, nbytes = c3
     achieved = flops / (ms * 1e-3) / 1e12
     roofline = {
-        "bound": "mfma", "kernel": "matMulKernel<AM_Conv> (3x3 convolutions, %d launches per step)" % (launches // max(args.steps, 1)),
+        "bound": "mfma", "kernel": "matMulKernel<AM_ConvTaps> (3x3 convolutions, %d launches per step)" % (launches // max(args.steps, 1)),
         "achieved": round(achieved, 2), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
         "traffic": CONV3X3_TRAFFIC_BYTES_B64_224 if (args.batch, args.image) == (64, 224) else None,
@@ -359,6 +370,8 @@ def main():
             # not of the sum, so the per-element bar is a strict one here; the reference's two GEMM backends show the scale
             builtin = cpu["logits_builtin_gemm"].reshape(-1, logits_gpu.shape[1])
             n = builtin.shape[0]
+            # ( all three on the same first images, so that the figures can be set side by side )
+            result["parity_logits_vs_cpu"]["same_images_vs_mlas_engine"] = distance(logits_gpu[:n], logits_cpu[:n])
             result["parity_logits_vs_cpu"]["vs_builtin_gemm_engine"] = distance(logits_gpu[:n], builtin)
             result["parity_logits_vs_cpu"]["reference_mlas_vs_builtin_gemm"] = distance(logits_cpu[:n], builtin)
         # the same network as an application of the reference runs it: NeoML's own CDnn and layer classes (compiled from the
