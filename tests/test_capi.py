@@ -62,8 +62,9 @@ def test_lstm_workspace_size():
     lib = neoml_amd.load()
     size = ctypes.c_size_t(0)
     neoml_amd.check(lib.nhLstmWorkspaceSize(256, 512, 128, 64, ctypes.byref(size)))
-    # gates for every step, summed free term, one step of cell state, two exchange buffers of 64-bit words, abort word
-    assert size.value == 4 * (128 * 64 * 1024 + 1024 + 64 * 256 + 2 * 2 * 64 * 256 + 2)
+    # gates for every step, summed free term, one step of cell state, two sets of two exchange buffers of 64-bit words
+    # ( one that every XCD sees, one for readers on the writer's XCD ), the per-XCD role counters, the abort word
+    assert size.value == 4 * (128 * 64 * 1024 + 1024 + 64 * 256 + 2 * 2 * 2 * 64 * 256 + 256 + 2)
 
 
 # ---- caching allocator on host memory (kind 1): same logic as on the device ------------------------------------
