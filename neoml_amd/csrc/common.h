@@ -14,14 +14,17 @@ void setLastError( const char* fmt, ... );
 
 // Streams on which two one-launch LSTMs that do not depend on each other may run side by side ( nhStreamOverlapLstm,
 // dnn_ops.hip ) need to know whether anything was enqueued between two nhLstm calls: every entry point turns its stream
-// handle into a stream here, so here is where that is noted. Costs one relaxed load while no stream has asked for it.
+// handle into a stream here, so here is where that is noted. Costs one relaxed load unless some stream's last launch is a
+// one-launch LSTM that still waits for a partner ( lstmPartnersAwaited: between an nhLstm call and the next call on its
+// stream ); only then are the device asked for and the lock taken.
 extern int overlapLstmStreams;
+extern int lstmPartnersAwaited;
 void noteStreamUse( hipStream_t stream );
 
 inline hipStream_t toStream( nhStream s )
 {
 	const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
-	if( __atomic_load_n( &overlapLstmStreams, __ATOMIC_RELAXED ) != 0 ) {
+	if( __atomic_load_n( &lstmPartnersAwaited, __ATOMIC_RELAXED ) != 0 ) {
 		noteStreamUse( stream );
 	}
 	return stream;

@@ -1019,7 +1019,9 @@ void lstmSequenceKernel( const CLstmSeqArgs a )
 //                h[ i ][ 64m + 16q + b ], q = 0..3: one register feeds sixteen instructions ( block b's value is
 //                broadcast by instruction b ), four 64-bit loads per lane and step.
 //                A wavefront waits with a light load ( one word of every store instruction that publishes into its k
-//                range ) and then asks for everything; what it uses is checked word by word.
+//                range ) and then asks for everything; what it uses is checked word by word. ( Waiting with the full
+//                request instead, 2 KB per wavefront and round, saves a round trip on paper and cost 15 %: 128 steps
+//                266 -> 308 us. The waiting loads of 128 workgroups per XCD stand in the way of the stores they wait for. )
 //   cells      : 128 cells, two wavefronts. Every load and store is a buffer access issued on every path ( a lane or
 //                step with nothing to move gets an offset beyond the range, which the hardware drops ), so the compiler
 //                can count what is in flight and wait for the gate loads alone; the wavefronts that publish never wait
@@ -1872,6 +1874,21 @@ static std::map<std::pair<int, hipStream_t>, CLstmOverlap>& lstmOverlaps()
 }
 
 int overlapLstmStreams = 0;
+int lstmPartnersAwaited = 0;
+
+// ( under sequenceLock ) the stream's last launch is / is no longer a one-launch LSTM that a partner may join; the count
+// of such streams is what every entry point looks at before it takes the lock
+static void setLastWasLstm( CLstmOverlap& o, bool value )
+{
+	if( o.LastWasLstm != value ) {
+		o.LastWasLstm = value;
+		if( value ) {
+			__atomic_fetch_add( &lstmPartnersAwaited, 1, __ATOMIC_RELAXED );
+		} else {
+			__atomic_fetch_sub( &lstmPartnersAwaited, 1, __ATOMIC_RELAXED );
+		}
+	}
+}
 
 // something is being enqueued on `stream` through this library: a one-launch LSTM on it has no partner any more
 void noteStreamUse( hipStream_t stream )
@@ -1884,7 +1901,7 @@ void noteStreamUse( hipStream_t stream )
 	std::lock_guard<std::mutex> guard( sequenceLock );
 	auto found = lstmOverlaps().find( std::make_pair( device, stream ) );
 	if( found != lstmOverlaps().end() ) {
-		found->second.LastWasLstm = false;
+		setLastWasLstm( found->second, false );
 	}
 }
 
@@ -1975,6 +1992,7 @@ void releaseSequenceStream( hipStream_t stream )
 		if( o.Enabled ) {
 			__atomic_fetch_sub( &overlapLstmStreams, 1, __ATOMIC_RELAXED );
 		}
+		setLastWasLstm( o, false );
 		lstmOverlaps().erase( overlap );
 	}
 }
@@ -3070,7 +3088,7 @@ int nhStreamOverlapLstm( nhStream s, int enable )
 		}
 		o.Enabled = enable != 0;
 	}
-	o.LastWasLstm = false;
+	setLastWasLstm( o, false );
 	return NH_OK;
 }
 
@@ -3153,7 +3171,7 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 						&& !rangesMeet( written[i], o.Read[j] );
 				}
 			}
-			o.LastWasLstm = false;
+			setLastWasLstm( o, false );
 			pair = o;
 		}
 	}
@@ -3211,7 +3229,7 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 			auto found = lstmOverlaps().find( std::make_pair( device, mainStream ) );
 			if( found != lstmOverlaps().end() ) {
 				CLstmOverlap& o = found->second;
-				o.LastWasLstm = true;
+				setLastWasLstm( o, true );
 				o.Generation = generation;
 				for( int i = 0; i < 3; ++i ) {
 					o.Written[i] = written[i];

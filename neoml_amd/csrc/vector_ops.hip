@@ -545,6 +545,14 @@ static int launchSum( nhStream s, const float* first, const float* second, int v
 	unsigned* counter = nullptr;
 	if( !streamMeetingPlace( toStream( s ), 2048, &partials, &counter ) ) {
 		partials = nullptr;
+		// a result that lies inside an operand must be read before it is written: zeroing it first would change the
+		// operand, so such a call ( rare: a capturing stream and an aliased result ) goes to one workgroup
+		const auto inside = [&]( const float* operand ) {
+			return operand != nullptr && result >= operand && result < operand + vectorSize;
+		};
+		if( inside( first ) || ( DOT && inside( second ) ) ) {
+			blocks = 1;
+		}
 		if( blocks == 1 ) {
 			partials = result; // ( not used by a single workgroup: only says that it may write the result itself )
 		} else if( !addToResult ) {
