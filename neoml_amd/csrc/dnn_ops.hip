@@ -2523,7 +2523,7 @@ template<int STRIDE, int KIN, bool CLIPPED>
 __global__ __launch_bounds__( 256, 2 )
 void expandDepthwiseKernel( const nhSeparableBlockDesc d, int outH, int outW, const float* input, const float* expandFilter,
 	const float* expandBias, const float* dwFilter, const float* dwBias, float* result, int tilesX, int tilesY, int totalTiles,
-	const CFusedActivation expandAct, const CFusedActivation dwAct )
+	const CFusedActivation expandAct, const CFusedActivation dwAct, unsigned resultBytes )
 {
 	constexpr int PH = STRIDE == 1 ? 8 : 7, PW = STRIDE == 1 ? 8 : 9;
 	constexpr int OH = ( PH - 3 ) / STRIDE + 1, OW = ( PW - 3 ) / STRIDE + 1;
@@ -2574,48 +2574,64 @@ void expandDepthwiseKernel( const nhSeparableBlockDesc d, int outH, int outW, co
 	// lane ( q, o ) sums 4 channels of the output pixels 8 pass + o: where their windows begin in the tile and where they go
 	constexpr int Passes = ( OH * OW + 7 ) / 8;
 	int windowAt[Passes];
-	long long storeAt[Passes]; // in floats from result, without the channel; negative: no such pixel
+	unsigned storeAt[Passes]; // byte offset in result, without the chunk's channels; out of range: no such pixel
 #pragma unroll
 	for( int pass = 0; pass < Passes; ++pass ) {
 		const int op = pass * 8 + ( lane >> 3 );
 		const int oy = op / OW, ox = op - oy * OW;
 		const int gy = ty * OH + oy, gx = tx * OW + ox;
-		windowAt[pass] = ( oy * STRIDE * PW + ox * STRIDE ) * PitchE + q4;
+		// ( lanes beyond the patch's outputs compute on the window at the origin; what they compute goes nowhere )
+		windowAt[pass] = ( op < OH * OW ? ( oy * STRIDE * PW + ox * STRIDE ) * PitchE : 0 ) + q4;
 		storeAt[pass] = ( op < OH * OW && gy < outH && gx < outW )
-			? ( ( static_cast<long long>( n ) * outH + gy ) * outW + gx ) * cexp + q4 : -1;
+			? static_cast<unsigned>( ( ( n * outH + gy ) * outW + gx ) * cexp + q4 ) * 4u : OutOfRange;
 	}
+	// Every load and store of the chunk loop is a buffer access issued on every path ( what has nothing to move gets an
+	// offset beyond the range: reads zeros, drops stores ), so that the compiler can count what is in flight: behind a
+	// branch it waits for everything, and a pass of outputs then began by waiting for the stores of the pass before it
+	// ( five round trips to memory per chunk, two thirds of the kernel's time ). A chunk's offset travels as the access's
+	// scalar offset, which the range check does not see: the lane's part says whether the lane has a row / a quad at all.
+	const __amdgpu_buffer_rsrc_t wBuffer = makeBuffer( expandFilter );
+	const __amdgpu_buffer_rsrc_t expandBiasBuffer = __builtin_amdgcn_make_buffer_rsrc(
+		const_cast<float*>( expandBias != nullptr ? expandBias : expandFilter ), 0, expandBias != nullptr ? BufferBytes : 0u, 0x00020000 );
+	const __amdgpu_buffer_rsrc_t fBuffer = makeBuffer( dwFilter );
+	const __amdgpu_buffer_rsrc_t dwBiasBuffer = __builtin_amdgcn_make_buffer_rsrc(
+		const_cast<float*>( dwBias != nullptr ? dwBias : dwFilter ), 0, dwBias != nullptr ? BufferBytes : 0u, 0x00020000 );
+	const __amdgpu_buffer_rsrc_t outBuffer = __builtin_amdgcn_make_buffer_rsrc( result, 0, resultBytes, 0x00020000 );
 	// a chunk's rows of the expand filter ( lane = channel c0 + l32 ) and its free term are requested one chunk ahead
 	float4 wNext[KG];
 	float biasNext = 0.f;
 	auto requestChunk = [&]( int c0 ) {
 		const bool rowOk = c0 + l32 < cexp;
-		const float* wRow = expandFilter + static_cast<long long>( rowOk ? c0 + l32 : 0 ) * KIN + half * 4;
+		const unsigned at = rowOk ? static_cast<unsigned>( l32 * KIN + half * 4 ) * 4u : OutOfRange;
 #pragma unroll
 		for( int g = 0; g < KG; ++g ) {
-			wNext[g] = *reinterpret_cast<const float4*>( wRow + g * 8 );
+			wNext[g] = bufferLoad4( wBuffer, at + g * 32u, static_cast<unsigned>( c0 ) * ( KIN * 4u ) );
 		}
-		biasNext = expandBias != nullptr ? expandBias[rowOk ? c0 + l32 : 0] : 0.f;
+		biasNext = __uint_as_float( __builtin_amdgcn_raw_buffer_load_b32( expandBiasBuffer, rowOk ? l32 * 4u : OutOfRange, c0 * 4, 0 ) );
 	};
 	requestChunk( 0 );
+	// ( the compiler's count of what may be in flight at the top of the loop is the worse of the two ways there: what
+	// follows a chunk's request in an iteration, ten loads' and Passes stores' worth, follows the first request too )
+#pragma unroll
+	for( int k = 0; k < 10 + Passes; ++k ) {
+		bufferStore4( outBuffer, OutOfRange + 16u * k, make_float4( 0.f, 0.f, 0.f, 0.f ) ); // ( distinct, or they are merged into one )
+	}
 	for( int c0 = 0; c0 < cexp; c0 += 32 ) {
-		const bool rowOk = c0 + l32 < cexp;
 		float4 w[KG];
 #pragma unroll
 		for( int g = 0; g < KG; ++g ) {
-			w[g] = rowOk ? wNext[g] : make_float4( 0.f, 0.f, 0.f, 0.f );
+			w[g] = wNext[g]; // ( rows beyond the last channel were read as zeros )
 		}
-		const float bias = rowOk ? biasNext : 0.f;
-		if( c0 + 32 < cexp ) {
-			requestChunk( c0 + 32 );
-		}
+		const float bias = biasNext;
+		requestChunk( c0 + 32 );
 		const bool quadOk = c0 + q4 < cexp;
+		const unsigned quadAt = quadOk ? q4 * 4u : OutOfRange;
 		float4 f[9];
 #pragma unroll
 		for( int k = 0; k < 9; ++k ) {
-			f[k] = quadOk ? *reinterpret_cast<const float4*>( dwFilter + k * cexp + c0 + q4 ) : make_float4( 0.f, 0.f, 0.f, 0.f );
+			f[k] = bufferLoad4( fBuffer, quadAt, static_cast<unsigned>( k * cexp + c0 ) * 4u );
 		}
-		const float4 bias4 = ( dwBias != nullptr && quadOk ) ? *reinterpret_cast<const float4*>( dwBias + c0 + q4 )
-			: make_float4( 0.f, 0.f, 0.f, 0.f );
+		const float4 bias4 = bufferLoad4( dwBiasBuffer, quadAt, static_cast<unsigned>( c0 ) * 4u );
 #pragma unroll
 		for( int b = 0; b < 2; ++b ) {
 			// the accumulator starts as the free term: every register of a lane belongs to the lane's channel
@@ -2650,17 +2666,16 @@ void expandDepthwiseKernel( const nhSeparableBlockDesc d, int outH, int outW, co
 		__builtin_amdgcn_fence( __ATOMIC_ACQUIRE, "wavefront" );
 #pragma unroll
 		for( int pass = 0; pass < Passes; ++pass ) {
-			if( storeAt[pass] >= 0 && quadOk ) {
-				const float* e = tile + windowAt[pass];
-				float4 acc = CChanVec<4>::fma( *reinterpret_cast<const float4*>( e ), f[0], bias4 );
+			const float* e = tile + windowAt[pass];
+			float4 acc = CChanVec<4>::fma( *reinterpret_cast<const float4*>( e ), f[0], bias4 );
 #pragma unroll
-				for( int k = 1; k < 9; ++k ) {
-					acc = CChanVec<4>::fma( *reinterpret_cast<const float4*>( e + ( ( k / 3 ) * PW + k % 3 ) * PitchE ), f[k], acc );
-				}
-				*reinterpret_cast<float4*>( result + storeAt[pass] + c0 )
-					= make_float4( activateExpanded<CLIPPED>( acc.x, dwAct ), activateExpanded<CLIPPED>( acc.y, dwAct ),
-						activateExpanded<CLIPPED>( acc.z, dwAct ), activateExpanded<CLIPPED>( acc.w, dwAct ) );
+			for( int k = 1; k < 9; ++k ) {
+				acc = CChanVec<4>::fma( *reinterpret_cast<const float4*>( e + ( ( k / 3 ) * PW + k % 3 ) * PitchE ), f[k], acc );
 			}
+			__builtin_amdgcn_raw_buffer_store_b128( u32x4{
+				__float_as_uint( activateExpanded<CLIPPED>( acc.x, dwAct ) ), __float_as_uint( activateExpanded<CLIPPED>( acc.y, dwAct ) ),
+				__float_as_uint( activateExpanded<CLIPPED>( acc.z, dwAct ) ), __float_as_uint( activateExpanded<CLIPPED>( acc.w, dwAct ) ) },
+				outBuffer, quadOk ? storeAt[pass] : OutOfRange, c0 * 4, 0 );
 		}
 		__builtin_amdgcn_fence( __ATOMIC_RELEASE, "wavefront" );
 		__builtin_amdgcn_wave_barrier();
@@ -2675,7 +2690,8 @@ static bool tryExpandDepthwise( nhStream s, const nhSeparableBlockDesc* d, const
 	const float* expandFilter, const float* expandBias, const float* dwFilter, const float* dwBias, float* reduced )
 {
 	const long long expandedBytes = static_cast<long long>( d->batch ) * d->height * d->width * d->expandedChannels * 4;
-	if( expandedBytes < ( 64LL << 20 ) || d->expandedChannels % 4 != 0 || !isAligned16( input ) || !isAligned16( expandFilter )
+	const long long resultBytes = static_cast<long long>( d->batch ) * dw.resultHeight * dw.resultWidth * d->expandedChannels * 4;
+	if( expandedBytes < ( 64LL << 20 ) || resultBytes >= 0x7fffff00LL || d->expandedChannels % 4 != 0 || !isAligned16( input ) || !isAligned16( expandFilter )
 		|| !isAligned16( dwFilter ) || ( dwBias != nullptr && !isAligned16( dwBias ) ) || !isAligned16( reduced )
 		|| ( d->inputChannels != 16 && d->inputChannels != 24 && d->inputChannels != 32 )
 		|| static_cast<long long>( d->height ) * d->width * d->inputChannels * 4 >= 0x7fffffffLL )
@@ -2695,7 +2711,7 @@ static bool tryExpandDepthwise( nhStream s, const nhSeparableBlockDesc* d, const
 		&& d->channelwiseParam > 0.f;
 #define NH_EXPAND_DW( STRIDE, KIN, CLIPPED ) hipLaunchKernelGGL( ( expandDepthwiseKernel<STRIDE, KIN, CLIPPED> ), dim3( groups ), \
 		dim3( 256 ), 0, toStream( s ), *d, dw.resultHeight, dw.resultWidth, input, expandFilter, expandBias, dwFilter, dwBias, reduced, \
-		tilesX, tilesY, static_cast<int>( tiles ), expandAct, dwAct )
+		tilesX, tilesY, static_cast<int>( tiles ), expandAct, dwAct, static_cast<unsigned>( resultBytes ) )
 #define NH_EXPAND_DW_K( STRIDE, CLIPPED ) if( d->inputChannels == 16 ) { NH_EXPAND_DW( STRIDE, 16, CLIPPED ); } \
 	else if( d->inputChannels == 24 ) { NH_EXPAND_DW( STRIDE, 24, CLIPPED ); } else { NH_EXPAND_DW( STRIDE, 32, CLIPPED ); }
 	if( d->stride == 1 ) {
