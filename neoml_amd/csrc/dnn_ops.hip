@@ -2519,8 +2519,9 @@ __device__ __forceinline__ float activateExpanded( float v, const CFusedActivati
 	return applyActivation( v, a );
 }
 
+// ( four workgroups per compute unit where the registers allow it without spills: 16 input channels )
 template<int STRIDE, int KIN, bool CLIPPED>
-__global__ __launch_bounds__( 256, 2 )
+__global__ __launch_bounds__( 256, KIN <= 16 ? 4 : 2 )
 void expandDepthwiseKernel( const nhSeparableBlockDesc d, int outH, int outW, const float* input, const float* expandFilter,
 	const float* expandBias, const float* dwFilter, const float* dwBias, float* result, int tilesX, int tilesY, int totalTiles,
 	const CFusedActivation expandAct, const CFusedActivation dwAct, unsigned resultBytes )
