@@ -1556,11 +1556,13 @@ static int launchTile( hipStream_t stream, CMatMulArgs& args, int batch, bool ve
 // accumulators per wavefront, is 0-25 % slower on the shapes of the benchmarks and 2 % faster only on 256 -> 256 channels
 // over 65 536 pixels),
 // and latency hiding across workgroups matters more at fp32 MFMA rates than the smaller tile's extra L2 traffic.
-// Narrow outputs (N <= 32) use 128x32 so that no MFMA block multiplies padding.
+// Narrow outputs (N <= 32, and 96 or 160 columns) use 128x32 so that no MFMA block multiplies padding.
 template<int AMODE, int BMODE>
 static int launchMatMul( hipStream_t stream, CMatMulArgs& args, int batch, bool vec, const CSliceMeeting* fixedMeeting = nullptr )
 {
-	if( args.N > 32 ) {
+	// ( 96 or 160 columns: three or five tiles of 32 columns instead of two or three of 64 the last of which is half padding;
+	// 25088 x 96 x 384 30.4 -> 26.0 us, 6272 x 160 x 576 21.8 -> 17.3, 6272 x 160 x 960 28.5 -> 24.2 )
+	if( args.N > 32 && !( args.N <= 160 && args.N % 64 == 32 ) ) {
 		return launchTile<64, 64, 2, 2, AMODE, BMODE>( stream, args, batch, vec, fixedMeeting );
 	}
 	return launchTile<128, 32, 4, 1, AMODE, BMODE>( stream, args, batch, vec, fixedMeeting );
