@@ -176,22 +176,28 @@ def other_workload(args):
     tags = set(t for _, _, t, _, _ in plan.launches if t)
     steps = args.steps
     pools = plan.make_events(tags, steps)
+    # what the engine adapter asks for its own stream: runs of small element-wise calls (the per-row scalars of the
+    # normalisation layers) go out several per launch; every launch and wait below goes through the library
+    deferring = args.workload == "transformer" and not args.no_defer
+    be.defer_small_ops(deferring)
     for _ in range(args.warmup):
         plan.run()
-    torch.cuda.synchronize()
+    be.synchronize()
     t_settle = time.perf_counter()
     while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
         plan.run()
-        torch.cuda.synchronize()
+        be.synchronize()
     # untimed-event pass for the throughput figure, then an event pass for the per-family split
     t0 = time.perf_counter()
     for _ in range(steps):
         plan.run()
-    torch.cuda.synchronize()
+    be.synchronize()
     elapsed = time.perf_counter() - t0
+    by_runs = deferring or args.time_by_runs
     for step in range(steps):
-        plan.run_with_events(pools[step])
-    torch.cuda.synchronize()
+        plan.run_with_events(pools[step], by_runs=by_runs)
+    be.synchronize()
+    be.defer_small_ops(False)
     fam = plan.family_totals()
     split = {}
     for tag, (cnt, tms, fl, by) in sorted(fam.items(), key=lambda kv: -kv[1][1]):
@@ -207,7 +213,8 @@ def other_workload(args):
         "metric": "%s (not the headline metric)" % unit, "value": round(items * steps / elapsed, 1), "unit": unit, "n_gpus": 1,
         "steps": steps, "warmup": args.warmup, "ms_per_step": round(elapsed / steps * 1e3, 3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": name + ", fp32, engine calls through the C ABI", "launches_per_step": len(plan.launches)},
+        "config": {"workload": name + ", fp32, engine calls through the C ABI", "launches_per_step": len(plan.launches),
+                   "small_ops_deferred": deferring, "families_timed": "per run of launches" if by_runs else "per launch"},
         "families": split, **extra}))
 
 
@@ -228,6 +235,10 @@ def main():
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--image", type=int, default=224)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--time-by-runs", action="store_true",
+                    help="other workloads: the per-family split from one pair of events per run of consecutive launches of a family")
+    ap.add_argument("--no-defer", action="store_true",
+                    help="transformer workload: every small element-wise call as a launch of its own (nhStreamDeferSmallOps off)")
     ap.add_argument("--cpu-replicas", type=int, default=min(16, os.cpu_count() or 1),
                     help="engines of the multi-replica CPU baseline (one thread each; 16 = the host cores that go with one GPU)")
     ap.add_argument("--per-kernel", action="store_true", help="print a per-op-family timing table to stderr")

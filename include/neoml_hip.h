@@ -430,6 +430,19 @@ NH_API int nhBlobMeanPoolingBackward(nhStream s, const nhPoolingDesc* desc_host,
  * caller's stream waits for it right there, so work enqueued later is ordered behind both. Only for streams whose work
  * all goes through this library (an engine's own stream). Results are those of the calls in order. */
 NH_API int nhStreamOverlapLstm(nhStream s, int enable);
+
+/* Several small element-wise calls in one launch. No counterpart in the reference: there every call runs at once on the
+ * calling thread. On a stream that has asked for it (enable != 0) a float element-wise call over at most 16384 elements
+ * (copy, add, sub, multiply, divide, negate, abs, max, min, sqrt, inv, and the forms with a device scalar: add value,
+ * multiply, neg-multiply, multiply-and-add, multiply-and-sub, eltwise multiply-add, eltwise neg-multiply) is put aside;
+ * up to eight of them are launched together, in call order and with bit-identical results, as soon as ANY other call
+ * on the stream through this library arrives: a larger or different operation, a copy, an event, nhStreamSynchronize,
+ * nhStreamDestroy, enable = 0, or a release of device memory (nhRawFree, a pool's clean-up). Until then their results are
+ * not in memory and their operands must stay valid, so this is only for streams whose work, synchronisation included,
+ * all goes through this library (an engine's own stream): synchronise with nhStreamSynchronize, not with HIP calls of
+ * your own. Nothing is put aside while the stream is being captured into a graph. What it saves: a row-normalising
+ * layer (CObjectNormalizationLayer) asks for five such calls per run, each a launch of about 4 us. */
+NH_API int nhStreamDeferSmallOps(nhStream s, int enable);
 /* LSTM (NME.h:1005-1011). Weights: inputWeights [4H x objectSize], recurrentWeights [4H x H]; gate order in
  * the 4H vector: main(tanh) | forget | input | output (src/CPU/CpuMathEngineDnnLstm.h:49-90).
  * Free terms, inputStateBackLink, inputMainBackLink and outputStateBackLink may be null.

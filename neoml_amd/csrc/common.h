@@ -21,9 +21,21 @@ extern int overlapLstmStreams;
 extern int lstmPartnersAwaited;
 void noteStreamUse( hipStream_t stream );
 
+// Small element-wise calls that a stream has put aside ( nhStreamDeferSmallOps, vector_ops.hip ) run before anything else
+// that is asked of the stream, so they too are caught here: tinyChainsPending counts the streams that hold some.
+// flushTinyOps launches what the stream of the current device holds; flushAllTinyOps does so for every stream of every
+// device ( before device memory is given back ). releaseTinyQueue: the stream is being destroyed.
+extern int tinyChainsPending;
+bool flushTinyOps( hipStream_t stream ); // true: something was launched
+void flushAllTinyOps();
+void releaseTinyQueue( hipStream_t stream );
+
 inline hipStream_t toStream( nhStream s )
 {
 	const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
+	if( __atomic_load_n( &tinyChainsPending, __ATOMIC_RELAXED ) != 0 ) {
+		flushTinyOps( stream );
+	}
 	if( __atomic_load_n( &lstmPartnersAwaited, __ATOMIC_RELAXED ) != 0 ) {
 		noteStreamUse( stream );
 	}

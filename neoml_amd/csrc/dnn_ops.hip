@@ -3138,8 +3138,12 @@ int nhLstm( nhStream s, int hiddenSize, int objectSize, const float* inputWeight
 	const int H = hiddenSize;
 	const int B = sequenceCount;
 	const int T = sequenceLength;
-	// ( not through toStream: whether something was enqueued since the last nhLstm is what is asked here )
+	// ( not through toStream: whether something was enqueued since the last nhLstm is what is asked here; small calls that
+	// the stream has put aside are launched now and count as enqueued )
 	const hipStream_t mainStream = reinterpret_cast<hipStream_t>( s );
+	if( __atomic_load_n( &tinyChainsPending, __ATOMIC_RELAXED ) != 0 && flushTinyOps( mainStream ) ) {
+		noteStreamUse( mainStream );
+	}
 	hipStream_t stream = mainStream;
 	const bool sequencePath = T > 1 && lstmSequenceFits( H, B, recurrentWeights, inputStateBackLink, inputMainBackLink, outputMainBackLink )
 		&& lstmSequenceAllowed( mainStream );

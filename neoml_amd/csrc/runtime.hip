@@ -93,6 +93,7 @@ int nhStreamDestroy( nhStream stream )
 		NH_HIP( hipStreamSynchronize( toStream( stream ) ) );
 		releaseSliceScratch( toStream( stream ), true );
 		releaseSequenceStream( toStream( stream ) );
+		releaseTinyQueue( toStream( stream ) );
 		NH_HIP( hipStreamDestroy( toStream( stream ) ) );
 	}
 	return NH_OK;
@@ -121,6 +122,7 @@ int nhRawAlloc( void** ptr, size_t size )
 int nhRawFree( void* ptr )
 {
 	if( ptr != nullptr ) {
+		flushAllTinyOps(); // a call that has been put aside may still name this block
 		NH_HIP( hipFree( ptr ) );
 	}
 	return NH_OK;

@@ -8,6 +8,10 @@
 // same thread, so no __restrict__ is put on the pointers.
 #include "common.h"
 #include <float.h>
+#include <map>
+#include <mutex>
+#include <type_traits>
+#include <utility>
 
 namespace nh {
 
@@ -102,6 +106,11 @@ void eltwiseKernel( const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, 
 	}
 }
 
+// A stream may put small calls aside and run several of them with one launch ( "tiny chains", below the functors ).
+// true: the call has been taken over, nothing is left to launch.
+template<int NIN, typename TIn, typename TOut, typename F>
+static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, const F& f );
+
 template<int NIN, typename TIn, typename TOut, typename F>
 static int launchEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, F f )
 {
@@ -115,6 +124,9 @@ static int launchEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 	if( out == nullptr || ( NIN >= 1 && a == nullptr ) || ( NIN >= 2 && b == nullptr ) || ( NIN >= 3 && c == nullptr ) ) {
 		setLastError( "null vector pointer" );
 		return NH_ERR_ARGUMENT;
+	}
+	if( deferEltwise<NIN, TIn, TOut, F>( s, a, b, c, out, n, f ) ) {
+		return NH_OK;
 	}
 	const bool vec = isAligned16( out ) && ( NIN < 1 || isAligned16( a ) ) && ( NIN < 2 || isAligned16( b ) )
 		&& ( NIN < 3 || isAligned16( c ) ) && n >= 4;
@@ -426,6 +438,323 @@ struct CTanhDiffOp : CNoScalar {
 };
 struct CTanhDiffOutOp : CNoScalar { __device__ float operator()( float y, float b, float ) const { return ( 1.f - y * y ) * b; } };
 
+// ---- tiny chains -----------------------------------------------------------------------------------------------------
+// A layer that normalises every row of a matrix ( CObjectNormalizationLayer::runOnceImpl,
+// NeoML/src/Dnn/Layers/ObjectNormalizationLayer.cpp:181-242 ) asks for runs of element-wise calls over one value per row:
+// a few thousand floats each, a launch of some 4 us that moves a few tens of KB. On a stream that has asked for it
+// ( nhStreamDeferSmallOps ) such calls are put aside, up to TinyChainMax of them, and run by ONE launch as soon as
+// anything else is asked of the stream ( toStream ), in the order of the calls and with the very functors of the
+// separate launches, so every value is the same bit for bit.
+//
+// Inside that launch thread t of the grid handles elements t, t + threads, ... of every call. A call whose operands are
+// either untouched by the calls in front of it in the chain, or begin exactly where an operand of one of them begins
+// ( then each element is read and written by the same thread, in program order ), needs nothing between it and the
+// call in front. Any other overlap ( a shifted view, a scalar that a call in front has produced ) needs every thread
+// to have finished the calls in front: the chain then runs in one workgroup with a barrier in front of such calls.
+
+constexpr int TinyChainMax = 8;
+constexpr int TinyOpMaxCount = 16384;
+constexpr int TinyThreads = 1024;
+constexpr int TinyMaxBlocks = 8;
+constexpr int TinyFunctorBytes = 16;
+
+struct CTinyOp {
+	const float* In[3];
+	float* Out;
+	const float* Scalar; // the device scalar that the functor reads when it starts ( host-side bookkeeping )
+	int Count;
+	short Kind; // index into CTinyKinds
+	short Barrier; // every thread must have finished the calls in front
+	alignas( 8 ) unsigned char Functor[TinyFunctorBytes];
+};
+
+struct CTinyChain {
+	int Length;
+	int Blocks;
+	CTinyOp Ops[TinyChainMax];
+};
+
+template<typename... T> struct CTypeList {};
+// the functors a chain may hold ( float in, float out, no more than TinyFunctorBytes of state )
+typedef CTypeList<CCopyOp<float>, CAddOp<float>, CSubOp<float>, CMulOp<float>, CDivOp, CNegOp, CAbsOp, CMaxOp, CMinOp, CSqrtOp, CInvOp,
+	CAddValueOp<float>, CMulValueOp<float>, CNegMulValueOp, CMultiplyAndAddOp, CMultiplyAndSubOp, CMulAddOp, CNegMulOp> CTinyKinds;
+
+template<typename F, typename List> struct CKindOf;
+template<typename F> struct CKindOf<F, CTypeList<>> { static constexpr int Value = -1; };
+template<typename F, typename Head, typename... Tail> struct CKindOf<F, CTypeList<Head, Tail...>> {
+	static constexpr int Rest = CKindOf<F, CTypeList<Tail...>>::Value;
+	static constexpr int Value = std::is_same<F, Head>::value ? 0 : ( Rest < 0 ? -1 : Rest + 1 );
+};
+
+template<typename F> __device__ __forceinline__ void runTinyOp( const CTinyOp& op, int first, int step )
+{
+	static_assert( sizeof( F ) <= TinyFunctorBytes && std::is_trivially_copyable<F>::value, "functor does not fit a chain" );
+	F f;
+	__builtin_memcpy( &f, op.Functor, sizeof( F ) );
+	f.prepare();
+	const float* a = op.In[0];
+	const float* b = op.In[1];
+	const float* c = op.In[2];
+	for( int i = first; i < op.Count; i += step ) {
+		const float x = a != nullptr ? a[i] : 0.f;
+		const float y = b != nullptr ? b[i] : 0.f;
+		const float z = c != nullptr ? c[i] : 0.f;
+		op.Out[i] = f( x, y, z );
+	}
+}
+
+template<typename List> struct CTinyDispatch;
+template<> struct CTinyDispatch<CTypeList<>> {
+	static __device__ __forceinline__ void Run( int, const CTinyOp&, int, int ) {}
+};
+template<typename Head, typename... Tail> struct CTinyDispatch<CTypeList<Head, Tail...>> {
+	static __device__ __forceinline__ void Run( int kind, const CTinyOp& op, int first, int step )
+	{
+		if( kind == 0 ) {
+			runTinyOp<Head>( op, first, step );
+		} else {
+			CTinyDispatch<CTypeList<Tail...>>::Run( kind - 1, op, first, step );
+		}
+	}
+};
+
+__global__ __launch_bounds__( TinyThreads ) void tinyChainKernel( const CTinyChain chain )
+{
+	const int first = blockIdx.x * TinyThreads + threadIdx.x;
+	const int step = gridDim.x * TinyThreads;
+	for( int k = 0; k < chain.Length; ++k ) {
+		const CTinyOp& op = chain.Ops[k];
+		if( op.Barrier != 0 ) {
+			// only in chains of one workgroup; the stores in front are visible to the whole workgroup behind it
+			__syncthreads();
+		}
+		CTinyDispatch<CTinyKinds>::Run( op.Kind, op, first, step );
+	}
+}
+
+struct CTinyQueue {
+	bool Enabled = false;
+	CTinyChain Chain = {};
+};
+
+typedef std::map<std::pair<int, hipStream_t>, CTinyQueue> CTinyQueues;
+static std::mutex tinyLock;
+static CTinyQueues& tinyQueues()
+{
+	static CTinyQueues* queues = new CTinyQueues; // never destroyed: calls may still arrive while the process unloads
+	return *queues;
+}
+int tinyChainsPending = 0;
+static int tinyDeferringStreams = 0;
+
+// With tinyLock held and the queue's device current. true: something was launched ( telling a stream's one-launch LSTMs
+// about it, noteStreamUse, is left to the callers: that takes a lock that a caller of toStream may hold ).
+static bool launchTinyChain( hipStream_t stream, CTinyChain& chain )
+{
+	if( chain.Length == 0 ) {
+		return false;
+	}
+	chain.Blocks = 1;
+	bool barrier = false;
+	int longest = 0;
+	for( int k = 0; k < chain.Length; ++k ) {
+		barrier = barrier || chain.Ops[k].Barrier != 0;
+		longest = chain.Ops[k].Count > longest ? chain.Ops[k].Count : longest;
+	}
+	if( !barrier ) {
+		const int blocks = ceilDiv( longest, TinyThreads );
+		chain.Blocks = blocks < TinyMaxBlocks ? blocks : TinyMaxBlocks;
+	}
+	hipLaunchKernelGGL( tinyChainKernel, dim3( chain.Blocks ), dim3( TinyThreads ), 0, stream, chain );
+	chain.Length = 0;
+	__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+	return true;
+}
+
+bool flushTinyOps( hipStream_t stream )
+{
+	int device = 0;
+	if( hipGetDevice( &device ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return false;
+	}
+	std::lock_guard<std::mutex> guard( tinyLock );
+	auto found = tinyQueues().find( std::make_pair( device, stream ) );
+	return found != tinyQueues().end() && launchTinyChain( stream, found->second.Chain );
+}
+
+void flushAllTinyOps()
+{
+	if( __atomic_load_n( &tinyChainsPending, __ATOMIC_RELAXED ) == 0 ) {
+		return;
+	}
+	int current = 0;
+	if( hipGetDevice( &current ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return;
+	}
+	int active = current;
+	std::pair<int, hipStream_t> launched[16];
+	int launchedCount = 0;
+	{
+		std::lock_guard<std::mutex> guard( tinyLock );
+		for( auto& entry : tinyQueues() ) {
+			if( entry.second.Chain.Length == 0 ) {
+				continue;
+			}
+			if( entry.first.first != active ) {
+				if( hipSetDevice( entry.first.first ) != hipSuccess ) {
+					( void )hipGetLastError();
+					continue;
+				}
+				active = entry.first.first;
+			}
+			if( launchTinyChain( entry.first.second, entry.second.Chain ) && launchedCount < 16 ) {
+				launched[launchedCount++] = entry.first;
+			}
+		}
+	}
+	if( __atomic_load_n( &lstmPartnersAwaited, __ATOMIC_RELAXED ) != 0 ) {
+		for( int i = 0; i < launchedCount; ++i ) {
+			if( launched[i].first != active ) {
+				if( hipSetDevice( launched[i].first ) != hipSuccess ) {
+					( void )hipGetLastError();
+					continue;
+				}
+				active = launched[i].first;
+			}
+			noteStreamUse( launched[i].second );
+		}
+	}
+	if( active != current ) {
+		( void )hipSetDevice( current );
+	}
+}
+
+// the stream is going away ( drained by the caller ): a later stream may be handed the same handle
+void releaseTinyQueue( hipStream_t stream )
+{
+	int device = 0;
+	if( hipGetDevice( &device ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return;
+	}
+	std::lock_guard<std::mutex> guard( tinyLock );
+	auto found = tinyQueues().find( std::make_pair( device, stream ) );
+	if( found != tinyQueues().end() ) {
+		launchTinyChain( stream, found->second.Chain );
+		if( found->second.Enabled ) {
+			__atomic_fetch_sub( &tinyDeferringStreams, 1, __ATOMIC_RELAXED );
+		}
+		tinyQueues().erase( found );
+	}
+}
+
+struct CFloatRange {
+	const float* Lo = nullptr;
+	const float* Hi = nullptr;
+};
+// the ranges share elements without beginning at the same one
+static bool rangesClash( const CFloatRange& x, const CFloatRange& y )
+{
+	return x.Lo != nullptr && y.Lo != nullptr && x.Lo != y.Lo && x.Lo < y.Hi && y.Lo < x.Hi;
+}
+static bool rangesTouch( const CFloatRange& x, const CFloatRange& y )
+{
+	return x.Lo != nullptr && y.Lo != nullptr && x.Lo < y.Hi && y.Lo < x.Hi;
+}
+
+// the device scalar a functor reads when the kernel starts, if it has one
+template<typename F> static auto scalarOf( const F& f, int ) -> decltype( static_cast<const float*>( f.Ptr ) ) { return f.Ptr; }
+template<typename F> static const float* scalarOf( const F&, long ) { return nullptr; }
+
+template<int NIN, typename TIn, typename TOut, typename F>
+static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, const F& f )
+{
+	if constexpr( std::is_same<TIn, float>::value && std::is_same<TOut, float>::value && CKindOf<F, CTinyKinds>::Value >= 0 ) {
+		if( n > TinyOpMaxCount || __atomic_load_n( &tinyDeferringStreams, __ATOMIC_RELAXED ) == 0 ) {
+			return false;
+		}
+		const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
+		int device = 0;
+		hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+		if( hipGetDevice( &device ) != hipSuccess || hipStreamIsCapturing( stream, &capture ) != hipSuccess ) {
+			( void )hipGetLastError();
+			return false;
+		}
+		if( capture != hipStreamCaptureStatusNone ) {
+			return false; // the recording ends outside this library: nothing may be left behind
+		}
+		std::lock_guard<std::mutex> guard( tinyLock );
+		auto found = tinyQueues().find( std::make_pair( device, stream ) );
+		if( found == tinyQueues().end() || !found->second.Enabled ) {
+			return false;
+		}
+		CTinyChain& chain = found->second.Chain;
+		if( chain.Length == TinyChainMax ) {
+			launchTinyChain( stream, chain );
+		}
+		CTinyOp& op = chain.Ops[chain.Length];
+		op = CTinyOp();
+		op.In[0] = NIN >= 1 ? a : nullptr;
+		op.In[1] = NIN >= 2 ? b : nullptr;
+		op.In[2] = NIN >= 3 ? c : nullptr;
+		op.Out = out;
+		op.Count = n;
+		op.Kind = static_cast<short>( CKindOf<F, CTinyKinds>::Value );
+		__builtin_memcpy( op.Functor, &f, sizeof( F ) );
+		// what the calls in front have to do with this one
+		CFloatRange reads[4], writes;
+		for( int i = 0; i < 3; ++i ) {
+			if( op.In[i] != nullptr ) {
+				reads[i].Lo = op.In[i];
+				reads[i].Hi = op.In[i] + n;
+			}
+		}
+		const float* scalar = scalarOf( f, 0 );
+		op.Scalar = scalar;
+		if( scalar != nullptr ) {
+			reads[3].Lo = scalar;
+			reads[3].Hi = scalar + 1;
+		}
+		writes.Lo = out;
+		writes.Hi = out + n;
+		bool barrier = false;
+		for( int k = 0; k < chain.Length && !barrier; ++k ) {
+			const CTinyOp& front = chain.Ops[k];
+			CFloatRange frontWrites;
+			frontWrites.Lo = front.Out;
+			frontWrites.Hi = front.Out + front.Count;
+			// ( the scalar: read by every thread, so a match of the first element is no excuse )
+			barrier = rangesClash( reads[0], frontWrites ) || rangesClash( reads[1], frontWrites ) || rangesClash( reads[2], frontWrites )
+				|| rangesTouch( reads[3], frontWrites ) || rangesClash( writes, frontWrites );
+			for( int i = 0; i < 3 && !barrier; ++i ) {
+				if( front.In[i] != nullptr ) {
+					CFloatRange frontReads;
+					frontReads.Lo = front.In[i];
+					frontReads.Hi = front.In[i] + front.Count;
+					barrier = rangesClash( writes, frontReads );
+				}
+			}
+			if( !barrier && front.Scalar != nullptr ) {
+				CFloatRange frontReads;
+				frontReads.Lo = front.Scalar;
+				frontReads.Hi = front.Scalar + 1;
+				barrier = rangesTouch( writes, frontReads );
+			}
+		}
+		op.Barrier = barrier ? 1 : 0;
+		if( chain.Length == 0 ) {
+			__atomic_fetch_add( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+		}
+		++chain.Length;
+		return true;
+	} else {
+		( void )s; ( void )a; ( void )b; ( void )c; ( void )out; ( void )n; ( void )f;
+		return false;
+	}
+}
+
 // ---- reductions to one value: one workgroup per 16K elements ------------------------------------------------------
 // The workgroups meet in the stream's scratch: each leaves its partial sum there and draws a ticket; the one that draws
 // the last ticket adds the partial sums up in a fixed order and only then touches the result ( stores, or adds onto it ).
@@ -580,6 +909,26 @@ static int launchSum( nhStream s, const float* first, const float* second, int v
 } // namespace nh
 
 using namespace nh;
+
+extern "C" int nhStreamDeferSmallOps( nhStream s, int enable )
+{
+	const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
+	int device = 0;
+	NH_HIP( hipGetDevice( &device ) );
+	std::lock_guard<std::mutex> guard( tinyLock );
+	CTinyQueue& queue = tinyQueues()[std::make_pair( device, stream )];
+	if( ( enable != 0 ) != queue.Enabled ) {
+		queue.Enabled = enable != 0;
+		if( queue.Enabled ) {
+			__atomic_fetch_add( &tinyDeferringStreams, 1, __ATOMIC_RELAXED );
+		} else {
+			__atomic_fetch_sub( &tinyDeferringStreams, 1, __ATOMIC_RELAXED );
+			launchTinyChain( stream, queue.Chain );
+			NH_LAUNCH_CHECK();
+		}
+	}
+	return NH_OK;
+}
 
 #define NH_UNARY( name, Op ) \
 	extern "C" int name( nhStream s, const float* first, float* result, int vectorSize ) \

@@ -104,6 +104,9 @@ CHipMathEngine::CHipMathEngine( int deviceIndex, size_t memoryLimit, int /*flags
 	NH_CALL( nhStreamBindPool( stream, pool ) );
 	// all of this engine's work is enqueued through the library: independent one-launch LSTMs may run side by side
 	NH_CALL( nhStreamOverlapLstm( stream, 1 ) );
+	// ... and runs of small element-wise calls ( the per-row scalars of CObjectNormalizationLayer ) may share a launch:
+	// every wait of this engine is nhStreamSynchronize or a copy through the library, which launch them first
+	NH_CALL( nhStreamDeferSmallOps( stream, 1 ) );
 	initialized = true;
 }
 

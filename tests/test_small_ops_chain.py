@@ -1,0 +1,237 @@
+"""nhStreamDeferSmallOps: small element-wise calls that a stream puts aside and launches together must leave the very
+bits that the separate launches leave, whatever the calls have to do with one another (in place, shifted views of
+one buffer, a device scalar that a call in front has produced), and nothing may overtake or be overtaken by them."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from test_oracle import rng
+
+pytestmark = pytest.mark.gpu
+
+ARENA = 1 << 16
+
+
+class Streams:
+    """Two streams of the library: one that launches every call by itself, one that puts small calls aside."""
+
+    def __init__(self):
+        import torch
+        import neoml_amd
+        self.torch, self.na, self.lib = torch, neoml_amd, neoml_amd.load()
+        self.dev = torch.device("cuda:0")
+        self.plain, self.deferring = ctypes.c_void_p(), ctypes.c_void_p()
+        neoml_amd.check(self.lib.nhStreamCreate(ctypes.byref(self.plain)))
+        neoml_amd.check(self.lib.nhStreamCreate(ctypes.byref(self.deferring)))
+        neoml_amd.check(self.lib.nhStreamDeferSmallOps(self.deferring, 1))
+
+    def close(self):
+        self.na.check(self.lib.nhStreamDestroy(self.plain))
+        self.na.check(self.lib.nhStreamDestroy(self.deferring))
+
+    def run(self, stream, program, start):
+        """program: [(entry point, [arguments; ("at", offset) stands for a pointer into the arena])]. Returns the arena
+        afterwards, fetched through the library (a copy to the host is one of the calls that launch what was put aside)."""
+        arena = self.torch.from_numpy(start).to(self.dev)
+        self.torch.cuda.synchronize()
+        base = arena.data_ptr()
+        for name, args in program:
+            real = [ctypes.c_void_p(base + 4 * a[1]) if isinstance(a, tuple) else a for a in args]
+            self.na.check(getattr(self.lib, name)(stream, *real))
+        out = np.empty_like(start)
+        self.na.check(self.lib.nhCopyDeviceToHost(stream, out.ctypes.data_as(ctypes.c_void_p), ctypes.c_void_p(base), out.nbytes))
+        return out
+
+
+@pytest.fixture(scope="module")
+def streams():
+    s = Streams()
+    yield s
+    s.close()
+
+
+def same_bits(a, b):
+    return np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def at(offset):
+    return ("at", int(offset))
+
+
+def test_row_normalisation_scalars_chain(streams):
+    """The small calls of CObjectNormalizationLayer::runOnceImpl (NeoML/src/Dnn/Layers/ObjectNormalizationLayer.cpp:
+    200-230) on one value per row, with the matrix-sized calls between them."""
+    g = rng(4001)
+    rows, width = 8192, 2
+    start = g.uniform(0.5, 2.0, ARENA).astype(np.float32)
+    x, sq, mean, inv_std, inv_w, eps = 0, rows * width, 2 * rows * width, 2 * rows * width + rows, ARENA - 8, ARENA - 4
+    start[inv_w], start[eps] = 1.0 / width, 1e-5
+    program = [
+        ("nhSumMatrixColumns", [at(mean), at(x), rows, width]),
+        ("nhVectorNegMultiply", [at(mean), at(mean), rows, at(inv_w)]),
+        ("nhAddVectorToMatrixColumns", [at(x), at(sq), rows, width, at(mean)]),
+        ("nhVectorEltwiseMultiply", [at(sq), at(sq), at(sq), rows * width]),
+        ("nhSumMatrixColumns", [at(inv_std), at(sq), rows, width]),
+        ("nhVectorMultiply", [at(inv_std), at(inv_std), rows, at(inv_w)]),
+        ("nhVectorAddValue", [at(inv_std), at(inv_std), rows, at(eps)]),
+        ("nhVectorSqrt", [at(inv_std), at(inv_std), rows]),
+        ("nhVectorInv", [at(inv_std), at(inv_std), rows]),
+        ("nhAddVectorToMatrixColumns", [at(x), at(sq), rows, width, at(mean)]),
+        ("nhMultiplyDiagMatrixByMatrix", [at(inv_std), rows, at(sq), width, at(sq), rows * width]),
+    ]
+    want = streams.run(streams.plain, program, start)
+    got = streams.run(streams.deferring, program, start)
+    assert same_bits(got, want)
+    # and the numbers are those of the formula
+    m = start[x:x + rows * width].reshape(rows, width).astype(np.float64)
+    ref = (m - m.mean(1, keepdims=True)) / np.sqrt(m.var(1, keepdims=True) + 1e-5)
+    # ( two values per row: where they nearly agree the variance is a difference of close numbers, hence the loose bar;
+    # the bar of this test is the line above )
+    assert np.allclose(got[sq:sq + rows * width].reshape(rows, width), ref, rtol=1e-3, atol=5e-3)
+
+
+UNARY = ("nhVectorSqrt", "nhVectorInv", "nhVectorNeg", "nhVectorAbs")
+BINARY = ("nhVectorAdd", "nhVectorSub", "nhVectorEltwiseMultiply", "nhVectorEltwiseDivide", "nhVectorEltwiseMax", "nhVectorEltwiseMin",
+          "nhVectorEltwiseMultiplyAdd", "nhVectorEltwiseNegMultiply")
+WITH_SCALAR = ("nhVectorAddValue", "nhVectorMultiply", "nhVectorNegMultiply")
+BINARY_WITH_SCALAR = ("nhVectorMultiplyAndAdd", "nhVectorMultiplyAndSub")
+# not of the kind that is put aside: launched at once, after what was put aside
+OTHER = ("nhVectorSigmoid", "nhVectorTanh")
+
+
+def random_program(g, length):
+    """Operands begin at a few fixed places of the arena, so that exact matches, shifted overlaps and disjoint operands
+    all come up; a result either begins where one of the call's own operands begins or keeps clear of them (what the
+    entry points ask for); scalars sit in the arena too, sometimes where a call in front writes."""
+    places = [0, 0, 0, 1, 3, 4, 64, 4096, 8192, 8195, 12288, 20000, 20000, 36000]
+    sizes = [1, 5, 64, 777, 1024, 4096, 8192, 8192, 16384, 16384, 20000]
+    program = []
+    while len(program) < length:
+        n = int(g.choice(sizes))
+        kind = g.integers(0, 10)
+        if kind < 3:
+            name, n_in, scalar = str(g.choice(UNARY)), 1, False
+        elif kind < 6:
+            name, n_in, scalar = str(g.choice(BINARY)), 2, False
+        elif kind < 8:
+            name, n_in, scalar = str(g.choice(WITH_SCALAR)), 1, True
+        elif kind < 9:
+            name, n_in, scalar = str(g.choice(BINARY_WITH_SCALAR)), 2, True
+        else:
+            name, n_in, scalar = str(g.choice(OTHER)), 1, False
+        ins = [int(g.choice(places)) for _ in range(n_in)]
+        if name == "nhVectorEltwiseMultiplyAdd":
+            # result += first * second: the result is the third operand
+            out = int(g.choice(places))
+            if any(i != out and i < out + n and out < i + n for i in ins):
+                continue
+        elif g.integers(0, 2) == 0:
+            out = ins[int(g.integers(0, n_in))]
+            if any(i != out and i < out + n and out < i + n for i in ins):
+                continue
+        else:
+            out = int(g.choice(places))
+            if any(i != out and i < out + n and out < i + n for i in ins):
+                continue
+        args = [at(i) for i in ins]
+        if scalar:
+            where = int(g.choice([ARENA - 4, ARENA - 3, 2, 4100, 8192]))
+            if out <= where < out + n:
+                continue  # a call may not overwrite its own scalar
+            args += [at(out), n, at(where)]
+        else:
+            args += [at(out), n]
+        program.append((name, args))
+    return program
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_chains_leave_the_same_bits(streams, seed):
+    g = rng(4100 + seed)
+    start = g.uniform(0.25, 4.0, ARENA).astype(np.float32) * g.choice([-1.0, 1.0], ARENA).astype(np.float32)
+    start[ARENA - 4:] = (1.5, -0.75, 0.0, 0.0)
+    program = random_program(g, 40)
+    want = streams.run(streams.plain, program, start)
+    got = streams.run(streams.deferring, program, start)
+    assert same_bits(got, want), [p[0] for p in program]
+
+
+def test_every_way_out_of_the_queue(streams):
+    """What was put aside is launched by: a ninth small call, an event, a synchronisation, switching the mode off, and
+    the release of device memory."""
+    import torch
+    lib, na = streams.lib, streams.na
+    s = streams.deferring
+    x = torch.full((4096,), 2.0, device=streams.dev)
+    two = torch.full((1,), 2.0, device=streams.dev)
+    torch.cuda.synchronize()
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def double(times):
+        for _ in range(times):
+            na.check(lib.nhVectorMultiply(s, P(x), P(x), 4096, P(two)))
+
+    double(11)  # more than one chain holds
+    na.check(lib.nhStreamSynchronize(s))
+    assert float(x[0]) == 2.0 * 2 ** 11 and float(x[4095]) == 2.0 * 2 ** 11
+    double(2)
+    event = ctypes.c_void_p()
+    na.check(lib.nhEventCreate(ctypes.byref(event)))
+    na.check(lib.nhEventRecord(event, s))
+    na.check(lib.nhEventSynchronize(event))
+    assert float(x[7]) == 2.0 * 2 ** 13
+    na.check(lib.nhEventDestroy(event))
+    double(1)
+    na.check(lib.nhStreamDeferSmallOps(s, 0))
+    torch.cuda.synchronize()
+    assert float(x[9]) == 2.0 * 2 ** 14
+    na.check(lib.nhStreamDeferSmallOps(s, 1))
+    block = ctypes.c_void_p()
+    na.check(lib.nhRawAlloc(ctypes.byref(block), 4096 * 4))
+    na.check(lib.nhVectorCopy(s, block, P(x), 4096))
+    na.check(lib.nhVectorMultiply(s, block, P(x), 4096, P(two)))
+    na.check(lib.nhRawFree(block))  # the two calls above name the block: they run before it goes
+    na.check(lib.nhStreamSynchronize(s))
+    assert float(x[11]) == 2.0 * 2 ** 15
+
+
+def test_small_call_between_two_lstms_keeps_its_place(streams):
+    """On a stream that also lets independent one-launch LSTMs run side by side: a small call between two nhLstm calls
+    that produces the second one's input is launched before it, and the second does not run beside the first."""
+    import torch
+    from nhtest import Cpu, assert_close
+    orc = Cpu("orc")
+    lib, na = streams.lib, streams.na
+    s = streams.deferring
+    g = rng(4200)
+    T, B, In, H = 16, 16, 64, 256   # the second call's input: T * B * In = 16384 floats, a small call
+    w_in = g.uniform(-0.2, 0.2, (2, 4 * H, In)).astype(np.float32)
+    w_rec = g.uniform(-0.1, 0.1, (2, 4 * H, H)).astype(np.float32)
+    bias = g.uniform(-0.5, 0.5, (2, 4 * H)).astype(np.float32)
+    x = g.uniform(-1, 1, (T, B, In)).astype(np.float32)
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(streams.dev)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    d_w_in, d_w_rec, d_bias, d_x = up(w_in), up(w_rec), up(bias), up(x)
+    size = ctypes.c_size_t(0)
+    na.check(lib.nhLstmWorkspaceSize(H, In, T, B, ctypes.byref(size)))
+    work = [torch.empty((size.value + 15) // 4, dtype=torch.float32, device=streams.dev) for _ in range(2)]
+    out = [torch.zeros((T, B, H), device=streams.dev) for _ in range(2)]
+    x2 = torch.zeros((T, B, In), device=streams.dev)
+    half = up(np.array([0.5], np.float32))
+    torch.cuda.synchronize()
+    na.check(lib.nhStreamOverlapLstm(s, 1))
+    try:
+        for _ in range(2):
+            na.check(lib.nhLstm(s, H, In, P(d_w_in[0]), P(d_bias[0]), P(d_w_rec[0]), None, 0, T, B, None, None, P(d_x), None, P(out[0]),
+                                P(work[0]), size.value))
+            na.check(lib.nhVectorMultiply(s, P(d_x), P(x2), x.size, P(half)))
+            na.check(lib.nhLstm(s, H, In, P(d_w_in[1]), P(d_bias[1]), P(d_w_rec[1]), None, 1, T, B, None, None, P(x2), None, P(out[1]),
+                                P(work[1]), size.value))
+            assert lib.nhStreamSynchronize(s) == 0
+            assert_close(out[0].cpu().numpy(), orc.lstm(w_in[0], bias[0], w_rec[0], None, x, False)[0], "first")
+            assert_close(out[1].cpu().numpy(), orc.lstm(w_in[1], bias[1], w_rec[1], None, 0.5 * x, True)[0], "second, input from the small call")
+            x2.zero_()
+            torch.cuda.synchronize()
+    finally:
+        na.check(lib.nhStreamOverlapLstm(s, 0))

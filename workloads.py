@@ -55,10 +55,18 @@ class HipBackend:
         return self.torch.empty(shape, dtype=self.torch.float32, device=self.dev)
 
     def to_numpy(self, t):
+        self.synchronize()
         return t.cpu().numpy()
 
     def synchronize(self):
+        # through the library first: it launches what the stream may have put aside (nhStreamDeferSmallOps)
+        self.na.check(self.lib.nhStreamSynchronize(self.stream))
         self.torch.cuda.synchronize()
+
+    def defer_small_ops(self, enable):
+        """Small element-wise calls of this backend's stream are launched several at a time. Only while every launch and
+        every synchronisation goes through the library: switch it off before torch touches the tensors again."""
+        self.na.check(self.lib.nhStreamDeferSmallOps(self.stream, 1 if enable else 0))
 
     @staticmethod
     def _p(t):
@@ -393,8 +401,28 @@ class LaunchPlan:
             pools.append(step)
         return pools
 
-    def run_with_events(self, pool):
+    def run_with_events(self, pool, by_runs=False):
+        """by_runs: one pair of events around every run of consecutive launches of one family (the launches of one layer)
+        rather than around every launch. An event is itself a call on the stream, so with small calls being put aside
+        (HipBackend.defer_small_ops) only this way shows what the stream then does."""
         record, stream = self.be.lib.nhEventRecord, self.be.stream
+        if by_runs:
+            launches, i = self.launches, 0
+            while i < len(launches):
+                tag, j, flops, nbytes = launches[i][2], i, 0, 0
+                while j < len(launches) and launches[j][2] == tag:
+                    flops, nbytes, j = flops + launches[j][3], nbytes + launches[j][4], j + 1
+                if pool[i] is not None:
+                    record(pool[i][0], stream)
+                for fn, args, _, _, _ in launches[i:j]:
+                    rc = fn(*args)
+                    if rc != 0:
+                        self.be.na.check(rc)
+                if pool[i] is not None:
+                    record(pool[i][1], stream)
+                    self.timed.append((tag, flops, nbytes, pool[i][0], pool[i][1], j - i))
+                i = j
+            return
         for (fn, args, tag, flops, nbytes), ev in zip(self.launches, pool):
             if ev is None:
                 rc = fn(*args)
@@ -411,10 +439,10 @@ class LaunchPlan:
         lib = self.be.lib
         fam = {}
         ms = ctypes.c_float(0)
-        for tag, flops, nbytes, a, b in self.timed:
+        for tag, flops, nbytes, a, b, *count in self.timed:
             self.be.na.check(lib.nhEventElapsedMs(a, b, ctypes.byref(ms)))
             f = fam.setdefault(tag, [0, 0.0, 0, 0])
-            f[0] += 1
+            f[0] += count[0] if count else 1
             f[1] += ms.value
             f[2] += flops
             f[3] += nbytes
