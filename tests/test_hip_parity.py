@@ -997,9 +997,9 @@ def test_separable_blocks(case, with_expand):
 
 
 # Blocks whose expanded tensor would be far larger than the caches: expand and depthwise stage run as one launch that
-# keeps the expanded values of a tile of pixels in LDS (tiles of 14 x 14 / 7 x 7 output pixels, 32 expanded channels at a
-# time). Sizes that are and are not multiples of the tile, a last chunk of 16 and of 4 channels, both strides, with and
-# without free terms, a residual that reuses the input blob.
+# keeps the expanded values of a patch of pixels in LDS (32 expanded channels at a time). Sizes that are and are not
+# multiples of the patch, a last chunk of 16 and of 4 channels, both strides, 16 / 24 / 32 input channels, with and
+# without free terms, a residual, also one that reuses the input blob.
 LARGE_SEPARABLE_CASES = [
     (16, 112, 112, 16, 96, 24, 2, False, ("relu", 6.0), ("relu", 6.0)),
     (40, 56, 56, 24, 144, 24, 1, True, ("relu", 6.0), ("relu", 6.0)),
@@ -1007,6 +1007,9 @@ LARGE_SEPARABLE_CASES = [
     (128, 28, 28, 32, 192, 32, 1, True, ("relu", 6.0), ("relu", 6.0)),
     (24, 100, 90, 16, 100, 24, 1, False, ("hswish", 0.0), ("relu", 0.0)),
     (24, 101, 91, 16, 96, 24, 2, False, ("relu", 6.0), (None, 0.0)),
+    # 32 input channels, without and with a residual
+    (48, 60, 52, 32, 128, 16, 1, False, ("hswish", 0.0), ("relu", 0.0)),
+    (48, 60, 52, 32, 192, 32, 1, True, ("relu", 6.0), ("relu", 6.0)),
 ]
 
 
