@@ -332,7 +332,8 @@ NH_API int nhBlobConvolutionNoAlloc(nhStream s, const nhConvDesc* desc_host, con
 /* Gradients of the convolution (NME.h:757-761), same descriptor as the forward pass.
  * Backward: inputDiff = the gradient by the source; freeTerm (per source channel, may be null) is added, as the
  * reference does for the layers that run a convolution backwards as their forward pass. workspace: the filter with its
- * channel axes swapped, nhBlobConvolutionBackwardWorkspaceSize bytes.
+ * channel axes swapped (for the 7x7/2 stem over 3 channels: the filter in the kernel's order and the windows of the
+ * input gradient that its tiles leave to be summed), nhBlobConvolutionBackwardWorkspaceSize bytes.
  * LearnAdd: filterDiff += the gradient by the filter. The gradient by the free term is a column sum of outputDiff
  * (nhSumMatrixRowsAdd over [pixels x filterCount]). */
 NH_API int nhBlobConvolutionBackwardWorkspaceSize(const nhConvDesc* desc_host, size_t* bytes);
@@ -433,7 +434,7 @@ NH_API int nhStreamOverlapLstm(nhStream s, int enable);
 
 /* Several small element-wise calls in one launch. No counterpart in the reference: there every call runs at once on the
  * calling thread. On a stream that has asked for it (enable != 0) a float element-wise call over at most 16384 elements
- * (copy, add, sub, multiply, divide, negate, abs, max, min, sqrt, inv, and the forms with a device scalar: add value,
+ * (fill, copy, add, sub, multiply, divide, negate, abs, max, min, sqrt, inv, and the forms with a device scalar: add value,
  * multiply, neg-multiply, multiply-and-add, multiply-and-sub, eltwise multiply-add, eltwise neg-multiply) is put aside;
  * up to eight of them are launched together, in call order and with bit-identical results, as soon as ANY other call
  * on the stream through this library arrives: a larger or different operation, a copy, an event, nhStreamSynchronize,

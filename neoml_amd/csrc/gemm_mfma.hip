@@ -2908,6 +2908,317 @@ static bool convBackwardDataByClasses( hipStream_t stream, const nhConvDesc& d, 
 	return true;
 }
 
+// ---- input gradient of a 7 x 7 / 2 convolution from 3 to 64 channels ( the stem of the ImageNet networks ) -----------
+// As a product per input pixel the result has 3 columns, and a matrix tile spends nine tenths of its work on padding
+// ( 1.4 ms at 64 x 224 x 224 ). Turned round, every pixel of the output gradient is a row of 64 values times the
+// filter as a 64 x 147 matrix, and the 147 products are the pixel's contributions to the 7 x 7 x 3 window of the input
+// gradient it looks at: a product with hardly any padding, followed by sums over overlapping windows.
+//
+// A workgroup takes tiles of 16 x 16 output-gradient pixels, one after the other: 256 operand rows, two blocks of 32 per
+// wave, a lane holding its pixel's 64 values in registers for the whole tile. The filter's columns ( column n = input
+// channel x 49 + tap, 64 values each, transposed by a small launch in front ) are walked 32 at a time: per block of rows
+// 32 v_mfma_f32_32x32x2 ( number j takes output channel 32 half + j from both operands, so a lane's values are adjacent
+// in memory ), then every accumulator register is added to its place in the WAVE's own window in LDS; the place is the
+// sum of a term of the row ( 8 per lane ) and a term of the column ( one per chunk ). The adds are plain LDS reads and
+// writes ( LDS float atomics took six times as long ), which needs the places of one round to differ over the whole wave:
+// two rows and two columns meet in one place only when 2 x + kx = 2 x' + kx' and 2 y + ky = 2 y' + ky', i.e. for pixels
+// at most 3 apart in x and in y. So wave w takes the pixel rows y = w, w + 4, w + 8, w + 12, and accumulator register
+// 4 q + i of a lane is pixel x = 4 X + i: register i of all eight groups ( 2 blocks x 4 ) and both half-waves are
+// 16 pixels 4 apart in x or y, one round. Four rounds per chunk, each read - add - write; a wave's LDS operations complete
+// in order. A wave's window is four bands of 7 rows x 37 x 3 values.
+//
+// The tile's 37 x 37 x 3 window ( the sum of the four waves' windows, in wave order ) overlaps its neighbours' by 5 pixels,
+// so it goes to scratch memory, and a second launch adds up the at most four windows that cover an input pixel, in a
+// fixed order, with the free term: no run differs from another.
+constexpr int SgWindow = 37;                        // 2 x + kx for x < 16, kx < 7
+constexpr int SgWindowFloats = SgWindow * SgWindow * 3;
+constexpr int SgBandFloats = 7 * SgWindow * 3;      // one row of source pixels: 7 rows of the window
+constexpr int SgWaveFloats = 4 * SgBandFloats;
+constexpr int SgColumns = 147;                      // 3 channels x 49 taps
+constexpr int SgStagePitch = 68;                    // floats per pixel where a row of pixels passes through LDS
+
+constexpr int SgPackedFilterFloats = 5 * 8 * 64 * 4;
+
+typedef float stemAcc __attribute__( ( ext_vector_type( 16 ) ) );
+
+// filter [64][49][3] -> [chunk][i][lane][e]: output channel 32 half + 4 i + e of column 32 chunk + l32 ( column n = input
+// channel n / 49, tap n % 49; zeros beyond column 146 ), so that a wave instruction of the main kernel reads 1 KB on end.
+// ( Read column by column, 256 bytes per lane, every instruction touched 64 cache lines, five times eight times a tile:
+// the refills of the first-level cache from the second took longer than the products. )
+__global__ __launch_bounds__( 256 ) void packStemFilterKernel( const float* filter, float* packed )
+{
+	const int idx = blockIdx.x * 256 + threadIdx.x;
+	if( idx >= SgPackedFilterFloats ) {
+		return;
+	}
+	const int e = idx & 3, lane = ( idx >> 2 ) & 63, i = ( idx >> 8 ) & 7, chunk = idx >> 11;
+	const int n = chunk * 32 + ( lane & 31 ), k = 32 * ( lane >> 5 ) + 4 * i + e;
+	packed[idx] = n < SgColumns ? filter[k * SgColumns + ( n % 49 ) * 3 + n / 49] : 0.f;
+}
+
+__global__ __launch_bounds__( 256, 2 )
+void stemInputGradientKernel( const float* outputDiff, const float* columns, float* tileWindows,
+	int outH, int outW, int tilesY, int tilesX, int totalTiles )
+{
+	// ( + a place per lane for the columns of padding, + a word that stays zero )
+	__shared__ __attribute__( ( aligned( 16 ) ) ) float windows[4][SgWaveFloats + 64 + 4];
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, half = lane >> 5;
+	// ( a row of pixels passes through the wave's window before the window is cleared for the tile )
+	static_assert( 16 * SgStagePitch <= SgWaveFloats, "the staging row fits the window" );
+	float* const stage = windows[wave];
+	// operand row rho of block b: pixel x = 4 ( 2 * bit 2 of rho + bit 3 of rho ) + ( rho & 3 ), y = 4 ( 2 b + bit 4 of rho ) + wave;
+	// as accumulator row rho = 8 q + 4 half + i that is X = 2 half + ( q & 1 ), band 2 b + ( q >> 1 )
+	const int ownX = 4 * ( 2 * ( ( l32 >> 2 ) & 1 ) + ( ( l32 >> 3 ) & 1 ) ) + ( l32 & 3 );
+	int rowTerm[2][4];
+#pragma unroll
+	for( int b = 0; b < 2; ++b ) {
+#pragma unroll
+		for( int q = 0; q < 4; ++q ) {
+			const int x4 = 4 * ( 2 * half + ( q & 1 ) );
+			const int band = 2 * b + ( q >> 1 );
+			rowTerm[b][q] = band * SgBandFloats + 2 * x4 * 3;
+		}
+	}
+	int columnTerm[5];
+#pragma unroll
+	for( int chunk = 0; chunk < 5; ++chunk ) {
+		const int n = chunk * 32 + l32;
+		const int c = n / 49, tap = n - c * 49, ky = tap / 7, kx = tap - ky * 7;
+		columnTerm[chunk] = n < SgColumns ? ( ky * SgWindow + kx ) * 3 + c : 0;
+	}
+	const bool paddingColumn = 4 * 32 + l32 >= SgColumns; // ( in the last chunk )
+	const __amdgpu_buffer_rsrc_t source = makeBuffer( outputDiff );
+	// the filter as the lanes want it: [chunk][i][lane][4], see packStemFilterKernel
+	const __amdgpu_buffer_rsrc_t filterColumns = __builtin_amdgcn_make_buffer_rsrc( const_cast<float*>( columns ), 0, SgPackedFilterFloats * 4, 0x00020000 );
+	float* const window = windows[wave];
+	if( lane == 0 ) {
+		window[SgWaveFloats + 64] = 0.f;
+	}
+	// The wave's four rows of 16 pixels ( 4 KB each, contiguous ) are fetched as they lie, a wave instruction 1 KB on end,
+	// and turned into the operand's layout ( a lane: 32 values of one pixel ) through LDS. Fetched in that layout
+	// directly, every instruction touched 64 cache lines for 16 bytes each and came back for them seven more times
+	// after the other waves' fetches had pushed them out.
+	float4 fetched[4][4];
+	auto request = [&]( int t ) {
+		const int tx = t % tilesX;
+		const int ty = ( t / tilesX ) % tilesY;
+		const int n = t / ( tilesX * tilesY );
+#pragma unroll
+		for( int band = 0; band < 4; ++band ) {
+			const int sy = 16 * ty + 4 * band + wave;
+#pragma unroll
+			for( int m = 0; m < 4; ++m ) {
+				const int sx = 16 * tx + 4 * m + ( lane >> 4 );
+				const unsigned at = ( t < totalTiles && sy < outH && sx < outW )
+					? static_cast<unsigned>( ( ( n * outH + sy ) * outW + sx ) * 64 + ( lane & 15 ) * 4 ) * 4u : OutOfRange;
+				fetched[band][m] = bufferLoad4( source, at );
+			}
+		}
+	};
+	for( int t = blockIdx.x; t < totalTiles; t += gridDim.x ) {
+		request( t );
+		float4 a[2][8];
+#pragma unroll
+		for( int band = 0; band < 4; ++band ) {
+#pragma unroll
+			for( int m = 0; m < 4; ++m ) {
+				*reinterpret_cast<float4*>( stage + ( 4 * m + ( lane >> 4 ) ) * SgStagePitch + ( lane & 15 ) * 4 ) = fetched[band][m];
+			}
+			__builtin_amdgcn_fence( __ATOMIC_RELEASE, "wavefront" );
+			__builtin_amdgcn_wave_barrier();
+			__builtin_amdgcn_fence( __ATOMIC_ACQUIRE, "wavefront" );
+			if( ( l32 >> 4 ) == ( band & 1 ) ) {
+#pragma unroll
+				for( int i = 0; i < 8; ++i ) {
+					a[band >> 1][i] = *reinterpret_cast<const float4*>( stage + ownX * SgStagePitch + 32 * half + 4 * i );
+				}
+			}
+			__builtin_amdgcn_fence( __ATOMIC_RELEASE, "wavefront" );
+			__builtin_amdgcn_wave_barrier();
+			__builtin_amdgcn_fence( __ATOMIC_ACQUIRE, "wavefront" );
+		}
+		float4 w[8];
+#pragma unroll
+		for( int i = 0; i < 8; ++i ) {
+			w[i] = bufferLoad4( filterColumns, i * 1024u + lane * 16u );
+		}
+		// ( nobody reads this wave's window of the tile before any more: the barrier at the end of the tile )
+		for( int i = lane; i < SgWaveFloats; i += 64 ) {
+			window[i] = 0.f;
+		}
+#pragma unroll
+		for( int chunk = 0; chunk < 5; ++chunk ) {
+			stemAcc acc[2];
+#pragma unroll
+			for( int b = 0; b < 2; ++b ) {
+#pragma unroll
+				for( int r = 0; r < 16; ++r ) {
+					acc[b][r] = 0.f;
+				}
+			}
+#pragma unroll
+			for( int i = 0; i < 8; ++i ) {
+				acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32( a[0][i].x, w[i].x, acc[0], 0, 0, 0 );
+				acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32( a[1][i].x, w[i].x, acc[1], 0, 0, 0 );
+				acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32( a[0][i].y, w[i].y, acc[0], 0, 0, 0 );
+				acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32( a[1][i].y, w[i].y, acc[1], 0, 0, 0 );
+				acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32( a[0][i].z, w[i].z, acc[0], 0, 0, 0 );
+				acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32( a[1][i].z, w[i].z, acc[1], 0, 0, 0 );
+				acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32( a[0][i].w, w[i].w, acc[0], 0, 0, 0 );
+				acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32( a[1][i].w, w[i].w, acc[1], 0, 0, 0 );
+			}
+			if( chunk < 4 ) {
+				// the next chunk's columns arrive while this chunk's products are added up
+#pragma unroll
+				for( int i = 0; i < 8; ++i ) {
+					w[i] = bufferLoad4( filterColumns, ( ( chunk + 1 ) * 8 + i ) * 1024u + lane * 16u );
+				}
+			}
+#pragma unroll
+			for( int i = 0; i < 4; ++i ) {
+				float before[2][4];
+				// ( columns of padding hold zeros; they go to a place of the lane's own )
+				const int columnPart = ( chunk == 4 && paddingColumn ) ? -1 : columnTerm[chunk] + 6 * i;
+#pragma unroll
+				for( int b = 0; b < 2; ++b ) {
+#pragma unroll
+					for( int q = 0; q < 4; ++q ) {
+						before[b][q] = window[columnPart < 0 ? SgWaveFloats + lane : rowTerm[b][q] + columnPart];
+					}
+				}
+#pragma unroll
+				for( int b = 0; b < 2; ++b ) {
+#pragma unroll
+					for( int q = 0; q < 4; ++q ) {
+						window[columnPart < 0 ? SgWaveFloats + lane : rowTerm[b][q] + columnPart] = before[b][q] + acc[b][q * 4 + i];
+					}
+				}
+				__builtin_amdgcn_fence( __ATOMIC_RELEASE, "wavefront" );
+				__builtin_amdgcn_wave_barrier();
+				__builtin_amdgcn_fence( __ATOMIC_ACQUIRE, "wavefront" );
+			}
+		}
+		__syncthreads();
+		// row wy of the tile's window: from wave w the band with 0 <= wy - 8 band - 2 w <= 6, if there is one
+		float* const out = tileWindows + static_cast<long long>( t ) * SgWindowFloats;
+		// ( half a workgroup per row, a thread per value of the row: which bands a row takes is the same for the whole
+		// half, so the addresses come from the scalar unit; what a wave has no band for is read from a word that holds
+		// zero, so that all the reads of a thread can be in flight together )
+		{
+			const int column = threadIdx.x & 127;
+			if( column < SgWindow * 3 ) {
+				float sums[( SgWindow + 1 ) / 2];
+#pragma unroll
+				for( int step = 0; step < ( SgWindow + 1 ) / 2; ++step ) {
+					const int wy = __builtin_amdgcn_readfirstlane( 2 * step + ( static_cast<int>( threadIdx.x ) >> 7 ) );
+					sums[step] = 0.f;
+#pragma unroll
+					for( int w4 = 0; w4 < 4; ++w4 ) {
+						const int band = ( wy - 2 * w4 ) >> 3; // ( floor: negative for wy < 2 w )
+						const int ky = wy - 2 * w4 - 8 * band;
+						const bool has = band >= 0 && band < 4 && ky <= 6 && wy < SgWindow;
+						sums[step] += windows[w4][has ? band * SgBandFloats + ky * ( SgWindow * 3 ) + column : SgWaveFloats + 64];
+					}
+				}
+#pragma unroll
+				for( int step = 0; step < ( SgWindow + 1 ) / 2; ++step ) {
+					const int wy = __builtin_amdgcn_readfirstlane( 2 * step + ( static_cast<int>( threadIdx.x ) >> 7 ) );
+					if( wy < SgWindow ) {
+						out[wy * ( SgWindow * 3 ) + column] = sums[step];
+					}
+				}
+			}
+		}
+		__syncthreads();
+	}
+}
+
+// input pixel ( gy, gx ): window row gy + 3 - 32 ty of tile row ty, for the one or two ty that have such a row
+// ( a row of workgroups per SgGatherRows rows of the batch's images: what depends on the row is scalar arithmetic, and a
+// thread has several rows' reads in flight )
+constexpr int SgGatherRows = 8;
+
+__global__ __launch_bounds__( 256 )
+void stemGatherWindowsKernel( const float* tileWindows, const float* freeTerm, float* inputDiff, int height, int width,
+	int tilesY, int tilesX, int rows )
+{
+	const int j = blockIdx.x * 256 + threadIdx.x;
+	if( j >= width * 3 ) {
+		return;
+	}
+	const int gx = j / 3, c = j - gx * 3;
+	const float bias = freeTerm != nullptr ? freeTerm[c] : 0.f;
+	const int tx1 = ( gx + 3 ) >> 5;
+	const int wx1 = gx + 3 - 32 * tx1, wx0 = wx1 + 32; // in tile tx1 and in the one to its left
+	const bool has1 = tx1 < tilesX, has0 = tx1 >= 1 && wx0 < SgWindow;
+	float sums[SgGatherRows];
+#pragma unroll
+	for( int r = 0; r < SgGatherRows; ++r ) {
+		const int row = blockIdx.y * SgGatherRows + r;
+		sums[r] = bias;
+		if( row < rows ) {
+			const int gy = row % height, n = row / height;
+			const int ty1 = ( gy + 3 ) >> 5;
+#pragma unroll
+			for( int dy = 1; dy >= 0; --dy ) {
+				const int ty = ty1 - dy, wy = gy + 3 - 32 * ty;
+				if( ty >= 0 && ty < tilesY && wy < SgWindow ) {
+					const float* const from = tileWindows + static_cast<long long>( ( n * tilesY + ty ) * tilesX ) * SgWindowFloats
+						+ wy * ( SgWindow * 3 ) + c;
+					if( has0 ) {
+						sums[r] += from[( tx1 - 1 ) * SgWindowFloats + wx0 * 3];
+					}
+					if( has1 ) {
+						sums[r] += from[tx1 * SgWindowFloats + wx1 * 3];
+					}
+				}
+			}
+		}
+	}
+#pragma unroll
+	for( int r = 0; r < SgGatherRows; ++r ) {
+		const int row = blockIdx.y * SgGatherRows + r;
+		if( row < rows ) {
+			inputDiff[static_cast<long long>( row ) * ( width * 3 ) + j] = sums[r];
+		}
+	}
+}
+
+// tiles of 16 x 16 output-gradient pixels, or 0 where the window-summing path does not apply
+static long long stemInputGradientTiles( const nhConvDesc& d )
+{
+	if( d.filterHeight != 7 || d.filterWidth != 7 || d.strideHeight != 2 || d.strideWidth != 2 || d.dilationHeight != 1 || d.dilationWidth != 1
+		|| d.paddingHeight != 3 || d.paddingWidth != 3 || d.channels != 3 || d.filterCount != 64 )
+	{
+		return 0;
+	}
+	const long long tiles = static_cast<long long>( d.batch ) * ceilDiv( d.resultHeight, 16 ) * ceilDiv( d.resultWidth, 16 );
+	// ( a handful of tiles: the general path spreads further; rows of the batch are a grid dimension of the second launch )
+	return tiles >= 32 && tiles * SgWindowFloats <= 0x7fffffffLL && static_cast<long long>( d.batch ) * d.height <= 65535LL * SgGatherRows ? tiles : 0;
+}
+
+static bool stemInputGradient( hipStream_t stream, const nhConvDesc& d, const float* outputDiff, const float* filter,
+	const float* freeTerm, float* inputDiff, float* workspace )
+{
+	const long long tiles = stemInputGradientTiles( d );
+	if( tiles == 0 || !isAligned16( outputDiff ) || !isAligned16( workspace )
+		|| !fitsBuffer( 1, 0, static_cast<long long>( d.batch ) * d.resultHeight * d.resultWidth * 64 ) )
+	{
+		return false;
+	}
+	const int tilesY = ceilDiv( d.resultHeight, 16 ), tilesX = ceilDiv( d.resultWidth, 16 );
+	// workspace: the filter in the main kernel's order, then every tile's window
+	float* const columns = workspace;
+	float* const tileWindows = workspace + SgPackedFilterFloats;
+	hipLaunchKernelGGL( packStemFilterKernel, dim3( SgPackedFilterFloats / 256 ), dim3( 256 ), 0, stream, filter, columns );
+	const unsigned groups = static_cast<unsigned>( tiles ); // ( workgroups that stay for several tiles gained nothing )
+	hipLaunchKernelGGL( stemInputGradientKernel, dim3( groups ), dim3( 256 ), 0, stream, outputDiff, columns, tileWindows,
+		d.resultHeight, d.resultWidth, tilesY, tilesX, static_cast<int>( tiles ) );
+	hipLaunchKernelGGL( stemGatherWindowsKernel, dim3( ceilDiv( d.width * 3, 256 ), ceilDiv( d.batch * d.height, SgGatherRows ) ), dim3( 256 ), 0, stream,
+		tileWindows, freeTerm, inputDiff, d.height, d.width, tilesY, tilesX, d.batch * d.height );
+	return true;
+}
+
 int convBackwardData( hipStream_t stream, const nhConvDesc& d, const float* outputDiff, const float* filter,
 	const float* freeTerm, float* inputDiff, float* swappedFilter )
 {
@@ -2915,6 +3226,9 @@ int convBackwardData( hipStream_t stream, const nhConvDesc& d, const float* outp
 		return NH_OK;
 	}
 	int rc = NH_OK;
+	if( stemInputGradient( stream, d, outputDiff, filter, freeTerm, inputDiff, swappedFilter ) ) {
+		return hipGetLastError() == hipSuccess ? NH_OK : NH_ERR_HIP;
+	}
 	if( convBackwardDataByClasses( stream, d, outputDiff, filter, freeTerm, inputDiff, swappedFilter, rc ) ) {
 		return rc;
 	}
@@ -3109,6 +3423,11 @@ int nhBlobConvolutionBackwardWorkspaceSize( const nhConvDesc* d, size_t* bytes )
 	}
 	NH_REQUIRE( bytes != nullptr );
 	*bytes = static_cast<size_t>( d->filterCount ) * d->filterHeight * d->filterWidth * d->channels * sizeof( float );
+	// ( the stem's input gradient: the filter with its columns padded, and the windows that its tiles leave there )
+	const size_t stemTiles = static_cast<size_t>( stemInputGradientTiles( *d ) );
+	if( stemTiles > 0 ) {
+		*bytes = ( SgPackedFilterFloats + stemTiles * SgWindowFloats ) * sizeof( float );
+	}
 	return NH_OK;
 }
 

@@ -476,7 +476,7 @@ struct CTinyChain {
 
 template<typename... T> struct CTypeList {};
 // the functors a chain may hold ( float in, float out, no more than TinyFunctorBytes of state )
-typedef CTypeList<CCopyOp<float>, CAddOp<float>, CSubOp<float>, CMulOp<float>, CDivOp, CNegOp, CAbsOp, CMaxOp, CMinOp, CSqrtOp, CInvOp,
+typedef CTypeList<CFillOp<float>, CFillFromOp<float>, CCopyOp<float>, CAddOp<float>, CSubOp<float>, CMulOp<float>, CDivOp, CNegOp, CAbsOp, CMaxOp, CMinOp, CSqrtOp, CInvOp,
 	CAddValueOp<float>, CMulValueOp<float>, CNegMulValueOp, CMultiplyAndAddOp, CMultiplyAndSubOp, CMulAddOp, CNegMulOp> CTinyKinds;
 
 template<typename F, typename List> struct CKindOf;

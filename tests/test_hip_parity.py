@@ -414,6 +414,11 @@ GPU_CONV_GRADIENT_CASES = CONV_CASES + [
     (1, 13, 13, 4, 16, 3, 3, 1, 1, 3, 3, 1, 1),     # the masked form over 16 gradient channels: taps in scalar registers
     (1, 9, 9, 4, 32, 5, 5, 2, 2, 2, 2, 2, 2),
     (8, 14, 14, 256, 512, 3, 3, 1, 1, 2, 2, 1, 1),  # few tiles per class, long reduction: K slices over a preset result
+    # the 7x7/2 stem from 3 to 64 channels at sizes that take the window-summing input gradient: tiles of 32 x 32 input
+    # pixels that fit exactly, even sizes with partial tiles, odd sizes
+    (1, 224, 224, 3, 64, 7, 7, 3, 3, 2, 2, 1, 1),
+    (3, 70, 100, 3, 64, 7, 7, 3, 3, 2, 2, 1, 1),
+    (6, 63, 65, 3, 64, 7, 7, 3, 3, 2, 2, 1, 1),
 ]
 
 

@@ -110,6 +110,10 @@ def random_program(g, length):
     while len(program) < length:
         n = int(g.choice(sizes))
         kind = g.integers(0, 10)
+        if kind < 1:
+            out = int(g.choice(places))
+            program.append(("nhVectorFill", [at(out), float(g.integers(-3, 4)) * 0.5, n]))
+            continue
         if kind < 3:
             name, n_in, scalar = str(g.choice(UNARY)), 1, False
         elif kind < 6:
