@@ -433,7 +433,7 @@ NH_API int nhBlobMeanPoolingBackward(nhStream s, const nhPoolingDesc* desc_host,
 NH_API int nhStreamOverlapLstm(nhStream s, int enable);
 
 /* Several small element-wise calls in one launch. No counterpart in the reference: there every call runs at once on the
- * calling thread. On a stream that has asked for it (enable != 0) a float element-wise call over at most 16384 elements
+ * calling thread. On a stream that has asked for it (enable != 0) a float element-wise call over at most 262144 elements
  * (fill, copy, add, sub, multiply, divide, negate, abs, max, min, sqrt, inv, and the forms with a device scalar: add value,
  * multiply, neg-multiply, multiply-and-add, multiply-and-sub, eltwise multiply-add, eltwise neg-multiply) is put aside;
  * up to eight of them are launched together, in call order and with bit-identical results, as soon as ANY other call

@@ -1505,23 +1505,39 @@ template<> struct CChanAtomic<1> {
 // registers ( every input row loaded once per strip ) and keeps the nine tap sums and the free-term sum of its strip in
 // registers. The threads of a workgroup then meet per channel in an LDS table ( LDS atomics ), and the workgroup leaves
 // with one global atomic add per table entry: a few hundred adds per address over the whole launch.
-template<int STRIDE, int WPT>
+//
+// PARTIALS ( the form that is launched wherever the stream has scratch memory ): a workgroup has a whole number of threads
+// per channel group ( blockDim = cg * threads per group ), a thread keeps its channel group for all its strips and its
+// sums in registers until the end, the threads of a group then meet in LDS through plain stores and one pass of
+// adds, and the workgroup leaves its 40 x cg sums in a row of its own in scratch memory; sumLearnPartialsKernel adds the
+// rows up in workgroup order. No atomic anywhere: LDS float atomics cost several hundred cycles per wave instruction
+// on this part ( 40 of them per strip were a third of the launch at 14 x 14 x 384 ), a few hundred global adds per
+// address another third, and the sums now come out the same on every run.
+template<int STRIDE, int WPT, bool PARTIALS>
 __global__ __launch_bounds__( 256 )
 void channelwiseLearn3x3Kernel( const nhConvDesc d, const float* input, const float* outputDiff, float* filterDiff,
-	float* freeTermDiff, int wGroups, int rowChunks, int rowsPerItem, int totalItems )
+	float* freeTermDiff, int wGroups, int rowChunks, int rowsPerItem, int totalItems, float* partials )
 {
 	constexpr int NC = ( WPT - 1 ) * STRIDE + 3;
 	constexpr int Keep = 3 - STRIDE;
 	constexpr int Sums = 10; // nine taps and the free term
 	__shared__ float table[Sums * 4 * 256];
 	const int cg = d.channels / 4; // at most 256: the table has a column per channel group
-	const int tableWidth = cg;
-	for( int idx = threadIdx.x; idx < Sums * 4 * tableWidth; idx += blockDim.x ) {
-		table[idx] = 0.f;
+	const int tableWidth = PARTIALS ? static_cast<int>( blockDim.x ) : cg;
+	if( !PARTIALS ) {
+		for( int idx = threadIdx.x; idx < Sums * 4 * tableWidth; idx += blockDim.x ) {
+			table[idx] = 0.f;
+		}
+		__syncthreads();
 	}
-	__syncthreads();
+	float4 kept[Sums];
+#pragma unroll
+	for( int k = 0; k < Sums; ++k ) {
+		kept[k] = make_float4( 0.f, 0.f, 0.f, 0.f );
+	}
 	// a few hundred workgroups walk the strips grid-stride and collect in their table: the global adds at the end are what
 	// limits this kernel when thousands of workgroups bring their own
+	// ( PARTIALS: items are counted group-first too, and blockDim is a multiple of cg: item % cg stays what it is )
 	for( int item = blockIdx.x * blockDim.x + threadIdx.x; item < totalItems; item += gridDim.x * blockDim.x ) {
 		int t = item;
 		const int group = t % cg;
@@ -1590,13 +1606,42 @@ void channelwiseLearn3x3Kernel( const nhConvDesc d, const float* input, const fl
 			hi += STRIDE;
 			diff += diffRow;
 		}
+		if( PARTIALS ) {
+#pragma unroll
+			for( int k = 0; k < Sums; ++k ) {
+				kept[k].x += sums[k].x; kept[k].y += sums[k].y; kept[k].z += sums[k].z; kept[k].w += sums[k].w;
+			}
+		} else {
+#pragma unroll
+			for( int k = 0; k < Sums; ++k ) {
+				atomicAdd( &table[( k * 4 + 0 ) * tableWidth + group], sums[k].x );
+				atomicAdd( &table[( k * 4 + 1 ) * tableWidth + group], sums[k].y );
+				atomicAdd( &table[( k * 4 + 2 ) * tableWidth + group], sums[k].z );
+				atomicAdd( &table[( k * 4 + 3 ) * tableWidth + group], sums[k].w );
+			}
+		}
+	}
+	if( PARTIALS ) {
+		// thread tid = sub * cg + group: every thread its column, then the threads below cg add their group's columns up
 #pragma unroll
 		for( int k = 0; k < Sums; ++k ) {
-			atomicAdd( &table[( k * 4 + 0 ) * tableWidth + group], sums[k].x );
-			atomicAdd( &table[( k * 4 + 1 ) * tableWidth + group], sums[k].y );
-			atomicAdd( &table[( k * 4 + 2 ) * tableWidth + group], sums[k].z );
-			atomicAdd( &table[( k * 4 + 3 ) * tableWidth + group], sums[k].w );
+			table[( k * 4 + 0 ) * tableWidth + threadIdx.x] = kept[k].x;
+			table[( k * 4 + 1 ) * tableWidth + threadIdx.x] = kept[k].y;
+			table[( k * 4 + 2 ) * tableWidth + threadIdx.x] = kept[k].z;
+			table[( k * 4 + 3 ) * tableWidth + threadIdx.x] = kept[k].w;
 		}
+		__syncthreads();
+		float* const mine = partials + static_cast<long long>( blockIdx.x ) * ( Sums * 4 * cg );
+		for( int idx = threadIdx.x; idx < Sums * 4 * cg; idx += blockDim.x ) {
+			const int k4 = idx / cg;
+			const int group = idx - k4 * cg;
+			float v = 0.f;
+			for( int at = group; at < tableWidth; at += cg ) {
+				v += table[k4 * tableWidth + at];
+			}
+			mine[idx] = v;
+		}
+		return;
 	}
 	__syncthreads();
 	for( int idx = threadIdx.x; idx < Sums * 4 * tableWidth; idx += blockDim.x ) {
@@ -1608,6 +1653,46 @@ void channelwiseLearn3x3Kernel( const nhConvDesc d, const float* input, const fl
 			unsafeAtomicAdd( filterDiff + ( k4 >> 2 ) * d.channels + channel, v );
 		} else if( freeTermDiff != nullptr ) {
 			unsafeAtomicAdd( freeTermDiff + channel, v );
+		}
+	}
+}
+
+// Entry k4 * cg + group of every workgroup's row: tap k4 / 4 ( 9: the free term ) of channel 4 group + k4 % 4. A workgroup
+// adds up 16 entries: 16 threads per entry take every 16th row with eight sums of their own in flight, then meet in LDS.
+__global__ __launch_bounds__( 256 )
+void sumLearnPartialsKernel( const float* partials, int rows, int cg, int channels, float* filterDiff, float* freeTermDiff )
+{
+	__shared__ float meet[16][17];
+	const int entries = 40 * cg; // ( a multiple of 8 )
+	const int column = threadIdx.x & 15, lane = threadIdx.x >> 4;
+	const int idx = blockIdx.x * 16 + column;
+	float sums[8] = { 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f };
+	if( idx < entries ) {
+		int r = lane;
+		for( ; r + 7 * 16 < rows; r += 8 * 16 ) {
+#pragma unroll
+			for( int u = 0; u < 8; ++u ) {
+				sums[u] += partials[static_cast<long long>( r + u * 16 ) * entries + idx];
+			}
+		}
+		for( int u = 0; r < rows; r += 16, ++u ) {
+			sums[u & 7] += partials[static_cast<long long>( r ) * entries + idx];
+		}
+	}
+	meet[lane][column] = ( ( sums[0] + sums[1] ) + ( sums[2] + sums[3] ) ) + ( ( sums[4] + sums[5] ) + ( sums[6] + sums[7] ) );
+	__syncthreads();
+	if( lane == 0 && idx < entries ) {
+		float v = 0.f;
+#pragma unroll
+		for( int l = 0; l < 16; ++l ) {
+			v += meet[l][column];
+		}
+		const int k4 = idx / cg;
+		const int channel = ( idx - k4 * cg ) * 4 + ( k4 & 3 );
+		if( k4 < 36 ) {
+			filterDiff[( k4 >> 2 ) * channels + channel] += v;
+		} else if( freeTermDiff != nullptr ) {
+			freeTermDiff[channel] += v;
 		}
 	}
 }
@@ -2455,13 +2540,37 @@ static int channelwiseLearn3x3Impl( nhStream s, const nhConvDesc* d, const float
 	int rowChunks = 1, rowsPerItem = 1;
 	// tall strips ( few row chunks ): every chunk re-reads two halo rows and ends with 40 LDS adds per thread
 	chooseRowChunks( perRow, d->resultHeight, 4, 256, &rowChunks, &rowsPerItem );
+	const int cg = d->channels / 4;
+	// with scratch memory: a row of 40 x cg sums per workgroup, added up by a second launch. 512 workgroups, two per compute
+	// unit ( every row of a strip is a round trip to memory, so one per unit leaves the memory system idle; measured at
+	// 128 / 256 / 384 / 512 / 768 / 1024: 14 x 14 x 384 36 / 26 / 27 / 26 / 31 / 36 us, 56 x 56 x 144 145 / 87 / 104 / 88 / 88 / 95,
+	// 112 x 112 x 96 stride 2 191 / 159 / 157 / 140 / 148 / 141; with LDS and global adds instead 64 / 114 / 177 )
+	{
+		const int threads = cg * ( 256 / cg ); // ( cg <= 256 )
+		const long long cap = 512;
+		int chunks = 1, rows = 1;
+		chooseRowChunks( perRow, d->resultHeight, 4, static_cast<int>( cap ), &chunks, &rows );
+		const long long items = perRow * chunks;
+		const long long blocks = ( items + threads - 1 ) / threads < cap ? ( items + threads - 1 ) / threads : cap;
+		float* partials = nullptr;
+		unsigned* counter = nullptr;
+		if( streamMeetingPlace( toStream( s ), static_cast<size_t>( blocks ) * 40 * cg, &partials, &counter ) ) {
+			hipLaunchKernelGGL( ( channelwiseLearn3x3Kernel<STRIDE, WPT, true> ), dim3( static_cast<unsigned>( blocks ) ), dim3( threads ), 0,
+				toStream( s ), *d, input, outputDiff, filterDiff, freeTermDiff, wGroups, chunks, rows, static_cast<int>( items ), partials );
+			NH_LAUNCH_CHECK();
+			hipLaunchKernelGGL( sumLearnPartialsKernel, dim3( ceilDiv( 40 * cg, 16 ) ), dim3( 256 ), 0, toStream( s ),
+				partials, static_cast<int>( blocks ), cg, d->channels, filterDiff, freeTermDiff );
+			NH_LAUNCH_CHECK();
+			return NH_OK;
+		}
+	}
+	// without ( a stream that is being captured ): LDS adds, then global adds. One workgroup per compute unit: measured
+	// best of 64..2048 ( more workgroups bring more global adds, fewer leave compute units idle )
 	const long long items = perRow * rowChunks;
-	// one workgroup per compute unit: measured best of 64..2048 ( more workgroups bring more global adds, fewer leave
-	// compute units idle; larger workgroups change nothing )
 	const long long cap = 256;
 	const long long blocks = ( items + 255 ) / 256 < cap ? ( items + 255 ) / 256 : cap;
-	hipLaunchKernelGGL( ( channelwiseLearn3x3Kernel<STRIDE, WPT> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0,
-		toStream( s ), *d, input, outputDiff, filterDiff, freeTermDiff, wGroups, rowChunks, rowsPerItem, static_cast<int>( items ) );
+	hipLaunchKernelGGL( ( channelwiseLearn3x3Kernel<STRIDE, WPT, false> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0,
+		toStream( s ), *d, input, outputDiff, filterDiff, freeTermDiff, wGroups, rowChunks, rowsPerItem, static_cast<int>( items ), nullptr );
 	NH_LAUNCH_CHECK();
 	return NH_OK;
 }

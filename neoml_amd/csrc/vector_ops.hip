@@ -450,12 +450,14 @@ struct CTanhDiffOutOp : CNoScalar { __device__ float operator()( float y, float 
 // either untouched by the calls in front of it in the chain, or begin exactly where an operand of one of them begins
 // ( then each element is read and written by the same thread, in program order ), needs nothing between it and the
 // call in front. Any other overlap ( a shifted view, a scalar that a call in front has produced ) needs every thread
-// to have finished the calls in front: the chain then runs in one workgroup with a barrier in front of such calls.
+// to have finished the calls in front: the chain then runs in one workgroup with a barrier in front of such calls ( calls
+// over more than TinyOpMaxCount elements do not join such a chain: it is launched, and they begin the next one ).
 
 constexpr int TinyChainMax = 8;
-constexpr int TinyOpMaxCount = 16384;
+constexpr int TinyOpMaxCount = 16384; // in a chain that runs as one workgroup
+constexpr int TinyWideMaxCount = 262144; // in a chain without barriers ( a solver's passes over a filter of a few hundred KB )
 constexpr int TinyThreads = 1024;
-constexpr int TinyMaxBlocks = 8;
+constexpr int TinyMaxBlocks = 256;
 constexpr int TinyFunctorBytes = 16;
 
 struct CTinyOp {
@@ -672,7 +674,7 @@ template<int NIN, typename TIn, typename TOut, typename F>
 static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, const F& f )
 {
 	if constexpr( std::is_same<TIn, float>::value && std::is_same<TOut, float>::value && CKindOf<F, CTinyKinds>::Value >= 0 ) {
-		if( n > TinyOpMaxCount || __atomic_load_n( &tinyDeferringStreams, __ATOMIC_RELAXED ) == 0 ) {
+		if( n > TinyWideMaxCount || __atomic_load_n( &tinyDeferringStreams, __ATOMIC_RELAXED ) == 0 ) {
 			return false;
 		}
 		const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
@@ -694,8 +696,7 @@ static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 		if( chain.Length == TinyChainMax ) {
 			launchTinyChain( stream, chain );
 		}
-		CTinyOp& op = chain.Ops[chain.Length];
-		op = CTinyOp();
+		CTinyOp op = CTinyOp();
 		op.In[0] = NIN >= 1 ? a : nullptr;
 		op.In[1] = NIN >= 2 ? b : nullptr;
 		op.In[2] = NIN >= 3 ? c : nullptr;
@@ -719,7 +720,10 @@ static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 		}
 		writes.Lo = out;
 		writes.Hi = out + n;
-		bool barrier = false;
+		bool barrier = false, wide = n > TinyOpMaxCount;
+		for( int k = 0; k < chain.Length; ++k ) {
+			wide = wide || chain.Ops[k].Count > TinyOpMaxCount;
+		}
 		for( int k = 0; k < chain.Length && !barrier; ++k ) {
 			const CTinyOp& front = chain.Ops[k];
 			CFloatRange frontWrites;
@@ -743,10 +747,17 @@ static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 				barrier = rangesTouch( writes, frontReads );
 			}
 		}
+		if( barrier && wide ) {
+			// a chain with a barrier is one workgroup, too few threads for this many elements: what is in front goes out
+			// now, and this call is the first of the next chain
+			launchTinyChain( stream, chain );
+			barrier = false;
+		}
 		op.Barrier = barrier ? 1 : 0;
 		if( chain.Length == 0 ) {
 			__atomic_fetch_add( &tinyChainsPending, 1, __ATOMIC_RELAXED );
 		}
+		chain.Ops[chain.Length] = op;
 		++chain.Length;
 		return true;
 	} else {

@@ -10,7 +10,7 @@ from test_oracle import rng
 
 pytestmark = pytest.mark.gpu
 
-ARENA = 1 << 16
+ARENA = 1 << 19
 
 
 class Streams:
@@ -104,8 +104,9 @@ def random_program(g, length):
     """Operands begin at a few fixed places of the arena, so that exact matches, shifted overlaps and disjoint operands
     all come up; a result either begins where one of the call's own operands begins or keeps clear of them (what the
     entry points ask for); scalars sit in the arena too, sometimes where a call in front writes."""
-    places = [0, 0, 0, 1, 3, 4, 64, 4096, 8192, 8195, 12288, 20000, 20000, 36000]
-    sizes = [1, 5, 64, 777, 1024, 4096, 8192, 8192, 16384, 16384, 20000]
+    places = [0, 0, 0, 1, 3, 4, 64, 4096, 8192, 8195, 12288, 20000, 20000, 36000, 100000, 100000, 210000]
+    # ( above 16384 elements a call joins a chain only while no call in it has to wait for another; above 262144 never )
+    sizes = [1, 5, 64, 777, 1024, 4096, 8192, 8192, 16384, 16384, 20000, 70000, 200000, 300000]
     program = []
     while len(program) < length:
         n = int(g.choice(sizes))
