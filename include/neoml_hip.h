@@ -441,7 +441,8 @@ NH_API int nhStreamOverlapLstm(nhStream s, int enable);
  * nhStreamDestroy, enable = 0, or a release of device memory (nhRawFree, a pool's clean-up). Until then their results are
  * not in memory and their operands must stay valid, so this is only for streams whose work, synchronisation included,
  * all goes through this library (an engine's own stream): synchronise with nhStreamSynchronize, not with HIP calls of
- * your own. Nothing is put aside while the stream is being captured into a graph. What it saves: a row-normalising
+ * your own. Nothing is put aside while the stream is being captured into a graph (synchronise through the library
+ * before a capture begins: what was put aside before it would otherwise become the graph's first launch). What it saves: a row-normalising
  * layer (CObjectNormalizationLayer) asks for five such calls per run, each a launch of about 4 us. */
 NH_API int nhStreamDeferSmallOps(nhStream s, int enable);
 /* LSTM (NME.h:1005-1011). Weights: inputWeights [4H x objectSize], recurrentWeights [4H x H]; gate order in

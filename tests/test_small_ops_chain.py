@@ -240,3 +240,32 @@ def test_small_call_between_two_lstms_keeps_its_place(streams):
             torch.cuda.synchronize()
     finally:
         na.check(lib.nhStreamOverlapLstm(s, 0))
+
+
+def test_nothing_is_put_aside_while_the_stream_is_captured():
+    """A graph recorded from a stream that puts small calls aside holds every call: the recording ends outside the library,
+    so a call left in the queue would be missing from the graph (and run once, later, outside it)."""
+    import torch
+    import neoml_amd
+    lib = neoml_amd.load()
+    dev = torch.device("cuda:0")
+    x = torch.full((4096,), 1.0, device=dev)
+    two = torch.full((1,), 2.0, device=dev)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    s = torch.cuda.Stream()
+    ps = ctypes.c_void_p(s.cuda_stream)
+    torch.cuda.synchronize()
+    neoml_amd.check(lib.nhStreamDeferSmallOps(ps, 1))
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            for _ in range(3):
+                neoml_amd.check(lib.nhVectorMultiply(ps, P(x), P(x), 4096, P(two)))
+        torch.cuda.synchronize()
+        assert float(x[0]) == 1.0 and float(x[4095]) == 1.0  # recorded, not run
+        for replay in range(1, 4):
+            graph.replay()
+            torch.cuda.synchronize()
+            assert float(x[0]) == 8.0 ** replay and float(x[4095]) == 8.0 ** replay
+    finally:
+        neoml_amd.check(lib.nhStreamDeferSmallOps(ps, 0))
