@@ -325,12 +325,23 @@ void maxPoolingIndexKernel( const nhPoolingDesc d, const float* source, int* max
 			v[0] = *p;
 		}
 	};
+	const bool narrow = total <= 0x7fffffffLL; // ( 32-bit divisions where the count allows it )
 	for( long long item = blockIdx.x * 256LL + threadIdx.x; item < total; item += step ) {
-		long long t = item;
-		const int c = static_cast<int>( t % channelGroups ) * VECW; t /= channelGroups;
-		const int wo = static_cast<int>( t % d.resultWidth ); t /= d.resultWidth;
-		const int ho = static_cast<int>( t % d.resultHeight ); t /= d.resultHeight;
-		const long long n = t;
+		int c, wo, ho;
+		long long n;
+		if( narrow ) {
+			unsigned t = static_cast<unsigned>( item );
+			c = static_cast<int>( t % static_cast<unsigned>( channelGroups ) ) * VECW; t /= static_cast<unsigned>( channelGroups );
+			wo = static_cast<int>( t % static_cast<unsigned>( d.resultWidth ) ); t /= static_cast<unsigned>( d.resultWidth );
+			ho = static_cast<int>( t % static_cast<unsigned>( d.resultHeight ) ); t /= static_cast<unsigned>( d.resultHeight );
+			n = t;
+		} else {
+			long long t = item;
+			c = static_cast<int>( t % channelGroups ) * VECW; t /= channelGroups;
+			wo = static_cast<int>( t % d.resultWidth ); t /= d.resultWidth;
+			ho = static_cast<int>( t % d.resultHeight ); t /= d.resultHeight;
+			n = t;
+		}
 		const int stripRow = ho * d.strideHeight;
 		const float* strip = source + ( n * d.height + stripRow ) * rowSize;
 		const int windowColumn = wo * d.strideWidth * d.channels;
@@ -1299,12 +1310,24 @@ void poolingBackwardKernel( const nhPoolingDesc d, const float* resultDiff, cons
 {
 	const float scale = 1.f / d.filterHeight / d.filterWidth;
 	const int cg = d.channels / VECW;
+	// ( an item's place from 32-bit divisions where the count allows it: four 64-bit ones were most of this kernel's instructions )
+	const bool narrow = totalItems <= 0x7fffffffLL;
 	for( long long item = blockIdx.x * 256LL + threadIdx.x; item < totalItems; item += static_cast<long long>( gridDim.x ) * 256 ) {
-		long long t = item;
-		const int c = static_cast<int>( t % cg ) * VECW; t /= cg;
-		const int wi = static_cast<int>( t % d.width ); t /= d.width;
-		const int hi = static_cast<int>( t % d.height );
-		const long long n = t / d.height;
+		int c, wi, hi;
+		long long n;
+		if( narrow ) {
+			unsigned t = static_cast<unsigned>( item );
+			c = static_cast<int>( t % static_cast<unsigned>( cg ) ) * VECW; t /= static_cast<unsigned>( cg );
+			wi = static_cast<int>( t % static_cast<unsigned>( d.width ) ); t /= static_cast<unsigned>( d.width );
+			hi = static_cast<int>( t % static_cast<unsigned>( d.height ) );
+			n = t / static_cast<unsigned>( d.height );
+		} else {
+			long long t = item;
+			c = static_cast<int>( t % cg ) * VECW; t /= cg;
+			wi = static_cast<int>( t % d.width ); t /= d.width;
+			hi = static_cast<int>( t % d.height );
+			n = t / d.height;
+		}
 		// windows ho with ho * s <= hi < ho * s + fh
 		const int hoFirst = hi >= d.filterHeight ? ( hi - d.filterHeight ) / d.strideHeight + 1 : 0;
 		const int hoLast = min( hi / d.strideHeight, d.resultHeight - 1 );
