@@ -294,6 +294,9 @@ def main():
         x, y = rand(n, h, w, c), empty(n, d.resultHeight, d.resultWidth, c)
         idx = torch.empty(y.shape, dtype=torch.int32, device=dev)
         neoml_amd.check(lib.nhBlobMaxPooling(stream, ctypes.byref(d), P(x), P(idx), P(y)))
+        measure("BlobMaxPooling with indices cfg2 %dx%dx%dx%d %dx%d/%d" % (n, h, w, c, f, f, s_),
+                lambda: lib.nhBlobMaxPooling(stream, ctypes.byref(d), P(x), P(idx), P(y)),
+                0, 4 * (x.numel() + 2 * y.numel()), 4 * (x.numel() + 2 * y.numel()))
         g, dx = rand(*y.shape), empty(n, h, w, c)
         measure("BlobMaxPoolingBackward cfg2 %dx%dx%dx%d %dx%d/%d" % (n, h, w, c, f, f, s_),
                 lambda: lib.nhBlobMaxPoolingBackward(stream, ctypes.byref(d), P(g), P(idx), P(dx)),

@@ -396,6 +396,77 @@ void maxPoolingIndexKernel( const nhPoolingDesc d, const float* source, int* max
 	}
 }
 
+// The same for a square window of FILTER x FILTER and 4 channels per thread: the window's loads and the loads of the
+// row-index lookup ( image columns 0 .. FILTER - 1 of the strip, whatever the window's column ) all go out together, and
+// the lookup's answer is picked by the winning column afterwards. Same comparisons in the same order as above.
+template<int FILTER>
+__global__ __launch_bounds__( 256 )
+void maxPoolingIndexSquareKernel( const nhPoolingDesc d, const float* source, int* maxIndices, float* result, int total )
+{
+	const int rowSize = d.width * d.channels;
+	const unsigned channelGroups = static_cast<unsigned>( d.channels / 4 );
+	for( int item = xcdSwizzle( blockIdx.x, gridDim.x ) * 256 + threadIdx.x; item < total; item += gridDim.x * 256 ) {
+		unsigned t = static_cast<unsigned>( item );
+		const int c = static_cast<int>( t % channelGroups ) * 4; t /= channelGroups;
+		const int wo = static_cast<int>( t % static_cast<unsigned>( d.resultWidth ) ); t /= static_cast<unsigned>( d.resultWidth );
+		const int ho = static_cast<int>( t % static_cast<unsigned>( d.resultHeight ) );
+		const long long n = t / static_cast<unsigned>( d.resultHeight );
+		const int stripRow = ho * d.strideHeight;
+		const float* strip = source + ( n * d.height + stripRow ) * rowSize;
+		const int windowColumn = wo * d.strideWidth * d.channels;
+		float4 window[FILTER][FILTER], lookup[FILTER][FILTER]; // [kh][kw]
+#pragma unroll
+		for( int kh = 0; kh < FILTER; ++kh ) {
+#pragma unroll
+			for( int kw = 0; kw < FILTER; ++kw ) {
+				window[kh][kw] = *reinterpret_cast<const float4*>( strip + static_cast<long long>( kh ) * rowSize + windowColumn + kw * d.channels + c );
+				lookup[kh][kw] = *reinterpret_cast<const float4*>( strip + static_cast<long long>( kh ) * rowSize + kw * d.channels + c );
+			}
+		}
+		float best[4];
+		int index[4];
+#pragma unroll
+		for( int e = 0; e < 4; ++e ) {
+			auto lane = [e]( const float4& v ) { return e == 0 ? v.x : ( e == 1 ? v.y : ( e == 2 ? v.z : v.w ) ); };
+			int bestCol = 0;
+#pragma unroll
+			for( int kw = 0; kw < FILTER; ++kw ) {
+				float col = lane( window[0][kw] );
+#pragma unroll
+				for( int kh = 1; kh < FILTER; ++kh ) {
+					const float v = lane( window[kh][kw] );
+					if( v > col ) {
+						col = v;
+					}
+				}
+				if( kw == 0 || col > best[e] ) {
+					best[e] = col;
+					bestCol = kw;
+				}
+			}
+			int rowIdx = 0;
+#pragma unroll
+			for( int kw = 0; kw < FILTER; ++kw ) {
+				float rowBest = lane( lookup[0][kw] );
+				int idx = 0;
+#pragma unroll
+				for( int kh = 1; kh < FILTER; ++kh ) {
+					const float v = lane( lookup[kh][kw] );
+					if( v > rowBest ) {
+						rowBest = v;
+						idx = kh;
+					}
+				}
+				rowIdx = bestCol == kw ? idx : rowIdx;
+			}
+			index[e] = ( stripRow + rowIdx ) * rowSize + windowColumn + bestCol * d.channels + c + e;
+		}
+		const long long out = static_cast<long long>( item ) * 4;
+		*reinterpret_cast<float4*>( result + out ) = make_float4( best[0], best[1], best[2], best[3] );
+		*reinterpret_cast<int4*>( maxIndices + out ) = make_int4( index[0], index[1], index[2], index[3] );
+	}
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // BlobResizeImage: pad (constant / edge / reflect) or crop the H and W dimensions
 
@@ -2955,7 +3026,15 @@ int nhBlobMaxPooling( nhStream s, const nhPoolingDesc* d, const float* source, i
 	const long long items = vec ? total / 4 : total;
 	long long blocks = ( items + 255 ) / 256;
 	blocks = blocks > 1048576 ? 1048576 : blocks;
-	if( vec ) {
+	// ( the lookup reads image columns 0 .. filterWidth - 1: they exist, the filter fits the image )
+	const bool square = vec && d->filterHeight == d->filterWidth && items <= 0x3fffffffLL;
+	if( square && d->filterHeight == 3 ) {
+		hipLaunchKernelGGL( maxPoolingIndexSquareKernel<3>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			*d, source, maxIndices, result, static_cast<int>( items ) );
+	} else if( square && d->filterHeight == 2 ) {
+		hipLaunchKernelGGL( maxPoolingIndexSquareKernel<2>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+			*d, source, maxIndices, result, static_cast<int>( items ) );
+	} else if( vec ) {
 		hipLaunchKernelGGL( maxPoolingIndexKernel<4>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
 			*d, source, maxIndices, result, items );
 	} else {
