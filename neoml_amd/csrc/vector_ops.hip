@@ -458,7 +458,6 @@ constexpr int TinyChainMax = 8;
 constexpr int TinyOpMaxCount = 16384; // in a chain that runs as one workgroup
 constexpr int TinyWideMaxCount = 262144; // in a chain without barriers ( a solver's passes over a filter of a few hundred KB )
 constexpr int TinyThreads = 1024;
-constexpr int TinyMaxBlocks = 256;
 constexpr int TinyFunctorBytes = 16;
 
 struct CTinyOp {
@@ -474,7 +473,7 @@ struct CTinyOp {
 struct CTinyChain {
 	int Length;
 	int Blocks;
-	int Straight; // no call has to wait for another, and Blocks * TinyThreads covers the longest call
+	int Straight; // no call has to wait for another: the grid has a thread per element of the longest call
 	int Reserved;
 	CTinyOp Ops[TinyChainMax];
 };
@@ -622,28 +621,18 @@ static bool launchTinyChain( hipStream_t stream, CTinyChain& chain )
 	if( chain.Length == 0 ) {
 		return false;
 	}
-	chain.Blocks = 1;
 	bool barrier = false;
 	int longest = 0;
 	for( int k = 0; k < chain.Length; ++k ) {
 		barrier = barrier || chain.Ops[k].Barrier != 0;
 		longest = chain.Ops[k].Count > longest ? chain.Ops[k].Count : longest;
 	}
-	chain.Straight = 0;
-	if( !barrier ) {
-		const int blocks = ceilDiv( longest, TinyThreads );
-		chain.Blocks = blocks < TinyMaxBlocks ? blocks : TinyMaxBlocks;
-		chain.Straight = chain.Blocks * TinyThreads >= longest ? 1 : 0;
-	}
-	if( chain.Straight != 0 ) {
-		constexpr int straightThreads = 256; // ( 64, 256 and 1024 take the same 4.6 us for four calls over 8192 elements )
-		chain.Blocks = ceilDiv( longest, straightThreads );
-		hipLaunchKernelGGL( tinyChainKernel, dim3( chain.Blocks ), dim3( straightThreads ), 0, stream, chain );
-		chain.Length = 0;
-		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
-		return true;
-	}
-	hipLaunchKernelGGL( tinyChainKernel, dim3( chain.Blocks ), dim3( TinyThreads ), 0, stream, chain );
+	// one workgroup with barriers, or a thread per element of the longest call ( workgroups of 64, 256 and 1024 threads take
+	// the same 4.6 us for four calls over 8192 elements )
+	constexpr int StraightThreads = 256;
+	chain.Straight = barrier ? 0 : 1;
+	chain.Blocks = barrier ? 1 : ceilDiv( longest, StraightThreads );
+	hipLaunchKernelGGL( tinyChainKernel, dim3( chain.Blocks ), dim3( barrier ? TinyThreads : StraightThreads ), 0, stream, chain );
 	chain.Length = 0;
 	__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
 	return true;
