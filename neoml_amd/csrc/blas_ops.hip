@@ -464,6 +464,49 @@ void transposePlainKernel( const T* in, T* out, int height, int width )
 	}
 }
 
+// The same with 128-bit accesses to memory ( both dimensions multiples of 4, 16-byte aligned ): a thread reads four
+// neighbours of a row, leaves them in a column of the tile, and collects four neighbours of a result row from four rows of it.
+template<typename T>
+__global__ __launch_bounds__( 256 )
+void transposePlainQuadKernel( const T* in, T* out, int height, int width )
+{
+	static_assert( sizeof( T ) == 4, "four elements are 128 bits" );
+	__shared__ T tile[64][65];
+	const long long base = static_cast<long long>( blockIdx.z ) * height * width;
+	const int x0 = blockIdx.x * 64;
+	const int y0 = blockIdx.y * 64;
+	const int q4 = ( threadIdx.x & 15 ) * 4;
+	const int r0 = threadIdx.x >> 4;
+	int4 v[4];
+#pragma unroll
+	for( int k = 0; k < 4; ++k ) {
+		const int y = y0 + r0 + 16 * k, x = x0 + q4;
+		v[k] = make_int4( 0, 0, 0, 0 );
+		if( y < height && x < width ) {
+			v[k] = *reinterpret_cast<const int4*>( in + base + static_cast<long long>( y ) * width + x );
+		}
+	}
+#pragma unroll
+	for( int k = 0; k < 4; ++k ) {
+		int* row = reinterpret_cast<int*>( &tile[r0 + 16 * k][q4] );
+		row[0] = v[k].x; row[1] = v[k].y; row[2] = v[k].z; row[3] = v[k].w;
+	}
+	__syncthreads();
+#pragma unroll
+	for( int k = 0; k < 4; ++k ) {
+		const int xr = r0 + 16 * k; // row of the result inside the tile
+		const int x = x0 + xr, y = y0 + q4;
+		if( x < width && y < height ) {
+			int4 w;
+			w.x = *reinterpret_cast<const int*>( &tile[q4 + 0][xr] );
+			w.y = *reinterpret_cast<const int*>( &tile[q4 + 1][xr] );
+			w.z = *reinterpret_cast<const int*>( &tile[q4 + 2][xr] );
+			w.w = *reinterpret_cast<const int*>( &tile[q4 + 3][xr] );
+			*reinterpret_cast<int4*>( out + base + static_cast<long long>( x ) * height + y ) = w;
+		}
+	}
+}
+
 template<typename T>
 static int transposeImpl( nhStream s, int batchSize, const T* first, int height, int medium, int width, int channels,
 	T* result, int resultBufferSize )
@@ -491,6 +534,11 @@ static int transposeImpl( nhStream s, int batchSize, const T* first, int height,
 	}
 	if( medium == 1 && channels == 1 ) {
 		const dim3 grid( ceilDiv( width, 64 ), ceilDiv( height, 64 ), batchSize );
+		if( grid.y <= 65535 && grid.z <= 65535 && height % 4 == 0 && width % 4 == 0 && isAligned16( first ) && isAligned16( result ) ) {
+			hipLaunchKernelGGL( transposePlainQuadKernel<T>, grid, dim3( 256 ), 0, toStream( s ), first, result, height, width );
+			NH_LAUNCH_CHECK();
+			return NH_OK;
+		}
 		if( grid.y <= 65535 && grid.z <= 65535 ) {
 			hipLaunchKernelGGL( transposePlainKernel<T>, grid, dim3( 256 ), 0, toStream( s ), first, result, height, width );
 			NH_LAUNCH_CHECK();

@@ -202,10 +202,14 @@ def test_ctc_greedy_pipeline_bit_exact():
 def test_transpose():
     g = rng(8)
     for shape in ((1, 1, 1, 1, 1), (2, 3, 1, 5, 1), (2, 4, 3, 5, 2), (1, 1, 3, 4, 2), (3, 7, 1, 1, 4), (2, 16, 1, 8, 64),
-                  (2, 100, 1, 130, 1), (4, 256, 1, 8, 64), (2, 70, 2, 33, 3)):
+                  (2, 100, 1, 130, 1), (4, 256, 1, 8, 64), (2, 70, 2, 33, 3),
+                  # plain matrices whose sides are multiples of 4 ( 128-bit accesses ): partial and whole 64 x 64 tiles
+                  (3, 100, 1, 132, 1), (2, 256, 1, 512, 1), (1, 4, 1, 68, 1)):
         x = g.uniform(-1, 1, shape).astype(np.float32)
         assert np.array_equal(hip().transpose(x), orc.transpose(x)), shape
     xi = g.integers(-5, 5, (2, 9, 2, 7, 3)).astype(np.int32)
+    assert np.array_equal(hip().transpose(xi, integer=True), np.transpose(xi, (0, 3, 2, 1, 4)))
+    xi = g.integers(-5, 5, (2, 72, 1, 60, 1)).astype(np.int32)
     assert np.array_equal(hip().transpose(xi, integer=True), np.transpose(xi, (0, 3, 2, 1, 4)))
 
 
