@@ -177,8 +177,9 @@ def other_workload(args):
     steps = args.steps
     pools = plan.make_events(tags, steps)
     # what the engine adapter asks for its own stream: runs of small element-wise calls (the per-row scalars of the
-    # normalisation layers) go out several per launch; every launch and wait below goes through the library
-    deferring = args.workload == "transformer" and not args.no_defer
+    # normalisation layers) go out several per launch, and a fully connected layer's product takes its free term along;
+    # every launch and wait below goes through the library
+    deferring = not args.no_defer
     be.defer_small_ops(deferring)
     for _ in range(args.warmup):
         plan.run()
@@ -238,7 +239,7 @@ def main():
     ap.add_argument("--time-by-runs", action="store_true",
                     help="other workloads: the per-family split from one pair of events per run of consecutive launches of a family")
     ap.add_argument("--no-defer", action="store_true",
-                    help="transformer workload: every small element-wise call as a launch of its own (nhStreamDeferSmallOps off)")
+                    help="other workloads: every call a launch of its own (nhStreamDeferSmallOps off)")
     ap.add_argument("--cpu-replicas", type=int, default=min(16, os.cpu_count() or 1),
                     help="engines of the multi-replica CPU baseline (one thread each; 16 = the host cores that go with one GPU)")
     ap.add_argument("--per-kernel", action="store_true", help="print a per-op-family timing table to stderr")

@@ -443,7 +443,13 @@ NH_API int nhStreamOverlapLstm(nhStream s, int enable);
  * all goes through this library (an engine's own stream): synchronise with nhStreamSynchronize, not with HIP calls of
  * your own. Nothing is put aside while the stream is being captured into a graph (synchronise through the library
  * before a capture begins: what was put aside before it would otherwise become the graph's first launch). What it saves: a row-normalising
- * layer (CObjectNormalizationLayer) asks for five such calls per run, each a launch of about 4 us. */
+ * layer (CObjectNormalizationLayer) asks for five such calls per run, each a launch of about 4 us.
+ * On such a stream nhMultiplyMatrixByTransposedMatrix with a dense result (resultRowSize == secondHeight) waits for the
+ * call behind it as well: nhAddVectorToMatrixRows over that result in place (batchSize 1, the same height and width) is
+ * then part of the product's launch, the vector added to the accumulators on their way out, as the fully connected
+ * layer's two calls ask (NeoML/src/Dnn/Layers/FullyConnectedLayer.cpp:91-99); any other call launches the product first,
+ * as it was asked for. The sum is the same; where the product is cut into slices of its reduction the vector is added
+ * in front of the slices instead of behind them, i.e. the last bits may differ from the two launches'. */
 NH_API int nhStreamDeferSmallOps(nhStream s, int enable);
 /* LSTM (NME.h:1005-1011). Weights: inputWeights [4H x objectSize], recurrentWeights [4H x H]; gate order in
  * the 4H vector: main(tanh) | forget | input | output (src/CPU/CpuMathEngineDnnLstm.h:49-90).

@@ -656,6 +656,12 @@ int nhAddVectorToMatrixRows( nhStream s, int batchSize, const float* matrix, flo
 {
 	NH_REQUIRE( batchSize >= 0 && matrixHeight >= 0 && matrixWidth >= 0 );
 	NH_REQUIRE( static_cast<long long>( matrixHeight ) * matrixWidth <= 0x7fffffffLL );
+	int rc = NH_OK;
+	if( batchSize == 1 && __atomic_load_n( &tinyChainsPending, __ATOMIC_RELAXED ) != 0
+		&& fusePendingProduct( s, matrix, result, matrixHeight, matrixWidth, vector, &rc ) )
+	{
+		return rc; // ( the product that waited for this call took the vector with it )
+	}
 	return launchRowBroadcast<BO_Add>( s, matrix, result, vector, batchSize, matrixHeight, matrixWidth,
 		matrixHeight * matrixWidth, matrixWidth );
 }

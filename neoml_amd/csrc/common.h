@@ -29,6 +29,11 @@ extern int tinyChainsPending;
 bool flushTinyOps( hipStream_t stream ); // true: something was launched
 void flushAllTinyOps();
 void releaseTinyQueue( hipStream_t stream );
+// On such a stream a product A * B^T with a dense result may wait for the call behind it ( deferProduct: true, nothing
+// launched ); an AddVectorToMatrixRows over that result in place then launches both as one ( fusePendingProduct: true,
+// *rc is the launch's code ), any other call sends the product out first, through toStream.
+bool deferProduct( nhStream s, const float* a, int lda, const float* b, int ldb, float* c, int ldc, int M, int N, int K );
+bool fusePendingProduct( nhStream s, const float* matrix, float* result, int height, int width, const float* vector, int* rc );
 
 inline hipStream_t toStream( nhStream s )
 {

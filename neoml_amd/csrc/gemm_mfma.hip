@@ -3369,6 +3369,11 @@ int nhMultiplyMatrixByTransposedMatrix( nhStream s, const float* first, int firs
 	// resultBufferSize is not looked at: the reference CPU engine ignores it (src/CPU/CpuMathEngineBlas.cpp:906-918)
 	// and CFullyConnectedLayer::RunOnce passes 0 (NeoML/src/Dnn/Layers/FullyConnectedLayer.cpp:91-94)
 	( void )resultBufferSize;
+	// ( on a stream that puts small calls aside the product waits for the call behind it: a free term added to its rows
+	// goes into the same launch )
+	if( deferProduct( s, first, firstRowSize, second, secondRowSize, result, resultRowSize, firstHeight, secondHeight, firstWidth ) ) {
+		return NH_OK;
+	}
 	return matMulNT( toStream( s ), first, firstRowSize, second, secondRowSize, result, resultRowSize,
 		firstHeight, secondHeight, firstWidth, 1, 0, 0, 0, nullptr, false );
 }

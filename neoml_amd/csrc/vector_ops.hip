@@ -599,13 +599,33 @@ __global__ __launch_bounds__( TinyThreads ) void tinyChainKernel( const CTinyCha
 	}
 }
 
+// A product A * B^T whose launch waits for the call behind it: a fully connected layer ( CFullyConnectedLayer::RunOnce,
+// NeoML/src/Dnn/Layers/FullyConnectedLayer.cpp:91-99 ) asks for the product and then for its free term to be added to the
+// product's rows in place, a pass over the whole result for one add per element. On a stream that puts small calls aside
+// the product is put aside too ( nothing else is pending then ), and if the next call is that AddVectorToMatrixRows, both
+// go out as the one launch the product's kernels have for it ( the free term added to the accumulators on their way
+// out ); any other call launches the product as it was asked for, first.
+struct CPendingProduct {
+	bool Pending = false;
+	const float* A = nullptr;
+	const float* B = nullptr;
+	float* C = nullptr;
+	int Lda = 0, Ldb = 0, Ldc = 0, M = 0, N = 0, K = 0;
+};
+
 struct CTinyQueue {
 	bool Enabled = false;
 	CTinyChain Chain = {};
+	CPendingProduct Product;
 };
 
+int matMulNT( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
+	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC, const float* bias, bool accumulate );
+
 typedef std::map<std::pair<int, hipStream_t>, CTinyQueue> CTinyQueues;
-static std::mutex tinyLock;
+// ( recursive: a product launched from under the lock may ask its stream's pool for scratch memory, a pool at its limit
+// gives memory back first, and giving memory back launches what every stream holds )
+static std::recursive_mutex tinyLock;
 static CTinyQueues& tinyQueues()
 {
 	static CTinyQueues* queues = new CTinyQueues; // never destroyed: calls may still arrive while the process unloads
@@ -638,6 +658,20 @@ static bool launchTinyChain( hipStream_t stream, CTinyChain& chain )
 	return true;
 }
 
+// what the queue holds: the product that waits for its successor ( then nothing else is queued ), or a chain
+static bool launchPending( hipStream_t stream, CTinyQueue& queue )
+{
+	if( queue.Product.Pending ) {
+		const CPendingProduct p = queue.Product;
+		queue.Product.Pending = false;
+		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+		// ( a launch that fails leaves its message with nhGetLastError and its HIP error to the next launch check )
+		( void )matMulNT( stream, p.A, p.Lda, p.B, p.Ldb, p.C, p.Ldc, p.M, p.N, p.K, 1, 0, 0, 0, nullptr, false );
+		return true;
+	}
+	return launchTinyChain( stream, queue.Chain );
+}
+
 bool flushTinyOps( hipStream_t stream )
 {
 	int device = 0;
@@ -645,9 +679,9 @@ bool flushTinyOps( hipStream_t stream )
 		( void )hipGetLastError();
 		return false;
 	}
-	std::lock_guard<std::mutex> guard( tinyLock );
+	std::lock_guard<std::recursive_mutex> guard( tinyLock );
 	auto found = tinyQueues().find( std::make_pair( device, stream ) );
-	return found != tinyQueues().end() && launchTinyChain( stream, found->second.Chain );
+	return found != tinyQueues().end() && launchPending( stream, found->second );
 }
 
 void flushAllTinyOps()
@@ -664,9 +698,9 @@ void flushAllTinyOps()
 	std::pair<int, hipStream_t> launched[16];
 	int launchedCount = 0;
 	{
-		std::lock_guard<std::mutex> guard( tinyLock );
+		std::lock_guard<std::recursive_mutex> guard( tinyLock );
 		for( auto& entry : tinyQueues() ) {
-			if( entry.second.Chain.Length == 0 ) {
+			if( entry.second.Chain.Length == 0 && !entry.second.Product.Pending ) {
 				continue;
 			}
 			if( entry.first.first != active ) {
@@ -676,7 +710,7 @@ void flushAllTinyOps()
 				}
 				active = entry.first.first;
 			}
-			if( launchTinyChain( entry.first.second, entry.second.Chain ) && launchedCount < 16 ) {
+			if( launchPending( entry.first.second, entry.second ) && launchedCount < 16 ) {
 				launched[launchedCount++] = entry.first;
 			}
 		}
@@ -706,15 +740,71 @@ void releaseTinyQueue( hipStream_t stream )
 		( void )hipGetLastError();
 		return;
 	}
-	std::lock_guard<std::mutex> guard( tinyLock );
+	std::lock_guard<std::recursive_mutex> guard( tinyLock );
 	auto found = tinyQueues().find( std::make_pair( device, stream ) );
 	if( found != tinyQueues().end() ) {
-		launchTinyChain( stream, found->second.Chain );
+		launchPending( stream, found->second );
 		if( found->second.Enabled ) {
 			__atomic_fetch_sub( &tinyDeferringStreams, 1, __ATOMIC_RELAXED );
 		}
 		tinyQueues().erase( found );
 	}
+}
+
+bool deferProduct( nhStream s, const float* a, int lda, const float* b, int ldb, float* c, int ldc, int M, int N, int K )
+{
+	if( __atomic_load_n( &tinyDeferringStreams, __ATOMIC_RELAXED ) == 0 || M <= 0 || N <= 0 || K <= 0 || ldc != N ) {
+		return false;
+	}
+	const hipStream_t stream = toStream( s ); // ( what the stream holds goes out first )
+	int device = 0;
+	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+	if( hipGetDevice( &device ) != hipSuccess || hipStreamIsCapturing( stream, &capture ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return false;
+	}
+	if( capture != hipStreamCaptureStatusNone ) {
+		return false;
+	}
+	std::lock_guard<std::recursive_mutex> guard( tinyLock );
+	auto found = tinyQueues().find( std::make_pair( device, stream ) );
+	if( found == tinyQueues().end() || !found->second.Enabled || found->second.Chain.Length != 0 || found->second.Product.Pending ) {
+		return false;
+	}
+	CPendingProduct& p = found->second.Product;
+	p.Pending = true;
+	p.A = a; p.Lda = lda; p.B = b; p.Ldb = ldb; p.C = c; p.Ldc = ldc; p.M = M; p.N = N; p.K = K;
+	__atomic_fetch_add( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+	return true;
+}
+
+bool fusePendingProduct( nhStream s, const float* matrix, float* result, int height, int width, const float* vector, int* rc )
+{
+	const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
+	int device = 0;
+	if( hipGetDevice( &device ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return false;
+	}
+	CPendingProduct p;
+	{
+		std::lock_guard<std::recursive_mutex> guard( tinyLock );
+		auto found = tinyQueues().find( std::make_pair( device, stream ) );
+		if( found == tinyQueues().end() || !found->second.Product.Pending ) {
+			return false;
+		}
+		p = found->second.Product;
+		if( matrix != p.C || result != p.C || height != p.M || width != p.N || vector == nullptr ) {
+			return false; // ( the caller's own launch sends the product out first, as it was asked for )
+		}
+		found->second.Product.Pending = false;
+		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+	}
+	*rc = matMulNT( stream, p.A, p.Lda, p.B, p.Ldb, p.C, p.Ldc, p.M, p.N, p.K, 1, 0, 0, 0, vector, false );
+	if( __atomic_load_n( &lstmPartnersAwaited, __ATOMIC_RELAXED ) != 0 ) {
+		noteStreamUse( stream );
+	}
+	return true;
 }
 
 struct CFloatRange {
@@ -755,10 +845,13 @@ static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 		if( capture != hipStreamCaptureStatusNone ) {
 			return false; // the recording ends outside this library: nothing may be left behind
 		}
-		std::lock_guard<std::mutex> guard( tinyLock );
+		std::lock_guard<std::recursive_mutex> guard( tinyLock );
 		auto found = tinyQueues().find( std::make_pair( device, stream ) );
 		if( found == tinyQueues().end() || !found->second.Enabled ) {
 			return false;
+		}
+		if( found->second.Product.Pending ) {
+			launchPending( stream, found->second ); // ( a product that waited for its successor: this call is not the one )
 		}
 		CTinyChain& chain = found->second.Chain;
 		if( chain.Length == TinyChainMax ) {
@@ -1001,7 +1094,7 @@ extern "C" int nhStreamDeferSmallOps( nhStream s, int enable )
 	const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
 	int device = 0;
 	NH_HIP( hipGetDevice( &device ) );
-	std::lock_guard<std::mutex> guard( tinyLock );
+	std::lock_guard<std::recursive_mutex> guard( tinyLock );
 	CTinyQueue& queue = tinyQueues()[std::make_pair( device, stream )];
 	if( ( enable != 0 ) != queue.Enabled ) {
 		queue.Enabled = enable != 0;
@@ -1009,7 +1102,7 @@ extern "C" int nhStreamDeferSmallOps( nhStream s, int enable )
 			__atomic_fetch_add( &tinyDeferringStreams, 1, __ATOMIC_RELAXED );
 		} else {
 			__atomic_fetch_sub( &tinyDeferringStreams, 1, __ATOMIC_RELAXED );
-			launchTinyChain( stream, queue.Chain );
+			launchPending( stream, queue );
 			NH_LAUNCH_CHECK();
 		}
 	}

@@ -269,3 +269,69 @@ def test_nothing_is_put_aside_while_the_stream_is_captured():
             assert float(x[0]) == 8.0 ** replay and float(x[4095]) == 8.0 ** replay
     finally:
         neoml_amd.check(lib.nhStreamDeferSmallOps(ps, 0))
+
+
+def test_product_waits_for_its_free_term(streams):
+    """On such a stream a product A * B^T is put aside as well, and an AddVectorToMatrixRows over its result in place goes
+    into the same launch (the two calls of CFullyConnectedLayer::RunOnce, NeoML/src/Dnn/Layers/FullyConnectedLayer.cpp:
+    91-99). Whatever else comes behind the product finds it done."""
+    import torch
+    from nhtest import assert_close
+    lib, na = streams.lib, streams.na
+    g = rng(4300)
+    dev = streams.dev
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    for m, n, k in ((8192, 512, 512), (300, 101, 64), (64, 1000, 512), (1000, 24, 8), (5, 7, 3)):
+        a = g.uniform(-1, 1, (m, k)).astype(np.float32)
+        w = (g.uniform(-1, 1, (n, k)) / np.sqrt(k)).astype(np.float32)
+        bias = g.uniform(-1, 1, n).astype(np.float32)
+        want = (a.astype(np.float64) @ w.astype(np.float64).T + bias).astype(np.float32)
+        d_a, d_w, d_bias = up(a), up(w), up(bias)
+        outs = {}
+        for name, stream in (("plain", streams.plain), ("deferring", streams.deferring)):
+            c = torch.zeros((m, n), device=dev)
+            torch.cuda.synchronize()
+            na.check(lib.nhMultiplyMatrixByTransposedMatrix(stream, P(d_a), m, k, k, P(d_w), n, k, P(c), n, m * n))
+            na.check(lib.nhAddVectorToMatrixRows(stream, 1, P(c), P(c), m, n, P(d_bias)))
+            na.check(lib.nhStreamSynchronize(stream))
+            outs[name] = c.cpu().numpy()
+        assert_close(outs["deferring"], want, "product + free term in one launch %s" % ((m, n, k),), atol=2e-5)
+        assert_close(outs["deferring"], outs["plain"], "one launch vs two %s" % ((m, n, k),), atol=2e-5)
+    # other successors: the product is launched as it was asked for, before them
+    m, n, k = 512, 256, 128
+    a = g.uniform(-1, 1, (m, k)).astype(np.float32)
+    w = g.uniform(-1, 1, (n, k)).astype(np.float32)
+    bias = g.uniform(-1, 1, n).astype(np.float32)
+    d_a, d_w, d_bias, zero = up(a), up(w), up(bias), up(np.zeros(1, np.float32))
+
+    def run(stream, successor):
+        c = torch.zeros((m, n), device=dev)
+        other = torch.zeros((m, n), device=dev)
+        torch.cuda.synchronize()
+        na.check(lib.nhMultiplyMatrixByTransposedMatrix(stream, P(d_a), m, k, k, P(d_w), n, k, P(c), n, m * n))
+        successor(stream, c, other)
+        na.check(lib.nhStreamSynchronize(stream))
+        return c.cpu().numpy(), other.cpu().numpy()
+
+    successors = {
+        "nothing but the wait": lambda s, c, o: None,
+        "free term into another matrix": lambda s, c, o: na.check(lib.nhAddVectorToMatrixRows(s, 1, P(c), P(o), m, n, P(d_bias))),
+        "free term of half the rows": lambda s, c, o: na.check(lib.nhAddVectorToMatrixRows(s, 1, P(c), P(c), m // 2, n, P(d_bias))),
+        "a large call on the result": lambda s, c, o: na.check(lib.nhVectorReLU(s, P(c), P(o), m * n, P(zero))),
+        "a small call on the result": lambda s, c, o: na.check(lib.nhVectorAbs(s, P(c), P(o), 4096)),
+        "a second product": lambda s, c, o: na.check(lib.nhMultiplyMatrixByTransposedMatrix(s, P(d_a), m, k, k, P(d_w), n, k, P(o), n, m * n)),
+    }
+    for what, successor in successors.items():
+        want_c, want_o = run(streams.plain, successor)
+        got_c, got_o = run(streams.deferring, successor)
+        assert same_bits(got_c, want_c) and same_bits(got_o, want_o), what
+    # memory given back while a product waits: it runs first
+    c = torch.zeros((m, n), device=dev)
+    block = ctypes.c_void_p()
+    na.check(lib.nhRawAlloc(ctypes.byref(block), 1 << 20))
+    torch.cuda.synchronize()
+    na.check(lib.nhMultiplyMatrixByTransposedMatrix(streams.deferring, P(d_a), m, k, k, P(d_w), n, k, P(c), n, m * n))
+    na.check(lib.nhRawFree(block))
+    torch.cuda.synchronize()
+    assert_close(c.cpu().numpy(), (a.astype(np.float64) @ w.astype(np.float64).T).astype(np.float32), "launched by nhRawFree", atol=2e-5)

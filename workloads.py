@@ -171,7 +171,8 @@ class HipBackend:
             out = self.empty(m, n)
         self._timed("fc", 2 * m * n * k, 4 * (m * k + n * k + m * n), self.lib.nhMultiplyMatrixByTransposedMatrix,
                     self._p(x), m, k, k, self._p(weight), n, k, self._p(out), n, m * n)
-        self._call(self.lib.nhAddVectorToMatrixRows, 1, self._p(out), self._p(out), m, n, self._p(bias))
+        # ( the layer's second call; the same family, so that a stream on which the product waits for it shows both as one )
+        self._timed("fc", 0, 8 * m * n, self.lib.nhAddVectorToMatrixRows, 1, self._p(out), self._p(out), m, n, self._p(bias))
         return out
 
     def softmax(self, x, out=None):
