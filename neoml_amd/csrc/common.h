@@ -34,6 +34,11 @@ void releaseTinyQueue( hipStream_t stream );
 // *rc is the launch's code ), any other call sends the product out first, through toStream.
 bool deferProduct( nhStream s, const float* a, int lda, const float* b, int ldb, float* c, int ldc, int M, int N, int K );
 bool fusePendingProduct( nhStream s, const float* matrix, float* result, int height, int width, const float* vector, int* rc );
+// The same for a convolution ( plain or channelwise, its descriptor checked by the caller ) and the VectorReLU over its
+// result in place that follows it in most networks.
+bool deferConvolution( nhStream s, bool channelwise, const nhConvDesc& d, const float* source, const float* filter,
+	const float* freeTerm, float* result );
+bool fusePendingConvolution( nhStream s, const float* first, float* result, long long count, const float* upperThreshold, int* rc );
 
 inline hipStream_t toStream( nhStream s )
 {
@@ -159,7 +164,19 @@ __device__ __forceinline__ int xcdSwizzle( int bid, int total )
 struct CFusedActivation {
 	int Type;    // NH_ACT_*
 	float Param; // upper threshold of NH_ACT_RELU when above zero
+	// where the threshold lives in device memory instead ( the engine's VectorReLU takes it there ): a kernel that is
+	// handed one reads it once, through withParam, before it looks at Param
+	const float* ParamPtr;
 };
+
+__device__ __forceinline__ CFusedActivation withParam( CFusedActivation a )
+{
+	if( a.ParamPtr != nullptr ) {
+		a.Param = *a.ParamPtr;
+		a.ParamPtr = nullptr;
+	}
+	return a;
+}
 
 __device__ __forceinline__ float applyActivation( float v, const CFusedActivation& a )
 {

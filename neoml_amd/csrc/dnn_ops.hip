@@ -13,6 +13,11 @@
 namespace nh {
 
 // matrix products defined in gemm_mfma.hip
+struct CSliceMeeting;
+int convImplicitGemm( hipStream_t stream, const nhConvDesc& d, const float* source, const float* filter,
+	const float* freeTerm, float* result, const CFusedActivation& act, const CSliceMeeting* fixedMeeting );
+int launchDeferredConvolution( hipStream_t stream, bool channelwise, const nhConvDesc& d, const float* source, const float* filter,
+	const float* freeTerm, float* result, const CFusedActivation& act );
 int matMulNT( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
 	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC,
 	const float* bias, bool accumulate );
@@ -53,8 +58,9 @@ template<> struct CChanVec<1> {
 template<int VECW, int WPT>
 __global__ __launch_bounds__( 256 )
 void channelwiseConvKernel( const nhConvDesc d, const float* source, const float* filter, const float* freeTerm,
-	float* result, int wGroups, long long totalItems, const CFusedActivation act )
+	float* result, int wGroups, long long totalItems, const CFusedActivation actAsGiven )
 {
+	const CFusedActivation act = withParam( actAsGiven );
 	typedef CChanVec<VECW> V;
 	typedef typename V::Type T;
 	const int cg = d.channels / VECW;
@@ -125,9 +131,10 @@ void channelwiseConvKernel( const nhConvDesc d, const float* source, const float
 template<int STRIDE, int WPT, int PRE, bool STREAM, int ACT>
 __global__ __launch_bounds__( 256 )
 void channelwiseConv3x3Kernel( const nhConvDesc d, const float* source, const float* filter, const float* freeTerm,
-	float* result, int wGroups, int rowChunks, int rowsPerItem, int totalItems, const CFusedActivation act, int flipTaps,
+	float* result, int wGroups, int rowChunks, int rowsPerItem, int totalItems, const CFusedActivation actAsGiven, int flipTaps,
 	unsigned resultBytes )
 {
+	const CFusedActivation act = withParam( actAsGiven );
 	constexpr int NC = ( WPT - 1 ) * STRIDE + 3;
 	constexpr int Ring = 3 + PRE * STRIDE;
 	const int item = xcdSwizzle( blockIdx.x, gridDim.x ) * blockDim.x + threadIdx.x;
@@ -1876,8 +1883,9 @@ void channelwiseConvLearnKernel( const nhConvDesc d, const float* input, const f
 template<int VECW>
 __global__ __launch_bounds__( 256 )
 void scaleChannelsKernel( const float* in, const float* scale, float* out, int pixelsPerImage, int channels, long long totalItems,
-	const CFusedActivation act )
+	const CFusedActivation actAsGiven )
 {
+	const CFusedActivation act = withParam( actAsGiven );
 	typedef CChanVec<VECW> V;
 	const int cg = channels / VECW;
 	const long long perImage = static_cast<long long>( pixelsPerImage ) * cg;
@@ -2953,6 +2961,16 @@ static int channelwiseConvolution( nhStream s, const nhConvDesc* d, const float*
 int nhBlobChannelwiseConvolution( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
 	const float* freeTerm, float* result )
 {
+	// ( on a stream that puts calls aside the convolution waits for the call behind it: a ReLU over its result in place
+	// goes into the same launch )
+	if( d != nullptr && source != nullptr && filter != nullptr && result != nullptr ) {
+		nhConvDesc check = *d;
+		if( nhInitBlobChannelwiseConvolution( &check ) == NH_OK && check.resultHeight == d->resultHeight && check.resultWidth == d->resultWidth
+			&& deferConvolution( s, true, check, source, filter, freeTerm, result ) )
+		{
+			return NH_OK;
+		}
+	}
 	const CFusedActivation none = { NH_ACT_NONE, 0.f };
 	return channelwiseConvolution( s, d, source, filter, freeTerm, result, none );
 }
@@ -2996,6 +3014,20 @@ static int channelwiseConvolution( nhStream s, const nhConvDesc* d, const float*
 	NH_LAUNCH_CHECK();
 	return NH_OK;
 }
+
+} // extern "C"
+
+// a convolution that waited for its successor ( vector_ops.hip ), with the activation the successor turned out to be
+int nh::launchDeferredConvolution( hipStream_t stream, bool channelwise, const nhConvDesc& d, const float* source, const float* filter,
+	const float* freeTerm, float* result, const CFusedActivation& act )
+{
+	if( channelwise ) {
+		return channelwiseConvolution( reinterpret_cast<nhStream>( stream ), &d, source, filter, freeTerm, result, act );
+	}
+	return convImplicitGemm( stream, d, source, filter, freeTerm, result, act, nullptr );
+}
+
+extern "C" {
 
 int nhInitPooling( nhPoolingDesc* d )
 {

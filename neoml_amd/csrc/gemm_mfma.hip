@@ -958,7 +958,8 @@ void matMulKernel( const CMatMulArgs launchArgs )
 	if constexpr( !IsClasses && BMODE != BM_ConvN ) {
 		if( args.CBytes != 0 && splitK == 1 && !args.Accumulate && args.Residual == nullptr ) {
 			const __amdgpu_buffer_rsrc_t bufC = __builtin_amdgcn_make_buffer_rsrc( C, 0, args.CBytes, 0x00020000 );
-			const float reluTop = args.Act.Param > 0.f ? args.Act.Param : __builtin_inff();
+			const float actParam = withParam( args.Act ).Param; // ( the threshold may live in device memory )
+			const float reluTop = actParam > 0.f ? actParam : __builtin_inff();
 			const unsigned pitchBytes = static_cast<unsigned>( args.Ldc ) * 4u;
 			const bool inside = m0 + BM <= M;
 			auto store = [&]( auto typeOf, auto insideOf ) {
@@ -1020,7 +1021,8 @@ void matMulKernel( const CMatMulArgs launchArgs )
 			n = kh * args.RowK + r;
 		}
 		const float bias = ( args.Bias != nullptr ) ? args.Bias[n] : 0.f;
-		const float reluTop = args.Act.Param > 0.f ? args.Act.Param : __builtin_inff();
+		const float actParam = withParam( args.Act ).Param; // ( the threshold may live in device memory )
+			const float reluTop = actParam > 0.f ? actParam : __builtin_inff();
 		// Mode: 0 adds onto C with atomics ( K slices that meet in C: it was set to the free term, or left as it was when
 		// accumulating, before the launch ), 1 stores act( acc + bias ), 2 also accumulates and / or adds the residual.
 		// What is the same for the whole tile is decided once per tile, not per element: with up to eight wavefronts per SIMD
@@ -1320,8 +1322,9 @@ __global__ __launch_bounds__( 256 ) void presetResultKernel( float* c, const flo
 }
 
 // C[b][m][n] = act( C[b][m][n] ): the activation pass behind a launch that met in C through K slices
-__global__ __launch_bounds__( 256 ) void activateResultKernel( float* c, int M, int N, int ldc, long long batchStride, const CFusedActivation act )
+__global__ __launch_bounds__( 256 ) void activateResultKernel( float* c, int M, int N, int ldc, long long batchStride, const CFusedActivation actAsGiven )
 {
+	const CFusedActivation act = withParam( actAsGiven );
 	const long long total = static_cast<long long>( M ) * N;
 	float* base = c + blockIdx.y * batchStride;
 	for( long long i = blockIdx.x * 256LL + threadIdx.x; i < total; i += static_cast<long long>( gridDim.x ) * 256 ) {
@@ -1653,8 +1656,9 @@ struct CRunState {
 template<int KC, int NB, bool RES, int RP>
 __global__ __launch_bounds__( Threads, 2 )
 void shortReductionKernel( const float* A, const float* W, const float* bias, float* C, int M, int N, int rowBlocks,
-	const CFusedActivation act, const float* residual, const CRowRuns geo )
+	const CFusedActivation actAsGiven, const float* residual, const CRowRuns geo )
 {
+	const CFusedActivation act = withParam( actAsGiven );
 	constexpr int K = KC * 8;
 	constexpr int Pitch = K + 4;
 	constexpr int PatchPitch = 36;
@@ -2330,7 +2334,8 @@ void longProductKernel( const CLongProductArgs args )
 	// lane ( l32, half ) holds, of each block, one column of rows ( r / 4 ) * 8 + half * 4 + r % 4
 	float* C = args.C + batch * args.BatchStrideC;
 	const float* residual = args.Residual != nullptr ? args.Residual + batch * args.BatchStrideC : nullptr;
-	const float reluTop = args.Act.Param > 0.f ? args.Act.Param : __builtin_inff();
+	const float actParam = withParam( args.Act ).Param; // ( the threshold may live in device memory )
+			const float reluTop = actParam > 0.f ? actParam : __builtin_inff();
 	const bool accumulate = args.Accumulate != 0;
 	const int rowBase = m0 + waveM * 32 * MI + half * 4;
 	// what is the same for the whole tile is decided once, here, and not per element: 32 or 64 elements per lane and up
@@ -3518,6 +3523,13 @@ int nhBlobConvolutionLearnAdd( nhStream s, const nhConvDesc* d, const float* inp
 int nhBlobConvolution( nhStream s, const nhConvDesc* d, const float* source, const float* filter,
 	const float* freeTerm, float* result )
 {
+	// ( on a stream that puts calls aside the convolution waits for the call behind it: a ReLU over its result in place
+	// goes into the same launch )
+	if( d != nullptr && source != nullptr && filter != nullptr && result != nullptr && checkedConvDesc( d ) == NH_OK
+		&& deferConvolution( s, false, *d, source, filter, freeTerm, result ) )
+	{
+		return NH_OK;
+	}
 	return nhBlobConvolutionWithActivation( s, d, source, filter, freeTerm, NH_ACT_NONE, 0.f, result );
 }
 

@@ -613,11 +613,29 @@ struct CPendingProduct {
 	int Lda = 0, Ldb = 0, Ldc = 0, M = 0, N = 0, K = 0;
 };
 
+// A convolution ( plain or channelwise ) that waits for the call behind it in the same way: CConvLayer / CChannelwiseConvLayer
+// are followed by CReLULayer in most networks, a pass over the whole result in place that the convolution's kernels do on
+// the accumulators' way out ( nhBlobConvolutionWithActivation ). VectorReLU over the convolution's result in place makes
+// the two one launch, the threshold read from where the engine keeps it in device memory.
+struct CPendingConvolution {
+	bool Pending = false;
+	bool Channelwise = false;
+	nhConvDesc Desc = {};
+	const float* Source = nullptr;
+	const float* Filter = nullptr;
+	const float* FreeTerm = nullptr;
+	float* Result = nullptr;
+};
+
 struct CTinyQueue {
 	bool Enabled = false;
 	CTinyChain Chain = {};
 	CPendingProduct Product;
+	CPendingConvolution Convolution;
 };
+
+int launchDeferredConvolution( hipStream_t stream, bool channelwise, const nhConvDesc& d, const float* source, const float* filter,
+	const float* freeTerm, float* result, const CFusedActivation& act );
 
 int matMulNT( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
 	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC, const float* bias, bool accumulate );
@@ -669,6 +687,14 @@ static bool launchPending( hipStream_t stream, CTinyQueue& queue )
 		( void )matMulNT( stream, p.A, p.Lda, p.B, p.Ldb, p.C, p.Ldc, p.M, p.N, p.K, 1, 0, 0, 0, nullptr, false );
 		return true;
 	}
+	if( queue.Convolution.Pending ) {
+		const CPendingConvolution c = queue.Convolution;
+		queue.Convolution.Pending = false;
+		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+		const CFusedActivation none = { NH_ACT_NONE, 0.f };
+		( void )launchDeferredConvolution( stream, c.Channelwise, c.Desc, c.Source, c.Filter, c.FreeTerm, c.Result, none );
+		return true;
+	}
 	return launchTinyChain( stream, queue.Chain );
 }
 
@@ -700,7 +726,7 @@ void flushAllTinyOps()
 	{
 		std::lock_guard<std::recursive_mutex> guard( tinyLock );
 		for( auto& entry : tinyQueues() ) {
-			if( entry.second.Chain.Length == 0 && !entry.second.Product.Pending ) {
+			if( entry.second.Chain.Length == 0 && !entry.second.Product.Pending && !entry.second.Convolution.Pending ) {
 				continue;
 			}
 			if( entry.first.first != active ) {
@@ -768,7 +794,9 @@ bool deferProduct( nhStream s, const float* a, int lda, const float* b, int ldb,
 	}
 	std::lock_guard<std::recursive_mutex> guard( tinyLock );
 	auto found = tinyQueues().find( std::make_pair( device, stream ) );
-	if( found == tinyQueues().end() || !found->second.Enabled || found->second.Chain.Length != 0 || found->second.Product.Pending ) {
+	if( found == tinyQueues().end() || !found->second.Enabled || found->second.Chain.Length != 0 || found->second.Product.Pending
+		|| found->second.Convolution.Pending )
+	{
 		return false;
 	}
 	CPendingProduct& p = found->second.Product;
@@ -801,6 +829,69 @@ bool fusePendingProduct( nhStream s, const float* matrix, float* result, int hei
 		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
 	}
 	*rc = matMulNT( stream, p.A, p.Lda, p.B, p.Ldb, p.C, p.Ldc, p.M, p.N, p.K, 1, 0, 0, 0, vector, false );
+	if( __atomic_load_n( &lstmPartnersAwaited, __ATOMIC_RELAXED ) != 0 ) {
+		noteStreamUse( stream );
+	}
+	return true;
+}
+
+bool deferConvolution( nhStream s, bool channelwise, const nhConvDesc& d, const float* source, const float* filter,
+	const float* freeTerm, float* result )
+{
+	if( __atomic_load_n( &tinyDeferringStreams, __ATOMIC_RELAXED ) == 0 || d.batch <= 0 ) {
+		return false;
+	}
+	const hipStream_t stream = toStream( s ); // ( what the stream holds goes out first )
+	int device = 0;
+	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+	if( hipGetDevice( &device ) != hipSuccess || hipStreamIsCapturing( stream, &capture ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return false;
+	}
+	if( capture != hipStreamCaptureStatusNone ) {
+		return false;
+	}
+	std::lock_guard<std::recursive_mutex> guard( tinyLock );
+	auto found = tinyQueues().find( std::make_pair( device, stream ) );
+	if( found == tinyQueues().end() || !found->second.Enabled || found->second.Chain.Length != 0 || found->second.Product.Pending
+		|| found->second.Convolution.Pending )
+	{
+		return false;
+	}
+	CPendingConvolution& c = found->second.Convolution;
+	c.Pending = true;
+	c.Channelwise = channelwise;
+	c.Desc = d;
+	c.Source = source; c.Filter = filter; c.FreeTerm = freeTerm; c.Result = result;
+	__atomic_fetch_add( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+	return true;
+}
+
+bool fusePendingConvolution( nhStream s, const float* first, float* result, long long count, const float* upperThreshold, int* rc )
+{
+	const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
+	int device = 0;
+	if( hipGetDevice( &device ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return false;
+	}
+	CPendingConvolution c;
+	{
+		std::lock_guard<std::recursive_mutex> guard( tinyLock );
+		auto found = tinyQueues().find( std::make_pair( device, stream ) );
+		if( found == tinyQueues().end() || !found->second.Convolution.Pending ) {
+			return false;
+		}
+		c = found->second.Convolution;
+		const long long resultCount = static_cast<long long>( c.Desc.batch ) * c.Desc.resultHeight * c.Desc.resultWidth * c.Desc.filterCount;
+		if( first != c.Result || result != c.Result || count != resultCount || upperThreshold == nullptr ) {
+			return false; // ( the caller's own launch sends the convolution out first, as it was asked for )
+		}
+		found->second.Convolution.Pending = false;
+		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+	}
+	const CFusedActivation relu = { NH_ACT_RELU, 0.f, upperThreshold };
+	*rc = launchDeferredConvolution( stream, c.Channelwise, c.Desc, c.Source, c.Filter, c.FreeTerm, c.Result, relu );
 	if( __atomic_load_n( &lstmPartnersAwaited, __ATOMIC_RELAXED ) != 0 ) {
 		noteStreamUse( stream );
 	}
@@ -850,8 +941,8 @@ static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 		if( found == tinyQueues().end() || !found->second.Enabled ) {
 			return false;
 		}
-		if( found->second.Product.Pending ) {
-			launchPending( stream, found->second ); // ( a product that waited for its successor: this call is not the one )
+		if( found->second.Product.Pending || found->second.Convolution.Pending ) {
+			launchPending( stream, found->second ); // ( a launch that waited for its successor: this call is not the one )
 		}
 		CTinyChain& chain = found->second.Chain;
 		if( chain.Length == TinyChainMax ) {
@@ -1159,6 +1250,12 @@ extern "C" int nhVectorConvertIntToFloat( nhStream s, const int* from, float* to
 extern "C" int nhVectorReLU( nhStream s, const float* first, float* result, int vectorSize, const float* upperThreshold )
 {
 	NH_REQUIRE( upperThreshold != nullptr );
+	int rc = NH_OK;
+	if( first == result && __atomic_load_n( &tinyChainsPending, __ATOMIC_RELAXED ) != 0
+		&& fusePendingConvolution( s, first, result, vectorSize, upperThreshold, &rc ) )
+	{
+		return rc; // ( the convolution that waited for this call took the activation with it )
+	}
 	CReLUOp op; op.Ptr = upperThreshold; op.Threshold = 0;
 	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
 }

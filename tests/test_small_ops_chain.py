@@ -335,3 +335,88 @@ def test_product_waits_for_its_free_term(streams):
     na.check(lib.nhRawFree(block))
     torch.cuda.synchronize()
     assert_close(c.cpu().numpy(), (a.astype(np.float64) @ w.astype(np.float64).T).astype(np.float32), "launched by nhRawFree", atol=2e-5)
+
+
+def test_convolution_waits_for_its_relu(streams):
+    """A convolution (plain or channelwise) is put aside as well, and a VectorReLU over its result in place goes into its
+    launch, the threshold read from device memory: the same bits as the two launches, whatever kernel the shape takes
+    (tap-step and tiled products, the short-reduction and window kernels, K slices that meet in scratch memory, the
+    depthwise strips). Other successors find the convolution done."""
+    import torch
+    import neoml_amd
+    lib, na = streams.lib, streams.na
+    g = rng(4400)
+    dev = streams.dev
+    P = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    six, zero = up(np.array([6.0], np.float32)), up(np.array([0.0], np.float32))
+    cases = [
+        # n, h, w, cin, cout, f, pad, stride
+        (4, 56, 56, 64, 64, 3, 1, 1), (4, 28, 28, 128, 128, 3, 1, 1), (8, 14, 14, 256, 512, 3, 1, 1), (2, 56, 56, 64, 128, 1, 0, 2),
+        (4, 64, 64, 3, 64, 7, 3, 2), (8, 56, 56, 24, 144, 1, 0, 1), (2, 9, 11, 5, 6, 3, 1, 1), (16, 32, 96, 1, 64, 3, 1, 1),
+    ]
+    for n, h, w, cin, cout, f, pad, stride in cases:
+        x = g.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+        filt = g.normal(0, 1.0 / np.sqrt(f * f * cin), (cout, f, f, cin)).astype(np.float32)
+        bias = g.uniform(-0.5, 0.5, cout).astype(np.float32)
+        d = neoml_amd.ConvDesc(n, h, w, cin, cout, f, f, pad, pad, stride, stride, 1, 1, 0, 0)
+        na.check(lib.nhInitBlobConvolution(ctypes.byref(d)))
+        d_x, d_f, d_b = up(x), up(filt), up(bias)
+        shape = (n, d.resultHeight, d.resultWidth, cout)
+        for threshold in (zero, six):
+            outs = []
+            for stream in (streams.plain, streams.deferring):
+                y = torch.zeros(shape, device=dev)
+                torch.cuda.synchronize()
+                na.check(lib.nhBlobConvolution(stream, ctypes.byref(d), P(d_x), P(d_f), P(d_b), P(y)))
+                na.check(lib.nhVectorReLU(stream, P(y), P(y), y.numel(), P(threshold)))
+                na.check(lib.nhStreamSynchronize(stream))
+                outs.append(y.cpu().numpy())
+            assert same_bits(outs[0], outs[1]), (n, h, w, cin, cout, f, pad, stride, float(threshold[0]))
+            assert outs[1].min() >= 0.0 and (float(threshold[0]) == 0.0 or outs[1].max() <= 6.0)
+    for n, h, w, c, stride in ((8, 56, 56, 144, 1), (8, 112, 112, 96, 2), (3, 9, 7, 6, 1)):
+        x = g.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+        filt = g.normal(0, 1.0 / 3, (3, 3, c)).astype(np.float32)
+        bias = g.uniform(-0.5, 0.5, c).astype(np.float32)
+        d = neoml_amd.ConvDesc(n, h, w, c, 0, 3, 3, 1, 1, stride, stride, 0, 0, 0, 0)
+        na.check(lib.nhInitBlobChannelwiseConvolution(ctypes.byref(d)))
+        d_x, d_f, d_b = up(x), up(filt), up(bias)
+        outs = []
+        for stream in (streams.plain, streams.deferring):
+            y = torch.zeros((n, d.resultHeight, d.resultWidth, c), device=dev)
+            torch.cuda.synchronize()
+            na.check(lib.nhBlobChannelwiseConvolution(stream, ctypes.byref(d), P(d_x), P(d_f), P(d_b), P(y)))
+            na.check(lib.nhVectorReLU(stream, P(y), P(y), y.numel(), P(six)))
+            na.check(lib.nhStreamSynchronize(stream))
+            outs.append(y.cpu().numpy())
+        assert same_bits(outs[0], outs[1]), ("channelwise", n, h, w, c, stride)
+    # other successors
+    n, h, w, cin, cout = 4, 28, 28, 32, 64
+    x = g.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    filt = g.normal(0, 1.0 / np.sqrt(9 * cin), (cout, 3, 3, cin)).astype(np.float32)
+    d = neoml_amd.ConvDesc(n, h, w, cin, cout, 3, 3, 1, 1, 1, 1, 1, 1, 0, 0)
+    na.check(lib.nhInitBlobConvolution(ctypes.byref(d)))
+    d_x, d_f = up(x), up(filt)
+    count = n * h * w * cout
+
+    def run(stream, successor):
+        y = torch.zeros((n, h, w, cout), device=dev)
+        other = torch.zeros((n, h, w, cout), device=dev)
+        torch.cuda.synchronize()
+        na.check(lib.nhBlobConvolution(stream, ctypes.byref(d), P(d_x), P(d_f), None, P(y)))
+        successor(stream, y, other)
+        na.check(lib.nhStreamSynchronize(stream))
+        return y.cpu().numpy(), other.cpu().numpy()
+
+    successors = {
+        "nothing but the wait": lambda s, y, o: None,
+        "ReLU into another blob": lambda s, y, o: na.check(lib.nhVectorReLU(s, P(y), P(o), count, P(zero))),
+        "ReLU over a part": lambda s, y, o: na.check(lib.nhVectorReLU(s, P(y), P(y), count // 2, P(zero))),
+        "another activation in place": lambda s, y, o: na.check(lib.nhVectorAbs(s, P(y), P(y), count)),
+        "a small call on the result": lambda s, y, o: na.check(lib.nhVectorNeg(s, P(y), P(o), 1000)),
+        "a second convolution": lambda s, y, o: na.check(lib.nhBlobConvolution(s, ctypes.byref(d), P(d_x), P(d_f), None, P(o))),
+    }
+    for what, successor in successors.items():
+        want_y, want_o = run(streams.plain, successor)
+        got_y, got_o = run(streams.deferring, successor)
+        assert same_bits(got_y, want_y) and same_bits(got_o, want_o), what
