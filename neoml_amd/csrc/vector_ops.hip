@@ -194,6 +194,20 @@ struct CReLUOp {
 		return r;
 	}
 };
+// ReLU of a sum: an element-wise sum whose launch waited for the ReLU behind it ( see CPendingSum )
+struct CAddReLUOp {
+	const float* Ptr; float Threshold;
+	__device__ void prepare() { Threshold = *Ptr; }
+	__device__ float operator()( float a, float b, float ) const
+	{
+		const float sum = a + b;
+		float r = sum > 0.f ? sum : 0.f;
+		if( Threshold > 0.f ) {
+			r = r < Threshold ? r : Threshold;
+		}
+		return r;
+	}
+};
 struct CELUOp {
 	const float* Ptr; float Alpha;
 	__device__ void prepare() { Alpha = *Ptr; }
@@ -627,12 +641,27 @@ struct CPendingConvolution {
 	float* Result = nullptr;
 };
 
+// The sum of two large vectors ( the junction of a residual block, CEltwiseSumLayer ) followed by CReLULayer in place:
+// one pass instead of two.
+struct CPendingSum {
+	bool Pending = false;
+	const float* First = nullptr;
+	const float* Second = nullptr;
+	float* Result = nullptr;
+	int Count = 0;
+};
+
 struct CTinyQueue {
 	bool Enabled = false;
 	CTinyChain Chain = {};
 	CPendingProduct Product;
 	CPendingConvolution Convolution;
+	CPendingSum Sum;
+
+	bool LaunchWaits() const { return Product.Pending || Convolution.Pending || Sum.Pending; }
 };
+
+static int launchPlainSum( hipStream_t stream, const CPendingSum& sum );
 
 int launchDeferredConvolution( hipStream_t stream, bool channelwise, const nhConvDesc& d, const float* source, const float* filter,
 	const float* freeTerm, float* result, const CFusedActivation& act );
@@ -695,6 +724,13 @@ static bool launchPending( hipStream_t stream, CTinyQueue& queue )
 		( void )launchDeferredConvolution( stream, c.Channelwise, c.Desc, c.Source, c.Filter, c.FreeTerm, c.Result, none );
 		return true;
 	}
+	if( queue.Sum.Pending ) {
+		const CPendingSum sum = queue.Sum;
+		queue.Sum.Pending = false;
+		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+		( void )launchPlainSum( stream, sum );
+		return true;
+	}
 	return launchTinyChain( stream, queue.Chain );
 }
 
@@ -726,7 +762,7 @@ void flushAllTinyOps()
 	{
 		std::lock_guard<std::recursive_mutex> guard( tinyLock );
 		for( auto& entry : tinyQueues() ) {
-			if( entry.second.Chain.Length == 0 && !entry.second.Product.Pending && !entry.second.Convolution.Pending ) {
+			if( entry.second.Chain.Length == 0 && !entry.second.LaunchWaits() ) {
 				continue;
 			}
 			if( entry.first.first != active ) {
@@ -794,8 +830,7 @@ bool deferProduct( nhStream s, const float* a, int lda, const float* b, int ldb,
 	}
 	std::lock_guard<std::recursive_mutex> guard( tinyLock );
 	auto found = tinyQueues().find( std::make_pair( device, stream ) );
-	if( found == tinyQueues().end() || !found->second.Enabled || found->second.Chain.Length != 0 || found->second.Product.Pending
-		|| found->second.Convolution.Pending )
+	if( found == tinyQueues().end() || !found->second.Enabled || found->second.Chain.Length != 0 || found->second.LaunchWaits() )
 	{
 		return false;
 	}
@@ -835,6 +870,67 @@ bool fusePendingProduct( nhStream s, const float* matrix, float* result, int hei
 	return true;
 }
 
+static int launchPlainSum( hipStream_t stream, const CPendingSum& sum )
+{
+	return launchEltwise<2, float, float>( reinterpret_cast<nhStream>( stream ), sum.First, sum.Second, static_cast<const float*>( nullptr ),
+		sum.Result, sum.Count, CAddOp<float>() );
+}
+
+// a sum of two vectors too large for a chain: it waits for the call behind it
+static bool deferSum( nhStream s, const float* first, const float* second, float* result, int count )
+{
+	if( __atomic_load_n( &tinyDeferringStreams, __ATOMIC_RELAXED ) == 0 || first == nullptr || second == nullptr || result == nullptr ) {
+		return false;
+	}
+	const hipStream_t stream = toStream( s ); // ( what the stream holds goes out first )
+	int device = 0;
+	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+	if( hipGetDevice( &device ) != hipSuccess || hipStreamIsCapturing( stream, &capture ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return false;
+	}
+	if( capture != hipStreamCaptureStatusNone ) {
+		return false;
+	}
+	std::lock_guard<std::recursive_mutex> guard( tinyLock );
+	auto found = tinyQueues().find( std::make_pair( device, stream ) );
+	if( found == tinyQueues().end() || !found->second.Enabled || found->second.Chain.Length != 0 || found->second.LaunchWaits() ) {
+		return false;
+	}
+	CPendingSum& sum = found->second.Sum;
+	sum.Pending = true;
+	sum.First = first; sum.Second = second; sum.Result = result; sum.Count = count;
+	__atomic_fetch_add( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+	return true;
+}
+
+static bool fusePendingSum( nhStream s, const float* first, float* result, int count, const float* upperThreshold, int* rc )
+{
+	const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
+	int device = 0;
+	if( hipGetDevice( &device ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return false;
+	}
+	CPendingSum sum;
+	{
+		std::lock_guard<std::recursive_mutex> guard( tinyLock );
+		auto found = tinyQueues().find( std::make_pair( device, stream ) );
+		if( found == tinyQueues().end() || !found->second.Sum.Pending ) {
+			return false;
+		}
+		sum = found->second.Sum;
+		if( first != sum.Result || result != sum.Result || count != sum.Count ) {
+			return false; // ( the caller's own launch sends the sum out first, as it was asked for )
+		}
+		found->second.Sum.Pending = false;
+		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+	}
+	CAddReLUOp op; op.Ptr = upperThreshold; op.Threshold = 0;
+	*rc = launchEltwise<2, float, float>( s, sum.First, sum.Second, static_cast<const float*>( nullptr ), sum.Result, sum.Count, op );
+	return true;
+}
+
 bool deferConvolution( nhStream s, bool channelwise, const nhConvDesc& d, const float* source, const float* filter,
 	const float* freeTerm, float* result )
 {
@@ -853,8 +949,7 @@ bool deferConvolution( nhStream s, bool channelwise, const nhConvDesc& d, const 
 	}
 	std::lock_guard<std::recursive_mutex> guard( tinyLock );
 	auto found = tinyQueues().find( std::make_pair( device, stream ) );
-	if( found == tinyQueues().end() || !found->second.Enabled || found->second.Chain.Length != 0 || found->second.Product.Pending
-		|| found->second.Convolution.Pending )
+	if( found == tinyQueues().end() || !found->second.Enabled || found->second.Chain.Length != 0 || found->second.LaunchWaits() )
 	{
 		return false;
 	}
@@ -941,7 +1036,7 @@ static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 		if( found == tinyQueues().end() || !found->second.Enabled ) {
 			return false;
 		}
-		if( found->second.Product.Pending || found->second.Convolution.Pending ) {
+		if( found->second.LaunchWaits() ) {
 			launchPending( stream, found->second ); // ( a launch that waited for its successor: this call is not the one )
 		}
 		CTinyChain& chain = found->second.Chain;
@@ -1252,9 +1347,10 @@ extern "C" int nhVectorReLU( nhStream s, const float* first, float* result, int 
 	NH_REQUIRE( upperThreshold != nullptr );
 	int rc = NH_OK;
 	if( first == result && __atomic_load_n( &tinyChainsPending, __ATOMIC_RELAXED ) != 0
-		&& fusePendingConvolution( s, first, result, vectorSize, upperThreshold, &rc ) )
+		&& ( fusePendingConvolution( s, first, result, vectorSize, upperThreshold, &rc )
+			|| fusePendingSum( s, first, result, vectorSize, upperThreshold, &rc ) ) )
 	{
-		return rc; // ( the convolution that waited for this call took the activation with it )
+		return rc; // ( the convolution or the sum that waited for this call took the activation with it )
 	}
 	CReLUOp op; op.Ptr = upperThreshold; op.Threshold = 0;
 	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
@@ -1362,7 +1458,14 @@ extern "C" int nhVectorL1DiffAdd( nhStream s, const float* first, const float* s
 
 NH_BINARY( nhVectorEltwiseMax, float, CMaxOp )
 NH_BINARY( nhVectorEltwiseMin, float, CMinOp )
-NH_BINARY( nhVectorAdd, float, CAddOp<float> )
+extern "C" int nhVectorAdd( nhStream s, const float* first, const float* second, float* result, int vectorSize )
+{
+	// ( on a stream that puts calls aside a large sum waits for the call behind it: a ReLU over it in place is the same pass )
+	if( vectorSize > TinyWideMaxCount && deferSum( s, first, second, result, vectorSize ) ) {
+		return NH_OK;
+	}
+	return launchEltwise<2, float, float>( s, first, second, (const float*)nullptr, result, vectorSize, CAddOp<float>() );
+}
 NH_BINARY( nhVectorAddInt, int, CAddOp<int> )
 NH_BINARY( nhVectorSub, float, CSubOp<float> )
 NH_BINARY( nhVectorSubInt, int, CSubOp<int> )

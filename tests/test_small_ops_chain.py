@@ -420,3 +420,47 @@ def test_convolution_waits_for_its_relu(streams):
         want_y, want_o = run(streams.plain, successor)
         got_y, got_o = run(streams.deferring, successor)
         assert same_bits(got_y, want_y) and same_bits(got_o, want_o), what
+
+
+def test_large_sum_waits_for_its_relu(streams):
+    """VectorAdd over more elements than a chain takes waits for the call behind it too: a VectorReLU over the sum in place
+    (CEltwiseSumLayer + CReLULayer at the end of a residual block) is the same pass. Same bits; other successors find
+    the sum done."""
+    import torch
+    lib, na = streams.lib, streams.na
+    g = rng(4500)
+    dev = streams.dev
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    n = 3 * 1000 * 1000 + 7
+    a, b = g.normal(0, 3, n).astype(np.float32), g.normal(0, 3, n).astype(np.float32)
+    a[5], b[5] = np.nan, 1.0  # NaN becomes 0, as in VectorReLU
+    zero, six = up(np.zeros(1, np.float32)), up(np.array([6.0], np.float32))
+
+    def run(stream, in_place, successor):
+        d_a, d_b = up(a), up(b)
+        out = d_a if in_place else torch.zeros(n, device=dev)
+        other = torch.zeros(n, device=dev)
+        torch.cuda.synchronize()
+        na.check(lib.nhVectorAdd(stream, P(d_a), P(d_b), P(out), n))
+        successor(stream, out, other)
+        na.check(lib.nhStreamSynchronize(stream))
+        return out.cpu().numpy(), other.cpu().numpy()
+
+    successors = {
+        "ReLU in place": lambda s, y, o: na.check(lib.nhVectorReLU(s, P(y), P(y), n, P(zero))),
+        "ReLU6 in place": lambda s, y, o: na.check(lib.nhVectorReLU(s, P(y), P(y), n, P(six))),
+        "nothing but the wait": lambda s, y, o: None,
+        "ReLU into another vector": lambda s, y, o: na.check(lib.nhVectorReLU(s, P(y), P(o), n, P(zero))),
+        "ReLU over a part": lambda s, y, o: na.check(lib.nhVectorReLU(s, P(y), P(y), n - 8, P(zero))),
+        "a second sum": lambda s, y, o: na.check(lib.nhVectorAdd(s, P(y), P(y), P(o), n)),
+        "a small call": lambda s, y, o: na.check(lib.nhVectorNeg(s, P(y), P(o), 100)),
+    }
+    for in_place in (False, True):
+        for what, successor in successors.items():
+            want = run(streams.plain, in_place, successor)
+            got = run(streams.deferring, in_place, successor)
+            assert same_bits(got[0], want[0]) and same_bits(got[1], want[1]), (what, in_place)
+    y, _ = run(streams.deferring, False, successors["ReLU6 in place"])
+    assert y[5] == 0.0 and y.min() >= 0.0 and y.max() <= 6.0
+    assert np.array_equal(np.delete(y, 5), np.clip(np.delete(a + b, 5), 0.0, 6.0))

@@ -413,8 +413,8 @@ class LaunchPlan:
                 tag, j, flops, nbytes = launches[i][2], i, 0, 0
                 while j < len(launches) and launches[j][2] == tag:
                     flops, nbytes, j = flops + launches[j][3], nbytes + launches[j][4], j + 1
-                if tag and (tag.startswith("conv") or tag == "depthwise") and j == i + 1 and j < len(launches) and launches[j][2] == "relu":
-                    # the activation in place behind a convolution: on such a stream it is the convolution's own launch
+                if tag and (tag.startswith("conv") or tag in ("depthwise", "add")) and j < len(launches) and launches[j][2] == "relu":
+                    # the activation in place behind a convolution or a sum: on such a stream it is that call's own launch
                     flops, nbytes, j = flops + launches[j][3], nbytes + launches[j][4], j + 1
                 if pool[i] is not None:
                     record(pool[i][0], stream)
