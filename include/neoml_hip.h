@@ -433,10 +433,13 @@ NH_API int nhBlobMeanPoolingBackward(nhStream s, const nhPoolingDesc* desc_host,
 NH_API int nhStreamOverlapLstm(nhStream s, int enable);
 
 /* Several small element-wise calls in one launch. No counterpart in the reference: there every call runs at once on the
- * calling thread. On a stream that has asked for it (enable != 0) a float element-wise call over at most 262144 elements
- * (fill, copy, add, sub, multiply, divide, negate, abs, max, min, sqrt, inv, and the forms with a device scalar: add value,
- * multiply, neg-multiply, multiply-and-add, multiply-and-sub, eltwise multiply-add, eltwise neg-multiply) is put aside;
- * up to eight of them are launched together, in call order and with bit-identical results, as soon as ANY other call
+ * calling thread. On a stream that has asked for it (enable != 0) a float element-wise call
+ * (fill, copy, add, sub, multiply, divide, negate, abs, max, min, sqrt, inv, ReLU, sigmoid, tanh, h-swish, and the forms
+ * with a device scalar: add value, multiply, neg-multiply, multiply-and-add, multiply-and-sub, eltwise multiply-add,
+ * eltwise neg-multiply) is put aside: calls over at most 262144 elements together whatever their counts, a call over more
+ * elements only with calls of its own count (the passes of an activation layer or of a solver over one blob: the three
+ * calls of CGELULayer's sigmoid form become one pass; a large call that no other joins goes out as the launch it
+ * always was). Up to eight of them are launched together, in call order and with bit-identical results, as soon as ANY other call
  * on the stream through this library arrives: a larger or different operation, a copy, an event, nhStreamSynchronize,
  * nhStreamDestroy, enable = 0, or a release of device memory (nhRawFree, a pool's clean-up). Until then their results are
  * not in memory and their operands must stay valid, so this is only for streams whose work, synchronisation included,
@@ -449,7 +452,12 @@ NH_API int nhStreamOverlapLstm(nhStream s, int enable);
  * then part of the product's launch, the vector added to the accumulators on their way out, as the fully connected
  * layer's two calls ask (NeoML/src/Dnn/Layers/FullyConnectedLayer.cpp:91-99); any other call launches the product first,
  * as it was asked for. The sum is the same; where the product is cut into slices of its reduction the vector is added
- * in front of the slices instead of behind them, i.e. the last bits may differ from the two launches'. */
+ * in front of the slices instead of behind them, i.e. the last bits may differ from the two launches'.
+ * In the same way nhBlobConvolution and nhBlobChannelwiseConvolution wait for an nhVectorReLU over their result in place
+ * (CConvLayer / CChannelwiseConvLayer followed by CReLULayer: the activation runs on the accumulators' way out, its
+ * threshold read from the device scalar), and an nhVectorAdd over more than 262144 elements waits for an nhVectorReLU
+ * over the sum in place (CEltwiseSumLayer + CReLULayer at the end of a residual block: one pass). Same bits as the two
+ * launches. */
 NH_API int nhStreamDeferSmallOps(nhStream s, int enable);
 /* LSTM (NME.h:1005-1011). Weights: inputWeights [4H x objectSize], recurrentWeights [4H x H]; gate order in
  * the 4H vector: main(tanh) | forget | input | output (src/CPU/CpuMathEngineDnnLstm.h:49-90).

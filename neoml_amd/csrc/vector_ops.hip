@@ -113,6 +113,9 @@ template<int NIN, typename TIn, typename TOut, typename F>
 static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, const F& f );
 
 template<int NIN, typename TIn, typename TOut, typename F>
+static int launchEltwisePlain( hipStream_t stream, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, F f );
+
+template<int NIN, typename TIn, typename TOut, typename F>
 static int launchEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, F f )
 {
 	if( n < 0 ) {
@@ -129,6 +132,13 @@ static int launchEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 	if( deferEltwise<NIN, TIn, TOut, F>( s, a, b, c, out, n, f ) ) {
 		return NH_OK;
 	}
+	return launchEltwisePlain<NIN, TIn, TOut, F>( toStream( s ), a, b, c, out, n, f );
+}
+
+// the launch of one call on its own ( operands checked by the caller )
+template<int NIN, typename TIn, typename TOut, typename F>
+static int launchEltwisePlain( hipStream_t stream, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, F f )
+{
 	const bool vec = isAligned16( out ) && ( NIN < 1 || isAligned16( a ) ) && ( NIN < 2 || isAligned16( b ) )
 		&& ( NIN < 3 || isAligned16( c ) ) && n >= 4;
 	const int perBlock = EltThreads * EltUnroll * 4;
@@ -138,16 +148,16 @@ static int launchEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 	// mid-sized ones streaming stores cost what streaming loads gain ). Below that the hint only loses cache hits.
 	constexpr int StreamLoadsFrom = 24 << 20, StreamStoresFrom = 100 << 20;
 	if( vec && NIN >= 1 && n >= StreamStoresFrom ) {
-		hipLaunchKernelGGL( ( eltwiseKernel<NIN, TIn, TOut, F, true, 3> ), dim3( blocks ), dim3( EltThreads ), 0, toStream( s ),
+		hipLaunchKernelGGL( ( eltwiseKernel<NIN, TIn, TOut, F, true, 3> ), dim3( blocks ), dim3( EltThreads ), 0, stream,
 			a, b, c, out, n, f );
 	} else if( vec && NIN >= 1 && n >= StreamLoadsFrom ) {
-		hipLaunchKernelGGL( ( eltwiseKernel<NIN, TIn, TOut, F, true, 1> ), dim3( blocks ), dim3( EltThreads ), 0, toStream( s ),
+		hipLaunchKernelGGL( ( eltwiseKernel<NIN, TIn, TOut, F, true, 1> ), dim3( blocks ), dim3( EltThreads ), 0, stream,
 			a, b, c, out, n, f );
 	} else if( vec ) {
-		hipLaunchKernelGGL( ( eltwiseKernel<NIN, TIn, TOut, F, true> ), dim3( blocks ), dim3( EltThreads ), 0, toStream( s ),
+		hipLaunchKernelGGL( ( eltwiseKernel<NIN, TIn, TOut, F, true> ), dim3( blocks ), dim3( EltThreads ), 0, stream,
 			a, b, c, out, n, f );
 	} else {
-		hipLaunchKernelGGL( ( eltwiseKernel<NIN, TIn, TOut, F, false> ), dim3( blocks ), dim3( EltThreads ), 0, toStream( s ),
+		hipLaunchKernelGGL( ( eltwiseKernel<NIN, TIn, TOut, F, false> ), dim3( blocks ), dim3( EltThreads ), 0, stream,
 			a, b, c, out, n, f );
 	}
 	NH_LAUNCH_CHECK();
@@ -259,7 +269,16 @@ template<typename T> struct CMulOp : CNoScalar { __device__ T operator()( T a, T
 struct CDivOp : CNoScalar { __device__ float operator()( float a, float b, float ) const { return a / b; } };
 struct CNegMulOp : CNoScalar { __device__ float operator()( float a, float b, float ) const { return -a * b; } };
 // result += first * second, two roundings like the reference's mul + add
-struct CMulAddOp : CNoScalar { __device__ float operator()( float a, float b, float c ) const { return __fadd_rn( c, __fmul_rn( a, b ) ); } };
+// ( the product rounded by itself, as the CPU engine's separate multiply and add do: the pragma keeps the compiler from
+// contracting the two into a fused multiply-add )
+struct CMulAddOp : CNoScalar {
+	__device__ float operator()( float a, float b, float c ) const
+	{
+#pragma clang fp contract( off )
+		const float product = a * b;
+		return c + product;
+	}
+};
 template<typename T> struct CAddValueOp {
 	const T* Ptr; T Value;
 	__device__ void prepare() { Value = *Ptr; }
@@ -280,12 +299,22 @@ struct CNegMulValueOp {
 struct CMultiplyAndAddOp {
 	const float* Ptr; float Mult;
 	__device__ void prepare() { Mult = *Ptr; }
-	__device__ float operator()( float a, float b, float ) const { return __fadd_rn( a, __fmul_rn( b, Mult ) ); }
+	__device__ float operator()( float a, float b, float ) const
+	{
+#pragma clang fp contract( off )
+		const float product = b * Mult;
+		return a + product;
+	}
 };
 struct CMultiplyAndSubOp {
 	const float* Ptr; float Mult;
 	__device__ void prepare() { Mult = *Ptr; }
-	__device__ float operator()( float a, float b, float ) const { return __fsub_rn( a, __fmul_rn( b, Mult ) ); }
+	__device__ float operator()( float a, float b, float ) const
+	{
+#pragma clang fp contract( off )
+		const float product = b * Mult;
+		return a - product;
+	}
 };
 struct CSqrtOp : CNoScalar { __device__ float operator()( float a, float, float ) const { return sqrtf( a ); } };
 struct CInvOp : CNoScalar {
@@ -487,7 +516,7 @@ struct CTinyOp {
 struct CTinyChain {
 	int Length;
 	int Blocks;
-	int Straight; // no call has to wait for another: the grid has a thread per element of the longest call
+	int Straight; // no call has to wait for another: the grid has a thread per element of the longest call ( 4: per four elements )
 	int Reserved;
 	CTinyOp Ops[TinyChainMax];
 };
@@ -495,7 +524,8 @@ struct CTinyChain {
 template<typename... T> struct CTypeList {};
 // the functors a chain may hold ( float in, float out, no more than TinyFunctorBytes of state )
 typedef CTypeList<CFillOp<float>, CFillFromOp<float>, CCopyOp<float>, CAddOp<float>, CSubOp<float>, CMulOp<float>, CDivOp, CNegOp, CAbsOp, CMaxOp, CMinOp, CSqrtOp, CInvOp,
-	CAddValueOp<float>, CMulValueOp<float>, CNegMulValueOp, CMultiplyAndAddOp, CMultiplyAndSubOp, CMulAddOp, CNegMulOp> CTinyKinds;
+	CAddValueOp<float>, CMulValueOp<float>, CNegMulValueOp, CMultiplyAndAddOp, CMultiplyAndSubOp, CMulAddOp, CNegMulOp,
+	CReLUOp, CSigmoidOp, CTanhOp, CHSwishOp> CTinyKinds;
 
 template<typename F, typename List> struct CKindOf;
 template<typename F> struct CKindOf<F, CTypeList<>> { static constexpr int Value = -1; };
@@ -536,71 +566,150 @@ template<typename Head, typename... Tail> struct CTinyDispatch<CTypeList<Head, T
 	}
 };
 
-// One element of one call, the functor's device scalar already in hand ( the functors that have one are { pointer, value }:
+// N elements of one call, the functor's device scalar already in hand ( the functors that have one are { pointer, value }:
 // the value sits behind the pointer )
-template<typename F> __device__ __forceinline__ float applyTinyOp( const CTinyOp& op, float scalar, float x, float y, float z )
+template<typename F, int N> __device__ __forceinline__ void applyTinyOp( const CTinyOp& op, float scalar, const float* x, const float* y,
+	const float* z, float* r )
 {
 	F f;
 	__builtin_memcpy( &f, op.Functor, sizeof( F ) );
 	if( sizeof( F ) == 16 && op.Scalar != nullptr ) {
 		__builtin_memcpy( reinterpret_cast<char*>( &f ) + 8, &scalar, sizeof( float ) );
 	}
-	return f( x, y, z );
+#pragma unroll
+	for( int i = 0; i < N; ++i ) {
+		r[i] = f( x[i], y[i], z[i] );
+	}
 }
 
-template<typename List> struct CTinyApply;
-template<> struct CTinyApply<CTypeList<>> {
-	static __device__ __forceinline__ float Run( int, const CTinyOp&, float, float, float, float ) { return 0.f; }
+// ( the kind is the same for the whole grid: a search by halves costs a wavefront five scalar branches per call )
+template<int I, typename List> struct CTypeAt;
+template<typename Head, typename... Tail> struct CTypeAt<0, CTypeList<Head, Tail...>> { typedef Head Type; };
+template<int I, typename Head, typename... Tail> struct CTypeAt<I, CTypeList<Head, Tail...>> {
+	typedef typename CTypeAt<I - 1, CTypeList<Tail...>>::Type Type;
 };
-template<typename Head, typename... Tail> struct CTinyApply<CTypeList<Head, Tail...>> {
-	static __device__ __forceinline__ float Run( int kind, const CTinyOp& op, float scalar, float x, float y, float z )
+template<typename List> struct CTypeCount;
+template<typename... T> struct CTypeCount<CTypeList<T...>> { static constexpr int Value = static_cast<int>( sizeof...( T ) ); };
+
+template<typename List, int Lo = 0, int Hi = CTypeCount<List>::Value> struct CTinyApply {
+	template<int N> static __device__ __forceinline__ void Run( int kind, const CTinyOp& op, float scalar, const float* x, const float* y,
+		const float* z, float* r )
 	{
-		if( kind == 0 ) {
-			return applyTinyOp<Head>( op, scalar, x, y, z );
+		if constexpr( Hi - Lo == 1 ) {
+			applyTinyOp<typename CTypeAt<Lo, List>::Type, N>( op, scalar, x, y, z, r );
+		} else {
+			constexpr int Mid = ( Lo + Hi ) / 2;
+			if( kind < Mid ) {
+				CTinyApply<List, Lo, Mid>::template Run<N>( kind, op, scalar, x, y, z, r );
+			} else {
+				CTinyApply<List, Mid, Hi>::template Run<N>( kind, op, scalar, x, y, z, r );
+			}
 		}
-		return CTinyApply<CTypeList<Tail...>>::Run( kind - 1, op, scalar, x, y, z );
 	}
 };
+
+// A chain in which no call waits for another, and a grid with a thread per Q * V elements of the longest call: a thread
+// owns elements [first + u * stride, first + u * stride + V), u < Q, of every call ( V = 4: every call has the same count,
+// a multiple of four, and operands on 16-byte boundaries; Q of these 128-bit accesses are in flight per operand, as in
+// eltwiseKernel ). The scalars ( written by none of the calls ) are fetched together in front, and a call that reads where
+// the call in front of it wrote, or what the first call read, takes the value from the register it is still in: one round
+// trip to memory for a run of calls that work in place, not one per call.
+template<int V> __device__ __forceinline__ void loadTinyValues( const float* p, float* v )
+{
+	if( V == 4 ) {
+		const float4 q = *reinterpret_cast<const float4*>( p );
+		v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+	} else {
+		v[0] = *p;
+	}
+}
+
+template<int V, int Q> __device__ __forceinline__ void runStraightChain( const CTinyChain& chain, long long first, int stride )
+{
+	constexpr int N = V * Q;
+	float scalars[TinyChainMax];
+#pragma unroll
+	for( int k = 0; k < TinyChainMax; ++k ) {
+		scalars[k] = k < chain.Length && chain.Ops[k].Scalar != nullptr ? *chain.Ops[k].Scalar : 0.f;
+	}
+	const float* lastOut = nullptr; // what the call in front wrote
+	float lastValue[N] = {};
+	bool lastMine[Q] = {};
+	const float* heldIn = nullptr; // what the first call read ( its first operand ), and what has been written there since
+	float heldValue[N] = {};
+	bool heldMine[Q] = {};
+#pragma unroll
+	for( int k = 0; k < TinyChainMax; ++k ) {
+		if( k >= chain.Length ) {
+			break;
+		}
+		const CTinyOp& op = chain.Ops[k];
+		bool mine[Q];
+#pragma unroll
+		for( int u = 0; u < Q; ++u ) {
+			mine[u] = first + static_cast<long long>( u ) * stride < op.Count;
+		}
+		float in[3][N] = {};
+#pragma unroll
+		for( int j = 0; j < 3; ++j ) {
+			if( op.In[j] == nullptr ) {
+				continue;
+			}
+			const bool fromLast = op.In[j] == lastOut, fromHeld = op.In[j] == heldIn;
+#pragma unroll
+			for( int u = 0; u < Q; ++u ) {
+				if( !mine[u] ) {
+					continue;
+				}
+				if( fromLast && lastMine[u] ) {
+#pragma unroll
+					for( int v = 0; v < V; ++v ) in[j][u * V + v] = lastValue[u * V + v];
+				} else if( fromHeld && heldMine[u] ) {
+#pragma unroll
+					for( int v = 0; v < V; ++v ) in[j][u * V + v] = heldValue[u * V + v];
+				} else {
+					loadTinyValues<V>( op.In[j] + first + static_cast<long long>( u ) * stride, &in[j][u * V] );
+				}
+			}
+		}
+		if( k == 0 && op.In[0] != nullptr ) {
+			heldIn = op.In[0];
+#pragma unroll
+			for( int u = 0; u < Q; ++u ) heldMine[u] = mine[u];
+#pragma unroll
+			for( int i = 0; i < N; ++i ) heldValue[i] = in[0][i];
+		}
+		// ( elements that are not the thread's are computed from zeros and go nowhere )
+		CTinyApply<CTinyKinds>::template Run<N>( op.Kind, op, scalars[k], in[0], in[1], in[2], lastValue );
+		const bool overHeld = op.Out == heldIn;
+#pragma unroll
+		for( int u = 0; u < Q; ++u ) {
+			if( mine[u] ) {
+				float* to = op.Out + first + static_cast<long long>( u ) * stride;
+				if( V == 4 ) {
+					*reinterpret_cast<float4*>( to ) = make_float4( lastValue[u * V], lastValue[u * V + 1], lastValue[u * V + 2], lastValue[u * V + 3] );
+				} else {
+					*to = lastValue[u * V];
+				}
+			}
+			if( overHeld ) {
+				// ( whoever writes there owns the same elements: the held value follows )
+				heldMine[u] = mine[u];
+#pragma unroll
+				for( int v = 0; v < V; ++v ) heldValue[u * V + v] = lastValue[u * V + v];
+			}
+			lastMine[u] = mine[u];
+		}
+		lastOut = op.Out;
+	}
+}
 
 __global__ __launch_bounds__( TinyThreads ) void tinyChainKernel( const CTinyChain chain )
 {
 	const int first = blockIdx.x * blockDim.x + threadIdx.x;
 	const int step = gridDim.x * blockDim.x;
 	if( chain.Straight != 0 ) {
-		// No call waits for another, and the grid has a thread per element of the longest: a thread owns element `first` of
-		// every call. The scalars ( written by none of the calls ) are fetched together in front, and a call that reads
-		// where the call in front of it wrote takes the value from the register it is still in: one round trip to memory
-		// for a run of calls that work in place, not one per call.
-		float scalars[TinyChainMax];
-#pragma unroll
-		for( int k = 0; k < TinyChainMax; ++k ) {
-			scalars[k] = k < chain.Length && chain.Ops[k].Scalar != nullptr ? *chain.Ops[k].Scalar : 0.f;
-		}
-		const float* lastOut = nullptr;
-		float lastValue = 0.f;
-		bool lastMine = false;
-#pragma unroll
-		for( int k = 0; k < TinyChainMax; ++k ) {
-			if( k >= chain.Length ) {
-				break;
-			}
-			const CTinyOp& op = chain.Ops[k];
-			const bool mine = first < op.Count;
-			float in[3];
-#pragma unroll
-			for( int j = 0; j < 3; ++j ) {
-				in[j] = 0.f;
-				if( mine && op.In[j] != nullptr ) {
-					in[j] = ( lastMine && op.In[j] == lastOut ) ? lastValue : op.In[j][first];
-				}
-			}
-			if( mine ) {
-				lastValue = CTinyApply<CTinyKinds>::Run( op.Kind, op, scalars[k], in[0], in[1], in[2] );
-				op.Out[first] = lastValue;
-			}
-			lastOut = op.Out;
-			lastMine = mine;
-		}
+		runStraightChain<1, 1>( chain, first, 0 );
 		return;
 	}
 	for( int k = 0; k < chain.Length; ++k ) {
@@ -611,6 +720,15 @@ __global__ __launch_bounds__( TinyThreads ) void tinyChainKernel( const CTinyCha
 		}
 		CTinyDispatch<CTinyKinds>::Run( op.Kind, op, first, step );
 	}
+}
+
+// the same for calls of one count over vectors on 16-byte boundaries: QuadsPerThread times four elements per thread
+// ( the three calls of a GELU over 16.7 M elements: 72.6 us as three launches, 69 us with one quad per thread, 50 us with four )
+constexpr int QuadThreads = 256, QuadsPerThread = 4;
+__global__ __launch_bounds__( QuadThreads ) void quadChainKernel( const CTinyChain chain )
+{
+	runStraightChain<4, QuadsPerThread>( chain,
+		4ll * ( static_cast<long long>( blockIdx.x ) * ( QuadThreads * QuadsPerThread ) + threadIdx.x ), 4 * QuadThreads );
 }
 
 // A product A * B^T whose launch waits for the call behind it: a fully connected layer ( CFullyConnectedLayer::RunOnce,
@@ -654,6 +772,10 @@ struct CPendingSum {
 struct CTinyQueue {
 	bool Enabled = false;
 	CTinyChain Chain = {};
+	// A call over more than TinyWideMaxCount elements begins a chain that only calls of the same count join ( the passes
+	// of an activation or of a solver over one blob, quadChainKernel ); if none does, the call goes out as the launch it
+	// would have been on any other stream:
+	void ( *FirstAlone )( hipStream_t, const CTinyOp& ) = nullptr;
 	CPendingProduct Product;
 	CPendingConvolution Convolution;
 	CPendingSum Sum;
@@ -683,16 +805,35 @@ static int tinyDeferringStreams = 0;
 
 // With tinyLock held and the queue's device current. true: something was launched ( telling a stream's one-launch LSTMs
 // about it, noteStreamUse, is left to the callers: that takes a lock that a caller of toStream may hold ).
-static bool launchTinyChain( hipStream_t stream, CTinyChain& chain )
+static bool launchTinyChain( hipStream_t stream, CTinyQueue& queue )
 {
+	CTinyChain& chain = queue.Chain;
 	if( chain.Length == 0 ) {
 		return false;
 	}
-	bool barrier = false;
+	if( chain.Length == 1 && chain.Ops[0].Count > TinyWideMaxCount && queue.FirstAlone != nullptr ) {
+		const CTinyOp op = chain.Ops[0];
+		chain.Length = 0;
+		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+		queue.FirstAlone( stream, op );
+		return true;
+	}
+	bool barrier = false, quads = true;
 	int longest = 0;
 	for( int k = 0; k < chain.Length; ++k ) {
-		barrier = barrier || chain.Ops[k].Barrier != 0;
-		longest = chain.Ops[k].Count > longest ? chain.Ops[k].Count : longest;
+		const CTinyOp& op = chain.Ops[k];
+		barrier = barrier || op.Barrier != 0;
+		longest = op.Count > longest ? op.Count : longest;
+		quads = quads && op.Count == chain.Ops[0].Count && op.Count % 4 == 0 && isAligned16( op.Out )
+			&& isAligned16( op.In[0] ) && isAligned16( op.In[1] ) && isAligned16( op.In[2] );
+	}
+	if( !barrier && quads && longest > TinyOpMaxCount ) {
+		chain.Straight = 4;
+		chain.Blocks = ceilDiv( longest / 4, QuadThreads * QuadsPerThread );
+		hipLaunchKernelGGL( quadChainKernel, dim3( chain.Blocks ), dim3( QuadThreads ), 0, stream, chain );
+		chain.Length = 0;
+		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+		return true;
 	}
 	// one workgroup with barriers, or a thread per element of the longest call ( workgroups of 64, 256 and 1024 threads take
 	// the same 4.6 us for four calls over 8192 elements )
@@ -731,7 +872,7 @@ static bool launchPending( hipStream_t stream, CTinyQueue& queue )
 		( void )launchPlainSum( stream, sum );
 		return true;
 	}
-	return launchTinyChain( stream, queue.Chain );
+	return launchTinyChain( stream, queue );
 }
 
 bool flushTinyOps( hipStream_t stream )
@@ -872,8 +1013,9 @@ bool fusePendingProduct( nhStream s, const float* matrix, float* result, int hei
 
 static int launchPlainSum( hipStream_t stream, const CPendingSum& sum )
 {
-	return launchEltwise<2, float, float>( reinterpret_cast<nhStream>( stream ), sum.First, sum.Second, static_cast<const float*>( nullptr ),
-		sum.Result, sum.Count, CAddOp<float>() );
+	// ( the launch itself: the sum has waited already )
+	return launchEltwisePlain<2, float, float>( stream, sum.First, sum.Second, static_cast<const float*>( nullptr ), sum.Result, sum.Count,
+		CAddOp<float>() );
 }
 
 // a sum of two vectors too large for a chain: it waits for the call behind it
@@ -881,6 +1023,19 @@ static bool deferSum( nhStream s, const float* first, const float* second, float
 {
 	if( __atomic_load_n( &tinyDeferringStreams, __ATOMIC_RELAXED ) == 0 || first == nullptr || second == nullptr || result == nullptr ) {
 		return false;
+	}
+	if( __atomic_load_n( &tinyChainsPending, __ATOMIC_RELAXED ) != 0 ) {
+		// behind calls of the same count that wait as a chain ( a solver's last pass over a blob ) the sum is one more of them
+		int current = 0;
+		if( hipGetDevice( &current ) != hipSuccess ) {
+			( void )hipGetLastError();
+			return false;
+		}
+		std::lock_guard<std::recursive_mutex> guard( tinyLock );
+		auto waiting = tinyQueues().find( std::make_pair( current, reinterpret_cast<hipStream_t>( s ) ) );
+		if( waiting != tinyQueues().end() && waiting->second.Chain.Length > 0 && waiting->second.Chain.Ops[0].Count == count ) {
+			return false;
+		}
 	}
 	const hipStream_t stream = toStream( s ); // ( what the stream holds goes out first )
 	int device = 0;
@@ -1014,11 +1169,19 @@ template<typename F> struct CHasScalar<F, decltype( static_cast<void>( std::decl
 template<typename F> static auto scalarOf( const F& f, int ) -> decltype( static_cast<const float*>( f.Ptr ) ) { return f.Ptr; }
 template<typename F> static const float* scalarOf( const F&, long ) { return nullptr; }
 
+template<int NIN, typename F> static void launchTinyOpAlone( hipStream_t stream, const CTinyOp& op )
+{
+	F f;
+	__builtin_memcpy( &f, op.Functor, sizeof( F ) );
+	// ( a launch that fails leaves its HIP error to the next launch check )
+	( void )launchEltwisePlain<NIN, float, float, F>( stream, op.In[0], op.In[1], op.In[2], op.Out, op.Count, f );
+}
+
 template<int NIN, typename TIn, typename TOut, typename F>
 static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, const F& f )
 {
 	if constexpr( std::is_same<TIn, float>::value && std::is_same<TOut, float>::value && CKindOf<F, CTinyKinds>::Value >= 0 ) {
-		if( n > TinyWideMaxCount || __atomic_load_n( &tinyDeferringStreams, __ATOMIC_RELAXED ) == 0 ) {
+		if( __atomic_load_n( &tinyDeferringStreams, __ATOMIC_RELAXED ) == 0 ) {
 			return false;
 		}
 		const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
@@ -1039,9 +1202,13 @@ static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 		if( found->second.LaunchWaits() ) {
 			launchPending( stream, found->second ); // ( a launch that waited for its successor: this call is not the one )
 		}
-		CTinyChain& chain = found->second.Chain;
+		CTinyQueue& queue = found->second;
+		CTinyChain& chain = queue.Chain;
+		if( chain.Length > 0 && ( n > TinyWideMaxCount || chain.Ops[0].Count > TinyWideMaxCount ) && chain.Ops[0].Count != n ) {
+			launchTinyChain( stream, queue ); // ( a chain with a call that large holds calls of one count only )
+		}
 		if( chain.Length == TinyChainMax ) {
-			launchTinyChain( stream, chain );
+			launchTinyChain( stream, queue );
 		}
 		CTinyOp op = CTinyOp();
 		op.In[0] = NIN >= 1 ? a : nullptr;
@@ -1104,12 +1271,13 @@ static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 		if( barrier && wide ) {
 			// a chain with a barrier is one workgroup, too few threads for this many elements: what is in front goes out
 			// now, and this call is the first of the next chain
-			launchTinyChain( stream, chain );
+			launchTinyChain( stream, queue );
 			barrier = false;
 		}
 		op.Barrier = barrier ? 1 : 0;
 		if( chain.Length == 0 ) {
 			__atomic_fetch_add( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+			queue.FirstAlone = &launchTinyOpAlone<NIN, F>;
 		}
 		chain.Ops[chain.Length] = op;
 		++chain.Length;

@@ -660,8 +660,13 @@ void linearInterpolationKernel( const float* data, float* result, long long tota
 			const float rightMul = old - left;
 			const float leftMul = 1.f - rightMul;
 			const long long cell = static_cast<long long>( static_cast<int>( old ) ) * objectSize;
-			// two products, one sum, as the reference's multiply / multiply / add
-			value = __fadd_rn( __fmul_rn( in[cell + objectSize], rightMul ), __fmul_rn( in[cell], leftMul ) );
+			// two products, one sum, as the reference's multiply / multiply / add ( no fused multiply-add )
+			{
+#pragma clang fp contract( off )
+				const float right = in[cell + objectSize] * rightMul;
+				const float leftPart = in[cell] * leftMul;
+				value = right + leftPart;
+			}
 		}
 		result[i] = value;
 	}

@@ -976,13 +976,15 @@ SHIM_API int shim_performance_counters( void* engine, int smallSize, int largeSi
 		std::strncpy( name64, ( *counters )[0].Name, 63 );
 		name64[63] = 0;
 		counters->Synchronise();
+		// ( VectorExp: a call that an engine's stream launches at once; repeated calls of the kinds it may put aside
+		// and run as one pass would not be `repeats` passes over memory )
 		for( int i = 0; i < repeats; ++i ) {
-			e.VectorAbs( in.Const(), out.Handle(), smallSize );
+			e.VectorExp( in.Const(), out.Handle(), smallSize );
 		}
 		counters->Synchronise();
 		*smallValue = ( *counters )[0].Value;
 		for( int i = 0; i < repeats; ++i ) {
-			e.VectorAbs( in.Const(), out.Handle(), largeSize );
+			e.VectorExp( in.Const(), out.Handle(), largeSize );
 		}
 		counters->Synchronise();
 		*largeValue = ( *counters )[0].Value;

@@ -94,10 +94,10 @@ def test_row_normalisation_scalars_chain(streams):
 UNARY = ("nhVectorSqrt", "nhVectorInv", "nhVectorNeg", "nhVectorAbs")
 BINARY = ("nhVectorAdd", "nhVectorSub", "nhVectorEltwiseMultiply", "nhVectorEltwiseDivide", "nhVectorEltwiseMax", "nhVectorEltwiseMin",
           "nhVectorEltwiseMultiplyAdd", "nhVectorEltwiseNegMultiply")
-WITH_SCALAR = ("nhVectorAddValue", "nhVectorMultiply", "nhVectorNegMultiply")
+WITH_SCALAR = ("nhVectorAddValue", "nhVectorMultiply", "nhVectorNegMultiply", "nhVectorReLU")
 BINARY_WITH_SCALAR = ("nhVectorMultiplyAndAdd", "nhVectorMultiplyAndSub")
-# not of the kind that is put aside: launched at once, after what was put aside
-OTHER = ("nhVectorSigmoid", "nhVectorTanh")
+# activations that are put aside too, and two that are not: those are launched at once, after what was put aside
+OTHER = ("nhVectorSigmoid", "nhVectorTanh", "nhVectorHSwish", "nhVectorExp", "nhVectorSquaredHinge")
 
 
 def random_program(g, length):
@@ -105,8 +105,9 @@ def random_program(g, length):
     all come up; a result either begins where one of the call's own operands begins or keeps clear of them (what the
     entry points ask for); scalars sit in the arena too, sometimes where a call in front writes."""
     places = [0, 0, 0, 1, 3, 4, 64, 4096, 8192, 8195, 12288, 20000, 20000, 36000, 100000, 100000, 210000]
-    # ( above 16384 elements a call joins a chain only while no call in it has to wait for another; above 262144 never )
-    sizes = [1, 5, 64, 777, 1024, 4096, 8192, 8192, 16384, 16384, 20000, 70000, 200000, 300000]
+    # ( above 16384 elements a call joins a chain only while no call in it has to wait for another; above 262144 only
+    # a chain of calls of its own count )
+    sizes = [1, 5, 64, 777, 1024, 4096, 8192, 8192, 16384, 16384, 20000, 70000, 200000, 300000, 300000, 300000, 280000]
     program = []
     while len(program) < length:
         n = int(g.choice(sizes))
@@ -461,6 +462,83 @@ def test_large_sum_waits_for_its_relu(streams):
             want = run(streams.plain, in_place, successor)
             got = run(streams.deferring, in_place, successor)
             assert same_bits(got[0], want[0]) and same_bits(got[1], want[1]), (what, in_place)
+    # a copy to the host through the library is the call behind it (what a test of the engine does with a result)
+    d_a, d_b, d_out = up(a), up(b), torch.zeros(n, device=dev)
+    torch.cuda.synchronize()
+    na.check(lib.nhVectorAdd(streams.deferring, P(d_a), P(d_b), P(d_out), n))
+    fetched = np.empty(n, np.float32)
+    na.check(lib.nhCopyDeviceToHost(streams.deferring, fetched.ctypes.data_as(ctypes.c_void_p), P(d_out), fetched.nbytes))
+    assert same_bits(np.delete(fetched, 5), np.delete(a + b, 5)) and np.isnan(fetched[5])
     y, _ = run(streams.deferring, False, successors["ReLU6 in place"])
     assert y[5] == 0.0 and y.min() >= 0.0 and y.max() <= 6.0
     assert np.array_equal(np.delete(y, 5), np.clip(np.delete(a + b, 5), 0.0, 6.0))
+
+
+def test_large_calls_of_one_count_go_as_one_pass(streams):
+    """Calls over more elements than a mixed chain takes wait too, for calls of the same count: the three calls of
+    CGELULayer::runFastApproximate (NeoML/src/Dnn/Layers/GELULayer.cpp:145-160), in the layer's own form and with the
+    product written over the input, and a solver's passes over one parameter blob
+    (CDnnSimpleGradientSolver::TrainLayer, NeoML/src/Dnn/DnnSolver.cpp) leave the bits of the separate launches: on
+    16-byte boundaries with a count that is a multiple of four (four elements per thread), and off them."""
+    import torch
+    lib, na = streams.lib, streams.na
+    g = rng(4600)
+    dev = streams.dev
+    P = lambda t, o=0: ctypes.c_void_p(t.data_ptr() + 4 * o)
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    scale, rate, moment, decay = (up(np.array([v], np.float32)) for v in (1.702, -0.01, 0.9, 1e-4))
+
+    def gelu_layer(s, x, y, z, n, o):
+        na.check(lib.nhVectorMultiply(s, P(x, o), P(y, o), n, P(scale)))
+        na.check(lib.nhVectorSigmoid(s, P(y, o), P(y, o), n))
+        na.check(lib.nhVectorEltwiseMultiply(s, P(x, o), P(y, o), P(y, o), n))
+
+    def gelu_over_input(s, x, y, z, n, o):
+        na.check(lib.nhVectorMultiply(s, P(x, o), P(y, o), n, P(scale)))
+        na.check(lib.nhVectorSigmoid(s, P(y, o), P(y, o), n))
+        na.check(lib.nhVectorEltwiseMultiply(s, P(x, o), P(y, o), P(x, o), n))
+
+    def solver(s, x, y, z, n, o):
+        # x: parameters, y: their gradient, z: the moving mean of the steps
+        na.check(lib.nhVectorMultiply(s, P(z, o), P(z, o), n, P(moment)))
+        na.check(lib.nhVectorMultiplyAndAdd(s, P(y, o), P(x, o), P(y, o), n, P(decay)))
+        na.check(lib.nhVectorMultiplyAndAdd(s, P(z, o), P(y, o), P(z, o), n, P(rate)))
+        na.check(lib.nhVectorAdd(s, P(x, o), P(z, o), P(x, o), n))
+
+    def two_counts(s, x, y, z, n, o):
+        # a call of another count, and a small one, between calls of one count: each run goes out before the next begins
+        na.check(lib.nhVectorMultiply(s, P(x, o), P(y, o), n, P(scale)))
+        na.check(lib.nhVectorTanh(s, P(y, o), P(y, o), n - 4))
+        na.check(lib.nhVectorNeg(s, P(y, o), P(z, o), 1000))
+        na.check(lib.nhVectorHSwish(s, P(x, o), P(x, o), n))
+        na.check(lib.nhVectorReLU(s, P(x, o), P(x, o), n, P(moment)))
+
+    def shifted(s, x, y, z, n, o):
+        # the second call reads what the first wrote one element further on: it may not join the first
+        na.check(lib.nhVectorMultiply(s, P(x, o), P(y, o), n, P(scale)))
+        na.check(lib.nhVectorAbs(s, P(y, o + 1), P(z, o), n))
+
+    def alone(s, x, y, z, n, o):
+        # one large call and then a call that is no element-wise one: the large one goes out as its own launch
+        na.check(lib.nhVectorSigmoid(s, P(x, o), P(y, o), n))
+        na.check(lib.nhSumMatrixColumns(s, P(z, o), P(y, o), 1000, 64))
+
+    total = 3 * 1000 * 1000 + 16
+    data = [g.normal(0, 2, total).astype(np.float32) for _ in range(3)]
+    for what in (gelu_layer, gelu_over_input, solver, two_counts, shifted, alone):
+        for n, o in ((3 * 1000 * 1000, 0), (3 * 1000 * 1000, 4), (3 * 1000 * 1000 + 2, 0), (3 * 1000 * 1000, 3), (262148, 8)):
+            results = []
+            for stream in (streams.plain, streams.deferring):
+                x, y, z = (up(d) for d in data)
+                torch.cuda.synchronize()
+                what(stream, x, y, z, n, o)
+                na.check(lib.nhStreamSynchronize(stream))
+                results.append([t.cpu().numpy() for t in (x, y, z)])
+            for got, want in zip(results[1], results[0]):
+                assert same_bits(got, want), (what.__name__, n, o)
+    # and the values are the layer's: x * sigmoid( 1.702 x ) within the sigmoid's own bar
+    x, y, z = (up(d) for d in data)
+    gelu_layer(streams.deferring, x, y, z, 3 * 1000 * 1000, 0)
+    na.check(lib.nhStreamSynchronize(streams.deferring))
+    v = data[0][:3 * 1000 * 1000].astype(np.float64)
+    assert np.allclose(y.cpu().numpy()[:3 * 1000 * 1000], v / (1.0 + np.exp(-1.702 * v)), rtol=2e-6, atol=1e-6)
