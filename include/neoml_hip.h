@@ -456,7 +456,9 @@ NH_API int nhStreamOverlapLstm(nhStream s, int enable);
  * In the same way nhBlobConvolution and nhBlobChannelwiseConvolution wait for an nhVectorReLU over their result in place
  * (CConvLayer / CChannelwiseConvLayer followed by CReLULayer: the activation runs on the accumulators' way out, its
  * threshold read from the device scalar), and an nhVectorAdd over more than 262144 elements waits for an nhVectorReLU
- * over the sum in place (CEltwiseSumLayer + CReLULayer at the end of a residual block: one pass). Same bits as the two
+ * over the sum in place (CEltwiseSumLayer + CReLULayer at the end of a residual block: one pass), and
+ * nhBatchMultiplyMatrixByMatrix with a reduction of at most 256 waits for an nhVectorMultiply over its whole result in
+ * place (CMatrixMultiplicationLayer + CLinearLayer: an attention layer's scores and their factor). Same bits as the two
  * launches. */
 NH_API int nhStreamDeferSmallOps(nhStream s, int enable);
 /* LSTM (NME.h:1005-1011). Weights: inputWeights [4H x objectSize], recurrentWeights [4H x H]; gate order in

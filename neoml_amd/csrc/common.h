@@ -34,6 +34,10 @@ void releaseTinyQueue( hipStream_t stream );
 // *rc is the launch's code ), any other call sends the product out first, through toStream.
 bool deferProduct( nhStream s, const float* a, int lda, const float* b, int ldb, float* c, int ldc, int M, int N, int K );
 bool fusePendingProduct( nhStream s, const float* matrix, float* result, int height, int width, const float* vector, int* rc );
+// A batch of small dense row-major products that waits for the call behind it ( nhBatchMultiplyMatrixByMatrix followed by
+// nhVectorMultiply over the whole result in place: one launch )
+bool deferBatchedProduct( nhStream s, int batch, const float* first, int height, int width, const float* second, int secondWidth,
+	float* result );
 // The same for a convolution ( plain or channelwise, its descriptor checked by the caller ) and the VectorReLU over its
 // result in place that follows it in most networks.
 bool deferConvolution( nhStream s, bool channelwise, const nhConvDesc& d, const float* source, const float* filter,

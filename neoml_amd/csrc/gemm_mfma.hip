@@ -2517,8 +2517,11 @@ static int matMulNTMeeting( hipStream_t stream, const float* a, int lda, const f
 template<int MI, int KS>
 __global__ __launch_bounds__( Threads, 2 )
 void batchedStripKernel( const float* A, const float* B, float* C, int M, int N, int K, int lda, int ldb, int ldc,
-	long long strideA, long long strideB, long long strideC, int tilesM, int tilesN, int kChunks )
+	long long strideA, long long strideB, long long strideC, int tilesM, int tilesN, int kChunks, const float* scale )
 {
+	// ( a factor for every element of the result, read from device memory: the VectorMultiply of a CLinearLayer behind the
+	// product, done on the accumulators' way out; the accumulator is the value that call would have read, so the bits are its )
+	const float alpha = scale != nullptr ? *scale : 1.f;
 	constexpr int BM = 64 * MI;
 	constexpr int PitchA = KS + 4, PitchB = 68;
 	constexpr int QA = KS / 4;                 // float4 columns of an A tile row
@@ -2636,7 +2639,7 @@ void batchedStripKernel( const float* A, const float* B, float* C, int M, int N,
 				for( int r = 0; r < 16; ++r ) {
 					const int m = m0 + waveM * 32 * MI + mi * 32 + ( r >> 2 ) * 8 + half * 4 + ( r & 3 );
 					if( m < M && n < N ) {
-						C[static_cast<long long>( m ) * ldc + n] = acc[mi][r];
+						C[static_cast<long long>( m ) * ldc + n] = acc[mi][r] * alpha;
 					}
 					acc[mi][r] = 0.f;
 				}
@@ -2648,7 +2651,7 @@ void batchedStripKernel( const float* A, const float* B, float* C, int M, int N,
 
 // Whether a batched row-major product goes to batchedStripKernel: vector loads possible, many strips, and a reduction of
 // at most 256 ( longer ones keep the general kernel busy long enough per tile ).
-static bool tryBatchedStrips( hipStream_t stream, const CMatMulArgs& args, int batch, bool vec )
+static bool tryBatchedStrips( hipStream_t stream, const CMatMulArgs& args, int batch, bool vec, const float* scale )
 {
 	if( !vec || batch < 2 || args.Accumulate || args.K <= 0 || args.K > 256 ) {
 		return false;
@@ -2664,14 +2667,20 @@ static bool tryBatchedStrips( hipStream_t stream, const CMatMulArgs& args, int b
 	}
 	hipLaunchKernelGGL( ( batchedStripKernel<1, KS> ), dim3( static_cast<unsigned>( groups ) ), dim3( Threads ), 0, stream,
 		args.A, args.B, args.C, args.M, args.N, args.K, args.Lda, args.Ldb, args.Ldc,
-		args.BatchStrideA, args.BatchStrideB, args.BatchStrideC, tilesM, ceilDiv( args.N, 64 ), ceilDiv( args.K, KS ) );
+		args.BatchStrideA, args.BatchStrideB, args.BatchStrideC, tilesM, ceilDiv( args.N, 64 ), ceilDiv( args.K, KS ), scale );
 	return true;
 }
 
 // C = A * B, A is M x K, B is K x N, all row-major.
+// scale: a device scalar that every element of the result is to be multiplied by, if the kernel that takes the product can
+// do that on the way out ( *scaled says whether it did; the caller multiplies behind the product otherwise )
 int matMulNN( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
-	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC, bool accumulate )
+	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC, bool accumulate,
+	const float* scale, bool* scaled )
 {
+	if( scaled != nullptr ) {
+		*scaled = false;
+	}
 	if( M == 0 || N == 0 || batch == 0 ) {
 		return NH_OK;
 	}
@@ -2683,7 +2692,10 @@ int matMulNN( hipStream_t stream, const float* a, int lda, const float* b, int l
 	args.Accumulate = accumulate ? 1 : 0;
 	const bool vec = isAligned16( a ) && isAligned16( b ) && K % 4 == 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0
 		&& strideA % 4 == 0 && strideB % 4 == 0 && fitsBuffer( M, lda, K ) && fitsBuffer( K, ldb, N );
-	if( tryBatchedStrips( stream, args, batch, vec ) ) {
+	if( tryBatchedStrips( stream, args, batch, vec, scaled != nullptr ? scale : nullptr ) ) {
+		if( scaled != nullptr ) {
+			*scaled = scale != nullptr;
+		}
 		NH_LAUNCH_CHECK();
 		return NH_OK;
 	}
@@ -3399,10 +3411,15 @@ int nhBatchMultiplyMatrixByMatrix( nhStream s, int batchSize, const float* first
 {
 	NH_REQUIRE( batchSize >= 0 && firstHeight >= 0 && firstWidth >= 0 && secondWidth >= 0 );
 	NH_REQUIRE( static_cast<long long>( batchSize ) * firstHeight * secondWidth <= resultBufferSize );
+	// ( on a stream that puts calls aside a batch of small products waits for the call behind it: CLinearLayer's multiplier
+	// behind the QK^T of an attention layer becomes part of the launch )
+	if( deferBatchedProduct( s, batchSize, first, firstHeight, firstWidth, second, secondWidth, result ) ) {
+		return NH_OK;
+	}
 	return matMulNN( toStream( s ), first, firstWidth, second, secondWidth, result, secondWidth,
 		firstHeight, secondWidth, firstWidth, batchSize,
 		static_cast<long long>( firstHeight ) * firstWidth, static_cast<long long>( firstWidth ) * secondWidth,
-		static_cast<long long>( firstHeight ) * secondWidth, false );
+		static_cast<long long>( firstHeight ) * secondWidth, false, nullptr, nullptr );
 }
 
 int nhMultiplyTransposedMatrixByMatrixAndAdd( nhStream s, const float* first, int firstHeight, int firstWidth,

@@ -769,6 +769,17 @@ struct CPendingSum {
 	int Count = 0;
 };
 
+// A batch of small products C[b] = A[b] * B[b] ( dense, row-major ) followed by VectorMultiply over the whole result in place
+// by a device scalar: CMatrixMultiplicationLayer + CLinearLayer, the scores of an attention layer and their 1 / sqrt( d )
+// ( NeoML/src/Dnn/Layers/MultiheadAttentionLayer.cpp:168-183 ). The kernel for such batches multiplies on the way out.
+struct CPendingBatched {
+	bool Pending = false;
+	const float* A = nullptr;
+	const float* B = nullptr;
+	float* C = nullptr;
+	int Batch = 0, M = 0, N = 0, K = 0;
+};
+
 struct CTinyQueue {
 	bool Enabled = false;
 	CTinyChain Chain = {};
@@ -779,8 +790,9 @@ struct CTinyQueue {
 	CPendingProduct Product;
 	CPendingConvolution Convolution;
 	CPendingSum Sum;
+	CPendingBatched Batched;
 
-	bool LaunchWaits() const { return Product.Pending || Convolution.Pending || Sum.Pending; }
+	bool LaunchWaits() const { return Product.Pending || Convolution.Pending || Sum.Pending || Batched.Pending; }
 };
 
 static int launchPlainSum( hipStream_t stream, const CPendingSum& sum );
@@ -790,6 +802,16 @@ int launchDeferredConvolution( hipStream_t stream, bool channelwise, const nhCon
 
 int matMulNT( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
 	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC, const float* bias, bool accumulate );
+
+int matMulNN( hipStream_t stream, const float* a, int lda, const float* b, int ldb, float* c, int ldc,
+	int M, int N, int K, int batch, long long strideA, long long strideB, long long strideC, bool accumulate,
+	const float* scale, bool* scaled );
+
+static int launchBatched( hipStream_t stream, const CPendingBatched& p, const float* scale, bool* scaled )
+{
+	return matMulNN( stream, p.A, p.K, p.B, p.N, p.C, p.N, p.M, p.N, p.K, p.Batch, static_cast<long long>( p.M ) * p.K,
+		static_cast<long long>( p.K ) * p.N, static_cast<long long>( p.M ) * p.N, false, scale, scaled );
+}
 
 typedef std::map<std::pair<int, hipStream_t>, CTinyQueue> CTinyQueues;
 // ( recursive: a product launched from under the lock may ask its stream's pool for scratch memory, a pool at its limit
@@ -863,6 +885,13 @@ static bool launchPending( hipStream_t stream, CTinyQueue& queue )
 		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
 		const CFusedActivation none = { NH_ACT_NONE, 0.f };
 		( void )launchDeferredConvolution( stream, c.Channelwise, c.Desc, c.Source, c.Filter, c.FreeTerm, c.Result, none );
+		return true;
+	}
+	if( queue.Batched.Pending ) {
+		const CPendingBatched p = queue.Batched;
+		queue.Batched.Pending = false;
+		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+		( void )launchBatched( stream, p, nullptr, nullptr );
 		return true;
 	}
 	if( queue.Sum.Pending ) {
@@ -1009,6 +1038,71 @@ bool fusePendingProduct( nhStream s, const float* matrix, float* result, int hei
 		noteStreamUse( stream );
 	}
 	return true;
+}
+
+bool deferBatchedProduct( nhStream s, int batch, const float* first, int height, int width, const float* second, int secondWidth,
+	float* result )
+{
+	// ( only what the kernel for batches of small products may take: the others have nothing to gain from waiting )
+	if( __atomic_load_n( &tinyDeferringStreams, __ATOMIC_RELAXED ) == 0 || batch < 2 || height <= 0 || width <= 0 || width > 256
+		|| secondWidth <= 0 || first == nullptr || second == nullptr || result == nullptr
+		|| static_cast<long long>( batch ) * height * secondWidth > 0x7fffffffLL ) {
+		return false;
+	}
+	const hipStream_t stream = toStream( s ); // ( what the stream holds goes out first )
+	int device = 0;
+	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+	if( hipGetDevice( &device ) != hipSuccess || hipStreamIsCapturing( stream, &capture ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return false;
+	}
+	if( capture != hipStreamCaptureStatusNone ) {
+		return false;
+	}
+	std::lock_guard<std::recursive_mutex> guard( tinyLock );
+	auto found = tinyQueues().find( std::make_pair( device, stream ) );
+	if( found == tinyQueues().end() || !found->second.Enabled || found->second.Chain.Length != 0 || found->second.LaunchWaits() ) {
+		return false;
+	}
+	CPendingBatched& p = found->second.Batched;
+	p.Pending = true;
+	p.A = first; p.B = second; p.C = result; p.Batch = batch; p.M = height; p.N = secondWidth; p.K = width;
+	__atomic_fetch_add( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+	return true;
+}
+
+// VectorMultiply( first -> result, count, multiplier ) asks whether it is the call a batch of products waits for. true: both
+// have been launched as one ( *rc ). false: the caller goes on as usual ( a waiting batch has then been launched by itself if
+// this call is over its result but its kernel cannot multiply; otherwise the caller's own launch sends it out first ).
+static bool fusePendingBatched( nhStream s, const float* first, float* result, int count, const float* multiplier, int* rc )
+{
+	const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
+	int device = 0;
+	if( hipGetDevice( &device ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return false;
+	}
+	CPendingBatched p;
+	{
+		std::lock_guard<std::recursive_mutex> guard( tinyLock );
+		auto found = tinyQueues().find( std::make_pair( device, stream ) );
+		if( found == tinyQueues().end() || !found->second.Batched.Pending ) {
+			return false;
+		}
+		p = found->second.Batched;
+		if( first != p.C || result != p.C || multiplier == nullptr
+			|| static_cast<long long>( count ) != static_cast<long long>( p.Batch ) * p.M * p.N ) {
+			return false;
+		}
+		found->second.Batched.Pending = false;
+		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+	}
+	bool scaled = false;
+	*rc = launchBatched( stream, p, multiplier, &scaled );
+	if( __atomic_load_n( &lstmPartnersAwaited, __ATOMIC_RELAXED ) != 0 ) {
+		noteStreamUse( stream );
+	}
+	return scaled || *rc != NH_OK;
 }
 
 static int launchPlainSum( hipStream_t stream, const CPendingSum& sum )
@@ -1662,6 +1756,11 @@ extern "C" int nhVectorAddValueInt( nhStream s, const int* first, int* result, i
 extern "C" int nhVectorMultiply( nhStream s, const float* first, float* result, int vectorSize, const float* multiplier )
 {
 	NH_REQUIRE( multiplier != nullptr );
+	int rc = NH_OK;
+	if( first == result && __atomic_load_n( &tinyChainsPending, __ATOMIC_RELAXED ) != 0
+		&& fusePendingBatched( s, first, result, vectorSize, multiplier, &rc ) ) {
+		return rc; // ( a batch of products was waiting for this call )
+	}
 	CMulValueOp<float> op; op.Ptr = multiplier; op.Value = 0;
 	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
 }

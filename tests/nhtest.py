@@ -1188,7 +1188,7 @@ class CpuBackend:
     def add(self, a, b, out=None):
         return self.cpu.binary("add", a, b).reshape(a.shape)
 
-    def mul_scalar_(self, x, value):
+    def mul_scalar_(self, x, value, family=None):
         x[...] = self.cpu.unary("multiply", x, np.float32(value)).reshape(x.shape)
         return x
 

@@ -542,3 +542,49 @@ def test_large_calls_of_one_count_go_as_one_pass(streams):
     na.check(lib.nhStreamSynchronize(streams.deferring))
     v = data[0][:3 * 1000 * 1000].astype(np.float64)
     assert np.allclose(y.cpu().numpy()[:3 * 1000 * 1000], v / (1.0 + np.exp(-1.702 * v)), rtol=2e-6, atol=1e-6)
+
+
+def test_batch_of_products_waits_for_its_factor(streams):
+    """nhBatchMultiplyMatrixByMatrix followed by nhVectorMultiply over the whole result in place (CMatrixMultiplicationLayer
+    + CLinearLayer: the scores of an attention layer and their 1/sqrt(d), NeoML/src/Dnn/Layers/MultiheadAttentionLayer.cpp:
+    168-183) is one launch where the kernel for batches of small products takes the batch, two launches as ever where it
+    does not; the bits are those of the two launches, and every other successor finds the products done."""
+    import torch
+    lib, na = streams.lib, streams.na
+    g = rng(4700)
+    dev = streams.dev
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    factor = up(np.array([0.125], np.float32))
+    # ( batch, M, K, N ): an attention layer's scores, a ragged batch, one too small for the strip kernel, a long reduction
+    for batch, m, k, n in ((256, 256, 64, 256), (70, 200, 36, 132), (3, 64, 16, 64), (16, 128, 320, 64)):
+        a = g.normal(0, 1, (batch, m, k)).astype(np.float32)
+        b = g.normal(0, 1, (batch, k, n)).astype(np.float32)
+        count = batch * m * n
+
+        def run(stream, successor):
+            d_a, d_b = up(a), up(b)
+            out, other = torch.zeros(count, device=dev), torch.zeros(count, device=dev)
+            torch.cuda.synchronize()
+            na.check(lib.nhBatchMultiplyMatrixByMatrix(stream, batch, P(d_a), m, k, P(d_b), n, P(out), count))
+            successor(stream, out, other)
+            na.check(lib.nhStreamSynchronize(stream))
+            return out.cpu().numpy(), other.cpu().numpy()
+
+        successors = {
+            "the factor in place": lambda s, y, o: na.check(lib.nhVectorMultiply(s, P(y), P(y), count, P(factor))),
+            "nothing but the wait": lambda s, y, o: None,
+            "the factor into another vector": lambda s, y, o: na.check(lib.nhVectorMultiply(s, P(y), P(o), count, P(factor))),
+            "the factor over a part": lambda s, y, o: na.check(lib.nhVectorMultiply(s, P(y), P(y), count - n, P(factor))),
+            "a softmax": lambda s, y, o: na.check(lib.nhMatrixSoftmaxByRows(s, P(y), batch * m, n, P(o))),
+            "a small call": lambda s, y, o: na.check(lib.nhVectorNeg(s, P(y), P(o), 100)),
+            "the factor twice": lambda s, y, o: (na.check(lib.nhVectorMultiply(s, P(y), P(y), count, P(factor))),
+                                                 na.check(lib.nhVectorMultiply(s, P(y), P(y), count, P(factor)))),
+        }
+        for what, successor in successors.items():
+            want = run(streams.plain, successor)
+            got = run(streams.deferring, successor)
+            assert same_bits(got[0], want[0]) and same_bits(got[1], want[1]), (what, batch, m, k, n)
+        got, _ = run(streams.deferring, successors["the factor in place"])
+        want = np.matmul(a.astype(np.float64), b.astype(np.float64)).reshape(-1) * 0.125
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-5 * np.sqrt(k))

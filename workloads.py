@@ -258,8 +258,8 @@ class HipBackend:
         self._timed("add", 0, 12 * a.numel(), self.lib.nhVectorAdd, self._p(a), self._p(b), self._p(out), a.numel())
         return out
 
-    def mul_scalar_(self, x, value):
-        self._timed("eltwise", 0, 8 * x.numel(), self.lib.nhVectorMultiply, self._p(x), self._p(x), x.numel(), self._p(self.scalar(value)))
+    def mul_scalar_(self, x, value, family="eltwise"):
+        self._timed(family, 0, 8 * x.numel(), self.lib.nhVectorMultiply, self._p(x), self._p(x), x.numel(), self._p(self.scalar(value)))
         return x
 
     def transpose(self, x, out=None):
@@ -697,7 +697,9 @@ class TransformerEncoder(Network):
             kt = run(n + "kt", be.transpose, k.reshape(B, S, 1, D, 1))           # [B,D,1,S,1] = [B,h,dk,S]
             vt = run(n + "vt", be.transpose, v.reshape(B, S, 1, h, dk))
             sc = run(n + "sc", be.bmm_nn, qt.reshape(B * h, S, dk), kt.reshape(B * h, dk, S))
-            be.mul_scalar_(sc, 1.0 / np.sqrt(dk))
+            # ( CLinearLayer behind the product, MultiheadAttentionLayer.cpp:175-183: the product's family, whose launch
+            # takes the factor along on a stream that puts calls aside )
+            be.mul_scalar_(sc, 1.0 / np.sqrt(dk), family="bmm")
             pr = run(n + "pr", be.softmax, sc.reshape(B * h * S, S))
             cx = run(n + "cx", be.bmm_nn, pr.reshape(B * h, S, S), vt.reshape(B * h, S, dk))
             ct = run(n + "ct", be.transpose, cx.reshape(B, h, 1, S, dk))          # [B,S,1,h,dk]
