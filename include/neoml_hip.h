@@ -439,7 +439,9 @@ NH_API int nhStreamOverlapLstm(nhStream s, int enable);
  * eltwise neg-multiply) is put aside: calls over at most 262144 elements together whatever their counts, a call over more
  * elements only with calls of its own count (the passes of an activation layer or of a solver over one blob: the three
  * calls of CGELULayer's sigmoid form become one pass; a large call that no other joins goes out as the launch it
- * always was). Up to eight of them are launched together, in call order and with bit-identical results, as soon as ANY other call
+ * always was; nhAddVectorToMatrixColumns, nhMultiplyDiagMatrixByMatrix, nhAddVectorToMatrixRows and
+ * nhBatchMultiplyMatrixByDiagMatrix with batch 1 over more than 262144 elements are such calls too, their vector spread
+ * over the rows or columns: the last four calls of CObjectNormalizationLayer are one pass). Up to eight of them are launched together, in call order and with bit-identical results, as soon as ANY other call
  * on the stream through this library arrives: a larger or different operation, a copy, an event, nhStreamSynchronize,
  * nhStreamDestroy, enable = 0, or a release of device memory (nhRawFree, a pool's clean-up). Until then their results are
  * not in memory and their operands must stay valid, so this is only for streams whose work, synchronisation included,

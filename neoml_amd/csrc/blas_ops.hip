@@ -62,7 +62,18 @@ void rowBroadcastKernel( const float* matrix, float* result, const float* vector
 }
 
 template<int OP>
+static int launchRowBroadcastOn( hipStream_t stream, const float* matrix, float* result, const float* vector, int batch,
+	int height, int width, int matBatchStride, int vecBatchStride );
+
+template<int OP>
 static int launchRowBroadcast( nhStream s, const float* matrix, float* result, const float* vector, int batch,
+	int height, int width, int matBatchStride, int vecBatchStride )
+{
+	return launchRowBroadcastOn<OP>( toStream( s ), matrix, result, vector, batch, height, width, matBatchStride, vecBatchStride );
+}
+
+template<int OP>
+static int launchRowBroadcastOn( hipStream_t stream, const float* matrix, float* result, const float* vector, int batch,
 	int height, int width, int matBatchStride, int vecBatchStride )
 {
 	const long long total = static_cast<long long>( batch ) * height * width;
@@ -75,10 +86,10 @@ static int launchRowBroadcast( nhStream s, const float* matrix, float* result, c
 	long long blocks = ( work + 1023 ) / 1024; // 4 items per thread
 	blocks = blocks > 65536 ? 65536 : blocks;
 	if( vec ) {
-		hipLaunchKernelGGL( ( rowBroadcastKernel<OP, true> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+		hipLaunchKernelGGL( ( rowBroadcastKernel<OP, true> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, stream,
 			matrix, result, vector, height, width, total, matBatchStride, vecBatchStride );
 	} else {
-		hipLaunchKernelGGL( ( rowBroadcastKernel<OP, false> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+		hipLaunchKernelGGL( ( rowBroadcastKernel<OP, false> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, stream,
 			matrix, result, vector, height, width, total, matBatchStride, vecBatchStride );
 	}
 	NH_LAUNCH_CHECK();
@@ -112,7 +123,16 @@ void columnBroadcastKernel( const float* matrix, float* result, const float* vec
 }
 
 template<int OP>
+static int launchColumnBroadcastOn( hipStream_t stream, const float* matrix, float* result, const float* vector, int height, int width );
+
+template<int OP>
 static int launchColumnBroadcast( nhStream s, const float* matrix, float* result, const float* vector, int height, int width )
+{
+	return launchColumnBroadcastOn<OP>( toStream( s ), matrix, result, vector, height, width );
+}
+
+template<int OP>
+static int launchColumnBroadcastOn( hipStream_t stream, const float* matrix, float* result, const float* vector, int height, int width )
 {
 	const long long total = static_cast<long long>( height ) * width;
 	if( total == 0 ) {
@@ -123,10 +143,10 @@ static int launchColumnBroadcast( nhStream s, const float* matrix, float* result
 	long long blocks = ( work + 1023 ) / 1024;
 	blocks = blocks > 65536 ? 65536 : blocks;
 	if( vec ) {
-		hipLaunchKernelGGL( ( columnBroadcastKernel<OP, true> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+		hipLaunchKernelGGL( ( columnBroadcastKernel<OP, true> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, stream,
 			matrix, result, vector, width, total );
 	} else {
-		hipLaunchKernelGGL( ( columnBroadcastKernel<OP, false> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
+		hipLaunchKernelGGL( ( columnBroadcastKernel<OP, false> ), dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, stream,
 			matrix, result, vector, width, total );
 	}
 	NH_LAUNCH_CHECK();
@@ -642,6 +662,20 @@ static int softmaxImpl( nhStream s, const float* matrix, int height, int width, 
 	return NH_OK;
 }
 
+// The launch of a call with a spread vector that a stream had put aside and nothing joined
+static void launchSpreadAlone( hipStream_t stream, bool multiply, int spread, const float* matrix, const float* vector, float* result,
+	int height, int width )
+{
+	// ( a launch that fails leaves its HIP error to the next launch check )
+	if( spread == TS_PerRow ) {
+		( void )( multiply ? launchColumnBroadcastOn<BO_Mul>( stream, matrix, result, vector, height, width )
+			: launchColumnBroadcastOn<BO_Add>( stream, matrix, result, vector, height, width ) );
+	} else {
+		( void )( multiply ? launchRowBroadcastOn<BO_Mul>( stream, matrix, result, vector, 1, height, width, 0, 0 )
+			: launchRowBroadcastOn<BO_Add>( stream, matrix, result, vector, 1, height, width, 0, 0 ) );
+	}
+}
+
 extern "C" {
 
 
@@ -662,6 +696,9 @@ int nhAddVectorToMatrixRows( nhStream s, int batchSize, const float* matrix, flo
 	{
 		return rc; // ( the product that waited for this call took the vector with it )
 	}
+	if( batchSize == 1 && deferSpreadOp( s, false, TS_PerColumn, matrix, vector, result, matrixHeight, matrixWidth, &launchSpreadAlone ) ) {
+		return NH_OK;
+	}
 	return launchRowBroadcast<BO_Add>( s, matrix, result, vector, batchSize, matrixHeight, matrixWidth,
 		matrixHeight * matrixWidth, matrixWidth );
 }
@@ -670,6 +707,10 @@ int nhAddVectorToMatrixColumns( nhStream s, const float* matrix, float* result, 
 	const float* vector )
 {
 	NH_REQUIRE( matrixHeight >= 0 && matrixWidth >= 0 );
+	// ( on a stream that puts calls aside: one of a run of passes over the matrix, CObjectNormalizationLayer's four last calls )
+	if( deferSpreadOp( s, false, TS_PerRow, matrix, vector, result, matrixHeight, matrixWidth, &launchSpreadAlone ) ) {
+		return NH_OK;
+	}
 	return launchColumnBroadcast<BO_Add>( s, matrix, result, vector, matrixHeight, matrixWidth );
 }
 
@@ -685,6 +726,9 @@ int nhMultiplyDiagMatrixByMatrix( nhStream s, const float* first, int firstSize,
 {
 	NH_REQUIRE( firstSize >= 0 && secondWidth >= 0 );
 	NH_REQUIRE( static_cast<long long>( firstSize ) * secondWidth <= resultBufferSize );
+	if( deferSpreadOp( s, true, TS_PerRow, second, first, result, firstSize, secondWidth, &launchSpreadAlone ) ) {
+		return NH_OK;
+	}
 	return launchColumnBroadcast<BO_Mul>( s, second, result, first, firstSize, secondWidth );
 }
 
@@ -736,6 +780,9 @@ int nhBatchMultiplyMatrixByDiagMatrix( nhStream s, int batchSize, const float* f
 {
 	NH_REQUIRE( batchSize >= 0 && height >= 0 && width >= 0 && firstMatrixOffset >= 0 && secondMatrixOffset >= 0 );
 	NH_REQUIRE( static_cast<long long>( batchSize ) * height * width <= resultBufferSize );
+	if( batchSize == 1 && deferSpreadOp( s, true, TS_PerColumn, first, second, result, height, width, &launchSpreadAlone ) ) {
+		return NH_OK;
+	}
 	return launchRowBroadcast<BO_Mul>( s, first, result, second, batchSize, height, width, firstMatrixOffset, secondMatrixOffset );
 }
 

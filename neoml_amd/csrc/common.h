@@ -34,6 +34,14 @@ void releaseTinyQueue( hipStream_t stream );
 // *rc is the launch's code ), any other call sends the product out first, through toStream.
 bool deferProduct( nhStream s, const float* a, int lda, const float* b, int ldb, float* c, int ldc, int M, int N, int K );
 bool fusePendingProduct( nhStream s, const float* matrix, float* result, int height, int width, const float* vector, int* rc );
+// An element-wise call over a height x width matrix ( more than 262144 elements ) whose second operand is a vector spread
+// over the rows or the columns joins the stream's chain of large calls of one count: matrix (+ or *) vector -> result.
+// alone: the call's own launch, for when nothing joins it.
+enum TTinySpread { TS_None = 0, TS_PerRow = 1, TS_PerColumn = 2 };
+typedef void ( *CSpreadAlone )( hipStream_t stream, bool multiply, int spread, const float* matrix, const float* vector, float* result,
+	int height, int width );
+bool deferSpreadOp( nhStream s, bool multiply, int spread, const float* matrix, const float* vector, float* result, int height, int width,
+	CSpreadAlone alone );
 // A batch of small dense row-major products that waits for the call behind it ( nhBatchMultiplyMatrixByMatrix followed by
 // nhVectorMultiply over the whole result in place: one launch )
 bool deferBatchedProduct( nhStream s, int batch, const float* first, int height, int width, const float* second, int secondWidth,

@@ -110,7 +110,8 @@ void eltwiseKernel( const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, 
 // A stream may put small calls aside and run several of them with one launch ( "tiny chains", below the functors ).
 // true: the call has been taken over, nothing is left to launch.
 template<int NIN, typename TIn, typename TOut, typename F>
-static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, const F& f );
+static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, const F& f, int spread = TS_None,
+	int width = 0, CSpreadAlone spreadAlone = nullptr );
 
 template<int NIN, typename TIn, typename TOut, typename F>
 static int launchEltwisePlain( hipStream_t stream, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, F f );
@@ -511,6 +512,12 @@ struct CTinyOp {
 	short Kind; // index into CTinyKinds
 	short Barrier; // every thread must have finished the calls in front
 	alignas( 8 ) unsigned char Functor[TinyFunctorBytes];
+	// The second operand of a call over a matrix of rows of Width elements may be a vector spread over it: one value per row
+	// ( TS_PerRow: In[1][i / Width], AddVectorToMatrixColumns, MultiplyDiagMatrixByMatrix ) or per column ( TS_PerColumn:
+	// In[1][i % Width], AddVectorToMatrixRows, MultiplyMatrixByDiagMatrix ). Only calls over more than TinyWideMaxCount
+	// elements come with one, so a chain with barriers never holds any.
+	int Spread;
+	int Width;
 };
 
 struct CTinyChain {
@@ -638,6 +645,8 @@ template<int V, int Q> __device__ __forceinline__ void runStraightChain( const C
 	const float* heldIn = nullptr; // what the first call read ( its first operand ), and what has been written there since
 	float heldValue[N] = {};
 	bool heldMine[Q] = {};
+	int spreadWidth = 0; // where the thread's elements lie in a matrix of rows of that many elements
+	unsigned row[Q] = {}, column[Q] = {};
 #pragma unroll
 	for( int k = 0; k < TinyChainMax; ++k ) {
 		if( k >= chain.Length ) {
@@ -653,6 +662,33 @@ template<int V, int Q> __device__ __forceinline__ void runStraightChain( const C
 #pragma unroll
 		for( int j = 0; j < 3; ++j ) {
 			if( op.In[j] == nullptr ) {
+				continue;
+			}
+			if( j == 1 && op.Spread != TS_None ) {
+				if( op.Width != spreadWidth ) {
+					// ( the divisions once per width: the calls of a chain are as a rule over one matrix )
+					spreadWidth = op.Width;
+#pragma unroll
+					for( int u = 0; u < Q; ++u ) {
+						const unsigned element = static_cast<unsigned>( first + static_cast<long long>( u ) * stride );
+						row[u] = element / static_cast<unsigned>( spreadWidth );
+						column[u] = element - row[u] * static_cast<unsigned>( spreadWidth );
+					}
+				}
+#pragma unroll
+				for( int u = 0; u < Q; ++u ) {
+					if( !mine[u] ) {
+						continue;
+					}
+					// ( with V = 4 the width is a multiple of four: the four elements lie in one row, on four columns in a row )
+					if( op.Spread == TS_PerRow ) {
+						const float value = op.In[1][row[u]];
+#pragma unroll
+						for( int v = 0; v < V; ++v ) in[1][u * V + v] = value;
+					} else {
+						loadTinyValues<V>( op.In[1] + column[u], &in[1][u * V] );
+					}
+				}
 				continue;
 			}
 			const bool fromLast = op.In[j] == lastOut, fromHeld = op.In[j] == heldIn;
@@ -724,6 +760,9 @@ __global__ __launch_bounds__( TinyThreads ) void tinyChainKernel( const CTinyCha
 
 // the same for calls of one count over vectors on 16-byte boundaries: QuadsPerThread times four elements per thread
 // ( the three calls of a GELU over 16.7 M elements: 72.6 us as three launches, 69 us with one quad per thread, 50 us with four )
+// ( the four last calls of a normalisation layer over 8192 x 512 values, 16 MB that stay in the caches: 25 us as four launches,
+// 12 us as one, with one quad per thread as with four: what is left is a wavefront waiting for one call's spread vector
+// after the other )
 constexpr int QuadThreads = 256, QuadsPerThread = 4;
 __global__ __launch_bounds__( QuadThreads ) void quadChainKernel( const CTinyChain chain )
 {
@@ -787,6 +826,7 @@ struct CTinyQueue {
 	// of an activation or of a solver over one blob, quadChainKernel ); if none does, the call goes out as the launch it
 	// would have been on any other stream:
 	void ( *FirstAlone )( hipStream_t, const CTinyOp& ) = nullptr;
+	CSpreadAlone FirstSpreadAlone = nullptr; // ( the same for a call with a spread operand: its own kernel lives with its entry point )
 	CPendingProduct Product;
 	CPendingConvolution Convolution;
 	CPendingSum Sum;
@@ -833,11 +873,17 @@ static bool launchTinyChain( hipStream_t stream, CTinyQueue& queue )
 	if( chain.Length == 0 ) {
 		return false;
 	}
-	if( chain.Length == 1 && chain.Ops[0].Count > TinyWideMaxCount && queue.FirstAlone != nullptr ) {
+	if( chain.Length == 1 && chain.Ops[0].Count > TinyWideMaxCount
+		&& ( chain.Ops[0].Spread != TS_None ? queue.FirstSpreadAlone != nullptr : queue.FirstAlone != nullptr ) ) {
 		const CTinyOp op = chain.Ops[0];
 		chain.Length = 0;
 		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
-		queue.FirstAlone( stream, op );
+		if( op.Spread != TS_None ) {
+			queue.FirstSpreadAlone( stream, op.Kind == CKindOf<CMulOp<float>, CTinyKinds>::Value, op.Spread, op.In[0], op.In[1], op.Out,
+				op.Count / op.Width, op.Width );
+		} else {
+			queue.FirstAlone( stream, op );
+		}
 		return true;
 	}
 	bool barrier = false, quads = true;
@@ -847,7 +893,8 @@ static bool launchTinyChain( hipStream_t stream, CTinyQueue& queue )
 		barrier = barrier || op.Barrier != 0;
 		longest = op.Count > longest ? op.Count : longest;
 		quads = quads && op.Count == chain.Ops[0].Count && op.Count % 4 == 0 && isAligned16( op.Out )
-			&& isAligned16( op.In[0] ) && isAligned16( op.In[1] ) && isAligned16( op.In[2] );
+			&& isAligned16( op.In[0] ) && isAligned16( op.In[1] ) && isAligned16( op.In[2] )
+			&& ( op.Spread == TS_None || op.Width % 4 == 0 );
 	}
 	if( !barrier && quads && longest > TinyOpMaxCount ) {
 		chain.Straight = 4;
@@ -1263,6 +1310,15 @@ template<typename F> struct CHasScalar<F, decltype( static_cast<void>( std::decl
 template<typename F> static auto scalarOf( const F& f, int ) -> decltype( static_cast<const float*>( f.Ptr ) ) { return f.Ptr; }
 template<typename F> static const float* scalarOf( const F&, long ) { return nullptr; }
 
+// what a call reads of its spread operand
+static CFloatRange spreadRange( const CTinyOp& op )
+{
+	CFloatRange range;
+	range.Lo = op.In[1];
+	range.Hi = op.In[1] + ( op.Spread == TS_PerRow ? op.Count / op.Width : op.Width );
+	return range;
+}
+
 template<int NIN, typename F> static void launchTinyOpAlone( hipStream_t stream, const CTinyOp& op )
 {
 	F f;
@@ -1272,7 +1328,8 @@ template<int NIN, typename F> static void launchTinyOpAlone( hipStream_t stream,
 }
 
 template<int NIN, typename TIn, typename TOut, typename F>
-static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, const F& f )
+static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, TOut* out, int n, const F& f, int spread, int width,
+	CSpreadAlone spreadAlone )
 {
 	if constexpr( std::is_same<TIn, float>::value && std::is_same<TOut, float>::value && CKindOf<F, CTinyKinds>::Value >= 0 ) {
 		if( __atomic_load_n( &tinyDeferringStreams, __ATOMIC_RELAXED ) == 0 ) {
@@ -1311,14 +1368,19 @@ static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 		op.Out = out;
 		op.Count = n;
 		op.Kind = static_cast<short>( CKindOf<F, CTinyKinds>::Value );
+		op.Spread = spread;
+		op.Width = width;
 		__builtin_memcpy( op.Functor, &f, sizeof( F ) );
-		// what the calls in front have to do with this one
-		CFloatRange reads[4], writes;
+		// what the calls in front have to do with this one ( reads[4]: a spread operand, read by many threads like the scalar )
+		CFloatRange reads[5], writes;
 		for( int i = 0; i < 3; ++i ) {
-			if( op.In[i] != nullptr ) {
+			if( op.In[i] != nullptr && ( i != 1 || spread == TS_None ) ) {
 				reads[i].Lo = op.In[i];
 				reads[i].Hi = op.In[i] + n;
 			}
+		}
+		if( spread != TS_None ) {
+			reads[4] = spreadRange( op );
 		}
 		const float* scalar = scalarOf( f, 0 );
 		// ( a functor with a device scalar is { pointer, value }: tinyChainKernel puts the value it has fetched behind the pointer )
@@ -1346,14 +1408,17 @@ static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 			frontWrites.Hi = front.Out + front.Count;
 			// ( the scalar: read by every thread, so a match of the first element is no excuse )
 			barrier = rangesClash( reads[0], frontWrites ) || rangesClash( reads[1], frontWrites ) || rangesClash( reads[2], frontWrites )
-				|| rangesTouch( reads[3], frontWrites ) || rangesClash( writes, frontWrites );
+				|| rangesTouch( reads[3], frontWrites ) || rangesTouch( reads[4], frontWrites ) || rangesClash( writes, frontWrites );
 			for( int i = 0; i < 3 && !barrier; ++i ) {
-				if( front.In[i] != nullptr ) {
+				if( front.In[i] != nullptr && ( i != 1 || front.Spread == TS_None ) ) {
 					CFloatRange frontReads;
 					frontReads.Lo = front.In[i];
 					frontReads.Hi = front.In[i] + front.Count;
 					barrier = rangesClash( writes, frontReads );
 				}
+			}
+			if( !barrier && front.Spread != TS_None ) {
+				barrier = rangesTouch( writes, spreadRange( front ) );
 			}
 			if( !barrier && front.Scalar != nullptr ) {
 				CFloatRange frontReads;
@@ -1372,14 +1437,33 @@ static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 		if( chain.Length == 0 ) {
 			__atomic_fetch_add( &tinyChainsPending, 1, __ATOMIC_RELAXED );
 			queue.FirstAlone = &launchTinyOpAlone<NIN, F>;
+			queue.FirstSpreadAlone = spreadAlone;
 		}
 		chain.Ops[chain.Length] = op;
 		++chain.Length;
 		return true;
 	} else {
-		( void )s; ( void )a; ( void )b; ( void )c; ( void )out; ( void )n; ( void )f;
+		( void )s; ( void )a; ( void )b; ( void )c; ( void )out; ( void )n; ( void )f; ( void )spread; ( void )width; ( void )spreadAlone;
 		return false;
 	}
+}
+
+bool deferSpreadOp( nhStream s, bool multiply, int spread, const float* matrix, const float* vector, float* result, int height, int width,
+	CSpreadAlone alone )
+{
+	const long long count = static_cast<long long>( height ) * width;
+	if( __atomic_load_n( &tinyDeferringStreams, __ATOMIC_RELAXED ) == 0 || count <= TinyWideMaxCount || count > 0x7fffffffLL
+		|| matrix == nullptr || vector == nullptr || result == nullptr || alone == nullptr
+		|| ( spread != TS_PerRow && spread != TS_PerColumn ) ) {
+		return false;
+	}
+	const float* none = nullptr;
+	if( multiply ) {
+		return deferEltwise<2, float, float, CMulOp<float>>( s, matrix, vector, none, result, static_cast<int>( count ), CMulOp<float>(),
+			spread, width, alone );
+	}
+	return deferEltwise<2, float, float, CAddOp<float>>( s, matrix, vector, none, result, static_cast<int>( count ), CAddOp<float>(),
+		spread, width, alone );
 }
 
 // ---- reductions to one value: one workgroup per 16K elements ------------------------------------------------------

@@ -588,3 +588,69 @@ def test_batch_of_products_waits_for_its_factor(streams):
         got, _ = run(streams.deferring, successors["the factor in place"])
         want = np.matmul(a.astype(np.float64), b.astype(np.float64)).reshape(-1) * 0.125
         assert np.allclose(got, want, rtol=1e-5, atol=1e-5 * np.sqrt(k))
+
+
+def test_passes_over_a_matrix_with_vectors_spread_over_it(streams):
+    """The thirteen calls of CObjectNormalizationLayer::runOnceImpl (NeoML/src/Dnn/Layers/ObjectNormalizationLayer.cpp:
+    181-242) at the size of a transformer layer: the calls that add a vector to the columns or rows of the matrix, or
+    multiply by a diagonal matrix, are element-wise calls with a vector spread over the matrix and join the chain of large
+    calls of one count (the layer's last four calls become one pass, the centring and squaring in front of the variance
+    another). Same bits as the separate launches: widths that are and are not multiples of four, in place and not,
+    off the 16-byte boundaries, and with other calls between them."""
+    import torch
+    lib, na = streams.lib, streams.na
+    g = rng(4800)
+    dev = streams.dev
+    P = lambda t, o=0: ctypes.c_void_p(t.data_ptr() + 4 * o)
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    def layer(s, x, out, sq, neg_mean, inv_std, scale, bias, inv_w, eps, rows, width, o):
+        n = rows * width
+        na.check(lib.nhSumMatrixColumns(s, P(neg_mean), P(x, o), rows, width))
+        na.check(lib.nhVectorNegMultiply(s, P(neg_mean), P(neg_mean), rows, P(inv_w)))
+        na.check(lib.nhAddVectorToMatrixColumns(s, P(x, o), P(sq, o), rows, width, P(neg_mean)))
+        na.check(lib.nhVectorEltwiseMultiply(s, P(sq, o), P(sq, o), P(sq, o), n))
+        na.check(lib.nhSumMatrixColumns(s, P(inv_std), P(sq, o), rows, width))
+        na.check(lib.nhVectorMultiply(s, P(inv_std), P(inv_std), rows, P(inv_w)))
+        na.check(lib.nhVectorAddValue(s, P(inv_std), P(inv_std), rows, P(eps)))
+        na.check(lib.nhVectorSqrt(s, P(inv_std), P(inv_std), rows))
+        na.check(lib.nhVectorInv(s, P(inv_std), P(inv_std), rows))
+        na.check(lib.nhAddVectorToMatrixColumns(s, P(x, o), P(out, o), rows, width, P(neg_mean)))
+        na.check(lib.nhMultiplyDiagMatrixByMatrix(s, P(inv_std), rows, P(out, o), width, P(out, o), n))
+        na.check(lib.nhBatchMultiplyMatrixByDiagMatrix(s, 1, P(out, o), rows, width, 0, P(scale), 0, P(out, o), n))
+        na.check(lib.nhAddVectorToMatrixRows(s, 1, P(out, o), P(out, o), rows, width, P(bias)))
+
+    def other_orders(s, x, out, sq, neg_mean, inv_std, scale, bias, inv_w, eps, rows, width, o):
+        n = rows * width
+        na.check(lib.nhSumMatrixColumns(s, P(neg_mean), P(x, o), rows, width))
+        # a vector per row and one per column into different results, then a call that reads the spread vector's memory as a
+        # matrix ( no hazard: reads only ), then one that writes where a call in front read its vector ( goes out alone )
+        na.check(lib.nhAddVectorToMatrixRows(s, 1, P(x, o), P(out, o), rows, width, P(bias)))
+        na.check(lib.nhMultiplyDiagMatrixByMatrix(s, P(neg_mean), rows, P(out, o), width, P(sq, o), n))
+        na.check(lib.nhVectorAbs(s, P(sq, o), P(sq, o), n))
+        na.check(lib.nhBatchMultiplyMatrixByDiagMatrix(s, 1, P(sq, o), rows, width, 0, P(sq, o), 0, P(out, o), n))
+        na.check(lib.nhAddVectorToMatrixColumns(s, P(out, o), P(x, o), rows, width, P(out, o)))
+        na.check(lib.nhVectorFill(s, P(neg_mean), ctypes.c_float(0.5), rows))
+        na.check(lib.nhAddVectorToMatrixColumns(s, P(x, o), P(x, o), rows, width, P(neg_mean)))
+
+    for rows, width, o in ((8192, 512, 0), (1000, 300, 0), (1000, 300, 3), (999, 263, 0), (700, 376, 4)):
+        n = rows * width
+        x0 = g.normal(0.3, 1.5, n + 8).astype(np.float32)
+        scale0, bias0 = g.normal(1, 0.2, width).astype(np.float32), g.normal(0, 0.5, width).astype(np.float32)
+        for what in (layer, other_orders):
+            results = []
+            for stream in (streams.plain, streams.deferring):
+                x, scale, bias = up(x0), up(scale0), up(bias0)
+                out, sq = torch.zeros(n + 8, device=dev), torch.zeros(n + 8, device=dev)
+                neg_mean, inv_std = torch.zeros(rows, device=dev), torch.zeros(rows, device=dev)
+                inv_w, eps = up(np.array([1.0 / width], np.float32)), up(np.array([1e-5], np.float32))
+                torch.cuda.synchronize()
+                what(stream, x, out, sq, neg_mean, inv_std, scale, bias, inv_w, eps, rows, width, o)
+                na.check(lib.nhStreamSynchronize(stream))
+                results.append([t.cpu().numpy() for t in (x, out, sq, neg_mean, inv_std)])
+            for got, want in zip(results[1], results[0]):
+                assert same_bits(got, want), (what.__name__, rows, width, o)
+            if what is layer:
+                v = x0[o:o + n].astype(np.float64).reshape(rows, width)
+                ref = (v - v.mean(1, keepdims=True)) / np.sqrt(v.var(1, keepdims=True) + 1e-5) * scale0 + bias0
+                assert np.allclose(results[1][1][o:o + n].reshape(rows, width), ref, rtol=1e-4, atol=1e-4)
