@@ -460,8 +460,9 @@ NH_API int nhStreamOverlapLstm(nhStream s, int enable);
  * threshold read from the device scalar), and an nhVectorAdd over more than 262144 elements waits for an nhVectorReLU
  * over the sum in place (CEltwiseSumLayer + CReLULayer at the end of a residual block: one pass), and
  * nhBatchMultiplyMatrixByMatrix with a reduction of at most 256 waits for an nhVectorMultiply over its whole result in
- * place (CMatrixMultiplicationLayer + CLinearLayer: an attention layer's scores and their factor). Same bits as the two
- * launches. */
+ * place (CMatrixMultiplicationLayer + CLinearLayer: an attention layer's scores and their factor), and nhBlobResizeImage
+ * with constant padding waits for an nhBlobMaxPooling (3x3, no indices) over the padded blob (CImageResizeLayer +
+ * CMaxPoolingLayer: one launch writes both blobs). Same bits as the two launches. */
 NH_API int nhStreamDeferSmallOps(nhStream s, int enable);
 /* LSTM (NME.h:1005-1011). Weights: inputWeights [4H x objectSize], recurrentWeights [4H x H]; gate order in
  * the 4H vector: main(tanh) | forget | input | output (src/CPU/CpuMathEngineDnnLstm.h:49-90).

@@ -42,6 +42,22 @@ typedef void ( *CSpreadAlone )( hipStream_t stream, bool multiply, int spread, c
 	int height, int width );
 bool deferSpreadOp( nhStream s, bool multiply, int spread, const float* matrix, const float* vector, float* result, int height, int width,
 	CSpreadAlone alone );
+// An image blob padded with a constant ( nhBlobResizeImage ) that waits for the call behind it: a 3 x 3 max pooling over the
+// padded blob ( CImageResizeLayer + CMaxPoolingLayer, the way a pooling layer without padding of its own gets its border )
+// writes the padded blob and the pooled one in one pass over the image.
+struct CPendingPadding {
+	bool Pending = false;
+	const float* From = nullptr;
+	float* To = nullptr;
+	long long Batch = 0;
+	int Height = 0, Width = 0, Channels = 0, ToHeight = 0, ToWidth = 0, DeltaLeft = 0, DeltaTop = 0, Padding = 0;
+	float DefaultValue = 0.f;
+};
+bool deferPadding( nhStream s, const CPendingPadding& padding );
+bool fusePendingPadding( nhStream s, const nhPoolingDesc& d, const float* source, float* result, int* rc );
+// ( dnn_ops.hip ) the padding by itself; the padding with the pooling over it, false if the pair is not one it takes
+int launchPadding( hipStream_t stream, const CPendingPadding& padding );
+bool launchPaddingWithPooling( hipStream_t stream, const CPendingPadding& padding, const nhPoolingDesc& d, float* result, int* rc );
 // A batch of small dense row-major products that waits for the call behind it ( nhBatchMultiplyMatrixByMatrix followed by
 // nhVectorMultiply over the whole result in place: one launch )
 bool deferBatchedProduct( nhStream s, int batch, const float* first, int height, int width, const float* second, int secondWidth,

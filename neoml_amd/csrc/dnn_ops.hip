@@ -309,6 +309,112 @@ void poolingKernel( const nhPoolingDesc d, const float* source, float* result, i
 	}
 }
 
+// An image padded with a constant and the 3 x 3 max pooling over the padded image, one launch: the thread of poolingKernel
+// ( four channels of one output column, a few output rows down ) takes its nine taps from the image itself, the constant
+// where a tap lies in the border, and also writes the pixels of the padded image that are its own: the rows and columns
+// from the first of its window up to the first of the next window ( up to the edge for the last window of a row or column ),
+// so every padded pixel is written once. The padded image is not read back: 470 MB move where the two launches moved 683 MB
+// ( 64 x 112 x 112 x 64 padded by one pixel, pooled with stride 2 ). Strides of at most 3, so that the pixels a thread
+// owns lie in its window ( the few beyond it, at the far edges, are fetched on their own ). The maxima are taken in
+// poolingKernel's order ( rows of a column first ), with the same comparisons.
+struct CPadPoolArgs {
+	const float* From;
+	float* Padded;
+	float* Result;
+	int Height, Width, Channels, ToHeight, ToWidth, DeltaTop, DeltaLeft;
+	float DefaultValue;
+	int StrideHeight, StrideWidth, ResultHeight, ResultWidth, RowChunks, RowsPerItem;
+	long long TotalItems;
+};
+
+__device__ __forceinline__ float4 paddedPixel( const CPadPoolArgs& a, const float* image, int py, int px )
+{
+	const int sy = py - a.DeltaTop, sx = px - a.DeltaLeft;
+	if( sy >= 0 && sy < a.Height && sx >= 0 && sx < a.Width ) {
+		return *reinterpret_cast<const float4*>( image + ( static_cast<long long>( sy ) * a.Width + sx ) * a.Channels );
+	}
+	return make_float4( a.DefaultValue, a.DefaultValue, a.DefaultValue, a.DefaultValue );
+}
+
+__global__ __launch_bounds__( 256 )
+void padMaxPool3x3Kernel( const CPadPoolArgs a )
+{
+	const int cg = a.Channels / 4;
+	const long long step = static_cast<long long>( gridDim.x ) * 256;
+	for( long long item = xcdSwizzle( blockIdx.x, gridDim.x ) * 256LL + threadIdx.x; item < a.TotalItems; item += step ) {
+		long long t = item;
+		const int c = static_cast<int>( t % cg ) * 4; t /= cg;
+		const int wo = static_cast<int>( t % a.ResultWidth ); t /= a.ResultWidth;
+		const int ho0 = static_cast<int>( t % a.RowChunks ) * a.RowsPerItem; t /= a.RowChunks;
+		const long long n = t;
+		const int hoEnd = min( ho0 + a.RowsPerItem, a.ResultHeight );
+		const float* image = a.From + n * a.Height * a.Width * a.Channels + c;
+		float* padded = a.Padded + n * a.ToHeight * a.ToWidth * a.Channels + c;
+		float* out = a.Result + ( ( n * a.ResultHeight + ho0 ) * a.ResultWidth + wo ) * a.Channels + c;
+		const int px0 = wo * a.StrideWidth;
+		const int columnsOwned = ( wo == a.ResultWidth - 1 ? a.ToWidth : px0 + a.StrideWidth ) - px0;
+		for( int ho = ho0; ho < hoEnd; ++ho ) {
+			const int py0 = ho * a.StrideHeight;
+			const int rowsOwned = ( ho == a.ResultHeight - 1 ? a.ToHeight : py0 + a.StrideHeight ) - py0;
+			float4 taps[3][3];
+#pragma unroll
+			for( int kh = 0; kh < 3; ++kh ) {
+#pragma unroll
+				for( int kw = 0; kw < 3; ++kw ) {
+					taps[kh][kw] = paddedPixel( a, image, py0 + kh, px0 + kw );
+				}
+			}
+			float acc[4];
+#pragma unroll
+			for( int kw = 0; kw < 3; ++kw ) {
+				float col[4];
+#pragma unroll
+				for( int kh = 0; kh < 3; ++kh ) {
+					const float v[4] = { taps[kh][kw].x, taps[kh][kw].y, taps[kh][kw].z, taps[kh][kw].w };
+#pragma unroll
+					for( int e = 0; e < 4; ++e ) {
+						if( kh == 0 ) {
+							col[e] = v[e];
+						} else if( v[e] > col[e] ) {
+							col[e] = v[e];
+						}
+					}
+				}
+#pragma unroll
+				for( int e = 0; e < 4; ++e ) {
+					if( kw == 0 ) {
+						acc[e] = col[e];
+					} else if( col[e] > acc[e] ) {
+						acc[e] = col[e];
+					}
+				}
+			}
+			*reinterpret_cast<float4*>( out ) = make_float4( acc[0], acc[1], acc[2], acc[3] );
+			out += static_cast<long long>( a.ResultWidth ) * a.Channels;
+			// the thread's own pixels of the padded image: from its window where they lie in it
+#pragma unroll
+			for( int dy = 0; dy < 3; ++dy ) {
+#pragma unroll
+				for( int dx = 0; dx < 3; ++dx ) {
+					if( dy < rowsOwned && dx < columnsOwned ) {
+						*reinterpret_cast<float4*>( padded + ( static_cast<long long>( py0 + dy ) * a.ToWidth + px0 + dx ) * a.Channels ) = taps[dy][dx];
+					}
+				}
+			}
+			if( rowsOwned > 3 || columnsOwned > 3 ) {
+				for( int dy = 0; dy < rowsOwned; ++dy ) {
+					for( int dx = 0; dx < columnsOwned; ++dx ) {
+						if( dy >= 3 || dx >= 3 ) {
+							*reinterpret_cast<float4*>( padded + ( static_cast<long long>( py0 + dy ) * a.ToWidth + px0 + dx ) * a.Channels )
+								= paddedPixel( a, image, py0 + dy, px0 + dx );
+						}
+					}
+				}
+			}
+		}
+	}
+}
+
 // Max pooling with the index output used by the backward pass. The index reproduces the reference CPU engine
 // (src/CPU/CpuMathEngineDnnPooling.cpp:40-84) exactly:
 //   - column maxima over the window rows keep the topmost row on ties (strict >);
@@ -2716,6 +2822,63 @@ static int poolingBackwardImpl( nhStream s, const nhPoolingDesc* d, const float*
 // 1.8 times ( the matrix pipe is idle otherwise: the reduction is 16 to 32 long ).
 namespace nh {
 
+// ( declared in common.h: what a stream that puts calls aside does with a padded image that waited )
+int launchPadding( hipStream_t stream, const CPendingPadding& p )
+{
+	const bool vec = p.Channels % 4 == 0 && isAligned16( p.From ) && isAligned16( p.To );
+	const long long items = p.Batch * p.ToHeight * p.ToWidth * ( vec ? p.Channels / 4 : p.Channels );
+	long long blocks = ( items + 255 ) / 256;
+	blocks = blocks > 1048576 ? 1048576 : blocks;
+	if( vec ) {
+		hipLaunchKernelGGL( resizeImageKernel<4>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, stream,
+			p.From, p.To, p.Height, p.Width, p.Channels, p.ToHeight, p.ToWidth, p.DeltaLeft, p.DeltaTop, p.Padding, p.DefaultValue, items );
+	} else {
+		hipLaunchKernelGGL( resizeImageKernel<1>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, stream,
+			p.From, p.To, p.Height, p.Width, p.Channels, p.ToHeight, p.ToWidth, p.DeltaLeft, p.DeltaTop, p.Padding, p.DefaultValue, items );
+	}
+	NH_LAUNCH_CHECK();
+	return NH_OK;
+}
+
+bool launchPaddingWithPooling( hipStream_t stream, const CPendingPadding& p, const nhPoolingDesc& d, float* result, int* rc )
+{
+	if( p.Padding != NH_PAD_CONSTANT || p.Channels % 4 != 0 || !isAligned16( p.From ) || !isAligned16( p.To ) || !isAligned16( result )
+		|| d.batch != p.Batch || d.height != p.ToHeight || d.width != p.ToWidth || d.channels != p.Channels
+		|| d.filterHeight != 3 || d.filterWidth != 3 || d.strideHeight < 1 || d.strideHeight > 3 || d.strideWidth < 1 || d.strideWidth > 3
+		|| d.resultHeight < 1 || d.resultWidth < 1 ) {
+		return false;
+	}
+	// ( the pooled image may lie anywhere but over the two images of the padding )
+	const float* padEnd = p.To + p.Batch * p.ToHeight * p.ToWidth * p.Channels;
+	const float* fromEnd = p.From + p.Batch * p.Height * p.Width * p.Channels;
+	const float* resultEnd = result + static_cast<long long>( d.batch ) * d.resultHeight * d.resultWidth * d.channels;
+	if( ( result < padEnd && p.To < resultEnd ) || ( result < fromEnd && p.From < resultEnd ) ) {
+		return false;
+	}
+	const long long perRow = static_cast<long long>( d.batch ) * d.resultWidth * ( d.channels / 4 );
+	int rowChunks = 1, rowsPerItem = 1;
+	chooseRowChunks( perRow, d.resultHeight, 4, 8192, &rowChunks, &rowsPerItem );
+	CPadPoolArgs a;
+	a.From = p.From; a.Padded = p.To; a.Result = result;
+	a.Height = p.Height; a.Width = p.Width; a.Channels = p.Channels; a.ToHeight = p.ToHeight; a.ToWidth = p.ToWidth;
+	a.DeltaTop = p.DeltaTop; a.DeltaLeft = p.DeltaLeft; a.DefaultValue = p.DefaultValue;
+	a.StrideHeight = d.strideHeight; a.StrideWidth = d.strideWidth; a.ResultHeight = d.resultHeight; a.ResultWidth = d.resultWidth;
+	a.RowChunks = rowChunks; a.RowsPerItem = rowsPerItem;
+	a.TotalItems = perRow * rowChunks;
+	long long blocks = ( a.TotalItems + 255 ) / 256;
+	blocks = blocks > 1048576 ? 1048576 : blocks;
+	hipLaunchKernelGGL( padMaxPool3x3Kernel, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, stream, a );
+	const hipError_t launched = hipGetLastError();
+	if( launched != hipSuccess ) {
+		setLastError( hipGetErrorString( launched ) );
+		*rc = NH_ERR_HIP;
+	} else {
+		*rc = NH_OK;
+	}
+	return true;
+}
+
+
 typedef float expandAcc __attribute__( ( ext_vector_type( 16 ) ) );
 
 // CLIPPED: both activations are ReLU with an upper threshold ( ReLU6, what MobileNetV2 uses ): two instructions per value
@@ -3048,6 +3211,10 @@ int nhBlobMaxPooling( nhStream s, const nhPoolingDesc* d, const float* source, i
 	}
 	NH_REQUIRE( source != nullptr && result != nullptr );
 	if( maxIndices == nullptr ) {
+		int fused = NH_OK;
+		if( __atomic_load_n( &tinyChainsPending, __ATOMIC_RELAXED ) != 0 && fusePendingPadding( s, *d, source, result, &fused ) ) {
+			return fused; // ( the padded image that waited for this call went out with it )
+		}
 		return poolingImpl<false>( s, d, source, result );
 	}
 	const long long total = static_cast<long long>( d->batch ) * d->resultHeight * d->resultWidth * d->channels;
@@ -3245,19 +3412,16 @@ int nhBlobResizeImage( nhStream s, const nhBlobDesc* from, const float* fromData
 	if( batch == 0 ) {
 		return NH_OK;
 	}
-	const bool vec = channels % 4 == 0 && isAligned16( fromData ) && isAligned16( toData );
-	const long long items = batch * toHeight * toWidth * ( vec ? channels / 4 : channels );
-	long long blocks = ( items + 255 ) / 256;
-	blocks = blocks > 1048576 ? 1048576 : blocks;
-	if( vec ) {
-		hipLaunchKernelGGL( resizeImageKernel<4>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
-			fromData, toData, height, width, channels, toHeight, toWidth, deltaLeft, deltaTop, padding, defaultValue, items );
-	} else {
-		hipLaunchKernelGGL( resizeImageKernel<1>, dim3( static_cast<unsigned>( blocks ) ), dim3( 256 ), 0, toStream( s ),
-			fromData, toData, height, width, channels, toHeight, toWidth, deltaLeft, deltaTop, padding, defaultValue, items );
+	CPendingPadding p;
+	p.From = fromData; p.To = toData; p.Batch = batch;
+	p.Height = height; p.Width = width; p.Channels = channels; p.ToHeight = toHeight; p.ToWidth = toWidth;
+	p.DeltaLeft = deltaLeft; p.DeltaTop = deltaTop; p.Padding = padding; p.DefaultValue = defaultValue;
+	// ( on a stream that puts calls aside a border of constants waits for the pooling over the padded image )
+	if( padding == NH_PAD_CONSTANT && deltaLeft >= 0 && deltaRight >= 0 && deltaTop >= 0 && deltaBottom >= 0 && channels % 4 == 0
+		&& isAligned16( fromData ) && isAligned16( toData ) && deferPadding( s, p ) ) {
+		return NH_OK;
 	}
-	NH_LAUNCH_CHECK();
-	return NH_OK;
+	return launchPadding( toStream( s ), p );
 }
 
 int nhBlobMergeByDim( nhStream s, int dim, const nhBlobDesc* from, const float* const* fromData, int fromCount,

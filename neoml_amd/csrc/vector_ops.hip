@@ -831,8 +831,9 @@ struct CTinyQueue {
 	CPendingConvolution Convolution;
 	CPendingSum Sum;
 	CPendingBatched Batched;
+	CPendingPadding Padding;
 
-	bool LaunchWaits() const { return Product.Pending || Convolution.Pending || Sum.Pending || Batched.Pending; }
+	bool LaunchWaits() const { return Product.Pending || Convolution.Pending || Sum.Pending || Batched.Pending || Padding.Pending; }
 };
 
 static int launchPlainSum( hipStream_t stream, const CPendingSum& sum );
@@ -873,8 +874,9 @@ static bool launchTinyChain( hipStream_t stream, CTinyQueue& queue )
 	if( chain.Length == 0 ) {
 		return false;
 	}
-	if( chain.Length == 1 && chain.Ops[0].Count > TinyWideMaxCount
-		&& ( chain.Ops[0].Spread != TS_None ? queue.FirstSpreadAlone != nullptr : queue.FirstAlone != nullptr ) ) {
+	// ( a call that nothing has joined goes out as the launch it would have been on any other stream: the large ones for
+	// their kernels' rates, the small ones because a chain's launch takes 5 us where theirs takes 4 )
+	if( chain.Length == 1 && ( chain.Ops[0].Spread != TS_None ? queue.FirstSpreadAlone != nullptr : queue.FirstAlone != nullptr ) ) {
 		const CTinyOp op = chain.Ops[0];
 		chain.Length = 0;
 		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
@@ -939,6 +941,13 @@ static bool launchPending( hipStream_t stream, CTinyQueue& queue )
 		queue.Batched.Pending = false;
 		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
 		( void )launchBatched( stream, p, nullptr, nullptr );
+		return true;
+	}
+	if( queue.Padding.Pending ) {
+		const CPendingPadding p = queue.Padding;
+		queue.Padding.Pending = false;
+		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+		( void )launchPadding( stream, p );
 		return true;
 	}
 	if( queue.Sum.Pending ) {
@@ -1085,6 +1094,56 @@ bool fusePendingProduct( nhStream s, const float* matrix, float* result, int hei
 		noteStreamUse( stream );
 	}
 	return true;
+}
+
+bool deferPadding( nhStream s, const CPendingPadding& padding )
+{
+	if( __atomic_load_n( &tinyDeferringStreams, __ATOMIC_RELAXED ) == 0 ) {
+		return false;
+	}
+	const hipStream_t stream = toStream( s ); // ( what the stream holds goes out first )
+	int device = 0;
+	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+	if( hipGetDevice( &device ) != hipSuccess || hipStreamIsCapturing( stream, &capture ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return false;
+	}
+	if( capture != hipStreamCaptureStatusNone ) {
+		return false;
+	}
+	std::lock_guard<std::recursive_mutex> guard( tinyLock );
+	auto found = tinyQueues().find( std::make_pair( device, stream ) );
+	if( found == tinyQueues().end() || !found->second.Enabled || found->second.Chain.Length != 0 || found->second.LaunchWaits() ) {
+		return false;
+	}
+	found->second.Padding = padding;
+	found->second.Padding.Pending = true;
+	__atomic_fetch_add( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+	return true;
+}
+
+// BlobMaxPooling ( no indices ) asks whether it is the call a padded image waits for. true: both have been launched as one.
+bool fusePendingPadding( nhStream s, const nhPoolingDesc& d, const float* source, float* result, int* rc )
+{
+	const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
+	int device = 0;
+	if( hipGetDevice( &device ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return false;
+	}
+	std::lock_guard<std::recursive_mutex> guard( tinyLock );
+	auto found = tinyQueues().find( std::make_pair( device, stream ) );
+	if( found == tinyQueues().end() || !found->second.Padding.Pending || found->second.Padding.To != source ) {
+		return false; // ( the caller's own launch sends the padding out first )
+	}
+	const CPendingPadding p = found->second.Padding;
+	found->second.Padding.Pending = false;
+	__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+	if( launchPaddingWithPooling( stream, p, d, result, rc ) ) {
+		return true;
+	}
+	( void )launchPadding( stream, p ); // ( not a pair for one launch: the padding as it was asked for, the pooling is the caller's )
+	return false;
 }
 
 bool deferBatchedProduct( nhStream s, int batch, const float* first, int height, int width, const float* second, int secondWidth,

@@ -654,3 +654,79 @@ def test_passes_over_a_matrix_with_vectors_spread_over_it(streams):
                 v = x0[o:o + n].astype(np.float64).reshape(rows, width)
                 ref = (v - v.mean(1, keepdims=True)) / np.sqrt(v.var(1, keepdims=True) + 1e-5) * scale0 + bias0
                 assert np.allclose(results[1][1][o:o + n].reshape(rows, width), ref, rtol=1e-4, atol=1e-4)
+
+
+def test_padded_image_waits_for_its_pooling(streams):
+    """nhBlobResizeImage that pads with a constant, followed by nhBlobMaxPooling 3x3 over the padded blob (CImageResizeLayer +
+    CMaxPoolingLayer: how a ResNet's first pooling gets its border), is one launch that writes both blobs. Same bits in
+    both as the two launches leave, for strides 1 to 3, borders of 0 to 2 pixels of any constant (above and below the
+    image's values), image sizes that leave rows and columns behind the last window, NaN in the image; any other successor
+    finds the padded blob done."""
+    import torch
+    lib, na = streams.lib, streams.na
+    g = rng(4900)
+    dev = streams.dev
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    def blob(n, h, w, c):
+        return na.BlobDesc.of(1, n, 1, h, w, 1, c)
+
+    cases = (
+        # batch, height, width, channels, (left, right, top, bottom), constant, filter, stride
+        (4, 24, 24, 64, (1, 1, 1, 1), 0.0, 3, 2),
+        (3, 17, 23, 8, (1, 1, 1, 1), -100.0, 3, 2),
+        (2, 16, 21, 12, (2, 0, 0, 2), 7.5, 3, 3),
+        (2, 9, 12, 4, (0, 1, 2, 1), 0.25, 3, 1),
+        (1, 7, 7, 16, (0, 0, 0, 0), 0.0, 3, 2),
+        (2, 12, 12, 8, (1, 1, 1, 1), 0.0, 2, 2),      # not a 3 x 3 window: two launches as ever
+        (2, 12, 12, 6, (1, 1, 1, 1), 0.0, 3, 2),      # channels not a multiple of four: two launches as ever
+    )
+    for n, h, w, c, (dl, dr, dt, db), value, f, stride in cases:
+        image = g.normal(0, 2, (n, h, w, c)).astype(np.float32)
+        image[0, 0, 0, 0] = np.nan
+        image[0, h // 2, w // 2, c - 1] = np.nan
+        th, tw = h + dt + db, w + dl + dr
+        pool = na.PoolingDesc(n, th, tw, c, f, f, stride, stride, 0, 0)
+        na.check(lib.nhInitPooling(ctypes.byref(pool)))
+        rh, rw = pool.resultHeight, pool.resultWidth
+        src, dst = blob(n, h, w, c), blob(n, th, tw, c)
+
+        def run(stream, successor):
+            d_image = up(image)
+            padded = torch.full((n * th * tw * c,), -7.0, device=dev)
+            pooled = torch.full((n * rh * rw * c,), -7.0, device=dev)
+            torch.cuda.synchronize()
+            na.check(lib.nhBlobResizeImage(stream, ctypes.byref(src), P(d_image), dl, dr, dt, db, 0, ctypes.c_float(value),
+                                           ctypes.byref(dst), P(padded)))
+            successor(stream, padded, pooled)
+            na.check(lib.nhStreamSynchronize(stream))
+            return padded.cpu().numpy(), pooled.cpu().numpy()
+
+        def pooling(s, padded, pooled):
+            na.check(lib.nhBlobMaxPooling(s, ctypes.byref(pool), P(padded), None, P(pooled)))
+
+        def pooling_with_indices(s, padded, pooled):
+            indices = torch.zeros(n * rh * rw * c, dtype=torch.int32, device=dev)
+            na.check(lib.nhBlobMaxPooling(s, ctypes.byref(pool), P(padded), P(indices), P(pooled)))
+
+        def mean_pooling(s, padded, pooled):
+            na.check(lib.nhBlobMeanPooling(s, ctypes.byref(pool), P(padded), P(pooled)))
+
+        def nothing(s, padded, pooled):
+            pass
+
+        def small_call(s, padded, pooled):
+            na.check(lib.nhVectorNeg(s, P(padded), P(pooled), 16))
+
+        for successor in (pooling, pooling_with_indices, mean_pooling, nothing, small_call):
+            want = run(streams.plain, successor)
+            got = run(streams.deferring, successor)
+            assert same_bits(got[0], want[0]) and same_bits(got[1], want[1]), (successor.__name__, n, h, w, c, stride)
+        # and the padded blob is the image inside its border
+        padded, pooled = run(streams.deferring, pooling)
+        padded = padded.reshape(n, th, tw, c)
+        assert same_bits(np.ascontiguousarray(padded[:, dt:dt + h, dl:dl + w, :]), image)
+        border = np.ones((th, tw), bool)
+        border[dt:dt + h, dl:dl + w] = False
+        assert np.all(padded[:, border, :] == np.float32(value))

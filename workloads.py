@@ -416,6 +416,9 @@ class LaunchPlan:
                 if tag and (tag.startswith("conv") or tag in ("depthwise", "add")) and j < len(launches) and launches[j][2] == "relu":
                     # the activation in place behind a convolution or a sum: on such a stream it is that call's own launch
                     flops, nbytes, j = flops + launches[j][3], nbytes + launches[j][4], j + 1
+                if tag == "pad" and j < len(launches) and launches[j][2] == "maxpool":
+                    # the pooling over a padded image: one launch with the padding on such a stream
+                    flops, nbytes, j = flops + launches[j][3], nbytes + launches[j][4], j + 1
                 if pool[i] is not None:
                     record(pool[i][0], stream)
                 for fn, args, _, _, _ in launches[i:j]:
