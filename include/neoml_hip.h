@@ -455,7 +455,7 @@ NH_API int nhStreamOverlapLstm(nhStream s, int enable);
  * layer's two calls ask (NeoML/src/Dnn/Layers/FullyConnectedLayer.cpp:91-99); any other call launches the product first,
  * as it was asked for. The sum is the same; where the product is cut into slices of its reduction the vector is added
  * in front of the slices instead of behind them, i.e. the last bits may differ from the two launches'.
- * In the same way nhBlobConvolution and nhBlobChannelwiseConvolution wait for an nhVectorReLU over their result in place
+ * In the same way nhBlobConvolution and nhBlobChannelwiseConvolution wait for an nhVectorReLU or nhVectorHSwish over their result in place
  * (CConvLayer / CChannelwiseConvLayer followed by CReLULayer: the activation runs on the accumulators' way out, its
  * threshold read from the device scalar), and an nhVectorAdd over more than 262144 elements waits for an nhVectorReLU
  * over the sum in place (CEltwiseSumLayer + CReLULayer at the end of a residual block: one pass), and

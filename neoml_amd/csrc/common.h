@@ -66,7 +66,8 @@ bool deferBatchedProduct( nhStream s, int batch, const float* first, int height,
 // result in place that follows it in most networks.
 bool deferConvolution( nhStream s, bool channelwise, const nhConvDesc& d, const float* source, const float* filter,
 	const float* freeTerm, float* result );
-bool fusePendingConvolution( nhStream s, const float* first, float* result, long long count, const float* upperThreshold, int* rc );
+bool fusePendingConvolution( nhStream s, const float* first, float* result, long long count, int activation,
+	const float* upperThreshold, int* rc );
 
 inline hipStream_t toStream( nhStream s )
 {

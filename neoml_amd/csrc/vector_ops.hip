@@ -1317,7 +1317,8 @@ bool deferConvolution( nhStream s, bool channelwise, const nhConvDesc& d, const 
 	return true;
 }
 
-bool fusePendingConvolution( nhStream s, const float* first, float* result, long long count, const float* upperThreshold, int* rc )
+bool fusePendingConvolution( nhStream s, const float* first, float* result, long long count, int activation,
+	const float* upperThreshold, int* rc )
 {
 	const hipStream_t stream = reinterpret_cast<hipStream_t>( s );
 	int device = 0;
@@ -1334,14 +1335,14 @@ bool fusePendingConvolution( nhStream s, const float* first, float* result, long
 		}
 		c = found->second.Convolution;
 		const long long resultCount = static_cast<long long>( c.Desc.batch ) * c.Desc.resultHeight * c.Desc.resultWidth * c.Desc.filterCount;
-		if( first != c.Result || result != c.Result || count != resultCount || upperThreshold == nullptr ) {
+		if( first != c.Result || result != c.Result || count != resultCount || ( activation == NH_ACT_RELU && upperThreshold == nullptr ) ) {
 			return false; // ( the caller's own launch sends the convolution out first, as it was asked for )
 		}
 		found->second.Convolution.Pending = false;
 		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
 	}
-	const CFusedActivation relu = { NH_ACT_RELU, 0.f, upperThreshold };
-	*rc = launchDeferredConvolution( stream, c.Channelwise, c.Desc, c.Source, c.Filter, c.FreeTerm, c.Result, relu );
+	const CFusedActivation act = { activation, 0.f, activation == NH_ACT_RELU ? upperThreshold : nullptr };
+	*rc = launchDeferredConvolution( stream, c.Channelwise, c.Desc, c.Source, c.Filter, c.FreeTerm, c.Result, act );
 	if( __atomic_load_n( &lstmPartnersAwaited, __ATOMIC_RELAXED ) != 0 ) {
 		noteStreamUse( stream );
 	}
@@ -1752,7 +1753,7 @@ extern "C" int nhVectorReLU( nhStream s, const float* first, float* result, int 
 	NH_REQUIRE( upperThreshold != nullptr );
 	int rc = NH_OK;
 	if( first == result && __atomic_load_n( &tinyChainsPending, __ATOMIC_RELAXED ) != 0
-		&& ( fusePendingConvolution( s, first, result, vectorSize, upperThreshold, &rc )
+		&& ( fusePendingConvolution( s, first, result, vectorSize, NH_ACT_RELU, upperThreshold, &rc )
 			|| fusePendingSum( s, first, result, vectorSize, upperThreshold, &rc ) ) )
 	{
 		return rc; // ( the convolution or the sum that waited for this call took the activation with it )
@@ -1787,7 +1788,16 @@ extern "C" int nhVectorMinMax( nhStream s, const float* first, float* result, in
 	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, op );
 }
 
-NH_UNARY( nhVectorHSwish, CHSwishOp )
+extern "C" int nhVectorHSwish( nhStream s, const float* first, float* result, int vectorSize )
+{
+	// ( in place behind a convolution that waits for its successor: the convolution's launch applies it, as it does a ReLU )
+	int rc = NH_OK;
+	if( first == result && first != nullptr && __atomic_load_n( &tinyChainsPending, __ATOMIC_RELAXED ) != 0
+		&& fusePendingConvolution( s, first, result, vectorSize, NH_ACT_HSWISH, nullptr, &rc ) ) {
+		return rc;
+	}
+	return launchEltwise<1, float, float>( s, first, (const float*)nullptr, (const float*)nullptr, result, vectorSize, CHSwishOp() );
+}
 NH_UNARY( nhVectorAbs, CAbsOp )
 NH_UNARY( nhVectorHardTanh, CHardTanhOp )
 NH_UNARY( nhVectorNeg, CNegOp )

@@ -375,6 +375,17 @@ def test_convolution_waits_for_its_relu(streams):
                 outs.append(y.cpu().numpy())
             assert same_bits(outs[0], outs[1]), (n, h, w, cin, cout, f, pad, stride, float(threshold[0]))
             assert outs[1].min() >= 0.0 and (float(threshold[0]) == 0.0 or outs[1].max() <= 6.0)
+        # VectorHSwish in place is taken along in the same way
+        outs = []
+        for stream in (streams.plain, streams.deferring):
+            y = torch.zeros(shape, device=dev)
+            d_x4 = up(x * 4)  # ( values on both sides of -3 and 3 )
+            torch.cuda.synchronize()
+            na.check(lib.nhBlobConvolution(stream, ctypes.byref(d), P(d_x4), P(d_f), P(d_b), P(y)))
+            na.check(lib.nhVectorHSwish(stream, P(y), P(y), y.numel()))
+            na.check(lib.nhStreamSynchronize(stream))
+            outs.append(y.cpu().numpy())
+        assert same_bits(outs[0], outs[1]), ("h-swish", n, h, w, cin, cout, f, pad, stride)
     for n, h, w, c, stride in ((8, 56, 56, 144, 1), (8, 112, 112, 96, 2), (3, 9, 7, 6, 1)):
         x = g.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
         filt = g.normal(0, 1.0 / 3, (3, 3, c)).astype(np.float32)
@@ -391,6 +402,16 @@ def test_convolution_waits_for_its_relu(streams):
             na.check(lib.nhStreamSynchronize(stream))
             outs.append(y.cpu().numpy())
         assert same_bits(outs[0], outs[1]), ("channelwise", n, h, w, c, stride)
+        outs = []
+        for stream in (streams.plain, streams.deferring):
+            y = torch.zeros((n, d.resultHeight, d.resultWidth, c), device=dev)
+            d_x4 = up(x * 6)
+            torch.cuda.synchronize()
+            na.check(lib.nhBlobChannelwiseConvolution(stream, ctypes.byref(d), P(d_x4), P(d_f), P(d_b), P(y)))
+            na.check(lib.nhVectorHSwish(stream, P(y), P(y), y.numel()))
+            na.check(lib.nhStreamSynchronize(stream))
+            outs.append(y.cpu().numpy())
+        assert same_bits(outs[0], outs[1]), ("channelwise h-swish", n, h, w, c, stride)
     # other successors
     n, h, w, cin, cout = 4, 28, 28, 32, 64
     x = g.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
