@@ -519,6 +519,11 @@ def test_large_calls_of_one_count_go_as_one_pass(streams):
         na.check(lib.nhVectorSigmoid(s, P(y, o), P(y, o), n))
         na.check(lib.nhVectorEltwiseMultiply(s, P(x, o), P(y, o), P(x, o), n))
 
+    def gelu_into_a_third(s, x, y, z, n, o):
+        na.check(lib.nhVectorMultiply(s, P(x, o), P(y, o), n, P(scale)))
+        na.check(lib.nhVectorSigmoid(s, P(y, o), P(y, o), n))
+        na.check(lib.nhVectorEltwiseMultiply(s, P(y, o), P(x, o), P(z, o), n))
+
     def solver(s, x, y, z, n, o):
         # x: parameters, y: their gradient, z: the moving mean of the steps
         na.check(lib.nhVectorMultiply(s, P(z, o), P(z, o), n, P(moment)))
@@ -546,7 +551,7 @@ def test_large_calls_of_one_count_go_as_one_pass(streams):
 
     total = 3 * 1000 * 1000 + 16
     data = [g.normal(0, 2, total).astype(np.float32) for _ in range(3)]
-    for what in (gelu_layer, gelu_over_input, solver, two_counts, shifted, alone):
+    for what in (gelu_layer, gelu_over_input, gelu_into_a_third, solver, two_counts, shifted, alone):
         for n, o in ((3 * 1000 * 1000, 0), (3 * 1000 * 1000, 4), (3 * 1000 * 1000 + 2, 0), (3 * 1000 * 1000, 3), (262148, 8)):
             results = []
             for stream in (streams.plain, streams.deferring):
@@ -641,6 +646,24 @@ def test_passes_over_a_matrix_with_vectors_spread_over_it(streams):
         na.check(lib.nhBatchMultiplyMatrixByDiagMatrix(s, 1, P(out, o), rows, width, 0, P(scale), 0, P(out, o), n))
         na.check(lib.nhAddVectorToMatrixRows(s, 1, P(out, o), P(out, o), rows, width, P(bias)))
 
+    def tail_into_two_blobs(s, x, out, sq, neg_mean, inv_std, scale, bias, inv_w, eps, rows, width, o):
+        # the layer with a blob of its own for the normalised input ( what it keeps for the backward pass ), and in place
+        n = rows * width
+        na.check(lib.nhSumMatrixColumns(s, P(neg_mean), P(x, o), rows, width))
+        na.check(lib.nhSumMatrixColumns(s, P(inv_std), P(x, o + 1), rows, width - 1))
+        na.check(lib.nhAddVectorToMatrixColumns(s, P(x, o), P(sq, o), rows, width, P(neg_mean)))
+        na.check(lib.nhMultiplyDiagMatrixByMatrix(s, P(inv_std), rows, P(sq, o), width, P(sq, o), n))
+        na.check(lib.nhBatchMultiplyMatrixByDiagMatrix(s, 1, P(sq, o), rows, width, 0, P(scale), 0, P(out, o), n))
+        na.check(lib.nhAddVectorToMatrixRows(s, 1, P(out, o), P(out, o), rows, width, P(bias)))
+        na.check(lib.nhSumMatrixColumns(s, P(neg_mean), P(out, o), rows, width))
+        na.check(lib.nhAddVectorToMatrixColumns(s, P(x, o), P(x, o), rows, width, P(neg_mean)))
+        na.check(lib.nhMultiplyDiagMatrixByMatrix(s, P(inv_std), rows, P(x, o), width, P(x, o), n))
+        na.check(lib.nhBatchMultiplyMatrixByDiagMatrix(s, 1, P(x, o), rows, width, 0, P(scale), 0, P(x, o), n))
+        na.check(lib.nhAddVectorToMatrixRows(s, 1, P(x, o), P(x, o), rows, width, P(bias)))
+        na.check(lib.nhSumMatrixColumns(s, P(inv_std), P(x, o), rows, width))
+        na.check(lib.nhAddVectorToMatrixColumns(s, P(out, o), P(out, o), rows, width, P(inv_std)))
+        na.check(lib.nhVectorEltwiseMultiply(s, P(out, o), P(out, o), P(out, o), n))
+
     def other_orders(s, x, out, sq, neg_mean, inv_std, scale, bias, inv_w, eps, rows, width, o):
         n = rows * width
         na.check(lib.nhSumMatrixColumns(s, P(neg_mean), P(x, o), rows, width))
@@ -658,7 +681,7 @@ def test_passes_over_a_matrix_with_vectors_spread_over_it(streams):
         n = rows * width
         x0 = g.normal(0.3, 1.5, n + 8).astype(np.float32)
         scale0, bias0 = g.normal(1, 0.2, width).astype(np.float32), g.normal(0, 0.5, width).astype(np.float32)
-        for what in (layer, other_orders):
+        for what in (layer, tail_into_two_blobs, other_orders):
             results = []
             for stream in (streams.plain, streams.deferring):
                 x, scale, bias = up(x0), up(scale0), up(bias0)
