@@ -969,6 +969,49 @@ __global__ __launch_bounds__( 256 ) void normalizeChainKernel( const float* x, f
 	}
 }
 
+// The passes of CDnnSimpleGradientSolver::TrainLayer over one parameter blob ( NeoML/src/Dnn/DnnSolver.cpp:481-507 ):
+// history *= moment; history += gradient * rate; with L2 regularisation history += parameters * decay; parameters += history
+__global__ __launch_bounds__( 256 ) void momentumChainKernel( float* parameters, const float* gradient, float* history,
+	const float* moment, const float* rate, const float* decay, int quads )
+{
+	CMulValueOp<float> byMoment; byMoment.Ptr = moment; byMoment.prepare();
+	CMultiplyAndAddOp step; step.Ptr = rate; step.prepare();
+	CMultiplyAndAddOp regularise; regularise.Ptr = decay != nullptr ? decay : rate; regularise.prepare();
+	const CAddOp<float> sum;
+	const int base = blockIdx.x * ( 256 * KnownQuads ) + threadIdx.x;
+	float4 p[KnownQuads], g[KnownQuads], h[KnownQuads];
+#pragma unroll
+	for( int u = 0; u < KnownQuads; ++u ) {
+		const int i = base + u * 256;
+		if( i < quads ) {
+			p[u] = reinterpret_cast<const float4*>( parameters )[i];
+			g[u] = reinterpret_cast<const float4*>( gradient )[i];
+			h[u] = reinterpret_cast<const float4*>( history )[i];
+		}
+	}
+#pragma unroll
+	for( int u = 0; u < KnownQuads; ++u ) {
+		const int i = base + u * 256;
+		if( i < quads ) {
+			const float pv[4] = { p[u].x, p[u].y, p[u].z, p[u].w };
+			const float gv[4] = { g[u].x, g[u].y, g[u].z, g[u].w };
+			float hv[4] = { h[u].x, h[u].y, h[u].z, h[u].w };
+			float moved[4];
+#pragma unroll
+			for( int e = 0; e < 4; ++e ) {
+				hv[e] = byMoment( hv[e], 0.f, 0.f );
+				hv[e] = step( hv[e], gv[e], 0.f );
+				if( decay != nullptr ) {
+					hv[e] = regularise( hv[e], pv[e], 0.f );
+				}
+				moved[e] = sum( pv[e], hv[e], 0.f );
+			}
+			reinterpret_cast<float4*>( history )[i] = make_float4( hv[0], hv[1], hv[2], hv[3] );
+			reinterpret_cast<float4*>( parameters )[i] = make_float4( moved[0], moved[1], moved[2], moved[3] );
+		}
+	}
+}
+
 template<typename F> static bool isKind( const CTinyOp& op ) { return op.Kind == CKindOf<F, CTinyKinds>::Value; }
 
 // A chain of calls of one count on 16-byte boundaries without barriers: true if it was one of the known sequences ( launched )
@@ -997,6 +1040,25 @@ static bool launchKnownChain( hipStream_t stream, const CTinyChain& chain )
 		if( op[1].In[0] == y && op[1].Out == y && op[2].In[0] == y && op[3].In[0] == out && op[3].Out == out ) {
 			hipLaunchKernelGGL( normalizeChainKernel<false>, grid, dim3( 256 ), 0, stream, op[0].In[0], y, out, op[0].In[1], op[1].In[1],
 				op[2].In[1], op[3].In[1], op[0].Width, quads );
+			return true;
+		}
+		return false;
+	}
+	if( ( chain.Length == 3 || chain.Length == 4 ) && isKind<CMulValueOp<float>>( op[0] ) && isKind<CMultiplyAndAddOp>( op[1] )
+		&& isKind<CAddOp<float>>( op[chain.Length - 1] ) && ( chain.Length == 3 || isKind<CMultiplyAndAddOp>( op[2] ) ) ) {
+		const CTinyOp& last = op[chain.Length - 1];
+		float* history = op[0].Out;
+		float* parameters = last.Out;
+		const float* gradient = op[1].In[1];
+		bool known = op[0].In[0] == history && op[1].In[0] == history && op[1].Out == history && last.Spread == TS_None
+			&& ( ( last.In[0] == parameters && last.In[1] == history ) || ( last.In[0] == history && last.In[1] == parameters ) )
+			&& parameters != history && gradient != history && gradient != parameters;
+		if( chain.Length == 4 ) {
+			known = known && op[2].In[0] == history && op[2].In[1] == parameters && op[2].Out == history;
+		}
+		if( known ) {
+			hipLaunchKernelGGL( momentumChainKernel, grid, dim3( 256 ), 0, stream, parameters, gradient, history, op[0].Scalar, op[1].Scalar,
+				chain.Length == 4 ? op[2].Scalar : static_cast<const float*>( nullptr ), quads );
 			return true;
 		}
 		return false;

@@ -531,6 +531,20 @@ def test_large_calls_of_one_count_go_as_one_pass(streams):
         na.check(lib.nhVectorMultiplyAndAdd(s, P(z, o), P(y, o), P(z, o), n, P(rate)))
         na.check(lib.nhVectorAdd(s, P(x, o), P(z, o), P(x, o), n))
 
+    def momentum_solver(s, x, y, z, n, o):
+        # the order of CDnnSimpleGradientSolver::TrainLayer (NeoML/src/Dnn/DnnSolver.cpp:481-507) with L2 regularisation
+        na.check(lib.nhVectorMultiply(s, P(z, o), P(z, o), n, P(moment)))
+        na.check(lib.nhVectorMultiplyAndAdd(s, P(z, o), P(y, o), P(z, o), n, P(rate)))
+        na.check(lib.nhVectorMultiplyAndAdd(s, P(z, o), P(x, o), P(z, o), n, P(decay)))
+        na.check(lib.nhVectorAdd(s, P(x, o), P(z, o), P(x, o), n))
+
+    def momentum_solver_plain(s, x, y, z, n, o):
+        # ... and without it, twice in a row ( two steps )
+        for _ in range(2):
+            na.check(lib.nhVectorMultiply(s, P(z, o), P(z, o), n, P(moment)))
+            na.check(lib.nhVectorMultiplyAndAdd(s, P(z, o), P(y, o), P(z, o), n, P(rate)))
+            na.check(lib.nhVectorAdd(s, P(z, o), P(x, o), P(x, o), n))
+
     def two_counts(s, x, y, z, n, o):
         # a call of another count, and a small one, between calls of one count: each run goes out before the next begins
         na.check(lib.nhVectorMultiply(s, P(x, o), P(y, o), n, P(scale)))
@@ -551,7 +565,8 @@ def test_large_calls_of_one_count_go_as_one_pass(streams):
 
     total = 3 * 1000 * 1000 + 16
     data = [g.normal(0, 2, total).astype(np.float32) for _ in range(3)]
-    for what in (gelu_layer, gelu_over_input, gelu_into_a_third, solver, two_counts, shifted, alone):
+    for what in (gelu_layer, gelu_over_input, gelu_into_a_third, solver, momentum_solver, momentum_solver_plain, two_counts, shifted,
+                 alone):
         for n, o in ((3 * 1000 * 1000, 0), (3 * 1000 * 1000, 4), (3 * 1000 * 1000 + 2, 0), (3 * 1000 * 1000, 3), (262148, 8)):
             results = []
             for stream in (streams.plain, streams.deferring):
