@@ -516,7 +516,11 @@ struct CTinyOp {
 	// ( TS_PerRow: In[1][i / Width], AddVectorToMatrixColumns, MultiplyDiagMatrixByMatrix ) or per column ( TS_PerColumn:
 	// In[1][i % Width], AddVectorToMatrixRows, MultiplyMatrixByDiagMatrix ). Only calls over more than TinyWideMaxCount
 	// elements come with one, so a chain with barriers never holds any.
-	int Spread;
+	short Spread;
+	// The result is not stored: a later call of the chain writes the same elements, and every call in between that reads
+	// them has them in registers ( chains without barriers whose calls all have one count; set when the chain is launched ).
+	// NeoML's blobs of gradients are cleared, copied into, copied out of and cleared again in one run of calls.
+	short Dead;
 	int Width;
 };
 
@@ -720,7 +724,7 @@ template<int V, int Q> __device__ __forceinline__ void runStraightChain( const C
 		const bool overHeld = op.Out == heldIn;
 #pragma unroll
 		for( int u = 0; u < Q; ++u ) {
-			if( mine[u] ) {
+			if( mine[u] && op.Dead == 0 ) {
 				float* to = op.Out + first + static_cast<long long>( u ) * stride;
 				if( V == 4 ) {
 					*reinterpret_cast<float4*>( to ) = make_float4( lastValue[u * V], lastValue[u * V + 1], lastValue[u * V + 2], lastValue[u * V + 3] );
@@ -1096,15 +1100,39 @@ static bool launchTinyChain( hipStream_t stream, CTinyQueue& queue )
 		}
 		return true;
 	}
-	bool barrier = false, quads = true;
+	bool barrier = false, quads = true, oneCount = true;
 	int longest = 0;
 	for( int k = 0; k < chain.Length; ++k ) {
-		const CTinyOp& op = chain.Ops[k];
+		CTinyOp& op = chain.Ops[k];
+		op.Dead = 0;
 		barrier = barrier || op.Barrier != 0;
+		oneCount = oneCount && op.Count == chain.Ops[0].Count;
 		longest = op.Count > longest ? op.Count : longest;
 		quads = quads && op.Count == chain.Ops[0].Count && op.Count % 4 == 0 && isAligned16( op.Out )
 			&& isAligned16( op.In[0] ) && isAligned16( op.In[1] ) && isAligned16( op.In[2] )
 			&& ( op.Spread == TS_None || op.Width % 4 == 0 );
+	}
+	if( !barrier && oneCount ) {
+		// results that a later call overwrites before anything reads them from memory: the kernel's thread takes an operand from
+		// a register if the call in front wrote it, or if it is what the first call read ( runStraightChain )
+		const float* held = chain.Ops[0].In[0];
+		for( int k = 0; k + 1 < chain.Length; ++k ) {
+			const float* out = chain.Ops[k].Out;
+			for( int j = k + 1; j < chain.Length; ++j ) {
+				const CTinyOp& later = chain.Ops[j];
+				bool readsFromMemory = false;
+				for( int i = 0; i < 3; ++i ) {
+					readsFromMemory = readsFromMemory || ( later.In[i] == out && j != k + 1 && out != held );
+				}
+				if( readsFromMemory ) {
+					break;
+				}
+				if( later.Out == out ) {
+					chain.Ops[k].Dead = 1;
+					break;
+				}
+			}
+		}
 	}
 	if( !barrier && quads && longest > TinyOpMaxCount ) {
 		if( !launchKnownChain( stream, chain ) ) {

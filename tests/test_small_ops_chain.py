@@ -545,6 +545,29 @@ def test_large_calls_of_one_count_go_as_one_pass(streams):
             na.check(lib.nhVectorMultiplyAndAdd(s, P(z, o), P(y, o), P(z, o), n, P(rate)))
             na.check(lib.nhVectorAdd(s, P(z, o), P(x, o), P(x, o), n))
 
+    def gradient_blob(s, x, y, z, n, o):
+        # how NeoML's layers treat a blob of gradients: cleared, copied into, copied out of, cleared again. Only the last
+        # value of z and the copy in y need to reach memory.
+        na.check(lib.nhVectorFill(s, P(z, o), ctypes.c_float(0.0), n))
+        na.check(lib.nhVectorCopy(s, P(z, o), P(x, o), n))
+        na.check(lib.nhVectorCopy(s, P(y, o), P(z, o), n))
+        na.check(lib.nhVectorFill(s, P(z, o), ctypes.c_float(0.0), n))
+
+    def overwritten_but_read_from_memory(s, x, y, z, n, o):
+        # z is overwritten by the last call, but the call in front of that reads it, and not from a register: it must be there
+        na.check(lib.nhVectorCopy(s, P(z, o), P(y, o), n))
+        na.check(lib.nhVectorNeg(s, P(x, o), P(x, o), n))
+        na.check(lib.nhVectorAbs(s, P(z, o), P(x, o), n))
+        na.check(lib.nhVectorFill(s, P(z, o), ctypes.c_float(0.5), n))
+
+    def overwritten_and_read_from_a_register(s, x, y, z, n, o):
+        # x is what the first call read: the thread keeps it, and what is written over it since
+        na.check(lib.nhVectorAbs(s, P(x, o), P(y, o), n))
+        na.check(lib.nhVectorNeg(s, P(y, o), P(x, o), n))
+        na.check(lib.nhVectorSqrt(s, P(y, o), P(y, o), n))
+        na.check(lib.nhVectorCopy(s, P(z, o), P(x, o), n))
+        na.check(lib.nhVectorFill(s, P(x, o), ctypes.c_float(1.0), n))
+
     def two_counts(s, x, y, z, n, o):
         # a call of another count, and a small one, between calls of one count: each run goes out before the next begins
         na.check(lib.nhVectorMultiply(s, P(x, o), P(y, o), n, P(scale)))
@@ -565,8 +588,8 @@ def test_large_calls_of_one_count_go_as_one_pass(streams):
 
     total = 3 * 1000 * 1000 + 16
     data = [g.normal(0, 2, total).astype(np.float32) for _ in range(3)]
-    for what in (gelu_layer, gelu_over_input, gelu_into_a_third, solver, momentum_solver, momentum_solver_plain, two_counts, shifted,
-                 alone):
+    for what in (gelu_layer, gelu_over_input, gelu_into_a_third, solver, momentum_solver, momentum_solver_plain, gradient_blob,
+                 overwritten_but_read_from_memory, overwritten_and_read_from_a_register, two_counts, shifted, alone):
         for n, o in ((3 * 1000 * 1000, 0), (3 * 1000 * 1000, 4), (3 * 1000 * 1000 + 2, 0), (3 * 1000 * 1000, 3), (262148, 8)):
             results = []
             for stream in (streams.plain, streams.deferring):
