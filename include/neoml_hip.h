@@ -441,13 +441,16 @@ NH_API int nhStreamOverlapLstm(nhStream s, int enable);
  * calls of CGELULayer's sigmoid form become one pass; a large call that no other joins goes out as the launch it
  * always was; nhAddVectorToMatrixColumns, nhMultiplyDiagMatrixByMatrix, nhAddVectorToMatrixRows and
  * nhBatchMultiplyMatrixByDiagMatrix with batch 1 over more than 262144 elements are such calls too, their vector spread
- * over the rows or columns: the last four calls of CObjectNormalizationLayer are one pass). Up to eight of them are launched together, in call order and with bit-identical results, as soon as ANY other call
+ * over the rows or columns: the last four calls of CObjectNormalizationLayer are one pass). Up to eight of them are
+ * launched together, in call order and with bit-identical results (a result that a later call of the same launch
+ * overwrites before anything reads it is not stored), as soon as ANY other call
  * on the stream through this library arrives: a larger or different operation, a copy, an event, nhStreamSynchronize,
  * nhStreamDestroy, enable = 0, or a release of device memory (nhRawFree, a pool's clean-up). Until then their results are
  * not in memory and their operands must stay valid, so this is only for streams whose work, synchronisation included,
  * all goes through this library (an engine's own stream): synchronise with nhStreamSynchronize, not with HIP calls of
  * your own. Nothing is put aside while the stream is being captured into a graph (synchronise through the library
- * before a capture begins: what was put aside before it would otherwise become the graph's first launch). What it saves: a row-normalising
+ * before a capture begins: what was put aside before it would otherwise become the graph's first launch). What it
+ * saves: a row-normalising
  * layer (CObjectNormalizationLayer) asks for five such calls per run, each a launch of about 4 us.
  * On such a stream nhMultiplyMatrixByTransposedMatrix with a dense result (resultRowSize == secondHeight) waits for the
  * call behind it as well: nhAddVectorToMatrixRows over that result in place (batchSize 1, the same height and width) is
@@ -455,7 +458,8 @@ NH_API int nhStreamOverlapLstm(nhStream s, int enable);
  * layer's two calls ask (NeoML/src/Dnn/Layers/FullyConnectedLayer.cpp:91-99); any other call launches the product first,
  * as it was asked for. The sum is the same; where the product is cut into slices of its reduction the vector is added
  * in front of the slices instead of behind them, i.e. the last bits may differ from the two launches'.
- * In the same way nhBlobConvolution and nhBlobChannelwiseConvolution wait for an nhVectorReLU or nhVectorHSwish over their result in place
+ * In the same way nhBlobConvolution and nhBlobChannelwiseConvolution wait for an nhVectorReLU or nhVectorHSwish over
+ * their result in place
  * (CConvLayer / CChannelwiseConvLayer followed by CReLULayer: the activation runs on the accumulators' way out, its
  * threshold read from the device scalar), and an nhVectorAdd over more than 262144 elements waits for an nhVectorReLU
  * over the sum in place (CEltwiseSumLayer + CReLULayer at the end of a residual block: one pass), and
