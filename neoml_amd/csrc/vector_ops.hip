@@ -497,10 +497,18 @@ struct CTanhDiffOutOp : CNoScalar { __device__ float operator()( float y, float 
 // call in front. Any other overlap ( a shifted view, a scalar that a call in front has produced ) needs every thread
 // to have finished the calls in front: the chain then runs in one workgroup with a barrier in front of such calls ( calls
 // over more than TinyOpMaxCount elements do not join such a chain: it is launched, and they begin the next one ).
+//
+// The same queue serves the passes of a layer over a whole blob: a call over more than TinyWideMaxCount elements begins
+// a chain that only calls of its own count join ( an activation's or a solver's passes over one blob, the passes of a
+// normalisation over its matrix, whose vectors per row or column are "spread" operands ). Such a chain never has barriers;
+// it runs four elements per thread with 128-bit accesses where the operands allow it ( quadChainKernel ), through a kernel
+// of its own if it is one of a few known sequences ( launchKnownChain ), and a call that nothing joined goes out as the
+// launch it always was. In every chain without barriers whose calls have one count, a result that a later call
+// overwrites before anything reads it from memory is computed but not stored ( CTinyOp::Dead ).
 
 constexpr int TinyChainMax = 8;
 constexpr int TinyOpMaxCount = 16384; // in a chain that runs as one workgroup
-constexpr int TinyWideMaxCount = 262144; // in a chain without barriers ( a solver's passes over a filter of a few hundred KB )
+constexpr int TinyWideMaxCount = 262144; // in a chain without barriers whose calls differ in count ( a filter and its free terms )
 constexpr int TinyThreads = 1024;
 constexpr int TinyFunctorBytes = 16;
 
