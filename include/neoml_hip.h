@@ -466,7 +466,9 @@ NH_API int nhStreamOverlapLstm(nhStream s, int enable);
  * nhBatchMultiplyMatrixByMatrix with a reduction of at most 256 waits for an nhVectorMultiply over its whole result in
  * place (CMatrixMultiplicationLayer + CLinearLayer: an attention layer's scores and their factor), and nhBlobResizeImage
  * with constant padding waits for an nhBlobMaxPooling (3x3, no indices) over the padded blob (CImageResizeLayer +
- * CMaxPoolingLayer: one launch writes both blobs). Same bits as the two launches. */
+ * CMaxPoolingLayer: one launch writes both blobs), and nhSumMatrixColumns waits for the element-wise calls with one
+ * operand in place over its sums (the mean and the inverse deviation of CObjectNormalizationLayer: the reduction's launch
+ * applies them to each row's value). Same bits as the separate launches. */
 NH_API int nhStreamDeferSmallOps(nhStream s, int enable);
 /* LSTM (NME.h:1005-1011). Weights: inputWeights [4H x objectSize], recurrentWeights [4H x H]; gate order in
  * the 4H vector: main(tanh) | forget | input | output (src/CPU/CpuMathEngineDnnLstm.h:49-90).

@@ -804,6 +804,10 @@ int nhSumMatrixColumns( nhStream s, float* result, const float* matrix, int matr
 	if( matrixHeight == 0 ) {
 		return NH_OK;
 	}
+	// ( on a stream that puts calls aside the sums wait for the small calls in place over them: one launch with those )
+	if( matrixWidth > 0 && deferColumnSum( s, result, matrix, matrixHeight, matrixWidth ) ) {
+		return NH_OK;
+	}
 	const int vec = ( matrixWidth % 4 == 0 && isAligned16( matrix ) ) ? 1 : 0;
 	hipLaunchKernelGGL( sumColumnsKernel, dim3( ceilDiv( matrixHeight, RowsPerBlock ) ), dim3( 256 ), 0, toStream( s ),
 		result, matrix, matrixHeight, matrixWidth, vec );

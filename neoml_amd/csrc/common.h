@@ -42,6 +42,8 @@ typedef void ( *CSpreadAlone )( hipStream_t stream, bool multiply, int spread, c
 	int height, int width );
 bool deferSpreadOp( nhStream s, bool multiply, int spread, const float* matrix, const float* vector, float* result, int height, int width,
 	CSpreadAlone alone );
+// The sums of a matrix's rows ( nhSumMatrixColumns ) wait for the element-wise calls in place over them: one launch
+bool deferColumnSum( nhStream s, float* result, const float* matrix, int height, int width );
 // An image blob padded with a constant ( nhBlobResizeImage ) that waits for the call behind it: a 3 x 3 max pooling over the
 // padded blob ( CImageResizeLayer + CMaxPoolingLayer, the way a pooling layer without padding of its own gets its border )
 // writes the padded blob and the pooled one in one pass over the image.

@@ -831,6 +831,18 @@ struct CPendingBatched {
 	int Batch = 0, M = 0, N = 0, K = 0;
 };
 
+// The sums of the rows of a matrix ( SumMatrixColumns: one value per row ) followed by element-wise calls with one operand
+// in place over those sums: the mean and the inverse deviation of CObjectNormalizationLayer ( sum, x -1/width; sum, x 1/width,
+// + epsilon, sqrt, 1/x ). The sum waits; such calls are queued behind it as its tail ( the queue's chain holds nothing else
+// while it waits ), and the launch of the sum applies them to each row's value before it is stored, with the calls' own
+// functors: one launch for the reduction and its tail. Any other call launches the sum with the tail it has by then.
+struct CPendingColumnSum {
+	bool Pending = false;
+	float* Result = nullptr;
+	const float* Matrix = nullptr;
+	int Height = 0, Width = 0;
+};
+
 struct CTinyQueue {
 	bool Enabled = false;
 	CTinyChain Chain = {};
@@ -844,8 +856,12 @@ struct CTinyQueue {
 	CPendingSum Sum;
 	CPendingBatched Batched;
 	CPendingPadding Padding;
+	CPendingColumnSum ColumnSum;
 
-	bool LaunchWaits() const { return Product.Pending || Convolution.Pending || Sum.Pending || Batched.Pending || Padding.Pending; }
+	bool LaunchWaits() const
+	{
+		return Product.Pending || Convolution.Pending || Sum.Pending || Batched.Pending || Padding.Pending || ColumnSum.Pending;
+	}
 };
 
 static int launchPlainSum( hipStream_t stream, const CPendingSum& sum );
@@ -1163,9 +1179,60 @@ static bool launchTinyChain( hipStream_t stream, CTinyQueue& queue )
 	return true;
 }
 
+// result[r] = tail( sum_c matrix[r][c] ): a wavefront per row ( sumColumnsKernel of blas_ops.hip, with the same order of
+// additions ), then the calls of the tail on the row's value, each with the functor and the device scalar of its own launch
+__global__ __launch_bounds__( 256 )
+void sumColumnsTailKernel( float* result, const float* matrix, int height, int width, int vec, const CTinyChain tail )
+{
+	const int row = blockIdx.x * 4 + ( threadIdx.x >> 6 );
+	if( row >= height ) {
+		return;
+	}
+	const int lane = threadIdx.x & 63;
+	const float* p = matrix + static_cast<long long>( row ) * width;
+	float s = 0.f;
+	if( vec ) {
+		const int w4 = width >> 2;
+		for( int i = lane; i < w4; i += 64 ) {
+			const float4 v = reinterpret_cast<const float4*>( p )[i];
+			s += ( v.x + v.y ) + ( v.z + v.w );
+		}
+	} else {
+		for( int i = lane; i < width; i += 64 ) {
+			s += p[i];
+		}
+	}
+	s = waveReduceSum( s );
+	if( lane == 0 ) {
+		const float none = 0.f;
+		for( int k = 0; k < tail.Length; ++k ) {
+			const CTinyOp& op = tail.Ops[k];
+			const float scalar = op.Scalar != nullptr ? *op.Scalar : 0.f;
+			float next = 0.f;
+			CTinyApply<CTinyKinds>::template Run<1>( op.Kind, op, scalar, &s, &none, &none, &next );
+			s = next;
+		}
+		result[row] = s;
+	}
+}
+
 // what the queue holds: the product that waits for its successor ( then nothing else is queued ), or a chain
 static bool launchPending( hipStream_t stream, CTinyQueue& queue )
 {
+	if( queue.ColumnSum.Pending ) {
+		const CPendingColumnSum sum = queue.ColumnSum;
+		queue.ColumnSum.Pending = false;
+		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+		CTinyChain& tail = queue.Chain; // ( calls in place over the sums, nothing else: deferEltwise sees to that )
+		const int vec = ( sum.Width % 4 == 0 && isAligned16( sum.Matrix ) ) ? 1 : 0;
+		hipLaunchKernelGGL( sumColumnsTailKernel, dim3( ceilDiv( sum.Height, 4 ) ), dim3( 256 ), 0, stream, sum.Result, sum.Matrix,
+			sum.Height, sum.Width, vec, tail );
+		if( tail.Length > 0 ) {
+			tail.Length = 0;
+			__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
+		}
+		return true;
+	}
 	if( queue.Product.Pending ) {
 		const CPendingProduct p = queue.Product;
 		queue.Product.Pending = false;
@@ -1339,6 +1406,34 @@ bool fusePendingProduct( nhStream s, const float* matrix, float* result, int hei
 	if( __atomic_load_n( &lstmPartnersAwaited, __ATOMIC_RELAXED ) != 0 ) {
 		noteStreamUse( stream );
 	}
+	return true;
+}
+
+bool deferColumnSum( nhStream s, float* result, const float* matrix, int height, int width )
+{
+	if( __atomic_load_n( &tinyDeferringStreams, __ATOMIC_RELAXED ) == 0 || result == nullptr || matrix == nullptr || height <= 0
+		|| width <= 0 ) {
+		return false;
+	}
+	const hipStream_t stream = toStream( s ); // ( what the stream holds goes out first )
+	int device = 0;
+	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+	if( hipGetDevice( &device ) != hipSuccess || hipStreamIsCapturing( stream, &capture ) != hipSuccess ) {
+		( void )hipGetLastError();
+		return false;
+	}
+	if( capture != hipStreamCaptureStatusNone ) {
+		return false;
+	}
+	std::lock_guard<std::recursive_mutex> guard( tinyLock );
+	auto found = tinyQueues().find( std::make_pair( device, stream ) );
+	if( found == tinyQueues().end() || !found->second.Enabled || found->second.Chain.Length != 0 || found->second.LaunchWaits() ) {
+		return false;
+	}
+	CPendingColumnSum& sum = found->second.ColumnSum;
+	sum.Pending = true;
+	sum.Result = result; sum.Matrix = matrix; sum.Height = height; sum.Width = width;
+	__atomic_fetch_add( &tinyChainsPending, 1, __ATOMIC_RELAXED );
 	return true;
 }
 
@@ -1656,7 +1751,16 @@ static bool deferEltwise( nhStream s, const TIn* a, const TIn* b, const TIn* c, 
 		if( found == tinyQueues().end() || !found->second.Enabled ) {
 			return false;
 		}
-		if( found->second.LaunchWaits() ) {
+		if( found->second.ColumnSum.Pending ) {
+			// row sums wait: a call with one operand, in place over exactly those sums, joins their tail
+			const CPendingColumnSum& sum = found->second.ColumnSum;
+			const float* own = scalarOf( f, 0 );
+			const bool tail = NIN == 1 && spread == TS_None && a == out && out == sum.Result && n == sum.Height
+				&& found->second.Chain.Length < TinyChainMax && ( own == nullptr || own + 1 <= out || own >= out + n );
+			if( !tail ) {
+				launchPending( stream, found->second );
+			}
+		} else if( found->second.LaunchWaits() ) {
 			launchPending( stream, found->second ); // ( a launch that waited for its successor: this call is not the one )
 		}
 		CTinyQueue& queue = found->second;

@@ -812,3 +812,37 @@ def test_padded_image_waits_for_its_pooling(streams):
         border = np.ones((th, tw), bool)
         border[dt:dt + h, dl:dl + w] = False
         assert np.all(padded[:, border, :] == np.float32(value))
+
+
+def test_row_sums_wait_for_the_calls_over_them(streams):
+    """nhSumMatrixColumns followed by element-wise calls with one operand in place over the sums (the mean and the inverse
+    deviation of CObjectNormalizationLayer, NeoML/src/Dnn/Layers/ObjectNormalizationLayer.cpp:190-214) is one launch;
+    same bits as the separate launches, also when the call behind the sums is no such call: over a part of them, into
+    another vector, with two operands, with its scalar among the sums, or more calls than a chain holds."""
+    g = rng(5000)
+    rows, width = 3000, 36
+    start = g.uniform(0.5, 2.0, ARENA).astype(np.float32)
+    x, sums, other, inv_w, eps = 0, 200000, 210000, ARENA - 8, ARENA - 4
+    start[inv_w], start[eps] = 1.0 / width, 1e-5
+    tails = {
+        "mean": [("nhVectorNegMultiply", [at(sums), at(sums), rows, at(inv_w)])],
+        "deviation": [("nhVectorMultiply", [at(sums), at(sums), rows, at(inv_w)]), ("nhVectorAddValue", [at(sums), at(sums), rows, at(eps)]),
+                      ("nhVectorSqrt", [at(sums), at(sums), rows]), ("nhVectorInv", [at(sums), at(sums), rows])],
+        "nothing": [],
+        "a part": [("nhVectorSqrt", [at(sums), at(sums), rows - 1])],
+        "into another vector": [("nhVectorSqrt", [at(sums), at(other), rows])],
+        "two operands": [("nhVectorAdd", [at(sums), at(sums), at(sums), rows])],
+        "its scalar among the sums": [("nhVectorMultiply", [at(sums), at(sums), rows, at(sums + 5)])],
+        "ten calls": [("nhVectorAbs" if k % 2 else "nhVectorNeg", [at(sums), at(sums), rows]) for k in range(10)],
+        "a second sum": [("nhVectorSqrt", [at(sums), at(sums), rows]), ("nhSumMatrixColumns", [at(other), at(x), rows, width]),
+                         ("nhVectorInv", [at(other), at(other), rows])],
+    }
+    for what, tail in tails.items():
+        for w in (width, width + 1):
+            program = [("nhSumMatrixColumns", [at(sums), at(x), rows, w])] + tail
+            want = streams.run(streams.plain, program, start)
+            got = streams.run(streams.deferring, program, start)
+            assert same_bits(got, want), (what, w)
+    got = streams.run(streams.deferring, [("nhSumMatrixColumns", [at(sums), at(x), rows, width])] + tails["mean"], start)
+    mean = start[:rows * width].astype(np.float64).reshape(rows, width).mean(1)
+    assert np.allclose(got[sums:sums + rows], -mean, rtol=1e-5, atol=1e-6)
