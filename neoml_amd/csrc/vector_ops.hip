@@ -841,6 +841,10 @@ struct CPendingColumnSum {
 	float* Result = nullptr;
 	const float* Matrix = nullptr;
 	int Height = 0, Width = 0;
+	// The matrix may itself be a sum of two that waited on the stream ( VectorAdd over the whole matrix: the residual sum in
+	// front of a normalisation ): the launch then adds the two, writes the matrix and sums its rows in one pass.
+	const float* AddFirst = nullptr;
+	const float* AddSecond = nullptr;
 };
 
 struct CTinyQueue {
@@ -1181,25 +1185,44 @@ static bool launchTinyChain( hipStream_t stream, CTinyQueue& queue )
 
 // result[r] = tail( sum_c matrix[r][c] ): a wavefront per row ( sumColumnsKernel of blas_ops.hip, with the same order of
 // additions ), then the calls of the tail on the row's value, each with the functor and the device scalar of its own launch
+// ( ADD: the matrix is first + second, written on the way )
+template<bool ADD>
 __global__ __launch_bounds__( 256 )
-void sumColumnsTailKernel( float* result, const float* matrix, int height, int width, int vec, const CTinyChain tail )
+void sumColumnsTailKernel( float* result, const float* matrix, const float* first, const float* second, float* sum, int height, int width,
+	int vec, const CTinyChain tail )
 {
 	const int row = blockIdx.x * 4 + ( threadIdx.x >> 6 );
 	if( row >= height ) {
 		return;
 	}
 	const int lane = threadIdx.x & 63;
-	const float* p = matrix + static_cast<long long>( row ) * width;
+	const long long offset = static_cast<long long>( row ) * width;
+	const float* p = matrix + offset;
 	float s = 0.f;
 	if( vec ) {
 		const int w4 = width >> 2;
 		for( int i = lane; i < w4; i += 64 ) {
-			const float4 v = reinterpret_cast<const float4*>( p )[i];
+			float4 v;
+			if( ADD ) {
+				const float4 x = reinterpret_cast<const float4*>( first + offset )[i];
+				const float4 y = reinterpret_cast<const float4*>( second + offset )[i];
+				v = make_float4( x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w );
+				reinterpret_cast<float4*>( sum + offset )[i] = v;
+			} else {
+				v = reinterpret_cast<const float4*>( p )[i];
+			}
 			s += ( v.x + v.y ) + ( v.z + v.w );
 		}
 	} else {
 		for( int i = lane; i < width; i += 64 ) {
-			s += p[i];
+			float v;
+			if( ADD ) {
+				v = first[offset + i] + second[offset + i];
+				sum[offset + i] = v;
+			} else {
+				v = p[i];
+			}
+			s += v;
 		}
 	}
 	s = waveReduceSum( s );
@@ -1224,9 +1247,15 @@ static bool launchPending( hipStream_t stream, CTinyQueue& queue )
 		queue.ColumnSum.Pending = false;
 		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
 		CTinyChain& tail = queue.Chain; // ( calls in place over the sums, nothing else: deferEltwise sees to that )
-		const int vec = ( sum.Width % 4 == 0 && isAligned16( sum.Matrix ) ) ? 1 : 0;
-		hipLaunchKernelGGL( sumColumnsTailKernel, dim3( ceilDiv( sum.Height, 4 ) ), dim3( 256 ), 0, stream, sum.Result, sum.Matrix,
-			sum.Height, sum.Width, vec, tail );
+		const int vec = ( sum.Width % 4 == 0 && isAligned16( sum.Matrix ) && isAligned16( sum.AddFirst ) && isAligned16( sum.AddSecond ) ) ? 1 : 0;
+		if( sum.AddFirst != nullptr ) {
+			hipLaunchKernelGGL( sumColumnsTailKernel<true>, dim3( ceilDiv( sum.Height, 4 ) ), dim3( 256 ), 0, stream, sum.Result, sum.Matrix,
+				sum.AddFirst, sum.AddSecond, const_cast<float*>( sum.Matrix ), sum.Height, sum.Width, vec, tail );
+		} else {
+			hipLaunchKernelGGL( sumColumnsTailKernel<false>, dim3( ceilDiv( sum.Height, 4 ) ), dim3( 256 ), 0, stream, sum.Result, sum.Matrix,
+				static_cast<const float*>( nullptr ), static_cast<const float*>( nullptr ), static_cast<float*>( nullptr ), sum.Height,
+				sum.Width, vec, tail );
+		}
 		if( tail.Length > 0 ) {
 			tail.Length = 0;
 			__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
@@ -1415,6 +1444,29 @@ bool deferColumnSum( nhStream s, float* result, const float* matrix, int height,
 		|| width <= 0 ) {
 		return false;
 	}
+	if( __atomic_load_n( &tinyChainsPending, __ATOMIC_RELAXED ) != 0 ) {
+		// a sum of two matrices that waits on the stream, and these are the sums of its rows: the two wait on as one
+		int current = 0;
+		if( hipGetDevice( &current ) != hipSuccess ) {
+			( void )hipGetLastError();
+			return false;
+		}
+		std::lock_guard<std::recursive_mutex> guard( tinyLock );
+		auto waiting = tinyQueues().find( std::make_pair( current, reinterpret_cast<hipStream_t>( s ) ) );
+		if( waiting != tinyQueues().end() && waiting->second.Sum.Pending ) {
+			const CPendingSum added = waiting->second.Sum;
+			const float* resultEnd = result + height;
+			const bool apart = resultEnd <= added.Result || added.Result + added.Count <= result;
+			if( added.Result == matrix && static_cast<long long>( added.Count ) == static_cast<long long>( height ) * width && apart ) {
+				waiting->second.Sum.Pending = false; // ( one thing waits where one waited: the count of waiting queues stays )
+				CPendingColumnSum& sum = waiting->second.ColumnSum;
+				sum.Pending = true;
+				sum.Result = result; sum.Matrix = matrix; sum.Height = height; sum.Width = width;
+				sum.AddFirst = added.First; sum.AddSecond = added.Second;
+				return true;
+			}
+		}
+	}
 	const hipStream_t stream = toStream( s ); // ( what the stream holds goes out first )
 	int device = 0;
 	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
@@ -1433,6 +1485,7 @@ bool deferColumnSum( nhStream s, float* result, const float* matrix, int height,
 	CPendingColumnSum& sum = found->second.ColumnSum;
 	sum.Pending = true;
 	sum.Result = result; sum.Matrix = matrix; sum.Height = height; sum.Width = width;
+	sum.AddFirst = nullptr; sum.AddSecond = nullptr;
 	__atomic_fetch_add( &tinyChainsPending, 1, __ATOMIC_RELAXED );
 	return true;
 }

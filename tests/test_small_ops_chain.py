@@ -702,6 +702,19 @@ def test_passes_over_a_matrix_with_vectors_spread_over_it(streams):
         na.check(lib.nhAddVectorToMatrixColumns(s, P(out, o), P(out, o), rows, width, P(inv_std)))
         na.check(lib.nhVectorEltwiseMultiply(s, P(out, o), P(out, o), P(out, o), n))
 
+    def residual_sum_in_front(s, x, out, sq, neg_mean, inv_std, scale, bias, inv_w, eps, rows, width, o):
+        # the sum of two matrices that waits on the stream and the sums of its rows are one pass; in place and not, and a
+        # reduction over fewer rows than the sum has, which leaves the two apart
+        n = rows * width
+        na.check(lib.nhVectorAdd(s, P(x, o), P(x, o), P(out, o), n))
+        na.check(lib.nhSumMatrixColumns(s, P(neg_mean), P(out, o), rows, width))
+        na.check(lib.nhVectorNegMultiply(s, P(neg_mean), P(neg_mean), rows, P(inv_w)))
+        na.check(lib.nhAddVectorToMatrixColumns(s, P(out, o), P(sq, o), rows, width, P(neg_mean)))
+        na.check(lib.nhVectorAdd(s, P(x, o), P(sq, o), P(x, o), n))
+        na.check(lib.nhSumMatrixColumns(s, P(inv_std), P(x, o), rows, width))
+        na.check(lib.nhVectorAdd(s, P(out, o), P(sq, o), P(out, o), n))
+        na.check(lib.nhSumMatrixColumns(s, P(neg_mean), P(out, o), rows - 1, width))
+
     def other_orders(s, x, out, sq, neg_mean, inv_std, scale, bias, inv_w, eps, rows, width, o):
         n = rows * width
         na.check(lib.nhSumMatrixColumns(s, P(neg_mean), P(x, o), rows, width))
@@ -719,7 +732,7 @@ def test_passes_over_a_matrix_with_vectors_spread_over_it(streams):
         n = rows * width
         x0 = g.normal(0.3, 1.5, n + 8).astype(np.float32)
         scale0, bias0 = g.normal(1, 0.2, width).astype(np.float32), g.normal(0, 0.5, width).astype(np.float32)
-        for what in (layer, tail_into_two_blobs, other_orders):
+        for what in (layer, tail_into_two_blobs, residual_sum_in_front, other_orders):
             results = []
             for stream in (streams.plain, streams.deferring):
                 x, scale, bias = up(x0), up(scale0), up(bias0)
