@@ -845,6 +845,10 @@ struct CPendingColumnSum {
 	// front of a normalisation ): the launch then adds the two, writes the matrix and sums its rows in one pass.
 	const float* AddFirst = nullptr;
 	const float* AddSecond = nullptr;
+	// ... or the squares of a matrix's distances from a value per row, the two calls in front of a normalisation's variance
+	// that waited as a chain ( matrix = ( SquareOf + SquareShift[row] )^2 ): computed, written and summed in one pass.
+	const float* SquareOf = nullptr;
+	const float* SquareShift = nullptr;
 };
 
 struct CTinyQueue {
@@ -1185,12 +1189,14 @@ static bool launchTinyChain( hipStream_t stream, CTinyQueue& queue )
 
 // result[r] = tail( sum_c matrix[r][c] ): a wavefront per row ( sumColumnsKernel of blas_ops.hip, with the same order of
 // additions ), then the calls of the tail on the row's value, each with the functor and the device scalar of its own launch
-// ( ADD: the matrix is first + second, written on the way )
-template<bool ADD>
+// ( PRODUCER 1: the matrix is first + second, 2: it is ( first + second[row] )^2; written on the way )
+template<int PRODUCER>
 __global__ __launch_bounds__( 256 )
 void sumColumnsTailKernel( float* result, const float* matrix, const float* first, const float* second, float* sum, int height, int width,
 	int vec, const CTinyChain tail )
 {
+	// ( a square must be rounded before it is added to its neighbour, as the separate launches' stored values are )
+#pragma clang fp contract( off )
 	const int row = blockIdx.x * 4 + ( threadIdx.x >> 6 );
 	if( row >= height ) {
 		return;
@@ -1198,15 +1204,21 @@ void sumColumnsTailKernel( float* result, const float* matrix, const float* firs
 	const int lane = threadIdx.x & 63;
 	const long long offset = static_cast<long long>( row ) * width;
 	const float* p = matrix + offset;
+	const float shift = PRODUCER == 2 ? second[row] : 0.f;
 	float s = 0.f;
 	if( vec ) {
 		const int w4 = width >> 2;
 		for( int i = lane; i < w4; i += 64 ) {
 			float4 v;
-			if( ADD ) {
+			if( PRODUCER == 1 ) {
 				const float4 x = reinterpret_cast<const float4*>( first + offset )[i];
 				const float4 y = reinterpret_cast<const float4*>( second + offset )[i];
 				v = make_float4( x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w );
+				reinterpret_cast<float4*>( sum + offset )[i] = v;
+			} else if( PRODUCER == 2 ) {
+				const float4 x = reinterpret_cast<const float4*>( first + offset )[i];
+				const float4 c = make_float4( x.x + shift, x.y + shift, x.z + shift, x.w + shift );
+				v = make_float4( c.x * c.x, c.y * c.y, c.z * c.z, c.w * c.w );
 				reinterpret_cast<float4*>( sum + offset )[i] = v;
 			} else {
 				v = reinterpret_cast<const float4*>( p )[i];
@@ -1216,8 +1228,12 @@ void sumColumnsTailKernel( float* result, const float* matrix, const float* firs
 	} else {
 		for( int i = lane; i < width; i += 64 ) {
 			float v;
-			if( ADD ) {
+			if( PRODUCER == 1 ) {
 				v = first[offset + i] + second[offset + i];
+				sum[offset + i] = v;
+			} else if( PRODUCER == 2 ) {
+				const float c = first[offset + i] + shift;
+				v = c * c;
 				sum[offset + i] = v;
 			} else {
 				v = p[i];
@@ -1247,12 +1263,16 @@ static bool launchPending( hipStream_t stream, CTinyQueue& queue )
 		queue.ColumnSum.Pending = false;
 		__atomic_fetch_sub( &tinyChainsPending, 1, __ATOMIC_RELAXED );
 		CTinyChain& tail = queue.Chain; // ( calls in place over the sums, nothing else: deferEltwise sees to that )
-		const int vec = ( sum.Width % 4 == 0 && isAligned16( sum.Matrix ) && isAligned16( sum.AddFirst ) && isAligned16( sum.AddSecond ) ) ? 1 : 0;
+		const int vec = ( sum.Width % 4 == 0 && isAligned16( sum.Matrix ) && isAligned16( sum.AddFirst ) && isAligned16( sum.AddSecond )
+			&& isAligned16( sum.SquareOf ) ) ? 1 : 0;
 		if( sum.AddFirst != nullptr ) {
-			hipLaunchKernelGGL( sumColumnsTailKernel<true>, dim3( ceilDiv( sum.Height, 4 ) ), dim3( 256 ), 0, stream, sum.Result, sum.Matrix,
+			hipLaunchKernelGGL( sumColumnsTailKernel<1>, dim3( ceilDiv( sum.Height, 4 ) ), dim3( 256 ), 0, stream, sum.Result, sum.Matrix,
 				sum.AddFirst, sum.AddSecond, const_cast<float*>( sum.Matrix ), sum.Height, sum.Width, vec, tail );
+		} else if( sum.SquareOf != nullptr ) {
+			hipLaunchKernelGGL( sumColumnsTailKernel<2>, dim3( ceilDiv( sum.Height, 4 ) ), dim3( 256 ), 0, stream, sum.Result, sum.Matrix,
+				sum.SquareOf, sum.SquareShift, const_cast<float*>( sum.Matrix ), sum.Height, sum.Width, vec, tail );
 		} else {
-			hipLaunchKernelGGL( sumColumnsTailKernel<false>, dim3( ceilDiv( sum.Height, 4 ) ), dim3( 256 ), 0, stream, sum.Result, sum.Matrix,
+			hipLaunchKernelGGL( sumColumnsTailKernel<0>, dim3( ceilDiv( sum.Height, 4 ) ), dim3( 256 ), 0, stream, sum.Result, sum.Matrix,
 				static_cast<const float*>( nullptr ), static_cast<const float*>( nullptr ), static_cast<float*>( nullptr ), sum.Height,
 				sum.Width, vec, tail );
 		}
@@ -1463,6 +1483,30 @@ bool deferColumnSum( nhStream s, float* result, const float* matrix, int height,
 				sum.Pending = true;
 				sum.Result = result; sum.Matrix = matrix; sum.Height = height; sum.Width = width;
 				sum.AddFirst = added.First; sum.AddSecond = added.Second;
+				sum.SquareOf = nullptr; sum.SquareShift = nullptr;
+				return true;
+			}
+		}
+		if( waiting != tinyQueues().end() && !waiting->second.LaunchWaits() && waiting->second.Chain.Length == 2 ) {
+			// the chain "matrix = source + value per row; matrix *= matrix" waits, and these are the sums of that matrix's rows
+			CTinyChain& chain = waiting->second.Chain;
+			const CTinyOp& centre = chain.Ops[0];
+			const CTinyOp& square = chain.Ops[1];
+			const float* resultEnd = result + height;
+			const long long count = static_cast<long long>( height ) * width;
+			const bool apart = ( resultEnd <= centre.Out || centre.Out + count <= result )
+				&& ( resultEnd <= centre.In[0] || centre.In[0] + count <= result )
+				&& ( resultEnd <= centre.In[1] || centre.In[1] + height <= result );
+			if( centre.Kind == CKindOf<CAddOp<float>, CTinyKinds>::Value && square.Kind == CKindOf<CMulOp<float>, CTinyKinds>::Value
+				&& centre.Spread == TS_PerRow && square.Spread == TS_None && centre.Width == width && centre.Count == count
+				&& square.Count == count && centre.Out == matrix && square.In[0] == matrix && square.In[1] == matrix && square.Out == matrix
+				&& centre.Barrier == 0 && square.Barrier == 0 && apart ) {
+				CPendingColumnSum& sum = waiting->second.ColumnSum;
+				sum.Pending = true;
+				sum.Result = result; sum.Matrix = matrix; sum.Height = height; sum.Width = width;
+				sum.AddFirst = nullptr; sum.AddSecond = nullptr;
+				sum.SquareOf = centre.In[0]; sum.SquareShift = centre.In[1];
+				chain.Length = 0; // ( one thing waits where one waited )
 				return true;
 			}
 		}
@@ -1486,6 +1530,7 @@ bool deferColumnSum( nhStream s, float* result, const float* matrix, int height,
 	sum.Pending = true;
 	sum.Result = result; sum.Matrix = matrix; sum.Height = height; sum.Width = width;
 	sum.AddFirst = nullptr; sum.AddSecond = nullptr;
+	sum.SquareOf = nullptr; sum.SquareShift = nullptr;
 	__atomic_fetch_add( &tinyChainsPending, 1, __ATOMIC_RELAXED );
 	return true;
 }

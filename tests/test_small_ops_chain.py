@@ -701,6 +701,12 @@ def test_passes_over_a_matrix_with_vectors_spread_over_it(streams):
         na.check(lib.nhSumMatrixColumns(s, P(inv_std), P(x, o), rows, width))
         na.check(lib.nhAddVectorToMatrixColumns(s, P(out, o), P(out, o), rows, width, P(inv_std)))
         na.check(lib.nhVectorEltwiseMultiply(s, P(out, o), P(out, o), P(out, o), n))
+        # sums over fewer rows than the squares have, and sums that would land in the vector the squares were centred with:
+        # the squares go out by themselves
+        na.check(lib.nhSumMatrixColumns(s, P(neg_mean), P(out, o), rows - 1, width))
+        na.check(lib.nhAddVectorToMatrixColumns(s, P(x, o), P(sq, o), rows, width, P(inv_std)))
+        na.check(lib.nhVectorEltwiseMultiply(s, P(sq, o), P(sq, o), P(sq, o), n))
+        na.check(lib.nhSumMatrixColumns(s, P(inv_std), P(sq, o), rows, width))
 
     def residual_sum_in_front(s, x, out, sq, neg_mean, inv_std, scale, bias, inv_w, eps, rows, width, o):
         # the sum of two matrices that waits on the stream and the sums of its rows are one pass; in place and not, and a
